@@ -1,0 +1,19 @@
+"""fly_amd -- MI355X (gfx950) implementation of the Scatterbrain / Pixelfly hot path of
+HazyResearch/fly: SBLocalAttention and the block-sparse matmul / softmax family, as hand-written
+HIP kernels behind the reference's module interfaces.  The kernels live in ``libflyhip.so``
+(built from ``csrc/`` by ``python -m fly_amd.build``); nothing here falls back to a CPU path."""
+from .masking import FullMask, LengthMask, TriangularCausalMask
+from .feature_maps_sb import SBPerformerFeatures, gaussian_orthogonal_random_matrix
+from .sblocal_attention import SBLocalAttention, sblocal_forward
+from .blocksparse_utils import sparsify_tensor, densify_tensor, mask_tensor, sparsify_broadcast_tensor
+from .blocksparse_matmul import matmul
+from .blocksparse_softmax import softmax, logsumexp, blocksparse_sum
+from .blocksparse_attention import BlockSparseAttention
+from .blocksparse_linear import BlockSparseLinear, FlatBlockButterflySparsityConfig
+from .fastlinear import LowRank, SparseLRLinear
+
+__all__ = ['FullMask', 'LengthMask', 'TriangularCausalMask', 'SBPerformerFeatures',
+           'gaussian_orthogonal_random_matrix', 'SBLocalAttention', 'sblocal_forward',
+           'sparsify_tensor', 'densify_tensor', 'mask_tensor', 'sparsify_broadcast_tensor',
+           'matmul', 'softmax', 'logsumexp', 'blocksparse_sum', 'BlockSparseAttention',
+           'BlockSparseLinear', 'FlatBlockButterflySparsityConfig', 'LowRank', 'SparseLRLinear']

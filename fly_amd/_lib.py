@@ -1,0 +1,87 @@
+"""ctypes binding of ``libflyhip.so`` (the C ABI declared in ``include/flyhip.h``).
+
+The library is loaded lazily from the package directory.  There is no CPU fallback: if the
+shared object is missing, or a tensor is not on a GPU, the call raises.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, 'libflyhip.so')
+
+c_int, c_i64, c_float, c_vp = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
+
+# name -> argument ctypes, in the order of include/flyhip.h
+SIGNATURES = {
+    'flyhip_version': [],
+    'flyhip_sb_plan': [c_int, c_int, c_int, ctypes.POINTER(c_int), ctypes.POINTER(c_int)],
+    'flyhip_sb_kv_reduce': [c_vp] * 11 + [c_int] * 8 + [c_i64] * 6 + [c_float, c_int, c_vp],
+    'flyhip_sblocal_fwd': [c_vp] * 12 + [c_int] * 9 + [c_i64] * 12 + [c_float, c_int, c_vp],
+    'flyhip_bs_sdd': [c_vp] * 4 + [c_int] * 4 + [c_i64] * 8 + [c_int, c_vp],
+    'flyhip_bs_dsd': [c_vp] * 6 + [c_int] * 6 + [c_i64] * 9 + [c_int, c_vp],
+    'flyhip_bs_dds': [c_vp] * 6 + [c_int] * 6 + [c_i64] * 9 + [c_int, c_vp],
+    'flyhip_bs_softmax': [c_vp] * 4 + [c_int] * 5 + [c_i64, c_float, c_vp, c_i64, c_int, c_vp, c_i64,
+                                                    c_int, c_int, c_vp],
+    'flyhip_bs_rowreduce': [c_vp] * 4 + [c_int] * 3 + [c_i64, c_int, c_int, c_vp],
+}
+
+_lib = None
+
+
+def load():
+    """Load libflyhip.so (once) and declare the prototypes."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(f'{LIB_PATH} is missing: build it with `python -m fly_amd.build` '
+                           '(there is no fallback implementation)')
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, argtypes in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.argtypes = argtypes
+        fn.restype = c_int
+    lib.flyhip_last_error.argtypes = []
+    lib.flyhip_last_error.restype = ctypes.c_char_p
+    _lib = lib
+    return lib
+
+
+def call(name, *args):
+    """Invoke an entry point; a negative return code becomes a RuntimeError with the library's
+    message."""
+    lib = load()
+    rc = getattr(lib, name)(*args)
+    if rc != 0:
+        raise RuntimeError(f'{name} failed ({rc}): {lib.flyhip_last_error().decode()}')
+
+
+DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
+
+
+def dtype_code(t):
+    try:
+        return DTYPE_CODE[t.dtype]
+    except KeyError:
+        raise ValueError(f'unsupported dtype {t.dtype}; expected float32, bfloat16 or float16') from None
+
+
+def ptr(t):
+    """Device pointer of a tensor, or NULL for None."""
+    return None if t is None else t.data_ptr()
+
+
+def stream_ptr(device):
+    """The hipStream_t PyTorch currently enqueues on for `device`."""
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def require_gpu(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise ValueError('the HIP kernels only accept GPU tensors (no CPU implementation is shipped)')
+    dev = {t.device for t in tensors if t is not None}
+    if len(dev) > 1:
+        raise ValueError(f'tensors live on different devices: {sorted(map(str, dev))}')

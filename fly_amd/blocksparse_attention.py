@@ -1,0 +1,117 @@
+"""Block-sparse softmax attention on the HIP kernels: drop-in for
+src/models/attention/blocksparse_attention.py:23-166 (SDD -> block softmax -> DSD)."""
+import importlib
+import math
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+from torch import distributed as dist
+
+from .blocksparse_matmul import matmul
+from .blocksparse_softmax import softmax
+from .blocksparse_utils import densify_tensor
+from .masking import FullMask, LengthMask, pad_mask
+from .padding import pad_to_multiple
+
+
+def instantiate(cfg, *args, **kwargs):
+    """Resolve a plugin description the way the reference's hydra.utils.instantiate call sites do
+    (blocksparse_attention.py:39, blocksparse_linear.py:49, fastlinear.py:789): a mapping with a
+    ``_target_`` dotted path plus keyword arguments becomes an object; anything else is taken to be
+    the object itself."""
+    if isinstance(cfg, dict) or (hasattr(cfg, 'keys') and '_target_' in cfg):
+        cfg = dict(cfg)
+        target = cfg.pop('_target_')
+        cfg.pop('_recursive_', None)
+        module, _, name = target.rpartition('.')
+        # reference paths resolve to this package's drop-ins
+        module = {'src.models.layers.blocksparse_linear': 'fly_amd.blocksparse_linear',
+                  'src.models.layers.fastlinear': 'fly_amd.fastlinear',
+                  'src.models.attention.sblocal_attention': 'fly_amd.sblocal_attention',
+                  'src.models.attention.blocksparse_attention': 'fly_amd.blocksparse_attention',
+                  }.get(module, module)
+        return getattr(importlib.import_module(module), name)(*args, **{**cfg, **kwargs})
+    return cfg
+
+
+class BlockSparseAttention(nn.Module):
+    """Softmax attention restricted to the nonzero blocks of ``sparsity_config.make_layout``.
+
+    sparsity_config: an object with ``.block`` and ``.make_layout(seq_len) -> (H, nb, nb)`` or a
+    mapping with ``_target_``.  Same forward convention as the reference: query (B,T,H,E), key
+    (B,S,H,E), value (B,S,H,D), optional FullMask attn_mask and key_padding_mask, returns
+    (out (B,T,H,D), attn or None)."""
+
+    def __init__(self, sparsity_config, softmax_temp=None, attention_dropout=0.1, max_seq_length=2048):
+        super().__init__()
+        self.sparsity_config = instantiate(sparsity_config)
+        self.softmax_temp = softmax_temp
+        self.dropout = nn.Dropout(attention_dropout)
+        master_layout = self.sparsity_config.make_layout(max_seq_length)
+        self.register_buffer("master_layout", master_layout)
+        self._need_layout_synchronization = True
+        self.ops_cache = dict()
+
+    def get_layout(self, T, S=None):
+        if S is None:
+            S = T
+        if self._need_layout_synchronization and dist.is_available() and dist.is_initialized():
+            dist.broadcast(self.master_layout, src=0)
+            self._need_layout_synchronization = False
+        block = self.sparsity_config.block
+        if (T % block != 0) or (S % block != 0):
+            raise ValueError(f'Sequence lengths, {T} and {S}, needs to be divisible by block size {block}!')
+        return self.master_layout[..., :T // block, :S // block].cpu()
+
+    def get_ops(self, T, S=None):
+        if S is None:
+            S = T
+        if (T, S) not in self.ops_cache:
+            layout = self.get_layout(T, S)
+            block = self.sparsity_config.block
+            self.ops_cache[T, S] = (matmul(layout, block, 'sdd', trans_a=False, trans_b=True),
+                                    matmul(layout, block, 'dsd', trans_a=False, trans_b=False),
+                                    softmax(layout, block))
+        return self.ops_cache[T, S]
+
+    def forward(self, query, key, value, attn_mask=None, key_padding_mask=None, need_weights=False):
+        block = self.sparsity_config.block
+        _, q_seqlen_og, n_head, q_dim_og = query.shape
+        k_seqlen_og = key.shape[1]
+        v_dim_og = value.shape[3]
+        query = pad_to_multiple(query, block, dims=(1, 3))          # :107-109
+        key = pad_to_multiple(key, block, dims=(1, 3))
+        value = pad_to_multiple(value, block, dims=(1, 3))
+        B, T, H, E = query.shape
+        S = value.shape[1]
+        softmax_temp = self.softmax_temp or 1 / math.sqrt(q_dim_og)  # :114
+
+        if S > k_seqlen_og:                                          # :117-123
+            if key_padding_mask is None:
+                key_padding_mask = LengthMask(key.new_full((key.shape[0],), k_seqlen_og, dtype=torch.long),
+                                              max_len=S)
+            else:
+                key_padding_mask = pad_mask(key_padding_mask, pad_length=S - k_seqlen_og, left=False,
+                                            value=False)
+        if attn_mask is not None and (S > k_seqlen_og or T > q_seqlen_og):   # :125-127
+            attn_mask = FullMask(F.pad(attn_mask._mask, (0, S - k_seqlen_og, 0, T - q_seqlen_og), value=False))
+
+        # the kernels read (B,T,H,E) through strides: no permuted copies (the reference makes
+        # contiguous (B,H,T,E) tensors at :130-132)
+        q, k, v = (x.permute(0, 2, 1, 3) for x in (query, key, value))
+        layout = self.get_layout(T, S)
+        sdd_nt, dsd_nn, sparse_softmax = self.get_ops(T, S)
+        qk = sdd_nt(q, k)
+        attn = sparse_softmax(qk, scale=softmax_temp,
+                              key_padding_mask=None if key_padding_mask is None else key_padding_mask.additive_matrix,
+                              attn_mask=None if attn_mask is None else attn_mask.additive_matrix,
+                              key_padding_mask_mode='add', attn_mask_mode='add')
+        if ((key_padding_mask is not None and not key_padding_mask.all_ones)
+                or (attn_mask is not None and not attn_mask.all_ones)):
+            attn.nan_to_num_()                                        # :156-158: fully masked rows -> 0
+        out = dsd_nn(self.dropout(attn), v)
+        weights = None
+        if need_weights:
+            weights = densify_tensor(attn, layout)[:, :, :q_seqlen_og, :k_seqlen_og]
+        return out.permute(0, 2, 1, 3)[:, :q_seqlen_og, :, :v_dim_og], weights

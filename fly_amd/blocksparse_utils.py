@@ -1,0 +1,101 @@
+"""The block-sparse storage format (src/models/attention/blocksparse_utils.py:8-74) and the index
+tables the HIP kernels walk.
+
+A sparse tensor is (..., nnz, blk, blk1): block n is the n-th nonzero of ``layout.flatten()`` for a
+layout (H, rows/blk, cols/blk1), i.e. nonzero blocks in (head, block-row, block-col) row-major
+order, each stored row-major.
+"""
+import torch
+
+
+def _as_layout3(layout):
+    layout = torch.as_tensor(layout)
+    if layout.ndim == 2:
+        layout = layout.unsqueeze(0)
+    if layout.ndim != 3:
+        raise ValueError('layout must be a 2- or 3-dimensional tensor of 0s and 1s')
+    return layout
+
+
+def sparsify_tensor(x, mask):
+    """x (..., H, T, S), mask (H, T/blk, S/blk1) -> (..., nnz, blk, blk1)   (:8-19)."""
+    H, p, r = mask.shape
+    blk, blk1 = x.shape[-2] // p, x.shape[-1] // r
+    lead = x.shape[:-3]
+    blocks = x.reshape(*lead, H, p, blk, r, blk1).transpose(-3, -2).reshape(*lead, H * p * r, blk, blk1)
+    return blocks[..., mask.flatten().bool().to(x.device), :, :]
+
+
+def densify_tensor(x, mask, value=0.0):
+    """x (..., nnz, blk, blk1), mask (H, p, r) -> (..., H, p*blk, r*blk1), `value` elsewhere (:22-40)."""
+    mask = mask.bool().to(x.device)
+    lead = x.shape[:-3]
+    nnz, blk, blk1 = x.shape[-3:]
+    H, p, r = mask.shape
+    assert nnz == mask.sum(), 'Mask has a different number of nonzero blocks than input'
+    dense = torch.full((*lead, H * p * r, blk, blk1), value, dtype=x.dtype, device=x.device)
+    dense[..., mask.flatten(), :, :] = x
+    return dense.reshape(*lead, H, p, r, blk, blk1).transpose(-3, -2).reshape(*lead, H, p * blk, r * blk1)
+
+
+def mask_tensor(x, mask, value=0.0):
+    """Keep the nonzero blocks of x (..., H, T, S), set the others to `value` (:45-57)."""
+    H, p, r = mask.shape
+    blk, blk1 = x.shape[-2] // p, x.shape[-1] // r
+    keep = mask.bool().to(x.device).repeat_interleave(blk, dim=1).repeat_interleave(blk1, dim=2)
+    return x.masked_fill(~keep, value)
+
+
+def sparsify_broadcast_tensor(x, mask, block=None):
+    """x (B, H, T) -> (B, nnz, blk, 1): for every nonzero block the slice of x for its rows (:60-74).
+    `block` is accepted and ignored: the reference's callers pass it although the reference
+    function takes two arguments (sbblocksparse_attention.py:197,199)."""
+    blk = x.shape[-1] // mask.shape[-2]
+    rows = x.reshape(x.shape[0], x.shape[1], mask.shape[-2], blk, 1)
+    h_idx, row_idx, _ = torch.nonzero(mask, as_tuple=True)
+    return rows[:, h_idx.to(x.device), row_idx.to(x.device)]
+
+
+# -----------------------------------------------------------------------------------------
+# index tables (host side, int32) -- the information of the reference's look-up tables
+# (blocksparse_matmul.py:261-276, 356-441; blocksparse_logsumexp.py:107-128) in the CSR-like
+# form the HIP kernels consume
+# -----------------------------------------------------------------------------------------
+def sdd_table(layout):
+    """int32 (nnz, 4): (head, block_row, block_col, block_id) per nonzero block, storage order."""
+    layout = _as_layout3(layout).cpu()
+    nz = layout.nonzero(as_tuple=False)
+    ids = torch.arange(nz.shape[0], dtype=nz.dtype).unsqueeze(1)
+    return torch.cat([nz, ids], dim=1).to(torch.int32).contiguous()
+
+
+def segment_table(layout, by_rows):
+    """Reduction lists per (head, block-row) [by_rows] or (head, block-col): returns
+    (seg_ptr int32 (n_seg+1), seg_blk int32 (nnz) block ids, seg_inner int32 (nnz) the block index
+    along the other axis), blocks of a segment in increasing inner index."""
+    layout = _as_layout3(layout).cpu().long()
+    H, p, r = layout.shape
+    nz = layout.nonzero(as_tuple=False)                      # storage order: (h, row, col)
+    ids = torch.arange(nz.shape[0])
+    if by_rows:
+        seg = nz[:, 0] * p + nz[:, 1]
+        inner = nz[:, 2]
+        n_seg = H * p
+    else:
+        key = (nz[:, 0] * r + nz[:, 2]) * p + nz[:, 1]       # sort by (h, col, row)
+        order = torch.argsort(key, stable=True)
+        nz, ids = nz[order], ids[order]
+        seg = nz[:, 0] * r + nz[:, 2]
+        inner = nz[:, 1]
+        n_seg = H * r
+    counts = torch.bincount(seg, minlength=n_seg)
+    ptr = torch.zeros(n_seg + 1, dtype=torch.int64)
+    ptr[1:] = torch.cumsum(counts, 0)
+    return ptr.to(torch.int32), ids.to(torch.int32).contiguous(), inner.to(torch.int32).contiguous()
+
+
+def row_table(layout):
+    """Per (head, block-row): (row_ptr, row_blk, row_col, max_row_nnz) for the row operations."""
+    ptr, blk, col = segment_table(layout, by_rows=True)
+    counts = ptr[1:] - ptr[:-1]
+    return ptr, blk, col, int(counts.max()) if counts.numel() else 0

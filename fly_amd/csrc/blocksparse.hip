@@ -1,0 +1,511 @@
+// Block-sparse matmuls (SDD / DSD / DDS) and block-sparse row operations for gfx950.
+//
+// Sparse tensors are (Z, nnz, blk, blk) with block n the n-th nonzero of the (H, rows, cols)
+// layout in row-major order.  Every matmul wave owns one register tile of the output (up to
+// 32x32, built from 16x16 MFMA results) and walks its reduction list, reading operand fragments
+// straight from global memory (16-byte / 8-byte vector loads when the contraction index is
+// contiguous, strided gathers otherwise).  Products are formed with the operand that supplies
+// the output columns on the MFMA "A" side, so a lane ends up with four consecutive output
+// columns of one row and writes them with a single vector store.
+#include "common.h"
+#include <math.h>
+
+namespace flyhip {
+
+template <typename T>
+__device__ __forceinline__ typename Frag<T>::type frag_at(const T* p, long k_stride) {
+    // four contraction elements starting at p, spaced by k_stride
+    if (k_stride == 1) return Frag<T>::load(p);
+    return Frag<T>::gather(p, k_stride);
+}
+
+template <typename T>
+__device__ __forceinline__ void store_tile_row(T* p, long col_stride, floatx4 v, int ncols_left) {
+    // v holds four consecutive output columns starting at p
+    if (col_stride == 1 && ncols_left >= 4) { store4_f32(p, v); return; }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        if (i < ncols_left) p[i * col_stride] = Elem<T>::from_f32(v[i]);
+}
+
+// ---------------------------------------------------------------------------------------
+// SDD: sparse = dense x dense^T
+// ---------------------------------------------------------------------------------------
+struct SddArgs {
+    const void* a; const void* b; void* c; const int32_t* lut;
+    int nnz, K;
+    long a_sz, a_sh, a_sm, a_sk, b_sz, b_sh, b_sn, b_sk;
+};
+
+template <typename T, int BLK>
+__global__ __launch_bounds__(256) void bs_sdd_kernel(SddArgs a) {
+    constexpr int TILE = BLK >= 32 ? 32 : 16, NTL = TILE / 16, SUB = BLK / TILE;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, r16 = lane & 15, g = lane >> 4;
+    const long wid = (long)blockIdx.x * 4 + w;
+    const int n = (int)(wid / (SUB * SUB)), sub = (int)(wid % (SUB * SUB));
+    if (n >= a.nnz) return;
+    const int z = blockIdx.y;
+    const int head = a.lut[4 * n], bi = a.lut[4 * n + 1], bj = a.lut[4 * n + 2], id = a.lut[4 * n + 3];
+    const int ml = (sub / SUB) * TILE, nl = (sub % SUB) * TILE;      // tile origin inside the block
+    const T* ap = reinterpret_cast<const T*>(a.a) + z * a.a_sz + head * a.a_sh + (long)(bi * BLK + ml) * a.a_sm;
+    const T* bp = reinterpret_cast<const T*>(a.b) + z * a.b_sz + head * a.b_sh + (long)(bj * BLK + nl) * a.b_sn;
+
+    floatx4 acc[NTL][NTL];
+#pragma unroll
+    for (int tm = 0; tm < NTL; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < NTL; ++tn) acc[tm][tn] = Frag<float>::zero();
+
+    for (int kk = 0; kk < a.K; kk += 16) {
+        typename Frag<T>::type fa[NTL], fb[NTL];
+#pragma unroll
+        for (int t = 0; t < NTL; ++t) {
+            fa[t] = frag_at<T>(ap + (long)(16 * t + r16) * a.a_sm + (long)(kk + 4 * g) * a.a_sk, a.a_sk);
+            fb[t] = frag_at<T>(bp + (long)(16 * t + r16) * a.b_sn + (long)(kk + 4 * g) * a.b_sk, a.b_sk);
+        }
+#pragma unroll
+        for (int tm = 0; tm < NTL; ++tm)
+#pragma unroll
+            for (int tn = 0; tn < NTL; ++tn) acc[tm][tn] = Frag<T>::mma(fb[tn], fa[tm], acc[tm][tn]);
+    }
+    // lane holds C[m = 16tm + r16][n = 16tn + 4g + i]
+    T* cp = reinterpret_cast<T*>(a.c) + ((long)z * a.nnz + id) * (BLK * BLK);
+#pragma unroll
+    for (int tm = 0; tm < NTL; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < NTL; ++tn)
+            store4_f32(cp + (ml + 16 * tm + r16) * BLK + nl + 16 * tn + 4 * g, acc[tm][tn]);
+}
+
+// ---------------------------------------------------------------------------------------
+// DSD: dense = sparse x dense
+// ---------------------------------------------------------------------------------------
+struct DxdArgs {
+    const void* sp; const void* dn; void* c;
+    const int32_t* seg_ptr; const int32_t* seg_blk; const int32_t* seg_inner;
+    int n_seg, per_head, X, trans;      // X = N (DSD: dense columns) or M (DDS: dense rows)
+    long sp_sz;
+    long dn_sz, dn_sh, dn_s0, dn_s1;    // DSD: (k, n) strides; DDS: (m, k) strides
+    long c_sz, c_sh, c_sm, c_sn;
+};
+
+template <typename T, int BLK>
+__global__ __launch_bounds__(256) void bs_dsd_kernel(DxdArgs a) {
+    constexpr int TILE = BLK >= 32 ? 32 : 16, NTL = TILE / 16, SUBM = BLK / TILE;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, r16 = lane & 15, g = lane >> 4;
+    const int ntn = (a.X + 31) / 32;
+    const long wid = (long)blockIdx.x * 4 + w;
+    const long per_seg = (long)SUBM * ntn;
+    const int seg = (int)(wid / per_seg);
+    if (seg >= a.n_seg) return;
+    const int rem = (int)(wid % per_seg), subm = rem / ntn, nt = rem % ntn;
+    const int z = blockIdx.y;
+    const int head = seg / a.per_head, brow = seg % a.per_head;
+    const int n0 = nt * 32;
+    const T* spz = reinterpret_cast<const T*>(a.sp) + z * a.sp_sz;
+    const T* dnp = reinterpret_cast<const T*>(a.dn) + z * a.dn_sz + head * a.dn_sh;
+
+    floatx4 acc[NTL][2];
+#pragma unroll
+    for (int tm = 0; tm < NTL; ++tm) { acc[tm][0] = Frag<float>::zero(); acc[tm][1] = Frag<float>::zero(); }
+    bool nok[2];
+    nok[0] = n0 + r16 < a.X;
+    nok[1] = n0 + 16 + r16 < a.X;
+
+    const int p1 = a.seg_ptr[seg + 1];
+    for (int p = a.seg_ptr[seg]; p < p1; ++p) {
+        const T* blkp = spz + (long)a.seg_blk[p] * (BLK * BLK);
+        const long krow0 = (long)a.seg_inner[p] * BLK;
+#pragma unroll
+        for (int kk = 0; kk < BLK; kk += 16) {
+            typename Frag<T>::type fs[NTL], fd[2];
+#pragma unroll
+            for (int tm = 0; tm < NTL; ++tm) {
+                const int m = subm * TILE + 16 * tm + r16;
+                fs[tm] = a.trans ? Frag<T>::gather(blkp + (kk + 4 * g) * BLK + m, BLK)
+                                 : Frag<T>::load(blkp + m * BLK + kk + 4 * g);
+            }
+#pragma unroll
+            for (int tn = 0; tn < 2; ++tn) {
+                fd[tn] = Frag<T>::zero();
+                if (nok[tn])
+                    fd[tn] = frag_at<T>(dnp + (krow0 + kk + 4 * g) * a.dn_s0 + (long)(n0 + 16 * tn + r16) * a.dn_s1, a.dn_s0);
+            }
+#pragma unroll
+            for (int tm = 0; tm < NTL; ++tm) {
+                acc[tm][0] = Frag<T>::mma(fd[0], fs[tm], acc[tm][0]);
+                acc[tm][1] = Frag<T>::mma(fd[1], fs[tm], acc[tm][1]);
+            }
+        }
+    }
+    T* cp = reinterpret_cast<T*>(a.c) + z * a.c_sz + head * a.c_sh;
+#pragma unroll
+    for (int tm = 0; tm < NTL; ++tm) {
+        const long m = (long)brow * BLK + subm * TILE + 16 * tm + r16;
+#pragma unroll
+        for (int tn = 0; tn < 2; ++tn) {
+            const int n = n0 + 16 * tn + 4 * g;
+            if (n < a.X) store_tile_row<T>(cp + m * a.c_sm + n * a.c_sn, a.c_sn, acc[tm][tn], a.X - n);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// DDS: dense = dense x sparse
+// ---------------------------------------------------------------------------------------
+template <typename T, int BLK>
+__global__ __launch_bounds__(256) void bs_dds_kernel(DxdArgs a) {
+    constexpr int TILE = BLK >= 32 ? 32 : 16, NTL = TILE / 16, SUBN = BLK / TILE;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, r16 = lane & 15, g = lane >> 4;
+    const long wid = (long)blockIdx.x * 4 + w;
+    const long per_mt = (long)a.n_seg * SUBN;
+    const long mt = wid / per_mt;
+    if (mt * 32 >= a.X) return;
+    const int rem = (int)(wid % per_mt), seg = rem / SUBN, subn = rem % SUBN;
+    const int z = blockIdx.y;
+    const int head = seg / a.per_head, bcol = seg % a.per_head;
+    const long m0 = mt * 32;
+    const T* spz = reinterpret_cast<const T*>(a.sp) + z * a.sp_sz;
+    const T* dnp = reinterpret_cast<const T*>(a.dn) + z * a.dn_sz + head * a.dn_sh;
+
+    floatx4 acc[2][NTL];
+#pragma unroll
+    for (int tn = 0; tn < NTL; ++tn) { acc[0][tn] = Frag<float>::zero(); acc[1][tn] = Frag<float>::zero(); }
+    bool mok[2];
+    mok[0] = m0 + r16 < a.X;
+    mok[1] = m0 + 16 + r16 < a.X;
+
+    const int p1 = a.seg_ptr[seg + 1];
+    for (int p = a.seg_ptr[seg]; p < p1; ++p) {
+        const T* blkp = spz + (long)a.seg_blk[p] * (BLK * BLK);
+        const long kcol0 = (long)a.seg_inner[p] * BLK;
+#pragma unroll
+        for (int kk = 0; kk < BLK; kk += 16) {
+            typename Frag<T>::type fs[NTL], fd[2];
+#pragma unroll
+            for (int tn = 0; tn < NTL; ++tn) {
+                const int n = subn * TILE + 16 * tn + r16;
+                fs[tn] = a.trans ? Frag<T>::load(blkp + n * BLK + kk + 4 * g)
+                                 : Frag<T>::gather(blkp + (kk + 4 * g) * BLK + n, BLK);
+            }
+#pragma unroll
+            for (int tm = 0; tm < 2; ++tm) {
+                fd[tm] = Frag<T>::zero();
+                if (mok[tm])
+                    fd[tm] = frag_at<T>(dnp + (m0 + 16 * tm + r16) * a.dn_s0 + (kcol0 + kk + 4 * g) * a.dn_s1, a.dn_s1);
+            }
+#pragma unroll
+            for (int tn = 0; tn < NTL; ++tn) {
+                acc[0][tn] = Frag<T>::mma(fs[tn], fd[0], acc[0][tn]);
+                acc[1][tn] = Frag<T>::mma(fs[tn], fd[1], acc[1][tn]);
+            }
+        }
+    }
+    // lane holds C[m = m0 + 16tm + r16][n = 16tn + 4g + i]
+    T* cp = reinterpret_cast<T*>(a.c) + z * a.c_sz + head * a.c_sh;
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm) {
+        if (!mok[tm]) continue;
+        const long m = m0 + 16 * tm + r16;
+#pragma unroll
+        for (int tn = 0; tn < NTL; ++tn) {
+            const long n = (long)bcol * BLK + subn * TILE + 16 * tn + 4 * g;
+            store_tile_row<T>(cp + m * a.c_sm + n * a.c_sn, a.c_sn, acc[tm][tn], 4);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// row operations: one wave per row of a block-row
+// ---------------------------------------------------------------------------------------
+struct RowArgs {
+    void* x; void* out;
+    const int32_t* row_ptr; const int32_t* row_blk; const int32_t* row_col;
+    int n_brow, brows_per_head, blk_shift;
+    long x_sz;
+    float scale;
+    const float* kpm; long kpm_stride; int kpm_mul;
+    const float* am; long am_stride; int am_mul;
+    int op;
+};
+
+__device__ __forceinline__ float mask_term(float v, int mul) {
+    if (!mul) return v;
+    return v == 0.f ? -INFINITY : 0.f;
+}
+
+// value of element e (0 <= e < nb*blk) of the row, with scale and masks applied
+template <typename T>
+__device__ __forceinline__ float row_value(const RowArgs& a, const T* xz, int p0, int rl, int e, int z, int grow,
+                                           long* addr) {
+    const int BLK = 1 << a.blk_shift;
+    const int bidx = e >> a.blk_shift, cl = e & (BLK - 1);
+    const long off = (long)a.row_blk[p0 + bidx] * (BLK * BLK) + rl * BLK + cl;
+    *addr = off;
+    float v = Elem<T>::to_f32(xz[off]) * a.scale;
+    if (a.kpm || a.am) {
+        const long col = (long)a.row_col[p0 + bidx] * BLK + cl;
+        if (a.kpm) v += mask_term(a.kpm[z * a.kpm_stride + col], a.kpm_mul);
+        if (a.am) v += mask_term(a.am[grow * a.am_stride + col], a.am_mul);
+    }
+    return v;
+}
+
+template <typename T, int NREG>
+__global__ __launch_bounds__(256) void bs_softmax_kernel(RowArgs a) {
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int BLK = 1 << a.blk_shift;
+    const long R = (long)blockIdx.x * 4 + w;
+    if (R >= (long)a.n_brow * BLK) return;
+    const int brow = (int)(R >> a.blk_shift), rl = (int)(R & (BLK - 1));
+    const int z = blockIdx.y;
+    const int p0 = a.row_ptr[brow], nb = a.row_ptr[brow + 1] - p0;
+    const int n = nb << a.blk_shift;
+    const int grow = (brow % a.brows_per_head) * BLK + rl;
+    T* xz = reinterpret_cast<T*>(a.x) + z * a.x_sz;
+
+    float vals[NREG];
+    long addr[NREG];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int it = 0; it < NREG; ++it) {
+        const int e = lane + 64 * it;
+        vals[it] = -INFINITY;
+        addr[it] = 0;
+        if (e < n) vals[it] = row_value<T>(a, xz, p0, rl, e, z, grow, &addr[it]);
+        mx = fmaxf(mx, vals[it]);
+    }
+    mx = wave_max(mx);
+    float sum = 0.f;
+#pragma unroll
+    for (int it = 0; it < NREG; ++it) {
+        const int e = lane + 64 * it;
+        if (e < n) { vals[it] = expf(vals[it] - mx); sum += vals[it]; }   // -inf - -inf = NaN, kept on purpose
+    }
+    sum = wave_sum(sum);
+    const float inv = 1.0f / sum;
+#pragma unroll
+    for (int it = 0; it < NREG; ++it) {
+        const int e = lane + 64 * it;
+        if (e < n) xz[addr[it]] = Elem<T>::from_f32(vals[it] * inv);
+    }
+}
+
+// rows longer than the register budget: three passes over the row
+template <typename T>
+__global__ __launch_bounds__(256) void bs_softmax_long_kernel(RowArgs a) {
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int BLK = 1 << a.blk_shift;
+    const long R = (long)blockIdx.x * 4 + w;
+    if (R >= (long)a.n_brow * BLK) return;
+    const int brow = (int)(R >> a.blk_shift), rl = (int)(R & (BLK - 1));
+    const int z = blockIdx.y;
+    const int p0 = a.row_ptr[brow], nb = a.row_ptr[brow + 1] - p0;
+    const int n = nb << a.blk_shift;
+    const int grow = (brow % a.brows_per_head) * BLK + rl;
+    T* xz = reinterpret_cast<T*>(a.x) + z * a.x_sz;
+    long addr;
+    float mx = -INFINITY;
+    for (int e = lane; e < n; e += 64) mx = fmaxf(mx, row_value<T>(a, xz, p0, rl, e, z, grow, &addr));
+    mx = wave_max(mx);
+    float sum = 0.f;
+    for (int e = lane; e < n; e += 64) sum += expf(row_value<T>(a, xz, p0, rl, e, z, grow, &addr) - mx);
+    sum = wave_sum(sum);
+    const float inv = 1.0f / sum;
+    for (int e = lane; e < n; e += 64) {
+        const float v = expf(row_value<T>(a, xz, p0, rl, e, z, grow, &addr) - mx) * inv;
+        xz[addr] = Elem<T>::from_f32(v);
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void bs_rowreduce_kernel(RowArgs a) {
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int BLK = 1 << a.blk_shift;
+    const long R = (long)blockIdx.x * 4 + w;
+    if (R >= (long)a.n_brow * BLK) return;
+    const int brow = (int)(R >> a.blk_shift), rl = (int)(R & (BLK - 1));
+    const int z = blockIdx.y;
+    const int p0 = a.row_ptr[brow], nb = a.row_ptr[brow + 1] - p0;
+    const int n = nb << a.blk_shift;
+    const T* xz = reinterpret_cast<const T*>(a.x) + z * a.x_sz;
+    T* out = reinterpret_cast<T*>(a.out) + (long)z * a.n_brow * BLK + R;
+    float res = 0.f;
+    if (n > 0) {
+        if (a.op == 1) {
+            float s = 0.f;
+            for (int e = lane; e < n; e += 64)
+                s += Elem<T>::to_f32(xz[(long)a.row_blk[p0 + (e >> a.blk_shift)] * (BLK * BLK) + rl * BLK + (e & (BLK - 1))]);
+            res = wave_sum(s);
+        } else {
+            float mx = -INFINITY;
+            for (int e = lane; e < n; e += 64)
+                mx = fmaxf(mx, Elem<T>::to_f32(xz[(long)a.row_blk[p0 + (e >> a.blk_shift)] * (BLK * BLK) + rl * BLK + (e & (BLK - 1))]));
+            mx = wave_max(mx);
+            float s = 0.f;
+            for (int e = lane; e < n; e += 64)
+                s += expf(Elem<T>::to_f32(xz[(long)a.row_blk[p0 + (e >> a.blk_shift)] * (BLK * BLK) + rl * BLK + (e & (BLK - 1))]) - mx);
+            s = wave_sum(s);
+            res = (mx == -INFINITY) ? -INFINITY : mx + logf(s);
+        }
+    }
+    if (lane == 0) *out = Elem<T>::from_f32(res);
+}
+
+// ---------------------------------------------------------------------------------------
+// host side dispatch
+// ---------------------------------------------------------------------------------------
+static int blk_shift_of(int blk) {
+    switch (blk) { case 16: return 4; case 32: return 5; case 64: return 6; case 128: return 7; default: return -1; }
+}
+
+#define BS_DISPATCH_BLK(KERN, T, GRID, ARGS)                                               \
+    switch (blk) {                                                                         \
+        case 16: hipLaunchKernelGGL((KERN<T, 16>), GRID, dim3(256), 0, st, ARGS); break;   \
+        case 32: hipLaunchKernelGGL((KERN<T, 32>), GRID, dim3(256), 0, st, ARGS); break;   \
+        case 64: hipLaunchKernelGGL((KERN<T, 64>), GRID, dim3(256), 0, st, ARGS); break;   \
+        case 128: hipLaunchKernelGGL((KERN<T, 128>), GRID, dim3(256), 0, st, ARGS); break; \
+    }
+#define BS_DISPATCH(KERN, GRID, ARGS)                                                      \
+    switch (dtype) {                                                                       \
+        case F32: BS_DISPATCH_BLK(KERN, float, GRID, ARGS) break;                          \
+        case BF16: BS_DISPATCH_BLK(KERN, bf16_t, GRID, ARGS) break;                        \
+        case F16: BS_DISPATCH_BLK(KERN, f16_t, GRID, ARGS) break;                          \
+    }
+
+static long waves_to_blocks(long waves) { return (waves + 3) / 4; }
+
+}  // namespace flyhip
+
+using namespace flyhip;
+
+static int check_common(const char* who, int blk, int dtype, int Z) {
+    FLY_REQUIRE(blk_shift_of(blk) >= 0, "%s: block size %d not in {16,32,64,128}", who, blk);
+    FLY_REQUIRE(dtype == F32 || dtype == BF16 || dtype == F16, "%s: unknown dtype code %d", who, dtype);
+    FLY_REQUIRE(Z >= 1 && Z <= 65535, "%s: batch %d outside [1, 65535]", who, Z);
+    return OK;
+}
+
+extern "C" int flyhip_bs_sdd(const void* a, const void* b, void* c, const int32_t* lut, int nnz,
+                             int Z, int K, int blk,
+                             int64_t a_sz, int64_t a_sh, int64_t a_sm, int64_t a_sk,
+                             int64_t b_sz, int64_t b_sh, int64_t b_sn, int64_t b_sk,
+                             int dtype, void* stream) {
+    int rc = check_common("bs_sdd", blk, dtype, Z);
+    if (rc) return rc;
+    FLY_REQUIRE(a && b && c && lut, "bs_sdd: null pointer");
+    FLY_REQUIRE(nnz >= 0, "bs_sdd: negative nnz");
+    FLY_REQUIRE(K > 0 && K % 16 == 0, "bs_sdd: reduction size %d must be a positive multiple of 16", K);
+    if (a_sk == 1) FLY_REQUIRE(((a_sz | a_sh | a_sm) % 4) == 0, "bs_sdd: A strides must be multiples of 4 elements");
+    if (b_sk == 1) FLY_REQUIRE(((b_sz | b_sh | b_sn) % 4) == 0, "bs_sdd: B strides must be multiples of 4 elements");
+    if (nnz == 0) return OK;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    SddArgs args{a, b, c, lut, nnz, K, a_sz, a_sh, a_sm, a_sk, b_sz, b_sh, b_sn, b_sk};
+    const int tile = blk >= 32 ? 32 : 16, sub = blk / tile;
+    const long nblocks = waves_to_blocks((long)nnz * sub * sub);
+    FLY_REQUIRE(nblocks <= 2147483647L, "bs_sdd: too many blocks");
+    dim3 grid((unsigned)nblocks, Z);
+    BS_DISPATCH(bs_sdd_kernel, grid, args)
+    return check_launch("bs_sdd_kernel");
+}
+
+extern "C" int flyhip_bs_dsd(const void* a_sp, const void* b, void* c,
+                             const int32_t* seg_ptr, const int32_t* seg_blk, const int32_t* seg_inner,
+                             int n_seg, int rows_per_head, int Z, int N, int blk, int trans_a,
+                             int64_t a_sz,
+                             int64_t b_sz, int64_t b_sh, int64_t b_sk, int64_t b_sn,
+                             int64_t c_sz, int64_t c_sh, int64_t c_sm, int64_t c_sn,
+                             int dtype, void* stream) {
+    int rc = check_common("bs_dsd", blk, dtype, Z);
+    if (rc) return rc;
+    FLY_REQUIRE(a_sp && b && c && seg_ptr && seg_blk && seg_inner, "bs_dsd: null pointer");
+    FLY_REQUIRE(n_seg > 0 && rows_per_head > 0 && n_seg % rows_per_head == 0, "bs_dsd: bad segment counts");
+    FLY_REQUIRE(N > 0, "bs_dsd: N must be positive");
+    if (b_sk == 1) FLY_REQUIRE(((b_sz | b_sh | b_sn) % 4) == 0, "bs_dsd: B strides must be multiples of 4 elements");
+    if (c_sn == 1) FLY_REQUIRE(((c_sz | c_sh | c_sm) % 4) == 0, "bs_dsd: C strides must be multiples of 4 elements");
+    FLY_REQUIRE(a_sz % 4 == 0, "bs_dsd: sparse batch stride must be a multiple of 4 elements");
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    DxdArgs args{a_sp, b, c, seg_ptr, seg_blk, seg_inner, n_seg, rows_per_head, N, trans_a,
+                 a_sz, b_sz, b_sh, b_sk, b_sn, c_sz, c_sh, c_sm, c_sn};
+    const int tile = blk >= 32 ? 32 : 16;
+    const long nblocks = waves_to_blocks((long)n_seg * (blk / tile) * ((N + 31) / 32));
+    FLY_REQUIRE(nblocks <= 2147483647L, "bs_dsd: too many blocks");
+    dim3 grid((unsigned)nblocks, Z);
+    BS_DISPATCH(bs_dsd_kernel, grid, args)
+    return check_launch("bs_dsd_kernel");
+}
+
+extern "C" int flyhip_bs_dds(const void* a, const void* b_sp, void* c,
+                             const int32_t* seg_ptr, const int32_t* seg_blk, const int32_t* seg_inner,
+                             int n_seg, int cols_per_head, int Z, int M, int blk, int trans_b,
+                             int64_t a_sz, int64_t a_sh, int64_t a_sm, int64_t a_sk,
+                             int64_t b_sz,
+                             int64_t c_sz, int64_t c_sh, int64_t c_sm, int64_t c_sn,
+                             int dtype, void* stream) {
+    int rc = check_common("bs_dds", blk, dtype, Z);
+    if (rc) return rc;
+    FLY_REQUIRE(a && b_sp && c && seg_ptr && seg_blk && seg_inner, "bs_dds: null pointer");
+    FLY_REQUIRE(n_seg > 0 && cols_per_head > 0 && n_seg % cols_per_head == 0, "bs_dds: bad segment counts");
+    FLY_REQUIRE(M > 0, "bs_dds: M must be positive");
+    if (a_sk == 1) FLY_REQUIRE(((a_sz | a_sh | a_sm) % 4) == 0, "bs_dds: A strides must be multiples of 4 elements");
+    if (c_sn == 1) FLY_REQUIRE(((c_sz | c_sh | c_sm) % 4) == 0, "bs_dds: C strides must be multiples of 4 elements");
+    FLY_REQUIRE(b_sz % 4 == 0, "bs_dds: sparse batch stride must be a multiple of 4 elements");
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    DxdArgs args{b_sp, a, c, seg_ptr, seg_blk, seg_inner, n_seg, cols_per_head, M, trans_b,
+                 b_sz, a_sz, a_sh, a_sm, a_sk, c_sz, c_sh, c_sm, c_sn};
+    const int tile = blk >= 32 ? 32 : 16;
+    const long nblocks = waves_to_blocks((long)((M + 31) / 32) * n_seg * (blk / tile));
+    FLY_REQUIRE(nblocks <= 2147483647L, "bs_dds: too many blocks");
+    dim3 grid((unsigned)nblocks, Z);
+    BS_DISPATCH(bs_dds_kernel, grid, args)
+    return check_launch("bs_dds_kernel");
+}
+
+template <typename T>
+static int launch_softmax(const RowArgs& args, dim3 grid, int max_elems, hipStream_t st) {
+    if (max_elems <= 64 * 8) hipLaunchKernelGGL((bs_softmax_kernel<T, 8>), grid, dim3(256), 0, st, args);
+    else if (max_elems <= 64 * 32) hipLaunchKernelGGL((bs_softmax_kernel<T, 32>), grid, dim3(256), 0, st, args);
+    else hipLaunchKernelGGL((bs_softmax_long_kernel<T>), grid, dim3(256), 0, st, args);
+    return check_launch("bs_softmax_kernel");
+}
+
+extern "C" int flyhip_bs_softmax(void* x, const int32_t* row_ptr, const int32_t* row_blk, const int32_t* row_col,
+                                 int n_brow, int brows_per_head, int max_row_nnz, int Z, int blk, int64_t x_sz,
+                                 float scale, const float* kpm, int64_t kpm_stride, int kpm_mul,
+                                 const float* am, int64_t am_stride, int am_mul, int dtype, void* stream) {
+    int rc = check_common("bs_softmax", blk, dtype, Z);
+    if (rc) return rc;
+    FLY_REQUIRE(x && row_ptr && row_blk && row_col, "bs_softmax: null pointer");
+    FLY_REQUIRE(n_brow > 0 && brows_per_head > 0 && n_brow % brows_per_head == 0, "bs_softmax: bad row counts");
+    FLY_REQUIRE(max_row_nnz >= 0, "bs_softmax: negative max_row_nnz");
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    RowArgs args{x, nullptr, row_ptr, row_blk, row_col, n_brow, brows_per_head, blk_shift_of(blk), x_sz, scale,
+                 kpm, kpm_stride, kpm_mul, am, am_stride, am_mul, 0};
+    const long nblocks = waves_to_blocks((long)n_brow * blk);
+    dim3 grid((unsigned)nblocks, Z);
+    const int max_elems = max_row_nnz * blk;   // selects the register-resident or the multi-pass kernel
+    switch (dtype) {
+        case F32: return launch_softmax<float>(args, grid, max_elems, st);
+        case BF16: return launch_softmax<bf16_t>(args, grid, max_elems, st);
+        default: return launch_softmax<f16_t>(args, grid, max_elems, st);
+    }
+}
+
+extern "C" int flyhip_bs_rowreduce(const void* x, void* out, const int32_t* row_ptr, const int32_t* row_blk,
+                                   int n_brow, int Z, int blk, int64_t x_sz, int op, int dtype, void* stream) {
+    int rc = check_common("bs_rowreduce", blk, dtype, Z);
+    if (rc) return rc;
+    FLY_REQUIRE(x && out && row_ptr && row_blk, "bs_rowreduce: null pointer");
+    FLY_REQUIRE(op == 0 || op == 1, "bs_rowreduce: op must be 0 (logsumexp) or 1 (sum)");
+    FLY_REQUIRE(n_brow > 0, "bs_rowreduce: no rows");
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    RowArgs args{const_cast<void*>(x), out, row_ptr, row_blk, nullptr, n_brow, 1, blk_shift_of(blk), x_sz, 1.f,
+                 nullptr, 0, 0, nullptr, 0, 0, op};
+    dim3 grid((unsigned)waves_to_blocks((long)n_brow * blk), Z);
+    switch (dtype) {
+        case F32: hipLaunchKernelGGL((bs_rowreduce_kernel<float>), grid, dim3(256), 0, st, args); break;
+        case BF16: hipLaunchKernelGGL((bs_rowreduce_kernel<bf16_t>), grid, dim3(256), 0, st, args); break;
+        default: hipLaunchKernelGGL((bs_rowreduce_kernel<f16_t>), grid, dim3(256), 0, st, args); break;
+    }
+    return check_launch("bs_rowreduce_kernel");
+}

@@ -1,0 +1,154 @@
+// Shared device/host helpers for the gfx950 kernels: error reporting for the C ABI,
+// element-type traits, 16-byte operand loads and the 16x16 MFMA wrappers.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+namespace flyhip {
+
+// ---------------------------------------------------------------------------------------
+// error convention: entry points return 0 or a negative code and leave a message here
+// ---------------------------------------------------------------------------------------
+enum { OK = 0, ERR_ARG = -1, ERR_UNSUPPORTED = -2, ERR_LAUNCH = -3 };
+char* error_buffer();   // thread-local, 512 bytes
+inline int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(error_buffer(), 512, fmt, ap);
+    va_end(ap);
+    return code;
+}
+inline int check_launch(const char* what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+    return OK;
+}
+#define FLY_REQUIRE(cond, ...) do { if (!(cond)) return ::flyhip::fail(::flyhip::ERR_ARG, __VA_ARGS__); } while (0)
+
+enum DType { F32 = 0, BF16 = 1, F16 = 2 };
+
+// ---------------------------------------------------------------------------------------
+// element types
+// ---------------------------------------------------------------------------------------
+struct bf16_t { uint16_t bits; };
+struct f16_t { _Float16 v; };
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef short shortx4 __attribute__((ext_vector_type(4)));
+typedef _Float16 halfx4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float bf16_to_f32(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {   // round to nearest even, NaN kept quiet
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+template <typename T> struct Elem;
+template <> struct Elem<float> {
+    static __device__ __forceinline__ float to_f32(float x) { return x; }
+    static __device__ __forceinline__ float from_f32(float x) { return x; }
+};
+template <> struct Elem<bf16_t> {
+    static __device__ __forceinline__ float to_f32(bf16_t x) { return bf16_to_f32(x.bits); }
+    static __device__ __forceinline__ bf16_t from_f32(float x) { bf16_t r; r.bits = f32_to_bf16(x); return r; }
+};
+template <> struct Elem<f16_t> {
+    static __device__ __forceinline__ float to_f32(f16_t x) { return (float)x.v; }
+    static __device__ __forceinline__ f16_t from_f32(float x) { f16_t r; r.v = (_Float16)x; return r; }
+};
+
+// four consecutive elements -> fp32 (pointer must be aligned to 4 elements)
+__device__ __forceinline__ floatx4 load4_f32(const float* p) { return *reinterpret_cast<const floatx4*>(p); }
+__device__ __forceinline__ floatx4 load4_f32(const bf16_t* p) {
+    uint2 u = *reinterpret_cast<const uint2*>(p);
+    floatx4 r;
+    r[0] = __uint_as_float(u.x << 16); r[1] = __uint_as_float(u.x & 0xffff0000u);
+    r[2] = __uint_as_float(u.y << 16); r[3] = __uint_as_float(u.y & 0xffff0000u);
+    return r;
+}
+__device__ __forceinline__ floatx4 load4_f32(const f16_t* p) {
+    halfx4 h = *reinterpret_cast<const halfx4*>(p);
+    floatx4 r = {(float)h[0], (float)h[1], (float)h[2], (float)h[3]};
+    return r;
+}
+__device__ __forceinline__ void store4_f32(float* p, floatx4 v) { *reinterpret_cast<floatx4*>(p) = v; }
+__device__ __forceinline__ void store4_f32(bf16_t* p, floatx4 v) {
+    uint2 u;
+    u.x = (uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16);
+    u.y = (uint32_t)f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16);
+    *reinterpret_cast<uint2*>(p) = u;
+}
+__device__ __forceinline__ void store4_f32(f16_t* p, floatx4 v) {
+    halfx4 h = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
+    *reinterpret_cast<halfx4*>(p) = h;
+}
+
+// ---------------------------------------------------------------------------------------
+// 16x16 MFMA "k16" step.  A fragment holds, for lane (r = lane%16, g = lane/16), the four
+// operand elements k = 4g..4g+3 of row r (A side) or column r (B side) of a 16-wide slice of
+// the contraction.  acc holds C[4g+i][r] for i = 0..3.
+// ---------------------------------------------------------------------------------------
+template <typename T> struct Frag;
+template <> struct Frag<float> {
+    typedef floatx4 type;
+    static __device__ __forceinline__ type zero() { type z = {0.f, 0.f, 0.f, 0.f}; return z; }
+    static __device__ __forceinline__ type load(const float* p) { return *reinterpret_cast<const type*>(p); }
+    static __device__ __forceinline__ type gather(const float* p, long s) {
+        type r = {p[0], p[s], p[2 * s], p[3 * s]}; return r;
+    }
+    static __device__ __forceinline__ floatx4 mma(type a, type b, floatx4 c) {
+        c = __builtin_amdgcn_mfma_f32_16x16x4f32(a[0], b[0], c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_16x16x4f32(a[1], b[1], c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_16x16x4f32(a[2], b[2], c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_16x16x4f32(a[3], b[3], c, 0, 0, 0);
+        return c;
+    }
+};
+template <> struct Frag<bf16_t> {
+    typedef shortx4 type;
+    static __device__ __forceinline__ type zero() { type z = {0, 0, 0, 0}; return z; }
+    static __device__ __forceinline__ type load(const bf16_t* p) { return *reinterpret_cast<const type*>(p); }
+    static __device__ __forceinline__ type gather(const bf16_t* p, long s) {
+        type r = {(short)p[0].bits, (short)p[s].bits, (short)p[2 * s].bits, (short)p[3 * s].bits}; return r;
+    }
+    static __device__ __forceinline__ floatx4 mma(type a, type b, floatx4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, b, c, 0, 0, 0);
+    }
+};
+template <> struct Frag<f16_t> {
+    typedef halfx4 type;
+    static __device__ __forceinline__ type zero() { type z = {0, 0, 0, 0}; return z; }
+    static __device__ __forceinline__ type load(const f16_t* p) { return *reinterpret_cast<const type*>(p); }
+    static __device__ __forceinline__ type gather(const f16_t* p, long s) {
+        type r = {p[0].v, p[s].v, p[2 * s].v, p[3 * s].v}; return r;
+    }
+    static __device__ __forceinline__ floatx4 mma(type a, type b, floatx4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x16f16(a, b, c, 0, 0, 0);
+    }
+};
+
+// wave-level butterflies across the four 16-lane groups (lanes r, r+16, r+32, r+48)
+__device__ __forceinline__ float group_max(float v) {
+    v = fmaxf(v, __shfl_xor(v, 16));
+    v = fmaxf(v, __shfl_xor(v, 32));
+    return v;
+}
+__device__ __forceinline__ float group_sum(float v) {
+    v += __shfl_xor(v, 16);
+    v += __shfl_xor(v, 32);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+
+}  // namespace flyhip

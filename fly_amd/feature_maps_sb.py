@@ -1,0 +1,79 @@
+"""Performer random features for Scatterbrain attention: the projection matrix and the module
+that owns it (src/models/attention/projection_utils.py:8-28, feature_maps_sb.py:85-156).
+
+The feature values themselves (feature_maps_sb.py:51-82) are never materialised by this
+package for the queries and only as a kernel-internal workspace for the keys: they are computed
+inside the HIP kernels behind ``SBLocalAttention``.
+"""
+import math
+
+import torch
+import torch.nn as nn
+
+
+def gaussian_orthogonal_random_matrix(nrows, ncols, scaling=0, device=None, dtype=None):
+    """(nrows, ncols) matrix whose ncols-row blocks are Haar-orthogonal, with rows rescaled to
+    chi-distributed norms (scaling=0) or to sqrt(ncols) (scaling=1) -- projection_utils.py:8-28.
+    Unlike the reference, which draws the row norms on the target device (:23), every random
+    number comes from the CPU generator so that a seed gives the same matrix on any machine."""
+    nblocks = int(math.ceil(nrows / ncols))
+    gauss = torch.randn((nblocks, ncols, ncols), device='cpu')
+    q, r = torch.linalg.qr(gauss)
+    q = q * torch.sign(torch.diagonal(r, dim1=-2, dim2=-1)).unsqueeze(-2)
+    rows = q.transpose(-1, -2).reshape(nblocks * ncols, ncols)[:nrows]
+    if scaling == 0:
+        norms = torch.randn((nrows, ncols), device='cpu').norm(dim=1)
+        rows = norms.unsqueeze(-1) * rows
+    elif scaling == 1:
+        rows = math.sqrt(ncols) * rows
+    else:
+        raise ValueError(f'Invalid scaling {scaling}')
+    return rows.to(device=device, dtype=dtype)
+
+
+class SBPerformerFeatures(nn.Module):
+    """Holder of the random projection (feature_maps_sb.py:85-156).
+
+    ``n_features`` defaults to int(E ln E); the cosh feature map uses n_features // 2 projection
+    rows and produces 2 * (n_features // 2) features.  ``new_feature_map`` draws the matrix on the
+    first call only (the reference sets ``redraw = pi`` so that ``calls % redraw == 0`` just once,
+    :119,135-137).  The buffer ``projection_matrix`` has shape (n_features // 2, query_dims); a
+    matrix loaded from a state dict or assigned by the caller is used as is when
+    ``freeze_projection()`` has been called.
+    """
+
+    def __init__(self, query_dims, n_features=None, ortho_scaling=0, softmax_temp=None,
+                 orthogonal=False, cosh=True, redraw=1, deterministic_eval=False, eps=0.0,
+                 device=None, dtype=None):
+        super().__init__()
+        if not cosh:
+            raise NotImplementedError('only the cosh (two-sided) feature map is implemented')
+        self.query_dims = query_dims
+        self.n_features = n_features or int(query_dims * math.log(query_dims))
+        self.ortho_scaling = ortho_scaling
+        self.orthogonal = orthogonal
+        self.softmax_temp = 1 / math.sqrt(query_dims) if softmax_temp is None else softmax_temp
+        self.cosh = cosh
+        self.redraw = math.pi
+        self.deterministic_eval = deterministic_eval
+        self.eps = eps
+        self.factory_kwargs = {'device': device, 'dtype': dtype}
+        self.register_buffer('projection_matrix',
+                             torch.zeros(self.n_features // 2, query_dims, **self.factory_kwargs))
+        self._calls = -1
+
+    def freeze_projection(self):
+        """Keep the current ``projection_matrix`` (e.g. one loaded from a checkpoint or set by a
+        test) instead of drawing a new one on the first forward."""
+        self._calls = 0
+
+    def new_feature_map(self, device):
+        if self.deterministic_eval and not self.training:
+            return
+        self._calls += 1
+        if (self._calls % self.redraw) != 0:
+            return
+        matrix = gaussian_orthogonal_random_matrix(self.n_features // 2, self.query_dims,
+                                                   scaling=self.ortho_scaling, device=device,
+                                                   dtype=self.factory_kwargs['dtype'])
+        self.register_buffer('projection_matrix', matrix)

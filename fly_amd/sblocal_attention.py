@@ -1,0 +1,153 @@
+"""Scatterbrain-local attention on the HIP kernels: drop-in for
+src/models/attention/sblocal_attention.py (class SBLocalAttention, :15-137)."""
+import ctypes
+import math
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import _lib
+from .feature_maps_sb import SBPerformerFeatures
+
+_HEAD_DIMS = (32, 64, 128)       # padded head dims the kernels are instantiated for
+_FEATURE_ROWS = (16, 32, 64, 128)  # padded projection rows (m/2)
+
+
+def _round_up_choice(n, choices, what):
+    for c in choices:
+        if n <= c:
+            return c
+    raise NotImplementedError(f'{what}={n} exceeds the largest supported size {choices[-1]}')
+
+
+def _vector_ready(x):
+    """16-byte vector access needs a unit inner stride, strides in multiples of 4 elements and an
+    aligned base pointer."""
+    return (x.stride(-1) == 1 and all(s % 4 == 0 for s in x.stride()[:-1])
+            and x.data_ptr() % 16 == 0)
+
+
+def sblocal_forward(query, key, value, projection_matrix, local_context, softmax_temp=None,
+                    key_lengths=None):
+    """Scatterbrain-local attention forward on the GPU.
+
+    query (B,T,H,E), key (B,S,H,E), value (B,S,H,D) float32 or bfloat16 CUDA tensors;
+    projection_matrix (m/2, E); key_lengths (B,) int64 or None.  Computes what
+    sblocal_attention.py:73-122 computes for causal=False, attn_mask=None, eps=0, no dropout.
+    Returns (out (B,T,H,D) in the input dtype, log_normalization (B,H,T,1) float32).
+    """
+    _lib.require_gpu(query, key, value, projection_matrix, key_lengths)
+    if query.dtype not in (torch.float32, torch.bfloat16):
+        raise NotImplementedError(f'SBLocal kernels support float32 and bfloat16, got {query.dtype}')
+    if key.dtype != query.dtype or value.dtype != query.dtype:
+        raise ValueError('query, key and value must share a dtype')
+    B, T, H, E = query.shape
+    Bk, S, Hk, Ek = key.shape
+    Bv, Sv, Hv, D = value.shape
+    if (Bk, Hk, Ek) != (B, H, E) or (Bv, Sv, Hv) != (B, S, H):
+        raise ValueError(f'inconsistent shapes q{tuple(query.shape)} k{tuple(key.shape)} v{tuple(value.shape)}')
+    if projection_matrix.dim() != 2 or projection_matrix.shape[1] != E:
+        raise ValueError(f'projection_matrix must be (m/2, {E}), got {tuple(projection_matrix.shape)}')
+    if local_context < 1:
+        raise ValueError('local_context must be >= 1')
+    t = softmax_temp or 1 / math.sqrt(E)          # sblocal_attention.py:59: 0 / None mean "unset"
+
+    dim = _round_up_choice(max(E, D), _HEAD_DIMS, 'head dimension')
+    mh_valid = projection_matrix.shape[0]
+    mh = _round_up_choice(mh_valid, _FEATURE_ROWS, 'number of projection rows')
+    m = 2 * mh
+
+    def prep(x):
+        if x.shape[-1] != dim:
+            x = F.pad(x, (0, dim - x.shape[-1]))      # zero columns change neither dots nor norms
+        return x if _vector_ready(x) else x.contiguous()
+    q, k, v = prep(query), prep(key), prep(value)
+    proj = torch.zeros(mh, dim, dtype=torch.float32, device=query.device)
+    proj[:mh_valid, :E] = projection_matrix.to(torch.float32)
+    lens = None
+    if key_lengths is not None:
+        lens = key_lengths.to(device=query.device, dtype=torch.int64).contiguous()
+        if lens.shape != (B,):
+            raise ValueError(f'key_lengths must have shape ({B},)')
+
+    n_chunks, n_split = ctypes.c_int(), ctypes.c_int()
+    _lib.call('flyhip_sb_plan', B, H, S, ctypes.byref(n_chunks), ctypes.byref(n_split))
+    n_chunks, n_split = n_chunks.value, n_split.value
+    dev, f32 = query.device, torch.float32
+    kfeat = torch.empty(B, H, n_chunks * 64, m, dtype=f32, device=dev)
+    chunk_scale = torch.empty(B, H, n_chunks, dtype=f32, device=dev)
+    kv_part = torch.empty(B, H, n_split, m * (dim + 1), dtype=f32, device=dev)
+    part_max = torch.empty(B, H, n_split, dtype=f32, device=dev)
+    kv = torch.empty(B, H, m, dim, dtype=f32, device=dev)
+    ksum = torch.empty(B, H, m, dtype=f32, device=dev)
+    kmax = torch.empty(B, H, dtype=f32, device=dev)
+    out = torch.empty(B, T, H, dim, dtype=query.dtype, device=dev)
+    log_norm = torch.empty(B, H, T, dtype=f32, device=dev)
+
+    code = _lib.dtype_code(query)
+    stream = _lib.stream_ptr(dev)
+    with torch.cuda.device(dev):
+        _lib.call('flyhip_sb_kv_reduce', k.data_ptr(), v.data_ptr(), proj.data_ptr(), _lib.ptr(lens),
+                  kfeat.data_ptr(), chunk_scale.data_ptr(), kv_part.data_ptr(), part_max.data_ptr(),
+                  kv.data_ptr(), ksum.data_ptr(), kmax.data_ptr(),
+                  B, H, S, dim, dim, mh, mh_valid, n_split,
+                  k.stride(0), k.stride(2), k.stride(1), v.stride(0), v.stride(2), v.stride(1),
+                  t, code, stream)
+        _lib.call('flyhip_sblocal_fwd', q.data_ptr(), k.data_ptr(), v.data_ptr(), proj.data_ptr(),
+                  kfeat.data_ptr(), chunk_scale.data_ptr(), kv.data_ptr(), ksum.data_ptr(), kmax.data_ptr(),
+                  _lib.ptr(lens), out.data_ptr(), log_norm.data_ptr(),
+                  B, H, T, S, dim, dim, mh, mh_valid, local_context,
+                  q.stride(0), q.stride(2), q.stride(1), k.stride(0), k.stride(2), k.stride(1),
+                  v.stride(0), v.stride(2), v.stride(1), out.stride(0), out.stride(2), out.stride(1),
+                  t, code, stream)
+    return out[..., :D], log_norm.unsqueeze(-1)
+
+
+class SBLocalAttention(nn.Module):
+    """Local (banded) softmax attention plus a Performer low-rank estimate of everything outside
+    the band, under one normaliser.  Query i attends exactly to keys j with
+    -(local_context // 2) <= j - i < (local_context + 1) // 2 and through random features to the rest.
+
+    Same constructor and forward signature as the reference class (sblocal_attention.py:29-44).
+    The GPU path covers what the reference itself exercises: non-causal, no attn_mask, optional
+    length-style key_padding_mask, softmax_eps = 0, dropout inactive, need_weights=False.  Any other
+    request raises NotImplementedError -- there is no slower fallback inside this module.
+    """
+
+    def __init__(self, local_context, dim_heads, nb_features=None, ortho_scaling=0,
+                 causal=False, softmax_temp=None, attention_dropout=0.0, softmax_eps=0.0,
+                 device=None, dtype=None):
+        super().__init__()
+        self.feature_map = SBPerformerFeatures(dim_heads, nb_features, ortho_scaling=ortho_scaling,
+                                               softmax_temp=softmax_temp, eps=softmax_eps,
+                                               device=device, dtype=dtype)
+        self.local_context = local_context
+        self.causal = causal
+        self.softmax_temp = softmax_temp
+        self.dropout = nn.Dropout(attention_dropout)
+        self.softmax_eps = softmax_eps
+
+    def forward(self, query, key, value, attn_mask=None, key_padding_mask=None, need_weights=False,
+                return_attn_unnormalized=False):
+        """query (B,T,H,E), key (B,S,H,E), value (B,S,H,D) -> (out (B,T,H,D), None)."""
+        if self.causal:
+            raise NotImplementedError('causal SBLocalAttention is not implemented (the reference '
+                                      'marks it unverified, sblocal_attention.py:61)')
+        if attn_mask is not None and not bool(attn_mask.all_ones):
+            raise NotImplementedError('attn_mask other than all-ones is not supported by the fused kernel')
+        if need_weights or return_attn_unnormalized:
+            raise NotImplementedError('need_weights=True would materialise the (T,S) matrix; not supported')
+        if self.softmax_eps != 0.0:
+            raise NotImplementedError('softmax_eps != 0 is not supported by the fused kernel')
+        if self.training and self.dropout.p > 0.0:
+            raise NotImplementedError('attention dropout is not implemented in the fused kernel')
+        lengths = None
+        if key_padding_mask is not None and not bool(key_padding_mask.all_ones):
+            lengths = key_padding_mask.lengths          # raises ValueError unless a length mask
+        self.feature_map.new_feature_map(query.device)
+        out, log_norm = sblocal_forward(query, key, value, self.feature_map.projection_matrix,
+                                        self.local_context, softmax_temp=self.softmax_temp,
+                                        key_lengths=lengths)
+        self.last_log_normalization = log_norm
+        return out, None

@@ -1,0 +1,139 @@
+/* flyhip -- C ABI of the MI355X (gfx950) kernels for the Scatterbrain-local attention path and
+ * the block-sparse matmul / row-op path of HazyResearch/fly.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer owned by the caller (PyTorch in the shipped host code);
+ *     the library never allocates, frees or synchronises; work is enqueued on `stream`
+ *     (a hipStream_t passed as void*, NULL = default stream);
+ *   - entry points return 0 on success and a negative code otherwise; the message is
+ *     available from flyhip_last_error() (thread-local);
+ *   - dtype: 0 = float32, 1 = bfloat16, 2 = float16 (storage type; accumulation is fp32);
+ *   - strides are in elements.
+ *
+ * "ref:" comments name the interface in the reference checkout that each entry point replaces.
+ */
+#ifndef FLYHIP_H
+#define FLYHIP_H
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { FLYHIP_F32 = 0, FLYHIP_BF16 = 1, FLYHIP_F16 = 2 };
+enum { FLYHIP_SB_CHUNK = 64 };           /* keys per feature chunk / key tile */
+
+int flyhip_version(void);
+const char* flyhip_last_error(void);
+
+/* ------------------------------------------------------------------------------------------
+ * Scatterbrain-local attention (ref: src/models/attention/sblocal_attention.py:43-137)
+ * ---------------------------------------------------------------------------------------- */
+
+/* Sizes of the caller-allocated scratch for one (B,H,S) problem: n_chunks = ceil(S/64) and the
+ * number n_split of partial K'^T V reductions per (batch, head). */
+int flyhip_sb_plan(int B, int H, int S, int* n_chunks, int* n_split);
+
+/* Key-side pass.  Replaces feature_map.forward_keys (ref: feature_maps_sb.py:51-82, key branch),
+ * the masking of padded keys (sblocal_attention.py:83-85) and the global reductions
+ * linear_attention / linear_attention_normalization (ref: scatterbrain_utils.py:18-22,48-52:
+ * K'^T V and sum_s K').
+ *   k (B,S,H,E), v (B,S,H,D) addressed through strides (batch, head, seq); innermost contiguous
+ *   proj (mh, E) fp32 row-major, rows >= mh_valid ignored (zero rows); E = D in {32,64,128},
+ *   m = 2*mh in {32,64,128,256}
+ *   key_lengths (B) int64 or NULL
+ * outputs (all fp32):
+ *   kfeat       (B,H,n_chunks*64,m)  positive random features of every key, stabilised per chunk
+ *   chunk_scale (B,H,n_chunks)       log-stabiliser each chunk of kfeat was written with
+ *   kv (B,H,m,D), ksum (B,H,m), kmax (B,H)  global reductions in units of exp(kmax)
+ * scratch: kv_part (B,H,n_split,m*(D+1)), part_max (B,H,n_split). */
+int flyhip_sb_kv_reduce(const void* k, const void* v, const float* proj, const int64_t* key_lengths,
+                        float* kfeat, float* chunk_scale, float* kv_part, float* part_max,
+                        float* kv, float* ksum, float* kmax,
+                        int B, int H, int S, int E, int D, int mh, int mh_valid, int n_split,
+                        int64_t k_sb, int64_t k_sh, int64_t k_ss,
+                        int64_t v_sb, int64_t v_sh, int64_t v_ss,
+                        float softmax_temp, int dtype, void* stream);
+
+/* Fused query-side pass.  Replaces feature_map.forward_queries, both local_dot_product calls, the
+ * joint normalisation and local_weighted_average + combine (ref: sblocal_attention.py:78,90-122;
+ * fast_transformers.local_product).  Consumes the outputs of flyhip_sb_kv_reduce.
+ *   q (B,T,H,E), out (B,T,H,D) via strides; log_norm (B,H,T) fp32 = the reference's
+ *   log_normalization; local_context = lc (band -(lc/2) <= s - i < (lc+1)/2). */
+int flyhip_sblocal_fwd(const void* q, const void* k, const void* v, const float* proj,
+                       const float* kfeat, const float* chunk_scale,
+                       const float* kv, const float* ksum, const float* kmax,
+                       const int64_t* key_lengths, void* out, float* log_norm,
+                       int B, int H, int T, int S, int E, int D, int mh, int mh_valid,
+                       int local_context,
+                       int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                       int64_t k_sb, int64_t k_sh, int64_t k_ss,
+                       int64_t v_sb, int64_t v_sh, int64_t v_ss,
+                       int64_t o_sb, int64_t o_sh, int64_t o_ss,
+                       float softmax_temp, int dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Block-sparse matmuls (ref: src/models/attention/blocksparse_matmul.py; matmul.__call__ :656,
+ * _sdd_matmul :279-346, _dds_matmul :444-488, _dsd_matmul :491-535).
+ * Sparse tensors are (Z, nnz, blk, blk); block n is the n-th nonzero of the (H, rows, cols)
+ * layout in row-major order (ref: blocksparse_utils.py:8-19).  blk in {16,32,64,128}.
+ * ---------------------------------------------------------------------------------------- */
+
+/* SDD: c[z, n] = A[z, h_n, rows of block-row i_n, :] . B[z, h_n, rows of block-col j_n, :]^T where
+ * A(m,k) / B(n,k) are addressed with (batch, head, row, k) strides (this covers trans_a/trans_b).
+ * lut: int32 (nnz,4) rows (head, block_row, block_col, block_id) (ref: make_sdd_lut :261-276). */
+int flyhip_bs_sdd(const void* a, const void* b, void* c, const int32_t* lut, int nnz,
+                  int Z, int K, int blk,
+                  int64_t a_sz, int64_t a_sh, int64_t a_sm, int64_t a_sk,
+                  int64_t b_sz, int64_t b_sh, int64_t b_sn, int64_t b_sk,
+                  int dtype, void* stream);
+
+/* DSD: c (Z,H,M,N) = op(sparse a) . dense b.  Segment s = (head, output block-row); seg_ptr
+ * (n_seg+1), seg_blk (block id), seg_inner (inner block index) int32 list the blocks reduced into
+ * it; n_seg = H * M/blk; an empty segment writes zeros (ref: make_dxx_lut :356-441 plays this
+ * role).  trans_a != 0 reads every sparse block transposed.  b(k,n) and c(m,n) via strides. */
+int flyhip_bs_dsd(const void* a_sp, const void* b, void* c,
+                  const int32_t* seg_ptr, const int32_t* seg_blk, const int32_t* seg_inner,
+                  int n_seg, int rows_per_head, int Z, int N, int blk, int trans_a,
+                  int64_t a_sz,
+                  int64_t b_sz, int64_t b_sh, int64_t b_sk, int64_t b_sn,
+                  int64_t c_sz, int64_t c_sh, int64_t c_sm, int64_t c_sn,
+                  int dtype, void* stream);
+
+/* DDS: c (Z,H,M,N) = dense a . op(sparse b).  Segment s = (head, output block-column); trans_b != 0
+ * reads every sparse block transposed (the BlockSparseLinear case, ref:
+ * src/models/layers/blocksparse_linear.py:119-120,152-162).  a(m,k) and c(m,n) via strides. */
+int flyhip_bs_dds(const void* a, const void* b_sp, void* c,
+                  const int32_t* seg_ptr, const int32_t* seg_blk, const int32_t* seg_inner,
+                  int n_seg, int cols_per_head, int Z, int M, int blk, int trans_b,
+                  int64_t a_sz, int64_t a_sh, int64_t a_sm, int64_t a_sk,
+                  int64_t b_sz,
+                  int64_t c_sz, int64_t c_sh, int64_t c_sm, int64_t c_sn,
+                  int dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Block-sparse row operations.  row_ptr (n_brow+1) / row_blk / row_col int32: for every
+ * (head, block-row) the ids and block-columns of its nonzero blocks (the information of the
+ * reference's row LUT, ref: blocksparse_logsumexp.py:107-128).  n_brow = H * M/blk.
+ * ---------------------------------------------------------------------------------------- */
+
+/* In-place softmax over the nonzero blocks of each row of x*scale + kpm[z,col] + am[row,col]
+ * (ref: triton.ops.blocksparse.softmax as called at blocksparse_attention.py:146-152).
+ * kpm (Z, kpm_stride) / am (rows, am_stride) fp32 additive or NULL; *_mul != 0 selects the
+ * 'mul' mode (0 -> -inf, nonzero -> 0).  A row with no finite entry becomes NaN.  max_row_nnz = the
+ * largest number of blocks in any block-row (an upper bound is fine). */
+int flyhip_bs_softmax(void* x, const int32_t* row_ptr, const int32_t* row_blk, const int32_t* row_col,
+                      int n_brow, int brows_per_head, int max_row_nnz, int Z, int blk, int64_t x_sz, float scale,
+                      const float* kpm, int64_t kpm_stride, int kpm_mul,
+                      const float* am, int64_t am_stride, int am_mul,
+                      int dtype, void* stream);
+
+/* Row reduction over nonzero blocks -> out (Z, n_brow*blk) in x's dtype: op 0 = logsumexp
+ * (ref: blocksparse_logsumexp.py:161-184), op 1 = sum (ref: blocksparse_sum.py:156-179).
+ * Rows of an empty block-row give 0. */
+int flyhip_bs_rowreduce(const void* x, void* out, const int32_t* row_ptr, const int32_t* row_blk,
+                        int n_brow, int Z, int blk, int64_t x_sz, int op, int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,182 @@
+"""Parity of the HIP block-sparse matmuls / row ops against the CPU oracle (GPU box only)."""
+import math
+
+import pytest
+import torch
+
+from conftest import rel_err
+from oracle import blocksparse as ob
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda:0'
+TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2, torch.float16: 2e-3}
+
+
+def random_layout(H, p, r, seed, density=0.5):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.rand(H, p, r, generator=g) < density).long()
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('block', [16, 32, 64, 128])
+def test_sdd_softmax_dsd_pipeline(block, dtype):
+    """The reference's own pipeline test (tests/models/attention/test_blocksparse_attention.py:32-81)
+    at several block sizes and dtypes."""
+    from fly_amd import matmul, softmax
+    print('case', block, dtype, flush=True)
+    Z, H, p, r, K = 2, 3, 4, 3, 48 if block == 16 else 64
+    g = torch.Generator().manual_seed(2357)
+    q = torch.randn(Z, H, p * block, K, generator=g).to(dtype)
+    k = torch.randn(Z, H, r * block, K, generator=g).to(dtype)
+    v = torch.randn(Z, H, r * block, K, generator=g).to(dtype)
+    layout = random_layout(H, p, r, 1)
+    layout[0, 1, :] = 0                                  # an empty block-row
+    tol = TOL[dtype]
+
+    qk = matmul(layout, block, 'sdd', trans_a=False, trans_b=True)(q.to(DEV), k.to(DEV))
+    qk_ref = ob.sdd(q, k, layout, block, trans_b=True)
+    assert qk.shape == qk_ref.shape
+    assert rel_err(qk, qk_ref) <= tol
+
+    attn = softmax(layout, block)(qk.clone(), scale=0.23)
+    attn_ref = ob.block_softmax(qk.cpu(), layout, block, scale=0.23)
+    assert rel_err(attn, attn_ref) <= tol
+
+    out = matmul(layout, block, 'dsd')(attn, v.to(DEV))
+    out_ref = ob.dsd(attn.cpu(), v, layout, block)
+    assert rel_err(out, out_ref) <= tol
+    assert out.shape == (Z, H, p * block, K)
+    # rows of the empty block-row are exactly zero
+    assert float(out[:, 0, block:2 * block].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize('trans_a,trans_b', [(False, False), (True, False), (False, True), (True, True)])
+@pytest.mark.parametrize('mode', ['sdd', 'dsd', 'dds'])
+def test_matmul_modes_and_transposes(mode, trans_a, trans_b):
+    from fly_amd import matmul
+    print('case', mode, trans_a, trans_b, flush=True)
+    block, Z, H, p, r = 32, 2, 2, 3, 5
+    layout = random_layout(H, p, r, 3)
+    g = torch.Generator().manual_seed(11)
+    nnz = int(layout.sum())
+    if mode == 'sdd':
+        K = 48
+        a = torch.randn((Z, H, K, p * block) if trans_a else (Z, H, p * block, K), generator=g)
+        b = torch.randn((Z, H, r * block, K) if trans_b else (Z, H, K, r * block), generator=g)
+        ref = ob.sdd(a, b, layout, block, trans_a, trans_b)
+    elif mode == 'dsd':
+        a = torch.randn(Z, nnz, block, block, generator=g)
+        inner = (p if trans_a else r) * block
+        N = 40
+        b = torch.randn((Z, H, N, inner) if trans_b else (Z, H, inner, N), generator=g)
+        ref = ob.dsd(a, b, layout, block, trans_a, trans_b)
+    else:
+        b = torch.randn(Z, nnz, block, block, generator=g)
+        inner = (r if trans_b else p) * block
+        M = 72
+        a = torch.randn((Z, H, inner, M) if trans_a else (Z, H, M, inner), generator=g)
+        ref = ob.dds(a, b, layout, block, trans_a, trans_b)
+    out = matmul(layout, block, mode, trans_a=trans_a, trans_b=trans_b)(a.to(DEV), b.to(DEV))
+    assert out.shape == ref.shape
+    assert rel_err(out, ref) <= 1e-5
+
+
+def test_softmax_masks_and_rowreduce():
+    from fly_amd import softmax, logsumexp, blocksparse_sum
+    block, Z, H, p, r = 32, 3, 2, 4, 6
+    layout = random_layout(H, p, r, 5, density=0.6)
+    layout[1, 2, :] = 0
+    g = torch.Generator().manual_seed(4)
+    nnz = int(layout.sum())
+    x = torch.randn(Z, nnz, block, block, generator=g)
+    lens = torch.tensor([r * block, 70, 1])
+    kpm = torch.log((torch.arange(r * block).view(1, -1) < lens.view(-1, 1)).float())
+    am_bool = torch.rand(p * block, r * block, generator=g) < 0.7
+    am = torch.log(am_bool.float())
+    for kw_dev, kw_ref in [
+        (dict(key_padding_mask=kpm.to(DEV)), dict(key_padding_mask=kpm)),
+        (dict(attn_mask=am.to(DEV)), dict(attn_mask=am)),
+        (dict(key_padding_mask=kpm.to(DEV), attn_mask=am.to(DEV)), dict(key_padding_mask=kpm, attn_mask=am)),
+        (dict(attn_mask=am_bool.float().to(DEV), attn_mask_mode='mul'),
+         dict(attn_mask=am_bool.float(), attn_mask_mode='mul')),
+    ]:
+        got = softmax(layout, block)(x.clone().to(DEV), scale=0.5, **kw_dev).cpu()
+        ref = ob.block_softmax(x, layout, block, scale=0.5, **kw_ref)
+        assert torch.equal(got.isnan(), ref.isnan())
+        assert rel_err(got.nan_to_num(), ref.nan_to_num()) <= 1e-5
+    assert rel_err(logsumexp(layout, block)(x.to(DEV)), ob.block_logsumexp(x, layout, block)) <= 1e-5
+    assert rel_err(blocksparse_sum(layout, block)(x.to(DEV)), ob.block_sum(x, layout, block)) <= 1e-5
+    # long rows take the multi-pass kernel
+    layout = torch.ones(1, 1, 80, dtype=torch.long)
+    x = torch.randn(2, 80, 32, 32, generator=g)
+    got = softmax(layout, 32)(x.clone().to(DEV), scale=1.3).cpu()
+    assert rel_err(got, ob.block_softmax(x, layout, 32, scale=1.3)) <= 1e-5
+
+
+def test_blocksparse_attention_module():
+    """BlockSparseAttention end to end with masks and sizes that need padding
+    (cf. tests/models/attention/test_blocksparse_attention.py:83-142)."""
+    from fly_amd import BlockSparseAttention, FullMask, LengthMask
+
+    class Cfg:
+        block = 16
+
+        def make_layout(self, seqlen):
+            nb = seqlen // self.block
+            lay = ob.band_layout(nb, nb, 1)
+            lay[:, 0] = 1
+            return lay.unsqueeze(0).repeat(3, 1, 1)
+
+    B, T, S, H, E, D = 2, 235, 179, 3, 15, 33
+    g = torch.Generator().manual_seed(0)
+    q = torch.randn(B, T, H, E, generator=g)
+    k = torch.randn(B, S, H, E, generator=g)
+    v = torch.randn(B, S, H, D, generator=g)
+    lengths = torch.tensor([S, 77])
+    am_bool = torch.rand(T, S, generator=g) < 0.8
+    mod = BlockSparseAttention(Cfg(), attention_dropout=0.0, max_seq_length=256).to(DEV)
+    out, _ = mod(q.to(DEV), k.to(DEV), v.to(DEV), attn_mask=FullMask(am_bool.to(DEV)),
+                 key_padding_mask=LengthMask(lengths.to(DEV), max_len=S))
+    ref = ob.blocksparse_attention(q, k, v, mod.master_layout.cpu(), 16, key_lengths=lengths,
+                                   attn_mask_bool=am_bool)
+    assert out.shape == (B, T, H, D)
+    assert rel_err(out, ref) <= 1e-5
+
+
+def test_blocksparse_linear_and_sparse_lr():
+    """Pixelfly linear at small, non-aligned sizes (cf. tests/models/layers/test_blocksparse_linear.py:88-134)."""
+    from fly_amd import BlockSparseLinear, FlatBlockButterflySparsityConfig, SparseLRLinear
+    torch.manual_seed(0)
+    cfg = FlatBlockButterflySparsityConfig(8, 2, block=32)
+    lin = BlockSparseLinear(497, 698, cfg).to(DEV)
+    x = torch.randn(3, 57, 497)
+    y = lin(x.to(DEV))
+    ref = ob.blocksparse_linear(x, lin.weight.detach().cpu(), lin.layout.cpu(), 32, lin.bias.detach().cpu(), 698)
+    assert y.shape == (3, 57, 698)
+    assert rel_err(y, ref) <= 1e-5
+
+    slr = SparseLRLinear(256, 512, {'_target_': 'src.models.layers.blocksparse_linear.BlockSparseLinear',
+                                    'sparsity_config': cfg}, rank=16).to(DEV)
+    x = torch.randn(100, 256)
+    y = slr(x.to(DEV))
+    sp = ob.blocksparse_linear(x, slr.sparse.weight.detach().cpu(), slr.sparse.layout.cpu(), 32, None, 512)
+    ref = ob.sparse_lr_linear(x, sp, slr.low_rank.lr_weight1.detach().cpu(), slr.low_rank.lr_weight2.detach().cpu(),
+                              slr.gate.weight.detach().cpu(), slr.gate.bias.detach().cpu(), slr.bias.detach().cpu())
+    assert rel_err(y, ref) <= 1e-4
+
+
+def test_config2_layout_stage_parity_reduced():
+    """BASELINE config 2 pattern (band +-4 OR flat butterfly (8,2), block 32, bf16) at B=1, H=2."""
+    from fly_amd import matmul, softmax, FlatBlockButterflySparsityConfig
+    L, d, block = 4096, 64, 32
+    lay = (FlatBlockButterflySparsityConfig(8, 2, block).make_layout(L) + ob.band_layout(L // block, L // block, 4)) > 0
+    assert int(lay.sum()) == 6204
+    layout = lay.long().unsqueeze(0).repeat(2, 1, 1)
+    g = torch.Generator().manual_seed(0)
+    q, k, v = (torch.randn(1, 2, L, d, generator=g).bfloat16() for _ in range(3))
+    qk = matmul(layout, block, 'sdd', trans_b=True)(q.to(DEV), k.to(DEV))
+    assert rel_err(qk, ob.sdd(q, k, layout, block, trans_b=True)) <= 2e-2
+    p = softmax(layout, block)(qk.clone(), scale=0.125)
+    assert rel_err(p, ob.block_softmax(qk.cpu(), layout, block, scale=0.125)) <= 2e-2
+    out = matmul(layout, block, 'dsd')(p, v.to(DEV))
+    assert rel_err(out, ob.dsd(p.cpu(), v, layout, block)) <= 2e-2
