@@ -1,0 +1,186 @@
+#!/usr/bin/env python3
+"""Benchmark of the Scatterbrain-local attention forward on one MI355X.
+
+One "step" is one forward of BASELINE config 1 (fp32, B=2, H=1, L=3136, d=64, band 256 each side,
+128 orthogonal-Gaussian random features) through the C ABI: the key-side pass
+(flyhip_sb_kv_reduce) followed by the fused band pass (flyhip_sblocal_fwd), inputs resident in
+HBM.  Prints ONE JSON line: tokens/s for the whole forward, the roofline of the dominant kernel
+(the fused band kernel, timed with events on its stream inside the timed region), the CPU oracle
+timed on this box's host cores, and -- as `extra` -- the block-sparse SDD / softmax / DSD stages
+of BASELINE config 2 (bf16, B=8, H=12, L=4096, d=64, block 32).
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+
+def sblocal_flops(B, H, T, S, E, D, m, lc):
+    """Algorithmic FLOPs of one forward (band pairs x 2(E+m+D), the two projections, K'^T V,
+    Q'(K'^T V) and the normaliser dot) and the share of them the fused band kernel computes."""
+    lo, hi = lc // 2, (lc + 1) // 2
+    pairs = B * H * sum(max(0, min(S, i + hi) - max(0, i - lo)) for i in range(T))
+    band = pairs * 2 * (E + m + D)
+    proj_q = 2 * B * H * T * E * (m // 2)
+    proj_k = 2 * B * H * S * E * (m // 2)
+    kv = 2 * B * H * S * m * D
+    qkv = 2 * B * H * T * m * D + 2 * B * H * T * m
+    total = band + proj_q + proj_k + kv + qkv
+    fused = band + proj_q + qkv            # what the fused band kernel computes
+    return total, fused
+
+
+def bench_sblocal(steps, warmup):
+    from fly_amd.sblocal_attention import SBLocalPlan
+    from oracle import sblocal as osb
+    dev = torch.device('cuda:0')
+    B, H, L, E, D, mh, lc = 2, 1, 3136, 64, 64, 64, 512
+    g = torch.Generator().manual_seed(0)
+    q = torch.randn(B, L, H, E, generator=g) * E ** -0.25
+    k = torch.randn(B, L, H, E, generator=g) * E ** -0.25
+    v = torch.randn(B, L, H, D, generator=g)
+    P = osb.gaussian_orthogonal_random_matrix(mh, E, generator=g)
+    t = 1 / math.sqrt(E)
+    qd, kd, vd, Pd = (x.to(dev) for x in (q, k, v, P))
+    plan = SBLocalPlan(B, H, L, L, E, mh, mh, torch.float32, dev)
+    out = torch.empty(B, L, H, D, device=dev)
+    ln = torch.empty(B, H, L, device=dev)
+
+    for _ in range(warmup):
+        plan.run(qd, kd, vd, Pd, None, lc, t, out, ln)
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for i in range(steps):
+        plan.run_keys(kd, vd, Pd, None, t)
+        ev[i][0].record()
+        plan.run_queries(qd, kd, vd, Pd, None, lc, t, out, ln)
+        ev[i][1].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    fwd_ms = sum(a.elapsed_time(b) for a, b in ev) / steps
+
+    # parity of what was just timed, against the float64 oracle
+    ref_out, ref_ln = osb.sblocal_attention(q.double(), k.double(), v.double(), P.double(), lc)
+    err_out = float((out.cpu().double() - ref_out).abs().max() / ref_out.abs().max())
+    err_ln = float((ln.cpu().double().unsqueeze(-1) - ref_ln).abs().max() / ref_ln.abs().max())
+
+    total_flops, fwd_flops = sblocal_flops(B, H, L, L, E, D, 2 * mh, lc)
+    ms_per_step = wall / steps * 1e3
+    achieved = fwd_flops / (fwd_ms * 1e-3) / 1e12
+    res = {
+        'tokens_per_s': B * L / (wall / steps),
+        'ms_per_step': ms_per_step,
+        'roofline': {'bound': 'mfma', 'kernel': 'sblocal_fwd_kernel<float,64,64,128>',
+                     'achieved': achieved, 'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s',
+                     'frac': achieved / PEAK_FP32_MFMA_TFLOPS, 'traffic': None,
+                     'kernel_ms': fwd_ms, 'flops_per_launch': fwd_flops},
+        'parity': {'out_rel_err': err_out, 'log_norm_rel_err': err_ln},
+        'flops_per_step': total_flops,
+    }
+
+    # CPU baseline: the oracle (a port of the reference op sequence) on the host cores, bounded
+    torch.set_num_threads(min(os.cpu_count() or 1, 16))
+    osb.sblocal_attention(q, k, v, P, lc)
+    n, t0 = 0, time.perf_counter()
+    while True:
+        osb.sblocal_attention(q, k, v, P, lc)
+        n += 1
+        el = time.perf_counter() - t0
+        if el > 10.0 or n >= 200:
+            break
+    res['cpu_baseline'] = {'value': B * L * n / el, 'unit': 'tokens/s', 'cores': torch.get_num_threads(),
+                           'kind': 'port',
+                           'sample': f'{n} full-size forwards of the same workload (fp32 oracle, {el:.1f} s)'}
+    return res
+
+
+def bench_blocksparse(steps, warmup):
+    """BASELINE config 2: SDD -> softmax -> DSD, bf16, B=8, H=12, L=4096, d=64, block 32."""
+    from fly_amd import matmul, softmax, FlatBlockButterflySparsityConfig
+    dev = torch.device('cuda:0')
+    B, H, L, d, block = 8, 12, 4096, 64, 32
+    nb = L // block
+    r = torch.arange(nb)
+    band = ((r.view(-1, 1) - r.view(1, -1)).abs() <= 4)
+    lay = (FlatBlockButterflySparsityConfig(8, 2, block).make_layout(L) > 0) | band
+    layout = lay.long().unsqueeze(0).repeat(H, 1, 1)
+    nnz = int(layout.sum())
+    g = torch.Generator().manual_seed(0)
+    q, k, v = (torch.randn(B, H, L, d, generator=g).bfloat16().to(dev) for _ in range(3))
+    sdd = matmul(layout, block, 'sdd', trans_b=True)
+    dsd = matmul(layout, block, 'dsd')
+    sm = softmax(layout, block)
+    out = {}
+
+    def timeit(fn):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps
+
+    qk = sdd(q, k)
+    flops = 2 * B * nnz * block * block * d
+    sp_bytes = B * nnz * block * block * 2
+    dense_bytes = B * H * L * d * 2
+    ms = timeit(lambda: sdd(q, k))
+    out['sdd'] = {'ms': ms, 'tflops': flops / ms / 1e9, 'gbs': (sp_bytes + 2 * dense_bytes) / ms / 1e6}
+    ms = timeit(lambda: sm(qk, scale=0.125))
+    out['softmax'] = {'ms': ms, 'gbs': 2 * sp_bytes / ms / 1e6}
+    ms = timeit(lambda: dsd(qk, v))
+    out['dsd'] = {'ms': ms, 'tflops': flops / ms / 1e9, 'gbs': (sp_bytes + 2 * dense_bytes) / ms / 1e6}
+    for st in out.values():
+        st['hbm_frac'] = st['gbs'] / PEAK_HBM_GBS
+    out['config'] = f'bf16 B={B} H={H} L={L} d={d} block={block} nnz/head={nnz // H}'
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=200)
+    ap.add_argument('--warmup', type=int, default=20)
+    ap.add_argument('--no-blocksparse', action='store_true')
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print('bench.py: this build measures one GPU; --gpus must be 1 (nothing here shards over devices)',
+              file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print('bench.py: no GPU visible', file=sys.stderr)
+        sys.exit(1)
+    sb = bench_sblocal(args.steps, args.warmup)
+    line = {
+        'metric': 'SBLocal attention forward tokens/s (fp32, L=3136, d=64)',
+        'value': sb['tokens_per_s'], 'unit': 'tokens/s', 'n_gpus': 1, 'steps': args.steps,
+        'warmup': args.warmup, 'ms_per_step': sb['ms_per_step'], 'higher_is_better': True,
+        'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f32', 'data': 'synthetic',
+        'config': {'workload': 'BASELINE config 1 (configs[0]): SBLocal fwd fp32 B=2 H=1 L=3136 d=64 '
+                               'local_context=512 nb_features=128, seeded orthogonal-Gaussian projection'},
+        'roofline': sb['roofline'], 'cpu_baseline': sb['cpu_baseline'],
+        'gpu_over_cpu': sb['tokens_per_s'] / sb['cpu_baseline']['value'],
+        'parity': sb['parity'],
+    }
+    if not args.no_blocksparse:
+        line['extra'] = {'blocksparse_config2': bench_blocksparse(max(5, args.steps // 10), 3)}
+    print(json.dumps(line))
+
+
+if __name__ == '__main__':
+    main()

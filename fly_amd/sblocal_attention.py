@@ -28,6 +28,60 @@ def _vector_ready(x):
             and x.data_ptr() % 16 == 0)
 
 
+class SBLocalPlan:
+    """Scratch buffers and the two C-ABI calls for one problem shape.  Callers that run the same
+    shape repeatedly (serving loops, benchmarks) keep one plan and call ``run`` with tensors that
+    are already padded and vector-ready; ``sblocal_forward`` builds a plan per call.
+
+    q (B,T,H,dim), k, v (B,S,H,dim), proj (mh, dim) float32, lens (B,) int64 or None,
+    out (B,T,H,dim), log_norm (B,H,T) float32.  Buffers of one plan are shared by its runs: runs
+    of the same plan on different streams race."""
+
+    def __init__(self, B, H, T, S, dim, mh, mh_valid, dtype, device):
+        n_chunks, n_split = ctypes.c_int(), ctypes.c_int()
+        _lib.call('flyhip_sb_plan', B, H, S, ctypes.byref(n_chunks), ctypes.byref(n_split))
+        self.n_chunks, self.n_split = n_chunks.value, n_split.value
+        self.shape = (B, H, T, S, dim, mh, mh_valid)
+        self.device = torch.device(device)
+        self.code = _lib.DTYPE_CODE[dtype]
+        m, f32 = 2 * mh, torch.float32
+        self.kfeat = torch.empty(B, H, self.n_chunks * 64, m, dtype=f32, device=device)
+        self.chunk_scale = torch.empty(B, H, self.n_chunks, dtype=f32, device=device)
+        self.kv_part = torch.empty(B, H, self.n_split, m * (dim + 1), dtype=f32, device=device)
+        self.part_max = torch.empty(B, H, self.n_split, dtype=f32, device=device)
+        self.kv = torch.empty(B, H, m, dim, dtype=f32, device=device)
+        self.ksum = torch.empty(B, H, m, dtype=f32, device=device)
+        self.kmax = torch.empty(B, H, dtype=f32, device=device)
+
+    def run_keys(self, k, v, proj, lens, t, stream=None):
+        B, H, T, S, dim, mh, mh_valid = self.shape
+        stream = _lib.stream_ptr(self.device) if stream is None else stream
+        _lib.call('flyhip_sb_kv_reduce', k.data_ptr(), v.data_ptr(), proj.data_ptr(), _lib.ptr(lens),
+                  self.kfeat.data_ptr(), self.chunk_scale.data_ptr(), self.kv_part.data_ptr(),
+                  self.part_max.data_ptr(), self.kv.data_ptr(), self.ksum.data_ptr(), self.kmax.data_ptr(),
+                  B, H, S, dim, dim, mh, mh_valid, self.n_split,
+                  k.stride(0), k.stride(2), k.stride(1), v.stride(0), v.stride(2), v.stride(1),
+                  t, self.code, stream)
+
+    def run_queries(self, q, k, v, proj, lens, local_context, t, out, log_norm, stream=None):
+        B, H, T, S, dim, mh, mh_valid = self.shape
+        stream = _lib.stream_ptr(self.device) if stream is None else stream
+        _lib.call('flyhip_sblocal_fwd', q.data_ptr(), k.data_ptr(), v.data_ptr(), proj.data_ptr(),
+                  self.kfeat.data_ptr(), self.chunk_scale.data_ptr(), self.kv.data_ptr(),
+                  self.ksum.data_ptr(), self.kmax.data_ptr(), _lib.ptr(lens),
+                  out.data_ptr(), log_norm.data_ptr(),
+                  B, H, T, S, dim, dim, mh, mh_valid, local_context,
+                  q.stride(0), q.stride(2), q.stride(1), k.stride(0), k.stride(2), k.stride(1),
+                  v.stride(0), v.stride(2), v.stride(1), out.stride(0), out.stride(2), out.stride(1),
+                  t, self.code, stream)
+
+    def run(self, q, k, v, proj, lens, local_context, t, out, log_norm):
+        with torch.cuda.device(self.device):
+            stream = _lib.stream_ptr(self.device)
+            self.run_keys(k, v, proj, lens, t, stream)
+            self.run_queries(q, k, v, proj, lens, local_context, t, out, log_norm, stream)
+
+
 def sblocal_forward(query, key, value, projection_matrix, local_context, softmax_temp=None,
                     key_lengths=None):
     """Scatterbrain-local attention forward on the GPU.
@@ -71,36 +125,10 @@ def sblocal_forward(query, key, value, projection_matrix, local_context, softmax
         if lens.shape != (B,):
             raise ValueError(f'key_lengths must have shape ({B},)')
 
-    n_chunks, n_split = ctypes.c_int(), ctypes.c_int()
-    _lib.call('flyhip_sb_plan', B, H, S, ctypes.byref(n_chunks), ctypes.byref(n_split))
-    n_chunks, n_split = n_chunks.value, n_split.value
-    dev, f32 = query.device, torch.float32
-    kfeat = torch.empty(B, H, n_chunks * 64, m, dtype=f32, device=dev)
-    chunk_scale = torch.empty(B, H, n_chunks, dtype=f32, device=dev)
-    kv_part = torch.empty(B, H, n_split, m * (dim + 1), dtype=f32, device=dev)
-    part_max = torch.empty(B, H, n_split, dtype=f32, device=dev)
-    kv = torch.empty(B, H, m, dim, dtype=f32, device=dev)
-    ksum = torch.empty(B, H, m, dtype=f32, device=dev)
-    kmax = torch.empty(B, H, dtype=f32, device=dev)
-    out = torch.empty(B, T, H, dim, dtype=query.dtype, device=dev)
-    log_norm = torch.empty(B, H, T, dtype=f32, device=dev)
-
-    code = _lib.dtype_code(query)
-    stream = _lib.stream_ptr(dev)
-    with torch.cuda.device(dev):
-        _lib.call('flyhip_sb_kv_reduce', k.data_ptr(), v.data_ptr(), proj.data_ptr(), _lib.ptr(lens),
-                  kfeat.data_ptr(), chunk_scale.data_ptr(), kv_part.data_ptr(), part_max.data_ptr(),
-                  kv.data_ptr(), ksum.data_ptr(), kmax.data_ptr(),
-                  B, H, S, dim, dim, mh, mh_valid, n_split,
-                  k.stride(0), k.stride(2), k.stride(1), v.stride(0), v.stride(2), v.stride(1),
-                  t, code, stream)
-        _lib.call('flyhip_sblocal_fwd', q.data_ptr(), k.data_ptr(), v.data_ptr(), proj.data_ptr(),
-                  kfeat.data_ptr(), chunk_scale.data_ptr(), kv.data_ptr(), ksum.data_ptr(), kmax.data_ptr(),
-                  _lib.ptr(lens), out.data_ptr(), log_norm.data_ptr(),
-                  B, H, T, S, dim, dim, mh, mh_valid, local_context,
-                  q.stride(0), q.stride(2), q.stride(1), k.stride(0), k.stride(2), k.stride(1),
-                  v.stride(0), v.stride(2), v.stride(1), out.stride(0), out.stride(2), out.stride(1),
-                  t, code, stream)
+    plan = SBLocalPlan(B, H, T, S, dim, mh, mh_valid, query.dtype, query.device)
+    out = torch.empty(B, T, H, dim, dtype=query.dtype, device=query.device)
+    log_norm = torch.empty(B, H, T, dtype=torch.float32, device=query.device)
+    plan.run(q, k, v, proj, lens, local_context, t, out, log_norm)
     return out[..., :D], log_norm.unsqueeze(-1)
 
 
