@@ -52,7 +52,7 @@ def bench_sblocal(steps, warmup):
     P = osb.gaussian_orthogonal_random_matrix(mh, E, generator=g)
     t = 1 / math.sqrt(E)
     qd, kd, vd, Pd = (x.to(dev) for x in (q, k, v, P))
-    plan = SBLocalPlan(B, H, L, L, E, mh, mh, torch.float32, dev)
+    plan = SBLocalPlan(B, H, L, L, E, mh, mh, torch.float32, dev, lc)
     out = torch.empty(B, L, H, D, device=dev)
     ln = torch.empty(B, H, L, device=dev)
 

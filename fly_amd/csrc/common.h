@@ -131,16 +131,26 @@ template <> struct Frag<f16_t> {
     }
 };
 
-// wave-level butterflies across the four 16-lane groups (lanes r, r+16, r+32, r+48)
+// wave-level butterflies across the four 16-lane groups (lanes r, r+16, r+32, r+48), on the
+// gfx950 row-swap instructions: permlane16_swap(v, v) yields {rows 0,0,2,2} and {rows 1,1,3,3},
+// permlane32_swap(v, v) yields {low half twice} and {high half twice}; no LDS traffic
+__device__ __forceinline__ void rows_pair16(float v, float& a, float& b) {
+    auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    a = __uint_as_float(r[0]); b = __uint_as_float(r[1]);
+}
+__device__ __forceinline__ void rows_pair32(float v, float& a, float& b) {
+    auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    a = __uint_as_float(r[0]); b = __uint_as_float(r[1]);
+}
 __device__ __forceinline__ float group_max(float v) {
-    v = fmaxf(v, __shfl_xor(v, 16));
-    v = fmaxf(v, __shfl_xor(v, 32));
-    return v;
+    float a, b;
+    rows_pair16(v, a, b); v = fmaxf(a, b);
+    rows_pair32(v, a, b); return fmaxf(a, b);
 }
 __device__ __forceinline__ float group_sum(float v) {
-    v += __shfl_xor(v, 16);
-    v += __shfl_xor(v, 32);
-    return v;
+    float a, b;
+    rows_pair16(v, a, b); v = a + b;
+    rows_pair32(v, a, b); return a + b;
 }
 __device__ __forceinline__ float wave_max(float v) {
     for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));

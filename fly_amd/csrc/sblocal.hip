@@ -6,11 +6,14 @@
 //                       written to HBM once, plus the partial K'^T V / sum K' reductions with an
 //                       online rescale to the running maximum.
 //   sb_combine_kernel : merges the partial reductions of one (batch, head).
-//   sblocal_fwd_kernel: per (batch, head, 64-query tile): query features in registers, then for
-//                       each 64-key tile of the band Q K^T and Q' K'^T on MFMA (transposed, so
-//                       that every lane owns one query), band/length masking, online softmax with
-//                       the low-rank overlap subtracted, P V on MFMA, and the epilogue that adds
-//                       the global low-rank term and writes out / log-normaliser.
+//   sblocal_fwd_kernel: per (batch, head, 64-query tile, part of the band): query features in
+//                       registers, then for each 32-key tile of its share of the band Q K^T and
+//                       Q' K'^T on MFMA (transposed, so that every lane owns one query),
+//                       band/length masking, online softmax with the low-rank overlap subtracted,
+//                       P V on MFMA; key tiles are double-buffered through LDS.  With one part the
+//                       epilogue adds the global low-rank term and writes out / log-normaliser;
+//                       with several parts (small problems, to fill the chip) each part writes an
+//                       un-normalised partial and sb_merge_kernel finishes the job.
 //
 // Layout of an MFMA 16x16 result in a lane (r = lane%16, g = lane/16): element i is
 // C[4g+i][r].  All products are formed "transposed" (rows = keys / features / value dims,
@@ -21,8 +24,11 @@
 
 namespace flyhip {
 
-constexpr int CH = 64;     // keys per chunk and per key tile
+constexpr int CH = 64;     // keys per feature chunk (granularity of the key-side stabiliser)
+constexpr int TK = 32;     // keys per tile of the fused band kernel
+constexpr int TQ = 64;     // queries per workgroup of the fused band kernel
 constexpr int NT = 256;    // threads per workgroup (4 waves)
+constexpr int NSTAT = 5;   // per-query statistics of a partial: m, ze, zp, qk1, lsq+kmax
 
 struct KvArgs {
     const void* k; const void* v; const float* proj; const int64_t* lens;
@@ -35,34 +41,46 @@ struct KvArgs {
 struct FwdArgs {
     const void* q; const void* k; const void* v; const float* proj;
     const float* kfeat; const float* chunk_scale; const float* kv; const float* ksum; const float* kmax;
-    const int64_t* lens; void* out; float* log_norm;
-    int B, H, T, S, mh_valid, lc, n_chunks;
+    const int64_t* lens; void* out; float* log_norm; float* part_ws;
+    int B, H, T, S, mh_valid, lc, n_chunks, n_parts;
     long q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss;
     float temp;
 };
 
-// rows [row0, row0+CH) of a (seq, W) matrix -> LDS tile with leading dimension LD; rows at or
-// beyond `limit` are zero filled
-template <typename T, int W, int LD>
-__device__ __forceinline__ void load_tile(float* dst, const T* src, long row_stride, int row0, int limit, int tid) {
-    constexpr int V4 = W / 4;
-    for (int idx = tid; idx < CH * V4; idx += NT) {
-        int row = idx / V4, c4 = idx % V4;
-        floatx4 val = {0.f, 0.f, 0.f, 0.f};
-        if (row0 + row < limit) val = load4_f32(src + (long)(row0 + row) * row_stride + 4 * c4);
-        *reinterpret_cast<floatx4*>(dst + row * LD + 4 * c4) = val;
+// ROWS x W tile of a (seq, W) matrix, moved global -> registers -> LDS in two steps so that all of
+// a thread's loads are in flight together (and, in the band kernel, fly during the MFMAs of the
+// previous tile).  Row indices are clamped to `last_row`: rows past the end re-read the last valid
+// row, which callers mask, so the loads need no branches and never leave the tensor.
+template <int ROWS, int W>
+struct RowTile {
+    static constexpr int V4 = W / 4, N = (ROWS * V4 + NT - 1) / NT;
+    floatx4 r[N];
+    template <typename T>
+    __device__ __forceinline__ void fetch(const T* src, long row_stride, int row0, int last_row, int tid) {
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+            const int idx = tid + NT * j, row = idx / V4, c4 = idx % V4;
+            if (N * NT == ROWS * V4 || idx < ROWS * V4)
+                r[j] = load4_f32(src + (long)min(row0 + row, last_row) * row_stride + 4 * c4);
+        }
     }
-}
+    template <int LD>
+    __device__ __forceinline__ void stash(float* dst, int tid, float scale = 1.0f) const {
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+            const int idx = tid + NT * j, row = idx / V4, c4 = idx % V4;
+            if (N * NT == ROWS * V4 || idx < ROWS * V4)
+                *reinterpret_cast<floatx4*>(dst + row * LD + 4 * c4) = r[j] * scale;
+        }
+    }
+};
 
+// projection matrix (MH, E) -> LDS rows of E+4 floats, scaled by sqrt(t)
 template <int E, int MH>
 __device__ __forceinline__ void load_proj(float* Ps, const float* proj, float scale, int tid) {
-    constexpr int V4 = E / 4, LD = E + 4;
-    for (int idx = tid; idx < MH * V4; idx += NT) {
-        int row = idx / V4, c4 = idx % V4;
-        floatx4 val = *reinterpret_cast<const floatx4*>(proj + row * E + 4 * c4);
-        val *= scale;
-        *reinterpret_cast<floatx4*>(Ps + row * LD + 4 * c4) = val;
-    }
+    RowTile<MH, E> t;
+    t.fetch(proj, E, 0, MH - 1, tid);
+    t.template stash<E + 4>(Ps, tid, scale);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -102,8 +120,14 @@ __global__ __launch_bounds__(NT) void sb_kfeat_kernel(KvArgs a) {
     for (int c = c0; c < c1; ++c) {
         const int s_base = c * CH;
         __syncthreads();
-        load_tile<T, E, LDK>(Ks, kptr, a.k_ss, s_base, len, tid);
-        load_tile<T, D, LDV>(Vs, vptr, a.v_ss, s_base, len, tid);
+        {
+            RowTile<CH, E> kt;
+            RowTile<CH, D> vt;
+            kt.fetch(kptr, a.k_ss, s_base, a.S - 1, tid);
+            vt.fetch(vptr, a.v_ss, s_base, a.S - 1, tid);
+            kt.template stash<LDK>(Ks, tid);
+            vt.template stash<LDV>(Vs, tid);
+        }
         __syncthreads();
 
         // projection of this wave's 16 keys: dd[fb][i] = (sqrt(t) P)[16fb+4g+i] . k[16w+r16]
@@ -216,21 +240,30 @@ __global__ __launch_bounds__(NT) void sb_kfeat_kernel(KvArgs a) {
     if (tid == 0) a.part_max[(long)bh * a.n_split + sp] = run_max;
 }
 
-// KV = sum_s exp(part_max_s - kmax) KV_s, same for Ksum; one thread per output element
-__global__ void sb_combine_kernel(const float* kv_part, const float* part_max, float* kv, float* ksum,
-                                  float* kmax_out, int n_split, int M, int D) {
+// KV = sum_s exp(part_max_s - kmax) KV_s, same for Ksum; one thread per output element, the
+// weights staged in LDS so that the loads over s are independent and stay in flight together
+constexpr int MAX_SPLIT = 1024;
+__global__ __launch_bounds__(256) void sb_combine_kernel(const float* kv_part, const float* part_max, float* kv,
+                                                         float* ksum, float* kmax_out, int n_split, int M, int D) {
+    __shared__ float wgt[MAX_SPLIT];
     const int bh = blockIdx.y;
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;
     const int per = M * (D + 1);
     float kmax = -INFINITY;
     for (int s = 0; s < n_split; ++s) kmax = fmaxf(kmax, part_max[(long)bh * n_split + s]);
+    for (int s = threadIdx.x; s < n_split; s += blockDim.x) {
+        const float pm = part_max[(long)bh * n_split + s];
+        // same expression as the band kernel's chunk weight, so that both sides of the
+        // "global minus band" low-rank difference carry bit-identical factors
+        wgt[s] = (pm == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((pm - kmax) * 1.4426950408889634f);
+    }
+    __syncthreads();
     if (idx == 0) kmax_out[bh] = (kmax == -INFINITY) ? 0.f : kmax;
     if (idx >= per) return;
+    const float* src = kv_part + (long)bh * n_split * per + idx;
     float acc = 0.f;
-    for (int s = 0; s < n_split; ++s) {
-        const float pm = part_max[(long)bh * n_split + s];
-        if (pm != -INFINITY) acc += expf(pm - kmax) * kv_part[((long)bh * n_split + s) * per + idx];
-    }
+#pragma unroll 16
+    for (int s = 0; s < n_split; ++s) acc += wgt[s] * src[(long)s * per];
     if (idx < M * D) kv[(long)bh * M * D + idx] = acc;
     else ksum[(long)bh * M + idx - M * D] = acc;
 }
@@ -238,27 +271,55 @@ __global__ void sb_combine_kernel(const float* kv_part, const float* part_max, f
 // ---------------------------------------------------------------------------------------
 // fused band kernel
 // ---------------------------------------------------------------------------------------
-template <typename T, int E, int D, int M>
+template <typename T, int E, int D, int M, bool SPLIT>
 __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
     constexpr int MH = M / 2, LDK = E + 4, LDV = D + 4, LDF = M + 4;
-    constexpr int FB = MH / 16, EC = E / 16, DB = D / 16, KB = CH / 16;
+    constexpr int FB = MH / 16, EC = E / 16, DB = D / 16, KB = TK / 16;
+    constexpr int STAGE = TK * (LDK + LDV + LDF);     // floats per LDS stage
     extern __shared__ float smem[];
-    float* Ks = smem;
-    float* Vs = Ks + CH * LDK;
-    float* Fs = Vs + CH * LDV;
-    float* Ps = smem;                         // only live before the key loop
+    float* Ps = smem;                                  // only live before the key loop
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
-    const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
-    const int q0 = blockIdx.x * 64;
+    const int bh = blockIdx.z, b = bh / a.H, h = bh % a.H;
+    const int part = blockIdx.y;
+    const int q0 = blockIdx.x * TQ;
     const int iq = q0 + 16 * w + r16;
     const bool qvalid = iq < a.T;
     const T* qptr = reinterpret_cast<const T*>(a.q) + b * a.q_sb + h * a.q_sh;
     const T* kptr = reinterpret_cast<const T*>(a.k) + b * a.k_sb + h * a.k_sh;
     const T* vptr = reinterpret_cast<const T*>(a.v) + b * a.v_sb + h * a.v_sh;
+    const float* fptr = a.kfeat + (long)bh * a.n_chunks * CH * M;
     const int len = a.lens ? min((int)a.lens[b], a.S) : a.S;
-    const float lnm_half = 0.5f * logf(2.0f * a.mh_valid);
+    const float lnm_half = 0.5f * __logf(2.0f * a.mh_valid);
     const int lc_lo = a.lc / 2, lc_hi = (a.lc + 1) / 2;    // band: -lc_lo <= s - i < lc_hi
+
+    // this workgroup's share of the band, in 32-key tiles
+    const int q_last = min(q0 + TQ - 1, a.T - 1);
+    const int lo = max(0, q0 - lc_lo);
+    const int hi = min(len, q_last + lc_hi);
+    int kt_lo = lo / TK;
+    int kt_hi = (hi > lo) ? (hi + TK - 1) / TK : kt_lo;
+    if (SPLIT) {
+        // the global low-rank epilogue of part 0 counts as one more tile when sharing out the band
+        const int per = (kt_hi - kt_lo + 1 + a.n_parts - 1) / a.n_parts;
+        const int first = kt_lo + part * per - (part > 0 ? 1 : 0);
+        const int last = kt_lo + (part + 1) * per - 1;
+        kt_lo = min(kt_hi, first);
+        kt_hi = min(kt_hi, last);
+    }
+
+    // start the first tile's loads before anything else
+    RowTile<TK, E> rk;
+    RowTile<TK, D> rv;
+    RowTile<TK, M> rf;
+    const int f_last = a.n_chunks * CH - 1;
+    if (kt_lo < kt_hi) {
+        rk.fetch(kptr, a.k_ss, kt_lo * TK, a.S - 1, tid);
+        rv.fetch(vptr, a.v_ss, kt_lo * TK, a.S - 1, tid);
+        rf.fetch(fptr, M, kt_lo * TK, f_last, tid);
+    }
+    const float* csp = a.chunk_scale + (long)bh * a.n_chunks;
+    float cscale = (kt_lo < kt_hi) ? csp[kt_lo * TK / CH] : 0.f;
 
     // query operand (B side: column = query, k = 16c+4g+j) and its squared norm
     floatx4 qr[EC];
@@ -297,125 +358,232 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const bool ok = 16 * fb + 4 * g + i < a.mh_valid;
-            qf[fb][i] = ok ? expf(dd[i] - qmax) : 0.f;
-            qf[FB + fb][i] = ok ? expf(-dd[i] - qmax) : 0.f;
+            qf[fb][i] = ok ? __expf(dd[i] - qmax) : 0.f;
+            qf[FB + fb][i] = ok ? __expf(-dd[i] - qmax) : 0.f;
         }
     }
+    __syncthreads();                 // Ps is dead; the tile buffers may overwrite it
 
+    // From here on all exponents are base 2 (one v_exp_f32 each): scores carry t*log2(e) through
+    // the query operand, the log-scales are converted once.
+    constexpr float LOG2E = 1.4426950408889634f, LN2 = 0.6931471805599453f;
     const float kmax = a.kmax[bh];
-    float m_run = lsq + kmax;       // reference exponent: max(running row max, log-scale of the low-rank part)
+    const float c0 = (lsq + kmax) * LOG2E;       // base-2 log-scale of the global low-rank term
+#pragma unroll
+    for (int c = 0; c < EC; ++c) qr[c] *= a.temp * LOG2E;
+    float m_run = c0;               // reference exponent: max(running row max, log-scale of the low-rank part)
     float ze = 0.f, zp = 0.f;       // per-lane partial sums (reduced over g at the end)
     floatx4 oacc[DB];
 #pragma unroll
     for (int db = 0; db < DB; ++db) oacc[db] = Frag<float>::zero();
-
-    const int q_last = min(q0 + 63, a.T - 1);
-    const int lo = max(0, q0 - lc_lo);
-    const int hi = min(len, q_last + lc_hi);
-    const int kt_lo = lo / CH;
-    const int kt_hi = (hi > lo) ? (hi + CH - 1) / CH : kt_lo;
     const int qw0 = q0 + 16 * w;    // first query of this wave
+    // keys this lane's query may see: smin <= s < smin + span
+    const int smin = max(iq - lc_lo, 0);
+    const unsigned span = qvalid ? (unsigned)max(min(iq + lc_hi, len) - smin, 0) : 0u;
+
+    if (kt_lo < kt_hi) {
+        rk.template stash<LDK>(smem, tid);
+        rv.template stash<LDV>(smem + TK * LDK, tid);
+        rf.template stash<LDF>(smem + TK * (LDK + LDV), tid);
+    }
+    __syncthreads();
 
     for (int kt = kt_lo; kt < kt_hi; ++kt) {
-        const int s_base = kt * CH;
-        __syncthreads();
-        load_tile<T, E, LDK>(Ks, kptr, a.k_ss, s_base, len, tid);
-        load_tile<T, D, LDV>(Vs, vptr, a.v_ss, s_base, len, tid);
-        load_tile<float, M, LDF>(Fs, a.kfeat + (long)bh * a.n_chunks * CH * M, M, s_base, a.n_chunks * CH, tid);
-        __syncthreads();
-        const float cscale = a.chunk_scale[(long)bh * a.n_chunks + kt];
-        const float beta_k = expf(cscale - kmax);            // <= 1
+        const int s_base = kt * TK;
+        const int cur = (kt - kt_lo) & 1;
+        const float* Ks = smem + cur * STAGE;
+        const float* Vs = Ks + TK * LDK;
+        const float* Fs = Vs + TK * LDV;
+        const bool more = kt + 1 < kt_hi;
+        float cscale_next = cscale;
+        if (more) {                                      // next tile's loads fly during the MFMAs
+            rk.fetch(kptr, a.k_ss, s_base + TK, a.S - 1, tid);
+            rv.fetch(vptr, a.v_ss, s_base + TK, a.S - 1, tid);
+            rf.fetch(fptr, M, s_base + TK, f_last, tid);
+            cscale_next = csp[(s_base + TK) / CH];
+        }
+        // weight of this chunk's features relative to the global key stabiliser (<= 1); the same
+        // expression weights the chunk in sb_combine_kernel
+        const float wc = __builtin_amdgcn_exp2f((cscale - kmax) * LOG2E);
 
+        // wave-uniform: does this tile touch the band of any of the wave's 16 queries?  (Blocks of a
+        // touched tile that lie outside the band are computed and masked: no branches among the MFMAs.)
+        const bool any = !(s_base + TK - 1 - qw0 < -lc_lo || s_base - (qw0 + 15) >= lc_hi || s_base >= len);
+        if (any) {
+            // scores^T: s1 = (t log2e) K q, s2 = K' q'.  The accumulation chains of the two key
+            // blocks and of the two products are interleaved so that no MFMA waits on its predecessor.
+            floatx4 s1[KB], s2[KB];
 #pragma unroll
-        for (int kb = 0; kb < KB; ++kb) {
-            const int s0 = s_base + 16 * kb;
-            // wave-uniform: does this 16-key block touch the band of any of the wave's 16 queries?
-            if (s0 + 15 - qw0 < -lc_lo || s0 - (qw0 + 15) >= lc_hi || s0 >= len) continue;
-            floatx4 s1 = Frag<float>::zero(), s2 = Frag<float>::zero();
-            const float* krow = Ks + (16 * kb + r16) * LDK + 4 * g;
+            for (int kb = 0; kb < KB; ++kb) { s1[kb] = Frag<float>::zero(); s2[kb] = Frag<float>::zero(); }
+            constexpr int CMAX = EC > 2 * FB ? EC : 2 * FB;
 #pragma unroll
-            for (int c = 0; c < EC; ++c)
-                s1 = Frag<float>::mma(*reinterpret_cast<const floatx4*>(krow + 16 * c), qr[c], s1);
-            const float* frow = Fs + (16 * kb + r16) * LDF + 4 * g;
+            for (int c = 0; c < CMAX; ++c) {
+                floatx4 ka[KB], fa[KB];
 #pragma unroll
-            for (int c = 0; c < 2 * FB; ++c)
-                s2 = Frag<float>::mma(*reinterpret_cast<const floatx4*>(frow + 16 * c), qf[c], s2);
+                for (int kb = 0; kb < KB; ++kb) {
+                    if (c < EC) ka[kb] = *reinterpret_cast<const floatx4*>(Ks + (16 * kb + r16) * LDK + 4 * g + 16 * c);
+                    if (c < 2 * FB) fa[kb] = *reinterpret_cast<const floatx4*>(Fs + (16 * kb + r16) * LDF + 4 * g + 16 * c);
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                    for (int kb = 0; kb < KB; ++kb) {
+                        if (c < EC) s1[kb] = __builtin_amdgcn_mfma_f32_16x16x4f32(ka[kb][j], qr[c][j], s1[kb], 0, 0, 0);
+                        if (c < 2 * FB) s2[kb] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[kb][j], qf[c][j], s2[kb], 0, 0, 0);
+                    }
+                }
+            }
 
-            // lane now holds the scores of query iq against keys s0 + 4g + i
-            bool ok[4];
-            float x[4];
+            // lane holds the scores of query iq against keys s_base + 16kb + 4g + i
+            bool ok[KB][4];
             float mx = -INFINITY;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int s = s0 + 4 * g + i;
-                const int rel = s - iq;
-                ok[i] = qvalid && rel >= -lc_lo && rel < lc_hi && s < len;
-                x[i] = a.temp * s1[i];
-                if (ok[i]) mx = fmaxf(mx, x[i]);
-            }
+            for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int s = s_base + 16 * kb + 4 * g + i;
+                    ok[kb][i] = (unsigned)(s - smin) < span;
+                    mx = fmaxf(mx, ok[kb][i] ? s1[kb][i] : -INFINITY);
+                }
             mx = group_max(mx);
-            if (mx > m_run) {
-                const float alpha = expf(m_run - mx);
-                m_run = mx;
-                ze *= alpha;
+            const float m_new = fmaxf(m_run, mx);
+            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+            m_run = m_new;
+            ze *= alpha;
 #pragma unroll
-                for (int db = 0; db < DB; ++db) oacc[db] *= alpha;
-            }
-            const float beta = expf(lsq + cscale - m_run);   // scale of the overlap term, <= 1
-            floatx4 p;
+            for (int db = 0; db < DB; ++db) oacc[db] *= alpha;
+            const float beta = wc * __builtin_amdgcn_exp2f(c0 - m_run);          // scale of the overlap term, <= 1
+            floatx4 p[KB];
+            float ovs = 0.f;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const float e = ok[i] ? expf(x[i] - m_run) : 0.f;
-                const float ov = ok[i] ? s2[i] : 0.f;
-                ze += e;
-                zp += ov * beta_k;
-                p[i] = e - ov * beta;
-            }
+            for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float e = ok[kb][i] ? __builtin_amdgcn_exp2f(s1[kb][i] - m_run) : 0.f;
+                    const float ov = ok[kb][i] ? s2[kb][i] : 0.f;
+                    ze += e;
+                    ovs += ov;
+                    p[kb][i] = e - ov * beta;
+                }
+            zp += ovs * wc;
             // O^T[d][query] += sum_keys V[key][d] p[key][query]
 #pragma unroll
-            for (int db = 0; db < DB; ++db) {
-                floatx4 va;
+            for (int kb = 0; kb < KB; ++kb) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) va[i] = Vs[(16 * kb + 4 * g + i) * LDV + 16 * db + r16];
-                oacc[db] = Frag<float>::mma(va, p, oacc[db]);
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int db = 0; db < DB; ++db)
+                        oacc[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(
+                            Vs[(16 * kb + 4 * g + i) * LDV + 16 * db + r16], p[kb][i], oacc[db], 0, 0, 0);
             }
         }
+        if (more) {
+            float* nxt = smem + (cur ^ 1) * STAGE;
+            rk.template stash<LDK>(nxt, tid);
+            rv.template stash<LDV>(nxt + TK * LDK, tid);
+            rf.template stash<LDF>(nxt + TK * (LDK + LDV), tid);
+        }
+        cscale = cscale_next;
+        __syncthreads();
     }
 
     // global low-rank term: qkv^T[d][query] = sum_r KV[r][d] q'[query][r],  qk1 = q' . Ksum
-    const float* kvp = a.kv + (long)bh * M * D;
-    const float* ksp = a.ksum + (long)bh * M;
+    // (with several parts only part 0 carries it)
     floatx4 lacc[DB];
 #pragma unroll
     for (int db = 0; db < DB; ++db) lacc[db] = Frag<float>::zero();
     float qk1 = 0.f;
-#pragma unroll
-    for (int c = 0; c < 2 * FB; ++c) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) qk1 += qf[c][j] * ksp[16 * c + 4 * g + j];
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-            floatx4 ka;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) ka[j] = kvp[(16 * c + 4 * g + j) * D + 16 * db + r16];
-            lacc[db] = Frag<float>::mma(ka, qf[c], lacc[db]);
+    if (!SPLIT || part == 0) {                       // workgroup-uniform
+        // K'^T V (M x D) and sum K' (M) staged in LDS: coalesced loads, all in flight together
+        float* KVs = smem;
+        float* KSs = smem + M * LDV;
+        {
+            RowTile<M, D> kvt;
+            kvt.fetch(a.kv + (long)bh * M * D, D, 0, M - 1, tid);
+            if (tid < M) KSs[tid] = a.ksum[(long)bh * M + tid];
+            kvt.template stash<LDV>(KVs, tid);
         }
+        __syncthreads();
+#pragma unroll
+        for (int c = 0; c < 2 * FB; ++c) {
+            const floatx4 ks = *reinterpret_cast<const floatx4*>(KSs + 16 * c + 4 * g);
+            qk1 += qf[c][0] * ks[0] + qf[c][1] * ks[1] + qf[c][2] * ks[2] + qf[c][3] * ks[3];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+                    lacc[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(
+                        KVs[(16 * c + 4 * g + j) * LDV + 16 * db + r16], qf[c][j], lacc[db], 0, 0, 0);
+        }
+        qk1 = group_sum(qk1);
     }
-    qk1 = group_sum(qk1);
     ze = group_sum(ze);
     zp = group_sum(zp);
-    const float gamma = expf(lsq + kmax - m_run);                     // <= 1
-    const float Z = ze + gamma * fmaxf(qk1 - zp, 1e-24f);
-    const float inv = 1.0f / Z;
-    if (qvalid) {
-        T* optr = reinterpret_cast<T*>(a.out) + b * a.o_sb + h * a.o_sh + (long)iq * a.o_ss;
+    const float gamma = __builtin_amdgcn_exp2f(c0 - m_run);               // <= 1
+    if (SPLIT) {
+        // un-normalised partial in this part's own (base-2) exponent m_run
+        float* ws = a.part_ws + (((long)bh * gridDim.x + blockIdx.x) * a.n_parts + part) * (TQ * (D + NSTAT));
+        const int ql = 16 * w + r16;
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
-            floatx4 o = (oacc[db] + gamma * lacc[db]) * inv;
-            store4_f32(optr + 16 * db + 4 * g, o);
+            floatx4 o = oacc[db] + gamma * lacc[db];
+            *reinterpret_cast<floatx4*>(ws + ql * D + 16 * db + 4 * g) = o;
         }
-        if (g == 0) a.log_norm[(long)bh * a.T + iq] = m_run + logf(Z);
+        if (g == 0) {
+            float* st = ws + TQ * D;
+            st[0 * TQ + ql] = m_run;
+            st[1 * TQ + ql] = ze;
+            st[2 * TQ + ql] = zp;
+            st[3 * TQ + ql] = qk1;
+            st[4 * TQ + ql] = c0;
+        }
+    } else {
+        const float Z = ze + gamma * fmaxf(qk1 - zp, 1e-24f);
+        const float inv = 1.0f / Z;
+        if (qvalid) {
+            T* optr = reinterpret_cast<T*>(a.out) + b * a.o_sb + h * a.o_sh + (long)iq * a.o_ss;
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                floatx4 o = (oacc[db] + gamma * lacc[db]) * inv;
+                store4_f32(optr + 16 * db + 4 * g, o);
+            }
+            if (g == 0) a.log_norm[(long)bh * a.T + iq] = m_run * LN2 + __logf(Z);
+        }
     }
+}
+
+// merge of the per-part partials: one thread per (query, four output columns); every load of a
+// thread is independent of the others so they are all in flight together
+template <typename T>
+__global__ __launch_bounds__(NT) void sb_merge_kernel(FwdArgs a, int D) {
+    constexpr float LN2 = 0.6931471805599453f;
+    const int d4 = D / 4;                                  // column groups per query
+    const int gid = blockIdx.x * NT + threadIdx.x;         // over TQ * d4 items of one query tile
+    const int qt = gid / (TQ * d4), rem = gid % (TQ * d4), ql = rem / d4, d = 4 * (rem % d4);
+    const int n_qt = (a.T + TQ - 1) / TQ;
+    if (qt >= n_qt) return;
+    const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
+    const int iq = qt * TQ + ql;
+    if (iq >= a.T) return;
+    const long stride = (long)TQ * (D + NSTAT);
+    const float* ws = a.part_ws + ((long)bh * n_qt + qt) * a.n_parts * stride;
+    const float* st = ws + TQ * D + ql;
+    float m_star = -INFINITY;
+#pragma unroll 8
+    for (int p = 0; p < a.n_parts; ++p) m_star = fmaxf(m_star, st[p * stride]);
+    float ze = 0.f, zp = 0.f;
+    floatx4 acc = Frag<float>::zero();
+#pragma unroll 8
+    for (int p = 0; p < a.n_parts; ++p) {
+        const float wgt = __builtin_amdgcn_exp2f(st[p * stride] - m_star);
+        ze += wgt * st[p * stride + TQ];
+        zp += st[p * stride + 2 * TQ];
+        acc += wgt * *reinterpret_cast<const floatx4*>(ws + p * stride + ql * D + d);
+    }
+    const float Z = ze + __builtin_amdgcn_exp2f(st[4 * TQ] - m_star) * fmaxf(st[3 * TQ] - zp, 1e-24f);
+    T* optr = reinterpret_cast<T*>(a.out) + b * a.o_sb + h * a.o_sh + (long)iq * a.o_ss;
+    store4_f32(optr + d, acc * (1.0f / Z));
+    if (d == 0) a.log_norm[(long)bh * a.T + iq] = m_star * LN2 + __logf(Z);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -425,29 +593,50 @@ template <int E, int M> constexpr size_t kfeat_smem() {
     return sizeof(float) * ((M / 2) * (E + 4) + CH * (E + 4) + CH * (E + 4) + CH * (M + 4) + 8);
 }
 template <int E, int M> constexpr size_t fwd_smem() {
-    return sizeof(float) * (CH * (E + 4) + CH * (E + 4) + CH * (M + 4));
+    constexpr size_t stage = (size_t)TK * ((E + 4) + (E + 4) + (M + 4));
+    constexpr size_t proj = (size_t)(M / 2) * (E + 4);
+    constexpr size_t lowrank = (size_t)M * (E + 4) + M;
+    constexpr size_t need = 2 * stage > proj ? (2 * stage > lowrank ? 2 * stage : lowrank)
+                                             : (proj > lowrank ? proj : lowrank);
+    return sizeof(float) * need;
 }
 
 template <typename T, int E, int M>
 static int launch_kfeat(const KvArgs& a, hipStream_t st) {
     auto kern = sb_kfeat_kernel<T, E, E, M>;
     constexpr size_t smem = kfeat_smem<E, M>();
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) return fail(ERR_LAUNCH, "sb_kfeat: LDS attribute: %s", hipGetErrorString(e));
+    static bool lds_ready = false;     // one instantiation = one kernel; set its LDS limit once
+    if (!lds_ready) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return fail(ERR_LAUNCH, "sb_kfeat: LDS attribute: %s", hipGetErrorString(e));
+        lds_ready = true;
+    }
     hipLaunchKernelGGL(kern, dim3(a.n_split, a.B * a.H), dim3(NT), smem, st, a);
     return check_launch("sb_kfeat_kernel");
 }
 
+template <typename T, int E, int M, bool SPLIT>
+static int launch_fwd_impl(const FwdArgs& a, hipStream_t st) {
+    auto kern = sblocal_fwd_kernel<T, E, E, M, SPLIT>;
+    constexpr size_t smem = fwd_smem<E, M>();
+    static bool lds_ready = false;
+    if (!lds_ready) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return fail(ERR_LAUNCH, "sblocal_fwd: LDS attribute: %s", hipGetErrorString(e));
+        lds_ready = true;
+    }
+    const int qt = (a.T + TQ - 1) / TQ;
+    hipLaunchKernelGGL(kern, dim3(qt, SPLIT ? a.n_parts : 1, a.B * a.H), dim3(NT), smem, st, a);
+    int rc = check_launch("sblocal_fwd_kernel");
+    if (rc || !SPLIT) return rc;
+    hipLaunchKernelGGL(sb_merge_kernel<T>, dim3((qt * TQ * (E / 4) + NT - 1) / NT, a.B * a.H), dim3(NT), 0, st, a, E);
+    return check_launch("sb_merge_kernel");
+}
 template <typename T, int E, int M>
 static int launch_fwd(const FwdArgs& a, hipStream_t st) {
-    auto kern = sblocal_fwd_kernel<T, E, E, M>;
-    constexpr size_t smem = fwd_smem<E, M>();
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) return fail(ERR_LAUNCH, "sblocal_fwd: LDS attribute: %s", hipGetErrorString(e));
-    hipLaunchKernelGGL(kern, dim3((a.T + 63) / 64, a.B * a.H), dim3(NT), smem, st, a);
-    return check_launch("sblocal_fwd_kernel");
+    return a.n_parts > 1 ? launch_fwd_impl<T, E, M, true>(a, st) : launch_fwd_impl<T, E, M, false>(a, st);
 }
 
 #define SB_DISPATCH_M(FN, T, EE, ARGS)                                       \
@@ -477,6 +666,19 @@ static int dispatch_fwd(int dtype, int E, int m, const FwdArgs& a, hipStream_t s
     return fail(ERR_UNSUPPORTED, "sblocal supports float32 and bfloat16, got dtype code %d", dtype);
 }
 
+// number of parts the band of every query tile is split into: enough workgroups for two per CU
+// on small problems, one part (no partials, no merge) once the grid fills the chip by itself
+static int plan_parts(int B, int H, int T, int S, int lc) {
+    const long tiles = (long)B * H * ((T + TQ - 1) / TQ);
+    long band = (long)lc + TQ;
+    if (band > S) band = S;
+    const int key_tiles = (int)((band + TK - 1) / TK);
+    long want = (512 + tiles - 1) / tiles;
+    if (want > 8) want = 8;
+    if (want > key_tiles / 2) want = key_tiles / 2;      // at least two key tiles per part
+    return want < 1 ? 1 : (int)want;
+}
+
 static int plan(int B, int H, int S, int* n_chunks, int* n_split) {
     const int nc = (S + CH - 1) / CH;
     // aim for about 1024 workgroups over the chip, at least one chunk each
@@ -493,8 +695,11 @@ static int plan(int B, int H, int S, int* n_chunks, int* n_split) {
 
 using namespace flyhip;
 
-extern "C" int flyhip_sb_plan(int B, int H, int S, int* n_chunks, int* n_split) {
-    FLY_REQUIRE(B > 0 && H > 0 && S > 0 && n_chunks && n_split, "sb_plan: bad arguments");
+extern "C" int flyhip_sb_plan(int B, int H, int T, int S, int local_context,
+                              int* n_chunks, int* n_split, int* n_parts) {
+    FLY_REQUIRE(B > 0 && H > 0 && T > 0 && S > 0 && local_context > 0 && n_chunks && n_split && n_parts,
+                "sb_plan: bad arguments");
+    *n_parts = plan_parts(B, H, T, S, local_context);
     return plan(B, H, S, n_chunks, n_split);
 }
 
@@ -523,7 +728,8 @@ extern "C" int flyhip_sb_kv_reduce(const void* k, const void* v, const float* pr
     if (rc) return rc;
     int nc, ns;
     plan(B, H, S, &nc, &ns);
-    FLY_REQUIRE(n_split >= 1 && n_split <= nc, "sb_kv_reduce: n_split=%d outside [1, %d]", n_split, nc);
+    FLY_REQUIRE(n_split >= 1 && n_split <= nc && n_split <= MAX_SPLIT,
+                "sb_kv_reduce: n_split=%d outside [1, min(%d, %d)]", n_split, nc, MAX_SPLIT);
     FLY_REQUIRE((long)B * H <= 65535, "sb_kv_reduce: B*H=%ld exceeds the grid limit 65535", (long)B * H);
     KvArgs a{k, v, proj, key_lengths, kfeat, chunk_scale, kv_part, part_max,
              B, H, S, mh_valid, nc, n_split, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, softmax_temp};
@@ -541,6 +747,7 @@ extern "C" int flyhip_sblocal_fwd(const void* q, const void* k, const void* v, c
                                   const float* kfeat, const float* chunk_scale,
                                   const float* kv, const float* ksum, const float* kmax,
                                   const int64_t* key_lengths, void* out, float* log_norm,
+                                  float* part_ws, int n_parts,
                                   int B, int H, int T, int S, int E, int D, int mh, int mh_valid,
                                   int local_context,
                                   int64_t q_sb, int64_t q_sh, int64_t q_ss,
@@ -557,10 +764,12 @@ extern "C" int flyhip_sblocal_fwd(const void* q, const void* k, const void* v, c
                            v_sb | v_sh | v_ss, o_sb | o_sh | o_ss);
     if (rc) return rc;
     FLY_REQUIRE((long)B * H <= 65535, "sblocal_fwd: B*H=%ld exceeds the grid limit 65535", (long)B * H);
+    FLY_REQUIRE(n_parts >= 1 && n_parts <= 64, "sblocal_fwd: n_parts=%d outside [1, 64]", n_parts);
+    FLY_REQUIRE(n_parts == 1 || part_ws, "sblocal_fwd: n_parts > 1 needs the partial workspace");
     int nc, ns;
     plan(B, H, S, &nc, &ns);
-    FwdArgs a{q, k, v, proj, kfeat, chunk_scale, kv, ksum, kmax, key_lengths, out, log_norm,
-              B, H, T, S, mh_valid, local_context, nc,
+    FwdArgs a{q, k, v, proj, kfeat, chunk_scale, kv, ksum, kmax, key_lengths, out, log_norm, part_ws,
+              B, H, T, S, mh_valid, local_context, nc, n_parts,
               q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss, softmax_temp};
     return dispatch_fwd(dtype, E, 2 * mh, a, reinterpret_cast<hipStream_t>(stream));
 }

@@ -37,10 +37,13 @@ class SBLocalPlan:
     out (B,T,H,dim), log_norm (B,H,T) float32.  Buffers of one plan are shared by its runs: runs
     of the same plan on different streams race."""
 
-    def __init__(self, B, H, T, S, dim, mh, mh_valid, dtype, device):
-        n_chunks, n_split = ctypes.c_int(), ctypes.c_int()
-        _lib.call('flyhip_sb_plan', B, H, S, ctypes.byref(n_chunks), ctypes.byref(n_split))
+    def __init__(self, B, H, T, S, dim, mh, mh_valid, dtype, device, local_context, n_parts=None):
+        n_chunks, n_split, parts = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+        _lib.call('flyhip_sb_plan', B, H, T, S, local_context, ctypes.byref(n_chunks), ctypes.byref(n_split),
+                  ctypes.byref(parts))
         self.n_chunks, self.n_split = n_chunks.value, n_split.value
+        self.n_parts = parts.value if n_parts is None else n_parts
+        self.local_context = local_context
         self.shape = (B, H, T, S, dim, mh, mh_valid)
         self.device = torch.device(device)
         self.code = _lib.DTYPE_CODE[dtype]
@@ -52,6 +55,10 @@ class SBLocalPlan:
         self.kv = torch.empty(B, H, m, dim, dtype=f32, device=device)
         self.ksum = torch.empty(B, H, m, dtype=f32, device=device)
         self.kmax = torch.empty(B, H, dtype=f32, device=device)
+        self.part_ws = None
+        if self.n_parts > 1:
+            self.part_ws = torch.empty(B * H * ((T + 63) // 64) * self.n_parts * 64 * (dim + 5), dtype=f32,
+                                       device=device)
 
     def run_keys(self, k, v, proj, lens, t, stream=None):
         B, H, T, S, dim, mh, mh_valid = self.shape
@@ -69,7 +76,7 @@ class SBLocalPlan:
         _lib.call('flyhip_sblocal_fwd', q.data_ptr(), k.data_ptr(), v.data_ptr(), proj.data_ptr(),
                   self.kfeat.data_ptr(), self.chunk_scale.data_ptr(), self.kv.data_ptr(),
                   self.ksum.data_ptr(), self.kmax.data_ptr(), _lib.ptr(lens),
-                  out.data_ptr(), log_norm.data_ptr(),
+                  out.data_ptr(), log_norm.data_ptr(), _lib.ptr(self.part_ws), self.n_parts,
                   B, H, T, S, dim, dim, mh, mh_valid, local_context,
                   q.stride(0), q.stride(2), q.stride(1), k.stride(0), k.stride(2), k.stride(1),
                   v.stride(0), v.stride(2), v.stride(1), out.stride(0), out.stride(2), out.stride(1),
@@ -125,7 +132,7 @@ def sblocal_forward(query, key, value, projection_matrix, local_context, softmax
         if lens.shape != (B,):
             raise ValueError(f'key_lengths must have shape ({B},)')
 
-    plan = SBLocalPlan(B, H, T, S, dim, mh, mh_valid, query.dtype, query.device)
+    plan = SBLocalPlan(B, H, T, S, dim, mh, mh_valid, query.dtype, query.device, local_context)
     out = torch.empty(B, T, H, dim, dtype=query.dtype, device=query.device)
     log_norm = torch.empty(B, H, T, dtype=torch.float32, device=query.device)
     plan.run(q, k, v, proj, lens, local_context, t, out, log_norm)

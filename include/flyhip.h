@@ -29,9 +29,11 @@ const char* flyhip_last_error(void);
  * Scatterbrain-local attention (ref: src/models/attention/sblocal_attention.py:43-137)
  * ---------------------------------------------------------------------------------------- */
 
-/* Sizes of the caller-allocated scratch for one (B,H,S) problem: n_chunks = ceil(S/64) and the
- * number n_split of partial K'^T V reductions per (batch, head). */
-int flyhip_sb_plan(int B, int H, int S, int* n_chunks, int* n_split);
+/* Sizes of the caller-allocated scratch for one problem: n_chunks = ceil(S/64), the number n_split
+ * of partial K'^T V reductions per (batch, head), and the number n_parts of pieces the band of
+ * every 64-query tile is split into by flyhip_sblocal_fwd (1 = no partial workspace needed). */
+int flyhip_sb_plan(int B, int H, int T, int S, int local_context,
+                   int* n_chunks, int* n_split, int* n_parts);
 
 /* Key-side pass.  Replaces feature_map.forward_keys (ref: feature_maps_sb.py:51-82, key branch),
  * the masking of padded keys (sblocal_attention.py:83-85) and the global reductions
@@ -58,11 +60,14 @@ int flyhip_sb_kv_reduce(const void* k, const void* v, const float* proj, const i
  * joint normalisation and local_weighted_average + combine (ref: sblocal_attention.py:78,90-122;
  * fast_transformers.local_product).  Consumes the outputs of flyhip_sb_kv_reduce.
  *   q (B,T,H,E), out (B,T,H,D) via strides; log_norm (B,H,T) fp32 = the reference's
- *   log_normalization; local_context = lc (band -(lc/2) <= s - i < (lc+1)/2). */
+ *   log_normalization; local_context = lc (band -(lc/2) <= s - i < (lc+1)/2).
+ *   n_parts from flyhip_sb_plan (any value in [1,64] is valid); when > 1, part_ws is scratch of
+ *   B*H*ceil(T/64)*n_parts*64*(D+5) floats, else it may be NULL. */
 int flyhip_sblocal_fwd(const void* q, const void* k, const void* v, const float* proj,
                        const float* kfeat, const float* chunk_scale,
                        const float* kv, const float* ksum, const float* kmax,
                        const int64_t* key_lengths, void* out, float* log_norm,
+                       float* part_ws, int n_parts,
                        int B, int H, int T, int S, int E, int D, int mh, int mh_valid,
                        int local_context,
                        int64_t q_sb, int64_t q_sh, int64_t q_ss,
