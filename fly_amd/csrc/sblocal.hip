@@ -28,7 +28,23 @@ constexpr int CH = 64;     // keys per feature chunk (granularity of the key-sid
 constexpr int TK = 32;     // keys per tile of the fused band kernel
 constexpr int TQ = 64;     // queries per workgroup of the fused band kernel
 constexpr int NT = 256;    // threads per workgroup (4 waves)
+constexpr int N_XCD = 8;   // accelerator dies (each with its own L2) the dispatcher cycles over
 constexpr int NSTAT = 5;   // per-query statistics of a partial: m, ze, zp, qk1, lsq+kmax
+
+// Optional phase timestamps of the fused kernel (a development build, -DFLY_PROFILE, reads them
+// back through flyhip_prof_read); compiled out of the shipped library.
+#ifdef FLY_PROFILE
+__device__ long long g_prof[16384 * 8];
+#define FLY_PROF(slot)                                                                                   \
+    do {                                                                                                 \
+        if (threadIdx.x == 0) {                                                                          \
+            const int wg_ = blockIdx.x;                                                                  \
+            if (wg_ < 16384) g_prof[wg_ * 8 + (slot)] = wall_clock64();                                  \
+        }                                                                                                \
+    } while (0)
+#else
+#define FLY_PROF(slot)
+#endif
 
 struct KvArgs {
     const void* k; const void* v; const float* proj; const int64_t* lens;
@@ -280,9 +296,18 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
     float* Ps = smem;                                  // only live before the key loop
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
-    const int bh = blockIdx.z, b = bh / a.H, h = bh % a.H;
-    const int part = blockIdx.y;
-    const int q0 = blockIdx.x * TQ;
+    // Workgroups are handed to the 8 XCDs round-robin in launch order, and every XCD has its own
+    // L2.  The linear id is therefore re-mapped so that one XCD works on a contiguous run of
+    // (batch-head, query tile, part) items: neighbours in that order share key tiles.
+    const int n_qt = (a.T + TQ - 1) / TQ;
+    const int n_items = a.B * a.H * n_qt * a.n_parts;
+    const int per_xcd = (n_items + N_XCD - 1) / N_XCD;
+    const int item = (blockIdx.x % N_XCD) * per_xcd + blockIdx.x / N_XCD;
+    if (item >= n_items) return;                       // workgroup-uniform
+    const int part = item % a.n_parts;
+    const int qt = (item / a.n_parts) % n_qt;
+    const int bh = item / (a.n_parts * n_qt), b = bh / a.H, h = bh % a.H;
+    const int q0 = qt * TQ;
     const int iq = q0 + 16 * w + r16;
     const bool qvalid = iq < a.T;
     const T* qptr = reinterpret_cast<const T*>(a.q) + b * a.q_sb + h * a.q_sh;
@@ -293,6 +318,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
     const float lnm_half = 0.5f * __logf(2.0f * a.mh_valid);
     const int lc_lo = a.lc / 2, lc_hi = (a.lc + 1) / 2;    // band: -lc_lo <= s - i < lc_hi
 
+    FLY_PROF(0);
     // this workgroup's share of the band, in 32-key tiles
     const int q_last = min(q0 + TQ - 1, a.T - 1);
     const int lo = max(0, q0 - lc_lo);
@@ -338,18 +364,24 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
     floatx4 qf[2 * FB];
     float qmax = 0.f;
 #pragma unroll
-    for (int fb = 0; fb < FB; ++fb) {
-        floatx4 dd = Frag<float>::zero();
+    for (int fb = 0; fb < FB; ++fb) qf[fb] = Frag<float>::zero();
 #pragma unroll
-        for (int c = 0; c < EC; ++c) {
-            floatx4 pa = *reinterpret_cast<const floatx4*>(Ps + (16 * fb + r16) * LDK + 16 * c + 4 * g);
-            dd = Frag<float>::mma(pa, qr[c], dd);
-        }
-        qf[fb] = dd;
+    for (int c = 0; c < EC; ++c) {                      // the FB accumulation chains advance together
+        floatx4 pa[FB];
+#pragma unroll
+        for (int fb = 0; fb < FB; ++fb)
+            pa[fb] = *reinterpret_cast<const floatx4*>(Ps + (16 * fb + r16) * LDK + 16 * c + 4 * g);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int fb = 0; fb < FB; ++fb)
+                qf[fb] = __builtin_amdgcn_mfma_f32_16x16x4f32(pa[fb][j], qr[c][j], qf[fb], 0, 0, 0);
+    }
+#pragma unroll
+    for (int fb = 0; fb < FB; ++fb)
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-            if (16 * fb + 4 * g + i < a.mh_valid) qmax = fmaxf(qmax, fabsf(dd[i]));
-    }
+            if (16 * fb + 4 * g + i < a.mh_valid) qmax = fmaxf(qmax, fabsf(qf[fb][i]));
     qmax = group_max(qmax);
     const float lsq = -diag_q + qmax - lnm_half;
 #pragma unroll
@@ -363,6 +395,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
         }
     }
     __syncthreads();                 // Ps is dead; the tile buffers may overwrite it
+    FLY_PROF(1);
 
     // From here on all exponents are base 2 (one v_exp_f32 each): scores carry t*log2(e) through
     // the query operand, the log-scales are converted once.
@@ -388,6 +421,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
     }
     __syncthreads();
 
+    FLY_PROF(2);
     for (int kt = kt_lo; kt < kt_hi; ++kt) {
         const int s_base = kt * TK;
         const int cur = (kt - kt_lo) & 1;
@@ -446,12 +480,14 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
                     mx = fmaxf(mx, ok[kb][i] ? s1[kb][i] : -INFINITY);
                 }
             mx = group_max(mx);
-            const float m_new = fmaxf(m_run, mx);
-            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-            m_run = m_new;
-            ze *= alpha;
+            if (__builtin_amdgcn_ballot_w64(mx > m_run) != 0) {      // wave-uniform: some row maximum grew
+                const float m_new = fmaxf(m_run, mx);
+                const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+                m_run = m_new;
+                ze *= alpha;
 #pragma unroll
-            for (int db = 0; db < DB; ++db) oacc[db] *= alpha;
+                for (int db = 0; db < DB; ++db) oacc[db] *= alpha;
+            }
             const float beta = wc * __builtin_amdgcn_exp2f(c0 - m_run);          // scale of the overlap term, <= 1
             floatx4 p[KB];
             float ovs = 0.f;
@@ -487,6 +523,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
         __syncthreads();
     }
 
+    FLY_PROF(3);
     // global low-rank term: qkv^T[d][query] = sum_r KV[r][d] q'[query][r],  qk1 = q' . Ksum
     // (with several parts only part 0 carries it)
     floatx4 lacc[DB];
@@ -519,10 +556,11 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
     }
     ze = group_sum(ze);
     zp = group_sum(zp);
+    FLY_PROF(4);
     const float gamma = __builtin_amdgcn_exp2f(c0 - m_run);               // <= 1
     if (SPLIT) {
         // un-normalised partial in this part's own (base-2) exponent m_run
-        float* ws = a.part_ws + (((long)bh * gridDim.x + blockIdx.x) * a.n_parts + part) * (TQ * (D + NSTAT));
+        float* ws = a.part_ws + (((long)bh * n_qt + qt) * a.n_parts + part) * (TQ * (D + NSTAT));
         const int ql = 16 * w + r16;
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
@@ -550,6 +588,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
             if (g == 0) a.log_norm[(long)bh * a.T + iq] = m_run * LN2 + __logf(Z);
         }
     }
+    FLY_PROF(5);
 }
 
 // merge of the per-part partials: one thread per (query, four output columns); every load of a
@@ -628,7 +667,10 @@ static int launch_fwd_impl(const FwdArgs& a, hipStream_t st) {
         lds_ready = true;
     }
     const int qt = (a.T + TQ - 1) / TQ;
-    hipLaunchKernelGGL(kern, dim3(qt, SPLIT ? a.n_parts : 1, a.B * a.H), dim3(NT), smem, st, a);
+    const long items = (long)a.B * a.H * qt * a.n_parts;
+    const long grid = (items + N_XCD - 1) / N_XCD * N_XCD;       // whole rounds over the XCDs
+    if (grid > 2147483647L) return fail(ERR_ARG, "sblocal_fwd: too many workgroups");
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NT), smem, st, a);
     int rc = check_launch("sblocal_fwd_kernel");
     if (rc || !SPLIT) return rc;
     hipLaunchKernelGGL(sb_merge_kernel<T>, dim3((qt * TQ * (E / 4) + NT - 1) / NT, a.B * a.H), dim3(NT), 0, st, a, E);
@@ -673,7 +715,7 @@ static int plan_parts(int B, int H, int T, int S, int lc) {
     long band = (long)lc + TQ;
     if (band > S) band = S;
     const int key_tiles = (int)((band + TK - 1) / TK);
-    long want = (512 + tiles - 1) / tiles;
+    long want = 512 / tiles;                             // never more than two workgroups per CU
     if (want > 8) want = 8;
     if (want > key_tiles / 2) want = key_tiles / 2;      // at least two key tiles per part
     return want < 1 ? 1 : (int)want;
@@ -694,6 +736,14 @@ static int plan(int B, int H, int S, int* n_chunks, int* n_split) {
 }  // namespace flyhip
 
 using namespace flyhip;
+
+#ifdef FLY_PROFILE
+extern "C" int flyhip_prof_read(long long* dst, int n_workgroups) {
+    hipDeviceSynchronize();
+    hipError_t e = hipMemcpyFromSymbol(dst, HIP_SYMBOL(g_prof), sizeof(long long) * 8 * n_workgroups);
+    return e == hipSuccess ? 0 : -1;
+}
+#endif
 
 extern "C" int flyhip_sb_plan(int B, int H, int T, int S, int local_context,
                               int* n_chunks, int* n_split, int* n_parts) {
