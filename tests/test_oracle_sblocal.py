@@ -1,0 +1,166 @@
+"""Pins the Scatterbrain-local oracle (oracle/sblocal.py) with checks that do not retype its
+formulas: brute-force loops, an independent float64 closed form, and invariants.  CPU only."""
+import math
+
+import pytest
+import torch
+
+from oracle import sblocal as osb
+
+
+def _inputs(B, T, S, H, E, D, mh, seed, scale=None):
+    g = torch.Generator().manual_seed(seed)
+    scale = E ** -0.25 if scale is None else scale
+    q = torch.randn(B, T, H, E, generator=g, dtype=torch.float64) * scale
+    k = torch.randn(B, S, H, E, generator=g, dtype=torch.float64) * scale
+    v = torch.randn(B, S, H, D, generator=g, dtype=torch.float64)
+    P = osb.gaussian_orthogonal_random_matrix(mh, E, generator=g, dtype=torch.float64)
+    return q, k, v, P
+
+
+@pytest.mark.parametrize('nrows,ncols', [(64, 64), (128, 64), (36, 21), (13, 21)])
+def test_projection_blocks_are_scaled_orthogonal(nrows, ncols):
+    g = torch.Generator().manual_seed(1)
+    P = osb.gaussian_orthogonal_random_matrix(nrows, ncols, generator=g, dtype=torch.float64)
+    assert P.shape == (nrows, ncols)
+    unit = P / P.norm(dim=1, keepdim=True)
+    for r0 in range(0, nrows, ncols):                      # rows of one QR block are orthonormal
+        blk = unit[r0:r0 + ncols]
+        assert torch.allclose(blk @ blk.t(), torch.eye(blk.shape[0], dtype=torch.float64), atol=1e-10)
+    # row norms follow chi(ncols): mean ~ sqrt(ncols - 1/2)
+    assert abs(P.norm(dim=1).mean() - math.sqrt(ncols - 0.5)) < 0.25 * math.sqrt(ncols)
+    P1 = osb.gaussian_orthogonal_random_matrix(nrows, ncols, scaling=1, generator=g, dtype=torch.float64)
+    assert torch.allclose(P1.norm(dim=1), torch.full((nrows,), math.sqrt(ncols), dtype=torch.float64))
+    with pytest.raises(ValueError):
+        osb.gaussian_orthogonal_random_matrix(4, 4, scaling=2)
+
+
+@pytest.mark.parametrize('t', [None, 1.0, 0.235])
+def test_feature_map_closed_form(t):
+    """feat_q . feat_k * exp(ls_q + ls_k) must equal the un-stabilised positive random feature
+    product (1/m) sum_r [e^{w_r.(q~+k~)} + e^{-w_r.(q~+k~)}] e^{-(|q~|^2+|k~|^2)/2}, x~ = sqrt(t) x,
+    evaluated here with explicit Python loops."""
+    q, k, _, P = _inputs(1, 5, 6, 1, 7, 3, 4, seed=3, scale=0.7)
+    temp = t if t is not None else 1 / math.sqrt(7)
+    fq, lq = osb.softmax_kernel(q[0, :, 0], P, True, softmax_temp=t)
+    fk, lk = osb.softmax_kernel(k[0, :, 0], P, False, softmax_temp=t)
+    assert fq.shape == (5, 8) and fk.shape == (6, 8) and lq.shape == (5, 1) and lk.shape == (1, 1)
+    assert float(fq.max()) <= 1.0 + 1e-12 and float(fk.max()) <= 1.0 + 1e-12     # stabilised
+    m = 8
+    for i in range(5):
+        for j in range(6):
+            qt, kt = math.sqrt(temp) * q[0, i, 0], math.sqrt(temp) * k[0, j, 0]
+            acc = 0.0
+            for r in range(4):
+                z = float(P[r] @ (qt + kt))
+                acc += math.exp(z) + math.exp(-z)
+            want = acc / m * math.exp(-0.5 * float(qt @ qt + kt @ kt))
+            got = float(fq[i] @ fk[j]) * math.exp(float(lq[i]) + float(lk))
+            assert got == pytest.approx(want, rel=1e-10)
+
+
+def test_feature_map_is_unbiased_for_exp_kernel():
+    """E[phi(q).phi(k)] = exp(t q.k): with 30000 features the relative error is small
+    (cf. tests/models/attention/test_sblocal_attention.py:90-97 of the reference)."""
+    q, k, _, _ = _inputs(1, 8, 8, 1, 16, 4, 2, seed=5)
+    g = torch.Generator().manual_seed(0)
+    P = osb.gaussian_orthogonal_random_matrix(15000, 16, generator=g, dtype=torch.float64)
+    fq, lq = osb.softmax_kernel(q[0, :, 0], P, True)
+    fk, lk = osb.softmax_kernel(k[0, :, 0], P, False)
+    est = (fq @ fk.t()) * torch.exp(lq + lk)
+    exact = torch.exp((q[0, :, 0] @ k[0, :, 0].t()) / 4.0)
+    assert ((est - exact) / exact).abs().mean() < 0.05
+
+
+@pytest.mark.parametrize('lc', [1, 3, 4, 7, 28, 200])
+def test_local_products_against_loops(lc):
+    g = torch.Generator().manual_seed(lc)
+    B, H, T, S, E, D = 2, 2, 11, 9, 5, 3
+    Q = torch.randn(B, H, T, E, generator=g, dtype=torch.float64)
+    K = torch.randn(B, H, S, E, generator=g, dtype=torch.float64)
+    V = torch.randn(B, H, S, D, generator=g, dtype=torch.float64)
+    lens = torch.tensor([9, 4])
+    got = osb.local_dot_product(Q, K, None, lens, lc, chunk=4)
+    want = torch.full((B, H, T, lc), -1e24, dtype=torch.float64)
+    for b in range(B):
+        for h in range(H):
+            for i in range(T):
+                for j in range(lc):
+                    s = i - lc // 2 + j
+                    if 0 <= s < int(lens[b]):
+                        want[b, h, i, j] = Q[b, h, i] @ K[b, h, s]
+    assert torch.allclose(got, want, rtol=1e-12, atol=1e-12)
+    A = torch.randn(B, H, T, lc, generator=g, dtype=torch.float64)
+    got = osb.local_weighted_average(A, V, chunk=4)
+    want = torch.zeros(B, H, T, D, dtype=torch.float64)
+    for b in range(B):
+        for h in range(H):
+            for i in range(T):
+                for j in range(lc):
+                    s = i - lc // 2 + j
+                    if 0 <= s < S:
+                        want[b, h, i] += A[b, h, i, j] * V[b, h, s]
+    assert torch.allclose(got, want, rtol=1e-12, atol=1e-12)
+
+
+def test_band_definition_even_and_odd_windows():
+    """Even lc: [i - lc/2, i + lc/2); odd lc: symmetric (test_sblocal_attention.py:77-82)."""
+    Q = torch.eye(6, dtype=torch.float64).view(1, 1, 6, 6)
+    K = torch.eye(6, dtype=torch.float64).view(1, 1, 6, 6)
+    lens = torch.tensor([6])
+    d4 = osb.local_dot_product(Q, K, None, lens, 4)[0, 0]
+    # query 3 sees keys 1,2,3,4 in slots 0..3; the self product (=1) sits in slot lc//2 = 2
+    assert d4[3].tolist() == [0.0, 0.0, 1.0, 0.0]
+    assert d4[0].tolist() == [-1e24, -1e24, 1.0, 0.0]          # keys -2, -1 do not exist
+    assert d4[5].tolist() == [0.0, 0.0, 1.0, -1e24]            # key 6 does not exist
+    d3 = osb.local_dot_product(Q, K, None, lens, 3)[0, 0]
+    assert d3[3].tolist() == [0.0, 1.0, 0.0]                   # keys 2,3,4
+    assert d3[5].tolist() == [0.0, 1.0, -1e24]
+
+
+@pytest.mark.parametrize('lc,mh,t,lens', [
+    (3, 36, None, None), (4, 13, 1.0, [39, 12, 20]), (28, 36, 0.235, [10, 39, 25]), (33, 13, None, [39, 9, 30]),
+    (512, 8, None, None)])
+def test_forward_matches_dense_closed_form(lc, mh, t, lens):
+    """The reference op sequence (band-packed tensors, stabilisers, overlap subtraction) against the
+    estimator written directly as a dense (T,S) matrix in float64."""
+    q, k, v, P = _inputs(3, 47, 39, 2, 21, 17, mh, seed=2357, scale=0.6)
+    lens = None if lens is None else torch.tensor(lens)
+    out, ln = osb.sblocal_attention(q, k, v, P, lc, softmax_temp=t, key_lengths=lens)
+    out2, ln2, A = osb.dense_closed_form(q, k, v, P, lc, softmax_temp=t, key_lengths=lens)
+    assert out.shape == (3, 47, 2, 17) and ln.shape == (3, 2, 47, 1)
+    assert torch.allclose(out, out2, rtol=1e-9, atol=1e-11)
+    assert torch.allclose(ln, ln2, rtol=1e-9, atol=1e-11)
+    # invariants of the reference's test: non-negative weights, exact values on the band
+    assert bool((A >= 0).all())
+    temp = t or 1 / math.sqrt(21)
+    exact = torch.exp(temp * torch.einsum('bthe,bshe->bhts', q, k))
+    i = torch.arange(47).view(47, 1)
+    j = torch.arange(39).view(1, 39)
+    band = ((j - i) >= -(lc // 2)) & ((j - i) < (lc + 1) // 2)
+    if lens is not None:
+        band = band.view(1, 1, 47, 39) & (j.view(1, 1, 1, 39) < lens.view(3, 1, 1, 1))
+    else:
+        band = band.view(1, 1, 47, 39).expand(3, 2, 47, 39)
+    band = band.expand(3, 2, 47, 39)
+    assert torch.allclose(A[band], exact[band], rtol=1e-12)
+
+
+def test_value_of_ones_gives_ones_and_wide_band_is_full_attention():
+    q, k, v, P = _inputs(2, 40, 40, 2, 16, 8, 6, seed=11)
+    out, _ = osb.sblocal_attention(q, k, torch.ones_like(v), P, 9, key_lengths=torch.tensor([40, 17]))
+    assert torch.allclose(out, torch.ones_like(out), atol=1e-12)
+    out, ln = osb.sblocal_attention(q, k, v, P, 200)
+    att = torch.softmax(torch.einsum('bthe,bshe->bhts', q, k) / 4.0, dim=-1)
+    full = torch.einsum('bhts,bshd->bthd', att, v)
+    assert torch.allclose(out, full, atol=1e-10)
+    lse = torch.logsumexp(torch.einsum('bthe,bshe->bhts', q, k) / 4.0, dim=-1, keepdim=True)
+    assert torch.allclose(ln, lse, atol=1e-10)
+
+
+def test_float32_oracle_is_close_to_float64():
+    q, k, v, P = _inputs(2, 300, 300, 1, 64, 64, 64, seed=0)
+    o64, l64 = osb.sblocal_attention(q, k, v, P, 128)
+    o32, l32 = osb.sblocal_attention(q.float(), k.float(), v.float(), P.float(), 128)
+    assert float((o32.double() - o64).abs().max() / o64.abs().max()) < 1e-5
+    assert float((l32.double() - l64).abs().max() / l64.abs().max()) < 1e-5
