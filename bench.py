@@ -40,7 +40,7 @@ def sblocal_flops(B, H, T, S, E, D, m, lc):
     return total, fused
 
 
-def bench_sblocal(steps, warmup):
+def bench_sblocal(steps, warmup, cpu_baseline=True):
     from fly_amd.sblocal_attention import SBLocalPlan
     from oracle import sblocal as osb
     dev = torch.device('cuda:0')
@@ -89,7 +89,11 @@ def bench_sblocal(steps, warmup):
         'flops_per_step': total_flops,
     }
 
-    # CPU baseline: the oracle (a port of the reference op sequence) on the host cores, bounded
+    if not cpu_baseline:
+        res['cpu_baseline'] = None
+        return res
+    # CPU baseline: the oracle (a port of the reference op sequence) on the host cores, bounded to
+    # about 12 s of work
     torch.set_num_threads(min(os.cpu_count() or 1, 16))
     osb.sblocal_attention(q, k, v, P, lc)
     n, t0 = 0, time.perf_counter()
@@ -97,7 +101,7 @@ def bench_sblocal(steps, warmup):
         osb.sblocal_attention(q, k, v, P, lc)
         n += 1
         el = time.perf_counter() - t0
-        if el > 10.0 or n >= 200:
+        if el > 12.0:
             break
     res['cpu_baseline'] = {'value': B * L * n / el, 'unit': 'tokens/s', 'cores': torch.get_num_threads(),
                            'kind': 'port',
@@ -156,7 +160,11 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=200)
     ap.add_argument('--warmup', type=int, default=20)
-    ap.add_argument('--no-blocksparse', action='store_true')
+    ap.add_argument('--no-blocksparse', action='store_true', help='skip the config 2 stages')
+    ap.add_argument('--skip-cpu', action='store_true', help='skip the CPU baseline leg (profiling runs)')
+    ap.add_argument('--copy-calibration', action='store_true',
+                    help='also run a plain 256 MiB device copy: its FETCH_SIZE / WRITE_SIZE readings '
+                         'give the scale of the traffic counters')
     args = ap.parse_args()
     if args.gpus != 1:
         print('bench.py: this build measures one GPU; --gpus must be 1 (nothing here shards over devices)',
@@ -165,7 +173,13 @@ def main():
     if not torch.cuda.is_available():
         print('bench.py: no GPU visible', file=sys.stderr)
         sys.exit(1)
-    sb = bench_sblocal(args.steps, args.warmup)
+    if args.copy_calibration:
+        src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device='cuda:0').normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+    sb = bench_sblocal(args.steps, args.warmup, cpu_baseline=not args.skip_cpu)
     line = {
         'metric': 'SBLocal attention forward tokens/s (fp32, L=3136, d=64)',
         'value': sb['tokens_per_s'], 'unit': 'tokens/s', 'n_gpus': 1, 'steps': args.steps,
@@ -174,7 +188,7 @@ def main():
         'config': {'workload': 'BASELINE config 1 (configs[0]): SBLocal fwd fp32 B=2 H=1 L=3136 d=64 '
                                'local_context=512 nb_features=128, seeded orthogonal-Gaussian projection'},
         'roofline': sb['roofline'], 'cpu_baseline': sb['cpu_baseline'],
-        'gpu_over_cpu': sb['tokens_per_s'] / sb['cpu_baseline']['value'],
+        'gpu_over_cpu': sb['tokens_per_s'] / sb['cpu_baseline']['value'] if sb['cpu_baseline'] else None,
         'parity': sb['parity'],
     }
     if not args.no_blocksparse:

@@ -161,12 +161,14 @@ class matmul:
             raise ValueError(f'SDD operands {tuple(a.shape)}, {tuple(b.shape)} do not match layout '
                              f'{tuple(self.spdims)} with block {self.block}')
         (lut,) = self._table('sdd', a.device)
+        row_ptr, row_blk, row_col = self._table('rows', a.device)
         nnz = lut.shape[0]
         c = torch.empty((Z, nnz, self.block, self.block), dtype=a.dtype, device=a.device)
         a_sm, a_sk = (a.stride(3), a.stride(2)) if trans_a else (a.stride(2), a.stride(3))
         b_sn, b_sk = (b.stride(2), b.stride(3)) if trans_b else (b.stride(3), b.stride(2))
         with torch.cuda.device(a.device):
             _lib.call('flyhip_bs_sdd', a.data_ptr(), b.data_ptr(), c.data_ptr(), lut.data_ptr(), nnz,
+                      row_ptr.data_ptr(), row_blk.data_ptr(), row_col.data_ptr(), H * p, p,
                       Z, K, self.block, a.stride(0), a.stride(1), a_sm, a_sk,
                       b.stride(0), b.stride(1), b_sn, b_sk, _lib.dtype_code(a), _lib.stream_ptr(a.device))
         return c

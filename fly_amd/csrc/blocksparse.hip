@@ -77,6 +77,57 @@ __global__ __launch_bounds__(256) void bs_sdd_kernel(SddArgs a) {
             store4_f32(cp + (ml + 16 * tm + r16) * BLK + nl + 16 * tn + 4 * g, acc[tm][tn]);
 }
 
+// Fast SDD for 32x32 blocks of a 2-byte type with contiguous contraction (K a multiple of 32, at
+// most 128): one workgroup per (head, block-row).  Every wave loads the A fragments of the block-row
+// once (16-byte loads, kept in registers) and then produces the row's blocks w, w+4, ... one after
+// the other: B fragments with 16-byte loads, 16x16x32 MFMAs, 8-byte stores of a 2 KiB block.
+struct SddRowArgs {
+    const void* a; const void* b; void* c;
+    const int32_t* row_ptr; const int32_t* row_blk; const int32_t* row_col;
+    int nnz, K, brows_per_head;
+    long a_sz, a_sh, a_sm, b_sz, b_sh, b_sn;
+};
+
+template <typename T, int KS>     // KS = K / 32
+__global__ __launch_bounds__(256) void bs_sdd32_kernel(SddRowArgs a) {
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, r16 = lane & 15, g = lane >> 4;
+    const int brow = blockIdx.x, z = blockIdx.y;
+    const int head = brow / a.brows_per_head, bi = brow % a.brows_per_head;
+    const int p0 = a.row_ptr[brow], nb = a.row_ptr[brow + 1] - p0;
+    const T* ap = reinterpret_cast<const T*>(a.a) + z * a.a_sz + head * a.a_sh + (long)(bi * 32 + r16) * a.a_sm + 8 * g;
+    const T* bp = reinterpret_cast<const T*>(a.b) + z * a.b_sz + head * a.b_sh + (long)r16 * a.b_sn + 8 * g;
+    T* cz = reinterpret_cast<T*>(a.c) + (long)z * a.nnz * 1024;
+    uint4 fa[2][KS];
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) fa[tm][ks] = *reinterpret_cast<const uint4*>(ap + 16 * tm * a.a_sm + 32 * ks);
+    for (int j = w; j < nb; j += 4) {
+        const long brow_b = (long)a.row_col[p0 + j] * 32;
+        uint4 fb[2][KS];
+#pragma unroll
+        for (int tn = 0; tn < 2; ++tn)
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+                fb[tn][ks] = *reinterpret_cast<const uint4*>(bp + (brow_b + 16 * tn) * a.b_sn + 32 * ks);
+        floatx4 acc[2][2];
+#pragma unroll
+        for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+            for (int tn = 0; tn < 2; ++tn) {
+                acc[tm][tn] = Frag<float>::zero();
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) acc[tm][tn] = Frag32<T>::mma(fb[tn][ks], fa[tm][ks], acc[tm][tn]);
+            }
+        // lane holds C[m = 16tm + r16][n = 16tn + 4g + i]
+        T* cp = cz + (long)a.row_blk[p0 + j] * 1024;
+#pragma unroll
+        for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+            for (int tn = 0; tn < 2; ++tn) store4_f32(cp + (16 * tm + r16) * 32 + 16 * tn + 4 * g, acc[tm][tn]);
+    }
+}
+
 // ---------------------------------------------------------------------------------------
 // DSD: dense = sparse x dense
 // ---------------------------------------------------------------------------------------
@@ -147,6 +198,90 @@ __global__ __launch_bounds__(256) void bs_dsd_kernel(DxdArgs a) {
             const int n = n0 + 16 * tn + 4 * g;
             if (n < a.X) store_tile_row<T>(cp + m * a.c_sm + n * a.c_sn, a.c_sn, acc[tm][tn], a.X - n);
         }
+    }
+}
+
+// Fast DSD for 32x32 blocks of a 2-byte type, dense operand with contiguous columns (the V of
+// attention): one workgroup per (head, block-row, 64-column tile).  Wave w reduces the row's blocks
+// w, w+4, ...: the sparse block supplies k-contiguous fragments straight from global memory; the
+// 32 x 64 tile of the dense operand is staged in a wave-private LDS buffer (16-byte global loads)
+// and read back column-wise, which is the transposition a [k][n] operand needs.  The four partial
+// sums meet in LDS and leave as 16-byte stores.
+constexpr int DSD_LD = 68;      // LDS row stride in elements: the four k-groups of a read hit distinct banks
+
+template <typename T>
+__global__ __launch_bounds__(256) void bs_dsd32_kernel(DxdArgs a) {
+    __shared__ __attribute__((aligned(16))) uint16_t vt[4][32 * DSD_LD];
+    __shared__ float part[4][32][64 + 1];
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
+    const int seg = blockIdx.x, n0 = blockIdx.y * 64, z = blockIdx.z;
+    const int head = seg / a.per_head, brow = seg % a.per_head;
+    const T* spz = reinterpret_cast<const T*>(a.sp) + z * a.sp_sz;
+    const T* dnp = reinterpret_cast<const T*>(a.dn) + z * a.dn_sz + head * a.dn_sh;
+    const int ncols = min(64, a.X - n0);            // valid columns of this tile (a multiple of 8)
+
+    floatx4 acc[2][4];
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < 4; ++tn) acc[tm][tn] = Frag<float>::zero();
+    uint16_t* my = vt[w];
+    const int p1 = a.seg_ptr[seg + 1];
+    for (int p = a.seg_ptr[seg] + w; p < p1; p += 4) {
+        const T* blkp = spz + (long)a.seg_blk[p] * 1024;
+        const long krow0 = (long)a.seg_inner[p] * 32;
+        // dense tile rows krow0..+31, columns n0..n0+63 -> LDS (lane: row 8*it + lane/8, 8 columns)
+        uint4 stage[4];
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            const int k = 8 * it + (lane >> 3), c8 = 8 * (lane & 7);
+            stage[it] = make_uint4(0, 0, 0, 0);
+            if (c8 < ncols) stage[it] = *reinterpret_cast<const uint4*>(dnp + (krow0 + k) * a.dn_s0 + n0 + c8);
+        }
+        uint4 fs[2];
+#pragma unroll
+        for (int tm = 0; tm < 2; ++tm) fs[tm] = *reinterpret_cast<const uint4*>(blkp + (16 * tm + r16) * 32 + 8 * g);
+        __builtin_amdgcn_wave_barrier();            // previous iteration's LDS reads are done (in-order DS)
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            const int k = 8 * it + (lane >> 3), c8 = 8 * (lane & 7);
+            uint2* dst = reinterpret_cast<uint2*>(my + k * DSD_LD + c8);
+            dst[0] = make_uint2(stage[it].x, stage[it].y);
+            dst[1] = make_uint2(stage[it].z, stage[it].w);
+        }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int tn = 0; tn < 4; ++tn) {
+            // column n = 16tn + r16 of the tile, rows k = 8g..8g+7
+            const uint16_t* src = my + (8 * g) * DSD_LD + 16 * tn + r16;
+            uint4 fd;
+            fd.x = (uint32_t)src[0] | ((uint32_t)src[DSD_LD] << 16);
+            fd.y = (uint32_t)src[2 * DSD_LD] | ((uint32_t)src[3 * DSD_LD] << 16);
+            fd.z = (uint32_t)src[4 * DSD_LD] | ((uint32_t)src[5 * DSD_LD] << 16);
+            fd.w = (uint32_t)src[6 * DSD_LD] | ((uint32_t)src[7 * DSD_LD] << 16);
+            acc[0][tn] = Frag32<T>::mma(fd, fs[0], acc[0][tn]);
+            acc[1][tn] = Frag32<T>::mma(fd, fs[1], acc[1][tn]);
+        }
+    }
+    // lane holds C[m = 16tm + r16][n = 16tn + 4g + i]; sum the four waves
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < 4; ++tn)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) part[w][16 * tm + r16][16 * tn + 4 * g + i] = acc[tm][tn][i];
+    __syncthreads();
+    const int m = tid >> 3, c8 = 8 * (tid & 7);
+    if (c8 < ncols) {
+        floatx4 lo, hi;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            lo[i] = (part[0][m][c8 + i] + part[1][m][c8 + i]) + (part[2][m][c8 + i] + part[3][m][c8 + i]);
+            hi[i] = (part[0][m][c8 + 4 + i] + part[1][m][c8 + 4 + i]) + (part[2][m][c8 + 4 + i] + part[3][m][c8 + 4 + i]);
+        }
+        T* cp = reinterpret_cast<T*>(a.c) + z * a.c_sz + head * a.c_sh + ((long)brow * 32 + m) * a.c_sm + n0 + c8;
+        store4_f32(cp, lo);
+        store4_f32(cp + 4, hi);
     }
 }
 
@@ -291,6 +426,85 @@ __global__ __launch_bounds__(256) void bs_softmax_kernel(RowArgs a) {
     }
 }
 
+// Fast path for 32x32 blocks of a 2-byte type: one workgroup per (block-row, 16-row half).  The
+// 16 x 32 half of a block is 1 KiB of contiguous memory, which one wave moves with a single 16-byte
+// load per lane (lane = 4*row + chunk of 8 columns); wave w owns blocks w, w+4, ... of the row and
+// keeps them in registers (raw 2-byte form) across the max / sum / write passes, so HBM sees each
+// element once in and once out.  Row statistics go quad -> wave (DPP) -> workgroup (LDS).
+template <typename T, int MAXB>
+__global__ __launch_bounds__(256) void bs_softmax32_kernel(RowArgs a) {
+    constexpr float LOG2E = 1.4426950408889634f;
+    __shared__ float red[2][4][16];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, rl = lane >> 2, chunk = lane & 3;
+    const int brow = blockIdx.x >> 1, row = (blockIdx.x & 1) * 16 + rl;       // row inside the block
+    const int z = blockIdx.y;
+    const int p0 = a.row_ptr[brow], nb = a.row_ptr[brow + 1] - p0;
+    const int grow = (brow % a.brows_per_head) * 32 + row;
+    T* xz = reinterpret_cast<T*>(a.x) + z * a.x_sz + row * 32 + chunk * 8;
+    const bool masked = a.kpm || a.am;
+
+    uint4 raw[MAXB];
+    long off[MAXB];
+#pragma unroll
+    for (int it = 0; it < MAXB; ++it) {
+        const int j = w + 4 * it;
+        off[it] = -1;
+        if (j < nb) {
+            off[it] = (long)a.row_blk[p0 + j] * 1024;
+            raw[it] = *reinterpret_cast<const uint4*>(xz + off[it]);
+        }
+    }
+    // element u (0..7) of block slot `it`, scaled and masked
+    auto value = [&](int it, int u) -> float {
+        const uint32_t word = (&raw[it].x)[u >> 1];
+        T e;
+        *reinterpret_cast<uint16_t*>(&e) = (u & 1) ? (uint16_t)(word >> 16) : (uint16_t)(word & 0xffffu);
+        float v = Elem<T>::to_f32(e) * a.scale;
+        if (masked) {
+            const long col = (long)a.row_col[p0 + w + 4 * it] * 32 + chunk * 8 + u;
+            if (a.kpm) v += mask_term(a.kpm[z * a.kpm_stride + col], a.kpm_mul);
+            if (a.am) v += mask_term(a.am[grow * a.am_stride + col], a.am_mul);
+        }
+        return v;
+    };
+    float mx = -INFINITY;
+#pragma unroll
+    for (int it = 0; it < MAXB; ++it)
+        if (off[it] >= 0)
+#pragma unroll
+            for (int u = 0; u < 8; ++u) mx = fmaxf(mx, value(it, u));
+    mx = fmaxf(mx, __shfl_xor(mx, 1));
+    mx = fmaxf(mx, __shfl_xor(mx, 2));
+    if (chunk == 0) red[0][w][rl] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(red[0][0][rl], red[0][1][rl]), fmaxf(red[0][2][rl], red[0][3][rl]));
+    const float mx2 = mx * LOG2E;
+    float sum = 0.f;
+#pragma unroll
+    for (int it = 0; it < MAXB; ++it)
+        if (off[it] >= 0)
+#pragma unroll
+            for (int u = 0; u < 8; ++u) sum += __builtin_amdgcn_exp2f(value(it, u) * LOG2E - mx2);   // -inf - -inf = NaN, kept
+    sum += __shfl_xor(sum, 1);
+    sum += __shfl_xor(sum, 2);
+    if (chunk == 0) red[1][w][rl] = sum;
+    __syncthreads();
+    sum = (red[1][0][rl] + red[1][1][rl]) + (red[1][2][rl] + red[1][3][rl]);
+    const float inv = 1.0f / sum;
+#pragma unroll
+    for (int it = 0; it < MAXB; ++it)
+        if (off[it] >= 0) {
+            uint32_t outw[4];
+#pragma unroll
+            for (int u2 = 0; u2 < 4; ++u2) {
+                T lo = Elem<T>::from_f32(__builtin_amdgcn_exp2f(value(it, 2 * u2) * LOG2E - mx2) * inv);
+                T hi = Elem<T>::from_f32(__builtin_amdgcn_exp2f(value(it, 2 * u2 + 1) * LOG2E - mx2) * inv);
+                outw[u2] = (uint32_t)*reinterpret_cast<uint16_t*>(&lo) | ((uint32_t)*reinterpret_cast<uint16_t*>(&hi) << 16);
+            }
+            *reinterpret_cast<uint4*>(xz + off[it]) = make_uint4(outw[0], outw[1], outw[2], outw[3]);
+        }
+}
+
 // rows longer than the register budget: three passes over the row
 template <typename T>
 __global__ __launch_bounds__(256) void bs_softmax_long_kernel(RowArgs a) {
@@ -387,6 +601,8 @@ static int check_common(const char* who, int blk, int dtype, int Z) {
 }
 
 extern "C" int flyhip_bs_sdd(const void* a, const void* b, void* c, const int32_t* lut, int nnz,
+                             const int32_t* row_ptr, const int32_t* row_blk, const int32_t* row_col,
+                             int n_brow, int brows_per_head,
                              int Z, int K, int blk,
                              int64_t a_sz, int64_t a_sh, int64_t a_sm, int64_t a_sk,
                              int64_t b_sz, int64_t b_sh, int64_t b_sn, int64_t b_sk,
@@ -400,6 +616,22 @@ extern "C" int flyhip_bs_sdd(const void* a, const void* b, void* c, const int32_
     if (b_sk == 1) FLY_REQUIRE(((b_sz | b_sh | b_sn) % 4) == 0, "bs_sdd: B strides must be multiples of 4 elements");
     if (nnz == 0) return OK;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (row_ptr && row_blk && row_col && blk == 32 && (dtype == BF16 || dtype == F16) && a_sk == 1 && b_sk == 1 &&
+        K % 32 == 0 && K <= 128 && ((a_sz | a_sh | a_sm | b_sz | b_sh | b_sn) % 8) == 0 && n_brow > 0 &&
+        brows_per_head > 0) {
+        SddRowArgs ra{a, b, c, row_ptr, row_blk, row_col, nnz, K, brows_per_head, a_sz, a_sh, a_sm, b_sz, b_sh, b_sn};
+        dim3 grid(n_brow, Z);
+#define SDD32_LAUNCH(T)                                                                         \
+        switch (K / 32) {                                                                       \
+            case 1: hipLaunchKernelGGL((bs_sdd32_kernel<T, 1>), grid, dim3(256), 0, st, ra); break; \
+            case 2: hipLaunchKernelGGL((bs_sdd32_kernel<T, 2>), grid, dim3(256), 0, st, ra); break; \
+            case 3: hipLaunchKernelGGL((bs_sdd32_kernel<T, 3>), grid, dim3(256), 0, st, ra); break; \
+            default: hipLaunchKernelGGL((bs_sdd32_kernel<T, 4>), grid, dim3(256), 0, st, ra); break; \
+        }
+        if (dtype == BF16) { SDD32_LAUNCH(bf16_t) } else { SDD32_LAUNCH(f16_t) }
+#undef SDD32_LAUNCH
+        return check_launch("bs_sdd32_kernel");
+    }
     SddArgs args{a, b, c, lut, nnz, K, a_sz, a_sh, a_sm, a_sk, b_sz, b_sh, b_sn, b_sk};
     const int tile = blk >= 32 ? 32 : 16, sub = blk / tile;
     const long nblocks = waves_to_blocks((long)nnz * sub * sub);
@@ -427,6 +659,13 @@ extern "C" int flyhip_bs_dsd(const void* a_sp, const void* b, void* c,
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     DxdArgs args{a_sp, b, c, seg_ptr, seg_blk, seg_inner, n_seg, rows_per_head, N, trans_a,
                  a_sz, b_sz, b_sh, b_sk, b_sn, c_sz, c_sh, c_sm, c_sn};
+    if (blk == 32 && (dtype == BF16 || dtype == F16) && !trans_a && b_sn == 1 && c_sn == 1 && N % 8 == 0 &&
+        ((a_sz | b_sz | b_sh | b_sk | c_sz | c_sh | c_sm) % 8) == 0 && Z <= 65535 && (N + 63) / 64 <= 65535) {
+        dim3 grid(n_seg, (N + 63) / 64, Z);
+        if (dtype == BF16) hipLaunchKernelGGL((bs_dsd32_kernel<bf16_t>), grid, dim3(256), 0, st, args);
+        else hipLaunchKernelGGL((bs_dsd32_kernel<f16_t>), grid, dim3(256), 0, st, args);
+        return check_launch("bs_dsd32_kernel");
+    }
     const int tile = blk >= 32 ? 32 : 16;
     const long nblocks = waves_to_blocks((long)n_seg * (blk / tile) * ((N + 31) / 32));
     FLY_REQUIRE(nblocks <= 2147483647L, "bs_dsd: too many blocks");
@@ -463,6 +702,12 @@ extern "C" int flyhip_bs_dds(const void* a, const void* b_sp, void* c,
 
 template <typename T>
 static int launch_softmax(const RowArgs& args, dim3 grid, int max_elems, hipStream_t st) {
+    if (sizeof(T) == 2 && args.blk_shift == 5 && max_elems <= 32 * 4 * 16 && (args.x_sz % 8) == 0) {
+        dim3 g2(2 * args.n_brow, grid.y);
+        if (max_elems <= 32 * 4 * 8) hipLaunchKernelGGL((bs_softmax32_kernel<T, 8>), g2, dim3(256), 0, st, args);
+        else hipLaunchKernelGGL((bs_softmax32_kernel<T, 16>), g2, dim3(256), 0, st, args);
+        return check_launch("bs_softmax32_kernel");
+    }
     if (max_elems <= 64 * 8) hipLaunchKernelGGL((bs_softmax_kernel<T, 8>), grid, dim3(256), 0, st, args);
     else if (max_elems <= 64 * 32) hipLaunchKernelGGL((bs_softmax_kernel<T, 32>), grid, dim3(256), 0, st, args);
     else hipLaunchKernelGGL((bs_softmax_long_kernel<T>), grid, dim3(256), 0, st, args);

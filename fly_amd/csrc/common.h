@@ -131,6 +131,25 @@ template <> struct Frag<f16_t> {
     }
 };
 
+// 16x16x32 MFMA step for 2-byte types (gfx950): a fragment is the eight contraction elements
+// k = 8g..8g+7 of row/column r (one 16-byte load when k is contiguous)
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 halfx8_t __attribute__((ext_vector_type(8)));
+template <typename T> struct Frag32;
+template <> struct Frag32<bf16_t> {
+    static __device__ __forceinline__ floatx4 mma(uint4 a, uint4 b, floatx4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+    }
+};
+template <> struct Frag32<f16_t> {
+    static __device__ __forceinline__ floatx4 mma(uint4 a, uint4 b, floatx4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(halfx8_t, a), __builtin_bit_cast(halfx8_t, b), c, 0, 0, 0);
+    }
+};
+template <> struct Frag32<float> {     // never used: keeps templates that branch on sizeof(T) compilable
+    static __device__ __forceinline__ floatx4 mma(uint4, uint4, floatx4 c) { return c; }
+};
+
 // wave-level butterflies across the four 16-lane groups (lanes r, r+16, r+32, r+48), on the
 // gfx950 row-swap instructions: permlane16_swap(v, v) yields {rows 0,0,2,2} and {rows 1,1,3,3},
 // permlane32_swap(v, v) yields {low half twice} and {high half twice}; no LDS traffic

@@ -85,8 +85,13 @@ int flyhip_sblocal_fwd(const void* q, const void* k, const void* v, const float*
 
 /* SDD: c[z, n] = A[z, h_n, rows of block-row i_n, :] . B[z, h_n, rows of block-col j_n, :]^T where
  * A(m,k) / B(n,k) are addressed with (batch, head, row, k) strides (this covers trans_a/trans_b).
- * lut: int32 (nnz,4) rows (head, block_row, block_col, block_id) (ref: make_sdd_lut :261-276). */
+ * lut: int32 (nnz,4) rows (head, block_row, block_col, block_id) (ref: make_sdd_lut :261-276).
+ * row_ptr / row_blk / row_col (optional, may be NULL): the same blocks grouped per (head, block-row),
+ * n_brow = H * rows/blk of them; with these, 32x32 blocks of a 2-byte type take a faster kernel that
+ * keeps the A tile of a block-row in registers. */
 int flyhip_bs_sdd(const void* a, const void* b, void* c, const int32_t* lut, int nnz,
+                  const int32_t* row_ptr, const int32_t* row_blk, const int32_t* row_col,
+                  int n_brow, int brows_per_head,
                   int Z, int K, int blk,
                   int64_t a_sz, int64_t a_sh, int64_t a_sm, int64_t a_sk,
                   int64_t b_sz, int64_t b_sh, int64_t b_sn, int64_t b_sk,
