@@ -60,12 +60,16 @@ def bench_sblocal(steps, warmup, cpu_baseline=True):
         plan.run(qd, kd, vd, Pd, None, lc, t, out, ln)
     torch.cuda.synchronize()
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    from fly_amd import _lib
+    for a, b in ev:                      # create the underlying hipEvent_t objects before timing
+        a.record(); b.record()
+    torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(steps):
         plan.run_keys(kd, vd, Pd, None, t)
-        ev[i][0].record()
+        # the library records these two events right around the fused band kernel, on its stream
+        _lib.call('flyhip_sb_time_next_fwd', ev[i][0].cuda_event, ev[i][1].cuda_event)
         plan.run_queries(qd, kd, vd, Pd, None, lc, t, out, ln)
-        ev[i][1].record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     fwd_ms = sum(a.elapsed_time(b) for a, b in ev) / steps

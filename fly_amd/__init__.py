@@ -11,9 +11,11 @@ from .blocksparse_softmax import softmax, logsumexp, blocksparse_sum
 from .blocksparse_attention import BlockSparseAttention
 from .blocksparse_linear import BlockSparseLinear, FlatBlockButterflySparsityConfig
 from .fastlinear import LowRank, SparseLRLinear
+from .t2t_vit import T2T_ViT, T2T_module, T2TAttention, Token_transformer, MlpCustom, t2t_vit_t_14
 
 __all__ = ['FullMask', 'LengthMask', 'TriangularCausalMask', 'SBPerformerFeatures',
            'gaussian_orthogonal_random_matrix', 'SBLocalAttention', 'sblocal_forward',
            'sparsify_tensor', 'densify_tensor', 'mask_tensor', 'sparsify_broadcast_tensor',
            'matmul', 'softmax', 'logsumexp', 'blocksparse_sum', 'BlockSparseAttention',
-           'BlockSparseLinear', 'FlatBlockButterflySparsityConfig', 'LowRank', 'SparseLRLinear']
+           'BlockSparseLinear', 'FlatBlockButterflySparsityConfig', 'LowRank', 'SparseLRLinear',
+           'T2T_ViT', 'T2T_module', 'T2TAttention', 'Token_transformer', 'MlpCustom', 't2t_vit_t_14']

@@ -655,6 +655,10 @@ static int launch_kfeat(const KvArgs& a, hipStream_t st) {
     return check_launch("sb_kfeat_kernel");
 }
 
+// Optional timing hooks: two caller-owned events recorded immediately before and after the fused
+// band kernel of the next flyhip_sblocal_fwd call made by this thread (then cleared).
+static thread_local hipEvent_t g_ev_before = nullptr, g_ev_after = nullptr;
+
 template <typename T, int E, int M, bool SPLIT>
 static int launch_fwd_impl(const FwdArgs& a, hipStream_t st) {
     auto kern = sblocal_fwd_kernel<T, E, E, M, SPLIT>;
@@ -670,7 +674,10 @@ static int launch_fwd_impl(const FwdArgs& a, hipStream_t st) {
     const long items = (long)a.B * a.H * qt * a.n_parts;
     const long grid = (items + N_XCD - 1) / N_XCD * N_XCD;       // whole rounds over the XCDs
     if (grid > 2147483647L) return fail(ERR_ARG, "sblocal_fwd: too many workgroups");
+    if (g_ev_before) (void)hipEventRecord(g_ev_before, st);
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NT), smem, st, a);
+    if (g_ev_after) (void)hipEventRecord(g_ev_after, st);
+    g_ev_before = g_ev_after = nullptr;
     int rc = check_launch("sblocal_fwd_kernel");
     if (rc || !SPLIT) return rc;
     hipLaunchKernelGGL(sb_merge_kernel<T>, dim3((qt * TQ * (E / 4) + NT - 1) / NT, a.B * a.H), dim3(NT), 0, st, a, E);
@@ -744,6 +751,12 @@ extern "C" int flyhip_prof_read(long long* dst, int n_workgroups) {
     return e == hipSuccess ? 0 : -1;
 }
 #endif
+
+extern "C" int flyhip_sb_time_next_fwd(void* event_before, void* event_after) {
+    g_ev_before = reinterpret_cast<hipEvent_t>(event_before);
+    g_ev_after = reinterpret_cast<hipEvent_t>(event_after);
+    return OK;
+}
 
 extern "C" int flyhip_sb_plan(int B, int H, int T, int S, int local_context,
                               int* n_chunks, int* n_split, int* n_parts) {

@@ -76,6 +76,11 @@ int flyhip_sblocal_fwd(const void* q, const void* k, const void* v, const float*
                        int64_t o_sb, int64_t o_sh, int64_t o_ss,
                        float softmax_temp, int dtype, void* stream);
 
+/* Measurement hook (no counterpart in the reference): the two caller-owned hipEvent_t are recorded
+ * on the launch stream immediately before and after the fused band kernel of the NEXT
+ * flyhip_sblocal_fwd call of the calling thread, then forgotten.  Pass NULLs to clear. */
+int flyhip_sb_time_next_fwd(void* event_before, void* event_after);
+
 /* ------------------------------------------------------------------------------------------
  * Block-sparse matmuls (ref: src/models/attention/blocksparse_matmul.py; matmul.__call__ :656,
  * _sdd_matmul :279-346, _dds_matmul :444-488, _dsd_matmul :491-535).

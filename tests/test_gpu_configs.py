@@ -1,0 +1,174 @@
+"""BASELINE configs 3, 4 and 5 on the GPU against the oracle (GPU box only)."""
+import copy
+import math
+
+import pytest
+import torch
+import torch.nn as nn
+
+from conftest import rel_err
+from oracle import sblocal as osb
+from oracle import blocksparse as ob
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda:0'
+
+
+class OracleSBLocal(nn.Module):
+    """Attention plugin that evaluates the CPU oracle with a given projection matrix."""
+    def __init__(self, P, lc, temp):
+        super().__init__()
+        self.P, self.lc, self.temp = P, lc, temp
+
+    def forward(self, q, k, v):
+        out, _ = osb.sblocal_attention(q, k, v, self.P, self.lc, softmax_temp=self.temp)
+        return out, None
+
+
+def _sb_cfg():
+    return {'_target_': 'src.models.attention.sblocal_attention.SBLocalAttention', 'local_context': 256,
+            'dim_heads': 64, 'nb_features': 128}
+
+
+def test_config3_t2t_vit_logits_parity():
+    """T2T-ViT-t-14, both T2T layers on SBLocalAttention (window 256, 128 features, temperatures
+    147^-0.5 and 576^-0.5): logits of the HIP-attention model on the GPU against the same weights
+    with oracle attention on the CPU (batch 2 for the CPU side), then the full batch of 64 on the GPU."""
+    import fly_amd
+    torch.manual_seed(0)
+    model = fly_amd.t2t_vit_t_14(t2tattn1_cfg=_sb_cfg(), t2tattn2_cfg=_sb_cfg()).eval()
+    layers = [model.patch_embed.attention1.attn, model.patch_embed.attention2.attn]
+    for lay in layers:                                   # fixed seeded projection per layer
+        lay.attention_layer.feature_map.new_feature_map('cpu')
+    ref = copy.deepcopy(model)
+    for lay_ref, lay in zip([ref.patch_embed.attention1.attn, ref.patch_embed.attention2.attn], layers):
+        P = lay.attention_layer.feature_map.projection_matrix.clone()
+        assert P.shape == (64, 64) and float(P.abs().sum()) > 0
+        lay_ref.attention_layer = OracleSBLocal(P, 256, lay.scale)
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(64, 3, 224, 224, generator=g)
+    with torch.no_grad():
+        want = ref(x[:2])
+        gpu = model.to(DEV)
+        got = gpu(x[:2].to(DEV)).cpu()
+        print('logits rel err', rel_err(got, want), 'max elementwise rel',
+              float(((got - want).abs() / want.abs().clamp_min(1e-3)).max()), flush=True)
+        assert got.shape == (2, 1000)
+        assert rel_err(got, want) <= 1e-4
+        full = gpu(x.to(DEV))
+        torch.cuda.synchronize()
+        assert full.shape == (64, 1000) and bool(torch.isfinite(full).all())
+        assert rel_err(full[:2].cpu(), want) <= 1e-4
+
+
+@pytest.mark.parametrize('L,dim', [(3136, 147), (784, 576)])
+def test_config3_attention_layers_parity(L, dim):
+    from fly_amd import sblocal_forward
+    g = torch.Generator().manual_seed(L)
+    q, k, v = (torch.randn(4, L, 1, 64, generator=g) for _ in range(3))
+    P = osb.gaussian_orthogonal_random_matrix(64, 64, generator=g)
+    t = dim ** -0.5
+    out, ln = sblocal_forward(q.to(DEV), k.to(DEV), v.to(DEV), P.to(DEV), 256, softmax_temp=t)
+    ref_out, ref_ln = osb.sblocal_attention(q.double(), k.double(), v.double(), P.double(), 256, softmax_temp=t)
+    assert rel_err(out, ref_out) <= 1e-4 and rel_err(ln, ref_ln) <= 1e-4
+
+
+def test_config4_pixelfly_mlp_bf16():
+    """MLP-Mixer-B channel MLP 768 -> 3072 -> 768 in bf16: SparseLRLinear = flat butterfly (8, 2) block 32
+    sparse term (HIP DDS kernel) + rank 96 low-rank term + sigmoid gate, on 256 x 196 tokens."""
+    import fly_amd
+    torch.manual_seed(0)
+    cfg = fly_amd.FlatBlockButterflySparsityConfig(8, 2, block=32)
+    lin = {'_target_': 'src.models.layers.fastlinear.SparseLRLinear',
+           'sparse_cfg': {'_target_': 'src.models.layers.blocksparse_linear.BlockSparseLinear', 'sparsity_config': cfg},
+           'rank': 96, 'gating': True}
+    mlp = fly_amd.MlpCustom(768, 3072, linear1_cfg=lin, linear2_cfg=lin)
+    assert int(mlp.fc1.sparse.layout.sum()) == 864 and int(mlp.fc2.sparse.layout.sum()) == 864
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(256 * 196, 768, generator=g).bfloat16()
+    gpu = copy.deepcopy(mlp).to(DEV).to(torch.bfloat16)
+    with torch.no_grad():
+        y = gpu(x.to(DEV))
+        torch.cuda.synchronize()
+        assert y.shape == (256 * 196, 768) and y.dtype == torch.bfloat16
+
+        def slr_ref(mod, inp):        # oracle: fp32 math on the bf16-rounded weights and inputs
+            w = lambda p: p.detach().bfloat16().float()
+            sp = ob.blocksparse_linear(inp, w(mod.sparse.weight), mod.sparse.layout, 32, None, mod.out_features)
+            return ob.sparse_lr_linear(inp, sp, w(mod.low_rank.lr_weight1), w(mod.low_rank.lr_weight2),
+                                       w(mod.gate.weight), w(mod.gate.bias), w(mod.bias))
+        n = 4096                                       # oracle on a slice of the tokens
+        xs = x[:n].float()
+        h_gpu = gpu.fc1(x[:n].to(DEV)).float().cpu()
+        h_ref = slr_ref(mlp.fc1, xs)
+        assert rel_err(h_gpu, h_ref) <= 2e-2
+        ref = slr_ref(mlp.fc2, torch.nn.functional.gelu(h_ref.bfloat16().float()).bfloat16().float())
+        assert rel_err(y[:n].float().cpu(), ref) <= 2e-2
+        # the sparse term alone, all tokens, fc1 shape: DDS against the dense formula
+        s_gpu = gpu.fc1.sparse(x.to(DEV)).float().cpu()
+        s_ref = ob.blocksparse_linear(x.float(), mlp.fc1.sparse.weight.detach().bfloat16().float(),
+                                      mlp.fc1.sparse.layout, 32, None, 3072)
+        assert rel_err(s_gpu, s_ref) <= 2e-2
+
+
+def test_config5_long_sequence_bf16():
+    """B=1, H=16, L=16384, d=64, window 1024, 256 features, bf16 inputs with 5 % of the key rows
+    scaled by 8.  The GPU runs all 16 heads; the oracle (fp32 on the bf16-rounded inputs) checks two."""
+    from fly_amd import sblocal_forward
+    g = torch.Generator().manual_seed(0)
+    B, L, H, E = 1, 16384, 16, 64
+    q = torch.randn(B, L, H, E, generator=g)
+    k = torch.randn(B, L, H, E, generator=g)
+    v = torch.randn(B, L, H, E, generator=g)
+    idx = torch.randperm(L, generator=g)[: L // 20]
+    k[:, idx] *= 8
+    P = osb.gaussian_orthogonal_random_matrix(128, 64, generator=g)
+    qb, kb, vb = q.bfloat16(), k.bfloat16(), v.bfloat16()
+    out, ln = sblocal_forward(qb.to(DEV), kb.to(DEV), vb.to(DEV), P.to(DEV), 1024)
+    torch.cuda.synchronize()
+    assert out.shape == (B, L, H, E) and out.dtype == torch.bfloat16 and bool(torch.isfinite(out.float()).all())
+    heads = [3, 12]
+    sel = lambda t: t[:, :, heads].float()
+    ref_out, ref_ln = osb.sblocal_attention(sel(qb), sel(kb), sel(vb), P, 1024, chunk=512)
+    assert rel_err(out[:, :, heads], ref_out) <= 2e-2
+    assert rel_err(ln[:, heads], ref_ln) <= 2e-2
+    # normalisation identity at full size: values of one give outputs of one
+    ones, _ = sblocal_forward(qb.to(DEV), kb.to(DEV), torch.ones_like(vb).to(DEV), P.to(DEV), 1024)
+    assert float((ones.float() - 1).abs().max()) <= 1e-2
+
+
+def test_matmul_backward_matches_dense_autograd():
+    """Gradients of the three modes against autograd through the dense formula (the reference's
+    backward re-uses its kernels with permuted roles, blocksparse_matmul.py:562-587)."""
+    from fly_amd import matmul
+    from fly_amd.blocksparse_utils import densify_tensor, sparsify_tensor
+    g = torch.Generator().manual_seed(0)
+    block, Z, H, p, r = 32, 2, 2, 3, 4
+    layout = (torch.rand(H, p, r, generator=g) < 0.6).long()
+    nnz = int(layout.sum())
+    a = torch.randn(Z, H, p * block, 48, generator=g).to(DEV).requires_grad_()
+    b = torch.randn(Z, H, r * block, 48, generator=g).to(DEV).requires_grad_()
+    c = matmul(layout, block, 'sdd', trans_b=True)(a, b)
+    w = torch.randn(c.shape, generator=g).to(DEV)
+    (c * w).sum().backward()
+    a2, b2 = a.detach().clone().requires_grad_(), b.detach().clone().requires_grad_()
+    (sparsify_tensor(a2 @ b2.transpose(-1, -2), layout) * w).sum().backward()
+    assert rel_err(a.grad, a2.grad) <= 1e-5 and rel_err(b.grad, b2.grad) <= 1e-5
+
+    sp = torch.randn(Z, nnz, block, block, generator=g).to(DEV).requires_grad_()
+    d = torch.randn(Z, H, r * block, 48, generator=g).to(DEV).requires_grad_()   # SDD in the backward needs K % 16 == 0
+    out = matmul(layout, block, 'dsd')(sp, d)
+    w = torch.randn(out.shape, generator=g).to(DEV)
+    (out * w).sum().backward()
+    sp2, d2 = sp.detach().clone().requires_grad_(), d.detach().clone().requires_grad_()
+    ((densify_tensor(sp2, layout) @ d2) * w).sum().backward()
+    assert rel_err(sp.grad, sp2.grad) <= 1e-5 and rel_err(d.grad, d2.grad) <= 1e-5
+
+    x = torch.randn(1, 1, 64, r * block, generator=g).to(DEV).requires_grad_()
+    wsp = torch.randn(1, int(layout[0].sum()), block, block, generator=g).to(DEV).requires_grad_()
+    y = matmul(layout[0], block, 'dds', trans_b=True)(x, wsp)
+    w = torch.randn(y.shape, generator=g).to(DEV)
+    (y * w).sum().backward()
+    x2, w2 = x.detach().clone().requires_grad_(), wsp.detach().clone().requires_grad_()
+    ((x2 @ densify_tensor(w2, layout[:1]).transpose(-1, -2)) * w).sum().backward()
+    assert rel_err(x.grad, x2.grad) <= 1e-5 and rel_err(wsp.grad, w2.grad) <= 1e-5
