@@ -3,7 +3,7 @@ src/models/attention/blocksparse_matmul.py:590-719 (modes 'sdd', 'dsd', 'dds')."
 import torch
 
 from . import _lib
-from .blocksparse_utils import sdd_table, segment_table
+from .blocksparse_utils import group_table, sdd_table, segment_table
 
 _BLOCKS = (16, 32, 64, 128)
 
@@ -86,6 +86,8 @@ class matmul:
         if key not in self.lut_cache:
             if kind == 'sdd':
                 tabs = (sdd_table(self.layout),)
+            elif kind in ('grp_rows', 'grp_cols'):
+                tabs = group_table(self.layout, by_rows=(kind == 'grp_rows'))
             else:
                 tabs = segment_table(self.layout, by_rows=(kind == 'rows'))
             self.lut_cache[key] = tuple(t.to(device) for t in tabs)
@@ -200,6 +202,7 @@ class matmul:
         H, p, r = self.spdims
         by_rows = trans_b
         seg_ptr, seg_blk, seg_inner = self._table('rows' if by_rows else 'cols', a.device)
+        grp_row0, grp_n = self._table('grp_rows' if by_rows else 'grp_cols', a.device)
         per_head = p if by_rows else r
         N = per_head * self.block
         Z = a.shape[0]
@@ -210,6 +213,8 @@ class matmul:
         with torch.cuda.device(a.device):
             _lib.call('flyhip_bs_dds', a.data_ptr(), b.data_ptr(), c.data_ptr(),
                       seg_ptr.data_ptr(), seg_blk.data_ptr(), seg_inner.data_ptr(),
+                      grp_row0.data_ptr(), grp_n.data_ptr(), grp_row0.shape[0],
+                      int(self.layout.sum(-1 if by_rows else -2).max()),
                       H * per_head, per_head, Z, M, self.block, int(trans_b),
                       a.stride(0), a.stride(1), a_sm, a_sk, b.stride(0),
                       c.stride(0), c.stride(1), c_sm, c_sn, _lib.dtype_code(a), _lib.stream_ptr(a.device))

@@ -99,3 +99,23 @@ def row_table(layout):
     ptr, blk, col = segment_table(layout, by_rows=True)
     counts = ptr[1:] - ptr[:-1]
     return ptr, blk, col, int(counts.max()) if counts.numel() else 0
+
+
+def group_table(layout, by_rows, max_group=4):
+    """Groups of up to `max_group` consecutive segments (of one head) whose reduction lists visit the
+    same inner blocks: returns (grp_row0 int32, grp_n int32).  Every segment belongs to one group."""
+    layout = _as_layout3(layout).cpu().long()
+    if not by_rows:
+        layout = layout.transpose(1, 2)
+    H, p, _ = layout.shape
+    row0, count = [], []
+    for h in range(H):
+        i = 0
+        while i < p:
+            n = 1
+            while n < max_group and i + n < p and torch.equal(layout[h, i + n], layout[h, i]):
+                n += 1
+            row0.append(h * p + i)
+            count.append(n)
+            i += n
+    return torch.tensor(row0, dtype=torch.int32), torch.tensor(count, dtype=torch.int32)

@@ -350,6 +350,139 @@ __global__ __launch_bounds__(256) void bs_dds_kernel(DxdArgs a) {
     }
 }
 
+// Fast DDS (y = x W^T, W block-sparse, blocks read transposed) for 32x32 blocks of a 2-byte type,
+// the Pixelfly linear.  Consecutive output block-rows that reduce over the same input blocks are
+// grouped (at most four per group, table built on the host): a group is a small dense GEMM
+// y[M x 32g] = x[:, listed input blocks] . W_group^T.  One workgroup per (group, 128-token tile):
+// per input block the 128 x 32 activation tile and the group's 32g x 32 weight tile are staged in
+// LDS (registers hold the next step's tiles while the MFMAs of the current one run), the 2 x 2
+// waves own 64 x 64 outputs each and form them with 16x16x32 MFMAs.
+struct DdsGroupArgs {
+    const void* sp; const void* dn; void* c;
+    const int32_t* seg_ptr; const int32_t* seg_blk; const int32_t* seg_inner;
+    const int32_t* grp_row0; const int32_t* grp_n;
+    int per_head, M;
+    long sp_sz, dn_sz, dn_sh, dn_sm, c_sz, c_sh, c_sm;
+};
+constexpr int DDS_MAX_STEPS = 128;   // longest reduction list the tiled kernel accepts
+
+template <typename T>
+__global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
+    constexpr int KB = 1;                                   // input blocks per pipeline step
+    constexpr int LD = 32 * KB + 8;                         // LDS row stride in elements
+    __shared__ __attribute__((aligned(16))) uint16_t xs[2][128 * LD];
+    __shared__ __attribute__((aligned(16))) uint16_t ws[2][128 * LD];
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
+    const int wm = w >> 1, wn = w & 1;                      // this wave: tokens 64wm.., outputs 64wn..
+    const int grp = blockIdx.x, z = blockIdx.z;
+    const long m0 = (long)blockIdx.y * 128;
+    const int row0 = a.grp_row0[grp], gn = a.grp_n[grp];    // first output block-row (segment) and count
+    const int head = row0 / a.per_head, bcol0 = row0 % a.per_head;
+    const int p0 = a.seg_ptr[row0], nin = a.seg_ptr[row0 + 1] - p0;
+    const uint16_t* spz = reinterpret_cast<const uint16_t*>(a.sp) + z * a.sp_sz;
+    const uint16_t* xp = reinterpret_cast<const uint16_t*>(a.dn) + z * a.dn_sz + head * a.dn_sh;
+
+    // the group's reduction list (inner block per step, block id per step and output block-row) is
+    // read once into LDS: the per-step loads then depend on no other global load
+    __shared__ int s_inner[DDS_MAX_STEPS];
+    __shared__ int s_blk[4][DDS_MAX_STEPS];
+    for (int i = tid; i < nin; i += 256) s_inner[i] = a.seg_inner[p0 + i];
+    for (int i = tid; i < 4 * nin; i += 256) {
+        const int ob = i / nin, t = i % nin;
+        s_blk[ob][t] = ob < gn ? a.seg_blk[a.seg_ptr[row0 + ob] + t] : -1;
+    }
+    __syncthreads();
+
+    // staging roles: thread -> (row = tid/4 [+64], 16-byte chunk = tid%4) of the x and W tiles of one
+    // input block; a step moves KB input blocks
+    const int srow = tid >> 2, schunk = (tid & 3) * 8;
+    const int n_steps = (nin + KB - 1) / KB;
+    // two register sets: the loads of step s+2 are issued while step s computes and are parked in LDS
+    // one iteration later, so every global load has two steps to arrive
+    uint4 rxa[KB][2], rwa[KB][2], rxb[KB][2], rwb[KB][2];
+    auto fetch = [&](int step, uint4 (&rx)[KB][2], uint4 (&rw)[KB][2]) {
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) {
+            const int t = step * KB + kb;
+            const bool live = t < nin;                       // a missing block contributes zero weights
+            const long kcol = (long)s_inner[live ? t : nin - 1] * 32 + schunk;
+#pragma unroll
+            for (int hh = 0; hh < 2; ++hh) {
+                const long m = min(m0 + srow + 64 * hh, (long)a.M - 1);        // clamped: masked at the store
+                rx[kb][hh] = *reinterpret_cast<const uint4*>(xp + m * a.dn_sm + kcol);
+                const int orow = srow + 64 * hh;                                 // output row inside the group
+                const int blk_id = live ? s_blk[orow >> 5][t] : -1;
+                rw[kb][hh] = make_uint4(0, 0, 0, 0);
+                if (blk_id >= 0)
+                    rw[kb][hh] = *reinterpret_cast<const uint4*>(spz + (long)blk_id * 1024 + (orow & 31) * 32 + schunk);
+            }
+        }
+    };
+    auto stash = [&](int buf, const uint4 (&rx)[KB][2], const uint4 (&rw)[KB][2]) {
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+            for (int hh = 0; hh < 2; ++hh) {
+                *reinterpret_cast<uint4*>(&xs[buf][(srow + 64 * hh) * LD + 32 * kb + schunk]) = rx[kb][hh];
+                *reinterpret_cast<uint4*>(&ws[buf][(srow + 64 * hh) * LD + 32 * kb + schunk]) = rw[kb][hh];
+            }
+    };
+
+    floatx4 acc[4][4];
+#pragma unroll
+    for (int tm = 0; tm < 4; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < 4; ++tn) acc[tm][tn] = Frag<float>::zero();
+    const bool wave_active = 2 * wn < gn;                   // its output blocks exist in this group
+
+    auto compute = [&](int cur) {
+        if (wave_active) {
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) {
+                uint4 fx[4], fw[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    fx[i] = *reinterpret_cast<const uint4*>(&xs[cur][(64 * wm + 16 * i + r16) * LD + 32 * kb + 8 * g]);
+                    fw[i] = *reinterpret_cast<const uint4*>(&ws[cur][(64 * wn + 16 * i + r16) * LD + 32 * kb + 8 * g]);
+                }
+#pragma unroll
+                for (int tm = 0; tm < 4; ++tm)
+#pragma unroll
+                    for (int tn = 0; tn < 4; ++tn) acc[tm][tn] = Frag32<T>::mma(fw[tn], fx[tm], acc[tm][tn]);
+            }
+        }
+    };
+    if (n_steps > 0) { fetch(0, rxa, rwa); stash(0, rxa, rwa); }
+    if (n_steps > 1) fetch(1, rxb, rwb);                   // set B holds odd steps, set A even steps
+    __syncthreads();
+    for (int step = 0; step < n_steps; step += 2) {
+        if (step + 2 < n_steps) fetch(step + 2, rxa, rwa);
+        compute(0);
+        if (step + 1 < n_steps) stash(1, rxb, rwb);
+        __syncthreads();
+        if (step + 1 >= n_steps) break;
+        if (step + 3 < n_steps) fetch(step + 3, rxb, rwb);
+        compute(1);
+        if (step + 2 < n_steps) stash(0, rxa, rwa);
+        __syncthreads();
+    }
+    // lane holds y[m = 64wm + 16tm + r16][n = 64wn + 16tn + 4g + i]
+    if (!wave_active) return;
+    T* cp = reinterpret_cast<T*>(a.c) + z * a.c_sz + head * a.c_sh;
+#pragma unroll
+    for (int tm = 0; tm < 4; ++tm) {
+        const long m = m0 + 64 * wm + 16 * tm + r16;
+        if (m >= a.M) continue;
+#pragma unroll
+        for (int tn = 0; tn < 4; ++tn) {
+            const int ob = 2 * wn + (tn >> 1);
+            if (ob >= gn) continue;
+            const long n = (long)(bcol0 + ob) * 32 + 16 * (tn & 1) + 4 * g;
+            store4_f32(cp + m * a.c_sm + n, acc[tm][tn]);
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------------------
 // row operations: one wave per row of a block-row
 // ---------------------------------------------------------------------------------------
@@ -676,6 +809,7 @@ extern "C" int flyhip_bs_dsd(const void* a_sp, const void* b, void* c,
 
 extern "C" int flyhip_bs_dds(const void* a, const void* b_sp, void* c,
                              const int32_t* seg_ptr, const int32_t* seg_blk, const int32_t* seg_inner,
+                             const int32_t* grp_row0, const int32_t* grp_n, int n_grp, int max_seg_len,
                              int n_seg, int cols_per_head, int Z, int M, int blk, int trans_b,
                              int64_t a_sz, int64_t a_sh, int64_t a_sm, int64_t a_sk,
                              int64_t b_sz,
@@ -690,6 +824,16 @@ extern "C" int flyhip_bs_dds(const void* a, const void* b_sp, void* c,
     if (c_sn == 1) FLY_REQUIRE(((c_sz | c_sh | c_sm) % 4) == 0, "bs_dds: C strides must be multiples of 4 elements");
     FLY_REQUIRE(b_sz % 4 == 0, "bs_dds: sparse batch stride must be a multiple of 4 elements");
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (grp_row0 && grp_n && n_grp > 0 && max_seg_len >= 0 && max_seg_len <= DDS_MAX_STEPS && blk == 32 &&
+        (dtype == BF16 || dtype == F16) && trans_b && a_sk == 1 &&
+        c_sn == 1 && ((a_sz | a_sh | a_sm | b_sz | c_sz | c_sh | c_sm) % 8) == 0 && (M + 127) / 128 <= 65535) {
+        DdsGroupArgs ga{b_sp, a, c, seg_ptr, seg_blk, seg_inner, grp_row0, grp_n, cols_per_head, M,
+                        b_sz, a_sz, a_sh, a_sm, c_sz, c_sh, c_sm};
+        dim3 grid(n_grp, (M + 127) / 128, Z);
+        if (dtype == BF16) hipLaunchKernelGGL((bs_dds32_kernel<bf16_t>), grid, dim3(256), 0, st, ga);
+        else hipLaunchKernelGGL((bs_dds32_kernel<f16_t>), grid, dim3(256), 0, st, ga);
+        return check_launch("bs_dds32_kernel");
+    }
     DxdArgs args{b_sp, a, c, seg_ptr, seg_blk, seg_inner, n_seg, cols_per_head, M, trans_b,
                  b_sz, a_sz, a_sh, a_sm, a_sk, c_sz, c_sh, c_sm, c_sn};
     const int tile = blk >= 32 ? 32 : 16;

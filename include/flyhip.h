@@ -116,9 +116,14 @@ int flyhip_bs_dsd(const void* a_sp, const void* b, void* c,
 
 /* DDS: c (Z,H,M,N) = dense a . op(sparse b).  Segment s = (head, output block-column); trans_b != 0
  * reads every sparse block transposed (the BlockSparseLinear case, ref:
- * src/models/layers/blocksparse_linear.py:119-120,152-162).  a(m,k) and c(m,n) via strides. */
+ * src/models/layers/blocksparse_linear.py:119-120,152-162).  a(m,k) and c(m,n) via strides.
+ * grp_row0 / grp_n (optional, may be NULL, n_grp entries): groups of at most four consecutive segments
+ * of one head whose reduction lists visit the same inner blocks in the same order (first segment
+ * and count per group, covering every segment once; max_seg_len = longest reduction list); with them, 32x32 blocks of a 2-byte type with
+ * trans_b take a tiled kernel that treats each group as a small dense GEMM. */
 int flyhip_bs_dds(const void* a, const void* b_sp, void* c,
                   const int32_t* seg_ptr, const int32_t* seg_blk, const int32_t* seg_inner,
+                  const int32_t* grp_row0, const int32_t* grp_n, int n_grp, int max_seg_len,
                   int n_seg, int cols_per_head, int Z, int M, int blk, int trans_b,
                   int64_t a_sz, int64_t a_sh, int64_t a_sm, int64_t a_sk,
                   int64_t b_sz,
