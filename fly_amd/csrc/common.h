@@ -171,6 +171,15 @@ __device__ __forceinline__ float group_sum(float v) {
     rows_pair16(v, a, b); v = a + b;
     rows_pair32(v, a, b); return a + b;
 }
+// sum over the 16 lanes of a row (lanes with equal lane/16) on DPP: quad butterflies, then the two
+// mirrors; every lane of the row ends with the row total
+__device__ __forceinline__ float row16_sum(float v) {
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, true));   // quad_perm 1,0,3,2
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, true));   // quad_perm 2,3,0,1
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, true));  // row_half_mirror
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xf, 0xf, true));  // row_mirror
+    return v;
+}
 __device__ __forceinline__ float wave_max(float v) {
     for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
     return v;

@@ -102,76 +102,98 @@ __device__ __forceinline__ void load_proj(float* Ps, const float* proj, float sc
 // ---------------------------------------------------------------------------------------
 // key features + partial K'^T V
 // ---------------------------------------------------------------------------------------
+// two waves per SIMD (two workgroups per CU) where the register budget allows it without spilling
+constexpr int kfeat_waves(int E, int M) { return (E <= 64 && M <= 128) ? 2 : 1; }
+
 template <typename T, int E, int D, int M>
-__global__ __launch_bounds__(NT) void sb_kfeat_kernel(KvArgs a) {
+__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(kfeat_waves(E, M), kfeat_waves(E, M))))
+void sb_kfeat_kernel(KvArgs a) {
     constexpr int MH = M / 2, LDK = E + 4, LDV = D + 4, LDF = M + 4;
-    constexpr int FB = MH / 16;                  // feature blocks of the projection
+    constexpr int FB = MH / 16, EC = E / 16, DB = D / 16;
     constexpr int RB = (M / 16 + 3) / 4;         // K'^T V row blocks per wave
+    constexpr float LOG2E = 1.4426950408889634f, LN2 = 0.6931471805599453f;
     extern __shared__ float smem[];
-    float* Ps = smem;
-    float* Ks = Ps + MH * LDK;
-    float* Vs = Ks + CH * LDK;
-    float* Fs = Vs + CH * LDV;
-    float* red = Fs + CH * LDF;
+    float* Ks = smem;                             // 64-key K tile
+    float* Vs = Ks + CH * LDK;                    // 64-key V tile
+    float* Fs = Vs + CH * LDV;                    // features of the current chunk
+    float* red = Fs + CH * LDF;                   // 4 wave maxima
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
     const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H, sp = blockIdx.x;
     const T* kptr = reinterpret_cast<const T*>(a.k) + b * a.k_sb + h * a.k_sh;
     const T* vptr = reinterpret_cast<const T*>(a.v) + b * a.v_sb + h * a.v_sh;
     const int len = a.lens ? min((int)a.lens[b], a.S) : a.S;
-    const float lnm_half = 0.5f * logf(2.0f * a.mh_valid);
-
-    load_proj<E, MH>(Ps, a.proj, sqrtf(a.temp), tid);
-
-    floatx4 kvacc[RB][D / 16];
-#pragma unroll
-    for (int x = 0; x < RB; ++x)
-#pragma unroll
-        for (int db = 0; db < D / 16; ++db) kvacc[x][db] = Frag<float>::zero();
-    float ksum_acc = 0.f;
-    float run_max = -INFINITY;
+    const float lnm_half2 = 0.5f * __log2f(2.0f * a.mh_valid);      // base-2 from here on
 
     const int per = (a.n_chunks + a.n_split - 1) / a.n_split;
     const int c0 = sp * per, c1 = min(a.n_chunks, c0 + per);
+    RowTile<CH, E> kt;
+    RowTile<CH, D> vt;
+    if (c0 < c1) {
+        kt.fetch(kptr, a.k_ss, c0 * CH, a.S - 1, tid);
+        vt.fetch(vptr, a.v_ss, c0 * CH, a.S - 1, tid);
+    }
+    // projection fragments (A side: row = feature 16fb + r16, k = 16cc + 4g + j) come straight from
+    // global memory: the matrix is small and stays in the L1/L2 caches
+    const float* pp = a.proj + r16 * E + 4 * g;
+    const float pscale = sqrtf(a.temp) * LOG2E;                      // projections come out in base-2 units
+    if (c0 < c1) {
+        kt.template stash<LDK>(Ks, tid);
+        vt.template stash<LDV>(Vs, tid);
+    }
+    __syncthreads();
+
+    floatx4 kvacc[RB][DB];
+#pragma unroll
+    for (int x = 0; x < RB; ++x)
+#pragma unroll
+        for (int db = 0; db < DB; ++db) kvacc[x][db] = Frag<float>::zero();
+    floatx4 ksp[FB], ksn[FB];                    // running sums of this lane's key column of K'
+#pragma unroll
+    for (int fb = 0; fb < FB; ++fb) { ksp[fb] = Frag<float>::zero(); ksn[fb] = Frag<float>::zero(); }
+    float run_max = -INFINITY;                   // base-2 running maximum of the chunk stabilisers
+
     for (int c = c0; c < c1; ++c) {
         const int s_base = c * CH;
-        __syncthreads();
-        {
-            RowTile<CH, E> kt;
-            RowTile<CH, D> vt;
-            kt.fetch(kptr, a.k_ss, s_base, a.S - 1, tid);
-            vt.fetch(vptr, a.v_ss, s_base, a.S - 1, tid);
-            kt.template stash<LDK>(Ks, tid);
-            vt.template stash<LDV>(Vs, tid);
+        if (c + 1 < c1) {                        // next chunk's K and V fly during this chunk's work
+            kt.fetch(kptr, a.k_ss, s_base + CH, a.S - 1, tid);
+            vt.fetch(vptr, a.v_ss, s_base + CH, a.S - 1, tid);
         }
-        __syncthreads();
-
-        // projection of this wave's 16 keys: dd[fb][i] = (sqrt(t) P)[16fb+4g+i] . k[16w+r16]
-        floatx4 kb[E / 16];
+        // projection of this wave's 16 keys, all feature blocks advancing together:
+        // dd[fb][i] = log2(e) * (sqrt(t) P)[16fb+4g+i] . k[16w+r16]
+        floatx4 kb[EC];
         float sq = 0.f;
 #pragma unroll
-        for (int cc = 0; cc < E / 16; ++cc) {
+        for (int cc = 0; cc < EC; ++cc) {
             kb[cc] = *reinterpret_cast<const floatx4*>(Ks + (16 * w + r16) * LDK + 16 * cc + 4 * g);
             sq += kb[cc][0] * kb[cc][0] + kb[cc][1] * kb[cc][1] + kb[cc][2] * kb[cc][2] + kb[cc][3] * kb[cc][3];
+            kb[cc] *= pscale;                    // the key operand carries sqrt(t) log2(e)
         }
-        const float diag = 0.5f * a.temp * group_sum(sq);
+        const float diag2 = 0.5f * a.temp * LOG2E * group_sum(sq);
         floatx4 dd[FB];
+#pragma unroll
+        for (int fb = 0; fb < FB; ++fb) dd[fb] = Frag<float>::zero();
+#pragma unroll
+        for (int cc = 0; cc < EC; ++cc) {
+            floatx4 pa[FB];
+#pragma unroll
+            for (int fb = 0; fb < FB; ++fb)
+                pa[fb] = *reinterpret_cast<const floatx4*>(pp + 16 * fb * E + 16 * cc);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int fb = 0; fb < FB; ++fb)
+                    dd[fb] = __builtin_amdgcn_mfma_f32_16x16x4f32(pa[fb][j], kb[cc][j], dd[fb], 0, 0, 0);
+        }
         float amax = 0.f;
 #pragma unroll
-        for (int fb = 0; fb < FB; ++fb) {
-            dd[fb] = Frag<float>::zero();
-#pragma unroll
-            for (int cc = 0; cc < E / 16; ++cc) {
-                floatx4 pa = *reinterpret_cast<const floatx4*>(Ps + (16 * fb + r16) * LDK + 16 * cc + 4 * g);
-                dd[fb] = Frag<float>::mma(pa, kb[cc], dd[fb]);
-            }
+        for (int fb = 0; fb < FB; ++fb)
 #pragma unroll
             for (int i = 0; i < 4; ++i)
                 if (16 * fb + 4 * g + i < a.mh_valid) amax = fmaxf(amax, fabsf(dd[fb][i]));
-        }
         amax = group_max(amax);
         const bool kvalid = (s_base + 16 * w + r16) < len;
-        float cs = kvalid ? (amax - diag - lnm_half) : -INFINITY;
+        float cs = kvalid ? (amax - diag2 - lnm_half2) : -INFINITY;
         cs = wave_max(cs);
         if (lane == 0) red[w] = cs;
         __syncthreads();
@@ -185,75 +207,92 @@ __global__ __launch_bounds__(NT) void sb_kfeat_kernel(KvArgs a) {
                 *reinterpret_cast<floatx4*>(frow_g + MH + 16 * fb + 4 * g) = Frag<float>::zero();
             }
             if (tid == 0) a.chunk_scale[(long)bh * a.n_chunks + c] = 0.f;
-            continue;
-        }
-        const float rescale = (run_max == -INFINITY) ? 0.f : expf(run_max - new_max);
-        run_max = new_max;
+        } else {
+            const float rescale = (run_max == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(run_max - new_max);
+            run_max = new_max;
 #pragma unroll
-        for (int x = 0; x < RB; ++x)
+            for (int x = 0; x < RB; ++x)
 #pragma unroll
-            for (int db = 0; db < D / 16; ++db) kvacc[x][db] *= rescale;
-        ksum_acc *= rescale;
-
-        const float off = -diag - lnm_half - new_max;
-        float* frow_s = Fs + (16 * w + r16) * LDF;
+                for (int db = 0; db < DB; ++db) kvacc[x][db] *= rescale;
+            const float off = -diag2 - lnm_half2 - new_max;
+            float* frow_s = Fs + (16 * w + r16) * LDF;
 #pragma unroll
-        for (int fb = 0; fb < FB; ++fb) {
-            floatx4 fp, fn;
+            for (int fb = 0; fb < FB; ++fb) {
+                floatx4 fp, fn;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const bool ok = kvalid && (16 * fb + 4 * g + i < a.mh_valid);
-                fp[i] = ok ? expf(dd[fb][i] + off) : 0.f;
-                fn[i] = ok ? expf(-dd[fb][i] + off) : 0.f;
+                for (int i = 0; i < 4; ++i) {
+                    const bool ok = kvalid && (16 * fb + 4 * g + i < a.mh_valid);
+                    fp[i] = ok ? __builtin_amdgcn_exp2f(dd[fb][i] + off) : 0.f;
+                    fn[i] = ok ? __builtin_amdgcn_exp2f(-dd[fb][i] + off) : 0.f;
+                }
+                ksp[fb] = ksp[fb] * rescale + fp;
+                ksn[fb] = ksn[fb] * rescale + fn;
+                *reinterpret_cast<floatx4*>(frow_s + 16 * fb + 4 * g) = fp;
+                *reinterpret_cast<floatx4*>(frow_s + MH + 16 * fb + 4 * g) = fn;
+                *reinterpret_cast<floatx4*>(frow_g + 16 * fb + 4 * g) = fp;
+                *reinterpret_cast<floatx4*>(frow_g + MH + 16 * fb + 4 * g) = fn;
             }
-            *reinterpret_cast<floatx4*>(frow_s + 16 * fb + 4 * g) = fp;
-            *reinterpret_cast<floatx4*>(frow_s + MH + 16 * fb + 4 * g) = fn;
-            *reinterpret_cast<floatx4*>(frow_g + 16 * fb + 4 * g) = fp;
-            *reinterpret_cast<floatx4*>(frow_g + MH + 16 * fb + 4 * g) = fn;
-        }
-        if (tid == 0) a.chunk_scale[(long)bh * a.n_chunks + c] = new_max;
-        __syncthreads();
-
-        // KV[r][d] += sum_keys F[key][r] V[key][d]; lane ends with KV[16rb+4g+i][16db+r16]
+            if (tid == 0) a.chunk_scale[(long)bh * a.n_chunks + c] = new_max * LN2;    // stored in natural-log units
+            __syncthreads();
+            // KV[r][d] += sum_keys F[key][r] V[key][d]; lane ends with KV[16rb+4g+i][16db+r16]
 #pragma unroll
-        for (int x = 0; x < RB; ++x) {
-            const int rb = w + 4 * x;
-            if (rb < M / 16) {
+            for (int kk = 0; kk < CH / 16; ++kk) {
+                floatx4 vb[DB];
 #pragma unroll
-                for (int kk = 0; kk < CH / 16; ++kk) {
-                    floatx4 fa;
+                for (int db = 0; db < DB; ++db)
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) fa[j] = Fs[(16 * kk + 4 * g + j) * LDF + 16 * rb + r16];
+                    for (int j = 0; j < 4; ++j) vb[db][j] = Vs[(16 * kk + 4 * g + j) * LDV + 16 * db + r16];
 #pragma unroll
-                    for (int db = 0; db < D / 16; ++db) {
-                        floatx4 vb;
+                for (int x = 0; x < RB; ++x) {
+                    const int rb = w + 4 * x;
+                    if (rb < M / 16) {
+                        floatx4 fa;
 #pragma unroll
-                        for (int j = 0; j < 4; ++j) vb[j] = Vs[(16 * kk + 4 * g + j) * LDV + 16 * db + r16];
-                        kvacc[x][db] = Frag<float>::mma(fa, vb, kvacc[x][db]);
+                        for (int j = 0; j < 4; ++j) fa[j] = Fs[(16 * kk + 4 * g + j) * LDF + 16 * rb + r16];
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+#pragma unroll
+                            for (int db = 0; db < DB; ++db)
+                                kvacc[x][db] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[j], vb[db][j], kvacc[x][db], 0, 0, 0);
                     }
                 }
             }
         }
-        if (tid < M) {
-            float s = 0.f;
-            for (int row = 0; row < CH; ++row) s += Fs[row * LDF + tid];
-            ksum_acc += s;
+        __syncthreads();                          // everyone is done with this chunk's tiles
+        if (c + 1 < c1) {
+            kt.template stash<LDK>(Ks, tid);
+            vt.template stash<LDV>(Vs, tid);
         }
+        __syncthreads();                          // next tile visible; Fs and red free again
     }
 
+    // partial K'^T V in accumulator order (tile (rb, db) -> 64 lanes x 4 floats): 16-byte stores,
+    // sb_combine_kernel undoes the order
     float* part = a.kv_part + ((long)bh * a.n_split + sp) * (M * (D + 1));
 #pragma unroll
     for (int x = 0; x < RB; ++x) {
         const int rb = w + 4 * x;
         if (rb < M / 16) {
 #pragma unroll
-            for (int db = 0; db < D / 16; ++db)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) part[(16 * rb + 4 * g + i) * D + 16 * db + r16] = kvacc[x][db][i];
+            for (int db = 0; db < DB; ++db)
+                *reinterpret_cast<floatx4*>(part + ((rb * DB + db) * 64 + lane) * 4) = kvacc[x][db];
         }
     }
-    if (tid < M) part[M * D + tid] = ksum_acc;
-    if (tid == 0) a.part_max[(long)bh * a.n_split + sp] = run_max;
+    // column sums of K': over the 16 key lanes of a wave (DPP), then over the 4 waves (LDS)
+    float* ks_lds = Fs;                           // 4 x M floats
+#pragma unroll
+    for (int fb = 0; fb < FB; ++fb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float p = row16_sum(ksp[fb][i]), n = row16_sum(ksn[fb][i]);
+            if (r16 == 0) {
+                ks_lds[w * M + 16 * fb + 4 * g + i] = p;
+                ks_lds[w * M + MH + 16 * fb + 4 * g + i] = n;
+            }
+        }
+    __syncthreads();
+    if (tid < M) part[M * D + tid] = (ks_lds[tid] + ks_lds[M + tid]) + (ks_lds[2 * M + tid] + ks_lds[3 * M + tid]);
+    if (tid == 0) a.part_max[(long)bh * a.n_split + sp] = run_max * LN2;
 }
 
 // KV = sum_s exp(part_max_s - kmax) KV_s, same for Ksum; one thread per output element, the
@@ -276,12 +315,21 @@ __global__ __launch_bounds__(256) void sb_combine_kernel(const float* kv_part, c
     __syncthreads();
     if (idx == 0) kmax_out[bh] = (kmax == -INFINITY) ? 0.f : kmax;
     if (idx >= per) return;
+    // threads walk a partial in its storage order (coalesced reads over the splits); the K'^T V part
+    // is in accumulator order: offset ((tile*64 + lane)*4 + i) holds element (r, d) of tile
+    // (r/16, d/16) with lane = 16*((r%16)/4) + d%16 and i = r%4
     const float* src = kv_part + (long)bh * n_split * per + idx;
     float acc = 0.f;
 #pragma unroll 16
     for (int s = 0; s < n_split; ++s) acc += wgt[s] * src[(long)s * per];
-    if (idx < M * D) kv[(long)bh * M * D + idx] = acc;
-    else ksum[(long)bh * M + idx - M * D] = acc;
+    if (idx < M * D) {
+        const int i = idx & 3, lane = (idx >> 2) & 63, tile = idx >> 8;
+        const int db_n = D >> 4, rb = tile / db_n, db = tile % db_n;
+        const int r = 16 * rb + 4 * (lane >> 4) + i, d = 16 * db + (lane & 15);
+        kv[(long)bh * M * D + r * D + d] = acc;
+    } else {
+        ksum[(long)bh * M + idx - M * D] = acc;
+    }
 }
 
 // ---------------------------------------------------------------------------------------
@@ -629,7 +677,8 @@ __global__ __launch_bounds__(NT) void sb_merge_kernel(FwdArgs a, int D) {
 // host side
 // ---------------------------------------------------------------------------------------
 template <int E, int M> constexpr size_t kfeat_smem() {
-    return sizeof(float) * ((M / 2) * (E + 4) + CH * (E + 4) + CH * (E + 4) + CH * (M + 4) + 8);
+    // one K and one V tile, one feature tile, reduction scratch
+    return sizeof(float) * (2 * CH * (E + 4) + CH * (M + 4) + 8);
 }
 template <int E, int M> constexpr size_t fwd_smem() {
     constexpr size_t stage = (size_t)TK * ((E + 4) + (E + 4) + (M + 4));
