@@ -155,6 +155,10 @@ def bench_blocksparse(steps, warmup):
     out['dsd'] = {'ms': ms, 'tflops': flops / ms / 1e9, 'gbs': (sp_bytes + 2 * dense_bytes) / ms / 1e6}
     for st in out.values():
         st['hbm_frac'] = st['gbs'] / PEAK_HBM_GBS
+    # what a plain device copy of the sparse tensor reaches on this box (read + write bytes per second)
+    dst = torch.empty_like(qk)
+    ms = timeit(lambda: dst.copy_(qk))
+    out['plain_copy_gbs'] = 2 * sp_bytes / ms / 1e6
     out['config'] = f'bf16 B={B} H={H} L={L} d={d} block={block} nnz/head={nnz // H}'
     return out
 

@@ -95,7 +95,10 @@ __global__ __launch_bounds__(256) void bs_sdd32_kernel(SddRowArgs a) {
     const int head = brow / a.brows_per_head, bi = brow % a.brows_per_head;
     const int p0 = a.row_ptr[brow], nb = a.row_ptr[brow + 1] - p0;
     const T* ap = reinterpret_cast<const T*>(a.a) + z * a.a_sz + head * a.a_sh + (long)(bi * 32 + r16) * a.a_sm + 8 * g;
-    const T* bp = reinterpret_cast<const T*>(a.b) + z * a.b_sz + head * a.b_sh + (long)r16 * a.b_sn + 8 * g;
+    // MFMA row i of B-tile tn is block column 8*(i/4) + 4*tn + i%4: the four results a lane gets from
+    // tile 0 and the four from tile 1 are then eight consecutive columns -> one 16-byte store
+    const T* bp = reinterpret_cast<const T*>(a.b) + z * a.b_sz + head * a.b_sh +
+                  (long)(8 * (r16 >> 2) + (r16 & 3)) * a.b_sn + 8 * g;
     T* cz = reinterpret_cast<T*>(a.c) + (long)z * a.nnz * 1024;
     uint4 fa[2][KS];
 #pragma unroll
@@ -109,7 +112,7 @@ __global__ __launch_bounds__(256) void bs_sdd32_kernel(SddRowArgs a) {
         for (int tn = 0; tn < 2; ++tn)
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks)
-                fb[tn][ks] = *reinterpret_cast<const uint4*>(bp + (brow_b + 16 * tn) * a.b_sn + 32 * ks);
+                fb[tn][ks] = *reinterpret_cast<const uint4*>(bp + (brow_b + 4 * tn) * a.b_sn + 32 * ks);
         floatx4 acc[2][2];
 #pragma unroll
         for (int tm = 0; tm < 2; ++tm)
@@ -119,12 +122,10 @@ __global__ __launch_bounds__(256) void bs_sdd32_kernel(SddRowArgs a) {
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) acc[tm][tn] = Frag32<T>::mma(fb[tn][ks], fa[tm][ks], acc[tm][tn]);
             }
-        // lane holds C[m = 16tm + r16][n = 16tn + 4g + i]
+        // lane holds C[m = 16tm + r16][n = 8g + 4tn + i]: rows of 64 bytes, 16 consecutive rows per store
         T* cp = cz + (long)a.row_blk[p0 + j] * 1024;
 #pragma unroll
-        for (int tm = 0; tm < 2; ++tm)
-#pragma unroll
-            for (int tn = 0; tn < 2; ++tn) store4_f32(cp + (16 * tm + r16) * 32 + 16 * tn + 4 * g, acc[tm][tn]);
+        for (int tm = 0; tm < 2; ++tm) store8_f32(cp + (16 * tm + r16) * 32 + 8 * g, acc[tm][0], acc[tm][1]);
     }
 }
 
@@ -443,7 +444,9 @@ __global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     fx[i] = *reinterpret_cast<const uint4*>(&xs[cur][(64 * wm + 16 * i + r16) * LD + 32 * kb + 8 * g]);
-                    fw[i] = *reinterpret_cast<const uint4*>(&ws[cur][(64 * wn + 16 * i + r16) * LD + 32 * kb + 8 * g]);
+                    // W-tile i covers output block i/2; its MFMA row r is block row 8*(r/4) + 4*(i%2) + r%4
+                    fw[i] = *reinterpret_cast<const uint4*>(
+                        &ws[cur][(64 * wn + 32 * (i >> 1) + 8 * (r16 >> 2) + 4 * (i & 1) + (r16 & 3)) * LD + 32 * kb + 8 * g]);
                 }
 #pragma unroll
                 for (int tm = 0; tm < 4; ++tm)
@@ -466,7 +469,7 @@ __global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
         if (step + 2 < n_steps) stash(0, rxa, rwa);
         __syncthreads();
     }
-    // lane holds y[m = 64wm + 16tm + r16][n = 64wn + 16tn + 4g + i]
+    // lane holds y[m = 64wm + 16tm + r16][n = 32*(output block) + 8g + 4*(tn%2) + i]: 16-byte stores
     if (!wave_active) return;
     T* cp = reinterpret_cast<T*>(a.c) + z * a.c_sz + head * a.c_sh;
 #pragma unroll
@@ -474,11 +477,10 @@ __global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
         const long m = m0 + 64 * wm + 16 * tm + r16;
         if (m >= a.M) continue;
 #pragma unroll
-        for (int tn = 0; tn < 4; ++tn) {
-            const int ob = 2 * wn + (tn >> 1);
+        for (int o2 = 0; o2 < 2; ++o2) {
+            const int ob = 2 * wn + o2;
             if (ob >= gn) continue;
-            const long n = (long)(bcol0 + ob) * 32 + 16 * (tn & 1) + 4 * g;
-            store4_f32(cp + m * a.c_sm + n, acc[tm][tn]);
+            store8_f32(cp + m * a.c_sm + (long)(bcol0 + ob) * 32 + 8 * g, acc[tm][2 * o2], acc[tm][2 * o2 + 1]);
         }
     }
 }
@@ -587,51 +589,71 @@ __global__ __launch_bounds__(256) void bs_softmax32_kernel(RowArgs a) {
             raw[it] = *reinterpret_cast<const uint4*>(xz + off[it]);
         }
     }
-    // element u (0..7) of block slot `it`, scaled and masked
-    auto value = [&](int it, int u) -> float {
+    // element u (0..7) of block slot `it` as float, unscaled
+    auto elem = [&](int it, int u) -> float {
         const uint32_t word = (&raw[it].x)[u >> 1];
         T e;
         *reinterpret_cast<uint16_t*>(&e) = (u & 1) ? (uint16_t)(word >> 16) : (uint16_t)(word & 0xffffu);
-        float v = Elem<T>::to_f32(e) * a.scale;
-        if (masked) {
-            const long col = (long)a.row_col[p0 + w + 4 * it] * 32 + chunk * 8 + u;
-            if (a.kpm) v += mask_term(a.kpm[z * a.kpm_stride + col], a.kpm_mul);
-            if (a.am) v += mask_term(a.am[grow * a.am_stride + col], a.am_mul);
-        }
+        return Elem<T>::to_f32(e);
+    };
+    // additive mask term of that element (masked launches only)
+    auto mask_of = [&](int it, int u) -> float {
+        const long col = (long)a.row_col[p0 + w + 4 * it] * 32 + chunk * 8 + u;
+        float v = 0.f;
+        if (a.kpm) v += mask_term(a.kpm[z * a.kpm_stride + col], a.kpm_mul);
+        if (a.am) v += mask_term(a.am[grow * a.am_stride + col], a.am_mul);
         return v;
     };
+    // pass 1: row maximum of x*scale (+ masks)
     float mx = -INFINITY;
+    if (!masked && a.scale > 0.f) {              // max commutes with a positive scale: one multiply per lane
 #pragma unroll
-    for (int it = 0; it < MAXB; ++it)
-        if (off[it] >= 0)
+        for (int it = 0; it < MAXB; ++it)
+            if (off[it] >= 0)
 #pragma unroll
-            for (int u = 0; u < 8; ++u) mx = fmaxf(mx, value(it, u));
+                for (int u = 0; u < 8; ++u) mx = fmaxf(mx, elem(it, u));
+        mx *= a.scale;
+    } else {
+#pragma unroll
+        for (int it = 0; it < MAXB; ++it)
+            if (off[it] >= 0)
+#pragma unroll
+                for (int u = 0; u < 8; ++u) mx = fmaxf(mx, elem(it, u) * a.scale + (masked ? mask_of(it, u) : 0.f));
+    }
     mx = fmaxf(mx, __shfl_xor(mx, 1));
     mx = fmaxf(mx, __shfl_xor(mx, 2));
     if (chunk == 0) red[0][w][rl] = mx;
     __syncthreads();
     mx = fmaxf(fmaxf(red[0][0][rl], red[0][1][rl]), fmaxf(red[0][2][rl], red[0][3][rl]));
-    const float mx2 = mx * LOG2E;
+    // pass 2: exponentials (kept as floats in registers) and their sum; -inf - -inf = NaN, kept
+    const float mx2 = mx * LOG2E, scale2 = a.scale * LOG2E;
+    float ev[MAXB][8];
     float sum = 0.f;
 #pragma unroll
     for (int it = 0; it < MAXB; ++it)
         if (off[it] >= 0)
 #pragma unroll
-            for (int u = 0; u < 8; ++u) sum += __builtin_amdgcn_exp2f(value(it, u) * LOG2E - mx2);   // -inf - -inf = NaN, kept
+            for (int u = 0; u < 8; ++u) {
+                float arg = elem(it, u) * scale2 - mx2;
+                if (masked) arg += mask_of(it, u) * LOG2E;
+                ev[it][u] = __builtin_amdgcn_exp2f(arg);
+                sum += ev[it][u];
+            }
     sum += __shfl_xor(sum, 1);
     sum += __shfl_xor(sum, 2);
     if (chunk == 0) red[1][w][rl] = sum;
     __syncthreads();
     sum = (red[1][0][rl] + red[1][1][rl]) + (red[1][2][rl] + red[1][3][rl]);
     const float inv = 1.0f / sum;
+    // pass 3: normalise, round once, store
 #pragma unroll
     for (int it = 0; it < MAXB; ++it)
         if (off[it] >= 0) {
             uint32_t outw[4];
 #pragma unroll
             for (int u2 = 0; u2 < 4; ++u2) {
-                T lo = Elem<T>::from_f32(__builtin_amdgcn_exp2f(value(it, 2 * u2) * LOG2E - mx2) * inv);
-                T hi = Elem<T>::from_f32(__builtin_amdgcn_exp2f(value(it, 2 * u2 + 1) * LOG2E - mx2) * inv);
+                T lo = Elem<T>::from_f32(ev[it][2 * u2] * inv);
+                T hi = Elem<T>::from_f32(ev[it][2 * u2 + 1] * inv);
                 outw[u2] = (uint32_t)*reinterpret_cast<uint16_t*>(&lo) | ((uint32_t)*reinterpret_cast<uint16_t*>(&hi) << 16);
             }
             *reinterpret_cast<uint4*>(xz + off[it]) = make_uint4(outw[0], outw[1], outw[2], outw[3]);
@@ -848,8 +870,12 @@ template <typename T>
 static int launch_softmax(const RowArgs& args, dim3 grid, int max_elems, hipStream_t st) {
     if (sizeof(T) == 2 && args.blk_shift == 5 && max_elems <= 32 * 4 * 16 && (args.x_sz % 8) == 0) {
         dim3 g2(2 * args.n_brow, grid.y);
-        if (max_elems <= 32 * 4 * 8) hipLaunchKernelGGL((bs_softmax32_kernel<T, 8>), g2, dim3(256), 0, st, args);
-        else hipLaunchKernelGGL((bs_softmax32_kernel<T, 16>), g2, dim3(256), 0, st, args);
+        const int slots = (max_elems / 32 + 3) / 4;          // blocks per wave: sizes the register arrays
+#define SM32(N) hipLaunchKernelGGL((bs_softmax32_kernel<T, N>), g2, dim3(256), 0, st, args)
+        if (slots <= 4) SM32(4); else if (slots <= 8) SM32(8); else if (slots <= 10) SM32(10);
+        else if (slots <= 12) SM32(12); else if (slots <= 13) SM32(13); else if (slots <= 14) SM32(14);
+        else SM32(16);
+#undef SM32
         return check_launch("bs_softmax32_kernel");
     }
     if (max_elems <= 64 * 8) hipLaunchKernelGGL((bs_softmax_kernel<T, 8>), grid, dim3(256), 0, st, args);

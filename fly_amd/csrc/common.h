@@ -39,13 +39,17 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef short shortx4 __attribute__((ext_vector_type(4)));
 typedef _Float16 halfx4 __attribute__((ext_vector_type(4)));
 
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+
 __device__ __forceinline__ float bf16_to_f32(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
-__device__ __forceinline__ uint16_t f32_to_bf16(float f) {   // round to nearest even, NaN kept quiet
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (uint16_t)(u >> 16);
+// two floats -> two bf16 in one 32-bit word (low half = first), round to nearest even in hardware
+// (v_cvt_pk_bf16_f32 on gfx950)
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    floatx2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) { return (uint16_t)(pack_bf16x2(f, 0.f) & 0xffffu); }
 
 template <typename T> struct Elem;
 template <> struct Elem<float> {
@@ -78,14 +82,27 @@ __device__ __forceinline__ floatx4 load4_f32(const f16_t* p) {
 __device__ __forceinline__ void store4_f32(float* p, floatx4 v) { *reinterpret_cast<floatx4*>(p) = v; }
 __device__ __forceinline__ void store4_f32(bf16_t* p, floatx4 v) {
     uint2 u;
-    u.x = (uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16);
-    u.y = (uint32_t)f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16);
+    u.x = pack_bf16x2(v[0], v[1]);
+    u.y = pack_bf16x2(v[2], v[3]);
     *reinterpret_cast<uint2*>(p) = u;
 }
 __device__ __forceinline__ void store4_f32(f16_t* p, floatx4 v) {
     halfx4 h = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
     *reinterpret_cast<halfx4*>(p) = h;
 }
+
+// eight consecutive elements (two accumulator quads) with one 16-byte store for 2-byte types
+__device__ __forceinline__ void store8_f32(bf16_t* p, floatx4 a, floatx4 b) {
+    *reinterpret_cast<uint4*>(p) = make_uint4(pack_bf16x2(a[0], a[1]), pack_bf16x2(a[2], a[3]),
+                                              pack_bf16x2(b[0], b[1]), pack_bf16x2(b[2], b[3]));
+}
+__device__ __forceinline__ void store8_f32(f16_t* p, floatx4 a, floatx4 b) {
+    typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
+    halfx8 h = {(_Float16)a[0], (_Float16)a[1], (_Float16)a[2], (_Float16)a[3],
+                (_Float16)b[0], (_Float16)b[1], (_Float16)b[2], (_Float16)b[3]};
+    *reinterpret_cast<halfx8*>(p) = h;
+}
+__device__ __forceinline__ void store8_f32(float* p, floatx4 a, floatx4 b) { store4_f32(p, a); store4_f32(p + 4, b); }
 
 // ---------------------------------------------------------------------------------------
 // 16x16 MFMA "k16" step.  A fragment holds, for lane (r = lane%16, g = lane/16), the four
