@@ -78,20 +78,22 @@ __global__ __launch_bounds__(256) void bs_sdd_kernel(SddArgs a) {
 }
 
 // Fast SDD for 32x32 blocks of a 2-byte type with contiguous contraction (K a multiple of 32, at
-// most 128): one workgroup per (head, block-row).  Every wave loads the A fragments of the block-row
-// once (16-byte loads, kept in registers) and then produces the row's blocks w, w+4, ... one after
-// the other: B fragments with 16-byte loads, 16x16x32 MFMAs, 8-byte stores of a 2 KiB block.
+// most 128): one wave per (head, block-row).  The wave loads the A fragments of its block-row once
+// (16-byte loads, kept in registers) and then produces the row's blocks one after the other: B fragments with 16-byte loads, 16x16x32 MFMAs, 8-byte stores of a 2 KiB block.
 struct SddRowArgs {
     const void* a; const void* b; void* c;
     const int32_t* row_ptr; const int32_t* row_blk; const int32_t* row_col;
-    int nnz, K, brows_per_head;
+    int nnz, K, brows_per_head, n_brow;
     long a_sz, a_sh, a_sm, b_sz, b_sh, b_sn;
 };
 
 template <typename T, int KS>     // KS = K / 32
 __global__ __launch_bounds__(256) void bs_sdd32_kernel(SddRowArgs a) {
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, r16 = lane & 15, g = lane >> 4;
-    const int brow = blockIdx.x, z = blockIdx.y;
+    // one block-row per wave: the four waves of a workgroup walk neighbouring block-rows, whose
+    // column lists mostly coincide, so their B-tile loads meet in the L1 cache
+    const int brow = blockIdx.x * 4 + w, z = blockIdx.y;
+    if (brow >= a.n_brow) return;
     const int head = brow / a.brows_per_head, bi = brow % a.brows_per_head;
     const int p0 = a.row_ptr[brow], nb = a.row_ptr[brow + 1] - p0;
     const T* ap = reinterpret_cast<const T*>(a.a) + z * a.a_sz + head * a.a_sh + (long)(bi * 32 + r16) * a.a_sm + 8 * g;
@@ -105,7 +107,7 @@ __global__ __launch_bounds__(256) void bs_sdd32_kernel(SddRowArgs a) {
     for (int tm = 0; tm < 2; ++tm)
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) fa[tm][ks] = *reinterpret_cast<const uint4*>(ap + 16 * tm * a.a_sm + 32 * ks);
-    for (int j = w; j < nb; j += 4) {
+    for (int j = 0; j < nb; ++j) {
         const long brow_b = (long)a.row_col[p0 + j] * 32;
         uint4 fb[2][KS];
 #pragma unroll
@@ -774,8 +776,8 @@ extern "C" int flyhip_bs_sdd(const void* a, const void* b, void* c, const int32_
     if (row_ptr && row_blk && row_col && blk == 32 && (dtype == BF16 || dtype == F16) && a_sk == 1 && b_sk == 1 &&
         K % 32 == 0 && K <= 128 && ((a_sz | a_sh | a_sm | b_sz | b_sh | b_sn) % 8) == 0 && n_brow > 0 &&
         brows_per_head > 0) {
-        SddRowArgs ra{a, b, c, row_ptr, row_blk, row_col, nnz, K, brows_per_head, a_sz, a_sh, a_sm, b_sz, b_sh, b_sn};
-        dim3 grid(n_brow, Z);
+        SddRowArgs ra{a, b, c, row_ptr, row_blk, row_col, nnz, K, brows_per_head, n_brow, a_sz, a_sh, a_sm, b_sz, b_sh, b_sn};
+        dim3 grid((n_brow + 3) / 4, Z);
 #define SDD32_LAUNCH(T)                                                                         \
         switch (K / 32) {                                                                       \
             case 1: hipLaunchKernelGGL((bs_sdd32_kernel<T, 1>), grid, dim3(256), 0, st, ra); break; \
