@@ -3,7 +3,12 @@ src/models/attention/blocksparse_matmul.py:590-719 (modes 'sdd', 'dsd', 'dds')."
 import torch
 
 from . import _lib
-from .blocksparse_utils import group_table, sdd_table, segment_table
+from .blocksparse_utils import group_table, sdd_table, segment_table, union_table
+
+# Sharing the dense operand's tiles among four block-rows pays when the rows have columns in
+# common: the union tables are passed to the kernels when the layout has at least this many
+# (row, column) pairs per union column on average.
+UNION_MIN_SHARING = 1.5
 
 _BLOCKS = (16, 32, 64, 128)
 
@@ -88,6 +93,10 @@ class matmul:
                 tabs = (sdd_table(self.layout),)
             elif kind in ('grp_rows', 'grp_cols'):
                 tabs = group_table(self.layout, by_rows=(kind == 'grp_rows'))
+            elif kind == 'union':
+                tabs = union_table(self.layout)
+                if int(self.layout.sum()) < UNION_MIN_SHARING * tabs[1].numel():
+                    tabs = ()
             else:
                 tabs = segment_table(self.layout, by_rows=(kind == 'rows'))
             self.lut_cache[key] = tuple(t.to(device) for t in tabs)
@@ -164,13 +173,14 @@ class matmul:
                              f'{tuple(self.spdims)} with block {self.block}')
         (lut,) = self._table('sdd', a.device)
         row_ptr, row_blk, row_col = self._table('rows', a.device)
+        uni = [t.data_ptr() for t in self._table('union', a.device)] or [None] * 3
         nnz = lut.shape[0]
         c = torch.empty((Z, nnz, self.block, self.block), dtype=a.dtype, device=a.device)
         a_sm, a_sk = (a.stride(3), a.stride(2)) if trans_a else (a.stride(2), a.stride(3))
         b_sn, b_sk = (b.stride(2), b.stride(3)) if trans_b else (b.stride(3), b.stride(2))
         with torch.cuda.device(a.device):
             _lib.call('flyhip_bs_sdd', a.data_ptr(), b.data_ptr(), c.data_ptr(), lut.data_ptr(), nnz,
-                      row_ptr.data_ptr(), row_blk.data_ptr(), row_col.data_ptr(), H * p, p,
+                      row_ptr.data_ptr(), row_blk.data_ptr(), row_col.data_ptr(), H * p, p, *uni,
                       Z, K, self.block, a.stride(0), a.stride(1), a_sm, a_sk,
                       b.stride(0), b.stride(1), b_sn, b_sk, _lib.dtype_code(a), _lib.stream_ptr(a.device))
         return c
@@ -181,6 +191,7 @@ class matmul:
         H, p, r = self.spdims
         by_rows = not trans_a
         seg_ptr, seg_blk, seg_inner = self._table('rows' if by_rows else 'cols', b.device)
+        uni = ([t.data_ptr() for t in self._table('union', b.device)] if by_rows else []) or [None] * 3
         per_head = p if by_rows else r
         M = per_head * self.block
         Z = b.shape[0]
@@ -190,7 +201,7 @@ class matmul:
         c_sm, c_sn = (c.stride(3), c.stride(2)) if trans_c else (c.stride(2), c.stride(3))
         with torch.cuda.device(b.device):
             _lib.call('flyhip_bs_dsd', a.data_ptr(), b.data_ptr(), c.data_ptr(),
-                      seg_ptr.data_ptr(), seg_blk.data_ptr(), seg_inner.data_ptr(),
+                      seg_ptr.data_ptr(), seg_blk.data_ptr(), seg_inner.data_ptr(), *uni,
                       H * per_head, per_head, Z, N, self.block, int(trans_a), a.stride(0),
                       b.stride(0), b.stride(1), b_sk, b_sn, c.stride(0), c.stride(1), c_sm, c_sn,
                       _lib.dtype_code(b), _lib.stream_ptr(b.device))

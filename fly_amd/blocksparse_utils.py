@@ -101,6 +101,27 @@ def row_table(layout):
     return ptr, blk, col, int(counts.max()) if counts.numel() else 0
 
 
+def union_table(layout, rows_per_group=4):
+    """Union of block-columns over groups of `rows_per_group` consecutive block-rows of a head
+    (ceil(rows / rows_per_group) groups per head, head-major): returns (uni_ptr int32 (n_groups+1),
+    uni_inner int32 (n_union) block-columns in increasing order per group, uni_blk int32
+    (n_union, rows_per_group) the block id at (row rows_per_group*g + w, that column) or -1)."""
+    layout = _as_layout3(layout).cpu().long()
+    H, p, r = layout.shape
+    R = rows_per_group
+    G = (p + R - 1) // R
+    ids = (torch.cumsum(layout.reshape(-1), 0) - 1).reshape(H, p, r)
+    ids = torch.where(layout > 0, ids, torch.full_like(ids, -1))
+    pad = torch.full((H, G * R - p, r), -1, dtype=ids.dtype)
+    ids = torch.cat([ids, pad], dim=1).reshape(H, G, R, r)
+    nz = (ids >= 0).any(dim=2).nonzero(as_tuple=False)              # (h, g, col), sorted
+    blk = ids[nz[:, 0], nz[:, 1], :, nz[:, 2]]                      # (n_union, R)
+    counts = torch.bincount(nz[:, 0] * G + nz[:, 1], minlength=H * G)
+    ptr = torch.zeros(H * G + 1, dtype=torch.int64)
+    ptr[1:] = torch.cumsum(counts, 0)
+    return ptr.to(torch.int32), nz[:, 2].to(torch.int32).contiguous(), blk.to(torch.int32).contiguous()
+
+
 def group_table(layout, by_rows, max_group=4):
     """Groups of up to `max_group` consecutive segments (of one head) whose reduction lists visit the
     same inner blocks: returns (grp_row0 int32, grp_n int32).  Every segment belongs to one group."""

@@ -80,21 +80,38 @@ __global__ __launch_bounds__(256) void bs_sdd_kernel(SddArgs a) {
 // Fast SDD for 32x32 blocks of a 2-byte type with contiguous contraction (K a multiple of 32, at
 // most 128): one wave per (head, block-row).  The wave loads the A fragments of its block-row once
 // (16-byte loads, kept in registers) and then produces the row's blocks one after the other: B fragments with 16-byte loads, 16x16x32 MFMAs, 8-byte stores of a 2 KiB block.
+// The hardware hands consecutive workgroup ids to the eight XCDs in turn, and every XCD has an L2
+// of its own.  unit_of() turns a 1-D workgroup id into (unit, position inside the unit) such
+// that all `per_unit` workgroups of a unit -- one (batch, head) matrix, whose dense operand they
+// all re-read -- run on one XCD, so that operand comes from HBM once instead of once per XCD.
+constexpr int BS_XCD = 8;
+__device__ __forceinline__ bool unit_of(unsigned id, int per_unit, int n_units, int& unit, int& pos) {
+    const unsigned xcd = id % BS_XCD, slot = id / BS_XCD;
+    unit = (int)(slot / per_unit) * BS_XCD + (int)xcd;
+    pos = (int)(slot % per_unit);
+    return unit < n_units;
+}
+static long unit_grid(long n_units, long per_unit) { return (n_units + BS_XCD - 1) / BS_XCD * BS_XCD * per_unit; }
+
 struct SddRowArgs {
     const void* a; const void* b; void* c;
     const int32_t* row_ptr; const int32_t* row_blk; const int32_t* row_col;
-    int nnz, K, brows_per_head, n_brow;
+    int nnz, K, brows_per_head, n_heads, Z;
     long a_sz, a_sh, a_sm, b_sz, b_sh, b_sn;
 };
 
+constexpr int SDD_RING = 3;
+
 template <typename T, int KS>     // KS = K / 32
-__global__ __launch_bounds__(256) void bs_sdd32_kernel(SddRowArgs a) {
+__global__ __launch_bounds__(256) void bs_sdd32_kernel(const SddRowArgs a) {
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, r16 = lane & 15, g = lane >> 4;
     // one block-row per wave: the four waves of a workgroup walk neighbouring block-rows, whose
     // column lists mostly coincide, so their B-tile loads meet in the L1 cache
-    const int brow = blockIdx.x * 4 + w, z = blockIdx.y;
-    if (brow >= a.n_brow) return;
-    const int head = brow / a.brows_per_head, bi = brow % a.brows_per_head;
+    int unit, grp;
+    if (!unit_of(blockIdx.x, (a.brows_per_head + 3) / 4, a.n_heads * a.Z, unit, grp)) return;
+    const int z = unit / a.n_heads, head = unit % a.n_heads, bi = grp * 4 + w;
+    if (bi >= a.brows_per_head) return;
+    const int brow = head * a.brows_per_head + bi;
     const int p0 = a.row_ptr[brow], nb = a.row_ptr[brow + 1] - p0;
     const T* ap = reinterpret_cast<const T*>(a.a) + z * a.a_sz + head * a.a_sh + (long)(bi * 32 + r16) * a.a_sm + 8 * g;
     // MFMA row i of B-tile tn is block column 8*(i/4) + 4*tn + i%4: the four results a lane gets from
@@ -102,32 +119,139 @@ __global__ __launch_bounds__(256) void bs_sdd32_kernel(SddRowArgs a) {
     const T* bp = reinterpret_cast<const T*>(a.b) + z * a.b_sz + head * a.b_sh +
                   (long)(8 * (r16 >> 2) + (r16 & 3)) * a.b_sn + 8 * g;
     T* cz = reinterpret_cast<T*>(a.c) + (long)z * a.nnz * 1024;
+    if (nb == 0) return;
     uint4 fa[2][KS];
 #pragma unroll
     for (int tm = 0; tm < 2; ++tm)
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) fa[tm][ks] = *reinterpret_cast<const uint4*>(ap + 16 * tm * a.a_sm + 32 * ks);
-    for (int j = 0; j < nb; ++j) {
-        const long brow_b = (long)a.row_col[p0 + j] * 32;
-        uint4 fb[2][KS];
+    // B tiles travel through a ring of SDD_RING register sets: the loads of block j + SDD_RING - 1
+    // are issued before block j is multiplied and stored, so a wave keeps several tiles in flight
+    uint4 fb[SDD_RING][2][KS];
+    auto fetch = [&](uint4 (&dst)[2][KS], int j) {
+        const long brow_b = (long)a.row_col[p0 + min(j, nb - 1)] * 32;
 #pragma unroll
         for (int tn = 0; tn < 2; ++tn)
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks)
-                fb[tn][ks] = *reinterpret_cast<const uint4*>(bp + (brow_b + 4 * tn) * a.b_sn + 32 * ks);
-        floatx4 acc[2][2];
+                dst[tn][ks] = *reinterpret_cast<const uint4*>(bp + (brow_b + 4 * tn) * a.b_sn + 32 * ks);
+    };
 #pragma unroll
-        for (int tm = 0; tm < 2; ++tm)
+    for (int u = 0; u < SDD_RING - 1; ++u) fetch(fb[u], u);
+    for (int j0 = 0; j0 < nb; j0 += SDD_RING) {
 #pragma unroll
-            for (int tn = 0; tn < 2; ++tn) {
-                acc[tm][tn] = Frag<float>::zero();
+        for (int u = 0; u < SDD_RING; ++u) {
+            const int j = j0 + u;
+            if (j >= nb) break;
+            fetch(fb[(u + SDD_RING - 1) % SDD_RING], j + SDD_RING - 1);
+            floatx4 acc[2][2];
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) acc[tm][tn] = Frag32<T>::mma(fb[tn][ks], fa[tm][ks], acc[tm][tn]);
-            }
-        // lane holds C[m = 16tm + r16][n = 8g + 4tn + i]: rows of 64 bytes, 16 consecutive rows per store
-        T* cp = cz + (long)a.row_blk[p0 + j] * 1024;
+            for (int tm = 0; tm < 2; ++tm)
 #pragma unroll
-        for (int tm = 0; tm < 2; ++tm) store8_f32(cp + (16 * tm + r16) * 32 + 8 * g, acc[tm][0], acc[tm][1]);
+                for (int tn = 0; tn < 2; ++tn) {
+                    acc[tm][tn] = Frag<float>::zero();
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) acc[tm][tn] = Frag32<T>::mma(fb[u][tn][ks], fa[tm][ks], acc[tm][tn]);
+                }
+            // lane holds C[m = 16tm + r16][n = 8g + 4tn + i]: rows of 64 bytes, 16 consecutive rows per store
+            T* cp = cz + (long)a.row_blk[p0 + j] * 1024;
+#pragma unroll
+            for (int tm = 0; tm < 2; ++tm) store8_f32(cp + (16 * tm + r16) * 32 + 8 * g, acc[tm][0], acc[tm][1]);
+        }
+    }
+}
+
+// SDD for layouts whose neighbouring block-rows share most of their columns (band and butterfly
+// patterns do): one workgroup per (batch, head, four consecutive block-rows), wave w owning row
+// 4*group + w with its A fragments in registers.  The workgroup walks the union of the four
+// column lists (uni_inner), stages each 32 x K tile of B once in LDS -- a quarter of the cache
+// traffic of the one-wave-per-row kernel -- and every wave whose row holds that column
+// (uni_blk[step][w] >= 0) multiplies and stores its 2 KiB block.  Tiles are double-buffered:
+// the global loads of step s+1 are in flight while step s is multiplied.
+struct SddUniArgs {
+    const void* a; const void* b; void* c;
+    const int32_t* uni_ptr; const int32_t* uni_inner; const int32_t* uni_blk;
+    int nnz, brows_per_head, grps_per_head, n_heads, Z;
+    long a_sz, a_sh, a_sm, b_sz, b_sh, b_sn;
+};
+
+template <typename T, int KS>     // KS = K / 32
+__global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
+    constexpr int K = 32 * KS, LD = K + 8;              // LDS row stride: 16 rows of a tile hit all banks once
+    constexpr int CPR = K / 8;                          // 16-byte chunks per tile row
+    constexpr int NCH = (32 * CPR + 255) / 256;         // chunks per thread
+    __shared__ __attribute__((aligned(16))) uint16_t tile[2][32 * LD];
+    const int tid = threadIdx.x, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    int unit, grp;
+    if (!unit_of(blockIdx.x, a.grps_per_head, a.n_heads * a.Z, unit, grp)) return;
+    const int z = unit / a.n_heads, head = unit % a.n_heads;
+    const int ug = head * a.grps_per_head + grp;
+    const int p0 = a.uni_ptr[ug], n = a.uni_ptr[ug + 1] - p0;
+    if (n == 0) return;
+    const int bi = grp * 4 + w;
+    const bool have_row = bi < a.brows_per_head;
+    const T* ap = reinterpret_cast<const T*>(a.a) + z * a.a_sz + head * a.a_sh +
+                  (long)(min(bi, a.brows_per_head - 1) * 32 + r16) * a.a_sm + 8 * g;
+    const T* bz = reinterpret_cast<const T*>(a.b) + z * a.b_sz + head * a.b_sh;
+    T* cz = reinterpret_cast<T*>(a.c) + (long)z * a.nnz * 1024;
+    uint4 fa[2][KS];
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) fa[tm][ks] = *reinterpret_cast<const uint4*>(ap + 16 * tm * a.a_sm + 32 * ks);
+
+    // staging: chunk c = tid + 256 i is 16 bytes of tile row c / CPR.  Block column n lands in LDS row
+    // 16*((n>>2)&1) + 4*(n>>3) + (n&3), so that MFMA tile tn reads the 16 consecutive LDS rows
+    // 16 tn .. 16 tn + 15 and its row i is block column 8*(i/4) + 4*tn + i%4: the four results a lane
+    // gets from tile 0 and the four from tile 1 are eight consecutive columns -> one 16-byte store
+    uint4 reg[NCH];
+    auto fetch = [&](int s) {
+        const long brow_b = (long)a.uni_inner[p0 + s] * 32;
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int c = tid + 256 * i;
+            if (c < 32 * CPR) reg[i] = *reinterpret_cast<const uint4*>(bz + (brow_b + c / CPR) * a.b_sn + 8 * (c % CPR));
+        }
+    };
+    auto stash = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int c = tid + 256 * i, nrow = c / CPR;
+            const int lrow = 16 * ((nrow >> 2) & 1) + 4 * (nrow >> 3) + (nrow & 3);
+            if (c < 32 * CPR) *reinterpret_cast<uint4*>(&tile[buf][lrow * LD + 8 * (c % CPR)]) = reg[i];
+        }
+    };
+    fetch(0);
+    stash(0);
+    __syncthreads();
+    for (int s = 0; s < n; ++s) {
+        const int blk = a.uni_blk[(long)(p0 + s) * 4 + w];
+        if (s + 1 < n) fetch(s + 1);
+        if (blk >= 0 && have_row) {
+            const uint16_t* tp = tile[s & 1];
+            floatx4 acc[2][2];
+            uint4 fb[2][KS];
+#pragma unroll
+            for (int tn = 0; tn < 2; ++tn)
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks)
+                    fb[tn][ks] = *reinterpret_cast<const uint4*>(tp + (16 * tn + r16) * LD + 32 * ks + 8 * g);
+#pragma unroll
+            for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+                for (int tn = 0; tn < 2; ++tn) {
+                    acc[tm][tn] = Frag<float>::zero();
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) acc[tm][tn] = Frag32<T>::mma(fb[tn][ks], fa[tm][ks], acc[tm][tn]);
+                }
+            // lane holds C[m = 16tm + r16][n = 8g + 4tn + i]
+            T* cp = cz + (long)blk * 1024;
+#pragma unroll
+            for (int tm = 0; tm < 2; ++tm) store8_f32(cp + (16 * tm + r16) * 32 + 8 * g, acc[tm][0], acc[tm][1]);
+        }
+        if (s + 1 < n) stash((s + 1) & 1);
+        __syncthreads();
     }
 }
 
@@ -141,6 +265,7 @@ struct DxdArgs {
     long sp_sz;
     long dn_sz, dn_sh, dn_s0, dn_s1;    // DSD: (k, n) strides; DDS: (m, k) strides
     long c_sz, c_sh, c_sm, c_sn;
+    int Z;
 };
 
 template <typename T, int BLK>
@@ -217,8 +342,11 @@ __global__ __launch_bounds__(256) void bs_dsd32_kernel(DxdArgs a) {
     __shared__ __attribute__((aligned(16))) uint16_t vt[4][32 * DSD_LD];
     __shared__ float part[4][32][64 + 1];
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
-    const int seg = blockIdx.x, n0 = blockIdx.y * 64, z = blockIdx.z;
-    const int head = seg / a.per_head, brow = seg % a.per_head;
+    const int ntn = (a.X + 63) / 64, n_heads = a.n_seg / a.per_head;
+    int unit, pos;
+    if (!unit_of(blockIdx.x, a.per_head * ntn, n_heads * a.Z, unit, pos)) return;
+    const int z = unit / n_heads, head = unit % n_heads, brow = pos / ntn, n0 = (pos % ntn) * 64;
+    const int seg = head * a.per_head + brow;
     const T* spz = reinterpret_cast<const T*>(a.sp) + z * a.sp_sz;
     const T* dnp = reinterpret_cast<const T*>(a.dn) + z * a.dn_sz + head * a.dn_sh;
     const int ncols = min(64, a.X - n0);            // valid columns of this tile (a multiple of 8)
@@ -286,6 +414,106 @@ __global__ __launch_bounds__(256) void bs_dsd32_kernel(DxdArgs a) {
         store4_f32(cp, lo);
         store4_f32(cp + 4, hi);
     }
+}
+
+// DSD for layouts whose neighbouring block-rows share most of their columns: one workgroup per
+// (batch, head, four consecutive block-rows, 64-column tile of the dense operand), wave w owning
+// output rows of block-row 4*group + w -- no split of the reduction, so no partial sums to merge.
+// The workgroup walks the union of the four column lists; each 32 x 64 tile of the dense operand
+// is loaded once (16-byte global loads) and written to LDS transposed, [column][k], which turns the
+// MFMA fragment of a [k][n] operand into one 16-byte LDS read.  Sparse blocks come straight from
+// global memory, each read by exactly one wave.  Tiles and sparse fragments of step s+1 are in
+// flight while step s is multiplied.
+struct DsdUniArgs {
+    const void* sp; const void* dn; void* c;
+    const int32_t* uni_ptr; const int32_t* uni_inner; const int32_t* uni_blk;
+    int per_head, grps_per_head, n_heads, Z, N;
+    long sp_sz, dn_sz, dn_sh, dn_sk, c_sz, c_sh, c_sm;
+};
+constexpr int DSDU_LD = 40;     // LDS row stride in elements ([column][k], 32 k + 8): 16 columns hit all banks once
+
+template <typename T>
+__global__ __launch_bounds__(256) void bs_dsd32u_kernel(const DsdUniArgs a) {
+    __shared__ __attribute__((aligned(16))) uint16_t vt[2][64 * DSDU_LD];
+    const int tid = threadIdx.x, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int ntn = (a.N + 63) / 64;
+    int unit, pos;
+    if (!unit_of(blockIdx.x, a.grps_per_head * ntn, a.n_heads * a.Z, unit, pos)) return;
+    const int z = unit / a.n_heads, head = unit % a.n_heads, grp = pos / ntn, n0 = (pos % ntn) * 64;
+    const int ug = head * a.grps_per_head + grp;
+    const int p0 = a.uni_ptr[ug], n = a.uni_ptr[ug + 1] - p0;
+    const int bi = grp * 4 + w;
+    const bool have_row = bi < a.per_head;
+    const int ncols = min(64, a.N - n0);            // valid columns of this tile (a multiple of 8)
+    const T* spz = reinterpret_cast<const T*>(a.sp) + z * a.sp_sz;
+    const T* dnp = reinterpret_cast<const T*>(a.dn) + z * a.dn_sz + head * a.dn_sh + n0;
+
+    floatx4 acc[2][4];
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < 4; ++tn) acc[tm][tn] = Frag<float>::zero();
+
+    // staging: thread holds dense row k = tid / 8, columns c8 .. c8 + 7.  Column n lands in LDS row
+    // 32*(n>>5) + 16*((n>>2)&1) + 4*((n>>3)&3) + (n&3): MFMA tile tn reads LDS rows 16 tn .. 16 tn + 15
+    // and its row i is column 32*(tn/2) + 8*(i/4) + 4*(tn%2) + i%4, so tiles 2q and 2q+1 give a lane
+    // eight consecutive output columns.
+    const int sk = tid >> 3, c8 = 8 * (tid & 7);
+    uint4 stage, fs[2], fs_next[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
+    int blk_next = -1;
+    auto fetch = [&](int s) {
+        const long krow0 = (long)a.uni_inner[p0 + s] * 32;
+        stage = make_uint4(0, 0, 0, 0);
+        if (c8 < ncols) stage = *reinterpret_cast<const uint4*>(dnp + (krow0 + sk) * a.dn_sk + c8);
+        blk_next = have_row ? a.uni_blk[(long)(p0 + s) * 4 + w] : -1;
+        if (blk_next >= 0) {
+            const T* blkp = spz + (long)blk_next * 1024;
+#pragma unroll
+            for (int tm = 0; tm < 2; ++tm) fs_next[tm] = *reinterpret_cast<const uint4*>(blkp + (16 * tm + r16) * 32 + 8 * g);
+        }
+    };
+    auto stash = [&](int buf) {
+        const uint32_t v[4] = {stage.x, stage.y, stage.z, stage.w};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int nn = c8 + i;
+            const int lrow = 32 * (nn >> 5) + 16 * ((nn >> 2) & 1) + 4 * ((nn >> 3) & 3) + (nn & 3);
+            vt[buf][lrow * DSDU_LD + sk] = (uint16_t)(v[i >> 1] >> (16 * (i & 1)));
+        }
+    };
+    if (n > 0) {
+        fetch(0);
+        stash(0);
+    }
+    __syncthreads();
+    for (int s = 0; s < n; ++s) {
+        const int blk = blk_next;
+        fs[0] = fs_next[0];
+        fs[1] = fs_next[1];
+        if (s + 1 < n) fetch(s + 1);
+        if (blk >= 0) {
+            const uint16_t* tp = vt[s & 1];
+#pragma unroll
+            for (int tn = 0; tn < 4; ++tn) {
+                const uint4 fd = *reinterpret_cast<const uint4*>(tp + (16 * tn + r16) * DSDU_LD + 8 * g);
+                acc[0][tn] = Frag32<T>::mma(fd, fs[0], acc[0][tn]);
+                acc[1][tn] = Frag32<T>::mma(fd, fs[1], acc[1][tn]);
+            }
+        }
+        if (s + 1 < n) stash((s + 1) & 1);
+        __syncthreads();
+    }
+    if (!have_row) return;
+    // lane holds C[m = 16tm + r16][n = 32q + 8g + 4(tn%2) + i], tn = 2q, 2q+1
+    T* cp = reinterpret_cast<T*>(a.c) + z * a.c_sz + head * a.c_sh + n0;
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const int nn = 32 * q + 8 * g;
+            if (nn < ncols) store8_f32(cp + ((long)bi * 32 + 16 * tm + r16) * a.c_sm + nn, acc[tm][2 * q], acc[tm][2 * q + 1]);
+        }
 }
 
 // ---------------------------------------------------------------------------------------
@@ -760,6 +988,7 @@ static int check_common(const char* who, int blk, int dtype, int Z) {
 extern "C" int flyhip_bs_sdd(const void* a, const void* b, void* c, const int32_t* lut, int nnz,
                              const int32_t* row_ptr, const int32_t* row_blk, const int32_t* row_col,
                              int n_brow, int brows_per_head,
+                             const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
                              int Z, int K, int blk,
                              int64_t a_sz, int64_t a_sh, int64_t a_sm, int64_t a_sk,
                              int64_t b_sz, int64_t b_sh, int64_t b_sn, int64_t b_sk,
@@ -776,8 +1005,30 @@ extern "C" int flyhip_bs_sdd(const void* a, const void* b, void* c, const int32_
     if (row_ptr && row_blk && row_col && blk == 32 && (dtype == BF16 || dtype == F16) && a_sk == 1 && b_sk == 1 &&
         K % 32 == 0 && K <= 128 && ((a_sz | a_sh | a_sm | b_sz | b_sh | b_sn) % 8) == 0 && n_brow > 0 &&
         brows_per_head > 0) {
-        SddRowArgs ra{a, b, c, row_ptr, row_blk, row_col, nnz, K, brows_per_head, n_brow, a_sz, a_sh, a_sm, b_sz, b_sh, b_sn};
-        dim3 grid((n_brow + 3) / 4, Z);
+        FLY_REQUIRE(n_brow % brows_per_head == 0, "bs_sdd: %d block-rows do not divide into heads of %d", n_brow, brows_per_head);
+        const int n_heads = n_brow / brows_per_head;
+        if (uni_ptr && uni_inner && uni_blk) {
+            const int gph = (brows_per_head + 3) / 4;
+            SddUniArgs ua{a, b, c, uni_ptr, uni_inner, uni_blk, nnz, brows_per_head, gph, n_heads, Z,
+                          a_sz, a_sh, a_sm, b_sz, b_sh, b_sn};
+            const long nwg = unit_grid((long)n_heads * Z, gph);
+            FLY_REQUIRE(nwg <= 2147483647L, "bs_sdd: too many workgroups");
+            dim3 grid((unsigned)nwg);
+#define SDD32U_LAUNCH(T)                                                                         \
+            switch (K / 32) {                                                                    \
+                case 1: hipLaunchKernelGGL((bs_sdd32u_kernel<T, 1>), grid, dim3(256), 0, st, ua); break; \
+                case 2: hipLaunchKernelGGL((bs_sdd32u_kernel<T, 2>), grid, dim3(256), 0, st, ua); break; \
+                case 3: hipLaunchKernelGGL((bs_sdd32u_kernel<T, 3>), grid, dim3(256), 0, st, ua); break; \
+                default: hipLaunchKernelGGL((bs_sdd32u_kernel<T, 4>), grid, dim3(256), 0, st, ua); break; \
+            }
+            if (dtype == BF16) { SDD32U_LAUNCH(bf16_t) } else { SDD32U_LAUNCH(f16_t) }
+#undef SDD32U_LAUNCH
+            return check_launch("bs_sdd32u_kernel");
+        }
+        SddRowArgs ra{a, b, c, row_ptr, row_blk, row_col, nnz, K, brows_per_head, n_heads, Z, a_sz, a_sh, a_sm, b_sz, b_sh, b_sn};
+        const long nwg = unit_grid((long)n_heads * Z, (brows_per_head + 3) / 4);
+        FLY_REQUIRE(nwg <= 2147483647L, "bs_sdd: too many workgroups");
+        dim3 grid((unsigned)nwg);
 #define SDD32_LAUNCH(T)                                                                         \
         switch (K / 32) {                                                                       \
             case 1: hipLaunchKernelGGL((bs_sdd32_kernel<T, 1>), grid, dim3(256), 0, st, ra); break; \
@@ -800,6 +1051,7 @@ extern "C" int flyhip_bs_sdd(const void* a, const void* b, void* c, const int32_
 
 extern "C" int flyhip_bs_dsd(const void* a_sp, const void* b, void* c,
                              const int32_t* seg_ptr, const int32_t* seg_blk, const int32_t* seg_inner,
+                             const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
                              int n_seg, int rows_per_head, int Z, int N, int blk, int trans_a,
                              int64_t a_sz,
                              int64_t b_sz, int64_t b_sh, int64_t b_sk, int64_t b_sn,
@@ -815,10 +1067,23 @@ extern "C" int flyhip_bs_dsd(const void* a_sp, const void* b, void* c,
     FLY_REQUIRE(a_sz % 4 == 0, "bs_dsd: sparse batch stride must be a multiple of 4 elements");
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     DxdArgs args{a_sp, b, c, seg_ptr, seg_blk, seg_inner, n_seg, rows_per_head, N, trans_a,
-                 a_sz, b_sz, b_sh, b_sk, b_sn, c_sz, c_sh, c_sm, c_sn};
+                 a_sz, b_sz, b_sh, b_sk, b_sn, c_sz, c_sh, c_sm, c_sn, Z};
     if (blk == 32 && (dtype == BF16 || dtype == F16) && !trans_a && b_sn == 1 && c_sn == 1 && N % 8 == 0 &&
-        ((a_sz | b_sz | b_sh | b_sk | c_sz | c_sh | c_sm) % 8) == 0 && Z <= 65535 && (N + 63) / 64 <= 65535) {
-        dim3 grid(n_seg, (N + 63) / 64, Z);
+        ((a_sz | b_sz | b_sh | b_sk | c_sz | c_sh | c_sm) % 8) == 0) {
+        if (uni_ptr && uni_inner && uni_blk) {
+            const int gph = (rows_per_head + 3) / 4, n_heads = n_seg / rows_per_head;
+            DsdUniArgs ua{a_sp, b, c, uni_ptr, uni_inner, uni_blk, rows_per_head, gph, n_heads, Z, N,
+                          a_sz, b_sz, b_sh, b_sk, c_sz, c_sh, c_sm};
+            const long nwg = unit_grid((long)n_heads * Z, (long)gph * ((N + 63) / 64));
+            FLY_REQUIRE(nwg <= 2147483647L, "bs_dsd: too many workgroups");
+            dim3 grid((unsigned)nwg);
+            if (dtype == BF16) hipLaunchKernelGGL((bs_dsd32u_kernel<bf16_t>), grid, dim3(256), 0, st, ua);
+            else hipLaunchKernelGGL((bs_dsd32u_kernel<f16_t>), grid, dim3(256), 0, st, ua);
+            return check_launch("bs_dsd32u_kernel");
+        }
+        const long nwg = unit_grid((long)(n_seg / rows_per_head) * Z, (long)rows_per_head * ((N + 63) / 64));
+        FLY_REQUIRE(nwg <= 2147483647L, "bs_dsd: too many workgroups");
+        dim3 grid((unsigned)nwg);
         if (dtype == BF16) hipLaunchKernelGGL((bs_dsd32_kernel<bf16_t>), grid, dim3(256), 0, st, args);
         else hipLaunchKernelGGL((bs_dsd32_kernel<f16_t>), grid, dim3(256), 0, st, args);
         return check_launch("bs_dsd32_kernel");

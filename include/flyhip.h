@@ -93,10 +93,17 @@ int flyhip_sb_time_next_fwd(void* event_before, void* event_after);
  * lut: int32 (nnz,4) rows (head, block_row, block_col, block_id) (ref: make_sdd_lut :261-276).
  * row_ptr / row_blk / row_col (optional, may be NULL): the same blocks grouped per (head, block-row),
  * n_brow = H * rows/blk of them; with these, 32x32 blocks of a 2-byte type take a faster kernel that
- * keeps the A tile of a block-row in registers. */
+ * keeps the A tile of a block-row in registers.
+ * uni_ptr / uni_inner / uni_blk (optional, may be NULL; used with the row tables): for every group of
+ * four consecutive block-rows of a head (ceil(rows/4) groups per head, head-major), the union of
+ * the rows' block-columns in increasing order: uni_ptr int32 (n_groups+1), uni_inner int32 (n_union)
+ * the block-column, uni_blk int32 (n_union,4) the block id of (row 4g+w, that column) or -1.  With
+ * them the four rows share every B tile through LDS; worth passing when neighbouring rows have
+ * most columns in common. */
 int flyhip_bs_sdd(const void* a, const void* b, void* c, const int32_t* lut, int nnz,
                   const int32_t* row_ptr, const int32_t* row_blk, const int32_t* row_col,
                   int n_brow, int brows_per_head,
+                  const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
                   int Z, int K, int blk,
                   int64_t a_sz, int64_t a_sh, int64_t a_sm, int64_t a_sk,
                   int64_t b_sz, int64_t b_sh, int64_t b_sn, int64_t b_sk,
@@ -105,9 +112,13 @@ int flyhip_bs_sdd(const void* a, const void* b, void* c, const int32_t* lut, int
 /* DSD: c (Z,H,M,N) = op(sparse a) . dense b.  Segment s = (head, output block-row); seg_ptr
  * (n_seg+1), seg_blk (block id), seg_inner (inner block index) int32 list the blocks reduced into
  * it; n_seg = H * M/blk; an empty segment writes zeros (ref: make_dxx_lut :356-441 plays this
- * role).  trans_a != 0 reads every sparse block transposed.  b(k,n) and c(m,n) via strides. */
+ * role).  trans_a != 0 reads every sparse block transposed.  b(k,n) and c(m,n) via strides.
+ * uni_ptr / uni_inner / uni_blk (optional, may be NULL; trans_a == 0 only): the union table of
+ * flyhip_bs_sdd over groups of four output block-rows; with it the four rows share every tile of
+ * b through LDS. */
 int flyhip_bs_dsd(const void* a_sp, const void* b, void* c,
                   const int32_t* seg_ptr, const int32_t* seg_blk, const int32_t* seg_inner,
+                  const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
                   int n_seg, int rows_per_head, int Z, int N, int blk, int trans_a,
                   int64_t a_sz,
                   int64_t b_sz, int64_t b_sh, int64_t b_sk, int64_t b_sn,

@@ -165,6 +165,41 @@ def test_blocksparse_linear_and_sparse_lr():
     assert rel_err(y, ref) <= 1e-4
 
 
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('p,r,K,N', [(8, 6, 64, 64), (7, 5, 32, 40), (9, 4, 128, 136), (2, 3, 96, 72)])
+def test_shared_tile_kernels(p, r, K, N, dtype, monkeypatch):
+    """The SDD / DSD kernels that share tiles among four block-rows (32x32 blocks, 2-byte types),
+    forced on for layouts with and without common columns: ragged last group, an empty group, an
+    empty row inside a group, reduction sizes 32..128, dense widths that are not multiples of 64."""
+    from fly_amd import matmul
+    import fly_amd.blocksparse_matmul as bm
+    monkeypatch.setattr(bm, 'UNION_MIN_SHARING', 0.0)
+    print('case', p, r, K, N, dtype, flush=True)
+    block, Z, H = 32, 2, 3
+    layout = random_layout(H, p, r, 7 + p)
+    layout[1] = layout[1, :1].expand(p, r)               # one head whose rows all share their columns
+    if p > 4:
+        layout[0, 4:8] = 0                               # an empty group
+        layout[2, 1] = 0                                 # an empty row inside a group
+    g = torch.Generator().manual_seed(5)
+    a = torch.randn(Z, H, p * block, K, generator=g).to(dtype)
+    b = torch.randn(Z, H, r * block, K, generator=g).to(dtype)
+    c = matmul(layout, block, 'sdd', trans_b=True)(a.to(DEV), b.to(DEV))
+    assert rel_err(c, ob.sdd(a, b, layout, block, trans_b=True)) <= TOL[dtype]
+    nnz = int(layout.sum())
+    sp = torch.randn(Z, nnz, block, block, generator=g).to(dtype)
+    v = torch.randn(Z, H, r * block, N, generator=g).to(dtype)
+    out = matmul(layout, block, 'dsd')(sp.to(DEV), v.to(DEV))
+    assert rel_err(out, ob.dsd(sp, v, layout, block)) <= TOL[dtype]
+    if p > 4:
+        assert float(out[:, 0, 4 * block:8 * block].abs().max()) == 0.0
+        assert float(out[:, 2, block:2 * block].abs().max()) == 0.0
+    # the kernels without tile sharing give the same bits in SDD (same products, same order)
+    monkeypatch.setattr(bm, 'UNION_MIN_SHARING', 1e9)
+    c2 = matmul(layout, block, 'sdd', trans_b=True)(a.to(DEV), b.to(DEV))
+    assert torch.equal(c, c2)
+
+
 def test_config2_layout_stage_parity_reduced():
     """BASELINE config 2 pattern (band +-4 OR flat butterfly (8,2), block 32, bf16) at B=1, H=2."""
     from fly_amd import matmul, softmax, FlatBlockButterflySparsityConfig

@@ -74,6 +74,34 @@ def test_index_tables_bit_exact():
     assert torch.equal(bu.sdd_table(layout[0]), ob.sdd_lut(layout[0]))
 
 
+def test_union_table_against_loops():
+    """Union of block-columns over groups of four block-rows, checked against explicit loops."""
+    for H, p, r, seed in ((2, 7, 5, 4), (1, 4, 9, 5), (3, 1, 3, 6)):
+        layout = _layout(H, p, r, seed)
+        if p > 5:
+            layout[0, 4:8, :] = 0                           # an empty group
+            layout[1, 1, :] = 0                             # an empty row inside a group
+        ids = {}
+        for n, (h, i, j) in enumerate(layout.nonzero().tolist()):
+            ids[(h, i, j)] = n
+        ptr, inner, blk = bu.union_table(layout)
+        assert ptr.dtype == inner.dtype == blk.dtype == torch.int32
+        G = (p + 3) // 4
+        assert ptr.numel() == H * G + 1 and blk.shape == (inner.numel(), 4)
+        want_ptr, want_inner, want_blk = [0], [], []
+        for h in range(H):
+            for gi in range(G):
+                for j in range(r):
+                    row = [ids.get((h, 4 * gi + w, j), -1) for w in range(4)]
+                    if max(row) >= 0:
+                        want_inner.append(j)
+                        want_blk.append(row)
+                want_ptr.append(len(want_inner))
+        assert ptr.tolist() == want_ptr and inner.tolist() == want_inner and blk.tolist() == want_blk
+        # every block appears exactly once
+        assert sorted(x for x in blk.reshape(-1).tolist() if x >= 0) == list(range(int(layout.sum())))
+
+
 def test_format_helpers_bit_exact():
     layout = _layout(2, 3, 4, 2)
     g = torch.Generator().manual_seed(0)
