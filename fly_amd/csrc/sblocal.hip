@@ -1,10 +1,11 @@
 // Scatterbrain-local attention forward for gfx950.
 //
-// Three kernels:
-//   sb_kfeat_kernel   : per (batch, head, range of 64-key chunks): positive random features of
-//                       the keys (projection on fp32 MFMA, wavefront max reductions, exp),
-//                       written to HBM once, plus the partial K'^T V / sum K' reductions with an
-//                       online rescale to the running maximum.
+// Kernels:
+//   sb_kfeat_kernel   : workgroups take one of two roles.  Key role, per (batch, head, range of
+//                       64-key chunks): positive random features of the keys (projection on fp32
+//                       MFMA, wavefront max reductions, exp), written to HBM once, plus the partial
+//                       K'^T V / sum K' reductions with an online rescale to the running maximum.
+//                       Query role (small problems only): the features of 64 queries.
 //   sb_combine_kernel : merges the partial reductions of one (batch, head).
 //   sblocal_fwd_kernel: per (batch, head, 64-query tile, part of the band): query features in
 //                       registers, then for each 32-key tile of its share of the band Q K^T and
@@ -52,11 +53,17 @@ struct KvArgs {
     int B, H, S, mh_valid, n_chunks, n_split;
     long k_sb, k_sh, k_ss, v_sb, v_sh, v_ss;
     float temp;
+    // optional query side: features of the queries and their log-scales, for the band kernel
+    const void* q; float* qfeat; float* q_lsq;
+    int T;
+    long q_sb, q_sh, q_ss;
+    int q_tiles;                    // query-role workgroups per (batch, head), after the n_split key-role ones
 };
 
 struct FwdArgs {
     const void* q; const void* k; const void* v; const float* proj;
     const float* kfeat; const float* chunk_scale; const float* kv; const float* ksum; const float* kmax;
+    const float* qfeat; const float* q_lsq;
     const int64_t* lens; void* out; float* log_norm; float* part_ws;
     int B, H, T, S, mh_valid, lc, n_chunks, n_parts;
     long q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss;
@@ -99,6 +106,43 @@ __device__ __forceinline__ void load_proj(float* Ps, const float* proj, float sc
     t.template stash<E + 4>(Ps, tid, scale);
 }
 
+// KV = sum_s exp(part_max_s - kmax) KV_s, same for Ksum; one thread per output element, the
+// weights staged in LDS so that the loads over s are independent and stay in flight together
+constexpr int MAX_SPLIT = 1024;
+__global__ __launch_bounds__(NT) void sb_combine_kernel(const float* kv_part, const float* part_max, float* kv,
+                                                        float* ksum, float* kmax_out, int n_split, int M, int D) {
+    __shared__ float wgt[MAX_SPLIT];
+    const int bh = blockIdx.y;
+    const int idx = blockIdx.x * NT + threadIdx.x;
+    const int per = M * (D + 1);
+    float kmax = -INFINITY;
+    for (int s = 0; s < n_split; ++s) kmax = fmaxf(kmax, part_max[(long)bh * n_split + s]);
+    for (int s = threadIdx.x; s < n_split; s += NT) {
+        const float pm = part_max[(long)bh * n_split + s];
+        // same expression as the band kernel's chunk weight, so that both sides of the
+        // "global minus band" low-rank difference carry bit-identical factors
+        wgt[s] = (pm == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((pm - kmax) * 1.4426950408889634f);
+    }
+    __syncthreads();
+    if (idx == 0) kmax_out[bh] = (kmax == -INFINITY) ? 0.f : kmax;
+    if (idx >= per) return;
+    // threads walk a partial in its storage order (coalesced reads over the splits); the K'^T V part
+    // is in accumulator order: offset ((tile*64 + lane)*4 + i) holds element (r, d) of tile
+    // (r/16, d/16) with lane = 16*((r%16)/4) + d%16 and i = r%4
+    const float* src = kv_part + (long)bh * n_split * per + idx;
+    float acc = 0.f;
+#pragma unroll 16
+    for (int s = 0; s < n_split; ++s) acc += wgt[s] * src[(long)s * per];
+    if (idx < M * D) {
+        const int i = idx & 3, lane = (idx >> 2) & 63, tile = idx >> 8;
+        const int db_n = D >> 4, rb = tile / db_n, db = tile % db_n;
+        const int r = 16 * rb + 4 * (lane >> 4) + i, d = 16 * db + (lane & 15);
+        kv[(long)bh * M * D + r * D + d] = acc;
+    } else {
+        ksum[(long)bh * M + idx - M * D] = acc;
+    }
+}
+
 // ---------------------------------------------------------------------------------------
 // key features + partial K'^T V
 // ---------------------------------------------------------------------------------------
@@ -112,7 +156,7 @@ void sb_kfeat_kernel(KvArgs a) {
     constexpr int FB = MH / 16, EC = E / 16, DB = D / 16;
     constexpr int RB = (M / 16 + 3) / 4;         // K'^T V row blocks per wave
     constexpr float LOG2E = 1.4426950408889634f, LN2 = 0.6931471805599453f;
-    extern __shared__ float smem[];
+    extern __shared__ __attribute__((aligned(128))) float smem[];
     float* Ks = smem;                             // 64-key K tile
     float* Vs = Ks + CH * LDK;                    // 64-key V tile
     float* Fs = Vs + CH * LDV;                    // features of the current chunk
@@ -120,6 +164,66 @@ void sb_kfeat_kernel(KvArgs a) {
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
     const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H, sp = blockIdx.x;
+    // projection fragments (A side: row = feature 16fb + r16, k = 16cc + 4g + j) come straight from
+    // global memory: the matrix is small and stays in the L1/L2 caches
+    const float* pp = a.proj + r16 * E + 4 * g;
+
+    if (sp >= a.n_split) {
+        // Query role (workgroups past the key splits, present when the caller asks for query
+        // features): q' = exp(+-sqrt(t) P q - max) of 64 queries, one per lane column, with the
+        // per-query log-scale lsq = -t|q|^2/2 + max - log(2 mh)/2.  Lane (r16, g) ends with features
+        // 16c + 4g + i of query 16w + r16, the B-side operand layout of the band kernel.
+        const int iq = (sp - a.n_split) * TQ + 16 * w + r16;
+        const T* qrow = reinterpret_cast<const T*>(a.q) + b * a.q_sb + h * a.q_sh + (long)min(iq, a.T - 1) * a.q_ss;
+        floatx4 qr[EC];
+        float sq = 0.f;
+#pragma unroll
+        for (int c = 0; c < EC; ++c) {
+            qr[c] = load4_f32(qrow + 16 * c + 4 * g);
+            sq += qr[c][0] * qr[c][0] + qr[c][1] * qr[c][1] + qr[c][2] * qr[c][2] + qr[c][3] * qr[c][3];
+        }
+        const float diag_q = 0.5f * a.temp * group_sum(sq);
+        const float st = sqrtf(a.temp);
+        floatx4 qf[FB];
+#pragma unroll
+        for (int fb = 0; fb < FB; ++fb) qf[fb] = Frag<float>::zero();
+#pragma unroll
+        for (int c = 0; c < EC; ++c) {                      // the FB accumulation chains advance together
+            floatx4 pa[FB];
+#pragma unroll
+            for (int fb = 0; fb < FB; ++fb) pa[fb] = *reinterpret_cast<const floatx4*>(pp + 16 * fb * E + 16 * c) * st;
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int fb = 0; fb < FB; ++fb)
+                    qf[fb] = __builtin_amdgcn_mfma_f32_16x16x4f32(pa[fb][j], qr[c][j], qf[fb], 0, 0, 0);
+        }
+        float qmax = 0.f;
+#pragma unroll
+        for (int fb = 0; fb < FB; ++fb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (16 * fb + 4 * g + i < a.mh_valid) qmax = fmaxf(qmax, fabsf(qf[fb][i]));
+        qmax = group_max(qmax);
+        if (iq < a.T) {
+            float* dst = a.qfeat + ((long)bh * a.T + iq) * M;
+#pragma unroll
+            for (int fb = 0; fb < FB; ++fb) {
+                floatx4 fp, fn;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const bool ok = 16 * fb + 4 * g + i < a.mh_valid;
+                    fp[i] = ok ? __expf(qf[fb][i] - qmax) : 0.f;
+                    fn[i] = ok ? __expf(-qf[fb][i] - qmax) : 0.f;
+                }
+                *reinterpret_cast<floatx4*>(dst + 16 * fb + 4 * g) = fp;
+                *reinterpret_cast<floatx4*>(dst + MH + 16 * fb + 4 * g) = fn;
+            }
+            if (g == 0) a.q_lsq[(long)bh * a.T + iq] = -diag_q + qmax - 0.5f * __logf(2.0f * a.mh_valid);
+        }
+        return;
+    }
+
     const T* kptr = reinterpret_cast<const T*>(a.k) + b * a.k_sb + h * a.k_sh;
     const T* vptr = reinterpret_cast<const T*>(a.v) + b * a.v_sb + h * a.v_sh;
     const int len = a.lens ? min((int)a.lens[b], a.S) : a.S;
@@ -133,9 +237,6 @@ void sb_kfeat_kernel(KvArgs a) {
         kt.fetch(kptr, a.k_ss, c0 * CH, a.S - 1, tid);
         vt.fetch(vptr, a.v_ss, c0 * CH, a.S - 1, tid);
     }
-    // projection fragments (A side: row = feature 16fb + r16, k = 16cc + 4g + j) come straight from
-    // global memory: the matrix is small and stays in the L1/L2 caches
-    const float* pp = a.proj + r16 * E + 4 * g;
     const float pscale = sqrtf(a.temp) * LOG2E;                      // projections come out in base-2 units
     if (c0 < c1) {
         kt.template stash<LDK>(Ks, tid);
@@ -267,7 +368,7 @@ void sb_kfeat_kernel(KvArgs a) {
     }
 
     // partial K'^T V in accumulator order (tile (rb, db) -> 64 lanes x 4 floats): 16-byte stores,
-    // sb_combine_kernel undoes the order
+    // the combine role undoes the order
     float* part = a.kv_part + ((long)bh * a.n_split + sp) * (M * (D + 1));
 #pragma unroll
     for (int x = 0; x < RB; ++x) {
@@ -295,41 +396,64 @@ void sb_kfeat_kernel(KvArgs a) {
     if (tid == 0) a.part_max[(long)bh * a.n_split + sp] = run_max * LN2;
 }
 
-// KV = sum_s exp(part_max_s - kmax) KV_s, same for Ksum; one thread per output element, the
-// weights staged in LDS so that the loads over s are independent and stay in flight together
-constexpr int MAX_SPLIT = 1024;
-__global__ __launch_bounds__(256) void sb_combine_kernel(const float* kv_part, const float* part_max, float* kv,
-                                                         float* ksum, float* kmax_out, int n_split, int M, int D) {
-    __shared__ float wgt[MAX_SPLIT];
-    const int bh = blockIdx.y;
-    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
-    const int per = M * (D + 1);
-    float kmax = -INFINITY;
-    for (int s = 0; s < n_split; ++s) kmax = fmaxf(kmax, part_max[(long)bh * n_split + s]);
-    for (int s = threadIdx.x; s < n_split; s += blockDim.x) {
-        const float pm = part_max[(long)bh * n_split + s];
-        // same expression as the band kernel's chunk weight, so that both sides of the
-        // "global minus band" low-rank difference carry bit-identical factors
-        wgt[s] = (pm == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((pm - kmax) * 1.4426950408889634f);
+// Merge of the per-part partials of one query tile by the 256 threads of a workgroup: thread
+// (query ql = tid / 4, column quarter tid % 4).  Parts are taken in batches whose loads are all
+// issued before the first is used (slots past n_parts re-read the last part and are ignored),
+// with an online rescale to the running maximum between batches.
+template <typename T, int D>
+__device__ __forceinline__ void sb_merge_tile(const FwdArgs& a, int bh, int qt, int n_qt) {
+    constexpr float LN2 = 0.6931471805599453f;
+    constexpr int NV = D / 16;                      // floatx4 per thread and part
+    constexpr int PB = D <= 64 ? 8 : 4;             // parts per batch
+    const int tid = threadIdx.x, ql = tid >> 2, d0 = (tid & 3) * (D / 4);
+    const int b = bh / a.H, h = bh % a.H;
+    const int iq = qt * TQ + ql;
+    const long stride = (long)TQ * (D + NSTAT);
+    const float* ws = a.part_ws + ((long)bh * n_qt + qt) * a.n_parts * stride;
+    const float* st = ws + TQ * D + ql;
+    const float qk1 = st[3 * TQ], c0 = st[4 * TQ];  // carried by part 0
+    float m_star = -INFINITY, ze = 0.f, zp = 0.f;
+    floatx4 acc[NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) acc[v] = Frag<float>::zero();
+    for (int p0 = 0; p0 < a.n_parts; p0 += PB) {
+        float mv[PB], zev[PB], zpv[PB];
+        floatx4 ov[PB][NV];
+#pragma unroll
+        for (int j = 0; j < PB; ++j) {
+            const long off = (long)min(p0 + j, a.n_parts - 1) * stride;
+            mv[j] = st[off];
+            zev[j] = st[off + TQ];
+            zpv[j] = st[off + 2 * TQ];
+#pragma unroll
+            for (int v = 0; v < NV; ++v) ov[j][v] = *reinterpret_cast<const floatx4*>(ws + off + ql * D + d0 + 4 * v);
+        }
+        float m_new = m_star;
+#pragma unroll
+        for (int j = 0; j < PB; ++j) m_new = fmaxf(m_new, mv[j]);      // repeated slots repeat a valid value
+        const float keep = (m_star == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_star - m_new);
+        m_star = m_new;
+        ze *= keep;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) acc[v] *= keep;
+#pragma unroll
+        for (int j = 0; j < PB; ++j) {
+            if (p0 + j < a.n_parts) {
+                const float wgt = __builtin_amdgcn_exp2f(mv[j] - m_star);
+                ze += wgt * zev[j];
+                zp += zpv[j];
+#pragma unroll
+                for (int v = 0; v < NV; ++v) acc[v] += wgt * ov[j][v];
+            }
+        }
     }
-    __syncthreads();
-    if (idx == 0) kmax_out[bh] = (kmax == -INFINITY) ? 0.f : kmax;
-    if (idx >= per) return;
-    // threads walk a partial in its storage order (coalesced reads over the splits); the K'^T V part
-    // is in accumulator order: offset ((tile*64 + lane)*4 + i) holds element (r, d) of tile
-    // (r/16, d/16) with lane = 16*((r%16)/4) + d%16 and i = r%4
-    const float* src = kv_part + (long)bh * n_split * per + idx;
-    float acc = 0.f;
-#pragma unroll 16
-    for (int s = 0; s < n_split; ++s) acc += wgt[s] * src[(long)s * per];
-    if (idx < M * D) {
-        const int i = idx & 3, lane = (idx >> 2) & 63, tile = idx >> 8;
-        const int db_n = D >> 4, rb = tile / db_n, db = tile % db_n;
-        const int r = 16 * rb + 4 * (lane >> 4) + i, d = 16 * db + (lane & 15);
-        kv[(long)bh * M * D + r * D + d] = acc;
-    } else {
-        ksum[(long)bh * M + idx - M * D] = acc;
-    }
+    if (iq >= a.T) return;
+    const float Z = ze + __builtin_amdgcn_exp2f(c0 - m_star) * fmaxf(qk1 - zp, 1e-24f);
+    const float inv = 1.0f / Z;
+    T* optr = reinterpret_cast<T*>(a.out) + b * a.o_sb + h * a.o_sh + (long)iq * a.o_ss + d0;
+#pragma unroll
+    for (int v = 0; v < NV; ++v) store4_f32(optr + 4 * v, acc[v] * inv);
+    if ((tid & 3) == 0) a.log_norm[(long)bh * a.T + iq] = m_star * LN2 + __logf(Z);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -340,7 +464,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
     constexpr int MH = M / 2, LDK = E + 4, LDV = D + 4, LDF = M + 4;
     constexpr int FB = MH / 16, EC = E / 16, DB = D / 16, KB = TK / 16;
     constexpr int STAGE = TK * (LDK + LDV + LDF);     // floats per LDS stage
-    extern __shared__ float smem[];
+    extern __shared__ __attribute__((aligned(128))) float smem[];
     float* Ps = smem;                                  // only live before the key loop
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
@@ -394,6 +518,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
     }
     const float* csp = a.chunk_scale + (long)bh * a.n_chunks;
     float cscale = (kt_lo < kt_hi) ? csp[kt_lo * TK / CH] : 0.f;
+    const float kmax = a.kmax[bh];
 
     // query operand (B side: column = query, k = 16c+4g+j) and its squared norm
     floatx4 qr[EC];
@@ -407,48 +532,56 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
     const float diag_q = 0.5f * a.temp * group_sum(sq);
 
     // query features, kept in registers: qf[c] is the B operand for feature slice c of K'
-    load_proj<E, MH>(Ps, a.proj, sqrtf(a.temp), tid);
-    __syncthreads();
     floatx4 qf[2 * FB];
-    float qmax = 0.f;
+    float lsq;
+    if (SPLIT) {
+        // several parts share a query tile: the key pass has computed the features once
+        const long qrow = (long)bh * a.T + min(iq, a.T - 1);
 #pragma unroll
-    for (int fb = 0; fb < FB; ++fb) qf[fb] = Frag<float>::zero();
+        for (int c = 0; c < 2 * FB; ++c) qf[c] = *reinterpret_cast<const floatx4*>(a.qfeat + qrow * M + 16 * c + 4 * g);
+        lsq = a.q_lsq[qrow];
+    } else {
+        load_proj<E, MH>(Ps, a.proj, sqrtf(a.temp), tid);
+        __syncthreads();
+        float qmax = 0.f;
 #pragma unroll
-    for (int c = 0; c < EC; ++c) {                      // the FB accumulation chains advance together
-        floatx4 pa[FB];
+        for (int fb = 0; fb < FB; ++fb) qf[fb] = Frag<float>::zero();
 #pragma unroll
-        for (int fb = 0; fb < FB; ++fb)
-            pa[fb] = *reinterpret_cast<const floatx4*>(Ps + (16 * fb + r16) * LDK + 16 * c + 4 * g);
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int c = 0; c < EC; ++c) {                      // the FB accumulation chains advance together
+            floatx4 pa[FB];
 #pragma unroll
             for (int fb = 0; fb < FB; ++fb)
-                qf[fb] = __builtin_amdgcn_mfma_f32_16x16x4f32(pa[fb][j], qr[c][j], qf[fb], 0, 0, 0);
-    }
+                pa[fb] = *reinterpret_cast<const floatx4*>(Ps + (16 * fb + r16) * LDK + 16 * c + 4 * g);
 #pragma unroll
-    for (int fb = 0; fb < FB; ++fb)
+            for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            if (16 * fb + 4 * g + i < a.mh_valid) qmax = fmaxf(qmax, fabsf(qf[fb][i]));
-    qmax = group_max(qmax);
-    const float lsq = -diag_q + qmax - lnm_half;
+                for (int fb = 0; fb < FB; ++fb)
+                    qf[fb] = __builtin_amdgcn_mfma_f32_16x16x4f32(pa[fb][j], qr[c][j], qf[fb], 0, 0, 0);
+        }
 #pragma unroll
-    for (int fb = 0; fb < FB; ++fb) {
-        floatx4 dd = qf[fb];
+        for (int fb = 0; fb < FB; ++fb)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const bool ok = 16 * fb + 4 * g + i < a.mh_valid;
-            qf[fb][i] = ok ? __expf(dd[i] - qmax) : 0.f;
-            qf[FB + fb][i] = ok ? __expf(-dd[i] - qmax) : 0.f;
+            for (int i = 0; i < 4; ++i)
+                if (16 * fb + 4 * g + i < a.mh_valid) qmax = fmaxf(qmax, fabsf(qf[fb][i]));
+        qmax = group_max(qmax);
+        lsq = -diag_q + qmax - lnm_half;
+#pragma unroll
+        for (int fb = 0; fb < FB; ++fb) {
+            floatx4 dd = qf[fb];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const bool ok = 16 * fb + 4 * g + i < a.mh_valid;
+                qf[fb][i] = ok ? __expf(dd[i] - qmax) : 0.f;
+                qf[FB + fb][i] = ok ? __expf(-dd[i] - qmax) : 0.f;
+            }
         }
     }
-    __syncthreads();                 // Ps is dead; the tile buffers may overwrite it
+    if (!SPLIT) __syncthreads();     // Ps is dead; the tile buffers may overwrite it
     FLY_PROF(1);
 
     // From here on all exponents are base 2 (one v_exp_f32 each): scores carry t*log2(e) through
     // the query operand, the log-scales are converted once.
     constexpr float LOG2E = 1.4426950408889634f, LN2 = 0.6931471805599453f;
-    const float kmax = a.kmax[bh];
     const float c0 = (lsq + kmax) * LOG2E;       // base-2 log-scale of the global low-rank term
 #pragma unroll
     for (int c = 0; c < EC; ++c) qr[c] *= a.temp * LOG2E;
@@ -485,7 +618,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
             cscale_next = csp[(s_base + TK) / CH];
         }
         // weight of this chunk's features relative to the global key stabiliser (<= 1); the same
-        // expression weights the chunk in sb_combine_kernel
+        // expression weights the chunk in the combine role
         const float wc = __builtin_amdgcn_exp2f((cscale - kmax) * LOG2E);
 
         // wave-uniform: does this tile touch the band of any of the wave's 16 queries?  (Blocks of a
@@ -639,38 +772,10 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
     FLY_PROF(5);
 }
 
-// merge of the per-part partials: one thread per (query, four output columns); every load of a
-// thread is independent of the others so they are all in flight together
-template <typename T>
-__global__ __launch_bounds__(NT) void sb_merge_kernel(FwdArgs a, int D) {
-    constexpr float LN2 = 0.6931471805599453f;
-    const int d4 = D / 4;                                  // column groups per query
-    const int gid = blockIdx.x * NT + threadIdx.x;         // over TQ * d4 items of one query tile
-    const int qt = gid / (TQ * d4), rem = gid % (TQ * d4), ql = rem / d4, d = 4 * (rem % d4);
-    const int n_qt = (a.T + TQ - 1) / TQ;
-    if (qt >= n_qt) return;
-    const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
-    const int iq = qt * TQ + ql;
-    if (iq >= a.T) return;
-    const long stride = (long)TQ * (D + NSTAT);
-    const float* ws = a.part_ws + ((long)bh * n_qt + qt) * a.n_parts * stride;
-    const float* st = ws + TQ * D + ql;
-    float m_star = -INFINITY;
-#pragma unroll 8
-    for (int p = 0; p < a.n_parts; ++p) m_star = fmaxf(m_star, st[p * stride]);
-    float ze = 0.f, zp = 0.f;
-    floatx4 acc = Frag<float>::zero();
-#pragma unroll 8
-    for (int p = 0; p < a.n_parts; ++p) {
-        const float wgt = __builtin_amdgcn_exp2f(st[p * stride] - m_star);
-        ze += wgt * st[p * stride + TQ];
-        zp += st[p * stride + 2 * TQ];
-        acc += wgt * *reinterpret_cast<const floatx4*>(ws + p * stride + ql * D + d);
-    }
-    const float Z = ze + __builtin_amdgcn_exp2f(st[4 * TQ] - m_star) * fmaxf(st[3 * TQ] - zp, 1e-24f);
-    T* optr = reinterpret_cast<T*>(a.out) + b * a.o_sb + h * a.o_sh + (long)iq * a.o_ss;
-    store4_f32(optr + d, acc * (1.0f / Z));
-    if (d == 0) a.log_norm[(long)bh * a.T + iq] = m_star * LN2 + __logf(Z);
+// one workgroup per query tile
+template <typename T, int D>
+__global__ __launch_bounds__(NT) void sb_merge_kernel(FwdArgs a) {
+    sb_merge_tile<T, D>(a, blockIdx.y, blockIdx.x, gridDim.x);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -700,7 +805,8 @@ static int launch_kfeat(const KvArgs& a, hipStream_t st) {
         if (e != hipSuccess) return fail(ERR_LAUNCH, "sb_kfeat: LDS attribute: %s", hipGetErrorString(e));
         lds_ready = true;
     }
-    hipLaunchKernelGGL(kern, dim3(a.n_split, a.B * a.H), dim3(NT), smem, st, a);
+    // per (batch, head): key-role workgroups, then query-role ones
+    hipLaunchKernelGGL(kern, dim3(a.n_split + a.q_tiles, a.B * a.H), dim3(NT), smem, st, a);
     return check_launch("sb_kfeat_kernel");
 }
 
@@ -729,7 +835,7 @@ static int launch_fwd_impl(const FwdArgs& a, hipStream_t st) {
     g_ev_before = g_ev_after = nullptr;
     int rc = check_launch("sblocal_fwd_kernel");
     if (rc || !SPLIT) return rc;
-    hipLaunchKernelGGL(sb_merge_kernel<T>, dim3((qt * TQ * (E / 4) + NT - 1) / NT, a.B * a.H), dim3(NT), 0, st, a, E);
+    hipLaunchKernelGGL((sb_merge_kernel<T, E>), dim3(qt, a.B * a.H), dim3(NT), 0, st, a);
     return check_launch("sb_merge_kernel");
 }
 template <typename T, int E, int M>
@@ -828,6 +934,8 @@ static int check_sb_dims(const char* who, int E, int D, int mh, int mh_valid, in
 extern "C" int flyhip_sb_kv_reduce(const void* k, const void* v, const float* proj, const int64_t* key_lengths,
                                    float* kfeat, float* chunk_scale, float* kv_part, float* part_max,
                                    float* kv, float* ksum, float* kmax,
+                                   const void* q, float* qfeat, float* q_lsq, int T,
+                                   int64_t q_sb, int64_t q_sh, int64_t q_ss,
                                    int B, int H, int S, int E, int D, int mh, int mh_valid, int n_split,
                                    int64_t k_sb, int64_t k_sh, int64_t k_ss,
                                    int64_t v_sb, int64_t v_sh, int64_t v_ss,
@@ -843,14 +951,20 @@ extern "C" int flyhip_sb_kv_reduce(const void* k, const void* v, const float* pr
     FLY_REQUIRE(n_split >= 1 && n_split <= nc && n_split <= MAX_SPLIT,
                 "sb_kv_reduce: n_split=%d outside [1, min(%d, %d)]", n_split, nc, MAX_SPLIT);
     FLY_REQUIRE((long)B * H <= 65535, "sb_kv_reduce: B*H=%ld exceeds the grid limit 65535", (long)B * H);
+    if (q) {
+        FLY_REQUIRE(qfeat && q_lsq && T > 0, "sb_kv_reduce: query features asked for without qfeat / q_lsq / T");
+        FLY_REQUIRE(((q_sb | q_sh | q_ss) % 4) == 0, "sb_kv_reduce: q strides must be multiples of 4 elements");
+    }
     KvArgs a{k, v, proj, key_lengths, kfeat, chunk_scale, kv_part, part_max,
-             B, H, S, mh_valid, nc, n_split, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, softmax_temp};
+             B, H, S, mh_valid, nc, n_split, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, softmax_temp,
+             q, qfeat, q_lsq, q ? T : 0, q_sb, q_sh, q_ss,
+             q ? (T + TQ - 1) / TQ : 0};
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     const int m = 2 * mh;
     rc = dispatch_kfeat(dtype, E, m, a, st);
     if (rc) return rc;
     const int per = m * (D + 1);
-    hipLaunchKernelGGL(sb_combine_kernel, dim3((per + 255) / 256, B * H), dim3(256), 0, st,
+    hipLaunchKernelGGL(sb_combine_kernel, dim3((per + NT - 1) / NT, B * H), dim3(NT), 0, st,
                        kv_part, part_max, kv, ksum, kmax, n_split, m, D);
     return check_launch("sb_combine_kernel");
 }
@@ -858,6 +972,7 @@ extern "C" int flyhip_sb_kv_reduce(const void* k, const void* v, const float* pr
 extern "C" int flyhip_sblocal_fwd(const void* q, const void* k, const void* v, const float* proj,
                                   const float* kfeat, const float* chunk_scale,
                                   const float* kv, const float* ksum, const float* kmax,
+                                  const float* qfeat, const float* q_lsq,
                                   const int64_t* key_lengths, void* out, float* log_norm,
                                   float* part_ws, int n_parts,
                                   int B, int H, int T, int S, int E, int D, int mh, int mh_valid,
@@ -877,10 +992,11 @@ extern "C" int flyhip_sblocal_fwd(const void* q, const void* k, const void* v, c
     if (rc) return rc;
     FLY_REQUIRE((long)B * H <= 65535, "sblocal_fwd: B*H=%ld exceeds the grid limit 65535", (long)B * H);
     FLY_REQUIRE(n_parts >= 1 && n_parts <= 64, "sblocal_fwd: n_parts=%d outside [1, 64]", n_parts);
-    FLY_REQUIRE(n_parts == 1 || part_ws, "sblocal_fwd: n_parts > 1 needs the partial workspace");
+    FLY_REQUIRE(n_parts == 1 || (part_ws && qfeat && q_lsq),
+                "sblocal_fwd: n_parts > 1 needs the partial workspace and the query features of the key pass");
     int nc, ns;
     plan(B, H, S, &nc, &ns);
-    FwdArgs a{q, k, v, proj, kfeat, chunk_scale, kv, ksum, kmax, key_lengths, out, log_norm, part_ws,
+    FwdArgs a{q, k, v, proj, kfeat, chunk_scale, kv, ksum, kmax, qfeat, q_lsq, key_lengths, out, log_norm, part_ws,
               B, H, T, S, mh_valid, local_context, nc, n_parts,
               q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss, softmax_temp};
     return dispatch_fwd(dtype, E, 2 * mh, a, reinterpret_cast<hipStream_t>(stream));

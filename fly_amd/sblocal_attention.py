@@ -55,18 +55,27 @@ class SBLocalPlan:
         self.kv = torch.empty(B, H, m, dim, dtype=f32, device=device)
         self.ksum = torch.empty(B, H, m, dtype=f32, device=device)
         self.kmax = torch.empty(B, H, dtype=f32, device=device)
-        self.part_ws = None
+        # with several parts per query tile the key pass also computes the query features, once
+        self.part_ws = self.qfeat = self.q_lsq = None
         if self.n_parts > 1:
             self.part_ws = torch.empty(B * H * ((T + 63) // 64) * self.n_parts * 64 * (dim + 5), dtype=f32,
                                        device=device)
+            self.qfeat = torch.empty(B, H, T, m, dtype=f32, device=device)
+            self.q_lsq = torch.empty(B, H, T, dtype=f32, device=device)
 
-    def run_keys(self, k, v, proj, lens, t, stream=None):
+    def run_keys(self, q, k, v, proj, lens, t, stream=None):
+        """The key-side pass (features of the keys, K'^T V, sum K'); with several parts per query
+        tile also the features of the queries `q`."""
         B, H, T, S, dim, mh, mh_valid = self.shape
         stream = _lib.stream_ptr(self.device) if stream is None else stream
+        q_args = (None, None, None, 0, 0, 0, 0)
+        if self.n_parts > 1:
+            q_args = (q.data_ptr(), self.qfeat.data_ptr(), self.q_lsq.data_ptr(), T,
+                      q.stride(0), q.stride(2), q.stride(1))
         _lib.call('flyhip_sb_kv_reduce', k.data_ptr(), v.data_ptr(), proj.data_ptr(), _lib.ptr(lens),
                   self.kfeat.data_ptr(), self.chunk_scale.data_ptr(), self.kv_part.data_ptr(),
                   self.part_max.data_ptr(), self.kv.data_ptr(), self.ksum.data_ptr(), self.kmax.data_ptr(),
-                  B, H, S, dim, dim, mh, mh_valid, self.n_split,
+                  *q_args, B, H, S, dim, dim, mh, mh_valid, self.n_split,
                   k.stride(0), k.stride(2), k.stride(1), v.stride(0), v.stride(2), v.stride(1),
                   t, self.code, stream)
 
@@ -75,8 +84,8 @@ class SBLocalPlan:
         stream = _lib.stream_ptr(self.device) if stream is None else stream
         _lib.call('flyhip_sblocal_fwd', q.data_ptr(), k.data_ptr(), v.data_ptr(), proj.data_ptr(),
                   self.kfeat.data_ptr(), self.chunk_scale.data_ptr(), self.kv.data_ptr(),
-                  self.ksum.data_ptr(), self.kmax.data_ptr(), _lib.ptr(lens),
-                  out.data_ptr(), log_norm.data_ptr(), _lib.ptr(self.part_ws), self.n_parts,
+                  self.ksum.data_ptr(), self.kmax.data_ptr(), _lib.ptr(self.qfeat), _lib.ptr(self.q_lsq),
+                  _lib.ptr(lens), out.data_ptr(), log_norm.data_ptr(), _lib.ptr(self.part_ws), self.n_parts,
                   B, H, T, S, dim, dim, mh, mh_valid, local_context,
                   q.stride(0), q.stride(2), q.stride(1), k.stride(0), k.stride(2), k.stride(1),
                   v.stride(0), v.stride(2), v.stride(1), out.stride(0), out.stride(2), out.stride(1),
@@ -85,7 +94,7 @@ class SBLocalPlan:
     def run(self, q, k, v, proj, lens, local_context, t, out, log_norm):
         with torch.cuda.device(self.device):
             stream = _lib.stream_ptr(self.device)
-            self.run_keys(k, v, proj, lens, t, stream)
+            self.run_keys(q, k, v, proj, lens, t, stream)
             self.run_queries(q, k, v, proj, lens, local_context, t, out, log_norm, stream)
 
 

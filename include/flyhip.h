@@ -47,10 +47,17 @@ int flyhip_sb_plan(int B, int H, int T, int S, int local_context,
  *   kfeat       (B,H,n_chunks*64,m)  positive random features of every key, stabilised per chunk
  *   chunk_scale (B,H,n_chunks)       log-stabiliser each chunk of kfeat was written with
  *   kv (B,H,m,D), ksum (B,H,m), kmax (B,H)  global reductions in units of exp(kmax)
- * scratch: kv_part (B,H,n_split,m*(D+1)), part_max (B,H,n_split). */
+ * scratch: kv_part (B,H,n_split,m*(D+1)), part_max (B,H,n_split).
+ * Optional query side (q may be NULL; needed when flyhip_sblocal_fwd runs with n_parts > 1, where
+ * several workgroups share a query tile): q (B,T,H,E) via strides -> qfeat (B,H,T,m) fp32, the
+ * query features exp(+-sqrt(t) P q - rowmax) (ref: softmax_kernel with is_query=True,
+ * src/models/attention/feature_maps_sb.py:51-82,148-151), and q_lsq (B,H,T) fp32, their log-scale
+ * -t|q|^2/2 + rowmax - log(m)/2. */
 int flyhip_sb_kv_reduce(const void* k, const void* v, const float* proj, const int64_t* key_lengths,
                         float* kfeat, float* chunk_scale, float* kv_part, float* part_max,
                         float* kv, float* ksum, float* kmax,
+                        const void* q, float* qfeat, float* q_lsq, int T,
+                        int64_t q_sb, int64_t q_sh, int64_t q_ss,
                         int B, int H, int S, int E, int D, int mh, int mh_valid, int n_split,
                         int64_t k_sb, int64_t k_sh, int64_t k_ss,
                         int64_t v_sb, int64_t v_sh, int64_t v_ss,
@@ -62,10 +69,13 @@ int flyhip_sb_kv_reduce(const void* k, const void* v, const float* proj, const i
  *   q (B,T,H,E), out (B,T,H,D) via strides; log_norm (B,H,T) fp32 = the reference's
  *   log_normalization; local_context = lc (band -(lc/2) <= s - i < (lc+1)/2).
  *   n_parts from flyhip_sb_plan (any value in [1,64] is valid); when > 1, part_ws is scratch of
- *   B*H*ceil(T/64)*n_parts*64*(D+5) floats, else it may be NULL. */
+ *   B*H*ceil(T/64)*n_parts*64*(D+5) floats and qfeat / q_lsq are the query-side outputs of
+ *   flyhip_sb_kv_reduce for the same q; with n_parts == 1 all three may be NULL (the kernel forms
+ *   the query features itself). */
 int flyhip_sblocal_fwd(const void* q, const void* k, const void* v, const float* proj,
                        const float* kfeat, const float* chunk_scale,
                        const float* kv, const float* ksum, const float* kmax,
+                       const float* qfeat, const float* q_lsq,
                        const int64_t* key_lengths, void* out, float* log_norm,
                        float* part_ws, int n_parts,
                        int B, int H, int T, int S, int E, int D, int mh, int mh_valid,

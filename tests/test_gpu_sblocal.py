@@ -86,6 +86,27 @@ def test_config1_full_size():
     check_fp32(*run_both(q, k, v, P, 512))
 
 
+@pytest.mark.parametrize('n_parts', [5, 3, 8, 12, 1])
+def test_reused_plan_and_part_merge(n_parts):
+    """One plan (its workspaces) run on three different inputs in a row: every result matches the
+    oracle, i.e. nothing of an earlier call is seen by a later one.  Covers the merge of the parts
+    of a query tile for several part counts (one and two batches of the merge, parts without any
+    key tile) and the one-part kernel."""
+    from fly_amd.sblocal_attention import SBLocalPlan
+    dev = torch.device('cuda:0')
+    B, H, T, E, mh, lc = 2, 2, 700, 64, 64, 200
+    plan = SBLocalPlan(B, H, T, T, E, mh, mh, torch.float32, dev, lc, n_parts=n_parts)
+    assert plan.n_parts == n_parts
+    out = torch.empty(B, T, H, E, device=dev)
+    ln = torch.empty(B, H, T, device=dev)
+    for seed in (21, 22, 23):
+        print('case', n_parts, seed, flush=True)
+        q, k, v, P = make_inputs(B, T, T, H, E, E, mh, seed=seed)
+        plan.run(q.to(dev), k.to(dev), v.to(dev), P.to(dev), None, lc, 1 / math.sqrt(E), out, ln)
+        ref_out, ref_ln = osb.sblocal_attention(q.double(), k.double(), v.double(), P.double(), lc)
+        check_fp32(out.cpu(), ln.cpu().unsqueeze(-1), ref_out, ref_ln)
+
+
 def test_value_of_ones_gives_ones():
     """Normalisation identity at full size: v == 1 -> out == 1 for any P, lc, t."""
     q, k, v, P = make_inputs(2, 3136, 3136, 1, 64, 64, 64, seed=3)
