@@ -23,6 +23,10 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
+# HBM bytes one launch of the fused band kernel moves at config 1: rocprofv3 FETCH_SIZE (7381 KiB,
+# scale 2.0 from a plain copy of known size) + WRITE_SIZE (8452 KiB, scale 1.0), as committed in
+# profiles/sblocal_fwd_config1_fp32.md.  Counters cannot be read from inside this process.
+BAND_KERNEL_TRAFFIC_BYTES = 23.8e6
 
 
 def sblocal_flops(B, H, T, S, E, D, m, lc):
@@ -93,7 +97,7 @@ def bench_sblocal(steps, warmup, cpu_baseline=True):
         'ms_per_step': ms_per_step,
         'roofline': {'bound': 'mfma', 'kernel': 'sblocal_fwd_kernel<float,64,64,128>',
                      'achieved': achieved, 'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s',
-                     'frac': achieved / PEAK_FP32_MFMA_TFLOPS, 'traffic': None,
+                     'frac': achieved / PEAK_FP32_MFMA_TFLOPS, 'traffic': BAND_KERNEL_TRAFFIC_BYTES,
                      'kernel_ms': fwd_ms, 'flops_per_launch': fwd_flops, 'launches_timed': len(ev)},
         'parity': {'out_rel_err': err_out, 'log_norm_rel_err': err_ln},
         'flops_per_step': total_flops,
