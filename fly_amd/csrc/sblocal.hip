@@ -22,6 +22,7 @@
 // consecutive keys/features -- which is exactly the operand layout the next product needs.
 #include "common.h"
 #include <math.h>
+#include <type_traits>
 
 namespace flyhip {
 
@@ -49,7 +50,7 @@ __device__ long long g_prof[16384 * 8];
 
 struct KvArgs {
     const void* k; const void* v; const float* proj; const int64_t* lens;
-    float* kfeat; float* chunk_scale; float* kv_part; float* part_max;
+    void* kfeat; float* chunk_scale; float* kv_part; float* part_max;
     int B, H, S, mh_valid, n_chunks, n_split;
     long k_sb, k_sh, k_ss, v_sb, v_sh, v_ss;
     float temp;
@@ -58,12 +59,13 @@ struct KvArgs {
     int T;
     long q_sb, q_sh, q_ss;
     int q_tiles;                    // query-role workgroups per (batch, head), after the n_split key-role ones
+    void* vt;                       // bf16 inputs: V per 32-key tile, transposed ([d][k-slot]) for the band kernel's P V
 };
 
 struct FwdArgs {
     const void* q; const void* k; const void* v; const float* proj;
-    const float* kfeat; const float* chunk_scale; const float* kv; const float* ksum; const float* kmax;
-    const float* qfeat; const float* q_lsq;
+    const void* kfeat; const float* chunk_scale; const float* kv; const float* ksum; const float* kmax;
+    const float* qfeat; const float* q_lsq; const void* vt; const void* kvt;
     const int64_t* lens; void* out; float* log_norm; float* part_ws;
     int B, H, T, S, mh_valid, lc, n_chunks, n_parts;
     long q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss;
@@ -110,7 +112,8 @@ __device__ __forceinline__ void load_proj(float* Ps, const float* proj, float sc
 // weights staged in LDS so that the loads over s are independent and stay in flight together
 constexpr int MAX_SPLIT = 1024;
 __global__ __launch_bounds__(NT) void sb_combine_kernel(const float* kv_part, const float* part_max, float* kv,
-                                                        float* ksum, float* kmax_out, int n_split, int M, int D) {
+                                                        float* ksum, float* kmax_out, uint16_t* kvt, int n_split,
+                                                        int M, int D) {
     __shared__ float wgt[MAX_SPLIT];
     const int bh = blockIdx.y;
     const int idx = blockIdx.x * NT + threadIdx.x;
@@ -138,6 +141,10 @@ __global__ __launch_bounds__(NT) void sb_combine_kernel(const float* kv_part, co
         const int db_n = D >> 4, rb = tile / db_n, db = tile % db_n;
         const int r = 16 * rb + 4 * (lane >> 4) + i, d = 16 * db + (lane & 15);
         kv[(long)bh * M * D + r * D + d] = acc;
+        if (kvt) {      // bf16 copy for the bf16 band kernel: [d][slot], feature r in the k-slot order of its MFMA
+            const int c = r >> 4, slot = 32 * (c >> 1) + 8 * ((r >> 2) & 3) + 4 * (c & 1) + (r & 3);
+            kvt[(long)bh * M * D + d * M + slot] = f32_to_bf16(acc);
+        }
     } else {
         ksum[(long)bh * M + idx - M * D] = acc;
     }
@@ -146,6 +153,23 @@ __global__ __launch_bounds__(NT) void sb_combine_kernel(const float* kv_part, co
 // ---------------------------------------------------------------------------------------
 // key features + partial K'^T V
 // ---------------------------------------------------------------------------------------
+// One block of 16 features (block fbp of the [positive | negative] feature row; the lane holds
+// features 16 fbp + 4g + i) of one key goes to the feature scratch.  float inputs: fp32, natural
+// feature order.  bfloat16 inputs: bf16, in the order the 16x16x32 MFMA of the band kernel consumes
+// (position 32 ks + 8 g + j holds feature 32 ks + 16 (j / 4) + 4 g + j % 4, so that a lane's eight
+// k-slots are 16 contiguous bytes and the query features need no shuffle either).
+template <typename T>
+__device__ __forceinline__ void store_feat(void* kfeat, long row, int M, int fbp, int g, floatx4 f) {
+    if (sizeof(T) == 4) {
+        *reinterpret_cast<floatx4*>(reinterpret_cast<float*>(kfeat) + row * M + 16 * fbp + 4 * g) = f;
+    } else {
+        uint2 u;
+        u.x = pack_bf16x2(f[0], f[1]);
+        u.y = pack_bf16x2(f[2], f[3]);
+        *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(kfeat) + row * M + 32 * (fbp >> 1) + 8 * g + 4 * (fbp & 1)) = u;
+    }
+}
+
 // two waves per SIMD (two workgroups per CU) where the register budget allows it without spilling
 constexpr int kfeat_waves(int E, int M) { return (E <= 64 && M <= 128) ? 2 : 1; }
 
@@ -256,6 +280,19 @@ void sb_kfeat_kernel(KvArgs a) {
 
     for (int c = c0; c < c1; ++c) {
         const int s_base = c * CH;
+        if (sizeof(T) == 2 && a.vt) {
+            // the chunk's V, as two 32-key tiles [d][slot] with slot 8g+j = key 16(j/4) + 4g + j%4: the
+            // k-slot order of the band kernel's P V product, so that it can copy 16-byte pieces
+            uint16_t* vt = reinterpret_cast<uint16_t*>(a.vt) + ((long)bh * a.n_chunks + c) * (CH * D);
+#pragma unroll
+            for (int j = 0; j < CH * D / 8 / NT; ++j) {
+                const int ci = tid + NT * j, tile = ci / (D * 4), rem = ci % (D * 4), d = rem / 4, c8 = rem % 4;
+                const float* col = Vs + (32 * tile + 4 * c8) * LDV + d;          // key 4 c8 of the tile, dim d
+                const uint4 u = make_uint4(pack_bf16x2(col[0], col[LDV]), pack_bf16x2(col[2 * LDV], col[3 * LDV]),
+                                           pack_bf16x2(col[16 * LDV], col[17 * LDV]), pack_bf16x2(col[18 * LDV], col[19 * LDV]));
+                *reinterpret_cast<uint4*>(vt + tile * (D * 32) + d * 32 + 8 * c8) = u;
+            }
+        }
         if (c + 1 < c1) {                        // next chunk's K and V fly during this chunk's work
             kt.fetch(kptr, a.k_ss, s_base + CH, a.S - 1, tid);
             vt.fetch(vptr, a.v_ss, s_base + CH, a.S - 1, tid);
@@ -300,12 +337,12 @@ void sb_kfeat_kernel(KvArgs a) {
         __syncthreads();
         const float lmax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
         const float new_max = fmaxf(run_max, lmax);
-        float* frow_g = a.kfeat + ((long)bh * a.n_chunks * CH + s_base + 16 * w + r16) * M;
+        const long frow_g = (long)bh * a.n_chunks * CH + s_base + 16 * w + r16;      // this lane's key row
         if (new_max == -INFINITY) {   // no valid key yet (workgroup-uniform): features are zero
 #pragma unroll
             for (int fb = 0; fb < FB; ++fb) {
-                *reinterpret_cast<floatx4*>(frow_g + 16 * fb + 4 * g) = Frag<float>::zero();
-                *reinterpret_cast<floatx4*>(frow_g + MH + 16 * fb + 4 * g) = Frag<float>::zero();
+                store_feat<T>(a.kfeat, frow_g, M, fb, g, Frag<float>::zero());
+                store_feat<T>(a.kfeat, frow_g, M, FB + fb, g, Frag<float>::zero());
             }
             if (tid == 0) a.chunk_scale[(long)bh * a.n_chunks + c] = 0.f;
         } else {
@@ -330,8 +367,8 @@ void sb_kfeat_kernel(KvArgs a) {
                 ksn[fb] = ksn[fb] * rescale + fn;
                 *reinterpret_cast<floatx4*>(frow_s + 16 * fb + 4 * g) = fp;
                 *reinterpret_cast<floatx4*>(frow_s + MH + 16 * fb + 4 * g) = fn;
-                *reinterpret_cast<floatx4*>(frow_g + 16 * fb + 4 * g) = fp;
-                *reinterpret_cast<floatx4*>(frow_g + MH + 16 * fb + 4 * g) = fn;
+                store_feat<T>(a.kfeat, frow_g, M, fb, g, fp);
+                store_feat<T>(a.kfeat, frow_g, M, FB + fb, g, fn);
             }
             if (tid == 0) a.chunk_scale[(long)bh * a.n_chunks + c] = new_max * LN2;    // stored in natural-log units
             __syncthreads();
@@ -394,6 +431,454 @@ void sb_kfeat_kernel(KvArgs a) {
     __syncthreads();
     if (tid < M) part[M * D + tid] = (ks_lds[tid] + ks_lds[M + tid]) + (ks_lds[2 * M + tid] + ks_lds[3 * M + tid]);
     if (tid == 0) a.part_max[(long)bh * a.n_split + sp] = run_max * LN2;
+}
+
+// ---------------------------------------------------------------------------------------
+// fused band kernel for bfloat16 inputs
+// ---------------------------------------------------------------------------------------
+// Same algorithm and the same transposed formulation as sblocal_fwd_kernel, with the three
+// contractions of the key loop (and the global low-rank term) on v_mfma_f32_16x16x32_bf16: a
+// lane (r = lane%16, g = lane/16) supplies eight consecutive k-slots 8g..8g+7 of row / column r,
+// 16 contiguous bytes, and receives D[4g+i][r].  The k-slot order of every product is chosen so
+// that the operands exist without shuffles:
+//   scores   K q      : slot = head-dim index, K rows and q rows as they are in memory
+//   overlap  K' q'    : slot 8g+j of step ks = feature 32ks + 16(j/4) + 4g + j%4 -- the order in which
+//                       the fp32 projection leaves the query features in a lane, and in which the
+//                       key pass stores the bf16 key features
+//   P V               : slot 8g+j = key 16(j/4) + 4g + j%4 of the 32-key tile -- the order in which the
+//                       score tiles leave the probabilities in a lane; the key pass leaves V in HBM
+//                       per 32-key tile already transposed, [d][slot]
+// q and k are bf16 already, so the scores are as exact as on the fp32 path (the softmax scale is
+// applied to the fp32 result, not to an operand); key features, probabilities and K'^T V are
+// rounded to bf16 for their products.  The query projection sqrt(t) P q also runs on the bf16 MFMA
+// without losing precision: q is bf16 already and P is split into a bf16 head and a bf16 remainder
+// (two MFMAs per step; the split represents P to 2^-17).
+
+// ROWS x W tile of 2-byte elements, global -> registers -> LDS (rows clamped like RowTile)
+typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));   // a native vector: stays in registers as a struct member
+
+template <int ROWS, int W, int NT>
+struct Tile16 {
+    static constexpr int C8 = W / 8, N = (ROWS * C8 + NT - 1) / NT;
+    uintx4 r[N];
+    __device__ __forceinline__ void fetch(const uint16_t* src, long row_stride, int row0, int last_row, int tid) {
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+            const int idx = tid + NT * j, row = idx / C8, c8 = idx % C8;
+            if (N * NT == ROWS * C8 || idx < ROWS * C8)
+                r[j] = *reinterpret_cast<const uintx4*>(src + (long)min(row0 + row, last_row) * row_stride + 8 * c8);
+        }
+    }
+    template <int LD>
+    __device__ __forceinline__ void stash(uint16_t* dst, int tid) const {
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+            const int idx = tid + NT * j, row = idx / C8, c8 = idx % C8;
+            if (N * NT == ROWS * C8 || idx < ROWS * C8) *reinterpret_cast<uintx4*>(dst + row * LD + 8 * c8) = r[j];
+        }
+    }
+};
+
+__device__ __forceinline__ floatx4 mma_bf16(uint4 a, uint4 b, floatx4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+
+// A workgroup is NW waves of 16 queries each: more waves share every key tile, which divides the
+// L2 -> CU traffic (the limit of this kernel: 24 KiB per 32-key tile at E = D = 64, m = 256).
+constexpr int BF16_WAVES = 8;
+
+template <int E, int D, int M, bool SPLIT, int NW>
+__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2))) void sblocal_fwd_bf16_kernel(FwdArgs a) {
+    static_assert(TK == 32, "the P V product takes one 32-key tile per MFMA step");
+    constexpr int NT = 64 * NW, TQ = 16 * NW;          // shadow the 4-wave constants of the fp32 kernels
+    constexpr int TQ64 = 64;                           // queries per tile of the partial workspace / merge
+    typedef bf16_t T;
+    constexpr int MH = M / 2, FB = MH / 16, EC = E / 16, DB = D / 16, KB = TK / 16;
+    constexpr int LDK = E + 8, LDF = M + 8, LDT = TK + 8, LDKV = M + 8;   // LDS row strides in elements
+    constexpr int STAGE = TK * LDK + TK * LDF + D * LDT;                  // elements per stage
+    extern __shared__ __attribute__((aligned(128))) float smem[];
+    uint16_t* lds = reinterpret_cast<uint16_t*>(smem);
+
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
+    const int n_qt = (a.T + TQ - 1) / TQ;
+    const int n_items = a.B * a.H * n_qt * a.n_parts;
+    const int per_xcd = (n_items + N_XCD - 1) / N_XCD;
+    const int item = (blockIdx.x % N_XCD) * per_xcd + blockIdx.x / N_XCD;   // see sblocal_fwd_kernel
+    if (item >= n_items) return;                       // workgroup-uniform
+    const int part = item % a.n_parts;
+    const int qt = (item / a.n_parts) % n_qt;
+    const int bh = item / (a.n_parts * n_qt), b = bh / a.H, h = bh % a.H;
+    const int q0 = qt * TQ;
+    const int iq = q0 + 16 * w + r16;
+    const bool qvalid = iq < a.T;
+    const uint16_t* qptr = reinterpret_cast<const uint16_t*>(a.q) + b * a.q_sb + h * a.q_sh;
+    const uint16_t* kptr = reinterpret_cast<const uint16_t*>(a.k) + b * a.k_sb + h * a.k_sh;
+    const uint16_t* vtp = reinterpret_cast<const uint16_t*>(a.vt) + (long)bh * a.n_chunks * CH * D;   // [tile][d][slot]
+    const uint16_t* fptr = reinterpret_cast<const uint16_t*>(a.kfeat) + (long)bh * a.n_chunks * CH * M;
+    const int len = a.lens ? min((int)a.lens[b], a.S) : a.S;
+    const float lnm_half = 0.5f * __logf(2.0f * a.mh_valid);
+    const int lc_lo = a.lc / 2, lc_hi = (a.lc + 1) / 2;    // band: -lc_lo <= s - i < lc_hi
+    constexpr float LOG2E = 1.4426950408889634f, LN2 = 0.6931471805599453f;
+
+    FLY_PROF(0);
+    // this workgroup's share of the band, in 32-key tiles (as in sblocal_fwd_kernel)
+    const int q_last = min(q0 + TQ - 1, a.T - 1);
+    const int lo = max(0, q0 - lc_lo);
+    const int hi = min(len, q_last + lc_hi);
+    int kt_lo = lo / TK;
+    int kt_hi = (hi > lo) ? (hi + TK - 1) / TK : kt_lo;
+    if (SPLIT) {
+        const int per = (kt_hi - kt_lo + 1 + a.n_parts - 1) / a.n_parts;
+        const int first = kt_lo + part * per - (part > 0 ? 1 : 0);
+        const int last = kt_lo + (part + 1) * per - 1;
+        kt_lo = min(kt_hi, first);
+        kt_hi = min(kt_hi, last);
+    }
+    const bool lowrank_here = !SPLIT || part == 0;     // workgroup-uniform
+
+    // Key tiles travel global -> registers -> LDS.  A tile is requested two iterations before it is
+    // used (one iteration of work is shorter than the latency of the loads under load), so two
+    // register sets alternate and the key loop is unrolled by two.
+    struct TileRegs {
+        Tile16<TK, E, NT> k;
+        Tile16<D, TK, NT> v;          // already transposed by the key pass: D rows of 32 k-slots
+        Tile16<TK, M, NT> f;
+        float cscale;
+    };
+    const int f_last = a.n_chunks * CH - 1;
+    const float* csp = a.chunk_scale + (long)bh * a.n_chunks;
+    auto fetch = [&](TileRegs& r, int kt) __attribute__((always_inline)) {
+        r.k.fetch(kptr, a.k_ss, kt * TK, a.S - 1, tid);
+        r.v.fetch(vtp + (long)kt * (D * TK), TK, 0, D - 1, tid);
+        r.f.fetch(fptr, M, kt * TK, f_last, tid);
+        r.cscale = csp[kt * TK / CH];
+    };
+    auto stash = [&](const TileRegs& r, int stage) __attribute__((always_inline)) {
+        uint16_t* dst = lds + stage * STAGE;
+        r.k.template stash<LDK>(dst, tid);
+        r.f.template stash<LDF>(dst + TK * LDK, tid);
+        r.v.template stash<LDT>(dst + TK * (LDK + LDF), tid);
+    };
+    TileRegs ra, rb;
+    ra.cscale = rb.cscale = 0.f;
+    // (clamped tile indices: the loads are unconditional so that the register sets are plain values)
+    fetch(ra, min(kt_lo, max(kt_hi - 1, 0)));
+    fetch(rb, min(kt_lo + 1, max(kt_hi - 1, 0)));
+    const float kmax = a.kmax[bh];
+
+    // score operand: the query row as it is in memory
+    const uint16_t* qrow = qptr + (long)min(iq, a.T - 1) * a.q_ss;
+    uint4 qb[E / 32];
+#pragma unroll
+    for (int ks = 0; ks < E / 32; ++ks) qb[ks] = *reinterpret_cast<const uint4*>(qrow + 32 * ks + 8 * g);
+
+    // query features in fp32: qf[c][i] = feature 16c + 4g + i of the [positive | negative] row
+    floatx4 qf[2 * FB];
+    float lsq;
+    if (SPLIT) {
+        const long qr_ = (long)bh * a.T + min(iq, a.T - 1);
+#pragma unroll
+        for (int c = 0; c < 2 * FB; ++c) qf[c] = *reinterpret_cast<const floatx4*>(a.qfeat + qr_ * M + 16 * c + 4 * g);
+        lsq = a.q_lsq[qr_];
+    } else {
+        // |q|^2 from the score operand (lane g holds elements 32ks + 8g .. + 7 of its query row)
+        float sq = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < E / 32; ++ks) {
+            const uint32_t wds[4] = {qb[ks].x, qb[ks].y, qb[ks].z, qb[ks].w};
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                const float lo = __uint_as_float(wds[x] << 16), hi = __uint_as_float(wds[x] & 0xffff0000u);
+                sq += lo * lo + hi * hi;
+            }
+        }
+        const float diag_q = 0.5f * a.temp * group_sum(sq);
+        // sqrt(t) P as bf16 head + bf16 remainder, rows of E + 8 elements
+        uint16_t* Phi = lds;
+        uint16_t* Plo = lds + MH * LDK;
+        const float pscale = sqrtf(a.temp);
+        for (int idx = tid; idx < MH * E / 4; idx += NT) {
+            const int f = idx / (E / 4), c4 = idx % (E / 4);
+            const floatx4 x = *reinterpret_cast<const floatx4*>(a.proj + (long)f * E + 4 * c4) * pscale;
+            floatx4 rem;
+            uint16_t hb[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                hb[i] = f32_to_bf16(x[i]);
+                rem[i] = x[i] - bf16_to_f32(hb[i]);
+            }
+            *reinterpret_cast<uint2*>(Phi + f * LDK + 4 * c4) = make_uint2(hb[0] | ((uint32_t)hb[1] << 16), hb[2] | ((uint32_t)hb[3] << 16));
+            *reinterpret_cast<uint2*>(Plo + f * LDK + 4 * c4) = make_uint2(pack_bf16x2(rem[0], rem[1]), pack_bf16x2(rem[2], rem[3]));
+        }
+        __syncthreads();
+#pragma unroll
+        for (int fb = 0; fb < FB; ++fb) qf[fb] = Frag<float>::zero();
+#pragma unroll
+        for (int ks = 0; ks < E / 32; ++ks)
+#pragma unroll
+            for (int fb = 0; fb < FB; ++fb) {
+                const int off = (16 * fb + r16) * LDK + 32 * ks + 8 * g;
+                qf[fb] = mma_bf16(*reinterpret_cast<const uint4*>(Phi + off), qb[ks], qf[fb]);
+                qf[fb] = mma_bf16(*reinterpret_cast<const uint4*>(Plo + off), qb[ks], qf[fb]);
+            }
+        float qmax = 0.f;
+#pragma unroll
+        for (int fb = 0; fb < FB; ++fb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (16 * fb + 4 * g + i < a.mh_valid) qmax = fmaxf(qmax, fabsf(qf[fb][i]));
+        qmax = group_max(qmax);
+        lsq = -diag_q + qmax - lnm_half;
+#pragma unroll
+        for (int fb = 0; fb < FB; ++fb) {
+            const floatx4 dd = qf[fb];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float keep = (16 * fb + 4 * g + i < a.mh_valid) ? 1.f : 0.f;
+                qf[fb][i] = keep * __builtin_amdgcn_exp2f((dd[i] - qmax) * LOG2E);
+                qf[FB + fb][i] = keep * __builtin_amdgcn_exp2f((-dd[i] - qmax) * LOG2E);
+            }
+        }
+        __syncthreads();                 // the projection rows are dead; the tile buffers may overwrite them
+    }
+    FLY_PROF(1);
+    // normaliser of the global low-rank term, from the fp32 features
+    float qk1 = 0.f;
+    if (lowrank_here) {
+#pragma unroll
+        for (int c = 0; c < 2 * FB; ++c) {
+            const floatx4 ks = *reinterpret_cast<const floatx4*>(a.ksum + (long)bh * M + 16 * c + 4 * g);
+            qk1 += qf[c][0] * ks[0] + qf[c][1] * ks[1] + qf[c][2] * ks[2] + qf[c][3] * ks[3];
+        }
+        qk1 = group_sum(qk1);
+    }
+    // overlap operand: two 16-feature blocks make the eight k-slots of one MFMA step
+    uint4 qfb[M / 32];
+#pragma unroll
+    for (int ks = 0; ks < M / 32; ++ks)
+        qfb[ks] = make_uint4(pack_bf16x2(qf[2 * ks][0], qf[2 * ks][1]), pack_bf16x2(qf[2 * ks][2], qf[2 * ks][3]),
+                             pack_bf16x2(qf[2 * ks + 1][0], qf[2 * ks + 1][1]), pack_bf16x2(qf[2 * ks + 1][2], qf[2 * ks + 1][3]));
+
+    const float sc = a.temp * LOG2E;             // scores leave the MFMA unscaled; exponents are base 2
+    const float c0 = (lsq + kmax) * LOG2E;       // base-2 log-scale of the global low-rank term
+    float m_run = c0;
+    float ze = 0.f, zp = 0.f;
+    floatx4 oacc[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) oacc[db] = Frag<float>::zero();
+    const int qw0 = q0 + 16 * w;
+    const int smin = max(iq - lc_lo, 0);
+    const unsigned span = qvalid ? (unsigned)max(min(iq + lc_hi, len) - smin, 0) : 0u;
+
+    if (kt_lo < kt_hi) stash(ra, 0);
+    __syncthreads();
+
+    // One key tile takes two phases: scores (LDS fragment reads and the two score MFMA products) and
+    // softmax (the arithmetic on the scores and P V).  The first phase loads the LDS and matrix
+    // pipes, the second the vector ALU; the waves of a workgroup pass them in lock step if left
+    // alone, so the upper half of the waves runs half a tile behind the lower half: while one half
+    // reads fragments and multiplies, the other half does its softmax arithmetic.  A wave's scores
+    // and V fragments of a tile stay in registers between the two phases.
+    floatx4 s1[KB], s2[KB];
+    uint4 vf[DB];
+    auto touches = [&](int kt) __attribute__((always_inline)) {      // wave-uniform: does the tile touch the band of any of the wave's queries?
+        const int s_base = kt * TK;
+        return !(s_base + TK - 1 - qw0 < -lc_lo || s_base - (qw0 + 15) >= lc_hi || s_base >= len);
+    };
+    auto score_phase = [&](int kt, int stage) __attribute__((always_inline)) {
+        if (!touches(kt)) return;
+        const uint16_t* Ks = lds + stage * STAGE;
+        const uint16_t* Fs = Ks + TK * LDK;
+        const uint16_t* Vt = Fs + TK * LDF;
+        // fragments are requested from LDS in batches ahead of the MFMAs that use them (the scheduling
+        // barriers keep the loads from sinking to their uses, where each would wait alone); the feature
+        // fragments come in two batches to stay inside the register budget
+        constexpr int FS = M / 32, FH = FS > 4 ? FS / 2 : FS;
+        uint4 kf[E / 32][KB], ff[FH][KB];
+#pragma unroll
+        for (int ks = 0; ks < E / 32; ++ks)
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb)
+                kf[ks][kb] = *reinterpret_cast<const uint4*>(Ks + (16 * kb + r16) * LDK + 32 * ks + 8 * g);
+#pragma unroll
+        for (int ks = 0; ks < FH; ++ks)
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb)
+                ff[ks][kb] = *reinterpret_cast<const uint4*>(Fs + (16 * kb + r16) * LDF + 32 * ks + 8 * g);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) { s1[kb] = Frag<float>::zero(); s2[kb] = Frag<float>::zero(); }
+#pragma unroll
+        for (int ks = 0; ks < E / 32; ++ks)
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) s1[kb] = mma_bf16(kf[ks][kb], qb[ks], s1[kb]);
+#pragma unroll
+        for (int ks = 0; ks < FH; ++ks)
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) s2[kb] = mma_bf16(ff[ks][kb], qfb[ks], s2[kb]);
+        if (FH < FS) {
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int ks = FH; ks < FS; ++ks)
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb)
+                    ff[ks - FH][kb] = *reinterpret_cast<const uint4*>(Fs + (16 * kb + r16) * LDF + 32 * ks + 8 * g);
+#pragma unroll
+            for (int db = 0; db < DB; ++db) vf[db] = *reinterpret_cast<const uint4*>(Vt + (16 * db + r16) * LDT + 8 * g);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int ks = FH; ks < FS; ++ks)
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb) s2[kb] = mma_bf16(ff[ks - FH][kb], qfb[ks], s2[kb]);
+        } else {
+#pragma unroll
+            for (int db = 0; db < DB; ++db) vf[db] = *reinterpret_cast<const uint4*>(Vt + (16 * db + r16) * LDT + 8 * g);
+        }
+    };
+    auto soft_phase = [&](int kt, float cscale) __attribute__((always_inline)) {
+        if (!touches(kt)) return;
+        const int s_base = kt * TK;
+        const float wc = __builtin_amdgcn_exp2f((cscale - kmax) * LOG2E);
+        // lane holds the raw scores q.k of query iq against keys s_base + 16kb + 4g + i (the softmax
+        // scale enters through one fma per exponent).  Tiles that lie inside the band of all 16
+        // queries of the wave -- most of them -- skip the masks.
+        const bool inside = s_base >= max(qw0 + 15 - lc_lo, 0) && s_base + TK <= min(qw0 + lc_hi, len) && qw0 + 15 < a.T;
+        floatx4 p[KB];
+        float ovs = 0.f;
+        auto soft = [&](auto masked_t) __attribute__((always_inline)) {
+            constexpr bool MASKED = decltype(masked_t)::value;
+            bool ok[KB][4];
+            float mx = -INFINITY;
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int s = s_base + 16 * kb + 4 * g + i;
+                    ok[kb][i] = !MASKED || (unsigned)(s - smin) < span;
+                    mx = fmaxf(mx, ok[kb][i] ? s1[kb][i] : -INFINITY);
+                }
+            mx = group_max(mx) * sc;                               // sc > 0
+            if (__builtin_amdgcn_ballot_w64(mx > m_run) != 0) {      // wave-uniform: some row maximum grew
+                const float m_new = fmaxf(m_run, mx);
+                const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+                m_run = m_new;
+                ze *= alpha;
+#pragma unroll
+                for (int db = 0; db < DB; ++db) oacc[db] *= alpha;
+            }
+            const float beta = wc * __builtin_amdgcn_exp2f(c0 - m_run);      // scale of the overlap term, <= 1
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float e = ok[kb][i] ? __builtin_amdgcn_exp2f(__builtin_fmaf(s1[kb][i], sc, -m_run)) : 0.f;
+                    const float ov = ok[kb][i] ? s2[kb][i] : 0.f;
+                    ze += e;
+                    ovs += ov;
+                    p[kb][i] = e - ov * beta;
+                }
+        };
+        if (inside) soft(std::false_type{}); else soft(std::true_type{});
+        zp += ovs * wc;
+        // O^T[d][query] += sum_keys V[key][d] p[key][query]: one MFMA step per 16 value dims
+        const uint4 pb = make_uint4(pack_bf16x2(p[0][0], p[0][1]), pack_bf16x2(p[0][2], p[0][3]),
+                                    pack_bf16x2(p[1][0], p[1][1]), pack_bf16x2(p[1][2], p[1][3]));
+#pragma unroll
+        for (int db = 0; db < DB; ++db) oacc[db] = mma_bf16(vf[db], pb, oacc[db]);
+    };
+    const bool late = w >= NW / 2;        // wave-uniform: this wave runs half a tile behind
+    float cs_prev = 0.f;                  // chunk scale of the tile a late wave still owes its softmax
+    auto tile_step = [&](int kt, int stage, float cscale) __attribute__((always_inline)) {
+        if (!late) {
+            score_phase(kt, stage);
+            soft_phase(kt, cscale);
+        } else {
+            if (kt > kt_lo) soft_phase(kt - 1, cs_prev);
+            score_phase(kt, stage);
+            cs_prev = cscale;
+        }
+    };
+
+    FLY_PROF(2);
+    // even steps: tile kt sits in stage 0 (from ra), rb holds kt + 1, ra is refilled with kt + 2;
+    // odd steps the other way round
+    for (int kt = kt_lo; kt < kt_hi; kt += 2) {
+        const float cs0 = ra.cscale;
+        if (kt + 2 < kt_hi) fetch(ra, kt + 2);
+        tile_step(kt, 0, cs0);
+        if (kt + 1 < kt_hi) stash(rb, 1);
+        __syncthreads();
+        if (kt + 1 >= kt_hi) break;
+        const float cs1 = rb.cscale;
+        if (kt + 3 < kt_hi) fetch(rb, kt + 3);
+        tile_step(kt + 1, 1, cs1);
+        if (kt + 2 < kt_hi) stash(ra, 0);
+        __syncthreads();
+    }
+    if (late && kt_lo < kt_hi) soft_phase(kt_hi - 1, cs_prev);
+
+    FLY_PROF(3);
+    // global low-rank term: qkv^T[d][query] = sum_r KV[r][d] q'[query][r]; K'^T V comes as bf16, transposed,
+    // features in the slot order of the overlap operand
+    floatx4 lacc[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) lacc[db] = Frag<float>::zero();
+    if (lowrank_here) {
+        uint16_t* KVt = lds;
+        // written by the combine kernel as bf16 [d][slot]: a plain copy in 16-byte pieces
+        const uint16_t* kvg = reinterpret_cast<const uint16_t*>(a.kvt) + (long)bh * M * D;
+        constexpr int KVC = D * M / 8;
+#pragma unroll
+        for (int j = 0; j < (KVC + NT - 1) / NT; ++j) {
+            const int idx = tid + NT * j, d = idx / (M / 8), c8 = idx % (M / 8);
+            if (KVC % NT == 0 || idx < KVC)
+                *reinterpret_cast<uint4*>(KVt + d * LDKV + 8 * c8) = *reinterpret_cast<const uint4*>(kvg + (long)d * M + 8 * c8);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int ks = 0; ks < M / 32; ++ks)
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+                lacc[db] = mma_bf16(*reinterpret_cast<const uint4*>(KVt + (16 * db + r16) * LDKV + 32 * ks + 8 * g), qfb[ks], lacc[db]);
+    }
+    FLY_PROF(4);
+    ze = group_sum(ze);
+    zp = group_sum(zp);
+    const float gamma = __builtin_amdgcn_exp2f(c0 - m_run);               // <= 1
+    if (SPLIT) {
+        // partials are kept per 64-query tile (the unit of sb_merge_kernel); this wave's tile:
+        const int n_qt64 = (a.T + TQ64 - 1) / TQ64, t64 = (q0 + 16 * w) / TQ64;
+        if (t64 < n_qt64) {                            // wave-uniform
+            float* ws = a.part_ws + (((long)bh * n_qt64 + t64) * a.n_parts + part) * (TQ64 * (D + NSTAT));
+            const int ql = (16 * w + r16) % TQ64;
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                floatx4 o = oacc[db] + gamma * lacc[db];
+                *reinterpret_cast<floatx4*>(ws + ql * D + 16 * db + 4 * g) = o;
+            }
+            if (g == 0) {
+                float* st = ws + TQ64 * D;
+                st[0 * TQ64 + ql] = m_run;
+                st[1 * TQ64 + ql] = ze;
+                st[2 * TQ64 + ql] = zp;
+                st[3 * TQ64 + ql] = qk1;
+                st[4 * TQ64 + ql] = c0;
+            }
+        }
+    } else {
+        const float Z = ze + gamma * fmaxf(qk1 - zp, 1e-24f);
+        const float inv = 1.0f / Z;
+        if (qvalid) {
+            T* optr = reinterpret_cast<T*>(a.out) + b * a.o_sb + h * a.o_sh + (long)iq * a.o_ss;
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                floatx4 o = (oacc[db] + gamma * lacc[db]) * inv;
+                store4_f32(optr + 16 * db + 4 * g, o);
+            }
+            if (g == 0) a.log_norm[(long)bh * a.T + iq] = m_run * LN2 + __logf(Z);
+        }
+    }
+    FLY_PROF(5);
 }
 
 // Merge of the per-part partials of one query tile by the 256 threads of a workgroup: thread
@@ -485,7 +970,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
     const T* qptr = reinterpret_cast<const T*>(a.q) + b * a.q_sb + h * a.q_sh;
     const T* kptr = reinterpret_cast<const T*>(a.k) + b * a.k_sb + h * a.k_sh;
     const T* vptr = reinterpret_cast<const T*>(a.v) + b * a.v_sb + h * a.v_sh;
-    const float* fptr = a.kfeat + (long)bh * a.n_chunks * CH * M;
+    const float* fptr = reinterpret_cast<const float*>(a.kfeat) + (long)bh * a.n_chunks * CH * M;
     const int len = a.lens ? min((int)a.lens[b], a.S) : a.S;
     const float lnm_half = 0.5f * __logf(2.0f * a.mh_valid);
     const int lc_lo = a.lc / 2, lc_hi = (a.lc + 1) / 2;    // band: -lc_lo <= s - i < lc_hi
@@ -814,10 +1299,31 @@ static int launch_kfeat(const KvArgs& a, hipStream_t st) {
 // band kernel of the next flyhip_sblocal_fwd call made by this thread (then cleared).
 static thread_local hipEvent_t g_ev_before = nullptr, g_ev_after = nullptr;
 
+template <int E, int M> constexpr size_t fwd_bf16_smem() {
+    constexpr size_t stage = (size_t)TK * (E + 8) + (size_t)TK * (M + 8) + (size_t)E * (TK + 8);   // 2-byte elements
+    constexpr size_t tiles = 2 * stage * 2;
+    constexpr size_t proj = (size_t)2 * (M / 2) * (E + 8) * 2;      // bf16 head and remainder of the projection
+    constexpr size_t lowrank = (size_t)E * (M + 8) * 2;
+    constexpr size_t need = tiles > proj ? (tiles > lowrank ? tiles : lowrank) : (proj > lowrank ? proj : lowrank);
+    return need;
+}
+
+// float inputs: fp32 MFMA kernel; bfloat16 inputs: bf16 MFMA kernel
+template <typename T, int E, int M, bool SPLIT> struct FwdKernel {
+    static constexpr size_t smem = fwd_smem<E, M>();
+    static constexpr int threads = NT, tq = TQ;       // threads and queries per workgroup
+    static auto get() { return sblocal_fwd_kernel<T, E, E, M, SPLIT>; }
+};
+template <int E, int M, bool SPLIT> struct FwdKernel<bf16_t, E, M, SPLIT> {
+    static constexpr size_t smem = fwd_bf16_smem<E, M>();
+    static constexpr int threads = 64 * BF16_WAVES, tq = 16 * BF16_WAVES;
+    static auto get() { return sblocal_fwd_bf16_kernel<E, E, M, SPLIT, BF16_WAVES>; }
+};
+
 template <typename T, int E, int M, bool SPLIT>
 static int launch_fwd_impl(const FwdArgs& a, hipStream_t st) {
-    auto kern = sblocal_fwd_kernel<T, E, E, M, SPLIT>;
-    constexpr size_t smem = fwd_smem<E, M>();
+    auto kern = FwdKernel<T, E, M, SPLIT>::get();
+    constexpr size_t smem = FwdKernel<T, E, M, SPLIT>::smem;
     static bool lds_ready = false;
     if (!lds_ready) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -825,12 +1331,13 @@ static int launch_fwd_impl(const FwdArgs& a, hipStream_t st) {
         if (e != hipSuccess) return fail(ERR_LAUNCH, "sblocal_fwd: LDS attribute: %s", hipGetErrorString(e));
         lds_ready = true;
     }
-    const int qt = (a.T + TQ - 1) / TQ;
-    const long items = (long)a.B * a.H * qt * a.n_parts;
+    typedef FwdKernel<T, E, M, SPLIT> K;
+    const int qt = (a.T + TQ - 1) / TQ;                           // 64-query tiles (partials, merge)
+    const long items = (long)a.B * a.H * ((a.T + K::tq - 1) / K::tq) * a.n_parts;
     const long grid = (items + N_XCD - 1) / N_XCD * N_XCD;       // whole rounds over the XCDs
     if (grid > 2147483647L) return fail(ERR_ARG, "sblocal_fwd: too many workgroups");
     if (g_ev_before) (void)hipEventRecord(g_ev_before, st);
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NT), smem, st, a);
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(K::threads), smem, st, a);
     if (g_ev_after) (void)hipEventRecord(g_ev_after, st);
     g_ev_before = g_ev_after = nullptr;
     int rc = check_launch("sblocal_fwd_kernel");
@@ -925,17 +1432,17 @@ static int check_sb_dims(const char* who, int E, int D, int mh, int mh_valid, in
                          int64_t s0, int64_t s1, int64_t s2) {
     FLY_REQUIRE(E == D, "%s: padded head dims must be equal (E=%d, D=%d)", who, E, D);
     FLY_REQUIRE(mh_valid >= 1 && mh_valid <= mh, "%s: mh_valid=%d outside [1, mh=%d]", who, mh_valid, mh);
-    FLY_REQUIRE((s0 % 4) == 0 && (s1 % 4) == 0 && (s2 % 4) == 0,
-                "%s: strides must be multiples of 4 elements (16-byte vector access)", who);
-    (void)dtype;
+    const int64_t gran = dtype == BF16 ? 8 : 4;
+    FLY_REQUIRE((s0 % gran) == 0 && (s1 % gran) == 0 && (s2 % gran) == 0,
+                "%s: strides must be multiples of %d elements (16-byte vector access)", who, (int)gran);
     return OK;
 }
 
 extern "C" int flyhip_sb_kv_reduce(const void* k, const void* v, const float* proj, const int64_t* key_lengths,
-                                   float* kfeat, float* chunk_scale, float* kv_part, float* part_max,
+                                   void* kfeat, float* chunk_scale, float* kv_part, float* part_max,
                                    float* kv, float* ksum, float* kmax,
                                    const void* q, float* qfeat, float* q_lsq, int T,
-                                   int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                                   int64_t q_sb, int64_t q_sh, int64_t q_ss, void* vt, void* kvt,
                                    int B, int H, int S, int E, int D, int mh, int mh_valid, int n_split,
                                    int64_t k_sb, int64_t k_sh, int64_t k_ss,
                                    int64_t v_sb, int64_t v_sh, int64_t v_ss,
@@ -951,6 +1458,8 @@ extern "C" int flyhip_sb_kv_reduce(const void* k, const void* v, const float* pr
     FLY_REQUIRE(n_split >= 1 && n_split <= nc && n_split <= MAX_SPLIT,
                 "sb_kv_reduce: n_split=%d outside [1, min(%d, %d)]", n_split, nc, MAX_SPLIT);
     FLY_REQUIRE((long)B * H <= 65535, "sb_kv_reduce: B*H=%ld exceeds the grid limit 65535", (long)B * H);
+    FLY_REQUIRE(dtype != BF16 || (vt && kvt), "sb_kv_reduce: bfloat16 inputs need the vt and kvt scratch");
+    if (dtype != BF16) vt = kvt = nullptr;
     if (q) {
         FLY_REQUIRE(qfeat && q_lsq && T > 0, "sb_kv_reduce: query features asked for without qfeat / q_lsq / T");
         FLY_REQUIRE(((q_sb | q_sh | q_ss) % 4) == 0, "sb_kv_reduce: q strides must be multiples of 4 elements");
@@ -958,21 +1467,21 @@ extern "C" int flyhip_sb_kv_reduce(const void* k, const void* v, const float* pr
     KvArgs a{k, v, proj, key_lengths, kfeat, chunk_scale, kv_part, part_max,
              B, H, S, mh_valid, nc, n_split, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, softmax_temp,
              q, qfeat, q_lsq, q ? T : 0, q_sb, q_sh, q_ss,
-             q ? (T + TQ - 1) / TQ : 0};
+             q ? (T + TQ - 1) / TQ : 0, vt};
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     const int m = 2 * mh;
     rc = dispatch_kfeat(dtype, E, m, a, st);
     if (rc) return rc;
     const int per = m * (D + 1);
     hipLaunchKernelGGL(sb_combine_kernel, dim3((per + NT - 1) / NT, B * H), dim3(NT), 0, st,
-                       kv_part, part_max, kv, ksum, kmax, n_split, m, D);
+                       kv_part, part_max, kv, ksum, kmax, reinterpret_cast<uint16_t*>(kvt), n_split, m, D);
     return check_launch("sb_combine_kernel");
 }
 
 extern "C" int flyhip_sblocal_fwd(const void* q, const void* k, const void* v, const float* proj,
-                                  const float* kfeat, const float* chunk_scale,
+                                  const void* kfeat, const float* chunk_scale,
                                   const float* kv, const float* ksum, const float* kmax,
-                                  const float* qfeat, const float* q_lsq,
+                                  const float* qfeat, const float* q_lsq, const void* vt, const void* kvt,
                                   const int64_t* key_lengths, void* out, float* log_norm,
                                   float* part_ws, int n_parts,
                                   int B, int H, int T, int S, int E, int D, int mh, int mh_valid,
@@ -992,11 +1501,12 @@ extern "C" int flyhip_sblocal_fwd(const void* q, const void* k, const void* v, c
     if (rc) return rc;
     FLY_REQUIRE((long)B * H <= 65535, "sblocal_fwd: B*H=%ld exceeds the grid limit 65535", (long)B * H);
     FLY_REQUIRE(n_parts >= 1 && n_parts <= 64, "sblocal_fwd: n_parts=%d outside [1, 64]", n_parts);
+    FLY_REQUIRE(dtype != BF16 || (vt && kvt), "sblocal_fwd: bfloat16 inputs need the vt and kvt scratch of the key pass");
     FLY_REQUIRE(n_parts == 1 || (part_ws && qfeat && q_lsq),
                 "sblocal_fwd: n_parts > 1 needs the partial workspace and the query features of the key pass");
     int nc, ns;
     plan(B, H, S, &nc, &ns);
-    FwdArgs a{q, k, v, proj, kfeat, chunk_scale, kv, ksum, kmax, qfeat, q_lsq, key_lengths, out, log_norm, part_ws,
+    FwdArgs a{q, k, v, proj, kfeat, chunk_scale, kv, ksum, kmax, qfeat, q_lsq, vt, kvt, key_lengths, out, log_norm, part_ws,
               B, H, T, S, mh_valid, local_context, nc, n_parts,
               q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss, softmax_temp};
     return dispatch_fwd(dtype, E, 2 * mh, a, reinterpret_cast<hipStream_t>(stream));

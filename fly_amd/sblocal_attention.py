@@ -48,13 +48,18 @@ class SBLocalPlan:
         self.device = torch.device(device)
         self.code = _lib.DTYPE_CODE[dtype]
         m, f32 = 2 * mh, torch.float32
-        self.kfeat = torch.empty(B, H, self.n_chunks * 64, m, dtype=f32, device=device)
+        self.kfeat = torch.empty(B, H, self.n_chunks * 64, m, dtype=dtype, device=device)   # opaque, in the input dtype
         self.chunk_scale = torch.empty(B, H, self.n_chunks, dtype=f32, device=device)
         self.kv_part = torch.empty(B, H, self.n_split, m * (dim + 1), dtype=f32, device=device)
         self.part_max = torch.empty(B, H, self.n_split, dtype=f32, device=device)
         self.kv = torch.empty(B, H, m, dim, dtype=f32, device=device)
         self.ksum = torch.empty(B, H, m, dtype=f32, device=device)
         self.kmax = torch.empty(B, H, dtype=f32, device=device)
+        # bf16 inputs: V per 32-key tile and K'^T V in the operand order of the bf16 MFMA (opaque)
+        self.vt = self.kvt = None
+        if dtype == torch.bfloat16:
+            self.vt = torch.empty(B, H, self.n_chunks * 64, dim, dtype=dtype, device=device)
+            self.kvt = torch.empty(B, H, dim, m, dtype=dtype, device=device)
         # with several parts per query tile the key pass also computes the query features, once
         self.part_ws = self.qfeat = self.q_lsq = None
         if self.n_parts > 1:
@@ -75,7 +80,7 @@ class SBLocalPlan:
         _lib.call('flyhip_sb_kv_reduce', k.data_ptr(), v.data_ptr(), proj.data_ptr(), _lib.ptr(lens),
                   self.kfeat.data_ptr(), self.chunk_scale.data_ptr(), self.kv_part.data_ptr(),
                   self.part_max.data_ptr(), self.kv.data_ptr(), self.ksum.data_ptr(), self.kmax.data_ptr(),
-                  *q_args, B, H, S, dim, dim, mh, mh_valid, self.n_split,
+                  *q_args, _lib.ptr(self.vt), _lib.ptr(self.kvt), B, H, S, dim, dim, mh, mh_valid, self.n_split,
                   k.stride(0), k.stride(2), k.stride(1), v.stride(0), v.stride(2), v.stride(1),
                   t, self.code, stream)
 
@@ -85,7 +90,7 @@ class SBLocalPlan:
         _lib.call('flyhip_sblocal_fwd', q.data_ptr(), k.data_ptr(), v.data_ptr(), proj.data_ptr(),
                   self.kfeat.data_ptr(), self.chunk_scale.data_ptr(), self.kv.data_ptr(),
                   self.ksum.data_ptr(), self.kmax.data_ptr(), _lib.ptr(self.qfeat), _lib.ptr(self.q_lsq),
-                  _lib.ptr(lens), out.data_ptr(), log_norm.data_ptr(), _lib.ptr(self.part_ws), self.n_parts,
+                  _lib.ptr(self.vt), _lib.ptr(self.kvt), _lib.ptr(lens), out.data_ptr(), log_norm.data_ptr(), _lib.ptr(self.part_ws), self.n_parts,
                   B, H, T, S, dim, dim, mh, mh_valid, local_context,
                   q.stride(0), q.stride(2), q.stride(1), k.stride(0), k.stride(2), k.stride(1),
                   v.stride(0), v.stride(2), v.stride(1), out.stride(0), out.stride(2), out.stride(1),

@@ -43,8 +43,10 @@ int flyhip_sb_plan(int B, int H, int T, int S, int local_context,
  *   proj (mh, E) fp32 row-major, rows >= mh_valid ignored (zero rows); E = D in {32,64,128},
  *   m = 2*mh in {32,64,128,256}
  *   key_lengths (B) int64 or NULL
- * outputs (all fp32):
- *   kfeat       (B,H,n_chunks*64,m)  positive random features of every key, stabilised per chunk
+ * outputs (fp32 unless noted):
+ *   kfeat       (B,H,n_chunks*64,m)  positive random features of every key, stabilised per chunk;
+ *                                    opaque scratch in the element type of k (fp32, or bf16 in the
+ *                                    k-slot order of the bf16 MFMA) -- only flyhip_sblocal_fwd reads it
  *   chunk_scale (B,H,n_chunks)       log-stabiliser each chunk of kfeat was written with
  *   kv (B,H,m,D), ksum (B,H,m), kmax (B,H)  global reductions in units of exp(kmax)
  * scratch: kv_part (B,H,n_split,m*(D+1)), part_max (B,H,n_split).
@@ -52,12 +54,15 @@ int flyhip_sb_plan(int B, int H, int T, int S, int local_context,
  * several workgroups share a query tile): q (B,T,H,E) via strides -> qfeat (B,H,T,m) fp32, the
  * query features exp(+-sqrt(t) P q - rowmax) (ref: softmax_kernel with is_query=True,
  * src/models/attention/feature_maps_sb.py:51-82,148-151), and q_lsq (B,H,T) fp32, their log-scale
- * -t|q|^2/2 + rowmax - log(m)/2. */
+ * -t|q|^2/2 + rowmax - log(m)/2.
+ * bfloat16 inputs only (NULL otherwise): vt (B,H,n_chunks*64,D) bf16 and kvt (B,H,D,m) bf16, opaque
+ * scratch for flyhip_sblocal_fwd -- V per 32-key tile and K'^T V, transposed into the operand
+ * order of the bf16 MFMA. */
 int flyhip_sb_kv_reduce(const void* k, const void* v, const float* proj, const int64_t* key_lengths,
-                        float* kfeat, float* chunk_scale, float* kv_part, float* part_max,
+                        void* kfeat, float* chunk_scale, float* kv_part, float* part_max,
                         float* kv, float* ksum, float* kmax,
                         const void* q, float* qfeat, float* q_lsq, int T,
-                        int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                        int64_t q_sb, int64_t q_sh, int64_t q_ss, void* vt, void* kvt,
                         int B, int H, int S, int E, int D, int mh, int mh_valid, int n_split,
                         int64_t k_sb, int64_t k_sh, int64_t k_ss,
                         int64_t v_sb, int64_t v_sh, int64_t v_ss,
@@ -71,11 +76,11 @@ int flyhip_sb_kv_reduce(const void* k, const void* v, const float* proj, const i
  *   n_parts from flyhip_sb_plan (any value in [1,64] is valid); when > 1, part_ws is scratch of
  *   B*H*ceil(T/64)*n_parts*64*(D+5) floats and qfeat / q_lsq are the query-side outputs of
  *   flyhip_sb_kv_reduce for the same q; with n_parts == 1 all three may be NULL (the kernel forms
- *   the query features itself). */
+ *   the query features itself).  vt / kvt: the bf16 scratch of flyhip_sb_kv_reduce (NULL for fp32). */
 int flyhip_sblocal_fwd(const void* q, const void* k, const void* v, const float* proj,
-                       const float* kfeat, const float* chunk_scale,
+                       const void* kfeat, const float* chunk_scale,
                        const float* kv, const float* ksum, const float* kmax,
-                       const float* qfeat, const float* q_lsq,
+                       const float* qfeat, const float* q_lsq, const void* vt, const void* kvt,
                        const int64_t* key_lengths, void* out, float* log_norm,
                        float* part_ws, int n_parts,
                        int B, int H, int T, int S, int E, int D, int mh, int mh_valid,
