@@ -9,6 +9,7 @@ from .blocksparse_utils import sparsify_tensor, densify_tensor, mask_tensor, spa
 from .blocksparse_matmul import matmul
 from .blocksparse_softmax import softmax, logsumexp, blocksparse_sum
 from .blocksparse_attention import BlockSparseAttention
+from .sbblocksparse_attention import SBBlockSparseAttention
 from .blocksparse_linear import BlockSparseLinear, FlatBlockButterflySparsityConfig
 from .fastlinear import LowRank, SparseLRLinear
 from .t2t_vit import T2T_ViT, T2T_module, T2TAttention, Token_transformer, MlpCustom, t2t_vit_t_14
@@ -17,5 +18,6 @@ __all__ = ['FullMask', 'LengthMask', 'TriangularCausalMask', 'SBPerformerFeature
            'gaussian_orthogonal_random_matrix', 'SBLocalAttention', 'sblocal_forward',
            'sparsify_tensor', 'densify_tensor', 'mask_tensor', 'sparsify_broadcast_tensor',
            'matmul', 'softmax', 'logsumexp', 'blocksparse_sum', 'BlockSparseAttention',
+           'SBBlockSparseAttention',
            'BlockSparseLinear', 'FlatBlockButterflySparsityConfig', 'LowRank', 'SparseLRLinear',
            'T2T_ViT', 'T2T_module', 'T2TAttention', 'Token_transformer', 'MlpCustom', 't2t_vit_t_14']

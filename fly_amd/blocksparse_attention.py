@@ -30,6 +30,7 @@ def instantiate(cfg, *args, **kwargs):
                   'src.models.layers.fastlinear': 'fly_amd.fastlinear',
                   'src.models.attention.sblocal_attention': 'fly_amd.sblocal_attention',
                   'src.models.attention.blocksparse_attention': 'fly_amd.blocksparse_attention',
+                  'src.models.attention.sbblocksparse_attention': 'fly_amd.sbblocksparse_attention',
                   'src.models.layers.mlp': 'fly_amd.t2t_vit',
                   }.get(module, module)
         return getattr(importlib.import_module(module), name)(*args, **{**cfg, **kwargs})

@@ -50,6 +50,7 @@ def sparsify_broadcast_tensor(x, mask, block=None):
     """x (B, H, T) -> (B, nnz, blk, 1): for every nonzero block the slice of x for its rows (:60-74).
     `block` is accepted and ignored: the reference's callers pass it although the reference
     function takes two arguments (sbblocksparse_attention.py:197,199)."""
+    mask = _as_layout3(mask)
     blk = x.shape[-1] // mask.shape[-2]
     rows = x.reshape(x.shape[0], x.shape[1], mask.shape[-2], blk, 1)
     h_idx, row_idx, _ = torch.nonzero(mask, as_tuple=True)

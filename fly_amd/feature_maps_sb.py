@@ -1,9 +1,10 @@
 """Performer random features for Scatterbrain attention: the projection matrix and the module
 that owns it (src/models/attention/projection_utils.py:8-28, feature_maps_sb.py:85-156).
 
-The feature values themselves (feature_maps_sb.py:51-82) are never materialised by this
-package for the queries and only as a kernel-internal workspace for the keys: they are computed
-inside the HIP kernels behind ``SBLocalAttention``.
+Behind ``SBLocalAttention`` the feature values (feature_maps_sb.py:51-82) are computed inside
+the HIP kernels and never reach the caller.  ``softmax_kernel`` / ``forward_queries`` /
+``forward_keys`` give them as tensors for the layers that feed them to the block-sparse matmuls
+(``SBBlockSparseAttention``).
 """
 import math
 
@@ -29,6 +30,37 @@ def gaussian_orthogonal_random_matrix(nrows, ncols, scaling=0, device=None, dtyp
     else:
         raise ValueError(f'Invalid scaling {scaling}')
     return rows.to(device=device, dtype=dtype)
+
+
+def softmax_kernel(data, *, projection_matrix, is_query, softmax_temp=None, eps=0., cosh=True,
+                   return_log=False):
+    """Positive random features of `data` (..., S, D) with their log-scale (feature_maps_sb.py:51-82):
+    features = exp(+-sqrt(t) P x - stabiliser), where queries are stabilised per row (and the
+    log-scale carries -t|x|^2/2 + rowmax - log(m)/2) and keys by one maximum over the last two
+    dimensions.  Returns (features or their logs, in the dtype of `data`; log_scale)."""
+    if return_log and eps != 0:
+        raise NotImplementedError('return_log is not compatible with nonzero eps')
+    if not cosh:
+        raise NotImplementedError('only the cosh (two-sided) feature map is implemented')
+    d = data.shape[-1]
+    m = 2 * projection_matrix.shape[0]
+    if softmax_temp is None:
+        softmax_temp = 1 / math.sqrt(d)
+    normalizer = math.sqrt(softmax_temp)
+    dash = torch.matmul(data, (normalizer * projection_matrix.type_as(data)).t())
+    dash = torch.cat([dash, -dash], dim=-1)
+    diag = data.square().sum(dim=-1, keepdim=True) / 2 * softmax_temp
+    if is_query:
+        row_max = torch.amax(dash, dim=-1, keepdim=True)
+        log_scale = -diag + row_max - math.log(m) / 2
+        dash_log = dash - row_max
+    else:
+        shifted = dash - diag - math.log(m) / 2
+        log_scale = torch.amax(shifted, dim=(-1, -2), keepdim=True)
+        dash_log = shifted - log_scale
+    if return_log:
+        return dash_log.type_as(data), log_scale
+    return (torch.exp(dash_log) + eps / math.sqrt(m)).type_as(data), log_scale
 
 
 class SBPerformerFeatures(nn.Module):
@@ -77,3 +109,13 @@ class SBPerformerFeatures(nn.Module):
                                                    scaling=self.ortho_scaling, device=device,
                                                    dtype=self.factory_kwargs['dtype'])
         self.register_buffer('projection_matrix', matrix)
+
+    def forward_queries(self, x, return_log=False):
+        return softmax_kernel(x, projection_matrix=self.projection_matrix, is_query=True,
+                              softmax_temp=self.softmax_temp, eps=self.eps, cosh=self.cosh,
+                              return_log=return_log)
+
+    def forward_keys(self, x, return_log=False):
+        return softmax_kernel(x, projection_matrix=self.projection_matrix, is_query=False,
+                              softmax_temp=self.softmax_temp, eps=self.eps, cosh=self.cosh,
+                              return_log=return_log)

@@ -1,0 +1,136 @@
+"""Scatterbrain attention on a block-sparse support: drop-in for ``SBBlockSparseAttention``
+(src/models/attention/sbblocksparse_attention.py:31-213).
+
+Exact softmax weights on the nonzero blocks of the layout, the Performer low-rank estimate
+everywhere else, one joint normalisation.  The block-sparse products (Q K^T and Q' K'^T on the
+support, weights x V), the row logsumexp / row sum and the fused weight formula run on the HIP
+kernels of this package; the feature maps and the global low-rank reductions are library GEMMs.
+"""
+import math
+
+import torch
+import torch.nn as nn
+from torch import distributed as dist
+
+from .blocksparse_attention import instantiate
+from .blocksparse_matmul import matmul
+from .blocksparse_softmax import blocksparse_sum, logsumexp
+from .blocksparse_utils import densify_tensor, sparsify_broadcast_tensor
+from .feature_maps_sb import SBPerformerFeatures
+from .padding import pad_to_multiple
+from .scatterbrain_utils import linear_attention, linear_attention_normalization
+
+
+class SBBlockSparseAttention(nn.Module):
+    """sparsity_config: an object with ``.block`` and ``.make_layout(seq_len) -> (H, nb, nb)`` or a
+    mapping with ``_target_``.  forward(query (B,T,H,E), key (B,S,H,E), value (B,S,H,D)) returns
+    (out (B,T,H,D), attn or None).  Like the reference (its assertion at :181) the layer takes no
+    masks, which also means sequence lengths that are multiples of the block."""
+
+    def __init__(self, sparsity_config, dim_heads, nb_features=None, ortho_scaling=0,
+                 causal=False, softmax_temp=None, attention_dropout=0.0, softmax_eps=0.0,
+                 max_seq_length=2048):
+        super().__init__()
+        if causal:
+            raise NotImplementedError('causal Scatterbrain attention is not part of this build '
+                                      '(the reference marks it unchecked, sbblocksparse_attention.py:147)')
+        self.sparsity_config = instantiate(sparsity_config)
+        self.feature_map = SBPerformerFeatures(dim_heads, nb_features, ortho_scaling=ortho_scaling,
+                                               softmax_temp=softmax_temp, eps=softmax_eps)
+        self.causal = causal
+        self.softmax_temp = softmax_temp
+        self.dropout = nn.Dropout(attention_dropout)
+        self.softmax_eps = softmax_eps
+        master_layout = self.sparsity_config.make_layout(max_seq_length)
+        self.register_buffer("master_layout", master_layout)
+        self._need_layout_synchronization = True
+        self.ops_cache = dict()
+
+    def get_layout(self, T, S=None):
+        if S is None:
+            S = T
+        if self._need_layout_synchronization and dist.is_available() and dist.is_initialized():
+            dist.broadcast(self.master_layout, src=0)
+            self._need_layout_synchronization = False
+        block = self.sparsity_config.block
+        if (T % block != 0) or (S % block != 0):
+            raise ValueError(f'Sequence lengths, {T} and {S}, needs to be divisible by block size {block}!')
+        layout = self.master_layout[..., :T // block, :S // block].cpu()
+        return layout if layout.dim() == 3 else layout.unsqueeze(0)      # a 2-D layout means one head
+
+    def get_ops(self, T, S=None):
+        if S is None:
+            S = T
+        if (T, S) not in self.ops_cache:
+            layout = self.get_layout(T, S)
+            block = self.sparsity_config.block
+            self.ops_cache[T, S] = (matmul(layout, block, 'sdd', trans_a=False, trans_b=True),
+                                    matmul(layout, block, 'dsd', trans_a=False, trans_b=False),
+                                    logsumexp(layout, block), blocksparse_sum(layout, block))
+        return self.ops_cache[T, S]
+
+    def forward(self, query, key, value, attn_mask=None, key_padding_mask=None, need_weights=False,
+                return_attn_unnormalized=False):
+        block = self.sparsity_config.block
+        if attn_mask is not None or key_padding_mask is not None:
+            raise NotImplementedError('SBBlockSparseAttention takes no masks (the reference asserts so, '
+                                      'sbblocksparse_attention.py:181)')
+        if query.shape[1] % block or key.shape[1] % block:
+            # padding would create a key padding mask, which the reference then refuses (:135-138, 181)
+            raise ValueError(f'Sequence lengths, {query.shape[1]} and {key.shape[1]}, needs to be divisible '
+                             f'by block size {block}!')
+        if query.shape[3] != self.feature_map.query_dims:
+            raise ValueError(f'query has head dim {query.shape[3]}, the feature map was built for '
+                             f'{self.feature_map.query_dims}')
+        query = pad_to_multiple(query, block, dims=(1, 3))          # :125-127 (no-ops for the lengths)
+        key = pad_to_multiple(key, block, dims=(1, 3))
+        value = pad_to_multiple(value, block, dims=(1, 3))
+        if query.shape[3] != self.feature_map.query_dims:
+            raise ValueError(f'head dim {self.feature_map.query_dims} must be a multiple of the block '
+                             f'size {block}: the padded queries no longer match the projection matrix')
+        B, T, H, E = query.shape
+        S = value.shape[1]
+        softmax_temp = self.softmax_temp or 1 / math.sqrt(E)       # :131
+
+        # 2-byte inputs are widened: the scores pass through HBM between the stages, and a score kept
+        # in bf16 (three significant digits, values of order 10) would cost percents in its exponential
+        in_dtype = query.dtype
+        query = query.permute(0, 2, 1, 3).float().contiguous()     # b h t e
+        key = key.permute(0, 2, 1, 3).float().contiguous()
+        value = value.permute(0, 2, 1, 3).float().contiguous()
+
+        self.feature_map.new_feature_map(query.device)
+        q_prime, q_prime_log_scale = self.feature_map.forward_queries(query)
+        k_prime, k_prime_log_scale = self.feature_map.forward_keys(key)
+        prime_log_scale = q_prime_log_scale + k_prime_log_scale     # (b h t 1)
+        q_prime_k_prime_1 = linear_attention_normalization(q_prime, k_prime)
+        q_prime_k_prime_v, attn_prime = linear_attention(q_prime, k_prime, value, need_weights=need_weights)
+
+        layout = self.get_layout(T, S)
+        sdd_nt, dsd_nn, sparse_logsumexp, sparse_sum = self.get_ops(T, S)
+        QK = sdd_nt(query, key)
+        QK.mul_(softmax_temp)
+        dots_prime = sdd_nt(q_prime, k_prime)
+
+        # joint normalisation first (:185-190)
+        QK_lse = sparse_logsumexp(QK).unsqueeze(-1)
+        dots_prime_sum = sparse_sum(dots_prime).unsqueeze(-1)
+        lr_log_normalization = torch.log((q_prime_k_prime_1.unsqueeze(-1) - dots_prime_sum).clamp_min_(1e-24)) \
+            + prime_log_scale
+        log_normalization = torch.logaddexp(QK_lse, lr_log_normalization)
+        prime_scale = torch.exp(prime_log_scale - log_normalization)
+
+        # weights on the support: exp(QK - log Z) with the low-rank overlap taken out (:195-200);
+        # dropout acts on the exact part only
+        log_normalization_sparse = sparsify_broadcast_tensor(log_normalization.squeeze(-1), layout, block)
+        prime_scale_sparse = sparsify_broadcast_tensor(prime_scale.squeeze(-1), layout, block)
+        dots = self.dropout(torch.exp(QK - log_normalization_sparse)) - dots_prime * prime_scale_sparse
+
+        out = (dsd_nn(dots, value) + q_prime_k_prime_v * prime_scale).to(in_dtype)
+
+        attn = None
+        if need_weights:
+            attn = densify_tensor(dots, layout) + attn_prime * prime_scale
+            if return_attn_unnormalized:
+                attn = (attn, attn * torch.exp(log_normalization), attn_prime * torch.exp(prime_log_scale))
+        return out.permute(0, 2, 1, 3), attn

@@ -215,3 +215,34 @@ def test_config2_layout_stage_parity_reduced():
     assert rel_err(p, ob.block_softmax(qk.cpu(), layout, block, scale=0.125)) <= 2e-2
     out = matmul(layout, block, 'dsd')(p, v.to(DEV))
     assert rel_err(out, ob.dsd(p.cpu(), v, layout, block)) <= 2e-2
+
+
+@pytest.mark.parametrize('dtype,block', [(torch.float32, 16), (torch.float32, 32), (torch.bfloat16, 32)])
+def test_sbblocksparse_attention_module(dtype, block):
+    """Scatterbrain on a block-sparse support (sbblocksparse_attention.py:109-213): output, and with
+    need_weights the dense attention matrix, against the oracle."""
+    from fly_amd import SBBlockSparseAttention, FlatBlockButterflySparsityConfig
+    from oracle import sbblocksparse as osbb
+    print('case', dtype, block, flush=True)
+    B, T, H, E = 2, 8 * block, 1, 64
+    torch.manual_seed(0)
+    layer = SBBlockSparseAttention(FlatBlockButterflySparsityConfig(4, 2, block=block), dim_heads=E,
+                                   nb_features=64, max_seq_length=T).to(DEV)
+    g = torch.Generator().manual_seed(4)
+    q, k, v = (torch.randn(B, T, H, E, generator=g).to(dtype) for _ in range(3))
+    q, k = q * E ** -0.25 * 2, k * E ** -0.25 * 2
+    out, attn = layer(q.to(DEV), k.to(DEV), v.to(DEV), need_weights=True)
+    P = layer.feature_map.projection_matrix.cpu().double()
+    layout = layer.get_layout(T)
+    ref_out, ref_ln = osbb.sbblocksparse_attention(q.double(), k.double(), v.double(), P, layout, block)
+    tol = 1e-4 if dtype == torch.float32 else 2e-2
+    assert out.shape == (B, T, H, E) and out.dtype == dtype
+    assert rel_err(out, ref_out) <= tol
+    # the attention matrix of the closed form: A / rowsum(A)
+    _, _ = osbb.dense_closed_form(q.double(), k.double(), v.double(), P, layout, block)
+    rows = attn.sum(-1)
+    assert float((rows.float().cpu() - 1).abs().max()) <= (1e-4 if dtype == torch.float32 else 3e-2)
+    ref_from_attn = torch.einsum('bhts,bshd->bthd', attn.double().cpu(), v.double())
+    assert rel_err(ref_from_attn, ref_out) <= tol
+    out2, none = layer(q.to(DEV), k.to(DEV), v.to(DEV))
+    assert none is None and torch.equal(out2, out)

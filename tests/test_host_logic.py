@@ -245,3 +245,23 @@ def test_blocksparse_linear_init_and_dense_backend():
         'bias', 'sparse.weight', 'low_rank.lr_weight1', 'low_rank.lr_weight2', 'gate.weight', 'gate.bias'}
     y = slr(torch.randn(10, 256))
     assert y.shape == (10, 512)
+
+
+def test_sbblocksparse_module_interface_and_refusals():
+    """Constructor / buffers of the block-sparse Scatterbrain layer and what it refuses before any launch
+    (the reference asserts masks away, sbblocksparse_attention.py:181; its causal path is unchecked, :147)."""
+    cfg = fly_amd.FlatBlockButterflySparsityConfig(4, 2, block=16)
+    layer = fly_amd.SBBlockSparseAttention(cfg, dim_heads=32, nb_features=32, max_seq_length=256)
+    assert tuple(layer.master_layout.shape) == (16, 16)           # a 2-D layout means one head
+    assert tuple(layer.feature_map.projection_matrix.shape) == (16, 32)
+    assert tuple(layer.get_layout(64).shape) == (1, 4, 4)
+    with pytest.raises(NotImplementedError):
+        fly_amd.SBBlockSparseAttention(cfg, dim_heads=32, causal=True)
+    q = torch.zeros(1, 40, 1, 32)
+    with pytest.raises(ValueError, match='divisible by block size'):
+        layer(q, q, q)
+    q = torch.zeros(1, 64, 1, 32)
+    with pytest.raises(NotImplementedError):
+        layer(q, q, q, key_padding_mask=fly_amd.LengthMask(torch.tensor([64]), max_len=64))
+    with pytest.raises(ValueError, match='head dim'):
+        layer(torch.zeros(1, 64, 1, 16), q, q)
