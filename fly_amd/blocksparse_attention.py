@@ -29,6 +29,7 @@ def instantiate(cfg, *args, **kwargs):
         module = {'src.models.layers.blocksparse_linear': 'fly_amd.blocksparse_linear',
                   'src.models.layers.fastlinear': 'fly_amd.fastlinear',
                   'src.models.attention.sblocal_attention': 'fly_amd.sblocal_attention',
+                  'src.models.attention.local_attention': 'fly_amd.local_attention',
                   'src.models.attention.blocksparse_attention': 'fly_amd.blocksparse_attention',
                   'src.models.attention.sbblocksparse_attention': 'fly_amd.sbblocksparse_attention',
                   'src.models.layers.mlp': 'fly_amd.t2t_vit',

@@ -881,6 +881,146 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
     FLY_PROF(5);
 }
 
+// ---------------------------------------------------------------------------------------
+// plain local attention (no random features): softmax over the band, P V
+// ---------------------------------------------------------------------------------------
+// The band kernel without its low-rank half: per (batch, head, 64-query tile) scores^T = (t log2e) K q
+// on fp32 MFMA, band / length masks, online softmax, P V; key tiles double-buffered through LDS.
+// A query without any valid key gets a zero output row.
+struct LocalArgs {
+    const void* q; const void* k; const void* v; const int64_t* lens; void* out;
+    int B, H, T, S, lc;
+    long q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss;
+    float temp;
+};
+
+template <typename T, int E, int D>
+__global__ __launch_bounds__(NT) void local_fwd_kernel(LocalArgs a) {
+    constexpr int LDK = E + 4, LDV = D + 4, EC = E / 16, DB = D / 16, KB = TK / 16;
+    constexpr int STAGE = TK * (LDK + LDV);
+    constexpr float LOG2E = 1.4426950408889634f;
+    extern __shared__ __attribute__((aligned(128))) float smem[];
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
+    const int n_qt = (a.T + TQ - 1) / TQ;
+    const int n_items = a.B * a.H * n_qt;
+    const int per_xcd = (n_items + N_XCD - 1) / N_XCD;
+    const int item = (blockIdx.x % N_XCD) * per_xcd + blockIdx.x / N_XCD;   // see sblocal_fwd_kernel
+    if (item >= n_items) return;                       // workgroup-uniform
+    const int qt = item % n_qt, bh = item / n_qt, b = bh / a.H, h = bh % a.H;
+    const int q0 = qt * TQ, iq = q0 + 16 * w + r16;
+    const bool qvalid = iq < a.T;
+    const T* qptr = reinterpret_cast<const T*>(a.q) + b * a.q_sb + h * a.q_sh;
+    const T* kptr = reinterpret_cast<const T*>(a.k) + b * a.k_sb + h * a.k_sh;
+    const T* vptr = reinterpret_cast<const T*>(a.v) + b * a.v_sb + h * a.v_sh;
+    const int len = a.lens ? min((int)a.lens[b], a.S) : a.S;
+    const int lc_lo = a.lc / 2, lc_hi = (a.lc + 1) / 2;    // band: -lc_lo <= s - i < lc_hi
+
+    const int q_last = min(q0 + TQ - 1, a.T - 1);
+    const int lo = max(0, q0 - lc_lo), hi = min(len, q_last + lc_hi);
+    const int kt_lo = lo / TK, kt_hi = (hi > lo) ? (hi + TK - 1) / TK : kt_lo;
+    RowTile<TK, E> rk;
+    RowTile<TK, D> rv;
+    if (kt_lo < kt_hi) {
+        rk.fetch(kptr, a.k_ss, kt_lo * TK, a.S - 1, tid);
+        rv.fetch(vptr, a.v_ss, kt_lo * TK, a.S - 1, tid);
+    }
+    floatx4 qr[EC];
+#pragma unroll
+    for (int c = 0; c < EC; ++c) {
+        qr[c] = Frag<float>::zero();
+        if (qvalid) qr[c] = load4_f32(qptr + (long)iq * a.q_ss + 16 * c + 4 * g) * (a.temp * LOG2E);
+    }
+    float m_run = -1e30f;           // finite, so that the first rescale is exp2(-huge) = 0 and not inf - inf
+    float ze = 0.f;
+    floatx4 oacc[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) oacc[db] = Frag<float>::zero();
+    const int qw0 = q0 + 16 * w;
+    const int smin = max(iq - lc_lo, 0);
+    const unsigned span = qvalid ? (unsigned)max(min(iq + lc_hi, len) - smin, 0) : 0u;
+    if (kt_lo < kt_hi) {
+        rk.template stash<LDK>(smem, tid);
+        rv.template stash<LDV>(smem + TK * LDK, tid);
+    }
+    __syncthreads();
+    for (int kt = kt_lo; kt < kt_hi; ++kt) {
+        const int s_base = kt * TK, cur = (kt - kt_lo) & 1;
+        const float* Ks = smem + cur * STAGE;
+        const float* Vs = Ks + TK * LDK;
+        const bool more = kt + 1 < kt_hi;
+        if (more) {
+            rk.fetch(kptr, a.k_ss, s_base + TK, a.S - 1, tid);
+            rv.fetch(vptr, a.v_ss, s_base + TK, a.S - 1, tid);
+        }
+        const bool any = !(s_base + TK - 1 - qw0 < -lc_lo || s_base - (qw0 + 15) >= lc_hi || s_base >= len);
+        if (any) {
+            floatx4 s1[KB];
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) s1[kb] = Frag<float>::zero();
+#pragma unroll
+            for (int c = 0; c < EC; ++c) {
+                floatx4 ka[KB];
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb)
+                    ka[kb] = *reinterpret_cast<const floatx4*>(Ks + (16 * kb + r16) * LDK + 4 * g + 16 * c);
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int kb = 0; kb < KB; ++kb)
+                        s1[kb] = __builtin_amdgcn_mfma_f32_16x16x4f32(ka[kb][j], qr[c][j], s1[kb], 0, 0, 0);
+            }
+            bool ok[KB][4];
+            float mx = -INFINITY;
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int s = s_base + 16 * kb + 4 * g + i;
+                    ok[kb][i] = (unsigned)(s - smin) < span;
+                    mx = fmaxf(mx, ok[kb][i] ? s1[kb][i] : -INFINITY);
+                }
+            mx = group_max(mx);
+            if (__builtin_amdgcn_ballot_w64(mx > m_run) != 0) {
+                const float m_new = fmaxf(m_run, mx);
+                const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+                m_run = m_new;
+                ze *= alpha;
+#pragma unroll
+                for (int db = 0; db < DB; ++db) oacc[db] *= alpha;
+            }
+            floatx4 p[KB];
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    p[kb][i] = ok[kb][i] ? __builtin_amdgcn_exp2f(s1[kb][i] - m_run) : 0.f;
+                    ze += p[kb][i];
+                }
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int db = 0; db < DB; ++db)
+                        oacc[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(
+                            Vs[(16 * kb + 4 * g + i) * LDV + 16 * db + r16], p[kb][i], oacc[db], 0, 0, 0);
+        }
+        if (more) {
+            float* nxt = smem + (cur ^ 1) * STAGE;
+            rk.template stash<LDK>(nxt, tid);
+            rv.template stash<LDV>(nxt + TK * LDK, tid);
+        }
+        __syncthreads();
+    }
+    ze = group_sum(ze);
+    if (qvalid) {
+        const float inv = ze > 0.f ? 1.0f / ze : 0.f;
+        T* optr = reinterpret_cast<T*>(a.out) + b * a.o_sb + h * a.o_sh + (long)iq * a.o_ss;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) store4_f32(optr + 16 * db + 4 * g, oacc[db] * inv);
+    }
+}
+
 // Merge of the per-part partials of one query tile by the 256 threads of a workgroup: thread
 // (query ql = tid / 4, column quarter tid % 4).  Parts are taken in batches whose loads are all
 // issued before the first is used (slots past n_parts re-read the last part and are ignored),
@@ -1350,6 +1490,24 @@ static int launch_fwd(const FwdArgs& a, hipStream_t st) {
     return a.n_parts > 1 ? launch_fwd_impl<T, E, M, true>(a, st) : launch_fwd_impl<T, E, M, false>(a, st);
 }
 
+template <typename T, int E>
+static int launch_local(const LocalArgs& a, hipStream_t st) {
+    auto kern = local_fwd_kernel<T, E, E>;
+    constexpr size_t smem = sizeof(float) * 2 * TK * 2 * (E + 4);
+    static bool lds_ready = false;
+    if (!lds_ready) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return fail(ERR_LAUNCH, "local_fwd: LDS attribute: %s", hipGetErrorString(e));
+        lds_ready = true;
+    }
+    const long items = (long)a.B * a.H * ((a.T + TQ - 1) / TQ);
+    const long grid = (items + N_XCD - 1) / N_XCD * N_XCD;
+    if (grid > 2147483647L) return fail(ERR_ARG, "local_fwd: too many workgroups");
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NT), smem, st, a);
+    return check_launch("local_fwd_kernel");
+}
+
 #define SB_DISPATCH_M(FN, T, EE, ARGS)                                       \
     switch (m) {                                                              \
         case 32: return FN<T, EE, 32>(ARGS, st);                              \
@@ -1510,4 +1668,34 @@ extern "C" int flyhip_sblocal_fwd(const void* q, const void* k, const void* v, c
               B, H, T, S, mh_valid, local_context, nc, n_parts,
               q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss, softmax_temp};
     return dispatch_fwd(dtype, E, 2 * mh, a, reinterpret_cast<hipStream_t>(stream));
+}
+
+extern "C" int flyhip_local_fwd(const void* q, const void* k, const void* v, const int64_t* key_lengths, void* out,
+                                int B, int H, int T, int S, int E, int D, int local_context,
+                                int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                                int64_t k_sb, int64_t k_sh, int64_t k_ss,
+                                int64_t v_sb, int64_t v_sh, int64_t v_ss,
+                                int64_t o_sb, int64_t o_sh, int64_t o_ss,
+                                float softmax_temp, int dtype, void* stream) {
+    FLY_REQUIRE(q && k && v && out, "local_fwd: null pointer");
+    FLY_REQUIRE(B > 0 && H > 0 && T > 0 && S > 0, "local_fwd: empty problem");
+    FLY_REQUIRE(local_context >= 1, "local_fwd: local_context must be >= 1");
+    FLY_REQUIRE(softmax_temp > 0.f, "local_fwd: softmax_temp must be positive");
+    FLY_REQUIRE(E == D, "local_fwd: padded head dims must be equal (E=%d, D=%d)", E, D);
+    FLY_REQUIRE(((q_sb | q_sh | q_ss | k_sb | k_sh | k_ss | v_sb | v_sh | v_ss | o_sb | o_sh | o_ss) % 4) == 0,
+                "local_fwd: strides must be multiples of 4 elements (16-byte vector access)");
+    LocalArgs a{q, k, v, key_lengths, out, B, H, T, S, local_context,
+                q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss, softmax_temp};
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+#define LOCAL_DISPATCH(TT)                                                                          \
+    switch (E) {                                                                                    \
+        case 32: return launch_local<TT, 32>(a, st);                                                \
+        case 64: return launch_local<TT, 64>(a, st);                                                \
+        case 128: return launch_local<TT, 128>(a, st);                                              \
+        default: return fail(ERR_UNSUPPORTED, "local_fwd: head dim E=%d not in {32,64,128}", E);     \
+    }
+    if (dtype == F32) { LOCAL_DISPATCH(float) }
+    if (dtype == BF16) { LOCAL_DISPATCH(bf16_t) }
+#undef LOCAL_DISPATCH
+    return fail(ERR_UNSUPPORTED, "local_fwd supports float32 and bfloat16, got dtype code %d", dtype);
 }

@@ -1,0 +1,76 @@
+"""Plain local (banded) softmax attention on the HIP kernel: drop-in for ``LocalAttention``
+(src/models/attention/local_attention.py:12-108)."""
+import math
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import _lib
+from .sblocal_attention import _HEAD_DIMS, _round_up_choice, _vector_ready
+
+
+def local_forward(query, key, value, local_context, softmax_temp=None, key_lengths=None):
+    """query (B,T,H,E), key (B,S,H,E), value (B,S,H,D) float32 or bfloat16 GPU tensors ->
+    out (B,T,H,D): query i attends to keys j with -(local_context // 2) <= j - i < (local_context + 1) // 2
+    and j < key_lengths[b] (local_attention.py:68-92 for attn_mask=None, no dropout)."""
+    _lib.require_gpu(query, key, value, key_lengths)
+    if query.dtype not in (torch.float32, torch.bfloat16):
+        raise NotImplementedError(f'the local attention kernel supports float32 and bfloat16, got {query.dtype}')
+    if key.dtype != query.dtype or value.dtype != query.dtype:
+        raise ValueError('query, key and value must share a dtype')
+    B, T, H, E = query.shape
+    Bk, S, Hk, Ek = key.shape
+    Bv, Sv, Hv, D = value.shape
+    if (Bk, Hk, Ek) != (B, H, E) or (Bv, Sv, Hv) != (B, S, H):
+        raise ValueError(f'inconsistent shapes q{tuple(query.shape)} k{tuple(key.shape)} v{tuple(value.shape)}')
+    if local_context < 1:
+        raise ValueError('local_context must be >= 1')
+    t = softmax_temp or 1 / math.sqrt(E)
+    dim = _round_up_choice(max(E, D), _HEAD_DIMS, 'head dimension')
+
+    def prep(x):
+        if x.shape[-1] != dim:
+            x = F.pad(x, (0, dim - x.shape[-1]))      # zero columns change no dot product
+        return x if _vector_ready(x) else x.contiguous()
+    q, k, v = prep(query), prep(key), prep(value)
+    lens = None
+    if key_lengths is not None:
+        lens = key_lengths.to(device=query.device, dtype=torch.int64).contiguous()
+        if lens.shape != (B,):
+            raise ValueError(f'key_lengths must have shape ({B},)')
+    out = torch.empty(B, T, H, dim, dtype=query.dtype, device=query.device)
+    with torch.cuda.device(query.device):
+        _lib.call('flyhip_local_fwd', q.data_ptr(), k.data_ptr(), v.data_ptr(), _lib.ptr(lens), out.data_ptr(),
+                  B, H, T, S, dim, dim, local_context,
+                  q.stride(0), q.stride(2), q.stride(1), k.stride(0), k.stride(2), k.stride(1),
+                  v.stride(0), v.stride(2), v.stride(1), out.stride(0), out.stride(2), out.stride(1),
+                  t, _lib.dtype_code(q), _lib.stream_ptr(query.device))
+    return out[..., :D]
+
+
+class LocalAttention(nn.Module):
+    """Softmax attention in which query i only sees keys j with
+    -(local_context // 2) <= j - i < (local_context + 1) // 2.  Same constructor and forward signature
+    as the reference class.  Covered on the GPU: no attn_mask, optional length-style key_padding_mask,
+    dropout inactive, need_weights=False; anything else raises NotImplementedError."""
+
+    def __init__(self, local_context, softmax_temp=None, attention_dropout=0.0, device=None, dtype=None):
+        super().__init__()
+        self.local_context = local_context
+        self.softmax_temp = softmax_temp
+        self.dropout = nn.Dropout(attention_dropout)
+
+    def forward(self, query, key, value, attn_mask=None, key_padding_mask=None, need_weights=False):
+        if attn_mask is not None and not bool(attn_mask.all_ones):
+            raise NotImplementedError('attn_mask other than all-ones is not supported by the fused kernel')
+        if need_weights:
+            raise NotImplementedError('need_weights=True would materialise the (T,S) matrix; not supported')
+        if self.training and self.dropout.p > 0.0:
+            raise NotImplementedError('attention dropout is not implemented in the fused kernel')
+        lengths = None
+        if key_padding_mask is not None and not bool(key_padding_mask.all_ones):
+            lengths = key_padding_mask.lengths
+        out = local_forward(query, key, value, self.local_context, softmax_temp=self.softmax_temp,
+                            key_lengths=lengths)
+        return out, None

@@ -91,6 +91,19 @@ int flyhip_sblocal_fwd(const void* q, const void* k, const void* v, const float*
                        int64_t o_sb, int64_t o_sh, int64_t o_ss,
                        float softmax_temp, int dtype, void* stream);
 
+/* Plain local attention, no random features (ref: src/models/attention/local_attention.py:68-92;
+ * fast_transformers.local_product): out[i] = softmax over the band -(lc/2) <= s - i < (lc+1)/2, s below
+ * the key length, of t q_i.k_s, times v.  q (B,T,H,E), k (B,S,H,E), v (B,S,H,D), out (B,T,H,D) via
+ * (batch, head, seq) strides, innermost contiguous; E = D in {32,64,128}; key_lengths (B) int64 or
+ * NULL.  A query with no valid key gets a zero row (local_attention.py:74-84). */
+int flyhip_local_fwd(const void* q, const void* k, const void* v, const int64_t* key_lengths, void* out,
+                     int B, int H, int T, int S, int E, int D, int local_context,
+                     int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                     int64_t k_sb, int64_t k_sh, int64_t k_ss,
+                     int64_t v_sb, int64_t v_sh, int64_t v_ss,
+                     int64_t o_sb, int64_t o_sh, int64_t o_ss,
+                     float softmax_temp, int dtype, void* stream);
+
 /* Measurement hook (no counterpart in the reference): the two caller-owned hipEvent_t are recorded
  * on the launch stream immediately before and after the fused band kernel of the NEXT
  * flyhip_sblocal_fwd call of the calling thread, then forgotten.  Pass NULLs to clear. */

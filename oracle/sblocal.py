@@ -230,3 +230,25 @@ def dense_closed_form(query, key, value, projection_matrix, local_context, softm
     Z = A.sum(-1, keepdim=True)
     out = (A @ v) / Z
     return out.permute(0, 2, 1, 3), torch.log(Z), A
+
+
+def local_attention(query, key, value, local_context, softmax_temp=None, key_lengths=None):
+    """LocalAttention.forward for attn_mask=None, no dropout (local_attention.py:50-92): band-packed
+    scores from local_dot_product, softmax over the packed axis, rows without a valid key zeroed when
+    a key padding mask is given, local_weighted_average.  query (B,T,H,E) -> out (B,T,H,D)."""
+    B, T, H, E = query.shape
+    S = key.shape[1]
+    t = softmax_temp or 1 / math.sqrt(E)
+    q = query.permute(0, 2, 1, 3)
+    k = key.permute(0, 2, 1, 3)
+    v = value.permute(0, 2, 1, 3)
+    lengths = torch.full((B,), S, dtype=torch.long) if key_lengths is None else key_lengths
+    QK = local_dot_product(q, k, torch.zeros(T, S, dtype=q.dtype), lengths, local_context)     # :68-74
+    attn = torch.softmax(t * QK, dim=-1)                                                       # :75
+    if key_lengths is not None:                                                                # :82-88
+        i = torch.arange(T).view(1, 1, T, 1)
+        j = torch.arange(local_context)
+        idx = i - local_context // 2 + j
+        valid = (idx >= 0) & (idx < lengths.view(B, 1, 1, 1))
+        attn = attn.masked_fill(~valid, 0.0)
+    return local_weighted_average(attn, v).permute(0, 2, 1, 3)                                 # :91

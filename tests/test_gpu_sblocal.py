@@ -139,3 +139,32 @@ def test_module_dropin():
     assert rel_err(attn.last_log_normalization, ref_ln) <= 1e-4
     with pytest.raises(NotImplementedError):
         attn(q.to(dev), k.to(dev), v.to(dev), need_weights=True)
+
+
+@pytest.mark.parametrize('case', [
+    dict(B=2, T=300, S=300, H=2, E=64, D=64, lc=64, lens=None, dtype=torch.float32),
+    dict(B=2, T=130, S=257, H=1, E=21, D=17, lc=33, lens=[257, 100], dtype=torch.float32),
+    dict(B=1, T=200, S=70, H=2, E=128, D=128, lc=40, lens=[50], dtype=torch.float32),
+    dict(B=2, T=256, S=256, H=4, E=64, D=64, lc=128, lens=None, dtype=torch.bfloat16),
+], ids=['square', 'odd-sizes-lengths', 'rows-without-keys', 'bf16'])
+def test_local_attention_matches_oracle(case):
+    """LocalAttention (local_attention.py:50-92) through flyhip_local_fwd against the oracle."""
+    from fly_amd import LocalAttention, LengthMask
+    c = dict(case)
+    dtype, lens = c.pop('dtype'), c.pop('lens')
+    print('case', c, dtype, flush=True)
+    g = torch.Generator().manual_seed(31)
+    q = (torch.randn(c['B'], c['T'], c['H'], c['E'], generator=g)).to(dtype)
+    k = (torch.randn(c['B'], c['S'], c['H'], c['E'], generator=g)).to(dtype)
+    v = torch.randn(c['B'], c['S'], c['H'], c['D'], generator=g).to(dtype)
+    kl = None if lens is None else torch.tensor(lens)
+    dev = torch.device('cuda:0')
+    layer = LocalAttention(c['lc'])
+    mask = None if kl is None else LengthMask(kl.to(dev), max_len=c['S'])
+    out, attn = layer(q.to(dev), k.to(dev), v.to(dev), key_padding_mask=mask)
+    assert attn is None and out.shape == (c['B'], c['T'], c['H'], c['D']) and out.dtype == dtype
+    ref = osb.local_attention(q.double(), k.double(), v.double(), c['lc'], key_lengths=kl)
+    assert rel_err(out, ref) <= (1e-4 if dtype == torch.float32 else 2e-2)
+    if case['S'] == 70:       # 50 valid keys, 20 each side: queries from 70 on see no key and give zero rows
+        assert float(ref[:, 70:].abs().max()) == 0.0 and float(out[:, 70:].abs().max()) == 0.0
+        assert float(out[:, 69].abs().max()) > 0.0

@@ -164,3 +164,26 @@ def test_float32_oracle_is_close_to_float64():
     o32, l32 = osb.sblocal_attention(q.float(), k.float(), v.float(), P.float(), 128)
     assert float((o32.double() - o64).abs().max() / o64.abs().max()) < 1e-5
     assert float((l32.double() - l64).abs().max() / l64.abs().max()) < 1e-5
+
+
+def test_local_attention_equals_dense_masked_softmax():
+    """LocalAttention restated from the band-packed op sequence against a dense softmax over the same
+    support (a different route: -inf mask on the full (T,S) matrix), with key lengths and T != S."""
+    g = torch.Generator().manual_seed(8)
+    for (B, T, S, H, E, D, lc, lens) in [(2, 40, 40, 2, 8, 5, 7, None), (2, 33, 50, 1, 4, 6, 12, [50, 21]),
+                                         (1, 50, 20, 2, 4, 4, 9, [13])]:
+        q = torch.randn(B, T, H, E, generator=g, dtype=torch.float64)
+        k = torch.randn(B, S, H, E, generator=g, dtype=torch.float64)
+        v = torch.randn(B, S, H, D, generator=g, dtype=torch.float64)
+        kl = None if lens is None else torch.tensor(lens)
+        out = osb.local_attention(q, k, v, lc, softmax_temp=0.4, key_lengths=kl)
+        i = torch.arange(T).view(T, 1)
+        j = torch.arange(S).view(1, S)
+        band = ((j - i) >= -(lc // 2)) & ((j - i) < (lc + 1) // 2)
+        limit = torch.full((B,), S) if kl is None else kl
+        ok = band.view(1, 1, T, S) & (j.view(1, 1, 1, S) < limit.view(B, 1, 1, 1))
+        s = 0.4 * torch.einsum('bthe,bshe->bhts', q, k)
+        w = torch.softmax(s.masked_fill(~ok, float('-inf')), dim=-1)
+        w = torch.where(ok.any(-1, keepdim=True), w, torch.zeros_like(w))      # rows without a valid key
+        ref = torch.einsum('bhts,bshd->bthd', w, v)
+        assert (out - ref).abs().max() < 1e-12
