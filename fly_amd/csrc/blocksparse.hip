@@ -588,6 +588,8 @@ __global__ __launch_bounds__(256) void bs_dds_kernel(DxdArgs a) {
 // per input block the 128 x 32 activation tile and the group's 32g x 32 weight tile are staged in
 // LDS (registers hold the next step's tiles while the MFMAs of the current one run), the 2 x 2
 // waves own 64 x 64 outputs each and form them with 16x16x32 MFMAs.
+typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
+
 struct DdsGroupArgs {
     const void* sp; const void* dn; void* c;
     const int32_t* seg_ptr; const int32_t* seg_blk; const int32_t* seg_inner;
@@ -630,8 +632,9 @@ __global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
     const int n_steps = (nin + KB - 1) / KB;
     // two register sets: the loads of step s+2 are issued while step s computes and are parked in LDS
     // one iteration later, so every global load has two steps to arrive
-    uint4 rxa[KB][2], rwa[KB][2], rxb[KB][2], rwb[KB][2];
-    auto fetch = [&](int step, uint4 (&rx)[KB][2], uint4 (&rw)[KB][2]) {
+    // (native vectors: arrays of the uint4 struct passed by reference do not stay in registers)
+    uintx4 rxa[KB][2], rwa[KB][2], rxb[KB][2], rwb[KB][2];
+    auto fetch = [&](int step, uintx4 (&rx)[KB][2], uintx4 (&rw)[KB][2]) __attribute__((always_inline)) {
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb) {
             const int t = step * KB + kb;
@@ -640,22 +643,22 @@ __global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
 #pragma unroll
             for (int hh = 0; hh < 2; ++hh) {
                 const long m = min(m0 + srow + 64 * hh, (long)a.M - 1);        // clamped: masked at the store
-                rx[kb][hh] = *reinterpret_cast<const uint4*>(xp + m * a.dn_sm + kcol);
+                rx[kb][hh] = *reinterpret_cast<const uintx4*>(xp + m * a.dn_sm + kcol);
                 const int orow = srow + 64 * hh;                                 // output row inside the group
                 const int blk_id = live ? s_blk[orow >> 5][t] : -1;
-                rw[kb][hh] = make_uint4(0, 0, 0, 0);
+                rw[kb][hh] = uintx4{0, 0, 0, 0};
                 if (blk_id >= 0)
-                    rw[kb][hh] = *reinterpret_cast<const uint4*>(spz + (long)blk_id * 1024 + (orow & 31) * 32 + schunk);
+                    rw[kb][hh] = *reinterpret_cast<const uintx4*>(spz + (long)blk_id * 1024 + (orow & 31) * 32 + schunk);
             }
         }
     };
-    auto stash = [&](int buf, const uint4 (&rx)[KB][2], const uint4 (&rw)[KB][2]) {
+    auto stash = [&](int buf, const uintx4 (&rx)[KB][2], const uintx4 (&rw)[KB][2]) __attribute__((always_inline)) {
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
             for (int hh = 0; hh < 2; ++hh) {
-                *reinterpret_cast<uint4*>(&xs[buf][(srow + 64 * hh) * LD + 32 * kb + schunk]) = rx[kb][hh];
-                *reinterpret_cast<uint4*>(&ws[buf][(srow + 64 * hh) * LD + 32 * kb + schunk]) = rw[kb][hh];
+                *reinterpret_cast<uintx4*>(&xs[buf][(srow + 64 * hh) * LD + 32 * kb + schunk]) = rx[kb][hh];
+                *reinterpret_cast<uintx4*>(&ws[buf][(srow + 64 * hh) * LD + 32 * kb + schunk]) = rw[kb][hh];
             }
     };
 
@@ -666,7 +669,7 @@ __global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
         for (int tn = 0; tn < 4; ++tn) acc[tm][tn] = Frag<float>::zero();
     const bool wave_active = 2 * wn < gn;                   // its output blocks exist in this group
 
-    auto compute = [&](int cur) {
+    auto compute = [&](int cur) __attribute__((always_inline)) {
         if (wave_active) {
 #pragma unroll
             for (int kb = 0; kb < KB; ++kb) {
