@@ -8,7 +8,7 @@ blocksparse_sum.py:156-179.
 import torch
 
 from . import _lib
-from .blocksparse_utils import _as_layout3, row_table
+from .blocksparse_utils import _as_layout3, row_table, sparsify_broadcast_tensor
 
 
 class _RowOp:
@@ -65,13 +65,51 @@ class softmax(_RowOp):
                                              'key_padding_mask', x.device)
         am, am_stride, am_mul = _mask_arg(attn_mask, attn_mask_mode, p * self.block, r * self.block,
                                           'attn_mask', x.device)
+        return _SoftmaxFn.apply(x, self, float(scale), (kpm, kpm_stride, kpm_mul), (am, am_stride, am_mul))
+
+    def _launch(self, x, scale, kpm_args, am_args):
+        H, p, r = self.spdims
+        kpm, kpm_stride, kpm_mul = kpm_args
+        am, am_stride, am_mul = am_args
         ptr, blk, col, max_nnz = self.make_lut(x.device)
         with torch.cuda.device(x.device):
             _lib.call('flyhip_bs_softmax', x.data_ptr(), ptr.data_ptr(), blk.data_ptr(), col.data_ptr(),
-                      H * p, p, max_nnz, Z, self.block, x.stride(0), float(scale),
+                      H * p, p, max_nnz, x.shape[0], self.block, x.stride(0), scale,
                       _lib.ptr(kpm), kpm_stride, kpm_mul, _lib.ptr(am), am_stride, am_mul,
                       _lib.dtype_code(x), _lib.stream_ptr(x.device))
+
+
+class _SoftmaxFn(torch.autograd.Function):
+    """In-place block softmax y = softmax(scale * x + masks); backward dx = scale * y * (dy - rowsum(dy * y))
+    with the row sums on the row-reduction kernel (the kernel it replaces differentiates the same way)."""
+
+    @staticmethod
+    def forward(ctx, x, op, scale, kpm_args, am_args):
+        op._launch(x, scale, kpm_args, am_args)
+        ctx.mark_dirty(x)
+        ctx.save_for_backward(x)
+        ctx.op, ctx.scale = op, scale
         return x
+
+    @staticmethod
+    def backward(ctx, dy):
+        (y,) = ctx.saved_tensors
+        op = ctx.op
+        dyy = (dy * y).contiguous()
+        rows = _reduce_rows(op, dyy, 1)                                   # (Z, H, M)
+        dx = (dyy - y * sparsify_broadcast_tensor(rows, op.layout, op.block)) * ctx.scale
+        return dx, None, None, None, None
+
+
+def _reduce_rows(op, x, op_code):
+    H, p, r = op.spdims
+    Z = x.shape[0]
+    ptr, blk, col, _ = op.make_lut(x.device)
+    out = torch.empty((Z, H, p * op.block), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        _lib.call('flyhip_bs_rowreduce', x.data_ptr(), out.data_ptr(), ptr.data_ptr(), blk.data_ptr(),
+                  H * p, Z, op.block, x.stride(0), op_code, _lib.dtype_code(x), _lib.stream_ptr(x.device))
+    return out
 
 
 class _Reduce(_RowOp):
@@ -79,16 +117,28 @@ class _Reduce(_RowOp):
 
     def __call__(self, x):
         self._check(x)
-        x = x.contiguous()
-        H, p, r = self.spdims
-        Z = x.shape[0]
-        ptr, blk, col, _ = self.make_lut(x.device)
-        out = torch.empty((Z, H, p * self.block), dtype=x.dtype, device=x.device)
-        with torch.cuda.device(x.device):
-            _lib.call('flyhip_bs_rowreduce', x.data_ptr(), out.data_ptr(), ptr.data_ptr(), blk.data_ptr(),
-                      H * p, Z, self.block, x.stride(0), self.op_code, _lib.dtype_code(x),
-                      _lib.stream_ptr(x.device))
+        return _ReduceFn.apply(x.contiguous(), self)
+
+
+class _ReduceFn(torch.autograd.Function):
+    """Row logsumexp / sum with their gradients (blocksparse_logsumexp.py:63-102, blocksparse_sum.py):
+    d logsumexp = exp(x - lse[row]) * dout[row], d sum = dout[row], on the nonzero blocks."""
+
+    @staticmethod
+    def forward(ctx, x, op):
+        out = _reduce_rows(op, x, op.op_code)
+        ctx.save_for_backward(x, out)
+        ctx.op = op
         return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        x, out = ctx.saved_tensors
+        op = ctx.op
+        d_rows = sparsify_broadcast_tensor(dout.contiguous(), op.layout, op.block)
+        if op.op_code == 1:
+            return d_rows.expand_as(x).contiguous(), None
+        return torch.exp(x - sparsify_broadcast_tensor(out, op.layout, op.block)) * d_rows, None
 
 
 class logsumexp(_Reduce):

@@ -172,3 +172,42 @@ def test_matmul_backward_matches_dense_autograd():
     x2, w2 = x.detach().clone().requires_grad_(), wsp.detach().clone().requires_grad_()
     ((x2 @ densify_tensor(w2, layout[:1]).transpose(-1, -2)) * w).sum().backward()
     assert rel_err(x.grad, x2.grad) <= 1e-5 and rel_err(wsp.grad, w2.grad) <= 1e-5
+
+
+def test_row_ops_backward_match_dense_autograd():
+    """Gradients of the block softmax (with scale and an additive key-padding mask), logsumexp and row sum
+    against autograd through the dense formulas on -inf / zero filled matrices
+    (the reference's own checks: tests/models/attention/test_blocksparse_logsumexp.py:25-33)."""
+    from fly_amd import softmax, logsumexp, blocksparse_sum
+    from fly_amd.blocksparse_utils import densify_tensor, sparsify_tensor
+    g = torch.Generator().manual_seed(3)
+    block, Z, H, p, r = 16, 2, 2, 3, 4
+    layout = (torch.rand(H, p, r, generator=g) < 0.6).long()
+    layout[:, :, 0] = 1                                   # no empty block-row: every row has a finite entry
+    nnz = int(layout.sum())
+    x0 = torch.randn(Z, nnz, block, block, generator=g).to(DEV)
+    w = torch.randn(Z, nnz, block, block, generator=g).to(DEV)
+    kpm = torch.zeros(Z, r * block)
+    kpm[1, -5:] = float('-inf')
+    for name in ('softmax', 'logsumexp', 'sum'):
+        print('case', name, flush=True)
+        x = x0.clone().requires_grad_()
+        xd = x0.clone().requires_grad_()
+        if name == 'softmax':
+            y = softmax(layout, block)(x * 1.0, scale=0.7, key_padding_mask=kpm.to(DEV))
+            dense = densify_tensor(xd * 0.7, layout, float('-inf')) + kpm.to(DEV)[:, None, None, :]
+            ref = sparsify_tensor(torch.softmax(dense, dim=-1), layout)
+            (y * w).sum().backward()
+            (ref * w).sum().backward()
+        else:
+            op = logsumexp(layout, block) if name == 'logsumexp' else blocksparse_sum(layout, block)
+            y = op(x)
+            wr = torch.randn(y.shape, generator=g).to(DEV)
+            if name == 'logsumexp':
+                ref = torch.logsumexp(densify_tensor(xd, layout, float('-inf')), dim=-1)
+            else:
+                ref = densify_tensor(xd, layout, 0.0).sum(-1)
+            (y * wr).sum().backward()
+            (ref * wr).sum().backward()
+        assert rel_err(y, ref) <= 1e-5
+        assert rel_err(x.grad, xd.grad) <= 1e-5, name
