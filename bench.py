@@ -7,7 +7,8 @@ One "step" is one forward of BASELINE config 1 (fp32, B=2, H=1, L=3136, d=64, ba
 HBM.  Prints ONE JSON line: tokens/s for the whole forward, the roofline of the dominant kernel
 (the fused band kernel, timed with events on its stream inside the timed region), the CPU oracle
 timed on this box's host cores, and -- as `extra` -- the block-sparse SDD / softmax / DSD stages
-of BASELINE config 2 (bf16, B=8, H=12, L=4096, d=64, block 32).
+of BASELINE config 2 (bf16, B=8, H=12, L=4096, d=64, block 32) and whole-forward timings of
+configs 3, 4 and 5.
 """
 import argparse
 import json
@@ -173,12 +174,83 @@ def bench_blocksparse(steps, warmup):
     return out
 
 
+def bench_other_configs():
+    """Timings of the remaining BASELINE configs (stream events around whole forwards):
+    3 = the two Scatterbrain-local layers of T2T-ViT-t-14 at batch 64 (fp32), 4 = the two Pixelfly
+    block-sparse linears of the Mixer-B channel MLP (bf16), 5 = long-sequence Scatterbrain-local (bf16)."""
+    import fly_amd
+    from fly_amd.sblocal_attention import SBLocalPlan
+    from oracle import sblocal as osb
+    dev = torch.device('cuda:0')
+    g = torch.Generator().manual_seed(0)
+    out = {}
+
+    def timeit(fn, n=10, w=2):
+        for _ in range(w):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n
+
+    for L, dim in ((3136, 147), (784, 576)):
+        B, H, E, mh, lc = 64, 1, 64, 64, 256
+        q, k, v = (torch.randn(B, L, H, E, generator=g).to(dev) for _ in range(3))
+        P = osb.gaussian_orthogonal_random_matrix(mh, E, generator=g).to(dev)
+        plan = SBLocalPlan(B, H, L, L, E, mh, mh, torch.float32, dev, lc)
+        o = torch.empty(B, L, H, E, device=dev)
+        ln = torch.empty(B, H, L, device=dev)
+        ms = timeit(lambda: plan.run(q, k, v, P, None, lc, dim ** -0.5, o, ln))
+        fl, _ = sblocal_flops(B, H, L, L, E, E, 2 * mh, lc)
+        out[f'config3_sblocal_fp32_B64_L{L}'] = {'ms': ms, 'tflops': fl / ms / 1e9, 'tokens_per_s': B * L / ms * 1e3,
+                                                 'mfma_fp32_frac': fl / ms / 1e9 / PEAK_FP32_MFMA_TFLOPS}
+        del q, k, v, o, ln, plan
+
+    cfg = fly_amd.FlatBlockButterflySparsityConfig(8, 2, block=32)
+    torch.manual_seed(0)
+    fc1 = fly_amd.BlockSparseLinear(768, 3072, cfg, bias=False).to(dev).to(torch.bfloat16)
+    fc2 = fly_amd.BlockSparseLinear(3072, 768, cfg, bias=False).to(dev).to(torch.bfloat16)
+    x = torch.randn(256 * 196, 768, generator=g).bfloat16().to(dev)
+    h = torch.randn(256 * 196, 3072, generator=g).bfloat16().to(dev)
+    w = torch.randn(3072, 768, generator=g).bfloat16().to(dev)
+    with torch.no_grad():
+        ms1, ms2 = timeit(lambda: fc1(x)), timeit(lambda: fc2(h))
+        msd = timeit(lambda: torch.nn.functional.linear(x, w))
+    fl = 2 * 50176 * 864 * 1024
+    out['config4_pixelfly_linear_bf16'] = {
+        'fc1_ms': ms1, 'fc1_tflops': fl / ms1 / 1e9, 'fc2_ms': ms2, 'fc2_tflops': fl / ms2 / 1e9,
+        'fc1_hbm_gbs': (x.numel() + 50176 * 3072 + 864 * 1024) * 2 / ms1 / 1e6,
+        'dense_library_gemm_768_3072_ms': msd}
+    del x, h, w, fc1, fc2
+
+    B, L, H, E, mh, lc = 1, 16384, 16, 64, 128, 1024
+    q, k, v = (torch.randn(B, L, H, E, generator=g) for _ in range(3))
+    idx = torch.randperm(L, generator=g)[: L // 20]
+    k[:, idx] *= 8
+    q, k, v = (x.bfloat16().to(dev) for x in (q, k, v))
+    P = osb.gaussian_orthogonal_random_matrix(mh, E, generator=g).to(dev)
+    plan = SBLocalPlan(B, H, L, L, E, mh, mh, torch.bfloat16, dev, lc)
+    o = torch.empty(B, L, H, E, device=dev, dtype=torch.bfloat16)
+    ln = torch.empty(B, H, L, device=dev)
+    ms = timeit(lambda: plan.run(q, k, v, P, None, lc, 0.125, o, ln))
+    msk = timeit(lambda: plan.run_keys(q, k, v, P, None, 0.125))
+    fl, _ = sblocal_flops(B, H, L, L, E, E, 2 * mh, lc)
+    out['config5_sblocal_bf16_L16384'] = {'ms': ms, 'key_pass_ms': msk, 'tflops': fl / ms / 1e9,
+                                          'tokens_per_s': B * L / ms * 1e3, 'mfma_bf16_frac': fl / ms / 1e9 / 2500.0}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=200)
     ap.add_argument('--warmup', type=int, default=20)
     ap.add_argument('--no-blocksparse', action='store_true', help='skip the config 2 stages')
+    ap.add_argument('--no-other-configs', action='store_true', help='skip the timings of configs 3, 4, 5')
     ap.add_argument('--skip-cpu', action='store_true', help='skip the CPU baseline leg (profiling runs)')
     ap.add_argument('--copy-calibration', action='store_true',
                     help='also run a plain 256 MiB device copy: its FETCH_SIZE / WRITE_SIZE readings '
@@ -209,8 +281,13 @@ def main():
         'gpu_over_cpu': sb['tokens_per_s'] / sb['cpu_baseline']['value'] if sb['cpu_baseline'] else None,
         'parity': sb['parity'],
     }
+    extra = {}
     if not args.no_blocksparse:
-        line['extra'] = {'blocksparse_config2': bench_blocksparse(max(5, args.steps // 10), 3)}
+        extra['blocksparse_config2'] = bench_blocksparse(max(5, args.steps // 10), 3)
+    if not args.no_other_configs:
+        extra.update(bench_other_configs())
+    if extra:
+        line['extra'] = extra
     print(json.dumps(line))
 
 
