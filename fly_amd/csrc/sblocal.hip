@@ -882,6 +882,260 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
 }
 
 // ---------------------------------------------------------------------------------------
+// key pass for bfloat16 inputs (key role only; used when no query features are asked for)
+// ---------------------------------------------------------------------------------------
+// The same outputs as the key role of sb_kfeat_kernel, with both contractions on the bf16 MFMA:
+//   projection : S[key][feature] = K . (sqrt(t) log2e P)^T with K as it is in memory (bf16) and the
+//                projection split into a bf16 head and remainder.  Rows = keys: a lane owns ONE
+//                feature and receives keys 4g+i of every 16-key block -- which is the operand
+//                layout (lane = feature, k-slots = keys) the second product needs, so the
+//                features go from registers straight into it.
+//   K'^T V     : KV[feature][d] = sum_keys F[key][feature] V[key][d] with V transposed through LDS
+//                to [d][key slot]; the same LDS tile is what the band kernel wants in HBM (vt).
+// Wave w owns the projection rows of blocks w, w+4, ... (both signs of each), for all 64 keys of
+// the chunk.  The feature scratch for the band kernel ([key][k-slot order]) is assembled in LDS
+// from 2-byte writes and leaves as 16-byte stores.
+template <int E, int D, int M>
+__global__ __launch_bounds__(NT) void sb_kfeat_bf16_kernel(KvArgs a) {
+    constexpr int MH = M / 2, FB = MH / 16, DB = D / 16, KS = E / 32, KBN = CH / 16;
+    constexpr int FPW = (FB + 3) / 4;                       // projection-row blocks per wave
+    constexpr int LDK = E + 8, LDVT = CH + 8, LDFO = M + 8; // LDS row strides in 2-byte elements
+    constexpr float LOG2E = 1.4426950408889634f, LN2 = 0.6931471805599453f;
+    extern __shared__ __attribute__((aligned(128))) float smem[];
+    uint16_t* Ks = reinterpret_cast<uint16_t*>(smem);      // [CH][LDK]   keys of the chunk
+    uint16_t* Vt = Ks + CH * LDK;                           // [D][LDVT]   values, transposed, slot order
+    uint16_t* Fo = Vt + D * LDVT;                           // [CH][LDFO]  features for the band kernel
+    float* diag = reinterpret_cast<float*>(Fo + CH * LDFO); // [CH]        t log2e |k|^2 / 2
+    float* red = diag + CH;                                 // [4]         wave maxima
+
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
+    const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H, sp = blockIdx.x;
+    const uint16_t* kptr = reinterpret_cast<const uint16_t*>(a.k) + b * a.k_sb + h * a.k_sh;
+    const uint16_t* vptr = reinterpret_cast<const uint16_t*>(a.v) + b * a.v_sb + h * a.v_sh;
+    const int len = a.lens ? min((int)a.lens[b], a.S) : a.S;
+    const float lnm_half2 = 0.5f * __log2f(2.0f * a.mh_valid);
+    const int per = (a.n_chunks + a.n_split - 1) / a.n_split;
+    const int c0 = sp * per, c1 = min(a.n_chunks, c0 + per);
+
+    Tile16<CH, E, NT> rk;
+    Tile16<CH, D, NT> rv;
+    if (c0 < c1) {
+        rk.fetch(kptr, a.k_ss, c0 * CH, a.S - 1, tid);
+        rv.fetch(vptr, a.v_ss, c0 * CH, a.S - 1, tid);
+    }
+    // this wave's projection rows (feature c of block w + 4 fi), scaled by sqrt(t) log2e, as bf16 head
+    // and remainder: lane (c = r16, g) holds columns 32ks + 8g .. + 7
+    uint4 phi[FPW][KS], plo[FPW][KS];
+    const float pscale = sqrtf(a.temp) * LOG2E;
+#pragma unroll
+    for (int fi = 0; fi < FPW; ++fi) {
+        const int row = min(16 * (w + 4 * fi) + r16, MH - 1);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const float* src = a.proj + (long)row * E + 32 * ks + 8 * g;
+            const floatx4 x0 = *reinterpret_cast<const floatx4*>(src) * pscale;
+            const floatx4 x1 = *reinterpret_cast<const floatx4*>(src + 4) * pscale;
+            float xs[8] = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+            uint32_t hw[4], lw[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                hw[j] = pack_bf16x2(xs[2 * j], xs[2 * j + 1]);
+                lw[j] = pack_bf16x2(xs[2 * j] - __uint_as_float(hw[j] << 16), xs[2 * j + 1] - __uint_as_float(hw[j] & 0xffff0000u));
+            }
+            phi[fi][ks] = make_uint4(hw[0], hw[1], hw[2], hw[3]);
+            plo[fi][ks] = make_uint4(lw[0], lw[1], lw[2], lw[3]);
+        }
+    }
+    // the tile in registers -> LDS: K rows as they are; V transposed into the slot order of the band
+    // kernel's P V (column 32 t + 8g + 4h + i <- key 32 t + 16 h + 4 g + i); |k|^2 per key on the way
+    auto stash = [&]() __attribute__((always_inline)) {
+        rk.template stash<LDK>(Ks, tid);
+#pragma unroll
+        for (int j = 0; j < Tile16<CH, E, NT>::N; ++j) {
+            constexpr int C8 = E / 8;
+            const int idx = tid + NT * j, row = idx / C8;
+            const uint32_t wds[4] = {rk.r[j][0], rk.r[j][1], rk.r[j][2], rk.r[j][3]};
+            float sq = 0.f;
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                const float lo = __uint_as_float(wds[x] << 16), hi = __uint_as_float(wds[x] & 0xffff0000u);
+                sq += lo * lo + hi * hi;
+            }
+#pragma unroll
+            for (int off = 1; off < C8; off <<= 1) sq += __shfl_xor(sq, off);      // the C8 lanes of one key row
+            if (idx % C8 == 0 && idx < CH * C8) diag[row] = 0.5f * a.temp * LOG2E * sq;
+        }
+#pragma unroll
+        for (int j = 0; j < Tile16<CH, D, NT>::N; ++j) {
+            constexpr int C8 = D / 8;
+            const int idx = tid + NT * j, key = idx / C8, c8 = idx % C8;
+            if (idx < CH * C8) {
+                const int col = 32 * (key >> 5) + 8 * ((key >> 2) & 3) + 4 * ((key >> 4) & 1) + (key & 3);
+                const uint32_t wds[4] = {rv.r[j][0], rv.r[j][1], rv.r[j][2], rv.r[j][3]};
+#pragma unroll
+                for (int x = 0; x < 8; ++x) Vt[(8 * c8 + x) * LDVT + col] = (uint16_t)(wds[x >> 1] >> (16 * (x & 1)));
+            }
+        }
+    };
+    if (c0 < c1) stash();
+    __syncthreads();
+
+    floatx4 kvacc[FPW][2][DB];                   // [block][sign][value block]
+    float ksum_p[FPW], ksum_n[FPW];              // this lane's feature, summed over its keys
+#pragma unroll
+    for (int fi = 0; fi < FPW; ++fi) {
+        ksum_p[fi] = ksum_n[fi] = 0.f;
+#pragma unroll
+        for (int sg = 0; sg < 2; ++sg)
+#pragma unroll
+            for (int db = 0; db < DB; ++db) kvacc[fi][sg][db] = Frag<float>::zero();
+    }
+    float run_max = -INFINITY;
+
+    for (int c = c0; c < c1; ++c) {
+        const int s_base = c * CH;
+        if (c + 1 < c1) {
+            rk.fetch(kptr, a.k_ss, s_base + CH, a.S - 1, tid);
+            rv.fetch(vptr, a.v_ss, s_base + CH, a.S - 1, tid);
+        }
+        // projections: dd[fi][kb][i] = log2e sqrt(t) P[feature] . k[key 16kb + 4g + i]
+        uint4 kf[KBN][KS];
+#pragma unroll
+        for (int kb = 0; kb < KBN; ++kb)
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+                kf[kb][ks] = *reinterpret_cast<const uint4*>(Ks + (16 * kb + r16) * LDK + 32 * ks + 8 * g);
+        floatx4 dg[KBN];
+#pragma unroll
+        for (int kb = 0; kb < KBN; ++kb) dg[kb] = *reinterpret_cast<const floatx4*>(diag + 16 * kb + 4 * g);
+        floatx4 dd[FPW][KBN];
+#pragma unroll
+        for (int fi = 0; fi < FPW; ++fi)
+#pragma unroll
+            for (int kb = 0; kb < KBN; ++kb) {
+                dd[fi][kb] = Frag<float>::zero();
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    dd[fi][kb] = mma_bf16(kf[kb][ks], phi[fi][ks], dd[fi][kb]);
+                    dd[fi][kb] = mma_bf16(kf[kb][ks], plo[fi][ks], dd[fi][kb]);
+                }
+            }
+        // chunk stabiliser: max over valid keys and features of |dd| - diag
+        float cs = -INFINITY;
+#pragma unroll
+        for (int fi = 0; fi < FPW; ++fi) {
+            const bool fvalid = (w + 4 * fi) < FB && 16 * (w + 4 * fi) + r16 < a.mh_valid;
+#pragma unroll
+            for (int kb = 0; kb < KBN; ++kb)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const bool ok = fvalid && (s_base + 16 * kb + 4 * g + i) < len;
+                    cs = fmaxf(cs, ok ? fabsf(dd[fi][kb][i]) - dg[kb][i] : -INFINITY);
+                }
+        }
+        // a valid key whose features are all masked (mh_valid rows only in other waves) still bounds the max
+#pragma unroll
+        for (int kb = 0; kb < KBN; ++kb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if ((s_base + 16 * kb + 4 * g + i) < len) cs = fmaxf(cs, -dg[kb][i]);
+        cs = wave_max(cs) - lnm_half2;
+        if (lane == 0) red[w] = cs;
+        __syncthreads();
+        const float lmax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+        const float new_max = fmaxf(run_max, lmax);
+        const bool live = new_max != -INFINITY;              // workgroup-uniform: some valid key so far
+        const float rescale = (run_max == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(run_max - new_max);
+        if (live) run_max = new_max;
+        // per (block, sign): features of the lane's feature for all 64 keys -> column sums, the feature
+        // scratch in LDS (band kernel's order: block bm of the [positive | negative] row, feature c of it
+        // -> position 32 (bm/2) + 8 (c/4) + 4 (bm%2) + c%4 of the key's row) and K'^T V
+#pragma unroll
+        for (int fi = 0; fi < FPW; ++fi) {
+            const bool fvalid = (w + 4 * fi) < FB && 16 * (w + 4 * fi) + r16 < a.mh_valid;
+            ksum_p[fi] *= rescale;
+            ksum_n[fi] *= rescale;
+#pragma unroll
+            for (int sg = 0; sg < 2; ++sg) {
+#pragma unroll
+                for (int db = 0; db < DB; ++db) kvacc[fi][sg][db] *= rescale;
+                floatx4 fv[KBN];
+                float tot = 0.f;
+#pragma unroll
+                for (int kb = 0; kb < KBN; ++kb)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const bool ok = live && fvalid && (s_base + 16 * kb + 4 * g + i) < len;
+                        const float x = sg ? -dd[fi][kb][i] : dd[fi][kb][i];
+                        fv[kb][i] = ok ? __builtin_amdgcn_exp2f(x - dg[kb][i] - lnm_half2 - new_max) : 0.f;
+                        tot += fv[kb][i];
+                    }
+                if (sg) ksum_n[fi] += tot; else ksum_p[fi] += tot;
+                if ((w + 4 * fi) < FB) {
+                    const int bm = sg * FB + w + 4 * fi;
+                    const int pos = 32 * (bm >> 1) + 8 * (r16 >> 2) + 4 * (bm & 1) + (r16 & 3);
+#pragma unroll
+                    for (int kb = 0; kb < KBN; ++kb)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) Fo[(16 * kb + 4 * g + i) * LDFO + pos] = f32_to_bf16(fv[kb][i]);
+                }
+                // KV[feature][d] += sum_keys F[key][feature] V[key][d], 32 keys per MFMA step
+#pragma unroll
+                for (int t = 0; t < CH / 32; ++t) {
+                    const floatx4 f0 = fv[2 * t], f1 = fv[2 * t + 1];
+                    const uint4 fa = make_uint4(pack_bf16x2(f0[0], f0[1]), pack_bf16x2(f0[2], f0[3]),
+                                                pack_bf16x2(f1[0], f1[1]), pack_bf16x2(f1[2], f1[3]));
+#pragma unroll
+                    for (int db = 0; db < DB; ++db)
+                        kvacc[fi][sg][db] = mma_bf16(fa, *reinterpret_cast<const uint4*>(Vt + (16 * db + r16) * LDVT + 32 * t + 8 * g),
+                                                     kvacc[fi][sg][db]);
+                }
+            }
+        }
+        if (tid == 0) a.chunk_scale[(long)bh * a.n_chunks + c] = live ? new_max * LN2 : 0.f;
+        __syncthreads();                         // Fo complete
+        // LDS -> HBM in 16-byte pieces: the chunk's features, and its V as two transposed 32-key tiles
+        {
+            uint16_t* fdst = reinterpret_cast<uint16_t*>(a.kfeat) + ((long)bh * a.n_chunks * CH + s_base) * M;
+#pragma unroll
+            for (int j = 0; j < CH * M / 8 / NT; ++j) {
+                const int idx = tid + NT * j, row = idx / (M / 8), c8 = idx % (M / 8);
+                *reinterpret_cast<uint4*>(fdst + (long)row * M + 8 * c8) = *reinterpret_cast<const uint4*>(Fo + row * LDFO + 8 * c8);
+            }
+            uint16_t* vdst = reinterpret_cast<uint16_t*>(a.vt) + ((long)bh * a.n_chunks + c) * (CH * D);
+#pragma unroll
+            for (int j = 0; j < (CH * D / 8 + NT - 1) / NT; ++j) {
+                const int idx = tid + NT * j, tile = idx / (D * 4), rem = idx % (D * 4), d = rem / 4, c8 = rem % 4;
+                if (idx < CH * D / 8)
+                    *reinterpret_cast<uint4*>(vdst + tile * (D * 32) + d * 32 + 8 * c8) =
+                        *reinterpret_cast<const uint4*>(Vt + d * LDVT + 32 * tile + 8 * c8);
+            }
+        }
+        __syncthreads();                         // everyone is done with this chunk's tiles
+        if (c + 1 < c1) stash();
+        __syncthreads();
+    }
+
+    // partial K'^T V in accumulator order: tile (rb, db) -> 64 lanes x 4 floats (see sb_combine_kernel)
+    float* part = a.kv_part + ((long)bh * a.n_split + sp) * (M * (D + 1));
+#pragma unroll
+    for (int fi = 0; fi < FPW; ++fi) {
+        if ((w + 4 * fi) < FB) {
+#pragma unroll
+            for (int sg = 0; sg < 2; ++sg) {
+                const int rb = sg * FB + w + 4 * fi;
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+                    *reinterpret_cast<floatx4*>(part + ((rb * DB + db) * 64 + lane) * 4) = kvacc[fi][sg][db];
+                const float tot = group_sum(sg ? ksum_n[fi] : ksum_p[fi]);       // over the four key groups g
+                if (g == 0) part[M * D + sg * MH + 16 * (w + 4 * fi) + r16] = tot;
+            }
+        }
+    }
+    if (tid == 0) a.part_max[(long)bh * a.n_split + sp] = run_max * LN2;
+}
+
+// ---------------------------------------------------------------------------------------
 // plain local attention (no random features): softmax over the band, P V
 // ---------------------------------------------------------------------------------------
 // The band kernel without its low-rank half: per (batch, head, 64-query tile) scores^T = (t log2e) K q
@@ -1419,8 +1673,24 @@ template <int E, int M> constexpr size_t fwd_smem() {
     return sizeof(float) * need;
 }
 
+template <int E, int M> constexpr size_t kfeat_bf16_smem() {
+    return 2 * ((size_t)CH * (E + 8) + (size_t)E * (CH + 8) + (size_t)CH * (M + 8)) + sizeof(float) * (CH + 8);
+}
 template <typename T, int E, int M>
 static int launch_kfeat(const KvArgs& a, hipStream_t st) {
+    if (sizeof(T) == 2 && !a.q) {            // bfloat16 keys, no query role: both products on the bf16 MFMA
+        auto kern16 = sb_kfeat_bf16_kernel<E, E, M>;
+        constexpr size_t smem16 = kfeat_bf16_smem<E, M>();
+        static bool lds16_ready = false;
+        if (!lds16_ready) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern16),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem16);
+            if (e != hipSuccess) return fail(ERR_LAUNCH, "sb_kfeat_bf16: LDS attribute: %s", hipGetErrorString(e));
+            lds16_ready = true;
+        }
+        hipLaunchKernelGGL(kern16, dim3(a.n_split, a.B * a.H), dim3(NT), smem16, st, a);
+        return check_launch("sb_kfeat_bf16_kernel");
+    }
     auto kern = sb_kfeat_kernel<T, E, E, M>;
     constexpr size_t smem = kfeat_smem<E, M>();
     static bool lds_ready = false;     // one instantiation = one kernel; set its LDS limit once
