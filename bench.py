@@ -42,8 +42,8 @@ def sblocal_flops(B, H, T, S, E, D, m, lc):
     kv = 2 * B * H * S * m * D
     qkv = 2 * B * H * T * m * D + 2 * B * H * T * m
     total = band + proj_q + proj_k + kv + qkv
-    fused = band + qkv                     # what the fused band kernel computes (with several parts per
-    return total, fused                    # query tile the query projection runs in the key pass)
+    fused = band                           # what the fused band kernel computes when the band of a query tile
+    return total, fused                    # is split: projections in the key pass, low-rank term in the merge
 
 
 def bench_sblocal(steps, warmup, cpu_baseline=True):

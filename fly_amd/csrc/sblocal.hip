@@ -6,7 +6,8 @@
 //                       MFMA, wavefront max reductions, exp), written to HBM once, plus the partial
 //                       K'^T V / sum K' reductions with an online rescale to the running maximum.
 //                       Query role (small problems only): the features of 64 queries.
-//   sb_combine_kernel : merges the partial reductions of one (batch, head).
+//   sb_combine_kernel : merges the partial reductions of one (batch, head) (large problems; on small
+//                       ones extra workgroups of the band kernel's launch do it).
 //   sblocal_fwd_kernel: per (batch, head, 64-query tile, part of the band): query features in
 //                       registers, then for each 32-key tile of its share of the band Q K^T and
 //                       Q' K'^T on MFMA (transposed, so that every lane owns one query),
@@ -14,7 +15,8 @@
 //                       P V on MFMA; key tiles are double-buffered through LDS.  With one part the
 //                       epilogue adds the global low-rank term and writes out / log-normaliser;
 //                       with several parts (small problems, to fill the chip) each part writes an
-//                       un-normalised partial and sb_merge_kernel finishes the job.
+//                       un-normalised partial and sb_merge_kernel finishes the job: it merges the
+//                       parts and adds the global low-rank term.
 //
 // Layout of an MFMA 16x16 result in a lane (r = lane%16, g = lane/16): element i is
 // C[4g+i][r].  All products are formed "transposed" (rows = keys / features / value dims,
@@ -66,6 +68,9 @@ struct FwdArgs {
     const void* q; const void* k; const void* v; const float* proj;
     const void* kfeat; const float* chunk_scale; const float* kv; const float* ksum; const float* kmax;
     const float* qfeat; const float* q_lsq; const void* vt; const void* kvt;
+    // several parts per query tile: the partial reductions of the key pass, merged by extra
+    // workgroups of the band kernel's launch (ids >= band_wgs) into kv / ksum / kmax for the merge kernel
+    const float* kv_part; const float* part_max; int n_split, band_wgs, cmb_wpb;    // cmb_wpb: combine workgroups per (batch, head)
     const int64_t* lens; void* out; float* log_norm; float* part_ws;
     int B, H, T, S, mh_valid, lc, n_chunks, n_parts;
     long q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss;
@@ -108,46 +113,63 @@ __device__ __forceinline__ void load_proj(float* Ps, const float* proj, float sc
     t.template stash<E + 4>(Ps, tid, scale);
 }
 
-// KV = sum_s exp(part_max_s - kmax) KV_s, same for Ksum; one thread per output element, the
-// weights staged in LDS so that the loads over s are independent and stay in flight together
+// KV = sum_s exp(part_max_s - kmax) KV_s, same for Ksum, of one (batch, head) by `wpb` workgroups
+// (this is number `ci` of them; the output elements are dealt to their threads round-robin), the
+// weights staged in LDS (`wgt`, n_split floats) so that the loads over s are independent and stay
+// in flight together
 constexpr int MAX_SPLIT = 1024;
-__global__ __launch_bounds__(NT) void sb_combine_kernel(const float* kv_part, const float* part_max, float* kv,
-                                                        float* ksum, float* kmax_out, uint16_t* kvt, int n_split,
-                                                        int M, int D) {
-    __shared__ float wgt[MAX_SPLIT];
-    const int bh = blockIdx.y;
-    const int idx = blockIdx.x * NT + threadIdx.x;
+__device__ __forceinline__ void sb_combine_body(float* wgt, const float* kv_part, const float* part_max, float* kv,
+                                                float* ksum, float* kmax_out, uint16_t* kvt, int bh, int ci, int wpb,
+                                                int n_split, int M, int D) {
+    const int nthr = blockDim.x;
     const int per = M * (D + 1);
     float kmax = -INFINITY;
     for (int s = 0; s < n_split; ++s) kmax = fmaxf(kmax, part_max[(long)bh * n_split + s]);
-    for (int s = threadIdx.x; s < n_split; s += NT) {
+    for (int s = threadIdx.x; s < n_split; s += nthr) {
         const float pm = part_max[(long)bh * n_split + s];
         // same expression as the band kernel's chunk weight, so that both sides of the
         // "global minus band" low-rank difference carry bit-identical factors
         wgt[s] = (pm == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((pm - kmax) * 1.4426950408889634f);
     }
     __syncthreads();
-    if (idx == 0) kmax_out[bh] = (kmax == -INFINITY) ? 0.f : kmax;
-    if (idx >= per) return;
-    // threads walk a partial in its storage order (coalesced reads over the splits); the K'^T V part
-    // is in accumulator order: offset ((tile*64 + lane)*4 + i) holds element (r, d) of tile
-    // (r/16, d/16) with lane = 16*((r%16)/4) + d%16 and i = r%4
-    const float* src = kv_part + (long)bh * n_split * per + idx;
-    float acc = 0.f;
+    if (ci == 0 && threadIdx.x == 0) kmax_out[bh] = (kmax == -INFINITY) ? 0.f : kmax;
+    for (int idx = ci * nthr + threadIdx.x; idx < per; idx += wpb * nthr) {
+        // threads walk a partial in its storage order (coalesced reads over the splits); the K'^T V part
+        // is in accumulator order: offset ((tile*64 + lane)*4 + i) holds element (r, d) of tile
+        // (r/16, d/16) with lane = 16*((r%16)/4) + d%16 and i = r%4
+        const float* src = kv_part + (long)bh * n_split * per + idx;
+        float acc = 0.f;
 #pragma unroll 16
-    for (int s = 0; s < n_split; ++s) acc += wgt[s] * src[(long)s * per];
-    if (idx < M * D) {
-        const int i = idx & 3, lane = (idx >> 2) & 63, tile = idx >> 8;
-        const int db_n = D >> 4, rb = tile / db_n, db = tile % db_n;
-        const int r = 16 * rb + 4 * (lane >> 4) + i, d = 16 * db + (lane & 15);
-        kv[(long)bh * M * D + r * D + d] = acc;
-        if (kvt) {      // bf16 copy for the bf16 band kernel: [d][slot], feature r in the k-slot order of its MFMA
-            const int c = r >> 4, slot = 32 * (c >> 1) + 8 * ((r >> 2) & 3) + 4 * (c & 1) + (r & 3);
-            kvt[(long)bh * M * D + d * M + slot] = f32_to_bf16(acc);
+        for (int s = 0; s < n_split; ++s) acc += wgt[s] * src[(long)s * per];
+        if (idx < M * D) {
+            const int i = idx & 3, lane = (idx >> 2) & 63, tile = idx >> 8;
+            const int db_n = D >> 4, rb = tile / db_n, db = tile % db_n;
+            const int r = 16 * rb + 4 * (lane >> 4) + i, d = 16 * db + (lane & 15);
+            kv[(long)bh * M * D + r * D + d] = acc;
+            if (kvt) {      // bf16 copy for the bf16 band kernel: [d][slot], feature r in the k-slot order of its MFMA
+                const int c = r >> 4, slot = 32 * (c >> 1) + 8 * ((r >> 2) & 3) + 4 * (c & 1) + (r & 3);
+                kvt[(long)bh * M * D + d * M + slot] = f32_to_bf16(acc);
+            }
+        } else {
+            ksum[(long)bh * M + idx - M * D] = acc;
         }
-    } else {
-        ksum[(long)bh * M + idx - M * D] = acc;
     }
+}
+
+__global__ __launch_bounds__(NT) void sb_combine_kernel(const float* kv_part, const float* part_max, float* kv,
+                                                        float* ksum, float* kmax_out, uint16_t* kvt, int n_split,
+                                                        int M, int D) {
+    __shared__ float wgt[MAX_SPLIT];
+    sb_combine_body(wgt, kv_part, part_max, kv, ksum, kmax_out, kvt, blockIdx.y, blockIdx.x, gridDim.x, n_split, M, D);
+}
+
+// The band kernels' view of the same maximum when the combine shares their launch (several parts per
+// query tile): every wave reduces the partial maxima itself.
+__device__ __forceinline__ float split_kmax(const float* part_max, int bh, int n_split) {
+    float pm = -INFINITY;
+    for (int s = threadIdx.x & 63; s < n_split; s += 64) pm = fmaxf(pm, part_max[(long)bh * n_split + s]);
+    pm = wave_max(pm);
+    return pm == -INFINITY ? 0.f : pm;
 }
 
 // ---------------------------------------------------------------------------------------
@@ -500,6 +522,12 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
     uint16_t* lds = reinterpret_cast<uint16_t*>(smem);
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
+    if (SPLIT && (int)blockIdx.x >= a.band_wgs) {       // combine role, see sblocal_fwd_kernel
+        const int ci = blockIdx.x - a.band_wgs;
+        sb_combine_body(smem, a.kv_part, a.part_max, const_cast<float*>(a.kv), const_cast<float*>(a.ksum),
+                        const_cast<float*>(a.kmax), nullptr, ci / a.cmb_wpb, ci % a.cmb_wpb, a.cmb_wpb, a.n_split, M, D);
+        return;
+    }
     const int n_qt = (a.T + TQ - 1) / TQ;
     const int n_items = a.B * a.H * n_qt * a.n_parts;
     const int per_xcd = (n_items + N_XCD - 1) / N_XCD;
@@ -528,13 +556,12 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
     int kt_lo = lo / TK;
     int kt_hi = (hi > lo) ? (hi + TK - 1) / TK : kt_lo;
     if (SPLIT) {
-        const int per = (kt_hi - kt_lo + 1 + a.n_parts - 1) / a.n_parts;
-        const int first = kt_lo + part * per - (part > 0 ? 1 : 0);
-        const int last = kt_lo + (part + 1) * per - 1;
+        const int per = (kt_hi - kt_lo + a.n_parts - 1) / a.n_parts;
+        const int first = kt_lo + part * per;
         kt_lo = min(kt_hi, first);
-        kt_hi = min(kt_hi, last);
+        kt_hi = min(kt_hi, first + per);
     }
-    const bool lowrank_here = !SPLIT || part == 0;     // workgroup-uniform
+    constexpr bool lowrank_here = !SPLIT;              // with several parts the merge kernel adds the low-rank term
 
     // Key tiles travel global -> registers -> LDS.  A tile is requested two iterations before it is
     // used (one iteration of work is shorter than the latency of the loads under load), so two
@@ -564,7 +591,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
     // (clamped tile indices: the loads are unconditional so that the register sets are plain values)
     fetch(ra, min(kt_lo, max(kt_hi - 1, 0)));
     fetch(rb, min(kt_lo + 1, max(kt_hi - 1, 0)));
-    const float kmax = a.kmax[bh];
+    const float kmax = SPLIT ? split_kmax(a.part_max, bh, a.n_split) : a.kmax[bh];
 
     // score operand: the query row as it is in memory
     const uint16_t* qrow = qptr + (long)min(iq, a.T - 1) * a.q_ss;
@@ -852,16 +879,13 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
             float* ws = a.part_ws + (((long)bh * n_qt64 + t64) * a.n_parts + part) * (TQ64 * (D + NSTAT));
             const int ql = (16 * w + r16) % TQ64;
 #pragma unroll
-            for (int db = 0; db < DB; ++db) {
-                floatx4 o = oacc[db] + gamma * lacc[db];
-                *reinterpret_cast<floatx4*>(ws + ql * D + 16 * db + 4 * g) = o;
-            }
+            for (int db = 0; db < DB; ++db) *reinterpret_cast<floatx4*>(ws + ql * D + 16 * db + 4 * g) = oacc[db];
             if (g == 0) {
                 float* st = ws + TQ64 * D;
                 st[0 * TQ64 + ql] = m_run;
                 st[1 * TQ64 + ql] = ze;
                 st[2 * TQ64 + ql] = zp;
-                st[3 * TQ64 + ql] = qk1;
+                st[3 * TQ64 + ql] = 0.f;
                 st[4 * TQ64 + ql] = c0;
             }
         }
@@ -1275,66 +1299,6 @@ __global__ __launch_bounds__(NT) void local_fwd_kernel(LocalArgs a) {
     }
 }
 
-// Merge of the per-part partials of one query tile by the 256 threads of a workgroup: thread
-// (query ql = tid / 4, column quarter tid % 4).  Parts are taken in batches whose loads are all
-// issued before the first is used (slots past n_parts re-read the last part and are ignored),
-// with an online rescale to the running maximum between batches.
-template <typename T, int D>
-__device__ __forceinline__ void sb_merge_tile(const FwdArgs& a, int bh, int qt, int n_qt) {
-    constexpr float LN2 = 0.6931471805599453f;
-    constexpr int NV = D / 16;                      // floatx4 per thread and part
-    constexpr int PB = D <= 64 ? 8 : 4;             // parts per batch
-    const int tid = threadIdx.x, ql = tid >> 2, d0 = (tid & 3) * (D / 4);
-    const int b = bh / a.H, h = bh % a.H;
-    const int iq = qt * TQ + ql;
-    const long stride = (long)TQ * (D + NSTAT);
-    const float* ws = a.part_ws + ((long)bh * n_qt + qt) * a.n_parts * stride;
-    const float* st = ws + TQ * D + ql;
-    const float qk1 = st[3 * TQ], c0 = st[4 * TQ];  // carried by part 0
-    float m_star = -INFINITY, ze = 0.f, zp = 0.f;
-    floatx4 acc[NV];
-#pragma unroll
-    for (int v = 0; v < NV; ++v) acc[v] = Frag<float>::zero();
-    for (int p0 = 0; p0 < a.n_parts; p0 += PB) {
-        float mv[PB], zev[PB], zpv[PB];
-        floatx4 ov[PB][NV];
-#pragma unroll
-        for (int j = 0; j < PB; ++j) {
-            const long off = (long)min(p0 + j, a.n_parts - 1) * stride;
-            mv[j] = st[off];
-            zev[j] = st[off + TQ];
-            zpv[j] = st[off + 2 * TQ];
-#pragma unroll
-            for (int v = 0; v < NV; ++v) ov[j][v] = *reinterpret_cast<const floatx4*>(ws + off + ql * D + d0 + 4 * v);
-        }
-        float m_new = m_star;
-#pragma unroll
-        for (int j = 0; j < PB; ++j) m_new = fmaxf(m_new, mv[j]);      // repeated slots repeat a valid value
-        const float keep = (m_star == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_star - m_new);
-        m_star = m_new;
-        ze *= keep;
-#pragma unroll
-        for (int v = 0; v < NV; ++v) acc[v] *= keep;
-#pragma unroll
-        for (int j = 0; j < PB; ++j) {
-            if (p0 + j < a.n_parts) {
-                const float wgt = __builtin_amdgcn_exp2f(mv[j] - m_star);
-                ze += wgt * zev[j];
-                zp += zpv[j];
-#pragma unroll
-                for (int v = 0; v < NV; ++v) acc[v] += wgt * ov[j][v];
-            }
-        }
-    }
-    if (iq >= a.T) return;
-    const float Z = ze + __builtin_amdgcn_exp2f(c0 - m_star) * fmaxf(qk1 - zp, 1e-24f);
-    const float inv = 1.0f / Z;
-    T* optr = reinterpret_cast<T*>(a.out) + b * a.o_sb + h * a.o_sh + (long)iq * a.o_ss + d0;
-#pragma unroll
-    for (int v = 0; v < NV; ++v) store4_f32(optr + 4 * v, acc[v] * inv);
-    if ((tid & 3) == 0) a.log_norm[(long)bh * a.T + iq] = m_star * LN2 + __logf(Z);
-}
-
 // ---------------------------------------------------------------------------------------
 // fused band kernel
 // ---------------------------------------------------------------------------------------
@@ -1347,6 +1311,14 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
     float* Ps = smem;                                  // only live before the key loop
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
+    if (SPLIT && (int)blockIdx.x >= a.band_wgs) {
+        // combine role: the partial K'^T V / sum K' of the key pass become kv / ksum / kmax for the merge
+        // kernel (nothing in THIS launch reads them: the parts take kmax from the partial maxima)
+        const int ci = blockIdx.x - a.band_wgs;
+        sb_combine_body(smem, a.kv_part, a.part_max, const_cast<float*>(a.kv), const_cast<float*>(a.ksum),
+                        const_cast<float*>(a.kmax), nullptr, ci / a.cmb_wpb, ci % a.cmb_wpb, a.cmb_wpb, a.n_split, M, D);
+        return;
+    }
     // Workgroups are handed to the 8 XCDs round-robin in launch order, and every XCD has its own
     // L2.  The linear id is therefore re-mapped so that one XCD works on a contiguous run of
     // (batch-head, query tile, part) items: neighbours in that order share key tiles.
@@ -1377,12 +1349,10 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
     int kt_lo = lo / TK;
     int kt_hi = (hi > lo) ? (hi + TK - 1) / TK : kt_lo;
     if (SPLIT) {
-        // the global low-rank epilogue of part 0 counts as one more tile when sharing out the band
-        const int per = (kt_hi - kt_lo + 1 + a.n_parts - 1) / a.n_parts;
-        const int first = kt_lo + part * per - (part > 0 ? 1 : 0);
-        const int last = kt_lo + (part + 1) * per - 1;
+        const int per = (kt_hi - kt_lo + a.n_parts - 1) / a.n_parts;
+        const int first = kt_lo + part * per;
         kt_lo = min(kt_hi, first);
-        kt_hi = min(kt_hi, last);
+        kt_hi = min(kt_hi, first + per);
     }
 
     // start the first tile's loads before anything else
@@ -1397,7 +1367,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
     }
     const float* csp = a.chunk_scale + (long)bh * a.n_chunks;
     float cscale = (kt_lo < kt_hi) ? csp[kt_lo * TK / CH] : 0.f;
-    const float kmax = a.kmax[bh];
+    const float kmax = SPLIT ? split_kmax(a.part_max, bh, a.n_split) : a.kmax[bh];
 
     // query operand (B side: column = query, k = 16c+4g+j) and its squared norm
     floatx4 qr[EC];
@@ -1585,12 +1555,12 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
 
     FLY_PROF(3);
     // global low-rank term: qkv^T[d][query] = sum_r KV[r][d] q'[query][r],  qk1 = q' . Ksum
-    // (with several parts only part 0 carries it)
+    // (with several parts the merge kernel adds it)
     floatx4 lacc[DB];
 #pragma unroll
     for (int db = 0; db < DB; ++db) lacc[db] = Frag<float>::zero();
     float qk1 = 0.f;
-    if (!SPLIT || part == 0) {                       // workgroup-uniform
+    if (!SPLIT) {
         // K'^T V (M x D) and sum K' (M) staged in LDS: coalesced loads, all in flight together
         float* KVs = smem;
         float* KSs = smem + M * LDV;
@@ -1623,16 +1593,13 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
         float* ws = a.part_ws + (((long)bh * n_qt + qt) * a.n_parts + part) * (TQ * (D + NSTAT));
         const int ql = 16 * w + r16;
 #pragma unroll
-        for (int db = 0; db < DB; ++db) {
-            floatx4 o = oacc[db] + gamma * lacc[db];
-            *reinterpret_cast<floatx4*>(ws + ql * D + 16 * db + 4 * g) = o;
-        }
+        for (int db = 0; db < DB; ++db) *reinterpret_cast<floatx4*>(ws + ql * D + 16 * db + 4 * g) = oacc[db];
         if (g == 0) {
             float* st = ws + TQ * D;
             st[0 * TQ + ql] = m_run;
             st[1 * TQ + ql] = ze;
             st[2 * TQ + ql] = zp;
-            st[3 * TQ + ql] = qk1;
+            st[3 * TQ + ql] = 0.f;
             st[4 * TQ + ql] = c0;
         }
     } else {
@@ -1651,10 +1618,92 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
     FLY_PROF(5);
 }
 
-// one workgroup per query tile
-template <typename T, int D>
+// Finish of a query tile that was computed in parts: one workgroup per (64-query tile, batch-head),
+// in the register layout of the band kernel (wave w, lane (r16, g): query 16w + r16, output columns
+// 16db + 4g + i).  It merges the parts' un-normalised partials -- taken in batches whose loads are all
+// issued before the first is used (slots past n_parts re-read the last part and are ignored), with an
+// online rescale to the running maximum between batches -- and adds the global low-rank term
+// q' (K'^T V), q' . sum K' on fp32 MFMA from the query features of the key pass and the combined
+// reductions, then normalises.
+template <typename T, int D, int M>
 __global__ __launch_bounds__(NT) void sb_merge_kernel(FwdArgs a) {
-    sb_merge_tile<T, D>(a, blockIdx.y, blockIdx.x, gridDim.x);
+    constexpr float LN2 = 0.6931471805599453f;
+    constexpr int FC = M / 16, LDV = 16 + 4;
+    constexpr int PB = 8;                            // parts per batch
+    __shared__ __attribute__((aligned(16))) float KVs[M * LDV];      // 16 columns of K'^T V
+    __shared__ __attribute__((aligned(16))) float KSs[M];            // sum K'
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
+    // one workgroup per (64-query tile, 16 output columns, batch-head): the tile's finish is spread over
+    // D/16 workgroups because it is all latency (a short chain of loads, 2 M/16 MFMAs, a store)
+    const int qt = blockIdx.x, n_qt = gridDim.x, db = blockIdx.y, bh = blockIdx.z, b = bh / a.H, h = bh % a.H;
+    const int ql = 16 * w + r16, iq = qt * TQ + ql;
+    {
+        RowTile<M, 16> kvt;
+        kvt.fetch(a.kv + (long)bh * M * D + 16 * db, D, 0, M - 1, tid);
+        if (tid < M) KSs[tid] = a.ksum[(long)bh * M + tid];
+        kvt.template stash<LDV>(KVs, tid);
+    }
+    const long qrow = (long)bh * a.T + min(iq, a.T - 1);
+    floatx4 qf[FC];
+#pragma unroll
+    for (int c = 0; c < FC; ++c) qf[c] = *reinterpret_cast<const floatx4*>(a.qfeat + qrow * M + 16 * c + 4 * g);
+
+    const long stride = (long)TQ * (D + NSTAT);
+    const float* ws = a.part_ws + ((long)bh * n_qt + qt) * a.n_parts * stride;
+    const float* st = ws + TQ * D + ql;
+    const float c0 = st[4 * TQ];                     // base-2 log-scale of the low-rank term (same in every part)
+    float m_star = -INFINITY, ze = 0.f, zp = 0.f;
+    floatx4 acc = Frag<float>::zero();
+    for (int p0 = 0; p0 < a.n_parts; p0 += PB) {
+        float mv[PB], zev[PB], zpv[PB];
+        floatx4 ov[PB];
+#pragma unroll
+        for (int j = 0; j < PB; ++j) {
+            const long off = (long)min(p0 + j, a.n_parts - 1) * stride;
+            mv[j] = st[off];
+            zev[j] = st[off + TQ];
+            zpv[j] = st[off + 2 * TQ];
+            ov[j] = *reinterpret_cast<const floatx4*>(ws + off + ql * D + 16 * db + 4 * g);
+        }
+        float m_new = m_star;
+#pragma unroll
+        for (int j = 0; j < PB; ++j) m_new = fmaxf(m_new, mv[j]);      // repeated slots repeat a valid value
+        const float keep = (m_star == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_star - m_new);
+        m_star = m_new;
+        ze *= keep;
+        acc *= keep;
+#pragma unroll
+        for (int j = 0; j < PB; ++j) {
+            if (p0 + j < a.n_parts) {
+                const float wgt = __builtin_amdgcn_exp2f(mv[j] - m_star);
+                ze += wgt * zev[j];
+                zp += zpv[j];
+                acc += wgt * ov[j];
+            }
+        }
+    }
+    __syncthreads();                                 // K'^T V and sum K' are in LDS
+    floatx4 lacc0 = Frag<float>::zero(), lacc1 = Frag<float>::zero();    // two chains
+    float qk1 = 0.f;
+#pragma unroll
+    for (int c = 0; c < FC; ++c) {
+        const floatx4 ks = *reinterpret_cast<const floatx4*>(KSs + 16 * c + 4 * g);
+        qk1 += qf[c][0] * ks[0] + qf[c][1] * ks[1] + qf[c][2] * ks[2] + qf[c][3] * ks[3];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float kvv = KVs[(16 * c + 4 * g + j) * LDV + r16];
+            if (j & 1) lacc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(kvv, qf[c][j], lacc1, 0, 0, 0);
+            else lacc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(kvv, qf[c][j], lacc0, 0, 0, 0);
+        }
+    }
+    qk1 = group_sum(qk1);
+    if (iq >= a.T) return;
+    const float gamma = __builtin_amdgcn_exp2f(c0 - m_star);              // <= 1: every part starts its maximum at c0
+    const float Z = ze + gamma * fmaxf(qk1 - zp, 1e-24f);
+    const float inv = 1.0f / Z;
+    T* optr = reinterpret_cast<T*>(a.out) + b * a.o_sb + h * a.o_sh + (long)iq * a.o_ss;
+    store4_f32(optr + 16 * db + 4 * g, (acc + gamma * (lacc0 + lacc1)) * inv);
+    if (g == 0 && db == 0) a.log_norm[(long)bh * a.T + iq] = m_star * LN2 + __logf(Z);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -1744,15 +1793,28 @@ static int launch_fwd_impl(const FwdArgs& a, hipStream_t st) {
     typedef FwdKernel<T, E, M, SPLIT> K;
     const int qt = (a.T + TQ - 1) / TQ;                           // 64-query tiles (partials, merge)
     const long items = (long)a.B * a.H * ((a.T + K::tq - 1) / K::tq) * a.n_parts;
-    const long grid = (items + N_XCD - 1) / N_XCD * N_XCD;       // whole rounds over the XCDs
+    long grid = (items + N_XCD - 1) / N_XCD * N_XCD;             // whole rounds over the XCDs
+    FwdArgs args = a;
+    args.band_wgs = (int)grid;
+    if (SPLIT) {
+        // combine role: as many workgroups per (batch, head) as fit beside the band workgroups in one
+        // residency round (two workgroups of this kernel per CU), at least one, at most one thread per output
+        const long bhn = (long)a.B * a.H, free_slots = 512 - grid;
+        long wpb = free_slots / bhn;
+        const long most = (M * (E + 1) + K::threads - 1) / K::threads;
+        if (wpb > most) wpb = most;
+        if (wpb < 1) wpb = 1;
+        args.cmb_wpb = (int)wpb;
+        grid += bhn * wpb;
+    }
     if (grid > 2147483647L) return fail(ERR_ARG, "sblocal_fwd: too many workgroups");
     if (g_ev_before) (void)hipEventRecord(g_ev_before, st);
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(K::threads), smem, st, a);
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(K::threads), smem, st, args);
     if (g_ev_after) (void)hipEventRecord(g_ev_after, st);
     g_ev_before = g_ev_after = nullptr;
     int rc = check_launch("sblocal_fwd_kernel");
     if (rc || !SPLIT) return rc;
-    hipLaunchKernelGGL((sb_merge_kernel<T, E>), dim3(qt, a.B * a.H), dim3(NT), 0, st, a);
+    hipLaunchKernelGGL((sb_merge_kernel<T, E, M>), dim3(qt, E / 16, a.B * a.H), dim3(NT), 0, st, args);
     return check_launch("sb_merge_kernel");
 }
 template <typename T, int E, int M>
@@ -1899,7 +1961,8 @@ extern "C" int flyhip_sb_kv_reduce(const void* k, const void* v, const float* pr
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     const int m = 2 * mh;
     rc = dispatch_kfeat(dtype, E, m, a, st);
-    if (rc) return rc;
+    if (rc || q) return rc;          // with query features asked for (several parts per query tile) the
+                                     // partial reductions are combined inside flyhip_sblocal_fwd's launch
     const int per = m * (D + 1);
     hipLaunchKernelGGL(sb_combine_kernel, dim3((per + NT - 1) / NT, B * H), dim3(NT), 0, st,
                        kv_part, part_max, kv, ksum, kmax, reinterpret_cast<uint16_t*>(kvt), n_split, m, D);
@@ -1908,8 +1971,9 @@ extern "C" int flyhip_sb_kv_reduce(const void* k, const void* v, const float* pr
 
 extern "C" int flyhip_sblocal_fwd(const void* q, const void* k, const void* v, const float* proj,
                                   const void* kfeat, const float* chunk_scale,
-                                  const float* kv, const float* ksum, const float* kmax,
+                                  float* kv, float* ksum, float* kmax,
                                   const float* qfeat, const float* q_lsq, const void* vt, const void* kvt,
+                                  const float* kv_part, const float* part_max, int n_split,
                                   const int64_t* key_lengths, void* out, float* log_norm,
                                   float* part_ws, int n_parts,
                                   int B, int H, int T, int S, int E, int D, int mh, int mh_valid,
@@ -1930,11 +1994,12 @@ extern "C" int flyhip_sblocal_fwd(const void* q, const void* k, const void* v, c
     FLY_REQUIRE((long)B * H <= 65535, "sblocal_fwd: B*H=%ld exceeds the grid limit 65535", (long)B * H);
     FLY_REQUIRE(n_parts >= 1 && n_parts <= 64, "sblocal_fwd: n_parts=%d outside [1, 64]", n_parts);
     FLY_REQUIRE(dtype != BF16 || (vt && kvt), "sblocal_fwd: bfloat16 inputs need the vt and kvt scratch of the key pass");
-    FLY_REQUIRE(n_parts == 1 || (part_ws && qfeat && q_lsq),
-                "sblocal_fwd: n_parts > 1 needs the partial workspace and the query features of the key pass");
+    FLY_REQUIRE(n_parts == 1 || (part_ws && qfeat && q_lsq && kv_part && part_max && n_split >= 1 && n_split <= MAX_SPLIT),
+                "sblocal_fwd: n_parts > 1 needs the partial workspace, the query features and the partial "
+                "reductions (kv_part, part_max, n_split) of the key pass");
     int nc, ns;
     plan(B, H, S, &nc, &ns);
-    FwdArgs a{q, k, v, proj, kfeat, chunk_scale, kv, ksum, kmax, qfeat, q_lsq, vt, kvt, key_lengths, out, log_norm, part_ws,
+    FwdArgs a{q, k, v, proj, kfeat, chunk_scale, kv, ksum, kmax, qfeat, q_lsq, vt, kvt, kv_part, part_max, n_split, 0, 1, key_lengths, out, log_norm, part_ws,
               B, H, T, S, mh_valid, local_context, nc, n_parts,
               q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss, softmax_temp};
     return dispatch_fwd(dtype, E, 2 * mh, a, reinterpret_cast<hipStream_t>(stream));

@@ -90,7 +90,8 @@ class SBLocalPlan:
         _lib.call('flyhip_sblocal_fwd', q.data_ptr(), k.data_ptr(), v.data_ptr(), proj.data_ptr(),
                   self.kfeat.data_ptr(), self.chunk_scale.data_ptr(), self.kv.data_ptr(),
                   self.ksum.data_ptr(), self.kmax.data_ptr(), _lib.ptr(self.qfeat), _lib.ptr(self.q_lsq),
-                  _lib.ptr(self.vt), _lib.ptr(self.kvt), _lib.ptr(lens), out.data_ptr(), log_norm.data_ptr(), _lib.ptr(self.part_ws), self.n_parts,
+                  _lib.ptr(self.vt), _lib.ptr(self.kvt), self.kv_part.data_ptr(), self.part_max.data_ptr(),
+                  self.n_split, _lib.ptr(lens), out.data_ptr(), log_norm.data_ptr(), _lib.ptr(self.part_ws), self.n_parts,
                   B, H, T, S, dim, dim, mh, mh_valid, local_context,
                   q.stride(0), q.stride(2), q.stride(1), k.stride(0), k.stride(2), k.stride(1),
                   v.stride(0), v.stride(2), v.stride(1), out.stride(0), out.stride(2), out.stride(1),

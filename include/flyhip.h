@@ -54,7 +54,9 @@ int flyhip_sb_plan(int B, int H, int T, int S, int local_context,
  * several workgroups share a query tile): q (B,T,H,E) via strides -> qfeat (B,H,T,m) fp32, the
  * query features exp(+-sqrt(t) P q - rowmax) (ref: softmax_kernel with is_query=True,
  * src/models/attention/feature_maps_sb.py:51-82,148-151), and q_lsq (B,H,T) fp32, their log-scale
- * -t|q|^2/2 + rowmax - log(m)/2.
+ * -t|q|^2/2 + rowmax - log(m)/2.  With q given, kv / ksum / kmax are NOT written: the partial
+ * reductions (kv_part, part_max) are combined inside flyhip_sblocal_fwd's launch instead, which
+ * saves a launch on problems this small.
  * bfloat16 inputs only (NULL otherwise): vt (B,H,n_chunks*64,D) bf16 and kvt (B,H,D,m) bf16, opaque
  * scratch for flyhip_sblocal_fwd -- V per 32-key tile and K'^T V, transposed into the operand
  * order of the bf16 MFMA. */
@@ -76,11 +78,16 @@ int flyhip_sb_kv_reduce(const void* k, const void* v, const float* proj, const i
  *   n_parts from flyhip_sb_plan (any value in [1,64] is valid); when > 1, part_ws is scratch of
  *   B*H*ceil(T/64)*n_parts*64*(D+5) floats and qfeat / q_lsq are the query-side outputs of
  *   flyhip_sb_kv_reduce for the same q; with n_parts == 1 all three may be NULL (the kernel forms
- *   the query features itself).  vt / kvt: the bf16 scratch of flyhip_sb_kv_reduce (NULL for fp32). */
+ *   the query features itself).  vt / kvt: the bf16 scratch of flyhip_sb_kv_reduce (NULL for fp32).
+ *   With n_parts > 1 the key pass has left its partial reductions uncombined: pass its kv_part,
+ *   part_max and n_split; extra workgroups of the band kernel's launch combine them into kv / ksum /
+ *   kmax (written here, read by the merge kernel that finishes the tiles).  With n_parts == 1 they
+ *   are ignored and kv / ksum / kmax are inputs. */
 int flyhip_sblocal_fwd(const void* q, const void* k, const void* v, const float* proj,
                        const void* kfeat, const float* chunk_scale,
-                       const float* kv, const float* ksum, const float* kmax,
+                       float* kv, float* ksum, float* kmax,
                        const float* qfeat, const float* q_lsq, const void* vt, const void* kvt,
+                       const float* kv_part, const float* part_max, int n_split,
                        const int64_t* key_lengths, void* out, float* log_norm,
                        float* part_ws, int n_parts,
                        int B, int H, int T, int S, int E, int D, int mh, int mh_valid,
