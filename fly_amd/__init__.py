@@ -9,6 +9,7 @@ from .local_attention import LocalAttention, local_forward
 from .blocksparse_utils import sparsify_tensor, densify_tensor, mask_tensor, sparsify_broadcast_tensor
 from .blocksparse_matmul import matmul
 from .blocksparse_softmax import softmax, logsumexp, blocksparse_sum
+from .blocksparse_fused import fused_attention
 from .blocksparse_attention import BlockSparseAttention
 from .sbblocksparse_attention import SBBlockSparseAttention
 from .blocksparse_linear import BlockSparseLinear, FlatBlockButterflySparsityConfig
@@ -18,7 +19,7 @@ from .t2t_vit import T2T_ViT, T2T_module, T2TAttention, Token_transformer, MlpCu
 __all__ = ['FullMask', 'LengthMask', 'TriangularCausalMask', 'SBPerformerFeatures',
            'gaussian_orthogonal_random_matrix', 'SBLocalAttention', 'sblocal_forward', 'LocalAttention', 'local_forward',
            'sparsify_tensor', 'densify_tensor', 'mask_tensor', 'sparsify_broadcast_tensor',
-           'matmul', 'softmax', 'logsumexp', 'blocksparse_sum', 'BlockSparseAttention',
+           'matmul', 'softmax', 'logsumexp', 'blocksparse_sum', 'BlockSparseAttention', 'fused_attention',
            'SBBlockSparseAttention',
            'BlockSparseLinear', 'FlatBlockButterflySparsityConfig', 'LowRank', 'SparseLRLinear',
            'T2T_ViT', 'T2T_module', 'T2TAttention', 'Token_transformer', 'MlpCustom', 't2t_vit_t_14']

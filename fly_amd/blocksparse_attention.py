@@ -8,6 +8,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 from torch import distributed as dist
 
+from .blocksparse_fused import fused_attention
 from .blocksparse_matmul import matmul
 from .blocksparse_softmax import softmax
 from .blocksparse_utils import densify_tensor
@@ -55,6 +56,10 @@ class BlockSparseAttention(nn.Module):
         self.register_buffer("master_layout", master_layout)
         self._need_layout_synchronization = True
         self.ops_cache = dict()
+        self.fused_cache = dict()
+        # forward passes that need neither gradients, attention weights, an attention mask nor
+        # dropout run as ONE kernel (no score tensor in memory); set to False to force the three ops
+        self.fuse = True
 
     def get_layout(self, T, S=None):
         if S is None:
@@ -104,6 +109,18 @@ class BlockSparseAttention(nn.Module):
         # contiguous (B,H,T,E) tensors at :130-132)
         q, k, v = (x.permute(0, 2, 1, 3) for x in (query, key, value))
         layout = self.get_layout(T, S)
+        needs_grad = torch.is_grad_enabled() and any(x.requires_grad for x in (query, key, value))
+        if (self.fuse and not need_weights and not needs_grad
+                and (attn_mask is None or attn_mask.all_ones)
+                and not (self.training and self.dropout.p > 0)
+                and fused_attention.supports(block, query.dtype, E, value.shape[3])):
+            if (T, S) not in self.fused_cache:
+                self.fused_cache[T, S] = fused_attention(layout, block)
+            key_mask = None
+            if key_padding_mask is not None and not key_padding_mask.all_ones:
+                key_mask = key_padding_mask.additive_matrix
+            out = self.fused_cache[T, S](q, k, v, softmax_temp, key_mask)
+            return out.permute(0, 2, 1, 3)[:, :q_seqlen_og, :, :v_dim_og], None
         sdd_nt, dsd_nn, sparse_softmax = self.get_ops(T, S)
         qk = sdd_nt(q, k)
         attn = sparse_softmax(qk, scale=softmax_temp,
@@ -112,7 +129,9 @@ class BlockSparseAttention(nn.Module):
                               key_padding_mask_mode='add', attn_mask_mode='add')
         if ((key_padding_mask is not None and not key_padding_mask.all_ones)
                 or (attn_mask is not None and not attn_mask.all_ones)):
-            attn.nan_to_num_()                                        # :156-158: fully masked rows -> 0
+            # :156-158: fully masked rows -> 0 (out of place under autograd: the softmax keeps its
+            # output for the backward pass)
+            attn = attn.nan_to_num() if attn.requires_grad else attn.nan_to_num_()
         out = dsd_nn(self.dropout(attn), v)
         weights = None
         if need_weights:

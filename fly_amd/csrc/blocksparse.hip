@@ -588,8 +588,6 @@ __global__ __launch_bounds__(256) void bs_dds_kernel(DxdArgs a) {
 // per input block the 128 x 32 activation tile and the group's 32g x 32 weight tile are staged in
 // LDS (registers hold the next step's tiles while the MFMAs of the current one run), the 2 x 2
 // waves own 64 x 64 outputs each and form them with 16x16x32 MFMAs.
-typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
-
 struct DdsGroupArgs {
     const void* sp; const void* dn; void* c;
     const int32_t* seg_ptr; const int32_t* seg_blk; const int32_t* seg_inner;
@@ -715,6 +713,186 @@ __global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
             if (ob >= gn) continue;
             store8_f32(cp + m * a.c_sm + (long)(bcol0 + ob) * 32 + 8 * g, acc[tm][2 * o2], acc[tm][2 * o2 + 1]);
         }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// fused block-sparse attention: out = softmax(scale * Q K^T + key mask) V over the nonzero blocks
+// ---------------------------------------------------------------------------------------
+// One pass for 32x32 blocks of a 2-byte type: the (Z, nnz, 32, 32) score and probability tensors of
+// the SDD -> softmax -> DSD sequence never exist.  One workgroup per (batch, head, NW consecutive
+// block-rows); wave w owns the 32 queries of block-row NW*group + w with their Q fragments in
+// registers.  The workgroup walks the union of the rows' column lists; each step stages one 32 x D
+// tile of K (row-major) and of V (transposed, [d][key slot]) in LDS, double-buffered, and every
+// wave whose row holds that column forms S^T = K Q^T (rows = keys, columns = queries: a lane then
+// owns one query per 16-column tile and its row statistics are lane scalars plus a 4-group
+// butterfly), runs the online softmax in base 2, and accumulates O^T += V^T P with the
+// probabilities going straight from the score registers into the MFMA operand: key 16kt + 4g + i
+// sits in contraction slot 8g + 4kt + i, which is the order the V tile is transposed into.
+struct AttnArgs {
+    const void* q; const void* k; const void* v; void* out;
+    const int32_t* uni_ptr; const int32_t* uni_inner; const int32_t* uni_blk;
+    const float* kpm; long kpm_stride;
+    int brows_per_head, grps_per_head, n_heads, Z;
+    long q_sz, q_sh, q_sm, k_sz, k_sh, k_sn, v_sz, v_sh, v_sn, o_sz, o_sh, o_sm;
+    float scale;
+};
+
+template <typename T> __device__ __forceinline__ uint32_t pack2(float lo, float hi);
+template <> __device__ __forceinline__ uint32_t pack2<bf16_t>(float lo, float hi) { return pack_bf16x2(lo, hi); }
+template <> __device__ __forceinline__ uint32_t pack2<f16_t>(float lo, float hi) {
+    const _Float16 l = (_Float16)lo, h = (_Float16)hi;
+    return (uint32_t)__builtin_bit_cast(uint16_t, l) | ((uint32_t)__builtin_bit_cast(uint16_t, h) << 16);
+}
+template <typename T> __device__ __forceinline__ floatx4 mma32(uintx4 a, uintx4 b, floatx4 c);
+template <> __device__ __forceinline__ floatx4 mma32<bf16_t>(uintx4 a, uintx4 b, floatx4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+template <> __device__ __forceinline__ floatx4 mma32<f16_t>(uintx4 a, uintx4 b, floatx4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(halfx8_t, a), __builtin_bit_cast(halfx8_t, b), c, 0, 0, 0);
+}
+
+constexpr int ATT_LDT = 40;     // LDS row stride of the transposed V tile in elements (32 slots + 8)
+
+template <typename T, int KS, int NW>     // head dim 32*KS, NW block-rows (waves) per workgroup
+__global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
+    constexpr int D = 32 * KS, LDK = D + 8, LDT = ATT_LDT, DT = D / 16, NTH = 64 * NW;
+    constexpr int CPR = D / 8;                            // 16-byte chunks per tile row
+    constexpr int NCH = (32 * CPR + NTH - 1) / NTH;       // chunks per thread
+    constexpr float LOG2E = 1.4426950408889634f;
+    __shared__ __attribute__((aligned(16))) uint16_t ks_[2][32 * LDK];
+    __shared__ __attribute__((aligned(16))) uint16_t vs_[2][D * LDT];
+    const int tid = threadIdx.x, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    int unit, grp;
+    if (!unit_of(blockIdx.x, a.grps_per_head, a.n_heads * a.Z, unit, grp)) return;
+    const int z = unit / a.n_heads, head = unit % a.n_heads;
+    const int ug = head * a.grps_per_head + grp;
+    const int p0 = a.uni_ptr[ug], n = a.uni_ptr[ug + 1] - p0;
+    const int bi = grp * NW + w;
+    const bool have_row = bi < a.brows_per_head;
+    const T* qp = reinterpret_cast<const T*>(a.q) + z * a.q_sz + head * a.q_sh +
+                  (long)(min(bi, a.brows_per_head - 1) * 32 + r16) * a.q_sm + 8 * g;
+    const T* kz = reinterpret_cast<const T*>(a.k) + z * a.k_sz + head * a.k_sh;
+    const T* vz = reinterpret_cast<const T*>(a.v) + z * a.v_sz + head * a.v_sh;
+    const float* kpm = a.kpm ? a.kpm + z * a.kpm_stride : nullptr;
+
+    uintx4 fq[2][KS];                                     // B operand: query 16qt + r16, dims 32ks + 8g ..
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) fq[qt][ks] = *reinterpret_cast<const uintx4*>(qp + 16 * qt * a.q_sm + 32 * ks);
+
+    uintx4 kreg[NCH], vreg[NCH];
+    auto fetch = [&](int s) __attribute__((always_inline)) {
+        const long row0 = (long)a.uni_inner[p0 + s] * 32;
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int c = tid + NTH * i;
+            if (c < 32 * CPR) {
+                kreg[i] = *reinterpret_cast<const uintx4*>(kz + (row0 + c / CPR) * a.k_sn + 8 * (c % CPR));
+                vreg[i] = *reinterpret_cast<const uintx4*>(vz + (row0 + c / CPR) * a.v_sn + 8 * (c % CPR));
+            }
+        }
+    };
+    auto stash = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int c = tid + NTH * i, row = c / CPR, ch = c % CPR;
+            if (c < 32 * CPR) {
+                *reinterpret_cast<uintx4*>(&ks_[buf][row * LDK + 8 * ch]) = kreg[i];
+                const int slot = 8 * ((row >> 2) & 3) + 4 * (row >> 4) + (row & 3);
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    vs_[buf][(8 * ch + e) * LDT + slot] = (uint16_t)(vreg[i][e >> 1] >> (16 * (e & 1)));
+            }
+        }
+    };
+
+    floatx4 o[DT][2];                                     // O^T[d = 16dt + 4g + i][query 16qt + r16]
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) { o[dt][0] = Frag<float>::zero(); o[dt][1] = Frag<float>::zero(); }
+    float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.f, 0.f};
+    const float scale2 = a.scale * LOG2E;
+
+    if (n > 0) {
+        fetch(0);
+        stash(0);
+    }
+    __syncthreads();
+    for (int s = 0; s < n; ++s) {
+        const bool present = have_row && a.uni_blk[(long)(p0 + s) * NW + w] >= 0;
+        if (s + 1 < n) fetch(s + 1);
+        if (present) {
+            const uint16_t* kp = ks_[s & 1];
+            const uint16_t* vp = vs_[s & 1];
+            uintx4 fk[2][KS];
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks)
+                    fk[kt][ks] = *reinterpret_cast<const uintx4*>(kp + (16 * kt + r16) * LDK + 32 * ks + 8 * g);
+            uintx4 fv[DT];
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) fv[dt] = *reinterpret_cast<const uintx4*>(vp + (16 * dt + r16) * LDT + 8 * g);
+            floatx4 sc[2][2];                             // S^T[key 16kt + 4g + i][query 16qt + r16]
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int qt = 0; qt < 2; ++qt) {
+                    sc[kt][qt] = Frag<float>::zero();
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) sc[kt][qt] = mma32<T>(fk[kt][ks], fq[qt][ks], sc[kt][qt]);
+                }
+            floatx4 mk[2] = {Frag<float>::zero(), Frag<float>::zero()};
+            if (kpm) {
+                const float* mp = kpm + (long)a.uni_inner[p0 + s] * 32 + 4 * g;
+                mk[0] = *reinterpret_cast<const floatx4*>(mp) * LOG2E;
+                mk[1] = *reinterpret_cast<const floatx4*>(mp + 16) * LOG2E;
+            }
+            uintx4 pb[2];
+#pragma unroll
+            for (int qt = 0; qt < 2; ++qt) {
+                floatx4 t0 = sc[0][qt] * scale2 + mk[0], t1 = sc[1][qt] * scale2 + mk[1];
+                float mx = fmaxf(fmaxf(fmaxf(t0[0], t0[1]), fmaxf(t0[2], t0[3])), fmaxf(fmaxf(t1[0], t1[1]), fmaxf(t1[2], t1[3])));
+                mx = group_max(mx);
+                if (__builtin_amdgcn_ballot_w64(mx > m_run[qt]) != 0) {      // wave-uniform: some row maximum grew
+                    const float m_new = fmaxf(m_run[qt], mx);
+                    const float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_run[qt] - m_new);
+                    m_run[qt] = m_new;
+                    l_run[qt] *= alpha;
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) o[dt][qt] *= alpha;
+                }
+                const float mref = (m_run[qt] == -INFINITY) ? 0.f : m_run[qt];     // all keys masked so far: p = 0
+                float p0_[4], p1_[4], sum = 0.f;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    p0_[i] = __builtin_amdgcn_exp2f(t0[i] - mref);
+                    p1_[i] = __builtin_amdgcn_exp2f(t1[i] - mref);
+                    sum += p0_[i] + p1_[i];
+                }
+                l_run[qt] += sum;
+                pb[qt] = uintx4{pack2<T>(p0_[0], p0_[1]), pack2<T>(p0_[2], p0_[3]), pack2<T>(p1_[0], p1_[1]), pack2<T>(p1_[2], p1_[3])};
+            }
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                o[dt][0] = mma32<T>(fv[dt], pb[0], o[dt][0]);
+                o[dt][1] = mma32<T>(fv[dt], pb[1], o[dt][1]);
+            }
+        }
+        if (s + 1 < n) stash((s + 1) & 1);
+        __syncthreads();
+    }
+    if (!have_row) return;
+    T* op = reinterpret_cast<T*>(a.out) + z * a.o_sz + head * a.o_sh;
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt) {
+        const float l = group_sum(l_run[qt]);
+        const float inv = l > 0.f ? 1.0f / l : 0.f;       // rows without a finite score come out as zeros
+        T* row = op + ((long)bi * 32 + 16 * qt + r16) * a.o_sm + 4 * g;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) store4_f32(row + 16 * dt, o[dt][qt] * inv);
     }
 }
 
@@ -1152,6 +1330,42 @@ static int launch_softmax(const RowArgs& args, dim3 grid, int max_elems, hipStre
     else if (max_elems <= 64 * 32) hipLaunchKernelGGL((bs_softmax_kernel<T, 32>), grid, dim3(256), 0, st, args);
     else hipLaunchKernelGGL((bs_softmax_long_kernel<T>), grid, dim3(256), 0, st, args);
     return check_launch("bs_softmax_kernel");
+}
+
+extern "C" int flyhip_bs_attn(const void* q, const void* k, const void* v, void* out,
+                              const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
+                              int rows_per_group, const float* key_mask, int64_t key_mask_stride,
+                              int Z, int H, int brows_per_head, int D, int blk,
+                              int64_t q_sz, int64_t q_sh, int64_t q_sm,
+                              int64_t k_sz, int64_t k_sh, int64_t k_sn,
+                              int64_t v_sz, int64_t v_sh, int64_t v_sn,
+                              int64_t o_sz, int64_t o_sh, int64_t o_sm,
+                              float scale, int dtype, void* stream) {
+    int rc = check_common("bs_attn", blk, dtype, Z);
+    if (rc) return rc;
+    FLY_REQUIRE(q && k && v && out && uni_ptr && uni_inner && uni_blk, "bs_attn: null pointer");
+    FLY_REQUIRE(blk == 32 && (dtype == BF16 || dtype == F16), "bs_attn: needs 32x32 blocks of bf16 / fp16 (got block %d, dtype %d)", blk, dtype);
+    FLY_REQUIRE(D == 32 || D == 64 || D == 128, "bs_attn: head dim %d not in {32,64,128}", D);
+    FLY_REQUIRE(rows_per_group == 4 || rows_per_group == 8, "bs_attn: rows_per_group must be 4 or 8");
+    FLY_REQUIRE(H > 0 && brows_per_head > 0, "bs_attn: bad sizes");
+    FLY_REQUIRE(((q_sz | q_sh | q_sm | k_sz | k_sh | k_sn | v_sz | v_sh | v_sn) % 8) == 0,
+                "bs_attn: q / k / v strides must be multiples of 8 elements");
+    FLY_REQUIRE(((o_sz | o_sh | o_sm) % 4) == 0, "bs_attn: out strides must be multiples of 4 elements");
+    FLY_REQUIRE(!key_mask || key_mask_stride % 4 == 0, "bs_attn: key mask stride must be a multiple of 4");
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    const int gph = (brows_per_head + rows_per_group - 1) / rows_per_group;
+    AttnArgs args{q, k, v, out, uni_ptr, uni_inner, uni_blk, key_mask, key_mask_stride, brows_per_head, gph, H, Z,
+                  q_sz, q_sh, q_sm, k_sz, k_sh, k_sn, v_sz, v_sh, v_sn, o_sz, o_sh, o_sm, scale};
+    const long nwg = unit_grid((long)H * Z, gph);
+    FLY_REQUIRE(nwg <= 2147483647L, "bs_attn: too many workgroups");
+    dim3 grid((unsigned)nwg);
+#define ATTN_LAUNCH(T, KS, NW) hipLaunchKernelGGL((bs_attn32_kernel<T, KS, NW>), grid, dim3(64 * NW), 0, st, args)
+#define ATTN_KS(T, NW) do { if (D == 32) ATTN_LAUNCH(T, 1, NW); else if (D == 64) ATTN_LAUNCH(T, 2, NW); else ATTN_LAUNCH(T, 4, NW); } while (0)
+    if (dtype == BF16) { if (rows_per_group == 4) ATTN_KS(bf16_t, 4); else ATTN_KS(bf16_t, 8); }
+    else { if (rows_per_group == 4) ATTN_KS(f16_t, 4); else ATTN_KS(f16_t, 8); }
+#undef ATTN_KS
+#undef ATTN_LAUNCH
+    return check_launch("bs_attn32_kernel");
 }
 
 extern "C" int flyhip_bs_softmax(void* x, const int32_t* row_ptr, const int32_t* row_blk, const int32_t* row_col,

@@ -41,6 +41,8 @@ typedef _Float16 halfx4 __attribute__((ext_vector_type(4)));
 
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef float floatx2 __attribute__((ext_vector_type(2)));
+// native 4 x 32-bit vector (arrays of HIP's uint4 struct do not always stay in registers)
+typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ float bf16_to_f32(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
 // two floats -> two bf16 in one 32-bit word (low half = first), round to nearest even in hardware

@@ -477,7 +477,6 @@ void sb_kfeat_kernel(KvArgs a) {
 // (two MFMAs per step; the split represents P to 2^-17).
 
 // ROWS x W tile of 2-byte elements, global -> registers -> LDS (rows clamped like RowTile)
-typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));   // a native vector: stays in registers as a struct member
 
 template <int ROWS, int W, int NT>
 struct Tile16 {

@@ -176,6 +176,27 @@ int flyhip_bs_dds(const void* a, const void* b_sp, void* c,
                   int64_t c_sz, int64_t c_sh, int64_t c_sm, int64_t c_sn,
                   int dtype, void* stream);
 
+/* Fused block-sparse attention: out = softmax(scale * q k^T + key mask) v over the nonzero blocks of
+ * the layout, in one pass -- the SDD -> block softmax -> DSD sequence of BlockSparseAttention.forward
+ * (ref: src/models/attention/blocksparse_attention.py:134-160) without the (Z, nnz, blk, blk) score
+ * and probability tensors.  32x32 blocks of bf16 / fp16 only; q (Z,H,rows,D), k / v (Z,H,cols,D),
+ * out (Z,H,rows,D) via (batch, head, row) strides with D contiguous, D in {32,64,128};
+ * rows = 32 * brows_per_head.  uni_ptr / uni_inner / uni_blk: the union table described at
+ * flyhip_bs_sdd built for groups of rows_per_group (4 or 8) consecutive block-rows (uni_blk is
+ * (n_union, rows_per_group); only its sign is used).  key_mask (optional, may be NULL): fp32
+ * (Z, cols) additive term per key (0 or -inf: the additive form of key_padding_mask,
+ * blocksparse_attention.py:148-150), row stride key_mask_stride.  A query whose keys are all
+ * masked, or whose block-row is empty, gets a zero row (the reference's nan_to_num_, :156-158). */
+int flyhip_bs_attn(const void* q, const void* k, const void* v, void* out,
+                   const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
+                   int rows_per_group, const float* key_mask, int64_t key_mask_stride,
+                   int Z, int H, int brows_per_head, int D, int blk,
+                   int64_t q_sz, int64_t q_sh, int64_t q_sm,
+                   int64_t k_sz, int64_t k_sh, int64_t k_sn,
+                   int64_t v_sz, int64_t v_sh, int64_t v_sn,
+                   int64_t o_sz, int64_t o_sh, int64_t o_sm,
+                   float scale, int dtype, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * Block-sparse row operations.  row_ptr (n_brow+1) / row_blk / row_col int32: for every
  * (head, block-row) the ids and block-columns of its nonzero blocks (the information of the

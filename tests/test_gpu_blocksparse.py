@@ -246,3 +246,86 @@ def test_sbblocksparse_attention_module(dtype, block):
     assert rel_err(ref_from_attn, ref_out) <= tol
     out2, none = layer(q.to(DEV), k.to(DEV), v.to(DEV))
     assert none is None and torch.equal(out2, out)
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('p,r,D,rpg', [(8, 8, 64, 4), (13, 9, 64, 8), (5, 7, 32, 8), (6, 6, 128, 4), (9, 12, 128, 8)])
+def test_fused_attention_matches_oracle(p, r, D, rpg, dtype):
+    """One-kernel attention against the oracle's SDD -> softmax -> nan_to_num -> DSD in fp64 and
+    against the three separate ops on the GPU; with an empty block-row, a key mask and queries
+    whose keys are all masked."""
+    from fly_amd import matmul, softmax
+    from fly_amd.blocksparse_fused import fused_attention
+    print('case', p, r, D, rpg, dtype, flush=True)
+    Z, H, block = 2, 3, 32
+    g = torch.Generator().manual_seed(100 * p + r)
+    layout = random_layout(H, p, r, p * r, density=0.4)
+    layout[1, min(2, p - 1), :] = 0                       # an empty block-row
+    layout[0, 0, :] = 0
+    layout[0, 0, 1] = 1                                   # a row whose only block is fully masked below
+    q = torch.randn(Z, p * 32, H, D, generator=g).to(dtype)
+    k = torch.randn(Z, r * 32, H, D, generator=g).to(dtype)
+    v = torch.randn(Z, r * 32, H, D, generator=g).to(dtype)
+    lens = torch.tensor([r * 32, 32])                     # batch 1 keeps only block-column 0
+    kpm = torch.log((torch.arange(r * 32).view(1, -1) < lens.view(Z, 1)).float())
+    scale = 0.31
+    qh, kh, vh = (x.permute(0, 2, 1, 3) for x in (q, k, v))
+    for mask in (None, kpm):
+        qk = ob.sdd(qh.double(), kh.double(), layout, block, trans_b=True)
+        pr = ob.block_softmax(qk, layout, block, scale=scale, key_padding_mask=mask).nan_to_num()
+        ref = ob.dsd(pr, vh.double(), layout, block)
+        op = fused_attention(layout, block, rows_per_group=rpg)
+        out = op(qh.to(DEV), kh.to(DEV), vh.to(DEV), scale, None if mask is None else mask.to(DEV))
+        assert out.shape == (Z, H, p * 32, D) and out.permute(0, 2, 1, 3).is_contiguous()
+        assert rel_err(out, ref) <= TOL[dtype]
+        assert float(out[:, 1, 32 * min(2, p - 1):32 * min(2, p - 1) + 32].abs().max()) == 0.0
+        if mask is not None:
+            assert float(out[1, 0, :32].abs().max()) == 0.0      # every key of that row is masked
+        # the three separate kernels give the same result up to their extra roundings
+        s3 = matmul(layout, block, 'sdd', trans_b=True)(qh.to(DEV), kh.to(DEV))
+        a3 = softmax(layout, block)(s3, scale=scale, key_padding_mask=None if mask is None else mask.to(DEV))
+        o3 = matmul(layout, block, 'dsd')(a3.nan_to_num_(), vh.to(DEV))
+        assert rel_err(out, o3.float()) <= 2 * TOL[dtype]
+
+
+def test_blocksparse_attention_module_fused_path():
+    """BlockSparseAttention.forward takes the one-kernel path for eligible calls (eval / no grad, no
+    attention mask) and the three-op path otherwise; both agree with the oracle, including padded
+    sequence lengths and head dims (:107-127)."""
+    from fly_amd import BlockSparseAttention, LengthMask
+
+    class Cfg:
+        block = 32
+
+        def make_layout(self, seqlen):
+            nb = seqlen // self.block
+            lay = ob.band_layout(nb, nb, 1)
+            lay[:, 0] = 1
+            return lay.unsqueeze(0).repeat(2, 1, 1)
+
+    B, T, S, H, E = 2, 300, 270, 2, 50
+    g = torch.Generator().manual_seed(5)
+    q = torch.randn(B, T, H, E, generator=g).bfloat16()
+    k = torch.randn(B, S, H, E, generator=g).bfloat16()
+    v = torch.randn(B, S, H, E, generator=g).bfloat16()
+    lengths = torch.tensor([S, 101])
+    mod = BlockSparseAttention(Cfg(), attention_dropout=0.0, max_seq_length=512).to(DEV)
+    ref = ob.blocksparse_attention(q.double(), k.double(), v.double(), mod.master_layout.cpu(), 32, key_lengths=lengths)
+    with torch.no_grad():
+        out, w = mod(q.to(DEV), k.to(DEV), v.to(DEV), key_padding_mask=LengthMask(lengths.to(DEV), max_len=S))
+    assert w is None and out.shape == (B, T, H, E)
+    assert len(mod.fused_cache) == 1 and len(mod.ops_cache) == 0        # the fused kernel ran
+    assert rel_err(out, ref) <= 2e-2
+    mod.fuse = False
+    out3, _ = mod(q.to(DEV), k.to(DEV), v.to(DEV), key_padding_mask=LengthMask(lengths.to(DEV), max_len=S))
+    assert len(mod.ops_cache) == 1
+    assert rel_err(out3, ref) <= 2e-2
+    assert rel_err(out, out3.float()) <= 2e-2
+    # a call that needs gradients keeps the differentiable three-op path
+    mod.fuse = True
+    mod.ops_cache.clear()
+    qg = q.to(DEV).requires_grad_()
+    outg, _ = mod(qg, k.to(DEV), v.to(DEV))
+    assert len(mod.ops_cache) == 1
+    outg.float().sum().backward()
+    assert qg.grad is not None and bool(torch.isfinite(qg.grad.float()).all())
