@@ -91,6 +91,12 @@ __device__ __forceinline__ bool unit_of(unsigned id, int per_unit, int n_units, 
     pos = (int)(slot % per_unit);
     return unit < n_units;
 }
+// Wait for every outstanding vector-memory load (vmcnt(0); the other counters are left alone).  Placed
+// in front of a pipelined loop it tells the compiler's wait-count bookkeeping that the operands
+// loaded before the loop have arrived; without it the loop body carries the first iteration's waits
+// for them, and those waits -- counters retire in order -- also drain the prefetch the body has
+// just issued, every iteration.
+__device__ __forceinline__ void drain_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 static long unit_grid(long n_units, long per_unit) { return (n_units + BS_XCD - 1) / BS_XCD * BS_XCD * per_unit; }
 
 struct SddRowArgs {
@@ -754,12 +760,17 @@ template <> __device__ __forceinline__ floatx4 mma32<f16_t>(uintx4 a, uintx4 b, 
 
 constexpr int ATT_LDT = 40;     // LDS row stride of the transposed V tile in elements (32 slots + 8)
 
-template <typename T, int KS, int NW>     // head dim 32*KS, NW block-rows (waves) per workgroup
+template <typename T, int KS, int NW, bool MASKED>     // head dim 32*KS, NW block-rows (waves) per workgroup
 __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
     constexpr int D = 32 * KS, LDK = D + 8, LDT = ATT_LDT, DT = D / 16, NTH = 64 * NW;
     constexpr int CPR = D / 8;                            // 16-byte chunks per tile row
-    constexpr int NCH = (32 * CPR + NTH - 1) / NTH;       // chunks per thread
+    constexpr int NCH = (64 * CPR + NTH - 1) / NTH;       // chunks per thread (K and V tiles together)
     constexpr float LOG2E = 1.4426950408889634f;
+    // The running reference exponent of a query is only raised (and its accumulators rescaled) when
+    // a block's maximum exceeds it by more than LAZY binary orders of magnitude; until then the
+    // probabilities may exceed 1 (by at most 2^LAZY), which fp32 sums and 2-byte operands hold
+    // without loss, and the result is the same quotient.
+    constexpr float LAZY = 8.f;
     __shared__ __attribute__((aligned(16))) uint16_t ks_[2][32 * LDK];
     __shared__ __attribute__((aligned(16))) uint16_t vs_[2][D * LDT];
     const int tid = threadIdx.x, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
@@ -783,28 +794,42 @@ __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) fq[qt][ks] = *reinterpret_cast<const uintx4*>(qp + 16 * qt * a.q_sm + 32 * ks);
 
-    uintx4 kreg[NCH], vreg[NCH];
-    auto fetch = [&](int s) __attribute__((always_inline)) {
-        const long row0 = (long)a.uni_inner[p0 + s] * 32;
+    // staging: chunk c = tid + NTH i (16 bytes).  The first 32 CPR chunks are the K tile, row-major
+    // (row c / CPR); the rest are the V tile with the key running fastest over the lanes (row c % 32),
+    // so that the 2-byte stores that transpose it spread over the LDS banks.
+    uintx4 reg[NCH];
+    const T* src[NCH];           // the chunk's address in block-column 0
+    long src_step[NCH];          // elements from one block-column to the next (wave-uniform)
+    int dst[NCH];                // the chunk's LDS position in buffer 0 (K: elements of ks_, V: of vs_)
 #pragma unroll
-        for (int i = 0; i < NCH; ++i) {
-            const int c = tid + NTH * i;
-            if (c < 32 * CPR) {
-                kreg[i] = *reinterpret_cast<const uintx4*>(kz + (row0 + c / CPR) * a.k_sn + 8 * (c % CPR));
-                vreg[i] = *reinterpret_cast<const uintx4*>(vz + (row0 + c / CPR) * a.v_sn + 8 * (c % CPR));
-            }
+    for (int i = 0; i < NCH; ++i) {
+        const int c = tid + NTH * i;
+        const bool is_k = 64 * w + NTH * i < 32 * CPR;      // whole waves stage K or V
+        if (is_k) {
+            src[i] = kz + (long)(c / CPR) * a.k_sn + 8 * (c % CPR);
+            src_step[i] = 32 * a.k_sn;
+            dst[i] = (c / CPR) * LDK + 8 * (c % CPR);
+        } else {
+            const int row = c & 31, ch = (c - 32 * CPR) >> 5;
+            src[i] = vz + (long)row * a.v_sn + 8 * ch;
+            src_step[i] = 32 * a.v_sn;
+            dst[i] = 8 * ch * LDT + 8 * ((row >> 2) & 3) + 4 * (row >> 4) + (row & 3);
         }
+    }
+    auto fetch = [&](int inner) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < NCH; ++i)
+            if (64 * w + NTH * i < 64 * CPR) reg[i] = *reinterpret_cast<const uintx4*>(src[i] + inner * src_step[i]);
     };
     auto stash = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < NCH; ++i) {
-            const int c = tid + NTH * i, row = c / CPR, ch = c % CPR;
-            if (c < 32 * CPR) {
-                *reinterpret_cast<uintx4*>(&ks_[buf][row * LDK + 8 * ch]) = kreg[i];
-                const int slot = 8 * ((row >> 2) & 3) + 4 * (row >> 4) + (row & 3);
+            if (64 * w + NTH * i < 32 * CPR) {
+                *reinterpret_cast<uintx4*>(&ks_[buf][dst[i]]) = reg[i];
+            } else if (64 * w + NTH * i < 64 * CPR) {
 #pragma unroll
                 for (int e = 0; e < 8; ++e)
-                    vs_[buf][(8 * ch + e) * LDT + slot] = (uint16_t)(vreg[i][e >> 1] >> (16 * (e & 1)));
+                    vs_[buf][dst[i] + e * LDT] = (uint16_t)(reg[i][e >> 1] >> (16 * (e & 1)));
             }
         }
     };
@@ -812,17 +837,27 @@ __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
     floatx4 o[DT][2];                                     // O^T[d = 16dt + 4g + i][query 16qt + r16]
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) { o[dt][0] = Frag<float>::zero(); o[dt][1] = Frag<float>::zero(); }
-    float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.f, 0.f};
+    float m_run[2] = {-INFINITY, -INFINITY};
+    floatx4 lsum[2] = {Frag<float>::zero(), Frag<float>::zero()};      // every element: sum of the query's probabilities
+    const uint32_t one2 = pack2<T>(1.f, 1.f);
+    const uintx4 ones = {one2, one2, one2, one2};
     const float scale2 = a.scale * LOG2E;
 
+    // the index lists are read two steps (block-column) and one step (presence) ahead of their use,
+    // so that no step waits for a table load
+    int inner_cur = n > 0 ? a.uni_inner[p0] : 0, inner_n1 = n > 1 ? a.uni_inner[p0 + 1] : 0;
+    int blk_cur = n > 0 ? a.uni_blk[(long)p0 * NW + w] : -1;
     if (n > 0) {
-        fetch(0);
+        fetch(inner_cur);
         stash(0);
     }
+    drain_loads();
     __syncthreads();
     for (int s = 0; s < n; ++s) {
-        const bool present = have_row && a.uni_blk[(long)(p0 + s) * NW + w] >= 0;
-        if (s + 1 < n) fetch(s + 1);
+        const int inner_n2 = s + 2 < n ? a.uni_inner[p0 + s + 2] : 0;
+        const int blk_n1 = s + 1 < n ? a.uni_blk[(long)(p0 + s + 1) * NW + w] : -1;
+        const bool present = have_row && blk_cur >= 0;
+        if (s + 1 < n) fetch(inner_n1);
         if (present) {
             const uint16_t* kp = ks_[s & 1];
             const uint16_t* vp = vs_[s & 1];
@@ -844,37 +879,67 @@ __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
 #pragma unroll
                     for (int ks = 0; ks < KS; ++ks) sc[kt][qt] = mma32<T>(fk[kt][ks], fq[qt][ks], sc[kt][qt]);
                 }
-            floatx4 mk[2] = {Frag<float>::zero(), Frag<float>::zero()};
-            if (kpm) {
-                const float* mp = kpm + (long)a.uni_inner[p0 + s] * 32 + 4 * g;
-                mk[0] = *reinterpret_cast<const floatx4*>(mp) * LOG2E;
-                mk[1] = *reinterpret_cast<const floatx4*>(mp + 16) * LOG2E;
-            }
             uintx4 pb[2];
+            if (!MASKED) {
+                // scale > 0 and no mask: the maximum is taken on the raw scores and the scale rides in
+                // the exponent's fma
 #pragma unroll
-            for (int qt = 0; qt < 2; ++qt) {
-                floatx4 t0 = sc[0][qt] * scale2 + mk[0], t1 = sc[1][qt] * scale2 + mk[1];
-                float mx = fmaxf(fmaxf(fmaxf(t0[0], t0[1]), fmaxf(t0[2], t0[3])), fmaxf(fmaxf(t1[0], t1[1]), fmaxf(t1[2], t1[3])));
-                mx = group_max(mx);
-                if (__builtin_amdgcn_ballot_w64(mx > m_run[qt]) != 0) {      // wave-uniform: some row maximum grew
-                    const float m_new = fmaxf(m_run[qt], mx);
-                    const float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_run[qt] - m_new);
-                    m_run[qt] = m_new;
-                    l_run[qt] *= alpha;
+                for (int qt = 0; qt < 2; ++qt) {
+                    const floatx4 s0 = sc[0][qt], s1 = sc[1][qt];
+                    float mx = fmaxf(fmaxf(fmaxf(s0[0], s0[1]), s0[2]), fmaxf(fmaxf(s0[3], s1[0]), s1[1]));
+                    mx = fmaxf(fmaxf(mx, s1[2]), s1[3]);
+                    mx = group_max(mx) * scale2;
+                    if (__builtin_amdgcn_ballot_w64(mx > m_run[qt] + LAZY) != 0) {      // wave-uniform: some row maximum grew a lot
+                        const float m_new = fmaxf(m_run[qt], mx);
+                        const float alpha = __builtin_amdgcn_exp2f(m_run[qt] - m_new);
+                        m_run[qt] = m_new;
+                        lsum[qt] *= alpha;
 #pragma unroll
-                    for (int dt = 0; dt < DT; ++dt) o[dt][qt] *= alpha;
+                        for (int dt = 0; dt < DT; ++dt) o[dt][qt] *= alpha;
+                    }
+                    const float nm = -m_run[qt];
+                    float e0[4], e1[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        e0[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s0[i], scale2, nm));
+                        e1[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s1[i], scale2, nm));
+                    }
+                    pb[qt] = uintx4{pack2<T>(e0[0], e0[1]), pack2<T>(e0[2], e0[3]), pack2<T>(e1[0], e1[1]), pack2<T>(e1[2], e1[3])};
                 }
-                const float mref = (m_run[qt] == -INFINITY) ? 0.f : m_run[qt];     // all keys masked so far: p = 0
-                float p0_[4], p1_[4], sum = 0.f;
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    p0_[i] = __builtin_amdgcn_exp2f(t0[i] - mref);
-                    p1_[i] = __builtin_amdgcn_exp2f(t1[i] - mref);
-                    sum += p0_[i] + p1_[i];
+            } else {
+                floatx4 mk[2] = {Frag<float>::zero(), Frag<float>::zero()};
+                if (kpm) {
+                    const float* mp = kpm + (long)inner_cur * 32 + 4 * g;
+                    mk[0] = *reinterpret_cast<const floatx4*>(mp) * LOG2E;
+                    mk[1] = *reinterpret_cast<const floatx4*>(mp + 16) * LOG2E;
                 }
-                l_run[qt] += sum;
-                pb[qt] = uintx4{pack2<T>(p0_[0], p0_[1]), pack2<T>(p0_[2], p0_[3]), pack2<T>(p1_[0], p1_[1]), pack2<T>(p1_[2], p1_[3])};
+#pragma unroll
+                for (int qt = 0; qt < 2; ++qt) {
+                    const floatx4 t0 = sc[0][qt] * scale2 + mk[0], t1 = sc[1][qt] * scale2 + mk[1];
+                    float mx = fmaxf(fmaxf(fmaxf(t0[0], t0[1]), t0[2]), fmaxf(fmaxf(t0[3], t1[0]), t1[1]));
+                    mx = fmaxf(fmaxf(mx, t1[2]), t1[3]);
+                    mx = group_max(mx);
+                    if (__builtin_amdgcn_ballot_w64(mx > m_run[qt] + LAZY) != 0) {
+                        const float m_new = fmaxf(m_run[qt], mx);
+                        const float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_run[qt] - m_new);
+                        m_run[qt] = m_new;
+                        lsum[qt] *= alpha;
+#pragma unroll
+                        for (int dt = 0; dt < DT; ++dt) o[dt][qt] *= alpha;
+                    }
+                    const float mref = (m_run[qt] == -INFINITY) ? 0.f : m_run[qt];     // all keys masked so far: p = 0
+                    float e0[4], e1[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        e0[i] = __builtin_amdgcn_exp2f(t0[i] - mref);
+                        e1[i] = __builtin_amdgcn_exp2f(t1[i] - mref);
+                    }
+                    pb[qt] = uintx4{pack2<T>(e0[0], e0[1]), pack2<T>(e0[2], e0[3]), pack2<T>(e1[0], e1[1]), pack2<T>(e1[2], e1[3])};
+                }
             }
+            // the row sums come from the matrix pipe as well: a row of ones times the rounded probabilities
+            lsum[0] = mma32<T>(ones, pb[0], lsum[0]);
+            lsum[1] = mma32<T>(ones, pb[1], lsum[1]);
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
                 o[dt][0] = mma32<T>(fv[dt], pb[0], o[dt][0]);
@@ -882,13 +947,16 @@ __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
             }
         }
         if (s + 1 < n) stash((s + 1) & 1);
+        inner_cur = inner_n1;
+        inner_n1 = inner_n2;
+        blk_cur = blk_n1;
         __syncthreads();
     }
     if (!have_row) return;
     T* op = reinterpret_cast<T*>(a.out) + z * a.o_sz + head * a.o_sh;
 #pragma unroll
     for (int qt = 0; qt < 2; ++qt) {
-        const float l = group_sum(l_run[qt]);
+        const float l = lsum[qt][0];
         const float inv = l > 0.f ? 1.0f / l : 0.f;       // rows without a finite score come out as zeros
         T* row = op + ((long)bi * 32 + 16 * qt + r16) * a.o_sm + 4 * g;
 #pragma unroll
@@ -1359,7 +1427,12 @@ extern "C" int flyhip_bs_attn(const void* q, const void* k, const void* v, void*
     const long nwg = unit_grid((long)H * Z, gph);
     FLY_REQUIRE(nwg <= 2147483647L, "bs_attn: too many workgroups");
     dim3 grid((unsigned)nwg);
-#define ATTN_LAUNCH(T, KS, NW) hipLaunchKernelGGL((bs_attn32_kernel<T, KS, NW>), grid, dim3(64 * NW), 0, st, args)
+    const bool masked = key_mask != nullptr || !(scale > 0.f);
+#define ATTN_LAUNCH(T, KS, NW)                                                                                  \
+    do {                                                                                                        \
+        if (masked) hipLaunchKernelGGL((bs_attn32_kernel<T, KS, NW, true>), grid, dim3(64 * NW), 0, st, args);  \
+        else hipLaunchKernelGGL((bs_attn32_kernel<T, KS, NW, false>), grid, dim3(64 * NW), 0, st, args);        \
+    } while (0)
 #define ATTN_KS(T, NW) do { if (D == 32) ATTN_LAUNCH(T, 1, NW); else if (D == 64) ATTN_LAUNCH(T, 2, NW); else ATTN_LAUNCH(T, 4, NW); } while (0)
     if (dtype == BF16) { if (rows_per_group == 4) ATTN_KS(bf16_t, 4); else ATTN_KS(bf16_t, 8); }
     else { if (rows_per_group == 4) ATTN_KS(f16_t, 4); else ATTN_KS(f16_t, 8); }
