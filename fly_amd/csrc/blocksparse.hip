@@ -758,6 +758,21 @@ template <> __device__ __forceinline__ floatx4 mma32<f16_t>(uintx4 a, uintx4 b, 
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(halfx8_t, a), __builtin_bit_cast(halfx8_t, b), c, 0, 0, 0);
 }
 
+// Maxima of scores.  A two-operand fmaxf costs three instructions here (each operand is first quieted
+// by a self-maximum); three-operand maxima are emitted as they are, so pairs get -inf as a third.
+__device__ __forceinline__ float max2_finite(float a, float b) { return fmaxf(fmaxf(a, b), -INFINITY); }
+__device__ __forceinline__ float max8_finite(floatx4 a, floatx4 b) {
+    const float m0 = fmaxf(fmaxf(a[0], a[1]), a[2]);
+    const float m1 = fmaxf(fmaxf(m0, a[3]), b[0]);
+    const float m2 = fmaxf(fmaxf(m1, b[1]), b[2]);
+    return max2_finite(m2, b[3]);
+}
+__device__ __forceinline__ float group_max_finite(float v) {
+    float a, b;
+    rows_pair16(v, a, b); v = max2_finite(a, b);
+    rows_pair32(v, a, b); return max2_finite(a, b);
+}
+
 constexpr int ATT_LDT = 40;     // LDS row stride of the transposed V tile in elements (32 slots + 8)
 
 template <typename T, int KS, int NW, bool MASKED>     // head dim 32*KS, NW block-rows (waves) per workgroup
@@ -772,7 +787,7 @@ __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
     // without loss, and the result is the same quotient.
     constexpr float LAZY = 8.f;
     __shared__ __attribute__((aligned(16))) uint16_t ks_[2][32 * LDK];
-    __shared__ __attribute__((aligned(16))) uint16_t vs_[2][D * LDT];
+    __shared__ __attribute__((aligned(16))) uint16_t vs_[3][D * LDT];
     const int tid = threadIdx.x, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     int unit, grp;
@@ -821,15 +836,15 @@ __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
         for (int i = 0; i < NCH; ++i)
             if (64 * w + NTH * i < 64 * CPR) reg[i] = *reinterpret_cast<const uintx4*>(src[i] + inner * src_step[i]);
     };
-    auto stash = [&](int buf) __attribute__((always_inline)) {
+    auto stash = [&](int kbuf, int vbuf) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < NCH; ++i) {
             if (64 * w + NTH * i < 32 * CPR) {
-                *reinterpret_cast<uintx4*>(&ks_[buf][dst[i]]) = reg[i];
+                *reinterpret_cast<uintx4*>(&ks_[kbuf][dst[i]]) = reg[i];
             } else if (64 * w + NTH * i < 64 * CPR) {
 #pragma unroll
                 for (int e = 0; e < 8; ++e)
-                    vs_[buf][dst[i] + e * LDT] = (uint16_t)(reg[i][e >> 1] >> (16 * (e & 1)));
+                    vs_[vbuf][dst[i] + e * LDT] = (uint16_t)(reg[i][e >> 1] >> (16 * (e & 1)));
             }
         }
     };
@@ -843,114 +858,138 @@ __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
     const uintx4 ones = {one2, one2, one2, one2};
     const float scale2 = a.scale * LOG2E;
 
-    // the index lists are read two steps (block-column) and one step (presence) ahead of their use,
-    // so that no step waits for a table load
-    int inner_cur = n > 0 ? a.uni_inner[p0] : 0, inner_n1 = n > 1 ? a.uni_inner[p0 + 1] : 0;
+    // S^T[key 16kt + 4g + i][query 16qt + r16] of the tile in K buffer `buf`
+    floatx4 sc[2][2];
+    auto score = [&](int buf) __attribute__((always_inline)) {
+        const uint16_t* kp = ks_[buf];
+        uintx4 fk[2][KS];
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+                fk[kt][ks] = *reinterpret_cast<const uintx4*>(kp + (16 * kt + r16) * LDK + 32 * ks + 8 * g);
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+            for (int qt = 0; qt < 2; ++qt) {
+                sc[kt][qt] = Frag<float>::zero();
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) sc[kt][qt] = mma32<T>(fk[kt][ks], fq[qt][ks], sc[kt][qt]);
+            }
+    };
+    // online softmax of sc and O^T += V^T P with the tile in V buffer `buf`; `inner` = its block-column
+    auto soft_pv = [&](int buf, int inner) __attribute__((always_inline)) {
+        const uint16_t* vp = vs_[buf];
+        uintx4 fv[DT];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) fv[dt] = *reinterpret_cast<const uintx4*>(vp + (16 * dt + r16) * LDT + 8 * g);
+        uintx4 pb[2];
+        if (!MASKED) {
+            // scale > 0 and no mask: the maximum is taken on the raw scores and the scale rides in
+            // the exponent's fma
+#pragma unroll
+            for (int qt = 0; qt < 2; ++qt) {
+                const floatx4 s0 = sc[0][qt], s1 = sc[1][qt];
+                const float mx = group_max_finite(max8_finite(s0, s1)) * scale2;
+                if (__builtin_amdgcn_ballot_w64(mx > m_run[qt] + LAZY) != 0) {      // wave-uniform: some row maximum grew a lot
+                    const float m_new = fmaxf(m_run[qt], mx);
+                    const float alpha = __builtin_amdgcn_exp2f(m_run[qt] - m_new);
+                    m_run[qt] = m_new;
+                    lsum[qt] *= alpha;
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) o[dt][qt] *= alpha;
+                }
+                const float nm = -m_run[qt];
+                float e0[4], e1[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    e0[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s0[i], scale2, nm));
+                    e1[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s1[i], scale2, nm));
+                }
+                pb[qt] = uintx4{pack2<T>(e0[0], e0[1]), pack2<T>(e0[2], e0[3]), pack2<T>(e1[0], e1[1]), pack2<T>(e1[2], e1[3])};
+            }
+        } else {
+            floatx4 mk[2] = {Frag<float>::zero(), Frag<float>::zero()};
+            if (kpm) {
+                const float* mp = kpm + (long)inner * 32 + 4 * g;
+                mk[0] = *reinterpret_cast<const floatx4*>(mp) * LOG2E;
+                mk[1] = *reinterpret_cast<const floatx4*>(mp + 16) * LOG2E;
+            }
+#pragma unroll
+            for (int qt = 0; qt < 2; ++qt) {
+                const floatx4 t0 = sc[0][qt] * scale2 + mk[0], t1 = sc[1][qt] * scale2 + mk[1];
+                float mx = fmaxf(fmaxf(fmaxf(t0[0], t0[1]), t0[2]), fmaxf(fmaxf(t0[3], t1[0]), t1[1]));
+                mx = fmaxf(fmaxf(mx, t1[2]), t1[3]);
+                mx = group_max(mx);
+                if (__builtin_amdgcn_ballot_w64(mx > m_run[qt] + LAZY) != 0) {
+                    const float m_new = fmaxf(m_run[qt], mx);
+                    const float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_run[qt] - m_new);
+                    m_run[qt] = m_new;
+                    lsum[qt] *= alpha;
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) o[dt][qt] *= alpha;
+                }
+                const float mref = (m_run[qt] == -INFINITY) ? 0.f : m_run[qt];     // all keys masked so far: p = 0
+                float e0[4], e1[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    e0[i] = __builtin_amdgcn_exp2f(t0[i] - mref);
+                    e1[i] = __builtin_amdgcn_exp2f(t1[i] - mref);
+                }
+                pb[qt] = uintx4{pack2<T>(e0[0], e0[1]), pack2<T>(e0[2], e0[3]), pack2<T>(e1[0], e1[1]), pack2<T>(e1[2], e1[3])};
+            }
+        }
+        // the row sums come from the matrix pipe as well: a row of ones times the rounded probabilities
+        lsum[0] = mma32<T>(ones, pb[0], lsum[0]);
+        lsum[1] = mma32<T>(ones, pb[1], lsum[1]);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            o[dt][0] = mma32<T>(fv[dt], pb[0], o[dt][0]);
+            o[dt][1] = mma32<T>(fv[dt], pb[1], o[dt][1]);
+        }
+    };
+
+    // The index lists are read two steps (block-column) and one step (presence) ahead of their use,
+    // so that no step waits for a table load.
+    // The upper half of the waves runs half a step behind the lower half: in iteration s an early
+    // wave does scores(s), softmax(s), PV(s); a late wave does softmax(s-1), PV(s-1), scores(s).
+    // A SIMD holds one wave of each kind per workgroup, so one's matrix phase coincides with the
+    // other's vector phase instead of both queueing for the same pipe.  K tiles are double-buffered,
+    // V tiles (still read one iteration later by the late waves) triple-buffered.
+    const bool late = w >= NW / 2;
+    int inner_cur = n > 0 ? a.uni_inner[p0] : 0, inner_n1 = n > 1 ? a.uni_inner[p0 + 1] : 0, inner_prev = 0;
     int blk_cur = n > 0 ? a.uni_blk[(long)p0 * NW + w] : -1;
+    bool had_prev = false;
     if (n > 0) {
         fetch(inner_cur);
-        stash(0);
+        stash(0, 0);
     }
     drain_loads();
     __syncthreads();
-    for (int s = 0; s < n; ++s) {
+    int vb = 0;                                           // V buffer of step s (s % 3)
+    for (int s = 0; s <= n; ++s) {
         const int inner_n2 = s + 2 < n ? a.uni_inner[p0 + s + 2] : 0;
         const int blk_n1 = s + 1 < n ? a.uni_blk[(long)(p0 + s + 1) * NW + w] : -1;
-        const bool present = have_row && blk_cur >= 0;
+        const bool present = s < n && have_row && blk_cur >= 0;
+        const int vb_next = vb == 2 ? 0 : vb + 1, vb_prev = vb == 0 ? 2 : vb - 1;
+#ifndef ATT_NOSTAGE
         if (s + 1 < n) fetch(inner_n1);
-        if (present) {
-            const uint16_t* kp = ks_[s & 1];
-            const uint16_t* vp = vs_[s & 1];
-            uintx4 fk[2][KS];
-#pragma unroll
-            for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-                for (int ks = 0; ks < KS; ++ks)
-                    fk[kt][ks] = *reinterpret_cast<const uintx4*>(kp + (16 * kt + r16) * LDK + 32 * ks + 8 * g);
-            uintx4 fv[DT];
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) fv[dt] = *reinterpret_cast<const uintx4*>(vp + (16 * dt + r16) * LDT + 8 * g);
-            floatx4 sc[2][2];                             // S^T[key 16kt + 4g + i][query 16qt + r16]
-#pragma unroll
-            for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-                for (int qt = 0; qt < 2; ++qt) {
-                    sc[kt][qt] = Frag<float>::zero();
-#pragma unroll
-                    for (int ks = 0; ks < KS; ++ks) sc[kt][qt] = mma32<T>(fk[kt][ks], fq[qt][ks], sc[kt][qt]);
-                }
-            uintx4 pb[2];
-            if (!MASKED) {
-                // scale > 0 and no mask: the maximum is taken on the raw scores and the scale rides in
-                // the exponent's fma
-#pragma unroll
-                for (int qt = 0; qt < 2; ++qt) {
-                    const floatx4 s0 = sc[0][qt], s1 = sc[1][qt];
-                    float mx = fmaxf(fmaxf(fmaxf(s0[0], s0[1]), s0[2]), fmaxf(fmaxf(s0[3], s1[0]), s1[1]));
-                    mx = fmaxf(fmaxf(mx, s1[2]), s1[3]);
-                    mx = group_max(mx) * scale2;
-                    if (__builtin_amdgcn_ballot_w64(mx > m_run[qt] + LAZY) != 0) {      // wave-uniform: some row maximum grew a lot
-                        const float m_new = fmaxf(m_run[qt], mx);
-                        const float alpha = __builtin_amdgcn_exp2f(m_run[qt] - m_new);
-                        m_run[qt] = m_new;
-                        lsum[qt] *= alpha;
-#pragma unroll
-                        for (int dt = 0; dt < DT; ++dt) o[dt][qt] *= alpha;
-                    }
-                    const float nm = -m_run[qt];
-                    float e0[4], e1[4];
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        e0[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s0[i], scale2, nm));
-                        e1[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s1[i], scale2, nm));
-                    }
-                    pb[qt] = uintx4{pack2<T>(e0[0], e0[1]), pack2<T>(e0[2], e0[3]), pack2<T>(e1[0], e1[1]), pack2<T>(e1[2], e1[3])};
-                }
-            } else {
-                floatx4 mk[2] = {Frag<float>::zero(), Frag<float>::zero()};
-                if (kpm) {
-                    const float* mp = kpm + (long)inner_cur * 32 + 4 * g;
-                    mk[0] = *reinterpret_cast<const floatx4*>(mp) * LOG2E;
-                    mk[1] = *reinterpret_cast<const floatx4*>(mp + 16) * LOG2E;
-                }
-#pragma unroll
-                for (int qt = 0; qt < 2; ++qt) {
-                    const floatx4 t0 = sc[0][qt] * scale2 + mk[0], t1 = sc[1][qt] * scale2 + mk[1];
-                    float mx = fmaxf(fmaxf(fmaxf(t0[0], t0[1]), t0[2]), fmaxf(fmaxf(t0[3], t1[0]), t1[1]));
-                    mx = fmaxf(fmaxf(mx, t1[2]), t1[3]);
-                    mx = group_max(mx);
-                    if (__builtin_amdgcn_ballot_w64(mx > m_run[qt] + LAZY) != 0) {
-                        const float m_new = fmaxf(m_run[qt], mx);
-                        const float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_run[qt] - m_new);
-                        m_run[qt] = m_new;
-                        lsum[qt] *= alpha;
-#pragma unroll
-                        for (int dt = 0; dt < DT; ++dt) o[dt][qt] *= alpha;
-                    }
-                    const float mref = (m_run[qt] == -INFINITY) ? 0.f : m_run[qt];     // all keys masked so far: p = 0
-                    float e0[4], e1[4];
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        e0[i] = __builtin_amdgcn_exp2f(t0[i] - mref);
-                        e1[i] = __builtin_amdgcn_exp2f(t1[i] - mref);
-                    }
-                    pb[qt] = uintx4{pack2<T>(e0[0], e0[1]), pack2<T>(e0[2], e0[3]), pack2<T>(e1[0], e1[1]), pack2<T>(e1[2], e1[3])};
-                }
-            }
-            // the row sums come from the matrix pipe as well: a row of ones times the rounded probabilities
-            lsum[0] = mma32<T>(ones, pb[0], lsum[0]);
-            lsum[1] = mma32<T>(ones, pb[1], lsum[1]);
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                o[dt][0] = mma32<T>(fv[dt], pb[0], o[dt][0]);
-                o[dt][1] = mma32<T>(fv[dt], pb[1], o[dt][1]);
-            }
-        }
-        if (s + 1 < n) stash((s + 1) & 1);
+#endif
+        if (late && had_prev) soft_pv(vb_prev, inner_prev);
+        if (present) score(s & 1);
+        if (!late && present) soft_pv(vb, inner_cur);
+#ifndef ATT_NOSTAGE
+        if (s + 1 < n) stash((s + 1) & 1, vb_next);
+#endif
+        had_prev = present;
+        inner_prev = inner_cur;
         inner_cur = inner_n1;
         inner_n1 = inner_n2;
         blk_cur = blk_n1;
+        vb = vb_next;
+#ifndef ATT_NOBAR
         __syncthreads();
+#endif
     }
     if (!have_row) return;
     T* op = reinterpret_cast<T*>(a.out) + z * a.o_sz + head * a.o_sh;
