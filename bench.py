@@ -168,6 +168,18 @@ def bench_blocksparse(steps, warmup):
     out['dsd'] = {'ms': ms, 'tflops': flops / ms / 1e9, 'gbs': (sp_bytes + 2 * dense_bytes) / ms / 1e6}
     for st in out.values():
         st['hbm_frac'] = st['gbs'] / PEAK_HBM_GBS
+    # the three stages as separate launches, and the one-kernel form BlockSparseAttention.forward uses
+    # when it needs no gradients, weights or attention mask (same inputs, same result)
+    from fly_amd import fused_attention
+    fused = fused_attention(layout, block)
+    ms3 = timeit(lambda: dsd(sm(sdd(q, k), scale=0.125), v))
+    ref = dsd(sm(sdd(q, k), scale=0.125), v).float()
+    got = fused(q, k, v, 0.125).float()
+    ms = timeit(lambda: fused(q, k, v, 0.125))
+    out['three_stage_attention_ms'] = ms3
+    out['fused_attention'] = {'ms': ms, 'tflops': 2 * flops / ms / 1e9, 'mfma_bf16_frac': 2 * flops / ms / 1e9 / 2500.0,
+                              'speedup_over_three_stages': ms3 / ms,
+                              'max_diff_vs_three_stages': float((got - ref).abs().max() / ref.abs().max())}
     # what a plain device copy of the sparse tensor reaches on this box (read + write bytes per second)
     dst = torch.empty_like(qk)
     ms = timeit(lambda: dst.copy_(qk))

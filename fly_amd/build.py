@@ -9,9 +9,12 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, 'csrc')
 LIB = os.path.join(HERE, 'libflyhip.so')
 SOURCES = ['api.cpp', 'sblocal.hip', 'blocksparse.hip']
-# packed-fp32 VALU forms are switched off for every kernel of this library
+# packed-fp32 VALU forms are switched off for every kernel of this library; MFMA accumulators stay in
+# ordinary VGPRs (the softmax arithmetic reads them between products, and every trip through the
+# accumulation registers costs a move per value)
 FLAGS = ['--offload-arch=gfx950', '-O3', '-fPIC', '-std=c++17',
-         '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops']
+         '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
+         '-mllvm', '-amdgpu-mfma-vgpr-form=1']
 
 
 def _hipcc():

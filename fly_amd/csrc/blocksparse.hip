@@ -99,6 +99,20 @@ __device__ __forceinline__ bool unit_of(unsigned id, int per_unit, int n_units, 
 __device__ __forceinline__ void drain_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 static long unit_grid(long n_units, long per_unit) { return (n_units + BS_XCD - 1) / BS_XCD * BS_XCD * per_unit; }
 
+template <typename T> __device__ __forceinline__ uint32_t pack2(float lo, float hi);
+template <> __device__ __forceinline__ uint32_t pack2<bf16_t>(float lo, float hi) { return pack_bf16x2(lo, hi); }
+template <> __device__ __forceinline__ uint32_t pack2<f16_t>(float lo, float hi) {
+    const _Float16 l = (_Float16)lo, h = (_Float16)hi;
+    return (uint32_t)__builtin_bit_cast(uint16_t, l) | ((uint32_t)__builtin_bit_cast(uint16_t, h) << 16);
+}
+template <typename T> __device__ __forceinline__ floatx4 mma32(uintx4 a, uintx4 b, floatx4 c);
+template <> __device__ __forceinline__ floatx4 mma32<bf16_t>(uintx4 a, uintx4 b, floatx4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+template <> __device__ __forceinline__ floatx4 mma32<f16_t>(uintx4 a, uintx4 b, floatx4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(halfx8_t, a), __builtin_bit_cast(halfx8_t, b), c, 0, 0, 0);
+}
+
 struct SddRowArgs {
     const void* a; const void* b; void* c;
     const int32_t* row_ptr; const int32_t* row_blk; const int32_t* row_col;
@@ -201,62 +215,74 @@ __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
                   (long)(min(bi, a.brows_per_head - 1) * 32 + r16) * a.a_sm + 8 * g;
     const T* bz = reinterpret_cast<const T*>(a.b) + z * a.b_sz + head * a.b_sh;
     T* cz = reinterpret_cast<T*>(a.c) + (long)z * a.nnz * 1024;
-    uint4 fa[2][KS];
+    uintx4 fa[2][KS];
 #pragma unroll
     for (int tm = 0; tm < 2; ++tm)
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) fa[tm][ks] = *reinterpret_cast<const uint4*>(ap + 16 * tm * a.a_sm + 32 * ks);
+        for (int ks = 0; ks < KS; ++ks) fa[tm][ks] = *reinterpret_cast<const uintx4*>(ap + 16 * tm * a.a_sm + 32 * ks);
 
     // staging: chunk c = tid + 256 i is 16 bytes of tile row c / CPR.  Block column n lands in LDS row
     // 16*((n>>2)&1) + 4*(n>>3) + (n&3), so that MFMA tile tn reads the 16 consecutive LDS rows
     // 16 tn .. 16 tn + 15 and its row i is block column 8*(i/4) + 4*tn + i%4: the four results a lane
     // gets from tile 0 and the four from tile 1 are eight consecutive columns -> one 16-byte store
-    uint4 reg[NCH];
-    auto fetch = [&](int s) {
-        const long brow_b = (long)a.uni_inner[p0 + s] * 32;
+    uintx4 reg[NCH];
+    auto fetch = [&](int inner) __attribute__((always_inline)) {
+        const long brow_b = (long)inner * 32;
 #pragma unroll
         for (int i = 0; i < NCH; ++i) {
             const int c = tid + 256 * i;
-            if (c < 32 * CPR) reg[i] = *reinterpret_cast<const uint4*>(bz + (brow_b + c / CPR) * a.b_sn + 8 * (c % CPR));
+            if (c < 32 * CPR) reg[i] = *reinterpret_cast<const uintx4*>(bz + (brow_b + c / CPR) * a.b_sn + 8 * (c % CPR));
         }
     };
-    auto stash = [&](int buf) {
+    auto stash = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < NCH; ++i) {
             const int c = tid + 256 * i, nrow = c / CPR;
             const int lrow = 16 * ((nrow >> 2) & 1) + 4 * (nrow >> 3) + (nrow & 3);
-            if (c < 32 * CPR) *reinterpret_cast<uint4*>(&tile[buf][lrow * LD + 8 * (c % CPR)]) = reg[i];
+            if (c < 32 * CPR) *reinterpret_cast<uintx4*>(&tile[buf][lrow * LD + 8 * (c % CPR)]) = reg[i];
         }
     };
-    fetch(0);
+    // the index lists are read two steps (block-column) and one step (block id) ahead of their use
+    int inner_n1 = n > 1 ? a.uni_inner[p0 + 1] : 0;
+    int blk = a.uni_blk[(long)p0 * 4 + w];
+    fetch(a.uni_inner[p0]);
     stash(0);
+    drain_loads();
     __syncthreads();
     for (int s = 0; s < n; ++s) {
-        const int blk = a.uni_blk[(long)(p0 + s) * 4 + w];
-        if (s + 1 < n) fetch(s + 1);
-        if (blk >= 0 && have_row) {
+        const int inner_n2 = s + 2 < n ? a.uni_inner[p0 + s + 2] : 0;
+        const int blk_n1 = s + 1 < n ? a.uni_blk[(long)(p0 + s + 1) * 4 + w] : -1;
+        if (s + 1 < n) fetch(inner_n1);
+        const bool mine = blk >= 0 && have_row;
+        floatx4 acc[2][2];
+        if (mine) {
             const uint16_t* tp = tile[s & 1];
-            floatx4 acc[2][2];
-            uint4 fb[2][KS];
+            uintx4 fb[2][KS];
 #pragma unroll
             for (int tn = 0; tn < 2; ++tn)
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks)
-                    fb[tn][ks] = *reinterpret_cast<const uint4*>(tp + (16 * tn + r16) * LD + 32 * ks + 8 * g);
+                    fb[tn][ks] = *reinterpret_cast<const uintx4*>(tp + (16 * tn + r16) * LD + 32 * ks + 8 * g);
 #pragma unroll
             for (int tm = 0; tm < 2; ++tm)
 #pragma unroll
                 for (int tn = 0; tn < 2; ++tn) {
                     acc[tm][tn] = Frag<float>::zero();
 #pragma unroll
-                    for (int ks = 0; ks < KS; ++ks) acc[tm][tn] = Frag32<T>::mma(fb[tn][ks], fa[tm][ks], acc[tm][tn]);
+                    for (int ks = 0; ks < KS; ++ks) acc[tm][tn] = mma32<T>(fb[tn][ks], fa[tm][ks], acc[tm][tn]);
                 }
+        }
+        // the next tile goes to LDS before this step's stores are issued: the wait for its loads would
+        // otherwise wait for the stores too (one counter covers both)
+        if (s + 1 < n) stash((s + 1) & 1);
+        if (mine) {
             // lane holds C[m = 16tm + r16][n = 8g + 4tn + i]
             T* cp = cz + (long)blk * 1024;
 #pragma unroll
             for (int tm = 0; tm < 2; ++tm) store8_f32(cp + (16 * tm + r16) * 32 + 8 * g, acc[tm][0], acc[tm][1]);
         }
-        if (s + 1 < n) stash((s + 1) & 1);
+        inner_n1 = inner_n2;
+        blk = blk_n1;
         __syncthreads();
     }
 }
@@ -468,11 +494,11 @@ __global__ __launch_bounds__(256) void bs_dsd32u_kernel(const DsdUniArgs a) {
     const int sk = tid >> 3, c8 = 8 * (tid & 7);
     uint4 stage, fs[2], fs_next[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
     int blk_next = -1;
-    auto fetch = [&](int s) {
-        const long krow0 = (long)a.uni_inner[p0 + s] * 32;
+    auto fetch = [&](int inner, int blk_id) {
+        const long krow0 = (long)inner * 32;
         stage = make_uint4(0, 0, 0, 0);
         if (c8 < ncols) stage = *reinterpret_cast<const uint4*>(dnp + (krow0 + sk) * a.dn_sk + c8);
-        blk_next = have_row ? a.uni_blk[(long)(p0 + s) * 4 + w] : -1;
+        blk_next = have_row ? blk_id : -1;
         if (blk_next >= 0) {
             const T* blkp = spz + (long)blk_next * 1024;
 #pragma unroll
@@ -488,16 +514,23 @@ __global__ __launch_bounds__(256) void bs_dsd32u_kernel(const DsdUniArgs a) {
             vt[buf][lrow * DSDU_LD + sk] = (uint16_t)(v[i >> 1] >> (16 * (i & 1)));
         }
     };
+    // the index lists are read one step ahead of the fetch that uses them
+    int inner_n1 = n > 1 ? a.uni_inner[p0 + 1] : 0, id_n1 = n > 1 ? a.uni_blk[(long)(p0 + 1) * 4 + w] : -1;
     if (n > 0) {
-        fetch(0);
+        fetch(a.uni_inner[p0], a.uni_blk[(long)p0 * 4 + w]);
         stash(0);
     }
+    drain_loads();
     __syncthreads();
     for (int s = 0; s < n; ++s) {
         const int blk = blk_next;
         fs[0] = fs_next[0];
         fs[1] = fs_next[1];
-        if (s + 1 < n) fetch(s + 1);
+        const int inner_n2 = s + 2 < n ? a.uni_inner[p0 + s + 2] : 0;
+        const int id_n2 = s + 2 < n ? a.uni_blk[(long)(p0 + s + 2) * 4 + w] : -1;
+        if (s + 1 < n) fetch(inner_n1, id_n1);
+        inner_n1 = inner_n2;
+        id_n1 = id_n2;
         if (blk >= 0) {
             const uint16_t* tp = vt[s & 1];
 #pragma unroll
@@ -743,20 +776,6 @@ struct AttnArgs {
     long q_sz, q_sh, q_sm, k_sz, k_sh, k_sn, v_sz, v_sh, v_sn, o_sz, o_sh, o_sm;
     float scale;
 };
-
-template <typename T> __device__ __forceinline__ uint32_t pack2(float lo, float hi);
-template <> __device__ __forceinline__ uint32_t pack2<bf16_t>(float lo, float hi) { return pack_bf16x2(lo, hi); }
-template <> __device__ __forceinline__ uint32_t pack2<f16_t>(float lo, float hi) {
-    const _Float16 l = (_Float16)lo, h = (_Float16)hi;
-    return (uint32_t)__builtin_bit_cast(uint16_t, l) | ((uint32_t)__builtin_bit_cast(uint16_t, h) << 16);
-}
-template <typename T> __device__ __forceinline__ floatx4 mma32(uintx4 a, uintx4 b, floatx4 c);
-template <> __device__ __forceinline__ floatx4 mma32<bf16_t>(uintx4 a, uintx4 b, floatx4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
-}
-template <> __device__ __forceinline__ floatx4 mma32<f16_t>(uintx4 a, uintx4 b, floatx4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(halfx8_t, a), __builtin_bit_cast(halfx8_t, b), c, 0, 0, 0);
-}
 
 // Maxima of scores.  A two-operand fmaxf costs three instructions here (each operand is first quieted
 // by a self-maximum); three-operand maxima are emitted as they are, so pairs get -inf as a third.
