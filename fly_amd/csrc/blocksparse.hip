@@ -502,7 +502,11 @@ __global__ __launch_bounds__(256) void bs_dsd32u_kernel(const DsdUniArgs a) {
         if (blk_next >= 0) {
             const T* blkp = spz + (long)blk_next * 1024;
 #pragma unroll
-            for (int tm = 0; tm < 2; ++tm) fs_next[tm] = *reinterpret_cast<const uint4*>(blkp + (16 * tm + r16) * 32 + 8 * g);
+            for (int tm = 0; tm < 2; ++tm) {
+                // every sparse block is read by exactly one wave: nontemporal
+                const uintx4 t_ = __builtin_nontemporal_load(reinterpret_cast<const uintx4*>(blkp + (16 * tm + r16) * 32 + 8 * g));
+                fs_next[tm] = make_uint4(t_[0], t_[1], t_[2], t_[3]);
+            }
         }
     };
     auto stash = [&](int buf) {
@@ -1123,7 +1127,9 @@ __global__ __launch_bounds__(256) void bs_softmax32_kernel(RowArgs a) {
         off[it] = -1;
         if (j < nb) {
             off[it] = (long)a.row_blk[p0 + j] * 1024;
-            raw[it] = *reinterpret_cast<const uint4*>(xz + off[it]);
+            // streamed once in, once out: nontemporal both ways
+            const uintx4 t_ = __builtin_nontemporal_load(reinterpret_cast<const uintx4*>(xz + off[it]));
+            raw[it] = make_uint4(t_[0], t_[1], t_[2], t_[3]);
         }
     }
     // element u (0..7) of block slot `it` as float, unscaled
@@ -1193,7 +1199,7 @@ __global__ __launch_bounds__(256) void bs_softmax32_kernel(RowArgs a) {
                 T hi = Elem<T>::from_f32(ev[it][2 * u2 + 1] * inv);
                 outw[u2] = (uint32_t)*reinterpret_cast<uint16_t*>(&lo) | ((uint32_t)*reinterpret_cast<uint16_t*>(&hi) << 16);
             }
-            *reinterpret_cast<uint4*>(xz + off[it]) = make_uint4(outw[0], outw[1], outw[2], outw[3]);
+            __builtin_nontemporal_store(uintx4{outw[0], outw[1], outw[2], outw[3]}, reinterpret_cast<uintx4*>(xz + off[it]));
         }
 }
 
