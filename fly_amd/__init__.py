@@ -4,7 +4,8 @@ HIP kernels behind the reference's module interfaces.  The kernels live in ``lib
 (built from ``csrc/`` by ``python -m fly_amd.build``); nothing here falls back to a CPU path."""
 from .masking import FullMask, LengthMask, TriangularCausalMask
 from .feature_maps_sb import SBPerformerFeatures, gaussian_orthogonal_random_matrix
-from .sblocal_attention import SBLocalAttention, sblocal_forward
+from .sblocal_attention import SBLocalAttention, sblocal_forward, sblocal_attention_fn
+from .sblocal_backward import sblocal_backward
 from .local_attention import LocalAttention, local_forward
 from .blocksparse_utils import sparsify_tensor, densify_tensor, mask_tensor, sparsify_broadcast_tensor
 from .blocksparse_matmul import matmul
@@ -17,7 +18,7 @@ from .fastlinear import LowRank, SparseLRLinear
 from .t2t_vit import T2T_ViT, T2T_module, T2TAttention, Token_transformer, MlpCustom, t2t_vit_t_14
 
 __all__ = ['FullMask', 'LengthMask', 'TriangularCausalMask', 'SBPerformerFeatures',
-           'gaussian_orthogonal_random_matrix', 'SBLocalAttention', 'sblocal_forward', 'LocalAttention', 'local_forward',
+           'gaussian_orthogonal_random_matrix', 'SBLocalAttention', 'sblocal_forward', 'sblocal_attention_fn', 'sblocal_backward', 'LocalAttention', 'local_forward',
            'sparsify_tensor', 'densify_tensor', 'mask_tensor', 'sparsify_broadcast_tensor',
            'matmul', 'softmax', 'logsumexp', 'blocksparse_sum', 'BlockSparseAttention', 'fused_attention',
            'SBBlockSparseAttention',

@@ -154,6 +154,38 @@ def sblocal_forward(query, key, value, projection_matrix, local_context, softmax
     return out[..., :D], log_norm.unsqueeze(-1)
 
 
+class _SBLocalFn(torch.autograd.Function):
+    """sblocal_forward with gradients for query, key and value (the projection is a buffer).  The
+    forward is the fused kernel path; the backward is sblocal_backward.sblocal_backward."""
+
+    @staticmethod
+    def forward(ctx, query, key, value, projection_matrix, local_context, softmax_temp, key_lengths):
+        out, log_norm = sblocal_forward(query, key, value, projection_matrix, local_context,
+                                        softmax_temp=softmax_temp, key_lengths=key_lengths)
+        ctx.save_for_backward(query, key, value, projection_matrix, out, log_norm)
+        ctx.args = (local_context, softmax_temp, key_lengths)
+        ctx.mark_non_differentiable(log_norm)
+        return out, log_norm
+
+    @staticmethod
+    def backward(ctx, grad_out, _grad_log_norm):
+        from .sblocal_backward import sblocal_backward
+        query, key, value, projection_matrix, out, log_norm = ctx.saved_tensors
+        local_context, softmax_temp, key_lengths = ctx.args
+        dq, dk, dv = sblocal_backward(query, key, value, projection_matrix, local_context, softmax_temp,
+                                      key_lengths, out, log_norm, grad_out)
+        return dq, dk, dv, None, None, None, None
+
+
+def sblocal_attention_fn(query, key, value, projection_matrix, local_context, softmax_temp=None,
+                         key_lengths=None):
+    """sblocal_forward, differentiable with respect to query, key and value."""
+    if torch.is_grad_enabled() and any(x.requires_grad for x in (query, key, value)):
+        return _SBLocalFn.apply(query, key, value, projection_matrix, local_context, softmax_temp, key_lengths)
+    return sblocal_forward(query, key, value, projection_matrix, local_context, softmax_temp=softmax_temp,
+                           key_lengths=key_lengths)
+
+
 class SBLocalAttention(nn.Module):
     """Local (banded) softmax attention plus a Performer low-rank estimate of everything outside
     the band, under one normaliser.  Query i attends exactly to keys j with
@@ -196,8 +228,8 @@ class SBLocalAttention(nn.Module):
         if key_padding_mask is not None and not bool(key_padding_mask.all_ones):
             lengths = key_padding_mask.lengths          # raises ValueError unless a length mask
         self.feature_map.new_feature_map(query.device)
-        out, log_norm = sblocal_forward(query, key, value, self.feature_map.projection_matrix,
-                                        self.local_context, softmax_temp=self.softmax_temp,
-                                        key_lengths=lengths)
-        self.last_log_normalization = log_norm
+        out, log_norm = sblocal_attention_fn(query, key, value, self.feature_map.projection_matrix,
+                                             self.local_context, softmax_temp=self.softmax_temp,
+                                             key_lengths=lengths)
+        self.last_log_normalization = log_norm.detach()
         return out, None

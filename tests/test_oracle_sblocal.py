@@ -187,3 +187,28 @@ def test_local_attention_equals_dense_masked_softmax():
         w = torch.where(ok.any(-1, keepdim=True), w, torch.zeros_like(w))      # rows without a valid key
         ref = torch.einsum('bhts,bshd->bthd', w, v)
         assert (out - ref).abs().max() < 1e-12
+
+
+@pytest.mark.parametrize('B,T,S,H,E,D,mh,lc,lens', [(1, 40, 40, 2, 16, 16, 8, 12, None),
+                                                    (2, 70, 55, 2, 16, 24, 8, 13, [55, 31]),
+                                                    (1, 300, 300, 1, 8, 8, 4, 64, None)])
+def test_written_out_backward_matches_autograd_through_the_oracle(B, T, S, H, E, D, mh, lc, lens):
+    """fly_amd.sblocal_backward (the gradients written out: band terms plus global low-rank terms plus
+    the feature-map chain rule) against autograd through the oracle's op sequence, in float64, with
+    chunks smaller than the sequence, T != S, an odd window and key lengths."""
+    from fly_amd.sblocal_backward import sblocal_backward
+    g = torch.Generator().manual_seed(0)
+    q = (torch.randn(B, T, H, E, generator=g).double() * 0.7).requires_grad_()
+    k = (torch.randn(B, S, H, E, generator=g).double() * 0.7).requires_grad_()
+    v = torch.randn(B, S, H, D, generator=g).double().requires_grad_()
+    P = osb.gaussian_orthogonal_random_matrix(mh, E, generator=g, dtype=torch.float64)
+    kl = None if lens is None else torch.tensor(lens)
+    out, ln = osb.sblocal_attention(q, k, v, P, lc, key_lengths=kl)
+    w = torch.randn(out.shape, generator=g).double()
+    (out * w).sum().backward()
+    dq, dk, dv = sblocal_backward(q.detach(), k.detach(), v.detach(), P, lc, None, kl, out.detach(), ln.detach(), w,
+                                  chunk=32)
+    for got, ref in ((dq, q.grad), (dk, k.grad), (dv, v.grad)):
+        assert float((got - ref).abs().max() / ref.abs().max()) < 1e-10
+    if lens is not None:
+        assert float(dk[1, lens[1]:].abs().max()) == 0.0 and float(dv[1, lens[1]:].abs().max()) == 0.0
