@@ -94,6 +94,25 @@ struct RowTile {
                 r[j] = load4_f32(src + (long)min(row0 + row, last_row) * row_stride + 4 * c4);
         }
     }
+    // byte offsets of this thread's pieces inside a tile whose rows all exist (computed once); with
+    // them a fetch is one load per piece from a wave-uniform tile base, no address arithmetic
+    template <typename T>
+    __device__ __forceinline__ void offsets(uint32_t (&off)[N], long row_stride, int tid) const {
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+            const int idx = tid + NT * j, row = idx / V4, c4 = idx % V4;
+            off[j] = (uint32_t)((row * row_stride + 4 * c4) * (long)sizeof(T));
+        }
+    }
+    template <typename T>
+    __device__ __forceinline__ void fetch_fast(const T* tile_base, const uint32_t (&off)[N], int tid) {
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+            const int idx = tid + NT * j;
+            if (N * NT == ROWS * V4 || idx < ROWS * V4)
+                r[j] = load4_f32(reinterpret_cast<const T*>(reinterpret_cast<const char*>(tile_base) + off[j]));
+        }
+    }
     template <int LD>
     __device__ __forceinline__ void stash(float* dst, int tid, float scale = 1.0f) const {
 #pragma unroll
@@ -1364,6 +1383,12 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
         rv.fetch(vptr, a.v_ss, kt_lo * TK, a.S - 1, tid);
         rf.fetch(fptr, M, kt_lo * TK, f_last, tid);
     }
+    // tiles after the first: per-thread offsets once, then one load per piece from the tile's base
+    // (tiles that run past the last key row keep the clamping fetch)
+    uint32_t offk[RowTile<TK, E>::N], offv[RowTile<TK, D>::N], offf[RowTile<TK, M>::N];
+    rk.template offsets<T>(offk, a.k_ss, tid);
+    rv.template offsets<T>(offv, a.v_ss, tid);
+    rf.template offsets<float>(offf, M, tid);
     const float* csp = a.chunk_scale + (long)bh * a.n_chunks;
     float cscale = (kt_lo < kt_hi) ? csp[kt_lo * TK / CH] : 0.f;
     const float kmax = SPLIT ? split_kmax(a.part_max, bh, a.n_split) : a.kmax[bh];
@@ -1460,9 +1485,15 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
         const bool more = kt + 1 < kt_hi;
         float cscale_next = cscale;
         if (more) {                                      // next tile's loads fly during the MFMAs
-            rk.fetch(kptr, a.k_ss, s_base + TK, a.S - 1, tid);
-            rv.fetch(vptr, a.v_ss, s_base + TK, a.S - 1, tid);
-            rf.fetch(fptr, M, s_base + TK, f_last, tid);
+            if (s_base + 2 * TK <= a.S) {
+                rk.fetch_fast(kptr + (long)(s_base + TK) * a.k_ss, offk, tid);
+                rv.fetch_fast(vptr + (long)(s_base + TK) * a.v_ss, offv, tid);
+                rf.fetch_fast(fptr + (long)(s_base + TK) * M, offf, tid);
+            } else {
+                rk.fetch(kptr, a.k_ss, s_base + TK, a.S - 1, tid);
+                rv.fetch(vptr, a.v_ss, s_base + TK, a.S - 1, tid);
+                rf.fetch(fptr, M, s_base + TK, f_last, tid);
+            }
             cscale_next = csp[(s_base + TK) / CH];
         }
         // weight of this chunk's features relative to the global key stabiliser (<= 1); the same
@@ -1497,39 +1528,49 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
                 }
             }
 
-            // lane holds the scores of query iq against keys s_base + 16kb + 4g + i
-            bool ok[KB][4];
-            float mx = -INFINITY;
-#pragma unroll
-            for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int s = s_base + 16 * kb + 4 * g + i;
-                    ok[kb][i] = (unsigned)(s - smin) < span;
-                    mx = fmaxf(mx, ok[kb][i] ? s1[kb][i] : -INFINITY);
-                }
-            mx = group_max(mx);
-            if (__builtin_amdgcn_ballot_w64(mx > m_run) != 0) {      // wave-uniform: some row maximum grew
-                const float m_new = fmaxf(m_run, mx);
-                const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-                m_run = m_new;
-                ze *= alpha;
-#pragma unroll
-                for (int db = 0; db < DB; ++db) oacc[db] *= alpha;
-            }
-            const float beta = wc * __builtin_amdgcn_exp2f(c0 - m_run);          // scale of the overlap term, <= 1
+            // lane holds the scores of query iq against keys s_base + 16kb + 4g + i.  A tile that lies
+            // inside the band of all 16 queries of the wave and below the key length (wave-uniform) needs
+            // no masks.
+            const bool interior = s_base - (qw0 + 15) >= -lc_lo && s_base + TK - 1 - qw0 < lc_hi &&
+                                  s_base + TK <= len && qw0 + 15 < a.T;
             floatx4 p[KB];
             float ovs = 0.f;
+            auto soft = [&](auto masked_tag) __attribute__((always_inline)) {
+                constexpr bool MASKED = decltype(masked_tag)::value;
+                bool ok[KB][4];
+                float mx = -INFINITY;
 #pragma unroll
-            for (int kb = 0; kb < KB; ++kb)
+                for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const float e = ok[kb][i] ? __builtin_amdgcn_exp2f(s1[kb][i] - m_run) : 0.f;
-                    const float ov = ok[kb][i] ? s2[kb][i] : 0.f;
-                    ze += e;
-                    ovs += ov;
-                    p[kb][i] = e - ov * beta;
+                    for (int i = 0; i < 4; ++i) {
+                        const int s = s_base + 16 * kb + 4 * g + i;
+                        ok[kb][i] = !MASKED || (unsigned)(s - smin) < span;
+                        mx = fmaxf(mx, ok[kb][i] ? s1[kb][i] : -INFINITY);
+                    }
+                mx = group_max(mx);
+                // the reference exponent is raised only when a tile exceeds it by more than 2^8: until
+                // then the exponentials may exceed 1, which fp32 holds without loss
+                if (__builtin_amdgcn_ballot_w64(mx > m_run + 8.f) != 0) {      // wave-uniform
+                    const float m_new = fmaxf(m_run, mx);
+                    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+                    m_run = m_new;
+                    ze *= alpha;
+#pragma unroll
+                    for (int db = 0; db < DB; ++db) oacc[db] *= alpha;
                 }
+                const float beta = wc * __builtin_amdgcn_exp2f(c0 - m_run);      // scale of the overlap term
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float e = ok[kb][i] ? __builtin_amdgcn_exp2f(s1[kb][i] - m_run) : 0.f;
+                        const float ov = ok[kb][i] ? s2[kb][i] : 0.f;
+                        ze += e;
+                        ovs += ov;
+                        p[kb][i] = e - ov * beta;
+                    }
+            };
+            if (interior) soft(std::false_type{}); else soft(std::true_type{});
             zp += ovs * wc;
             // O^T[d][query] += sum_keys V[key][d] p[key][query]
 #pragma unroll
