@@ -803,7 +803,8 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
                     mx = fmaxf(mx, ok[kb][i] ? s1[kb][i] : -INFINITY);
                 }
             mx = group_max(mx) * sc;                               // sc > 0
-            if (__builtin_amdgcn_ballot_w64(mx > m_run) != 0) {      // wave-uniform: some row maximum grew
+            // (the reference exponent is raised only when a tile exceeds it by more than 2^8)
+            if (__builtin_amdgcn_ballot_w64(mx > m_run + 8.f) != 0) {      // wave-uniform
                 const float m_new = fmaxf(m_run, mx);
                 const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
                 m_run = m_new;
@@ -811,7 +812,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
 #pragma unroll
                 for (int db = 0; db < DB; ++db) oacc[db] *= alpha;
             }
-            const float beta = wc * __builtin_amdgcn_exp2f(c0 - m_run);      // scale of the overlap term, <= 1
+            const float beta = wc * __builtin_amdgcn_exp2f(c0 - m_run);      // scale of the overlap term
 #pragma unroll
             for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
@@ -1276,7 +1277,7 @@ __global__ __launch_bounds__(NT) void local_fwd_kernel(LocalArgs a) {
                     mx = fmaxf(mx, ok[kb][i] ? s1[kb][i] : -INFINITY);
                 }
             mx = group_max(mx);
-            if (__builtin_amdgcn_ballot_w64(mx > m_run) != 0) {
+            if (__builtin_amdgcn_ballot_w64(mx > m_run + 8.f) != 0) {
                 const float m_new = fmaxf(m_run, mx);
                 const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
                 m_run = m_new;
