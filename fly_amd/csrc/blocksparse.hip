@@ -97,6 +97,14 @@ __device__ __forceinline__ bool unit_of(unsigned id, int per_unit, int n_units, 
 // for them, and those waits -- counters retire in order -- also drain the prefetch the body has
 // just issued, every iteration.
 __device__ __forceinline__ void drain_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+// The same for "all but the newest N": in a loop that keeps two register sets of loads in flight,
+// placed after the older set has been consumed it records that only the newer set is outstanding,
+// so the refill of the older set's registers does not wait for the newer set.
+template <int N>
+__device__ __forceinline__ void drain_loads_but() {
+    static_assert(N >= 0 && N < 64, "vmcnt holds 6 bits");
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 0xF) | ((N >> 4) << 14));
+}
 static long unit_grid(long n_units, long per_unit) { return (n_units + BS_XCD - 1) / BS_XCD * BS_XCD * per_unit; }
 
 template <typename T> __device__ __forceinline__ uint32_t pack2(float lo, float hi);
@@ -674,32 +682,37 @@ __global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
     // two register sets: the loads of step s+2 are issued while step s computes and are parked in LDS
     // one iteration later, so every global load has two steps to arrive
     // (native vectors: arrays of the uint4 struct passed by reference do not stay in registers)
+    // Every fetch issues the same number of loads on every path (a step past the end re-reads the last
+    // one, an absent weight block reads block 0 and is zeroed when it is parked): only then can the
+    // compiler count how many newer loads may stay in flight when it waits for the older set.
     uintx4 rxa[KB][2], rwa[KB][2], rxb[KB][2], rwb[KB][2];
-    auto fetch = [&](int step, uintx4 (&rx)[KB][2], uintx4 (&rw)[KB][2]) __attribute__((always_inline)) {
+    bool wla[KB][2], wlb[KB][2];                            // weight block present?
+    auto fetch = [&](int step, uintx4 (&rx)[KB][2], uintx4 (&rw)[KB][2], bool (&wl)[KB][2]) __attribute__((always_inline)) {
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb) {
             const int t = step * KB + kb;
             const bool live = t < nin;                       // a missing block contributes zero weights
-            const long kcol = (long)s_inner[live ? t : nin - 1] * 32 + schunk;
+            const int tc = live ? t : nin - 1;
+            const long kcol = (long)s_inner[tc] * 32 + schunk;
 #pragma unroll
             for (int hh = 0; hh < 2; ++hh) {
                 const long m = min(m0 + srow + 64 * hh, (long)a.M - 1);        // clamped: masked at the store
                 rx[kb][hh] = *reinterpret_cast<const uintx4*>(xp + m * a.dn_sm + kcol);
                 const int orow = srow + 64 * hh;                                 // output row inside the group
-                const int blk_id = live ? s_blk[orow >> 5][t] : -1;
-                rw[kb][hh] = uintx4{0, 0, 0, 0};
-                if (blk_id >= 0)
-                    rw[kb][hh] = *reinterpret_cast<const uintx4*>(spz + (long)blk_id * 1024 + (orow & 31) * 32 + schunk);
+                const int blk_id = s_blk[orow >> 5][tc];
+                wl[kb][hh] = live && blk_id >= 0;
+                rw[kb][hh] = *reinterpret_cast<const uintx4*>(spz + (long)max(blk_id, 0) * 1024 + (orow & 31) * 32 + schunk);
             }
         }
     };
-    auto stash = [&](int buf, const uintx4 (&rx)[KB][2], const uintx4 (&rw)[KB][2]) __attribute__((always_inline)) {
+    auto stash = [&](int buf, const uintx4 (&rx)[KB][2], const uintx4 (&rw)[KB][2], const bool (&wl)[KB][2]) __attribute__((always_inline)) {
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
             for (int hh = 0; hh < 2; ++hh) {
                 *reinterpret_cast<uintx4*>(&xs[buf][(srow + 64 * hh) * LD + 32 * kb + schunk]) = rx[kb][hh];
-                *reinterpret_cast<uintx4*>(&ws[buf][(srow + 64 * hh) * LD + 32 * kb + schunk]) = rw[kb][hh];
+                *reinterpret_cast<uintx4*>(&ws[buf][(srow + 64 * hh) * LD + 32 * kb + schunk]) =
+                    wl[kb][hh] ? rw[kb][hh] : uintx4{0, 0, 0, 0};
             }
     };
 
@@ -729,18 +742,21 @@ __global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
             }
         }
     };
-    if (n_steps > 0) { fetch(0, rxa, rwa); stash(0, rxa, rwa); }
-    if (n_steps > 1) fetch(1, rxb, rwb);                   // set B holds odd steps, set A even steps
+    if (n_steps > 0) { fetch(0, rxa, rwa, wla); stash(0, rxa, rwa, wla); }
+    if (n_steps > 0) fetch(1, rxb, rwb, wlb);              // set B holds odd steps, set A even steps
+    drain_loads_but<4 * KB>();                              // only set B (4 KB loads a thread) is in flight
     __syncthreads();
     for (int step = 0; step < n_steps; step += 2) {
-        if (step + 2 < n_steps) fetch(step + 2, rxa, rwa);
+        fetch(step + 2, rxa, rwa, wla);
         compute(0);
-        if (step + 1 < n_steps) stash(1, rxb, rwb);
+        stash(1, rxb, rwb, wlb);
+        drain_loads_but<4 * KB>();                          // set B is parked: only set A is in flight
         __syncthreads();
         if (step + 1 >= n_steps) break;
-        if (step + 3 < n_steps) fetch(step + 3, rxb, rwb);
+        fetch(step + 3, rxb, rwb, wlb);
         compute(1);
-        if (step + 2 < n_steps) stash(0, rxa, rwa);
+        stash(0, rxa, rwa, wla);
+        drain_loads_but<4 * KB>();
         __syncthreads();
     }
     // lane holds y[m = 64wm + 16tm + r16][n = 32*(output block) + 8g + 4*(tn%2) + i]: 16-byte stores
