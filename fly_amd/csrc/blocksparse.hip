@@ -91,20 +91,6 @@ __device__ __forceinline__ bool unit_of(unsigned id, int per_unit, int n_units, 
     pos = (int)(slot % per_unit);
     return unit < n_units;
 }
-// Wait for every outstanding vector-memory load (vmcnt(0); the other counters are left alone).  Placed
-// in front of a pipelined loop it tells the compiler's wait-count bookkeeping that the operands
-// loaded before the loop have arrived; without it the loop body carries the first iteration's waits
-// for them, and those waits -- counters retire in order -- also drain the prefetch the body has
-// just issued, every iteration.
-__device__ __forceinline__ void drain_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }
-// The same for "all but the newest N": in a loop that keeps two register sets of loads in flight,
-// placed after the older set has been consumed it records that only the newer set is outstanding,
-// so the refill of the older set's registers does not wait for the newer set.
-template <int N>
-__device__ __forceinline__ void drain_loads_but() {
-    static_assert(N >= 0 && N < 64, "vmcnt holds 6 bits");
-    __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 0xF) | ((N >> 4) << 14));
-}
 static long unit_grid(long n_units, long per_unit) { return (n_units + BS_XCD - 1) / BS_XCD * BS_XCD * per_unit; }
 
 template <typename T> __device__ __forceinline__ uint32_t pack2(float lo, float hi);
@@ -752,9 +738,10 @@ __global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
         stash(1, rxb, rwb, wlb);
         drain_loads_but<4 * KB>();                          // set B is parked: only set A is in flight
         __syncthreads();
-        if (step + 1 >= n_steps) break;
+        // (no early exit between the halves: the compiler would count a path that leaves here, with
+        // set A in flight, as a way back to the top of the loop, and drain before every refill)
         fetch(step + 3, rxb, rwb, wlb);
-        compute(1);
+        if (step + 1 < n_steps) compute(1);
         stash(0, rxa, rwa, wla);
         drain_loads_but<4 * KB>();
         __syncthreads();

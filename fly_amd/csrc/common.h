@@ -171,6 +171,21 @@ template <> struct Frag32<float> {     // never used: keeps templates that branc
     static __device__ __forceinline__ floatx4 mma(uint4, uint4, floatx4 c) { return c; }
 };
 
+// Wait for every outstanding vector-memory load (vmcnt(0); the other counters are left alone).  Placed
+// in front of a pipelined loop it tells the compiler's wait-count bookkeeping that the operands
+// loaded before the loop have arrived; without it the loop body carries the first iteration's waits
+// for them, and those waits -- counters retire in order -- also drain the prefetch the body has
+// just issued, every iteration.
+__device__ __forceinline__ void drain_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+// The same for "all but the newest N": in a loop that keeps two register sets of loads in flight,
+// placed after the older set has been consumed it records that only the newer set is outstanding,
+// so the refill of the older set's registers does not wait for the newer set.
+template <int N>
+__device__ __forceinline__ void drain_loads_but() {
+    static_assert(N >= 0 && N < 64, "vmcnt holds 6 bits");
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 0xF) | ((N >> 4) << 14));
+}
+
 // wave-level butterflies across the four 16-lane groups (lanes r, r+16, r+32, r+48), on the
 // gfx950 row-swap instructions: permlane16_swap(v, v) yields {rows 0,0,2,2} and {rows 1,1,3,3},
 // permlane32_swap(v, v) yields {low half twice} and {high half twice}; no LDS traffic

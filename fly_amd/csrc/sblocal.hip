@@ -501,26 +501,91 @@ template <int ROWS, int W, int NT>
 struct Tile16 {
     static constexpr int C8 = W / 8, N = (ROWS * C8 + NT - 1) / NT;
     uintx4 r[N];
+    // the same with a wave-uniform tile base and per-thread byte offsets computed once (all rows exist)
+    __device__ __forceinline__ void offsets(uint32_t (&off)[N], long row_stride, int tid) const {
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+            const int idx = (tid + NT * j) % (ROWS * C8), row = idx / C8, c8 = idx % C8;
+            off[j] = (uint32_t)((row * row_stride + 8 * c8) * 2);
+        }
+    }
+    __device__ __forceinline__ void fetch_at(const uint16_t* tile_base, const uint32_t (&off)[N]) {
+#pragma unroll
+        for (int j = 0; j < N; ++j)
+            r[j] = *reinterpret_cast<const uintx4*>(reinterpret_cast<const char*>(tile_base) + off[j]);
+    }
+    // (a tile with fewer pieces than threads wraps around: every thread loads and stores, see TileKV16)
     __device__ __forceinline__ void fetch(const uint16_t* src, long row_stride, int row0, int last_row, int tid) {
 #pragma unroll
         for (int j = 0; j < N; ++j) {
-            const int idx = tid + NT * j, row = idx / C8, c8 = idx % C8;
-            if (N * NT == ROWS * C8 || idx < ROWS * C8)
-                r[j] = *reinterpret_cast<const uintx4*>(src + (long)min(row0 + row, last_row) * row_stride + 8 * c8);
+            const int idx = (tid + NT * j) % (ROWS * C8), row = idx / C8, c8 = idx % C8;
+            r[j] = *reinterpret_cast<const uintx4*>(src + (long)min(row0 + row, last_row) * row_stride + 8 * c8);
         }
     }
     template <int LD>
     __device__ __forceinline__ void stash(uint16_t* dst, int tid) const {
 #pragma unroll
         for (int j = 0; j < N; ++j) {
-            const int idx = tid + NT * j, row = idx / C8, c8 = idx % C8;
-            if (N * NT == ROWS * C8 || idx < ROWS * C8) *reinterpret_cast<uintx4*>(dst + row * LD + 8 * c8) = r[j];
+            const int idx = (tid + NT * j) % (ROWS * C8), row = idx / C8, c8 = idx % C8;
+            *reinterpret_cast<uintx4*>(dst + row * LD + 8 * c8) = r[j];
         }
+    }
+};
+
+// The K tile (TK rows of E, row-major) and the V tile (D rows of TK, contiguous) of one step as ONE
+// list of 16-byte pieces dealt to the threads round-robin, so that every thread issues the same
+// number of loads whatever it holds (whole waves hold K or V pieces: both piece counts are
+// multiples of 64).  Addresses are a wave-uniform tile base plus a per-thread byte offset computed
+// once: the key loop then contains no vector address arithmetic, whose temporaries the register
+// allocator likes to place in the registers of the previous fetch, behind a full wait.  The K tile
+// that runs past the last key row uses a second, clamped set of offsets.  A list shorter than the
+// workgroup wraps around: the surplus threads repeat pieces (same data to the same LDS address).
+template <int E, int D, int NT>
+struct TileKV16 {
+    static constexpr int KC = TK * E / 8, VC = D * TK / 8, TOT = KC + VC, N = (TOT + NT - 1) / NT;
+    static_assert(KC % 64 == 0 && VC % 64 == 0, "whole waves hold K or V pieces");
+    uintx4 r[N];
+    struct Plan {
+        uint32_t off[N], off_last[N];        // byte offsets from the tile base (off_last: K rows clamped)
+        int lds[N];                          // element offset in the K region or the V region of a stage
+        bool is_k[N];                        // wave-uniform
+    };
+    template <int LDK, int LDT>
+    static __device__ __forceinline__ void plan(Plan& p, long k_stride, int rows_in_last_tile, int tid) {
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+            const int idx = (tid + NT * j) % TOT, vi = idx - KC;
+            p.is_k[j] = __builtin_amdgcn_readfirstlane(idx < KC);
+            const int row = idx / (E / 8), c8 = idx % (E / 8);
+            p.off[j] = p.is_k[j] ? (uint32_t)((row * k_stride + 8 * c8) * 2) : (uint32_t)(16 * vi);
+            p.off_last[j] = p.is_k[j] ? (uint32_t)((min(row, rows_in_last_tile - 1) * k_stride + 8 * c8) * 2) : (uint32_t)(16 * vi);
+            p.lds[j] = p.is_k[j] ? row * LDK + 8 * c8 : (vi / (TK / 8)) * LDT + 8 * (vi % (TK / 8));
+        }
+    }
+    __device__ __forceinline__ void fetch(const Plan& p, const uint16_t* k_tile, const uint16_t* v_tile, bool last_tile) {
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+            const char* base = reinterpret_cast<const char*>(p.is_k[j] ? k_tile : v_tile);      // scalar select
+            r[j] = *reinterpret_cast<const uintx4*>(base + (last_tile ? p.off_last[j] : p.off[j]));
+        }
+    }
+    __device__ __forceinline__ void stash(const Plan& p, uint16_t* kdst, uint16_t* vdst) const {
+#pragma unroll
+        for (int j = 0; j < N; ++j) *reinterpret_cast<uintx4*>((p.is_k[j] ? kdst : vdst) + p.lds[j]) = r[j];
     }
 };
 
 __device__ __forceinline__ floatx4 mma_bf16(uint4 a, uint4 b, floatx4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+
+template <int E, int M> constexpr size_t fwd_bf16_smem() {
+    constexpr size_t stage = (size_t)TK * (E + 8) + (size_t)TK * (M + 8) + (size_t)E * (TK + 8);   // 2-byte elements
+    constexpr size_t tiles = 2 * stage * 2;
+    constexpr size_t proj = (size_t)2 * (M / 2) * (E + 8) * 2;      // bf16 head and remainder of the projection
+    constexpr size_t lowrank = (size_t)E * (M + 8) * 2;
+    constexpr size_t need = tiles > proj ? (tiles > lowrank ? tiles : lowrank) : (proj > lowrank ? proj : lowrank);
+    return need;
 }
 
 // A workgroup is NW waves of 16 queries each: more waves share every key tile, which divides the
@@ -585,27 +650,36 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
     // used (one iteration of work is shorter than the latency of the loads under load), so two
     // register sets alternate and the key loop is unrolled by two.
     struct TileRegs {
-        Tile16<TK, E, NT> k;
-        Tile16<D, TK, NT> v;          // already transposed by the key pass: D rows of 32 k-slots
+        TileKV16<E, D, NT> kv;        // K rows, and V already transposed by the key pass: D rows of 32 k-slots
         Tile16<TK, M, NT> f;
-        float cscale;
     };
-    const int f_last = a.n_chunks * CH - 1;
-    const float* csp = a.chunk_scale + (long)bh * a.n_chunks;
+    // the chunk log-scales of this workgroup's share of the band sit in LDS behind the tile stages
+    // (the host sizes the region): a load of them inside the loop would have to be waited for at
+    // the start of a step, and the memory counter retires in order -- behind it the tile prefetch
+    float* cs_lds = reinterpret_cast<float*>(reinterpret_cast<char*>(smem) + fwd_bf16_smem<E, M>());
+    const int c_lo = kt_lo * TK / CH;
+    {
+        const int n_cs = kt_hi > kt_lo ? (kt_hi - 1) * TK / CH - c_lo + 1 : 0;
+        const float* csg = a.chunk_scale + (long)bh * a.n_chunks + c_lo;
+        for (int i = tid; i < n_cs; i += NT) cs_lds[i] = csg[i];
+    }
+    constexpr int LOADS = TileKV16<E, D, NT>::N + Tile16<TK, M, NT>::N;     // vector loads of one fetch, per thread
+    typename TileKV16<E, D, NT>::Plan kvp;
+    const int last_tile = (a.S - 1) / TK;                 // the only K tile whose rows may not all exist
+    TileKV16<E, D, NT>::template plan<LDK, LDT>(kvp, a.k_ss, a.S - last_tile * TK, tid);
+    uint32_t foff[Tile16<TK, M, NT>::N];
+    Tile16<TK, M, NT>().offsets(foff, M, tid);
     auto fetch = [&](TileRegs& r, int kt) __attribute__((always_inline)) {
-        r.k.fetch(kptr, a.k_ss, kt * TK, a.S - 1, tid);
-        r.v.fetch(vtp + (long)kt * (D * TK), TK, 0, D - 1, tid);
-        r.f.fetch(fptr, M, kt * TK, f_last, tid);
-        r.cscale = csp[kt * TK / CH];
+        const int ktc = min(kt, last_tile);               // (tiles past the keys are never used; stay in bounds)
+        r.kv.fetch(kvp, kptr + (long)ktc * TK * a.k_ss, vtp + (long)kt * (D * TK), ktc == last_tile);
+        r.f.fetch_at(fptr + (long)kt * TK * M, foff);
     };
     auto stash = [&](const TileRegs& r, int stage) __attribute__((always_inline)) {
         uint16_t* dst = lds + stage * STAGE;
-        r.k.template stash<LDK>(dst, tid);
+        r.kv.stash(kvp, dst, dst + TK * (LDK + LDF));
         r.f.template stash<LDF>(dst + TK * LDK, tid);
-        r.v.template stash<LDT>(dst + TK * (LDK + LDF), tid);
     };
     TileRegs ra, rb;
-    ra.cscale = rb.cscale = 0.f;
     // (clamped tile indices: the loads are unconditional so that the register sets are plain values)
     fetch(ra, min(kt_lo, max(kt_hi - 1, 0)));
     fetch(rb, min(kt_lo + 1, max(kt_hi - 1, 0)));
@@ -715,7 +789,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
     const int smin = max(iq - lc_lo, 0);
     const unsigned span = qvalid ? (unsigned)max(min(iq + lc_hi, len) - smin, 0) : 0u;
 
-    if (kt_lo < kt_hi) stash(ra, 0);
+    stash(ra, 0);                          // (unconditional like every fetch and stash: see the key loop)
     __syncthreads();
 
     // One key tile takes two phases: scores (LDS fragment reads and the two score MFMA products) and
@@ -848,17 +922,25 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
     FLY_PROF(2);
     // even steps: tile kt sits in stage 0 (from ra), rb holds kt + 1, ra is refilled with kt + 2;
     // odd steps the other way round
+    // Fetches and stashes run on every pass, past the end with the last tile again: with loads under
+    // conditions the compiler cannot tell which set is the newer one and drains both whenever it
+    // waits for one.  After a stash only the other set is in flight, which the explicit counts record.
+    drain_loads();                         // once, before the loop: from here on the counts below are exact
     for (int kt = kt_lo; kt < kt_hi; kt += 2) {
-        const float cs0 = ra.cscale;
-        if (kt + 2 < kt_hi) fetch(ra, kt + 2);
+        const float cs0 = cs_lds[kt * TK / CH - c_lo];
+        fetch(ra, min(kt + 2, kt_hi - 1));
         tile_step(kt, 0, cs0);
-        if (kt + 1 < kt_hi) stash(rb, 1);
+        stash(rb, 1);
+        drain_loads_but<LOADS>();
         __syncthreads();
-        if (kt + 1 >= kt_hi) break;
-        const float cs1 = rb.cscale;
-        if (kt + 3 < kt_hi) fetch(rb, kt + 3);
-        tile_step(kt + 1, 1, cs1);
-        if (kt + 2 < kt_hi) stash(ra, 0);
+        // (no early exit between the halves: a path that leaves here with set A still in flight would
+        // count, for the compiler, as a way back to the top of the loop)
+        const bool second = kt + 1 < kt_hi;
+        const float cs1 = cs_lds[min(kt + 1, kt_hi - 1) * TK / CH - c_lo];
+        fetch(rb, min(kt + 3, kt_hi - 1));
+        if (second) tile_step(kt + 1, 1, cs1);
+        stash(ra, 0);
+        drain_loads_but<LOADS>();
         __syncthreads();
     }
     if (late && kt_lo < kt_hi) soft_phase(kt_hi - 1, cs_prev);
@@ -1799,15 +1881,6 @@ static int launch_kfeat(const KvArgs& a, hipStream_t st) {
 // band kernel of the next flyhip_sblocal_fwd call made by this thread (then cleared).
 static thread_local hipEvent_t g_ev_before = nullptr, g_ev_after = nullptr;
 
-template <int E, int M> constexpr size_t fwd_bf16_smem() {
-    constexpr size_t stage = (size_t)TK * (E + 8) + (size_t)TK * (M + 8) + (size_t)E * (TK + 8);   // 2-byte elements
-    constexpr size_t tiles = 2 * stage * 2;
-    constexpr size_t proj = (size_t)2 * (M / 2) * (E + 8) * 2;      // bf16 head and remainder of the projection
-    constexpr size_t lowrank = (size_t)E * (M + 8) * 2;
-    constexpr size_t need = tiles > proj ? (tiles > lowrank ? tiles : lowrank) : (proj > lowrank ? proj : lowrank);
-    return need;
-}
-
 // float inputs: fp32 MFMA kernel; bfloat16 inputs: bf16 MFMA kernel
 template <typename T, int E, int M, bool SPLIT> struct FwdKernel {
     static constexpr size_t smem = fwd_smem<E, M>();
@@ -1823,15 +1896,19 @@ template <int E, int M, bool SPLIT> struct FwdKernel<bf16_t, E, M, SPLIT> {
 template <typename T, int E, int M, bool SPLIT>
 static int launch_fwd_impl(const FwdArgs& a, hipStream_t st) {
     auto kern = FwdKernel<T, E, M, SPLIT>::get();
-    constexpr size_t smem = FwdKernel<T, E, M, SPLIT>::smem;
+    typedef FwdKernel<T, E, M, SPLIT> K;
+    // the bf16 kernel keeps the chunk log-scales of a workgroup's share of the band behind its tile stages
+    const long band_keys = (long)a.lc + K::tq + 2 * CH;
+    const size_t smem = K::smem + (sizeof(T) == 2 ? (size_t)(band_keys / CH + 2) * sizeof(float) : 0);
+    constexpr size_t LDS_MAX = 160 * 1024;
+    if (smem > LDS_MAX) return fail(ERR_ARG, "sblocal_fwd: local_context %d needs %zu bytes of LDS (limit %zu)", a.lc, smem, LDS_MAX);
     static bool lds_ready = false;
     if (!lds_ready) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_MAX);
         if (e != hipSuccess) return fail(ERR_LAUNCH, "sblocal_fwd: LDS attribute: %s", hipGetErrorString(e));
         lds_ready = true;
     }
-    typedef FwdKernel<T, E, M, SPLIT> K;
     const int qt = (a.T + TQ - 1) / TQ;                           // 64-query tiles (partials, merge)
     const long items = (long)a.B * a.H * ((a.T + K::tq - 1) / K::tq) * a.n_parts;
     long grid = (items + N_XCD - 1) / N_XCD * N_XCD;             // whole rounds over the XCDs
