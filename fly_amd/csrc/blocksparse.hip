@@ -998,24 +998,18 @@ __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
         const int blk_n1 = s + 1 < n ? a.uni_blk[(long)(p0 + s + 1) * NW + w] : -1;
         const bool present = s < n && have_row && blk_cur >= 0;
         const int vb_next = vb == 2 ? 0 : vb + 1, vb_prev = vb == 0 ? 2 : vb - 1;
-#ifndef ATT_NOSTAGE
         if (s + 1 < n) fetch(inner_n1);
-#endif
         if (late && had_prev) soft_pv(vb_prev, inner_prev);
         if (present) score(s & 1);
         if (!late && present) soft_pv(vb, inner_cur);
-#ifndef ATT_NOSTAGE
         if (s + 1 < n) stash((s + 1) & 1, vb_next);
-#endif
         had_prev = present;
         inner_prev = inner_cur;
         inner_cur = inner_n1;
         inner_n1 = inner_n2;
         blk_cur = blk_n1;
         vb = vb_next;
-#ifndef ATT_NOBAR
         __syncthreads();
-#endif
     }
     if (!have_row) return;
     T* op = reinterpret_cast<T*>(a.out) + z * a.o_sz + head * a.o_sh;
