@@ -86,13 +86,6 @@ def bench_sblocal(steps, warmup, cpu_baseline=True):
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     fwd_ms = sum(a.elapsed_time(b) for a, b in ev.values()) / len(ev)
-    # what the same two records read with nothing between them: the share of kernel_ms that is the
-    # event pair itself (a kernel trace of the same launches reads lower by about this much)
-    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(32)]
-    for a, b in pairs:
-        a.record(); b.record()
-    torch.cuda.synchronize()
-    empty_pair_ms = sum(a.elapsed_time(b) for a, b in pairs) / len(pairs)
 
     total_flops, fwd_flops = sblocal_flops(B, H, L, L, E, D, 2 * mh, lc)
     ms_per_step = wall / steps * 1e3
@@ -103,8 +96,7 @@ def bench_sblocal(steps, warmup, cpu_baseline=True):
         'roofline': {'bound': 'mfma', 'kernel': 'sblocal_fwd_kernel<float,64,64,128>',
                      'achieved': achieved, 'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s',
                      'frac': achieved / PEAK_FP32_MFMA_TFLOPS, 'traffic': BAND_KERNEL_TRAFFIC_BYTES,
-                     'kernel_ms': fwd_ms, 'empty_event_pair_ms': empty_pair_ms, 'flops_per_launch': fwd_flops,
-                     'launches_timed': len(ev)},
+                     'kernel_ms': fwd_ms, 'flops_per_launch': fwd_flops, 'launches_timed': len(ev)},
         'parity': None,
         'flops_per_step': total_flops,
     }

@@ -639,10 +639,11 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
     int kt_lo = lo / TK;
     int kt_hi = (hi > lo) ? (hi + TK - 1) / TK : kt_lo;
     if (SPLIT) {
-        const int per = (kt_hi - kt_lo + a.n_parts - 1) / a.n_parts;
-        const int first = kt_lo + part * per;
-        kt_lo = min(kt_hi, first);
-        kt_hi = min(kt_hi, first + per);
+        // an even split: the first (tiles % parts) parts take one tile more
+        const int nt = kt_hi - kt_lo, base = nt / a.n_parts, extra = nt % a.n_parts;
+        const int first = kt_lo + part * base + min(part, extra);
+        kt_lo = first;
+        kt_hi = first + base + (part < extra ? 1 : 0);
     }
     constexpr bool lowrank_here = !SPLIT;              // with several parts the merge kernel adds the low-rank term
 
@@ -1450,10 +1451,11 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
     int kt_lo = lo / TK;
     int kt_hi = (hi > lo) ? (hi + TK - 1) / TK : kt_lo;
     if (SPLIT) {
-        const int per = (kt_hi - kt_lo + a.n_parts - 1) / a.n_parts;
-        const int first = kt_lo + part * per;
-        kt_lo = min(kt_hi, first);
-        kt_hi = min(kt_hi, first + per);
+        // an even split: the first (tiles % parts) parts take one tile more
+        const int nt = kt_hi - kt_lo, base = nt / a.n_parts, extra = nt % a.n_parts;
+        const int first = kt_lo + part * base + min(part, extra);
+        kt_lo = first;
+        kt_hi = first + base + (part < extra ? 1 : 0);
     }
 
     // start the first tile's loads before anything else
