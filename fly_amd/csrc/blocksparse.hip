@@ -634,7 +634,7 @@ struct DdsGroupArgs {
 };
 constexpr int DDS_MAX_STEPS = 128;   // longest reduction list the tiled kernel accepts
 
-template <typename T>
+template <typename T, bool WT>     // WT: blocks are [k][n] (y = x W) and are transposed on their way into LDS
 __global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
     constexpr int KB = 1;                                   // input blocks per pipeline step
     constexpr int LD = 32 * KB + 8;                         // LDS row stride in elements
@@ -697,8 +697,18 @@ __global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
 #pragma unroll
             for (int hh = 0; hh < 2; ++hh) {
                 *reinterpret_cast<uintx4*>(&xs[buf][(srow + 64 * hh) * LD + 32 * kb + schunk]) = rx[kb][hh];
-                *reinterpret_cast<uintx4*>(&ws[buf][(srow + 64 * hh) * LD + 32 * kb + schunk]) =
-                    wl[kb][hh] ? rw[kb][hh] : uintx4{0, 0, 0, 0};
+                const uintx4 wv = wl[kb][hh] ? rw[kb][hh] : uintx4{0, 0, 0, 0};
+                if (!WT) {
+                    *reinterpret_cast<uintx4*>(&ws[buf][(srow + 64 * hh) * LD + 32 * kb + schunk]) = wv;
+                } else {
+                    // the thread holds row k = orow % 32 of the block, columns n = schunk .. schunk + 7: the
+                    // LDS tile is [n][k] either way, so these eight go out one by one
+                    const int orow = srow + 64 * hh;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        ws[buf][(32 * (orow >> 5) + schunk + e) * LD + 32 * kb + (orow & 31)] =
+                            (uint16_t)(wv[e >> 1] >> (16 * (e & 1)));
+                }
             }
     };
 
@@ -1424,13 +1434,18 @@ extern "C" int flyhip_bs_dds(const void* a, const void* b_sp, void* c,
     FLY_REQUIRE(b_sz % 4 == 0, "bs_dds: sparse batch stride must be a multiple of 4 elements");
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     if (grp_row0 && grp_n && n_grp > 0 && max_seg_len >= 0 && max_seg_len <= DDS_MAX_STEPS && blk == 32 &&
-        (dtype == BF16 || dtype == F16) && trans_b && a_sk == 1 &&
+        (dtype == BF16 || dtype == F16) && a_sk == 1 &&
         c_sn == 1 && ((a_sz | a_sh | a_sm | b_sz | c_sz | c_sh | c_sm) % 8) == 0 && (M + 127) / 128 <= 65535) {
         DdsGroupArgs ga{b_sp, a, c, seg_ptr, seg_blk, seg_inner, grp_row0, grp_n, cols_per_head, M,
                         b_sz, a_sz, a_sh, a_sm, c_sz, c_sh, c_sm};
         dim3 grid(n_grp, (M + 127) / 128, Z);
-        if (dtype == BF16) hipLaunchKernelGGL((bs_dds32_kernel<bf16_t>), grid, dim3(256), 0, st, ga);
-        else hipLaunchKernelGGL((bs_dds32_kernel<f16_t>), grid, dim3(256), 0, st, ga);
+        if (dtype == BF16) {
+            if (trans_b) hipLaunchKernelGGL((bs_dds32_kernel<bf16_t, false>), grid, dim3(256), 0, st, ga);
+            else hipLaunchKernelGGL((bs_dds32_kernel<bf16_t, true>), grid, dim3(256), 0, st, ga);
+        } else {
+            if (trans_b) hipLaunchKernelGGL((bs_dds32_kernel<f16_t, false>), grid, dim3(256), 0, st, ga);
+            else hipLaunchKernelGGL((bs_dds32_kernel<f16_t, true>), grid, dim3(256), 0, st, ga);
+        }
         return check_launch("bs_dds32_kernel");
     }
     DxdArgs args{b_sp, a, c, seg_ptr, seg_blk, seg_inner, n_seg, cols_per_head, M, trans_b,
