@@ -9,6 +9,8 @@ from .blocksparse_utils import group_table, sdd_table, segment_table, union_tabl
 # common: the union tables are passed to the kernels when the layout has at least this many
 # (row, column) pairs per union column on average.
 UNION_MIN_SHARING = 1.5
+# sdd with both operands contraction-major (a^T b) takes the split-K kernel from this contraction length on
+KMAJOR_MIN_K = 512
 
 _BLOCKS = (16, 32, 64, 128)
 
@@ -171,6 +173,10 @@ class matmul:
         if a.shape[1] != H or b.shape[1] != H or b.shape[0] != Z or M != p * self.block or N != r * self.block:
             raise ValueError(f'SDD operands {tuple(a.shape)}, {tuple(b.shape)} do not match layout '
                              f'{tuple(self.spdims)} with block {self.block}')
+        if (trans_a and not trans_b and self.block == 32 and a.dtype in (torch.bfloat16, torch.float16)
+                and K >= KMAJOR_MIN_K and a.stride(3) == 1 and b.stride(3) == 1
+                and all(s % 8 == 0 for s in a.stride()[:3] + b.stride()[:3])):
+            return self._sdd_kmajor(a, b, Z, K)
         (lut,) = self._table('sdd', a.device)
         row_ptr, row_blk, row_col = self._table('rows', a.device)
         uni = [t.data_ptr() for t in self._table('union', a.device)] or [None] * 3
@@ -184,6 +190,26 @@ class matmul:
                       Z, K, self.block, a.stride(0), a.stride(1), a_sm, a_sk,
                       b.stride(0), b.stride(1), b_sn, b_sk, _lib.dtype_code(a), _lib.stream_ptr(a.device))
         return c
+
+    def _sdd_kmajor(self, a, b, Z, K):
+        """sparse = a^T b with the contraction index slowest in both operands and long (the weight
+        gradient of a block-sparse linear layer: K = tokens): split over K, accumulated in fp32."""
+        H, p, r = self.spdims
+        row_ptr, row_blk, row_col = self._table('rows', a.device)
+        grp_row0, grp_n = self._table('grp_rows', a.device)
+        nnz = int(self.layout.sum())
+        max_row_nnz = int(self.layout.sum(-1).max())
+        tiles = grp_row0.shape[0] * ((max_row_nnz + 3) // 4) * Z
+        slices = max(1, min(K // 256, -(-2048 // tiles)))       # about eight workgroups per CU
+        k_slice = -(-(-(-K // slices)) // 32) * 32
+        c32 = torch.zeros((Z, nnz, 32, 32), dtype=torch.float32, device=a.device)
+        with torch.cuda.device(a.device):
+            _lib.call('flyhip_bs_sdd_kmajor', a.data_ptr(), b.data_ptr(), c32.data_ptr(),
+                      row_ptr.data_ptr(), row_blk.data_ptr(), row_col.data_ptr(),
+                      grp_row0.data_ptr(), grp_n.data_ptr(), grp_row0.shape[0], max_row_nnz,
+                      p, nnz, Z, K, k_slice, 32, a.stride(0), a.stride(1), a.stride(2),
+                      b.stride(0), b.stride(1), b.stride(2), _lib.dtype_code(a), _lib.stream_ptr(a.device))
+        return c32.to(a.dtype)
 
     def _dsd(self, a, b, trans_a, trans_b, trans_c):
         b = _dense_operand(b)

@@ -282,6 +282,130 @@ __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------
+// SDD with the contraction index slowest in both operands: sparse = A^T B, A (K x M), B (K x N)
+// ---------------------------------------------------------------------------------------
+// The weight gradient of a block-sparse linear layer: K = tokens (tens of thousands), M / N = output /
+// input features, 32x32 blocks of a 2-byte type.  One workgroup per (group of <= 4 consecutive
+// block-rows with identical column lists, chunk of <= 4 of their block-columns, slice of K): a
+// 128 x 128 output tile, the 2 x 2 waves owning 64 x 64 each.  Per step of 32 tokens the 32 x 128
+// tiles of A and B are loaded with 16-byte pieces along the features and written to LDS
+// transposed ([feature][token]), which makes every MFMA fragment one 16-byte LDS read; the
+// slices' partial blocks meet in an fp32 buffer through hardware float atomics (the caller zeroes
+// it and rounds it to the output type afterwards).
+struct SddKArgs {
+    const void* a; const void* b; float* c32;
+    const int32_t* seg_ptr; const int32_t* seg_blk; const int32_t* seg_inner;
+    const int32_t* grp_row0; const int32_t* grp_n;
+    int per_head, K, k_slice, chunks, nnz;
+    long a_sz, a_sh, a_sk, b_sz, b_sh, b_sk;
+};
+constexpr int SDDK_LD = 40;     // LDS row stride in elements ([feature][token], 32 tokens + 8)
+
+template <typename T>
+__global__ __launch_bounds__(256) void bs_sdd32k_kernel(const SddKArgs a) {
+    constexpr int LD = SDDK_LD;
+    __shared__ __attribute__((aligned(16))) uint16_t at[2][128 * LD];
+    __shared__ __attribute__((aligned(16))) uint16_t bt[2][128 * LD];
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
+    const int wm = w >> 1, wn = w & 1;
+    const int grp = blockIdx.x / a.chunks, chunk = blockIdx.x % a.chunks, z = blockIdx.z;
+    const int row0 = a.grp_row0[grp], gn = a.grp_n[grp];
+    const int head = row0 / a.per_head, brow0 = row0 % a.per_head;
+    const int p0 = a.seg_ptr[row0], nin = a.seg_ptr[row0 + 1] - p0;
+    const int j0 = chunk * 4, jn = min(4, nin - j0);       // this chunk's block-columns: list entries j0 .. j0 + jn - 1
+    if (jn <= 0) return;                                    // workgroup-uniform
+    const int k0 = blockIdx.y * a.k_slice, k1 = min(a.K, k0 + a.k_slice);
+    if (k0 >= k1) return;
+    const uint16_t* ap = reinterpret_cast<const uint16_t*>(a.a) + z * a.a_sz + head * a.a_sh + (long)brow0 * 32;
+    const uint16_t* bp = reinterpret_cast<const uint16_t*>(a.b) + z * a.b_sz + head * a.b_sh;
+
+    // staging: piece c = tid + 256 i (i < 2) of each tile is token c / 16, features 8 (c % 16) .. + 7;
+    // feature block c % 16 / 4 is output block-row ob (A) or list entry j0 + jb (B); absent blocks read
+    // block 0 of the tile and are zeroed when parked
+    int fcol_a[2], fcol_b[2];                               // feature offset of the piece in its operand
+    bool live_a[2], live_b[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int c = tid + 256 * i, fb = (c & 15) >> 2, f8 = 8 * (c & 3);
+        live_a[i] = fb < gn;
+        live_b[i] = fb < jn;
+        fcol_a[i] = 32 * (live_a[i] ? fb : 0) + f8;
+        fcol_b[i] = a.seg_inner[p0 + j0 + (live_b[i] ? fb : 0)] * 32 + f8;
+    }
+    uintx4 ra[2], rb[2];
+    auto fetch = [&](int kt) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int tok = min(kt + ((tid + 256 * i) >> 4), a.K - 1);     // clamped; tokens past k1 are zeroed below
+            ra[i] = *reinterpret_cast<const uintx4*>(ap + (long)tok * a.a_sk + fcol_a[i]);
+            rb[i] = *reinterpret_cast<const uintx4*>(bp + (long)tok * a.b_sk + fcol_b[i]);
+        }
+    };
+    auto stash = [&](int buf, int kt) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int c = tid + 256 * i, tok = c >> 4, f0 = 8 * (c & 15);
+            const bool in = kt + tok < k1;
+            const uintx4 va = (live_a[i] && in) ? ra[i] : uintx4{0, 0, 0, 0};
+            const uintx4 vb = (live_b[i] && in) ? rb[i] : uintx4{0, 0, 0, 0};
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                at[buf][(f0 + e) * LD + tok] = (uint16_t)(va[e >> 1] >> (16 * (e & 1)));
+                bt[buf][(f0 + e) * LD + tok] = (uint16_t)(vb[e >> 1] >> (16 * (e & 1)));
+            }
+        }
+    };
+
+    floatx4 acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = Frag<float>::zero();
+    const bool wave_active = 2 * wm < gn && 2 * wn < jn;    // its output blocks exist
+
+    fetch(k0);
+    stash(0, k0);
+    drain_loads();
+    __syncthreads();
+    int buf = 0;
+    for (int kt = k0; kt < k1; kt += 32) {
+        fetch(min(kt + 32, a.K - 1));                      // (past the slice: loaded, zeroed, never used)
+        if (wave_active) {
+            uintx4 fa[4], fb[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                fa[i] = *reinterpret_cast<const uintx4*>(&at[buf][(64 * wm + 16 * i + r16) * LD + 8 * g]);
+                fb[i] = *reinterpret_cast<const uintx4*>(&bt[buf][(64 * wn + 16 * i + r16) * LD + 8 * g]);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = mma32<T>(fa[i], fb[j], acc[i][j]);
+        }
+        stash(buf ^ 1, kt + 32);
+        buf ^= 1;
+        __syncthreads();
+    }
+    if (!wave_active) return;
+    // lane holds C[out = 64 wm + 16 i + 4 g + x][in = 64 wn + 16 j + r16]
+    float* cz = a.c32 + (long)z * a.nnz * 1024;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int ob = 2 * wm + (i >> 1);
+        if (ob >= gn) continue;
+        const int* blks = a.seg_blk + a.seg_ptr[row0 + ob] + j0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int jb = 2 * wn + (j >> 1);
+            if (jb >= jn) continue;
+            float* cb = cz + (long)blks[jb] * 1024 + (16 * (i & 1) + 4 * g) * 32 + 16 * (j & 1) + r16;
+#pragma unroll
+            for (int x = 0; x < 4; ++x) unsafeAtomicAdd(cb + 32 * x, acc[i][j][x]);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
 // DSD: dense = sparse x dense
 // ---------------------------------------------------------------------------------------
 struct DxdArgs {
@@ -1367,6 +1491,31 @@ extern "C" int flyhip_bs_sdd(const void* a, const void* b, void* c, const int32_
     dim3 grid((unsigned)nblocks, Z);
     BS_DISPATCH(bs_sdd_kernel, grid, args)
     return check_launch("bs_sdd_kernel");
+}
+
+extern "C" int flyhip_bs_sdd_kmajor(const void* a, const void* b, float* c32,
+                                    const int32_t* row_ptr, const int32_t* row_blk, const int32_t* row_col,
+                                    const int32_t* grp_row0, const int32_t* grp_n, int n_grp, int max_row_nnz,
+                                    int brows_per_head, int nnz, int Z, int K, int k_slice, int blk,
+                                    int64_t a_sz, int64_t a_sh, int64_t a_sk,
+                                    int64_t b_sz, int64_t b_sh, int64_t b_sk,
+                                    int dtype, void* stream) {
+    int rc = check_common("bs_sdd_kmajor", blk, dtype, Z);
+    if (rc) return rc;
+    FLY_REQUIRE(a && b && c32 && row_ptr && row_blk && row_col && grp_row0 && grp_n, "bs_sdd_kmajor: null pointer");
+    FLY_REQUIRE(blk == 32 && (dtype == BF16 || dtype == F16), "bs_sdd_kmajor: needs 32x32 blocks of bf16 / fp16");
+    FLY_REQUIRE(n_grp > 0 && max_row_nnz > 0 && brows_per_head > 0 && nnz > 0 && K > 0, "bs_sdd_kmajor: bad sizes");
+    FLY_REQUIRE(k_slice >= 32 && k_slice % 32 == 0, "bs_sdd_kmajor: k_slice must be a positive multiple of 32");
+    FLY_REQUIRE(((a_sz | a_sh | a_sk | b_sz | b_sh | b_sk) % 8) == 0, "bs_sdd_kmajor: strides must be multiples of 8 elements");
+    const int chunks = (max_row_nnz + 3) / 4, slices = (K + k_slice - 1) / k_slice;
+    FLY_REQUIRE((long)n_grp * chunks <= 2147483647L && slices <= 65535, "bs_sdd_kmajor: too many workgroups");
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    SddKArgs args{a, b, c32, row_ptr, row_blk, row_col, grp_row0, grp_n, brows_per_head, K, k_slice, chunks, nnz,
+                  a_sz, a_sh, a_sk, b_sz, b_sh, b_sk};
+    dim3 grid((unsigned)(n_grp * chunks), slices, Z);
+    if (dtype == BF16) hipLaunchKernelGGL((bs_sdd32k_kernel<bf16_t>), grid, dim3(256), 0, st, args);
+    else hipLaunchKernelGGL((bs_sdd32k_kernel<f16_t>), grid, dim3(256), 0, st, args);
+    return check_launch("bs_sdd32k_kernel");
 }
 
 extern "C" int flyhip_bs_dsd(const void* a_sp, const void* b, void* c,

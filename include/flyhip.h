@@ -144,6 +144,23 @@ int flyhip_bs_sdd(const void* a, const void* b, void* c, const int32_t* lut, int
                   int64_t b_sz, int64_t b_sh, int64_t b_sn, int64_t b_sk,
                   int dtype, void* stream);
 
+/* SDD with the contraction index slowest in both operands: c32[z, n] += A[z, h_n, :, block-row i_n]^T .
+ * B[z, h_n, :, block-col j_n], A (Z,H,K,M) and B (Z,H,K,N) with (batch, head, k) strides and contiguous
+ * features -- the weight gradient x^T dy of a block-sparse linear layer, K = tokens (ref: the 'sdd'
+ * call of the backward pass, blocksparse_matmul.py:562-587 -> _sdd_matmul :279-346).  32x32 blocks
+ * of bf16 / fp16.  c32 is fp32 (Z, nnz, 32, 32), ZEROED by the caller: slices of k_slice tokens
+ * (a multiple of 32) are accumulated into it with float atomics; the caller rounds it to the
+ * output type.  row_ptr / row_blk / row_col as in flyhip_bs_sdd; grp_row0 / grp_n: groups of at most
+ * four consecutive block-rows of a head with identical column lists (every block-row in exactly one
+ * group); max_row_nnz = the longest column list. */
+int flyhip_bs_sdd_kmajor(const void* a, const void* b, float* c32,
+                         const int32_t* row_ptr, const int32_t* row_blk, const int32_t* row_col,
+                         const int32_t* grp_row0, const int32_t* grp_n, int n_grp, int max_row_nnz,
+                         int brows_per_head, int nnz, int Z, int K, int k_slice, int blk,
+                         int64_t a_sz, int64_t a_sh, int64_t a_sk,
+                         int64_t b_sz, int64_t b_sh, int64_t b_sk,
+                         int dtype, void* stream);
+
 /* DSD: c (Z,H,M,N) = op(sparse a) . dense b.  Segment s = (head, output block-row); seg_ptr
  * (n_seg+1), seg_blk (block id), seg_inner (inner block index) int32 list the blocks reduced into
  * it; n_seg = H * M/blk; an empty segment writes zeros (ref: make_dxx_lut :356-441 plays this

@@ -329,3 +329,47 @@ def test_blocksparse_attention_module_fused_path():
     assert len(mod.ops_cache) == 1
     outg.float().sum().backward()
     assert qg.grad is not None and bool(torch.isfinite(qg.grad.float()).all())
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('p,r,K', [(8, 6, 1024), (5, 7, 2000), (12, 3, 777 * 16)])
+def test_sdd_with_contraction_major_operands(p, r, K, dtype):
+    """sparse = a^T b with a (K, M), b (K, N) and a long K -- the weight gradient of a block-sparse linear
+    layer -- on the split-K kernel (fp32 accumulation over slices of K), with rows that share column
+    lists (groups of up to four), rows that do not, an empty row, and K not a multiple of the step."""
+    from fly_amd import matmul
+    print('case', p, r, K, dtype, flush=True)
+    Z, H, block = 1, 2, 32
+    layout = random_layout(H, p, r, 17 * p + r, density=0.5)
+    layout[0, :4] = layout[0, 0]                          # a group of four rows with one column list
+    layout[1, min(2, p - 1)] = 0                          # an empty block-row
+    g = torch.Generator().manual_seed(K)
+    a = torch.randn(Z, H, K, p * block, generator=g).to(dtype)
+    b = torch.randn(Z, H, K, r * block, generator=g).to(dtype)
+    op = matmul(layout, block, 'sdd', trans_a=True, trans_b=False)
+    out = op(a.to(DEV), b.to(DEV))
+    ref = ob.sdd(a.double(), b.double(), layout, block, trans_a=True, trans_b=False)
+    assert out.shape == ref.shape and out.dtype == dtype
+    assert rel_err(out, ref) <= TOL[dtype]
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('trans_b', [True, False])
+def test_fast_dds_both_block_orientations(trans_b, dtype):
+    """dense = x . op(sparse) on the tiled kernel for 2-byte types: blocks read as they are (y = x W^T,
+    the forward of the Pixelfly linear) and transposed on their way into LDS (dx = dy W, its input
+    gradient); token counts that are not multiples of the tile, grouped and ungrouped segments."""
+    from fly_amd import matmul
+    print('case', trans_b, dtype, flush=True)
+    Z, H, block, p, r, M = 1, 2, 32, 9, 7, 333
+    layout = random_layout(H, p, r, 23, density=0.5)
+    layout[0, :3] = layout[0, 0]
+    layout[1, :, 1] = 0                                   # an empty block-column
+    g = torch.Generator().manual_seed(9)
+    nnz = int(layout.sum())
+    w = torch.randn(Z, nnz, block, block, generator=g).to(dtype)
+    x = torch.randn(Z, H, M, (r if trans_b else p) * block, generator=g).to(dtype)
+    out = matmul(layout, block, 'dds', trans_a=False, trans_b=trans_b)(x.to(DEV), w.to(DEV))
+    ref = ob.dds(x.double(), w.double(), layout, block, False, trans_b)
+    assert out.shape == ref.shape
+    assert rel_err(out, ref) <= TOL[dtype]
