@@ -319,14 +319,16 @@ __global__ __launch_bounds__(256) void bs_sdd32k_kernel(const SddKArgs a) {
     const uint16_t* ap = reinterpret_cast<const uint16_t*>(a.a) + z * a.a_sz + head * a.a_sh + (long)brow0 * 32;
     const uint16_t* bp = reinterpret_cast<const uint16_t*>(a.b) + z * a.b_sz + head * a.b_sh;
 
-    // staging: piece c = tid + 256 i (i < 2) of each tile is token c / 16, features 8 (c % 16) .. + 7;
-    // feature block c % 16 / 4 is output block-row ob (A) or list entry j0 + jb (B); absent blocks read
+    // staging: piece c = tid + 256 i (i < 2) of each tile is token c % 32, features 8 (c / 32) .. + 7 -- the
+    // token runs fastest over the lanes, so that the 2-byte stores that transpose the piece into
+    // [feature][token] spread over the LDS banks (with the feature fastest they pile onto four).
+    // Feature block c / 32 / 4 is output block-row ob (A) or list entry j0 + jb (B); absent blocks read
     // block 0 of the tile and are zeroed when parked
     int fcol_a[2], fcol_b[2];                               // feature offset of the piece in its operand
     bool live_a[2], live_b[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-        const int c = tid + 256 * i, fb = (c & 15) >> 2, f8 = 8 * (c & 3);
+        const int c = tid + 256 * i, fb = (c >> 5) >> 2, f8 = 8 * ((c >> 5) & 3);
         live_a[i] = fb < gn;
         live_b[i] = fb < jn;
         fcol_a[i] = 32 * (live_a[i] ? fb : 0) + f8;
@@ -336,7 +338,7 @@ __global__ __launch_bounds__(256) void bs_sdd32k_kernel(const SddKArgs a) {
     auto fetch = [&](int kt) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-            const int tok = min(kt + ((tid + 256 * i) >> 4), a.K - 1);     // clamped; tokens past k1 are zeroed below
+            const int tok = min(kt + ((tid + 256 * i) & 31), a.K - 1);     // clamped; tokens past k1 are zeroed below
             ra[i] = *reinterpret_cast<const uintx4*>(ap + (long)tok * a.a_sk + fcol_a[i]);
             rb[i] = *reinterpret_cast<const uintx4*>(bp + (long)tok * a.b_sk + fcol_b[i]);
         }
@@ -344,7 +346,7 @@ __global__ __launch_bounds__(256) void bs_sdd32k_kernel(const SddKArgs a) {
     auto stash = [&](int buf, int kt) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-            const int c = tid + 256 * i, tok = c >> 4, f0 = 8 * (c & 15);
+            const int c = tid + 256 * i, tok = c & 31, f0 = 8 * (c >> 5);
             const bool in = kt + tok < k1;
             const uintx4 va = (live_a[i] && in) ? ra[i] : uintx4{0, 0, 0, 0};
             const uintx4 vb = (live_b[i] && in) ? rb[i] : uintx4{0, 0, 0, 0};
