@@ -239,7 +239,24 @@ def bench_other_configs():
         'fc1_ms': ms1, 'fc1_tflops': fl / ms1 / 1e9, 'fc2_ms': ms2, 'fc2_tflops': fl / ms2 / 1e9,
         'fc1_hbm_gbs': (x.numel() + 50176 * 3072 + 864 * 1024) * 2 / ms1 / 1e6,
         'dense_library_gemm_768_3072_ms': msd}
-    del x, h, w, fc1, fc2
+
+    # one training step of the layer: forward, input gradient (DDS on untransposed blocks) and weight
+    # gradient (split-K SDD), beside the same for a dense nn.Linear of the same shape
+    def fwd_bwd(mod, inp):
+        def run():
+            y = mod(inp)
+            y.backward(gy[: y.numel()].view_as(y))
+            inp.grad = None
+            for p_ in mod.parameters():
+                p_.grad = None
+        return run
+    gy = torch.randn(50176 * 3072, generator=g).bfloat16().to(dev)
+    xg, hg = x.clone().requires_grad_(), h.clone().requires_grad_()
+    dense = torch.nn.Linear(768, 3072, bias=False).to(dev).to(torch.bfloat16)
+    out['config4_pixelfly_linear_bf16'].update({
+        'fc1_fwd_bwd_ms': timeit(fwd_bwd(fc1, xg), n=5), 'fc2_fwd_bwd_ms': timeit(fwd_bwd(fc2, hg), n=5),
+        'dense_768_3072_fwd_bwd_ms': timeit(fwd_bwd(dense, xg), n=5)})
+    del x, h, w, fc1, fc2, gy, xg, hg, dense
 
     B, L, H, E, mh, lc = 1, 16384, 16, 64, 128, 1024
     q, k, v = (torch.randn(B, L, H, E, generator=g) for _ in range(3))
