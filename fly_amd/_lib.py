@@ -28,6 +28,7 @@ SIGNATURES = {
     'flyhip_bs_attn': [c_vp] * 7 + [c_int, c_vp, c_i64] + [c_int] * 5 + [c_i64] * 12 + [c_float, c_int, c_vp],
     'flyhip_bs_softmax': [c_vp] * 4 + [c_int] * 5 + [c_i64, c_float, c_vp, c_i64, c_int, c_vp, c_i64,
                                                     c_int, c_int, c_vp],
+    'flyhip_bs_softmax_bwd': [c_vp] * 5 + [c_int] * 4 + [c_i64, c_float, c_int, c_vp],
     'flyhip_bs_rowreduce': [c_vp] * 4 + [c_int] * 3 + [c_i64, c_int, c_int, c_vp],
 }
 

@@ -95,6 +95,17 @@ class _SoftmaxFn(torch.autograd.Function):
     def backward(ctx, dy):
         (y,) = ctx.saved_tensors
         op = ctx.op
+        ptr, blk, col, max_nnz = op.make_lut(y.device)
+        if (op.block == 32 and y.dtype in (torch.bfloat16, torch.float16) and max_nnz <= 64
+                and y.stride(0) % 8 == 0):
+            dy = dy.contiguous()
+            dx = torch.empty_like(y)
+            H, p, r = op.spdims
+            with torch.cuda.device(y.device):
+                _lib.call('flyhip_bs_softmax_bwd', y.data_ptr(), dy.data_ptr(), dx.data_ptr(), ptr.data_ptr(),
+                          blk.data_ptr(), H * p, max_nnz, y.shape[0], 32, y.stride(0), ctx.scale,
+                          _lib.dtype_code(y), _lib.stream_ptr(y.device))
+            return dx, None, None, None, None
         dyy = (dy * y).contiguous()
         rows = _reduce_rows(op, dyy, 1)                                   # (Z, H, M)
         dx = (dyy - y * sparsify_broadcast_tensor(rows, op.layout, op.block)) * ctx.scale

@@ -1336,6 +1336,72 @@ __global__ __launch_bounds__(256) void bs_softmax32_kernel(RowArgs a) {
         }
 }
 
+// Backward of the block softmax for 32x32 blocks of a 2-byte type, one pass: dx = scale * y * (dy - sum_row(dy * y)).
+// Same work split as bs_softmax32_kernel (workgroup per (block-row, 16-row half), wave w takes blocks
+// w, w+4, ...; a lane holds 8 consecutive elements of one row per block): y and dy stay in registers
+// in their 2-byte form between the row sum and the result, so HBM sees two reads and one write.
+struct RowBwdArgs {
+    const void* y; const void* dy; void* dx;
+    const int32_t* row_ptr; const int32_t* row_blk;
+    long y_sz;
+    float scale;
+};
+
+template <typename T, int MAXB>
+__global__ __launch_bounds__(256) void bs_softmax32_bwd_kernel(RowBwdArgs a) {
+    __shared__ float red[4][16];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, rl = lane >> 2, chunk = lane & 3;
+    const int brow = blockIdx.x >> 1, row = (blockIdx.x & 1) * 16 + rl;
+    const int z = blockIdx.y;
+    const int p0 = a.row_ptr[brow], nb = a.row_ptr[brow + 1] - p0;
+    const long base = z * a.y_sz + row * 32 + chunk * 8;
+    const T* yz = reinterpret_cast<const T*>(a.y) + base;
+    const T* dz = reinterpret_cast<const T*>(a.dy) + base;
+    T* xz = reinterpret_cast<T*>(a.dx) + base;
+
+    uintx4 ry[MAXB], rd[MAXB];
+    int blk[MAXB];
+#pragma unroll
+    for (int it = 0; it < MAXB; ++it) {
+        const int j = w + 4 * it;
+        blk[it] = -1;
+        if (j < nb) {
+            blk[it] = a.row_blk[p0 + j];
+            ry[it] = __builtin_nontemporal_load(reinterpret_cast<const uintx4*>(yz + (long)blk[it] * 1024));
+            rd[it] = __builtin_nontemporal_load(reinterpret_cast<const uintx4*>(dz + (long)blk[it] * 1024));
+        }
+    }
+    auto elem = [&](uint32_t word, int hi) -> float {
+        T e;
+        *reinterpret_cast<uint16_t*>(&e) = hi ? (uint16_t)(word >> 16) : (uint16_t)(word & 0xffffu);
+        return Elem<T>::to_f32(e);
+    };
+    float s = 0.f;
+#pragma unroll
+    for (int it = 0; it < MAXB; ++it)
+        if (blk[it] >= 0)
+#pragma unroll
+            for (int u = 0; u < 8; ++u) s += elem(ry[it][u >> 1], u & 1) * elem(rd[it][u >> 1], u & 1);
+    s += __shfl_xor(s, 1);
+    s += __shfl_xor(s, 2);
+    if (chunk == 0) red[w][rl] = s;
+    __syncthreads();
+    s = (red[0][rl] + red[1][rl]) + (red[2][rl] + red[3][rl]);
+#pragma unroll
+    for (int it = 0; it < MAXB; ++it)
+        if (blk[it] >= 0) {
+            uint32_t outw[4];
+#pragma unroll
+            for (int u2 = 0; u2 < 4; ++u2) {
+                const float lo = a.scale * elem(ry[it][u2], 0) * (elem(rd[it][u2], 0) - s);
+                const float hi = a.scale * elem(ry[it][u2], 1) * (elem(rd[it][u2], 1) - s);
+                outw[u2] = pack2<T>(lo, hi);
+            }
+            __builtin_nontemporal_store(uintx4{outw[0], outw[1], outw[2], outw[3]},
+                                        reinterpret_cast<uintx4*>(xz + (long)blk[it] * 1024));
+        }
+}
+
 // rows longer than the register budget: three passes over the row
 template <typename T>
 __global__ __launch_bounds__(256) void bs_softmax_long_kernel(RowArgs a) {
@@ -1688,6 +1754,28 @@ extern "C" int flyhip_bs_softmax(void* x, const int32_t* row_ptr, const int32_t*
         case BF16: return launch_softmax<bf16_t>(args, grid, max_elems, st);
         default: return launch_softmax<f16_t>(args, grid, max_elems, st);
     }
+}
+
+extern "C" int flyhip_bs_softmax_bwd(const void* y, const void* dy, void* dx,
+                                     const int32_t* row_ptr, const int32_t* row_blk,
+                                     int n_brow, int max_row_nnz, int Z, int blk, int64_t y_sz,
+                                     float scale, int dtype, void* stream) {
+    int rc = check_common("bs_softmax_bwd", blk, dtype, Z);
+    if (rc) return rc;
+    FLY_REQUIRE(y && dy && dx && row_ptr && row_blk, "bs_softmax_bwd: null pointer");
+    FLY_REQUIRE(blk == 32 && (dtype == BF16 || dtype == F16), "bs_softmax_bwd: needs 32x32 blocks of bf16 / fp16");
+    FLY_REQUIRE(n_brow > 0 && max_row_nnz >= 0 && max_row_nnz <= 64, "bs_softmax_bwd: at most 64 blocks per block-row (got %d)", max_row_nnz);
+    FLY_REQUIRE(y_sz % 8 == 0, "bs_softmax_bwd: batch stride must be a multiple of 8 elements");
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    RowBwdArgs args{y, dy, dx, row_ptr, row_blk, y_sz, scale};
+    dim3 grid(2 * n_brow, Z);
+    const int slots = (max_row_nnz + 3) / 4;
+#define SMB(T, N) hipLaunchKernelGGL((bs_softmax32_bwd_kernel<T, N>), grid, dim3(256), 0, st, args)
+#define SMB_T(T) do { if (slots <= 4) SMB(T, 4); else if (slots <= 8) SMB(T, 8); else if (slots <= 13) SMB(T, 13); else SMB(T, 16); } while (0)
+    if (dtype == BF16) SMB_T(bf16_t); else SMB_T(f16_t);
+#undef SMB_T
+#undef SMB
+    return check_launch("bs_softmax32_bwd_kernel");
 }
 
 extern "C" int flyhip_bs_rowreduce(const void* x, void* out, const int32_t* row_ptr, const int32_t* row_blk,

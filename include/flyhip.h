@@ -231,6 +231,15 @@ int flyhip_bs_softmax(void* x, const int32_t* row_ptr, const int32_t* row_blk, c
                       const float* am, int64_t am_stride, int am_mul,
                       int dtype, void* stream);
 
+/* Backward of flyhip_bs_softmax without masks in the gradient: dx = scale * y * (dy - rowsum(dy * y)) over
+ * the nonzero blocks, y the softmax output (ref: the backward of triton.ops.blocksparse.softmax,
+ * reached from blocksparse_attention.py:146-152 under autograd).  32x32 blocks of bf16 / fp16, at most
+ * 64 blocks per block-row; y, dy, dx (Z, nnz, 32, 32) contiguous per batch, batch stride y_sz. */
+int flyhip_bs_softmax_bwd(const void* y, const void* dy, void* dx,
+                          const int32_t* row_ptr, const int32_t* row_blk,
+                          int n_brow, int max_row_nnz, int Z, int blk, int64_t y_sz,
+                          float scale, int dtype, void* stream);
+
 /* Row reduction over nonzero blocks -> out (Z, n_brow*blk) in x's dtype: op 0 = logsumexp
  * (ref: blocksparse_logsumexp.py:161-184), op 1 = sum (ref: blocksparse_sum.py:156-179).
  * Rows of an empty block-row give 0. */

@@ -211,3 +211,33 @@ def test_row_ops_backward_match_dense_autograd():
             (ref * wr).sum().backward()
         assert rel_err(y, ref) <= 1e-5
         assert rel_err(x.grad, xd.grad) <= 1e-5, name
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('p,r', [(4, 6), (3, 40), (5, 61)])
+def test_softmax_backward_kernel_matches_dense_autograd(p, r, dtype):
+    """The one-pass gradient kernel of the block softmax (32x32 blocks, 2-byte types; 4 / 13 / 16
+    register slots) against autograd through the dense softmax on the same rounded inputs."""
+    from fly_amd import softmax
+    from fly_amd.blocksparse_utils import densify_tensor, sparsify_tensor
+    print('case', p, r, dtype, flush=True)
+    g = torch.Generator().manual_seed(10 * p + r)
+    block, Z, H = 32, 2, 2
+    layout = (torch.rand(H, p, r, generator=g) < 0.7).long()
+    layout[:, :, 0] = 1
+    layout[0, 1, :] = 1                                   # a full block-row: the longest column list
+    nnz = int(layout.sum())
+    x0 = torch.randn(Z, nnz, block, block, generator=g).to(dtype).to(DEV)
+    w = torch.randn(Z, nnz, block, block, generator=g).to(dtype).to(DEV)
+    kpm = torch.zeros(Z, r * block)
+    kpm[1, -37:] = float('-inf')
+    x = x0.clone().requires_grad_()
+    y = softmax(layout, block)(x * 1.0, scale=0.3, key_padding_mask=kpm.to(DEV))
+    (y.float() * w.float()).sum().backward()
+    xd = x0.float().clone().requires_grad_()
+    dense = densify_tensor(xd * 0.3, layout, float('-inf')) + kpm.to(DEV)[:, None, None, :]
+    ref = sparsify_tensor(torch.softmax(dense, dim=-1), layout)
+    (ref * w.float()).sum().backward()
+    assert x.grad.dtype == dtype
+    tol = 2e-2 if dtype == torch.bfloat16 else 4e-3
+    assert rel_err(x.grad.float(), xd.grad) <= tol, rel_err(x.grad.float(), xd.grad)
