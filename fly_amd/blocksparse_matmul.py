@@ -95,8 +95,8 @@ class matmul:
                 tabs = (sdd_table(self.layout),)
             elif kind in ('grp_rows', 'grp_cols'):
                 tabs = group_table(self.layout, by_rows=(kind == 'grp_rows'))
-            elif kind == 'union':
-                tabs = union_table(self.layout)
+            elif kind in ('union', 'union_t'):
+                tabs = union_table(self.layout, transposed=(kind == 'union_t'))
                 if int(self.layout.sum()) < UNION_MIN_SHARING * tabs[1].numel():
                     tabs = ()
             else:
@@ -217,7 +217,7 @@ class matmul:
         H, p, r = self.spdims
         by_rows = not trans_a
         seg_ptr, seg_blk, seg_inner = self._table('rows' if by_rows else 'cols', b.device)
-        uni = ([t.data_ptr() for t in self._table('union', b.device)] if by_rows else []) or [None] * 3
+        uni = [t.data_ptr() for t in self._table('union' if by_rows else 'union_t', b.device)] or [None] * 3
         per_head = p if by_rows else r
         M = per_head * self.block
         Z = b.shape[0]
@@ -234,6 +234,10 @@ class matmul:
         return c
 
     def _dds(self, a, b, trans_a, trans_b, trans_c):
+        if trans_a and trans_c and not trans_b:
+            # (a^T b)^T = b^T a: the same numbers as a dsd with the sparse operand transposed, which has
+            # a tiled kernel (this is the gradient of the second operand of an sdd, e.g. dK = dS^T Q)
+            return self._dsd(b, a, True, False, False)
         a = _dense_operand(a)
         b = b.contiguous()
         H, p, r = self.spdims

@@ -102,17 +102,21 @@ def row_table(layout):
     return ptr, blk, col, int(counts.max()) if counts.numel() else 0
 
 
-def union_table(layout, rows_per_group=4):
+def union_table(layout, rows_per_group=4, transposed=False):
     """Union of block-columns over groups of `rows_per_group` consecutive block-rows of a head
     (ceil(rows / rows_per_group) groups per head, head-major): returns (uni_ptr int32 (n_groups+1),
     uni_inner int32 (n_union) block-columns in increasing order per group, uni_blk int32
-    (n_union, rows_per_group) the block id at (row rows_per_group*g + w, that column) or -1)."""
+    (n_union, rows_per_group) the block id at (row rows_per_group*g + w, that column) or -1).
+    transposed=True: the same with the roles of rows and columns exchanged (groups of block-columns,
+    unions of their block-rows), block ids still those of the layout's own storage order."""
     layout = _as_layout3(layout).cpu().long()
+    ids = (torch.cumsum(layout.reshape(-1), 0) - 1).reshape(layout.shape)
+    ids = torch.where(layout > 0, ids, torch.full_like(ids, -1))
+    if transposed:
+        layout, ids = layout.transpose(1, 2), ids.transpose(1, 2)
     H, p, r = layout.shape
     R = rows_per_group
     G = (p + R - 1) // R
-    ids = (torch.cumsum(layout.reshape(-1), 0) - 1).reshape(H, p, r)
-    ids = torch.where(layout > 0, ids, torch.full_like(ids, -1))
     pad = torch.full((H, G * R - p, r), -1, dtype=ids.dtype)
     ids = torch.cat([ids, pad], dim=1).reshape(H, G, R, r)
     nz = (ids >= 0).any(dim=2).nonzero(as_tuple=False)              # (h, g, col), sorted

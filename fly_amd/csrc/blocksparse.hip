@@ -584,9 +584,11 @@ struct DsdUniArgs {
 };
 constexpr int DSDU_LD = 40;     // LDS row stride in elements ([column][k], 32 k + 8): 16 columns hit all banks once
 
-template <typename T>
+template <typename T, bool TA>     // TA: every sparse block is used transposed (segments are block-columns of the layout)
 __global__ __launch_bounds__(256) void bs_dsd32u_kernel(const DsdUniArgs a) {
     __shared__ __attribute__((aligned(16))) uint16_t vt[2][64 * DSDU_LD];
+    // TA: a wave turns its 32x32 block through a private LDS tile, [column][row]
+    __shared__ __attribute__((aligned(16))) uint16_t bt[TA ? 4 : 1][TA ? 32 * DSDU_LD : 8];
     const int tid = threadIdx.x, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int ntn = (a.N + 63) / 64;
@@ -656,6 +658,23 @@ __global__ __launch_bounds__(256) void bs_dsd32u_kernel(const DsdUniArgs a) {
         inner_n1 = inner_n2;
         id_n1 = id_n2;
         if (blk >= 0) {
+            if (TA) {
+                // the lane holds rows 16 tm + r16 of the block, columns 8g .. 8g + 7: they go to LDS as
+                // [column][row] and come back as fragments of the transposed block (a wave-private tile;
+                // LDS operations of a wave complete in order)
+                uint16_t* my = bt[w];
+#pragma unroll
+                for (int tm = 0; tm < 2; ++tm) {
+                    const uint32_t v[4] = {fs[tm].x, fs[tm].y, fs[tm].z, fs[tm].w};
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        my[(8 * g + e) * DSDU_LD + 16 * tm + r16] = (uint16_t)(v[e >> 1] >> (16 * (e & 1)));
+                }
+                __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                for (int tm = 0; tm < 2; ++tm) fs[tm] = *reinterpret_cast<const uint4*>(my + (16 * tm + r16) * DSDU_LD + 8 * g);
+                __builtin_amdgcn_wave_barrier();
+            }
             const uint16_t* tp = vt[s & 1];
 #pragma unroll
             for (int tn = 0; tn < 4; ++tn) {
@@ -1605,7 +1624,8 @@ extern "C" int flyhip_bs_dsd(const void* a_sp, const void* b, void* c,
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     DxdArgs args{a_sp, b, c, seg_ptr, seg_blk, seg_inner, n_seg, rows_per_head, N, trans_a,
                  a_sz, b_sz, b_sh, b_sk, b_sn, c_sz, c_sh, c_sm, c_sn, Z};
-    if (blk == 32 && (dtype == BF16 || dtype == F16) && !trans_a && b_sn == 1 && c_sn == 1 && N % 8 == 0 &&
+    if (blk == 32 && (dtype == BF16 || dtype == F16) && (!trans_a || (uni_ptr && uni_inner && uni_blk)) && b_sn == 1 &&
+        c_sn == 1 && N % 8 == 0 &&
         ((a_sz | b_sz | b_sh | b_sk | c_sz | c_sh | c_sm) % 8) == 0) {
         if (uni_ptr && uni_inner && uni_blk) {
             const int gph = (rows_per_head + 3) / 4, n_heads = n_seg / rows_per_head;
@@ -1614,8 +1634,13 @@ extern "C" int flyhip_bs_dsd(const void* a_sp, const void* b, void* c,
             const long nwg = unit_grid((long)n_heads * Z, (long)gph * ((N + 63) / 64));
             FLY_REQUIRE(nwg <= 2147483647L, "bs_dsd: too many workgroups");
             dim3 grid((unsigned)nwg);
-            if (dtype == BF16) hipLaunchKernelGGL((bs_dsd32u_kernel<bf16_t>), grid, dim3(256), 0, st, ua);
-            else hipLaunchKernelGGL((bs_dsd32u_kernel<f16_t>), grid, dim3(256), 0, st, ua);
+            if (dtype == BF16) {
+                if (trans_a) hipLaunchKernelGGL((bs_dsd32u_kernel<bf16_t, true>), grid, dim3(256), 0, st, ua);
+                else hipLaunchKernelGGL((bs_dsd32u_kernel<bf16_t, false>), grid, dim3(256), 0, st, ua);
+            } else {
+                if (trans_a) hipLaunchKernelGGL((bs_dsd32u_kernel<f16_t, true>), grid, dim3(256), 0, st, ua);
+                else hipLaunchKernelGGL((bs_dsd32u_kernel<f16_t, false>), grid, dim3(256), 0, st, ua);
+            }
             return check_launch("bs_dsd32u_kernel");
         }
         const long nwg = unit_grid((long)(n_seg / rows_per_head) * Z, (long)rows_per_head * ((N + 63) / 64));

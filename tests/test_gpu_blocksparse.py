@@ -373,3 +373,33 @@ def test_fast_dds_both_block_orientations(trans_b, dtype):
     ref = ob.dds(x.double(), w.double(), layout, block, False, trans_b)
     assert out.shape == ref.shape
     assert rel_err(out, ref) <= TOL[dtype]
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('p,r,N', [(8, 8, 64), (11, 6, 72), (5, 13, 128)])
+def test_dsd_with_transposed_sparse_operand(p, r, N, dtype):
+    """dense = sparse^T . dense (dV = P^T dO, and dK = dS^T Q which arrives as a transposed dds) on the
+    tiled kernel: groups of four block-columns share the dense tiles, every block is turned through
+    LDS.  Band-like layouts (neighbouring columns share rows) so that the shared-tile path is taken."""
+    from fly_amd import matmul
+    print('case', p, r, N, dtype, flush=True)
+    Z, H, block = 2, 2, 32
+    rows = torch.arange(p).view(-1, 1) * r // p
+    layout = ((rows - torch.arange(r).view(1, -1)).abs() <= 2).long().unsqueeze(0).repeat(H, 1, 1)
+    layout[1, :, r - 1] = 0                               # an empty block-column
+    nnz = int(layout.sum())
+    g = torch.Generator().manual_seed(p * r)
+    sp = torch.randn(Z, nnz, block, block, generator=g).to(dtype)
+    dn = torch.randn(Z, H, p * block, N, generator=g).to(dtype)
+    op = matmul(layout, block, 'dsd', trans_a=True, trans_b=False)
+    out = op(sp.to(DEV), dn.to(DEV))
+    ref = ob.dsd(sp.double(), dn.double(), layout, block, trans_a=True, trans_b=False)
+    assert out.shape == ref.shape == (Z, H, r * block, N)
+    assert rel_err(out, ref) <= TOL[dtype]
+    assert float(out[:, 1, (r - 1) * block:].abs().max()) == 0.0
+    # the same numbers through the dds form the backward pass of an sdd produces: (a^T b)^T
+    a = dn.transpose(2, 3).contiguous()                   # (Z, H, N, p*block): op(a) = a is (N x K)
+    out2 = matmul(layout, block, 'dds', trans_a=False, trans_b=False)(a.to(DEV), sp.to(DEV))
+    ref2 = ob.dds(a.double(), sp.double(), layout, block, False, False)
+    assert rel_err(out2, ref2) <= TOL[dtype]
+    assert rel_err(out2.transpose(2, 3), ref) <= TOL[dtype]
