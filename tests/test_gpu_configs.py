@@ -241,3 +241,38 @@ def test_softmax_backward_kernel_matches_dense_autograd(p, r, dtype):
     assert x.grad.dtype == dtype
     tol = 2e-2 if dtype == torch.bfloat16 else 4e-3
     assert rel_err(x.grad.float(), xd.grad) <= tol, rel_err(x.grad.float(), xd.grad)
+
+
+def test_bf16_gradients_on_the_tiled_kernels():
+    """The gradient paths of the 2-byte tiled kernels against autograd through the dense formulas on the
+    same rounded inputs: dQ / dK (dsd, transposed dsd), dP (sdd), dV (transposed dsd) of an attention-like
+    sdd -> dsd chain on a band layout, and dx (dds on untransposed blocks) / dW (split-K sdd over 1024
+    tokens) of a block-sparse linear layer."""
+    from fly_amd import matmul
+    from fly_amd.blocksparse_utils import densify_tensor, sparsify_tensor
+    g = torch.Generator().manual_seed(1)
+    block, Z, H, nb, d = 32, 2, 2, 12, 64
+    r_ = torch.arange(nb)
+    layout = ((r_.view(-1, 1) - r_.view(1, -1)).abs() <= 2).long().unsqueeze(0).repeat(H, 1, 1)
+    bf = torch.bfloat16
+    q, k, v = (torch.randn(Z, H, nb * block, d, generator=g).to(bf).to(DEV).requires_grad_() for _ in range(3))
+    s = matmul(layout, block, 'sdd', trans_b=True)(q, k)
+    o = matmul(layout, block, 'dsd')(s * 0.05, v)
+    w = torch.randn(o.shape, generator=g).to(DEV)
+    (o.float() * w).sum().backward()
+    q2, k2, v2 = (x.detach().float().requires_grad_() for x in (q, k, v))
+    s2 = sparsify_tensor(q2 @ k2.transpose(-1, -2), layout)
+    o2 = densify_tensor(s2 * 0.05, layout) @ v2
+    (o2 * w).sum().backward()
+    for got, ref, name in ((q.grad, q2.grad, 'dq'), (k.grad, k2.grad, 'dk'), (v.grad, v2.grad, 'dv')):
+        assert rel_err(got.float(), ref) <= 3e-2, (name, rel_err(got.float(), ref))
+
+    lay1 = layout[0]
+    x = torch.randn(1, 1, 1024, nb * block, generator=g).to(bf).to(DEV).requires_grad_()
+    wsp = (torch.randn(1, int(lay1.sum()), block, block, generator=g) * 0.1).to(bf).to(DEV).requires_grad_()
+    y = matmul(lay1, block, 'dds', trans_b=True)(x, wsp)
+    wy = torch.randn(y.shape, generator=g).to(bf).to(DEV)
+    y.backward(wy)
+    x2, w2 = x.detach().float().requires_grad_(), wsp.detach().float().requires_grad_()
+    (x2 @ densify_tensor(w2, lay1.unsqueeze(0)).transpose(-1, -2)).backward(wy.float())
+    assert rel_err(x.grad.float(), x2.grad) <= 2e-2 and rel_err(wsp.grad.float(), w2.grad) <= 2e-2
