@@ -177,6 +177,17 @@ def bench_blocksparse(steps, warmup):
     got = fused(q, k, v, 0.125).float()
     ms = timeit(lambda: fused(q, k, v, 0.125))
     out['three_stage_attention_ms'] = ms3
+    # a training step of the same attention (the three ops are autograd functions; the gradients run
+    # on the tiled SDD / DSD kernels, the transposed-DSD kernel and the one-pass softmax gradient)
+    qg, kg, vg = (t.detach().clone().requires_grad_() for t in (q, k, v))
+    go = torch.randn(B, H, L, d, generator=g).bfloat16().to(dev)
+
+    def train_step():
+        o = dsd(sm(sdd(qg, kg), scale=0.125), vg)
+        o.backward(go)
+        qg.grad = kg.grad = vg.grad = None
+    out['three_stage_attention_fwd_bwd_ms'] = timeit(train_step)
+    del qg, kg, vg, go
     out['fused_attention'] = {'ms': ms, 'tflops': 2 * flops / ms / 1e9, 'mfma_bf16_frac': 2 * flops / ms / 1e9 / 2500.0,
                               'speedup_over_three_stages': ms3 / ms,
                               'max_diff_vs_three_stages': float((got - ref).abs().max() / ref.abs().max())}
