@@ -1259,10 +1259,10 @@ __global__ __launch_bounds__(256) void bs_softmax_kernel(RowArgs a) {
 // load per lane (lane = 4*row + chunk of 8 columns); wave w owns blocks w, w+4, ... of the row and
 // keeps them in registers (raw 2-byte form) across the max / sum / write passes, so HBM sees each
 // element once in and once out.  Row statistics go quad -> wave (DPP) -> workgroup (LDS).
-template <typename T, int MAXB>
-__global__ __launch_bounds__(256) void bs_softmax32_kernel(RowArgs a) {
+template <typename T, int MAXB, int NW>     // NW waves share a (block-row, 16-row half); wave w takes blocks w, w + NW, ...
+__global__ __launch_bounds__(64 * NW) void bs_softmax32_kernel(RowArgs a) {
     constexpr float LOG2E = 1.4426950408889634f;
-    __shared__ float red[2][4][16];
+    __shared__ float red[2][NW][16];
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, rl = lane >> 2, chunk = lane & 3;
     const int brow = blockIdx.x >> 1, row = (blockIdx.x & 1) * 16 + rl;       // row inside the block
     const int z = blockIdx.y;
@@ -1275,7 +1275,7 @@ __global__ __launch_bounds__(256) void bs_softmax32_kernel(RowArgs a) {
     long off[MAXB];
 #pragma unroll
     for (int it = 0; it < MAXB; ++it) {
-        const int j = w + 4 * it;
+        const int j = w + NW * it;
         off[it] = -1;
         if (j < nb) {
             off[it] = (long)a.row_blk[p0 + j] * 1024;
@@ -1293,7 +1293,7 @@ __global__ __launch_bounds__(256) void bs_softmax32_kernel(RowArgs a) {
     };
     // additive mask term of that element (masked launches only)
     auto mask_of = [&](int it, int u) -> float {
-        const long col = (long)a.row_col[p0 + w + 4 * it] * 32 + chunk * 8 + u;
+        const long col = (long)a.row_col[p0 + w + NW * it] * 32 + chunk * 8 + u;
         float v = 0.f;
         if (a.kpm) v += mask_term(a.kpm[z * a.kpm_stride + col], a.kpm_mul);
         if (a.am) v += mask_term(a.am[grow * a.am_stride + col], a.am_mul);
@@ -1319,7 +1319,9 @@ __global__ __launch_bounds__(256) void bs_softmax32_kernel(RowArgs a) {
     mx = fmaxf(mx, __shfl_xor(mx, 2));
     if (chunk == 0) red[0][w][rl] = mx;
     __syncthreads();
-    mx = fmaxf(fmaxf(red[0][0][rl], red[0][1][rl]), fmaxf(red[0][2][rl], red[0][3][rl]));
+    mx = red[0][0][rl];
+#pragma unroll
+    for (int ww = 1; ww < NW; ++ww) mx = fmaxf(mx, red[0][ww][rl]);
     // pass 2: exponentials (kept as floats in registers) and their sum; -inf - -inf = NaN, kept
     const float mx2 = mx * LOG2E, scale2 = a.scale * LOG2E;
     float ev[MAXB][8];
@@ -1338,7 +1340,9 @@ __global__ __launch_bounds__(256) void bs_softmax32_kernel(RowArgs a) {
     sum += __shfl_xor(sum, 2);
     if (chunk == 0) red[1][w][rl] = sum;
     __syncthreads();
-    sum = (red[1][0][rl] + red[1][1][rl]) + (red[1][2][rl] + red[1][3][rl]);
+    sum = red[1][0][rl];
+#pragma unroll
+    for (int ww = 1; ww < NW; ++ww) sum += red[1][ww][rl];
     const float inv = 1.0f / sum;
     // pass 3: normalise, round once, store
 #pragma unroll
@@ -1357,7 +1361,7 @@ __global__ __launch_bounds__(256) void bs_softmax32_kernel(RowArgs a) {
 
 // Backward of the block softmax for 32x32 blocks of a 2-byte type, one pass: dx = scale * y * (dy - sum_row(dy * y)).
 // Same work split as bs_softmax32_kernel (workgroup per (block-row, 16-row half), wave w takes blocks
-// w, w+4, ...; a lane holds 8 consecutive elements of one row per block): y and dy stay in registers
+// w, w+NW, ...; a lane holds 8 consecutive elements of one row per block): y and dy stay in registers
 // in their 2-byte form between the row sum and the result, so HBM sees two reads and one write.
 struct RowBwdArgs {
     const void* y; const void* dy; void* dx;
@@ -1366,9 +1370,9 @@ struct RowBwdArgs {
     float scale;
 };
 
-template <typename T, int MAXB>
-__global__ __launch_bounds__(256) void bs_softmax32_bwd_kernel(RowBwdArgs a) {
-    __shared__ float red[4][16];
+template <typename T, int MAXB, int NW>
+__global__ __launch_bounds__(64 * NW) void bs_softmax32_bwd_kernel(RowBwdArgs a) {
+    __shared__ float red[NW][16];
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, rl = lane >> 2, chunk = lane & 3;
     const int brow = blockIdx.x >> 1, row = (blockIdx.x & 1) * 16 + rl;
     const int z = blockIdx.y;
@@ -1382,7 +1386,7 @@ __global__ __launch_bounds__(256) void bs_softmax32_bwd_kernel(RowBwdArgs a) {
     int blk[MAXB];
 #pragma unroll
     for (int it = 0; it < MAXB; ++it) {
-        const int j = w + 4 * it;
+        const int j = w + NW * it;
         blk[it] = -1;
         if (j < nb) {
             blk[it] = a.row_blk[p0 + j];
@@ -1405,7 +1409,9 @@ __global__ __launch_bounds__(256) void bs_softmax32_bwd_kernel(RowBwdArgs a) {
     s += __shfl_xor(s, 2);
     if (chunk == 0) red[w][rl] = s;
     __syncthreads();
-    s = (red[0][rl] + red[1][rl]) + (red[2][rl] + red[3][rl]);
+    s = red[0][rl];
+#pragma unroll
+    for (int ww = 1; ww < NW; ++ww) s += red[ww][rl];
 #pragma unroll
     for (int it = 0; it < MAXB; ++it)
         if (blk[it] >= 0) {
@@ -1704,11 +1710,13 @@ template <typename T>
 static int launch_softmax(const RowArgs& args, dim3 grid, int max_elems, hipStream_t st) {
     if (sizeof(T) == 2 && args.blk_shift == 5 && max_elems <= 32 * 4 * 16 && (args.x_sz % 8) == 0) {
         dim3 g2(2 * args.n_brow, grid.y);
-        const int slots = (max_elems / 32 + 3) / 4;          // blocks per wave: sizes the register arrays
-#define SM32(N) hipLaunchKernelGGL((bs_softmax32_kernel<T, N>), g2, dim3(256), 0, st, args)
-        if (slots <= 4) SM32(4); else if (slots <= 8) SM32(8); else if (slots <= 10) SM32(10);
-        else if (slots <= 12) SM32(12); else if (slots <= 13) SM32(13); else if (slots <= 14) SM32(14);
-        else SM32(16);
+        const int slots = (max_elems / 32 + 3) / 4;          // blocks per wave with four waves: sizes the register arrays
+#define SM32(N) hipLaunchKernelGGL((bs_softmax32_kernel<T, N, 4>), g2, dim3(256), 0, st, args)
+#define SM32W(N) hipLaunchKernelGGL((bs_softmax32_kernel<T, N, 8>), g2, dim3(512), 0, st, args)
+        if (slots <= 4) SM32(4); else if (slots <= 8) SM32(8);
+        else if (slots <= 10) SM32W(5); else if (slots <= 12) SM32W(6); else if (slots <= 14) SM32W(7);
+        else SM32W(8);
+#undef SM32W
 #undef SM32
         return check_launch("bs_softmax32_kernel");
     }
@@ -1795,7 +1803,8 @@ extern "C" int flyhip_bs_softmax_bwd(const void* y, const void* dy, void* dx,
     RowBwdArgs args{y, dy, dx, row_ptr, row_blk, y_sz, scale};
     dim3 grid(2 * n_brow, Z);
     const int slots = (max_row_nnz + 3) / 4;
-#define SMB(T, N) hipLaunchKernelGGL((bs_softmax32_bwd_kernel<T, N>), grid, dim3(256), 0, st, args)
+#define SMB(T, N) hipLaunchKernelGGL((bs_softmax32_bwd_kernel<T, N, 4>), grid, dim3(256), 0, st, args)
+    // (four waves measured faster than eight here -- 0.68 against 0.77 ms at config 2 -- the opposite of the forward kernel)
 #define SMB_T(T) do { if (slots <= 4) SMB(T, 4); else if (slots <= 8) SMB(T, 8); else if (slots <= 13) SMB(T, 13); else SMB(T, 16); } while (0)
     if (dtype == BF16) SMB_T(bf16_t); else SMB_T(f16_t);
 #undef SMB_T
