@@ -339,7 +339,7 @@ def test_sdd_with_contraction_major_operands(p, r, K, dtype):
     lists (groups of up to four), rows that do not, an empty row, and K not a multiple of the step."""
     from fly_amd import matmul
     print('case', p, r, K, dtype, flush=True)
-    Z, H, block = 1, 2, 32
+    Z, H, block = (2 if K < 2000 else 1), 2, 32
     layout = random_layout(H, p, r, 17 * p + r, density=0.5)
     layout[0, :4] = layout[0, 0]                          # a group of four rows with one column list
     layout[1, min(2, p - 1)] = 0                          # an empty block-row
