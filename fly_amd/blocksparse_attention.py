@@ -16,6 +16,52 @@ from .masking import FullMask, LengthMask, pad_mask
 from .padding import pad_to_multiple
 
 
+class _AttentionCoreFn(torch.autograd.Function):
+    """softmax(scale * q k^T + masks) v on the nonzero blocks, for calls that need gradients: the forward is
+    the reference's three ops (blocksparse_attention.py:134-160; the probabilities are kept for the
+    backward), the backward runs four kernels instead of the op-by-op chain's six plus elementwise passes:
+    dV = P^T dO, dS = scale * P * (dO V^T - rowsum(dO * O)) in one kernel (the sdd fused with the softmax
+    gradient), dQ = dS K, dK = dS^T Q.  32x32 blocks of bf16 / fp16 with shared-tile tables only."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, sdd, dsd, sm, scale, kpm, am):
+        p = sm(sdd._run('sdd', q, k, False, True, False), scale=scale, key_padding_mask=kpm, attn_mask=am,
+               key_padding_mask_mode='add', attn_mask_mode='add')
+        if kpm is not None or am is not None:
+            p.nan_to_num_()
+        out = dsd._run('dsd', p, v, False, False, False)
+        ctx.save_for_backward(q, k, v, p, out)
+        ctx.ops, ctx.scale = (sdd, dsd), scale
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        from . import _lib
+        q, k, v, p, out = ctx.saved_tensors
+        sdd, dsd = ctx.ops
+        dout = dout.contiguous()
+        dv = dsd._run('dsd', p, dout, True, False, False)
+        delta = (dout.float() * out.float()).sum(-1).contiguous()
+        H, rows, cols = sdd.spdims
+        uni_ptr, uni_inner, uni_blk = sdd._table('union', q.device)
+        ds = torch.empty_like(p)
+        vv = v if (v.stride(3) == 1 and all(s_ % 8 == 0 for s_ in v.stride()[:3])) else v.contiguous()
+        with torch.cuda.device(q.device):
+            _lib.call('flyhip_bs_sdd_dsoftmax', dout.data_ptr(), vv.data_ptr(), p.data_ptr(), delta.data_ptr(),
+                      ds.data_ptr(), uni_ptr.data_ptr(), uni_inner.data_ptr(), uni_blk.data_ptr(),
+                      p.shape[1], H, rows, q.shape[0], v.shape[3], 32,
+                      dout.stride(0), dout.stride(1), dout.stride(2), vv.stride(0), vv.stride(1), vv.stride(2),
+                      float(ctx.scale), _lib.dtype_code(q), _lib.stream_ptr(q.device))
+        dq = dsd._run('dsd', ds, k, False, False, False)
+        dk = dsd._run('dsd', ds, q, True, False, False)
+        return dq, dk, dv, None, None, None, None, None, None
+
+    @staticmethod
+    def supports(sdd, block, dtype, head_dim, device):
+        return (block == 32 and dtype in (torch.bfloat16, torch.float16) and head_dim % 32 == 0
+                and head_dim <= 128 and len(sdd._table('union', device)) == 3)
+
+
 def instantiate(cfg, *args, **kwargs):
     """Resolve a plugin description the way the reference's hydra.utils.instantiate call sites do
     (blocksparse_attention.py:39, blocksparse_linear.py:49, fastlinear.py:789): a mapping with a
@@ -57,6 +103,7 @@ class BlockSparseAttention(nn.Module):
         self._need_layout_synchronization = True
         self.ops_cache = dict()
         self.fused_cache = dict()
+        self._layout_cache = dict()
         # forward passes that need neither gradients, attention weights, an attention mask nor
         # dropout run as ONE kernel (no score tensor in memory); set to False to force the three ops
         self.fuse = True
@@ -70,7 +117,13 @@ class BlockSparseAttention(nn.Module):
         block = self.sparsity_config.block
         if (T % block != 0) or (S % block != 0):
             raise ValueError(f'Sequence lengths, {T} and {S}, needs to be divisible by block size {block}!')
-        return self.master_layout[..., :T // block, :S // block].cpu()
+        # the host copy is made once per shape: the master layout does not change after construction
+        # (and synchronisation; the key carries its address and version counter in case it is replaced or
+        # loaded into), and a device-to-host copy per call would stall the stream
+        key = (T, S, self.master_layout.data_ptr(), self.master_layout._version)
+        if key not in self._layout_cache:
+            self._layout_cache[key] = self.master_layout[..., :T // block, :S // block].cpu()
+        return self._layout_cache[key]
 
     def get_ops(self, T, S=None):
         if S is None:
@@ -122,6 +175,13 @@ class BlockSparseAttention(nn.Module):
             out = self.fused_cache[T, S](q, k, v, softmax_temp, key_mask)
             return out.permute(0, 2, 1, 3)[:, :q_seqlen_og, :, :v_dim_og], None
         sdd_nt, dsd_nn, sparse_softmax = self.get_ops(T, S)
+        if (needs_grad and not need_weights and not (self.training and self.dropout.p > 0)
+                and E == value.shape[3] and _AttentionCoreFn.supports(sdd_nt, block, query.dtype, E, query.device)):
+            out = _AttentionCoreFn.apply(
+                q, k, v, sdd_nt, dsd_nn, sparse_softmax, softmax_temp,
+                None if key_padding_mask is None else key_padding_mask.additive_matrix,
+                None if attn_mask is None else attn_mask.additive_matrix)
+            return out.permute(0, 2, 1, 3)[:, :q_seqlen_og, :, :v_dim_og], None
         qk = sdd_nt(q, k)
         attn = sparse_softmax(qk, scale=softmax_temp,
                               key_padding_mask=None if key_padding_mask is None else key_padding_mask.additive_matrix,

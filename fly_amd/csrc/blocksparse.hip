@@ -187,9 +187,12 @@ struct SddUniArgs {
     const int32_t* uni_ptr; const int32_t* uni_inner; const int32_t* uni_blk;
     int nnz, brows_per_head, grps_per_head, n_heads, Z;
     long a_sz, a_sh, a_sm, b_sz, b_sh, b_sn;
+    // DSOFT: c = scale * p * (a b^T - delta[row]) on the nonzero blocks, the gradient of the scores of a
+    // softmax(scale * s) -> p -> p v chain from a = d out, b = v, delta = rowsum(d out * out)
+    const void* p; const float* delta; float scale;
 };
 
-template <typename T, int KS>     // KS = K / 32
+template <typename T, int KS, bool DSOFT = false>     // KS = K / 32
 __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
     constexpr int K = 32 * KS, LD = K + 8;              // LDS row stride: 16 rows of a tile hit all banks once
     constexpr int CPR = K / 8;                          // 16-byte chunks per tile row
@@ -209,6 +212,10 @@ __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
                   (long)(min(bi, a.brows_per_head - 1) * 32 + r16) * a.a_sm + 8 * g;
     const T* bz = reinterpret_cast<const T*>(a.b) + z * a.b_sz + head * a.b_sh;
     T* cz = reinterpret_cast<T*>(a.c) + (long)z * a.nnz * 1024;
+    // DSOFT: this lane's rows are 16 tm + r16 of block-row bi
+    const float* dlt = DSOFT ? a.delta + ((long)z * a.n_heads + head) * a.brows_per_head * 32 +
+                                   (long)min(bi, a.brows_per_head - 1) * 32 + r16
+                             : nullptr;
     uintx4 fa[2][KS];
 #pragma unroll
     for (int tm = 0; tm < 2; ++tm)
@@ -249,6 +256,13 @@ __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
         if (s + 1 < n) fetch(inner_n1);
         const bool mine = blk >= 0 && have_row;
         floatx4 acc[2][2];
+        uintx4 pv[2];
+        if (DSOFT && mine) {                              // requested before the products, used after them
+            const T* pp = reinterpret_cast<const T*>(a.p) + ((long)z * a.nnz + blk) * 1024;
+#pragma unroll
+            for (int tm = 0; tm < 2; ++tm)
+                pv[tm] = __builtin_nontemporal_load(reinterpret_cast<const uintx4*>(pp + (16 * tm + r16) * 32 + 8 * g));
+        }
         if (mine) {
             const uint16_t* tp = tile[s & 1];
             uintx4 fb[2][KS];
@@ -273,7 +287,21 @@ __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
             // lane holds C[m = 16tm + r16][n = 8g + 4tn + i]
             T* cp = cz + (long)blk * 1024;
 #pragma unroll
-            for (int tm = 0; tm < 2; ++tm) store8_f32(cp + (16 * tm + r16) * 32 + 8 * g, acc[tm][0], acc[tm][1]);
+            for (int tm = 0; tm < 2; ++tm) {
+                if (DSOFT) {
+                    const float dl = dlt[16 * tm];
+#pragma unroll
+                    for (int tn = 0; tn < 2; ++tn)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const uint32_t word = pv[tm][2 * tn + (i >> 1)];
+                            T e;
+                            *reinterpret_cast<uint16_t*>(&e) = (i & 1) ? (uint16_t)(word >> 16) : (uint16_t)(word & 0xffffu);
+                            acc[tm][tn][i] = a.scale * Elem<T>::to_f32(e) * (acc[tm][tn][i] - dl);
+                        }
+                }
+                store8_f32(cp + (16 * tm + r16) * 32 + 8 * g, acc[tm][0], acc[tm][1]);
+            }
         }
         inner_n1 = inner_n2;
         blk = blk_n1;
@@ -1547,7 +1575,7 @@ extern "C" int flyhip_bs_sdd(const void* a, const void* b, void* c, const int32_
         if (uni_ptr && uni_inner && uni_blk) {
             const int gph = (brows_per_head + 3) / 4;
             SddUniArgs ua{a, b, c, uni_ptr, uni_inner, uni_blk, nnz, brows_per_head, gph, n_heads, Z,
-                          a_sz, a_sh, a_sm, b_sz, b_sh, b_sn};
+                          a_sz, a_sh, a_sm, b_sz, b_sh, b_sn, nullptr, nullptr, 1.f};
             const long nwg = unit_grid((long)n_heads * Z, gph);
             FLY_REQUIRE(nwg <= 2147483647L, "bs_sdd: too many workgroups");
             dim3 grid((unsigned)nwg);
@@ -1584,6 +1612,38 @@ extern "C" int flyhip_bs_sdd(const void* a, const void* b, void* c, const int32_
     dim3 grid((unsigned)nblocks, Z);
     BS_DISPATCH(bs_sdd_kernel, grid, args)
     return check_launch("bs_sdd_kernel");
+}
+
+extern "C" int flyhip_bs_sdd_dsoftmax(const void* dout, const void* v, const void* p, const float* delta, void* ds,
+                                      const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
+                                      int nnz, int n_heads, int brows_per_head, int Z, int K, int blk,
+                                      int64_t a_sz, int64_t a_sh, int64_t a_sm,
+                                      int64_t b_sz, int64_t b_sh, int64_t b_sn,
+                                      float scale, int dtype, void* stream) {
+    int rc = check_common("bs_sdd_dsoftmax", blk, dtype, Z);
+    if (rc) return rc;
+    FLY_REQUIRE(dout && v && p && delta && ds && uni_ptr && uni_inner && uni_blk, "bs_sdd_dsoftmax: null pointer");
+    FLY_REQUIRE(blk == 32 && (dtype == BF16 || dtype == F16), "bs_sdd_dsoftmax: needs 32x32 blocks of bf16 / fp16");
+    FLY_REQUIRE(K % 32 == 0 && K >= 32 && K <= 128, "bs_sdd_dsoftmax: head dim %d not a multiple of 32 up to 128", K);
+    FLY_REQUIRE(nnz > 0 && n_heads > 0 && brows_per_head > 0, "bs_sdd_dsoftmax: bad sizes");
+    FLY_REQUIRE(((a_sz | a_sh | a_sm | b_sz | b_sh | b_sn) % 8) == 0, "bs_sdd_dsoftmax: strides must be multiples of 8 elements");
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    const int gph = (brows_per_head + 3) / 4;
+    SddUniArgs ua{dout, v, ds, uni_ptr, uni_inner, uni_blk, nnz, brows_per_head, gph, n_heads, Z,
+                  a_sz, a_sh, a_sm, b_sz, b_sh, b_sn, p, delta, scale};
+    const long nwg = unit_grid((long)n_heads * Z, gph);
+    FLY_REQUIRE(nwg <= 2147483647L, "bs_sdd_dsoftmax: too many workgroups");
+    dim3 grid((unsigned)nwg);
+#define SDDS_LAUNCH(T)                                                                                  \
+    switch (K / 32) {                                                                                   \
+        case 1: hipLaunchKernelGGL((bs_sdd32u_kernel<T, 1, true>), grid, dim3(256), 0, st, ua); break;  \
+        case 2: hipLaunchKernelGGL((bs_sdd32u_kernel<T, 2, true>), grid, dim3(256), 0, st, ua); break;  \
+        case 3: hipLaunchKernelGGL((bs_sdd32u_kernel<T, 3, true>), grid, dim3(256), 0, st, ua); break;  \
+        default: hipLaunchKernelGGL((bs_sdd32u_kernel<T, 4, true>), grid, dim3(256), 0, st, ua); break; \
+    }
+    if (dtype == BF16) { SDDS_LAUNCH(bf16_t) } else { SDDS_LAUNCH(f16_t) }
+#undef SDDS_LAUNCH
+    return check_launch("bs_sdd32u_kernel (dsoftmax)");
 }
 
 extern "C" int flyhip_bs_sdd_kmajor(const void* a, const void* b, float* c32,

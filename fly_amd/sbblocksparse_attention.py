@@ -45,6 +45,7 @@ class SBBlockSparseAttention(nn.Module):
         self.register_buffer("master_layout", master_layout)
         self._need_layout_synchronization = True
         self.ops_cache = dict()
+        self._layout_cache = dict()
 
     def get_layout(self, T, S=None):
         if S is None:
@@ -55,8 +56,13 @@ class SBBlockSparseAttention(nn.Module):
         block = self.sparsity_config.block
         if (T % block != 0) or (S % block != 0):
             raise ValueError(f'Sequence lengths, {T} and {S}, needs to be divisible by block size {block}!')
-        layout = self.master_layout[..., :T // block, :S // block].cpu()
-        return layout if layout.dim() == 3 else layout.unsqueeze(0)      # a 2-D layout means one head
+        # one host copy per shape (keyed by the buffer's address and version counter): a device-to-host
+        # copy per call would stall the stream
+        key = (T, S, self.master_layout.data_ptr(), self.master_layout._version)
+        if key not in self._layout_cache:
+            layout = self.master_layout[..., :T // block, :S // block].cpu()
+            self._layout_cache[key] = layout if layout.dim() == 3 else layout.unsqueeze(0)   # 2-D: one head
+        return self._layout_cache[key]
 
     def get_ops(self, T, S=None):
         if S is None:

@@ -144,6 +144,19 @@ int flyhip_bs_sdd(const void* a, const void* b, void* c, const int32_t* lut, int
                   int64_t b_sz, int64_t b_sh, int64_t b_sn, int64_t b_sk,
                   int dtype, void* stream);
 
+/* Score gradient of a block-sparse attention core in one kernel: ds[z, n] = scale * p[z, n] * (dout[rows of
+ * block-row i_n] . v[rows of block-col j_n]^T - delta[row]), i.e. the sdd that forms dP = dO V^T fused with
+ * the backward of softmax(scale * s) (ref: the autograd chain behind blocksparse_attention.py:134-160:
+ * _sdd_matmul :279-346 followed by the softmax backward).  p, ds (Z, nnz, 32, 32) of bf16 / fp16;
+ * dout (Z,H,rows,K), v (Z,H,cols,K) with (batch, head, row) strides and contiguous K in {32,..,128};
+ * delta fp32 (Z, H, rows) = rowsum(dout * out); uni_* the union table of flyhip_bs_sdd (required). */
+int flyhip_bs_sdd_dsoftmax(const void* dout, const void* v, const void* p, const float* delta, void* ds,
+                           const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
+                           int nnz, int n_heads, int brows_per_head, int Z, int K, int blk,
+                           int64_t a_sz, int64_t a_sh, int64_t a_sm,
+                           int64_t b_sz, int64_t b_sh, int64_t b_sn,
+                           float scale, int dtype, void* stream);
+
 /* SDD with the contraction index slowest in both operands: c32[z, n] += A[z, h_n, :, block-row i_n]^T .
  * B[z, h_n, :, block-col j_n], A (Z,H,K,M) and B (Z,H,K,N) with (batch, head, k) strides and contiguous
  * features -- the weight gradient x^T dy of a block-sparse linear layer, K = tokens (ref: the 'sdd'

@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     header = open(os.path.join(ROOT, 'include', 'flyhip.h')).read()
     declared = set(re.findall(r'\b(flyhip_\w+)\s*\(', header))
     assert {'flyhip_sb_kv_reduce', 'flyhip_sblocal_fwd', 'flyhip_local_fwd', 'flyhip_bs_sdd', 'flyhip_bs_dsd', 'flyhip_bs_dds',
-            'flyhip_bs_softmax', 'flyhip_bs_softmax_bwd', 'flyhip_bs_attn', 'flyhip_bs_sdd_kmajor', 'flyhip_bs_rowreduce', 'flyhip_sb_plan', 'flyhip_version',
+            'flyhip_bs_softmax', 'flyhip_bs_softmax_bwd', 'flyhip_bs_attn', 'flyhip_bs_sdd_kmajor', 'flyhip_bs_sdd_dsoftmax', 'flyhip_bs_rowreduce', 'flyhip_sb_plan', 'flyhip_version',
             'flyhip_last_error'} <= declared
     lib = _lib.load()
     for name in declared:
