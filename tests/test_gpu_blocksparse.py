@@ -217,6 +217,49 @@ def test_config2_layout_stage_parity_reduced():
     assert rel_err(out, ob.dsd(p.cpu(), v, layout, block)) <= 2e-2
 
 
+@pytest.mark.parametrize('Z', [8, 30])
+def test_config2_full_size_heads_against_oracle(Z):
+    """BASELINE config 2 at its full size (Z=8, H=12) and with a sparse tensor of more than 2^31
+    elements (Z=30: 30 * 74448 * 1024 = 2.29e9): every stage of a few (batch, head) pairs, the last one
+    of the tensor among them, against the oracle run on that pair alone; the one-kernel attention
+    against the three stages over the whole output."""
+    from fly_amd import matmul, softmax, FlatBlockButterflySparsityConfig
+    from fly_amd.blocksparse_fused import fused_attention
+    print('case', Z, flush=True)
+    L, d, block, H = 4096, 64, 32, 12
+    lay = ((FlatBlockButterflySparsityConfig(8, 2, block).make_layout(L) + ob.band_layout(L // block, L // block, 4)) > 0).long()
+    per_head = int(lay.sum())
+    assert per_head == 6204
+    layout = lay.unsqueeze(0).repeat(H, 1, 1)
+    torch.manual_seed(Z)
+    q, k, v = (torch.randn(Z, H, L, d, device=DEV).bfloat16() for _ in range(3))
+    qk = matmul(layout, block, 'sdd', trans_b=True)(q, k)
+    assert qk.shape == (Z, H * per_head, block, block)
+    if Z == 30:
+        assert qk.numel() > 2 ** 31
+    p = softmax(layout, block)(qk.clone(), scale=0.125)
+    out = matmul(layout, block, 'dsd')(p, v)
+    one = lay.unsqueeze(0)
+    for z, h in [(0, 0), (Z // 2, 5), (Z - 1, H - 1)]:
+        sl = slice(h * per_head, (h + 1) * per_head)
+        qh, kh, vh = (t[z:z + 1, h:h + 1].cpu() for t in (q, k, v))
+        qk_h = qk[z:z + 1, sl].cpu()
+        assert rel_err(qk_h, ob.sdd(qh, kh, one, block, trans_b=True)) <= 2e-2
+        p_h = p[z:z + 1, sl].cpu()
+        assert rel_err(p_h, ob.block_softmax(qk_h, one, block, scale=0.125)) <= 2e-2
+        assert rel_err(out[z:z + 1, h:h + 1], ob.dsd(p_h, vh, one, block)) <= 2e-2
+    # size-independent property: every row of the softmax sums to one
+    rows = p.view(Z, H, per_head, block, block).sum(-1, dtype=torch.float32)               # (Z, H, nnz, block)
+    idx = lay.nonzero()[:, 0].to(DEV)                                                   # block-row of every block
+    sums = torch.zeros(Z, H, L // block, block, device=DEV).index_add_(2, idx, rows)
+    assert float((sums - 1).abs().max()) <= 2e-2
+    del rows, sums, qk
+    fused = fused_attention(layout, block)(q, k, v, 0.125)
+    assert fused.shape == out.shape
+    diff = float((fused.float() - out.float()).abs().max() / out.float().abs().max())
+    assert diff <= 2e-2
+
+
 @pytest.mark.parametrize('dtype,block', [(torch.float32, 16), (torch.float32, 32), (torch.bfloat16, 32)])
 def test_sbblocksparse_attention_module(dtype, block):
     """Scatterbrain on a block-sparse support (sbblocksparse_attention.py:109-213): output, and with
