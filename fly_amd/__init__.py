@@ -6,7 +6,7 @@ from .masking import FullMask, LengthMask, TriangularCausalMask
 from .feature_maps_sb import SBPerformerFeatures, gaussian_orthogonal_random_matrix
 from .sblocal_attention import SBLocalAttention, sblocal_forward, sblocal_attention_fn
 from .sblocal_backward import sblocal_backward
-from .local_attention import LocalAttention, local_forward
+from .local_attention import LocalAttention, local_forward, local_attention_fn, local_backward
 from .blocksparse_utils import sparsify_tensor, densify_tensor, mask_tensor, sparsify_broadcast_tensor
 from .blocksparse_matmul import matmul
 from .blocksparse_softmax import softmax, logsumexp, blocksparse_sum
@@ -18,7 +18,7 @@ from .fastlinear import LowRank, SparseLRLinear
 from .t2t_vit import T2T_ViT, T2T_module, T2TAttention, Token_transformer, MlpCustom, t2t_vit_t_14
 
 __all__ = ['FullMask', 'LengthMask', 'TriangularCausalMask', 'SBPerformerFeatures',
-           'gaussian_orthogonal_random_matrix', 'SBLocalAttention', 'sblocal_forward', 'sblocal_attention_fn', 'sblocal_backward', 'LocalAttention', 'local_forward',
+           'gaussian_orthogonal_random_matrix', 'SBLocalAttention', 'sblocal_forward', 'sblocal_attention_fn', 'sblocal_backward', 'LocalAttention', 'local_forward', 'local_attention_fn', 'local_backward',
            'sparsify_tensor', 'densify_tensor', 'mask_tensor', 'sparsify_broadcast_tensor',
            'matmul', 'softmax', 'logsumexp', 'blocksparse_sum', 'BlockSparseAttention', 'fused_attention',
            'SBBlockSparseAttention',

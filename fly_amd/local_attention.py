@@ -49,6 +49,71 @@ def local_forward(query, key, value, local_context, softmax_temp=None, key_lengt
     return out[..., :D]
 
 
+def local_backward(query, key, value, local_context, softmax_temp, key_lengths, grad_out, chunk=256):
+    """Gradients of local attention with respect to query, key and value (the reference takes them from
+    autograd through fast_transformers.local_product, local_attention.py:68-92).  The band softmax is
+    evaluated again for chunks of queries against the slice of keys their bands touch; with
+    P = softmax over the band, g = d out and delta_i = sum_s P_is g_i.v_s:
+    d v_s = sum_i P_is g_i,  d(t q_i.k_s) = P_is (g_i.v_s - delta_i).  Queries without any visible
+    key get zero gradients.  Ordinary tensor algebra on whatever device the tensors live on."""
+    B, T, H, E = query.shape
+    S, D = key.shape[1], value.shape[3]
+    t = softmax_temp or 1 / math.sqrt(E)
+    lc_lo, lc_hi = local_context // 2, (local_context + 1) // 2
+    wdt = torch.float64 if query.dtype == torch.float64 else torch.float32
+
+    def bh(x):                                   # (B,L,H,C) -> (B*H, L, C)
+        return x.permute(0, 2, 1, 3).reshape(B * H, x.shape[1], x.shape[3]).to(wdt)
+    Q, K, V, G = bh(query), bh(key), bh(value), bh(grad_out)
+    lens = None
+    if key_lengths is not None:
+        lens = key_lengths.to(Q.device).repeat_interleave(H).view(B * H, 1, 1)
+    dQ, dK, dV = torch.zeros_like(Q), torch.zeros_like(K), torch.zeros_like(V)
+    for i0 in range(0, T, chunk):
+        i1 = min(T, i0 + chunk)
+        s0, s1 = max(0, i0 - lc_lo), min(S, i1 - 1 + lc_hi)
+        if s1 <= s0:
+            continue
+        qi, gi, ks, vs = Q[:, i0:i1], G[:, i0:i1], K[:, s0:s1], V[:, s0:s1]
+        rel = torch.arange(s0, s1, device=Q.device).view(1, -1) - torch.arange(i0, i1, device=Q.device).view(-1, 1)
+        band = ((rel >= -lc_lo) & (rel < lc_hi)).unsqueeze(0)
+        if lens is not None:
+            band = band & (torch.arange(s0, s1, device=Q.device).view(1, 1, -1) < lens)
+        scores = (t * (qi @ ks.transpose(1, 2))).masked_fill(~band, -math.inf)
+        p = torch.softmax(scores, dim=-1).nan_to_num(0.0)          # rows without a visible key: zeros
+        dp = gi @ vs.transpose(1, 2)
+        ds = p * (dp - (p * dp).sum(-1, keepdim=True))
+        dV[:, s0:s1] += p.transpose(1, 2) @ gi
+        dQ[:, i0:i1] += t * (ds @ ks)
+        dK[:, s0:s1] += t * (ds.transpose(1, 2) @ qi)
+
+    def back(x, like):                           # (B*H, L, C) -> (B,L,H,C)
+        return x.reshape(B, H, x.shape[1], x.shape[2]).permute(0, 2, 1, 3).to(like.dtype)
+    return back(dQ, query), back(dK, key), back(dV, value)
+
+
+class _LocalFn(torch.autograd.Function):
+    """Forward on the fused kernel, gradients from local_backward."""
+
+    @staticmethod
+    def forward(ctx, query, key, value, local_context, softmax_temp, key_lengths):
+        out = local_forward(query, key, value, local_context, softmax_temp=softmax_temp, key_lengths=key_lengths)
+        ctx.save_for_backward(query, key, value, key_lengths)
+        ctx.local_context, ctx.softmax_temp = local_context, softmax_temp
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        query, key, value, key_lengths = ctx.saved_tensors
+        dq, dk, dv = local_backward(query, key, value, ctx.local_context, ctx.softmax_temp, key_lengths, grad_out)
+        return dq, dk, dv, None, None, None
+
+
+def local_attention_fn(query, key, value, local_context, softmax_temp=None, key_lengths=None):
+    """local_forward that autograd can differentiate."""
+    return _LocalFn.apply(query, key, value, local_context, softmax_temp, key_lengths)
+
+
 class LocalAttention(nn.Module):
     """Softmax attention in which query i only sees keys j with
     -(local_context // 2) <= j - i < (local_context + 1) // 2.  Same constructor and forward signature
@@ -71,6 +136,6 @@ class LocalAttention(nn.Module):
         lengths = None
         if key_padding_mask is not None and not bool(key_padding_mask.all_ones):
             lengths = key_padding_mask.lengths
-        out = local_forward(query, key, value, self.local_context, softmax_temp=self.softmax_temp,
-                            key_lengths=lengths)
+        out = local_attention_fn(query, key, value, self.local_context, softmax_temp=self.softmax_temp,
+                                 key_lengths=lengths)
         return out, None

@@ -212,3 +212,25 @@ def test_written_out_backward_matches_autograd_through_the_oracle(B, T, S, H, E,
         assert float((got - ref).abs().max() / ref.abs().max()) < 1e-10
     if lens is not None:
         assert float(dk[1, lens[1]:].abs().max()) == 0.0 and float(dv[1, lens[1]:].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize('B,T,S,H,E,D,lc,lens', [(1, 40, 40, 2, 16, 16, 12, None), (2, 70, 55, 2, 16, 24, 13, [55, 31]),
+                                                 (1, 300, 300, 1, 8, 8, 64, None)])
+def test_local_backward_matches_autograd_through_the_oracle(B, T, S, H, E, D, lc, lens):
+    """fly_amd.local_backward (band softmax evaluated again per chunk of queries) against autograd
+    through the oracle's LocalAttention op sequence, in float64, with chunks smaller than the
+    sequence, T != S, an odd window and key lengths (queries past every visible key included)."""
+    from fly_amd.local_attention import local_backward
+    g = torch.Generator().manual_seed(1)
+    q = torch.randn(B, T, H, E, generator=g).double().requires_grad_()
+    k = torch.randn(B, S, H, E, generator=g).double().requires_grad_()
+    v = torch.randn(B, S, H, D, generator=g).double().requires_grad_()
+    kl = None if lens is None else torch.tensor(lens)
+    out = osb.local_attention(q, k, v, lc, key_lengths=kl)
+    w = torch.randn(out.shape, generator=g).double()
+    (out * w).sum().backward()
+    dq, dk, dv = local_backward(q.detach(), k.detach(), v.detach(), lc, None, kl, w, chunk=32)
+    for got, ref in ((dq, q.grad), (dk, k.grad), (dv, v.grad)):
+        assert float((got - ref).abs().max() / ref.abs().max()) < 1e-10
+    if lens is not None:
+        assert float(dk[1, lens[1]:].abs().max()) == 0.0 and float(dv[1, lens[1]:].abs().max()) == 0.0
