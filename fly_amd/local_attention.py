@@ -8,6 +8,7 @@ import torch.nn.functional as F
 
 from . import _lib
 from .sblocal_attention import _HEAD_DIMS, _round_up_choice, _vector_ready
+from .sblocal_backward import BandWindows
 
 
 def local_forward(query, key, value, local_context, softmax_temp=None, key_lengths=None):
@@ -49,17 +50,18 @@ def local_forward(query, key, value, local_context, softmax_temp=None, key_lengt
     return out[..., :D]
 
 
-def local_backward(query, key, value, local_context, softmax_temp, key_lengths, grad_out, chunk=256):
+def local_backward(query, key, value, local_context, softmax_temp, key_lengths, grad_out, chunk=256,
+                   max_elements=1 << 27):
     """Gradients of local attention with respect to query, key and value (the reference takes them from
     autograd through fast_transformers.local_product, local_attention.py:68-92).  The band softmax is
-    evaluated again for chunks of queries against the slice of keys their bands touch; with
+    evaluated again for all chunks of queries at once against the windows of keys their bands touch
+    (sblocal_backward.BandWindows); with
     P = softmax over the band, g = d out and delta_i = sum_s P_is g_i.v_s:
     d v_s = sum_i P_is g_i,  d(t q_i.k_s) = P_is (g_i.v_s - delta_i).  Queries without any visible
     key get zero gradients.  Ordinary tensor algebra on whatever device the tensors live on."""
     B, T, H, E = query.shape
     S, D = key.shape[1], value.shape[3]
     t = softmax_temp or 1 / math.sqrt(E)
-    lc_lo, lc_hi = local_context // 2, (local_context + 1) // 2
     wdt = torch.float64 if query.dtype == torch.float64 else torch.float32
 
     def bh(x):                                   # (B,L,H,C) -> (B*H, L, C)
@@ -68,24 +70,22 @@ def local_backward(query, key, value, local_context, softmax_temp, key_lengths, 
     lens = None
     if key_lengths is not None:
         lens = key_lengths.to(Q.device).repeat_interleave(H).view(B * H, 1, 1)
-    dQ, dK, dV = torch.zeros_like(Q), torch.zeros_like(K), torch.zeros_like(V)
-    for i0 in range(0, T, chunk):
-        i1 = min(T, i0 + chunk)
-        s0, s1 = max(0, i0 - lc_lo), min(S, i1 - 1 + lc_hi)
-        if s1 <= s0:
-            continue
-        qi, gi, ks, vs = Q[:, i0:i1], G[:, i0:i1], K[:, s0:s1], V[:, s0:s1]
-        rel = torch.arange(s0, s1, device=Q.device).view(1, -1) - torch.arange(i0, i1, device=Q.device).view(-1, 1)
-        band = ((rel >= -lc_lo) & (rel < lc_hi)).unsqueeze(0)
-        if lens is not None:
-            band = band & (torch.arange(s0, s1, device=Q.device).view(1, 1, -1) < lens)
-        scores = (t * (qi @ ks.transpose(1, 2))).masked_fill(~band, -math.inf)
+    band = BandWindows(T, S, local_context, chunk, Q.device, lens, max_elements)
+    Qc, Gc = band.chunks(Q), band.chunks(G)
+    acc_k, acc_v = band.key_accumulator(E, wdt), band.key_accumulator(D, wdt)
+    dQc = torch.zeros_like(Qc)
+    Kw, Vw = band.windows(K), band.windows(V)
+    for j0, j1 in band.groups(B * H):
+        sl = slice(j0, j1)
+        ks, vs = Kw[:, sl], Vw[:, sl]
+        scores = (t * (Qc[:, sl] @ ks.transpose(2, 3))).masked_fill(~band.mask(j0, j1), -math.inf)
         p = torch.softmax(scores, dim=-1).nan_to_num(0.0)          # rows without a visible key: zeros
-        dp = gi @ vs.transpose(1, 2)
+        dp = Gc[:, sl] @ vs.transpose(2, 3)
         ds = p * (dp - (p * dp).sum(-1, keepdim=True))
-        dV[:, s0:s1] += p.transpose(1, 2) @ gi
-        dQ[:, i0:i1] += t * (ds @ ks)
-        dK[:, s0:s1] += t * (ds.transpose(1, 2) @ qi)
+        dQc[:, sl] = t * (ds @ ks)
+        band.add_windows(acc_k, j0, t * (ds.transpose(2, 3) @ Qc[:, sl]))
+        band.add_windows(acc_v, j0, p.transpose(2, 3) @ Gc[:, sl])
+    dQ, dK, dV = band.unchunk(dQc), band.fold(acc_k), band.fold(acc_v)
 
     def back(x, like):                           # (B*H, L, C) -> (B,L,H,C)
         return x.reshape(B, H, x.shape[1], x.shape[2]).permute(0, 2, 1, 3).to(like.dtype)

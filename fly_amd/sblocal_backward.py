@@ -15,8 +15,9 @@ Here they are written out.  With g = d out, c_i = g_i.out_i and Df_is = g_i.v_s 
 Sums over "outside the band" are taken as (sum over all keys) - (sum over the band): the first is a
 product with the global reductions K'^T V, sum K' (queries) or Q'^T g, Q'^T c (keys), the second
 a band-limited product evaluated for chunks of queries against the slice of keys their bands
-touch.  Everything is ordinary tensor algebra (library GEMMs on whatever device the tensors
-live on); the clamp of the low-rank normaliser (sblocal_attention.py:111) is taken as inactive.
+touch -- all chunks at once as batched products over overlapping windows of the keys (BandWindows).
+Everything is ordinary tensor algebra (library GEMMs on whatever device the tensors live on); the
+clamp of the low-rank normaliser (sblocal_attention.py:111) is taken as inactive.
 """
 import math
 
@@ -25,10 +26,85 @@ import torch
 from .feature_maps_sb import softmax_kernel
 
 
+class BandWindows:
+    """Index bookkeeping for band-limited products taken for all chunks of queries at once.
+
+    Queries are cut into n chunks of C (the last one zero-padded); chunk j meets the window of W keys
+    starting at key j*C - lc_lo, W = the multiple of C that covers C + local_context - 1.  Query a of a
+    chunk and key b of its window are i = jC + a and s = jC - lc_lo + b, so s - i = b - a - lc_lo:
+    the band -lc_lo <= s - i < lc_hi is the pattern 0 <= b - a < local_context for every chunk; on
+    top of it keys must exist (0 <= s < S) and lie below the key length."""
+
+    def __init__(self, T, S, local_context, chunk, device, lens=None, max_elements=1 << 27):
+        self.T, self.S, self.C = T, S, chunk
+        self.lc_lo = local_context // 2
+        self.n = -(-T // chunk)
+        self.P = -(-(chunk + local_context - 1) // chunk)        # chunk-sized pieces per window
+        self.W = self.P * chunk
+        self.device, self.lens, self.max_elements = device, lens, max_elements
+        a = torch.arange(chunk, device=device).view(-1, 1)
+        b = torch.arange(self.W, device=device).view(1, -1)
+        self.pattern = ((b - a >= 0) & (b - a < local_context)).view(1, 1, chunk, self.W)
+
+    def chunks(self, x):
+        """(BH, T, F) -> (BH, n, C, F), zero rows after T."""
+        pad = self.n * self.C - self.T
+        if pad:
+            x = torch.nn.functional.pad(x, (0, 0, 0, pad))
+        return x.reshape(x.shape[0], self.n, self.C, x.shape[2])
+
+    def unchunk(self, x):
+        return x.reshape(x.shape[0], self.n * self.C, x.shape[3])[:, :self.T]
+
+    def windows(self, x):
+        """(BH, S, F) -> view (BH, n, W, F) of the zero-padded keys (windows overlap)."""
+        total = (self.n - 1) * self.C + self.W
+        xp = torch.nn.functional.pad(x, (0, 0, self.lc_lo, max(0, total - self.lc_lo - self.S)))[:, :total]
+        return xp.unfold(1, self.W, self.C).transpose(2, 3)
+
+    def groups(self, batch):
+        """Ranges of chunks whose (batch, g, C, W) intermediates stay below max_elements."""
+        g = max(1, self.max_elements // (batch * self.C * self.W))
+        return [(j0, min(self.n, j0 + g)) for j0 in range(0, self.n, g)]
+
+    def mask(self, j0, j1):
+        """(1 or BH, g, C, W) bool: inside the band, key exists and lies below the key length."""
+        s = (torch.arange(j0, j1, device=self.device) * self.C - self.lc_lo).view(1, -1, 1, 1) \
+            + torch.arange(self.W, device=self.device).view(1, 1, 1, -1)
+        ok = (s >= 0) & (s < self.S)
+        if self.lens is not None:
+            ok = ok & (s < self.lens.view(-1, 1, 1, 1))
+        return self.pattern & ok
+
+    def key_accumulator(self, F, dtype):
+        return torch.zeros(0, dtype=dtype, device=self.device), F     # allocated on first use (batch known then)
+
+    def add_windows(self, acc, j0, win):
+        """Overlap-add windows j0.. (BH, g, W, F): piece p of window j lands on key chunk j + p."""
+        buf, F = acc
+        BH, g = win.shape[0], win.shape[1]
+        if buf.numel() == 0:
+            buf.resize_(BH, self.n + self.P - 1, self.C, F).zero_()
+        wv = win.reshape(BH, g, self.P, self.C, F)
+        for p in range(self.P):
+            buf[:, j0 + p:j0 + p + g] += wv[:, :, p]
+
+    def fold(self, acc):
+        """Accumulated windows -> (BH, S, F)."""
+        buf, F = acc
+        flat = buf.reshape(buf.shape[0], -1, F)                 # row r is key r - lc_lo
+        out = flat.new_zeros(buf.shape[0], self.S, F)
+        hi = min(flat.shape[1], self.lc_lo + self.S)
+        out[:, :hi - self.lc_lo] = flat[:, self.lc_lo:hi]
+        return out
+
+
 def sblocal_backward(query, key, value, projection_matrix, local_context, softmax_temp, key_lengths,
-                     out, log_normalization, grad_out, chunk=256):
+                     out, log_normalization, grad_out, chunk=256, max_elements=1 << 27):
     """query (B,T,H,E), key (B,S,H,E), value (B,S,H,D), out / grad_out (B,T,H,D),
     log_normalization (B,H,T,1) as returned by the forward; key_lengths (B,) or None.
+    max_elements bounds the
+    size of the (batch, chunks, chunk, window) intermediates: chunks are taken in groups that stay below it.
     Returns (d query, d key, d value) in the dtypes of the inputs."""
     B, T, H, E = query.shape
     S, D = key.shape[1], value.shape[3]
@@ -62,27 +138,32 @@ def sblocal_backward(query, key, value, projection_matrix, local_context, softma
     dQ = torch.zeros_like(Q)
     dK = torch.zeros_like(K)
 
-    for i0 in range(0, T, chunk):
-        i1 = min(T, i0 + chunk)
-        s0, s1 = max(0, i0 - lc_lo), min(S, i1 - 1 + lc_hi)
-        if s1 <= s0:
-            continue
-        qi, gi, psi_i = Q[:, i0:i1], G[:, i0:i1], psi[:, i0:i1]
-        ks, vs, pk = K[:, s0:s1], V[:, s0:s1], phik[:, s0:s1]
-        rel = torch.arange(s0, s1, device=Q.device).view(1, -1) - torch.arange(i0, i1, device=Q.device).view(-1, 1)
-        band = ((rel >= -lc_lo) & (rel < lc_hi)).unsqueeze(0)
-        if lens is not None:
-            band = band & (torch.arange(s0, s1, device=Q.device).view(1, 1, -1) < lens)
-        band = band.to(wdt)
-        a_bar = torch.exp(t * (qi @ ks.transpose(1, 2)) - LN[:, i0:i1]) * band
-        k_bar = (psi_i @ pk.transpose(1, 2)) * band
-        df = (gi @ vs.transpose(1, 2) - c[:, i0:i1]) * band
+    # band terms, all chunks of queries at once: chunk j (queries jC .. jC+C-1) against the window of
+    # keys jC - lc_lo .. jC - lc_lo + W - 1 that its bands touch; inside a window the band is the same
+    # (C, W) pattern for every chunk
+    band = BandWindows(T, S, local_context, chunk, Q.device, lens, max_elements)
+    Qc, Gc, Pc, cc, LNc = (band.chunks(x) for x in (Q, G, psi, c, LN))
+    acc_k, acc_v, acc_u = band.key_accumulator(E, wdt), band.key_accumulator(D, wdt), band.key_accumulator(2 * mh, wdt)
+    dQc, uqc = torch.zeros_like(Qc), torch.zeros_like(Pc)
+    Kw, Vw, PKw = band.windows(K), band.windows(V), band.windows(phik)
+    for j0, j1 in band.groups(B * H):
+        sl = slice(j0, j1)
+        ks, vs, pk = Kw[:, sl], Vw[:, sl], PKw[:, sl]               # (BH, g, W, .)
+        valid = band.mask(j0, j1).to(wdt)
+        a_bar = torch.exp(t * (Qc[:, sl] @ ks.transpose(2, 3)) - LNc[:, sl]) * valid
+        k_bar = (Pc[:, sl] @ pk.transpose(2, 3)) * valid
+        df = (Gc[:, sl] @ vs.transpose(2, 3) - cc[:, sl]) * valid
         dm = a_bar * df
-        dQ[:, i0:i1] += t * (dm @ ks)
-        dK[:, s0:s1] += t * (dm.transpose(1, 2) @ qi)
-        dV[:, s0:s1] += (a_bar - k_bar).transpose(1, 2) @ gi
-        uq[:, i0:i1] -= psi_i * (df @ pk)
-        uk[:, s0:s1] -= pk * (df.transpose(1, 2) @ psi_i)
+        dQc[:, sl] = t * (dm @ ks)
+        uqc[:, sl] = df @ pk
+        band.add_windows(acc_k, j0, t * (dm.transpose(2, 3) @ Qc[:, sl]))
+        band.add_windows(acc_v, j0, (a_bar - k_bar).transpose(2, 3) @ Gc[:, sl])
+        band.add_windows(acc_u, j0, df.transpose(2, 3) @ Pc[:, sl])
+    dQ += band.unchunk(dQc)
+    uq -= psi * band.unchunk(uqc)
+    dK += band.fold(acc_k)
+    dV += band.fold(acc_v)
+    uk -= phik * band.fold(acc_u)
 
     st = math.sqrt(t)
     dQ += st * ((uq[..., :mh] - uq[..., mh:]) @ P) - t * Q * uq.sum(-1, keepdim=True)

@@ -210,6 +210,11 @@ def test_written_out_backward_matches_autograd_through_the_oracle(B, T, S, H, E,
                                   chunk=32)
     for got, ref in ((dq, q.grad), (dk, k.grad), (dv, v.grad)):
         assert float((got - ref).abs().max() / ref.abs().max()) < 1e-10
+    # chunks taken one group at a time give the same sums
+    again = sblocal_backward(q.detach(), k.detach(), v.detach(), P, lc, None, kl, out.detach(), ln.detach(), w,
+                             chunk=32, max_elements=1)
+    for got, ref in zip(again, (dq, dk, dv)):
+        assert float((got - ref).abs().max()) < 1e-12
     if lens is not None:
         assert float(dk[1, lens[1]:].abs().max()) == 0.0 and float(dv[1, lens[1]:].abs().max()) == 0.0
 
@@ -232,5 +237,8 @@ def test_local_backward_matches_autograd_through_the_oracle(B, T, S, H, E, D, lc
     dq, dk, dv = local_backward(q.detach(), k.detach(), v.detach(), lc, None, kl, w, chunk=32)
     for got, ref in ((dq, q.grad), (dk, k.grad), (dv, v.grad)):
         assert float((got - ref).abs().max() / ref.abs().max()) < 1e-10
+    again = local_backward(q.detach(), k.detach(), v.detach(), lc, None, kl, w, chunk=32, max_elements=1)
+    for got, ref in zip(again, (dq, dk, dv)):
+        assert float((got - ref).abs().max()) < 1e-12
     if lens is not None:
         assert float(dk[1, lens[1]:].abs().max()) == 0.0 and float(dv[1, lens[1]:].abs().max()) == 0.0
