@@ -1960,6 +1960,246 @@ static int launch_local(const LocalArgs& a, hipStream_t st) {
     return check_launch("local_fwd_kernel");
 }
 
+// ---------------------------------------------------------------------------------------
+// band terms of the backward pass
+// ---------------------------------------------------------------------------------------
+// Inside the band a (query i, key s) pair carries  a = exp(t q_i.k_s - log Z_i),  kb = psi_i.phik_s
+// (the low-rank weight, psi = Phi(q) scaled by 1/Z),  df = g_i.v_s - c_i  and  dm = a df.  The
+// gradients need five band-limited sums of them:
+//   over keys    : sum_s dm k_s (-> d q),  sum_s df phik_s                     (query-major pass)
+//   over queries : sum_i dm q_i (-> d k),  sum_i df psi_i,  sum_i (a - kb) g_i (key-major pass)
+// Both passes are one kernel: an "outer" side whose rows are owned by lanes (64 per workgroup, 16 per
+// wave, operands in registers) meets 32-row tiles of the "inner" side staged through LDS, with the
+// products formed transposed (rows = inner, columns = outer) exactly as in the forward kernel, so the
+// pair weights leave the score MFMAs in the operand layout of the output MFMAs.
+//   query-major: outer = (q, -, g), inner = (k, phik, v): s1 = K q, s3 = V g;
+//                out1 = t K^T dm, out2 = phik^T df
+//   key-major  : outer = (k, phik, v), inner = (q, psi, g): s1 = Q k, s2 = psi phik, s3 = G v;
+//                out1 = t Q^T dm, out2 = psi^T df, out3 = G^T (a - kb)
+// log Z and c belong to the query: lane-owned in the query-major pass, staged with the tile (two
+// extra LDS rows) in the key-major pass.  All tensors are fp32, contiguous (batch*head, rows, width).
+struct BwdArgs {
+    const float* x1; const float* x2; const float* x3;      // outer rows (x2 only key-major)
+    const float* y1; const float* y2; const float* y3;      // inner rows
+    const float* ln; const float* c;                        // per query: log Z, g.out
+    const int64_t* lens;
+    float* o1; float* o2; float* o3;                        // outer rows (o3 only key-major)
+    int BH, H, T, S, lc;
+    float temp;
+};
+
+template <int E, int M, bool KEYMAJOR>
+__global__ __launch_bounds__(NT) void sblocal_bwd_band_kernel(BwdArgs a) {
+    constexpr int D = E, LDK = E + 4, LDV = D + 4, LDF = M + 4;
+    constexpr int EC = E / 16, FC = M / 16, DB = D / 16, KB = TK / 16;
+    constexpr int STAGE = TK * (LDK + LDV + LDF) + 2 * TK;      // floats per LDS stage (+ log Z and c of the tile)
+    constexpr float LOG2E = 1.4426950408889634f;
+    extern __shared__ __attribute__((aligned(128))) float smem[];
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
+    const int Lo = KEYMAJOR ? a.S : a.T, Li = KEYMAJOR ? a.T : a.S;
+    const int n_ot = (Lo + TQ - 1) / TQ;
+    const int n_items = a.BH * n_ot;
+    const int per_xcd = (n_items + N_XCD - 1) / N_XCD;
+    const int item = (blockIdx.x % N_XCD) * per_xcd + blockIdx.x / N_XCD;   // see sblocal_fwd_kernel
+    if (item >= n_items) return;                       // workgroup-uniform
+    const int ot = item % n_ot, bh = item / n_ot, b = bh / a.H;
+    const int o0 = ot * TQ, ow0 = o0 + 16 * w, o = ow0 + r16;
+    const int len = a.lens ? min((int)a.lens[b], a.S) : a.S;
+    const int lc_lo = a.lc / 2, lc_hi = (a.lc + 1) / 2;    // band: -lc_lo <= s - i < lc_hi
+    // the same band seen from the outer row: lo <= n - o < hi
+    const int lo = KEYMAJOR ? -(lc_hi - 1) : -lc_lo, hi = KEYMAJOR ? lc_lo + 1 : lc_hi;
+    const int o_limit = KEYMAJOR ? len : a.T, n_limit = KEYMAJOR ? a.T : len;
+    const bool ovalid = o < o_limit;
+
+    const float* y1 = a.y1 + (long)bh * Li * E;
+    const float* y2 = a.y2 + (long)bh * Li * M;
+    const float* y3 = a.y3 + (long)bh * Li * D;
+    const float* lnp = a.ln + (long)bh * a.T;
+    const float* cp = a.c + (long)bh * a.T;
+
+    // inner tiles this workgroup meets
+    const int o_last = min(o0 + TQ - 1, o_limit - 1);
+    const int n_lo = max(0, o0 + lo), n_hi = min(n_limit, o_last + hi);
+    const int kt_lo = n_lo / TK;
+    const int kt_hi = (o_last >= o0 && n_hi > n_lo) ? (n_hi + TK - 1) / TK : kt_lo;
+
+    RowTile<TK, E> r1;
+    RowTile<TK, M> r2;
+    RowTile<TK, D> r3;
+    float rs = 0.f;                                   // key-major: log Z (threads 0..31) / c (32..63) of the tile
+    auto fetch = [&](int kt) __attribute__((always_inline)) {
+        r1.fetch(y1, E, kt * TK, Li - 1, tid);
+        r2.fetch(y2, M, kt * TK, Li - 1, tid);
+        r3.fetch(y3, D, kt * TK, Li - 1, tid);
+        if (KEYMAJOR && tid < 2 * TK) {
+            const int row = min(kt * TK + (tid & (TK - 1)), Li - 1);
+            rs = tid < TK ? lnp[row] * LOG2E : cp[row];
+        }
+    };
+    auto stash = [&](int buf) __attribute__((always_inline)) {
+        float* st = smem + buf * STAGE;
+        r1.template stash<LDK>(st, tid);
+        r3.template stash<LDV>(st + TK * LDK, tid);
+        r2.template stash<LDF>(st + TK * (LDK + LDV), tid);
+        if (KEYMAJOR && tid < 2 * TK) st[TK * (LDK + LDV + LDF) + tid] = rs;
+    };
+    if (kt_lo < kt_hi) fetch(kt_lo);
+
+    // outer operands (B side: column = outer row, k = 16c + 4g + j); exponents are base 2
+    const int orow = min(o, Lo - 1);
+    floatx4 x1[EC], x3[DB], x2[KEYMAJOR ? FC : 1];
+#pragma unroll
+    for (int c = 0; c < EC; ++c)
+        x1[c] = load4_f32(a.x1 + ((long)bh * Lo + orow) * E + 16 * c + 4 * g) * (a.temp * LOG2E);
+#pragma unroll
+    for (int c = 0; c < DB; ++c) x3[c] = load4_f32(a.x3 + ((long)bh * Lo + orow) * D + 16 * c + 4 * g);
+    if (KEYMAJOR) {
+#pragma unroll
+        for (int c = 0; c < FC; ++c) x2[c] = load4_f32(a.x2 + ((long)bh * Lo + orow) * M + 16 * c + 4 * g);
+    }
+    const float ln_o = KEYMAJOR ? 0.f : lnp[orow] * LOG2E, c_o = KEYMAJOR ? 0.f : cp[orow];
+    // inner rows this lane's outer row may meet: nmin <= n < nmin + span
+    const int nmin = max(o + lo, 0);
+    const unsigned span = ovalid ? (unsigned)max(min(o + hi, n_limit) - nmin, 0) : 0u;
+
+    floatx4 acc1[EC], acc2[FC], acc3[KEYMAJOR ? DB : 1];
+#pragma unroll
+    for (int c = 0; c < EC; ++c) acc1[c] = Frag<float>::zero();
+#pragma unroll
+    for (int c = 0; c < FC; ++c) acc2[c] = Frag<float>::zero();
+#pragma unroll
+    for (int c = 0; c < (KEYMAJOR ? DB : 1); ++c) acc3[c] = Frag<float>::zero();
+
+    if (kt_lo < kt_hi) stash(0);
+    __syncthreads();
+
+    for (int kt = kt_lo; kt < kt_hi; ++kt) {
+        const int n_base = kt * TK;
+        const int cur = (kt - kt_lo) & 1;
+        const float* Y1s = smem + cur * STAGE;
+        const float* Y3s = Y1s + TK * LDK;
+        const float* Y2s = Y3s + TK * LDV;
+        const float* Ss = Y2s + TK * LDF;
+        const bool more = kt + 1 < kt_hi;
+        if (more) fetch(kt + 1);                       // next tile's loads fly during the MFMAs
+
+        // wave-uniform: does this tile meet the band of any of the wave's 16 outer rows?
+        const bool any = !(n_base + TK - 1 - ow0 < lo || n_base - (ow0 + 15) >= hi || n_base >= n_limit || ow0 >= o_limit);
+        if (any) {
+            floatx4 s1[KB], s2[KB], s3[KB];
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) { s1[kb] = Frag<float>::zero(); s2[kb] = Frag<float>::zero(); s3[kb] = Frag<float>::zero(); }
+#pragma unroll
+            for (int c = 0; c < EC; ++c) {               // E == D: the two chains advance together
+                floatx4 ya[KB], yc[KB];
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb) {
+                    ya[kb] = *reinterpret_cast<const floatx4*>(Y1s + (16 * kb + r16) * LDK + 4 * g + 16 * c);
+                    yc[kb] = *reinterpret_cast<const floatx4*>(Y3s + (16 * kb + r16) * LDV + 4 * g + 16 * c);
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int kb = 0; kb < KB; ++kb) {
+                        s1[kb] = __builtin_amdgcn_mfma_f32_16x16x4f32(ya[kb][j], x1[c][j], s1[kb], 0, 0, 0);
+                        s3[kb] = __builtin_amdgcn_mfma_f32_16x16x4f32(yc[kb][j], x3[c][j], s3[kb], 0, 0, 0);
+                    }
+            }
+            if (KEYMAJOR) {
+#pragma unroll
+                for (int c = 0; c < FC; ++c) {
+                    floatx4 yb[KB];
+#pragma unroll
+                    for (int kb = 0; kb < KB; ++kb)
+                        yb[kb] = *reinterpret_cast<const floatx4*>(Y2s + (16 * kb + r16) * LDF + 4 * g + 16 * c);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+#pragma unroll
+                        for (int kb = 0; kb < KB; ++kb)
+                            s2[kb] = __builtin_amdgcn_mfma_f32_16x16x4f32(yb[kb][j], x2[c][j], s2[kb], 0, 0, 0);
+                }
+            }
+            // lane holds the pair (outer row o, inner row n_base + 16kb + 4g + i)
+            floatx4 wdm[KB], wdf[KB], wak[KB];
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) {
+                floatx4 lnq, cq;
+                if (KEYMAJOR) {
+                    lnq = *reinterpret_cast<const floatx4*>(Ss + 16 * kb + 4 * g);
+                    cq = *reinterpret_cast<const floatx4*>(Ss + TK + 16 * kb + 4 * g);
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int n = n_base + 16 * kb + 4 * g + i;
+                    const bool ok = (unsigned)(n - nmin) < span;
+                    const float av = ok ? __builtin_amdgcn_exp2f(s1[kb][i] - (KEYMAJOR ? lnq[i] : ln_o)) : 0.f;
+                    const float df = ok ? s3[kb][i] - (KEYMAJOR ? cq[i] : c_o) : 0.f;
+                    wdm[kb][i] = av * df;
+                    wdf[kb][i] = df;
+                    wak[kb][i] = av - (ok ? s2[kb][i] : 0.f);
+                }
+            }
+            // out^T[col][outer] += sum_inner Y[inner][col] w[inner][outer]
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int row = 16 * kb + 4 * g + i;
+#pragma unroll
+                    for (int c = 0; c < EC; ++c)
+                        acc1[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(Y1s[row * LDK + 16 * c + r16], wdm[kb][i], acc1[c], 0, 0, 0);
+#pragma unroll
+                    for (int c = 0; c < FC; ++c)
+                        acc2[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(Y2s[row * LDF + 16 * c + r16], wdf[kb][i], acc2[c], 0, 0, 0);
+                    if (KEYMAJOR) {
+#pragma unroll
+                        for (int c = 0; c < DB; ++c)
+                            acc3[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(Y3s[row * LDV + 16 * c + r16], wak[kb][i], acc3[c], 0, 0, 0);
+                    }
+                }
+        }
+        if (more) stash(cur ^ 1);
+        __syncthreads();
+    }
+
+    if (o < Lo) {
+        float* p1 = a.o1 + ((long)bh * Lo + o) * E;
+        float* p2 = a.o2 + ((long)bh * Lo + o) * M;
+#pragma unroll
+        for (int c = 0; c < EC; ++c) store4_f32(p1 + 16 * c + 4 * g, acc1[c] * a.temp);
+#pragma unroll
+        for (int c = 0; c < FC; ++c) store4_f32(p2 + 16 * c + 4 * g, acc2[c]);
+        if (KEYMAJOR) {
+            float* p3 = a.o3 + ((long)bh * Lo + o) * D;
+#pragma unroll
+            for (int c = 0; c < DB; ++c) store4_f32(p3 + 16 * c + 4 * g, acc3[c]);
+        }
+    }
+}
+
+template <int E, int M, bool KEYMAJOR>
+static int launch_bwd_band(const BwdArgs& a, hipStream_t st) {
+    auto kern = sblocal_bwd_band_kernel<E, M, KEYMAJOR>;
+    constexpr size_t smem = sizeof(float) * 2 * (TK * (3 * 4 + 2 * E + M) + 2 * TK);
+    static bool lds_ready = false;
+    if (!lds_ready) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return fail(ERR_LAUNCH, "sblocal_bwd_band: LDS attribute: %s", hipGetErrorString(e));
+        lds_ready = true;
+    }
+    const long items = (long)a.BH * (((KEYMAJOR ? a.S : a.T) + TQ - 1) / TQ);
+    const long grid = (items + N_XCD - 1) / N_XCD * N_XCD;
+    if (grid > 2147483647L) return fail(ERR_ARG, "sblocal_bwd_band: too many workgroups");
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NT), smem, st, a);
+    return check_launch("sblocal_bwd_band_kernel");
+}
+
+template <int E, int M>
+static int launch_bwd_band_both(const BwdArgs& a, bool key_major, hipStream_t st) {
+    return key_major ? launch_bwd_band<E, M, true>(a, st) : launch_bwd_band<E, M, false>(a, st);
+}
+
 #define SB_DISPATCH_M(FN, T, EE, ARGS)                                       \
     switch (m) {                                                              \
         case 32: return FN<T, EE, 32>(ARGS, st);                              \
@@ -2153,4 +2393,26 @@ extern "C" int flyhip_local_fwd(const void* q, const void* k, const void* v, con
     if (dtype == BF16) { LOCAL_DISPATCH(bf16_t) }
 #undef LOCAL_DISPATCH
     return fail(ERR_UNSUPPORTED, "local_fwd supports float32 and bfloat16, got dtype code %d", dtype);
+}
+
+extern "C" int flyhip_sblocal_bwd_band(const float* x1, const float* x2, const float* x3,
+                                       const float* y1, const float* y2, const float* y3,
+                                       const float* log_norm, const float* c, const int64_t* key_lengths,
+                                       float* o1, float* o2, float* o3,
+                                       int BH, int H, int T, int S, int E, int M, int local_context,
+                                       float softmax_temp, int key_major, void* stream) {
+    FLY_REQUIRE(x1 && x3 && y1 && y2 && y3 && log_norm && c && o1 && o2, "sblocal_bwd_band: null pointer");
+    FLY_REQUIRE(!key_major || (x2 && o3), "sblocal_bwd_band: the key-major pass needs x2 and o3");
+    FLY_REQUIRE(BH > 0 && H > 0 && BH % H == 0 && T > 0 && S > 0, "sblocal_bwd_band: empty or inconsistent problem");
+    FLY_REQUIRE(local_context >= 1, "sblocal_bwd_band: local_context must be >= 1");
+    FLY_REQUIRE(softmax_temp > 0.f, "sblocal_bwd_band: softmax_temp must be positive");
+    BwdArgs a{x1, x2, x3, y1, y2, y3, log_norm, c, key_lengths, o1, o2, o3, BH, H, T, S, local_context, softmax_temp};
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (E == 32 && M == 32) return launch_bwd_band_both<32, 32>(a, key_major != 0, st);
+    if (E == 32 && M == 64) return launch_bwd_band_both<32, 64>(a, key_major != 0, st);
+    if (E == 64 && M == 32) return launch_bwd_band_both<64, 32>(a, key_major != 0, st);
+    if (E == 64 && M == 64) return launch_bwd_band_both<64, 64>(a, key_major != 0, st);
+    if (E == 64 && M == 128) return launch_bwd_band_both<64, 128>(a, key_major != 0, st);
+    return fail(ERR_UNSUPPORTED, "sblocal_bwd_band: (head dim, features) = (%d, %d) not in "
+                                 "{(32,32), (32,64), (64,32), (64,64), (64,128)}", E, M);
 }

@@ -99,12 +99,90 @@ class BandWindows:
         return out
 
 
+_BAND_KERNEL_FEATURES = {32: (32, 64), 64: (32, 64, 128)}       # head dim -> feature counts the band kernels are built for
+
+
+def _band_kernel_dims(E, D, M):
+    """(head dim, feature count) of the band kernels that fit (zero padding up to them changes no
+    product), or None."""
+    for dim, feats in _BAND_KERNEL_FEATURES.items():
+        if max(E, D) <= dim:
+            for m in feats:
+                if M <= m:
+                    return dim, m
+    return None
+
+
+def _band_terms_hip(Q, K, V, G, psi, phik, LN, c, lens_b, H, local_context, t, dims):
+    """The five band-limited sums on flyhip_sblocal_bwd_band.  Q, G, psi, LN, c: (BH, T, .); K, V, phik:
+    (BH, S, .); float32 on the GPU.  Returns (t sum_s dm k, sum_s df phik, t sum_i dm q, sum_i df psi,
+    sum_i (a - kb) g) cut back to the callers' widths."""
+    from . import _lib
+    BH, T, E = Q.shape
+    S, D, M = K.shape[1], V.shape[2], psi.shape[2]
+    dim, mk = dims
+
+    def fit(x, width):
+        if x.shape[2] != width:
+            x = torch.nn.functional.pad(x, (0, width - x.shape[2]))
+        return x.contiguous()
+    q_, k_, v_, g_ = fit(Q, dim), fit(K, dim), fit(V, dim), fit(G, dim)
+    psi_, phik_ = fit(psi, mk), fit(phik, mk)
+    ln_, c_ = LN.reshape(BH, T).contiguous(), c.reshape(BH, T).contiguous()
+    dq, uq = Q.new_empty(BH, T, dim), Q.new_empty(BH, T, mk)
+    dk, uk, dv = Q.new_empty(BH, S, dim), Q.new_empty(BH, S, mk), Q.new_empty(BH, S, dim)
+    with torch.cuda.device(Q.device):
+        st = _lib.stream_ptr(Q.device)
+        _lib.call('flyhip_sblocal_bwd_band', q_.data_ptr(), None, g_.data_ptr(), k_.data_ptr(), phik_.data_ptr(),
+                  v_.data_ptr(), ln_.data_ptr(), c_.data_ptr(), _lib.ptr(lens_b), dq.data_ptr(), uq.data_ptr(), None,
+                  BH, H, T, S, dim, mk, local_context, float(t), 0, st)
+        _lib.call('flyhip_sblocal_bwd_band', k_.data_ptr(), phik_.data_ptr(), v_.data_ptr(), q_.data_ptr(),
+                  psi_.data_ptr(), g_.data_ptr(), ln_.data_ptr(), c_.data_ptr(), _lib.ptr(lens_b), dk.data_ptr(),
+                  uk.data_ptr(), dv.data_ptr(), BH, H, T, S, dim, mk, local_context, float(t), 1, st)
+    return dq[..., :E], uq[..., :M], dk[..., :E], uk[..., :M], dv[..., :D]
+
+
+def _band_terms_torch(Q, K, V, G, psi, phik, LN, c, lens, local_context, t, chunk, max_elements, dQ, dK, dV, uq, uk):
+    """The same sums as batched library products, added into dQ, dK, dV, uq, uk (any device, float32 or
+    float64)."""
+    # band terms, all chunks of queries at once: chunk j (queries jC .. jC+C-1) against the window of
+    # keys jC - lc_lo .. jC - lc_lo + W - 1 that its bands touch; inside a window the band is the same
+    # (C, W) pattern for every chunk
+    BH, T, E = Q.shape
+    S, D, mh2, wdt = K.shape[1], V.shape[2], psi.shape[2], Q.dtype
+    band = BandWindows(T, S, local_context, chunk, Q.device, lens, max_elements)
+    Qc, Gc, Pc, cc, LNc = (band.chunks(x) for x in (Q, G, psi, c, LN))
+    acc_k, acc_v, acc_u = band.key_accumulator(E, wdt), band.key_accumulator(D, wdt), band.key_accumulator(mh2, wdt)
+    dQc, uqc = torch.zeros_like(Qc), torch.zeros_like(Pc)
+    Kw, Vw, PKw = band.windows(K), band.windows(V), band.windows(phik)
+    for j0, j1 in band.groups(BH):
+        sl = slice(j0, j1)
+        ks, vs, pk = Kw[:, sl], Vw[:, sl], PKw[:, sl]               # (BH, g, W, .)
+        valid = band.mask(j0, j1).to(wdt)
+        a_bar = torch.exp(t * (Qc[:, sl] @ ks.transpose(2, 3)) - LNc[:, sl]) * valid
+        k_bar = (Pc[:, sl] @ pk.transpose(2, 3)) * valid
+        df = (Gc[:, sl] @ vs.transpose(2, 3) - cc[:, sl]) * valid
+        dm = a_bar * df
+        dQc[:, sl] = t * (dm @ ks)
+        uqc[:, sl] = df @ pk
+        band.add_windows(acc_k, j0, t * (dm.transpose(2, 3) @ Qc[:, sl]))
+        band.add_windows(acc_v, j0, (a_bar - k_bar).transpose(2, 3) @ Gc[:, sl])
+        band.add_windows(acc_u, j0, df.transpose(2, 3) @ Pc[:, sl])
+    dQ += band.unchunk(dQc)
+    uq -= psi * band.unchunk(uqc)
+    dK += band.fold(acc_k)
+    dV += band.fold(acc_v)
+    uk -= phik * band.fold(acc_u)
+
+
 def sblocal_backward(query, key, value, projection_matrix, local_context, softmax_temp, key_lengths,
-                     out, log_normalization, grad_out, chunk=256, max_elements=1 << 27):
+                     out, log_normalization, grad_out, chunk=256, max_elements=1 << 27, band_kernel=None):
     """query (B,T,H,E), key (B,S,H,E), value (B,S,H,D), out / grad_out (B,T,H,D),
     log_normalization (B,H,T,1) as returned by the forward; key_lengths (B,) or None.
     max_elements bounds the
     size of the (batch, chunks, chunk, window) intermediates: chunks are taken in groups that stay below it.
+    band_kernel: None = the fused band kernels where they apply (GPU, head dims <= 64, <= 128 features),
+    False = batched library products, True = the kernels or NotImplementedError.
     Returns (d query, d key, d value) in the dtypes of the inputs."""
     B, T, H, E = query.shape
     S, D = key.shape[1], value.shape[3]
@@ -138,32 +216,21 @@ def sblocal_backward(query, key, value, projection_matrix, local_context, softma
     dQ = torch.zeros_like(Q)
     dK = torch.zeros_like(K)
 
-    # band terms, all chunks of queries at once: chunk j (queries jC .. jC+C-1) against the window of
-    # keys jC - lc_lo .. jC - lc_lo + W - 1 that its bands touch; inside a window the band is the same
-    # (C, W) pattern for every chunk
-    band = BandWindows(T, S, local_context, chunk, Q.device, lens, max_elements)
-    Qc, Gc, Pc, cc, LNc = (band.chunks(x) for x in (Q, G, psi, c, LN))
-    acc_k, acc_v, acc_u = band.key_accumulator(E, wdt), band.key_accumulator(D, wdt), band.key_accumulator(2 * mh, wdt)
-    dQc, uqc = torch.zeros_like(Qc), torch.zeros_like(Pc)
-    Kw, Vw, PKw = band.windows(K), band.windows(V), band.windows(phik)
-    for j0, j1 in band.groups(B * H):
-        sl = slice(j0, j1)
-        ks, vs, pk = Kw[:, sl], Vw[:, sl], PKw[:, sl]               # (BH, g, W, .)
-        valid = band.mask(j0, j1).to(wdt)
-        a_bar = torch.exp(t * (Qc[:, sl] @ ks.transpose(2, 3)) - LNc[:, sl]) * valid
-        k_bar = (Pc[:, sl] @ pk.transpose(2, 3)) * valid
-        df = (Gc[:, sl] @ vs.transpose(2, 3) - cc[:, sl]) * valid
-        dm = a_bar * df
-        dQc[:, sl] = t * (dm @ ks)
-        uqc[:, sl] = df @ pk
-        band.add_windows(acc_k, j0, t * (dm.transpose(2, 3) @ Qc[:, sl]))
-        band.add_windows(acc_v, j0, (a_bar - k_bar).transpose(2, 3) @ Gc[:, sl])
-        band.add_windows(acc_u, j0, df.transpose(2, 3) @ Pc[:, sl])
-    dQ += band.unchunk(dQc)
-    uq -= psi * band.unchunk(uqc)
-    dK += band.fold(acc_k)
-    dV += band.fold(acc_v)
-    uk -= phik * band.fold(acc_u)
+    dims = _band_kernel_dims(E, D, 2 * mh) if band_kernel is not False else None
+    if band_kernel and dims is None:
+        raise NotImplementedError(f'no band kernel for head dims ({E}, {D}) with {2 * mh} features')
+    if dims is not None and Q.is_cuda and wdt == torch.float32:
+        # band terms on the fused kernels: one launch with lane-owned queries, one with lane-owned keys
+        lens_b = None if key_lengths is None else key_lengths.to(device=Q.device, dtype=torch.int64).contiguous()
+        dQ_b, uq_b, dK_b, uk_b, dV_b = _band_terms_hip(Q, K, V, G, psi, phik, LN, c, lens_b, H, local_context, t, dims)
+        dQ += dQ_b
+        uq -= psi * uq_b
+        dK += dK_b
+        uk -= phik * uk_b
+        dV += dV_b
+    else:
+        _band_terms_torch(Q, K, V, G, psi, phik, LN, c, lens, local_context, t, chunk, max_elements,
+                          dQ, dK, dV, uq, uk)
 
     st = math.sqrt(t)
     dQ += st * ((uq[..., :mh] - uq[..., mh:]) @ P) - t * Q * uq.sum(-1, keepdim=True)

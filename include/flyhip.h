@@ -98,6 +98,23 @@ int flyhip_sblocal_fwd(const void* q, const void* k, const void* v, const float*
                        int64_t o_sb, int64_t o_sh, int64_t o_ss,
                        float softmax_temp, int dtype, void* stream);
 
+/* Band terms of the backward pass of Scatterbrain-local attention (the reference differentiates its op
+ * sequence sblocal_attention.py:90-122 with autograd and the backward kernels of
+ * fast_transformers.local_product).  For a (query i, key s) pair inside the band, with
+ * a = exp(t q_i.k_s - log_norm_i), kb = psi_i.phik_s, df = g_i.v_s - c_i, dm = a df:
+ *   key_major = 0 (outer = queries, T rows; inner = keys):  x1 = q, x3 = g, y1 = k, y2 = phik, y3 = v;
+ *       o1 = t sum_s dm k_s (T,E), o2 = sum_s df phik_s (T,M); x2, o3 unused (may be NULL)
+ *   key_major = 1 (outer = keys, S rows; inner = queries):  x1 = k, x2 = phik, x3 = v, y1 = q, y2 = psi,
+ *       y3 = g;  o1 = t sum_i dm q_i (S,E), o2 = sum_i df psi_i (S,M), o3 = sum_i (a - kb) g_i (S,E)
+ * All tensors float32, contiguous (BH, rows, width), widths E, M, E; log_norm and c are (BH, T);
+ * key_lengths (BH / H) int64 or NULL; (E, M) in {(32,32),(32,64),(64,32),(64,64),(64,128)}. */
+int flyhip_sblocal_bwd_band(const float* x1, const float* x2, const float* x3,
+                            const float* y1, const float* y2, const float* y3,
+                            const float* log_norm, const float* c, const int64_t* key_lengths,
+                            float* o1, float* o2, float* o3,
+                            int BH, int H, int T, int S, int E, int M, int local_context,
+                            float softmax_temp, int key_major, void* stream);
+
 /* Plain local attention, no random features (ref: src/models/attention/local_attention.py:68-92;
  * fast_transformers.local_product): out[i] = softmax over the band -(lc/2) <= s - i < (lc+1)/2, s below
  * the key length, of t q_i.k_s, times v.  q (B,T,H,E), k (B,S,H,E), v (B,S,H,D), out (B,T,H,D) via

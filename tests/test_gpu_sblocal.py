@@ -226,3 +226,31 @@ def test_local_attention_module_gradients(dtype, tol):
     for got, ref in ((qg.grad, qd.grad), (kg.grad, kd.grad), (vg.grad, vd.grad)):
         assert got.dtype == dtype and rel_err(got.float(), ref) <= tol, rel_err(got.float(), ref)
     assert float(kg.grad[1, 200:].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize('B,T,S,H,E,D,mh,lc,lens', [(2, 300, 280, 2, 64, 64, 32, 64, [280, 200]),
+                                                    (1, 257, 391, 3, 50, 40, 24, 77, None),
+                                                    (2, 130, 130, 1, 32, 32, 16, 301, [130, 1]),
+                                                    (1, 100, 600, 2, 64, 64, 64, 48, [500]),
+                                                    (2, 3136, 3136, 1, 64, 64, 64, 512, None)])
+def test_backward_band_kernels_match_library_products(B, T, S, H, E, D, mh, lc, lens):
+    """The two band kernels of the backward pass (lane-owned queries, lane-owned keys) against the same
+    sums as batched library products, which the CPU suite checks against autograd through the oracle:
+    T != S, odd windows, windows wider than the sequence, key lengths (a batch entry with one key),
+    head dims and feature counts that need padding, and BASELINE config 1's size."""
+    from fly_amd import sblocal_backward
+    from fly_amd.sblocal_attention import sblocal_forward
+    print('case', B, T, S, H, E, D, mh, lc, lens, flush=True)
+    dev = torch.device('cuda:0')
+    g = torch.Generator().manual_seed(7)
+    q = (torch.randn(B, T, H, E, generator=g) * E ** -0.25).to(dev)
+    k = (torch.randn(B, S, H, E, generator=g) * E ** -0.25).to(dev)
+    v = torch.randn(B, S, H, D, generator=g).to(dev)
+    go = torch.randn(B, T, H, D, generator=g).to(dev)
+    P = osb.gaussian_orthogonal_random_matrix(mh, E, generator=g).to(dev)
+    kl = None if lens is None else torch.tensor(lens, device=dev)
+    out, ln = sblocal_forward(q, k, v, P, lc, key_lengths=kl)
+    ref = sblocal_backward(q, k, v, P, lc, None, kl, out, ln, go, band_kernel=False)
+    got = sblocal_backward(q, k, v, P, lc, None, kl, out, ln, go, band_kernel=True)
+    for a, b in zip(got, ref):
+        assert rel_err(a, b) <= 1e-4, rel_err(a, b)
