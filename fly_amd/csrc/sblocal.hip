@@ -1986,9 +1986,21 @@ struct BwdArgs {
     float* o1; float* o2; float* o3;                        // outer rows (o3 only key-major)
     int BH, H, T, S, lc;
     float temp;
+    // finishing pass: global low-rank terms and the chain rule through the feature map in the epilogue
+    const float* gmat; const float* gvec; const float* proj;
 };
 
-template <int E, int M, bool KEYMAJOR>
+//
+// With FINISH the epilogue turns the sums into the gradients themselves.  The low-rank weight outside
+// the band is "all keys minus the band", and the sums over all keys are products with small per-head
+// matrices computed beforehand: gmat | gvec = K'^T V | sum K' for the query-major pass (K' = phik),
+// Q'^T g | Q'^T c for the key-major pass (Q' = psi).  With x2 = the outer row's own features (psi
+// resp. phik), u_f = x2_f (gmat_f . x3 - c gvec_f - out2_f) is the gradient with respect to the log of
+// feature f (c = the query's g.out, resp. 1 for a key), and
+//   d x1 = out1 + sqrt(t) P^T (u+ - u-) - t x1 sum_f u_f,    d v = out3 + gmat^T phik   (key-major)
+// where features f < M/2 are the exp(+.) half and f + M/2 their exp(-.) partners.  o1 (and o3)
+// receive the gradients; o2 is not written.
+template <int E, int M, bool KEYMAJOR, bool FINISH>
 __global__ __launch_bounds__(NT) void sblocal_bwd_band_kernel(BwdArgs a) {
     constexpr int D = E, LDK = E + 4, LDV = D + 4, LDF = M + 4;
     constexpr int EC = E / 16, FC = M / 16, DB = D / 16, KB = TK / 16;
@@ -2047,13 +2059,13 @@ __global__ __launch_bounds__(NT) void sblocal_bwd_band_kernel(BwdArgs a) {
 
     // outer operands (B side: column = outer row, k = 16c + 4g + j); exponents are base 2
     const int orow = min(o, Lo - 1);
-    floatx4 x1[EC], x3[DB], x2[KEYMAJOR ? FC : 1];
+    floatx4 x1[EC], x3[DB], x2[(KEYMAJOR || FINISH) ? FC : 1];
 #pragma unroll
     for (int c = 0; c < EC; ++c)
         x1[c] = load4_f32(a.x1 + ((long)bh * Lo + orow) * E + 16 * c + 4 * g) * (a.temp * LOG2E);
 #pragma unroll
     for (int c = 0; c < DB; ++c) x3[c] = load4_f32(a.x3 + ((long)bh * Lo + orow) * D + 16 * c + 4 * g);
-    if (KEYMAJOR) {
+    if (KEYMAJOR || FINISH) {
 #pragma unroll
         for (int c = 0; c < FC; ++c) x2[c] = load4_f32(a.x2 + ((long)bh * Lo + orow) * M + 16 * c + 4 * g);
     }
@@ -2162,6 +2174,85 @@ __global__ __launch_bounds__(NT) void sblocal_bwd_band_kernel(BwdArgs a) {
         __syncthreads();
     }
 
+    if (FINISH) {
+        // per-head matrices into the tile stages (dead now; the loop ended on a barrier)
+        constexpr int MH = M / 2;
+        float* GMs = smem;                          // gmat (M, D), rows of LDV
+        float* GVs = GMs + M * LDV;                 // gvec (M)
+        float* Ps = GVs + M;                        // projection (M/2, E), rows of LDK
+        static_assert(M * LDV + M + MH * LDK <= 2 * STAGE, "epilogue operands must fit the tile stages");
+        {
+            RowTile<M, D> gm;
+            gm.fetch(a.gmat + (long)bh * M * D, D, 0, M - 1, tid);
+            RowTile<MH, E> pt;
+            pt.fetch(a.proj, E, 0, MH - 1, tid);
+            if (tid < M) GVs[tid] = a.gvec[(long)bh * M + tid];
+            gm.template stash<LDV>(GMs, tid);
+            pt.template stash<LDK>(Ps, tid);
+        }
+        __syncthreads();
+        // u^T[f][outer] = sum_d gmat[f][d] x3[d][outer]
+        floatx4 u[FC];
+#pragma unroll
+        for (int c = 0; c < FC; ++c) u[c] = Frag<float>::zero();
+#pragma unroll
+        for (int cd = 0; cd < DB; ++cd) {
+            floatx4 ga[FC];
+#pragma unroll
+            for (int c = 0; c < FC; ++c) ga[c] = *reinterpret_cast<const floatx4*>(GMs + (16 * c + r16) * LDV + 16 * cd + 4 * g);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int c = 0; c < FC; ++c) u[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(ga[c][j], x3[cd][j], u[c], 0, 0, 0);
+        }
+        const float cmul = KEYMAJOR ? 1.0f : c_o;
+        float usum = 0.f;
+#pragma unroll
+        for (int c = 0; c < FC; ++c) {
+            const floatx4 gv = *reinterpret_cast<const floatx4*>(GVs + 16 * c + 4 * g);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                u[c][i] = x2[c][i] * (u[c][i] - cmul * gv[i] - acc2[c][i]);
+                usum += u[c][i];
+            }
+        }
+        usum = group_sum(usum);
+        // chain rule through the projection: dp^T[e][outer] = sum_r P[r][e] (u_r - u_{r + M/2})
+        floatx4 dp[EC];
+#pragma unroll
+        for (int c = 0; c < EC; ++c) dp[c] = Frag<float>::zero();
+#pragma unroll
+        for (int c = 0; c < FC / 2; ++c) {
+            const floatx4 du = u[c] - u[c + FC / 2];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int eb = 0; eb < EC; ++eb)
+                    dp[eb] = __builtin_amdgcn_mfma_f32_16x16x4f32(Ps[(16 * c + 4 * g + j) * LDK + 16 * eb + r16], du[j], dp[eb], 0, 0, 0);
+        }
+        if (KEYMAJOR) {
+            // d v^T[d][key] += sum_f gmat[f][d] phik[f][key]
+#pragma unroll
+            for (int c = 0; c < FC; ++c)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int db = 0; db < DB; ++db)
+                        acc3[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(GMs[(16 * c + 4 * g + j) * LDV + 16 * db + r16], x2[c][j], acc3[db], 0, 0, 0);
+        }
+        if (o < Lo) {
+            const float st = sqrtf(a.temp), back = 1.0f / LOG2E;     // x1 carries t log2(e)
+            float* p1 = a.o1 + ((long)bh * Lo + o) * E;
+#pragma unroll
+            for (int c = 0; c < EC; ++c) store4_f32(p1 + 16 * c + 4 * g, acc1[c] * a.temp + dp[c] * st - x1[c] * (back * usum));
+            if (KEYMAJOR) {
+                float* p3 = a.o3 + ((long)bh * Lo + o) * D;
+#pragma unroll
+                for (int c = 0; c < DB; ++c) store4_f32(p3 + 16 * c + 4 * g, acc3[c]);
+            }
+        }
+        return;
+    }
     if (o < Lo) {
         float* p1 = a.o1 + ((long)bh * Lo + o) * E;
         float* p2 = a.o2 + ((long)bh * Lo + o) * M;
@@ -2177,9 +2268,9 @@ __global__ __launch_bounds__(NT) void sblocal_bwd_band_kernel(BwdArgs a) {
     }
 }
 
-template <int E, int M, bool KEYMAJOR>
+template <int E, int M, bool KEYMAJOR, bool FINISH>
 static int launch_bwd_band(const BwdArgs& a, hipStream_t st) {
-    auto kern = sblocal_bwd_band_kernel<E, M, KEYMAJOR>;
+    auto kern = sblocal_bwd_band_kernel<E, M, KEYMAJOR, FINISH>;
     constexpr size_t smem = sizeof(float) * 2 * (TK * (3 * 4 + 2 * E + M) + 2 * TK);
     static bool lds_ready = false;
     if (!lds_ready) {
@@ -2197,7 +2288,9 @@ static int launch_bwd_band(const BwdArgs& a, hipStream_t st) {
 
 template <int E, int M>
 static int launch_bwd_band_both(const BwdArgs& a, bool key_major, hipStream_t st) {
-    return key_major ? launch_bwd_band<E, M, true>(a, st) : launch_bwd_band<E, M, false>(a, st);
+    if (a.gmat)
+        return key_major ? launch_bwd_band<E, M, true, true>(a, st) : launch_bwd_band<E, M, false, true>(a, st);
+    return key_major ? launch_bwd_band<E, M, true, false>(a, st) : launch_bwd_band<E, M, false, false>(a, st);
 }
 
 #define SB_DISPATCH_M(FN, T, EE, ARGS)                                       \
@@ -2395,6 +2488,8 @@ extern "C" int flyhip_local_fwd(const void* q, const void* k, const void* v, con
     return fail(ERR_UNSUPPORTED, "local_fwd supports float32 and bfloat16, got dtype code %d", dtype);
 }
 
+static int dispatch_bwd_band(const BwdArgs& a, int E, int M, int key_major, void* stream);
+
 extern "C" int flyhip_sblocal_bwd_band(const float* x1, const float* x2, const float* x3,
                                        const float* y1, const float* y2, const float* y3,
                                        const float* log_norm, const float* c, const int64_t* key_lengths,
@@ -2406,7 +2501,30 @@ extern "C" int flyhip_sblocal_bwd_band(const float* x1, const float* x2, const f
     FLY_REQUIRE(BH > 0 && H > 0 && BH % H == 0 && T > 0 && S > 0, "sblocal_bwd_band: empty or inconsistent problem");
     FLY_REQUIRE(local_context >= 1, "sblocal_bwd_band: local_context must be >= 1");
     FLY_REQUIRE(softmax_temp > 0.f, "sblocal_bwd_band: softmax_temp must be positive");
-    BwdArgs a{x1, x2, x3, y1, y2, y3, log_norm, c, key_lengths, o1, o2, o3, BH, H, T, S, local_context, softmax_temp};
+    BwdArgs a{x1, x2, x3, y1, y2, y3, log_norm, c, key_lengths, o1, o2, o3, BH, H, T, S, local_context, softmax_temp,
+              nullptr, nullptr, nullptr};
+    return dispatch_bwd_band(a, E, M, key_major, stream);
+}
+
+extern "C" int flyhip_sblocal_bwd(const float* x1, const float* x2, const float* x3,
+                                  const float* y1, const float* y2, const float* y3,
+                                  const float* log_norm, const float* c, const int64_t* key_lengths,
+                                  const float* gmat, const float* gvec, const float* proj,
+                                  float* d1, float* d3,
+                                  int BH, int H, int T, int S, int E, int M, int local_context,
+                                  float softmax_temp, int key_major, void* stream) {
+    FLY_REQUIRE(x1 && x2 && x3 && y1 && y2 && y3 && log_norm && c && gmat && gvec && proj && d1,
+                "sblocal_bwd: null pointer");
+    FLY_REQUIRE(!key_major || d3, "sblocal_bwd: the key-major pass needs d3");
+    FLY_REQUIRE(BH > 0 && H > 0 && BH % H == 0 && T > 0 && S > 0, "sblocal_bwd: empty or inconsistent problem");
+    FLY_REQUIRE(local_context >= 1, "sblocal_bwd: local_context must be >= 1");
+    FLY_REQUIRE(softmax_temp > 0.f, "sblocal_bwd: softmax_temp must be positive");
+    BwdArgs a{x1, x2, x3, y1, y2, y3, log_norm, c, key_lengths, d1, nullptr, d3, BH, H, T, S, local_context, softmax_temp,
+              gmat, gvec, proj};
+    return dispatch_bwd_band(a, E, M, key_major, stream);
+}
+
+static int dispatch_bwd_band(const BwdArgs& a, int E, int M, int key_major, void* stream) {
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     if (E == 32 && M == 32) return launch_bwd_band_both<32, 32>(a, key_major != 0, st);
     if (E == 32 && M == 64) return launch_bwd_band_both<32, 64>(a, key_major != 0, st);

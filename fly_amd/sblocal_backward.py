@@ -113,6 +113,49 @@ def _band_kernel_dims(E, D, M):
     return None
 
 
+def _fit(x, width):
+    if x.shape[-1] != width:
+        x = torch.nn.functional.pad(x, (0, width - x.shape[-1]))
+    return x.contiguous()
+
+
+def _fit_features(x, mk):
+    """(.., 2 mh) -> (.., mk) keeping the two halves (exp(+.), exp(-.)) at f and f + mk/2."""
+    mh = x.shape[-1] // 2
+    if 2 * mh == mk:
+        return x.contiguous()
+    pad = (0, mk // 2 - mh)
+    return torch.cat([torch.nn.functional.pad(x[..., :mh], pad), torch.nn.functional.pad(x[..., mh:], pad)], dim=-1)
+
+
+def _backward_hip(Q, K, V, G, psi, phik, LN, c, P, lens_b, H, local_context, t, dims):
+    """d query, d key, d value (BH, rows, width) on two launches of flyhip_sblocal_bwd: the small
+    per-head reductions over all keys / all queries are library products, everything per (query, key)
+    pair and per row runs in the kernels."""
+    from . import _lib
+    BH, T, E = Q.shape
+    S, D = K.shape[1], V.shape[2]
+    dim, mk = dims
+    q_, k_, v_, g_ = _fit(Q, dim), _fit(K, dim), _fit(V, dim), _fit(G, dim)
+    psi_, phik_ = _fit_features(psi, mk), _fit_features(phik, mk)
+    proj = _fit(torch.nn.functional.pad(P, (0, 0, 0, mk // 2 - P.shape[0])), dim)
+    ln_, c_ = LN.reshape(BH, T).contiguous(), c.reshape(BH, T).contiguous()
+    kv = (phik_.transpose(1, 2) @ v_).contiguous()           # (BH, mk, dim)   sum_s phik_s v_s^T
+    ksum = phik_.sum(1)                                      # (BH, mk)
+    qg = (psi_.transpose(1, 2) @ g_).contiguous()            # (BH, mk, dim)   sum_i psi_i g_i^T
+    qc = torch.einsum('btm,bt->bm', psi_, c_).contiguous()   # (BH, mk)
+    dq, dk, dv = Q.new_empty(BH, T, dim), Q.new_empty(BH, S, dim), Q.new_empty(BH, S, dim)
+    with torch.cuda.device(Q.device):
+        st = _lib.stream_ptr(Q.device)
+        _lib.call('flyhip_sblocal_bwd', q_.data_ptr(), psi_.data_ptr(), g_.data_ptr(), k_.data_ptr(), phik_.data_ptr(),
+                  v_.data_ptr(), ln_.data_ptr(), c_.data_ptr(), _lib.ptr(lens_b), kv.data_ptr(), ksum.data_ptr(),
+                  proj.data_ptr(), dq.data_ptr(), None, BH, H, T, S, dim, mk, local_context, float(t), 0, st)
+        _lib.call('flyhip_sblocal_bwd', k_.data_ptr(), phik_.data_ptr(), v_.data_ptr(), q_.data_ptr(), psi_.data_ptr(),
+                  g_.data_ptr(), ln_.data_ptr(), c_.data_ptr(), _lib.ptr(lens_b), qg.data_ptr(), qc.data_ptr(),
+                  proj.data_ptr(), dk.data_ptr(), dv.data_ptr(), BH, H, T, S, dim, mk, local_context, float(t), 1, st)
+    return dq[..., :E], dk[..., :E], dv[..., :D]
+
+
 def _band_terms_hip(Q, K, V, G, psi, phik, LN, c, lens_b, H, local_context, t, dims):
     """The five band-limited sums on flyhip_sblocal_bwd_band.  Q, G, psi, LN, c: (BH, T, .); K, V, phik:
     (BH, S, .); float32 on the GPU.  Returns (t sum_s dm k, sum_s df phik, t sum_i dm q, sum_i df psi,
@@ -121,13 +164,8 @@ def _band_terms_hip(Q, K, V, G, psi, phik, LN, c, lens_b, H, local_context, t, d
     BH, T, E = Q.shape
     S, D, M = K.shape[1], V.shape[2], psi.shape[2]
     dim, mk = dims
-
-    def fit(x, width):
-        if x.shape[2] != width:
-            x = torch.nn.functional.pad(x, (0, width - x.shape[2]))
-        return x.contiguous()
-    q_, k_, v_, g_ = fit(Q, dim), fit(K, dim), fit(V, dim), fit(G, dim)
-    psi_, phik_ = fit(psi, mk), fit(phik, mk)
+    q_, k_, v_, g_ = _fit(Q, dim), _fit(K, dim), _fit(V, dim), _fit(G, dim)
+    psi_, phik_ = _fit(psi, mk), _fit(phik, mk)
     ln_, c_ = LN.reshape(BH, T).contiguous(), c.reshape(BH, T).contiguous()
     dq, uq = Q.new_empty(BH, T, dim), Q.new_empty(BH, T, mk)
     dk, uk, dv = Q.new_empty(BH, S, dim), Q.new_empty(BH, S, mk), Q.new_empty(BH, S, dim)
@@ -181,8 +219,9 @@ def sblocal_backward(query, key, value, projection_matrix, local_context, softma
     log_normalization (B,H,T,1) as returned by the forward; key_lengths (B,) or None.
     max_elements bounds the
     size of the (batch, chunks, chunk, window) intermediates: chunks are taken in groups that stay below it.
-    band_kernel: None = the fused band kernels where they apply (GPU, head dims <= 64, <= 128 features),
-    False = batched library products, True = the kernels or NotImplementedError.
+    band_kernel: None = the fused kernels where they apply (GPU, head dims <= 64, <= 128 features): band
+    sums, global low-rank terms and the feature-map chain rule in two launches; 'sums' = only the band
+    sums on the kernels; False = batched library products; True = the kernels or NotImplementedError.
     Returns (d query, d key, d value) in the dtypes of the inputs."""
     B, T, H, E = query.shape
     S, D = key.shape[1], value.shape[3]
@@ -206,35 +245,38 @@ def sblocal_backward(query, key, value, projection_matrix, local_context, softma
     psi = phiq * torch.exp(lsq + lsk - LN)       # Phi(q_i) Phi(k_s) / Z_i = psi_i . phik_s
     c = (G * O).sum(-1, keepdim=True)
 
-    kv = phik.transpose(1, 2) @ V                # (BH, m, D)   sum_s phik_s v_s^T
-    ksum = phik.sum(1)                           # (BH, m)
-    qg = psi.transpose(1, 2) @ G                 # (BH, m, D)   sum_i psi_i g_i^T
-    qc = (psi * c).sum(1)                        # (BH, m)
-    uq = psi * (G @ kv.transpose(1, 2) - c * ksum.unsqueeze(1))
-    uk = phik * (V @ qg.transpose(1, 2) - qc.unsqueeze(1))
-    dV = phik @ qg
-    dQ = torch.zeros_like(Q)
-    dK = torch.zeros_like(K)
-
     dims = _band_kernel_dims(E, D, 2 * mh) if band_kernel is not False else None
     if band_kernel and dims is None:
         raise NotImplementedError(f'no band kernel for head dims ({E}, {D}) with {2 * mh} features')
-    if dims is not None and Q.is_cuda and wdt == torch.float32:
-        # band terms on the fused kernels: one launch with lane-owned queries, one with lane-owned keys
-        lens_b = None if key_lengths is None else key_lengths.to(device=Q.device, dtype=torch.int64).contiguous()
-        dQ_b, uq_b, dK_b, uk_b, dV_b = _band_terms_hip(Q, K, V, G, psi, phik, LN, c, lens_b, H, local_context, t, dims)
-        dQ += dQ_b
-        uq -= psi * uq_b
-        dK += dK_b
-        uk -= phik * uk_b
-        dV += dV_b
+    on_kernels = dims is not None and Q.is_cuda and wdt == torch.float32
+    lens_b = None if key_lengths is None else key_lengths.to(device=Q.device, dtype=torch.int64).contiguous()
+    if on_kernels and band_kernel != 'sums':
+        # everything after the features on the two passes of the fused kernel
+        dQ, dK, dV = _backward_hip(Q, K, V, G, psi, phik, LN, c, P, lens_b, H, local_context, t, dims)
     else:
-        _band_terms_torch(Q, K, V, G, psi, phik, LN, c, lens, local_context, t, chunk, max_elements,
-                          dQ, dK, dV, uq, uk)
-
-    st = math.sqrt(t)
-    dQ += st * ((uq[..., :mh] - uq[..., mh:]) @ P) - t * Q * uq.sum(-1, keepdim=True)
-    dK += st * ((uk[..., :mh] - uk[..., mh:]) @ P) - t * K * uk.sum(-1, keepdim=True)
+        kv = phik.transpose(1, 2) @ V                # (BH, m, D)   sum_s phik_s v_s^T
+        ksum = phik.sum(1)                           # (BH, m)
+        qg = psi.transpose(1, 2) @ G                 # (BH, m, D)   sum_i psi_i g_i^T
+        qc = (psi * c).sum(1)                        # (BH, m)
+        uq = psi * (G @ kv.transpose(1, 2) - c * ksum.unsqueeze(1))
+        uk = phik * (V @ qg.transpose(1, 2) - qc.unsqueeze(1))
+        dV = phik @ qg
+        dQ = torch.zeros_like(Q)
+        dK = torch.zeros_like(K)
+        if on_kernels:
+            # only the band-limited sums on the kernels
+            dQ_b, uq_b, dK_b, uk_b, dV_b = _band_terms_hip(Q, K, V, G, psi, phik, LN, c, lens_b, H, local_context, t, dims)
+            dQ += dQ_b
+            uq -= psi * uq_b
+            dK += dK_b
+            uk -= phik * uk_b
+            dV += dV_b
+        else:
+            _band_terms_torch(Q, K, V, G, psi, phik, LN, c, lens, local_context, t, chunk, max_elements,
+                              dQ, dK, dV, uq, uk)
+        st = math.sqrt(t)
+        dQ += st * ((uq[..., :mh] - uq[..., mh:]) @ P) - t * Q * uq.sum(-1, keepdim=True)
+        dK += st * ((uk[..., :mh] - uk[..., mh:]) @ P) - t * K * uk.sum(-1, keepdim=True)
 
     def back(x, like):                           # (B*H, L, C) -> (B,L,H,C)
         return x.reshape(B, H, x.shape[1], x.shape[2]).permute(0, 2, 1, 3).to(like.dtype)

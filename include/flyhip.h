@@ -115,6 +115,22 @@ int flyhip_sblocal_bwd_band(const float* x1, const float* x2, const float* x3,
                             int BH, int H, int T, int S, int E, int M, int local_context,
                             float softmax_temp, int key_major, void* stream);
 
+/* The whole backward pass after the feature maps, one call per side (same operand roles as
+ * flyhip_sblocal_bwd_band, x2 = the outer rows' own features in both passes: psi for key_major = 0,
+ * phik for key_major = 1).  The epilogue adds the low-rank weight outside the band ("all keys minus the
+ * band") through the per-head reductions gmat (BH,M,E) | gvec (BH,M) -- phik^T v | sum phik for
+ * key_major = 0, psi^T g | psi^T c for key_major = 1 -- and the chain rule through the feature map
+ * (feature_maps_sb.py:51-82: features f < M/2 are exp(+sqrt(t) p_f.x - ..), f + M/2 their exp(-..)
+ * partners; proj (M/2, E) float32):  d1 = gradient of x1 (d query (T,E) resp. d key (S,E)),
+ * d3 = d value (S,E), key_major = 1 only. */
+int flyhip_sblocal_bwd(const float* x1, const float* x2, const float* x3,
+                       const float* y1, const float* y2, const float* y3,
+                       const float* log_norm, const float* c, const int64_t* key_lengths,
+                       const float* gmat, const float* gvec, const float* proj,
+                       float* d1, float* d3,
+                       int BH, int H, int T, int S, int E, int M, int local_context,
+                       float softmax_temp, int key_major, void* stream);
+
 /* Plain local attention, no random features (ref: src/models/attention/local_attention.py:68-92;
  * fast_transformers.local_product): out[i] = softmax over the band -(lc/2) <= s - i < (lc+1)/2, s below
  * the key length, of t q_i.k_s, times v.  q (B,T,H,E), k (B,S,H,E), v (B,S,H,D), out (B,T,H,D) via

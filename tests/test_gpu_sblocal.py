@@ -251,6 +251,7 @@ def test_backward_band_kernels_match_library_products(B, T, S, H, E, D, mh, lc, 
     kl = None if lens is None else torch.tensor(lens, device=dev)
     out, ln = sblocal_forward(q, k, v, P, lc, key_lengths=kl)
     ref = sblocal_backward(q, k, v, P, lc, None, kl, out, ln, go, band_kernel=False)
-    got = sblocal_backward(q, k, v, P, lc, None, kl, out, ln, go, band_kernel=True)
-    for a, b in zip(got, ref):
-        assert rel_err(a, b) <= 1e-4, rel_err(a, b)
+    for mode in ('sums', True):          # band sums only / everything after the features on the kernels
+        got = sblocal_backward(q, k, v, P, lc, None, kl, out, ln, go, band_kernel=mode)
+        for a, b in zip(got, ref):
+            assert rel_err(a, b) <= 1e-4, (mode, rel_err(a, b))
