@@ -23,7 +23,6 @@ import math
 
 import torch
 
-from .feature_maps_sb import softmax_kernel
 
 
 class BandWindows:
@@ -213,6 +212,30 @@ def _band_terms_torch(Q, K, V, G, psi, phik, LN, c, lens, local_context, t, chun
     uk -= phik * band.fold(acc_u)
 
 
+def _scaled_features(Q, K, P, t, LN, lens):
+    """psi (BH,T,m) and phik (BH,S,m) with psi_i . phik_s = Phi(q_i) . Phi(k_s) / Z_i, the low-rank weight
+    of the pair (feature_maps_sb.py:51-82 gives Phi_r(x) = exp(+-sqrt(t) p_r.x - t |x|^2 / 2) / sqrt(m),
+    the + half first).  One stabiliser kappa per (batch, head), the largest log-feature of a valid key,
+    is taken out of the keys and put into the queries together with -log Z; keys at or past the key
+    length get zero features."""
+    mh = P.shape[0]
+    Pt = (math.sqrt(t) * P).t()
+    dq, dk = Q @ Pt, K @ Pt                                              # (BH, rows, mh)
+    off = math.log(2 * mh) / 2
+    bk = K.square().sum(-1, keepdim=True).mul_(-t / 2).sub_(off)        # (BH, S, 1): log-feature = +-dk + bk
+    if lens is not None:
+        bk = bk.masked_fill(torch.arange(K.shape[1], device=K.device).view(1, -1, 1) >= lens, -math.inf)
+    kappa = (dk.abs().amax(-1, keepdim=True) + bk).amax(1, keepdim=True).nan_to_num_(neginf=0.0)
+    bk = bk - kappa
+    bq = kappa - LN - Q.square().sum(-1, keepdim=True).mul_(t / 2) - off
+    psi, phik = Q.new_empty(*dq.shape[:2], 2 * mh), K.new_empty(*dk.shape[:2], 2 * mh)
+    torch.exp(dq + bq, out=psi[..., :mh])
+    torch.exp(bq - dq, out=psi[..., mh:])
+    torch.exp(dk + bk, out=phik[..., :mh])
+    torch.exp(bk - dk, out=phik[..., mh:])
+    return psi, phik
+
+
 def sblocal_backward(query, key, value, projection_matrix, local_context, softmax_temp, key_lengths,
                      out, log_normalization, grad_out, chunk=256, max_elements=1 << 27, band_kernel=None):
     """query (B,T,H,E), key (B,S,H,E), value (B,S,H,D), out / grad_out (B,T,H,D),
@@ -236,13 +259,10 @@ def sblocal_backward(query, key, value, projection_matrix, local_context, softma
     P = projection_matrix.to(wdt)
     mh = P.shape[0]
 
-    phiq, lsq = softmax_kernel(Q, projection_matrix=P, is_query=True, softmax_temp=t)
-    phik, lsk = softmax_kernel(K, projection_matrix=P, is_query=False, softmax_temp=t)
     lens = None
     if key_lengths is not None:
         lens = key_lengths.to(Q.device).repeat_interleave(H).view(B * H, 1, 1)
-        phik = phik * (torch.arange(S, device=Q.device).view(1, S, 1) < lens)
-    psi = phiq * torch.exp(lsq + lsk - LN)       # Phi(q_i) Phi(k_s) / Z_i = psi_i . phik_s
+    psi, phik = _scaled_features(Q, K, P, t, LN, lens)
     c = (G * O).sum(-1, keepdim=True)
 
     dims = _band_kernel_dims(E, D, 2 * mh) if band_kernel is not False else None
