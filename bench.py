@@ -199,6 +199,20 @@ def bench_blocksparse(steps, warmup):
     return out
 
 
+def sblocal_train_step(q, k, v, P, lc, temp):
+    """A closure running one forward + backward of Scatterbrain-local attention with respect to q, k, v."""
+    import fly_amd
+    qg, kg, vg = (x.clone().requires_grad_() for x in (q, k, v))
+    go = torch.randn_like(v)
+
+    def run():
+        o = fly_amd.sblocal_attention_fn(qg, kg, vg, P, lc, temp, None)
+        o = o[0] if isinstance(o, tuple) else o
+        o.backward(go)
+        qg.grad = kg.grad = vg.grad = None
+    return run
+
+
 def bench_other_configs():
     """Timings of the remaining BASELINE configs (stream events around whole forwards):
     3 = the two Scatterbrain-local layers of T2T-ViT-t-14 at batch 64 (fp32), 4 = the two Pixelfly
@@ -232,8 +246,17 @@ def bench_other_configs():
         ms = timeit(lambda: plan.run(q, k, v, P, None, lc, dim ** -0.5, o, ln))
         fl, _ = sblocal_flops(B, H, L, L, E, E, 2 * mh, lc)
         out[f'config3_sblocal_fp32_B64_L{L}'] = {'ms': ms, 'tflops': fl / ms / 1e9, 'tokens_per_s': B * L / ms * 1e3,
-                                                 'mfma_fp32_frac': fl / ms / 1e9 / PEAK_FP32_MFMA_TFLOPS}
+                                                 'mfma_fp32_frac': fl / ms / 1e9 / PEAK_FP32_MFMA_TFLOPS,
+                                                 'fwd_bwd_ms': timeit(sblocal_train_step(q, k, v, P, lc, dim ** -0.5), n=5)}
         del q, k, v, o, ln, plan
+
+    # training step of the headline configuration: forward on the fused kernels, gradients of q, k, v
+    # on the two passes of the backward band kernel
+    B, H, L, E, mh, lc = 2, 1, 3136, 64, 64, 512
+    q, k, v = (torch.randn(B, L, H, E, generator=g).to(dev) * E ** -0.25 for _ in range(3))
+    P = fly_amd.gaussian_orthogonal_random_matrix(mh, E).to(dev)
+    out['config1_sblocal_fp32_fwd_bwd_ms'] = timeit(sblocal_train_step(q, k, v, P, lc, None), n=10)
+    del q, k, v
 
     cfg = fly_amd.FlatBlockButterflySparsityConfig(8, 2, block=32)
     torch.manual_seed(0)
