@@ -1272,6 +1272,7 @@ struct LocalArgs {
     int B, H, T, S, lc;
     long q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss;
     float temp;
+    float* lse;                     // optional (B, H, T): log of the softmax denominator, for the backward pass
 };
 
 template <typename T, int E, int D>
@@ -1398,6 +1399,8 @@ __global__ __launch_bounds__(NT) void local_fwd_kernel(LocalArgs a) {
         T* optr = reinterpret_cast<T*>(a.out) + b * a.o_sb + h * a.o_sh + (long)iq * a.o_ss;
 #pragma unroll
         for (int db = 0; db < DB; ++db) store4_f32(optr + 16 * db + 4 * g, oacc[db] * inv);
+        if (a.lse && g == 0)        // a query without visible keys has no pair that would read its entry
+            a.lse[((long)b * a.H + h) * a.T + iq] = ze > 0.f ? m_run * 0.6931471805599453f + __logf(ze) : 0.f;
     }
 }
 
@@ -2458,7 +2461,8 @@ extern "C" int flyhip_sblocal_fwd(const void* q, const void* k, const void* v, c
     return dispatch_fwd(dtype, E, 2 * mh, a, reinterpret_cast<hipStream_t>(stream));
 }
 
-extern "C" int flyhip_local_fwd(const void* q, const void* k, const void* v, const int64_t* key_lengths, void* out,
+extern "C" int flyhip_local_fwd_lse(const void* q, const void* k, const void* v, const int64_t* key_lengths, void* out,
+                                    float* lse,
                                 int B, int H, int T, int S, int E, int D, int local_context,
                                 int64_t q_sb, int64_t q_sh, int64_t q_ss,
                                 int64_t k_sb, int64_t k_sh, int64_t k_ss,
@@ -2473,7 +2477,7 @@ extern "C" int flyhip_local_fwd(const void* q, const void* k, const void* v, con
     FLY_REQUIRE(((q_sb | q_sh | q_ss | k_sb | k_sh | k_ss | v_sb | v_sh | v_ss | o_sb | o_sh | o_ss) % 4) == 0,
                 "local_fwd: strides must be multiples of 4 elements (16-byte vector access)");
     LocalArgs a{q, k, v, key_lengths, out, B, H, T, S, local_context,
-                q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss, softmax_temp};
+                q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss, softmax_temp, lse};
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
 #define LOCAL_DISPATCH(TT)                                                                          \
     switch (E) {                                                                                    \
@@ -2486,6 +2490,18 @@ extern "C" int flyhip_local_fwd(const void* q, const void* k, const void* v, con
     if (dtype == BF16) { LOCAL_DISPATCH(bf16_t) }
 #undef LOCAL_DISPATCH
     return fail(ERR_UNSUPPORTED, "local_fwd supports float32 and bfloat16, got dtype code %d", dtype);
+}
+
+extern "C" int flyhip_local_fwd(const void* q, const void* k, const void* v, const int64_t* key_lengths, void* out,
+                                int B, int H, int T, int S, int E, int D, int local_context,
+                                int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                                int64_t k_sb, int64_t k_sh, int64_t k_ss,
+                                int64_t v_sb, int64_t v_sh, int64_t v_ss,
+                                int64_t o_sb, int64_t o_sh, int64_t o_ss,
+                                float softmax_temp, int dtype, void* stream) {
+    return flyhip_local_fwd_lse(q, k, v, key_lengths, out, nullptr, B, H, T, S, E, D, local_context,
+                                q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss,
+                                softmax_temp, dtype, stream);
 }
 
 static int dispatch_bwd_band(const BwdArgs& a, int E, int M, int key_major, void* stream);

@@ -8,13 +8,14 @@ import torch.nn.functional as F
 
 from . import _lib
 from .sblocal_attention import _HEAD_DIMS, _round_up_choice, _vector_ready
-from .sblocal_backward import BandWindows
+from .sblocal_backward import BandWindows, _band_kernel_dims, _band_terms_hip
 
 
-def local_forward(query, key, value, local_context, softmax_temp=None, key_lengths=None):
+def local_forward(query, key, value, local_context, softmax_temp=None, key_lengths=None, return_lse=False):
     """query (B,T,H,E), key (B,S,H,E), value (B,S,H,D) float32 or bfloat16 GPU tensors ->
     out (B,T,H,D): query i attends to keys j with -(local_context // 2) <= j - i < (local_context + 1) // 2
-    and j < key_lengths[b] (local_attention.py:68-92 for attn_mask=None, no dropout)."""
+    and j < key_lengths[b] (local_attention.py:68-92 for attn_mask=None, no dropout).  With return_lse
+    also the log of every query's softmax denominator, (B,H,T) float32 (0 for a query without keys)."""
     _lib.require_gpu(query, key, value, key_lengths)
     if query.dtype not in (torch.float32, torch.bfloat16):
         raise NotImplementedError(f'the local attention kernel supports float32 and bfloat16, got {query.dtype}')
@@ -41,24 +42,29 @@ def local_forward(query, key, value, local_context, softmax_temp=None, key_lengt
         if lens.shape != (B,):
             raise ValueError(f'key_lengths must have shape ({B},)')
     out = torch.empty(B, T, H, dim, dtype=query.dtype, device=query.device)
+    lse = torch.empty(B, H, T, dtype=torch.float32, device=query.device) if return_lse else None
     with torch.cuda.device(query.device):
-        _lib.call('flyhip_local_fwd', q.data_ptr(), k.data_ptr(), v.data_ptr(), _lib.ptr(lens), out.data_ptr(),
-                  B, H, T, S, dim, dim, local_context,
+        _lib.call('flyhip_local_fwd_lse', q.data_ptr(), k.data_ptr(), v.data_ptr(), _lib.ptr(lens), out.data_ptr(),
+                  _lib.ptr(lse), B, H, T, S, dim, dim, local_context,
                   q.stride(0), q.stride(2), q.stride(1), k.stride(0), k.stride(2), k.stride(1),
                   v.stride(0), v.stride(2), v.stride(1), out.stride(0), out.stride(2), out.stride(1),
                   t, _lib.dtype_code(q), _lib.stream_ptr(query.device))
-    return out[..., :D]
+    return (out[..., :D], lse) if return_lse else out[..., :D]
 
 
 def local_backward(query, key, value, local_context, softmax_temp, key_lengths, grad_out, chunk=256,
-                   max_elements=1 << 27):
+                   max_elements=1 << 27, out=None, lse=None):
     """Gradients of local attention with respect to query, key and value (the reference takes them from
     autograd through fast_transformers.local_product, local_attention.py:68-92).  The band softmax is
     evaluated again for all chunks of queries at once against the windows of keys their bands touch
     (sblocal_backward.BandWindows); with
     P = softmax over the band, g = d out and delta_i = sum_s P_is g_i.v_s:
     d v_s = sum_i P_is g_i,  d(t q_i.k_s) = P_is (g_i.v_s - delta_i).  Queries without any visible
-    key get zero gradients.  Ordinary tensor algebra on whatever device the tensors live on."""
+    key get zero gradients.  Given the forward's out and lse (local_forward(..., return_lse=True)), float32
+    or bfloat16 GPU tensors and head dims <= 64, the sums run on the backward band kernel of
+    Scatterbrain-local attention with its feature operands zero (flyhip_sblocal_bwd_band: P_is =
+    exp(t q_i.k_s - lse_i), delta_i = g_i.out_i); otherwise as ordinary tensor algebra on whatever device
+    the tensors live on."""
     B, T, H, E = query.shape
     S, D = key.shape[1], value.shape[3]
     t = softmax_temp or 1 / math.sqrt(E)
@@ -67,6 +73,17 @@ def local_backward(query, key, value, local_context, softmax_temp, key_lengths, 
     def bh(x):                                   # (B,L,H,C) -> (B*H, L, C)
         return x.permute(0, 2, 1, 3).reshape(B * H, x.shape[1], x.shape[3]).to(wdt)
     Q, K, V, G = bh(query), bh(key), bh(value), bh(grad_out)
+
+    def back(x, like):                           # (B*H, L, C) -> (B,L,H,C)
+        return x.reshape(B, H, x.shape[1], x.shape[2]).permute(0, 2, 1, 3).to(like.dtype)
+    dims = _band_kernel_dims(E, D, 0)
+    if out is not None and lse is not None and Q.is_cuda and wdt == torch.float32 and dims is not None:
+        zq, zk = Q.new_zeros(B * H, T, dims[1]), Q.new_zeros(B * H, S, dims[1])
+        delta = (G * bh(out)).sum(-1, keepdim=True)
+        lens_b = None if key_lengths is None else key_lengths.to(device=Q.device, dtype=torch.int64).contiguous()
+        dQ, _, dK, _, dV = _band_terms_hip(Q, K, V, G, zq, zk, lse.reshape(B * H, T, 1), delta, lens_b, H,
+                                           local_context, t, dims)
+        return back(dQ, query), back(dK, key), back(dV, value)
     lens = None
     if key_lengths is not None:
         lens = key_lengths.to(Q.device).repeat_interleave(H).view(B * H, 1, 1)
@@ -86,9 +103,6 @@ def local_backward(query, key, value, local_context, softmax_temp, key_lengths, 
         band.add_windows(acc_k, j0, t * (ds.transpose(2, 3) @ Qc[:, sl]))
         band.add_windows(acc_v, j0, p.transpose(2, 3) @ Gc[:, sl])
     dQ, dK, dV = band.unchunk(dQc), band.fold(acc_k), band.fold(acc_v)
-
-    def back(x, like):                           # (B*H, L, C) -> (B,L,H,C)
-        return x.reshape(B, H, x.shape[1], x.shape[2]).permute(0, 2, 1, 3).to(like.dtype)
     return back(dQ, query), back(dK, key), back(dV, value)
 
 
@@ -97,15 +111,17 @@ class _LocalFn(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, query, key, value, local_context, softmax_temp, key_lengths):
-        out = local_forward(query, key, value, local_context, softmax_temp=softmax_temp, key_lengths=key_lengths)
-        ctx.save_for_backward(query, key, value, key_lengths)
+        out, lse = local_forward(query, key, value, local_context, softmax_temp=softmax_temp, key_lengths=key_lengths,
+                                 return_lse=True)
+        ctx.save_for_backward(query, key, value, key_lengths, out, lse)
         ctx.local_context, ctx.softmax_temp = local_context, softmax_temp
         return out
 
     @staticmethod
     def backward(ctx, grad_out):
-        query, key, value, key_lengths = ctx.saved_tensors
-        dq, dk, dv = local_backward(query, key, value, ctx.local_context, ctx.softmax_temp, key_lengths, grad_out)
+        query, key, value, key_lengths, out, lse = ctx.saved_tensors
+        dq, dk, dv = local_backward(query, key, value, ctx.local_context, ctx.softmax_temp, key_lengths, grad_out,
+                                    out=out, lse=lse)
         return dq, dk, dv, None, None, None
 
 

@@ -144,6 +144,19 @@ int flyhip_local_fwd(const void* q, const void* k, const void* v, const int64_t*
                      int64_t o_sb, int64_t o_sh, int64_t o_ss,
                      float softmax_temp, int dtype, void* stream);
 
+/* flyhip_local_fwd that also writes, when lse is not NULL, the log of every query's softmax
+ * denominator (B,H,T) float32 -- what the backward pass needs to evaluate the weights again (the
+ * reference keeps the whole (B,H,T,local_context) weight tensor for autograd, local_attention.py:75-91);
+ * 0 for a query without keys. */
+int flyhip_local_fwd_lse(const void* q, const void* k, const void* v, const int64_t* key_lengths, void* out,
+                         float* lse,
+                         int B, int H, int T, int S, int E, int D, int local_context,
+                         int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                         int64_t k_sb, int64_t k_sh, int64_t k_ss,
+                         int64_t v_sb, int64_t v_sh, int64_t v_ss,
+                         int64_t o_sb, int64_t o_sh, int64_t o_ss,
+                         float softmax_temp, int dtype, void* stream);
+
 /* Measurement hook (no counterpart in the reference): the two caller-owned hipEvent_t are recorded
  * on the launch stream immediately before and after the fused band kernel of the NEXT
  * flyhip_sblocal_fwd call of the calling thread, then forgotten.  Pass NULLs to clear. */
