@@ -815,8 +815,17 @@ __global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
     __shared__ __attribute__((aligned(16))) uint16_t ws[2][128 * LD];
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
     const int wm = w >> 1, wn = w & 1;                      // this wave: tokens 64wm.., outputs 64wn..
-    const int grp = blockIdx.x, z = blockIdx.z;
-    const long m0 = (long)blockIdx.y * 128;
+    const int z = blockIdx.z;
+    // Workgroups go to the 8 XCDs (each with its own L2) round-robin in launch order.  The launch
+    // index is re-mapped so that the groups working on one stream of token tiles -- they read the same
+    // activations -- run on one XCD, one after the other: stream = 8 * (slot / groups) + XCD.
+    const int lin = blockIdx.x + gridDim.x * blockIdx.y, slot = lin >> 3;
+    const int grp = slot % (int)gridDim.x, ty = 8 * (slot / (int)gridDim.x) + (lin & 7), gy = gridDim.y;   // gridDim.y is a multiple of 8
+    // token tiles ty, ty + gy, ... : the group's tables are read once and the load -> LDS -> MFMA
+    // pipeline runs on across tile boundaries
+    const int tiles_all = (a.M + 127) / 128;
+    if (ty >= tiles_all) return;                            // workgroup-uniform
+    const int my_tiles = (tiles_all - ty + gy - 1) / gy;
     const int row0 = a.grp_row0[grp], gn = a.grp_n[grp];    // first output block-row (segment) and count
     const int head = row0 / a.per_head, bcol0 = row0 % a.per_head;
     const int p0 = a.seg_ptr[row0], nin = a.seg_ptr[row0 + 1] - p0;
@@ -837,7 +846,8 @@ __global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
     // staging roles: thread -> (row = tid/4 [+64], 16-byte chunk = tid%4) of the x and W tiles of one
     // input block; a step moves KB input blocks
     const int srow = tid >> 2, schunk = (tid & 3) * 8;
-    const int n_steps = (nin + KB - 1) / KB;
+    static_assert(KB == 1, "the tile cursors below advance one input block per step");
+    const int n_steps = my_tiles * nin;
     // two register sets: the loads of step s+2 are issued while step s computes and are parked in LDS
     // one iteration later, so every global load has two steps to arrive
     // (native vectors: arrays of the uint4 struct passed by reference do not stay in registers)
@@ -846,43 +856,57 @@ __global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
     // compiler count how many newer loads may stay in flight when it waits for the older set.
     uintx4 rxa[KB][2], rwa[KB][2], rxb[KB][2], rwb[KB][2];
     bool wla[KB][2], wlb[KB][2];                            // weight block present?
-    auto fetch = [&](int step, uintx4 (&rx)[KB][2], uintx4 (&rw)[KB][2], bool (&wl)[KB][2]) __attribute__((always_inline)) {
-#pragma unroll
-        for (int kb = 0; kb < KB; ++kb) {
-            const int t = step * KB + kb;
-            const bool live = t < nin;                       // a missing block contributes zero weights
-            const int tc = live ? t : nin - 1;
-            const long kcol = (long)s_inner[tc] * 32 + schunk;
+    int f_tile = 0, f_t = 0;                                // fetch cursor: (token tile, step inside it)
+    // A load is "wave-uniform base + per-thread byte offset": the input block and the weight block of a
+    // step are the same for the whole wave (a wave stages rows of one output block: (tid / 4) / 32 = w / 2),
+    // so they come out of LDS once through the first lane and the bases are formed on the scalar unit;
+    // the per-thread offsets change only with the token tile.
+    const int obw = w >> 1;                                 // output block (of the group's four) of this wave's rows, +2 for the upper half
+    const uint32_t woff = (uint32_t)(((srow & 31) * 32 + schunk) * 2);
+    uint32_t xoff[2] = {0, 0};
+    auto fetch = [&](uintx4 (&rx)[KB][2], uintx4 (&rw)[KB][2], bool (&wl)[KB][2]) __attribute__((always_inline)) {
+        const bool live = f_tile < my_tiles;                 // past the end: re-read the last step, zero weights
+        const int tc = live ? f_t : nin - 1;
+        if (f_t == 0) {
+            const long m0 = ((long)ty + (long)min(f_tile, my_tiles - 1) * gy) * 128;
 #pragma unroll
             for (int hh = 0; hh < 2; ++hh) {
-                const long m = min(m0 + srow + 64 * hh, (long)a.M - 1);        // clamped: masked at the store
-                rx[kb][hh] = *reinterpret_cast<const uintx4*>(xp + m * a.dn_sm + kcol);
-                const int orow = srow + 64 * hh;                                 // output row inside the group
-                const int blk_id = s_blk[orow >> 5][tc];
-                wl[kb][hh] = live && blk_id >= 0;
-                rw[kb][hh] = *reinterpret_cast<const uintx4*>(spz + (long)max(blk_id, 0) * 1024 + (orow & 31) * 32 + schunk);
+                const long m = min(m0 + srow + 64 * hh, (long)a.M - 1);          // clamped: masked at the store
+                xoff[hh] = (uint32_t)((m * a.dn_sm + schunk) * 2);
             }
         }
+        const int inner = __builtin_amdgcn_readfirstlane(s_inner[tc]);
+        const char* xb = reinterpret_cast<const char*>(xp + (long)inner * 32);
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+            rx[0][hh] = *reinterpret_cast<const uintx4*>(xb + xoff[hh]);
+            const int blk_id = __builtin_amdgcn_readfirstlane(s_blk[obw + 2 * hh][tc]);
+            wl[0][hh] = live && blk_id >= 0;                 // a missing block contributes zero weights
+            rw[0][hh] = *reinterpret_cast<const uintx4*>(reinterpret_cast<const char*>(spz + (long)max(blk_id, 0) * 1024) + woff);
+        }
+        if (++f_t == nin) { f_t = 0; ++f_tile; }
     };
+    // The weight tile sits in LDS in the order the MFMAs read it: row 64*(n/64) + 16*i + r holds output
+    // n = 64*(n/64) + 32*(i/2) + 8*(r/4) + 4*(i%2) + r%4, so that a wave's fragment read walks 16
+    // consecutive LDS rows (rows 16 apart share their banks at this row stride).
+    auto wrow = [](int n) { const int b = n & 31; return (n & 64) + 16 * (2 * ((n >> 5) & 1) + ((b >> 2) & 1)) + 4 * (b >> 3) + (b & 3); };
+    const int wrow0 = wrow(srow);
     auto stash = [&](int buf, const uintx4 (&rx)[KB][2], const uintx4 (&rw)[KB][2], const bool (&wl)[KB][2]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int kb = 0; kb < KB; ++kb)
+        for (int hh = 0; hh < 2; ++hh) {
+            *reinterpret_cast<uintx4*>(&xs[buf][(srow + 64 * hh) * LD + schunk]) = rx[0][hh];
+            const uintx4 wv = wl[0][hh] ? rw[0][hh] : uintx4{0, 0, 0, 0};
+            if (!WT) {
+                *reinterpret_cast<uintx4*>(&ws[buf][(wrow0 + 64 * hh) * LD + schunk]) = wv;
+            } else {
+                // the thread holds row k = orow % 32 of the block, columns n = schunk .. schunk + 7: the
+                // LDS tile is [n][k] either way, so these eight go out one by one
+                const int orow = srow + 64 * hh;
 #pragma unroll
-            for (int hh = 0; hh < 2; ++hh) {
-                *reinterpret_cast<uintx4*>(&xs[buf][(srow + 64 * hh) * LD + 32 * kb + schunk]) = rx[kb][hh];
-                const uintx4 wv = wl[kb][hh] ? rw[kb][hh] : uintx4{0, 0, 0, 0};
-                if (!WT) {
-                    *reinterpret_cast<uintx4*>(&ws[buf][(srow + 64 * hh) * LD + 32 * kb + schunk]) = wv;
-                } else {
-                    // the thread holds row k = orow % 32 of the block, columns n = schunk .. schunk + 7: the
-                    // LDS tile is [n][k] either way, so these eight go out one by one
-                    const int orow = srow + 64 * hh;
-#pragma unroll
-                    for (int e = 0; e < 8; ++e)
-                        ws[buf][(32 * (orow >> 5) + schunk + e) * LD + 32 * kb + (orow & 31)] =
-                            (uint16_t)(wv[e >> 1] >> (16 * (e & 1)));
-                }
+                for (int e = 0; e < 8; ++e)
+                    ws[buf][wrow(32 * (orow >> 5) + schunk + e) * LD + (orow & 31)] = (uint16_t)(wv[e >> 1] >> (16 * (e & 1)));
             }
+        }
     };
 
     floatx4 acc[4][4];
@@ -892,6 +916,24 @@ __global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
         for (int tn = 0; tn < 4; ++tn) acc[tm][tn] = Frag<float>::zero();
     const bool wave_active = 2 * wn < gn;                   // its output blocks exist in this group
 
+    T* cp = reinterpret_cast<T*>(a.c) + z * a.c_sz + head * a.c_sh;
+    // lane holds y[m = 64wm + 16tm + r16][n = 32*(output block) + 8g + 4*(tn%2) + i]: 16-byte stores
+    auto store_tile = [&](int tile) __attribute__((always_inline)) {
+        const long m0 = ((long)ty + (long)tile * gy) * 128;
+#pragma unroll
+        for (int tm = 0; tm < 4; ++tm) {
+            const long m = m0 + 64 * wm + 16 * tm + r16;
+#pragma unroll
+            for (int o2 = 0; o2 < 2; ++o2) {
+                const int ob = 2 * wn + o2;
+                if (m < a.M && ob < gn)
+                    store8_f32(cp + m * a.c_sm + (long)(bcol0 + ob) * 32 + 8 * g, acc[tm][2 * o2], acc[tm][2 * o2 + 1]);
+            }
+#pragma unroll
+            for (int tn = 0; tn < 4; ++tn) acc[tm][tn] = Frag<float>::zero();
+        }
+    };
+    int c_tile = 0, c_t = 0;                                // compute cursor
     auto compute = [&](int cur) __attribute__((always_inline)) {
         if (wave_active) {
 #pragma unroll
@@ -901,47 +943,39 @@ __global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
                 for (int i = 0; i < 4; ++i) {
                     fx[i] = *reinterpret_cast<const uint4*>(&xs[cur][(64 * wm + 16 * i + r16) * LD + 32 * kb + 8 * g]);
                     // W-tile i covers output block i/2; its MFMA row r is block row 8*(r/4) + 4*(i%2) + r%4
-                    fw[i] = *reinterpret_cast<const uint4*>(
-                        &ws[cur][(64 * wn + 32 * (i >> 1) + 8 * (r16 >> 2) + 4 * (i & 1) + (r16 & 3)) * LD + 32 * kb + 8 * g]);
+                    fw[i] = *reinterpret_cast<const uint4*>(&ws[cur][(64 * wn + 16 * i + r16) * LD + 32 * kb + 8 * g]);
                 }
 #pragma unroll
                 for (int tm = 0; tm < 4; ++tm)
 #pragma unroll
                     for (int tn = 0; tn < 4; ++tn) acc[tm][tn] = Frag32<T>::mma(fw[tn], fx[tm], acc[tm][tn]);
             }
+            if (++c_t == nin) { store_tile(c_tile); c_t = 0; ++c_tile; }     // the tile's last input block
         }
     };
-    if (n_steps > 0) { fetch(0, rxa, rwa, wla); stash(0, rxa, rwa, wla); }
-    if (n_steps > 0) fetch(1, rxb, rwb, wlb);              // set B holds odd steps, set A even steps
+    if (nin == 0) {                                         // no input block: zero rows
+        if (wave_active)
+            for (int tile = 0; tile < my_tiles; ++tile) store_tile(tile);
+        return;
+    }
+    fetch(rxa, rwa, wla);
+    stash(0, rxa, rwa, wla);
+    fetch(rxb, rwb, wlb);                                   // set B holds odd steps, set A even steps
     drain_loads_but<4 * KB>();                              // only set B (4 KB loads a thread) is in flight
     __syncthreads();
     for (int step = 0; step < n_steps; step += 2) {
-        fetch(step + 2, rxa, rwa, wla);
+        fetch(rxa, rwa, wla);
         compute(0);
         stash(1, rxb, rwb, wlb);
         drain_loads_but<4 * KB>();                          // set B is parked: only set A is in flight
         __syncthreads();
         // (no early exit between the halves: the compiler would count a path that leaves here, with
         // set A in flight, as a way back to the top of the loop, and drain before every refill)
-        fetch(step + 3, rxb, rwb, wlb);
+        fetch(rxb, rwb, wlb);
         if (step + 1 < n_steps) compute(1);
         stash(0, rxa, rwa, wla);
         drain_loads_but<4 * KB>();
         __syncthreads();
-    }
-    // lane holds y[m = 64wm + 16tm + r16][n = 32*(output block) + 8g + 4*(tn%2) + i]: 16-byte stores
-    if (!wave_active) return;
-    T* cp = reinterpret_cast<T*>(a.c) + z * a.c_sz + head * a.c_sh;
-#pragma unroll
-    for (int tm = 0; tm < 4; ++tm) {
-        const long m = m0 + 64 * wm + 16 * tm + r16;
-        if (m >= a.M) continue;
-#pragma unroll
-        for (int o2 = 0; o2 < 2; ++o2) {
-            const int ob = 2 * wn + o2;
-            if (ob >= gn) continue;
-            store8_f32(cp + m * a.c_sm + (long)(bcol0 + ob) * 32 + 8 * g, acc[tm][2 * o2], acc[tm][2 * o2 + 1]);
-        }
     }
 }
 
@@ -1742,11 +1776,16 @@ extern "C" int flyhip_bs_dds(const void* a, const void* b_sp, void* c,
     FLY_REQUIRE(b_sz % 4 == 0, "bs_dds: sparse batch stride must be a multiple of 4 elements");
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     if (grp_row0 && grp_n && n_grp > 0 && max_seg_len >= 0 && max_seg_len <= DDS_MAX_STEPS && blk == 32 &&
-        (dtype == BF16 || dtype == F16) && a_sk == 1 &&
+        (dtype == BF16 || dtype == F16) && a_sk == 1 && (long)M * a_sm * 2 < (1L << 32) &&
         c_sn == 1 && ((a_sz | a_sh | a_sm | b_sz | c_sz | c_sh | c_sm) % 8) == 0 && (M + 127) / 128 <= 65535) {
         DdsGroupArgs ga{b_sp, a, c, seg_ptr, seg_blk, seg_inner, grp_row0, grp_n, cols_per_head, M,
                         b_sz, a_sz, a_sh, a_sm, c_sz, c_sh, c_sm};
-        dim3 grid(n_grp, (M + 127) / 128, Z);
+        // as many workgroups as are resident together (three fit a CU); each walks its share of the token tiles
+        const long tiles = (M + 127) / 128;
+        long gy = (3L * 256 + (long)n_grp * Z - 1) / ((long)n_grp * Z);
+        if (gy > tiles) gy = tiles;
+        gy = (gy + 7) / 8 * 8;                               // the kernel deals streams of token tiles to the 8 XCDs
+        dim3 grid(n_grp, (unsigned)gy, Z);
         if (dtype == BF16) {
             if (trans_b) hipLaunchKernelGGL((bs_dds32_kernel<bf16_t, false>), grid, dim3(256), 0, st, ga);
             else hipLaunchKernelGGL((bs_dds32_kernel<bf16_t, true>), grid, dim3(256), 0, st, ga);

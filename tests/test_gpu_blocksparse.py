@@ -418,6 +418,29 @@ def test_fast_dds_both_block_orientations(trans_b, dtype):
     assert rel_err(out, ref) <= TOL[dtype]
 
 
+@pytest.mark.parametrize('trans_b', [True, False])
+def test_fast_dds_many_token_tiles_per_workgroup(trans_b):
+    """The tiled dds kernel walks several 128-token tiles per workgroup once there are more tiles than
+    workgroups wanted: enough tokens for two to three tiles each, a ragged last tile, an empty
+    block-row (no input block at all) among the outputs."""
+    from fly_amd import matmul
+    print('case', trans_b, flush=True)
+    Z, H, block, p, r, M = 1, 1, 32, 4, 3, 128 * 2500 + 37
+    layout = torch.tensor([[[1, 0, 1], [1, 0, 1], [0, 1, 1], [1, 1, 0]]])
+    if trans_b:
+        layout[0, 1] = 0
+    else:
+        layout[0, :, 1] = 0
+    g = torch.Generator().manual_seed(10)
+    nnz = int(layout.sum())
+    w = torch.randn(Z, nnz, block, block, generator=g).bfloat16()
+    x = torch.randn(Z, H, M, (r if trans_b else p) * block, generator=g).bfloat16()
+    out = matmul(layout, block, 'dds', trans_a=False, trans_b=trans_b)(x.to(DEV), w.to(DEV))
+    ref = ob.dds(x.float(), w.float(), layout, block, False, trans_b)
+    assert out.shape == ref.shape
+    assert rel_err(out, ref) <= TOL[torch.bfloat16]
+
+
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize('p,r,N', [(8, 8, 64), (11, 6, 72), (5, 13, 128)])
 def test_dsd_with_transposed_sparse_operand(p, r, N, dtype):
