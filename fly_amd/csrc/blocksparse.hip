@@ -810,9 +810,14 @@ constexpr int DDS_MAX_STEPS = 128;   // longest reduction list the tiled kernel 
 template <typename T, bool WT>     // WT: blocks are [k][n] (y = x W) and are transposed on their way into LDS
 __global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
     constexpr int KB = 1;                                   // input blocks per pipeline step
-    constexpr int LD = 32 * KB + 8;                         // LDS row stride in elements
+    // LDS tiles are [row][32 k] with 64-byte rows and no padding; the four 16-byte chunks of a row are
+    // stored at chunk ^ swz(row), swz(r) = ((r >> 1) & 3) ^ ((r >> 3) & 1).  Then both the 16-byte
+    // fragment reads (16 consecutive rows, one chunk) and the staging writes (4 rows x 4 chunks per 16
+    // lanes) spread evenly over the banks, whether 8 or 16 lanes are served per clock.
+    constexpr int LD = 32;
     __shared__ __attribute__((aligned(16))) uint16_t xs[2][128 * LD];
     __shared__ __attribute__((aligned(16))) uint16_t ws[2][128 * LD];
+    auto swz = [](int r) { return ((r >> 1) & 3) ^ ((r >> 3) & 1); };
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
     const int wm = w >> 1, wn = w & 1;                      // this wave: tokens 64wm.., outputs 64wn..
     const int z = blockIdx.z;
@@ -891,20 +896,24 @@ __global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
     // consecutive LDS rows (rows 16 apart share their banks at this row stride).
     auto wrow = [](int n) { const int b = n & 31; return (n & 64) + 16 * (2 * ((n >> 5) & 1) + ((b >> 2) & 1)) + 4 * (b >> 3) + (b & 3); };
     const int wrow0 = wrow(srow);
+    const int xs_off = srow * LD + 8 * ((tid & 3) ^ swz(srow));        // + 64 rows for the upper half (same swizzle)
+    const int ws_off = wrow0 * LD + 8 * ((tid & 3) ^ swz(wrow0));
     auto stash = [&](int buf, const uintx4 (&rx)[KB][2], const uintx4 (&rw)[KB][2], const bool (&wl)[KB][2]) __attribute__((always_inline)) {
 #pragma unroll
         for (int hh = 0; hh < 2; ++hh) {
-            *reinterpret_cast<uintx4*>(&xs[buf][(srow + 64 * hh) * LD + schunk]) = rx[0][hh];
+            *reinterpret_cast<uintx4*>(&xs[buf][xs_off + 64 * hh * LD]) = rx[0][hh];
             const uintx4 wv = wl[0][hh] ? rw[0][hh] : uintx4{0, 0, 0, 0};
             if (!WT) {
-                *reinterpret_cast<uintx4*>(&ws[buf][(wrow0 + 64 * hh) * LD + schunk]) = wv;
+                *reinterpret_cast<uintx4*>(&ws[buf][ws_off + 64 * hh * LD]) = wv;
             } else {
                 // the thread holds row k = orow % 32 of the block, columns n = schunk .. schunk + 7: the
                 // LDS tile is [n][k] either way, so these eight go out one by one
-                const int orow = srow + 64 * hh;
+                const int orow = srow + 64 * hh, k = orow & 31;
 #pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    ws[buf][wrow(32 * (orow >> 5) + schunk + e) * LD + (orow & 31)] = (uint16_t)(wv[e >> 1] >> (16 * (e & 1)));
+                for (int e = 0; e < 8; ++e) {
+                    const int n = wrow(32 * (orow >> 5) + schunk + e);
+                    ws[buf][n * LD + 8 * ((k >> 3) ^ swz(n)) + (k & 7)] = (uint16_t)(wv[e >> 1] >> (16 * (e & 1)));
+                }
             }
         }
     };
@@ -934,6 +943,7 @@ __global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
         }
     };
     int c_tile = 0, c_t = 0;                                // compute cursor
+    const int frag_off = r16 * LD + 8 * (g ^ swz(r16));     // this lane's 16 bytes inside a 16-row fragment
     auto compute = [&](int cur) __attribute__((always_inline)) {
         if (wave_active) {
 #pragma unroll
@@ -941,9 +951,9 @@ __global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
                 uint4 fx[4], fw[4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    fx[i] = *reinterpret_cast<const uint4*>(&xs[cur][(64 * wm + 16 * i + r16) * LD + 32 * kb + 8 * g]);
+                    fx[i] = *reinterpret_cast<const uint4*>(&xs[cur][(64 * wm + 16 * i) * LD + frag_off]);
                     // W-tile i covers output block i/2; its MFMA row r is block row 8*(r/4) + 4*(i%2) + r%4
-                    fw[i] = *reinterpret_cast<const uint4*>(&ws[cur][(64 * wn + 16 * i + r16) * LD + 32 * kb + 8 * g]);
+                    fw[i] = *reinterpret_cast<const uint4*>(&ws[cur][(64 * wn + 16 * i) * LD + frag_off]);
                 }
 #pragma unroll
                 for (int tm = 0; tm < 4; ++tm)
