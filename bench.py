@@ -188,6 +188,27 @@ def bench_blocksparse(steps, warmup):
         qg.grad = kg.grad = vg.grad = None
     out['three_stage_attention_fwd_bwd_ms'] = timeit(train_step)
     del qg, kg, vg, go
+
+    # the same training step through BlockSparseAttention: forward on the one-kernel attention (it keeps
+    # a log-denominator per row), backward = probabilities again, dV, fused score gradient, dQ, dK
+    from fly_amd import BlockSparseAttention
+
+    class Layout:
+        def __init__(self):
+            self.block = block
+
+        def make_layout(self, seqlen):
+            return layout
+    mod = BlockSparseAttention(Layout(), attention_dropout=0.0, max_seq_length=L).to(dev)
+    qm, km, vm = (t.detach().transpose(1, 2).contiguous().requires_grad_() for t in (q, k, v))      # (B, L, H, d)
+    gm = torch.randn(B, L, H, d, generator=g).bfloat16().to(dev)
+
+    def module_step():
+        o, _ = mod(qm, km, vm)
+        o.backward(gm)
+        qm.grad = km.grad = vm.grad = None
+    out['module_fwd_bwd_ms'] = timeit(module_step)
+    del qm, km, vm, gm, mod
     out['fused_attention'] = {'ms': ms, 'tflops': 2 * flops / ms / 1e9, 'mfma_bf16_frac': 2 * flops / ms / 1e9 / 2500.0,
                               'speedup_over_three_stages': ms3 / ms,
                               'max_diff_vs_three_stages': float((got - ref).abs().max() / ref.abs().max())}

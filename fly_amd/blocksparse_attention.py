@@ -17,35 +17,61 @@ from .padding import pad_to_multiple
 
 
 class _AttentionCoreFn(torch.autograd.Function):
-    """softmax(scale * q k^T + masks) v on the nonzero blocks, for calls that need gradients: the forward is
-    the reference's three ops (blocksparse_attention.py:134-160; the probabilities are kept for the
-    backward), the backward runs four kernels instead of the op-by-op chain's six plus elementwise passes:
+    """softmax(scale * q k^T + masks) v on the nonzero blocks, for calls that need gradients.  With masks
+    the forward is the reference's three ops (blocksparse_attention.py:134-160; the probabilities are
+    kept for the backward); without, the one-kernel attention, which keeps one log-denominator per row,
+    and the backward forms the probabilities again.  The backward runs four kernels instead of the
+    op-by-op chain's six plus elementwise passes:
     dV = P^T dO, dS = scale * P * (dO V^T - rowsum(dO * O)) in one kernel (the sdd fused with the softmax
     gradient), dQ = dS K, dK = dS^T Q.  32x32 blocks of bf16 / fp16 with shared-tile tables only."""
 
     @staticmethod
-    def forward(ctx, q, k, v, sdd, dsd, sm, scale, kpm, am):
+    def forward(ctx, q, k, v, sdd, dsd, sm, scale, kpm, am, fused):
+        ctx.ops, ctx.scale = (sdd, dsd), scale
+        if fused is not None and kpm is None and am is None:
+            # no masks: the one-kernel forward; it keeps the rows' log-denominators instead of the
+            # probabilities, which the backward forms again (one sdd with an exponential epilogue)
+            out, lse2 = fused(q, k, v, scale, None, return_lse=True)
+            ctx.save_for_backward(q, k, v, out, lse2)
+            ctx.recompute = True
+            return out
         p = sm(sdd._run('sdd', q, k, False, True, False), scale=scale, key_padding_mask=kpm, attn_mask=am,
                key_padding_mask_mode='add', attn_mask_mode='add')
         if kpm is not None or am is not None:
             p.nan_to_num_()
         out = dsd._run('dsd', p, v, False, False, False)
         ctx.save_for_backward(q, k, v, p, out)
-        ctx.ops, ctx.scale = (sdd, dsd), scale
+        ctx.recompute = False
         return out
 
     @staticmethod
     def backward(ctx, dout):
         from . import _lib
-        q, k, v, p, out = ctx.saved_tensors
         sdd, dsd = ctx.ops
+        H, rows, cols = sdd.spdims
+        uni_ptr, uni_inner, uni_blk = sdd._table('union', dout.device)
+
+        def vec(x):          # 16-byte loads: last dim contiguous, other strides multiples of 8
+            ok = x.stride(3) == 1 and all(s_ % 8 == 0 for s_ in x.stride()[:3]) and x.data_ptr() % 16 == 0
+            return x if ok else x.contiguous()
+        if ctx.recompute:
+            q, k, v, out, lse2 = ctx.saved_tensors
+            nnz = int(sdd.layout.sum())
+            p = torch.empty((q.shape[0], nnz, 32, 32), dtype=q.dtype, device=q.device)
+            qq, kk = vec(q), vec(k)
+            with torch.cuda.device(q.device):
+                _lib.call('flyhip_bs_sdd_prob', qq.data_ptr(), kk.data_ptr(), lse2.data_ptr(), p.data_ptr(),
+                          uni_ptr.data_ptr(), uni_inner.data_ptr(), uni_blk.data_ptr(),
+                          nnz, H, rows, q.shape[0], q.shape[3], 32,
+                          qq.stride(0), qq.stride(1), qq.stride(2), kk.stride(0), kk.stride(1), kk.stride(2),
+                          float(ctx.scale), _lib.dtype_code(q), _lib.stream_ptr(q.device))
+        else:
+            q, k, v, p, out = ctx.saved_tensors
         dout = dout.contiguous()
         dv = dsd._run('dsd', p, dout, True, False, False)
         delta = (dout.float() * out.float()).sum(-1).contiguous()
-        H, rows, cols = sdd.spdims
-        uni_ptr, uni_inner, uni_blk = sdd._table('union', q.device)
         ds = torch.empty_like(p)
-        vv = v if (v.stride(3) == 1 and all(s_ % 8 == 0 for s_ in v.stride()[:3])) else v.contiguous()
+        vv = vec(v)
         with torch.cuda.device(q.device):
             _lib.call('flyhip_bs_sdd_dsoftmax', dout.data_ptr(), vv.data_ptr(), p.data_ptr(), delta.data_ptr(),
                       ds.data_ptr(), uni_ptr.data_ptr(), uni_inner.data_ptr(), uni_blk.data_ptr(),
@@ -54,7 +80,7 @@ class _AttentionCoreFn(torch.autograd.Function):
                       float(ctx.scale), _lib.dtype_code(q), _lib.stream_ptr(q.device))
         dq = dsd._run('dsd', ds, k, False, False, False)
         dk = dsd._run('dsd', ds, q, True, False, False)
-        return dq, dk, dv, None, None, None, None, None, None
+        return dq, dk, dv, None, None, None, None, None, None, None
 
     @staticmethod
     def supports(sdd, block, dtype, head_dim, device):
@@ -177,10 +203,17 @@ class BlockSparseAttention(nn.Module):
         sdd_nt, dsd_nn, sparse_softmax = self.get_ops(T, S)
         if (needs_grad and not need_weights and not (self.training and self.dropout.p > 0)
                 and E == value.shape[3] and _AttentionCoreFn.supports(sdd_nt, block, query.dtype, E, query.device)):
+            fused = None
+            if (self.fuse and (key_padding_mask is None or key_padding_mask.all_ones)
+                    and (attn_mask is None or attn_mask.all_ones)
+                    and fused_attention.supports(block, query.dtype, E, value.shape[3])):
+                if (T, S) not in self.fused_cache:
+                    self.fused_cache[T, S] = fused_attention(layout, block)
+                fused = self.fused_cache[T, S]
             out = _AttentionCoreFn.apply(
                 q, k, v, sdd_nt, dsd_nn, sparse_softmax, softmax_temp,
-                None if key_padding_mask is None else key_padding_mask.additive_matrix,
-                None if attn_mask is None else attn_mask.additive_matrix)
+                None if fused is not None or key_padding_mask is None else key_padding_mask.additive_matrix,
+                None if fused is not None or attn_mask is None else attn_mask.additive_matrix, fused)
             return out.permute(0, 2, 1, 3)[:, :q_seqlen_og, :, :v_dim_og], None
         qk = sdd_nt(q, k)
         attn = sparse_softmax(qk, scale=softmax_temp,

@@ -31,7 +31,7 @@ class fused_attention:
             self.lut_cache[device] = tuple(t.to(device) for t in union_table(self.layout, self.rows_per_group))
         return self.lut_cache[device]
 
-    def __call__(self, q, k, v, scale, key_mask=None):
+    def __call__(self, q, k, v, scale, key_mask=None, return_lse=False):
         _lib.require_gpu(q, k, v)
         H, p, r = self.spdims
         Z, D = q.shape[0], q.shape[3]
@@ -55,11 +55,14 @@ class fused_attention:
             km, km_stride = key_mask.data_ptr(), key_mask.stride(0)
         uni_ptr, uni_inner, uni_blk = self.make_lut(q.device)
         out = torch.empty((Z, p * 32, H, D), dtype=q.dtype, device=q.device).permute(0, 2, 1, 3)
+        # base-2 log of every row's softmax denominator (+inf for a row without a finite score): what a
+        # backward pass needs to form the probabilities again
+        lse2 = torch.empty((Z, H, p * 32), dtype=torch.float32, device=q.device) if return_lse else None
         with torch.cuda.device(q.device):
-            _lib.call('flyhip_bs_attn', q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+            _lib.call('flyhip_bs_attn_lse', q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), _lib.ptr(lse2),
                       uni_ptr.data_ptr(), uni_inner.data_ptr(), uni_blk.data_ptr(), self.rows_per_group,
                       km, km_stride, Z, H, p, D, 32,
                       q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
                       v.stride(0), v.stride(1), v.stride(2), out.stride(0), out.stride(1), out.stride(2),
                       float(scale), _lib.dtype_code(q), _lib.stream_ptr(q.device))
-        return out
+        return (out, lse2) if return_lse else out

@@ -187,13 +187,16 @@ struct SddUniArgs {
     const int32_t* uni_ptr; const int32_t* uni_inner; const int32_t* uni_blk;
     int nnz, brows_per_head, grps_per_head, n_heads, Z;
     long a_sz, a_sh, a_sm, b_sz, b_sh, b_sn;
-    // DSOFT: c = scale * p * (a b^T - delta[row]) on the nonzero blocks, the gradient of the scores of a
+    // EPI 1: c = scale * p * (a b^T - delta[row]) on the nonzero blocks, the gradient of the scores of a
     // softmax(scale * s) -> p -> p v chain from a = d out, b = v, delta = rowsum(d out * out)
+    // EPI 2: c = 2^(scale * a b^T - delta[row]): the probabilities again from a = q, b = k, scale =
+    // softmax scale * log2(e) and delta = the rows' base-2 log-denominators of the one-kernel attention
     const void* p; const float* delta; float scale;
 };
 
-template <typename T, int KS, bool DSOFT = false>     // KS = K / 32
+template <typename T, int KS, int EPI = 0>     // KS = K / 32; EPI: 0 product, 1 softmax gradient, 2 probabilities
 __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
+    constexpr bool DSOFT = EPI == 1, PROB = EPI == 2;
     constexpr int K = 32 * KS, LD = K + 8;              // LDS row stride: 16 rows of a tile hit all banks once
     constexpr int CPR = K / 8;                          // 16-byte chunks per tile row
     constexpr int NCH = (32 * CPR + 255) / 256;         // chunks per thread
@@ -213,7 +216,7 @@ __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
     const T* bz = reinterpret_cast<const T*>(a.b) + z * a.b_sz + head * a.b_sh;
     T* cz = reinterpret_cast<T*>(a.c) + (long)z * a.nnz * 1024;
     // DSOFT: this lane's rows are 16 tm + r16 of block-row bi
-    const float* dlt = DSOFT ? a.delta + ((long)z * a.n_heads + head) * a.brows_per_head * 32 +
+    const float* dlt = (DSOFT || PROB) ? a.delta + ((long)z * a.n_heads + head) * a.brows_per_head * 32 +
                                    (long)min(bi, a.brows_per_head - 1) * 32 + r16
                              : nullptr;
     uintx4 fa[2][KS];
@@ -299,6 +302,14 @@ __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
                             *reinterpret_cast<uint16_t*>(&e) = (i & 1) ? (uint16_t)(word >> 16) : (uint16_t)(word & 0xffffu);
                             acc[tm][tn][i] = a.scale * Elem<T>::to_f32(e) * (acc[tm][tn][i] - dl);
                         }
+                }
+                if (PROB) {
+                    const float dl = dlt[16 * tm];
+#pragma unroll
+                    for (int tn = 0; tn < 2; ++tn)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                            acc[tm][tn][i] = __builtin_amdgcn_exp2f(__builtin_fmaf(acc[tm][tn][i], a.scale, -dl));
                 }
                 store8_f32(cp + (16 * tm + r16) * 32 + 8 * g, acc[tm][0], acc[tm][1]);
             }
@@ -1009,6 +1020,7 @@ struct AttnArgs {
     int brows_per_head, grps_per_head, n_heads, Z;
     long q_sz, q_sh, q_sm, k_sz, k_sh, k_sn, v_sz, v_sh, v_sn, o_sz, o_sh, o_sm;
     float scale;
+    float* lse2;        // optional (Z, H, 32 * brows_per_head): base-2 log of every row's softmax denominator
 };
 
 // Maxima of scores.  A two-operand fmaxf costs three instructions here (each operand is first quieted
@@ -1247,6 +1259,9 @@ __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
         T* row = op + ((long)bi * 32 + 16 * qt + r16) * a.o_sm + 4 * g;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) store4_f32(row + 16 * dt, o[dt][qt] * inv);
+        if (a.lse2 && g == 0)       // a row without a finite score: +inf, so that 2^(score - lse2) is 0
+            a.lse2[(((long)z * a.n_heads + head) * a.brows_per_head + bi) * 32 + 16 * qt + r16] =
+                l > 0.f ? m_run[qt] + __log2f(l) : INFINITY;
     }
 }
 
@@ -1658,36 +1673,57 @@ extern "C" int flyhip_bs_sdd(const void* a, const void* b, void* c, const int32_
     return check_launch("bs_sdd_kernel");
 }
 
+template <int EPI>
+static int launch_sdd_epilogue(const char* what, const void* a_dn, const void* b_dn, const void* p, const float* rowvec, void* c,
+                               const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
+                               int nnz, int n_heads, int brows_per_head, int Z, int K, int blk,
+                               int64_t a_sz, int64_t a_sh, int64_t a_sm, int64_t b_sz, int64_t b_sh, int64_t b_sn,
+                               float scale, int dtype, void* stream) {
+    int rc = check_common(what, blk, dtype, Z);
+    if (rc) return rc;
+    FLY_REQUIRE(a_dn && b_dn && (EPI != 1 || p) && rowvec && c && uni_ptr && uni_inner && uni_blk, "%s: null pointer", what);
+    FLY_REQUIRE(blk == 32 && (dtype == BF16 || dtype == F16), "%s: needs 32x32 blocks of bf16 / fp16", what);
+    FLY_REQUIRE(K % 32 == 0 && K >= 32 && K <= 128, "%s: head dim %d not a multiple of 32 up to 128", what, K);
+    FLY_REQUIRE(nnz > 0 && n_heads > 0 && brows_per_head > 0, "%s: bad sizes", what);
+    FLY_REQUIRE(((a_sz | a_sh | a_sm | b_sz | b_sh | b_sn) % 8) == 0, "%s: strides must be multiples of 8 elements", what);
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    const int gph = (brows_per_head + 3) / 4;
+    SddUniArgs ua{a_dn, b_dn, c, uni_ptr, uni_inner, uni_blk, nnz, brows_per_head, gph, n_heads, Z,
+                  a_sz, a_sh, a_sm, b_sz, b_sh, b_sn, p, rowvec, scale};
+    const long nwg = unit_grid((long)n_heads * Z, gph);
+    FLY_REQUIRE(nwg <= 2147483647L, "%s: too many workgroups", what);
+    dim3 grid((unsigned)nwg);
+#define SDDS_LAUNCH(T)                                                                                  \
+    switch (K / 32) {                                                                                   \
+        case 1: hipLaunchKernelGGL((bs_sdd32u_kernel<T, 1, EPI>), grid, dim3(256), 0, st, ua); break;  \
+        case 2: hipLaunchKernelGGL((bs_sdd32u_kernel<T, 2, EPI>), grid, dim3(256), 0, st, ua); break;  \
+        case 3: hipLaunchKernelGGL((bs_sdd32u_kernel<T, 3, EPI>), grid, dim3(256), 0, st, ua); break;  \
+        default: hipLaunchKernelGGL((bs_sdd32u_kernel<T, 4, EPI>), grid, dim3(256), 0, st, ua); break; \
+    }
+    if (dtype == BF16) { SDDS_LAUNCH(bf16_t) } else { SDDS_LAUNCH(f16_t) }
+#undef SDDS_LAUNCH
+    return check_launch(what);
+}
+
 extern "C" int flyhip_bs_sdd_dsoftmax(const void* dout, const void* v, const void* p, const float* delta, void* ds,
                                       const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
                                       int nnz, int n_heads, int brows_per_head, int Z, int K, int blk,
                                       int64_t a_sz, int64_t a_sh, int64_t a_sm,
                                       int64_t b_sz, int64_t b_sh, int64_t b_sn,
                                       float scale, int dtype, void* stream) {
-    int rc = check_common("bs_sdd_dsoftmax", blk, dtype, Z);
-    if (rc) return rc;
-    FLY_REQUIRE(dout && v && p && delta && ds && uni_ptr && uni_inner && uni_blk, "bs_sdd_dsoftmax: null pointer");
-    FLY_REQUIRE(blk == 32 && (dtype == BF16 || dtype == F16), "bs_sdd_dsoftmax: needs 32x32 blocks of bf16 / fp16");
-    FLY_REQUIRE(K % 32 == 0 && K >= 32 && K <= 128, "bs_sdd_dsoftmax: head dim %d not a multiple of 32 up to 128", K);
-    FLY_REQUIRE(nnz > 0 && n_heads > 0 && brows_per_head > 0, "bs_sdd_dsoftmax: bad sizes");
-    FLY_REQUIRE(((a_sz | a_sh | a_sm | b_sz | b_sh | b_sn) % 8) == 0, "bs_sdd_dsoftmax: strides must be multiples of 8 elements");
-    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    const int gph = (brows_per_head + 3) / 4;
-    SddUniArgs ua{dout, v, ds, uni_ptr, uni_inner, uni_blk, nnz, brows_per_head, gph, n_heads, Z,
-                  a_sz, a_sh, a_sm, b_sz, b_sh, b_sn, p, delta, scale};
-    const long nwg = unit_grid((long)n_heads * Z, gph);
-    FLY_REQUIRE(nwg <= 2147483647L, "bs_sdd_dsoftmax: too many workgroups");
-    dim3 grid((unsigned)nwg);
-#define SDDS_LAUNCH(T)                                                                                  \
-    switch (K / 32) {                                                                                   \
-        case 1: hipLaunchKernelGGL((bs_sdd32u_kernel<T, 1, true>), grid, dim3(256), 0, st, ua); break;  \
-        case 2: hipLaunchKernelGGL((bs_sdd32u_kernel<T, 2, true>), grid, dim3(256), 0, st, ua); break;  \
-        case 3: hipLaunchKernelGGL((bs_sdd32u_kernel<T, 3, true>), grid, dim3(256), 0, st, ua); break;  \
-        default: hipLaunchKernelGGL((bs_sdd32u_kernel<T, 4, true>), grid, dim3(256), 0, st, ua); break; \
-    }
-    if (dtype == BF16) { SDDS_LAUNCH(bf16_t) } else { SDDS_LAUNCH(f16_t) }
-#undef SDDS_LAUNCH
-    return check_launch("bs_sdd32u_kernel (dsoftmax)");
+    return launch_sdd_epilogue<1>("bs_sdd_dsoftmax", dout, v, p, delta, ds, uni_ptr, uni_inner, uni_blk, nnz, n_heads,
+                                  brows_per_head, Z, K, blk, a_sz, a_sh, a_sm, b_sz, b_sh, b_sn, scale, dtype, stream);
+}
+
+extern "C" int flyhip_bs_sdd_prob(const void* q, const void* k, const float* lse2, void* p,
+                                  const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
+                                  int nnz, int n_heads, int brows_per_head, int Z, int K, int blk,
+                                  int64_t a_sz, int64_t a_sh, int64_t a_sm,
+                                  int64_t b_sz, int64_t b_sh, int64_t b_sn,
+                                  float scale, int dtype, void* stream) {
+    return launch_sdd_epilogue<2>("bs_sdd_prob", q, k, nullptr, lse2, p, uni_ptr, uni_inner, uni_blk, nnz, n_heads,
+                                  brows_per_head, Z, K, blk, a_sz, a_sh, a_sm, b_sz, b_sh, b_sn,
+                                  scale * 1.4426950408889634f, dtype, stream);
 }
 
 extern "C" int flyhip_bs_sdd_kmajor(const void* a, const void* b, float* c32,
@@ -1835,7 +1871,7 @@ static int launch_softmax(const RowArgs& args, dim3 grid, int max_elems, hipStre
     return check_launch("bs_softmax_kernel");
 }
 
-extern "C" int flyhip_bs_attn(const void* q, const void* k, const void* v, void* out,
+extern "C" int flyhip_bs_attn_lse(const void* q, const void* k, const void* v, void* out, float* lse2,
                               const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
                               int rows_per_group, const float* key_mask, int64_t key_mask_stride,
                               int Z, int H, int brows_per_head, int D, int blk,
@@ -1858,7 +1894,7 @@ extern "C" int flyhip_bs_attn(const void* q, const void* k, const void* v, void*
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     const int gph = (brows_per_head + rows_per_group - 1) / rows_per_group;
     AttnArgs args{q, k, v, out, uni_ptr, uni_inner, uni_blk, key_mask, key_mask_stride, brows_per_head, gph, H, Z,
-                  q_sz, q_sh, q_sm, k_sz, k_sh, k_sn, v_sz, v_sh, v_sn, o_sz, o_sh, o_sm, scale};
+                  q_sz, q_sh, q_sm, k_sz, k_sh, k_sn, v_sz, v_sh, v_sn, o_sz, o_sh, o_sm, scale, lse2};
     const long nwg = unit_grid((long)H * Z, gph);
     FLY_REQUIRE(nwg <= 2147483647L, "bs_attn: too many workgroups");
     dim3 grid((unsigned)nwg);
@@ -1874,6 +1910,20 @@ extern "C" int flyhip_bs_attn(const void* q, const void* k, const void* v, void*
 #undef ATTN_KS
 #undef ATTN_LAUNCH
     return check_launch("bs_attn32_kernel");
+}
+
+extern "C" int flyhip_bs_attn(const void* q, const void* k, const void* v, void* out,
+                              const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
+                              int rows_per_group, const float* key_mask, int64_t key_mask_stride,
+                              int Z, int H, int brows_per_head, int D, int blk,
+                              int64_t q_sz, int64_t q_sh, int64_t q_sm,
+                              int64_t k_sz, int64_t k_sh, int64_t k_sn,
+                              int64_t v_sz, int64_t v_sh, int64_t v_sn,
+                              int64_t o_sz, int64_t o_sh, int64_t o_sm,
+                              float scale, int dtype, void* stream) {
+    return flyhip_bs_attn_lse(q, k, v, out, nullptr, uni_ptr, uni_inner, uni_blk, rows_per_group, key_mask, key_mask_stride,
+                              Z, H, brows_per_head, D, blk, q_sz, q_sh, q_sm, k_sz, k_sh, k_sn, v_sz, v_sh, v_sn,
+                              o_sz, o_sh, o_sm, scale, dtype, stream);
 }
 
 extern "C" int flyhip_bs_softmax(void* x, const int32_t* row_ptr, const int32_t* row_blk, const int32_t* row_col,

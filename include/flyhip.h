@@ -273,6 +273,31 @@ int flyhip_bs_attn(const void* q, const void* k, const void* v, void* out,
                    int64_t o_sz, int64_t o_sh, int64_t o_sm,
                    float scale, int dtype, void* stream);
 
+/* flyhip_bs_attn that also writes, when lse2 is not NULL, the base-2 logarithm of every row's softmax
+ * denominator, (Z, H, 32 * brows_per_head) float32, +inf for a row without a finite score: all a
+ * backward pass needs to form the probabilities again (the reference keeps the (Z, nnz, 32, 32)
+ * probability tensor for autograd, blocksparse_attention.py:146-160). */
+int flyhip_bs_attn_lse(const void* q, const void* k, const void* v, void* out, float* lse2,
+                       const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
+                       int rows_per_group, const float* key_mask, int64_t key_mask_stride,
+                       int Z, int H, int brows_per_head, int D, int blk,
+                       int64_t q_sz, int64_t q_sh, int64_t q_sm,
+                       int64_t k_sz, int64_t k_sh, int64_t k_sn,
+                       int64_t v_sz, int64_t v_sh, int64_t v_sn,
+                       int64_t o_sz, int64_t o_sh, int64_t o_sm,
+                       float scale, int dtype, void* stream);
+
+/* The probabilities of that attention again, in the block-sparse format: p = exp(scale * q k^T - lse) on
+ * the nonzero blocks, as one sdd (blocksparse_matmul.py:279-346) with an exponential epilogue;
+ * lse2 as written by flyhip_bs_attn_lse; tables as for flyhip_bs_sdd's shared-tile path (four
+ * block-rows per group). */
+int flyhip_bs_sdd_prob(const void* q, const void* k, const float* lse2, void* p,
+                       const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
+                       int nnz, int n_heads, int brows_per_head, int Z, int K, int blk,
+                       int64_t a_sz, int64_t a_sh, int64_t a_sm,
+                       int64_t b_sz, int64_t b_sh, int64_t b_sn,
+                       float scale, int dtype, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * Block-sparse row operations.  row_ptr (n_brow+1) / row_blk / row_col int32: for every
  * (head, block-row) the ids and block-columns of its nonzero blocks (the information of the

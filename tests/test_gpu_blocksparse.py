@@ -471,10 +471,13 @@ def test_dsd_with_transposed_sparse_operand(p, r, N, dtype):
     assert rel_err(out2.transpose(2, 3), ref) <= TOL[dtype]
 
 
-def test_blocksparse_attention_module_gradients():
+@pytest.mark.parametrize('masked', [True, False])
+def test_blocksparse_attention_module_gradients(masked):
     """Training path of BlockSparseAttention for 2-byte inputs: one autograd node whose backward runs
     dV, the fused score gradient, dQ and dK on the tiled kernels; gradients against autograd through
-    the oracle in float64 on the same rounded inputs, with padded keys."""
+    the oracle in float64 on the same rounded inputs.  With padded keys the forward is the three ops and
+    keeps the probabilities; without masks it is the one-kernel attention and the backward forms the
+    probabilities again from the rows' log-denominators."""
     from fly_amd import BlockSparseAttention, LengthMask
 
     class Cfg:
@@ -490,13 +493,14 @@ def test_blocksparse_attention_module_gradients():
     g = torch.Generator().manual_seed(8)
     q, k, v = (torch.randn(B, T, H, E, generator=g).bfloat16() for _ in range(3))
     w = torch.randn(B, T, H, E, generator=g)
-    lengths = torch.tensor([T, 200])
+    lengths = torch.tensor([T, 200]) if masked else None
     mod = BlockSparseAttention(Cfg(), attention_dropout=0.0, max_seq_length=512).to(DEV)
     qd, kd, vd = (x.double().requires_grad_() for x in (q, k, v))
     ref = ob.blocksparse_attention(qd, kd, vd, mod.master_layout.cpu(), 32, key_lengths=lengths)
     (ref * w.double()).sum().backward()
     qg, kg, vg = (x.to(DEV).requires_grad_() for x in (q, k, v))
-    out, _ = mod(qg, kg, vg, key_padding_mask=LengthMask(lengths.to(DEV), max_len=T))
+    out, _ = mod(qg, kg, vg, key_padding_mask=LengthMask(lengths.to(DEV), max_len=T) if masked else None)
+    assert (len(mod.fused_cache) == 1) == (not masked)
     seen, todo = set(), [out.grad_fn]
     while todo:                                           # the node sits behind the views that un-pad the output
         fn = todo.pop()
@@ -509,4 +513,5 @@ def test_blocksparse_attention_module_gradients():
     (out.float() * w.to(DEV)).sum().backward()
     for got, want, name in ((qg.grad, qd.grad, 'dq'), (kg.grad, kd.grad, 'dk'), (vg.grad, vd.grad, 'dv')):
         assert rel_err(got.float(), want) <= 3e-2, (name, rel_err(got.float(), want))
-    assert float(kg.grad[1, 200:].abs().max()) == 0.0
+    if masked:
+        assert float(kg.grad[1, 200:].abs().max()) == 0.0
