@@ -255,3 +255,48 @@ def test_backward_band_kernels_match_library_products(B, T, S, H, E, D, mh, lc, 
         got = sblocal_backward(q, k, v, P, lc, None, kl, out, ln, go, band_kernel=mode)
         for a, b in zip(got, ref):
             assert rel_err(a, b) <= 1e-4, (mode, rel_err(a, b))
+
+
+def test_random_shapes_sweep():
+    """Forty seeded random problems (ragged T != S, head dims that need padding, odd and even windows up
+    to wider than the sequence, feature counts from 2 to 256, key lengths down to one key, one to three
+    heads, fp32 and bf16): forward against the oracle in float64 on the same rounded inputs, and -- where
+    the backward kernels apply -- the gradients on the kernels against the library-product path."""
+    from fly_amd import sblocal_backward
+    from fly_amd.sblocal_attention import sblocal_forward
+    dev = torch.device('cuda:0')
+    rng = torch.Generator().manual_seed(20240)
+
+    def pick(lo, hi):
+        return int(torch.randint(lo, hi + 1, (1,), generator=rng))
+    for case in range(40):
+        B, H = pick(1, 3), pick(1, 3)
+        T, S = pick(1, 400), pick(1, 400)
+        E, D = pick(1, 128), pick(1, 128)
+        mh = [1, 3, 8, 16, 24, 32, 64, 100, 128][pick(0, 8)]
+        lc = pick(1, 2 * max(T, S))
+        dtype = torch.bfloat16 if case % 4 == 3 else torch.float32
+        lengths = None
+        if case % 3 == 0:
+            lengths = torch.randint(1, S + 1, (B,), generator=rng)
+        print('case', case, B, H, T, S, E, D, mh, lc, dtype, None if lengths is None else lengths.tolist(), flush=True)
+        q, k, v, P = make_inputs(B, T, S, H, E, D, mh, seed=1000 + case, dtype=dtype)
+        out, ln, ref_out, ref_ln = run_both(q, k, v, P, lc, None, lengths)
+        if dtype == torch.float32:
+            # few features make the estimator ill conditioned: the bar is a small multiple of the float32
+            # oracle's own distance from its float64 evaluation, never tighter than 1e-4
+            o32, l32 = osb.sblocal_attention(q, k, v, P, lc, key_lengths=lengths)
+            assert rel_err(out, ref_out) <= max(1e-4, 4 * rel_err(o32, ref_out)), rel_err(out, ref_out)
+            assert rel_err(ln, ref_ln) <= max(1e-4, 4 * rel_err(l32, ref_ln)), rel_err(ln, ref_ln)
+        else:
+            assert rel_err(out, ref_out) <= 2e-2, rel_err(out, ref_out)
+            assert rel_err(ln, ref_ln) <= 2e-2, rel_err(ln, ref_ln)
+        if dtype == torch.float32 and max(E, D) <= 64 and 2 * mh <= 128 and case % 2 == 0:
+            go = torch.randn(B, T, H, D, generator=rng).to(dev)
+            kl = None if lengths is None else lengths.to(dev)
+            o_dev, ln_dev = sblocal_forward(q.to(dev), k.to(dev), v.to(dev), P.to(dev), lc, key_lengths=kl)
+            args = (q.to(dev), k.to(dev), v.to(dev), P.to(dev), lc, None, kl, o_dev, ln_dev, go)
+            ref = sblocal_backward(*args, band_kernel=False)
+            got = sblocal_backward(*args, band_kernel=True)
+            for a, b in zip(got, ref):
+                assert rel_err(a, b) <= 2e-4, rel_err(a, b)
