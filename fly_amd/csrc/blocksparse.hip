@@ -192,15 +192,20 @@ struct SddUniArgs {
     // EPI 2: c = 2^(scale * a b^T - delta[row]): the probabilities again from a = q, b = k, scale =
     // softmax scale * log2(e) and delta = the rows' base-2 log-denominators of the one-kernel attention
     const void* p; const float* delta; float scale;
+    // EPI 3: both at once from a = d out, b = v and a2 = q, b2 = k (strides as a, b): p2 = 2^(scale2 * a2 b2^T -
+    // lse2[row]) is written to p2 and c = scale * p2 * (a b^T - delta[row])
+    const void* a2; const void* b2; const float* lse2; void* p2; float scale2;
+    long a2_sz, a2_sh, a2_sm, b2_sz, b2_sh, b2_sn;
 };
 
 template <typename T, int KS, int EPI = 0>     // KS = K / 32; EPI: 0 product, 1 softmax gradient, 2 probabilities
 __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
-    constexpr bool DSOFT = EPI == 1, PROB = EPI == 2;
+    constexpr bool DSOFT = EPI == 1, PROB = EPI == 2, BOTH = EPI == 3;
     constexpr int K = 32 * KS, LD = K + 8;              // LDS row stride: 16 rows of a tile hit all banks once
     constexpr int CPR = K / 8;                          // 16-byte chunks per tile row
     constexpr int NCH = (32 * CPR + 255) / 256;         // chunks per thread
     __shared__ __attribute__((aligned(16))) uint16_t tile[2][32 * LD];
+    __shared__ __attribute__((aligned(16))) uint16_t tile2[BOTH ? 2 : 1][BOTH ? 32 * LD : 8];
     const int tid = threadIdx.x, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     int unit, grp;
@@ -216,26 +221,43 @@ __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
     const T* bz = reinterpret_cast<const T*>(a.b) + z * a.b_sz + head * a.b_sh;
     T* cz = reinterpret_cast<T*>(a.c) + (long)z * a.nnz * 1024;
     // DSOFT: this lane's rows are 16 tm + r16 of block-row bi
-    const float* dlt = (DSOFT || PROB) ? a.delta + ((long)z * a.n_heads + head) * a.brows_per_head * 32 +
-                                   (long)min(bi, a.brows_per_head - 1) * 32 + r16
-                             : nullptr;
+    const long rowvec_off = ((long)z * a.n_heads + head) * a.brows_per_head * 32 + (long)min(bi, a.brows_per_head - 1) * 32 + r16;
+    const float* dlt = (DSOFT || PROB || BOTH) ? a.delta + rowvec_off : nullptr;
     uintx4 fa[2][KS];
 #pragma unroll
     for (int tm = 0; tm < 2; ++tm)
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) fa[tm][ks] = *reinterpret_cast<const uintx4*>(ap + 16 * tm * a.a_sm + 32 * ks);
+    // EPI 3: the second product's row operand, column tiles and row vector
+    uintx4 fa2[BOTH ? 2 : 1][BOTH ? KS : 1];
+    const T* bz2 = nullptr;
+    float lse_row[2] = {0.f, 0.f}, dl_row[2] = {0.f, 0.f};
+    if (BOTH) {
+        const T* ap2 = reinterpret_cast<const T*>(a.a2) + z * a.a2_sz + head * a.a2_sh +
+                       (long)(min(bi, a.brows_per_head - 1) * 32 + r16) * a.a2_sm + 8 * g;
+#pragma unroll
+        for (int tm = 0; tm < 2; ++tm) {
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) fa2[BOTH ? tm : 0][BOTH ? ks : 0] = *reinterpret_cast<const uintx4*>(ap2 + 16 * tm * a.a2_sm + 32 * ks);
+            lse_row[tm] = a.lse2[rowvec_off + 16 * tm];
+            dl_row[tm] = dlt[16 * tm];
+        }
+        bz2 = reinterpret_cast<const T*>(a.b2) + z * a.b2_sz + head * a.b2_sh;
+    }
 
     // staging: chunk c = tid + 256 i is 16 bytes of tile row c / CPR.  Block column n lands in LDS row
     // 16*((n>>2)&1) + 4*(n>>3) + (n&3), so that MFMA tile tn reads the 16 consecutive LDS rows
     // 16 tn .. 16 tn + 15 and its row i is block column 8*(i/4) + 4*tn + i%4: the four results a lane
     // gets from tile 0 and the four from tile 1 are eight consecutive columns -> one 16-byte store
-    uintx4 reg[NCH];
+    uintx4 reg[NCH], reg2[BOTH ? NCH : 1];
     auto fetch = [&](int inner) __attribute__((always_inline)) {
         const long brow_b = (long)inner * 32;
 #pragma unroll
         for (int i = 0; i < NCH; ++i) {
             const int c = tid + 256 * i;
             if (c < 32 * CPR) reg[i] = *reinterpret_cast<const uintx4*>(bz + (brow_b + c / CPR) * a.b_sn + 8 * (c % CPR));
+            if (BOTH && c < 32 * CPR)
+                reg2[BOTH ? i : 0] = *reinterpret_cast<const uintx4*>(bz2 + (brow_b + c / CPR) * a.b2_sn + 8 * (c % CPR));
         }
     };
     auto stash = [&](int buf) __attribute__((always_inline)) {
@@ -244,6 +266,7 @@ __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
             const int c = tid + 256 * i, nrow = c / CPR;
             const int lrow = 16 * ((nrow >> 2) & 1) + 4 * (nrow >> 3) + (nrow & 3);
             if (c < 32 * CPR) *reinterpret_cast<uintx4*>(&tile[buf][lrow * LD + 8 * (c % CPR)]) = reg[i];
+            if (BOTH && c < 32 * CPR) *reinterpret_cast<uintx4*>(&tile2[BOTH ? buf : 0][lrow * LD + 8 * (c % CPR)]) = reg2[BOTH ? i : 0];
         }
     };
     // the index lists are read two steps (block-column) and one step (block id) ahead of their use
@@ -258,7 +281,7 @@ __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
         const int blk_n1 = s + 1 < n ? a.uni_blk[(long)(p0 + s + 1) * 4 + w] : -1;
         if (s + 1 < n) fetch(inner_n1);
         const bool mine = blk >= 0 && have_row;
-        floatx4 acc[2][2];
+        floatx4 acc[2][2], acc2[2][2];
         uintx4 pv[2];
         if (DSOFT && mine) {                              // requested before the products, used after them
             const T* pp = reinterpret_cast<const T*>(a.p) + ((long)z * a.nnz + blk) * 1024;
@@ -282,6 +305,23 @@ __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
 #pragma unroll
                     for (int ks = 0; ks < KS; ++ks) acc[tm][tn] = mma32<T>(fb[tn][ks], fa[tm][ks], acc[tm][tn]);
                 }
+            if (BOTH) {
+                const uint16_t* tp2 = tile2[BOTH ? (s & 1) : 0];
+#pragma unroll
+                for (int tn = 0; tn < 2; ++tn)
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks)
+                        fb[tn][ks] = *reinterpret_cast<const uintx4*>(tp2 + (16 * tn + r16) * LD + 32 * ks + 8 * g);
+#pragma unroll
+                for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+                    for (int tn = 0; tn < 2; ++tn) {
+                        acc2[tm][tn] = Frag<float>::zero();
+#pragma unroll
+                        for (int ks = 0; ks < KS; ++ks)
+                            acc2[tm][tn] = mma32<T>(fb[tn][ks], fa2[BOTH ? tm : 0][BOTH ? ks : 0], acc2[tm][tn]);
+                    }
+            }
         }
         // the next tile goes to LDS before this step's stores are issued: the wait for its loads would
         // otherwise wait for the stores too (one counter covers both)
@@ -302,6 +342,18 @@ __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
                             *reinterpret_cast<uint16_t*>(&e) = (i & 1) ? (uint16_t)(word >> 16) : (uint16_t)(word & 0xffffu);
                             acc[tm][tn][i] = a.scale * Elem<T>::to_f32(e) * (acc[tm][tn][i] - dl);
                         }
+                }
+                if (BOTH) {
+#pragma unroll
+                    for (int tn = 0; tn < 2; ++tn)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(acc2[tm][tn][i], a.scale2, -lse_row[tm]));
+                            acc2[tm][tn][i] = pr;
+                            acc[tm][tn][i] = a.scale * pr * (acc[tm][tn][i] - dl_row[tm]);
+                        }
+                    T* pp2 = reinterpret_cast<T*>(a.p2) + ((long)z * a.nnz + blk) * 1024;
+                    store8_f32(pp2 + (16 * tm + r16) * 32 + 8 * g, acc2[tm][0], acc2[tm][1]);
                 }
                 if (PROB) {
                     const float dl = dlt[16 * tm];
@@ -1678,7 +1730,7 @@ static int launch_sdd_epilogue(const char* what, const void* a_dn, const void* b
                                const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
                                int nnz, int n_heads, int brows_per_head, int Z, int K, int blk,
                                int64_t a_sz, int64_t a_sh, int64_t a_sm, int64_t b_sz, int64_t b_sh, int64_t b_sn,
-                               float scale, int dtype, void* stream) {
+                               float scale, int dtype, void* stream, const SddUniArgs* second = nullptr) {
     int rc = check_common(what, blk, dtype, Z);
     if (rc) return rc;
     FLY_REQUIRE(a_dn && b_dn && (EPI != 1 || p) && rowvec && c && uni_ptr && uni_inner && uni_blk, "%s: null pointer", what);
@@ -1690,6 +1742,14 @@ static int launch_sdd_epilogue(const char* what, const void* a_dn, const void* b
     const int gph = (brows_per_head + 3) / 4;
     SddUniArgs ua{a_dn, b_dn, c, uni_ptr, uni_inner, uni_blk, nnz, brows_per_head, gph, n_heads, Z,
                   a_sz, a_sh, a_sm, b_sz, b_sh, b_sn, p, rowvec, scale};
+    if (EPI == 3) {
+        FLY_REQUIRE(second && second->a2 && second->b2 && second->lse2 && second->p2, "%s: null pointer", what);
+        FLY_REQUIRE(((second->a2_sz | second->a2_sh | second->a2_sm | second->b2_sz | second->b2_sh | second->b2_sn) % 8) == 0,
+                    "%s: strides must be multiples of 8 elements", what);
+        ua.a2 = second->a2; ua.b2 = second->b2; ua.lse2 = second->lse2; ua.p2 = second->p2; ua.scale2 = second->scale2;
+        ua.a2_sz = second->a2_sz; ua.a2_sh = second->a2_sh; ua.a2_sm = second->a2_sm;
+        ua.b2_sz = second->b2_sz; ua.b2_sh = second->b2_sh; ua.b2_sn = second->b2_sn;
+    }
     const long nwg = unit_grid((long)n_heads * Z, gph);
     FLY_REQUIRE(nwg <= 2147483647L, "%s: too many workgroups", what);
     dim3 grid((unsigned)nwg);
@@ -1713,6 +1773,24 @@ extern "C" int flyhip_bs_sdd_dsoftmax(const void* dout, const void* v, const voi
                                       float scale, int dtype, void* stream) {
     return launch_sdd_epilogue<1>("bs_sdd_dsoftmax", dout, v, p, delta, ds, uni_ptr, uni_inner, uni_blk, nnz, n_heads,
                                   brows_per_head, Z, K, blk, a_sz, a_sh, a_sm, b_sz, b_sh, b_sn, scale, dtype, stream);
+}
+
+extern "C" int flyhip_bs_sdd_prob_dsoftmax(const void* dout, const void* v, const void* q, const void* k,
+                                           const float* delta, const float* lse2, void* ds, void* p,
+                                           const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
+                                           int nnz, int n_heads, int brows_per_head, int Z, int K, int blk,
+                                           int64_t do_sz, int64_t do_sh, int64_t do_sm,
+                                           int64_t v_sz, int64_t v_sh, int64_t v_sn,
+                                           int64_t q_sz, int64_t q_sh, int64_t q_sm,
+                                           int64_t k_sz, int64_t k_sh, int64_t k_sn,
+                                           float scale, int dtype, void* stream) {
+    SddUniArgs second{};
+    second.a2 = q; second.b2 = k; second.lse2 = lse2; second.p2 = p; second.scale2 = scale * 1.4426950408889634f;
+    second.a2_sz = q_sz; second.a2_sh = q_sh; second.a2_sm = q_sm;
+    second.b2_sz = k_sz; second.b2_sh = k_sh; second.b2_sn = k_sn;
+    return launch_sdd_epilogue<3>("bs_sdd_prob_dsoftmax", dout, v, nullptr, delta, ds, uni_ptr, uni_inner, uni_blk, nnz,
+                                  n_heads, brows_per_head, Z, K, blk, do_sz, do_sh, do_sm, v_sz, v_sh, v_sn, scale, dtype,
+                                  stream, &second);
 }
 
 extern "C" int flyhip_bs_sdd_prob(const void* q, const void* k, const float* lse2, void* p,

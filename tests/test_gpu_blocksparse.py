@@ -515,3 +515,32 @@ def test_blocksparse_attention_module_gradients(masked):
         assert rel_err(got.float(), want) <= 3e-2, (name, rel_err(got.float(), want))
     if masked:
         assert float(kg.grad[1, 200:].abs().max()) == 0.0
+
+
+def test_probabilities_from_log_denominators():
+    """flyhip_bs_attn_lse + flyhip_bs_sdd_prob: the one-kernel attention's per-row log-denominators
+    turn an sdd into the softmax probabilities (what the training path's backward starts from); against
+    the oracle's block softmax, with an empty block-row."""
+    from fly_amd import _lib, matmul
+    from fly_amd.blocksparse_fused import fused_attention
+    Z, H, p, r, D, block = 2, 3, 9, 7, 64, 32
+    g = torch.Generator().manual_seed(77)
+    rows = torch.arange(p).view(-1, 1) * r // p
+    layout = ((rows - torch.arange(r).view(1, -1)).abs() <= 2).long().unsqueeze(0).repeat(H, 1, 1)     # neighbouring rows share columns
+    layout[1, 2, :] = 0
+    q = torch.randn(Z, H, p * block, D, generator=g).bfloat16()
+    k = torch.randn(Z, H, r * block, D, generator=g).bfloat16()
+    v = torch.randn(Z, H, r * block, D, generator=g).bfloat16()
+    out, lse2 = fused_attention(layout, block)(q.to(DEV), k.to(DEV), v.to(DEV), 0.2, return_lse=True)
+    assert lse2.shape == (Z, H, p * block) and bool(torch.isinf(lse2[:, 1, 2 * block:3 * block]).all())
+    sdd = matmul(layout, block, 'sdd', trans_b=True)
+    uni_ptr, uni_inner, uni_blk = sdd._table('union', torch.device(DEV))
+    nnz = int(layout.sum())
+    qd, kd = q.to(DEV), k.to(DEV)
+    probs = torch.empty(Z, nnz, block, block, dtype=torch.bfloat16, device=DEV)
+    _lib.call('flyhip_bs_sdd_prob', qd.data_ptr(), kd.data_ptr(), lse2.data_ptr(), probs.data_ptr(),
+              uni_ptr.data_ptr(), uni_inner.data_ptr(), uni_blk.data_ptr(), nnz, H, p, Z, D, block,
+              qd.stride(0), qd.stride(1), qd.stride(2), kd.stride(0), kd.stride(1), kd.stride(2),
+              0.2, _lib.dtype_code(qd), _lib.stream_ptr(torch.device(DEV)))
+    ref = ob.block_softmax(ob.sdd(q.float(), k.float(), layout, block, trans_b=True), layout, block, scale=0.2)
+    assert rel_err(probs, ref.nan_to_num()) <= 2e-2
