@@ -857,10 +857,11 @@ __global__ __launch_bounds__(256) void bs_dds_kernel(DxdArgs a) {
 // Fast DDS (y = x W^T, W block-sparse, blocks read transposed) for 32x32 blocks of a 2-byte type,
 // the Pixelfly linear.  Consecutive output block-rows that reduce over the same input blocks are
 // grouped (at most four per group, table built on the host): a group is a small dense GEMM
-// y[M x 32g] = x[:, listed input blocks] . W_group^T.  One workgroup per (group, 128-token tile):
-// per input block the 128 x 32 activation tile and the group's 32g x 32 weight tile are staged in
-// LDS (registers hold the next step's tiles while the MFMAs of the current one run), the 2 x 2
-// waves own 64 x 64 outputs each and form them with 16x16x32 MFMAs.
+// y[M x 32g] = x[:, listed input blocks] . W_group^T.  A workgroup owns one group and walks a stream
+// of 128-token tiles with one continuous pipeline: per input block the 128 x 32 activation tile and
+// the group's 32g x 32 weight tile are staged in LDS (registers hold the next-but-one step's tiles
+// while the MFMAs of the current one run, across tile boundaries), the 2 x 2 waves own 64 x 64
+// outputs each, form them with 16x16x32 MFMAs and store them after the tile's last input block.
 struct DdsGroupArgs {
     const void* sp; const void* dn; void* c;
     const int32_t* seg_ptr; const int32_t* seg_blk; const int32_t* seg_inner;

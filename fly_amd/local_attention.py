@@ -89,7 +89,7 @@ def local_backward(query, key, value, local_context, softmax_temp, key_lengths, 
         lens = key_lengths.to(Q.device).repeat_interleave(H).view(B * H, 1, 1)
     band = BandWindows(T, S, local_context, chunk, Q.device, lens, max_elements)
     Qc, Gc = band.chunks(Q), band.chunks(G)
-    acc_k, acc_v = band.key_accumulator(E, wdt), band.key_accumulator(D, wdt)
+    acc_k, acc_v = band.key_accumulator(B * H, E, wdt), band.key_accumulator(B * H, D, wdt)
     dQc = torch.zeros_like(Qc)
     Kw, Vw = band.windows(K), band.windows(V)
     for j0, j1 in band.groups(B * H):

@@ -75,22 +75,20 @@ class BandWindows:
             ok = ok & (s < self.lens.view(-1, 1, 1, 1))
         return self.pattern & ok
 
-    def key_accumulator(self, F, dtype):
-        return torch.zeros(0, dtype=dtype, device=self.device), F     # allocated on first use (batch known then)
+    def key_accumulator(self, batch, F, dtype):
+        """Zeroed (batch, n + P - 1, C, F): the zero-padded key axis cut into chunk-sized pieces."""
+        return torch.zeros(batch, self.n + self.P - 1, self.C, F, dtype=dtype, device=self.device)
 
-    def add_windows(self, acc, j0, win):
+    def add_windows(self, buf, j0, win):
         """Overlap-add windows j0.. (BH, g, W, F): piece p of window j lands on key chunk j + p."""
-        buf, F = acc
-        BH, g = win.shape[0], win.shape[1]
-        if buf.numel() == 0:
-            buf.resize_(BH, self.n + self.P - 1, self.C, F).zero_()
+        BH, g, F = win.shape[0], win.shape[1], win.shape[3]
         wv = win.reshape(BH, g, self.P, self.C, F)
         for p in range(self.P):
             buf[:, j0 + p:j0 + p + g] += wv[:, :, p]
 
-    def fold(self, acc):
+    def fold(self, buf):
         """Accumulated windows -> (BH, S, F)."""
-        buf, F = acc
+        F = buf.shape[3]
         flat = buf.reshape(buf.shape[0], -1, F)                 # row r is key r - lc_lo
         out = flat.new_zeros(buf.shape[0], self.S, F)
         hi = min(flat.shape[1], self.lc_lo + self.S)
@@ -189,7 +187,7 @@ def _band_terms_torch(Q, K, V, G, psi, phik, LN, c, lens, local_context, t, chun
     S, D, mh2, wdt = K.shape[1], V.shape[2], psi.shape[2], Q.dtype
     band = BandWindows(T, S, local_context, chunk, Q.device, lens, max_elements)
     Qc, Gc, Pc, cc, LNc = (band.chunks(x) for x in (Q, G, psi, c, LN))
-    acc_k, acc_v, acc_u = band.key_accumulator(E, wdt), band.key_accumulator(D, wdt), band.key_accumulator(mh2, wdt)
+    acc_k, acc_v, acc_u = (band.key_accumulator(BH, F, wdt) for F in (E, D, mh2))
     dQc, uqc = torch.zeros_like(Qc), torch.zeros_like(Pc)
     Kw, Vw, PKw = band.windows(K), band.windows(V), band.windows(phik)
     for j0, j1 in band.groups(BH):
