@@ -63,16 +63,19 @@ class _AttentionCoreFn(torch.autograd.Function):
             ds = torch.empty_like(p)
             delta = (dout.float() * out.float()).sum(-1).contiguous()
             qq, kk, vv = vec(q), vec(k), vec(v)
+            dq = torch.empty(q.shape, dtype=q.dtype, device=q.device)
             with torch.cuda.device(q.device):
                 _lib.call('flyhip_bs_sdd_prob_dsoftmax', dout.data_ptr(), vv.data_ptr(), qq.data_ptr(), kk.data_ptr(),
-                          delta.data_ptr(), lse2.data_ptr(), ds.data_ptr(), p.data_ptr(),
+                          delta.data_ptr(), lse2.data_ptr(), ds.data_ptr(), p.data_ptr(), dq.data_ptr(),
                           uni_ptr.data_ptr(), uni_inner.data_ptr(), uni_blk.data_ptr(),
                           nnz, H, rows, q.shape[0], q.shape[3], 32,
                           dout.stride(0), dout.stride(1), dout.stride(2), vv.stride(0), vv.stride(1), vv.stride(2),
                           qq.stride(0), qq.stride(1), qq.stride(2), kk.stride(0), kk.stride(1), kk.stride(2),
+                          dq.stride(0), dq.stride(1), dq.stride(2),
                           float(ctx.scale), _lib.dtype_code(q), _lib.stream_ptr(q.device))
             dv = dsd._run('dsd', p, dout, True, False, False)
         else:
+            dq = None
             q, k, v, p, out = ctx.saved_tensors
             dv = dsd._run('dsd', p, dout, True, False, False)
             delta = (dout.float() * out.float()).sum(-1).contiguous()
@@ -84,7 +87,8 @@ class _AttentionCoreFn(torch.autograd.Function):
                           p.shape[1], H, rows, q.shape[0], v.shape[3], 32,
                           dout.stride(0), dout.stride(1), dout.stride(2), vv.stride(0), vv.stride(1), vv.stride(2),
                           float(ctx.scale), _lib.dtype_code(q), _lib.stream_ptr(q.device))
-        dq = dsd._run('dsd', ds, k, False, False, False)
+        if dq is None:
+            dq = dsd._run('dsd', ds, k, False, False, False)
         dk = dsd._run('dsd', ds, q, True, False, False)
         return dq, dk, dv, None, None, None, None, None, None, None
 

@@ -196,6 +196,8 @@ struct SddUniArgs {
     // lse2[row]) is written to p2 and c = scale * p2 * (a b^T - delta[row])
     const void* a2; const void* b2; const float* lse2; void* p2; float scale2;
     long a2_sz, a2_sh, a2_sm, b2_sz, b2_sh, b2_sn;
+    // ... and the gradient of a2 on the way: dq = c b2 (rows of a2), accumulated over the row's blocks
+    void* dq; long dq_sz, dq_sh, dq_sm;
 };
 
 template <typename T, int KS, int EPI = 0>     // KS = K / 32; EPI: 0 product, 1 softmax gradient, 2 probabilities
@@ -206,6 +208,8 @@ __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
     constexpr int NCH = (32 * CPR + 255) / 256;         // chunks per thread
     __shared__ __attribute__((aligned(16))) uint16_t tile[2][32 * LD];
     __shared__ __attribute__((aligned(16))) uint16_t tile2[BOTH ? 2 : 1][BOTH ? 32 * LD : 8];
+    constexpr int LDT2 = 40;                            // row stride of the transposed copy: [feature][32 columns + pad]
+    __shared__ __attribute__((aligned(16))) uint16_t tile2t[BOTH ? 2 : 1][BOTH ? K * LDT2 : 8];
     const int tid = threadIdx.x, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     int unit, grp;
@@ -213,9 +217,16 @@ __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
     const int z = unit / a.n_heads, head = unit % a.n_heads;
     const int ug = head * a.grps_per_head + grp;
     const int p0 = a.uni_ptr[ug], n = a.uni_ptr[ug + 1] - p0;
-    if (n == 0) return;
     const int bi = grp * 4 + w;
     const bool have_row = bi < a.brows_per_head;
+    if (n == 0) {
+        if (EPI == 3 && have_row) {                     // rows without blocks: zero gradient
+            T* dqp = reinterpret_cast<T*>(a.dq) + z * a.dq_sz + head * a.dq_sh;
+            for (int e = lane; e < 32 * K / 4; e += 64)
+                store4_f32(dqp + (long)(bi * 32 + e / (K / 4)) * a.dq_sm + 4 * (e % (K / 4)), Frag<float>::zero());
+        }
+        return;
+    }
     const T* ap = reinterpret_cast<const T*>(a.a) + z * a.a_sz + head * a.a_sh +
                   (long)(min(bi, a.brows_per_head - 1) * 32 + r16) * a.a_sm + 8 * g;
     const T* bz = reinterpret_cast<const T*>(a.b) + z * a.b_sz + head * a.b_sh;
@@ -266,9 +277,21 @@ __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
             const int c = tid + 256 * i, nrow = c / CPR;
             const int lrow = 16 * ((nrow >> 2) & 1) + 4 * (nrow >> 3) + (nrow & 3);
             if (c < 32 * CPR) *reinterpret_cast<uintx4*>(&tile[buf][lrow * LD + 8 * (c % CPR)]) = reg[i];
-            if (BOTH && c < 32 * CPR) *reinterpret_cast<uintx4*>(&tile2[BOTH ? buf : 0][lrow * LD + 8 * (c % CPR)]) = reg2[BOTH ? i : 0];
+            if (BOTH && c < 32 * CPR) {
+                const uintx4 rv = reg2[BOTH ? i : 0];
+                *reinterpret_cast<uintx4*>(&tile2[BOTH ? buf : 0][lrow * LD + 8 * (c % CPR)]) = rv;
+                // transposed copy for dq = ds b2: [feature][column], natural column order
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    tile2t[BOTH ? buf : 0][(8 * (c % CPR) + e) * LDT2 + nrow] = (uint16_t)(rv[e >> 1] >> (16 * (e & 1)));
+            }
         }
     };
+    floatx4 dqa[BOTH ? 2 * KS : 1][2];                  // dq^T[feature 16dt + 4g + i][row 16tm + r16]
+    if (BOTH) {
+#pragma unroll
+        for (int dt = 0; dt < 2 * KS; ++dt) { dqa[BOTH ? dt : 0][0] = Frag<float>::zero(); dqa[BOTH ? dt : 0][1] = Frag<float>::zero(); }
+    }
     // the index lists are read two steps (block-column) and one step (block id) ahead of their use
     int inner_n1 = n > 1 ? a.uni_inner[p0 + 1] : 0;
     int blk = a.uni_blk[(long)p0 * 4 + w];
@@ -354,6 +377,15 @@ __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
                         }
                     T* pp2 = reinterpret_cast<T*>(a.p2) + ((long)z * a.nnz + blk) * 1024;
                     store8_f32(pp2 + (16 * tm + r16) * 32 + 8 * g, acc2[tm][0], acc2[tm][1]);
+                    // the lane's eight ds values are columns 8g .. 8g+7 of row 16tm + r16: an MFMA operand as they are
+                    const uintx4 dsb = {pack2<T>(acc[tm][0][0], acc[tm][0][1]), pack2<T>(acc[tm][0][2], acc[tm][0][3]),
+                                        pack2<T>(acc[tm][1][0], acc[tm][1][1]), pack2<T>(acc[tm][1][2], acc[tm][1][3])};
+                    const uint16_t* tt = tile2t[BOTH ? (s & 1) : 0];
+#pragma unroll
+                    for (int dt = 0; dt < 2 * KS; ++dt) {
+                        const uintx4 fk = *reinterpret_cast<const uintx4*>(tt + (16 * dt + r16) * LDT2 + 8 * g);
+                        dqa[BOTH ? dt : 0][tm] = mma32<T>(fk, dsb, dqa[BOTH ? dt : 0][tm]);
+                    }
                 }
                 if (PROB) {
                     const float dl = dlt[16 * tm];
@@ -369,6 +401,14 @@ __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
         inner_n1 = inner_n2;
         blk = blk_n1;
         __syncthreads();
+    }
+    if (BOTH && have_row) {
+        T* dqp = reinterpret_cast<T*>(a.dq) + z * a.dq_sz + head * a.dq_sh;
+#pragma unroll
+        for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+            for (int dt = 0; dt < 2 * KS; ++dt)
+                store4_f32(dqp + (long)(bi * 32 + 16 * tm + r16) * a.dq_sm + 16 * dt + 4 * g, dqa[BOTH ? dt : 0][tm]);
     }
 }
 
@@ -1750,6 +1790,9 @@ static int launch_sdd_epilogue(const char* what, const void* a_dn, const void* b
         ua.a2 = second->a2; ua.b2 = second->b2; ua.lse2 = second->lse2; ua.p2 = second->p2; ua.scale2 = second->scale2;
         ua.a2_sz = second->a2_sz; ua.a2_sh = second->a2_sh; ua.a2_sm = second->a2_sm;
         ua.b2_sz = second->b2_sz; ua.b2_sh = second->b2_sh; ua.b2_sn = second->b2_sn;
+        FLY_REQUIRE(second->dq && ((second->dq_sz | second->dq_sh | second->dq_sm) % 4) == 0,
+                    "%s: dq missing or its strides are not multiples of 4 elements", what);
+        ua.dq = second->dq; ua.dq_sz = second->dq_sz; ua.dq_sh = second->dq_sh; ua.dq_sm = second->dq_sm;
     }
     const long nwg = unit_grid((long)n_heads * Z, gph);
     FLY_REQUIRE(nwg <= 2147483647L, "%s: too many workgroups", what);
@@ -1777,15 +1820,17 @@ extern "C" int flyhip_bs_sdd_dsoftmax(const void* dout, const void* v, const voi
 }
 
 extern "C" int flyhip_bs_sdd_prob_dsoftmax(const void* dout, const void* v, const void* q, const void* k,
-                                           const float* delta, const float* lse2, void* ds, void* p,
+                                           const float* delta, const float* lse2, void* ds, void* p, void* dq,
                                            const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
                                            int nnz, int n_heads, int brows_per_head, int Z, int K, int blk,
                                            int64_t do_sz, int64_t do_sh, int64_t do_sm,
                                            int64_t v_sz, int64_t v_sh, int64_t v_sn,
                                            int64_t q_sz, int64_t q_sh, int64_t q_sm,
                                            int64_t k_sz, int64_t k_sh, int64_t k_sn,
+                                           int64_t dq_sz, int64_t dq_sh, int64_t dq_sm,
                                            float scale, int dtype, void* stream) {
     SddUniArgs second{};
+    second.dq = dq; second.dq_sz = dq_sz; second.dq_sh = dq_sh; second.dq_sm = dq_sm;
     second.a2 = q; second.b2 = k; second.lse2 = lse2; second.p2 = p; second.scale2 = scale * 1.4426950408889634f;
     second.a2_sz = q_sz; second.a2_sh = q_sh; second.a2_sm = q_sm;
     second.b2_sz = k_sz; second.b2_sh = k_sh; second.b2_sn = k_sn;

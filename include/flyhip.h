@@ -302,15 +302,17 @@ int flyhip_bs_sdd_prob(const void* q, const void* k, const float* lse2, void* p,
  * (q k^T and d out v^T) per block, p = exp(scale q k^T - lse) written to p and
  * ds = scale * p * (d out v^T - delta[row]) to ds, both (Z, nnz, 32, 32); neither the scores nor
  * d p exist in memory (the reference's autograd chain through blocksparse_attention.py:134-160
- * materialises both). */
+ * materialises both).  The gradient of q comes out of the same pass: dq = ds k over the row's blocks
+ * (Z, H, rows, K) through (batch, head, row) strides. */
 int flyhip_bs_sdd_prob_dsoftmax(const void* dout, const void* v, const void* q, const void* k,
-                                const float* delta, const float* lse2, void* ds, void* p,
+                                const float* delta, const float* lse2, void* ds, void* p, void* dq,
                                 const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
                                 int nnz, int n_heads, int brows_per_head, int Z, int K, int blk,
                                 int64_t do_sz, int64_t do_sh, int64_t do_sm,
                                 int64_t v_sz, int64_t v_sh, int64_t v_sn,
                                 int64_t q_sz, int64_t q_sh, int64_t q_sm,
                                 int64_t k_sz, int64_t k_sh, int64_t k_sn,
+                                int64_t dq_sz, int64_t dq_sh, int64_t dq_sm,
                                 float scale, int dtype, void* stream);
 
 /* ------------------------------------------------------------------------------------------
