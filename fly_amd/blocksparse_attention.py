@@ -54,24 +54,24 @@ class _AttentionCoreFn(torch.autograd.Function):
         def vec(x):          # 16-byte loads: last dim contiguous, other strides multiples of 8
             ok = x.stride(3) == 1 and all(s_ % 8 == 0 for s_ in x.stride()[:3]) and x.data_ptr() % 16 == 0
             return x if ok else x.contiguous()
-        dout = dout.contiguous()
+        dout = vec(dout)
         if ctx.recompute:
-            # probabilities and score gradient from one kernel: both products (q k^T, d out v^T) per block
+            # probabilities, score gradient, dq and the rows' delta = rowsum(d out * out) from one kernel: both
+            # products (q k^T, d out v^T) per block
             q, k, v, out, lse2 = ctx.saved_tensors
             nnz = int(sdd.layout.sum())
             p = torch.empty((q.shape[0], nnz, 32, 32), dtype=q.dtype, device=q.device)
             ds = torch.empty_like(p)
-            delta = (dout.float() * out.float()).sum(-1).contiguous()
-            qq, kk, vv = vec(q), vec(k), vec(v)
+            qq, kk, vv, oo = vec(q), vec(k), vec(v), vec(out)
             dq = torch.empty(q.shape, dtype=q.dtype, device=q.device)
             with torch.cuda.device(q.device):
                 _lib.call('flyhip_bs_sdd_prob_dsoftmax', dout.data_ptr(), vv.data_ptr(), qq.data_ptr(), kk.data_ptr(),
-                          delta.data_ptr(), lse2.data_ptr(), ds.data_ptr(), p.data_ptr(), dq.data_ptr(),
+                          None, oo.data_ptr(), lse2.data_ptr(), ds.data_ptr(), p.data_ptr(), dq.data_ptr(),
                           uni_ptr.data_ptr(), uni_inner.data_ptr(), uni_blk.data_ptr(),
                           nnz, H, rows, q.shape[0], q.shape[3], 32,
                           dout.stride(0), dout.stride(1), dout.stride(2), vv.stride(0), vv.stride(1), vv.stride(2),
                           qq.stride(0), qq.stride(1), qq.stride(2), kk.stride(0), kk.stride(1), kk.stride(2),
-                          dq.stride(0), dq.stride(1), dq.stride(2),
+                          dq.stride(0), dq.stride(1), dq.stride(2), oo.stride(0), oo.stride(1), oo.stride(2),
                           float(ctx.scale), _lib.dtype_code(q), _lib.stream_ptr(q.device))
             dv = dsd._run('dsd', p, dout, True, False, False)
         else:

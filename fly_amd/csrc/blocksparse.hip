@@ -198,6 +198,8 @@ struct SddUniArgs {
     long a2_sz, a2_sh, a2_sm, b2_sz, b2_sh, b2_sn;
     // ... and the gradient of a2 on the way: dq = c b2 (rows of a2), accumulated over the row's blocks
     void* dq; long dq_sz, dq_sh, dq_sm;
+    // ... with delta formed here when `out` is given (delta may then be null): rowsum(a * out), out laid out like a
+    const void* out; long o_sz, o_sh, o_sm;
 };
 
 template <typename T, int KS, int EPI = 0>     // KS = K / 32; EPI: 0 product, 1 softmax gradient, 2 probabilities
@@ -233,7 +235,7 @@ __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
     T* cz = reinterpret_cast<T*>(a.c) + (long)z * a.nnz * 1024;
     // DSOFT: this lane's rows are 16 tm + r16 of block-row bi
     const long rowvec_off = ((long)z * a.n_heads + head) * a.brows_per_head * 32 + (long)min(bi, a.brows_per_head - 1) * 32 + r16;
-    const float* dlt = (DSOFT || PROB || BOTH) ? a.delta + rowvec_off : nullptr;
+    const float* dlt = (DSOFT || PROB || (BOTH && a.delta)) ? a.delta + rowvec_off : nullptr;
     uintx4 fa[2][KS];
 #pragma unroll
     for (int tm = 0; tm < 2; ++tm)
@@ -251,7 +253,28 @@ __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) fa2[BOTH ? tm : 0][BOTH ? ks : 0] = *reinterpret_cast<const uintx4*>(ap2 + 16 * tm * a.a2_sm + 32 * ks);
             lse_row[tm] = a.lse2[rowvec_off + 16 * tm];
-            dl_row[tm] = dlt[16 * tm];
+            if (a.out) {
+                // delta = sum over the head dim of d out * out for this lane's row: the lane holds 8 KS of the
+                // row's values, the four lanes r16 + 16g the rest
+                const T* op = reinterpret_cast<const T*>(a.out) + z * a.o_sz + head * a.o_sh +
+                              (long)(min(bi, a.brows_per_head - 1) * 32 + 16 * tm + r16) * a.o_sm + 8 * g;
+                float part = 0.f;
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    const uintx4 ov = *reinterpret_cast<const uintx4*>(op + 32 * ks);
+                    const uintx4 gv = fa[tm][ks];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        T x, y;
+                        *reinterpret_cast<uint16_t*>(&x) = (uint16_t)(gv[e >> 1] >> (16 * (e & 1)));
+                        *reinterpret_cast<uint16_t*>(&y) = (uint16_t)(ov[e >> 1] >> (16 * (e & 1)));
+                        part += Elem<T>::to_f32(x) * Elem<T>::to_f32(y);
+                    }
+                }
+                dl_row[tm] = group_sum(part);
+            } else {
+                dl_row[tm] = dlt[16 * tm];
+            }
         }
         bz2 = reinterpret_cast<const T*>(a.b2) + z * a.b2_sz + head * a.b2_sh;
     }
@@ -1774,7 +1797,8 @@ static int launch_sdd_epilogue(const char* what, const void* a_dn, const void* b
                                float scale, int dtype, void* stream, const SddUniArgs* second = nullptr) {
     int rc = check_common(what, blk, dtype, Z);
     if (rc) return rc;
-    FLY_REQUIRE(a_dn && b_dn && (EPI != 1 || p) && rowvec && c && uni_ptr && uni_inner && uni_blk, "%s: null pointer", what);
+    FLY_REQUIRE(a_dn && b_dn && (EPI != 1 || p) && (rowvec || (EPI == 3 && second && second->out)) && c && uni_ptr &&
+                uni_inner && uni_blk, "%s: null pointer", what);
     FLY_REQUIRE(blk == 32 && (dtype == BF16 || dtype == F16), "%s: needs 32x32 blocks of bf16 / fp16", what);
     FLY_REQUIRE(K % 32 == 0 && K >= 32 && K <= 128, "%s: head dim %d not a multiple of 32 up to 128", what, K);
     FLY_REQUIRE(nnz > 0 && n_heads > 0 && brows_per_head > 0, "%s: bad sizes", what);
@@ -1793,6 +1817,9 @@ static int launch_sdd_epilogue(const char* what, const void* a_dn, const void* b
         FLY_REQUIRE(second->dq && ((second->dq_sz | second->dq_sh | second->dq_sm) % 4) == 0,
                     "%s: dq missing or its strides are not multiples of 4 elements", what);
         ua.dq = second->dq; ua.dq_sz = second->dq_sz; ua.dq_sh = second->dq_sh; ua.dq_sm = second->dq_sm;
+        FLY_REQUIRE(!second->out || ((second->o_sz | second->o_sh | second->o_sm) % 8) == 0,
+                    "%s: out strides must be multiples of 8 elements", what);
+        ua.out = second->out; ua.o_sz = second->o_sz; ua.o_sh = second->o_sh; ua.o_sm = second->o_sm;
     }
     const long nwg = unit_grid((long)n_heads * Z, gph);
     FLY_REQUIRE(nwg <= 2147483647L, "%s: too many workgroups", what);
@@ -1820,7 +1847,7 @@ extern "C" int flyhip_bs_sdd_dsoftmax(const void* dout, const void* v, const voi
 }
 
 extern "C" int flyhip_bs_sdd_prob_dsoftmax(const void* dout, const void* v, const void* q, const void* k,
-                                           const float* delta, const float* lse2, void* ds, void* p, void* dq,
+                                           const float* delta, const void* out, const float* lse2, void* ds, void* p, void* dq,
                                            const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
                                            int nnz, int n_heads, int brows_per_head, int Z, int K, int blk,
                                            int64_t do_sz, int64_t do_sh, int64_t do_sm,
@@ -1828,8 +1855,10 @@ extern "C" int flyhip_bs_sdd_prob_dsoftmax(const void* dout, const void* v, cons
                                            int64_t q_sz, int64_t q_sh, int64_t q_sm,
                                            int64_t k_sz, int64_t k_sh, int64_t k_sn,
                                            int64_t dq_sz, int64_t dq_sh, int64_t dq_sm,
+                                           int64_t o_sz, int64_t o_sh, int64_t o_sm,
                                            float scale, int dtype, void* stream) {
     SddUniArgs second{};
+    second.out = out; second.o_sz = o_sz; second.o_sh = o_sh; second.o_sm = o_sm;
     second.dq = dq; second.dq_sz = dq_sz; second.dq_sh = dq_sh; second.dq_sm = dq_sm;
     second.a2 = q; second.b2 = k; second.lse2 = lse2; second.p2 = p; second.scale2 = scale * 1.4426950408889634f;
     second.a2_sz = q_sz; second.a2_sh = q_sh; second.a2_sm = q_sm;

@@ -303,9 +303,10 @@ int flyhip_bs_sdd_prob(const void* q, const void* k, const float* lse2, void* p,
  * ds = scale * p * (d out v^T - delta[row]) to ds, both (Z, nnz, 32, 32); neither the scores nor
  * d p exist in memory (the reference's autograd chain through blocksparse_attention.py:134-160
  * materialises both).  The gradient of q comes out of the same pass: dq = ds k over the row's blocks
- * (Z, H, rows, K) through (batch, head, row) strides. */
+ * (Z, H, rows, K) through (batch, head, row) strides.  delta (Z, H, rows) float32 = rowsum(d out * out)
+ * may be NULL when out (the forward's result, strided like d out) is given: it is then formed here. */
 int flyhip_bs_sdd_prob_dsoftmax(const void* dout, const void* v, const void* q, const void* k,
-                                const float* delta, const float* lse2, void* ds, void* p, void* dq,
+                                const float* delta, const void* out, const float* lse2, void* ds, void* p, void* dq,
                                 const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
                                 int nnz, int n_heads, int brows_per_head, int Z, int K, int blk,
                                 int64_t do_sz, int64_t do_sh, int64_t do_sm,
@@ -313,6 +314,7 @@ int flyhip_bs_sdd_prob_dsoftmax(const void* dout, const void* v, const void* q, 
                                 int64_t q_sz, int64_t q_sh, int64_t q_sm,
                                 int64_t k_sz, int64_t k_sh, int64_t k_sn,
                                 int64_t dq_sz, int64_t dq_sh, int64_t dq_sm,
+                                int64_t o_sz, int64_t o_sh, int64_t o_sm,
                                 float scale, int dtype, void* stream);
 
 /* ------------------------------------------------------------------------------------------
