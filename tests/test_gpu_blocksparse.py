@@ -471,8 +471,9 @@ def test_dsd_with_transposed_sparse_operand(p, r, N, dtype):
     assert rel_err(out2.transpose(2, 3), ref) <= TOL[dtype]
 
 
-@pytest.mark.parametrize('masked,E', [(True, 64), (False, 64), (False, 32), (False, 128)])
-def test_blocksparse_attention_module_gradients(masked, E):
+@pytest.mark.parametrize('masked,E,dtype', [(True, 64, torch.bfloat16), (False, 64, torch.bfloat16), (False, 32, torch.bfloat16),
+                                            (False, 128, torch.bfloat16), (False, 64, torch.float16)])
+def test_blocksparse_attention_module_gradients(masked, E, dtype):
     """Training path of BlockSparseAttention for 2-byte inputs: one autograd node whose backward runs
     dV, the fused score gradient, dQ and dK on the tiled kernels; gradients against autograd through
     the oracle in float64 on the same rounded inputs.  With padded keys the forward is the three ops and
@@ -490,9 +491,9 @@ def test_blocksparse_attention_module_gradients(masked, E):
             return lay.unsqueeze(0).repeat(2, 1, 1)
 
     B, T, H = 2, 384, 2
-    print('case', masked, E, flush=True)
+    print('case', masked, E, dtype, flush=True)
     g = torch.Generator().manual_seed(8)
-    q, k, v = (torch.randn(B, T, H, E, generator=g).bfloat16() for _ in range(3))
+    q, k, v = (torch.randn(B, T, H, E, generator=g).to(dtype) for _ in range(3))
     w = torch.randn(B, T, H, E, generator=g)
     lengths = torch.tensor([T, 200]) if masked else None
     mod = BlockSparseAttention(Cfg(), attention_dropout=0.0, max_seq_length=512).to(DEV)
