@@ -442,8 +442,9 @@ __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
 // input features, 32x32 blocks of a 2-byte type.  One workgroup per (group of <= 4 consecutive
 // block-rows with identical column lists, chunk of <= 4 of their block-columns, slice of K): a
 // 128 x 128 output tile, the 2 x 2 waves owning 64 x 64 each.  Per step of 32 tokens the 32 x 128
-// tiles of A and B are loaded with 16-byte pieces along the features and written to LDS
-// transposed ([feature][token]), which makes every MFMA fragment one 16-byte LDS read; the
+// tiles of A and B are loaded with 16-byte pieces along the features and kept row-major in LDS; the
+// MFMA fragments, whose contraction index runs down the rows, are two transposing 8-byte LDS reads
+// each (ds_read_b64_tr_b16), so nothing is transposed with 2-byte stores; the
 // slices' partial blocks meet in an fp32 buffer through hardware float atomics (the caller zeroes
 // it and rounds it to the output type afterwards).
 struct SddKArgs {
@@ -453,13 +454,31 @@ struct SddKArgs {
     int per_head, K, k_slice, chunks, nnz;
     long a_sz, a_sh, a_sk, b_sz, b_sh, b_sk;
 };
-constexpr int SDDK_LD = 40;     // LDS row stride in elements ([feature][token], 32 tokens + 8)
+constexpr int SDDK_LD = 144;    // LDS row stride in elements ([token][128 features + 16]: the four token rows a
+                                // 16-lane group reads together start 32 bytes apart modulo 256)
+
+// Operand of a 16x16x32 MFMA whose contraction index runs down the rows of a row-major LDS tile
+// ([k][feature]): lane (r16, g) needs feature f0 + r16 at k = 8g .. 8g + 7.  ds_read_b64_tr_b16 hands a lane
+// the element column of a 16-lane group's 16 x 4 block of 2-byte values: with lane j of the group
+// pointing at row j / 4, columns 4 (j % 4) .. + 3, lane j receives column j of rows 0 .. 3.  Two such reads
+// (rows 8g .. 8g + 3 and 8g + 4 .. 8g + 7) make the eight k-slots; both operands of a product are built
+// this way, so their k-slots pair up.
+typedef short shortx4 __attribute__((ext_vector_type(4)));
+typedef unsigned int uintx2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uintx4 frag_down_rows(const uint16_t* tile, int ld, int f0, int r16, int g) {
+    const uint16_t* p = tile + (8 * g + (r16 >> 2)) * ld + f0 + 4 * (r16 & 3);
+    typedef __attribute__((address_space(3))) shortx4 lds_shortx4;
+    const shortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(p));
+    const shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(p + 4 * ld));
+    const uintx2 l = __builtin_bit_cast(uintx2, lo), h = __builtin_bit_cast(uintx2, hi);
+    return uintx4{l[0], l[1], h[0], h[1]};
+}
 
 template <typename T>
 __global__ __launch_bounds__(256) void bs_sdd32k_kernel(const SddKArgs a) {
     constexpr int LD = SDDK_LD;
-    __shared__ __attribute__((aligned(16))) uint16_t at[2][128 * LD];
-    __shared__ __attribute__((aligned(16))) uint16_t bt[2][128 * LD];
+    __shared__ __attribute__((aligned(16))) uint16_t at[2][32 * LD];
+    __shared__ __attribute__((aligned(16))) uint16_t bt[2][32 * LD];
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
     const int wm = w >> 1, wn = w & 1;
     const int grp = blockIdx.x / a.chunks, chunk = blockIdx.x % a.chunks, z = blockIdx.z;
@@ -473,42 +492,40 @@ __global__ __launch_bounds__(256) void bs_sdd32k_kernel(const SddKArgs a) {
     const uint16_t* ap = reinterpret_cast<const uint16_t*>(a.a) + z * a.a_sz + head * a.a_sh + (long)brow0 * 32;
     const uint16_t* bp = reinterpret_cast<const uint16_t*>(a.b) + z * a.b_sz + head * a.b_sh;
 
-    // staging: piece c = tid + 256 i (i < 2) of each tile is token c % 32, features 8 (c / 32) .. + 7 -- the
-    // token runs fastest over the lanes, so that the 2-byte stores that transpose the piece into
-    // [feature][token] spread over the LDS banks (with the feature fastest they pile onto four).
-    // Feature block c / 32 / 4 is output block-row ob (A) or list entry j0 + jb (B); absent blocks read
+    // staging: piece c = tid + 256 i (i < 2) of each 32-token x 128-feature tile is token c / 16, features
+    // 8 (c % 16) .. + 7: the tiles stay row-major ([token][feature]) in LDS, one 16-byte store per piece; the
+    // MFMA fragments -- tokens are the contraction index -- come out of them through the transposing read.
+    // Feature block (c % 16) / 4 is output block-row ob (A) or list entry j0 + jb (B); absent blocks read
     // block 0 of the tile and are zeroed when parked
     int fcol_a[2], fcol_b[2];                               // feature offset of the piece in its operand
     bool live_a[2], live_b[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-        const int c = tid + 256 * i, fb = (c >> 5) >> 2, f8 = 8 * ((c >> 5) & 3);
+        const int c = tid + 256 * i, fb = (c & 15) >> 2, f8 = 8 * (c & 3);
         live_a[i] = fb < gn;
         live_b[i] = fb < jn;
         fcol_a[i] = 32 * (live_a[i] ? fb : 0) + f8;
         fcol_b[i] = a.seg_inner[p0 + j0 + (live_b[i] ? fb : 0)] * 32 + f8;
     }
-    uintx4 ra[2], rb[2];
-    auto fetch = [&](int kt) __attribute__((always_inline)) {
+    // two register sets: the loads of step s+2 are issued while step s is multiplied and are parked in LDS
+    // one step later, so every global load has two steps to arrive (every fetch issues the same four
+    // loads per thread on every path, so the wait for the older set can leave the newer one in flight)
+    uintx4 ra0[2], rb0[2], ra1[2], rb1[2];
+    auto fetch = [&](int kt, uintx4 (&ra)[2], uintx4 (&rb)[2]) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-            const int tok = min(kt + ((tid + 256 * i) & 31), a.K - 1);     // clamped; tokens past k1 are zeroed below
+            const int tok = min(kt + ((tid + 256 * i) >> 4), a.K - 1);     // clamped; tokens past k1 are zeroed below
             ra[i] = *reinterpret_cast<const uintx4*>(ap + (long)tok * a.a_sk + fcol_a[i]);
             rb[i] = *reinterpret_cast<const uintx4*>(bp + (long)tok * a.b_sk + fcol_b[i]);
         }
     };
-    auto stash = [&](int buf, int kt) __attribute__((always_inline)) {
+    auto stash = [&](int buf, int kt, const uintx4 (&ra)[2], const uintx4 (&rb)[2]) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-            const int c = tid + 256 * i, tok = c & 31, f0 = 8 * (c >> 5);
+            const int c = tid + 256 * i, tok = c >> 4, f0 = 8 * (c & 15);
             const bool in = kt + tok < k1;
-            const uintx4 va = (live_a[i] && in) ? ra[i] : uintx4{0, 0, 0, 0};
-            const uintx4 vb = (live_b[i] && in) ? rb[i] : uintx4{0, 0, 0, 0};
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                at[buf][(f0 + e) * LD + tok] = (uint16_t)(va[e >> 1] >> (16 * (e & 1)));
-                bt[buf][(f0 + e) * LD + tok] = (uint16_t)(vb[e >> 1] >> (16 * (e & 1)));
-            }
+            *reinterpret_cast<uintx4*>(&at[buf][tok * LD + f0]) = (live_a[i] && in) ? ra[i] : uintx4{0, 0, 0, 0};
+            *reinterpret_cast<uintx4*>(&bt[buf][tok * LD + f0]) = (live_b[i] && in) ? rb[i] : uintx4{0, 0, 0, 0};
         }
     };
 
@@ -519,27 +536,35 @@ __global__ __launch_bounds__(256) void bs_sdd32k_kernel(const SddKArgs a) {
         for (int j = 0; j < 4; ++j) acc[i][j] = Frag<float>::zero();
     const bool wave_active = 2 * wm < gn && 2 * wn < jn;    // its output blocks exist
 
-    fetch(k0);
-    stash(0, k0);
-    drain_loads();
-    __syncthreads();
-    int buf = 0;
-    for (int kt = k0; kt < k1; kt += 32) {
-        fetch(min(kt + 32, a.K - 1));                      // (past the slice: loaded, zeroed, never used)
+    auto compute = [&](int buf) __attribute__((always_inline)) {
         if (wave_active) {
             uintx4 fa[4], fb[4];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                fa[i] = *reinterpret_cast<const uintx4*>(&at[buf][(64 * wm + 16 * i + r16) * LD + 8 * g]);
-                fb[i] = *reinterpret_cast<const uintx4*>(&bt[buf][(64 * wn + 16 * i + r16) * LD + 8 * g]);
+                fa[i] = frag_down_rows(at[buf], LD, 64 * wm + 16 * i, r16, g);
+                fb[i] = frag_down_rows(bt[buf], LD, 64 * wn + 16 * i, r16, g);
             }
 #pragma unroll
             for (int i = 0; i < 4; ++i)
 #pragma unroll
                 for (int j = 0; j < 4; ++j) acc[i][j] = mma32<T>(fa[i], fb[j], acc[i][j]);
         }
-        stash(buf ^ 1, kt + 32);
-        buf ^= 1;
+    };
+    fetch(k0, ra0, rb0);
+    stash(0, k0, ra0, rb0);
+    fetch(k0 + 32, ra1, rb1);                               // set 1 holds odd steps, set 0 even steps
+    drain_loads_but<4>();                                   // only set 1 (four loads a thread) is in flight
+    __syncthreads();
+    for (int kt = k0; kt < k1; kt += 64) {
+        fetch(kt + 64, ra0, rb0);                           // (past the slice: loaded, zeroed, never used)
+        compute(0);
+        stash(1, kt + 32, ra1, rb1);
+        drain_loads_but<4>();                               // set 1 is parked: only set 0 is in flight
+        __syncthreads();
+        fetch(kt + 96, ra1, rb1);
+        if (kt + 32 < k1) compute(1);
+        stash(0, kt + 64, ra0, rb0);
+        drain_loads_but<4>();
         __syncthreads();
     }
     if (!wave_active) return;
