@@ -175,6 +175,27 @@ __global__ __launch_bounds__(256) void bs_sdd32_kernel(const SddRowArgs a) {
     }
 }
 
+// Operand of a 16x16x32 MFMA whose contraction index runs down the rows of a row-major LDS tile
+// ([k][feature]): lane (r16, g) needs feature f0 + r16 at k = 8g .. 8g + 7.  ds_read_b64_tr_b16 hands a lane
+// the element column of a 16-lane group's 16 x 4 block of 2-byte values: with lane j of the group
+// pointing at some row (its choice) for k-slot j / 4, columns 4 (j % 4) .. + 3, lane j receives column j of the
+// four rows.  Two such reads (k-slots 8g .. 8g + 3 and 8g + 4 .. 8g + 7) make the eight k-slots; row_lo /
+// row_hi are the LDS rows that hold k = 8g + r16 / 4 and k = 8g + 4 + r16 / 4 (tiles may keep their rows
+// in any order).
+typedef short shortx4 __attribute__((ext_vector_type(4)));
+typedef unsigned int uintx2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uintx4 frag_down_rows_at(const uint16_t* tile, int ld, int f0, int r16, int row_lo, int row_hi) {
+    typedef __attribute__((address_space(3))) shortx4 lds_shortx4;
+    const uint16_t* p = tile + f0 + 4 * (r16 & 3);
+    const shortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(p + row_lo * ld));
+    const shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(p + row_hi * ld));
+    const uintx2 l = __builtin_bit_cast(uintx2, lo), h = __builtin_bit_cast(uintx2, hi);
+    return uintx4{l[0], l[1], h[0], h[1]};
+}
+__device__ __forceinline__ uintx4 frag_down_rows(const uint16_t* tile, int ld, int f0, int r16, int g) {
+    return frag_down_rows_at(tile, ld, f0, r16, 8 * g + (r16 >> 2), 8 * g + 4 + (r16 >> 2));
+}
+
 // SDD for layouts whose neighbouring block-rows share most of their columns (band and butterfly
 // patterns do): one workgroup per (batch, head, four consecutive block-rows), wave w owning row
 // 4*group + w with its A fragments in registers.  The workgroup walks the union of the four
@@ -210,8 +231,6 @@ __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
     constexpr int NCH = (32 * CPR + 255) / 256;         // chunks per thread
     __shared__ __attribute__((aligned(16))) uint16_t tile[2][32 * LD];
     __shared__ __attribute__((aligned(16))) uint16_t tile2[BOTH ? 2 : 1][BOTH ? 32 * LD : 8];
-    constexpr int LDT2 = 40;                            // row stride of the transposed copy: [feature][32 columns + pad]
-    __shared__ __attribute__((aligned(16))) uint16_t tile2t[BOTH ? 2 : 1][BOTH ? K * LDT2 : 8];
     const int tid = threadIdx.x, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     int unit, grp;
@@ -300,14 +319,7 @@ __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
             const int c = tid + 256 * i, nrow = c / CPR;
             const int lrow = 16 * ((nrow >> 2) & 1) + 4 * (nrow >> 3) + (nrow & 3);
             if (c < 32 * CPR) *reinterpret_cast<uintx4*>(&tile[buf][lrow * LD + 8 * (c % CPR)]) = reg[i];
-            if (BOTH && c < 32 * CPR) {
-                const uintx4 rv = reg2[BOTH ? i : 0];
-                *reinterpret_cast<uintx4*>(&tile2[BOTH ? buf : 0][lrow * LD + 8 * (c % CPR)]) = rv;
-                // transposed copy for dq = ds b2: [feature][column], natural column order
-#pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    tile2t[BOTH ? buf : 0][(8 * (c % CPR) + e) * LDT2 + nrow] = (uint16_t)(rv[e >> 1] >> (16 * (e & 1)));
-            }
+            if (BOTH && c < 32 * CPR) *reinterpret_cast<uintx4*>(&tile2[BOTH ? buf : 0][lrow * LD + 8 * (c % CPR)]) = reg2[BOTH ? i : 0];
         }
     };
     floatx4 dqa[BOTH ? 2 * KS : 1][2];                  // dq^T[feature 16dt + 4g + i][row 16tm + r16]
@@ -403,10 +415,15 @@ __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
                     // the lane's eight ds values are columns 8g .. 8g+7 of row 16tm + r16: an MFMA operand as they are
                     const uintx4 dsb = {pack2<T>(acc[tm][0][0], acc[tm][0][1]), pack2<T>(acc[tm][0][2], acc[tm][0][3]),
                                         pack2<T>(acc[tm][1][0], acc[tm][1][1]), pack2<T>(acc[tm][1][2], acc[tm][1][3])};
-                    const uint16_t* tt = tile2t[BOTH ? (s & 1) : 0];
+                    // ... against the b2 tile read down its rows (block column n sits in LDS row
+                    // 16 ((n >> 2) & 1) + 4 (n >> 3) + (n & 3), see the staging)
+                    const uint16_t* tt = tile2[BOTH ? (s & 1) : 0];
+                    const int n_lo = 8 * g + (r16 >> 2), n_hi = n_lo + 4;
+                    const int row_lo = 16 * ((n_lo >> 2) & 1) + 4 * (n_lo >> 3) + (n_lo & 3);
+                    const int row_hi = 16 * ((n_hi >> 2) & 1) + 4 * (n_hi >> 3) + (n_hi & 3);
 #pragma unroll
                     for (int dt = 0; dt < 2 * KS; ++dt) {
-                        const uintx4 fk = *reinterpret_cast<const uintx4*>(tt + (16 * dt + r16) * LDT2 + 8 * g);
+                        const uintx4 fk = frag_down_rows_at(tt, LD, 16 * dt, r16, row_lo, row_hi);
                         dqa[BOTH ? dt : 0][tm] = mma32<T>(fk, dsb, dqa[BOTH ? dt : 0][tm]);
                     }
                 }
@@ -456,23 +473,6 @@ struct SddKArgs {
 };
 constexpr int SDDK_LD = 144;    // LDS row stride in elements ([token][128 features + 16]: the four token rows a
                                 // 16-lane group reads together start 32 bytes apart modulo 256)
-
-// Operand of a 16x16x32 MFMA whose contraction index runs down the rows of a row-major LDS tile
-// ([k][feature]): lane (r16, g) needs feature f0 + r16 at k = 8g .. 8g + 7.  ds_read_b64_tr_b16 hands a lane
-// the element column of a 16-lane group's 16 x 4 block of 2-byte values: with lane j of the group
-// pointing at row j / 4, columns 4 (j % 4) .. + 3, lane j receives column j of rows 0 .. 3.  Two such reads
-// (rows 8g .. 8g + 3 and 8g + 4 .. 8g + 7) make the eight k-slots; both operands of a product are built
-// this way, so their k-slots pair up.
-typedef short shortx4 __attribute__((ext_vector_type(4)));
-typedef unsigned int uintx2 __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ uintx4 frag_down_rows(const uint16_t* tile, int ld, int f0, int r16, int g) {
-    const uint16_t* p = tile + (8 * g + (r16 >> 2)) * ld + f0 + 4 * (r16 & 3);
-    typedef __attribute__((address_space(3))) shortx4 lds_shortx4;
-    const shortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(p));
-    const shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(p + 4 * ld));
-    const uintx2 l = __builtin_bit_cast(uintx2, lo), h = __builtin_bit_cast(uintx2, hi);
-    return uintx4{l[0], l[1], h[0], h[1]};
-}
 
 template <typename T>
 __global__ __launch_bounds__(256) void bs_sdd32k_kernel(const SddKArgs a) {
