@@ -279,6 +279,25 @@ def bench_other_configs():
     out['config1_sblocal_fp32_fwd_bwd_ms'] = timeit(sblocal_train_step(q, k, v, P, lc, None), n=10)
     del q, k, v
 
+    # Scatterbrain on a block-sparse support at the first T2T layer's size (the sbbs-* attention configs:
+    # block 32, three sliding-window blocks, 32 features; here with one global block row / column)
+    class WindowPlusGlobal:
+        block = 32
+
+        def make_layout(self, seqlen):
+            nb = seqlen // self.block
+            r = torch.arange(nb)
+            lay = ((r.view(-1, 1) - r.view(1, -1)).abs() <= 1).long()
+            lay[:, 0] = 1
+            lay[0, :] = 1
+            return lay.unsqueeze(0)
+    B, L, E = 64, 3136, 64
+    sbbs = fly_amd.SBBlockSparseAttention(WindowPlusGlobal(), dim_heads=E, nb_features=32, max_seq_length=L).to(dev)
+    q, k, v = (torch.randn(B, L, 1, E, generator=g).to(dev) * E ** -0.25 for _ in range(3))
+    with torch.no_grad():
+        out['sbblocksparse_fp32_B64_L3136_block32_m32'] = {'ms': timeit(lambda: sbbs(q, k, v), n=5)}
+    del q, k, v, sbbs
+
     cfg = fly_amd.FlatBlockButterflySparsityConfig(8, 2, block=32)
     torch.manual_seed(0)
     fc1 = fly_amd.BlockSparseLinear(768, 3072, cfg, bias=False).to(dev).to(torch.bfloat16)

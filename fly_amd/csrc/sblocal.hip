@@ -75,6 +75,10 @@ struct FwdArgs {
     int B, H, T, S, mh_valid, lc, n_chunks, n_parts;
     long q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss;
     float temp;
+    // block-sparse support instead of a band (32 x 32 blocks; the fp32 kernel's LIST variant): per (head,
+    // 64-query tile) the key blocks its two block-rows touch -- tl_ptr (H * tiles + 1), tl_inner (block
+    // column per entry), tl_blk (2 per entry: block id of block-row 2 tile, 2 tile + 1, or -1 if absent)
+    const int32_t* tl_ptr; const int32_t* tl_inner; const int32_t* tl_blk;
 };
 
 // ROWS x W tile of a (seq, W) matrix, moved global -> registers -> LDS in two steps so that all of
@@ -1407,8 +1411,9 @@ __global__ __launch_bounds__(NT) void local_fwd_kernel(LocalArgs a) {
 // ---------------------------------------------------------------------------------------
 // fused band kernel
 // ---------------------------------------------------------------------------------------
-template <typename T, int E, int D, int M, bool SPLIT>
+template <typename T, int E, int D, int M, bool SPLIT, bool LIST = false>
 __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
+    static_assert(!(SPLIT && LIST), "the block-sparse support runs with one part per query tile");
     constexpr int MH = M / 2, LDK = E + 4, LDV = D + 4, LDF = M + 4;
     constexpr int FB = MH / 16, EC = E / 16, DB = D / 16, KB = TK / 16;
     constexpr int STAGE = TK * (LDK + LDV + LDF);     // floats per LDS stage
@@ -1460,6 +1465,23 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
         kt_lo = first;
         kt_hi = first + base + (part < extra ? 1 : 0);
     }
+    // LIST: the loop counter walks the tile's list of key blocks instead of a range of key tiles (a key
+    // block is a key tile: both are 32 keys); the block column and this wave's presence flag of an entry
+    // are read one iteration ahead of their use
+    const int32_t* tl_inner = nullptr;
+    const int32_t* tl_blk = nullptr;
+    int tile_cur = 0, tile_next = 0;
+    bool pres_cur = false, pres_next = false, seen_block = false;
+    if (LIST) {
+        const int lp0 = a.tl_ptr[h * n_qt + qt];
+        kt_lo = 0;
+        kt_hi = a.tl_ptr[h * n_qt + qt + 1] - lp0;
+        tl_inner = a.tl_inner + lp0;
+        tl_blk = a.tl_blk + 2 * (long)lp0 + (w >> 1);       // waves 0, 1: block-row 2 qt; waves 2, 3: 2 qt + 1
+        if (kt_hi > 0) { tile_cur = tl_inner[0]; pres_cur = tl_blk[0] >= 0; }
+        if (kt_hi > 1) { tile_next = tl_inner[1]; pres_next = tl_blk[2] >= 0; }
+    }
+    const int first_tile = LIST ? tile_cur : kt_lo;
 
     // start the first tile's loads before anything else
     RowTile<TK, E> rk;
@@ -1467,9 +1489,9 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
     RowTile<TK, M> rf;
     const int f_last = a.n_chunks * CH - 1;
     if (kt_lo < kt_hi) {
-        rk.fetch(kptr, a.k_ss, kt_lo * TK, a.S - 1, tid);
-        rv.fetch(vptr, a.v_ss, kt_lo * TK, a.S - 1, tid);
-        rf.fetch(fptr, M, kt_lo * TK, f_last, tid);
+        rk.fetch(kptr, a.k_ss, first_tile * TK, a.S - 1, tid);
+        rv.fetch(vptr, a.v_ss, first_tile * TK, a.S - 1, tid);
+        rf.fetch(fptr, M, first_tile * TK, f_last, tid);
     }
     // tiles after the first: per-thread offsets once, then one load per piece from the tile's base
     // (tiles that run past the last key row keep the clamping fetch)
@@ -1478,7 +1500,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
     rv.template offsets<T>(offv, a.v_ss, tid);
     rf.template offsets<float>(offf, M, tid);
     const float* csp = a.chunk_scale + (long)bh * a.n_chunks;
-    float cscale = (kt_lo < kt_hi) ? csp[kt_lo * TK / CH] : 0.f;
+    float cscale = (kt_lo < kt_hi) ? csp[first_tile * TK / CH] : 0.f;
     const float kmax = SPLIT ? split_kmax(a.part_max, bh, a.n_split) : a.kmax[bh];
 
     // query operand (B side: column = query, k = 16c+4g+j) and its squared norm
@@ -1565,24 +1587,29 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
 
     FLY_PROF(2);
     for (int kt = kt_lo; kt < kt_hi; ++kt) {
-        const int s_base = kt * TK;
+        const int s_base = (LIST ? tile_cur : kt) * TK;
+        const int s_next = LIST ? tile_next * TK : s_base + TK;      // first key of the next tile
         const int cur = (kt - kt_lo) & 1;
         const float* Ks = smem + cur * STAGE;
         const float* Vs = Ks + TK * LDK;
         const float* Fs = Vs + TK * LDV;
         const bool more = kt + 1 < kt_hi;
         float cscale_next = cscale;
+        // LIST: the entry after the next one (block column, presence) is requested now
+        int tile_n2 = 0;
+        bool pres_n2 = false;
+        if (LIST && kt + 2 < kt_hi) { tile_n2 = tl_inner[kt + 2]; pres_n2 = tl_blk[2 * (kt + 2)] >= 0; }
         if (more) {                                      // next tile's loads fly during the MFMAs
-            if (s_base + 2 * TK <= a.S) {
-                rk.fetch_fast(kptr + (long)(s_base + TK) * a.k_ss, offk, tid);
-                rv.fetch_fast(vptr + (long)(s_base + TK) * a.v_ss, offv, tid);
-                rf.fetch_fast(fptr + (long)(s_base + TK) * M, offf, tid);
+            if (s_next + TK <= a.S) {
+                rk.fetch_fast(kptr + (long)s_next * a.k_ss, offk, tid);
+                rv.fetch_fast(vptr + (long)s_next * a.v_ss, offv, tid);
+                rf.fetch_fast(fptr + (long)s_next * M, offf, tid);
             } else {
-                rk.fetch(kptr, a.k_ss, s_base + TK, a.S - 1, tid);
-                rv.fetch(vptr, a.v_ss, s_base + TK, a.S - 1, tid);
-                rf.fetch(fptr, M, s_base + TK, f_last, tid);
+                rk.fetch(kptr, a.k_ss, s_next, a.S - 1, tid);
+                rv.fetch(vptr, a.v_ss, s_next, a.S - 1, tid);
+                rf.fetch(fptr, M, s_next, f_last, tid);
             }
-            cscale_next = csp[(s_base + TK) / CH];
+            cscale_next = csp[s_next / CH];
         }
         // weight of this chunk's features relative to the global key stabiliser (<= 1); the same
         // expression weights the chunk in the combine role
@@ -1590,7 +1617,8 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
 
         // wave-uniform: does this tile touch the band of any of the wave's 16 queries?  (Blocks of a
         // touched tile that lie outside the band are computed and masked: no branches among the MFMAs.)
-        const bool any = !(s_base + TK - 1 - qw0 < -lc_lo || s_base - (qw0 + 15) >= lc_hi || s_base >= len);
+        const bool any = LIST ? pres_cur
+                              : !(s_base + TK - 1 - qw0 < -lc_lo || s_base - (qw0 + 15) >= lc_hi || s_base >= len);
         if (any) {
             // scores^T: s1 = (t log2e) K q, s2 = K' q'.  The accumulation chains of the two key
             // blocks and of the two products are interleaved so that no MFMA waits on its predecessor.
@@ -1619,8 +1647,9 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
             // lane holds the scores of query iq against keys s_base + 16kb + 4g + i.  A tile that lies
             // inside the band of all 16 queries of the wave and below the key length (wave-uniform) needs
             // no masks.
-            const bool interior = s_base - (qw0 + 15) >= -lc_lo && s_base + TK - 1 - qw0 < lc_hi &&
-                                  s_base + TK <= len && qw0 + 15 < a.T;
+            // (LIST: a present block is wholly visible; the caller guarantees whole blocks of keys and queries)
+            const bool interior = LIST || (s_base - (qw0 + 15) >= -lc_lo && s_base + TK - 1 - qw0 < lc_hi &&
+                                           s_base + TK <= len && qw0 + 15 < a.T);
             floatx4 p[KB];
             float ovs = 0.f;
             auto soft = [&](auto masked_tag) __attribute__((always_inline)) {
@@ -1678,7 +1707,14 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
             rf.template stash<LDF>(nxt + TK * (LDK + LDV), tid);
         }
         cscale = cscale_next;
+        if (LIST) { seen_block |= pres_cur; tile_cur = tile_next; tile_next = tile_n2; pres_cur = pres_next; pres_next = pres_n2; }
         __syncthreads();
+    }
+    if (LIST && !seen_block) {
+        // A block-row without any block: the reference's row logsumexp returns 0 there, not -inf
+        // (blocksparse_logsumexp.py:132), so its normaliser carries an extra exp(0); reproduced.
+        m_run = fmaxf(m_run, 0.f);
+        ze = g == 0 ? __builtin_amdgcn_exp2f(-m_run) : 0.f;
     }
 
     FLY_PROF(3);
@@ -1943,6 +1979,27 @@ static int launch_fwd_impl(const FwdArgs& a, hipStream_t st) {
 template <typename T, int E, int M>
 static int launch_fwd(const FwdArgs& a, hipStream_t st) {
     return a.n_parts > 1 ? launch_fwd_impl<T, E, M, true>(a, st) : launch_fwd_impl<T, E, M, false>(a, st);
+}
+
+// fp32 kernel on a block-sparse support (lists of key blocks per query tile), one part per tile
+template <typename T, int E, int M>
+static int launch_fwd_list(const FwdArgs& a, hipStream_t st) {
+    auto kern = sblocal_fwd_kernel<float, E, E, M, false, true>;
+    constexpr size_t smem = fwd_smem<E, M>();
+    static bool lds_ready = false;
+    if (!lds_ready) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return fail(ERR_LAUNCH, "sbblocksparse_fwd: LDS attribute: %s", hipGetErrorString(e));
+        lds_ready = true;
+    }
+    const long items = (long)a.B * a.H * ((a.T + TQ - 1) / TQ);
+    const long grid = (items + N_XCD - 1) / N_XCD * N_XCD;
+    if (grid > 2147483647L) return fail(ERR_ARG, "sbblocksparse_fwd: too many workgroups");
+    FwdArgs args = a;
+    args.band_wgs = (int)grid;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NT), smem, st, args);
+    return check_launch("sblocal_fwd_kernel (block-sparse support)");
 }
 
 template <typename T, int E>
@@ -2457,8 +2514,41 @@ extern "C" int flyhip_sblocal_fwd(const void* q, const void* k, const void* v, c
     plan(B, H, S, &nc, &ns);
     FwdArgs a{q, k, v, proj, kfeat, chunk_scale, kv, ksum, kmax, qfeat, q_lsq, vt, kvt, kv_part, part_max, n_split, 0, 1, key_lengths, out, log_norm, part_ws,
               B, H, T, S, mh_valid, local_context, nc, n_parts,
-              q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss, softmax_temp};
+              q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss, softmax_temp,
+              nullptr, nullptr, nullptr};
     return dispatch_fwd(dtype, E, 2 * mh, a, reinterpret_cast<hipStream_t>(stream));
+}
+
+extern "C" int flyhip_sbblocksparse_fwd(const void* q, const void* k, const void* v, const float* proj,
+                                        const void* kfeat, const float* chunk_scale,
+                                        const float* kv, const float* ksum, const float* kmax,
+                                        const int32_t* tl_ptr, const int32_t* tl_inner, const int32_t* tl_blk,
+                                        void* out, float* log_norm,
+                                        int B, int H, int T, int S, int E, int D, int mh, int mh_valid,
+                                        int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                                        int64_t k_sb, int64_t k_sh, int64_t k_ss,
+                                        int64_t v_sb, int64_t v_sh, int64_t v_ss,
+                                        int64_t o_sb, int64_t o_sh, int64_t o_ss,
+                                        float softmax_temp, int dtype, void* stream) {
+    FLY_REQUIRE(q && k && v && proj && kfeat && chunk_scale && kv && ksum && kmax && tl_ptr && tl_inner && tl_blk &&
+                out && log_norm, "sbblocksparse_fwd: null pointer");
+    FLY_REQUIRE(B > 0 && H > 0 && T > 0 && S > 0, "sbblocksparse_fwd: empty problem");
+    FLY_REQUIRE(T % 32 == 0 && S % 32 == 0, "sbblocksparse_fwd: sequence lengths %d, %d must be multiples of the block size 32", T, S);
+    FLY_REQUIRE(softmax_temp > 0.f, "sbblocksparse_fwd: softmax_temp must be positive");
+    FLY_REQUIRE(dtype == F32, "sbblocksparse_fwd: float32 inputs only (got dtype code %d)", dtype);
+    int rc = check_sb_dims("sbblocksparse_fwd", E, D, mh, mh_valid, dtype, q_sb | q_sh | q_ss | k_sb | k_sh | k_ss,
+                           v_sb | v_sh | v_ss, o_sb | o_sh | o_ss);
+    if (rc) return rc;
+    int nc, ns;
+    plan(B, H, S, &nc, &ns);
+    FwdArgs a{q, k, v, proj, kfeat, chunk_scale, kv, ksum, kmax, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 1,
+              nullptr, out, log_norm, nullptr,
+              B, H, T, S, mh_valid, 1, nc, 1,
+              q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss, softmax_temp,
+              tl_ptr, tl_inner, tl_blk};
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    const int m = 2 * mh;
+    SB_DISPATCH_E(launch_fwd_list, float, a)
 }
 
 extern "C" int flyhip_local_fwd_lse(const void* q, const void* k, const void* v, const int64_t* key_lengths, void* out,

@@ -15,7 +15,8 @@ from torch import distributed as dist
 from .blocksparse_attention import instantiate
 from .blocksparse_matmul import matmul
 from .blocksparse_softmax import blocksparse_sum, logsumexp
-from .blocksparse_utils import densify_tensor, sparsify_broadcast_tensor
+from .blocksparse_utils import densify_tensor, sparsify_broadcast_tensor, union_table
+from .sblocal_attention import sbblocksparse_forward, sbblocksparse_forward_supported
 from .feature_maps_sb import SBPerformerFeatures
 from .padding import pad_to_multiple
 from .scatterbrain_utils import linear_attention, linear_attention_normalization
@@ -46,6 +47,9 @@ class SBBlockSparseAttention(nn.Module):
         self._need_layout_synchronization = True
         self.ops_cache = dict()
         self._layout_cache = dict()
+        self.fused_tables = dict()
+        # eligible forward passes run on the fused kernels; set to False to force the op-by-op path
+        self.fuse = True
 
     def get_layout(self, T, S=None):
         if S is None:
@@ -97,6 +101,24 @@ class SBBlockSparseAttention(nn.Module):
         B, T, H, E = query.shape
         S = value.shape[1]
         softmax_temp = self.softmax_temp or 1 / math.sqrt(E)       # :131
+
+        # 32 x 32 blocks, float32, nothing but the output wanted: the whole forward on the fused kernels of
+        # Scatterbrain-local attention, walking the layout's blocks instead of a band
+        self.feature_map.new_feature_map(query.device)
+        layout = self.get_layout(T, S)
+        needs_grad = torch.is_grad_enabled() and any(x.requires_grad for x in (query, key, value))
+        if (self.fuse and not need_weights and not needs_grad and not (self.training and self.dropout.p > 0)
+                and self.softmax_eps == 0
+                and query.dtype in (torch.float32, torch.bfloat16, torch.float16)
+                and sbblocksparse_forward_supported(block, torch.float32, E, value.shape[3],
+                                                    self.feature_map.projection_matrix.shape[0], layout.shape[0], H)):
+            key_ = (T, S, query.device)
+            if key_ not in self.fused_tables:
+                self.fused_tables[key_] = tuple(x.to(query.device) for x in union_table(layout, rows_per_group=2))
+            # (2-byte inputs are widened, as on the op-by-op path below)
+            out, _ = sbblocksparse_forward(query.float(), key.float(), value.float(),
+                                           self.feature_map.projection_matrix, self.fused_tables[key_], softmax_temp)
+            return out.to(query.dtype), None
 
         # 2-byte inputs are widened: the scores pass through HBM between the stages, and a score kept
         # in bf16 (three significant digits, values of order 10) would cost percents in its exponential

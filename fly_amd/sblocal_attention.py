@@ -97,6 +97,24 @@ class SBLocalPlan:
                   v.stride(0), v.stride(2), v.stride(1), out.stride(0), out.stride(2), out.stride(1),
                   t, self.code, stream)
 
+    def run_block_sparse(self, q, k, v, proj, t, tables, out, log_norm):
+        """Scatterbrain attention whose exact part lives on a block-sparse support instead of a band: the
+        key pass as in ``run``, then the fp32 band kernel walking lists of 32-key blocks (``tables`` =
+        union_table(layout, rows_per_group=2) on the device).  One part per query tile, no key lengths."""
+        B, H, T, S, dim, mh, mh_valid = self.shape
+        tl_ptr, tl_inner, tl_blk = tables
+        with torch.cuda.device(self.device):
+            stream = _lib.stream_ptr(self.device)
+            self.run_keys(q, k, v, proj, None, t, stream)
+            _lib.call('flyhip_sbblocksparse_fwd', q.data_ptr(), k.data_ptr(), v.data_ptr(), proj.data_ptr(),
+                      self.kfeat.data_ptr(), self.chunk_scale.data_ptr(), self.kv.data_ptr(),
+                      self.ksum.data_ptr(), self.kmax.data_ptr(), tl_ptr.data_ptr(), tl_inner.data_ptr(),
+                      tl_blk.data_ptr(), out.data_ptr(), log_norm.data_ptr(),
+                      B, H, T, S, dim, dim, mh, mh_valid,
+                      q.stride(0), q.stride(2), q.stride(1), k.stride(0), k.stride(2), k.stride(1),
+                      v.stride(0), v.stride(2), v.stride(1), out.stride(0), out.stride(2), out.stride(1),
+                      t, self.code, stream)
+
     def run(self, q, k, v, proj, lens, local_context, t, out, log_norm):
         with torch.cuda.device(self.device):
             stream = _lib.stream_ptr(self.device)
@@ -151,6 +169,42 @@ def sblocal_forward(query, key, value, projection_matrix, local_context, softmax
     out = torch.empty(B, T, H, dim, dtype=query.dtype, device=query.device)
     log_norm = torch.empty(B, H, T, dtype=torch.float32, device=query.device)
     plan.run(q, k, v, proj, lens, local_context, t, out, log_norm)
+    return out[..., :D], log_norm.unsqueeze(-1)
+
+
+def sbblocksparse_forward_supported(block, dtype, E, D, n_projection_rows, layout_heads, H):
+    """Whether sbblocksparse_forward applies: 32 x 32 blocks, float32, one layout per attention head."""
+    return (block == 32 and dtype == torch.float32 and max(E, D) <= _HEAD_DIMS[-1]
+            and n_projection_rows <= _FEATURE_ROWS[-1] and layout_heads == H)
+
+
+def sbblocksparse_forward(query, key, value, projection_matrix, tables, softmax_temp=None):
+    """Scatterbrain attention on a block-sparse support (sbblocksparse_attention.py:109-213 for
+    need_weights=False, no dropout) on the fused kernels: exact softmax weights on the nonzero 32 x 32
+    blocks, the Performer estimate everywhere else, one normaliser.  query (B,T,H,E), key (B,S,H,E), value
+    (B,S,H,D) float32 GPU tensors, T and S multiples of 32; tables = union_table(layout, rows_per_group=2)
+    as int32 tensors on the device.  Returns (out (B,T,H,D), log_normalization (B,H,T,1))."""
+    _lib.require_gpu(query, key, value, projection_matrix)
+    B, T, H, E = query.shape
+    S, D = key.shape[1], value.shape[3]
+    if T % 32 or S % 32:
+        raise ValueError(f'sequence lengths {T}, {S} must be multiples of the block size 32')
+    t = softmax_temp or 1 / math.sqrt(E)
+    dim = _round_up_choice(max(E, D), _HEAD_DIMS, 'head dimension')
+    mh_valid = projection_matrix.shape[0]
+    mh = _round_up_choice(mh_valid, _FEATURE_ROWS, 'number of projection rows')
+
+    def prep(x):
+        if x.shape[-1] != dim:
+            x = F.pad(x, (0, dim - x.shape[-1]))
+        return x if _vector_ready(x) else x.contiguous()
+    q, k, v = prep(query), prep(key), prep(value)
+    proj = torch.zeros(mh, dim, dtype=torch.float32, device=query.device)
+    proj[:mh_valid, :E] = projection_matrix.to(torch.float32)
+    plan = SBLocalPlan(B, H, T, S, dim, mh, mh_valid, query.dtype, query.device, 64, n_parts=1)
+    out = torch.empty(B, T, H, dim, dtype=query.dtype, device=query.device)
+    log_norm = torch.empty(B, H, T, dtype=torch.float32, device=query.device)
+    plan.run_block_sparse(q, k, v, proj, t, tables, out, log_norm)
     return out[..., :D], log_norm.unsqueeze(-1)
 
 

@@ -131,6 +131,24 @@ int flyhip_sblocal_bwd(const float* x1, const float* x2, const float* x3,
                        int BH, int H, int T, int S, int E, int M, int local_context,
                        float softmax_temp, int key_major, void* stream);
 
+/* Scatterbrain attention on a block-sparse support (ref: src/models/attention/sbblocksparse_attention.py:109-213
+ * for need_weights = False, no dropout, no masks): as flyhip_sblocal_fwd with one part per query tile, but the
+ * exact part covers the nonzero 32 x 32 blocks of a layout instead of a band.  Key-side inputs (kfeat,
+ * chunk_scale, kv, ksum, kmax) from flyhip_sb_kv_reduce.  tl_ptr (H * ceil(T/64) + 1), tl_inner, tl_blk (2 per
+ * entry): per (head, 64-query tile) the union of the block columns of its two block-rows, and per entry the block
+ * id of each of the two rows or -1 where the row lacks that column.  float32 only; T, S multiples of 32. */
+int flyhip_sbblocksparse_fwd(const void* q, const void* k, const void* v, const float* proj,
+                             const void* kfeat, const float* chunk_scale,
+                             const float* kv, const float* ksum, const float* kmax,
+                             const int32_t* tl_ptr, const int32_t* tl_inner, const int32_t* tl_blk,
+                             void* out, float* log_norm,
+                             int B, int H, int T, int S, int E, int D, int mh, int mh_valid,
+                             int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                             int64_t k_sb, int64_t k_sh, int64_t k_ss,
+                             int64_t v_sb, int64_t v_sh, int64_t v_ss,
+                             int64_t o_sb, int64_t o_sh, int64_t o_ss,
+                             float softmax_temp, int dtype, void* stream);
+
 /* Plain local attention, no random features (ref: src/models/attention/local_attention.py:68-92;
  * fast_transformers.local_product): out[i] = softmax over the band -(lc/2) <= s - i < (lc+1)/2, s below
  * the key length, of t q_i.k_s, times v.  q (B,T,H,E), k (B,S,H,E), v (B,S,H,D), out (B,T,H,D) via

@@ -287,8 +287,14 @@ def test_sbblocksparse_attention_module(dtype, block):
     assert float((rows.float().cpu() - 1).abs().max()) <= (1e-4 if dtype == torch.float32 else 3e-2)
     ref_from_attn = torch.einsum('bhts,bshd->bthd', attn.double().cpu(), v.double())
     assert rel_err(ref_from_attn, ref_out) <= tol
+    # without the weights: 32 x 32 blocks take the fused kernels (the band kernel of Scatterbrain-local attention
+    # walking the layout's blocks), other block sizes the same ops as above
     out2, none = layer(q.to(DEV), k.to(DEV), v.to(DEV))
-    assert none is None and torch.equal(out2, out)
+    assert none is None and (len(layer.fused_tables) == 1) == (block == 32)
+    assert rel_err(out2, ref_out) <= tol
+    layer.fuse = False
+    out3, _ = layer(q.to(DEV), k.to(DEV), v.to(DEV))
+    assert torch.equal(out3, out)
 
 
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
@@ -546,3 +552,30 @@ def test_probabilities_from_log_denominators():
               0.2, _lib.dtype_code(qd), _lib.stream_ptr(torch.device(DEV)))
     ref = ob.block_softmax(ob.sdd(q.float(), k.float(), layout, block, trans_b=True), layout, block, scale=0.2)
     assert rel_err(probs, ref.nan_to_num()) <= 2e-2
+
+
+@pytest.mark.parametrize('B,H,T,S,E,D,m,seed', [(2, 2, 256, 256, 64, 64, 64, 1), (1, 3, 224, 352, 32, 32, 32, 2),
+                                                (2, 1, 96, 64, 128, 128, 256, 3), (1, 2, 416, 160, 40, 24, 26, 4)])
+def test_sbblocksparse_fused_forward(B, H, T, S, E, D, m, seed):
+    """Scatterbrain attention on a block-sparse support on the fused kernels (flyhip_sbblocksparse_fwd): random
+    layouts per head with an empty block-row, an odd number of block-rows (a query tile with one block-row),
+    T != S, head dims and feature counts that need padding; output and log-normaliser against the oracle."""
+    from fly_amd.blocksparse_utils import union_table
+    from fly_amd.sblocal_attention import sbblocksparse_forward
+    from oracle import sbblocksparse as osbb
+    from oracle import sblocal as osb
+    print('case', B, H, T, S, E, D, m, flush=True)
+    g = torch.Generator().manual_seed(seed)
+    layout = (torch.rand(H, T // 32, S // 32, generator=g) < 0.4).long()
+    layout[:, :, 0] = 1
+    layout[0, 1, :] = 0
+    q = torch.randn(B, T, H, E, generator=g) * E ** -0.25
+    k = torch.randn(B, S, H, E, generator=g) * E ** -0.25
+    v = torch.randn(B, S, H, D, generator=g)
+    P = osb.gaussian_orthogonal_random_matrix(m // 2, E, generator=g)
+    tables = tuple(x.to(DEV) for x in union_table(layout, rows_per_group=2))
+    out, ln = sbblocksparse_forward(q.to(DEV), k.to(DEV), v.to(DEV), P.to(DEV), tables)
+    ref_out, ref_ln = osbb.sbblocksparse_attention(q.double(), k.double(), v.double(), P.double(), layout, 32)
+    assert out.shape == (B, T, H, D) and ln.shape == (B, H, T, 1)
+    assert rel_err(out, ref_out) <= 1e-4, rel_err(out, ref_out)
+    assert rel_err(ln.reshape(ref_ln.shape), ref_ln) <= 1e-4, rel_err(ln.reshape(ref_ln.shape), ref_ln)
