@@ -15,7 +15,9 @@ from .blocksparse_attention import BlockSparseAttention
 from .sbblocksparse_attention import SBBlockSparseAttention
 from .blocksparse_linear import BlockSparseLinear, FlatBlockButterflySparsityConfig
 from .fastlinear import LowRank, SparseLRLinear
-from .t2t_vit import T2T_ViT, T2T_module, T2TAttention, Token_transformer, MlpCustom, t2t_vit_t_14
+from .t2t_vit import (T2T_ViT, T2T_module, T2TAttention, Token_transformer, MlpCustom, t2t_vit_t_14,
+                      convert_t2t_vit_state_dict)
+from .multihead_attention import MultiheadAttention
 
 __all__ = ['FullMask', 'LengthMask', 'TriangularCausalMask', 'SBPerformerFeatures',
            'gaussian_orthogonal_random_matrix', 'SBLocalAttention', 'sblocal_forward', 'sblocal_attention_fn', 'sblocal_backward', 'LocalAttention', 'local_forward', 'local_attention_fn', 'local_backward',
@@ -23,4 +25,5 @@ __all__ = ['FullMask', 'LengthMask', 'TriangularCausalMask', 'SBPerformerFeature
            'matmul', 'softmax', 'logsumexp', 'blocksparse_sum', 'BlockSparseAttention', 'fused_attention',
            'SBBlockSparseAttention',
            'BlockSparseLinear', 'FlatBlockButterflySparsityConfig', 'LowRank', 'SparseLRLinear',
-           'T2T_ViT', 'T2T_module', 'T2TAttention', 'Token_transformer', 'MlpCustom', 't2t_vit_t_14']
+           'T2T_ViT', 'T2T_module', 'T2TAttention', 'Token_transformer', 'MlpCustom', 't2t_vit_t_14',
+           'convert_t2t_vit_state_dict', 'MultiheadAttention']

@@ -215,3 +215,22 @@ def t2t_vit_t_14(**kwargs):
     """T2T-ViT-t-14: transformer tokens-to-token, embed 384, depth 14, 6 heads, mlp_ratio 3
     (t2t_vit.py:197-206)."""
     return T2T_ViT(embed_dim=384, depth=14, num_heads=6, mlp_ratio=3., **kwargs)
+
+
+def convert_t2t_vit_state_dict(state_dict):
+    """State dict of a published T2T-ViT checkpoint -> the names of this model (the mapping of the
+    reference's conversion script, scripts/convert_checkpoint_t2t_vit.py:19-31, and the unwrapping of
+    its loader, src/eval.py:22-32): the weights may sit under the single key 'state_dict_ema';
+    'pos_embed' becomes 'pos_embed.pe' and the 'tokens_to_token.' prefix 'patch_embed.'.  Returns a
+    new dict; the tensors are not copied.  Already converted dicts come back unchanged."""
+    if set(state_dict.keys()) == {'state_dict_ema'}:
+        state_dict = state_dict['state_dict_ema']
+
+    def rename(key):
+        if key == 'pos_embed':
+            return 'pos_embed.pe'
+        if key.startswith('tokens_to_token.'):
+            return 'patch_embed.' + key[len('tokens_to_token.'):]
+        return key
+
+    return {rename(k): v for k, v in state_dict.items()}

@@ -95,3 +95,25 @@ def test_mlp_custom_with_plugin_linears():
     assert torch.allclose(mlp(x), want)
     plain = MlpCustom(16, 32)
     assert isinstance(plain.fc1, nn.Linear) and plain(torch.randn(2, 16)).shape == (2, 16)
+
+
+def test_published_checkpoint_names_convert_and_load():
+    """A state dict under the names of the published T2T-ViT checkpoints ('tokens_to_token.*', a bare
+    'pos_embed', everything under 'state_dict_ema') loads after conversion, strictly
+    (scripts/convert_checkpoint_t2t_vit.py:19-31)."""
+    torch.manual_seed(0)
+    small = dict(embed_dim=64, depth=1, num_heads=2, mlp_ratio=1., token_dim=16, num_classes=10)
+    src = fly_amd.T2T_ViT(**small)
+    published = {}
+    for k, v in src.state_dict().items():
+        k = 'pos_embed' if k == 'pos_embed.pe' else k
+        k = 'tokens_to_token.' + k[len('patch_embed.'):] if k.startswith('patch_embed.') else k
+        published[k] = v.clone()
+    assert 'pos_embed' in published and any(k.startswith('tokens_to_token.attention1') for k in published)
+    converted = fly_amd.convert_t2t_vit_state_dict({'state_dict_ema': published})
+    assert set(converted) == set(src.state_dict())
+    dst = fly_amd.T2T_ViT(**small)
+    dst.load_state_dict(converted, strict=True)
+    x = torch.randn(2, 3, 224, 224)
+    assert torch.equal(src.eval()(x), dst.eval()(x))
+    assert fly_amd.convert_t2t_vit_state_dict(converted).keys() == converted.keys()      # idempotent

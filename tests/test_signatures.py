@@ -50,6 +50,10 @@ CASES = [
     ('attention/blocksparse_utils.py', None, 'mask_tensor', 'mask_tensor'),
     ('attention/blocksparse_utils.py', None, 'sparsify_broadcast_tensor', 'sparsify_broadcast_tensor'),
     ('attention/projection_utils.py', None, 'gaussian_orthogonal_random_matrix', 'gaussian_orthogonal_random_matrix'),
+    ('modules/multihead_attention.py', 'MultiheadAttention', '__init__', 'MultiheadAttention.__init__'),
+    ('modules/multihead_attention.py', 'MultiheadAttention', 'forward', 'MultiheadAttention.forward'),
+    ('modules/multihead_attention.py', 'InProjContainer', '__init__', 'multihead_attention.InProjContainer.__init__'),
+    ('modules/multihead_attention.py', 'InProjContainer', 'forward', 'multihead_attention.InProjContainer.forward'),
 ]
 
 
