@@ -2399,7 +2399,18 @@ static int plan(int B, int H, int S, int* n_chunks, int* n_split) {
     long want = (1024 + (long)B * H - 1) / ((long)B * H);
     if (want < 1) want = 1;
     if (want > nc) want = nc;
-    const int per = (nc + (int)want - 1) / (int)want;
+    int per = (nc + (int)want - 1) / (int)want;
+    if ((long)B * H * nc > 512) {
+        // more work than one residency round (two workgroups per CU): the pass takes about
+        // rounds x chunks per workgroup, and a round that is full costs no more than one that is not; among
+        // equals the larger share wins (fewer partial reductions to combine)
+        long best = -1;
+        for (int p = 1; p <= nc; ++p) {
+            const long wgs = (long)B * H * ((nc + p - 1) / p);
+            const long cost = ((wgs + 511) / 512) * p;
+            if (best < 0 || cost <= best) { best = cost; per = p; }
+        }
+    }
     *n_chunks = nc;
     *n_split = (nc + per - 1) / per;
     return OK;
