@@ -127,6 +127,13 @@ def union_table(layout, rows_per_group=4, transposed=False):
     return ptr.to(torch.int32), nz[:, 2].to(torch.int32).contiguous(), blk.to(torch.int32).contiguous()
 
 
+def union_order(uni_ptr, n_heads):
+    """Per head, its groups of union_table sorted by the length of their lists, longest first (ties in
+    index order): int32 (n_heads * groups_per_head), entries are group indices within the head."""
+    counts = (uni_ptr[1:] - uni_ptr[:-1]).cpu().long().reshape(n_heads, -1)
+    return torch.argsort(counts, dim=1, descending=True, stable=True).to(torch.int32).reshape(-1).contiguous()
+
+
 def group_table(layout, by_rows, max_group=4):
     """Groups of up to `max_group` consecutive segments (of one head) whose reduction lists visit the
     same inner blocks: returns (grp_row0 int32, grp_n int32).  Every segment belongs to one group."""

@@ -79,6 +79,8 @@ struct FwdArgs {
     // 64-query tile) the key blocks its two block-rows touch -- tl_ptr (H * tiles + 1), tl_inner (block
     // column per entry), tl_blk (2 per entry: block id of block-row 2 tile, 2 tile + 1, or -1 if absent)
     const int32_t* tl_ptr; const int32_t* tl_inner; const int32_t* tl_blk;
+    // optional: per head the query tiles in the order they should start (longest list first)
+    const int32_t* tl_order;
 };
 
 // ROWS x W tile of a (seq, W) matrix, moved global -> registers -> LDS in two steps so that all of
@@ -1433,13 +1435,28 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
     // L2.  The linear id is therefore re-mapped so that one XCD works on a contiguous run of
     // (batch-head, query tile, part) items: neighbours in that order share key tiles.
     const int n_qt = (a.T + TQ - 1) / TQ;
-    const int n_items = a.B * a.H * n_qt * a.n_parts;
-    const int per_xcd = (n_items + N_XCD - 1) / N_XCD;
-    const int item = (blockIdx.x % N_XCD) * per_xcd + blockIdx.x / N_XCD;
-    if (item >= n_items) return;                       // workgroup-uniform
-    const int part = item % a.n_parts;
-    const int qt = (item / a.n_parts) % n_qt;
-    const int bh = item / (a.n_parts * n_qt), b = bh / a.H, h = bh % a.H;
+    int part, qt, bh;
+    if (LIST) {
+        // Lists differ in length by orders of magnitude (a block-row of global tokens against a window), so
+        // the tiles start longest first: an XCD takes the (batch, head) pairs congruent to its number and
+        // walks them rank by rank -- all their longest tiles, then all their second longest ...
+        const int nbh = a.B * a.H, x = blockIdx.x % N_XCD, i = blockIdx.x / N_XCD;
+        const int mine = (nbh - x + N_XCD - 1) / N_XCD;            // pairs of this XCD
+        if (mine <= 0 || i >= mine * n_qt) return;                 // workgroup-uniform
+        const int rank = i / mine;
+        bh = x + N_XCD * (i % mine);
+        qt = a.tl_order ? a.tl_order[(bh % a.H) * n_qt + rank] : rank;
+        part = 0;
+    } else {
+        const int n_items = a.B * a.H * n_qt * a.n_parts;
+        const int per_xcd = (n_items + N_XCD - 1) / N_XCD;
+        const int item = (blockIdx.x % N_XCD) * per_xcd + blockIdx.x / N_XCD;
+        if (item >= n_items) return;                       // workgroup-uniform
+        part = item % a.n_parts;
+        qt = (item / a.n_parts) % n_qt;
+        bh = item / (a.n_parts * n_qt);
+    }
+    const int b = bh / a.H, h = bh % a.H;
     const int q0 = qt * TQ;
     const int iq = q0 + 16 * w + r16;
     const bool qvalid = iq < a.T;
@@ -1993,8 +2010,8 @@ static int launch_fwd_list(const FwdArgs& a, hipStream_t st) {
         if (e != hipSuccess) return fail(ERR_LAUNCH, "sbblocksparse_fwd: LDS attribute: %s", hipGetErrorString(e));
         lds_ready = true;
     }
-    const long items = (long)a.B * a.H * ((a.T + TQ - 1) / TQ);
-    const long grid = (items + N_XCD - 1) / N_XCD * N_XCD;
+    // every XCD gets room for ceil(B H / 8) (batch, head) pairs
+    const long grid = (((long)a.B * a.H + N_XCD - 1) / N_XCD) * ((a.T + TQ - 1) / TQ) * N_XCD;
     if (grid > 2147483647L) return fail(ERR_ARG, "sbblocksparse_fwd: too many workgroups");
     FwdArgs args = a;
     args.band_wgs = (int)grid;
@@ -2534,7 +2551,7 @@ extern "C" int flyhip_sbblocksparse_fwd(const void* q, const void* k, const void
                                         const void* kfeat, const float* chunk_scale,
                                         const float* kv, const float* ksum, const float* kmax,
                                         const int32_t* tl_ptr, const int32_t* tl_inner, const int32_t* tl_blk,
-                                        void* out, float* log_norm,
+                                        const int32_t* tl_order, void* out, float* log_norm,
                                         int B, int H, int T, int S, int E, int D, int mh, int mh_valid,
                                         int64_t q_sb, int64_t q_sh, int64_t q_ss,
                                         int64_t k_sb, int64_t k_sh, int64_t k_ss,
@@ -2556,7 +2573,7 @@ extern "C" int flyhip_sbblocksparse_fwd(const void* q, const void* k, const void
               nullptr, out, log_norm, nullptr,
               B, H, T, S, mh_valid, 1, nc, 1,
               q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss, softmax_temp,
-              tl_ptr, tl_inner, tl_blk};
+              tl_ptr, tl_inner, tl_blk, tl_order};
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     const int m = 2 * mh;
     SB_DISPATCH_E(launch_fwd_list, float, a)

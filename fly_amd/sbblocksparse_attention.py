@@ -15,7 +15,7 @@ from torch import distributed as dist
 from .blocksparse_attention import instantiate
 from .blocksparse_matmul import matmul
 from .blocksparse_softmax import blocksparse_sum, logsumexp
-from .blocksparse_utils import densify_tensor, sparsify_broadcast_tensor, union_table
+from .blocksparse_utils import densify_tensor, sparsify_broadcast_tensor, union_order, union_table
 from .sblocal_attention import sbblocksparse_forward, sbblocksparse_forward_supported
 from .feature_maps_sb import SBPerformerFeatures
 from .padding import pad_to_multiple
@@ -114,7 +114,9 @@ class SBBlockSparseAttention(nn.Module):
                                                     self.feature_map.projection_matrix.shape[0], layout.shape[0], H)):
             key_ = (T, S, query.device)
             if key_ not in self.fused_tables:
-                self.fused_tables[key_] = tuple(x.to(query.device) for x in union_table(layout, rows_per_group=2))
+                tabs = union_table(layout, rows_per_group=2)
+                tabs = tabs + (union_order(tabs[0], layout.shape[0]),)
+                self.fused_tables[key_] = tuple(x.to(query.device) for x in tabs)
             # (2-byte inputs are widened, as on the op-by-op path below)
             out, _ = sbblocksparse_forward(query.float(), key.float(), value.float(),
                                            self.feature_map.projection_matrix, self.fused_tables[key_], softmax_temp)

@@ -102,14 +102,15 @@ class SBLocalPlan:
         key pass as in ``run``, then the fp32 band kernel walking lists of 32-key blocks (``tables`` =
         union_table(layout, rows_per_group=2) on the device).  One part per query tile, no key lengths."""
         B, H, T, S, dim, mh, mh_valid = self.shape
-        tl_ptr, tl_inner, tl_blk = tables
+        tl_ptr, tl_inner, tl_blk = tables[:3]
+        tl_order = tables[3] if len(tables) > 3 else None      # union_order(tl_ptr, H): longest lists first
         with torch.cuda.device(self.device):
             stream = _lib.stream_ptr(self.device)
             self.run_keys(q, k, v, proj, None, t, stream)
             _lib.call('flyhip_sbblocksparse_fwd', q.data_ptr(), k.data_ptr(), v.data_ptr(), proj.data_ptr(),
                       self.kfeat.data_ptr(), self.chunk_scale.data_ptr(), self.kv.data_ptr(),
                       self.ksum.data_ptr(), self.kmax.data_ptr(), tl_ptr.data_ptr(), tl_inner.data_ptr(),
-                      tl_blk.data_ptr(), out.data_ptr(), log_norm.data_ptr(),
+                      tl_blk.data_ptr(), _lib.ptr(tl_order), out.data_ptr(), log_norm.data_ptr(),
                       B, H, T, S, dim, dim, mh, mh_valid,
                       q.stride(0), q.stride(2), q.stride(1), k.stride(0), k.stride(2), k.stride(1),
                       v.stride(0), v.stride(2), v.stride(1), out.stride(0), out.stride(2), out.stride(1),
@@ -183,7 +184,7 @@ def sbblocksparse_forward(query, key, value, projection_matrix, tables, softmax_
     need_weights=False, no dropout) on the fused kernels: exact softmax weights on the nonzero 32 x 32
     blocks, the Performer estimate everywhere else, one normaliser.  query (B,T,H,E), key (B,S,H,E), value
     (B,S,H,D) float32 GPU tensors, T and S multiples of 32; tables = union_table(layout, rows_per_group=2)
-    as int32 tensors on the device.  Returns (out (B,T,H,D), log_normalization (B,H,T,1))."""
+    as int32 tensors on the device, optionally followed by union_order(tables[0], H).  Returns (out (B,T,H,D), log_normalization (B,H,T,1))."""
     _lib.require_gpu(query, key, value, projection_matrix)
     B, T, H, E = query.shape
     S, D = key.shape[1], value.shape[3]

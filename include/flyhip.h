@@ -136,11 +136,14 @@ int flyhip_sblocal_bwd(const float* x1, const float* x2, const float* x3,
  * exact part covers the nonzero 32 x 32 blocks of a layout instead of a band.  Key-side inputs (kfeat,
  * chunk_scale, kv, ksum, kmax) from flyhip_sb_kv_reduce.  tl_ptr (H * ceil(T/64) + 1), tl_inner, tl_blk (2 per
  * entry): per (head, 64-query tile) the union of the block columns of its two block-rows, and per entry the block
- * id of each of the two rows or -1 where the row lacks that column.  float32 only; T, S multiples of 32. */
+ * id of each of the two rows or -1 where the row lacks that column.  tl_order (H * ceil(T/64), may be NULL): per
+ * head a permutation of its query tiles, the order in which they are started -- longest list first keeps a
+ * block-row of global tokens from becoming the tail of the launch.  float32 only; T, S multiples of 32. */
 int flyhip_sbblocksparse_fwd(const void* q, const void* k, const void* v, const float* proj,
                              const void* kfeat, const float* chunk_scale,
                              const float* kv, const float* ksum, const float* kmax,
                              const int32_t* tl_ptr, const int32_t* tl_inner, const int32_t* tl_blk,
+                             const int32_t* tl_order,
                              void* out, float* log_norm,
                              int B, int H, int T, int S, int E, int D, int mh, int mh_valid,
                              int64_t q_sb, int64_t q_sh, int64_t q_ss,

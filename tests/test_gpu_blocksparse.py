@@ -555,7 +555,8 @@ def test_probabilities_from_log_denominators():
 
 
 @pytest.mark.parametrize('B,H,T,S,E,D,m,seed', [(2, 2, 256, 256, 64, 64, 64, 1), (1, 3, 224, 352, 32, 32, 32, 2),
-                                                (2, 1, 96, 64, 128, 128, 256, 3), (1, 2, 416, 160, 40, 24, 26, 4)])
+                                                (2, 1, 96, 64, 128, 128, 256, 3), (1, 2, 416, 160, 40, 24, 26, 4),
+                                                (11, 3, 160, 192, 32, 32, 32, 5)])
 def test_sbblocksparse_fused_forward(B, H, T, S, E, D, m, seed):
     """Scatterbrain attention on a block-sparse support on the fused kernels (flyhip_sbblocksparse_fwd): random
     layouts per head with an empty block-row, an odd number of block-rows (a query tile with one block-row),
@@ -579,3 +580,8 @@ def test_sbblocksparse_fused_forward(B, H, T, S, E, D, m, seed):
     assert out.shape == (B, T, H, D) and ln.shape == (B, H, T, 1)
     assert rel_err(out, ref_out) <= 1e-4, rel_err(out, ref_out)
     assert rel_err(ln.reshape(ref_ln.shape), ref_ln) <= 1e-4, rel_err(ln.reshape(ref_ln.shape), ref_ln)
+    # the same with the tiles started longest list first: every tile is still computed once, by the same code
+    from fly_amd.blocksparse_utils import union_order
+    ordered = tables + (union_order(tables[0], H).to(DEV),)
+    out2, ln2 = sbblocksparse_forward(q.to(DEV), k.to(DEV), v.to(DEV), P.to(DEV), ordered)
+    assert torch.equal(out2, out) and torch.equal(ln2, ln)

@@ -74,6 +74,23 @@ def test_index_tables_bit_exact():
     assert torch.equal(bu.sdd_table(layout[0]), ob.sdd_lut(layout[0]))
 
 
+def test_union_order_longest_lists_first():
+    """Per head a permutation of its groups, list lengths non-increasing, ties in index order."""
+    for H, p, r, seed in ((2, 8, 6, 1), (3, 5, 9, 2), (1, 2, 3, 3)):
+        layout = _layout(H, p, r, seed)
+        layout[0, 0, :] = 1                                  # a block-row of global tokens
+        ptr, _, _ = bu.union_table(layout, rows_per_group=2)
+        order = bu.union_order(ptr, H)
+        G = (p + 1) // 2
+        assert order.dtype == torch.int32 and order.shape == (H * G,)
+        counts = (ptr[1:] - ptr[:-1]).reshape(H, G).tolist()
+        for h in range(H):
+            o = order[h * G:(h + 1) * G].tolist()
+            assert sorted(o) == list(range(G))
+            assert o == sorted(range(G), key=lambda g: (-counts[h][g], g))
+        assert order[0] == 0                                 # the global row's group has every column
+
+
 def test_union_table_against_loops():
     """Union of block-columns over groups of four block-rows, checked against explicit loops."""
     for H, p, r, seed in ((2, 7, 5, 4), (1, 4, 9, 5), (3, 1, 3, 6)):
