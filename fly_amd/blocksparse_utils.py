@@ -134,6 +134,26 @@ def union_order(uni_ptr, n_heads):
     return torch.argsort(counts, dim=1, descending=True, stable=True).to(torch.int32).reshape(-1).contiguous()
 
 
+def union_heavy(uni_ptr, uni_blk, n_heavy_min=32, entries_per_part=12, max_parts=16):
+    """The groups of union_table whose lists are long enough to be walked in parts: returns (heavy int32
+    (n_heavy) global group indices head * groups + group, parts) with parts = longest list //
+    entries_per_part clipped to [2, max_parts]; (empty, 1) when no list has n_heavy_min entries.  A group
+    qualifies only if every one of its rows that has any entry in the table's padding sense -- i.e. each of
+    its block-rows -- owns at least one block (a part cannot know whether another part saw a block)."""
+    ptr = uni_ptr.cpu().long()
+    blk = uni_blk.cpu()
+    counts = ptr[1:] - ptr[:-1]
+    heavy = []
+    for gidx in (counts >= n_heavy_min).nonzero().flatten().tolist():
+        rows = blk[ptr[gidx]:ptr[gidx + 1]]
+        if bool((rows >= 0).any(dim=0).all()):
+            heavy.append(gidx)
+    if not heavy:
+        return torch.zeros(0, dtype=torch.int32), 1
+    longest = int(counts[heavy].max())
+    return torch.tensor(heavy, dtype=torch.int32), max(2, min(max_parts, longest // entries_per_part))
+
+
 def group_table(layout, by_rows, max_group=4):
     """Groups of up to `max_group` consecutive segments (of one head) whose reduction lists visit the
     same inner blocks: returns (grp_row0 int32, grp_n int32).  Every segment belongs to one group."""

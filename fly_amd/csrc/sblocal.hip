@@ -79,8 +79,15 @@ struct FwdArgs {
     // 64-query tile) the key blocks its two block-rows touch -- tl_ptr (H * tiles + 1), tl_inner (block
     // column per entry), tl_blk (2 per entry: block id of block-row 2 tile, 2 tile + 1, or -1 if absent)
     const int32_t* tl_ptr; const int32_t* tl_inner; const int32_t* tl_blk;
-    // optional: per head the query tiles in the order they should start (longest list first)
+    // optional: per head the query tiles in the order they should start (longest list first); an entry
+    // -1 - tile marks a tile the one-part launch leaves to the launch below
     const int32_t* tl_order;
+    // long lists: tl_heavy (n_heavy entries head * tiles + tile) names the query tiles whose lists are walked
+    // in n_parts parts by a second launch (SPLIT and LIST; items (batch, heavy entry, part)), each part writing
+    // a partial for the merge kernel.  Its parts form the query features themselves (part 0 leaves them in
+    // qfeat), take kmax from the combined reductions, and index partials / query features by batch * n_heavy
+    // + entry.
+    const int32_t* tl_heavy; int n_heavy;
 };
 
 // ROWS x W tile of a (seq, W) matrix, moved global -> registers -> LDS in two steps so that all of
@@ -1415,7 +1422,6 @@ __global__ __launch_bounds__(NT) void local_fwd_kernel(LocalArgs a) {
 // ---------------------------------------------------------------------------------------
 template <typename T, int E, int D, int M, bool SPLIT, bool LIST = false>
 __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
-    static_assert(!(SPLIT && LIST), "the block-sparse support runs with one part per query tile");
     constexpr int MH = M / 2, LDK = E + 4, LDV = D + 4, LDF = M + 4;
     constexpr int FB = MH / 16, EC = E / 16, DB = D / 16, KB = TK / 16;
     constexpr int STAGE = TK * (LDK + LDV + LDF);     // floats per LDS stage
@@ -1423,7 +1429,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
     float* Ps = smem;                                  // only live before the key loop
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
-    if (SPLIT && (int)blockIdx.x >= a.band_wgs) {
+    if (SPLIT && !LIST && (int)blockIdx.x >= a.band_wgs) {
         // combine role: the partial K'^T V / sum K' of the key pass become kv / ksum / kmax for the merge
         // kernel (nothing in THIS launch reads them: the parts take kmax from the partial maxima)
         const int ci = blockIdx.x - a.band_wgs;
@@ -1436,7 +1442,16 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
     // (batch-head, query tile, part) items: neighbours in that order share key tiles.
     const int n_qt = (a.T + TQ - 1) / TQ;
     int part, qt, bh;
-    if (LIST) {
+    long slot = 0;                  // SPLIT and LIST: index of the tile's partials and compact query features
+    if (SPLIT && LIST) {
+        const int idx = blockIdx.x;
+        if (idx >= a.B * a.n_heavy * a.n_parts) return;            // workgroup-uniform
+        part = idx % a.n_parts;
+        slot = idx / a.n_parts;
+        const int hq = a.tl_heavy[slot % a.n_heavy];
+        qt = hq % n_qt;
+        bh = (int)(slot / a.n_heavy) * a.H + hq / n_qt;
+    } else if (LIST) {
         // Lists differ in length by orders of magnitude (a block-row of global tokens against a window), so
         // the tiles start longest first: an XCD takes the (batch, head) pairs congruent to its number and
         // walks them rank by rank -- all their longest tiles, then all their second longest ...
@@ -1446,6 +1461,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
         const int rank = i / mine;
         bh = x + N_XCD * (i % mine);
         qt = a.tl_order ? a.tl_order[(bh % a.H) * n_qt + rank] : rank;
+        if (qt < 0) return;                                        // a long list: left to the launch in parts
         part = 0;
     } else {
         const int n_items = a.B * a.H * n_qt * a.n_parts;
@@ -1475,7 +1491,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
     const int hi = min(len, q_last + lc_hi);
     int kt_lo = lo / TK;
     int kt_hi = (hi > lo) ? (hi + TK - 1) / TK : kt_lo;
-    if (SPLIT) {
+    if (SPLIT && !LIST) {
         // an even split: the first (tiles % parts) parts take one tile more
         const int nt = kt_hi - kt_lo, base = nt / a.n_parts, extra = nt % a.n_parts;
         const int first = kt_lo + part * base + min(part, extra);
@@ -1490,9 +1506,15 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
     int tile_cur = 0, tile_next = 0;
     bool pres_cur = false, pres_next = false, seen_block = false;
     if (LIST) {
-        const int lp0 = a.tl_ptr[h * n_qt + qt];
+        int lp0 = a.tl_ptr[h * n_qt + qt];
         kt_lo = 0;
         kt_hi = a.tl_ptr[h * n_qt + qt + 1] - lp0;
+        if (SPLIT) {
+            // this part's share of the list: the first (entries % parts) parts take one entry more
+            const int base = kt_hi / a.n_parts, extra = kt_hi % a.n_parts;
+            lp0 += part * base + min(part, extra);
+            kt_hi = base + (part < extra ? 1 : 0);
+        }
         tl_inner = a.tl_inner + lp0;
         tl_blk = a.tl_blk + 2 * (long)lp0 + (w >> 1);       // waves 0, 1: block-row 2 qt; waves 2, 3: 2 qt + 1
         if (kt_hi > 0) { tile_cur = tl_inner[0]; pres_cur = tl_blk[0] >= 0; }
@@ -1518,7 +1540,8 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
     rf.template offsets<float>(offf, M, tid);
     const float* csp = a.chunk_scale + (long)bh * a.n_chunks;
     float cscale = (kt_lo < kt_hi) ? csp[first_tile * TK / CH] : 0.f;
-    const float kmax = SPLIT ? split_kmax(a.part_max, bh, a.n_split) : a.kmax[bh];
+    constexpr bool OWN_Q = !SPLIT || LIST;       // query features formed here (not by the key pass), kmax combined
+    const float kmax = OWN_Q ? a.kmax[bh] : split_kmax(a.part_max, bh, a.n_split);
 
     // query operand (B side: column = query, k = 16c+4g+j) and its squared norm
     floatx4 qr[EC];
@@ -1534,7 +1557,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
     // query features, kept in registers: qf[c] is the B operand for feature slice c of K'
     floatx4 qf[2 * FB];
     float lsq;
-    if (SPLIT) {
+    if (!OWN_Q) {
         // several parts share a query tile: the key pass has computed the features once
         const long qrow = (long)bh * a.T + min(iq, a.T - 1);
 #pragma unroll
@@ -1576,7 +1599,13 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
             }
         }
     }
-    if (!SPLIT) __syncthreads();     // Ps is dead; the tile buffers may overwrite it
+    if (OWN_Q) __syncthreads();      // Ps is dead; the tile buffers may overwrite it
+    if (SPLIT && LIST && part == 0) {
+        // the merge kernel's operand for the global low-rank term
+        float* dst = const_cast<float*>(a.qfeat) + (slot * TQ + 16 * w + r16) * M;
+#pragma unroll
+        for (int c = 0; c < 2 * FB; ++c) *reinterpret_cast<floatx4*>(dst + 16 * c + 4 * g) = qf[c];
+    }
     FLY_PROF(1);
 
     // From here on all exponents are base 2 (one v_exp_f32 each): scores carry t*log2(e) through
@@ -1727,7 +1756,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
         if (LIST) { seen_block |= pres_cur; tile_cur = tile_next; tile_next = tile_n2; pres_cur = pres_next; pres_next = pres_n2; }
         __syncthreads();
     }
-    if (LIST && !seen_block) {
+    if (LIST && !SPLIT && !seen_block) {
         // A block-row without any block: the reference's row logsumexp returns 0 there, not -inf
         // (blocksparse_logsumexp.py:132), so its normaliser carries an extra exp(0); reproduced.
         m_run = fmaxf(m_run, 0.f);
@@ -1771,7 +1800,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
     const float gamma = __builtin_amdgcn_exp2f(c0 - m_run);               // <= 1
     if (SPLIT) {
         // un-normalised partial in this part's own (base-2) exponent m_run
-        float* ws = a.part_ws + (((long)bh * n_qt + qt) * a.n_parts + part) * (TQ * (D + NSTAT));
+        float* ws = a.part_ws + ((LIST ? slot : (long)bh * n_qt + qt) * a.n_parts + part) * (TQ * (D + NSTAT));
         const int ql = 16 * w + r16;
 #pragma unroll
         for (int db = 0; db < DB; ++db) *reinterpret_cast<floatx4*>(ws + ql * D + 16 * db + 4 * g) = oacc[db];
@@ -1816,7 +1845,14 @@ __global__ __launch_bounds__(NT) void sb_merge_kernel(FwdArgs a) {
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
     // one workgroup per (64-query tile, 16 output columns, batch-head): the tile's finish is spread over
     // D/16 workgroups because it is all latency (a short chain of loads, 2 M/16 MFMAs, a store)
-    const int qt = blockIdx.x, n_qt = gridDim.x, db = blockIdx.y, bh = blockIdx.z, b = bh / a.H, h = bh % a.H;
+    // (long lists of a block-sparse support: blockIdx.x = batch * n_heavy + entry of tl_heavy, see FwdArgs)
+    const bool heavy = a.tl_heavy != nullptr;
+    const int n_qt = heavy ? (a.T + TQ - 1) / TQ : gridDim.x;
+    const int hq = heavy ? a.tl_heavy[blockIdx.x % a.n_heavy] : 0;
+    const int qt = heavy ? hq % n_qt : blockIdx.x;
+    const int db = blockIdx.y, bh = heavy ? (blockIdx.x / a.n_heavy) * a.H + hq / n_qt : blockIdx.z;
+    const int b = bh / a.H, h = bh % a.H;
+    const long slot = heavy ? blockIdx.x : (long)bh * n_qt + qt;
     const int ql = 16 * w + r16, iq = qt * TQ + ql;
     {
         RowTile<M, 16> kvt;
@@ -1824,13 +1860,13 @@ __global__ __launch_bounds__(NT) void sb_merge_kernel(FwdArgs a) {
         if (tid < M) KSs[tid] = a.ksum[(long)bh * M + tid];
         kvt.template stash<LDV>(KVs, tid);
     }
-    const long qrow = (long)bh * a.T + min(iq, a.T - 1);
+    const long qrow = heavy ? slot * TQ + ql : (long)bh * a.T + min(iq, a.T - 1);
     floatx4 qf[FC];
 #pragma unroll
     for (int c = 0; c < FC; ++c) qf[c] = *reinterpret_cast<const floatx4*>(a.qfeat + qrow * M + 16 * c + 4 * g);
 
     const long stride = (long)TQ * (D + NSTAT);
-    const float* ws = a.part_ws + ((long)bh * n_qt + qt) * a.n_parts * stride;
+    const float* ws = a.part_ws + slot * a.n_parts * stride;
     const float* st = ws + TQ * D + ql;
     const float c0 = st[4 * TQ];                     // base-2 log-scale of the low-rank term (same in every part)
     float m_star = -INFINITY, ze = 0.f, zp = 0.f;
@@ -2015,8 +2051,29 @@ static int launch_fwd_list(const FwdArgs& a, hipStream_t st) {
     if (grid > 2147483647L) return fail(ERR_ARG, "sbblocksparse_fwd: too many workgroups");
     FwdArgs args = a;
     args.band_wgs = (int)grid;
+    args.tl_heavy = nullptr;
+    args.n_parts = 1;
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NT), smem, st, args);
-    return check_launch("sblocal_fwd_kernel (block-sparse support)");
+    int rc = check_launch("sblocal_fwd_kernel (block-sparse support)");
+    if (rc || a.n_heavy <= 0) return rc;
+    // the long lists, in parts
+    auto kern_parts = sblocal_fwd_kernel<float, E, E, M, true, true>;
+    static bool lds_parts_ready = false;
+    if (!lds_parts_ready) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern_parts),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return fail(ERR_LAUNCH, "sbblocksparse_fwd: LDS attribute: %s", hipGetErrorString(e));
+        lds_parts_ready = true;
+    }
+    const long tiles = (long)a.B * a.n_heavy, grid_parts = tiles * a.n_parts;
+    if (grid_parts > 2147483647L) return fail(ERR_ARG, "sbblocksparse_fwd: too many workgroups");
+    args = a;
+    args.band_wgs = (int)grid_parts;
+    hipLaunchKernelGGL(kern_parts, dim3((unsigned)grid_parts), dim3(NT), smem, st, args);
+    rc = check_launch("sblocal_fwd_kernel (block-sparse support, long lists)");
+    if (rc) return rc;
+    hipLaunchKernelGGL((sb_merge_kernel<float, E, M>), dim3((unsigned)tiles, E / 16, 1), dim3(NT), 0, st, args);
+    return check_launch("sb_merge_kernel (long lists)");
 }
 
 template <typename T, int E>
@@ -2551,7 +2608,8 @@ extern "C" int flyhip_sbblocksparse_fwd(const void* q, const void* k, const void
                                         const void* kfeat, const float* chunk_scale,
                                         const float* kv, const float* ksum, const float* kmax,
                                         const int32_t* tl_ptr, const int32_t* tl_inner, const int32_t* tl_blk,
-                                        const int32_t* tl_order, void* out, float* log_norm,
+                                        const int32_t* tl_order, const int32_t* tl_heavy, int n_heavy, int heavy_parts,
+                                        float* part_ws, float* qfeat, void* out, float* log_norm,
                                         int B, int H, int T, int S, int E, int D, int mh, int mh_valid,
                                         int64_t q_sb, int64_t q_sh, int64_t q_ss,
                                         int64_t k_sb, int64_t k_sh, int64_t k_ss,
@@ -2569,11 +2627,14 @@ extern "C" int flyhip_sbblocksparse_fwd(const void* q, const void* k, const void
     if (rc) return rc;
     int nc, ns;
     plan(B, H, S, &nc, &ns);
-    FwdArgs a{q, k, v, proj, kfeat, chunk_scale, kv, ksum, kmax, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 1,
-              nullptr, out, log_norm, nullptr,
-              B, H, T, S, mh_valid, 1, nc, 1,
+    FLY_REQUIRE(n_heavy >= 0 && (n_heavy == 0 || (tl_heavy && tl_order && part_ws && qfeat && heavy_parts >= 2 && heavy_parts <= 64)),
+                "sbblocksparse_fwd: long lists need tl_heavy, tl_order (with the long tiles marked), part_ws, qfeat and "
+                "2 <= heavy_parts <= 64");
+    FwdArgs a{q, k, v, proj, kfeat, chunk_scale, kv, ksum, kmax, qfeat, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 1,
+              nullptr, out, log_norm, part_ws,
+              B, H, T, S, mh_valid, 1, nc, n_heavy > 0 ? heavy_parts : 1,
               q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss, softmax_temp,
-              tl_ptr, tl_inner, tl_blk, tl_order};
+              tl_ptr, tl_inner, tl_blk, tl_order, tl_heavy, n_heavy};
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     const int m = 2 * mh;
     SB_DISPATCH_E(launch_fwd_list, float, a)

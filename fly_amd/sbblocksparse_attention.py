@@ -15,11 +15,30 @@ from torch import distributed as dist
 from .blocksparse_attention import instantiate
 from .blocksparse_matmul import matmul
 from .blocksparse_softmax import blocksparse_sum, logsumexp
-from .blocksparse_utils import densify_tensor, sparsify_broadcast_tensor, union_order, union_table
+from .blocksparse_utils import densify_tensor, sparsify_broadcast_tensor, union_heavy, union_order, union_table
 from .sblocal_attention import sbblocksparse_forward, sbblocksparse_forward_supported
 from .feature_maps_sb import SBPerformerFeatures
 from .padding import pad_to_multiple
 from .scatterbrain_utils import linear_attention, linear_attention_normalization
+
+
+def fused_tables(layout, device):
+    """Index tables of the fused forward for a (H, T/32, S/32) layout: the union lists of the query tiles
+    (two block-rows each), their start order (longest first), and the tiles whose lists are long enough to
+    be walked in parts -- (ptr, inner, blk, order, heavy, parts), tensors on `device`."""
+    ptr, inner, blk = union_table(layout, rows_per_group=2)
+    H = layout.shape[0]
+    order = union_order(ptr, H)
+    heavy, parts = union_heavy(ptr, blk)
+    if heavy.numel():
+        groups = order.numel() // H
+        marked = order.reshape(H, groups).clone()
+        is_heavy = torch.zeros(H * groups, dtype=torch.bool)
+        is_heavy[heavy.long()] = True
+        flat = torch.arange(H).unsqueeze(1) * groups + marked.long()
+        marked[is_heavy[flat]] = -1 - marked[is_heavy[flat]]
+        order = marked.reshape(-1).contiguous()
+    return tuple(x.to(device) for x in (ptr, inner, blk, order, heavy)) + (parts,)
 
 
 class SBBlockSparseAttention(nn.Module):
@@ -114,9 +133,7 @@ class SBBlockSparseAttention(nn.Module):
                                                     self.feature_map.projection_matrix.shape[0], layout.shape[0], H)):
             key_ = (T, S, query.device)
             if key_ not in self.fused_tables:
-                tabs = union_table(layout, rows_per_group=2)
-                tabs = tabs + (union_order(tabs[0], layout.shape[0]),)
-                self.fused_tables[key_] = tuple(x.to(query.device) for x in tabs)
+                self.fused_tables[key_] = fused_tables(layout, query.device)
             # (2-byte inputs are widened, as on the op-by-op path below)
             out, _ = sbblocksparse_forward(query.float(), key.float(), value.float(),
                                            self.feature_map.projection_matrix, self.fused_tables[key_], softmax_temp)

@@ -104,13 +104,24 @@ class SBLocalPlan:
         B, H, T, S, dim, mh, mh_valid = self.shape
         tl_ptr, tl_inner, tl_blk = tables[:3]
         tl_order = tables[3] if len(tables) > 3 else None      # union_order(tl_ptr, H): longest lists first
+        # long lists walked in parts (sbblocksparse_attention.fused_tables): scratch for their partials
+        tl_heavy, n_heavy, parts = None, 0, 1
+        if len(tables) > 5 and tables[4].numel() > 0:
+            tl_heavy, n_heavy, parts = tables[4], tables[4].numel(), int(tables[5])
+            need = (B * n_heavy * parts * 64 * (dim + 5), B * n_heavy * 64 * 2 * mh)
+            if getattr(self, '_heavy_sizes', None) != need:
+                self.part_ws = torch.empty(need[0], dtype=torch.float32, device=self.device)
+                self.qfeat = torch.empty(need[1], dtype=torch.float32, device=self.device)
+                self._heavy_sizes = need
         with torch.cuda.device(self.device):
             stream = _lib.stream_ptr(self.device)
             self.run_keys(q, k, v, proj, None, t, stream)
             _lib.call('flyhip_sbblocksparse_fwd', q.data_ptr(), k.data_ptr(), v.data_ptr(), proj.data_ptr(),
                       self.kfeat.data_ptr(), self.chunk_scale.data_ptr(), self.kv.data_ptr(),
                       self.ksum.data_ptr(), self.kmax.data_ptr(), tl_ptr.data_ptr(), tl_inner.data_ptr(),
-                      tl_blk.data_ptr(), _lib.ptr(tl_order), out.data_ptr(), log_norm.data_ptr(),
+                      tl_blk.data_ptr(), _lib.ptr(tl_order), _lib.ptr(tl_heavy), n_heavy, parts,
+                      _lib.ptr(self.part_ws) if n_heavy else None, _lib.ptr(self.qfeat) if n_heavy else None,
+                      out.data_ptr(), log_norm.data_ptr(),
                       B, H, T, S, dim, dim, mh, mh_valid,
                       q.stride(0), q.stride(2), q.stride(1), k.stride(0), k.stride(2), k.stride(1),
                       v.stride(0), v.stride(2), v.stride(1), out.stride(0), out.stride(2), out.stride(1),
@@ -184,7 +195,8 @@ def sbblocksparse_forward(query, key, value, projection_matrix, tables, softmax_
     need_weights=False, no dropout) on the fused kernels: exact softmax weights on the nonzero 32 x 32
     blocks, the Performer estimate everywhere else, one normaliser.  query (B,T,H,E), key (B,S,H,E), value
     (B,S,H,D) float32 GPU tensors, T and S multiples of 32; tables = union_table(layout, rows_per_group=2)
-    as int32 tensors on the device, optionally followed by union_order(tables[0], H).  Returns (out (B,T,H,D), log_normalization (B,H,T,1))."""
+    as int32 tensors on the device, optionally followed by union_order(tables[0], H), or the six entries of
+    sbblocksparse_attention.fused_tables (start order with the long lists marked, those lists, their parts).  Returns (out (B,T,H,D), log_normalization (B,H,T,1))."""
     _lib.require_gpu(query, key, value, projection_matrix)
     B, T, H, E = query.shape
     S, D = key.shape[1], value.shape[3]

@@ -585,3 +585,38 @@ def test_sbblocksparse_fused_forward(B, H, T, S, E, D, m, seed):
     ordered = tables + (union_order(tables[0], H).to(DEV),)
     out2, ln2 = sbblocksparse_forward(q.to(DEV), k.to(DEV), v.to(DEV), P.to(DEV), ordered)
     assert torch.equal(out2, out) and torch.equal(ln2, ln)
+
+
+def test_sbblocksparse_long_lists_in_parts():
+    """Block-rows of global tokens: their query tiles' lists are walked in parts by a second launch and merged
+    (fused_tables marks them); output and log-normaliser against the oracle and against the one-part path."""
+    from fly_amd.blocksparse_utils import union_table
+    from fly_amd.sbblocksparse_attention import fused_tables
+    from fly_amd.sblocal_attention import sbblocksparse_forward
+    from oracle import sbblocksparse as osbb
+    from oracle import sblocal as osb
+    B, H, L, E, m = 3, 2, 1280, 64, 64
+    nb = L // 32
+    g = torch.Generator().manual_seed(11)
+    idx = torch.arange(nb)
+    window = ((idx[:, None] - idx[None, :]).abs() <= 1).long()
+    layout = torch.stack([window.clone(), window.clone()])
+    layout[0, 0, :] = 1                       # head 0: block-row 0 global (tile 0: 40 entries, its second row a window)
+    layout[0, :, 0] = 1
+    layout[1, 21, :] = 1                      # head 1: block-row 21 global (second row of tile 10)
+    layout[1, 38:40, :] = 1                   # and a tile whose two rows are both long
+    q = torch.randn(B, L, H, E, generator=g) * E ** -0.25
+    k = torch.randn(B, L, H, E, generator=g) * E ** -0.25
+    v = torch.randn(B, L, H, E, generator=g)
+    P = osb.gaussian_orthogonal_random_matrix(m // 2, E, generator=g)
+    tables = fused_tables(layout, DEV)
+    assert sorted(tables[4].tolist()) == [0, 20 + 10, 20 + 19] and tables[5] >= 2
+    assert sorted(-1 - x for x in tables[3].tolist() if x < 0) == [0, 10, 19]
+    print('case long lists', tables[4].tolist(), tables[5], flush=True)
+    out, ln = sbblocksparse_forward(q.to(DEV), k.to(DEV), v.to(DEV), P.to(DEV), tables)
+    ref_out, ref_ln = osbb.sbblocksparse_attention(q.double(), k.double(), v.double(), P.double(), layout, 32)
+    assert rel_err(out, ref_out) <= 1e-4, rel_err(out, ref_out)
+    assert rel_err(ln.reshape(ref_ln.shape), ref_ln) <= 1e-4, rel_err(ln.reshape(ref_ln.shape), ref_ln)
+    plain = tuple(x.to(DEV) for x in union_table(layout, rows_per_group=2))
+    out1, ln1 = sbblocksparse_forward(q.to(DEV), k.to(DEV), v.to(DEV), P.to(DEV), plain)
+    assert rel_err(out, out1) <= 1e-5 and rel_err(ln, ln1) <= 1e-5
