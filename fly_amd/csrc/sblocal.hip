@@ -80,13 +80,13 @@ struct FwdArgs {
     // column per entry), tl_blk (2 per entry: block id of block-row 2 tile, 2 tile + 1, or -1 if absent)
     const int32_t* tl_ptr; const int32_t* tl_inner; const int32_t* tl_blk;
     // optional: per head the query tiles in the order they should start (longest list first); an entry
-    // -1 - tile marks a tile the one-part launch leaves to the launch below
+    // -1 - tile marks a tile that is left to the workgroups walking long lists in parts
     const int32_t* tl_order;
     // long lists: tl_heavy (n_heavy entries head * tiles + tile) names the query tiles whose lists are walked
-    // in n_parts parts by a second launch (SPLIT and LIST; items (batch, heavy entry, part)), each part writing
-    // a partial for the merge kernel.  Its parts form the query features themselves (part 0 leaves them in
-    // qfeat), take kmax from the combined reductions, and index partials / query features by batch * n_heavy
-    // + entry.
+    // in n_parts parts: the first B * n_heavy * n_parts workgroups of the launch (rounded up to a multiple of the
+    // XCD count) take one (batch, heavy entry, part) each and write a partial for the merge kernel.  They form
+    // the query features themselves (part 0 leaves them in qfeat), take kmax from the combined reductions, and
+    // index partials / query features by batch * n_heavy + entry.
     const int32_t* tl_heavy; int n_heavy;
 };
 
@@ -1442,10 +1442,15 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
     // (batch-head, query tile, part) items: neighbours in that order share key tiles.
     const int n_qt = (a.T + TQ - 1) / TQ;
     int part, qt, bh;
-    long slot = 0;                  // SPLIT and LIST: index of the tile's partials and compact query features
-    if (SPLIT && LIST) {
+    // part_role: this workgroup writes an un-normalised partial for the merge kernel.  Always with SPLIT; on a
+    // block-sparse support the first workgroups of the launch, which walk the long lists in parts
+    bool part_role = SPLIT;
+    long slot = 0;                  // long lists: index of the tile's partials and compact query features
+    const int n_part_wgs = LIST ? (a.B * a.n_heavy * a.n_parts + N_XCD - 1) / N_XCD * N_XCD : 0;
+    if (LIST && (int)blockIdx.x < n_part_wgs) {
         const int idx = blockIdx.x;
         if (idx >= a.B * a.n_heavy * a.n_parts) return;            // workgroup-uniform
+        part_role = true;
         part = idx % a.n_parts;
         slot = idx / a.n_parts;
         const int hq = a.tl_heavy[slot % a.n_heavy];
@@ -1455,13 +1460,14 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
         // Lists differ in length by orders of magnitude (a block-row of global tokens against a window), so
         // the tiles start longest first: an XCD takes the (batch, head) pairs congruent to its number and
         // walks them rank by rank -- all their longest tiles, then all their second longest ...
-        const int nbh = a.B * a.H, x = blockIdx.x % N_XCD, i = blockIdx.x / N_XCD;
+        const int blk_id = blockIdx.x - n_part_wgs;
+        const int nbh = a.B * a.H, x = blk_id % N_XCD, i = blk_id / N_XCD;
         const int mine = (nbh - x + N_XCD - 1) / N_XCD;            // pairs of this XCD
         if (mine <= 0 || i >= mine * n_qt) return;                 // workgroup-uniform
         const int rank = i / mine;
         bh = x + N_XCD * (i % mine);
         qt = a.tl_order ? a.tl_order[(bh % a.H) * n_qt + rank] : rank;
-        if (qt < 0) return;                                        // a long list: left to the launch in parts
+        if (qt < 0) return;                                        // a long list: walked in parts by the first workgroups
         part = 0;
     } else {
         const int n_items = a.B * a.H * n_qt * a.n_parts;
@@ -1509,7 +1515,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
         int lp0 = a.tl_ptr[h * n_qt + qt];
         kt_lo = 0;
         kt_hi = a.tl_ptr[h * n_qt + qt + 1] - lp0;
-        if (SPLIT) {
+        if (part_role) {
             // this part's share of the list: the first (entries % parts) parts take one entry more
             const int base = kt_hi / a.n_parts, extra = kt_hi % a.n_parts;
             lp0 += part * base + min(part, extra);
@@ -1600,7 +1606,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
         }
     }
     if (OWN_Q) __syncthreads();      // Ps is dead; the tile buffers may overwrite it
-    if (SPLIT && LIST && part == 0) {
+    if (LIST && part_role && part == 0) {
         // the merge kernel's operand for the global low-rank term
         float* dst = const_cast<float*>(a.qfeat) + (slot * TQ + 16 * w + r16) * M;
 #pragma unroll
@@ -1756,7 +1762,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
         if (LIST) { seen_block |= pres_cur; tile_cur = tile_next; tile_next = tile_n2; pres_cur = pres_next; pres_next = pres_n2; }
         __syncthreads();
     }
-    if (LIST && !SPLIT && !seen_block) {
+    if (LIST && !part_role && !seen_block) {
         // A block-row without any block: the reference's row logsumexp returns 0 there, not -inf
         // (blocksparse_logsumexp.py:132), so its normaliser carries an extra exp(0); reproduced.
         m_run = fmaxf(m_run, 0.f);
@@ -1770,7 +1776,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
 #pragma unroll
     for (int db = 0; db < DB; ++db) lacc[db] = Frag<float>::zero();
     float qk1 = 0.f;
-    if (!SPLIT) {
+    if (!part_role) {
         // K'^T V (M x D) and sum K' (M) staged in LDS: coalesced loads, all in flight together
         float* KVs = smem;
         float* KSs = smem + M * LDV;
@@ -1798,7 +1804,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
     zp = group_sum(zp);
     FLY_PROF(4);
     const float gamma = __builtin_amdgcn_exp2f(c0 - m_run);               // <= 1
-    if (SPLIT) {
+    if (part_role) {
         // un-normalised partial in this part's own (base-2) exponent m_run
         float* ws = a.part_ws + ((LIST ? slot : (long)bh * n_qt + qt) * a.n_parts + part) * (TQ * (D + NSTAT));
         const int ql = 16 * w + r16;
@@ -2049,29 +2055,15 @@ static int launch_fwd_list(const FwdArgs& a, hipStream_t st) {
     // every XCD gets room for ceil(B H / 8) (batch, head) pairs
     const long grid = (((long)a.B * a.H + N_XCD - 1) / N_XCD) * ((a.T + TQ - 1) / TQ) * N_XCD;
     if (grid > 2147483647L) return fail(ERR_ARG, "sbblocksparse_fwd: too many workgroups");
+    // long lists: the first workgroups of the launch walk them in parts (they are the longest pieces of work)
+    const long tiles = (long)a.B * a.n_heavy;
+    const long part_wgs = (tiles * a.n_parts + N_XCD - 1) / N_XCD * N_XCD;
+    if (grid + part_wgs > 2147483647L) return fail(ERR_ARG, "sbblocksparse_fwd: too many workgroups");
     FwdArgs args = a;
-    args.band_wgs = (int)grid;
-    args.tl_heavy = nullptr;
-    args.n_parts = 1;
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NT), smem, st, args);
+    args.band_wgs = (int)(grid + part_wgs);
+    hipLaunchKernelGGL(kern, dim3((unsigned)(grid + part_wgs)), dim3(NT), smem, st, args);
     int rc = check_launch("sblocal_fwd_kernel (block-sparse support)");
     if (rc || a.n_heavy <= 0) return rc;
-    // the long lists, in parts
-    auto kern_parts = sblocal_fwd_kernel<float, E, E, M, true, true>;
-    static bool lds_parts_ready = false;
-    if (!lds_parts_ready) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern_parts),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        if (e != hipSuccess) return fail(ERR_LAUNCH, "sbblocksparse_fwd: LDS attribute: %s", hipGetErrorString(e));
-        lds_parts_ready = true;
-    }
-    const long tiles = (long)a.B * a.n_heavy, grid_parts = tiles * a.n_parts;
-    if (grid_parts > 2147483647L) return fail(ERR_ARG, "sbblocksparse_fwd: too many workgroups");
-    args = a;
-    args.band_wgs = (int)grid_parts;
-    hipLaunchKernelGGL(kern_parts, dim3((unsigned)grid_parts), dim3(NT), smem, st, args);
-    rc = check_launch("sblocal_fwd_kernel (block-sparse support, long lists)");
-    if (rc) return rc;
     hipLaunchKernelGGL((sb_merge_kernel<float, E, M>), dim3((unsigned)tiles, E / 16, 1), dim3(NT), 0, st, args);
     return check_launch("sb_merge_kernel (long lists)");
 }

@@ -139,10 +139,10 @@ int flyhip_sblocal_bwd(const float* x1, const float* x2, const float* x3,
  * id of each of the two rows or -1 where the row lacks that column.  tl_order (H * ceil(T/64), may be NULL): per
  * head a permutation of its query tiles, the order in which they are started -- longest list first keeps a
  * block-row of global tokens from becoming the tail of the launch.
- * Long lists (n_heavy > 0): tl_heavy (n_heavy entries head * ceil(T/64) + tile) names query tiles whose lists a
- * second launch walks in heavy_parts parts (2..64), finished by a merge launch; those tiles carry the entry
- * -1 - tile in tl_order so that the one-part launch leaves them alone, and every block-row of such a tile must
- * have at least one block.  Scratch for them: part_ws of B*n_heavy*heavy_parts*64*(D+5) floats and qfeat of
+ * Long lists (n_heavy > 0): tl_heavy (n_heavy entries head * ceil(T/64) + tile) names query tiles whose lists are
+ * walked in heavy_parts parts (2..64) by the first workgroups of the launch and finished by a merge launch; those
+ * tiles carry the entry -1 - tile in tl_order so that no workgroup takes them whole, and every block-row of such
+ * a tile must have at least one block.  Scratch for them: part_ws of B*n_heavy*heavy_parts*64*(D+5) floats and qfeat of
  * B*n_heavy*64*m floats (both NULL when n_heavy == 0).  float32 only; T, S multiples of 32. */
 int flyhip_sbblocksparse_fwd(const void* q, const void* k, const void* v, const float* proj,
                              const void* kfeat, const float* chunk_scale,
