@@ -158,3 +158,46 @@ def test_wrapper_around_sblocal_attention_matches_oracle_layer():
     ref, _ = mha.double().cpu()(OracleLayer(), x.double().cpu(), x.double().cpu(), x.double().cpu(),
                                 key_padding_mask=LengthMask(lengths, max_len=T))
     assert rel_err(out.cpu(), ref) <= 1e-4, rel_err(out.cpu(), ref)
+
+
+@pytest.mark.gpu
+def test_wrapper_around_blocksparse_attention_matches_dense_masked_softmax():
+    """Seq-first inputs, bias_k / zero position off, a key-padding mask: the wrapper around
+    BlockSparseAttention (bf16, fused kernel) against the same wrapper around a plain softmax layer
+    restricted to the layout's blocks."""
+    from conftest import rel_err
+    from fly_amd import BlockSparseAttention
+    torch.manual_seed(0)
+    dev = torch.device('cuda:0')
+    E, H, B, T = 256, 4, 2, 256
+
+    class BandPerHead:
+        """One layout per head: a band whose width grows with the head, plus the first block-column."""
+        block = 32
+
+        def make_layout(self, seqlen):
+            r = torch.arange(seqlen // self.block)
+            lay = torch.stack([((r.view(-1, 1) - r.view(1, -1)).abs() <= h).long() for h in range(H)])
+            lay[:, :, 0] = 1
+            return lay
+
+    mha = MultiheadAttention(E, H).to(dev)
+    attn = BlockSparseAttention(BandPerHead(), attention_dropout=0.0, max_seq_length=T).to(dev).eval()
+    x = torch.randn(T, B, E, device=dev)
+    lengths = torch.tensor([256, 160], device=dev)
+    with torch.no_grad():
+        out, w = mha.bfloat16()(attn, x.bfloat16(), x.bfloat16(), x.bfloat16(),
+                                key_padding_mask=LengthMask(lengths, max_len=T))
+    assert w is None and out.shape == (T, B, E)
+    dense = attn.get_layout(T).to(dev).bool().repeat_interleave(32, 1).repeat_interleave(32, 2)      # (H, T, T)
+
+    class MaskedLayer(torch.nn.Module):
+        def forward(self, q, k, v, attn_mask=None, key_padding_mask=None, need_weights=False):
+            s = torch.einsum('bthd,bshd->bhts', q, k) / math.sqrt(q.shape[-1])
+            s = s + key_padding_mask.additive_matrix[:, None, None, :]
+            s = s.masked_fill(~dense[None], float('-inf'))
+            return torch.einsum('bhts,bshd->bthd', s.softmax(dim=-1), v), None
+
+    with torch.no_grad():
+        ref, _ = mha.float()(MaskedLayer(), x, x, x, key_padding_mask=LengthMask(lengths, max_len=T))
+    assert rel_err(out.float().cpu(), ref.cpu()) <= 3e-2, rel_err(out.float().cpu(), ref.cpu())
