@@ -243,7 +243,7 @@ def test_blocksparse_linear_init_and_dense_backend():
     # Kaiming-uniform(a=sqrt5) on the dense matrix scaled by sqrt(ncol/nnz cols): bound = sqrt(1/nnz_in)
     nnz_cols = lin.layout.sum(-1).float() * 32
     bound = (1.0 / nnz_cols).sqrt().max()
-    assert float(lin.weight.abs().max()) <= float(bound) + 1e-6
+    assert float(lin.weight.detach().abs().max()) <= float(bound) + 1e-6
     assert float(lin.bias.abs().max()) <= 1 / (512 ** 0.5) + 1e-6
     x = torch.randn(3, 5, 497)
     ref = ob.blocksparse_linear(x, lin.weight.detach(), lin.layout, 32, lin.bias.detach(), 698)

@@ -126,7 +126,7 @@ def test_extra_key_positions_extend_the_masks_on_the_left():
     assert torch.equal(seen_am.bool_matrix[:, 2:], am.bool_matrix)
     assert w.shape == (B, H, T, T + 2) and out.shape == (B, T, E)
     # keys: zero position, bias_k, then the projected keys; masked keys get no weight
-    assert float(w[1, :, :, 4:].abs().max()) == 0.0
+    assert float(w[1, :, :, 4:].detach().abs().max()) == 0.0
     with pytest.raises(RuntimeError):
         m(layer, x, x, x, attn_mask=FullMask(torch.ones(T, T + 1, dtype=torch.bool)))
     with pytest.raises(AssertionError):
