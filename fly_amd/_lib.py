@@ -20,6 +20,7 @@ SIGNATURES = {
     'flyhip_sb_time_next_fwd': [c_vp, c_vp],
     'flyhip_sb_kv_reduce': [c_vp] * 14 + [c_int] + [c_i64] * 3 + [c_vp] * 2 + [c_int] * 8 + [c_i64] * 6 + [c_float, c_int, c_vp],
     'flyhip_sblocal_fwd': [c_vp] * 13 + [c_vp] * 2 + [c_int] + [c_vp] * 4 + [c_int] * 10 + [c_i64] * 12 + [c_float, c_int, c_vp],
+    'flyhip_sblocal_fwd_static': [c_vp] * 13 + [c_vp] * 2 + [c_int] + [c_vp] * 3 + [c_int] * 10 + [c_i64] * 12 + [c_float, c_int, c_vp],
     'flyhip_sblocal_bwd_band': [c_vp] * 12 + [c_int] * 7 + [c_float, c_int, c_vp],
     'flyhip_sblocal_bwd': [c_vp] * 14 + [c_int] * 7 + [c_float, c_int, c_vp],
     'flyhip_sbblocksparse_fwd': [c_vp] * 14 + [c_int] * 2 + [c_vp] * 4 + [c_int] * 8 + [c_i64] * 12 + [c_float, c_int, c_vp],

@@ -25,6 +25,7 @@
 #include "common.h"
 #include <math.h>
 #include <type_traits>
+#include <atomic>
 
 namespace flyhip {
 
@@ -2594,6 +2595,73 @@ extern "C" int flyhip_sblocal_fwd(const void* q, const void* k, const void* v, c
               q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss, softmax_temp,
               nullptr, nullptr, nullptr};
     return dispatch_fwd(dtype, E, 2 * mh, a, reinterpret_cast<hipStream_t>(stream));
+}
+
+// ---------------------------------------------------------------------------------------
+// flyhip_sblocal_fwd for callers that cannot allocate
+// ---------------------------------------------------------------------------------------
+// The un-normalised partial outputs of the band kernel (one per part of a query tile) live in a
+// fixed array inside the library's code object instead of a caller-provided workspace.  Every GPU
+// the library runs on holds its own copy of the array for the life of the process.
+constexpr size_t STATIC_SCRATCH_FLOATS = (size_t)4 << 20;                  // 16 MiB
+static __device__ __align__(256) float scratch[STATIC_SCRATCH_FLOATS];
+
+// The array's address on each device, resolved once per device on first use.  In host code the
+// array's name is only a handle for hipGetSymbolAddress, never an address a kernel may receive.
+constexpr int MAX_DEVICES = 64;
+static std::atomic<float*> g_scratch_ptr[MAX_DEVICES];
+
+static int static_scratch(float** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(ERR_LAUNCH, "sblocal_fwd_static: hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= MAX_DEVICES) return fail(ERR_UNSUPPORTED, "sblocal_fwd_static: device index %d outside [0, %d)", dev, MAX_DEVICES);
+    float* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        // (two threads racing here resolve the same address; the second store is harmless)
+        void* sym = nullptr;
+        e = hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !sym)
+            return fail(ERR_LAUNCH, "sblocal_fwd_static: hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+        p = reinterpret_cast<float*>(sym);
+        g_scratch_ptr[dev].store(p, std::memory_order_release);
+    }
+    *out = p;
+    return OK;
+}
+
+extern "C" int flyhip_sblocal_fwd_static(const void* q, const void* k, const void* v, const float* proj,
+                                         const void* kfeat, const float* chunk_scale,
+                                         float* kv, float* ksum, float* kmax,
+                                         const float* qfeat, const float* q_lsq, const void* vt, const void* kvt,
+                                         const float* kv_part, const float* part_max, int n_split,
+                                         const int64_t* key_lengths, void* out, float* log_norm,
+                                         int n_parts,
+                                         int B, int H, int T, int S, int E, int D, int mh, int mh_valid,
+                                         int local_context,
+                                         int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                                         int64_t k_sb, int64_t k_sh, int64_t k_ss,
+                                         int64_t v_sb, int64_t v_sh, int64_t v_ss,
+                                         int64_t o_sb, int64_t o_sh, int64_t o_ss,
+                                         float softmax_temp, int dtype, void* stream) {
+    FLY_REQUIRE(B > 0 && H > 0 && T > 0 && D > 0, "sblocal_fwd_static: empty problem");
+    FLY_REQUIRE(n_parts >= 1 && n_parts <= 64, "sblocal_fwd_static: n_parts=%d outside [1, 64]", n_parts);
+    float* ws = nullptr;
+    if (n_parts > 1) {
+        // the partials of flyhip_sblocal_fwd's part_ws: every part writes all 64 rows of its tile and its
+        // five statistics before the merge kernel reads them, so nothing has to start at zero
+        const size_t need = (size_t)B * H * ((T + TQ - 1) / TQ) * n_parts * TQ * (size_t)(D + NSTAT);
+        FLY_REQUIRE(need <= STATIC_SCRATCH_FLOATS,
+                    "sblocal_fwd_static: the partial outputs of this problem need %zu floats, the built-in scratch "
+                    "holds %zu (B*H*ceil(T/64)*n_parts*64*(D+5) must not exceed it); use flyhip_sblocal_fwd with a "
+                    "caller-allocated part_ws", need, STATIC_SCRATCH_FLOATS);
+        int rc = static_scratch(&ws);
+        if (rc) return rc;
+    }
+    return flyhip_sblocal_fwd(q, k, v, proj, kfeat, chunk_scale, kv, ksum, kmax, qfeat, q_lsq, vt, kvt, kv_part, part_max,
+                              n_split, key_lengths, out, log_norm, ws, n_parts, B, H, T, S, E, D, mh, mh_valid,
+                              local_context, q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss,
+                              softmax_temp, dtype, stream);
 }
 
 extern "C" int flyhip_sbblocksparse_fwd(const void* q, const void* k, const void* v, const float* proj,

@@ -97,6 +97,21 @@ class SBLocalPlan:
                   v.stride(0), v.stride(2), v.stride(1), out.stride(0), out.stride(2), out.stride(1),
                   t, self.code, stream)
 
+    def run_queries_static(self, q, k, v, proj, lens, local_context, t, out, log_norm, stream=None):
+        """``run_queries`` through flyhip_sblocal_fwd_static: the partial outputs go to the library's
+        built-in scratch array instead of ``self.part_ws`` (nothing is allocated by the call)."""
+        B, H, T, S, dim, mh, mh_valid = self.shape
+        stream = _lib.stream_ptr(self.device) if stream is None else stream
+        _lib.call('flyhip_sblocal_fwd_static', q.data_ptr(), k.data_ptr(), v.data_ptr(), proj.data_ptr(),
+                  self.kfeat.data_ptr(), self.chunk_scale.data_ptr(), self.kv.data_ptr(),
+                  self.ksum.data_ptr(), self.kmax.data_ptr(), _lib.ptr(self.qfeat), _lib.ptr(self.q_lsq),
+                  _lib.ptr(self.vt), _lib.ptr(self.kvt), self.kv_part.data_ptr(), self.part_max.data_ptr(),
+                  self.n_split, _lib.ptr(lens), out.data_ptr(), log_norm.data_ptr(), self.n_parts,
+                  B, H, T, S, dim, dim, mh, mh_valid, local_context,
+                  q.stride(0), q.stride(2), q.stride(1), k.stride(0), k.stride(2), k.stride(1),
+                  v.stride(0), v.stride(2), v.stride(1), out.stride(0), out.stride(2), out.stride(1),
+                  t, self.code, stream)
+
     def run_block_sparse(self, q, k, v, proj, t, tables, out, log_norm):
         """Scatterbrain attention whose exact part lives on a block-sparse support instead of a band: the
         key pass as in ``run``, then the fp32 band kernel walking lists of 32-key blocks (``tables`` =

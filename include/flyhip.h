@@ -98,6 +98,30 @@ int flyhip_sblocal_fwd(const void* q, const void* k, const void* v, const float*
                        int64_t o_sb, int64_t o_sh, int64_t o_ss,
                        float softmax_temp, int dtype, void* stream);
 
+/* flyhip_sblocal_fwd for callers that cannot allocate device memory -- code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.
+ * Same arguments and results as flyhip_sblocal_fwd except that there is no part_ws: the partial
+ * outputs of the parts of a query tile go to a fixed 16 MiB array inside the library (one copy per
+ * GPU, held until the process ends).  The call allocates and frees nothing.  It fails with a
+ * message when B*H*ceil(T/64)*n_parts*64*(D+5) exceeds 4 Mi floats (n_parts > 1 only; with
+ * n_parts == 1 no scratch is used).  All calls on one GPU share that array: calls that overlap in
+ * time on one GPU (different streams or threads) race.  Its address is looked up on the first call
+ * on each device, with that device current; make that first call outside a graph capture. */
+int flyhip_sblocal_fwd_static(const void* q, const void* k, const void* v, const float* proj,
+                              const void* kfeat, const float* chunk_scale,
+                              float* kv, float* ksum, float* kmax,
+                              const float* qfeat, const float* q_lsq, const void* vt, const void* kvt,
+                              const float* kv_part, const float* part_max, int n_split,
+                              const int64_t* key_lengths, void* out, float* log_norm,
+                              int n_parts,
+                              int B, int H, int T, int S, int E, int D, int mh, int mh_valid,
+                              int local_context,
+                              int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                              int64_t k_sb, int64_t k_sh, int64_t k_ss,
+                              int64_t v_sb, int64_t v_sh, int64_t v_ss,
+                              int64_t o_sb, int64_t o_sh, int64_t o_ss,
+                              float softmax_temp, int dtype, void* stream);
+
 /* Band terms of the backward pass of Scatterbrain-local attention (the reference differentiates its op
  * sequence sblocal_attention.py:90-122 with autograd and the backward kernels of
  * fast_transformers.local_product).  For a (query i, key s) pair inside the band, with
