@@ -67,25 +67,21 @@ class matmul:
             raise NotImplementedError('Supported modes are: sdd, dsd, dds')
         if block not in _BLOCKS:
             raise NotImplementedError(f'block size {block} not in {_BLOCKS}')
+        assert layout.ndim in (2, 3), "Layout should be a 2 or 3 dimensional tensor of 0s and 1s"
+        self.block, self.mode, self.trans_a, self.trans_b = block, mode, trans_a, trans_b
         self.lut_cache = dict()
-        self.block = block
-        self.mode = mode
-        self.trans_a = trans_a
-        self.trans_b = trans_b
-        layout_dim = layout.ndim
-        assert layout_dim in (2, 3), "Layout should be a 2 or 3 dimensional tensor of 0s and 1s"
-        if not mode == 'sdd':
-            # which dim of the dense operand is contracted, and its required size (:639-646)
-            trans_dense, trans_sparse, sparse_inner = (trans_b, trans_a, -1) if mode == 'dsd' else (trans_a, trans_b, -2)
-            self.dense_inner_dim = -((sparse_inner % 2) + 1) if not trans_dense else sparse_inner
-            sparse_inner = sparse_inner if not trans_sparse else -((sparse_inner % 2) + 1)
-            self.dense_inner_size = layout.shape[sparse_inner] * block
-            self.sparse_shape = (layout.sum().item(), block, block)
-        if layout_dim == 2:
-            layout = layout.unsqueeze(0)
-        layout = layout.long()
-        self.layout = layout
-        self.spdims = layout.shape
+        self.layout = _as_heads(layout)            # (H, block-rows, block-cols), integral; 2-D means one head
+        self.spdims = self.layout.shape
+        if mode != 'sdd':
+            # The contraction runs over one axis of the sparse operand's layout and one dim of the dense
+            # operand: sparse first ('dsd') contracts its columns unless transposed, and meets dim -2 of
+            # op(b); dense first ('dds') contracts dim -1 of op(a) with the sparse operand's rows.
+            if mode == 'dsd':
+                layout_axis, self.dense_inner_dim = (-2 if trans_a else -1), (-1 if trans_b else -2)
+            else:
+                layout_axis, self.dense_inner_dim = (-1 if trans_b else -2), (-2 if trans_a else -1)
+            self.dense_inner_size = self.layout.shape[layout_axis] * block
+            self.sparse_shape = (int(self.layout.sum()), block, block)
 
     # ------------------------------------------------------------------ tables
     def _table(self, kind, device):
@@ -122,33 +118,30 @@ class matmul:
         return c
 
     def _validate_inputs(self, a, b):
+        """Device, dtype and shape checks with the reference's messages (:678-702); returns both
+        operands as 4-D views (leading singleton dims added)."""
         if a.device != b.device:
             raise ValueError(f"Inputs must be on the same device; got {a.device} for tensor A "
                              f"and {b.device} for tensor B")
         if not a.is_cuda:
             raise ValueError("Only GPU devices are supported for now")
-        if torch.is_autocast_enabled():
+        if torch.is_autocast_enabled():            # like torch.matmul under autocast
             a, b = a.half(), b.half()
         elif a.dtype != b.dtype:
             raise ValueError(f"Inputs must be the same dtype; got {a.dtype} for A and {b.dtype} for B")
         if self.mode != 'sdd':
-            dense, dense_name, sparse, sparse_name = (a, 'A', b, 'B') if self.mode == 'dds' else (b, 'B', a, 'A')
-            dense_inner = dense.shape[self.dense_inner_dim]
-            if dense_inner != self.dense_inner_size:
+            (dense, dense_name), (sparse, sparse_name) = ((a, 'A'), (b, 'B')) if self.mode == 'dds' else ((b, 'B'), (a, 'A'))
+            got = dense.shape[self.dense_inner_dim]
+            if got != self.dense_inner_size:
                 raise ValueError(f"Expected tensor {dense_name} to have size {self.dense_inner_size} at dim "
-                                 f"{self.dense_inner_dim % dense.ndim}, got {dense_inner}.")
-            if sparse.shape[-len(self.sparse_shape):] != self.sparse_shape:
+                                 f"{self.dense_inner_dim % dense.ndim}, got {got}.")
+            if tuple(sparse.shape[-3:]) != self.sparse_shape:
                 raise ValueError(f"Expected tensor with trailing dimensions of shape {self.sparse_shape} for argument "
                                  f"{sparse_name}, got {sparse.shape}")
-
-        def add_extra_dims(x):
-            dims_needed = 4 - x.ndim
-            if dims_needed > 0:
-                x = x.view(*([1] * dims_needed), *x.shape)
-            elif dims_needed < 0:
+        for x in (a, b):
+            if x.ndim > 4:
                 raise ValueError("Tensors with more than 4 dimensions are not currently supported")
-            return x
-        return add_extra_dims(a), add_extra_dims(b)
+        return tuple(x.reshape((1,) * (4 - x.ndim) + tuple(x.shape)) if x.ndim < 4 else x for x in (a, b))
 
     # ------------------------------------------------------------------ kernels
     def _run(self, mode, a, b, trans_a, trans_b, trans_c):
@@ -173,6 +166,8 @@ class matmul:
         if a.shape[1] != H or b.shape[1] != H or b.shape[0] != Z or M != p * self.block or N != r * self.block:
             raise ValueError(f'SDD operands {tuple(a.shape)}, {tuple(b.shape)} do not match layout '
                              f'{tuple(self.spdims)} with block {self.block}')
+        if int(self.layout.sum()) == 0:              # a layout without blocks: nothing to compute or launch
+            return torch.empty((Z, 0, self.block, self.block), dtype=a.dtype, device=a.device)
         if (trans_a and not trans_b and self.block == 32 and a.dtype in (torch.bfloat16, torch.float16)
                 and K >= KMAJOR_MIN_K and a.stride(3) == 1 and b.stride(3) == 1
                 and all(s % 8 == 0 for s in a.stride()[:3] + b.stride()[:3])):
@@ -260,6 +255,10 @@ class matmul:
                       a.stride(0), a.stride(1), a_sm, a_sk, b.stride(0),
                       c.stride(0), c.stride(1), c_sm, c_sn, _lib.dtype_code(a), _lib.stream_ptr(a.device))
         return c
+
+
+def _as_heads(layout):
+    return (layout.unsqueeze(0) if layout.ndim == 2 else layout).long()
 
 
 def _dim_to_name(x):

@@ -89,12 +89,17 @@ class _SoftmaxFn(torch.autograd.Function):
         ctx.mark_dirty(x)
         ctx.save_for_backward(x)
         ctx.op, ctx.scale = op, scale
+        ctx.masked = kpm_args[0] is not None or am_args[0] is not None
         return x
 
     @staticmethod
     def backward(ctx, dy):
         (y,) = ctx.saved_tensors
         op = ctx.op
+        if ctx.masked:
+            # a row whose every entry was masked came out as NaN; it has no gradient (the caller has
+            # replaced it by zeros, blocksparse_attention.py:156-158), and 0 * NaN must not leak into dx
+            y = y.nan_to_num()
         ptr, blk, col, max_nnz = op.make_lut(y.device)
         if (op.block == 32 and y.dtype in (torch.bfloat16, torch.float16) and max_nnz <= 64
                 and y.stride(0) % 8 == 0):

@@ -80,19 +80,22 @@ class SBPerformerFeatures(nn.Module):
         super().__init__()
         if not cosh:
             raise NotImplementedError('only the cosh (two-sided) feature map is implemented')
-        self.query_dims = query_dims
-        self.n_features = n_features or int(query_dims * math.log(query_dims))
-        self.ortho_scaling = ortho_scaling
-        self.orthogonal = orthogonal
-        self.softmax_temp = 1 / math.sqrt(query_dims) if softmax_temp is None else softmax_temp
-        self.cosh = cosh
-        self.redraw = math.pi
-        self.deterministic_eval = deterministic_eval
-        self.eps = eps
-        self.factory_kwargs = {'device': device, 'dtype': dtype}
-        self.register_buffer('projection_matrix',
-                             torch.zeros(self.n_features // 2, query_dims, **self.factory_kwargs))
-        self._calls = -1
+        if n_features is None or n_features == 0:
+            n_features = int(query_dims * math.log(query_dims))
+        if softmax_temp is None:
+            softmax_temp = query_dims ** -0.5
+        # `orthogonal` and `redraw` are accepted and ignored like in the reference, which fixes the redraw
+        # period to an irrational number: only call number 0 is a multiple of it
+        vars(self).update(query_dims=query_dims, n_features=n_features, ortho_scaling=ortho_scaling,
+                          softmax_temp=softmax_temp, orthogonal=orthogonal, cosh=cosh, redraw=math.pi,
+                          deterministic_eval=deterministic_eval, eps=eps,
+                          factory_kwargs=dict(device=device, dtype=dtype), _calls=-1)
+        self.register_buffer('projection_matrix', torch.zeros(self.projection_rows, query_dims, device=device, dtype=dtype))
+
+    @property
+    def projection_rows(self):
+        """Rows of the projection: each gives an exp(+.) and an exp(-.) feature."""
+        return self.n_features // 2
 
     def freeze_projection(self):
         """Keep the current ``projection_matrix`` (e.g. one loaded from a checkpoint or set by a
@@ -100,22 +103,22 @@ class SBPerformerFeatures(nn.Module):
         self._calls = 0
 
     def new_feature_map(self, device):
+        """Called once per forward by the attention layers; draws the projection when a redraw is due."""
         if self.deterministic_eval and not self.training:
             return
         self._calls += 1
-        if (self._calls % self.redraw) != 0:
-            return
-        matrix = gaussian_orthogonal_random_matrix(self.n_features // 2, self.query_dims,
-                                                   scaling=self.ortho_scaling, device=device,
-                                                   dtype=self.factory_kwargs['dtype'])
-        self.register_buffer('projection_matrix', matrix)
+        due = math.fmod(self._calls, self.redraw) == 0
+        if due:
+            self.projection_matrix = gaussian_orthogonal_random_matrix(
+                self.projection_rows, self.query_dims, scaling=self.ortho_scaling, device=device,
+                dtype=self.factory_kwargs['dtype'])
+
+    def _features(self, x, is_query, return_log):
+        return softmax_kernel(x, projection_matrix=self.projection_matrix, is_query=is_query,
+                              softmax_temp=self.softmax_temp, eps=self.eps, cosh=self.cosh, return_log=return_log)
 
     def forward_queries(self, x, return_log=False):
-        return softmax_kernel(x, projection_matrix=self.projection_matrix, is_query=True,
-                              softmax_temp=self.softmax_temp, eps=self.eps, cosh=self.cosh,
-                              return_log=return_log)
+        return self._features(x, True, return_log)
 
     def forward_keys(self, x, return_log=False):
-        return softmax_kernel(x, projection_matrix=self.projection_matrix, is_query=False,
-                              softmax_temp=self.softmax_temp, eps=self.eps, cosh=self.cosh,
-                              return_log=return_log)
+        return self._features(x, False, return_log)

@@ -90,22 +90,21 @@ class FullMask(BaseMask):
 
 
 class LengthMask(BaseMask):
-    """Rows of ones followed by zeros, given by their lengths (masking.py:159-186)."""
+    """Rows of ones followed by zeros, given by their lengths (masking.py:159-186).  ``max_len``
+    defaults to the largest length; ``device`` to the device of ``lengths``."""
 
     def __init__(self, lengths, max_len=None, device=None):
-        self._device = device or lengths.device
-        with torch.no_grad():
-            self._lengths = lengths.clone().to(self._device)
-        self._max_len = max_len or self._lengths.max()
+        self._device = lengths.device if device is None else device
+        self._lengths = lengths.detach().clone().to(self._device)
+        self._max_len = self._lengths.max() if not max_len else max_len
+        self._all_ones = bool((self._lengths == self._max_len).all())
         self._bool_matrix = None
-        self._all_ones = torch.all(self._lengths == self._max_len).item()
 
     @property
     def bool_matrix(self):
         if self._bool_matrix is None:
-            with torch.no_grad():
-                idx = torch.arange(self._max_len, device=self._device)
-                self._bool_matrix = idx.view(1, -1) < self._lengths.view(-1, 1)
+            positions = torch.arange(self._max_len, device=self._device)
+            self._bool_matrix = positions.unsqueeze(0) < self._lengths.unsqueeze(-1)
         return self._bool_matrix
 
 

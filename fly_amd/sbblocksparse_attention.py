@@ -146,7 +146,6 @@ class SBBlockSparseAttention(nn.Module):
         key = key.permute(0, 2, 1, 3).float().contiguous()
         value = value.permute(0, 2, 1, 3).float().contiguous()
 
-        self.feature_map.new_feature_map(query.device)
         q_prime, q_prime_log_scale = self.feature_map.forward_queries(query)
         k_prime, k_prime_log_scale = self.feature_map.forward_keys(key)
         prime_log_scale = q_prime_log_scale + k_prime_log_scale     # (b h t 1)

@@ -4,15 +4,15 @@ import torch
 
 
 def linear_attention_normalization(q, k, causal=False):
-    """q' . sum_s k'_s per query: (..., T, m), (..., S, m) -> (..., T)."""
+    """q' . sum_s k'_s per query: q (..., T, m), k (..., S, m) -> (..., T)."""
     if causal:
         raise NotImplementedError('causal linear attention is not part of this build')
-    return torch.einsum('...nm,...m->...n', q, k.sum(dim=-2))
+    key_total = k.sum(dim=-2).unsqueeze(-1)                   # (..., m, 1)
+    return torch.matmul(q, key_total).squeeze(-1)
 
 
 def linear_attention(q, k, v, need_weights=False):
-    """q' (k'^T v): returns ((..., T, D), attention weights or None)."""
-    k_v = torch.einsum('...nm,...nd->...md', k, v)
-    q_k_v = torch.einsum('...nm,...md->...nd', q, k_v)
-    attn = None if not need_weights else torch.einsum('...im,...jm->...ij', q, k)
-    return q_k_v, attn
+    """q' (k'^T v) without forming the (T, S) weights unless asked for: returns ((..., T, D), weights or None)."""
+    summary = torch.matmul(k.transpose(-1, -2), v)            # (..., m, D)
+    weights = torch.matmul(q, k.transpose(-1, -2)) if need_weights else None
+    return torch.matmul(q, summary), weights

@@ -193,13 +193,26 @@ class T2T_ViT(nn.Module):
 
     @staticmethod
     def _init_weights(m):
+        """Truncated-normal(0.02) weights and zero biases for every linear-like layer, the Pixelfly ones
+        (block-sparse, low-rank, sparse + low-rank) through their dense-initialisation hooks; unit / zero
+        LayerNorm affine parameters (t2t_vit.py:88-99)."""
+        from .blocksparse_linear import BlockSparseLinear
+        from .fastlinear import LowRank, SparseLRLinear
+        if isinstance(m, nn.LayerNorm):
+            nn.init.ones_(m.weight)
+            nn.init.zeros_(m.bias)
+            return
+        if not isinstance(m, (nn.Linear, BlockSparseLinear, LowRank, SparseLRLinear)):
+            return
+        if m.bias is not None:
+            nn.init.zeros_(m.bias)
+
+        def small_normal_(w):
+            return nn.init.trunc_normal_(w, std=.02)
         if isinstance(m, nn.Linear):
-            nn.init.trunc_normal_(m.weight, std=.02)
-            if m.bias is not None:
-                nn.init.constant_(m.bias, 0)
-        elif isinstance(m, nn.LayerNorm):
-            nn.init.constant_(m.bias, 0)
-            nn.init.constant_(m.weight, 1.0)
+            small_normal_(m.weight)
+        elif isinstance(m, (BlockSparseLinear, LowRank)):     # (SparseLRLinear's two halves are visited as children)
+            m.set_weights_from_dense_init(small_normal_)
 
     def forward_features(self, x):
         x = self.patch_embed(x)

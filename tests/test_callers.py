@@ -117,3 +117,28 @@ def test_published_checkpoint_names_convert_and_load():
     x = torch.randn(2, 3, 224, 224)
     assert torch.equal(src.eval()(x), dst.eval()(x))
     assert fly_amd.convert_t2t_vit_state_dict(converted).keys() == converted.keys()      # idempotent
+
+
+def test_vit_initialisation_reaches_the_pixelfly_layers():
+    """T2T_ViT._init_weights (t2t_vit.py:88-99): with Pixelfly linears plugged into the blocks' MLPs the
+    biases are zero and the weights come from a truncated normal(0.02) dense draw -- block-sparse weights
+    rescaled per block-row, low-rank factors from its projection -- not from the layers' own defaults."""
+    torch.manual_seed(0)
+    cfg = fly_amd.FlatBlockButterflySparsityConfig(4, 2, block=16)
+    lin = {'_target_': 'src.models.layers.fastlinear.SparseLRLinear',
+           'sparse_cfg': {'_target_': 'src.models.layers.blocksparse_linear.BlockSparseLinear',
+                          'sparsity_config': cfg, 'backend': 'dense'},
+           'rank': 4, 'gating': True}
+    mlp_cfg = {'_target_': 'src.models.layers.mlp.MlpCustom', 'linear1_cfg': lin, 'linear2_cfg': lin}
+    model = fly_amd.T2T_ViT(embed_dim=64, depth=1, num_heads=2, mlp_ratio=1., token_dim=16, num_classes=10,
+                            mlp_cfg=mlp_cfg)
+    fc1 = model.blocks[0].mlp.fc1
+    assert isinstance(fc1, fly_amd.SparseLRLinear)
+    assert float(fc1.bias.detach().abs().max()) == 0.0 and float(fc1.gate.bias.detach().abs().max()) == 0.0
+    # normal with std 0.02, block-rows rescaled by sqrt(cols / nonzero cols) = sqrt(4 / 3): std 0.0231
+    # (the layer's own default, uniform(+-1/8) times the same factor, has std 0.083)
+    w = fc1.sparse.weight.detach()
+    assert 0.021 < float(w.std()) < 0.025
+    # the low-rank factors reproduce a rank-4 matrix whose entries are of the dense draw's size
+    lr = (fc1.low_rank.lr_weight2 @ fc1.low_rank.lr_weight1).detach()
+    assert lr.shape == (64, 64) and float(lr.std()) < 0.02

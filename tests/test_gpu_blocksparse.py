@@ -400,6 +400,9 @@ def test_sdd_with_contraction_major_operands(p, r, K, dtype):
     ref = ob.sdd(a.double(), b.double(), layout, block, trans_a=True, trans_b=False)
     assert out.shape == ref.shape and out.dtype == dtype
     assert rel_err(out, ref) <= TOL[dtype]
+    # a layout without any block: an empty result, whichever kernel the shape would have selected
+    empty = matmul(torch.zeros_like(layout), block, 'sdd', trans_a=True, trans_b=False)(a.to(DEV), b.to(DEV))
+    assert empty.shape == (Z, 0, block, block)
 
 
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
@@ -523,6 +526,55 @@ def test_blocksparse_attention_module_gradients(masked, E, dtype):
         assert rel_err(got.float(), want) <= 3e-2, (name, rel_err(got.float(), want))
     if masked:
         assert float(kg.grad[1, 200:].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize('dtype,dropout', [(torch.float32, 0.0), (torch.bfloat16, 0.3)])
+def test_blocksparse_attention_gradients_with_fully_masked_rows(dtype, dropout):
+    """Band-only layout plus a length mask: the query rows past the band of the last valid key see no key
+    at all.  The three-op path under autograd (fp32 inputs, or training with dropout) must give finite
+    gradients, zero on padded keys -- and, without dropout, the oracle's."""
+    from fly_amd import BlockSparseAttention, LengthMask
+
+    class Cfg:
+        block = 32
+
+        def make_layout(self, seqlen):
+            nb = seqlen // self.block
+            return ob.band_layout(nb, nb, 1).unsqueeze(0).repeat(2, 1, 1)
+
+    B, T, H, E = 2, 256, 2, 64
+    print('case', dtype, dropout, flush=True)
+    g = torch.Generator().manual_seed(18)
+    q, k, v = (torch.randn(B, T, H, E, generator=g).to(dtype) for _ in range(3))
+    w = torch.randn(B, T, H, E, generator=g)
+    lengths = torch.tensor([T, 70])              # batch 1: block-rows 4.. see only masked keys
+    mod = BlockSparseAttention(Cfg(), attention_dropout=dropout, max_seq_length=T).to(DEV).train()
+    qg, kg, vg = (x.to(DEV).requires_grad_() for x in (q, k, v))
+    torch.manual_seed(0)
+    out, _ = mod(qg, kg, vg, key_padding_mask=LengthMask(lengths.to(DEV), max_len=T))
+    assert len(mod.fused_cache) == 0
+    assert float(out[1, 128:].detach().abs().max()) == 0.0
+    (out.float() * w.to(DEV)).sum().backward()
+    for grad in (qg.grad, kg.grad, vg.grad):
+        assert bool(torch.isfinite(grad).all())
+    assert float(kg.grad[1, 70:].abs().max()) == 0.0 and float(vg.grad[1, 70:].abs().max()) == 0.0
+    assert float(qg.grad[1, 128:].abs().max()) == 0.0
+    if dropout == 0.0:
+        # dense masked softmax in float64 whose rows without any visible key are zero rows (autograd through
+        # the oracle's NaN -> 0 replacement would itself yield NaN there)
+        qd, kd, vd = (x.double().requires_grad_() for x in (q, k, v))
+        lay = ob.densify_tensor(torch.ones(1, int(mod.master_layout.sum()), 32, 32), mod.master_layout.cpu())[0].bool()
+        vis = lay.unsqueeze(0) & (torch.arange(T).view(1, 1, 1, T) < lengths.view(B, 1, 1, 1))      # (B, H, T, S)
+        s = torch.einsum('bthe,bshe->bhts', qd, kd) / math.sqrt(E)
+        live = vis.any(-1, keepdim=True)
+        p = torch.softmax(torch.where(live, s.masked_fill(~vis, float('-inf')), torch.zeros_like(s)), -1) * live
+        ref = torch.einsum('bhts,bshd->bthd', p, vd)
+        (ref * w.double()).sum().backward()
+        assert rel_err(out, ref) <= 1e-4
+        assert rel_err(out, ob.blocksparse_attention(q.double(), k.double(), v.double(), mod.master_layout.cpu(), 32,
+                                                     key_lengths=lengths)) <= 1e-4
+        for got, want in ((qg.grad, qd.grad), (kg.grad, kd.grad), (vg.grad, vd.grad)):
+            assert rel_err(got, want) <= 1e-4, rel_err(got, want)
 
 
 def test_probabilities_from_log_denominators():
