@@ -47,8 +47,18 @@ __device__ long long g_prof[16384 * 8];
             if (wg_ < 16384) g_prof[wg_ * 8 + (slot)] = wall_clock64();                                  \
         }                                                                                                \
     } while (0)
+// (the key pass has its own table: its grid is two-dimensional)
+__device__ long long g_prof_k[4096 * 8];
+#define FLY_PROFK(slot)                                                                                  \
+    do {                                                                                                 \
+        if (threadIdx.x == 0) {                                                                          \
+            const int wg_ = blockIdx.y * gridDim.x + blockIdx.x;                                         \
+            if (wg_ < 4096) g_prof_k[wg_ * 8 + (slot)] = wall_clock64();                                 \
+        }                                                                                                \
+    } while (0)
 #else
 #define FLY_PROF(slot)
+#define FLY_PROFK(slot)
 #endif
 
 struct KvArgs {
@@ -225,12 +235,122 @@ __device__ __forceinline__ void store_feat(void* kfeat, long row, int M, int fbp
     }
 }
 
+// ---------------------------------------------------------------------------------------
+// fp32 inputs on the bf16 matrix pipe: operands as sums of bf16 pieces
+// ---------------------------------------------------------------------------------------
+// The band kernel for float inputs forms its three products on v_mfma_f32_16x16x32_bf16 (16 times the
+// rate of the fp32 MFMA) from operands split into bf16 pieces, x = hi + lo (+ a third piece), with
+// fp32 accumulation.  Products of bf16 pairs are exact in fp32, so a product that takes every pair of
+// pieces above the fp32 rounding level is as accurate as the fp32 MFMA:
+//   features : q', k' are ROUNDED TO 16 SIGNIFICANT BITS where they are formed (key pass), two pieces
+//              represent them exactly, and all four piece products are taken: the overlap q'.k' of the
+//              band is then the exact product of the same numbers whose sums over all keys the global
+//              low-rank term uses (also formed from the rounded features), so the "all keys minus the
+//              band" difference cancels as well as it does in fp32 arithmetic.  The rounding itself
+//              perturbs a feature by 2^-17 relative, consistently everywhere.
+//   scores   : q, k in two pieces, three products (the lo.lo product, 2^-16 relative, is dropped: an
+//              error in an exponent, not in a difference).
+//   P V      : probabilities and values in three pieces each (exact), the six products above 2^-24.
+// The key pass leaves every 32-key tile as an image of what the band kernel wants in LDS: in the
+// feature / operand scratch, per tile, [K hi][K lo][V^T h][V^T m][V^T l] (the "kv image") and
+// [K' hi][K' lo] (the "feature image"); rows of K and K' in the k-slot order of the MFMA, V
+// transposed to [d][key slot], and the 16-byte chunks of every row XOR-swizzled so that the
+// fragment reads of 8 consecutive rows fall into different LDS banks without padding.
+template <int E, int D, int M>
+struct X3Tile {
+    static constexpr int K_ROW = 2 * E, F_ROW = 2 * M, V_ROW = 2 * TK;           // bytes per row
+    static constexpr int K_PIECE = TK * K_ROW, F_PIECE = TK * F_ROW, V_PIECE = D * V_ROW;
+    static constexpr int KV_BYTES = 2 * K_PIECE + 3 * V_PIECE;                    // per tile, operand scratch
+    static constexpr int F_BYTES = 2 * F_PIECE;                                   // per tile, feature scratch
+    static constexpr int BYTES = KV_BYTES + F_BYTES;                              // one LDS stage
+};
+// chunk c of a row -> the chunk it is stored at
+__device__ __forceinline__ int x3_swz(int row, int c, int row_bytes) {
+    return row_bytes >= 128 ? (c ^ (row & 7)) : (c ^ ((row >> 1) & 3));
+}
+// an fp32 value rounded to 16 significant bits: bf16 head plus the bf16 head of the rest
+__device__ __forceinline__ float quant16(float x) {
+    const float h = bf16_to_f32(f32_to_bf16(x));
+    return h + bf16_to_f32(f32_to_bf16(x - h));
+}
+__device__ __forceinline__ floatx4 quant16(floatx4 x) {
+    floatx4 r = {quant16(x[0]), quant16(x[1]), quant16(x[2]), quant16(x[3])};
+    return r;
+}
+// eight floats -> bf16 head and remainder (eight k-slots each)
+__device__ __forceinline__ void split2(floatx4 x0, floatx4 x1, uintx4& hi, uintx4& lo) {
+    hi = uintx4{pack_bf16x2(x0[0], x0[1]), pack_bf16x2(x0[2], x0[3]), pack_bf16x2(x1[0], x1[1]), pack_bf16x2(x1[2], x1[3])};
+    floatx4 r0, r1;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t w0 = hi[i >> 1], w1 = hi[2 + (i >> 1)];
+        r0[i] = x0[i] - ((i & 1) ? __uint_as_float(w0 & 0xffff0000u) : __uint_as_float(w0 << 16));
+        r1[i] = x1[i] - ((i & 1) ? __uint_as_float(w1 & 0xffff0000u) : __uint_as_float(w1 << 16));
+    }
+    lo = uintx4{pack_bf16x2(r0[0], r0[1]), pack_bf16x2(r0[2], r0[3]), pack_bf16x2(r1[0], r1[1]), pack_bf16x2(r1[2], r1[3])};
+}
+// eight floats -> three bf16 pieces whose sum is the value exactly
+__device__ __forceinline__ void split3(floatx4 x0, floatx4 x1, uintx4& h, uintx4& m, uintx4& l) {
+    h = uintx4{pack_bf16x2(x0[0], x0[1]), pack_bf16x2(x0[2], x0[3]), pack_bf16x2(x1[0], x1[1]), pack_bf16x2(x1[2], x1[3])};
+    floatx4 r0, r1;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t w0 = h[i >> 1], w1 = h[2 + (i >> 1)];
+        r0[i] = x0[i] - ((i & 1) ? __uint_as_float(w0 & 0xffff0000u) : __uint_as_float(w0 << 16));
+        r1[i] = x1[i] - ((i & 1) ? __uint_as_float(w1 & 0xffff0000u) : __uint_as_float(w1 << 16));
+    }
+    split2(r0, r1, m, l);
+}
+// 64 rows x W floats in LDS (row stride LD floats) -> the two-piece images of the two 32-row tiles:
+// position 32ks + 8g + 4h + i of a row <- element 32ks + 16h + 4g + i (the k-slot order of the MFMA)
+template <int W, int LD>
+__device__ __forceinline__ void x3_emit_rows(const float* src, char* tile0, long tile_stride, int piece_bytes, int tid) {
+    constexpr int CH8 = W / 8, ROWB = 2 * W, TOT = CH * CH8;
+#pragma unroll
+    for (int j = 0; j < (TOT + NT - 1) / NT; ++j) {
+        const int idx = tid + NT * j;
+        if (TOT % NT == 0 || idx < TOT) {
+            const int row64 = idx / CH8, cch = idx % CH8, ks = cch >> 2, gq = cch & 3, row = row64 & (TK - 1);
+            const float* sp = src + row64 * LD + 32 * ks + 4 * gq;
+            uintx4 hi, lo;
+            split2(*reinterpret_cast<const floatx4*>(sp), *reinterpret_cast<const floatx4*>(sp + 16), hi, lo);
+            char* dst = tile0 + (row64 / TK) * tile_stride + row * ROWB + x3_swz(row, cch, ROWB) * 16;
+            *reinterpret_cast<uintx4*>(dst) = hi;
+            *reinterpret_cast<uintx4*>(dst + piece_bytes) = lo;
+        }
+    }
+}
+// 64 keys x D floats in LDS -> the three-piece transposed images [d][key slot] of the two 32-key tiles:
+// slot 8g + j of a tile <- key 16 (j / 4) + 4 g + j % 4 (the order in which score tiles leave the probabilities)
+template <int D, int LD>
+__device__ __forceinline__ void x3_emit_vt(const float* src, char* tile0, long tile_stride, int tid) {
+    constexpr int TOT = 2 * D * 4, PIECE = D * 2 * TK;
+#pragma unroll
+    for (int j = 0; j < (TOT + NT - 1) / NT; ++j) {
+        const int idx = tid + NT * j;
+        if (TOT % NT == 0 || idx < TOT) {
+            const int tile = idx / (4 * D), rem = idx % (4 * D), d = rem >> 2, gq = rem & 3;
+            const float* col = src + (TK * tile + 4 * gq) * LD + d;
+            const floatx4 x0 = {col[0], col[LD], col[2 * LD], col[3 * LD]};
+            const floatx4 x1 = {col[16 * LD], col[17 * LD], col[18 * LD], col[19 * LD]};
+            uintx4 h, m, l;
+            split3(x0, x1, h, m, l);
+            char* dst = tile0 + tile * tile_stride + d * (2 * TK) + x3_swz(d, gq, 2 * TK) * 16;
+            *reinterpret_cast<uintx4*>(dst) = h;
+            *reinterpret_cast<uintx4*>(dst + PIECE) = m;
+            *reinterpret_cast<uintx4*>(dst + 2 * PIECE) = l;
+        }
+    }
+}
+
 // two waves per SIMD (two workgroups per CU) where the register budget allows it without spilling
 constexpr int kfeat_waves(int E, int M) { return (E <= 64 && M <= 128) ? 2 : 1; }
 
-template <typename T, int E, int D, int M>
+template <typename T, int E, int D, int M, bool X3 = false>
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(kfeat_waves(E, M), kfeat_waves(E, M))))
 void sb_kfeat_kernel(KvArgs a) {
+    static_assert(!X3 || sizeof(T) == 4, "piece images are for float inputs");
+    typedef X3Tile<E, D, M> TL;
     constexpr int MH = M / 2, LDK = E + 4, LDV = D + 4, LDF = M + 4;
     constexpr int FB = MH / 16, EC = E / 16, DB = D / 16;
     constexpr int RB = (M / 16 + 3) / 4;         // K'^T V row blocks per wave
@@ -247,6 +367,7 @@ void sb_kfeat_kernel(KvArgs a) {
     // global memory: the matrix is small and stays in the L1/L2 caches
     const float* pp = a.proj + r16 * E + 4 * g;
 
+    FLY_PROFK(0);
     if (sp >= a.n_split) {
         // Query role (workgroups past the key splits, present when the caller asks for query
         // features): q' = exp(+-sqrt(t) P q - max) of 64 queries, one per lane column, with the
@@ -295,11 +416,13 @@ void sb_kfeat_kernel(KvArgs a) {
                     fp[i] = ok ? __expf(qf[fb][i] - qmax) : 0.f;
                     fn[i] = ok ? __expf(-qf[fb][i] - qmax) : 0.f;
                 }
+                if (X3) { fp = quant16(fp); fn = quant16(fn); }
                 *reinterpret_cast<floatx4*>(dst + 16 * fb + 4 * g) = fp;
                 *reinterpret_cast<floatx4*>(dst + MH + 16 * fb + 4 * g) = fn;
             }
             if (g == 0) a.q_lsq[(long)bh * a.T + iq] = -diag_q + qmax - 0.5f * __logf(2.0f * a.mh_valid);
         }
+        FLY_PROFK(6);
         return;
     }
 
@@ -323,6 +446,7 @@ void sb_kfeat_kernel(KvArgs a) {
     }
     __syncthreads();
 
+    FLY_PROFK(1);
     floatx4 kvacc[RB][DB];
 #pragma unroll
     for (int x = 0; x < RB; ++x)
@@ -352,6 +476,16 @@ void sb_kfeat_kernel(KvArgs a) {
             kt.fetch(kptr, a.k_ss, s_base + CH, a.S - 1, tid);
             vt.fetch(vptr, a.v_ss, s_base + CH, a.S - 1, tid);
         }
+        char* kv_img = nullptr;
+        char* f_img = nullptr;
+        if (X3) {
+            // the chunk's two 32-key tiles as the band kernel wants them in LDS: K in two bf16 pieces, V transposed in three
+            kv_img = reinterpret_cast<char*>(a.vt) + ((long)bh * a.n_chunks + c) * (2 * (long)TL::KV_BYTES);
+            f_img = reinterpret_cast<char*>(a.kfeat) + ((long)bh * a.n_chunks + c) * (2 * (long)TL::F_BYTES);
+            x3_emit_rows<E, LDK>(Ks, kv_img, TL::KV_BYTES, TL::K_PIECE, tid);
+            x3_emit_vt<D, LDV>(Vs, kv_img + 2 * TL::K_PIECE, TL::KV_BYTES, tid);
+        }
+        FLY_PROFK(2);
         // projection of this wave's 16 keys, all feature blocks advancing together:
         // dd[fb][i] = log2(e) * (sqrt(t) P)[16fb+4g+i] . k[16w+r16]
         floatx4 kb[EC];
@@ -394,8 +528,13 @@ void sb_kfeat_kernel(KvArgs a) {
         const float new_max = fmaxf(run_max, lmax);
         const long frow_g = (long)bh * a.n_chunks * CH + s_base + 16 * w + r16;      // this lane's key row
         if (new_max == -INFINITY) {   // no valid key yet (workgroup-uniform): features are zero
+            if (X3) {
+                for (int idx = tid; idx < 2 * TL::F_BYTES / 16; idx += NT)
+                    reinterpret_cast<uintx4*>(f_img)[idx] = uintx4{0u, 0u, 0u, 0u};
+            }
 #pragma unroll
             for (int fb = 0; fb < FB; ++fb) {
+                if (X3) break;
                 store_feat<T>(a.kfeat, frow_g, M, fb, g, Frag<float>::zero());
                 store_feat<T>(a.kfeat, frow_g, M, FB + fb, g, Frag<float>::zero());
             }
@@ -418,15 +557,21 @@ void sb_kfeat_kernel(KvArgs a) {
                     fp[i] = ok ? __builtin_amdgcn_exp2f(dd[fb][i] + off) : 0.f;
                     fn[i] = ok ? __builtin_amdgcn_exp2f(-dd[fb][i] + off) : 0.f;
                 }
+                if (X3) { fp = quant16(fp); fn = quant16(fn); }     // every later use sees the rounded features
                 ksp[fb] = ksp[fb] * rescale + fp;
                 ksn[fb] = ksn[fb] * rescale + fn;
                 *reinterpret_cast<floatx4*>(frow_s + 16 * fb + 4 * g) = fp;
                 *reinterpret_cast<floatx4*>(frow_s + MH + 16 * fb + 4 * g) = fn;
-                store_feat<T>(a.kfeat, frow_g, M, fb, g, fp);
-                store_feat<T>(a.kfeat, frow_g, M, FB + fb, g, fn);
+                if (!X3) {
+                    store_feat<T>(a.kfeat, frow_g, M, fb, g, fp);
+                    store_feat<T>(a.kfeat, frow_g, M, FB + fb, g, fn);
+                }
             }
             if (tid == 0) a.chunk_scale[(long)bh * a.n_chunks + c] = new_max * LN2;    // stored in natural-log units
             __syncthreads();
+            FLY_PROFK(3);
+            if (X3) x3_emit_rows<M, LDF>(Fs, f_img, TL::F_BYTES, TL::F_PIECE, tid);
+            FLY_PROFK(4);
             // KV[r][d] += sum_keys F[key][r] V[key][d]; lane ends with KV[16rb+4g+i][16db+r16]
 #pragma unroll
             for (int kk = 0; kk < CH / 16; ++kk) {
@@ -451,6 +596,7 @@ void sb_kfeat_kernel(KvArgs a) {
                 }
             }
         }
+        FLY_PROFK(5);
         __syncthreads();                          // everyone is done with this chunk's tiles
         if (c + 1 < c1) {
             kt.template stash<LDK>(Ks, tid);
@@ -486,6 +632,7 @@ void sb_kfeat_kernel(KvArgs a) {
     __syncthreads();
     if (tid < M) part[M * D + tid] = (ks_lds[tid] + ks_lds[M + tid]) + (ks_lds[2 * M + tid] + ks_lds[3 * M + tid]);
     if (tid == 0) a.part_max[(long)bh * a.n_split + sp] = run_max * LN2;
+    FLY_PROFK(6);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -590,6 +737,9 @@ struct TileKV16 {
 };
 
 __device__ __forceinline__ floatx4 mma_bf16(uint4 a, uint4 b, floatx4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+__device__ __forceinline__ floatx4 mma_bf16(uintx4 a, uintx4 b, floatx4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
 }
 
@@ -1835,6 +1985,351 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
     FLY_PROF(5);
 }
 
+// ---------------------------------------------------------------------------------------
+// fused band kernel for float inputs on the bf16 matrix pipe (operands in bf16 pieces)
+// ---------------------------------------------------------------------------------------
+// Same work decomposition, masks, online softmax and outputs as sblocal_fwd_kernel; the three products
+// of the key loop run on v_mfma_f32_16x16x32_bf16 from the tile images the key pass has left (see
+// X3Tile): per 32-key tile and wave 12 MFMAs for the scores (three piece products), 4 M / 16 for the
+// overlap (four), 6 D / 16 for P V (six) instead of (E + M + D) / 2 fp32 MFMAs of twice the duration.
+// A tile image is copied global -> registers -> LDS as it is (16-byte pieces in thread order), two LDS
+// stages.
+template <int E, int D, int M, bool SPLIT>
+__global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
+    typedef X3Tile<E, D, M> TL;
+    constexpr int MH = M / 2, LDK = E + 4, LDV = D + 4;
+    constexpr int FB = MH / 16, EC = E / 16, DB = D / 16, KB = TK / 16, KS = E / 32, FS = M / 32;
+    static_assert(KB == 2 && TK == 32, "one P V step per tile: eight k-slots per lane are the lane's two score quads");
+    extern __shared__ __attribute__((aligned(128))) float smem[];
+    char* lds = reinterpret_cast<char*>(smem);
+    float* Ps = smem;                                  // only live before the key loop
+
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
+    if (SPLIT && (int)blockIdx.x >= a.band_wgs) {       // combine role, see sblocal_fwd_kernel
+        const int ci = blockIdx.x - a.band_wgs;
+        sb_combine_body(smem, a.kv_part, a.part_max, const_cast<float*>(a.kv), const_cast<float*>(a.ksum),
+                        const_cast<float*>(a.kmax), nullptr, ci / a.cmb_wpb, ci % a.cmb_wpb, a.cmb_wpb, a.n_split, M, D);
+        return;
+    }
+    const int n_qt = (a.T + TQ - 1) / TQ;
+    const int n_items = a.B * a.H * n_qt * a.n_parts;
+    const int per_xcd = (n_items + N_XCD - 1) / N_XCD;
+    const int item = (blockIdx.x % N_XCD) * per_xcd + blockIdx.x / N_XCD;   // see sblocal_fwd_kernel
+    if (item >= n_items) return;                       // workgroup-uniform
+    const int part = item % a.n_parts;
+    const int qt = (item / a.n_parts) % n_qt;
+    const int bh = item / (a.n_parts * n_qt), b = bh / a.H, h = bh % a.H;
+    const int q0 = qt * TQ;
+    const int iq = q0 + 16 * w + r16;
+    const bool qvalid = iq < a.T;
+    const float* qptr = reinterpret_cast<const float*>(a.q) + b * a.q_sb + h * a.q_sh;
+    const char* kv_img = reinterpret_cast<const char*>(a.vt) + (long)bh * a.n_chunks * (2 * (long)TL::KV_BYTES);
+    const char* f_img = reinterpret_cast<const char*>(a.kfeat) + (long)bh * a.n_chunks * (2 * (long)TL::F_BYTES);
+    const int len = a.lens ? min((int)a.lens[b], a.S) : a.S;
+    const float lnm_half = 0.5f * __logf(2.0f * a.mh_valid);
+    const int lc_lo = a.lc / 2, lc_hi = (a.lc + 1) / 2;    // band: -lc_lo <= s - i < lc_hi
+
+    FLY_PROF(0);
+    const int q_last = min(q0 + TQ - 1, a.T - 1);
+    const int lo = max(0, q0 - lc_lo);
+    const int hi = min(len, q_last + lc_hi);
+    int kt_lo = lo / TK;
+    int kt_hi = (hi > lo) ? (hi + TK - 1) / TK : kt_lo;
+    if (SPLIT) {
+        const int nt = kt_hi - kt_lo, base = nt / a.n_parts, extra = nt % a.n_parts;
+        const int first = kt_lo + part * base + min(part, extra);
+        kt_lo = first;
+        kt_hi = first + base + (part < extra ? 1 : 0);
+    }
+
+    // tile images: flat copies, 16-byte pieces in thread order
+    constexpr int NKV = (TL::KV_BYTES / 16 + NT - 1) / NT, NF = (TL::F_BYTES / 16 + NT - 1) / NT;
+    constexpr bool KV_EXACT = TL::KV_BYTES / 16 % NT == 0, F_EXACT = TL::F_BYTES / 16 % NT == 0;
+    uintx4 rkv[NKV], rf[NF];
+    auto fetch = [&](int kt) __attribute__((always_inline)) {
+        const uintx4* gk = reinterpret_cast<const uintx4*>(kv_img + (long)kt * TL::KV_BYTES);
+        const uintx4* gf = reinterpret_cast<const uintx4*>(f_img + (long)kt * TL::F_BYTES);
+#pragma unroll
+        for (int j = 0; j < NKV; ++j)
+            if (KV_EXACT || tid + NT * j < TL::KV_BYTES / 16) rkv[j] = gk[tid + NT * j];
+#pragma unroll
+        for (int j = 0; j < NF; ++j)
+            if (F_EXACT || tid + NT * j < TL::F_BYTES / 16) rf[j] = gf[tid + NT * j];
+    };
+    auto stash = [&](int stage) __attribute__((always_inline)) {
+        uintx4* dk = reinterpret_cast<uintx4*>(lds + stage * TL::BYTES);
+        uintx4* df = reinterpret_cast<uintx4*>(lds + stage * TL::BYTES + TL::KV_BYTES);
+#pragma unroll
+        for (int j = 0; j < NKV; ++j)
+            if (KV_EXACT || tid + NT * j < TL::KV_BYTES / 16) dk[tid + NT * j] = rkv[j];
+#pragma unroll
+        for (int j = 0; j < NF; ++j)
+            if (F_EXACT || tid + NT * j < TL::F_BYTES / 16) df[tid + NT * j] = rf[j];
+    };
+    if (kt_lo < kt_hi) fetch(kt_lo);
+    const float* csp = a.chunk_scale + (long)bh * a.n_chunks;
+    float cscale = (kt_lo < kt_hi) ? csp[kt_lo * TK / CH] : 0.f;
+    const float kmax = SPLIT ? split_kmax(a.part_max, bh, a.n_split) : a.kmax[bh];
+
+    // query operand: lane (r16, g) holds elements 16c + 4g + i of its query row
+    floatx4 qr[EC];
+    float sq = 0.f;
+#pragma unroll
+    for (int c = 0; c < EC; ++c) {
+        qr[c] = Frag<float>::zero();
+        if (qvalid) qr[c] = load4_f32(qptr + (long)iq * a.q_ss + 16 * c + 4 * g);
+        sq += qr[c][0] * qr[c][0] + qr[c][1] * qr[c][1] + qr[c][2] * qr[c][2] + qr[c][3] * qr[c][3];
+    }
+    const float diag_q = 0.5f * a.temp * group_sum(sq);
+
+    // query features rounded to 16 bits, as two bf16 pieces in B-operand order (k-slot 8g + 4h + i of step ks
+    // = feature 32 ks + 16 h + 4 g + i, i.e. blocks 2 ks and 2 ks + 1 of the lane's features)
+    uintx4 qfh[FS], qfl[FS];
+    float lsq;
+    {
+        floatx4 qf[2 * FB];
+        if (SPLIT) {
+            const long qrow = (long)bh * a.T + min(iq, a.T - 1);
+#pragma unroll
+            for (int c = 0; c < 2 * FB; ++c) qf[c] = *reinterpret_cast<const floatx4*>(a.qfeat + qrow * M + 16 * c + 4 * g);
+            lsq = a.q_lsq[qrow];
+        } else {
+            load_proj<E, MH>(Ps, a.proj, sqrtf(a.temp), tid);
+            __syncthreads();
+            float qmax = 0.f;
+#pragma unroll
+            for (int fb = 0; fb < FB; ++fb) qf[fb] = Frag<float>::zero();
+#pragma unroll
+            for (int c = 0; c < EC; ++c) {
+                floatx4 pa[FB];
+#pragma unroll
+                for (int fb = 0; fb < FB; ++fb)
+                    pa[fb] = *reinterpret_cast<const floatx4*>(Ps + (16 * fb + r16) * LDK + 16 * c + 4 * g);
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int fb = 0; fb < FB; ++fb)
+                        qf[fb] = __builtin_amdgcn_mfma_f32_16x16x4f32(pa[fb][j], qr[c][j], qf[fb], 0, 0, 0);
+            }
+#pragma unroll
+            for (int fb = 0; fb < FB; ++fb)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (16 * fb + 4 * g + i < a.mh_valid) qmax = fmaxf(qmax, fabsf(qf[fb][i]));
+            qmax = group_max(qmax);
+            lsq = -diag_q + qmax - lnm_half;
+#pragma unroll
+            for (int fb = 0; fb < FB; ++fb) {
+                floatx4 dd = qf[fb];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const bool ok = 16 * fb + 4 * g + i < a.mh_valid;
+                    qf[fb][i] = ok ? quant16(__expf(dd[i] - qmax)) : 0.f;
+                    qf[FB + fb][i] = ok ? quant16(__expf(-dd[i] - qmax)) : 0.f;
+                }
+            }
+            __syncthreads();      // Ps is dead; the tile buffers may overwrite it
+        }
+#pragma unroll
+        for (int ks = 0; ks < FS; ++ks) split2(qf[2 * ks], qf[2 * ks + 1], qfh[ks], qfl[ks]);   // exact: 16-bit values
+    }
+    FLY_PROF(1);
+
+    // From here on all exponents are base 2: the score operand carries t log2(e)
+    constexpr float LOG2E = 1.4426950408889634f, LN2 = 0.6931471805599453f;
+    const float c0 = (lsq + kmax) * LOG2E;       // base-2 log-scale of the global low-rank term
+    uintx4 qh[KS], ql[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) split2(qr[2 * ks] * (a.temp * LOG2E), qr[2 * ks + 1] * (a.temp * LOG2E), qh[ks], ql[ks]);
+    float m_run = c0;
+    float ze = 0.f, zp = 0.f;
+    floatx4 oacc[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) oacc[db] = Frag<float>::zero();
+    const int qw0 = q0 + 16 * w;
+    const int smin = max(iq - lc_lo, 0);
+    const unsigned span = qvalid ? (unsigned)max(min(iq + lc_hi, len) - smin, 0) : 0u;
+
+    // fragment addresses inside a stage (bytes): rows 16 kb + r16 share the swizzle of r16
+    int koff[KS], foff[FS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) koff[ks] = r16 * TL::K_ROW + x3_swz(r16, 4 * ks + g, TL::K_ROW) * 16;
+#pragma unroll
+    for (int ks = 0; ks < FS; ++ks) foff[ks] = TL::KV_BYTES + r16 * TL::F_ROW + x3_swz(r16, 4 * ks + g, TL::F_ROW) * 16;
+    const int voff = 2 * TL::K_PIECE + r16 * TL::V_ROW + x3_swz(r16, g, TL::V_ROW) * 16;
+
+    if (kt_lo < kt_hi) stash(0);
+    __syncthreads();
+
+    FLY_PROF(2);
+    for (int kt = kt_lo; kt < kt_hi; ++kt) {
+        const int s_base = kt * TK;
+        const int cur = (kt - kt_lo) & 1;
+        const char* st = lds + cur * TL::BYTES;
+        const bool more = kt + 1 < kt_hi;
+        float cscale_next = cscale;
+        if (more) {                                      // next tile's loads fly during the MFMAs
+            fetch(kt + 1);
+            cscale_next = csp[(s_base + TK) / CH];
+        }
+        const float wc = __builtin_amdgcn_exp2f((cscale - kmax) * LOG2E);
+        const bool any = !(s_base + TK - 1 - qw0 < -lc_lo || s_base - (qw0 + 15) >= lc_hi || s_base >= len);
+        if (any) {
+            floatx4 s1[KB], s2[KB];
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) { s1[kb] = Frag<float>::zero(); s2[kb] = Frag<float>::zero(); }
+            // scores: three piece products, smallest first
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb) {
+                    const uintx4 khi = *reinterpret_cast<const uintx4*>(st + koff[ks] + 16 * kb * TL::K_ROW);
+                    const uintx4 klo = *reinterpret_cast<const uintx4*>(st + koff[ks] + 16 * kb * TL::K_ROW + TL::K_PIECE);
+                    s1[kb] = mma_bf16(klo, qh[ks], s1[kb]);
+                    s1[kb] = mma_bf16(khi, ql[ks], s1[kb]);
+                    s1[kb] = mma_bf16(khi, qh[ks], s1[kb]);
+                }
+            // overlap: all four piece products (exact product of the rounded features)
+#pragma unroll
+            for (int ks = 0; ks < FS; ++ks)
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb) {
+                    const uintx4 fhi = *reinterpret_cast<const uintx4*>(st + foff[ks] + 16 * kb * TL::F_ROW);
+                    const uintx4 flo = *reinterpret_cast<const uintx4*>(st + foff[ks] + 16 * kb * TL::F_ROW + TL::F_PIECE);
+                    s2[kb] = mma_bf16(flo, qfl[ks], s2[kb]);
+                    s2[kb] = mma_bf16(flo, qfh[ks], s2[kb]);
+                    s2[kb] = mma_bf16(fhi, qfl[ks], s2[kb]);
+                    s2[kb] = mma_bf16(fhi, qfh[ks], s2[kb]);
+                }
+            const bool interior = s_base - (qw0 + 15) >= -lc_lo && s_base + TK - 1 - qw0 < lc_hi &&
+                                  s_base + TK <= len && qw0 + 15 < a.T;
+            floatx4 p[KB];
+            float ovs = 0.f;
+            auto soft = [&](auto masked_tag) __attribute__((always_inline)) {
+                constexpr bool MASKED = decltype(masked_tag)::value;
+                bool ok[KB][4];
+                float mx = -INFINITY;
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int s = s_base + 16 * kb + 4 * g + i;
+                        ok[kb][i] = !MASKED || (unsigned)(s - smin) < span;
+                        mx = fmaxf(mx, ok[kb][i] ? s1[kb][i] : -INFINITY);
+                    }
+                mx = group_max(mx);
+                if (__builtin_amdgcn_ballot_w64(mx > m_run + 8.f) != 0) {      // wave-uniform
+                    const float m_new = fmaxf(m_run, mx);
+                    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+                    m_run = m_new;
+                    ze *= alpha;
+#pragma unroll
+                    for (int db = 0; db < DB; ++db) oacc[db] *= alpha;
+                }
+                const float beta = wc * __builtin_amdgcn_exp2f(c0 - m_run);      // scale of the overlap term
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float e = ok[kb][i] ? __builtin_amdgcn_exp2f(s1[kb][i] - m_run) : 0.f;
+                        const float ov = ok[kb][i] ? s2[kb][i] : 0.f;
+                        ze += e;
+                        ovs += ov;
+                        p[kb][i] = e - ov * beta;
+                    }
+            };
+            if (interior) soft(std::false_type{}); else soft(std::true_type{});
+            zp += ovs * wc;
+            // O^T[d][query] += sum_keys V[key][d] p[key][query]: P exactly in three pieces, six products
+            uintx4 ph, pm, pl;
+            split3(p[0], p[1], ph, pm, pl);
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                const uintx4 vh = *reinterpret_cast<const uintx4*>(st + voff + 16 * db * TL::V_ROW);
+                const uintx4 vm = *reinterpret_cast<const uintx4*>(st + voff + 16 * db * TL::V_ROW + TL::V_PIECE);
+                const uintx4 vl = *reinterpret_cast<const uintx4*>(st + voff + 16 * db * TL::V_ROW + 2 * TL::V_PIECE);
+                floatx4 o = oacc[db];
+                o = mma_bf16(vl, ph, o);
+                o = mma_bf16(vh, pl, o);
+                o = mma_bf16(vm, pm, o);
+                o = mma_bf16(vm, ph, o);
+                o = mma_bf16(vh, pm, o);
+                o = mma_bf16(vh, ph, o);
+                oacc[db] = o;
+            }
+        }
+        if (more) stash(cur ^ 1);
+        cscale = cscale_next;
+        __syncthreads();
+    }
+
+    FLY_PROF(3);
+    floatx4 lacc[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) lacc[db] = Frag<float>::zero();
+    float qk1 = 0.f;
+    if (!SPLIT) {
+        // global low-rank term on the fp32 MFMA from the rounded query features (hi + lo is exact)
+        float* KVs = smem;
+        float* KSs = smem + M * LDV;
+        {
+            RowTile<M, D> kvt;
+            kvt.fetch(a.kv + (long)bh * M * D, D, 0, M - 1, tid);
+            if (tid < M) KSs[tid] = a.ksum[(long)bh * M + tid];
+            kvt.template stash<LDV>(KVs, tid);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int c = 0; c < 2 * FB; ++c) {
+            const uintx4 hw = qfh[c >> 1], lw = qfl[c >> 1];
+            floatx4 qf;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t wh = hw[2 * (c & 1) + (i >> 1)], wl = lw[2 * (c & 1) + (i >> 1)];
+                qf[i] = ((i & 1) ? __uint_as_float(wh & 0xffff0000u) : __uint_as_float(wh << 16)) +
+                        ((i & 1) ? __uint_as_float(wl & 0xffff0000u) : __uint_as_float(wl << 16));
+            }
+            const floatx4 ks = *reinterpret_cast<const floatx4*>(KSs + 16 * c + 4 * g);
+            qk1 += qf[0] * ks[0] + qf[1] * ks[1] + qf[2] * ks[2] + qf[3] * ks[3];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+                    lacc[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(
+                        KVs[(16 * c + 4 * g + j) * LDV + 16 * db + r16], qf[j], lacc[db], 0, 0, 0);
+        }
+        qk1 = group_sum(qk1);
+    }
+    ze = group_sum(ze);
+    zp = group_sum(zp);
+    FLY_PROF(4);
+    const float gamma = __builtin_amdgcn_exp2f(c0 - m_run);               // <= 1
+    if (SPLIT) {
+        float* ws = a.part_ws + (((long)bh * n_qt + qt) * a.n_parts + part) * (TQ * (D + NSTAT));
+        const int ql_ = 16 * w + r16;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) *reinterpret_cast<floatx4*>(ws + ql_ * D + 16 * db + 4 * g) = oacc[db];
+        if (g == 0) {
+            float* stp = ws + TQ * D;
+            stp[0 * TQ + ql_] = m_run;
+            stp[1 * TQ + ql_] = ze;
+            stp[2 * TQ + ql_] = zp;
+            stp[3 * TQ + ql_] = 0.f;
+            stp[4 * TQ + ql_] = c0;
+        }
+    } else {
+        const float Z = ze + gamma * fmaxf(qk1 - zp, 1e-24f);
+        const float inv = 1.0f / Z;
+        if (qvalid) {
+            float* optr = reinterpret_cast<float*>(a.out) + b * a.o_sb + h * a.o_sh + (long)iq * a.o_ss;
+#pragma unroll
+            for (int db = 0; db < DB; ++db) store4_f32(optr + 16 * db + 4 * g, (oacc[db] + gamma * lacc[db]) * inv);
+            if (g == 0) a.log_norm[(long)bh * a.T + iq] = m_run * LN2 + __logf(Z);
+        }
+    }
+    FLY_PROF(5);
+}
+
 // Finish of a query tile that was computed in parts: one workgroup per (64-query tile, batch-head),
 // in the register layout of the band kernel (wave w, lane (r16, g): query 16w + r16, output columns
 // 16db + 4g + i).  It merges the parts' un-normalised partials -- taken in batches whose loads are all
@@ -1930,6 +2425,106 @@ __global__ __launch_bounds__(NT) void sb_merge_kernel(FwdArgs a) {
     if (g == 0 && db == 0) a.log_norm[(long)bh * a.T + iq] = m_star * LN2 + __logf(Z);
 }
 
+// The same finish for the band kernel on bf16 pieces, arranged for locality: a workgroup takes 16 NDB output
+// columns of a tile (NDB = D / 16: the whole tile, so that the query features and the parts' statistics are
+// read once), and the one-dimensional grid is laid out so that a tile is finished on the XCD whose
+// workgroups wrote its parts (the dispatcher deals consecutive workgroup ids to the XCDs in turn): the
+// partials are then still in that XCD's L2.  xcd_items = band items (tile, part) per XCD of the band launch.
+template <int D, int M, int NDB>
+__global__ __launch_bounds__(NT) void sb_merge_x_kernel(FwdArgs a, int xcd_items, int tiles_per_xcd) {
+    constexpr float LN2 = 0.6931471805599453f;
+    constexpr int FC = M / 16, COLS = 16 * NDB, LDV = COLS + 4, NSL = D / COLS;
+    constexpr int PB = NDB >= 4 ? 5 : 8;              // parts per batch (their loads are all in flight together)
+    __shared__ __attribute__((aligned(16))) float KVs[M * LDV];
+    __shared__ __attribute__((aligned(16))) float KSs[M];
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
+    const int n_qt = (a.T + TQ - 1) / TQ, n_tiles = a.B * a.H * n_qt;
+    const int x = blockIdx.x % N_XCD, i = blockIdx.x / N_XCD, slice = i % NSL, j = i / NSL;
+    // tiles whose first part is one of XCD x's band items
+    const int t_lo = (x * xcd_items + a.n_parts - 1) / a.n_parts;
+    const int t_hi = min(((x + 1) * xcd_items + a.n_parts - 1) / a.n_parts, n_tiles);
+    const int tl = t_lo + j;
+    if (j >= tiles_per_xcd || tl >= t_hi) return;     // workgroup-uniform
+    const int qt = tl % n_qt, bh = tl / n_qt, b = bh / a.H, h = bh % a.H;
+    const int col0 = slice * COLS;
+    const int ql = 16 * w + r16, iq = qt * TQ + ql;
+    {
+        RowTile<M, COLS> kvt;
+        kvt.fetch(a.kv + (long)bh * M * D + col0, D, 0, M - 1, tid);
+        if (tid < M) KSs[tid] = a.ksum[(long)bh * M + tid];
+        kvt.template stash<LDV>(KVs, tid);
+    }
+    const long qrow = (long)bh * a.T + min(iq, a.T - 1);
+    floatx4 qf[FC];
+#pragma unroll
+    for (int c = 0; c < FC; ++c) qf[c] = *reinterpret_cast<const floatx4*>(a.qfeat + qrow * M + 16 * c + 4 * g);
+
+    const long stride = (long)TQ * (D + NSTAT);
+    const float* ws = a.part_ws + (long)tl * a.n_parts * stride;
+    const float* st = ws + TQ * D + ql;
+    const float c0 = st[4 * TQ];
+    float m_star = -INFINITY, ze = 0.f, zp = 0.f;
+    floatx4 acc[NDB];
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) acc[db] = Frag<float>::zero();
+    for (int p0 = 0; p0 < a.n_parts; p0 += PB) {
+        float mv[PB], zev[PB], zpv[PB];
+        floatx4 ov[PB][NDB];
+#pragma unroll
+        for (int jj = 0; jj < PB; ++jj) {
+            const long off = (long)min(p0 + jj, a.n_parts - 1) * stride;
+            mv[jj] = st[off];
+            zev[jj] = st[off + TQ];
+            zpv[jj] = st[off + 2 * TQ];
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+                ov[jj][db] = *reinterpret_cast<const floatx4*>(ws + off + ql * D + col0 + 16 * db + 4 * g);
+        }
+        float m_new = m_star;
+#pragma unroll
+        for (int jj = 0; jj < PB; ++jj) m_new = fmaxf(m_new, mv[jj]);
+        const float keep = (m_star == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_star - m_new);
+        m_star = m_new;
+        ze *= keep;
+#pragma unroll
+        for (int db = 0; db < NDB; ++db) acc[db] *= keep;
+#pragma unroll
+        for (int jj = 0; jj < PB; ++jj) {
+            if (p0 + jj < a.n_parts) {
+                const float wgt = __builtin_amdgcn_exp2f(mv[jj] - m_star);
+                ze += wgt * zev[jj];
+                zp += zpv[jj];
+#pragma unroll
+                for (int db = 0; db < NDB; ++db) acc[db] += wgt * ov[jj][db];
+            }
+        }
+    }
+    __syncthreads();                                 // K'^T V and sum K' are in LDS
+    floatx4 lacc[NDB];
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) lacc[db] = Frag<float>::zero();
+    float qk1 = 0.f;
+#pragma unroll
+    for (int c = 0; c < FC; ++c) {
+        const floatx4 ks = *reinterpret_cast<const floatx4*>(KSs + 16 * c + 4 * g);
+        qk1 += qf[c][0] * ks[0] + qf[c][1] * ks[1] + qf[c][2] * ks[2] + qf[c][3] * ks[3];
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj)
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+                lacc[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(KVs[(16 * c + 4 * g + jj) * LDV + 16 * db + r16], qf[c][jj], lacc[db], 0, 0, 0);
+    }
+    qk1 = group_sum(qk1);
+    if (iq >= a.T) return;
+    const float gamma = __builtin_amdgcn_exp2f(c0 - m_star);
+    const float Z = ze + gamma * fmaxf(qk1 - zp, 1e-24f);
+    const float inv = 1.0f / Z;
+    float* optr = reinterpret_cast<float*>(a.out) + b * a.o_sb + h * a.o_sh + (long)iq * a.o_ss + col0;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) store4_f32(optr + 16 * db + 4 * g, (acc[db] + gamma * lacc[db]) * inv);
+    if (g == 0 && slice == 0) a.log_norm[(long)bh * a.T + iq] = m_star * LN2 + __logf(Z);
+}
+
 // ---------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------
@@ -1949,6 +2544,21 @@ template <int E, int M> constexpr size_t fwd_smem() {
 template <int E, int M> constexpr size_t kfeat_bf16_smem() {
     return 2 * ((size_t)CH * (E + 8) + (size_t)E * (CH + 8) + (size_t)CH * (M + 8)) + sizeof(float) * (CH + 8);
 }
+template <int E, int M>
+static int launch_kfeat_x3(const KvArgs& a, hipStream_t st) {
+    auto kern = sb_kfeat_kernel<float, E, E, M, true>;
+    constexpr size_t smem = kfeat_smem<E, M>();
+    static bool lds_ready = false;
+    if (!lds_ready) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return fail(ERR_LAUNCH, "sb_kfeat (piece images): LDS attribute: %s", hipGetErrorString(e));
+        lds_ready = true;
+    }
+    hipLaunchKernelGGL(kern, dim3(a.n_split + a.q_tiles, a.B * a.H), dim3(NT), smem, st, a);
+    return check_launch("sb_kfeat_kernel (piece images)");
+}
+
 template <typename T, int E, int M>
 static int launch_kfeat(const KvArgs& a, hipStream_t st) {
     if (sizeof(T) == 2 && !a.q) {            // bfloat16 keys, no query role: both products on the bf16 MFMA
@@ -1964,6 +2574,7 @@ static int launch_kfeat(const KvArgs& a, hipStream_t st) {
         hipLaunchKernelGGL(kern16, dim3(a.n_split, a.B * a.H), dim3(NT), smem16, st, a);
         return check_launch("sb_kfeat_bf16_kernel");
     }
+    if (sizeof(T) == 4 && a.vt) return launch_kfeat_x3<E, M>(a, st);      // float inputs, piece images asked for
     auto kern = sb_kfeat_kernel<T, E, E, M>;
     constexpr size_t smem = kfeat_smem<E, M>();
     static bool lds_ready = false;     // one instantiation = one kernel; set its LDS limit once
@@ -2036,8 +2647,60 @@ static int launch_fwd_impl(const FwdArgs& a, hipStream_t st) {
     hipLaunchKernelGGL((sb_merge_kernel<T, E, M>), dim3(qt, E / 16, a.B * a.H), dim3(NT), 0, st, args);
     return check_launch("sb_merge_kernel");
 }
+#ifndef MERGE_NDB
+#define MERGE_NDB 2
+#endif
+// float inputs with the piece images of the key pass: the band kernel on the bf16 matrix pipe
+template <int E, int M> constexpr size_t fwd_x3_smem() {
+    constexpr size_t tiles = 2 * (size_t)X3Tile<E, E, M>::BYTES;
+    constexpr size_t proj = sizeof(float) * (size_t)(M / 2) * (E + 4);
+    constexpr size_t lowrank = sizeof(float) * ((size_t)M * (E + 4) + M);
+    return tiles > proj ? (tiles > lowrank ? tiles : lowrank) : (proj > lowrank ? proj : lowrank);
+}
+template <int E, int M, bool SPLIT>
+static int launch_fwd_x3(const FwdArgs& a, hipStream_t st) {
+    auto kern = sblocal_fwd_x3_kernel<E, E, M, SPLIT>;
+    constexpr size_t smem = fwd_x3_smem<E, M>();
+    static_assert(smem <= 160 * 1024, "two tile stages must fit the LDS");
+    static bool lds_ready = false;
+    if (!lds_ready) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return fail(ERR_LAUNCH, "sblocal_fwd (bf16 pieces): LDS attribute: %s", hipGetErrorString(e));
+        lds_ready = true;
+    }
+    const int qt = (a.T + TQ - 1) / TQ;
+    const long items = (long)a.B * a.H * qt * a.n_parts;
+    long grid = (items + N_XCD - 1) / N_XCD * N_XCD;
+    FwdArgs args = a;
+    args.band_wgs = (int)grid;
+    if (SPLIT) {
+        const long bhn = (long)a.B * a.H, free_slots = 512 - grid;
+        long wpb = free_slots / bhn;
+        const long most = (M * (E + 1) + NT - 1) / NT;
+        if (wpb > most) wpb = most;
+        if (wpb < 1) wpb = 1;
+        args.cmb_wpb = (int)wpb;
+        grid += bhn * wpb;
+    }
+    if (grid > 2147483647L) return fail(ERR_ARG, "sblocal_fwd: too many workgroups");
+    if (g_ev_before) (void)hipEventRecord(g_ev_before, st);
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NT), smem, st, args);
+    if (g_ev_after) (void)hipEventRecord(g_ev_after, st);
+    g_ev_before = g_ev_after = nullptr;
+    int rc = check_launch("sblocal_fwd_x3_kernel");
+    if (rc || !SPLIT) return rc;
+    constexpr int NDB = MERGE_NDB < E / 16 ? MERGE_NDB : E / 16;
+    const int xcd_items = (int)((items + N_XCD - 1) / N_XCD);
+    const int tiles_per_xcd = (xcd_items + a.n_parts - 1) / a.n_parts + 1;
+    hipLaunchKernelGGL((sb_merge_x_kernel<E, M, NDB>), dim3((unsigned)(N_XCD * tiles_per_xcd * (E / 16 / NDB))), dim3(NT), 0, st,
+                       args, xcd_items, tiles_per_xcd);
+    return check_launch("sb_merge_x_kernel");
+}
 template <typename T, int E, int M>
 static int launch_fwd(const FwdArgs& a, hipStream_t st) {
+    if (sizeof(T) == 4 && a.vt)
+        return a.n_parts > 1 ? launch_fwd_x3<E, M, true>(a, st) : launch_fwd_x3<E, M, false>(a, st);
     return a.n_parts > 1 ? launch_fwd_impl<T, E, M, true>(a, st) : launch_fwd_impl<T, E, M, false>(a, st);
 }
 
@@ -2488,6 +3151,11 @@ static int plan(int B, int H, int S, int* n_chunks, int* n_split) {
 using namespace flyhip;
 
 #ifdef FLY_PROFILE
+extern "C" int flyhip_prof_read_k(long long* dst, int n_workgroups) {
+    hipDeviceSynchronize();
+    hipError_t e = hipMemcpyFromSymbol(dst, HIP_SYMBOL(g_prof_k), sizeof(long long) * 8 * n_workgroups);
+    return e == hipSuccess ? 0 : -1;
+}
 extern "C" int flyhip_prof_read(long long* dst, int n_workgroups) {
     hipDeviceSynchronize();
     hipError_t e = hipMemcpyFromSymbol(dst, HIP_SYMBOL(g_prof), sizeof(long long) * 8 * n_workgroups);
@@ -2540,7 +3208,7 @@ extern "C" int flyhip_sb_kv_reduce(const void* k, const void* v, const float* pr
                 "sb_kv_reduce: n_split=%d outside [1, min(%d, %d)]", n_split, nc, MAX_SPLIT);
     FLY_REQUIRE((long)B * H <= 65535, "sb_kv_reduce: B*H=%ld exceeds the grid limit 65535", (long)B * H);
     FLY_REQUIRE(dtype != BF16 || (vt && kvt), "sb_kv_reduce: bfloat16 inputs need the vt and kvt scratch");
-    if (dtype != BF16) vt = kvt = nullptr;
+    if (dtype != BF16) kvt = nullptr;           // (float inputs: vt, when given, receives the operand images)
     if (q) {
         FLY_REQUIRE(qfeat && q_lsq && T > 0, "sb_kv_reduce: query features asked for without qfeat / q_lsq / T");
         FLY_REQUIRE(((q_sb | q_sh | q_ss) % 4) == 0, "sb_kv_reduce: q strides must be multiples of 4 elements");

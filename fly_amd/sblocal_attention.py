@@ -37,7 +37,8 @@ class SBLocalPlan:
     out (B,T,H,dim), log_norm (B,H,T) float32.  Buffers of one plan are shared by its runs: runs
     of the same plan on different streams race."""
 
-    def __init__(self, B, H, T, S, dim, mh, mh_valid, dtype, device, local_context, n_parts=None):
+    def __init__(self, B, H, T, S, dim, mh, mh_valid, dtype, device, local_context, n_parts=None,
+                 operand_images=True):
         n_chunks, n_split, parts = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
         _lib.call('flyhip_sb_plan', B, H, T, S, local_context, ctypes.byref(n_chunks), ctypes.byref(n_split),
                   ctypes.byref(parts))
@@ -57,6 +58,12 @@ class SBLocalPlan:
         self.kmax = torch.empty(B, H, dtype=f32, device=device)
         # bf16 inputs: V per 32-key tile and K'^T V in the operand order of the bf16 MFMA (opaque)
         self.vt = self.kvt = None
+        if dtype == torch.float32 and operand_images:
+            # float inputs: the band kernel runs on the bf16 matrix pipe from images of every 32-key tile
+            # (K in two bf16 pieces, V transposed in three; kfeat then holds the features in two pieces);
+            # 128 E + 192 D bytes per tile, two tiles per 64-key chunk.  Without it (block-sparse supports)
+            # the fp32-MFMA kernels run from fp32 features.
+            self.vt = torch.empty(B, H, self.n_chunks, 2 * (128 * dim + 192 * dim), dtype=torch.uint8, device=device)
         if dtype == torch.bfloat16:
             self.vt = torch.empty(B, H, self.n_chunks * 64, dim, dtype=dtype, device=device)
             self.kvt = torch.empty(B, H, dim, m, dtype=dtype, device=device)
@@ -229,7 +236,8 @@ def sbblocksparse_forward(query, key, value, projection_matrix, tables, softmax_
     q, k, v = prep(query), prep(key), prep(value)
     proj = torch.zeros(mh, dim, dtype=torch.float32, device=query.device)
     proj[:mh_valid, :E] = projection_matrix.to(torch.float32)
-    plan = SBLocalPlan(B, H, T, S, dim, mh, mh_valid, query.dtype, query.device, 64, n_parts=1)
+    plan = SBLocalPlan(B, H, T, S, dim, mh, mh_valid, query.dtype, query.device, 64, n_parts=1,
+                       operand_images=False)
     out = torch.empty(B, T, H, dim, dtype=query.dtype, device=query.device)
     log_norm = torch.empty(B, H, T, dtype=torch.float32, device=query.device)
     plan.run_block_sparse(q, k, v, proj, t, tables, out, log_norm)
