@@ -176,25 +176,40 @@ __device__ __forceinline__ void sb_combine_body(float* wgt, const float* kv_part
     }
     __syncthreads();
     if (ci == 0 && threadIdx.x == 0) kmax_out[bh] = (kmax == -INFINITY) ? 0.f : kmax;
-    for (int idx = ci * nthr + threadIdx.x; idx < per; idx += wpb * nthr) {
-        // threads walk a partial in its storage order (coalesced reads over the splits); the K'^T V part
-        // is in accumulator order: offset ((tile*64 + lane)*4 + i) holds element (r, d) of tile
-        // (r/16, d/16) with lane = 16*((r%16)/4) + d%16 and i = r%4
-        const float* src = kv_part + (long)bh * n_split * per + idx;
-        float acc = 0.f;
-#pragma unroll 16
-        for (int s = 0; s < n_split; ++s) acc += wgt[s] * src[(long)s * per];
+    // Threads walk a partial in its storage order, four consecutive floats each (16-byte loads, coalesced
+    // over the splits), in batches of 16 splits whose loads are all in flight together: the partials come
+    // from memory, and one round trip per split would make this the longest job of the launch.  The K'^T V
+    // part is in accumulator order: offset ((tile*64 + lane)*4 + i) holds element (r, d) of tile (r/16, d/16)
+    // with lane = 16*((r%16)/4) + d%16 and i = r%4.
+    const int per4 = per / 4;                                   // M (D + 1) is a multiple of 4
+    for (int q4 = ci * nthr + threadIdx.x; q4 < per4; q4 += wpb * nthr) {
+        const floatx4* src = reinterpret_cast<const floatx4*>(kv_part + (long)bh * n_split * per) + q4;
+        floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+        for (int s0 = 0; s0 < n_split; s0 += 16) {
+            floatx4 pv[16];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) pv[u] = src[(long)min(s0 + u, n_split - 1) * per4];
+#pragma unroll
+            for (int u = 0; u < 16; ++u)
+                if (s0 + u < n_split) acc += wgt[s0 + u] * pv[u];
+        }
+        const int idx = 4 * q4;
         if (idx < M * D) {
-            const int i = idx & 3, lane = (idx >> 2) & 63, tile = idx >> 8;
+            const int lane = (idx >> 2) & 63, tile = idx >> 8;
             const int db_n = D >> 4, rb = tile / db_n, db = tile % db_n;
-            const int r = 16 * rb + 4 * (lane >> 4) + i, d = 16 * db + (lane & 15);
-            kv[(long)bh * M * D + r * D + d] = acc;
-            if (kvt) {      // bf16 copy for the bf16 band kernel: [d][slot], feature r in the k-slot order of its MFMA
-                const int c = r >> 4, slot = 32 * (c >> 1) + 8 * ((r >> 2) & 3) + 4 * (c & 1) + (r & 3);
-                kvt[(long)bh * M * D + d * M + slot] = f32_to_bf16(acc);
+            const int r0 = 16 * rb + 4 * (lane >> 4), d = 16 * db + (lane & 15);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int r = r0 + i;
+                kv[(long)bh * M * D + r * D + d] = acc[i];
+                if (kvt) {      // bf16 copy for the bf16 band kernel: [d][slot], feature r in the k-slot order of its MFMA
+                    const int c = r >> 4, slot = 32 * (c >> 1) + 8 * ((r >> 2) & 3) + 4 * (c & 1) + (r & 3);
+                    kvt[(long)bh * M * D + d * M + slot] = f32_to_bf16(acc[i]);
+                }
             }
         } else {
-            ksum[(long)bh * M + idx - M * D] = acc;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) ksum[(long)bh * M + idx - M * D + i] = acc[i];
         }
     }
 }
@@ -233,6 +248,33 @@ __device__ __forceinline__ void store_feat(void* kfeat, long row, int M, int fbp
         u.y = pack_bf16x2(f[2], f[3]);
         *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(kfeat) + row * M + 32 * (fbp >> 1) + 8 * g + 4 * (fbp & 1)) = u;
     }
+}
+
+// stores of data that the next launch reads (tile images, partial results)
+#if !defined(FLY_PLAIN_STORES)
+// write-through to memory (device scope): nothing of it is left dirty in the L2 when the kernel ends (the
+// write-back of megabytes of dirty lines at the end of a launch is time nothing overlaps), and a workgroup
+// on another XCD that reads the line for the first time in its launch finds the data in memory
+template <typename V>
+__device__ __forceinline__ void store16_wt(V val, V* ptr) {
+    static_assert(sizeof(V) == 16, "16-byte pieces");
+    // (the wait states keep a following VALU write away from the data registers, which a store of more than
+    // eight bytes reads a little after it issues; the compiler does that for its own stores)
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(ptr), "v"(val) : "memory");
+}
+#define FLY_STORE(val, ptr) store16_wt((val), (ptr))
+#elif defined(FLY_NT_STORES)
+#define FLY_STORE(val, ptr) __builtin_nontemporal_store((val), (ptr))
+#else
+#define FLY_STORE(val, ptr) (*(ptr) = (val))
+#endif
+
+// one 16x16x32 step on the bf16 matrix pipe: eight k-slots per lane on either side
+__device__ __forceinline__ floatx4 mma_bf16(uint4 a, uint4 b, floatx4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+__device__ __forceinline__ floatx4 mma_bf16(uintx4 a, uintx4 b, floatx4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -636,6 +678,369 @@ void sb_kfeat_kernel(KvArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------
+// key pass for float inputs with both products on the bf16 matrix pipe (tile images built in LDS)
+// ---------------------------------------------------------------------------------------
+// The outputs of sb_kfeat_kernel<float, .., X3 = true> -- tile images, chunk scales, partial K'^T V / sum K' --
+// with the images assembled in LDS, where they double as MFMA operands:
+//   projection : dd[feature][key] = (sqrt(t) log2e P) . k with P in three bf16 pieces (exact) as the row
+//                operand and the K image (two pieces) as the column operand, five piece products; a lane
+//                ends with four features of its key, as in sb_kfeat_kernel
+//   features   : exp2, rounded to 16 bits, written as two pieces into the feature image (16-byte writes:
+//                the lane's blocks 2p, 2p+1 are the eight k-slots of one chunk)
+//   K'^T V     : rows = feature positions of the image (transposing LDS reads hand a lane one feature
+//                column of four key rows), columns = value dims from the V^T image, five piece products;
+//                the partial leaves in the natural feature order the combine step expects
+// One chunk of 64 keys = two tile images = 2 * X3Tile::BYTES of LDS, copied to global memory in 16-byte
+// pieces.  Instantiated where that fits next to the fp32 V chunk and the projection image (E <= 64, m <= 128).
+template <int E, int D, int M>
+__global__ __launch_bounds__(NT) void sb_kfeat_x3_kernel(KvArgs a) {
+    typedef X3Tile<E, D, M> TL;
+    constexpr int MH = M / 2, FB = MH / 16, EC = E / 16, DB = D / 16, KS = E / 32, FS = M / 32;
+    constexpr int LDV = D + 4, P_ROW = 2 * E, P_PIECE = MH * P_ROW;
+    constexpr int NBLK = M / 16, RB = (NBLK + 3) / 4;      // K'^T V row blocks (of feature positions) per wave
+    constexpr float LOG2E = 1.4426950408889634f, LN2 = 0.6931471805599453f;
+    extern __shared__ __attribute__((aligned(128))) float smem[];
+    char* img = reinterpret_cast<char*>(smem);                         // two tile images
+    float* Vs = reinterpret_cast<float*>(img + 2 * TL::BYTES);         // fp32 V chunk (for the transposition)
+    char* Pimg = reinterpret_cast<char*>(Vs + CH * LDV);               // projection rows, three pieces
+    float* diag = reinterpret_cast<float*>(Pimg + 3 * P_PIECE);        // t log2e |k|^2 / 2 per key
+    float* red = diag + CH;                                            // 4 wave maxima
+    float* ks_lds = red + 4;                                           // 4 x M column sums
+
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
+    const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H, sp = blockIdx.x;
+    FLY_PROFK(0);
+    if (sp >= a.n_split) {
+        // Query role: the features of 64 queries, rounded to 16 bits, and their log-scales (see sb_kfeat_kernel)
+        const float* pp = a.proj + r16 * E + 4 * g;
+        const int iq = (sp - a.n_split) * TQ + 16 * w + r16;
+        const float* qrow = reinterpret_cast<const float*>(a.q) + b * a.q_sb + h * a.q_sh + (long)min(iq, a.T - 1) * a.q_ss;
+        floatx4 qr[EC];
+        float sq = 0.f;
+#pragma unroll
+        for (int c = 0; c < EC; ++c) {
+            qr[c] = load4_f32(qrow + 16 * c + 4 * g);
+            sq += qr[c][0] * qr[c][0] + qr[c][1] * qr[c][1] + qr[c][2] * qr[c][2] + qr[c][3] * qr[c][3];
+        }
+        const float diag_q = 0.5f * a.temp * group_sum(sq);
+        const float st = sqrtf(a.temp);
+        floatx4 pa[EC][FB];
+#pragma unroll
+        for (int c = 0; c < EC; ++c)
+#pragma unroll
+            for (int fb = 0; fb < FB; ++fb) pa[c][fb] = *reinterpret_cast<const floatx4*>(pp + 16 * fb * E + 16 * c) * st;
+        floatx4 qf[FB];
+#pragma unroll
+        for (int fb = 0; fb < FB; ++fb) qf[fb] = Frag<float>::zero();
+#pragma unroll
+        for (int c = 0; c < EC; ++c)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int fb = 0; fb < FB; ++fb)
+                    qf[fb] = __builtin_amdgcn_mfma_f32_16x16x4f32(pa[c][fb][j], qr[c][j], qf[fb], 0, 0, 0);
+        float qmax = 0.f;
+#pragma unroll
+        for (int fb = 0; fb < FB; ++fb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (16 * fb + 4 * g + i < a.mh_valid) qmax = fmaxf(qmax, fabsf(qf[fb][i]));
+        qmax = group_max(qmax);
+        if (iq < a.T) {
+            float* dst = a.qfeat + ((long)bh * a.T + iq) * M;
+#pragma unroll
+            for (int fb = 0; fb < FB; ++fb) {
+                floatx4 fp, fn;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const bool ok = 16 * fb + 4 * g + i < a.mh_valid;
+                    fp[i] = ok ? quant16(__expf(qf[fb][i] - qmax)) : 0.f;
+                    fn[i] = ok ? quant16(__expf(-qf[fb][i] - qmax)) : 0.f;
+                }
+                FLY_STORE(fp, reinterpret_cast<floatx4*>(dst + 16 * fb + 4 * g));
+                FLY_STORE(fn, reinterpret_cast<floatx4*>(dst + MH + 16 * fb + 4 * g));
+            }
+            if (g == 0) a.q_lsq[(long)bh * a.T + iq] = -diag_q + qmax - 0.5f * __logf(2.0f * a.mh_valid);
+        }
+        FLY_PROFK(6);
+        return;
+    }
+
+    const float* kptr = reinterpret_cast<const float*>(a.k) + b * a.k_sb + h * a.k_sh;
+    const float* vptr = reinterpret_cast<const float*>(a.v) + b * a.v_sb + h * a.v_sh;
+    const int len = a.lens ? min((int)a.lens[b], a.S) : a.S;
+    const float lnm_half2 = 0.5f * __log2f(2.0f * a.mh_valid);
+    const int per = (a.n_chunks + a.n_split - 1) / a.n_split;
+    const int c0 = sp * per, c1 = min(a.n_chunks, c0 + per);
+    RowTile<CH, E> kt;
+    RowTile<CH, D> vt;
+    if (c0 < c1) {
+        kt.fetch(kptr, a.k_ss, c0 * CH, a.S - 1, tid);
+        vt.fetch(vptr, a.v_ss, c0 * CH, a.S - 1, tid);
+    }
+    // projection rows scaled by sqrt(t) log2e, as three bf16 pieces in the k-slot order of the K image
+    {
+        const float pscale = sqrtf(a.temp) * LOG2E;
+        constexpr int CH8 = E / 8, TOT = MH * CH8;
+#pragma unroll
+        for (int j = 0; j < (TOT + NT - 1) / NT; ++j) {
+            const int idx = tid + NT * j;
+            if (TOT % NT == 0 || idx < TOT) {
+                const int row = idx / CH8, cch = idx % CH8, ks = cch >> 2, gq = cch & 3;
+                const float* sp_ = a.proj + (long)row * E + 32 * ks + 4 * gq;
+                uintx4 ph, pm, pl;
+                split3(*reinterpret_cast<const floatx4*>(sp_) * pscale, *reinterpret_cast<const floatx4*>(sp_ + 16) * pscale, ph, pm, pl);
+                char* dst = Pimg + row * P_ROW + x3_swz(row, cch, P_ROW) * 16;
+                *reinterpret_cast<uintx4*>(dst) = ph;
+                *reinterpret_cast<uintx4*>(dst + P_PIECE) = pm;
+                *reinterpret_cast<uintx4*>(dst + 2 * P_PIECE) = pl;
+            }
+        }
+    }
+    // a chunk in registers -> K image (two pieces) and |k|^2 per key, V as fp32 rows for the transposition
+    auto stash = [&]() __attribute__((always_inline)) {
+        constexpr int V4 = E / 4;                         // RowTile pieces: idx -> row idx / V4, columns 4 (idx % V4) ..
+#pragma unroll
+        for (int j = 0; j < RowTile<CH, E>::N; ++j) {
+            const int idx = tid + NT * j, row64 = idx / V4;
+            const floatx4 x = kt.r[j];
+            float sq = x[0] * x[0] + x[1] * x[1] + x[2] * x[2] + x[3] * x[3];
+#pragma unroll
+            for (int off = 1; off < V4; off <<= 1) sq += __shfl_xor(sq, off);      // the V4 lanes of one key row
+            if (idx % V4 == 0) diag[row64] = 0.5f * a.temp * LOG2E * sq;
+        }
+        // the K image takes elements 32ks + 4gq + i and 32ks + 16 + 4gq + i into one chunk: go through Vs' neighbour?
+        // (no: the two quads sit in different threads' registers, so K goes through an fp32 staging tile too)
+        kt.template stash<E + 4>(reinterpret_cast<float*>(img), tid);             // fp32 K rows, overlaid on the images
+        vt.template stash<LDV>(Vs, tid);
+    };
+    if (c0 < c1) stash();
+    __syncthreads();
+    FLY_PROFK(1);
+
+    floatx4 kvacc[RB][DB];
+#pragma unroll
+    for (int x = 0; x < RB; ++x)
+#pragma unroll
+        for (int db = 0; db < DB; ++db) kvacc[x][db] = Frag<float>::zero();
+    floatx4 ksp[FB], ksn[FB];
+#pragma unroll
+    for (int fb = 0; fb < FB; ++fb) { ksp[fb] = Frag<float>::zero(); ksn[fb] = Frag<float>::zero(); }
+    float run_max = -INFINITY;
+    const int tile_w = w >> 1, row_w = 16 * (w & 1) + r16;              // this lane's key: tile and row inside it
+
+    for (int c = c0; c < c1; ++c) {
+        const int s_base = c * CH;
+        if (c + 1 < c1) {
+            kt.fetch(kptr, a.k_ss, s_base + CH, a.S - 1, tid);
+            vt.fetch(vptr, a.v_ss, s_base + CH, a.S - 1, tid);
+        }
+        // fp32 K rows (staged over the image area) -> registers -> K image; V^T image from Vs
+        {
+            constexpr int CH8 = E / 8, TOT = CH * CH8, NJ = (TOT + NT - 1) / NT;
+            uintx4 khi[NJ], klo[NJ];
+            const float* Kf = reinterpret_cast<const float*>(img);
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                const int idx = tid + NT * j;
+                if (TOT % NT == 0 || idx < TOT) {
+                    const int row64 = idx / CH8, cch = idx % CH8, ks = cch >> 2, gq = cch & 3;
+                    const float* sp_ = Kf + row64 * (E + 4) + 32 * ks + 4 * gq;
+                    split2(*reinterpret_cast<const floatx4*>(sp_), *reinterpret_cast<const floatx4*>(sp_ + 16), khi[j], klo[j]);
+                }
+            }
+            __syncthreads();                             // every thread has its K quads: the staging tile may be overwritten
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                const int idx = tid + NT * j;
+                if (TOT % NT == 0 || idx < TOT) {
+                    const int row64 = idx / CH8, cch = idx % CH8, row = row64 & (TK - 1);
+                    char* dst = img + (row64 / TK) * TL::BYTES + row * TL::K_ROW + x3_swz(row, cch, TL::K_ROW) * 16;
+                    *reinterpret_cast<uintx4*>(dst) = khi[j];
+                    *reinterpret_cast<uintx4*>(dst + TL::K_PIECE) = klo[j];
+                }
+            }
+            x3_emit_vt<D, LDV>(Vs, img + 2 * TL::K_PIECE, TL::BYTES, tid);
+        }
+        __syncthreads();
+        FLY_PROFK(2);
+        // projection of this wave's 16 keys: five piece products per step
+        floatx4 dd[FB];
+#pragma unroll
+        for (int fb = 0; fb < FB; ++fb) dd[fb] = Frag<float>::zero();
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const char* kp = img + tile_w * TL::BYTES + row_w * TL::K_ROW + x3_swz(row_w, 4 * ks + g, TL::K_ROW) * 16;
+            const uintx4 kh = *reinterpret_cast<const uintx4*>(kp), kl = *reinterpret_cast<const uintx4*>(kp + TL::K_PIECE);
+#pragma unroll
+            for (int fb = 0; fb < FB; ++fb) {
+                const char* pp_ = Pimg + (16 * fb + r16) * P_ROW + x3_swz(r16, 4 * ks + g, P_ROW) * 16;
+                const uintx4 ph = *reinterpret_cast<const uintx4*>(pp_), pm = *reinterpret_cast<const uintx4*>(pp_ + P_PIECE),
+                             pl = *reinterpret_cast<const uintx4*>(pp_ + 2 * P_PIECE);
+                floatx4 d_ = dd[fb];
+                d_ = mma_bf16(pl, kh, d_);
+                d_ = mma_bf16(pm, kl, d_);
+                d_ = mma_bf16(ph, kl, d_);
+                d_ = mma_bf16(pm, kh, d_);
+                d_ = mma_bf16(ph, kh, d_);
+                dd[fb] = d_;
+            }
+        }
+        const float diag2 = diag[16 * w + r16];
+        float amax = 0.f;
+#pragma unroll
+        for (int fb = 0; fb < FB; ++fb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (16 * fb + 4 * g + i < a.mh_valid) amax = fmaxf(amax, fabsf(dd[fb][i]));
+        amax = group_max(amax);
+        const bool kvalid = (s_base + 16 * w + r16) < len;
+        float cs = kvalid ? (amax - diag2 - lnm_half2) : -INFINITY;
+        cs = wave_max(cs);
+        if (lane == 0) red[w] = cs;
+        __syncthreads();
+        const float lmax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+        const float new_max = fmaxf(run_max, lmax);
+        const bool live = new_max != -INFINITY;            // workgroup-uniform: some valid key so far
+        const float rescale = (run_max == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(run_max - new_max);
+        if (live) run_max = new_max;
+        const float off = -diag2 - lnm_half2 - new_max;
+        floatx4 fblk[2 * FB];                              // the lane's features: blocks of the [positive | negative] row
+#pragma unroll
+        for (int fb = 0; fb < FB; ++fb) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const bool ok = live && kvalid && (16 * fb + 4 * g + i < a.mh_valid);
+                fblk[fb][i] = ok ? quant16(__builtin_amdgcn_exp2f(dd[fb][i] + off)) : 0.f;
+                fblk[FB + fb][i] = ok ? quant16(__builtin_amdgcn_exp2f(-dd[fb][i] + off)) : 0.f;
+            }
+            ksp[fb] = ksp[fb] * rescale + fblk[fb];
+            ksn[fb] = ksn[fb] * rescale + fblk[FB + fb];
+        }
+        {
+            char* frow = img + tile_w * TL::BYTES + TL::KV_BYTES + row_w * TL::F_ROW;
+#pragma unroll
+            for (int p_ = 0; p_ < FS; ++p_) {
+                uintx4 fh, fl;
+                split2(fblk[2 * p_], fblk[2 * p_ + 1], fh, fl);
+                char* dst = frow + x3_swz(row_w, 4 * p_ + g, TL::F_ROW) * 16;
+                *reinterpret_cast<uintx4*>(dst) = fh;
+                *reinterpret_cast<uintx4*>(dst + TL::F_PIECE) = fl;
+            }
+        }
+        if (tid == 0) a.chunk_scale[(long)bh * a.n_chunks + c] = live ? new_max * LN2 : 0.f;
+        __syncthreads();                                   // images complete
+        FLY_PROFK(3);
+        // images -> global memory, 16-byte pieces in thread order
+        {
+            char* kv_g = reinterpret_cast<char*>(a.vt) + ((long)bh * a.n_chunks + c) * (2 * (long)TL::KV_BYTES);
+            char* f_g = reinterpret_cast<char*>(a.kfeat) + ((long)bh * a.n_chunks + c) * (2 * (long)TL::F_BYTES);
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+#pragma unroll
+                for (int j = 0; j < (TL::KV_BYTES / 16 + NT - 1) / NT; ++j) {
+                    const int idx = tid + NT * j;
+                    if (TL::KV_BYTES / 16 % NT == 0 || idx < TL::KV_BYTES / 16)
+                        FLY_STORE(reinterpret_cast<const uintx4*>(img + t * TL::BYTES)[idx], reinterpret_cast<uintx4*>(kv_g + t * TL::KV_BYTES) + idx);
+                }
+#pragma unroll
+                for (int j = 0; j < (TL::F_BYTES / 16 + NT - 1) / NT; ++j) {
+                    const int idx = tid + NT * j;
+                    if (TL::F_BYTES / 16 % NT == 0 || idx < TL::F_BYTES / 16)
+                        FLY_STORE(reinterpret_cast<const uintx4*>(img + t * TL::BYTES + TL::KV_BYTES)[idx], reinterpret_cast<uintx4*>(f_g + t * TL::F_BYTES) + idx);
+                }
+            }
+        }
+        FLY_PROFK(4);
+        // K'^T V: rows = feature positions 16 blk + r16, k = keys of a tile (transposing reads of the feature
+        // image), columns = value dims (V^T image rows); five piece products
+        if (live) {
+#pragma unroll
+            for (int x = 0; x < RB; ++x)
+#pragma unroll
+                for (int db = 0; db < DB; ++db) kvacc[x][db] *= rescale;
+            typedef __attribute__((address_space(3))) shortx4 lds_s4;
+            typedef unsigned int uintx2_t __attribute__((ext_vector_type(2)));
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const char* ti = img + t * TL::BYTES;
+                uintx4 vh[DB], vm[DB], vl[DB];
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+                    const char* vp = ti + 2 * TL::K_PIECE + (16 * db + r16) * TL::V_ROW + x3_swz(r16, g, TL::V_ROW) * 16;
+                    vh[db] = *reinterpret_cast<const uintx4*>(vp);
+                    vm[db] = *reinterpret_cast<const uintx4*>(vp + TL::V_PIECE);
+                    vl[db] = *reinterpret_cast<const uintx4*>(vp + 2 * TL::V_PIECE);
+                }
+#pragma unroll
+                for (int x = 0; x < RB; ++x) {
+                    const int blk = w + 4 * x;
+                    if (blk < NBLK) {
+                        // lane (r16, g) points at key rows 4g + r16/4 and 16 + 4g + r16/4, position quad 16 blk + 4 (r16 % 4)
+                        const int pos = 16 * blk + 4 * (r16 & 3), cch = pos >> 3, sub = (pos & 4) * 2;
+                        const int row_lo = 4 * g + (r16 >> 2), row_hi = 16 + row_lo;
+                        const char* flo_ = ti + TL::KV_BYTES + row_lo * TL::F_ROW + x3_swz(row_lo, cch, TL::F_ROW) * 16 + sub;
+                        const char* fhi_ = ti + TL::KV_BYTES + row_hi * TL::F_ROW + x3_swz(row_hi, cch, TL::F_ROW) * 16 + sub;
+                        uintx4 fh, fl;
+                        {
+                            const uintx2_t a0 = __builtin_bit_cast(uintx2_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)flo_));
+                            const uintx2_t a1 = __builtin_bit_cast(uintx2_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)fhi_));
+                            const uintx2_t b0 = __builtin_bit_cast(uintx2_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(flo_ + TL::F_PIECE)));
+                            const uintx2_t b1 = __builtin_bit_cast(uintx2_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(fhi_ + TL::F_PIECE)));
+                            fh = uintx4{a0[0], a0[1], a1[0], a1[1]};
+                            fl = uintx4{b0[0], b0[1], b1[0], b1[1]};
+                        }
+#pragma unroll
+                        for (int db = 0; db < DB; ++db) {
+                            floatx4 o = kvacc[x][db];
+                            o = mma_bf16(fl, vm[db], o);
+                            o = mma_bf16(fh, vl[db], o);
+                            o = mma_bf16(fl, vh[db], o);
+                            o = mma_bf16(fh, vm[db], o);
+                            o = mma_bf16(fh, vh[db], o);
+                            kvacc[x][db] = o;
+                        }
+                    }
+                }
+            }
+        }
+        FLY_PROFK(5);
+        __syncthreads();                                   // everyone is done with the images
+        if (c + 1 < c1) stash();
+        __syncthreads();
+    }
+
+    // partial K'^T V in the combine step's order: tile (rb, db) -> 64 lanes x 4 floats with element
+    // (feature 16 rb + 4 g'' + i, dim 16 db + r16) at lane 16 g'' + r16.  This lane's accumulator row 4g + i of
+    // position block blk is feature 32 (blk / 2) + 16 (g % 2) + 8 (blk % 2) + 4 (g / 2) + i.
+    float* part = a.kv_part + ((long)bh * a.n_split + sp) * (M * (D + 1));
+#pragma unroll
+    for (int x = 0; x < RB; ++x) {
+        const int blk = w + 4 * x;
+        if (blk < NBLK) {
+            const int rb = 2 * (blk >> 1) + (g & 1), g2 = 2 * (blk & 1) + (g >> 1);
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+                FLY_STORE(kvacc[x][db], reinterpret_cast<floatx4*>(part + ((rb * DB + db) * 64 + 16 * g2 + r16) * 4));
+        }
+    }
+#pragma unroll
+    for (int fb = 0; fb < FB; ++fb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float p_ = row16_sum(ksp[fb][i]), n_ = row16_sum(ksn[fb][i]);
+            if (r16 == 0) {
+                ks_lds[w * M + 16 * fb + 4 * g + i] = p_;
+                ks_lds[w * M + MH + 16 * fb + 4 * g + i] = n_;
+            }
+        }
+    __syncthreads();
+    if (tid < M) part[M * D + tid] = (ks_lds[tid] + ks_lds[M + tid]) + (ks_lds[2 * M + tid] + ks_lds[3 * M + tid]);
+    if (tid == 0) a.part_max[(long)bh * a.n_split + sp] = run_max * LN2;
+    FLY_PROFK(6);
+}
+
+// ---------------------------------------------------------------------------------------
 // fused band kernel for bfloat16 inputs
 // ---------------------------------------------------------------------------------------
 // Same algorithm and the same transposed formulation as sblocal_fwd_kernel, with the three
@@ -736,12 +1141,6 @@ struct TileKV16 {
     }
 };
 
-__device__ __forceinline__ floatx4 mma_bf16(uint4 a, uint4 b, floatx4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
-}
-__device__ __forceinline__ floatx4 mma_bf16(uintx4 a, uintx4 b, floatx4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
-}
 
 template <int E, int M> constexpr size_t fwd_bf16_smem() {
     constexpr size_t stage = (size_t)TK * (E + 8) + (size_t)TK * (M + 8) + (size_t)E * (TK + 8);   // 2-byte elements
@@ -2005,13 +2404,13 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
     float* Ps = smem;                                  // only live before the key loop
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
+    const int n_qt = (a.T + TQ - 1) / TQ;
     if (SPLIT && (int)blockIdx.x >= a.band_wgs) {       // combine role, see sblocal_fwd_kernel
         const int ci = blockIdx.x - a.band_wgs;
         sb_combine_body(smem, a.kv_part, a.part_max, const_cast<float*>(a.kv), const_cast<float*>(a.ksum),
                         const_cast<float*>(a.kmax), nullptr, ci / a.cmb_wpb, ci % a.cmb_wpb, a.cmb_wpb, a.n_split, M, D);
         return;
     }
-    const int n_qt = (a.T + TQ - 1) / TQ;
     const int n_items = a.B * a.H * n_qt * a.n_parts;
     const int per_xcd = (n_items + N_XCD - 1) / N_XCD;
     const int item = (blockIdx.x % N_XCD) * per_xcd + blockIdx.x / N_XCD;   // see sblocal_fwd_kernel
@@ -2307,10 +2706,10 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
     if (SPLIT) {
         float* ws = a.part_ws + (((long)bh * n_qt + qt) * a.n_parts + part) * (TQ * (D + NSTAT));
         const int ql_ = 16 * w + r16;
+        float* stp = ws + TQ * D;
 #pragma unroll
-        for (int db = 0; db < DB; ++db) *reinterpret_cast<floatx4*>(ws + ql_ * D + 16 * db + 4 * g) = oacc[db];
+        for (int db = 0; db < DB; ++db) FLY_STORE(oacc[db], reinterpret_cast<floatx4*>(ws + ql_ * D + 16 * db + 4 * g));
         if (g == 0) {
-            float* stp = ws + TQ * D;
             stp[0 * TQ + ql_] = m_run;
             stp[1 * TQ + ql_] = ze;
             stp[2 * TQ + ql_] = zp;
@@ -2430,30 +2829,22 @@ __global__ __launch_bounds__(NT) void sb_merge_kernel(FwdArgs a) {
 // read once), and the one-dimensional grid is laid out so that a tile is finished on the XCD whose
 // workgroups wrote its parts (the dispatcher deals consecutive workgroup ids to the XCDs in turn): the
 // partials are then still in that XCD's L2.  xcd_items = band items (tile, part) per XCD of the band launch.
+// (the finish of tile tl, columns 16 NDB slice .. of it, by one workgroup; KVs: M rows of 16 NDB + 4 floats, KSs: M floats of LDS)
 template <int D, int M, int NDB>
-__global__ __launch_bounds__(NT) void sb_merge_x_kernel(FwdArgs a, int xcd_items, int tiles_per_xcd) {
+__device__ __forceinline__ void sb_merge_tile(const FwdArgs& a, int tl, int slice, float* KVs, float* KSs) {
     constexpr float LN2 = 0.6931471805599453f;
-    constexpr int FC = M / 16, COLS = 16 * NDB, LDV = COLS + 4, NSL = D / COLS;
+    constexpr int FC = M / 16, COLS = 16 * NDB, LDV = COLS + 4;
     constexpr int PB = NDB >= 4 ? 5 : 8;              // parts per batch (their loads are all in flight together)
-    __shared__ __attribute__((aligned(16))) float KVs[M * LDV];
-    __shared__ __attribute__((aligned(16))) float KSs[M];
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
-    const int n_qt = (a.T + TQ - 1) / TQ, n_tiles = a.B * a.H * n_qt;
-    const int x = blockIdx.x % N_XCD, i = blockIdx.x / N_XCD, slice = i % NSL, j = i / NSL;
-    // tiles whose first part is one of XCD x's band items
-    const int t_lo = (x * xcd_items + a.n_parts - 1) / a.n_parts;
-    const int t_hi = min(((x + 1) * xcd_items + a.n_parts - 1) / a.n_parts, n_tiles);
-    const int tl = t_lo + j;
-    if (j >= tiles_per_xcd || tl >= t_hi) return;     // workgroup-uniform
+    const int n_qt = (a.T + TQ - 1) / TQ;
     const int qt = tl % n_qt, bh = tl / n_qt, b = bh / a.H, h = bh % a.H;
     const int col0 = slice * COLS;
     const int ql = 16 * w + r16, iq = qt * TQ + ql;
-    {
-        RowTile<M, COLS> kvt;
-        kvt.fetch(a.kv + (long)bh * M * D + col0, D, 0, M - 1, tid);
-        if (tid < M) KSs[tid] = a.ksum[(long)bh * M + tid];
-        kvt.template stash<LDV>(KVs, tid);
-    }
+    // every operand comes from memory (another launch, or another workgroup, wrote it): all loads are issued
+    // before the first is used, so that the finish costs one round trip, not one per operand
+    RowTile<M, COLS> kvt;
+    kvt.fetch(a.kv + (long)bh * M * D + col0, D, 0, M - 1, tid);
+    const float ksv = a.ksum[(long)bh * M + min(tid, M - 1)];
     const long qrow = (long)bh * a.T + min(iq, a.T - 1);
     floatx4 qf[FC];
 #pragma unroll
@@ -2479,6 +2870,10 @@ __global__ __launch_bounds__(NT) void sb_merge_x_kernel(FwdArgs a, int xcd_items
 #pragma unroll
             for (int db = 0; db < NDB; ++db)
                 ov[jj][db] = *reinterpret_cast<const floatx4*>(ws + off + ql * D + col0 + 16 * db + 4 * g);
+        }
+        if (p0 == 0) {
+            kvt.template stash<LDV>(KVs, tid);
+            if (tid < M) KSs[tid] = ksv;
         }
         float m_new = m_star;
 #pragma unroll
@@ -2525,6 +2920,21 @@ __global__ __launch_bounds__(NT) void sb_merge_x_kernel(FwdArgs a, int xcd_items
     if (g == 0 && slice == 0) a.log_norm[(long)bh * a.T + iq] = m_star * LN2 + __logf(Z);
 }
 
+template <int D, int M, int NDB>
+__global__ __launch_bounds__(NT) void sb_merge_x_kernel(FwdArgs a, int xcd_items, int tiles_per_xcd) {
+    constexpr int COLS = 16 * NDB, LDV = COLS + 4, NSL = D / COLS;
+    __shared__ __attribute__((aligned(16))) float KVs[M * LDV];
+    __shared__ __attribute__((aligned(16))) float KSs[M];
+    const int n_qt = (a.T + TQ - 1) / TQ, n_tiles = a.B * a.H * n_qt;
+    const int x = blockIdx.x % N_XCD, i = blockIdx.x / N_XCD, slice = i % NSL, j = i / NSL;
+    // tiles whose first part is one of XCD x's band items
+    const int t_lo = (x * xcd_items + a.n_parts - 1) / a.n_parts;
+    const int t_hi = min(((x + 1) * xcd_items + a.n_parts - 1) / a.n_parts, n_tiles);
+    const int tl = t_lo + j;
+    if (j >= tiles_per_xcd || tl >= t_hi) return;     // workgroup-uniform
+    sb_merge_tile<D, M, NDB>(a, tl, slice, KVs, KSs);
+}
+
 // ---------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------
@@ -2544,8 +2954,27 @@ template <int E, int M> constexpr size_t fwd_smem() {
 template <int E, int M> constexpr size_t kfeat_bf16_smem() {
     return 2 * ((size_t)CH * (E + 8) + (size_t)E * (CH + 8) + (size_t)CH * (M + 8)) + sizeof(float) * (CH + 8);
 }
+template <int E, int M> constexpr size_t kfeat_x3_smem() {
+    return 2 * (size_t)X3Tile<E, E, M>::BYTES + sizeof(float) * CH * (E + 4) + 3 * (size_t)(M / 2) * 2 * E +
+           sizeof(float) * (CH + 4 + 4 * M);
+}
 template <int E, int M>
 static int launch_kfeat_x3(const KvArgs& a, hipStream_t st) {
+    if constexpr (E <= 64 && M <= 128) {
+        // both products on the bf16 matrix pipe, images assembled in LDS
+        auto kern = sb_kfeat_x3_kernel<E, E, M>;
+        constexpr size_t smem = kfeat_x3_smem<E, M>();
+        static_assert(smem <= 160 * 1024, "two tile images, the V chunk and the projection image must fit the LDS");
+        static bool lds_ready = false;
+        if (!lds_ready) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+            if (e != hipSuccess) return fail(ERR_LAUNCH, "sb_kfeat_x3: LDS attribute: %s", hipGetErrorString(e));
+            lds_ready = true;
+        }
+        hipLaunchKernelGGL(kern, dim3(a.n_split + a.q_tiles, a.B * a.H), dim3(NT), smem, st, a);
+        return check_launch("sb_kfeat_x3_kernel");
+    }
     auto kern = sb_kfeat_kernel<float, E, E, M, true>;
     constexpr size_t smem = kfeat_smem<E, M>();
     static bool lds_ready = false;
@@ -2631,7 +3060,7 @@ static int launch_fwd_impl(const FwdArgs& a, hipStream_t st) {
         // residency round (two workgroups of this kernel per CU), at least one, at most one thread per output
         const long bhn = (long)a.B * a.H, free_slots = 512 - grid;
         long wpb = free_slots / bhn;
-        const long most = (M * (E + 1) + K::threads - 1) / K::threads;
+        const long most = (M * (E + 1) / 4 + K::threads - 1) / K::threads;   // one 16-byte piece of the result per thread
         if (wpb > most) wpb = most;
         if (wpb < 1) wpb = 1;
         args.cmb_wpb = (int)wpb;
@@ -2677,7 +3106,7 @@ static int launch_fwd_x3(const FwdArgs& a, hipStream_t st) {
     if (SPLIT) {
         const long bhn = (long)a.B * a.H, free_slots = 512 - grid;
         long wpb = free_slots / bhn;
-        const long most = (M * (E + 1) + NT - 1) / NT;
+        const long most = (M * (E + 1) / 4 + NT - 1) / NT;      // one 16-byte piece of the result per thread
         if (wpb > most) wpb = most;
         if (wpb < 1) wpb = 1;
         args.cmb_wpb = (int)wpb;
@@ -3151,6 +3580,15 @@ static int plan(int B, int H, int S, int* n_chunks, int* n_split) {
 using namespace flyhip;
 
 #ifdef FLY_PROFILE
+extern "C" int flyhip_prof_reset(void) {
+    hipDeviceSynchronize();
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_prof)) != hipSuccess) return -1;
+    if (hipMemset(p, 0, sizeof(long long) * 16384 * 8) != hipSuccess) return -1;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_prof_k)) != hipSuccess) return -1;
+    if (hipMemset(p, 0, sizeof(long long) * 4096 * 8) != hipSuccess) return -1;
+    return hipDeviceSynchronize() == hipSuccess ? 0 : -1;
+}
 extern "C" int flyhip_prof_read_k(long long* dst, int n_workgroups) {
     hipDeviceSynchronize();
     hipError_t e = hipMemcpyFromSymbol(dst, HIP_SYMBOL(g_prof_k), sizeof(long long) * 8 * n_workgroups);
@@ -3223,12 +3661,12 @@ extern "C" int flyhip_sb_kv_reduce(const void* k, const void* v, const float* pr
     if (rc || q) return rc;          // with query features asked for (several parts per query tile) the
                                      // partial reductions are combined inside flyhip_sblocal_fwd's launch
     const int per = m * (D + 1);
-    hipLaunchKernelGGL(sb_combine_kernel, dim3((per + NT - 1) / NT, B * H), dim3(NT), 0, st,
+    hipLaunchKernelGGL(sb_combine_kernel, dim3((per / 4 + NT - 1) / NT, B * H), dim3(NT), 0, st,
                        kv_part, part_max, kv, ksum, kmax, reinterpret_cast<uint16_t*>(kvt), n_split, m, D);
     return check_launch("sb_combine_kernel");
 }
 
-extern "C" int flyhip_sblocal_fwd(const void* q, const void* k, const void* v, const float* proj,
+static int sblocal_fwd_checked(const void* q, const void* k, const void* v, const float* proj,
                                   const void* kfeat, const float* chunk_scale,
                                   float* kv, float* ksum, float* kmax,
                                   const float* qfeat, const float* q_lsq, const void* vt, const void* kvt,
@@ -3263,6 +3701,101 @@ extern "C" int flyhip_sblocal_fwd(const void* q, const void* k, const void* v, c
               q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss, softmax_temp,
               nullptr, nullptr, nullptr};
     return dispatch_fwd(dtype, E, 2 * mh, a, reinterpret_cast<hipStream_t>(stream));
+}
+
+extern "C" int flyhip_sblocal_fwd(const void* q, const void* k, const void* v, const float* proj,
+                                  const void* kfeat, const float* chunk_scale,
+                                  float* kv, float* ksum, float* kmax,
+                                  const float* qfeat, const float* q_lsq, const void* vt, const void* kvt,
+                                  const float* kv_part, const float* part_max, int n_split,
+                                  const int64_t* key_lengths, void* out, float* log_norm,
+                                  float* part_ws, int n_parts,
+                                  int B, int H, int T, int S, int E, int D, int mh, int mh_valid,
+                                  int local_context,
+                                  int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                                  int64_t k_sb, int64_t k_sh, int64_t k_ss,
+                                  int64_t v_sb, int64_t v_sh, int64_t v_ss,
+                                  int64_t o_sb, int64_t o_sh, int64_t o_ss,
+                                  float softmax_temp, int dtype, void* stream) {
+    return sblocal_fwd_checked(q, k, v, proj, kfeat, chunk_scale, kv, ksum, kmax, qfeat, q_lsq, vt, kvt, kv_part, part_max,
+                               n_split, key_lengths, out, log_norm, part_ws, n_parts, B, H, T, S, E, D, mh, mh_valid,
+                               local_context, q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss,
+                               softmax_temp, dtype, stream);
+}
+
+// ---------------------------------------------------------------------------------------
+// the whole forward on one caller-provided workspace
+// ---------------------------------------------------------------------------------------
+namespace {
+struct SbWorkspace {
+    size_t kfeat, chunk_scale, kv_part, part_max, kv, ksum, kmax, vt, kvt, part_ws, qfeat, q_lsq, total;
+    int n_chunks, n_split, n_parts;
+};
+// Every piece starts at a multiple of 256 bytes.  E: padded head dim (= D), mh: padded projection rows.
+SbWorkspace sb_workspace(int B, int H, int T, int S, int E, int mh, int local_context, int dtype) {
+    SbWorkspace w{};
+    plan(B, H, S, &w.n_chunks, &w.n_split);
+    w.n_parts = plan_parts(B, H, T, S, local_context);
+    const size_t bh = (size_t)B * H, nc = w.n_chunks, ns = w.n_split, m = 2 * (size_t)mh, n_qt = (T + TQ - 1) / TQ;
+    const size_t esize = dtype == F32 ? 4 : 2;
+    size_t off = 0;
+    auto take = [&](size_t bytes) { const size_t at = off; off += (bytes + 255) / 256 * 256; return at; };
+    w.kfeat = take(bh * nc * CH * m * esize);
+    w.chunk_scale = take(bh * nc * 4);
+    w.kv_part = take(bh * ns * m * (E + 1) * 4);
+    w.part_max = take(bh * ns * 4);
+    w.kv = take(bh * m * E * 4);
+    w.ksum = take(bh * m * 4);
+    w.kmax = take(bh * 4);
+    w.vt = take(dtype == F32 ? bh * nc * 2 * (128 * (size_t)E + 192 * (size_t)E) : bh * nc * CH * E * 2);
+    w.kvt = take(dtype == F32 ? 0 : bh * E * m * 2);
+    w.part_ws = take(w.n_parts > 1 ? bh * n_qt * w.n_parts * TQ * (E + NSTAT) * 4 : 0);
+    w.qfeat = take(w.n_parts > 1 ? bh * T * m * 4 : 0);
+    w.q_lsq = take(w.n_parts > 1 ? bh * T * 4 : 0);
+    w.total = off;
+    return w;
+}
+}  // namespace
+
+extern "C" int64_t flyhip_sb_workspace_bytes(int B, int H, int T, int S, int E, int mh, int local_context, int dtype) {
+    if (B <= 0 || H <= 0 || T <= 0 || S <= 0 || E <= 0 || mh <= 0 || local_context <= 0 || (dtype != F32 && dtype != BF16)) return -1;
+    return (int64_t)sb_workspace(B, H, T, S, E, mh, local_context, dtype).total;
+}
+
+extern "C" int flyhip_sblocal_forward(const void* q, const void* k, const void* v, const float* proj,
+                                      const int64_t* key_lengths, void* out, float* log_norm,
+                                      void* workspace, int64_t workspace_bytes,
+                                      int B, int H, int T, int S, int E, int D, int mh, int mh_valid, int local_context,
+                                      int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                                      int64_t k_sb, int64_t k_sh, int64_t k_ss,
+                                      int64_t v_sb, int64_t v_sh, int64_t v_ss,
+                                      int64_t o_sb, int64_t o_sh, int64_t o_ss,
+                                      float softmax_temp, int dtype, void* stream) {
+    FLY_REQUIRE(q && k && v && proj && out && log_norm && workspace, "sblocal_forward: null pointer");
+    FLY_REQUIRE(B > 0 && H > 0 && T > 0 && S > 0 && local_context >= 1, "sblocal_forward: empty problem");
+    FLY_REQUIRE(dtype == F32 || dtype == BF16, "sblocal_forward supports float32 and bfloat16, got dtype code %d", dtype);
+    FLY_REQUIRE(E == D && E > 0 && mh > 0, "sblocal_forward: padded head dims must be equal (E=%d, D=%d)", E, D);
+    FLY_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0, "sblocal_forward: the workspace must be aligned to 256 bytes");
+    const SbWorkspace w = sb_workspace(B, H, T, S, E, mh, local_context, dtype);
+    FLY_REQUIRE(workspace_bytes >= (int64_t)w.total, "sblocal_forward: the workspace holds %lld bytes, this problem needs %lld "
+                "(flyhip_sb_workspace_bytes)", (long long)workspace_bytes, (long long)w.total);
+    char* ws = reinterpret_cast<char*>(workspace);
+    auto f = [&](size_t at) { return reinterpret_cast<float*>(ws + at); };
+    const bool split = w.n_parts > 1;
+    void* vt = ws + w.vt;
+    void* kvt = dtype == BF16 ? ws + w.kvt : nullptr;
+    int rc = flyhip_sb_kv_reduce(k, v, proj, key_lengths, ws + w.kfeat, f(w.chunk_scale), f(w.kv_part), f(w.part_max),
+                                 f(w.kv), f(w.ksum), f(w.kmax),
+                                 split ? q : nullptr, split ? f(w.qfeat) : nullptr, split ? f(w.q_lsq) : nullptr, T,
+                                 q_sb, q_sh, q_ss, vt, kvt, B, H, S, E, D, mh, mh_valid, w.n_split,
+                                 k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, softmax_temp, dtype, stream);
+    if (rc) return rc;
+    return sblocal_fwd_checked(q, k, v, proj, ws + w.kfeat, f(w.chunk_scale), f(w.kv), f(w.ksum), f(w.kmax),
+                               split ? f(w.qfeat) : nullptr, split ? f(w.q_lsq) : nullptr, vt, kvt,
+                               f(w.kv_part), f(w.part_max), w.n_split, key_lengths, out, log_norm,
+                               split ? f(w.part_ws) : nullptr, w.n_parts, B, H, T, S, E, D, mh, mh_valid, local_context,
+                               q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss,
+                               softmax_temp, dtype, stream);
 }
 
 // ---------------------------------------------------------------------------------------

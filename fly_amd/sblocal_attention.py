@@ -29,13 +29,17 @@ def _vector_ready(x):
 
 
 class SBLocalPlan:
-    """Scratch buffers and the two C-ABI calls for one problem shape.  Callers that run the same
-    shape repeatedly (serving loops, benchmarks) keep one plan and call ``run`` with tensors that
-    are already padded and vector-ready; ``sblocal_forward`` builds a plan per call.
+    """The device scratch and the C-ABI calls for one problem shape.  Callers that run the same shape
+    repeatedly (serving loops, benchmarks, the module below) keep one plan and call ``run`` with tensors
+    that are already padded and vector-ready; nothing is allocated after the first call.
 
     q (B,T,H,dim), k, v (B,S,H,dim), proj (mh, dim) float32, lens (B,) int64 or None,
-    out (B,T,H,dim), log_norm (B,H,T) float32.  Buffers of one plan are shared by its runs: runs
-    of the same plan on different streams race."""
+    out (B,T,H,dim), log_norm (B,H,T) float32.  The scratch of one plan is shared by its runs: runs
+    of the same plan on different streams race.
+
+    ``run`` is one library call (flyhip_sblocal_forward) on one workspace;
+    ``run_keys`` / ``run_queries`` are the two halves as separate calls (flyhip_sb_kv_reduce,
+    flyhip_sblocal_fwd) on individually allocated buffers, which are created on first use."""
 
     def __init__(self, B, H, T, S, dim, mh, mh_valid, dtype, device, local_context, n_parts=None,
                  operand_images=True):
@@ -43,11 +47,32 @@ class SBLocalPlan:
         _lib.call('flyhip_sb_plan', B, H, T, S, local_context, ctypes.byref(n_chunks), ctypes.byref(n_split),
                   ctypes.byref(parts))
         self.n_chunks, self.n_split = n_chunks.value, n_split.value
+        self.planned_parts = parts.value
         self.n_parts = parts.value if n_parts is None else n_parts
         self.local_context = local_context
         self.shape = (B, H, T, S, dim, mh, mh_valid)
         self.device = torch.device(device)
+        self.dtype = dtype
         self.code = _lib.DTYPE_CODE[dtype]
+        self.operand_images = operand_images
+        self.workspace = None
+        self._buffers = False
+
+    def _workspace(self):
+        if self.workspace is None:
+            B, H, T, S, dim, mh, _ = self.shape
+            size = _lib.load().flyhip_sb_workspace_bytes(B, H, T, S, dim, mh, self.local_context, self.code)
+            if size < 0:
+                raise ValueError('flyhip_sb_workspace_bytes rejected the problem shape')
+            self.workspace = torch.empty(size, dtype=torch.uint8, device=self.device)
+        return self.workspace
+
+    def _make_buffers(self):
+        """Scratch of the two-call path, one tensor each."""
+        if self._buffers:
+            return
+        B, H, T, S, dim, mh, _ = self.shape
+        dtype, device = self.dtype, self.device
         m, f32 = 2 * mh, torch.float32
         self.kfeat = torch.empty(B, H, self.n_chunks * 64, m, dtype=dtype, device=device)   # opaque, in the input dtype
         self.chunk_scale = torch.empty(B, H, self.n_chunks, dtype=f32, device=device)
@@ -56,15 +81,15 @@ class SBLocalPlan:
         self.kv = torch.empty(B, H, m, dim, dtype=f32, device=device)
         self.ksum = torch.empty(B, H, m, dtype=f32, device=device)
         self.kmax = torch.empty(B, H, dtype=f32, device=device)
-        # bf16 inputs: V per 32-key tile and K'^T V in the operand order of the bf16 MFMA (opaque)
         self.vt = self.kvt = None
-        if dtype == torch.float32 and operand_images:
+        if dtype == torch.float32 and self.operand_images:
             # float inputs: the band kernel runs on the bf16 matrix pipe from images of every 32-key tile
             # (K in two bf16 pieces, V transposed in three; kfeat then holds the features in two pieces);
             # 128 E + 192 D bytes per tile, two tiles per 64-key chunk.  Without it (block-sparse supports)
             # the fp32-MFMA kernels run from fp32 features.
             self.vt = torch.empty(B, H, self.n_chunks, 2 * (128 * dim + 192 * dim), dtype=torch.uint8, device=device)
         if dtype == torch.bfloat16:
+            # bf16 inputs: V per 32-key tile and K'^T V in the operand order of the bf16 MFMA (opaque)
             self.vt = torch.empty(B, H, self.n_chunks * 64, dim, dtype=dtype, device=device)
             self.kvt = torch.empty(B, H, dim, m, dtype=dtype, device=device)
         # with several parts per query tile the key pass also computes the query features, once
@@ -74,11 +99,13 @@ class SBLocalPlan:
                                        device=device)
             self.qfeat = torch.empty(B, H, T, m, dtype=f32, device=device)
             self.q_lsq = torch.empty(B, H, T, dtype=f32, device=device)
+        self._buffers = True
 
     def run_keys(self, q, k, v, proj, lens, t, stream=None):
         """The key-side pass (features of the keys, K'^T V, sum K'); with several parts per query
         tile also the features of the queries `q`."""
         B, H, T, S, dim, mh, mh_valid = self.shape
+        self._make_buffers()
         stream = _lib.stream_ptr(self.device) if stream is None else stream
         q_args = (None, None, None, 0, 0, 0, 0)
         if self.n_parts > 1:
@@ -93,6 +120,7 @@ class SBLocalPlan:
 
     def run_queries(self, q, k, v, proj, lens, local_context, t, out, log_norm, stream=None):
         B, H, T, S, dim, mh, mh_valid = self.shape
+        self._make_buffers()
         stream = _lib.stream_ptr(self.device) if stream is None else stream
         _lib.call('flyhip_sblocal_fwd', q.data_ptr(), k.data_ptr(), v.data_ptr(), proj.data_ptr(),
                   self.kfeat.data_ptr(), self.chunk_scale.data_ptr(), self.kv.data_ptr(),
@@ -108,6 +136,7 @@ class SBLocalPlan:
         """``run_queries`` through flyhip_sblocal_fwd_static: the partial outputs go to the library's
         built-in scratch array instead of ``self.part_ws`` (nothing is allocated by the call)."""
         B, H, T, S, dim, mh, mh_valid = self.shape
+        self._make_buffers()
         stream = _lib.stream_ptr(self.device) if stream is None else stream
         _lib.call('flyhip_sblocal_fwd_static', q.data_ptr(), k.data_ptr(), v.data_ptr(), proj.data_ptr(),
                   self.kfeat.data_ptr(), self.chunk_scale.data_ptr(), self.kv.data_ptr(),
@@ -124,6 +153,7 @@ class SBLocalPlan:
         key pass as in ``run``, then the fp32 band kernel walking lists of 32-key blocks (``tables`` =
         union_table(layout, rows_per_group=2) on the device).  One part per query tile, no key lengths."""
         B, H, T, S, dim, mh, mh_valid = self.shape
+        self._make_buffers()
         tl_ptr, tl_inner, tl_blk = tables[:3]
         tl_order = tables[3] if len(tables) > 3 else None      # union_order(tl_ptr, H): longest lists first
         # long lists walked in parts (sbblocksparse_attention.fused_tables): scratch for their partials
@@ -150,10 +180,22 @@ class SBLocalPlan:
                       t, self.code, stream)
 
     def run(self, q, k, v, proj, lens, local_context, t, out, log_norm):
+        B, H, T, S, dim, mh, mh_valid = self.shape
+        if self.n_parts != self.planned_parts or not self.operand_images or local_context != self.local_context:
+            # a part count or band the library would not choose itself: the two-call path takes them as arguments
+            with torch.cuda.device(self.device):
+                stream = _lib.stream_ptr(self.device)
+                self.run_keys(q, k, v, proj, lens, t, stream)
+                self.run_queries(q, k, v, proj, lens, local_context, t, out, log_norm, stream)
+            return
+        ws = self._workspace()
         with torch.cuda.device(self.device):
-            stream = _lib.stream_ptr(self.device)
-            self.run_keys(q, k, v, proj, lens, t, stream)
-            self.run_queries(q, k, v, proj, lens, local_context, t, out, log_norm, stream)
+            _lib.call('flyhip_sblocal_forward', q.data_ptr(), k.data_ptr(), v.data_ptr(), proj.data_ptr(), _lib.ptr(lens),
+                      out.data_ptr(), log_norm.data_ptr(), ws.data_ptr(), ws.numel(),
+                      B, H, T, S, dim, dim, mh, mh_valid, local_context,
+                      q.stride(0), q.stride(2), q.stride(1), k.stride(0), k.stride(2), k.stride(1),
+                      v.stride(0), v.stride(2), v.stride(1), out.stride(0), out.stride(2), out.stride(1),
+                      t, self.code, _lib.stream_ptr(self.device))
 
 
 def sblocal_forward(query, key, value, projection_matrix, local_context, softmax_temp=None,

@@ -98,6 +98,25 @@ int flyhip_sblocal_fwd(const void* q, const void* k, const void* v, const float*
                        int64_t o_sb, int64_t o_sh, int64_t o_ss,
                        float softmax_temp, int dtype, void* stream);
 
+/* The whole forward of Scatterbrain-local attention in one call (ref: SBLocalAttention.forward,
+ * src/models/attention/sblocal_attention.py:73-122, for causal = False, attn_mask = None, eps = 0, no dropout):
+ * flyhip_sb_kv_reduce followed by flyhip_sblocal_fwd on ONE caller-provided workspace, which the library divides
+ * into the scratch of both calls (for float inputs that includes the tile images of the key pass, so the band
+ * kernel runs on the bf16 matrix pipe).  flyhip_sb_workspace_bytes gives its size for a problem (E = D: padded
+ * head dim, mh: padded projection rows; -1 for bad arguments).  The workspace must be aligned to 256 bytes; its
+ * contents need no initialisation and mean nothing between calls; one call at a time may use it.
+ * Arguments as for flyhip_sb_kv_reduce / flyhip_sblocal_fwd. */
+int64_t flyhip_sb_workspace_bytes(int B, int H, int T, int S, int E, int mh, int local_context, int dtype);
+int flyhip_sblocal_forward(const void* q, const void* k, const void* v, const float* proj,
+                           const int64_t* key_lengths, void* out, float* log_norm,
+                           void* workspace, int64_t workspace_bytes,
+                           int B, int H, int T, int S, int E, int D, int mh, int mh_valid, int local_context,
+                           int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                           int64_t k_sb, int64_t k_sh, int64_t k_ss,
+                           int64_t v_sb, int64_t v_sh, int64_t v_ss,
+                           int64_t o_sb, int64_t o_sh, int64_t o_ss,
+                           float softmax_temp, int dtype, void* stream);
+
 /* flyhip_sblocal_fwd for callers that cannot allocate device memory -- code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.
  * Same arguments and results as flyhip_sblocal_fwd except that there is no part_ws: the partial
