@@ -2,10 +2,9 @@
 """Benchmark of the Scatterbrain-local attention forward on one MI355X.
 
 One "step" is one forward of BASELINE config 1 (fp32, B=2, H=1, L=3136, d=64, band 256 each side,
-128 orthogonal-Gaussian random features) through the C ABI: the key-side pass
-(flyhip_sb_kv_reduce, one launch) followed by the fused band pass (flyhip_sblocal_fwd: the band
-kernel and the kernel that merges its partial results and adds the low-rank term), inputs resident
-in HBM.  Prints ONE JSON line: tokens/s for the whole forward, the roofline of the dominant kernel
+128 orthogonal-Gaussian random features) through the C ABI (flyhip_sblocal_forward: the key-side
+pass, the fused band kernel, and the kernel that merges its partial results and adds the low-rank
+term), inputs resident in HBM.  Prints ONE JSON line: tokens/s for the whole forward, the roofline of the dominant kernel
 (the fused band kernel, timed with events on its stream inside the timed region), the CPU oracle
 timed on this box's host cores, and -- as `extra` -- the block-sparse SDD / softmax / DSD stages
 of BASELINE config 2 (bf16, B=8, H=12, L=4096, d=64, block 32) and whole-forward timings of
@@ -25,10 +24,19 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
-# HBM bytes one launch of the fused band kernel moves at config 1: rocprofv3 FETCH_SIZE (8785 KiB,
-# scale 2.0 from a plain copy of known size) + WRITE_SIZE (8518 KiB, scale 1.0), as committed in
-# profiles/sblocal_fwd_config1_fp32.md.  Counters cannot be read from inside this process.
-BAND_KERNEL_TRAFFIC_BYTES = 26.7e6
+# HBM bytes one launch of the dominant kernel moves at the benchmarked workload: rocprofv3 FETCH_SIZE / WRITE_SIZE
+# readings scaled by a plain copy of known size, kept with the profile summaries they come from
+TRAFFIC_FILE = os.path.join(ROOT, 'profiles', 'sblocal_fwd_config1_fp32_traffic.json')
+
+
+def band_kernel_traffic():
+    """Scaled read + write bytes per launch of the band kernel from the committed counter summary, or None."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            t = json.load(f)
+        return float(t['band_kernel']['hbm_read_bytes']) + float(t['band_kernel']['hbm_write_bytes'])
+    except (OSError, KeyError, ValueError):
+        return None
 
 
 def sblocal_flops(B, H, T, S, E, D, m, lc):
@@ -49,13 +57,12 @@ def sblocal_flops(B, H, T, S, E, D, m, lc):
 
 def bench_sblocal(steps, warmup, cpu_baseline=True):
     import fly_amd
+    from fly_amd import _lib
     from fly_amd.sblocal_attention import SBLocalPlan
     dev = torch.device('cuda:0')
     B, H, L, E, D, mh, lc = 2, 1, 3136, 64, 64, 64, 512
     g = torch.Generator().manual_seed(0)
-    q = torch.randn(B, L, H, E, generator=g) * E ** -0.25
-    k = torch.randn(B, L, H, E, generator=g) * E ** -0.25
-    v = torch.randn(B, L, H, D, generator=g)
+    q, k, v = (torch.randn(B, L, H, E, generator=g) * E ** -0.25 for _ in range(3))      # q, k, v ~ N(0,1) d^-1/4
     torch.manual_seed(0)
     P = fly_amd.gaussian_orthogonal_random_matrix(mh, E)
     t = 1 / math.sqrt(E)
@@ -67,25 +74,38 @@ def bench_sblocal(steps, warmup, cpu_baseline=True):
     for _ in range(warmup):
         plan.run(qd, kd, vd, Pd, None, lc, t, out, ln)
     torch.cuda.synchronize()
-    # The dominant kernel is timed inside the timed region on every EVERY-th step: the library
-    # records two events right around the fused band kernel, on its stream.  (An event pair costs a
-    # few microseconds of a 60 microsecond step, so it is not put around every launch.)
-    EVERY = 8
-    sampled = [i for i in range(steps) if i % EVERY == 0]
+    # The dominant kernel is timed inside the timed region: on sampled steps the library records two events
+    # right around the band kernel, on its stream.  At least 16 samples whatever the step count (an event pair
+    # costs a few microseconds of a 35 microsecond step, so it is not put around every launch of a long run).
+    every = max(1, steps // 16)
+    sampled = [i for i in range(steps) if i % every == 0]
     ev = {i: (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for i in sampled}
-    from fly_amd import _lib
     for a, b in ev.values():             # create the underlying hipEvent_t objects before timing
         a.record(); b.record()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(steps):
-        plan.run_keys(qd, kd, vd, Pd, None, t)
         if i in ev:
             _lib.call('flyhip_sb_time_next_fwd', ev[i][0].cuda_event, ev[i][1].cuda_event)
-        plan.run_queries(qd, kd, vd, Pd, None, lc, t, out, ln)
+        plan.run(qd, kd, vd, Pd, None, lc, t, out, ln)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     fwd_ms = sum(a.elapsed_time(b) for a, b in ev.values()) / len(ev)
+
+    # the same forward through the drop-in module (reference signature sblocal_attention.py:43-44): argument
+    # checks, cached scratch, two result tensors per call
+    mod = fly_amd.SBLocalAttention(lc, dim_heads=E, nb_features=2 * mh).to(dev).eval()
+    mod.feature_map.projection_matrix.copy_(Pd)
+    mod.feature_map.freeze_projection()
+    with torch.no_grad():
+        for _ in range(max(warmup, 3)):
+            mod(qd, kd, vd)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(steps):
+            mod(qd, kd, vd)
+        torch.cuda.synchronize()
+        module_ms = (time.perf_counter() - t1) / steps * 1e3
 
     total_flops, fwd_flops = sblocal_flops(B, H, L, L, E, D, 2 * mh, lc)
     ms_per_step = wall / steps * 1e3
@@ -93,10 +113,14 @@ def bench_sblocal(steps, warmup, cpu_baseline=True):
     res = {
         'tokens_per_s': B * L / (wall / steps),
         'ms_per_step': ms_per_step,
-        'roofline': {'bound': 'mfma', 'kernel': 'sblocal_fwd_kernel<float,64,64,128>',
+        'module_forward_ms': module_ms,
+        'roofline': {'bound': 'mfma', 'kernel': 'sblocal_fwd_x3_kernel<64,64,128,split>',
                      'achieved': achieved, 'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s',
-                     'frac': achieved / PEAK_FP32_MFMA_TFLOPS, 'traffic': BAND_KERNEL_TRAFFIC_BYTES,
-                     'kernel_ms': fwd_ms, 'flops_per_launch': fwd_flops, 'launches_timed': len(ev)},
+                     'frac': achieved / PEAK_FP32_MFMA_TFLOPS, 'traffic': band_kernel_traffic(),
+                     'kernel_ms': fwd_ms, 'flops_per_launch': fwd_flops, 'launches_timed': len(ev),
+                     'arithmetic': 'fp32 inputs, outputs and accumulation; products on v_mfma_f32_16x16x32_bf16 from '
+                                   'operands split into bf16 pieces (scores 3 piece products, feature overlap 4 on '
+                                   'features rounded to 16 bits, P V 6); priced against the fp32 MFMA peak'},
         'parity': None,
         'flops_per_step': total_flops,
     }
@@ -111,7 +135,8 @@ def bench_sblocal(steps, warmup, cpu_baseline=True):
     res['parity'] = {
         'out_rel_err': float((out.cpu().double() - ref_out).abs().max() / ref_out.abs().max()),
         'log_norm_rel_err': float((ln.cpu().double().unsqueeze(-1) - ref_ln).abs().max() / ref_ln.abs().max())}
-    torch.set_num_threads(min(os.cpu_count() or 1, 16))
+    host_cpus = os.cpu_count() or 1
+    torch.set_num_threads(min(host_cpus, 16))          # the box's CPU share for one GPU is 16 cores
     osb.sblocal_attention(q, k, v, P, lc)
     n, t0 = 0, time.perf_counter()
     while True:
@@ -121,8 +146,9 @@ def bench_sblocal(steps, warmup, cpu_baseline=True):
         if el > 12.0:
             break
     res['cpu_baseline'] = {'value': B * L * n / el, 'unit': 'tokens/s', 'cores': torch.get_num_threads(),
-                           'kind': 'port',
-                           'sample': f'{n} full-size forwards of the same workload (fp32 oracle, {el:.1f} s)'}
+                           'host_cpus': host_cpus, 'kind': 'port',
+                           'sample': f'{n} full-size forwards of the same workload (fp32 oracle, {el:.1f} s, '
+                                     f'{torch.get_num_threads()} threads of {host_cpus} host CPUs)'}
     return res
 
 
@@ -382,6 +408,7 @@ def main():
         'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f32', 'data': 'synthetic',
         'config': {'workload': 'BASELINE config 1 (configs[0]): SBLocal fwd fp32 B=2 H=1 L=3136 d=64 '
                                'local_context=512 nb_features=128, seeded orthogonal-Gaussian projection'},
+        'module_forward_ms': sb['module_forward_ms'],
         'roofline': sb['roofline'], 'cpu_baseline': sb['cpu_baseline'],
         'gpu_over_cpu': sb['tokens_per_s'] / sb['cpu_baseline']['value'] if sb['cpu_baseline'] else None,
         'parity': sb['parity'],

@@ -161,6 +161,10 @@ __device__ __forceinline__ void load_proj(float* Ps, const float* proj, float sc
 // weights staged in LDS (`wgt`, n_split floats) so that the loads over s are independent and stay
 // in flight together
 constexpr int MAX_SPLIT = 1024;
+#ifndef FLY_CMB_BATCH
+#define FLY_CMB_BATCH 25
+#endif
+constexpr int CMB_BATCH = FLY_CMB_BATCH;     // partial reductions whose loads a combining thread keeps in flight together
 __device__ __forceinline__ void sb_combine_body(float* wgt, const float* kv_part, const float* part_max, float* kv,
                                                 float* ksum, float* kmax_out, uint16_t* kvt, int bh, int ci, int wpb,
                                                 int n_split, int M, int D) {
@@ -177,7 +181,7 @@ __device__ __forceinline__ void sb_combine_body(float* wgt, const float* kv_part
     __syncthreads();
     if (ci == 0 && threadIdx.x == 0) kmax_out[bh] = (kmax == -INFINITY) ? 0.f : kmax;
     // Threads walk a partial in its storage order, four consecutive floats each (16-byte loads, coalesced
-    // over the splits), in batches of 16 splits whose loads are all in flight together: the partials come
+    // over the splits), in batches of CMB_BATCH splits whose loads are all in flight together: the partials come
     // from memory, and one round trip per split would make this the longest job of the launch.  The K'^T V
     // part is in accumulator order: offset ((tile*64 + lane)*4 + i) holds element (r, d) of tile (r/16, d/16)
     // with lane = 16*((r%16)/4) + d%16 and i = r%4.
@@ -185,12 +189,12 @@ __device__ __forceinline__ void sb_combine_body(float* wgt, const float* kv_part
     for (int q4 = ci * nthr + threadIdx.x; q4 < per4; q4 += wpb * nthr) {
         const floatx4* src = reinterpret_cast<const floatx4*>(kv_part + (long)bh * n_split * per) + q4;
         floatx4 acc = {0.f, 0.f, 0.f, 0.f};
-        for (int s0 = 0; s0 < n_split; s0 += 16) {
-            floatx4 pv[16];
+        for (int s0 = 0; s0 < n_split; s0 += CMB_BATCH) {
+            floatx4 pv[CMB_BATCH];
 #pragma unroll
-            for (int u = 0; u < 16; ++u) pv[u] = src[(long)min(s0 + u, n_split - 1) * per4];
+            for (int u = 0; u < CMB_BATCH; ++u) pv[u] = src[(long)min(s0 + u, n_split - 1) * per4];
 #pragma unroll
-            for (int u = 0; u < 16; ++u)
+            for (int u = 0; u < CMB_BATCH; ++u)
                 if (s0 + u < n_split) acc += wgt[s0 + u] * pv[u];
         }
         const int idx = 4 * q4;
@@ -2407,8 +2411,12 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
     const int n_qt = (a.T + TQ - 1) / TQ;
     if (SPLIT && (int)blockIdx.x >= a.band_wgs) {       // combine role, see sblocal_fwd_kernel
         const int ci = blockIdx.x - a.band_wgs;
+        FLY_PROF(0);
+#ifndef FLY_EXP_NOCOMBINE
         sb_combine_body(smem, a.kv_part, a.part_max, const_cast<float*>(a.kv), const_cast<float*>(a.ksum),
                         const_cast<float*>(a.kmax), nullptr, ci / a.cmb_wpb, ci % a.cmb_wpb, a.cmb_wpb, a.n_split, M, D);
+#endif
+        FLY_PROF(7);
         return;
     }
     const int n_items = a.B * a.H * n_qt * a.n_parts;
@@ -2568,7 +2576,9 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
         const bool more = kt + 1 < kt_hi;
         float cscale_next = cscale;
         if (more) {                                      // next tile's loads fly during the MFMAs
+#ifndef FLY_EXP_NOFETCH
             fetch(kt + 1);
+#endif
             cscale_next = csp[(s_base + TK) / CH];
         }
         const float wc = __builtin_amdgcn_exp2f((cscale - kmax) * LOG2E);
@@ -2589,6 +2599,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
                     s1[kb] = mma_bf16(khi, qh[ks], s1[kb]);
                 }
             // overlap: all four piece products (exact product of the rounded features)
+#ifndef FLY_EXP_NOS2
 #pragma unroll
             for (int ks = 0; ks < FS; ++ks)
 #pragma unroll
@@ -2600,6 +2611,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
                     s2[kb] = mma_bf16(fhi, qfl[ks], s2[kb]);
                     s2[kb] = mma_bf16(fhi, qfh[ks], s2[kb]);
                 }
+#endif
             const bool interior = s_base - (qw0 + 15) >= -lc_lo && s_base + TK - 1 - qw0 < lc_hi &&
                                   s_base + TK <= len && qw0 + 15 < a.T;
             floatx4 p[KB];
@@ -2637,11 +2649,20 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
                         p[kb][i] = e - ov * beta;
                     }
             };
+#ifdef FLY_EXP_NOSOFT
+            p[0] = s1[0] + s2[0]; p[1] = s1[1] + s2[1];
+#else
             if (interior) soft(std::false_type{}); else soft(std::true_type{});
+#endif
             zp += ovs * wc;
             // O^T[d][query] += sum_keys V[key][d] p[key][query]: P exactly in three pieces, six products
             uintx4 ph, pm, pl;
+#ifdef FLY_EXP_NOSPLIT
+            ph = pm = pl = uintx4{__float_as_uint(p[0][0]), __float_as_uint(p[0][1]), __float_as_uint(p[1][0]), __float_as_uint(p[1][1])};
+#else
             split3(p[0], p[1], ph, pm, pl);
+#endif
+#ifndef FLY_EXP_NOPV
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
                 const uintx4 vh = *reinterpret_cast<const uintx4*>(st + voff + 16 * db * TL::V_ROW);
@@ -2656,10 +2677,17 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
                 o = mma_bf16(vh, ph, o);
                 oacc[db] = o;
             }
+#else
+            oacc[0] += __builtin_bit_cast(floatx4, ph) + __builtin_bit_cast(floatx4, pm) + __builtin_bit_cast(floatx4, pl);
+#endif
         }
+#ifndef FLY_EXP_NOFETCH
         if (more) stash(cur ^ 1);
+#endif
         cscale = cscale_next;
+#ifndef FLY_EXP_NOBARRIER
         __syncthreads();
+#endif
     }
 
     FLY_PROF(3);

@@ -198,14 +198,35 @@ class SBLocalPlan:
                       t, self.code, _lib.stream_ptr(self.device))
 
 
+def _padded_projection(projection_matrix, mh, dim, cache):
+    """The projection as the kernels want it: float32, (mh, dim), zero rows / columns as padding.  The caller's
+    tensor itself when it already has that form; otherwise a padded copy, kept in `cache` until the
+    caller's tensor is replaced or written to."""
+    mh_valid, E = projection_matrix.shape
+    if (mh_valid, E) == (mh, dim) and projection_matrix.dtype == torch.float32 and projection_matrix.is_contiguous():
+        return projection_matrix
+    stamp = (projection_matrix.data_ptr(), projection_matrix._version, mh, dim)
+    if cache is not None and cache.get('projection_stamp') == stamp:
+        return cache['projection']
+    proj = torch.zeros(mh, dim, dtype=torch.float32, device=projection_matrix.device)
+    proj[:mh_valid, :E] = projection_matrix.to(torch.float32)
+    if cache is not None:
+        cache['projection_stamp'], cache['projection'] = stamp, proj
+    return proj
+
+
 def sblocal_forward(query, key, value, projection_matrix, local_context, softmax_temp=None,
-                    key_lengths=None):
+                    key_lengths=None, cache=None):
     """Scatterbrain-local attention forward on the GPU.
 
     query (B,T,H,E), key (B,S,H,E), value (B,S,H,D) float32 or bfloat16 CUDA tensors;
     projection_matrix (m/2, E); key_lengths (B,) int64 or None.  Computes what
     sblocal_attention.py:73-122 computes for causal=False, attn_mask=None, eps=0, no dropout.
     Returns (out (B,T,H,D) in the input dtype, log_normalization (B,H,T,1) float32).
+
+    cache: an optional dict the caller keeps between calls (SBLocalAttention keeps one per module).  It holds
+    the plan -- the device scratch -- of every problem shape seen and the padded projection, so that a repeated
+    call allocates nothing but its two results.  Calls that share a cache share scratch: one at a time.
     """
     _lib.require_gpu(query, key, value, projection_matrix, key_lengths)
     if query.dtype not in (torch.float32, torch.bfloat16):
@@ -233,15 +254,19 @@ def sblocal_forward(query, key, value, projection_matrix, local_context, softmax
             x = F.pad(x, (0, dim - x.shape[-1]))      # zero columns change neither dots nor norms
         return x if _vector_ready(x) else x.contiguous()
     q, k, v = prep(query), prep(key), prep(value)
-    proj = torch.zeros(mh, dim, dtype=torch.float32, device=query.device)
-    proj[:mh_valid, :E] = projection_matrix.to(torch.float32)
+    proj = _padded_projection(projection_matrix, mh, dim, cache)
     lens = None
     if key_lengths is not None:
         lens = key_lengths.to(device=query.device, dtype=torch.int64).contiguous()
         if lens.shape != (B,):
             raise ValueError(f'key_lengths must have shape ({B},)')
 
-    plan = SBLocalPlan(B, H, T, S, dim, mh, mh_valid, query.dtype, query.device, local_context)
+    plan_key = (B, H, T, S, dim, mh, mh_valid, query.dtype, query.device, local_context)
+    plan = None if cache is None else cache.get(plan_key)
+    if plan is None:
+        plan = SBLocalPlan(B, H, T, S, dim, mh, mh_valid, query.dtype, query.device, local_context)
+        if cache is not None:
+            cache[plan_key] = plan
     out = torch.empty(B, T, H, dim, dtype=query.dtype, device=query.device)
     log_norm = torch.empty(B, H, T, dtype=torch.float32, device=query.device)
     plan.run(q, k, v, proj, lens, local_context, t, out, log_norm)
@@ -291,9 +316,9 @@ class _SBLocalFn(torch.autograd.Function):
     forward is the fused kernel path; the backward is sblocal_backward.sblocal_backward."""
 
     @staticmethod
-    def forward(ctx, query, key, value, projection_matrix, local_context, softmax_temp, key_lengths):
+    def forward(ctx, query, key, value, projection_matrix, local_context, softmax_temp, key_lengths, cache=None):
         out, log_norm = sblocal_forward(query, key, value, projection_matrix, local_context,
-                                        softmax_temp=softmax_temp, key_lengths=key_lengths)
+                                        softmax_temp=softmax_temp, key_lengths=key_lengths, cache=cache)
         ctx.save_for_backward(query, key, value, projection_matrix, out, log_norm)
         ctx.args = (local_context, softmax_temp, key_lengths)
         ctx.mark_non_differentiable(log_norm)
@@ -306,16 +331,16 @@ class _SBLocalFn(torch.autograd.Function):
         local_context, softmax_temp, key_lengths = ctx.args
         dq, dk, dv = sblocal_backward(query, key, value, projection_matrix, local_context, softmax_temp,
                                       key_lengths, out, log_norm, grad_out)
-        return dq, dk, dv, None, None, None, None
+        return dq, dk, dv, None, None, None, None, None
 
 
 def sblocal_attention_fn(query, key, value, projection_matrix, local_context, softmax_temp=None,
-                         key_lengths=None):
+                         key_lengths=None, cache=None):
     """sblocal_forward, differentiable with respect to query, key and value."""
     if torch.is_grad_enabled() and any(x.requires_grad for x in (query, key, value)):
-        return _SBLocalFn.apply(query, key, value, projection_matrix, local_context, softmax_temp, key_lengths)
+        return _SBLocalFn.apply(query, key, value, projection_matrix, local_context, softmax_temp, key_lengths, cache)
     return sblocal_forward(query, key, value, projection_matrix, local_context, softmax_temp=softmax_temp,
-                           key_lengths=key_lengths)
+                           key_lengths=key_lengths, cache=cache)
 
 
 class SBLocalAttention(nn.Module):
@@ -341,6 +366,8 @@ class SBLocalAttention(nn.Module):
         self.softmax_temp = softmax_temp
         self.dropout = nn.Dropout(attention_dropout)
         self.softmax_eps = softmax_eps
+        # device scratch per problem shape and the padded projection, kept between calls (see sblocal_forward)
+        self._scratch_cache = {}
 
     def forward(self, query, key, value, attn_mask=None, key_padding_mask=None, need_weights=False,
                 return_attn_unnormalized=False):
@@ -362,6 +389,6 @@ class SBLocalAttention(nn.Module):
         self.feature_map.new_feature_map(query.device)
         out, log_norm = sblocal_attention_fn(query, key, value, self.feature_map.projection_matrix,
                                              self.local_context, softmax_temp=self.softmax_temp,
-                                             key_lengths=lengths)
+                                             key_lengths=lengths, cache=self._scratch_cache)
         self.last_log_normalization = log_norm.detach()
         return out, None

@@ -10,12 +10,12 @@ from oracle import sblocal as osb
 pytestmark = pytest.mark.gpu
 
 
-def make_inputs(B, T, S, H, E, D, mh, seed, dtype=torch.float32, scale=None):
+def make_inputs(B, T, S, H, E, D, mh, seed, dtype=torch.float32, scale=None, scale_v=False):
     g = torch.Generator().manual_seed(seed)
     scale = E ** -0.25 if scale is None else scale
     q = torch.randn(B, T, H, E, generator=g) * scale
     k = torch.randn(B, S, H, E, generator=g) * scale
-    v = torch.randn(B, S, H, D, generator=g)
+    v = torch.randn(B, S, H, D, generator=g) * (scale if scale_v else 1.0)
     P = osb.gaussian_orthogonal_random_matrix(mh, E, generator=g)
     return q.to(dtype), k.to(dtype), v.to(dtype), P
 
@@ -81,8 +81,8 @@ def test_fp32_odd_sizes_and_lengths():
 
 
 def test_config1_full_size():
-    """BASELINE config 1: B=2, H=1, L=3136, d=64, window 512, 128 features, fp32."""
-    q, k, v, P = make_inputs(2, 3136, 3136, 1, 64, 64, 64, seed=0)
+    """BASELINE config 1: B=2, H=1, L=3136, d=64, window 512, 128 features, fp32; q, k, v ~ N(0,1) d^-1/4."""
+    q, k, v, P = make_inputs(2, 3136, 3136, 1, 64, 64, 64, seed=0, scale_v=True)
     check_fp32(*run_both(q, k, v, P, 512))
 
 
@@ -139,6 +139,36 @@ def test_module_dropin():
     assert rel_err(attn.last_log_normalization, ref_ln) <= 1e-4
     with pytest.raises(NotImplementedError):
         attn(q.to(dev), k.to(dev), v.to(dev), need_weights=True)
+
+
+def test_module_keeps_its_scratch_between_calls():
+    """The drop-in module caches the plan (device scratch) and the padded projection per problem shape: a
+    repeated call creates its two result tensors and nothing else, asks the driver for no new memory, and
+    gives the same numbers; a changed projection is picked up."""
+    from fly_amd import SBLocalAttention
+    dev = torch.device('cuda:0')
+    attn = SBLocalAttention(local_context=512, dim_heads=64, nb_features=128).to(dev).eval()
+    q, k, v, P = make_inputs(2, 3136, 3136, 1, 64, 64, 64, seed=4)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    with torch.no_grad():
+        first, _ = attn(qd, kd, vd)
+        torch.cuda.synchronize()
+        stats = torch.cuda.memory_stats(dev)
+        allocs, segments = stats['allocation.all.allocated'], stats['segment.all.allocated']
+        second, _ = attn(qd, kd, vd)
+        torch.cuda.synchronize()
+        stats = torch.cuda.memory_stats(dev)
+    assert stats['allocation.all.allocated'] - allocs <= 2          # out and log_normalization
+    assert stats['segment.all.allocated'] == segments
+    assert torch.equal(first, second)
+    ref_out, _ = osb.sblocal_attention(q.double(), k.double(), v.double(),
+                                       attn.feature_map.projection_matrix.cpu().double(), 512)
+    assert rel_err(second, ref_out) <= 1e-4
+    with torch.no_grad():
+        attn.feature_map.projection_matrix.copy_(P)                  # in place: same storage, new version
+        third, _ = attn(qd, kd, vd)
+    ref_out, _ = osb.sblocal_attention(q.double(), k.double(), v.double(), P.double(), 512)
+    assert rel_err(third, ref_out) <= 1e-4
 
 
 @pytest.mark.parametrize('case', [
