@@ -80,18 +80,20 @@ __global__ __launch_bounds__(256) void bs_sdd_kernel(SddArgs a) {
 // Fast SDD for 32x32 blocks of a 2-byte type with contiguous contraction (K a multiple of 32, at
 // most 128): one wave per (head, block-row).  The wave loads the A fragments of its block-row once
 // (16-byte loads, kept in registers) and then produces the row's blocks one after the other: B fragments with 16-byte loads, 16x16x32 MFMAs, 8-byte stores of a 2 KiB block.
-// The hardware hands consecutive workgroup ids to the eight XCDs in turn, and every XCD has an L2
+// The hardware hands consecutive workgroup ids to the XCDs in turn (n_xcd of them), and every XCD has an L2
 // of its own.  unit_of() turns a 1-D workgroup id into (unit, position inside the unit) such
 // that all `per_unit` workgroups of a unit -- one (batch, head) matrix, whose dense operand they
 // all re-read -- run on one XCD, so that operand comes from HBM once instead of once per XCD.
-constexpr int BS_XCD = 8;
-__device__ __forceinline__ bool unit_of(unsigned id, int per_unit, int n_units, int& unit, int& pos) {
-    const unsigned xcd = id % BS_XCD, slot = id / BS_XCD;
-    unit = (int)(slot / per_unit) * BS_XCD + (int)xcd;
+__device__ __forceinline__ bool unit_of(unsigned id, int n_xcd, int per_unit, int n_units, int& unit, int& pos) {
+    const unsigned xcd = id % (unsigned)n_xcd, slot = id / (unsigned)n_xcd;
+    unit = (int)(slot / per_unit) * n_xcd + (int)xcd;
     pos = (int)(slot % per_unit);
     return unit < n_units;
 }
-static long unit_grid(long n_units, long per_unit) { return (n_units + BS_XCD - 1) / BS_XCD * BS_XCD * per_unit; }
+static long unit_grid(long n_units, long per_unit) {
+    const long x = machine().xcds;
+    return (n_units + x - 1) / x * x * per_unit;
+}
 
 template <typename T> __device__ __forceinline__ uint32_t pack2(float lo, float hi);
 template <> __device__ __forceinline__ uint32_t pack2<bf16_t>(float lo, float hi) { return pack_bf16x2(lo, hi); }
@@ -112,6 +114,7 @@ struct SddRowArgs {
     const int32_t* row_ptr; const int32_t* row_blk; const int32_t* row_col;
     int nnz, K, brows_per_head, n_heads, Z;
     long a_sz, a_sh, a_sm, b_sz, b_sh, b_sn;
+    int n_xcd;          // dies the dispatcher deals workgroup ids to (set where the kernel is launched)
 };
 
 constexpr int SDD_RING = 3;
@@ -122,7 +125,7 @@ __global__ __launch_bounds__(256) void bs_sdd32_kernel(const SddRowArgs a) {
     // one block-row per wave: the four waves of a workgroup walk neighbouring block-rows, whose
     // column lists mostly coincide, so their B-tile loads meet in the L1 cache
     int unit, grp;
-    if (!unit_of(blockIdx.x, (a.brows_per_head + 3) / 4, a.n_heads * a.Z, unit, grp)) return;
+    if (!unit_of(blockIdx.x, a.n_xcd, (a.brows_per_head + 3) / 4, a.n_heads * a.Z, unit, grp)) return;
     const int z = unit / a.n_heads, head = unit % a.n_heads, bi = grp * 4 + w;
     if (bi >= a.brows_per_head) return;
     const int brow = head * a.brows_per_head + bi;
@@ -221,6 +224,7 @@ struct SddUniArgs {
     void* dq; long dq_sz, dq_sh, dq_sm;
     // ... with delta formed here when `out` is given (delta may then be null): rowsum(a * out), out laid out like a
     const void* out; long o_sz, o_sh, o_sm;
+    int n_xcd;          // dies the dispatcher deals workgroup ids to (set where the kernel is launched)
 };
 
 template <typename T, int KS, int EPI = 0>     // KS = K / 32; EPI: 0 product, 1 softmax gradient, 2 probabilities
@@ -234,7 +238,7 @@ __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
     const int tid = threadIdx.x, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     int unit, grp;
-    if (!unit_of(blockIdx.x, a.grps_per_head, a.n_heads * a.Z, unit, grp)) return;
+    if (!unit_of(blockIdx.x, a.n_xcd, a.grps_per_head, a.n_heads * a.Z, unit, grp)) return;
     const int z = unit / a.n_heads, head = unit % a.n_heads;
     const int ug = head * a.grps_per_head + grp;
     const int p0 = a.uni_ptr[ug], n = a.uni_ptr[ug + 1] - p0;
@@ -597,6 +601,7 @@ struct DxdArgs {
     long dn_sz, dn_sh, dn_s0, dn_s1;    // DSD: (k, n) strides; DDS: (m, k) strides
     long c_sz, c_sh, c_sm, c_sn;
     int Z;
+    int n_xcd;          // dies the dispatcher deals workgroup ids to (set where the kernel is launched)
 };
 
 template <typename T, int BLK>
@@ -675,7 +680,7 @@ __global__ __launch_bounds__(256) void bs_dsd32_kernel(DxdArgs a) {
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
     const int ntn = (a.X + 63) / 64, n_heads = a.n_seg / a.per_head;
     int unit, pos;
-    if (!unit_of(blockIdx.x, a.per_head * ntn, n_heads * a.Z, unit, pos)) return;
+    if (!unit_of(blockIdx.x, a.n_xcd, a.per_head * ntn, n_heads * a.Z, unit, pos)) return;
     const int z = unit / n_heads, head = unit % n_heads, brow = pos / ntn, n0 = (pos % ntn) * 64;
     const int seg = head * a.per_head + brow;
     const T* spz = reinterpret_cast<const T*>(a.sp) + z * a.sp_sz;
@@ -760,6 +765,7 @@ struct DsdUniArgs {
     const int32_t* uni_ptr; const int32_t* uni_inner; const int32_t* uni_blk;
     int per_head, grps_per_head, n_heads, Z, N;
     long sp_sz, dn_sz, dn_sh, dn_sk, c_sz, c_sh, c_sm;
+    int n_xcd;          // dies the dispatcher deals workgroup ids to (set where the kernel is launched)
 };
 constexpr int DSDU_LD = 40;     // LDS row stride in elements ([column][k], 32 k + 8): 16 columns hit all banks once
 
@@ -772,7 +778,7 @@ __global__ __launch_bounds__(256) void bs_dsd32u_kernel(const DsdUniArgs a) {
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int ntn = (a.N + 63) / 64;
     int unit, pos;
-    if (!unit_of(blockIdx.x, a.grps_per_head * ntn, a.n_heads * a.Z, unit, pos)) return;
+    if (!unit_of(blockIdx.x, a.n_xcd, a.grps_per_head * ntn, a.n_heads * a.Z, unit, pos)) return;
     const int z = unit / a.n_heads, head = unit % a.n_heads, grp = pos / ntn, n0 = (pos % ntn) * 64;
     const int ug = head * a.grps_per_head + grp;
     const int p0 = a.uni_ptr[ug], n = a.uni_ptr[ug + 1] - p0;
@@ -956,6 +962,7 @@ struct DdsGroupArgs {
     const int32_t* grp_row0; const int32_t* grp_n;
     int per_head, M;
     long sp_sz, dn_sz, dn_sh, dn_sm, c_sz, c_sh, c_sm;
+    int n_xcd;          // dies the dispatcher deals workgroup ids to (set where the kernel is launched)
 };
 constexpr int DDS_MAX_STEPS = 128;   // longest reduction list the tiled kernel accepts
 
@@ -973,11 +980,11 @@ __global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
     const int wm = w >> 1, wn = w & 1;                      // this wave: tokens 64wm.., outputs 64wn..
     const int z = blockIdx.z;
-    // Workgroups go to the 8 XCDs (each with its own L2) round-robin in launch order.  The launch
+    // Workgroups go to the XCDs (each with its own L2) round-robin in launch order.  The launch
     // index is re-mapped so that the groups working on one stream of token tiles -- they read the same
-    // activations -- run on one XCD, one after the other: stream = 8 * (slot / groups) + XCD.
-    const int lin = blockIdx.x + gridDim.x * blockIdx.y, slot = lin >> 3;
-    const int grp = slot % (int)gridDim.x, ty = 8 * (slot / (int)gridDim.x) + (lin & 7), gy = gridDim.y;   // gridDim.y is a multiple of 8
+    // activations -- run on one XCD, one after the other: stream = n_xcd * (slot / groups) + XCD.
+    const int lin = blockIdx.x + gridDim.x * blockIdx.y, slot = lin / a.n_xcd;
+    const int grp = slot % (int)gridDim.x, ty = a.n_xcd * (slot / (int)gridDim.x) + lin % a.n_xcd, gy = gridDim.y;   // gridDim.y is a multiple of n_xcd
     // token tiles ty, ty + gy, ... : the group's tables are read once and the load -> LDS -> MFMA
     // pipeline runs on across tile boundaries
     const int tiles_all = (a.M + 127) / 128;
@@ -1162,6 +1169,7 @@ struct AttnArgs {
     long q_sz, q_sh, q_sm, k_sz, k_sh, k_sn, v_sz, v_sh, v_sn, o_sz, o_sh, o_sm;
     float scale;
     float* lse2;        // optional (Z, H, 32 * brows_per_head): base-2 log of every row's softmax denominator
+    int n_xcd;          // dies the dispatcher deals workgroup ids to (set where the kernel is launched)
 };
 
 // Maxima of scores.  A two-operand fmaxf costs three instructions here (each operand is first quieted
@@ -1197,7 +1205,7 @@ __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
     const int tid = threadIdx.x, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     int unit, grp;
-    if (!unit_of(blockIdx.x, a.grps_per_head, a.n_heads * a.Z, unit, grp)) return;
+    if (!unit_of(blockIdx.x, a.n_xcd, a.grps_per_head, a.n_heads * a.Z, unit, grp)) return;
     const int z = unit / a.n_heads, head = unit % a.n_heads;
     const int ug = head * a.grps_per_head + grp;
     const int p0 = a.uni_ptr[ug], n = a.uni_ptr[ug + 1] - p0;
@@ -1777,6 +1785,7 @@ extern "C" int flyhip_bs_sdd(const void* a, const void* b, void* c, const int32_
             SddUniArgs ua{a, b, c, uni_ptr, uni_inner, uni_blk, nnz, brows_per_head, gph, n_heads, Z,
                           a_sz, a_sh, a_sm, b_sz, b_sh, b_sn, nullptr, nullptr, 1.f};
             const long nwg = unit_grid((long)n_heads * Z, gph);
+            ua.n_xcd = machine().xcds;
             FLY_REQUIRE(nwg <= 2147483647L, "bs_sdd: too many workgroups");
             dim3 grid((unsigned)nwg);
 #define SDD32U_LAUNCH(T)                                                                         \
@@ -1792,6 +1801,7 @@ extern "C" int flyhip_bs_sdd(const void* a, const void* b, void* c, const int32_
         }
         SddRowArgs ra{a, b, c, row_ptr, row_blk, row_col, nnz, K, brows_per_head, n_heads, Z, a_sz, a_sh, a_sm, b_sz, b_sh, b_sn};
         const long nwg = unit_grid((long)n_heads * Z, (brows_per_head + 3) / 4);
+        ra.n_xcd = machine().xcds;
         FLY_REQUIRE(nwg <= 2147483647L, "bs_sdd: too many workgroups");
         dim3 grid((unsigned)nwg);
 #define SDD32_LAUNCH(T)                                                                         \
@@ -1847,6 +1857,7 @@ static int launch_sdd_epilogue(const char* what, const void* a_dn, const void* b
         ua.out = second->out; ua.o_sz = second->o_sz; ua.o_sh = second->o_sh; ua.o_sm = second->o_sm;
     }
     const long nwg = unit_grid((long)n_heads * Z, gph);
+    ua.n_xcd = machine().xcds;
     FLY_REQUIRE(nwg <= 2147483647L, "%s: too many workgroups", what);
     dim3 grid((unsigned)nwg);
 #define SDDS_LAUNCH(T)                                                                                  \
@@ -1956,6 +1967,7 @@ extern "C" int flyhip_bs_dsd(const void* a_sp, const void* b, void* c,
             DsdUniArgs ua{a_sp, b, c, uni_ptr, uni_inner, uni_blk, rows_per_head, gph, n_heads, Z, N,
                           a_sz, b_sz, b_sh, b_sk, c_sz, c_sh, c_sm};
             const long nwg = unit_grid((long)n_heads * Z, (long)gph * ((N + 63) / 64));
+            ua.n_xcd = machine().xcds;
             FLY_REQUIRE(nwg <= 2147483647L, "bs_dsd: too many workgroups");
             dim3 grid((unsigned)nwg);
             if (dtype == BF16) {
@@ -1968,6 +1980,7 @@ extern "C" int flyhip_bs_dsd(const void* a_sp, const void* b, void* c,
             return check_launch("bs_dsd32u_kernel");
         }
         const long nwg = unit_grid((long)(n_seg / rows_per_head) * Z, (long)rows_per_head * ((N + 63) / 64));
+        args.n_xcd = machine().xcds;
         FLY_REQUIRE(nwg <= 2147483647L, "bs_dsd: too many workgroups");
         dim3 grid((unsigned)nwg);
         if (dtype == BF16) hipLaunchKernelGGL((bs_dsd32_kernel<bf16_t>), grid, dim3(256), 0, st, args);
@@ -2006,9 +2019,11 @@ extern "C" int flyhip_bs_dds(const void* a, const void* b_sp, void* c,
                         b_sz, a_sz, a_sh, a_sm, c_sz, c_sh, c_sm};
         // as many workgroups as are resident together (three fit a CU); each walks its share of the token tiles
         const long tiles = (M + 127) / 128;
-        long gy = (3L * 256 + (long)n_grp * Z - 1) / ((long)n_grp * Z);
+        const Machine& mach = machine();
+        ga.n_xcd = mach.xcds;
+        long gy = (3L * mach.cus + (long)n_grp * Z - 1) / ((long)n_grp * Z);
         if (gy > tiles) gy = tiles;
-        gy = (gy + 7) / 8 * 8;                               // the kernel deals streams of token tiles to the 8 XCDs
+        gy = (gy + mach.xcds - 1) / mach.xcds * mach.xcds;   // the kernel deals streams of token tiles to the XCDs
         dim3 grid(n_grp, (unsigned)gy, Z);
         if (dtype == BF16) {
             if (trans_b) hipLaunchKernelGGL((bs_dds32_kernel<bf16_t, false>), grid, dim3(256), 0, st, ga);
@@ -2074,6 +2089,7 @@ extern "C" int flyhip_bs_attn_lse(const void* q, const void* k, const void* v, v
     AttnArgs args{q, k, v, out, uni_ptr, uni_inner, uni_blk, key_mask, key_mask_stride, brows_per_head, gph, H, Z,
                   q_sz, q_sh, q_sm, k_sz, k_sh, k_sn, v_sz, v_sh, v_sn, o_sz, o_sh, o_sm, scale, lse2};
     const long nwg = unit_grid((long)H * Z, gph);
+    args.n_xcd = machine().xcds;
     FLY_REQUIRE(nwg <= 2147483647L, "bs_attn: too many workgroups");
     dim3 grid((unsigned)nwg);
     const bool masked = key_mask != nullptr || !(scale > 0.f);

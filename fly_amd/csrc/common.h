@@ -5,6 +5,7 @@
 #include <stdint.h>
 #include <stdio.h>
 #include <stdarg.h>
+#include <atomic>
 
 namespace flyhip {
 
@@ -26,6 +27,19 @@ inline int check_launch(const char* what) {
     return OK;
 }
 #define FLY_REQUIRE(cond, ...) do { if (!(cond)) return ::flyhip::fail(::flyhip::ERR_ARG, __VA_ARGS__); } while (0)
+
+// ---------------------------------------------------------------------------------------
+// facts of the device the calling thread has current, queried from the runtime once per device
+// ---------------------------------------------------------------------------------------
+struct Machine {
+    int cus;       // compute units
+    int xcds;      // accelerator dies, each with its own L2; the dispatcher deals consecutive workgroup ids to them in turn
+    int slots;     // workgroups of 256 threads that are resident together at two per compute unit
+};
+const Machine& machine();      // (without a device: the MI355X's 256 compute units on 8 dies)
+// hipFuncSetAttribute(MaxDynamicSharedMemorySize) once per kernel and device; `done` is the caller's
+// per-kernel set of devices already served (one bit each)
+int ensure_dynamic_lds(const void* kernel, size_t bytes, std::atomic<unsigned long long>& done, const char* what);
 
 enum DType { F32 = 0, BF16 = 1, F16 = 2 };
 

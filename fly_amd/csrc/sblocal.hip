@@ -33,7 +33,6 @@ constexpr int CH = 64;     // keys per feature chunk (granularity of the key-sid
 constexpr int TK = 32;     // keys per tile of the fused band kernel
 constexpr int TQ = 64;     // queries per workgroup of the fused band kernel
 constexpr int NT = 256;    // threads per workgroup (4 waves)
-constexpr int N_XCD = 8;   // accelerator dies (each with its own L2) the dispatcher cycles over
 constexpr int NSTAT = 5;   // per-query statistics of a partial: m, ze, zp, qk1, lsq+kmax
 
 // Optional phase timestamps of the fused kernel (a development build, -DFLY_PROFILE, reads them
@@ -99,6 +98,7 @@ struct FwdArgs {
     // the query features themselves (part 0 leaves them in qfeat), take kmax from the combined reductions, and
     // index partials / query features by batch * n_heavy + entry.
     const int32_t* tl_heavy; int n_heavy;
+    int n_xcd;                      // dies the dispatcher deals workgroup ids to (set at launch)
 };
 
 // ROWS x W tile of a (seq, W) matrix, moved global -> registers -> LDS in two steps so that all of
@@ -1180,8 +1180,8 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
     }
     const int n_qt = (a.T + TQ - 1) / TQ;
     const int n_items = a.B * a.H * n_qt * a.n_parts;
-    const int per_xcd = (n_items + N_XCD - 1) / N_XCD;
-    const int item = (blockIdx.x % N_XCD) * per_xcd + blockIdx.x / N_XCD;   // see sblocal_fwd_kernel
+    const int per_xcd = (n_items + a.n_xcd - 1) / a.n_xcd;
+    const int item = (blockIdx.x % a.n_xcd) * per_xcd + blockIdx.x / a.n_xcd;   // see sblocal_fwd_kernel
     if (item >= n_items) return;                       // workgroup-uniform
     const int part = item % a.n_parts;
     const int qt = (item / a.n_parts) % n_qt;
@@ -1840,6 +1840,7 @@ struct LocalArgs {
     long q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss;
     float temp;
     float* lse;                     // optional (B, H, T): log of the softmax denominator, for the backward pass
+    int n_xcd;                      // dies the dispatcher deals workgroup ids to (set at launch)
 };
 
 template <typename T, int E, int D>
@@ -1851,8 +1852,8 @@ __global__ __launch_bounds__(NT) void local_fwd_kernel(LocalArgs a) {
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
     const int n_qt = (a.T + TQ - 1) / TQ;
     const int n_items = a.B * a.H * n_qt;
-    const int per_xcd = (n_items + N_XCD - 1) / N_XCD;
-    const int item = (blockIdx.x % N_XCD) * per_xcd + blockIdx.x / N_XCD;   // see sblocal_fwd_kernel
+    const int per_xcd = (n_items + a.n_xcd - 1) / a.n_xcd;
+    const int item = (blockIdx.x % a.n_xcd) * per_xcd + blockIdx.x / a.n_xcd;   // see sblocal_fwd_kernel
     if (item >= n_items) return;                       // workgroup-uniform
     const int qt = item % n_qt, bh = item / n_qt, b = bh / a.H, h = bh % a.H;
     const int q0 = qt * TQ, iq = q0 + 16 * w + r16;
@@ -2000,7 +2001,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
     // block-sparse support the first workgroups of the launch, which walk the long lists in parts
     bool part_role = SPLIT;
     long slot = 0;                  // long lists: index of the tile's partials and compact query features
-    const int n_part_wgs = LIST ? (a.B * a.n_heavy * a.n_parts + N_XCD - 1) / N_XCD * N_XCD : 0;
+    const int n_part_wgs = LIST ? (a.B * a.n_heavy * a.n_parts + a.n_xcd - 1) / a.n_xcd * a.n_xcd : 0;
     if (LIST && (int)blockIdx.x < n_part_wgs) {
         const int idx = blockIdx.x;
         if (idx >= a.B * a.n_heavy * a.n_parts) return;            // workgroup-uniform
@@ -2015,18 +2016,18 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
         // the tiles start longest first: an XCD takes the (batch, head) pairs congruent to its number and
         // walks them rank by rank -- all their longest tiles, then all their second longest ...
         const int blk_id = blockIdx.x - n_part_wgs;
-        const int nbh = a.B * a.H, x = blk_id % N_XCD, i = blk_id / N_XCD;
-        const int mine = (nbh - x + N_XCD - 1) / N_XCD;            // pairs of this XCD
+        const int nbh = a.B * a.H, x = blk_id % a.n_xcd, i = blk_id / a.n_xcd;
+        const int mine = (nbh - x + a.n_xcd - 1) / a.n_xcd;            // pairs of this XCD
         if (mine <= 0 || i >= mine * n_qt) return;                 // workgroup-uniform
         const int rank = i / mine;
-        bh = x + N_XCD * (i % mine);
+        bh = x + a.n_xcd * (i % mine);
         qt = a.tl_order ? a.tl_order[(bh % a.H) * n_qt + rank] : rank;
         if (qt < 0) return;                                        // a long list: walked in parts by the first workgroups
         part = 0;
     } else {
         const int n_items = a.B * a.H * n_qt * a.n_parts;
-        const int per_xcd = (n_items + N_XCD - 1) / N_XCD;
-        const int item = (blockIdx.x % N_XCD) * per_xcd + blockIdx.x / N_XCD;
+        const int per_xcd = (n_items + a.n_xcd - 1) / a.n_xcd;
+        const int item = (blockIdx.x % a.n_xcd) * per_xcd + blockIdx.x / a.n_xcd;
         if (item >= n_items) return;                       // workgroup-uniform
         part = item % a.n_parts;
         qt = (item / a.n_parts) % n_qt;
@@ -2412,16 +2413,14 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
     if (SPLIT && (int)blockIdx.x >= a.band_wgs) {       // combine role, see sblocal_fwd_kernel
         const int ci = blockIdx.x - a.band_wgs;
         FLY_PROF(0);
-#ifndef FLY_EXP_NOCOMBINE
         sb_combine_body(smem, a.kv_part, a.part_max, const_cast<float*>(a.kv), const_cast<float*>(a.ksum),
                         const_cast<float*>(a.kmax), nullptr, ci / a.cmb_wpb, ci % a.cmb_wpb, a.cmb_wpb, a.n_split, M, D);
-#endif
         FLY_PROF(7);
         return;
     }
     const int n_items = a.B * a.H * n_qt * a.n_parts;
-    const int per_xcd = (n_items + N_XCD - 1) / N_XCD;
-    const int item = (blockIdx.x % N_XCD) * per_xcd + blockIdx.x / N_XCD;   // see sblocal_fwd_kernel
+    const int per_xcd = (n_items + a.n_xcd - 1) / a.n_xcd;
+    const int item = (blockIdx.x % a.n_xcd) * per_xcd + blockIdx.x / a.n_xcd;   // see sblocal_fwd_kernel
     if (item >= n_items) return;                       // workgroup-uniform
     const int part = item % a.n_parts;
     const int qt = (item / a.n_parts) % n_qt;
@@ -2576,9 +2575,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
         const bool more = kt + 1 < kt_hi;
         float cscale_next = cscale;
         if (more) {                                      // next tile's loads fly during the MFMAs
-#ifndef FLY_EXP_NOFETCH
             fetch(kt + 1);
-#endif
             cscale_next = csp[(s_base + TK) / CH];
         }
         const float wc = __builtin_amdgcn_exp2f((cscale - kmax) * LOG2E);
@@ -2599,7 +2596,6 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
                     s1[kb] = mma_bf16(khi, qh[ks], s1[kb]);
                 }
             // overlap: all four piece products (exact product of the rounded features)
-#ifndef FLY_EXP_NOS2
 #pragma unroll
             for (int ks = 0; ks < FS; ++ks)
 #pragma unroll
@@ -2611,7 +2607,6 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
                     s2[kb] = mma_bf16(fhi, qfl[ks], s2[kb]);
                     s2[kb] = mma_bf16(fhi, qfh[ks], s2[kb]);
                 }
-#endif
             const bool interior = s_base - (qw0 + 15) >= -lc_lo && s_base + TK - 1 - qw0 < lc_hi &&
                                   s_base + TK <= len && qw0 + 15 < a.T;
             floatx4 p[KB];
@@ -2649,20 +2644,11 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
                         p[kb][i] = e - ov * beta;
                     }
             };
-#ifdef FLY_EXP_NOSOFT
-            p[0] = s1[0] + s2[0]; p[1] = s1[1] + s2[1];
-#else
             if (interior) soft(std::false_type{}); else soft(std::true_type{});
-#endif
             zp += ovs * wc;
             // O^T[d][query] += sum_keys V[key][d] p[key][query]: P exactly in three pieces, six products
             uintx4 ph, pm, pl;
-#ifdef FLY_EXP_NOSPLIT
-            ph = pm = pl = uintx4{__float_as_uint(p[0][0]), __float_as_uint(p[0][1]), __float_as_uint(p[1][0]), __float_as_uint(p[1][1])};
-#else
             split3(p[0], p[1], ph, pm, pl);
-#endif
-#ifndef FLY_EXP_NOPV
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
                 const uintx4 vh = *reinterpret_cast<const uintx4*>(st + voff + 16 * db * TL::V_ROW);
@@ -2677,17 +2663,10 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
                 o = mma_bf16(vh, ph, o);
                 oacc[db] = o;
             }
-#else
-            oacc[0] += __builtin_bit_cast(floatx4, ph) + __builtin_bit_cast(floatx4, pm) + __builtin_bit_cast(floatx4, pl);
-#endif
         }
-#ifndef FLY_EXP_NOFETCH
         if (more) stash(cur ^ 1);
-#endif
         cscale = cscale_next;
-#ifndef FLY_EXP_NOBARRIER
         __syncthreads();
-#endif
     }
 
     FLY_PROF(3);
@@ -2954,7 +2933,7 @@ __global__ __launch_bounds__(NT) void sb_merge_x_kernel(FwdArgs a, int xcd_items
     __shared__ __attribute__((aligned(16))) float KVs[M * LDV];
     __shared__ __attribute__((aligned(16))) float KSs[M];
     const int n_qt = (a.T + TQ - 1) / TQ, n_tiles = a.B * a.H * n_qt;
-    const int x = blockIdx.x % N_XCD, i = blockIdx.x / N_XCD, slice = i % NSL, j = i / NSL;
+    const int x = blockIdx.x % a.n_xcd, i = blockIdx.x / a.n_xcd, slice = i % NSL, j = i / NSL;
     // tiles whose first part is one of XCD x's band items
     const int t_lo = (x * xcd_items + a.n_parts - 1) / a.n_parts;
     const int t_hi = min(((x + 1) * xcd_items + a.n_parts - 1) / a.n_parts, n_tiles);
@@ -2993,25 +2972,15 @@ static int launch_kfeat_x3(const KvArgs& a, hipStream_t st) {
         auto kern = sb_kfeat_x3_kernel<E, E, M>;
         constexpr size_t smem = kfeat_x3_smem<E, M>();
         static_assert(smem <= 160 * 1024, "two tile images, the V chunk and the projection image must fit the LDS");
-        static bool lds_ready = false;
-        if (!lds_ready) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-            if (e != hipSuccess) return fail(ERR_LAUNCH, "sb_kfeat_x3: LDS attribute: %s", hipGetErrorString(e));
-            lds_ready = true;
-        }
+        static std::atomic<unsigned long long> lds_set{0};     // (devices on which this kernel has its LDS limit)
+        if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_set, "sb_kfeat_x3")) return rc;
         hipLaunchKernelGGL(kern, dim3(a.n_split + a.q_tiles, a.B * a.H), dim3(NT), smem, st, a);
         return check_launch("sb_kfeat_x3_kernel");
     }
     auto kern = sb_kfeat_kernel<float, E, E, M, true>;
     constexpr size_t smem = kfeat_smem<E, M>();
-    static bool lds_ready = false;
-    if (!lds_ready) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        if (e != hipSuccess) return fail(ERR_LAUNCH, "sb_kfeat (piece images): LDS attribute: %s", hipGetErrorString(e));
-        lds_ready = true;
-    }
+    static std::atomic<unsigned long long> lds_set{0};     // (devices on which this kernel has its LDS limit)
+    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_set, "sb_kfeat (piece images)")) return rc;
     hipLaunchKernelGGL(kern, dim3(a.n_split + a.q_tiles, a.B * a.H), dim3(NT), smem, st, a);
     return check_launch("sb_kfeat_kernel (piece images)");
 }
@@ -3021,26 +2990,16 @@ static int launch_kfeat(const KvArgs& a, hipStream_t st) {
     if (sizeof(T) == 2 && !a.q) {            // bfloat16 keys, no query role: both products on the bf16 MFMA
         auto kern16 = sb_kfeat_bf16_kernel<E, E, M>;
         constexpr size_t smem16 = kfeat_bf16_smem<E, M>();
-        static bool lds16_ready = false;
-        if (!lds16_ready) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern16),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem16);
-            if (e != hipSuccess) return fail(ERR_LAUNCH, "sb_kfeat_bf16: LDS attribute: %s", hipGetErrorString(e));
-            lds16_ready = true;
-        }
+        static std::atomic<unsigned long long> lds_set{0};     // (devices on which this kernel has its LDS limit)
+        if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern16), smem16, lds_set, "sb_kfeat_bf16")) return rc;
         hipLaunchKernelGGL(kern16, dim3(a.n_split, a.B * a.H), dim3(NT), smem16, st, a);
         return check_launch("sb_kfeat_bf16_kernel");
     }
     if (sizeof(T) == 4 && a.vt) return launch_kfeat_x3<E, M>(a, st);      // float inputs, piece images asked for
     auto kern = sb_kfeat_kernel<T, E, E, M>;
     constexpr size_t smem = kfeat_smem<E, M>();
-    static bool lds_ready = false;     // one instantiation = one kernel; set its LDS limit once
-    if (!lds_ready) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        if (e != hipSuccess) return fail(ERR_LAUNCH, "sb_kfeat: LDS attribute: %s", hipGetErrorString(e));
-        lds_ready = true;
-    }
+    static std::atomic<unsigned long long> lds_set{0};     // (devices on which this kernel has its LDS limit)
+    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_set, "sb_kfeat")) return rc;
     // per (batch, head): key-role workgroups, then query-role ones
     hipLaunchKernelGGL(kern, dim3(a.n_split + a.q_tiles, a.B * a.H), dim3(NT), smem, st, a);
     return check_launch("sb_kfeat_kernel");
@@ -3071,22 +3030,19 @@ static int launch_fwd_impl(const FwdArgs& a, hipStream_t st) {
     const size_t smem = K::smem + (sizeof(T) == 2 ? (size_t)(band_keys / CH + 2) * sizeof(float) : 0);
     constexpr size_t LDS_MAX = 160 * 1024;
     if (smem > LDS_MAX) return fail(ERR_ARG, "sblocal_fwd: local_context %d needs %zu bytes of LDS (limit %zu)", a.lc, smem, LDS_MAX);
-    static bool lds_ready = false;
-    if (!lds_ready) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_MAX);
-        if (e != hipSuccess) return fail(ERR_LAUNCH, "sblocal_fwd: LDS attribute: %s", hipGetErrorString(e));
-        lds_ready = true;
-    }
+    static std::atomic<unsigned long long> lds_set{0};     // (devices on which this kernel has its LDS limit)
+    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), LDS_MAX, lds_set, "sblocal_fwd")) return rc;
+    const Machine& mach = machine();
     const int qt = (a.T + TQ - 1) / TQ;                           // 64-query tiles (partials, merge)
     const long items = (long)a.B * a.H * ((a.T + K::tq - 1) / K::tq) * a.n_parts;
-    long grid = (items + N_XCD - 1) / N_XCD * N_XCD;             // whole rounds over the XCDs
+    long grid = (items + mach.xcds - 1) / mach.xcds * mach.xcds;             // whole rounds over the XCDs
     FwdArgs args = a;
+    args.n_xcd = mach.xcds;
     args.band_wgs = (int)grid;
     if (SPLIT) {
         // combine role: as many workgroups per (batch, head) as fit beside the band workgroups in one
         // residency round (two workgroups of this kernel per CU), at least one, at most one thread per output
-        const long bhn = (long)a.B * a.H, free_slots = 512 - grid;
+        const long bhn = (long)a.B * a.H, free_slots = mach.slots - grid;
         long wpb = free_slots / bhn;
         const long most = (M * (E + 1) / 4 + K::threads - 1) / K::threads;   // one 16-byte piece of the result per thread
         if (wpb > most) wpb = most;
@@ -3119,20 +3075,17 @@ static int launch_fwd_x3(const FwdArgs& a, hipStream_t st) {
     auto kern = sblocal_fwd_x3_kernel<E, E, M, SPLIT>;
     constexpr size_t smem = fwd_x3_smem<E, M>();
     static_assert(smem <= 160 * 1024, "two tile stages must fit the LDS");
-    static bool lds_ready = false;
-    if (!lds_ready) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        if (e != hipSuccess) return fail(ERR_LAUNCH, "sblocal_fwd (bf16 pieces): LDS attribute: %s", hipGetErrorString(e));
-        lds_ready = true;
-    }
+    static std::atomic<unsigned long long> lds_set{0};     // (devices on which this kernel has its LDS limit)
+    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_set, "sblocal_fwd (bf16 pieces)")) return rc;
+    const Machine& mach = machine();
     const int qt = (a.T + TQ - 1) / TQ;
     const long items = (long)a.B * a.H * qt * a.n_parts;
-    long grid = (items + N_XCD - 1) / N_XCD * N_XCD;
+    long grid = (items + mach.xcds - 1) / mach.xcds * mach.xcds;
     FwdArgs args = a;
+    args.n_xcd = mach.xcds;
     args.band_wgs = (int)grid;
     if (SPLIT) {
-        const long bhn = (long)a.B * a.H, free_slots = 512 - grid;
+        const long bhn = (long)a.B * a.H, free_slots = mach.slots - grid;
         long wpb = free_slots / bhn;
         const long most = (M * (E + 1) / 4 + NT - 1) / NT;      // one 16-byte piece of the result per thread
         if (wpb > most) wpb = most;
@@ -3148,9 +3101,9 @@ static int launch_fwd_x3(const FwdArgs& a, hipStream_t st) {
     int rc = check_launch("sblocal_fwd_x3_kernel");
     if (rc || !SPLIT) return rc;
     constexpr int NDB = MERGE_NDB < E / 16 ? MERGE_NDB : E / 16;
-    const int xcd_items = (int)((items + N_XCD - 1) / N_XCD);
+    const int xcd_items = (int)((items + mach.xcds - 1) / mach.xcds);
     const int tiles_per_xcd = (xcd_items + a.n_parts - 1) / a.n_parts + 1;
-    hipLaunchKernelGGL((sb_merge_x_kernel<E, M, NDB>), dim3((unsigned)(N_XCD * tiles_per_xcd * (E / 16 / NDB))), dim3(NT), 0, st,
+    hipLaunchKernelGGL((sb_merge_x_kernel<E, M, NDB>), dim3((unsigned)(mach.xcds * tiles_per_xcd * (E / 16 / NDB))), dim3(NT), 0, st,
                        args, xcd_items, tiles_per_xcd);
     return check_launch("sb_merge_x_kernel");
 }
@@ -3166,21 +3119,18 @@ template <typename T, int E, int M>
 static int launch_fwd_list(const FwdArgs& a, hipStream_t st) {
     auto kern = sblocal_fwd_kernel<float, E, E, M, false, true>;
     constexpr size_t smem = fwd_smem<E, M>();
-    static bool lds_ready = false;
-    if (!lds_ready) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        if (e != hipSuccess) return fail(ERR_LAUNCH, "sbblocksparse_fwd: LDS attribute: %s", hipGetErrorString(e));
-        lds_ready = true;
-    }
-    // every XCD gets room for ceil(B H / 8) (batch, head) pairs
-    const long grid = (((long)a.B * a.H + N_XCD - 1) / N_XCD) * ((a.T + TQ - 1) / TQ) * N_XCD;
+    static std::atomic<unsigned long long> lds_set{0};     // (devices on which this kernel has its LDS limit)
+    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_set, "sbblocksparse_fwd")) return rc;
+    // every XCD gets room for ceil(B H / dies) (batch, head) pairs
+    const Machine& mach = machine();
+    const long grid = (((long)a.B * a.H + mach.xcds - 1) / mach.xcds) * ((a.T + TQ - 1) / TQ) * mach.xcds;
     if (grid > 2147483647L) return fail(ERR_ARG, "sbblocksparse_fwd: too many workgroups");
     // long lists: the first workgroups of the launch walk them in parts (they are the longest pieces of work)
     const long tiles = (long)a.B * a.n_heavy;
-    const long part_wgs = (tiles * a.n_parts + N_XCD - 1) / N_XCD * N_XCD;
+    const long part_wgs = (tiles * a.n_parts + mach.xcds - 1) / mach.xcds * mach.xcds;
     if (grid + part_wgs > 2147483647L) return fail(ERR_ARG, "sbblocksparse_fwd: too many workgroups");
     FwdArgs args = a;
+    args.n_xcd = mach.xcds;
     args.band_wgs = (int)(grid + part_wgs);
     hipLaunchKernelGGL(kern, dim3((unsigned)(grid + part_wgs)), dim3(NT), smem, st, args);
     int rc = check_launch("sblocal_fwd_kernel (block-sparse support)");
@@ -3193,17 +3143,15 @@ template <typename T, int E>
 static int launch_local(const LocalArgs& a, hipStream_t st) {
     auto kern = local_fwd_kernel<T, E, E>;
     constexpr size_t smem = sizeof(float) * 2 * TK * 2 * (E + 4);
-    static bool lds_ready = false;
-    if (!lds_ready) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        if (e != hipSuccess) return fail(ERR_LAUNCH, "local_fwd: LDS attribute: %s", hipGetErrorString(e));
-        lds_ready = true;
-    }
+    static std::atomic<unsigned long long> lds_set{0};     // (devices on which this kernel has its LDS limit)
+    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_set, "local_fwd")) return rc;
+    const Machine& mach = machine();
     const long items = (long)a.B * a.H * ((a.T + TQ - 1) / TQ);
-    const long grid = (items + N_XCD - 1) / N_XCD * N_XCD;
+    const long grid = (items + mach.xcds - 1) / mach.xcds * mach.xcds;
     if (grid > 2147483647L) return fail(ERR_ARG, "local_fwd: too many workgroups");
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NT), smem, st, a);
+    LocalArgs args = a;
+    args.n_xcd = mach.xcds;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NT), smem, st, args);
     return check_launch("local_fwd_kernel");
 }
 
@@ -3235,6 +3183,7 @@ struct BwdArgs {
     float temp;
     // finishing pass: global low-rank terms and the chain rule through the feature map in the epilogue
     const float* gmat; const float* gvec; const float* proj;
+    int n_xcd;                      // dies the dispatcher deals workgroup ids to (set at launch)
 };
 
 //
@@ -3258,8 +3207,8 @@ __global__ __launch_bounds__(NT) void sblocal_bwd_band_kernel(BwdArgs a) {
     const int Lo = KEYMAJOR ? a.S : a.T, Li = KEYMAJOR ? a.T : a.S;
     const int n_ot = (Lo + TQ - 1) / TQ;
     const int n_items = a.BH * n_ot;
-    const int per_xcd = (n_items + N_XCD - 1) / N_XCD;
-    const int item = (blockIdx.x % N_XCD) * per_xcd + blockIdx.x / N_XCD;   // see sblocal_fwd_kernel
+    const int per_xcd = (n_items + a.n_xcd - 1) / a.n_xcd;
+    const int item = (blockIdx.x % a.n_xcd) * per_xcd + blockIdx.x / a.n_xcd;   // see sblocal_fwd_kernel
     if (item >= n_items) return;                       // workgroup-uniform
     const int ot = item % n_ot, bh = item / n_ot, b = bh / a.H;
     const int o0 = ot * TQ, ow0 = o0 + 16 * w, o = ow0 + r16;
@@ -3519,17 +3468,15 @@ template <int E, int M, bool KEYMAJOR, bool FINISH>
 static int launch_bwd_band(const BwdArgs& a, hipStream_t st) {
     auto kern = sblocal_bwd_band_kernel<E, M, KEYMAJOR, FINISH>;
     constexpr size_t smem = sizeof(float) * 2 * (TK * (3 * 4 + 2 * E + M) + 2 * TK);
-    static bool lds_ready = false;
-    if (!lds_ready) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        if (e != hipSuccess) return fail(ERR_LAUNCH, "sblocal_bwd_band: LDS attribute: %s", hipGetErrorString(e));
-        lds_ready = true;
-    }
+    static std::atomic<unsigned long long> lds_set{0};     // (devices on which this kernel has its LDS limit)
+    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_set, "sblocal_bwd_band")) return rc;
+    const Machine& mach = machine();
     const long items = (long)a.BH * (((KEYMAJOR ? a.S : a.T) + TQ - 1) / TQ);
-    const long grid = (items + N_XCD - 1) / N_XCD * N_XCD;
+    const long grid = (items + mach.xcds - 1) / mach.xcds * mach.xcds;
     if (grid > 2147483647L) return fail(ERR_ARG, "sblocal_bwd_band: too many workgroups");
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NT), smem, st, a);
+    BwdArgs args = a;
+    args.n_xcd = mach.xcds;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NT), smem, st, args);
     return check_launch("sblocal_bwd_band_kernel");
 }
 
@@ -3574,7 +3521,7 @@ static int plan_parts(int B, int H, int T, int S, int lc) {
     long band = (long)lc + TQ;
     if (band > S) band = S;
     const int key_tiles = (int)((band + TK - 1) / TK);
-    long want = 512 / tiles;                             // never more than two workgroups per CU
+    long want = machine().slots / tiles;                 // never more than two workgroups per CU
     if (want > 8) want = 8;
     if (want > key_tiles / 2) want = key_tiles / 2;      // at least two key tiles per part
     return want < 1 ? 1 : (int)want;
@@ -3582,19 +3529,20 @@ static int plan_parts(int B, int H, int T, int S, int lc) {
 
 static int plan(int B, int H, int S, int* n_chunks, int* n_split) {
     const int nc = (S + CH - 1) / CH;
-    // aim for about 1024 workgroups over the chip, at least one chunk each
-    long want = (1024 + (long)B * H - 1) / ((long)B * H);
+    // aim for about four workgroups per CU over the chip, at least one chunk each
+    const long slots = machine().slots;
+    long want = (2 * slots + (long)B * H - 1) / ((long)B * H);
     if (want < 1) want = 1;
     if (want > nc) want = nc;
     int per = (nc + (int)want - 1) / (int)want;
-    if ((long)B * H * nc > 512) {
+    if ((long)B * H * nc > slots) {
         // more work than one residency round (two workgroups per CU): the pass takes about
         // rounds x chunks per workgroup, and a round that is full costs no more than one that is not; among
         // equals the larger share wins (fewer partial reductions to combine)
         long best = -1;
         for (int p = 1; p <= nc; ++p) {
             const long wgs = (long)B * H * ((nc + p - 1) / p);
-            const long cost = ((wgs + 511) / 512) * p;
+            const long cost = ((wgs + slots - 1) / slots) * p;
             if (best < 0 || cost <= best) { best = cost; per = p; }
         }
     }
