@@ -57,9 +57,15 @@ int flyhip_sb_plan(int B, int H, int T, int S, int local_context,
  * -t|q|^2/2 + rowmax - log(m)/2.  With q given, kv / ksum / kmax are NOT written: the partial
  * reductions (kv_part, part_max) are combined inside flyhip_sblocal_fwd's launch instead, which
  * saves a launch on problems this small.
- * bfloat16 inputs only (NULL otherwise): vt (B,H,n_chunks*64,D) bf16 and kvt (B,H,D,m) bf16, opaque
- * scratch for flyhip_sblocal_fwd -- V per 32-key tile and K'^T V, transposed into the operand
- * order of the bf16 MFMA. */
+ * bfloat16 inputs: vt (B,H,n_chunks*64,D) bf16 and kvt (B,H,D,m) bf16, opaque scratch for
+ * flyhip_sblocal_fwd -- V per 32-key tile and K'^T V, transposed into the operand order of the bf16
+ * MFMA.
+ * float inputs: vt may be NULL (all products on the fp32 matrix pipe, kfeat holds fp32 features).
+ * With vt given -- B*H*n_chunks*2*(128*E + 192*D) bytes, 16-byte aligned -- the key pass writes
+ * per 32-key tile an image of K and V^T split into bfloat16 pieces there, and into kfeat (same
+ * byte size as the fp32 features) an image of the features split into two pieces; passing the same
+ * vt to flyhip_sblocal_fwd then runs the band on the bf16 matrix pipe with fp32-level accuracy
+ * (features are rounded to 16 significant bits where they are formed).  kvt is unused for float. */
 int flyhip_sb_kv_reduce(const void* k, const void* v, const float* proj, const int64_t* key_lengths,
                         void* kfeat, float* chunk_scale, float* kv_part, float* part_max,
                         float* kv, float* ksum, float* kmax,
@@ -78,7 +84,8 @@ int flyhip_sb_kv_reduce(const void* k, const void* v, const float* proj, const i
  *   n_parts from flyhip_sb_plan (any value in [1,64] is valid); when > 1, part_ws is scratch of
  *   B*H*ceil(T/64)*n_parts*64*(D+5) floats and qfeat / q_lsq are the query-side outputs of
  *   flyhip_sb_kv_reduce for the same q; with n_parts == 1 all three may be NULL (the kernel forms
- *   the query features itself).  vt / kvt: the bf16 scratch of flyhip_sb_kv_reduce (NULL for fp32).
+ *   the query features itself).  vt / kvt: the scratch of flyhip_sb_kv_reduce (float inputs: vt as
+ *   it was passed there, NULL or the piece images; kvt NULL).
  *   With n_parts > 1 the key pass has left its partial reductions uncombined: pass its kv_part,
  *   part_max and n_split; extra workgroups of the band kernel's launch combine them into kv / ksum /
  *   kmax (written here, read by the merge kernel that finishes the tiles).  With n_parts == 1 they
