@@ -378,8 +378,8 @@ def bench_other_configs():
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
-    ap.add_argument('--steps', type=int, default=200)
-    ap.add_argument('--warmup', type=int, default=20)
+    ap.add_argument('--steps', type=int, default=2000)
+    ap.add_argument('--warmup', type=int, default=50)
     ap.add_argument('--no-blocksparse', action='store_true', help='skip the config 2 stages')
     ap.add_argument('--no-other-configs', action='store_true', help='skip the timings of configs 3, 4, 5')
     ap.add_argument('--skip-cpu', action='store_true', help='skip the CPU baseline leg (profiling runs)')
@@ -415,7 +415,7 @@ def main():
     }
     extra = {}
     if not args.no_blocksparse:
-        extra['blocksparse_config2'] = bench_blocksparse(max(5, args.steps // 10), 3)
+        extra['blocksparse_config2'] = bench_blocksparse(min(20, max(5, args.steps // 10)), 3)
     if not args.no_other_configs:
         extra.update(bench_other_configs())
     if extra:

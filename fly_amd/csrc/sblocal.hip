@@ -2584,29 +2584,78 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
             floatx4 s1[KB], s2[KB];
 #pragma unroll
             for (int kb = 0; kb < KB; ++kb) { s1[kb] = Frag<float>::zero(); s2[kb] = Frag<float>::zero(); }
+            // LDS fragments are requested a phase ahead of the MFMAs that use them (the scheduling barriers keep the
+            // requests where they are written): K and the first half of K' before the scores, the second half
+            // of K' before the first half of the overlap, V^T before the second half and the softmax arithmetic
+            // (small problems, where a workgroup's few tiles are a chain of latencies; with one part per tile the registers
+            // this takes would cost the second workgroup of a compute unit, and fragments are requested where they are used)
+            constexpr bool AHEAD = SPLIT;
+            constexpr int FA = (FS + 1) / 2, DA = (DB + 1) / 2;
+            uintx4 kf[KS][KB][2], ff[FS][KB][2], vf[DB][3];
+            auto load_f = [&](int ks) __attribute__((always_inline)) {
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb) {
+                    ff[ks][kb][0] = *reinterpret_cast<const uintx4*>(st + foff[ks] + 16 * kb * TL::F_ROW);
+                    ff[ks][kb][1] = *reinterpret_cast<const uintx4*>(st + foff[ks] + 16 * kb * TL::F_ROW + TL::F_PIECE);
+                }
+            };
+            auto load_v = [&](int db) __attribute__((always_inline)) {
+                vf[db][0] = *reinterpret_cast<const uintx4*>(st + voff + 16 * db * TL::V_ROW);
+                vf[db][1] = *reinterpret_cast<const uintx4*>(st + voff + 16 * db * TL::V_ROW + TL::V_PIECE);
+                vf[db][2] = *reinterpret_cast<const uintx4*>(st + voff + 16 * db * TL::V_ROW + 2 * TL::V_PIECE);
+            };
+            // overlap of one feature step: all four piece products (exact product of the rounded features)
+            auto overlap = [&](int ks) __attribute__((always_inline)) {
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb) {
+                    s2[kb] = mma_bf16(ff[ks][kb][1], qfl[ks], s2[kb]);
+                    s2[kb] = mma_bf16(ff[ks][kb][1], qfh[ks], s2[kb]);
+                    s2[kb] = mma_bf16(ff[ks][kb][0], qfl[ks], s2[kb]);
+                    s2[kb] = mma_bf16(ff[ks][kb][0], qfh[ks], s2[kb]);
+                }
+            };
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb) {
+                    kf[ks][kb][0] = *reinterpret_cast<const uintx4*>(st + koff[ks] + 16 * kb * TL::K_ROW);
+                    kf[ks][kb][1] = *reinterpret_cast<const uintx4*>(st + koff[ks] + 16 * kb * TL::K_ROW + TL::K_PIECE);
+                }
+            if (AHEAD) {
+#pragma unroll
+                for (int ks = 0; ks < FA; ++ks) load_f(ks);
+                __builtin_amdgcn_sched_barrier(0);
+            }
             // scores: three piece products, smallest first
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
                 for (int kb = 0; kb < KB; ++kb) {
-                    const uintx4 khi = *reinterpret_cast<const uintx4*>(st + koff[ks] + 16 * kb * TL::K_ROW);
-                    const uintx4 klo = *reinterpret_cast<const uintx4*>(st + koff[ks] + 16 * kb * TL::K_ROW + TL::K_PIECE);
-                    s1[kb] = mma_bf16(klo, qh[ks], s1[kb]);
-                    s1[kb] = mma_bf16(khi, ql[ks], s1[kb]);
-                    s1[kb] = mma_bf16(khi, qh[ks], s1[kb]);
+                    s1[kb] = mma_bf16(kf[ks][kb][1], qh[ks], s1[kb]);
+                    s1[kb] = mma_bf16(kf[ks][kb][0], ql[ks], s1[kb]);
+                    s1[kb] = mma_bf16(kf[ks][kb][0], qh[ks], s1[kb]);
                 }
-            // overlap: all four piece products (exact product of the rounded features)
+            if (AHEAD) {
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int ks = 0; ks < FS; ++ks)
+                for (int ks = FA; ks < FS; ++ks) load_f(ks);
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int kb = 0; kb < KB; ++kb) {
-                    const uintx4 fhi = *reinterpret_cast<const uintx4*>(st + foff[ks] + 16 * kb * TL::F_ROW);
-                    const uintx4 flo = *reinterpret_cast<const uintx4*>(st + foff[ks] + 16 * kb * TL::F_ROW + TL::F_PIECE);
-                    s2[kb] = mma_bf16(flo, qfl[ks], s2[kb]);
-                    s2[kb] = mma_bf16(flo, qfh[ks], s2[kb]);
-                    s2[kb] = mma_bf16(fhi, qfl[ks], s2[kb]);
-                    s2[kb] = mma_bf16(fhi, qfh[ks], s2[kb]);
-                }
+                for (int ks = 0; ks < FA; ++ks) overlap(ks);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int db = 0; db < DA; ++db) load_v(db);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int ks = FA; ks < FS; ++ks) overlap(ks);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int db = DA; db < DB; ++db) load_v(db);
+                __builtin_amdgcn_sched_barrier(0);
+            } else {
+#pragma unroll
+                for (int ks = 0; ks < FS; ++ks) { load_f(ks); overlap(ks); }
+            }
             const bool interior = s_base - (qw0 + 15) >= -lc_lo && s_base + TK - 1 - qw0 < lc_hi &&
                                   s_base + TK <= len && qw0 + 15 < a.T;
             floatx4 p[KB];
@@ -2651,9 +2700,8 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
             split3(p[0], p[1], ph, pm, pl);
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
-                const uintx4 vh = *reinterpret_cast<const uintx4*>(st + voff + 16 * db * TL::V_ROW);
-                const uintx4 vm = *reinterpret_cast<const uintx4*>(st + voff + 16 * db * TL::V_ROW + TL::V_PIECE);
-                const uintx4 vl = *reinterpret_cast<const uintx4*>(st + voff + 16 * db * TL::V_ROW + 2 * TL::V_PIECE);
+                if (!AHEAD) load_v(db);
+                const uintx4 vh = vf[db][0], vm = vf[db][1], vl = vf[db][2];
                 floatx4 o = oacc[db];
                 o = mma_bf16(vl, ph, o);
                 o = mma_bf16(vh, pl, o);
