@@ -314,10 +314,11 @@ struct X3Tile {
 __device__ __forceinline__ int x3_swz(int row, int c, int row_bytes) {
     return row_bytes >= 128 ? (c ^ (row & 7)) : (c ^ ((row >> 1) & 3));
 }
-// an fp32 value rounded to 16 significant bits: bf16 head plus the bf16 head of the rest
+// an fp32 value rounded to 17 significant bits (its bf16 head and the bf16 head of the rest then add up to it exactly)
 __device__ __forceinline__ float quant16(float x) {
-    const float h = bf16_to_f32(f32_to_bf16(x));
-    return h + bf16_to_f32(f32_to_bf16(x - h));
+    // (finite x; ties away from zero.  17 significant bits split exactly: the head is rounded to nearest, so the rest is
+    //  at most half a unit of its last place, and its sign carries the ninth bit)
+    return __uint_as_float((__float_as_uint(x) + 0x40u) & 0xffffff80u);
 }
 __device__ __forceinline__ floatx4 quant16(floatx4 x) {
     floatx4 r = {quant16(x[0]), quant16(x[1]), quant16(x[2]), quant16(x[3])};
@@ -368,8 +369,10 @@ __device__ __forceinline__ void x3_emit_rows(const float* src, char* tile0, long
 }
 // 64 keys x D floats in LDS -> the three-piece transposed images [d][key slot] of the two 32-key tiles:
 // slot 8g + j of a tile <- key 16 (j / 4) + 4 g + j % 4 (the order in which score tiles leave the probabilities)
+// (with `gtile0` the same pieces also go to global memory, tiles `gtile_stride` bytes apart, write-through)
 template <int D, int LD>
-__device__ __forceinline__ void x3_emit_vt(const float* src, char* tile0, long tile_stride, int tid) {
+__device__ __forceinline__ void x3_emit_vt(const float* src, char* tile0, long tile_stride, int tid,
+                                           char* gtile0 = nullptr, long gtile_stride = 0) {
     constexpr int TOT = 2 * D * 4, PIECE = D * 2 * TK;
 #pragma unroll
     for (int j = 0; j < (TOT + NT - 1) / NT; ++j) {
@@ -385,6 +388,12 @@ __device__ __forceinline__ void x3_emit_vt(const float* src, char* tile0, long t
             *reinterpret_cast<uintx4*>(dst) = h;
             *reinterpret_cast<uintx4*>(dst + PIECE) = m;
             *reinterpret_cast<uintx4*>(dst + 2 * PIECE) = l;
+            if (gtile0) {
+                char* gd = gtile0 + tile * gtile_stride + d * (2 * TK) + x3_swz(d, gq, 2 * TK) * 16;
+                FLY_STORE(h, reinterpret_cast<uintx4*>(gd));
+                FLY_STORE(m, reinterpret_cast<uintx4*>(gd + PIECE));
+                FLY_STORE(l, reinterpret_cast<uintx4*>(gd + 2 * PIECE));
+            }
         }
     }
 }
@@ -709,7 +718,6 @@ __global__ __launch_bounds__(NT) void sb_kfeat_x3_kernel(KvArgs a) {
     char* Pimg = reinterpret_cast<char*>(Vs + CH * LDV);               // projection rows, three pieces
     float* diag = reinterpret_cast<float*>(Pimg + 3 * P_PIECE);        // t log2e |k|^2 / 2 per key
     float* red = diag + CH;                                            // 4 wave maxima
-    float* ks_lds = red + 4;                                           // 4 x M column sums
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
     const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H, sp = blockIdx.x;
@@ -776,10 +784,23 @@ __global__ __launch_bounds__(NT) void sb_kfeat_x3_kernel(KvArgs a) {
     const float lnm_half2 = 0.5f * __log2f(2.0f * a.mh_valid);
     const int per = (a.n_chunks + a.n_split - 1) / a.n_split;
     const int c0 = sp * per, c1 = min(a.n_chunks, c0 + per);
-    RowTile<CH, E> kt;
+    // K is fetched in the pattern of its image: piece j of a thread is 16-byte chunk idx % (E / 8) of key row
+    // idx / (E / 8), i.e. elements 32 ks + 4 gq + i and 32 ks + 16 + 4 gq + i -- two quads from global memory
+    constexpr int KCH8 = E / 8, KTOT = CH * KCH8, KNJ = (KTOT + NT - 1) / NT;
+    static_assert(KTOT % NT == 0 && NT % KCH8 == 0, "whole key rows per pass of the workgroup");
+    floatx4 kq0[KNJ], kq1[KNJ];
+    auto fetch_k = [&](int s_base) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < KNJ; ++j) {
+            const int idx = tid + NT * j, row64 = idx / KCH8, cch = idx % KCH8;
+            const float* sp_ = kptr + (long)min(s_base + row64, a.S - 1) * a.k_ss + 32 * (cch >> 2) + 4 * (cch & 3);
+            kq0[j] = load4_f32(sp_);
+            kq1[j] = load4_f32(sp_ + 16);
+        }
+    };
     RowTile<CH, D> vt;
     if (c0 < c1) {
-        kt.fetch(kptr, a.k_ss, c0 * CH, a.S - 1, tid);
+        fetch_k(c0 * CH);
         vt.fetch(vptr, a.v_ss, c0 * CH, a.S - 1, tid);
     }
     // projection rows scaled by sqrt(t) log2e, as three bf16 pieces in the k-slot order of the K image
@@ -801,74 +822,60 @@ __global__ __launch_bounds__(NT) void sb_kfeat_x3_kernel(KvArgs a) {
             }
         }
     }
-    // a chunk in registers -> K image (two pieces) and |k|^2 per key, V as fp32 rows for the transposition
-    auto stash = [&]() __attribute__((always_inline)) {
-        constexpr int V4 = E / 4;                         // RowTile pieces: idx -> row idx / V4, columns 4 (idx % V4) ..
+    // a chunk in registers -> K image (two pieces, into LDS and, write-through, into global memory: the stores drain
+    // while the projection runs) and |k|^2 per key; V as fp32 rows for the transposition
+    auto stash = [&](int c) __attribute__((always_inline)) {
+        char* kv_g = reinterpret_cast<char*>(a.vt) + ((long)bh * a.n_chunks + c) * (2 * (long)TL::KV_BYTES);
 #pragma unroll
-        for (int j = 0; j < RowTile<CH, E>::N; ++j) {
-            const int idx = tid + NT * j, row64 = idx / V4;
-            const floatx4 x = kt.r[j];
-            float sq = x[0] * x[0] + x[1] * x[1] + x[2] * x[2] + x[3] * x[3];
+        for (int j = 0; j < KNJ; ++j) {
+            const int idx = tid + NT * j, row64 = idx / KCH8, cch = idx % KCH8, row = row64 & (TK - 1);
+            const floatx4 x = kq0[j], y = kq1[j];
+            float sq = x[0] * x[0] + x[1] * x[1] + x[2] * x[2] + x[3] * x[3] + y[0] * y[0] + y[1] * y[1] + y[2] * y[2] + y[3] * y[3];
 #pragma unroll
-            for (int off = 1; off < V4; off <<= 1) sq += __shfl_xor(sq, off);      // the V4 lanes of one key row
-            if (idx % V4 == 0) diag[row64] = 0.5f * a.temp * LOG2E * sq;
+            for (int off = 1; off < KCH8; off <<= 1) sq += __shfl_xor(sq, off);    // the lanes of one key row
+            if (cch == 0) diag[row64] = 0.5f * a.temp * LOG2E * sq;
+            uintx4 khi, klo;
+            split2(x, y, khi, klo);
+            const int o = row * TL::K_ROW + x3_swz(row, cch, TL::K_ROW) * 16;
+            char* dst = img + (row64 / TK) * TL::BYTES + o;
+            *reinterpret_cast<uintx4*>(dst) = khi;
+            *reinterpret_cast<uintx4*>(dst + TL::K_PIECE) = klo;
+            char* gd = kv_g + (row64 / TK) * (long)TL::KV_BYTES + o;
+            FLY_STORE(khi, reinterpret_cast<uintx4*>(gd));
+            FLY_STORE(klo, reinterpret_cast<uintx4*>(gd + TL::K_PIECE));
         }
-        // the K image takes elements 32ks + 4gq + i and 32ks + 16 + 4gq + i into one chunk: go through Vs' neighbour?
-        // (no: the two quads sit in different threads' registers, so K goes through an fp32 staging tile too)
-        kt.template stash<E + 4>(reinterpret_cast<float*>(img), tid);             // fp32 K rows, overlaid on the images
         vt.template stash<LDV>(Vs, tid);
     };
-    if (c0 < c1) stash();
+    if (c0 < c1) stash(c0);
     __syncthreads();
     FLY_PROFK(1);
 
-    floatx4 kvacc[RB][DB];
+    floatx4 kvacc[RB][DB + 1];          // column block DB: the products with a column of ones = the sums of the features
 #pragma unroll
     for (int x = 0; x < RB; ++x)
 #pragma unroll
-        for (int db = 0; db < DB; ++db) kvacc[x][db] = Frag<float>::zero();
-    floatx4 ksp[FB], ksn[FB];
-#pragma unroll
-    for (int fb = 0; fb < FB; ++fb) { ksp[fb] = Frag<float>::zero(); ksn[fb] = Frag<float>::zero(); }
+        for (int db = 0; db <= DB; ++db) kvacc[x][db] = Frag<float>::zero();
     float run_max = -INFINITY;
     const int tile_w = w >> 1, row_w = 16 * (w & 1) + r16;              // this lane's key: tile and row inside it
+    // the projection fragments of this lane stay in registers for all chunks (one workgroup per compute unit: the
+    // register file is not what limits this kernel)
+    uintx4 pf[KS][FB][3];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int fb = 0; fb < FB; ++fb) {
+            const char* pp_ = Pimg + (16 * fb + r16) * P_ROW + x3_swz(r16, 4 * ks + g, P_ROW) * 16;
+#pragma unroll
+            for (int pc = 0; pc < 3; ++pc) pf[ks][fb][pc] = *reinterpret_cast<const uintx4*>(pp_ + pc * P_PIECE);
+        }
 
     for (int c = c0; c < c1; ++c) {
         const int s_base = c * CH;
         if (c + 1 < c1) {
-            kt.fetch(kptr, a.k_ss, s_base + CH, a.S - 1, tid);
+            fetch_k(s_base + CH);
             vt.fetch(vptr, a.v_ss, s_base + CH, a.S - 1, tid);
         }
-        // fp32 K rows (staged over the image area) -> registers -> K image; V^T image from Vs
-        {
-            constexpr int CH8 = E / 8, TOT = CH * CH8, NJ = (TOT + NT - 1) / NT;
-            uintx4 khi[NJ], klo[NJ];
-            const float* Kf = reinterpret_cast<const float*>(img);
-#pragma unroll
-            for (int j = 0; j < NJ; ++j) {
-                const int idx = tid + NT * j;
-                if (TOT % NT == 0 || idx < TOT) {
-                    const int row64 = idx / CH8, cch = idx % CH8, ks = cch >> 2, gq = cch & 3;
-                    const float* sp_ = Kf + row64 * (E + 4) + 32 * ks + 4 * gq;
-                    split2(*reinterpret_cast<const floatx4*>(sp_), *reinterpret_cast<const floatx4*>(sp_ + 16), khi[j], klo[j]);
-                }
-            }
-            __syncthreads();                             // every thread has its K quads: the staging tile may be overwritten
-#pragma unroll
-            for (int j = 0; j < NJ; ++j) {
-                const int idx = tid + NT * j;
-                if (TOT % NT == 0 || idx < TOT) {
-                    const int row64 = idx / CH8, cch = idx % CH8, row = row64 & (TK - 1);
-                    char* dst = img + (row64 / TK) * TL::BYTES + row * TL::K_ROW + x3_swz(row, cch, TL::K_ROW) * 16;
-                    *reinterpret_cast<uintx4*>(dst) = khi[j];
-                    *reinterpret_cast<uintx4*>(dst + TL::K_PIECE) = klo[j];
-                }
-            }
-            x3_emit_vt<D, LDV>(Vs, img + 2 * TL::K_PIECE, TL::BYTES, tid);
-        }
-        __syncthreads();
-        FLY_PROFK(2);
-        // projection of this wave's 16 keys: five piece products per step
+        // projection of this wave's 16 keys: five piece products per step (the K image is complete: stash() wrote it)
         floatx4 dd[FB];
 #pragma unroll
         for (int fb = 0; fb < FB; ++fb) dd[fb] = Frag<float>::zero();
@@ -878,9 +885,7 @@ __global__ __launch_bounds__(NT) void sb_kfeat_x3_kernel(KvArgs a) {
             const uintx4 kh = *reinterpret_cast<const uintx4*>(kp), kl = *reinterpret_cast<const uintx4*>(kp + TL::K_PIECE);
 #pragma unroll
             for (int fb = 0; fb < FB; ++fb) {
-                const char* pp_ = Pimg + (16 * fb + r16) * P_ROW + x3_swz(r16, 4 * ks + g, P_ROW) * 16;
-                const uintx4 ph = *reinterpret_cast<const uintx4*>(pp_), pm = *reinterpret_cast<const uintx4*>(pp_ + P_PIECE),
-                             pl = *reinterpret_cast<const uintx4*>(pp_ + 2 * P_PIECE);
+                const uintx4 ph = pf[ks][fb][0], pm = pf[ks][fb][1], pl = pf[ks][fb][2];
                 floatx4 d_ = dd[fb];
                 d_ = mma_bf16(pl, kh, d_);
                 d_ = mma_bf16(pm, kl, d_);
@@ -890,6 +895,12 @@ __global__ __launch_bounds__(NT) void sb_kfeat_x3_kernel(KvArgs a) {
                 dd[fb] = d_;
             }
         }
+        // V^T image from Vs (LDS and global memory), in the shadow of the projection; K'^T V below is its first reader
+        {
+            char* kv_g = reinterpret_cast<char*>(a.vt) + ((long)bh * a.n_chunks + c) * (2 * (long)TL::KV_BYTES);
+            x3_emit_vt<D, LDV>(Vs, img + 2 * TL::K_PIECE, TL::BYTES, tid, kv_g + 2 * TL::K_PIECE, TL::KV_BYTES);
+        }
+        FLY_PROFK(2);
         const float diag2 = diag[16 * w + r16];
         float amax = 0.f;
 #pragma unroll
@@ -900,7 +911,7 @@ __global__ __launch_bounds__(NT) void sb_kfeat_x3_kernel(KvArgs a) {
         amax = group_max(amax);
         const bool kvalid = (s_base + 16 * w + r16) < len;
         float cs = kvalid ? (amax - diag2 - lnm_half2) : -INFINITY;
-        cs = wave_max(cs);
+        cs = row16_max(cs);                                // (amax is already the maximum over the four lane groups)
         if (lane == 0) red[w] = cs;
         __syncthreads();
         const float lmax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
@@ -918,8 +929,6 @@ __global__ __launch_bounds__(NT) void sb_kfeat_x3_kernel(KvArgs a) {
                 fblk[fb][i] = ok ? quant16(__builtin_amdgcn_exp2f(dd[fb][i] + off)) : 0.f;
                 fblk[FB + fb][i] = ok ? quant16(__builtin_amdgcn_exp2f(-dd[fb][i] + off)) : 0.f;
             }
-            ksp[fb] = ksp[fb] * rescale + fblk[fb];
-            ksn[fb] = ksn[fb] * rescale + fblk[FB + fb];
         }
         {
             char* frow = img + tile_w * TL::BYTES + TL::KV_BYTES + row_w * TL::F_ROW;
@@ -935,18 +944,11 @@ __global__ __launch_bounds__(NT) void sb_kfeat_x3_kernel(KvArgs a) {
         if (tid == 0) a.chunk_scale[(long)bh * a.n_chunks + c] = live ? new_max * LN2 : 0.f;
         __syncthreads();                                   // images complete
         FLY_PROFK(3);
-        // images -> global memory, 16-byte pieces in thread order
+        // feature images -> global memory, 16-byte pieces in thread order
         {
-            char* kv_g = reinterpret_cast<char*>(a.vt) + ((long)bh * a.n_chunks + c) * (2 * (long)TL::KV_BYTES);
             char* f_g = reinterpret_cast<char*>(a.kfeat) + ((long)bh * a.n_chunks + c) * (2 * (long)TL::F_BYTES);
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
-#pragma unroll
-                for (int j = 0; j < (TL::KV_BYTES / 16 + NT - 1) / NT; ++j) {
-                    const int idx = tid + NT * j;
-                    if (TL::KV_BYTES / 16 % NT == 0 || idx < TL::KV_BYTES / 16)
-                        FLY_STORE(reinterpret_cast<const uintx4*>(img + t * TL::BYTES)[idx], reinterpret_cast<uintx4*>(kv_g + t * TL::KV_BYTES) + idx);
-                }
 #pragma unroll
                 for (int j = 0; j < (TL::F_BYTES / 16 + NT - 1) / NT; ++j) {
                     const int idx = tid + NT * j;
@@ -962,7 +964,8 @@ __global__ __launch_bounds__(NT) void sb_kfeat_x3_kernel(KvArgs a) {
 #pragma unroll
             for (int x = 0; x < RB; ++x)
 #pragma unroll
-                for (int db = 0; db < DB; ++db) kvacc[x][db] *= rescale;
+                for (int db = 0; db <= DB; ++db) kvacc[x][db] *= rescale;
+            const uintx4 ones = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};     // bf16 1.0 in every k-slot
             typedef __attribute__((address_space(3))) shortx4 lds_s4;
             typedef unsigned int uintx2_t __attribute__((ext_vector_type(2)));
 #pragma unroll
@@ -1004,14 +1007,17 @@ __global__ __launch_bounds__(NT) void sb_kfeat_x3_kernel(KvArgs a) {
                             o = mma_bf16(fh, vh[db], o);
                             kvacc[x][db] = o;
                         }
+                        kvacc[x][DB] = mma_bf16(fh, ones, mma_bf16(fl, ones, kvacc[x][DB]));
                     }
                 }
             }
         }
         FLY_PROFK(5);
-        __syncthreads();                                   // everyone is done with the images
-        if (c + 1 < c1) stash();
-        __syncthreads();
+        if (c + 1 < c1) {
+            __syncthreads();                               // everyone is done with the images
+            stash(c + 1);
+            __syncthreads();
+        }
     }
 
     // partial K'^T V in the combine step's order: tile (rb, db) -> 64 lanes x 4 floats with element
@@ -1026,20 +1032,10 @@ __global__ __launch_bounds__(NT) void sb_kfeat_x3_kernel(KvArgs a) {
 #pragma unroll
             for (int db = 0; db < DB; ++db)
                 FLY_STORE(kvacc[x][db], reinterpret_cast<floatx4*>(part + ((rb * DB + db) * 64 + 16 * g2 + r16) * 4));
+            // every column of the ones block holds the sum over the keys of the row's feature: features 16 rb + 4 g2 + i
+            if (r16 == 0) FLY_STORE(kvacc[x][DB], reinterpret_cast<floatx4*>(part + M * D + 16 * rb + 4 * g2));
         }
     }
-#pragma unroll
-    for (int fb = 0; fb < FB; ++fb)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const float p_ = row16_sum(ksp[fb][i]), n_ = row16_sum(ksn[fb][i]);
-            if (r16 == 0) {
-                ks_lds[w * M + 16 * fb + 4 * g + i] = p_;
-                ks_lds[w * M + MH + 16 * fb + 4 * g + i] = n_;
-            }
-        }
-    __syncthreads();
-    if (tid < M) part[M * D + tid] = (ks_lds[tid] + ks_lds[M + tid]) + (ks_lds[2 * M + tid] + ks_lds[3 * M + tid]);
     if (tid == 0) a.part_max[(long)bh * a.n_split + sp] = run_max * LN2;
     FLY_PROFK(6);
 }
