@@ -698,7 +698,7 @@ void sb_kfeat_kernel(KvArgs a) {
 //   projection : dd[feature][key] = (sqrt(t) log2e P) . k with P in three bf16 pieces (exact) as the row
 //                operand and the K image (two pieces) as the column operand, five piece products; a lane
 //                ends with four features of its key, as in sb_kfeat_kernel
-//   features   : exp2, rounded to 16 bits, written as two pieces into the feature image (16-byte writes:
+//   features   : exp2, rounded to 17 bits, written as two pieces into the feature image (16-byte writes:
 //                the lane's blocks 2p, 2p+1 are the eight k-slots of one chunk)
 //   K'^T V     : rows = feature positions of the image (transposing LDS reads hand a lane one feature
 //                column of four key rows), columns = value dims from the V^T image, five piece products;
@@ -723,7 +723,7 @@ __global__ __launch_bounds__(NT) void sb_kfeat_x3_kernel(KvArgs a) {
     const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H, sp = blockIdx.x;
     FLY_PROFK(0);
     if (sp >= a.n_split) {
-        // Query role: the features of 64 queries, rounded to 16 bits, and their log-scales (see sb_kfeat_kernel)
+        // Query role: the features of 64 queries, rounded to 17 bits, and their log-scales (see sb_kfeat_kernel)
         const float* pp = a.proj + r16 * E + 4 * g;
         const int iq = (sp - a.n_split) * TQ + 16 * w + r16;
         const float* qrow = reinterpret_cast<const float*>(a.q) + b * a.q_sb + h * a.q_sh + (long)min(iq, a.T - 1) * a.q_ss;
@@ -2406,18 +2406,23 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
     const int n_qt = (a.T + TQ - 1) / TQ;
-    if (SPLIT && (int)blockIdx.x >= a.band_wgs) {       // combine role, see sblocal_fwd_kernel
-        const int ci = blockIdx.x - a.band_wgs;
+    const int n_items = a.B * a.H * n_qt * a.n_parts;
+    const int per_xcd = (n_items + a.n_xcd - 1) / a.n_xcd;
+    const bool tail = (int)blockIdx.x >= a.band_wgs;
+    const int item = tail ? n_items : (blockIdx.x % a.n_xcd) * per_xcd + blockIdx.x / a.n_xcd;   // see sblocal_fwd_kernel
+    if (item >= n_items) {                             // workgroup-uniform
+        // Combine role, see sblocal_fwd_kernel: the workgroups behind the band workgroups, and the band range's own
+        // padding (its size is a whole number of rounds over the XCDs), which would otherwise hold a slot for nothing
+        if (!SPLIT) return;
+        const int n_pad = a.band_wgs - n_items;
+        const int ci = tail ? n_pad + (int)blockIdx.x - a.band_wgs : item - n_items;
+        if (ci >= a.B * a.H * a.cmb_wpb) return;
         FLY_PROF(0);
         sb_combine_body(smem, a.kv_part, a.part_max, const_cast<float*>(a.kv), const_cast<float*>(a.ksum),
                         const_cast<float*>(a.kmax), nullptr, ci / a.cmb_wpb, ci % a.cmb_wpb, a.cmb_wpb, a.n_split, M, D);
         FLY_PROF(7);
         return;
     }
-    const int n_items = a.B * a.H * n_qt * a.n_parts;
-    const int per_xcd = (n_items + a.n_xcd - 1) / a.n_xcd;
-    const int item = (blockIdx.x % a.n_xcd) * per_xcd + blockIdx.x / a.n_xcd;   // see sblocal_fwd_kernel
-    if (item >= n_items) return;                       // workgroup-uniform
     const int part = item % a.n_parts;
     const int qt = (item / a.n_parts) % n_qt;
     const int bh = item / (a.n_parts * n_qt), b = bh / a.H, h = bh % a.H;
@@ -2484,7 +2489,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
     }
     const float diag_q = 0.5f * a.temp * group_sum(sq);
 
-    // query features rounded to 16 bits, as two bf16 pieces in B-operand order (k-slot 8g + 4h + i of step ks
+    // query features rounded to 17 bits, as two bf16 pieces in B-operand order (k-slot 8g + 4h + i of step ks
     // = feature 32 ks + 16 h + 4 g + i, i.e. blocks 2 ks and 2 ks + 1 of the lane's features)
     uintx4 qfh[FS], qfl[FS];
     float lsq;
@@ -2533,7 +2538,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
             __syncthreads();      // Ps is dead; the tile buffers may overwrite it
         }
 #pragma unroll
-        for (int ks = 0; ks < FS; ++ks) split2(qf[2 * ks], qf[2 * ks + 1], qfh[ks], qfl[ks]);   // exact: 16-bit values
+        for (int ks = 0; ks < FS; ++ks) split2(qf[2 * ks], qf[2 * ks + 1], qfh[ks], qfl[ks]);   // exact: 17-bit values
     }
     FLY_PROF(1);
 
@@ -3129,13 +3134,16 @@ static int launch_fwd_x3(const FwdArgs& a, hipStream_t st) {
     args.n_xcd = mach.xcds;
     args.band_wgs = (int)grid;
     if (SPLIT) {
-        const long bhn = (long)a.B * a.H, free_slots = mach.slots - grid;
+        // combine role: as many workgroups per (batch, head) as fit beside the band workgroups in one residency round,
+        // at least one, at most one thread per 16-byte piece of the result; the padding of the band range serves first
+        const long bhn = (long)a.B * a.H, free_slots = mach.slots - items;
         long wpb = free_slots / bhn;
-        const long most = (M * (E + 1) / 4 + NT - 1) / NT;      // one 16-byte piece of the result per thread
+        const long most = (M * (E + 1) / 4 + NT - 1) / NT;
         if (wpb > most) wpb = most;
         if (wpb < 1) wpb = 1;
         args.cmb_wpb = (int)wpb;
-        grid += bhn * wpb;
+        const long pad = grid - items;
+        if (bhn * wpb > pad) grid += bhn * wpb - pad;
     }
     if (grid > 2147483647L) return fail(ERR_ARG, "sblocal_fwd: too many workgroups");
     if (g_ev_before) (void)hipEventRecord(g_ev_before, st);

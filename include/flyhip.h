@@ -65,7 +65,7 @@ int flyhip_sb_plan(int B, int H, int T, int S, int local_context,
  * per 32-key tile an image of K and V^T split into bfloat16 pieces there, and into kfeat (same
  * byte size as the fp32 features) an image of the features split into two pieces; passing the same
  * vt to flyhip_sblocal_fwd then runs the band on the bf16 matrix pipe with fp32-level accuracy
- * (features are rounded to 16 significant bits where they are formed).  kvt is unused for float. */
+ * (features are rounded to 17 significant bits where they are formed).  kvt is unused for float. */
 int flyhip_sb_kv_reduce(const void* k, const void* v, const float* proj, const int64_t* key_lengths,
                         void* kfeat, float* chunk_scale, float* kv_part, float* part_max,
                         float* kv, float* ksum, float* kmax,
