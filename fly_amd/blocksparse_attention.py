@@ -200,15 +200,16 @@ class BlockSparseAttention(nn.Module):
         layout = self.get_layout(T, S)
         needs_grad = torch.is_grad_enabled() and any(x.requires_grad for x in (query, key, value))
         if (self.fuse and not need_weights and not needs_grad
-                and (attn_mask is None or attn_mask.all_ones)
                 and not (self.training and self.dropout.p > 0)
                 and fused_attention.supports(block, query.dtype, E, value.shape[3])):
             if (T, S) not in self.fused_cache:
                 self.fused_cache[T, S] = fused_attention(layout, block)
-            key_mask = None
+            key_mask = add_mask = None
             if key_padding_mask is not None and not key_padding_mask.all_ones:
                 key_mask = key_padding_mask.additive_matrix
-            out = self.fused_cache[T, S](q, k, v, softmax_temp, key_mask)
+            if attn_mask is not None and not attn_mask.all_ones:
+                add_mask = attn_mask.additive_matrix        # (T, S), read per nonzero block inside the kernel
+            out = self.fused_cache[T, S](q, k, v, softmax_temp, key_mask, attn_mask=add_mask)
             return out.permute(0, 2, 1, 3)[:, :q_seqlen_og, :, :v_dim_og], None
         sdd_nt, dsd_nn, sparse_softmax = self.get_ops(T, S)
         if (needs_grad and not need_weights and not (self.training and self.dropout.p > 0)

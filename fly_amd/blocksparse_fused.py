@@ -8,11 +8,12 @@ from .blocksparse_utils import _as_layout3, union_table
 
 
 class fused_attention:
-    """``fused_attention(layout, block)(q, k, v, scale, key_mask=None)`` with q (Z,H,rows,D),
+    """``fused_attention(layout, block)(q, k, v, scale, key_mask=None, attn_mask=None)`` with q (Z,H,rows,D),
     k / v (Z,H,cols,D) (any batch / head / row strides, D contiguous) returns
-    softmax(scale * q k^T + key_mask[z, col]) v over the nonzero blocks of `layout`, shaped
-    (Z,H,rows,D) over memory laid out (Z,rows,H,D).  key_mask: fp32 (Z, cols), 0 or -inf.  Forward
-    only, 32x32 blocks of bf16 / fp16, D in {32,64,128}: `supports()` says whether a call qualifies."""
+    softmax(scale * q k^T + key_mask[z, col] + attn_mask[row, col]) v over the nonzero blocks of `layout`, shaped
+    (Z,H,rows,D) over memory laid out (Z,rows,H,D).  key_mask: fp32 (Z, cols), attn_mask: fp32 (rows, cols), both
+    additive (0 / -inf from the mask classes, blocksparse_attention.py:146-152).  Forward only, 32x32 blocks of
+    bf16 / fp16, D in {32,64,128}: `supports()` says whether a call qualifies."""
 
     def __init__(self, layout, block, rows_per_group=8):
         self.layout = _as_layout3(layout)
@@ -31,7 +32,7 @@ class fused_attention:
             self.lut_cache[device] = tuple(t.to(device) for t in union_table(self.layout, self.rows_per_group))
         return self.lut_cache[device]
 
-    def __call__(self, q, k, v, scale, key_mask=None, return_lse=False):
+    def __call__(self, q, k, v, scale, key_mask=None, return_lse=False, attn_mask=None):
         _lib.require_gpu(q, k, v)
         H, p, r = self.spdims
         Z, D = q.shape[0], q.shape[3]
@@ -53,15 +54,21 @@ class fused_attention:
                 raise ValueError(f'key_mask must have shape ({Z}, {r * 32}), got {tuple(key_mask.shape)}')
             key_mask = key_mask.to(device=q.device, dtype=torch.float32).contiguous()
             km, km_stride = key_mask.data_ptr(), key_mask.stride(0)
+        am, am_stride = None, 0
+        if attn_mask is not None:
+            if tuple(attn_mask.shape) != (p * 32, r * 32):
+                raise ValueError(f'attn_mask must have shape ({p * 32}, {r * 32}), got {tuple(attn_mask.shape)}')
+            attn_mask = attn_mask.to(device=q.device, dtype=torch.float32).contiguous()
+            am, am_stride = attn_mask.data_ptr(), attn_mask.stride(0)
         uni_ptr, uni_inner, uni_blk = self.make_lut(q.device)
         out = torch.empty((Z, p * 32, H, D), dtype=q.dtype, device=q.device).permute(0, 2, 1, 3)
         # base-2 log of every row's softmax denominator (+inf for a row without a finite score): what a
         # backward pass needs to form the probabilities again
         lse2 = torch.empty((Z, H, p * 32), dtype=torch.float32, device=q.device) if return_lse else None
         with torch.cuda.device(q.device):
-            _lib.call('flyhip_bs_attn_lse', q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), _lib.ptr(lse2),
+            _lib.call('flyhip_bs_attn_masks', q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), _lib.ptr(lse2),
                       uni_ptr.data_ptr(), uni_inner.data_ptr(), uni_blk.data_ptr(), self.rows_per_group,
-                      km, km_stride, Z, H, p, D, 32,
+                      km, km_stride, am, am_stride, Z, H, p, D, 32,
                       q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
                       v.stride(0), v.stride(1), v.stride(2), out.stride(0), out.stride(1), out.stride(2),
                       float(scale), _lib.dtype_code(q), _lib.stream_ptr(q.device))

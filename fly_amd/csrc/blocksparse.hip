@@ -1170,6 +1170,7 @@ struct AttnArgs {
     float scale;
     float* lse2;        // optional (Z, H, 32 * brows_per_head): base-2 log of every row's softmax denominator
     int n_xcd;          // dies the dispatcher deals workgroup ids to (set where the kernel is launched)
+    const float* am; long am_stride;     // optional (rows, cols) additive term per (query, key), shared by batch and heads
 };
 
 // Maxima of scores.  A two-operand fmaxf costs three instructions here (each operand is first quieted
@@ -1274,7 +1275,16 @@ __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
 
     // S^T[key 16kt + 4g + i][query 16qt + r16] of the tile in K buffer `buf`
     floatx4 sc[2][2];
-    auto score = [&](int buf) __attribute__((always_inline)) {
+    floatx4 amk[2][2];                                    // the attention-mask entries of sc (asked for with the scores)
+    const float* amrow = (MASKED && a.am) ? a.am + (long)(min(bi, a.brows_per_head - 1) * 32 + r16) * a.am_stride + 4 * g : nullptr;
+    auto score = [&](int buf, int inner) __attribute__((always_inline)) {
+        if (MASKED && amrow) {
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int qt = 0; qt < 2; ++qt)
+                    amk[kt][qt] = *reinterpret_cast<const floatx4*>(amrow + 16 * qt * a.am_stride + (long)inner * 32 + 16 * kt);
+        }
         const uint16_t* kp = ks_[buf];
         uintx4 fk[2][KS];
 #pragma unroll
@@ -1331,7 +1341,8 @@ __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
             }
 #pragma unroll
             for (int qt = 0; qt < 2; ++qt) {
-                const floatx4 t0 = sc[0][qt] * scale2 + mk[0], t1 = sc[1][qt] * scale2 + mk[1];
+                floatx4 t0 = sc[0][qt] * scale2 + mk[0], t1 = sc[1][qt] * scale2 + mk[1];
+                if (amrow) { t0 += amk[0][qt] * LOG2E; t1 += amk[1][qt] * LOG2E; }
                 float mx = fmaxf(fmaxf(fmaxf(t0[0], t0[1]), t0[2]), fmaxf(fmaxf(t0[3], t1[0]), t1[1]));
                 mx = fmaxf(fmaxf(mx, t1[2]), t1[3]);
                 mx = group_max(mx);
@@ -1388,7 +1399,7 @@ __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
         const int vb_next = vb == 2 ? 0 : vb + 1, vb_prev = vb == 0 ? 2 : vb - 1;
         if (s + 1 < n) fetch(inner_n1);
         if (late && had_prev) soft_pv(vb_prev, inner_prev);
-        if (present) score(s & 1);
+        if (present) score(s & 1, inner_cur);
         if (!late && present) soft_pv(vb, inner_cur);
         if (s + 1 < n) stash((s + 1) & 1, vb_next);
         had_prev = present;
@@ -2064,9 +2075,10 @@ static int launch_softmax(const RowArgs& args, dim3 grid, int max_elems, hipStre
     return check_launch("bs_softmax_kernel");
 }
 
-extern "C" int flyhip_bs_attn_lse(const void* q, const void* k, const void* v, void* out, float* lse2,
+extern "C" int flyhip_bs_attn_masks(const void* q, const void* k, const void* v, void* out, float* lse2,
                               const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
                               int rows_per_group, const float* key_mask, int64_t key_mask_stride,
+                              const float* attn_mask, int64_t attn_mask_stride,
                               int Z, int H, int brows_per_head, int D, int blk,
                               int64_t q_sz, int64_t q_sh, int64_t q_sm,
                               int64_t k_sz, int64_t k_sh, int64_t k_sn,
@@ -2084,15 +2096,18 @@ extern "C" int flyhip_bs_attn_lse(const void* q, const void* k, const void* v, v
                 "bs_attn: q / k / v strides must be multiples of 8 elements");
     FLY_REQUIRE(((o_sz | o_sh | o_sm) % 4) == 0, "bs_attn: out strides must be multiples of 4 elements");
     FLY_REQUIRE(!key_mask || key_mask_stride % 4 == 0, "bs_attn: key mask stride must be a multiple of 4");
+    FLY_REQUIRE(!attn_mask || attn_mask_stride % 4 == 0, "bs_attn: attention mask stride must be a multiple of 4");
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     const int gph = (brows_per_head + rows_per_group - 1) / rows_per_group;
     AttnArgs args{q, k, v, out, uni_ptr, uni_inner, uni_blk, key_mask, key_mask_stride, brows_per_head, gph, H, Z,
                   q_sz, q_sh, q_sm, k_sz, k_sh, k_sn, v_sz, v_sh, v_sn, o_sz, o_sh, o_sm, scale, lse2};
+    args.am = attn_mask;
+    args.am_stride = attn_mask_stride;
     const long nwg = unit_grid((long)H * Z, gph);
     args.n_xcd = machine().xcds;
     FLY_REQUIRE(nwg <= 2147483647L, "bs_attn: too many workgroups");
     dim3 grid((unsigned)nwg);
-    const bool masked = key_mask != nullptr || !(scale > 0.f);
+    const bool masked = key_mask != nullptr || attn_mask != nullptr || !(scale > 0.f);
 #define ATTN_LAUNCH(T, KS, NW)                                                                                  \
     do {                                                                                                        \
         if (masked) hipLaunchKernelGGL((bs_attn32_kernel<T, KS, NW, true>), grid, dim3(64 * NW), 0, st, args);  \
@@ -2104,6 +2119,20 @@ extern "C" int flyhip_bs_attn_lse(const void* q, const void* k, const void* v, v
 #undef ATTN_KS
 #undef ATTN_LAUNCH
     return check_launch("bs_attn32_kernel");
+}
+
+extern "C" int flyhip_bs_attn_lse(const void* q, const void* k, const void* v, void* out, float* lse2,
+                              const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
+                              int rows_per_group, const float* key_mask, int64_t key_mask_stride,
+                              int Z, int H, int brows_per_head, int D, int blk,
+                              int64_t q_sz, int64_t q_sh, int64_t q_sm,
+                              int64_t k_sz, int64_t k_sh, int64_t k_sn,
+                              int64_t v_sz, int64_t v_sh, int64_t v_sn,
+                              int64_t o_sz, int64_t o_sh, int64_t o_sm,
+                              float scale, int dtype, void* stream) {
+    return flyhip_bs_attn_masks(q, k, v, out, lse2, uni_ptr, uni_inner, uni_blk, rows_per_group, key_mask, key_mask_stride,
+                                nullptr, 0, Z, H, brows_per_head, D, blk, q_sz, q_sh, q_sm, k_sz, k_sh, k_sn, v_sz, v_sh, v_sn,
+                                o_sz, o_sh, o_sm, scale, dtype, stream);
 }
 
 extern "C" int flyhip_bs_attn(const void* q, const void* k, const void* v, void* out,

@@ -364,6 +364,23 @@ int flyhip_bs_attn_lse(const void* q, const void* k, const void* v, void* out, f
                        int64_t o_sz, int64_t o_sh, int64_t o_sm,
                        float scale, int dtype, void* stream);
 
+/* flyhip_bs_attn_lse with the attention mask of BlockSparseAttention.forward as well (ref:
+ * src/models/attention/blocksparse_attention.py:124-127,146-152: attn_mask.additive_matrix handed to the block
+ * softmax with attn_mask_mode='add'): attn_mask (optional, may be NULL) is fp32 (32 * brows_per_head, cols), row
+ * stride attn_mask_stride (a multiple of 4), an additive term per (query, key) shared by every batch entry and head --
+ * 0 / -inf from a FullMask, or any finite bias.  Only entries inside nonzero blocks are read.  A query without a
+ * finite score gets a zero row (:156-158). */
+int flyhip_bs_attn_masks(const void* q, const void* k, const void* v, void* out, float* lse2,
+                         const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
+                         int rows_per_group, const float* key_mask, int64_t key_mask_stride,
+                         const float* attn_mask, int64_t attn_mask_stride,
+                         int Z, int H, int brows_per_head, int D, int blk,
+                         int64_t q_sz, int64_t q_sh, int64_t q_sm,
+                         int64_t k_sz, int64_t k_sh, int64_t k_sn,
+                         int64_t v_sz, int64_t v_sh, int64_t v_sn,
+                         int64_t o_sz, int64_t o_sh, int64_t o_sm,
+                         float scale, int dtype, void* stream);
+
 /* The probabilities of that attention again, in the block-sparse format: p = exp(scale * q k^T - lse) on
  * the nonzero blocks, as one sdd (blocksparse_matmul.py:279-346) with an exponential epilogue;
  * lse2 as written by flyhip_bs_attn_lse; tables as for flyhip_bs_sdd's shared-tile path (four

@@ -381,6 +381,78 @@ def test_blocksparse_attention_module_fused_path():
 
 
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('p,r,D,rpg', [(7, 6, 64, 8), (5, 9, 32, 4), (9, 4, 128, 8)])
+def test_fused_attention_with_attention_mask(p, r, D, rpg, dtype):
+    """One-kernel attention with an additive (rows, cols) attention mask -- a random 0 / -inf mask, alone and
+    together with a key mask, and a finite bias -- against the oracle's SDD -> softmax(attn_mask, mode 'add')
+    -> nan_to_num -> DSD (blocksparse_attention.py:146-158); queries whose every score is masked give zero rows."""
+    from fly_amd.blocksparse_fused import fused_attention
+    print('case', p, r, D, rpg, dtype, flush=True)
+    Z, H, block = 2, 3, 32
+    g = torch.Generator().manual_seed(7 * p + r)
+    layout = random_layout(H, p, r, 3 * p + r, density=0.5)
+    layout[1, min(2, p - 1), :] = 0                       # an empty block-row
+    q = torch.randn(Z, p * 32, H, D, generator=g).to(dtype)
+    k = torch.randn(Z, r * 32, H, D, generator=g).to(dtype)
+    v = torch.randn(Z, r * 32, H, D, generator=g).to(dtype)
+    keep = torch.rand(p * 32, r * 32, generator=g) < 0.7
+    keep[5] = False                                       # a query that may attend to nothing
+    am_inf = torch.log(keep.float())
+    am_bias = torch.randn(p * 32, r * 32, generator=g)
+    lens = torch.tensor([r * 32, 40])
+    kpm = torch.log((torch.arange(r * 32).view(1, -1) < lens.view(Z, 1)).float())
+    scale = 0.27
+    qh, kh, vh = (x.permute(0, 2, 1, 3) for x in (q, k, v))
+    op = fused_attention(layout, block, rows_per_group=rpg)
+    for am, km in ((am_inf, None), (am_inf, kpm), (am_bias, None)):
+        qk = ob.sdd(qh.double(), kh.double(), layout, block, trans_b=True)
+        pr = ob.block_softmax(qk, layout, block, scale=scale, key_padding_mask=km, attn_mask=am).nan_to_num()
+        ref = ob.dsd(pr, vh.double(), layout, block)
+        out = op(qh.to(DEV), kh.to(DEV), vh.to(DEV), scale, None if km is None else km.to(DEV), attn_mask=am.to(DEV))
+        assert rel_err(out, ref) <= TOL[dtype]
+        if am is am_inf:
+            assert float(out[:, :, 5].abs().max()) == 0.0
+
+
+def test_blocksparse_attention_module_fused_with_full_mask():
+    """BlockSparseAttention.forward with a FullMask attention mask and a LengthMask stays on the one-kernel path
+    (eval, no gradients, bf16, 32x32 blocks), with sequence lengths and head dims that need padding
+    (blocksparse_attention.py:107-127,146-158; cf. tests/models/attention/test_blocksparse_attention.py:83-142)."""
+    from fly_amd import BlockSparseAttention, FullMask, LengthMask
+
+    class Cfg:
+        block = 32
+
+        def make_layout(self, seqlen):
+            nb = seqlen // self.block
+            lay = ob.band_layout(nb, nb, 1)
+            lay[:, 0] = 1
+            return lay.unsqueeze(0).repeat(3, 1, 1)
+
+    B, T, S, H, E = 2, 235, 179, 3, 40
+    g = torch.Generator().manual_seed(0)
+    q = torch.randn(B, T, H, E, generator=g).bfloat16()
+    k = torch.randn(B, S, H, E, generator=g).bfloat16()
+    v = torch.randn(B, S, H, E, generator=g).bfloat16()
+    lengths = torch.tensor([S, 77])
+    am_bool = torch.rand(T, S, generator=g) < 0.8
+    mod = BlockSparseAttention(Cfg(), attention_dropout=0.0, max_seq_length=256).to(DEV).eval()
+    with torch.no_grad():
+        out, w = mod(q.to(DEV), k.to(DEV), v.to(DEV), attn_mask=FullMask(am_bool.to(DEV)),
+                     key_padding_mask=LengthMask(lengths.to(DEV), max_len=S))
+    assert w is None and out.shape == (B, T, H, E)
+    assert len(mod.fused_cache) == 1 and len(mod.ops_cache) == 0        # the fused kernel ran
+    ref = ob.blocksparse_attention(q.double(), k.double(), v.double(), mod.master_layout.cpu(), 32,
+                                   key_lengths=lengths, attn_mask_bool=am_bool)
+    assert rel_err(out, ref) <= 2e-2
+    mod.fuse = False
+    with torch.no_grad():
+        out3, _ = mod(q.to(DEV), k.to(DEV), v.to(DEV), attn_mask=FullMask(am_bool.to(DEV)),
+                      key_padding_mask=LengthMask(lengths.to(DEV), max_len=S))
+    assert rel_err(out, out3.float()) <= 2e-2
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize('p,r,K', [(8, 6, 1024), (5, 7, 2000), (12, 3, 777 * 16)])
 def test_sdd_with_contraction_major_operands(p, r, K, dtype):
     """sparse = a^T b with a (K, M), b (K, N) and a long K -- the weight gradient of a block-sparse linear
