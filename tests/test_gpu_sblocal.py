@@ -233,6 +233,39 @@ def test_module_gradients_match_autograd_through_the_oracle(dtype, tol):
     assert torch.equal(out2, out.detach())
 
 
+@pytest.mark.parametrize('case', [
+    dict(B=2, L=3136, lc=512, temp=None, scale=64 ** -0.25),           # the benchmarked configuration
+    dict(B=4, L=3136, lc=256, temp=147 ** -0.5, scale=1.0),            # first T2T attention layer (4 of its 64 images)
+    dict(B=4, L=784, lc=256, temp=576 ** -0.5, scale=1.0),             # second T2T attention layer
+], ids=['config1', 'config3-L3136', 'config3-L784'])
+def test_gradients_at_benchmark_sizes_match_autograd_through_the_oracle(case):
+    """Training step of SBLocalAttention at the sizes the benchmark quotes (fp32, one head of 64 dims, 128
+    features): output and the gradients of query, key and value from the HIP forward and backward kernels against
+    autograd through the oracle in float64 (sblocal_attention.py:73-122)."""
+    from fly_amd import SBLocalAttention
+    B, L, lc, temp = case['B'], case['L'], case['lc'], case['temp']
+    H, E, mh = 1, 64, 64
+    g = torch.Generator().manual_seed(31)
+    q, k, v = (torch.randn(B, L, H, E, generator=g) * case['scale'] for _ in range(3))
+    P = osb.gaussian_orthogonal_random_matrix(mh, E, generator=g)
+    w = torch.randn(B, L, H, E, generator=g)
+    qd, kd, vd = (x.double().requires_grad_() for x in (q, k, v))
+    ref_out, _ = osb.sblocal_attention(qd, kd, vd, P.double(), lc, softmax_temp=temp)
+    (ref_out * w.double()).sum().backward()
+
+    dev = torch.device('cuda:0')
+    mod = SBLocalAttention(lc, dim_heads=E, nb_features=2 * mh, softmax_temp=temp, attention_dropout=0.0).to(dev)
+    mod.feature_map.projection_matrix.copy_(P)
+    mod.feature_map.freeze_projection()
+    mod.train()
+    qg, kg, vg = (x.to(dev).requires_grad_() for x in (q, k, v))
+    out, _ = mod(qg, kg, vg)
+    assert rel_err(out, ref_out.detach()) <= 1e-4
+    (out * w.to(dev)).sum().backward()
+    for name, got, ref in (('dq', qg.grad, qd.grad), ('dk', kg.grad, kd.grad), ('dv', vg.grad, vd.grad)):
+        assert rel_err(got, ref) <= 2e-4, (name, rel_err(got, ref))
+
+
 @pytest.mark.parametrize('dtype,tol', [(torch.float32, 1e-4), (torch.bfloat16, 3e-2)])
 def test_local_attention_module_gradients(dtype, tol):
     """LocalAttention is trainable: forward on the fused kernel, gradients against autograd through the
