@@ -46,6 +46,12 @@ __device__ long long g_prof[16384 * 8];
             if (wg_ < 16384) g_prof[wg_ * 8 + (slot)] = wall_clock64();                                  \
         }                                                                                                \
     } while (0)
+// (shader-clock stamps inside one iteration of the band kernel's key loop)
+__device__ long long g_prof2[16384 * 16];
+#define FLY_PROF2(cond, slot)                                                                            \
+    do {                                                                                                 \
+        if ((cond) && threadIdx.x == 0 && blockIdx.x < 16384) g_prof2[blockIdx.x * 16 + (slot)] = __builtin_readcyclecounter(); \
+    } while (0)
 // (the key pass has its own table: its grid is two-dimensional)
 __device__ long long g_prof_k[4096 * 8];
 #define FLY_PROFK(slot)                                                                                  \
@@ -57,6 +63,7 @@ __device__ long long g_prof_k[4096 * 8];
     } while (0)
 #else
 #define FLY_PROF(slot)
+#define FLY_PROF2(cond, slot)
 #define FLY_PROFK(slot)
 #endif
 
@@ -2581,6 +2588,8 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
         }
         const float wc = __builtin_amdgcn_exp2f((cscale - kmax) * LOG2E);
         const bool any = !(s_base + TK - 1 - qw0 < -lc_lo || s_base - (qw0 + 15) >= lc_hi || s_base >= len);
+        const bool stamp = kt == kt_lo + 1;
+        FLY_PROF2(stamp, 0);
         if (any) {
             floatx4 s1[KB], s2[KB];
 #pragma unroll
@@ -2606,14 +2615,17 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
                 vf[db][2] = *reinterpret_cast<const uintx4*>(st + voff + 16 * db * TL::V_ROW + 2 * TL::V_PIECE);
             };
             // overlap of one feature step: all four piece products (exact product of the rounded features)
+            // (consecutive MFMAs go to different accumulators: one that adds to the result of the one before it waits
+            //  for that result)
             auto overlap = [&](int ks) __attribute__((always_inline)) {
 #pragma unroll
-                for (int kb = 0; kb < KB; ++kb) {
-                    s2[kb] = mma_bf16(ff[ks][kb][1], qfl[ks], s2[kb]);
-                    s2[kb] = mma_bf16(ff[ks][kb][1], qfh[ks], s2[kb]);
-                    s2[kb] = mma_bf16(ff[ks][kb][0], qfl[ks], s2[kb]);
-                    s2[kb] = mma_bf16(ff[ks][kb][0], qfh[ks], s2[kb]);
-                }
+                for (int kb = 0; kb < KB; ++kb) s2[kb] = mma_bf16(ff[ks][kb][1], qfl[ks], s2[kb]);
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb) s2[kb] = mma_bf16(ff[ks][kb][1], qfh[ks], s2[kb]);
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb) s2[kb] = mma_bf16(ff[ks][kb][0], qfl[ks], s2[kb]);
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb) s2[kb] = mma_bf16(ff[ks][kb][0], qfh[ks], s2[kb]);
             };
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks)
@@ -2627,29 +2639,34 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
                 for (int ks = 0; ks < FA; ++ks) load_f(ks);
                 __builtin_amdgcn_sched_barrier(0);
             }
+            FLY_PROF2(stamp, 1);
             // scores: three piece products, smallest first
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks)
+            for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
-                for (int kb = 0; kb < KB; ++kb) {
-                    s1[kb] = mma_bf16(kf[ks][kb][1], qh[ks], s1[kb]);
-                    s1[kb] = mma_bf16(kf[ks][kb][0], ql[ks], s1[kb]);
-                    s1[kb] = mma_bf16(kf[ks][kb][0], qh[ks], s1[kb]);
-                }
+                for (int kb = 0; kb < KB; ++kb) s1[kb] = mma_bf16(kf[ks][kb][1], qh[ks], s1[kb]);
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb) s1[kb] = mma_bf16(kf[ks][kb][0], ql[ks], s1[kb]);
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb) s1[kb] = mma_bf16(kf[ks][kb][0], qh[ks], s1[kb]);
+            }
             if (AHEAD) {
                 __builtin_amdgcn_sched_barrier(0);
+                FLY_PROF2(stamp, 2);
 #pragma unroll
                 for (int ks = FA; ks < FS; ++ks) load_f(ks);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int ks = 0; ks < FA; ++ks) overlap(ks);
                 __builtin_amdgcn_sched_barrier(0);
+                FLY_PROF2(stamp, 3);
 #pragma unroll
                 for (int db = 0; db < DA; ++db) load_v(db);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int ks = FA; ks < FS; ++ks) overlap(ks);
                 __builtin_amdgcn_sched_barrier(0);
+                FLY_PROF2(stamp, 4);
 #pragma unroll
                 for (int db = DA; db < DB; ++db) load_v(db);
                 __builtin_amdgcn_sched_barrier(0);
@@ -2695,27 +2712,34 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
                     }
             };
             if (interior) soft(std::false_type{}); else soft(std::true_type{});
+            FLY_PROF2(stamp, 5);
             zp += ovs * wc;
             // O^T[d][query] += sum_keys V[key][d] p[key][query]: P exactly in three pieces, six products
             uintx4 ph, pm, pl;
             split3(p[0], p[1], ph, pm, pl);
+            if (!AHEAD) {
 #pragma unroll
-            for (int db = 0; db < DB; ++db) {
-                if (!AHEAD) load_v(db);
-                const uintx4 vh = vf[db][0], vm = vf[db][1], vl = vf[db][2];
-                floatx4 o = oacc[db];
-                o = mma_bf16(vl, ph, o);
-                o = mma_bf16(vh, pl, o);
-                o = mma_bf16(vm, pm, o);
-                o = mma_bf16(vm, ph, o);
-                o = mma_bf16(vh, pm, o);
-                o = mma_bf16(vh, ph, o);
-                oacc[db] = o;
+                for (int db = 0; db < DB; ++db) load_v(db);
             }
+#pragma unroll
+            for (int db = 0; db < DB; ++db) oacc[db] = mma_bf16(vf[db][2], ph, oacc[db]);
+#pragma unroll
+            for (int db = 0; db < DB; ++db) oacc[db] = mma_bf16(vf[db][0], pl, oacc[db]);
+#pragma unroll
+            for (int db = 0; db < DB; ++db) oacc[db] = mma_bf16(vf[db][1], pm, oacc[db]);
+#pragma unroll
+            for (int db = 0; db < DB; ++db) oacc[db] = mma_bf16(vf[db][1], ph, oacc[db]);
+#pragma unroll
+            for (int db = 0; db < DB; ++db) oacc[db] = mma_bf16(vf[db][0], pm, oacc[db]);
+#pragma unroll
+            for (int db = 0; db < DB; ++db) oacc[db] = mma_bf16(vf[db][0], ph, oacc[db]);
         }
+        FLY_PROF2(stamp, 6);
         if (more) stash(cur ^ 1);
         cscale = cscale_next;
+        FLY_PROF2(stamp, 7);
         __syncthreads();
+        FLY_PROF2(stamp, 8);
     }
 
     FLY_PROF(3);
@@ -3122,7 +3146,11 @@ template <int E, int M> constexpr size_t fwd_x3_smem() {
 template <int E, int M, bool SPLIT>
 static int launch_fwd_x3(const FwdArgs& a, hipStream_t st) {
     auto kern = sblocal_fwd_x3_kernel<E, E, M, SPLIT>;
+#ifdef FLY_X3_PAD
+    constexpr size_t smem = fwd_x3_smem<E, M>() + FLY_X3_PAD;
+#else
     constexpr size_t smem = fwd_x3_smem<E, M>();
+#endif
     static_assert(smem <= 160 * 1024, "two tile stages must fit the LDS");
     static std::atomic<unsigned long long> lds_set{0};     // (devices on which this kernel has its LDS limit)
     if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_set, "sblocal_fwd (bf16 pieces)")) return rc;
@@ -3620,6 +3648,11 @@ extern "C" int flyhip_prof_reset(void) {
 extern "C" int flyhip_prof_read_k(long long* dst, int n_workgroups) {
     hipDeviceSynchronize();
     hipError_t e = hipMemcpyFromSymbol(dst, HIP_SYMBOL(g_prof_k), sizeof(long long) * 8 * n_workgroups);
+    return e == hipSuccess ? 0 : -1;
+}
+extern "C" int flyhip_prof_read2(long long* dst, int n_workgroups) {
+    hipDeviceSynchronize();
+    hipError_t e = hipMemcpyFromSymbol(dst, HIP_SYMBOL(g_prof2), sizeof(long long) * 16 * n_workgroups);
     return e == hipSuccess ? 0 : -1;
 }
 extern "C" int flyhip_prof_read(long long* dst, int n_workgroups) {
