@@ -52,6 +52,12 @@ __device__ long long g_prof2[16384 * 16];
     do {                                                                                                 \
         if ((cond) && threadIdx.x == 0 && blockIdx.x < 16384) g_prof2[blockIdx.x * 16 + (slot)] = __builtin_readcyclecounter(); \
     } while (0)
+// (the same for waves 0 and 4 of a workgroup: slots 0..7 and 8..15)
+#define FLY_PROF3(cond, slot)                                                                            \
+    do {                                                                                                 \
+        if ((cond) && (threadIdx.x & 0x1bf) == 0 && blockIdx.x < 16384)                                  \
+            g_prof2[blockIdx.x * 16 + (threadIdx.x >> 8) * 8 + (slot)] = __builtin_readcyclecounter();   \
+    } while (0)
 // (the key pass has its own table: its grid is two-dimensional)
 __device__ long long g_prof_k[4096 * 8];
 #define FLY_PROFK(slot)                                                                                  \
@@ -64,6 +70,7 @@ __device__ long long g_prof_k[4096 * 8];
 #else
 #define FLY_PROF(slot)
 #define FLY_PROF2(cond, slot)
+#define FLY_PROF3(cond, slot)
 #define FLY_PROFK(slot)
 #endif
 
@@ -1480,14 +1487,18 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
     const bool late = w >= NW / 2;        // wave-uniform: this wave runs half a tile behind
     float cs_prev = 0.f;                  // chunk scale of the tile a late wave still owes its softmax
     auto tile_step = [&](int kt, int stage, float cscale) __attribute__((always_inline)) {
+        const bool stamp = kt == kt_lo + 8;
         if (!late) {
             score_phase(kt, stage);
+            FLY_PROF3(stamp, 2);
             soft_phase(kt, cscale);
         } else {
             if (kt > kt_lo) soft_phase(kt - 1, cs_prev);
+            FLY_PROF3(stamp, 2);
             score_phase(kt, stage);
             cs_prev = cscale;
         }
+        FLY_PROF3(stamp, 3);
     };
 
     FLY_PROF(2);
@@ -1499,11 +1510,16 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
     drain_loads();                         // once, before the loop: from here on the counts below are exact
     for (int kt = kt_lo; kt < kt_hi; kt += 2) {
         const float cs0 = cs_lds[kt * TK / CH - c_lo];
+        FLY_PROF3(kt == kt_lo + 8, 0);
         fetch(ra, min(kt + 2, kt_hi - 1));
+        FLY_PROF3(kt == kt_lo + 8, 1);
         tile_step(kt, 0, cs0);
         stash(rb, 1);
+        FLY_PROF3(kt == kt_lo + 8, 4);
         drain_loads_but<LOADS>();
+        FLY_PROF3(kt == kt_lo + 8, 5);
         __syncthreads();
+        FLY_PROF3(kt == kt_lo + 8, 6);
         // (no early exit between the halves: a path that leaves here with set A still in flight would
         // count, for the compiler, as a way back to the top of the loop)
         const bool second = kt + 1 < kt_hi;
@@ -1576,6 +1592,471 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
     }
     FLY_PROF(5);
 }
+
+// ---------------------------------------------------------------------------------------
+// fused band kernel for bfloat16 inputs, 32 queries per wave
+// ---------------------------------------------------------------------------------------
+// The algorithm, tile formats and scratch layouts of sblocal_fwd_bf16_kernel on v_mfma_f32_32x32x16_bf16: a
+// wave owns 32 queries, so every fragment it reads from LDS feeds twice the arithmetic (the 16-query kernel
+// spends most of its time on those reads).  Lane (c = lane % 32, h = lane / 32) supplies eight consecutive
+// k-slots 8h .. 8h+7 of row / column c per 16-slot step and receives D[8b + 4h + i][c], b = 0..3, i = 0..3, as
+// element 4b + i: one query per lane, whose 32 keys of a tile are split between the lane pair (c, c + 32).
+// The k-slot orders of the key pass's scratch fit without shuffles:
+//   overlap K' q' : position 32ks + 8g + j holds feature 32ks + 16(j/4) + 4g + j%4; step s = 2ks + t takes
+//                   positions 16s + 8h + j, i.e. (g = 2t + h) features 32ks + 8(2(j/4) + t) + 4h + j%4 -- elements
+//                   4t + j%4 and 4(2 + t) + j%4 of the lane's own block of 32 projected features
+//   P V           : position 8g + j of the V^T tile holds key 16(j/4) + 4g + j%4; step t takes positions
+//                   16t + 8h + j, i.e. keys 8(2(j/4) + t) + 4h + j%4 -- the lane's own score elements again
+// A workgroup is B32_WAVES waves of 32 queries.
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+__device__ __forceinline__ floatx16 mma32_bf16(uint4 a, uint4 b, floatx16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+__device__ __forceinline__ float pair32_max(float v) { float x, y; rows_pair32(v, x, y); return fmaxf(x, y); }
+__device__ __forceinline__ float pair32_sum(float v) { float x, y; rows_pair32(v, x, y); return x + y; }
+
+// The tile loads of sblocal_fwd_b32_kernel: per-lane byte offsets from the tile bases, computed once (the K tile that
+// runs past the last key row has its own), and the loads themselves -- wave w issues wave-loads w, w + NW, .. of every region.
+template <int E, int D, int M, int NW>
+struct B32Loads {
+    static constexpr int K_ROW = 2 * E, F_ROW = 2 * M, V_ROW = 2 * TK;
+    static constexpr int K_BYTES = TK * K_ROW, F_BYTES = TK * F_ROW, V_BYTES = D * V_ROW;
+    static constexpr int NKL = (K_BYTES / 1024 + NW - 1) / NW, NFL = (F_BYTES / 1024 + NW - 1) / NW, NVL = (V_BYTES / 1024 + NW - 1) / NW;
+    uint32_t kgo[NKL], kgo_last[NKL], fgo[NFL], vgo[NVL];
+    __device__ __forceinline__ void plan(long k_ss, int rows_last, int w, int lane) {
+#pragma unroll
+        for (int x = 0; x < NKL; ++x) {
+            const int o = 1024 * (NW * x + w) + 16 * lane, row = o / K_ROW, cp = (o % K_ROW) / 16;
+            kgo[x] = (uint32_t)(row * k_ss * 2 + x3_swz(row, cp, K_ROW) * 16);
+            kgo_last[x] = (uint32_t)(min(row, rows_last - 1) * k_ss * 2 + x3_swz(row, cp, K_ROW) * 16);
+        }
+#pragma unroll
+        for (int x = 0; x < NFL; ++x) {
+            const int o = 1024 * (NW * x + w) + 16 * lane, row = o / F_ROW, cp = (o % F_ROW) / 16;
+            fgo[x] = (uint32_t)(row * F_ROW + x3_swz(row, cp, F_ROW) * 16);
+        }
+#pragma unroll
+        for (int x = 0; x < NVL; ++x) {
+            const int o = 1024 * (NW * x + w) + 16 * lane, row = o / V_ROW, cp = (o % V_ROW) / 16;
+            vgo[x] = (uint32_t)(row * V_ROW + x3_swz(row, cp, V_ROW) * 16);
+        }
+    }
+    __device__ __forceinline__ void issue(char* st, int w, bool last, const char* kg, const char* fg, const char* vg) const {
+        typedef __attribute__((address_space(3))) void* lds_ptr;
+#pragma unroll
+        for (int x = 0; x < NKL; ++x)
+            if (K_BYTES / 1024 % NW == 0 || NW * x + w < K_BYTES / 1024)
+                __builtin_amdgcn_global_load_lds(kg + (last ? kgo_last[x] : kgo[x]), (lds_ptr)(st + 1024 * (NW * x + w)), 16, 0, 0);
+#pragma unroll
+        for (int x = 0; x < NFL; ++x)
+            if (F_BYTES / 1024 % NW == 0 || NW * x + w < F_BYTES / 1024)
+                __builtin_amdgcn_global_load_lds(fg + fgo[x], (lds_ptr)(st + K_BYTES + 1024 * (NW * x + w)), 16, 0, 0);
+#pragma unroll
+        for (int x = 0; x < NVL; ++x)
+            if (V_BYTES / 1024 % NW == 0 || NW * x + w < V_BYTES / 1024)
+                __builtin_amdgcn_global_load_lds(vg + vgo[x], (lds_ptr)(st + K_BYTES + F_BYTES + 1024 * (NW * x + w)), 16, 0, 0);
+    }
+};
+
+template <int E, int M> constexpr size_t fwd_b32_smem() { return fwd_bf16_smem<E, M>(); }
+// Four waves per workgroup (two workgroups per compute unit, which then overlap by themselves).  Eight with the skew
+// below measured the same at 64 and 128 features and slower at 256, where the skewed form spills registers.
+#ifndef B32_WAVES
+#define B32_WAVES 4
+#endif
+
+template <int E, int D, int M, bool SPLIT, int NW>
+__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2))) void sblocal_fwd_b32_kernel(FwdArgs a) {
+    static_assert(TK == 32, "one 32-key tile is one row block of the 32x32 MFMA");
+    constexpr int NT = 64 * NW, TQ = 32 * NW;          // shadow the constants of the fp32 kernels
+    constexpr int TQ64 = 64;                           // queries per tile of the partial workspace / merge
+    typedef bf16_t T;
+    constexpr int MH = M / 2, PB = MH / 32, KS = E / 16, FS = M / 16, DB = D / 32;
+    static_assert(MH % 32 == 0 && D % 32 == 0, "whole 32-row blocks");
+    constexpr int LDK = E + 8, LDKV = M + 8;           // LDS row strides in elements (projection rows, K'^T V)
+    // a tile stage: K rows, feature rows and V^T rows without padding, the 16-byte chunks of every row XOR-swizzled
+    // (x3_swz) -- the tiles come straight from global memory into LDS, a wave's 64 chunks to 1024 consecutive bytes
+    constexpr int K_ROW = 2 * E, F_ROW = 2 * M, V_ROW = 2 * TK;           // row sizes in bytes
+    constexpr int K_BYTES = TK * K_ROW, F_BYTES = TK * F_ROW, V_BYTES = D * V_ROW, STAGE_BYTES = K_BYTES + F_BYTES + V_BYTES;
+    static_assert(K_BYTES % 1024 == 0 && F_BYTES % 1024 == 0 && V_BYTES % 1024 == 0, "whole wave loads");
+    extern __shared__ __attribute__((aligned(128))) float smem[];
+    uint16_t* lds = reinterpret_cast<uint16_t*>(smem);
+
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c = lane & 31, h = lane >> 5;
+    if (SPLIT && (int)blockIdx.x >= a.band_wgs) {       // combine role, see sblocal_fwd_kernel
+        const int ci = blockIdx.x - a.band_wgs;
+        sb_combine_body(smem, a.kv_part, a.part_max, const_cast<float*>(a.kv), const_cast<float*>(a.ksum),
+                        const_cast<float*>(a.kmax), nullptr, ci / a.cmb_wpb, ci % a.cmb_wpb, a.cmb_wpb, a.n_split, M, D);
+        return;
+    }
+    const int n_qt = (a.T + TQ - 1) / TQ;
+    const int n_items = a.B * a.H * n_qt * a.n_parts;
+    const int per_xcd = (n_items + a.n_xcd - 1) / a.n_xcd;
+    const int item = (blockIdx.x % a.n_xcd) * per_xcd + blockIdx.x / a.n_xcd;   // see sblocal_fwd_kernel
+    if (item >= n_items) return;                       // workgroup-uniform
+    const int part = item % a.n_parts;
+    const int qt = (item / a.n_parts) % n_qt;
+    const int bh = item / (a.n_parts * n_qt), b = bh / a.H, hd = bh % a.H;
+    const int q0 = qt * TQ;
+    const int iq = q0 + 32 * w + c;
+    const bool qvalid = iq < a.T;
+    const uint16_t* qptr = reinterpret_cast<const uint16_t*>(a.q) + b * a.q_sb + hd * a.q_sh;
+    const uint16_t* kptr = reinterpret_cast<const uint16_t*>(a.k) + b * a.k_sb + hd * a.k_sh;
+    const uint16_t* vtp = reinterpret_cast<const uint16_t*>(a.vt) + (long)bh * a.n_chunks * CH * D;   // [tile][d][slot]
+    const uint16_t* fptr = reinterpret_cast<const uint16_t*>(a.kfeat) + (long)bh * a.n_chunks * CH * M;
+    const int len = a.lens ? min((int)a.lens[b], a.S) : a.S;
+    const float lnm_half = 0.5f * __logf(2.0f * a.mh_valid);
+    const int lc_lo = a.lc / 2, lc_hi = (a.lc + 1) / 2;    // band: -lc_lo <= s - i < lc_hi
+    constexpr float LOG2E = 1.4426950408889634f, LN2 = 0.6931471805599453f;
+
+    // this workgroup's share of the band, in 32-key tiles (as in sblocal_fwd_kernel)
+    const int q_last = min(q0 + TQ - 1, a.T - 1);
+    const int lo = max(0, q0 - lc_lo);
+    const int hi = min(len, q_last + lc_hi);
+    int kt_lo = lo / TK;
+    int kt_hi = (hi > lo) ? (hi + TK - 1) / TK : kt_lo;
+    if (SPLIT) {
+        const int nt = kt_hi - kt_lo, base = nt / a.n_parts, extra = nt % a.n_parts;
+        const int first = kt_lo + part * base + min(part, extra);
+        kt_lo = first;
+        kt_hi = first + base + (part < extra ? 1 : 0);
+    }
+
+    // Key tiles travel global memory -> LDS directly, one step ahead of their use (two stages): wave-load j of a
+    // region fills bytes 1024 j .. of it, lane l the chunk at 1024 j + 16 l, i.e. chunk position (1024 j + 16 l) % row
+    // / 16 of row (1024 j + 16 l) / row -- which holds the row's chunk x3_swz(row, position).  The waves share the loads.
+    const int last_tile = (a.S - 1) / TK;                 // the only K tile whose rows may not all exist
+    B32Loads<E, D, M, NW> tl;
+    tl.plan(a.k_ss, a.S - last_tile * TK, w, lane);
+    const float* csp = a.chunk_scale + (long)bh * a.n_chunks;
+    float cscale = (kt_lo < kt_hi) ? csp[kt_lo * TK / CH] : 0.f;
+    const float kmax = SPLIT ? split_kmax(a.part_max, bh, a.n_split) : a.kmax[bh];
+
+    // score operand: the query row as it is in memory, dims 16ks + 8h .. + 7
+    const uint16_t* qrow = qptr + (long)min(iq, a.T - 1) * a.q_ss;
+    uint4 qb[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qb[ks] = *reinterpret_cast<const uint4*>(qrow + 16 * ks + 8 * h);
+
+    // overlap operand: step s = 2 kq + t holds features 32 kq + 8 (2 jj + t) + 4h + i of the [positive | negative] row
+    uint4 qfb[FS];
+    float lsq, qk1 = 0.f;
+    if (SPLIT) {
+        const long qr_ = (long)bh * a.T + min(iq, a.T - 1);
+        const float* qfg = a.qfeat + qr_ * M;
+#pragma unroll
+        for (int s = 0; s < FS; ++s) {
+            const floatx4 x0 = *reinterpret_cast<const floatx4*>(qfg + 32 * (s >> 1) + 8 * (s & 1) + 4 * h);
+            const floatx4 x1 = *reinterpret_cast<const floatx4*>(qfg + 32 * (s >> 1) + 16 + 8 * (s & 1) + 4 * h);
+            qfb[s] = make_uint4(pack_bf16x2(x0[0], x0[1]), pack_bf16x2(x0[2], x0[3]), pack_bf16x2(x1[0], x1[1]), pack_bf16x2(x1[2], x1[3]));
+        }
+        lsq = a.q_lsq[qr_];
+    } else {
+        // |q|^2 from the score operand (the lane pair holds the two halves of every 16 dims)
+        float sq = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const uint32_t wds[4] = {qb[ks].x, qb[ks].y, qb[ks].z, qb[ks].w};
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                const float lo_ = __uint_as_float(wds[x] << 16), hi_ = __uint_as_float(wds[x] & 0xffff0000u);
+                sq += lo_ * lo_ + hi_ * hi_;
+            }
+        }
+        const float diag_q = 0.5f * a.temp * pair32_sum(sq);
+        // sqrt(t) P as bf16 head + bf16 remainder, rows of E + 8 elements
+        uint16_t* Phi = lds;
+        uint16_t* Plo = lds + MH * LDK;
+        const float pscale = sqrtf(a.temp);
+        for (int idx = tid; idx < MH * E / 4; idx += NT) {
+            const int f = idx / (E / 4), c4 = idx % (E / 4);
+            const floatx4 x = *reinterpret_cast<const floatx4*>(a.proj + (long)f * E + 4 * c4) * pscale;
+            floatx4 rem;
+            uint16_t hb[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                hb[i] = f32_to_bf16(x[i]);
+                rem[i] = x[i] - bf16_to_f32(hb[i]);
+            }
+            *reinterpret_cast<uint2*>(Phi + f * LDK + 4 * c4) = make_uint2(hb[0] | ((uint32_t)hb[1] << 16), hb[2] | ((uint32_t)hb[3] << 16));
+            *reinterpret_cast<uint2*>(Plo + f * LDK + 4 * c4) = make_uint2(pack_bf16x2(rem[0], rem[1]), pack_bf16x2(rem[2], rem[3]));
+        }
+        __syncthreads();
+        floatx16 dd[PB];                      // dd[pb][4b + i] = projection row 32 pb + 8b + 4h + i of this lane's query
+        float qmax = 0.f;
+#pragma unroll
+        for (int pb = 0; pb < PB; ++pb) {
+            floatx16 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const int off = (32 * pb + c) * LDK + 16 * ks + 8 * h;
+                acc = mma32_bf16(*reinterpret_cast<const uint4*>(Phi + off), qb[ks], acc);
+                acc = mma32_bf16(*reinterpret_cast<const uint4*>(Plo + off), qb[ks], acc);
+            }
+            dd[pb] = acc;
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+                if (32 * pb + 8 * (e >> 2) + 4 * h + (e & 3) < a.mh_valid) qmax = fmaxf(qmax, fabsf(acc[e]));
+        }
+        qmax = pair32_max(qmax);
+        lsq = -diag_q + qmax - lnm_half;
+        // features, the normaliser q' . sum K' on the way, and the operand (positive blocks first, then negative)
+        const float* ksg = a.ksum + (long)bh * M;
+#pragma unroll
+        for (int pb = 0; pb < PB; ++pb)
+#pragma unroll
+            for (int sg = 0; sg < 2; ++sg) {
+                float f[16];
+#pragma unroll
+                for (int bq = 0; bq < 4; ++bq) {
+                    const floatx4 ks4 = *reinterpret_cast<const floatx4*>(ksg + sg * MH + 32 * pb + 8 * bq + 4 * h);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float x = sg ? -dd[pb][4 * bq + i] : dd[pb][4 * bq + i];
+                        const bool ok = 32 * pb + 8 * bq + 4 * h + i < a.mh_valid;
+                        f[4 * bq + i] = ok ? __builtin_amdgcn_exp2f((x - qmax) * LOG2E) : 0.f;
+                        qk1 += f[4 * bq + i] * ks4[i];
+                    }
+                }
+                const int kq = sg * PB + pb;                  // 32-feature block of the [positive | negative] row
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+                    qfb[2 * kq + t] = make_uint4(pack_bf16x2(f[4 * t], f[4 * t + 1]), pack_bf16x2(f[4 * t + 2], f[4 * t + 3]),
+                                                 pack_bf16x2(f[4 * (2 + t)], f[4 * (2 + t) + 1]), pack_bf16x2(f[4 * (2 + t) + 2], f[4 * (2 + t) + 3]));
+            }
+        qk1 = pair32_sum(qk1);
+        __syncthreads();                 // the projection rows are dead; the tile buffers may overwrite them
+    }
+
+    const float sc = a.temp * LOG2E;             // scores leave the MFMA unscaled; exponents are base 2
+    const float c0 = (lsq + kmax) * LOG2E;       // base-2 log-scale of the global low-rank term
+    float m_run = c0;
+    float ze = 0.f, zp = 0.f;
+    floatx16 oacc[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) oacc[db][e] = 0.f;
+    const int qw0 = q0 + 32 * w;
+    const int smin = max(iq - lc_lo, 0);
+    const unsigned span = qvalid ? (unsigned)max(min(iq + lc_hi, len) - smin, 0) : 0u;
+
+    // fragment offsets inside a stage: step s of a row of 128 bytes or more reads chunk (2s + h) ^ (row & 7), i.e. one of
+    // four lane-dependent offsets (by s % 4) plus 128 (s / 4) bytes
+    static_assert(F_ROW >= 128, "feature rows of 64 features or more");
+    int foff4[4], koff4[4];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        foff4[v] = c * F_ROW + (((2 * v + h) ^ (c & 7)) * 16);
+        koff4[v] = K_ROW >= 128 ? c * K_ROW + (((2 * v + h) ^ (c & 7)) * 16) : c * K_ROW + x3_swz(c, (2 * v + h) & 3, K_ROW) * 16;
+    }
+
+    // One key tile takes two phases: scores (LDS fragment reads and the two score MFMA products) and softmax (the
+    // arithmetic on the scores, and P V).  The first loads the LDS and matrix pipes, the second the vector ALU.  With
+    // more than four waves per workgroup a SIMD holds two waves of it, and the upper half of the waves runs half a tile
+    // behind the lower half (one reads fragments and multiplies while the other does its softmax arithmetic); a wave's
+    // scores and V fragments of a tile stay in registers between the two phases.
+    floatx16 s1, s2;
+    uint4 vf[DB][2];
+    auto touches = [&](int kt) __attribute__((always_inline)) {      // wave-uniform: does the tile touch the band of any of the wave's queries?
+        const int s_base = kt * TK;
+        return !(s_base + TK - 1 - qw0 < -lc_lo || s_base - (qw0 + 31) >= lc_hi || s_base >= len);
+    };
+    auto score_phase = [&](int kt, int stage) __attribute__((always_inline)) {
+        if (!touches(kt)) return;
+        const char* Ks = reinterpret_cast<const char*>(lds) + stage * STAGE_BYTES;
+        const char* Fs = Ks + K_BYTES;
+        const char* Vt = Fs + F_BYTES;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) { s1[e] = 0.f; s2[e] = 0.f; }
+        // fragments are requested from LDS in batches ahead of the MFMAs that use them
+        uint4 kf[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) kf[ks] = *reinterpret_cast<const uint4*>(Ks + koff4[ks & 3] + 128 * (ks >> 2));
+        // (feature fragments in small batches, the next batch requested before the MFMAs of the current one)
+        constexpr int FBATCH = FS >= 16 ? 2 : (FS < 4 ? FS : 4), NBATCH = FS / FBATCH;    // (256 features leave room for pairs only)
+        static_assert(FS % FBATCH == 0, "whole batches");
+        uint4 ff[2][FBATCH];
+#pragma unroll
+        for (int s = 0; s < FBATCH; ++s) ff[0][s] = *reinterpret_cast<const uint4*>(Fs + foff4[s & 3] + 128 * (s >> 2));
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) s1 = mma32_bf16(kf[ks], qb[ks], s1);
+#pragma unroll
+        for (int bt = 0; bt < NBATCH; ++bt) {
+            if (bt + 1 < NBATCH) {
+#pragma unroll
+                for (int s = 0; s < FBATCH; ++s) {
+                    const int sn = (bt + 1) * FBATCH + s;
+                    ff[(bt + 1) & 1][s] = *reinterpret_cast<const uint4*>(Fs + foff4[sn & 3] + 128 * (sn >> 2));
+                }
+            } else {
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+#pragma unroll
+                    for (int t = 0; t < 2; ++t)
+                        vf[db][t] = *reinterpret_cast<const uint4*>(Vt + (32 * db + c) * V_ROW + x3_swz(32 * db + c, 2 * t + h, V_ROW) * 16);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int s = 0; s < FBATCH; ++s) s2 = mma32_bf16(ff[bt & 1][s], qfb[bt * FBATCH + s], s2);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    auto soft_phase = [&](int kt, float cs) __attribute__((always_inline)) {
+        if (!touches(kt)) return;
+        const int s_base = kt * TK;
+        const float wc = __builtin_amdgcn_exp2f((cs - kmax) * LOG2E);
+        // the lane holds the raw scores q.k of its query against keys s_base + 8b + 4h + i (element 4b + i)
+        const bool inside = s_base >= max(qw0 + 31 - lc_lo, 0) && s_base + TK <= min(qw0 + lc_hi, len) && qw0 + 31 < a.T;
+        float p[16];
+        float ovs = 0.f;
+        auto soft = [&](auto masked_t) __attribute__((always_inline)) {
+            constexpr bool MASKED = decltype(masked_t)::value;
+            bool ok[16];
+            float mx = -INFINITY;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int s = s_base + 8 * (e >> 2) + 4 * h + (e & 3);
+                ok[e] = !MASKED || (unsigned)(s - smin) < span;
+                mx = fmaxf(mx, ok[e] ? s1[e] : -INFINITY);
+            }
+            mx = pair32_max(mx) * sc;                               // sc > 0
+            // (the reference exponent is raised only when a tile exceeds it by more than 2^8)
+            if (__builtin_amdgcn_ballot_w64(mx > m_run + 8.f) != 0) {      // wave-uniform
+                const float m_new = fmaxf(m_run, mx);
+                const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+                m_run = m_new;
+                ze *= alpha;
+#pragma unroll
+                for (int db = 0; db < DB; ++db) oacc[db] *= alpha;
+            }
+            const float beta = wc * __builtin_amdgcn_exp2f(c0 - m_run);      // scale of the overlap term
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const float ex = ok[e] ? __builtin_amdgcn_exp2f(__builtin_fmaf(s1[e], sc, -m_run)) : 0.f;
+                const float ov = ok[e] ? s2[e] : 0.f;
+                ze += ex;
+                ovs += ov;
+                p[e] = ex - ov * beta;
+            }
+        };
+        if (inside) soft(std::false_type{}); else soft(std::true_type{});
+        zp += ovs * wc;
+        // O^T[d][query] += sum_keys V[key][d] p[key][query]: step t takes the lane's elements 4t + i and 4(2 + t) + i
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const uint4 pb_ = make_uint4(pack_bf16x2(p[4 * t], p[4 * t + 1]), pack_bf16x2(p[4 * t + 2], p[4 * t + 3]),
+                                         pack_bf16x2(p[4 * (2 + t)], p[4 * (2 + t) + 1]), pack_bf16x2(p[4 * (2 + t) + 2], p[4 * (2 + t) + 3]));
+#pragma unroll
+            for (int db = 0; db < DB; ++db) oacc[db] = mma32_bf16(vf[db][t], pb_, oacc[db]);
+        }
+    };
+    const bool late = NW > 4 && w >= NW / 2;      // wave-uniform: this wave runs half a tile behind
+    float cs_prev = 0.f;                          // chunk scale of the tile a late wave still owes its softmax
+    // (the first pass, kt = kt_lo - 1, only brings the first tile in)
+    for (int kt = kt_lo - 1; kt < kt_hi; ++kt) {
+        const int cur = (kt - kt_lo) & 1;
+        const bool more = kt + 1 < kt_hi;
+        float cscale_next = cscale;
+        if (more) {                                      // next tile's loads fly during the MFMAs (every wave is past the barrier
+            const int ktn = kt + 1, ktc = min(ktn, last_tile);      // that ended the last use of that stage; tiles past the keys
+            tl.issue(reinterpret_cast<char*>(lds) + (cur ^ 1) * STAGE_BYTES, w, ktc == last_tile,      // are never used: stay in bounds)
+                     reinterpret_cast<const char*>(kptr + (long)ktc * TK * a.k_ss),
+                     reinterpret_cast<const char*>(fptr + (long)ktn * TK * M), reinterpret_cast<const char*>(vtp + (long)ktn * (D * TK)));
+            cscale_next = csp[(kt + 1) * TK / CH];
+        }
+        if (kt >= kt_lo) {
+            if (!late) {
+                score_phase(kt, cur);
+                soft_phase(kt, cscale);
+            } else {
+                if (kt > kt_lo) soft_phase(kt - 1, cs_prev);
+                score_phase(kt, cur);
+                cs_prev = cscale;
+            }
+        }
+        drain_loads();                                   // this wave's share of the next tile is in LDS
+        cscale = cscale_next;
+        __syncthreads();
+    }
+    if (late && kt_lo < kt_hi) soft_phase(kt_hi - 1, cs_prev);
+
+    // global low-rank term: qkv^T[d][query] = sum_r KV[r][d] q'[query][r]; K'^T V comes as bf16, transposed,
+    // features in the slot order of the overlap operand
+    floatx16 lacc[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) lacc[db][e] = 0.f;
+    if (!SPLIT) {
+        uint16_t* KVt = lds;
+        const uint16_t* kvg = reinterpret_cast<const uint16_t*>(a.kvt) + (long)bh * M * D;
+        constexpr int KVC = D * M / 8;
+#pragma unroll
+        for (int j = 0; j < (KVC + NT - 1) / NT; ++j) {
+            const int idx = tid + NT * j, d = idx / (M / 8), c8 = idx % (M / 8);
+            if (KVC % NT == 0 || idx < KVC)
+                *reinterpret_cast<uint4*>(KVt + d * LDKV + 8 * c8) = *reinterpret_cast<const uint4*>(kvg + (long)d * M + 8 * c8);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int s = 0; s < FS; ++s)
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+                lacc[db] = mma32_bf16(*reinterpret_cast<const uint4*>(KVt + (32 * db + c) * LDKV + 16 * s + 8 * h), qfb[s], lacc[db]);
+    }
+    ze = pair32_sum(ze);
+    zp = pair32_sum(zp);
+    const float gamma = __builtin_amdgcn_exp2f(c0 - m_run);               // <= 1
+    if (SPLIT) {
+        // partials are kept per 64-query tile (the unit of sb_merge_kernel); this wave's tile:
+        const int n_qt64 = (a.T + TQ64 - 1) / TQ64, t64 = (q0 + 32 * w) / TQ64;
+        if (t64 < n_qt64) {                            // wave-uniform
+            float* ws = a.part_ws + (((long)bh * n_qt64 + t64) * a.n_parts + part) * (TQ64 * (D + NSTAT));
+            const int ql = (32 * w + c) % TQ64;
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int bq = 0; bq < 4; ++bq) {
+                    const floatx4 o4 = {oacc[db][4 * bq], oacc[db][4 * bq + 1], oacc[db][4 * bq + 2], oacc[db][4 * bq + 3]};
+                    *reinterpret_cast<floatx4*>(ws + ql * D + 32 * db + 8 * bq + 4 * h) = o4;
+                }
+            if (h == 0) {
+                float* st = ws + TQ64 * D;
+                st[0 * TQ64 + ql] = m_run;
+                st[1 * TQ64 + ql] = ze;
+                st[2 * TQ64 + ql] = zp;
+                st[3 * TQ64 + ql] = 0.f;
+                st[4 * TQ64 + ql] = c0;
+            }
+        }
+    } else {
+        const float Z = ze + gamma * fmaxf(qk1 - zp, 1e-24f);
+        const float inv = 1.0f / Z;
+        if (qvalid) {
+            T* optr = reinterpret_cast<T*>(a.out) + b * a.o_sb + hd * a.o_sh + (long)iq * a.o_ss;
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int bq = 0; bq < 4; ++bq) {
+                    floatx4 o4;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) o4[i] = (oacc[db][4 * bq + i] + gamma * lacc[db][4 * bq + i]) * inv;
+                    store4_f32(optr + 32 * db + 8 * bq + 4 * h, o4);
+                }
+            if (h == 0) a.log_norm[(long)bh * a.T + iq] = m_run * LN2 + __logf(Z);
+        }
+    }
+}
+
+// (explicit instantiations: the launcher refers to these through a deduced return type)
+#define FLY_B32_INST(EE, MM)                                                        \
+    template __global__ void sblocal_fwd_b32_kernel<EE, EE, MM, false, B32_WAVES>(FwdArgs);   \
+    template __global__ void sblocal_fwd_b32_kernel<EE, EE, MM, true, B32_WAVES>(FwdArgs);
+FLY_B32_INST(32, 64) FLY_B32_INST(32, 128) FLY_B32_INST(32, 256)
+FLY_B32_INST(64, 64) FLY_B32_INST(64, 128) FLY_B32_INST(64, 256)
+#undef FLY_B32_INST
 
 // ---------------------------------------------------------------------------------------
 // key pass for bfloat16 inputs (key role only; used when no query features are asked for)
@@ -3088,10 +3569,20 @@ template <typename T, int E, int M, bool SPLIT> struct FwdKernel {
     static constexpr int threads = NT, tq = TQ;       // threads and queries per workgroup
     static auto get() { return sblocal_fwd_kernel<T, E, E, M, SPLIT>; }
 };
+#ifndef FLY_BF16_WIDE
+#define FLY_BF16_WIDE 1
+#endif
+// bfloat16 inputs: 32 queries per wave where the registers hold the wider operands (head dim up to 64) and the
+// projection rows fill 32-row blocks (64 features or more); 16 queries per wave otherwise.  Both: 128 queries per workgroup.
+template <int E, int M> constexpr bool bf16_wide() { return FLY_BF16_WIDE && M >= 64 && E <= 64; }
 template <int E, int M, bool SPLIT> struct FwdKernel<bf16_t, E, M, SPLIT> {
     static constexpr size_t smem = fwd_bf16_smem<E, M>();
-    static constexpr int threads = 64 * BF16_WAVES, tq = 16 * BF16_WAVES;
-    static auto get() { return sblocal_fwd_bf16_kernel<E, E, M, SPLIT, BF16_WAVES>; }
+    static constexpr int threads = bf16_wide<E, M>() ? 64 * B32_WAVES : 64 * BF16_WAVES;
+    static constexpr int tq = bf16_wide<E, M>() ? 32 * B32_WAVES : 16 * BF16_WAVES;
+    static auto get() {
+        if constexpr (bf16_wide<E, M>()) return sblocal_fwd_b32_kernel<E, E, M, SPLIT, B32_WAVES>;
+        else return sblocal_fwd_bf16_kernel<E, E, M, SPLIT, BF16_WAVES>;
+    }
 };
 
 template <typename T, int E, int M, bool SPLIT>
