@@ -26,12 +26,14 @@ def _hipcc():
 
 def build(verbose=False):
     hipcc = _hipcc()
+    # extra compiler flags for measurement builds (e.g. -DFLY_BF16_WIDE=0: the 16-queries-per-wave bfloat16 band kernel everywhere)
+    extra = os.environ.get('FLYHIP_EXTRA_FLAGS', '').split()
     objdir = os.path.join(HERE, 'build')
     os.makedirs(objdir, exist_ok=True)
 
     def compile_one(src):
         obj = os.path.join(objdir, os.path.splitext(src)[0] + '.o')
-        cmd = [hipcc] + FLAGS + ['-x', 'hip', '-c', os.path.join(CSRC, src), '-o', obj]
+        cmd = [hipcc] + FLAGS + extra + ['-x', 'hip', '-c', os.path.join(CSRC, src), '-o', obj]
         res = subprocess.run(cmd, capture_output=True, text=True)
         if res.returncode != 0:
             raise RuntimeError(f'hipcc failed on {src}:\n{res.stderr}')
