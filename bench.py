@@ -275,13 +275,16 @@ def bench_other_configs():
         for _ in range(w):
             fn()
         torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(n):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / n
+        reps = []
+        for _ in range(3):                      # median of three timed runs of n calls (clocks settle between workloads)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(n):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            reps.append(e0.elapsed_time(e1) / n)
+        return sorted(reps)[1]
 
     for L, dim in ((3136, 147), (784, 576)):
         B, H, E, mh, lc = 64, 1, 64, 64, 256
