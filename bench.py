@@ -120,7 +120,7 @@ def bench_sblocal(steps, warmup, cpu_baseline=True):
                      'kernel_ms': fwd_ms, 'flops_per_launch': fwd_flops, 'launches_timed': len(ev),
                      'arithmetic': 'fp32 inputs, outputs and accumulation; products on v_mfma_f32_16x16x32_bf16 from '
                                    'operands split into bf16 pieces (scores 3 piece products, feature overlap 4 on '
-                                   'features rounded to 17 bits, P V 6); priced against the fp32 MFMA peak'},
+                                   'features rounded to 17 bits, P V 5 with V rounded to 16 bits); priced against the fp32 MFMA peak'},
         'parity': None,
         'flops_per_step': total_flops,
     }

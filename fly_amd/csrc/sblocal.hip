@@ -310,17 +310,27 @@ __device__ __forceinline__ floatx4 mma_bf16(uintx4 a, uintx4 b, floatx4 c) {
 //              perturbs a feature by 2^-17 relative, consistently everywhere.
 //   scores   : q, k in two pieces, three products (the lo.lo product, 2^-16 relative, is dropped: an
 //              error in an exponent, not in a difference).
-//   P V      : probabilities and values in three pieces each (exact), the six products above 2^-24.
+//   P V      : probabilities in three pieces (exact), values in X3_VP pieces: two (V rounded to 16 bits, five products;
+//              K'^T V of the key pass multiplies the same rounded V) or three (exact, six products).
 // The key pass leaves every 32-key tile as an image of what the band kernel wants in LDS: in the
-// feature / operand scratch, per tile, [K hi][K lo][V^T h][V^T m][V^T l] (the "kv image") and
+// feature / operand scratch, per tile, [K hi][K lo][V^T h][V^T m]([V^T l]) (the "kv image") and
 // [K' hi][K' lo] (the "feature image"); rows of K and K' in the k-slot order of the MFMA, V
 // transposed to [d][key slot], and the 16-byte chunks of every row XOR-swizzled so that the
 // fragment reads of 8 consecutive rows fall into different LDS banks without padding.
+// bf16 pieces of V in the images: two carry 16 significant bits of V -- every product that involves V (P V in the band
+// kernel, K'^T V in the key pass) then uses the same rounded V, so the cancellation between the band's low-rank part and
+// the global term is untouched and the result moves by at most 2^-17 |V| -- three are exact to fp32 and cost a sixth more
+// matrix and LDS work per tile.
+#ifndef FLY_X3_VP
+#define FLY_X3_VP 2
+#endif
+constexpr int X3_VP = FLY_X3_VP;
+static_assert(X3_VP == 2 || X3_VP == 3, "two or three pieces");
 template <int E, int D, int M>
 struct X3Tile {
     static constexpr int K_ROW = 2 * E, F_ROW = 2 * M, V_ROW = 2 * TK;           // bytes per row
     static constexpr int K_PIECE = TK * K_ROW, F_PIECE = TK * F_ROW, V_PIECE = D * V_ROW;
-    static constexpr int KV_BYTES = 2 * K_PIECE + 3 * V_PIECE;                    // per tile, operand scratch
+    static constexpr int KV_BYTES = 2 * K_PIECE + X3_VP * V_PIECE;                // per tile, operand scratch
     static constexpr int F_BYTES = 2 * F_PIECE;                                   // per tile, feature scratch
     static constexpr int BYTES = KV_BYTES + F_BYTES;                              // one LDS stage
 };
@@ -397,16 +407,16 @@ __device__ __forceinline__ void x3_emit_vt(const float* src, char* tile0, long t
             const floatx4 x0 = {col[0], col[LD], col[2 * LD], col[3 * LD]};
             const floatx4 x1 = {col[16 * LD], col[17 * LD], col[18 * LD], col[19 * LD]};
             uintx4 h, m, l;
-            split3(x0, x1, h, m, l);
+            if (X3_VP == 3) split3(x0, x1, h, m, l); else split2(x0, x1, h, m);
             char* dst = tile0 + tile * tile_stride + d * (2 * TK) + x3_swz(d, gq, 2 * TK) * 16;
             *reinterpret_cast<uintx4*>(dst) = h;
             *reinterpret_cast<uintx4*>(dst + PIECE) = m;
-            *reinterpret_cast<uintx4*>(dst + 2 * PIECE) = l;
+            if (X3_VP == 3) *reinterpret_cast<uintx4*>(dst + 2 * PIECE) = l;
             if (gtile0) {
                 char* gd = gtile0 + tile * gtile_stride + d * (2 * TK) + x3_swz(d, gq, 2 * TK) * 16;
                 FLY_STORE(h, reinterpret_cast<uintx4*>(gd));
                 FLY_STORE(m, reinterpret_cast<uintx4*>(gd + PIECE));
-                FLY_STORE(l, reinterpret_cast<uintx4*>(gd + 2 * PIECE));
+                if (X3_VP == 3) FLY_STORE(l, reinterpret_cast<uintx4*>(gd + 2 * PIECE));
             }
         }
     }
@@ -991,7 +1001,7 @@ __global__ __launch_bounds__(NT) void sb_kfeat_x3_kernel(KvArgs a) {
                     const char* vp = ti + 2 * TL::K_PIECE + (16 * db + r16) * TL::V_ROW + x3_swz(r16, g, TL::V_ROW) * 16;
                     vh[db] = *reinterpret_cast<const uintx4*>(vp);
                     vm[db] = *reinterpret_cast<const uintx4*>(vp + TL::V_PIECE);
-                    vl[db] = *reinterpret_cast<const uintx4*>(vp + 2 * TL::V_PIECE);
+                    if (X3_VP == 3) vl[db] = *reinterpret_cast<const uintx4*>(vp + 2 * TL::V_PIECE);
                 }
 #pragma unroll
                 for (int x = 0; x < RB; ++x) {
@@ -1015,7 +1025,7 @@ __global__ __launch_bounds__(NT) void sb_kfeat_x3_kernel(KvArgs a) {
                         for (int db = 0; db < DB; ++db) {
                             floatx4 o = kvacc[x][db];
                             o = mma_bf16(fl, vm[db], o);
-                            o = mma_bf16(fh, vl[db], o);
+                            if (X3_VP == 3) o = mma_bf16(fh, vl[db], o);
                             o = mma_bf16(fl, vh[db], o);
                             o = mma_bf16(fh, vm[db], o);
                             o = mma_bf16(fh, vh[db], o);
@@ -2879,7 +2889,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
 // Same work decomposition, masks, online softmax and outputs as sblocal_fwd_kernel; the three products
 // of the key loop run on v_mfma_f32_16x16x32_bf16 from the tile images the key pass has left (see
 // X3Tile): per 32-key tile and wave 12 MFMAs for the scores (three piece products), 4 M / 16 for the
-// overlap (four), 6 D / 16 for P V (six) instead of (E + M + D) / 2 fp32 MFMAs of twice the duration.
+// overlap (four), 5 D / 16 for P V (five; six with three V pieces) instead of (E + M + D) / 2 fp32 MFMAs of twice the duration.
 // A tile image is copied global -> registers -> LDS as it is (16-byte pieces in thread order), two LDS
 // stages.
 template <int E, int D, int M, bool SPLIT>
@@ -3082,7 +3092,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
             // this takes would cost the second workgroup of a compute unit, and fragments are requested where they are used)
             constexpr bool AHEAD = SPLIT;
             constexpr int FA = (FS + 1) / 2, DA = (DB + 1) / 2;
-            uintx4 kf[KS][KB][2], ff[FS][KB][2], vf[DB][3];
+            uintx4 kf[KS][KB][2], ff[FS][KB][2], vf[DB][X3_VP];
             auto load_f = [&](int ks) __attribute__((always_inline)) {
 #pragma unroll
                 for (int kb = 0; kb < KB; ++kb) {
@@ -3093,7 +3103,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
             auto load_v = [&](int db) __attribute__((always_inline)) {
                 vf[db][0] = *reinterpret_cast<const uintx4*>(st + voff + 16 * db * TL::V_ROW);
                 vf[db][1] = *reinterpret_cast<const uintx4*>(st + voff + 16 * db * TL::V_ROW + TL::V_PIECE);
-                vf[db][2] = *reinterpret_cast<const uintx4*>(st + voff + 16 * db * TL::V_ROW + 2 * TL::V_PIECE);
+                if (X3_VP == 3) vf[db][X3_VP - 1] = *reinterpret_cast<const uintx4*>(st + voff + 16 * db * TL::V_ROW + 2 * TL::V_PIECE);
             };
             // overlap of one feature step: all four piece products (exact product of the rounded features)
             // (consecutive MFMAs go to different accumulators: one that adds to the result of the one before it waits
@@ -3195,15 +3205,19 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
             if (interior) soft(std::false_type{}); else soft(std::true_type{});
             FLY_PROF2(stamp, 5);
             zp += ovs * wc;
-            // O^T[d][query] += sum_keys V[key][d] p[key][query]: P exactly in three pieces, six products
+            // O^T[d][query] += sum_keys V[key][d] p[key][query]: P exactly in three pieces, five or six products
+            // (P always in three exact pieces: its in-band low-rank part cancels against the global term, which is formed
+            //  in fp32.  V may be two: the key pass multiplies the same rounded V, so that cancellation is not touched.)
             uintx4 ph, pm, pl;
             split3(p[0], p[1], ph, pm, pl);
             if (!AHEAD) {
 #pragma unroll
                 for (int db = 0; db < DB; ++db) load_v(db);
             }
+            if (X3_VP == 3) {
 #pragma unroll
-            for (int db = 0; db < DB; ++db) oacc[db] = mma_bf16(vf[db][2], ph, oacc[db]);
+                for (int db = 0; db < DB; ++db) oacc[db] = mma_bf16(vf[db][X3_VP - 1], ph, oacc[db]);
+            }
 #pragma unroll
             for (int db = 0; db < DB; ++db) oacc[db] = mma_bf16(vf[db][0], pl, oacc[db]);
 #pragma unroll
@@ -4299,7 +4313,7 @@ SbWorkspace sb_workspace(int B, int H, int T, int S, int E, int mh, int local_co
     w.kv = take(bh * m * E * 4);
     w.ksum = take(bh * m * 4);
     w.kmax = take(bh * 4);
-    w.vt = take(dtype == F32 ? bh * nc * 2 * (128 * (size_t)E + 192 * (size_t)E) : bh * nc * CH * E * 2);
+    w.vt = take(dtype == F32 ? bh * nc * 2 * (128 * (size_t)E + 64 * (size_t)X3_VP * (size_t)E) : bh * nc * CH * E * 2);
     w.kvt = take(dtype == F32 ? 0 : bh * E * m * 2);
     w.part_ws = take(w.n_parts > 1 ? bh * n_qt * w.n_parts * TQ * (E + NSTAT) * 4 : 0);
     w.qfeat = take(w.n_parts > 1 ? bh * T * m * 4 : 0);

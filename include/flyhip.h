@@ -61,11 +61,11 @@ int flyhip_sb_plan(int B, int H, int T, int S, int local_context,
  * flyhip_sblocal_fwd -- V per 32-key tile and K'^T V, transposed into the operand order of the bf16
  * MFMA.
  * float inputs: vt may be NULL (all products on the fp32 matrix pipe, kfeat holds fp32 features).
- * With vt given -- B*H*n_chunks*2*(128*E + 192*D) bytes, 16-byte aligned -- the key pass writes
+ * With vt given -- B*H*n_chunks*2*(128*E + 192*D) bytes suffice, 16-byte aligned -- the key pass writes
  * per 32-key tile an image of K and V^T split into bfloat16 pieces there, and into kfeat (same
  * byte size as the fp32 features) an image of the features split into two pieces; passing the same
  * vt to flyhip_sblocal_fwd then runs the band on the bf16 matrix pipe with fp32-level accuracy
- * (features are rounded to 17 significant bits where they are formed).  kvt is unused for float. */
+ * (features are rounded to 17 significant bits where they are formed, V to 16 in both of its products).  kvt is unused for float. */
 int flyhip_sb_kv_reduce(const void* k, const void* v, const float* proj, const int64_t* key_lengths,
                         void* kfeat, float* chunk_scale, float* kv_part, float* part_max,
                         float* kv, float* ksum, float* kmax,
