@@ -134,24 +134,42 @@ class LocalAttention(nn.Module):
     """Softmax attention in which query i only sees keys j with
     -(local_context // 2) <= j - i < (local_context + 1) // 2.  Same constructor and forward signature
     as the reference class.  Covered on the GPU: no attn_mask, optional length-style key_padding_mask,
-    dropout inactive, need_weights=False; anything else raises NotImplementedError."""
+    dropout inactive; anything else raises NotImplementedError.  need_weights=True also returns the dense
+    (B,H,T,S) matrix (local_attention.py:94-106), exp(t q.k - lse) on the band with the kernel's own
+    log-denominators, as ordinary tensor algebra: an inspection path for problems of up to
+    max_weight_elements entries."""
 
     def __init__(self, local_context, softmax_temp=None, attention_dropout=0.0, device=None, dtype=None):
         super().__init__()
         self.local_context = local_context
         self.softmax_temp = softmax_temp
         self.dropout = nn.Dropout(attention_dropout)
+        self.max_weight_elements = 1 << 26
 
     def forward(self, query, key, value, attn_mask=None, key_padding_mask=None, need_weights=False):
         if attn_mask is not None and not bool(attn_mask.all_ones):
             raise NotImplementedError('attn_mask other than all-ones is not supported by the fused kernel')
-        if need_weights:
-            raise NotImplementedError('need_weights=True would materialise the (T,S) matrix; not supported')
         if self.training and self.dropout.p > 0.0:
             raise NotImplementedError('attention dropout is not implemented in the fused kernel')
         lengths = None
         if key_padding_mask is not None and not bool(key_padding_mask.all_ones):
             lengths = key_padding_mask.lengths
-        out = local_attention_fn(query, key, value, self.local_context, softmax_temp=self.softmax_temp,
-                                 key_lengths=lengths)
-        return out, None
+        if not need_weights:
+            out = local_attention_fn(query, key, value, self.local_context, softmax_temp=self.softmax_temp,
+                                     key_lengths=lengths)
+            return out, None
+        B, T, H, E = query.shape
+        S = key.shape[1]
+        if B * H * T * S > self.max_weight_elements:
+            raise NotImplementedError(f'need_weights=True materialises the (B,H,T,S) matrix: {B * H * T * S} entries '
+                                      f'exceed max_weight_elements = {self.max_weight_elements}')
+        out, lse = local_forward(query, key, value, self.local_context, softmax_temp=self.softmax_temp,
+                                 key_lengths=lengths, return_lse=True)
+        t = self.softmax_temp or 1 / math.sqrt(E)
+        scores = t * torch.einsum('bthe,bshe->bhts', query.float(), key.float())
+        idx = torch.arange(S, device=query.device).view(1, S) - torch.arange(T, device=query.device).view(T, 1)
+        band = ((idx >= -(self.local_context // 2)) & (idx < (self.local_context + 1) // 2)).view(1, 1, T, S)
+        if lengths is not None:
+            band = band & (torch.arange(S, device=query.device).view(1, 1, 1, S) < lengths.view(B, 1, 1, 1))
+        attn = torch.where(band, torch.exp(scores - lse.unsqueeze(-1)), scores.new_zeros(()))
+        return out, attn

@@ -8,7 +8,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from . import _lib
-from .feature_maps_sb import SBPerformerFeatures
+from .feature_maps_sb import SBPerformerFeatures, softmax_kernel
 
 _HEAD_DIMS = (32, 64, 128)       # padded head dims the kernels are instantiated for
 _FEATURE_ROWS = (16, 32, 64, 128)  # padded projection rows (m/2)
@@ -350,8 +350,10 @@ class SBLocalAttention(nn.Module):
 
     Same constructor and forward signature as the reference class (sblocal_attention.py:29-44).
     The GPU path covers what the reference itself exercises: non-causal, no attn_mask, optional
-    length-style key_padding_mask, softmax_eps = 0, dropout inactive, need_weights=False.  Any other
-    request raises NotImplementedError -- there is no slower fallback inside this module.
+    length-style key_padding_mask, softmax_eps = 0, dropout inactive.  ``need_weights`` /
+    ``return_attn_unnormalized`` (:124-136) give the dense matrix for small problems, formed with library products around
+    the fused kernels' ``log_normalization``; ``out`` always comes from the kernels.  Any other request raises
+    NotImplementedError -- there is no slower fallback inside this module.
     """
 
     def __init__(self, local_context, dim_heads, nb_features=None, ortho_scaling=0,
@@ -368,6 +370,8 @@ class SBLocalAttention(nn.Module):
         self.softmax_eps = softmax_eps
         # device scratch per problem shape and the padded projection, kept between calls (see sblocal_forward)
         self._scratch_cache = {}
+        # need_weights builds the dense (B,H,T,S) matrix with library products: an inspection aid, not a fast path
+        self.max_weight_elements = 1 << 26
 
     def forward(self, query, key, value, attn_mask=None, key_padding_mask=None, need_weights=False,
                 return_attn_unnormalized=False):
@@ -377,8 +381,10 @@ class SBLocalAttention(nn.Module):
                                       'marks it unverified, sblocal_attention.py:61)')
         if attn_mask is not None and not bool(attn_mask.all_ones):
             raise NotImplementedError('attn_mask other than all-ones is not supported by the fused kernel')
-        if need_weights or return_attn_unnormalized:
-            raise NotImplementedError('need_weights=True would materialise the (T,S) matrix; not supported')
+        if (need_weights or return_attn_unnormalized) and (
+                query.shape[0] * query.shape[2] * query.shape[1] * key.shape[1] > self.max_weight_elements):
+            raise NotImplementedError('need_weights=True materialises the (B,H,T,S) matrix; supported for inspection '
+                                      f'of small problems only (at most {self.max_weight_elements} elements)')
         if self.softmax_eps != 0.0:
             raise NotImplementedError('softmax_eps != 0 is not supported by the fused kernel')
         if self.training and self.dropout.p > 0.0:
@@ -391,4 +397,36 @@ class SBLocalAttention(nn.Module):
                                              self.local_context, softmax_temp=self.softmax_temp,
                                              key_lengths=lengths, cache=self._scratch_cache)
         self.last_log_normalization = log_norm.detach()
-        return out, None
+        attn = None
+        if need_weights or return_attn_unnormalized:
+            attn = self._dense_weights(query.detach(), key.detach(), lengths, log_norm.detach(),
+                                       return_attn_unnormalized)
+        return out, attn
+
+    def _dense_weights(self, query, key, lengths, log_norm, unnormalized):
+        """The (B,H,T,S) attention matrix the output corresponds to (sblocal_attention.py:124-136), for inspection of
+        small problems: exact weights exp(t q.k - log_normalization) inside the band, Performer weights
+        q'.k' exp(prime_log_scale - log_normalization) outside it, with ``log_normalization`` taken from the fused
+        kernels (nothing here feeds back into ``out``).  With ``unnormalized`` the reference's triple
+        (attn, attn * exp(log_normalization), attn_prime * exp(prime_log_scale))."""
+        B, T, H, E = query.shape
+        S = key.shape[1]
+        t = self.softmax_temp or 1 / math.sqrt(E)
+        q, k = query.permute(0, 2, 1, 3).float(), key.permute(0, 2, 1, 3).float()
+        P = self.feature_map.projection_matrix.float()
+        q_prime, q_ls = softmax_kernel(q, projection_matrix=P, is_query=True, softmax_temp=t)
+        k_prime, k_ls = softmax_kernel(k, projection_matrix=P, is_query=False, softmax_temp=t)
+        j = torch.arange(S, device=query.device)
+        valid = torch.ones(B, 1, 1, S, dtype=torch.bool, device=query.device) if lengths is None \
+            else (j.view(1, 1, 1, S) < lengths.view(B, 1, 1, 1))
+        k_prime = k_prime * valid.transpose(-1, -2)                        # :83-85
+        prime_log_scale = q_ls + k_ls                                      # (B,H,T,1)
+        ln = log_norm.float()                                              # (B,H,T,1)
+        attn_prime = q_prime @ k_prime.transpose(-1, -2)
+        idx = j.view(1, S) - torch.arange(T, device=query.device).view(T, 1)
+        band = ((idx >= -(self.local_context // 2)) & (idx < (self.local_context + 1) // 2)).view(1, 1, T, S) & valid
+        exact = torch.exp(t * (q @ k.transpose(-1, -2)) - ln)
+        attn = torch.where(band, exact, attn_prime * torch.exp(prime_log_scale - ln))
+        if not unnormalized:
+            return attn
+        return attn, attn * torch.exp(ln), attn_prime * torch.exp(prime_log_scale)

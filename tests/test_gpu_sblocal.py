@@ -137,8 +137,90 @@ def test_module_dropin():
     ref_out, ref_ln = osb.sblocal_attention(q.double(), k.double(), v.double(), P.double(), 64, key_lengths=lengths)
     assert rel_err(out, ref_out) <= 1e-4
     assert rel_err(attn.last_log_normalization, ref_ln) <= 1e-4
-    with pytest.raises(NotImplementedError):
+    attn.max_weight_elements = 1000
+    with pytest.raises(NotImplementedError):                          # the dense matrix is for small problems only
         attn(q.to(dev), k.to(dev), v.to(dev), need_weights=True)
+
+
+@pytest.mark.parametrize('lc,nb_features,t,out_tol', [(3, 73, None, 1e-3), (4, 26, 1.0, 1e-3), (28, 73, 0.235, 1e-3),
+                                                     (33, 26, None, 1e-2)])
+def test_attention_weights_satisfy_the_references_invariants(lc, nb_features, t, out_tol):
+    """need_weights / return_attn_unnormalized on the module (sblocal_attention.py:124-136) with the invariants of
+    the reference's own test (tests/models/attention/test_sblocal_attention.py:49-88) and its sizes: the rows of the
+    matrix sum to one (or zero), out = A v, the unnormalised matrix is exp(t q.k) inside the band and the low-rank
+    estimate outside it.  The reference's tolerances, but for out = A v in the last case: with 13 random features
+    and a band over nearly all keys the band's low-rank mass cancels against the global term in the linear-time
+    output (float32 run of the reference's own operations: up to 9e-4 of the maximum away from float64, see
+    test_fp32_odd_sizes_and_lengths), a cancellation the dense matrix does not have."""
+    from fly_amd import SBLocalAttention, LengthMask
+    dev = torch.device('cuda:0')
+    B, T, S, H, E, D = 18, 47, 39, 7, 21, 17
+    q, k, v, P = make_inputs(B, T, S, H, E, D, nb_features // 2, seed=2357, scale=1.0)
+    g = torch.Generator().manual_seed(5)
+    lengths = torch.randint(S // 4, S, (B,), generator=g)
+    mod = SBLocalAttention(lc, dim_heads=E, nb_features=nb_features, softmax_temp=t).to(dev).eval()
+    mod.feature_map.projection_matrix.copy_(P)
+    mod.feature_map.freeze_projection()
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    out, (A, A_un, A_lr) = mod(qd, kd, vd, key_padding_mask=LengthMask(lengths.to(dev), max_len=S), need_weights=True,
+                              return_attn_unnormalized=True)
+    assert out.shape == (B, T, H, D) and A.shape == (B, H, T, S)
+    assert bool((A >= 0).all())
+    rows = A.sum(-1)
+    assert bool((torch.isclose(rows, torch.ones_like(rows), atol=1e-2) | torch.isclose(rows, torch.zeros_like(rows), atol=1e-2)).all())
+    assert torch.allclose(out, torch.einsum('bhts,bshd->bthd', A, vd), rtol=out_tol, atol=out_tol)
+    temp = 1 / math.sqrt(E) if t is None else t
+    full = torch.exp(torch.einsum('bthe,bshe->bhts', qd * temp, kd))
+    j = torch.arange(S, device=dev)
+    keyok = (j.view(1, 1, 1, S) < lengths.to(dev).view(B, 1, 1, 1))
+    full = full * keyok
+    idx = j.view(1, S) - torch.arange(T, device=dev).view(T, 1)
+    local = ((idx >= -(lc // 2)) & (idx < (lc + 1) // 2)).view(1, 1, T, S) & keyok
+    local = local.expand(B, H, T, S)
+    assert torch.allclose(A_un[local], full[local], rtol=1e-3, atol=1e-4)
+    assert torch.allclose(A_un[~local], A_lr[~local], rtol=1e-3, atol=1e-4)
+    # and the plain call gives the same output
+    out2, none = mod(qd, kd, vd, key_padding_mask=LengthMask(lengths.to(dev), max_len=S))
+    assert none is None and torch.equal(out, out2)
+
+
+@pytest.mark.parametrize('lc', [3, 4, 28, 33])
+@pytest.mark.parametrize('t', [None, 1.0, 0.235])
+def test_local_attention_weights_satisfy_the_references_invariants(lc, t):
+    """need_weights of LocalAttention (local_attention.py:94-106) with the invariants and sizes of the reference's
+    test (tests/models/attention/test_local_attention.py:48-100): rows sum to one or zero, at most local_context
+    entries per row, out = A v, and A is full softmax attention with the entries outside the band set to zero and
+    the rows renormalised.  Key lengths start at zero as there."""
+    from fly_amd import LocalAttention, LengthMask
+    dev = torch.device('cuda:0')
+    B, T, S, H, E, D = 18, 47, 39, 7, 21, 17
+    q, k, v, _ = make_inputs(B, T, S, H, E, D, 4, seed=2357, scale=1.0)
+    g = torch.Generator().manual_seed(7)
+    lengths = torch.randint(0, S, (B,), generator=g).to(dev)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    mod = LocalAttention(lc, softmax_temp=t).to(dev).eval()
+    out, A = mod(qd, kd, vd, None, LengthMask(lengths, max_len=S), need_weights=True)
+    assert out.shape == (B, T, H, D) and A.shape == (B, H, T, S)
+    assert bool((A >= 0).all())
+    rows = A.sum(-1)
+    assert bool((torch.isclose(rows, torch.ones_like(rows), atol=1e-5) | torch.isclose(rows, torch.zeros_like(rows))).all())
+    assert bool(((A >= 1e-6).sum(-1) <= lc).all())
+    assert torch.allclose(out, torch.einsum('bhts,bshd->bthd', A, vd), rtol=1e-5, atol=1e-5)
+    temp = 1 / math.sqrt(E) if t is None else t
+    scores = temp * torch.einsum('bthe,bshe->bhts', qd, kd)
+    j = torch.arange(S, device=dev)
+    scores = scores.masked_fill(~(j.view(1, 1, 1, S) < lengths.view(B, 1, 1, 1)), -math.inf)
+    A_full = torch.softmax(scores, dim=-1).nan_to_num(0.0)
+    idx = j.view(1, S) - torch.arange(T, device=dev).view(T, 1)
+    local = ((idx >= -(lc // 2)) & (idx < (lc + 1) // 2)).view(1, 1, T, S)
+    A_sel = A_full.masked_fill(~local, 0.0)
+    A_sel = A_sel / A_sel.sum(-1, keepdim=True).clamp_min(1e-30)
+    assert torch.allclose(A, A_sel, rtol=1e-4, atol=1e-6)
+    out2, none = mod(qd, kd, vd, None, LengthMask(lengths, max_len=S))
+    assert none is None and torch.equal(out, out2)
+    mod.max_weight_elements = 1000
+    with pytest.raises(NotImplementedError):
+        mod(qd, kd, vd, None, LengthMask(lengths, max_len=S), need_weights=True)
 
 
 def test_module_keeps_its_scratch_between_calls():
