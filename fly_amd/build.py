@@ -8,7 +8,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, 'csrc')
 LIB = os.path.join(HERE, 'libflyhip.so')
-SOURCES = ['api.cpp', 'sblocal.hip', 'blocksparse.hip']
+SOURCES = ['api.cpp', 'sblocal.hip', 'sblocal_prep.hip', 'blocksparse.hip']
 # packed-fp32 VALU forms are switched off for every kernel of this library; MFMA accumulators stay in
 # ordinary VGPRs (the softmax arithmetic reads them between products, and every trip through the
 # accumulation registers costs a move per value)

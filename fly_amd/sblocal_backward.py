@@ -125,25 +125,30 @@ def _fit_features(x, mk):
     return torch.cat([torch.nn.functional.pad(x[..., :mh], pad), torch.nn.functional.pad(x[..., mh:], pad)], dim=-1)
 
 
-def _backward_hip(Q, K, V, G, psi, phik, LN, c, P, lens_b, H, local_context, t, dims):
-    """d query, d key, d value (BH, rows, width) on two launches of flyhip_sblocal_bwd: the small
-    per-head reductions over all keys / all queries are library products, everything per (query, key)
-    pair and per row runs in the kernels."""
+def _backward_hip(Q, K, V, G, O, LN, P, lens_b, H, local_context, t, dims):
+    """d query, d key, d value (BH, rows, width) in five launches: flyhip_sblocal_bwd_prep (scaled features of
+    queries and keys, c = g . out, and the per-head sums over all keys / all queries) and the two passes of
+    flyhip_sblocal_bwd (everything per (query, key) pair, the low-rank epilogue, the chain rule through the
+    feature map)."""
     from . import _lib
     BH, T, E = Q.shape
     S, D = K.shape[1], V.shape[2]
     dim, mk = dims
-    q_, k_, v_, g_ = _fit(Q, dim), _fit(K, dim), _fit(V, dim), _fit(G, dim)
-    psi_, phik_ = _fit_features(psi, mk), _fit_features(phik, mk)
-    proj = _fit(torch.nn.functional.pad(P, (0, 0, 0, mk // 2 - P.shape[0])), dim)
-    ln_, c_ = LN.reshape(BH, T).contiguous(), c.reshape(BH, T).contiguous()
-    kv = (phik_.transpose(1, 2) @ v_).contiguous()           # (BH, mk, dim)   sum_s phik_s v_s^T
-    ksum = phik_.sum(1)                                      # (BH, mk)
-    qg = (psi_.transpose(1, 2) @ g_).contiguous()            # (BH, mk, dim)   sum_i psi_i g_i^T
-    qc = torch.einsum('btm,bt->bm', psi_, c_).contiguous()   # (BH, mk)
-    dq, dk, dv = Q.new_empty(BH, T, dim), Q.new_empty(BH, S, dim), Q.new_empty(BH, S, dim)
+    q_, k_, v_, g_, o_ = _fit(Q, dim), _fit(K, dim), _fit(V, dim), _fit(G, dim), _fit(O, dim)
+    mh = P.shape[0]
+    proj = _fit(torch.nn.functional.pad(P, (0, 0, 0, mk // 2 - mh)), dim)
+    ln_ = LN.reshape(BH, T).contiguous()
+    new = Q.new_empty
+    psi_, phik_, c_ = new(BH, T, mk), new(BH, S, mk), new(BH, T)
+    kv, ksum, qg, qc = new(BH, mk, dim), new(BH, mk), new(BH, mk, dim), new(BH, mk)
+    scratch = new(_lib.load().flyhip_sblocal_bwd_prep_scratch(BH, T, S, dim, mk))
+    dq, dk, dv = new(BH, T, dim), new(BH, S, dim), new(BH, S, dim)
     with torch.cuda.device(Q.device):
         st = _lib.stream_ptr(Q.device)
+        _lib.call('flyhip_sblocal_bwd_prep', q_.data_ptr(), k_.data_ptr(), v_.data_ptr(), g_.data_ptr(), o_.data_ptr(),
+                  ln_.data_ptr(), proj.data_ptr(), _lib.ptr(lens_b), psi_.data_ptr(), phik_.data_ptr(), c_.data_ptr(),
+                  kv.data_ptr(), ksum.data_ptr(), qg.data_ptr(), qc.data_ptr(), scratch.data_ptr(), scratch.numel(),
+                  BH, H, T, S, dim, mk, mh, float(t), st)
         _lib.call('flyhip_sblocal_bwd', q_.data_ptr(), psi_.data_ptr(), g_.data_ptr(), k_.data_ptr(), phik_.data_ptr(),
                   v_.data_ptr(), ln_.data_ptr(), c_.data_ptr(), _lib.ptr(lens_b), kv.data_ptr(), ksum.data_ptr(),
                   proj.data_ptr(), dq.data_ptr(), None, BH, H, T, S, dim, mk, local_context, float(t), 0, st)
@@ -240,9 +245,9 @@ def sblocal_backward(query, key, value, projection_matrix, local_context, softma
     log_normalization (B,H,T,1) as returned by the forward; key_lengths (B,) or None.
     max_elements bounds the
     size of the (batch, chunks, chunk, window) intermediates: chunks are taken in groups that stay below it.
-    band_kernel: None = the fused kernels where they apply (GPU, head dims <= 64, <= 128 features): band
-    sums, global low-rank terms and the feature-map chain rule in two launches; 'sums' = only the band
-    sums on the kernels; False = batched library products; True = the kernels or NotImplementedError.
+    band_kernel: None = the fused kernels where they apply (GPU, head dims <= 64, <= 128 features): the
+    feature maps and per-head sums in three launches, then band sums, global low-rank terms and the feature-map
+    chain rule in two; 'sums' = only the band sums on the kernels, the rest as tensor algebra; False = batched library products; True = the kernels or NotImplementedError.
     Returns (d query, d key, d value) in the dtypes of the inputs."""
     B, T, H, E = query.shape
     S, D = key.shape[1], value.shape[3]
@@ -260,18 +265,17 @@ def sblocal_backward(query, key, value, projection_matrix, local_context, softma
     lens = None
     if key_lengths is not None:
         lens = key_lengths.to(Q.device).repeat_interleave(H).view(B * H, 1, 1)
-    psi, phik = _scaled_features(Q, K, P, t, LN, lens)
-    c = (G * O).sum(-1, keepdim=True)
-
     dims = _band_kernel_dims(E, D, 2 * mh) if band_kernel is not False else None
     if band_kernel and dims is None:
         raise NotImplementedError(f'no band kernel for head dims ({E}, {D}) with {2 * mh} features')
     on_kernels = dims is not None and Q.is_cuda and wdt == torch.float32
     lens_b = None if key_lengths is None else key_lengths.to(device=Q.device, dtype=torch.int64).contiguous()
     if on_kernels and band_kernel != 'sums':
-        # everything after the features on the two passes of the fused kernel
-        dQ, dK, dV = _backward_hip(Q, K, V, G, psi, phik, LN, c, P, lens_b, H, local_context, t, dims)
+        # features, per-head sums and the two passes of the fused kernel
+        dQ, dK, dV = _backward_hip(Q, K, V, G, O, LN, P, lens_b, H, local_context, t, dims)
     else:
+        psi, phik = _scaled_features(Q, K, P, t, LN, lens)
+        c = (G * O).sum(-1, keepdim=True)
         kv = phik.transpose(1, 2) @ V                # (BH, m, D)   sum_s phik_s v_s^T
         ksum = phik.sum(1)                           # (BH, m)
         qg = psi.transpose(1, 2) @ G                 # (BH, m, D)   sum_i psi_i g_i^T

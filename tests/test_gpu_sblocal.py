@@ -402,6 +402,59 @@ def test_backward_band_kernels_match_library_products(B, T, S, H, E, D, mh, lc, 
             assert rel_err(a, b) <= 1e-4, (mode, rel_err(a, b))
 
 
+@pytest.mark.parametrize('BH,H,T,S,dim,mk,mh,lens', [(4, 2, 300, 280, 64, 64, 32, [280, 200]),
+                                                     (3, 3, 257, 391, 64, 64, 24, None),
+                                                     (2, 1, 130, 135, 32, 32, 16, [135, 1]),
+                                                     (2, 1, 70, 600, 32, 64, 20, [0, 600]),
+                                                     (2, 2, 100, 64, 64, 32, 9, [33]),
+                                                     (2, 1, 3136, 3136, 64, 128, 64, None)])
+def test_backward_preparation_kernels_match_tensor_algebra(BH, H, T, S, dim, mk, mh, lens):
+    """flyhip_sblocal_bwd_prep (scaled features of queries and keys, c = g . out, the four per-head sums) against
+    the same quantities as ordinary tensor algebra (sblocal_backward._scaled_features and library products, which
+    the gradient tests check against autograd through the oracle): ragged lengths, a batch entry without any key,
+    fewer projection rows than the kernel's feature width, and BASELINE config 1's size."""
+    from fly_amd import _lib
+    from fly_amd.sblocal_backward import _scaled_features
+    print('case', BH, H, T, S, dim, mk, mh, lens, flush=True)
+    dev = torch.device('cuda:0')
+    g = torch.Generator().manual_seed(11)
+    Q = (torch.randn(BH, T, dim, generator=g) * dim ** -0.25).to(dev)
+    K = (torch.randn(BH, S, dim, generator=g) * dim ** -0.25).to(dev)
+    V, G, O = (torch.randn(BH, n, dim, generator=g).to(dev) for n in (S, T, T))
+    LN = torch.randn(BH, T, 1, generator=g).to(dev)
+    P = osb.gaussian_orthogonal_random_matrix(mh, dim, generator=g).to(dev)
+    t = 0.9 * dim ** -0.5
+    kl = None if lens is None else torch.tensor(lens, device=dev)
+    lens_bh = None if kl is None else kl.repeat_interleave(H).view(BH, 1, 1)
+    psi, phik = _scaled_features(Q, K, P, t, LN, lens_bh)
+    c = (G * O).sum(-1)
+    ref = dict(c=c, kv=phik.transpose(1, 2) @ V, ksum=phik.sum(1), qg=psi.transpose(1, 2) @ G,
+               qc=torch.einsum('btm,bt->bm', psi, c))
+    new = Q.new_empty
+    got = dict(psi=new(BH, T, mk), phik=new(BH, S, mk), c=new(BH, T), kv=new(BH, mk, dim), ksum=new(BH, mk),
+               qg=new(BH, mk, dim), qc=new(BH, mk))
+    proj = torch.zeros(mk // 2, dim, device=dev)
+    proj[:mh] = P
+    scratch = new(_lib.load().flyhip_sblocal_bwd_prep_scratch(BH, T, S, dim, mk))
+    _lib.call('flyhip_sblocal_bwd_prep', Q.data_ptr(), K.data_ptr(), V.data_ptr(), G.data_ptr(), O.data_ptr(),
+              LN.data_ptr(), proj.data_ptr(), _lib.ptr(kl), *(got[n].data_ptr() for n in ('psi', 'phik', 'c', 'kv', 'ksum', 'qg', 'qc')),
+              scratch.data_ptr(), scratch.numel(), BH, H, T, S, dim, mk, mh, t, _lib.stream_ptr(dev))
+    torch.cuda.synchronize()
+
+    def unpad(x, axis):                            # (.., mk, ..) -> (.., 2 mh, ..)
+        lo, hi = x.narrow(axis, 0, mh), x.narrow(axis, mk // 2, mh)
+        rest = torch.cat([x.narrow(axis, mh, mk // 2 - mh), x.narrow(axis, mk // 2 + mh, mk // 2 - mh)], axis)
+        assert rest.numel() == 0 or float(rest.abs().max()) == 0.0
+        return torch.cat([lo, hi], axis)
+    assert rel_err(unpad(got['psi'], 2), psi) <= 1e-5
+    assert rel_err(unpad(got['phik'], 2), phik) <= 1e-5
+    assert torch.allclose(unpad(got['psi'], 2), psi, rtol=1e-4, atol=0)
+    assert torch.allclose(unpad(got['phik'], 2), phik, rtol=1e-4, atol=0)
+    assert rel_err(got['c'], ref['c']) <= 1e-5
+    for name in ('kv', 'ksum', 'qg', 'qc'):
+        assert rel_err(unpad(got[name], 1), ref[name]) <= 2e-5, name
+
+
 def test_random_shapes_sweep():
     """Forty seeded random problems (ragged T != S, head dims that need padding, odd and even windows up
     to wider than the sequence, feature counts from 2 to 256, key lengths down to one key, one to three
