@@ -246,4 +246,52 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
+// ---- operands as sums of bf16 pieces (float inputs on the bf16 matrix pipe) ----
+// one 16x16x32 step on the bf16 matrix pipe: eight k-slots per lane on either side
+__device__ __forceinline__ floatx4 mma_bf16(uint4 a, uint4 b, floatx4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+__device__ __forceinline__ floatx4 mma_bf16(uintx4 a, uintx4 b, floatx4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+
+// chunk c of a row -> the chunk it is stored at
+__device__ __forceinline__ int x3_swz(int row, int c, int row_bytes) {
+    return row_bytes >= 128 ? (c ^ (row & 7)) : (c ^ ((row >> 1) & 3));
+}
+// an fp32 value rounded to 17 significant bits (its bf16 head and the bf16 head of the rest then add up to it exactly)
+__device__ __forceinline__ float quant16(float x) {
+    // (finite x; ties away from zero.  17 significant bits split exactly: the head is rounded to nearest, so the rest is
+    //  at most half a unit of its last place, and its sign carries the ninth bit)
+    return __uint_as_float((__float_as_uint(x) + 0x40u) & 0xffffff80u);
+}
+__device__ __forceinline__ floatx4 quant16(floatx4 x) {
+    floatx4 r = {quant16(x[0]), quant16(x[1]), quant16(x[2]), quant16(x[3])};
+    return r;
+}
+// eight floats -> bf16 head and remainder (eight k-slots each)
+__device__ __forceinline__ void split2(floatx4 x0, floatx4 x1, uintx4& hi, uintx4& lo) {
+    hi = uintx4{pack_bf16x2(x0[0], x0[1]), pack_bf16x2(x0[2], x0[3]), pack_bf16x2(x1[0], x1[1]), pack_bf16x2(x1[2], x1[3])};
+    floatx4 r0, r1;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t w0 = hi[i >> 1], w1 = hi[2 + (i >> 1)];
+        r0[i] = x0[i] - ((i & 1) ? __uint_as_float(w0 & 0xffff0000u) : __uint_as_float(w0 << 16));
+        r1[i] = x1[i] - ((i & 1) ? __uint_as_float(w1 & 0xffff0000u) : __uint_as_float(w1 << 16));
+    }
+    lo = uintx4{pack_bf16x2(r0[0], r0[1]), pack_bf16x2(r0[2], r0[3]), pack_bf16x2(r1[0], r1[1]), pack_bf16x2(r1[2], r1[3])};
+}
+// eight floats -> three bf16 pieces whose sum is the value exactly
+__device__ __forceinline__ void split3(floatx4 x0, floatx4 x1, uintx4& h, uintx4& m, uintx4& l) {
+    h = uintx4{pack_bf16x2(x0[0], x0[1]), pack_bf16x2(x0[2], x0[3]), pack_bf16x2(x1[0], x1[1]), pack_bf16x2(x1[2], x1[3])};
+    floatx4 r0, r1;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t w0 = h[i >> 1], w1 = h[2 + (i >> 1)];
+        r0[i] = x0[i] - ((i & 1) ? __uint_as_float(w0 & 0xffff0000u) : __uint_as_float(w0 << 16));
+        r1[i] = x1[i] - ((i & 1) ? __uint_as_float(w1 & 0xffff0000u) : __uint_as_float(w1 << 16));
+    }
+    split2(r0, r1, m, l);
+}
+
 }  // namespace flyhip

@@ -27,12 +27,62 @@ struct PrepArgs {
     float* kv; float* ksum; float* qg; float* qc;       // (BH, MK, DIM), (BH, MK) twice
     float* pmax;                     // (BH, n_kblk)
     float* part;                     // (BH, n_split_k + n_split_q, MK * (DIM + 1))
+    char* qimg; char* kimg;          // tile images for the band kernels on the bf16 matrix pipe (BwdTile), or null
     int BH, H, T, S, mh_valid, n_kblk, n_split_k, n_split_q;
     float temp;
 };
 
 constexpr int PREP_ROWS = 64;        // rows per step of a workgroup: 16 per wave
 constexpr int PREP_NT = 256;
+
+// four floats -> bf16 head and rest, four k-slots each
+__device__ __forceinline__ void split2_4(floatx4 x, uint2& hi, uint2& lo) {
+    hi = make_uint2(pack_bf16x2(x[0], x[1]), pack_bf16x2(x[2], x[3]));
+    const floatx4 r = {x[0] - __uint_as_float(hi.x << 16), x[1] - __uint_as_float(hi.x & 0xffff0000u),
+                       x[2] - __uint_as_float(hi.y << 16), x[3] - __uint_as_float(hi.y & 0xffff0000u)};
+    lo = make_uint2(pack_bf16x2(r[0], r[1]), pack_bf16x2(r[2], r[3]));
+}
+
+// 64 rows x W floats in LDS (row stride LD floats) -> their NP-piece images in the two 32-row tiles at `tile0` and
+// `tile0 + tile_stride`: chunk c of a row = elements 8c .. 8c + 7, 16 bytes per piece
+template <int W, int LD, int NP>
+__device__ __forceinline__ void prep_emit_rows(const float* src, char* tile0, long tile_stride, int piece_bytes, int tid) {
+    constexpr int CH8 = W / 8, ROWB = 2 * W, TOT = 64 * CH8;
+#pragma unroll
+    for (int j = 0; j < (TOT + 255) / 256; ++j) {
+        const int idx = tid + 256 * j;
+        if (TOT % 256 == 0 || idx < TOT) {
+            const int row64 = idx / CH8, ch = idx % CH8, row = row64 & 31;
+            const float* sp = src + row64 * LD + 8 * ch;
+            uintx4 h, m, l;
+            if (NP == 3) split3(*reinterpret_cast<const floatx4*>(sp), *reinterpret_cast<const floatx4*>(sp + 4), h, m, l);
+            else split2(*reinterpret_cast<const floatx4*>(sp), *reinterpret_cast<const floatx4*>(sp + 4), h, m);
+            char* dst = tile0 + (row64 >> 5) * tile_stride + row * ROWB + x3_swz(row, ch, ROWB) * 16;
+            *reinterpret_cast<uintx4*>(dst) = h;
+            *reinterpret_cast<uintx4*>(dst + piece_bytes) = m;
+            if (NP == 3) *reinterpret_cast<uintx4*>(dst + 2 * piece_bytes) = l;
+        }
+    }
+}
+
+// Image of 32 rows of one side (queries: q, g, psi; keys: k, v, phik) for the band kernels on the bf16 matrix
+// pipe: every operand as two bf16 pieces (head and rest: 16 to 17 significant bits; the features are rounded to
+// 17 bits first, so their pieces are exact), elements of a row in their natural order (both operands of every
+// product come from images, so lane g's eight k-slots of a 32-wide MFMA step are simply elements 8g .. 8g + 7 of
+// it), 16-byte chunks XOR-swizzled (x3_swz) so that fragment reads of neighbouring rows fall into different LDS
+// banks -- the row reads of the score products and the transposed reads of the output products alike.  One image is one LDS stage of the band
+// kernel, copied linearly:  [x hi][x lo][y h][y m][y l][features hi][features lo][log2(e) log Z of the 32 rows][c].
+// y (the values, resp. d out) comes in three pieces, exact to fp32: df = g.v - g.out is a difference of nearly
+// equal numbers wherever one key carries a query's whole weight.
+template <int DIM, int MK>
+struct BwdTile {
+    static constexpr int ROWS = 32;
+    static constexpr int X_ROW = 2 * DIM, F_ROW = 2 * MK;                       // bytes per row of a piece
+    static constexpr int X_PIECE = ROWS * X_ROW, F_PIECE = ROWS * F_ROW;
+    static constexpr int X_OFF = 0, Y_OFF = 2 * X_PIECE, F_OFF = 5 * X_PIECE, S_OFF = F_OFF + 2 * F_PIECE;
+    static constexpr int MAIN = S_OFF, BYTES = S_OFF + 2 * ROWS * 4;
+    static_assert(MAIN % 1024 == 0, "whole wave loads of 16 bytes per lane");
+};
 
 // sqrt(t) P x for the 16 rows of a wave.  prep_load: lane (r16, g) takes elements 16 c + 4 g .. + 3 of input row
 // r16 of the wave; prep_project returns in dd[fb][i] the projection of that row on row 16 fb + 4 g + i of P, and
@@ -112,7 +162,8 @@ __global__ __launch_bounds__(PREP_NT) void sb_prep_kernel(PrepArgs a) {
     const int rows = key_role ? a.S : a.T;
     const int len = key_role ? (a.lens ? min((int)a.lens[b], a.S) : a.S) : a.T;
     const float* X = (key_role ? a.k : a.q) + (long)bh * rows * DIM;
-    float* F = (key_role ? a.phik : a.psi) + (long)bh * rows * MK;
+    float* F = key_role ? a.phik : a.psi;        // may be null: only the images are wanted
+    if (F) F += (long)bh * rows * MK;
 
     // kappa: the maximum over the key blocks of pass 1 (0 when no key is valid)
     float kappa = -INFINITY;
@@ -193,6 +244,31 @@ __global__ __launch_bounds__(PREP_NT) void sb_prep_kernel(PrepArgs a) {
         const int row = base + 16 * w + r16;
         const bool valid = row < len;
         const float wrow = key_role ? 1.f : crow[16 * w + r16];
+        using TL = BwdTile<DIM, MK>;
+        char* img = key_role ? a.kimg : a.qimg;
+        const int trow = (16 * w + r16) & 31;     // this lane's row inside its 32-row tile
+        char* img0 = nullptr;                     // the chunk's first tile
+        if (img) {
+            img0 = img + ((long)bh * 2 * n_chunks + 2 * c) * TL::BYTES;
+            img = img0 + (w >> 1) * TL::BYTES;
+            // x of the lane's row: its elements 16 cc + 4 g .. + 3 are half g % 2 of chunk 2 cc + g / 2
+#pragma unroll
+            for (int cc = 0; cc < DIM / 16; ++cc) {
+                const int at = x3_swz(trow, 2 * cc + (g >> 1), TL::X_ROW) * 16 + 8 * (g & 1);
+                char* dst = img + TL::X_OFF + trow * TL::X_ROW + at;
+                uint2 p0, p1;
+                split2_4(xb[cc], p0, p1);
+                *reinterpret_cast<uint2*>(dst) = p0;
+                *reinterpret_cast<uint2*>(dst + TL::X_PIECE) = p1;
+            }
+            // y rows from their LDS copy, 16 bytes per piece and thread
+            prep_emit_rows<DIM, LDY, 3>(Ys, img0 + TL::Y_OFF, TL::BYTES, TL::X_PIECE, tid);
+            if (g == 0) {
+                float* tr = reinterpret_cast<float*>(img + TL::S_OFF);
+                tr[trow] = key_role ? 0.f : ln_row * 1.4426950408889634f;
+                tr[32 + trow] = wrow;
+            }
+        }
         floatx4 dd[FB];
         float sq;
         prep_project<DIM, FB>(xb, a.proj, st, r16, g, dd, sq);
@@ -201,7 +277,7 @@ __global__ __launch_bounds__(PREP_NT) void sb_prep_kernel(PrepArgs a) {
         else bias = kappa - ln_row - 0.5f * a.temp * sq - off;
         __syncthreads();                          // every c of this chunk has been read
         float* frow_s = Fs + (16 * w + r16) * LDF;
-        float* frow_g = F + (long)row * MK;
+        floatx4 fblk[2 * FB];                     // the row's features: blocks of 16, [exp(+.) | exp(-.)]
 #pragma unroll
         for (int fb = 0; fb < FB; ++fb) {
             floatx4 fp, fn;
@@ -211,16 +287,21 @@ __global__ __launch_bounds__(PREP_NT) void sb_prep_kernel(PrepArgs a) {
                 fp[i] = ok ? expf(dd[fb][i] + bias) : 0.f;
                 fn[i] = ok ? expf(bias - dd[fb][i]) : 0.f;
             }
+            if (img) { fp = quant16(fp); fn = quant16(fn); }     // every use sees the features rounded to 17 bits
             sp_[fb] += fp * wrow;
             sn_[fb] += fn * wrow;
             *reinterpret_cast<floatx4*>(frow_s + 16 * fb + 4 * g) = fp;
             *reinterpret_cast<floatx4*>(frow_s + MH + 16 * fb + 4 * g) = fn;
-            if (row < rows) {
-                *reinterpret_cast<floatx4*>(frow_g + 16 * fb + 4 * g) = fp;
-                *reinterpret_cast<floatx4*>(frow_g + MH + 16 * fb + 4 * g) = fn;
-            }
+            fblk[fb] = fp;
+            fblk[FB + fb] = fn;
+        }
+        if (F && row < rows) {
+            float* frow_g = F + (long)row * MK;
+#pragma unroll
+            for (int fb = 0; fb < 2 * FB; ++fb) *reinterpret_cast<floatx4*>(frow_g + 16 * fb + 4 * g) = fblk[fb];
         }
         __syncthreads();
+        if (img) prep_emit_rows<MK, LDF, 2>(Fs, img0 + TL::F_OFF, TL::BYTES, TL::F_PIECE, tid);
         // acc[r][d] += sum_rows F[row][r] Y[row][d]; lane ends with element (16 rb + 4g + i, 16 db + r16)
 #pragma unroll
         for (int kk = 0; kk < PREP_ROWS / 16; ++kk) {
@@ -304,6 +385,358 @@ __global__ __launch_bounds__(PREP_NT) void sb_prep_reduce_kernel(PrepArgs a) {
     *dst = s;
 }
 
+// ---------------------------------------------------------------------------------------
+// band terms of the backward pass on the bf16 matrix pipe
+// ---------------------------------------------------------------------------------------
+// The arithmetic of sblocal_bwd_band_kernel (pair weights a = exp(t q.k - log Z), kb = psi.phik, df = g.v - c,
+// dm = a df; five band-limited sums; the finishing epilogue with the per-head matrices and the chain rule through
+// the feature map), with every product on v_mfma_f32_16x16x32_bf16 from operands in two bf16 pieces and fp32
+// accumulation: three piece products for q.k and two of the output sums (the rest-times-rest product, 2^-16
+// relative, is dropped); six for g.v from three pieces each (exact to fp32: df = g.v - c cancels where one key carries
+// a query's weight) and five for phik^T df with df in three pieces; all four for psi.phik, whose operands are exact in two pieces -- the band's low-rank
+// weight then cancels against the per-head sums, which the preparation pass forms from the same rounded features.
+// The inner side comes as the images of BwdTile, one image = one LDS stage, copied by loads that write LDS
+// directly; the outer side's operands are read once from the images of its own rows.  The output products need
+// the inner rows transposed (k = inner row): ds_read_b64_tr_b16 delivers that from the row-major pieces -- 16
+// lanes pass the addresses of 4 rows x 4 groups of 4 columns and receive, lane l, column l of the 4 rows -- so
+// no transposed copy exists anywhere.
+struct BwdX3Args {
+    const char* oimg; const char* iimg;        // images of the outer and of the inner side
+    const float* x1; const float* x3;          // the outer rows themselves (BH, Lo, E), for the epilogue
+    const float* ln; const float* c;           // (BH, T)
+    const int64_t* lens;
+    float* o1; float* o3;                      // d x1 (BH, Lo, E); d v (BH, S, E), key-major only
+    int BH, H, T, S, lc;
+    float temp;
+    const float* gmat; const float* gvec; const float* proj;
+    int n_xcd;
+};
+
+typedef short shortx4 __attribute__((ext_vector_type(4)));
+typedef short shortx8 __attribute__((ext_vector_type(8)));
+// eight k-slots (inner rows) of one column: two transposed reads of 4 rows each
+__device__ __forceinline__ uintx4 lds_read_tr8(const char* p0, const char* p1) {
+    typedef __attribute__((address_space(3))) shortx4* lds_ptr;
+    const shortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)p0);
+    const shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)p1);
+    return __builtin_bit_cast(uintx4, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+}
+
+// one tile image, global memory -> LDS stage `dst` (linear; each wave load writes 1024 consecutive bytes); TAIL: also
+// the 256 bytes behind the MAIN ones (log Z and c of the tile's queries; a full wave load, lanes 16.. repeat them)
+template <int MAIN, bool TAIL>
+__device__ __forceinline__ void bwd_tile_to_lds(const char* src, char* dst, int tid) {
+    typedef __attribute__((address_space(3))) void* lds_ptr;
+    const int w = tid >> 6, lane = tid & 63;
+#pragma unroll
+    for (int j = 0; j < MAIN / 4096; ++j)
+        __builtin_amdgcn_global_load_lds(src + 4096 * j + 16 * tid, (lds_ptr)(dst + 4096 * j + 1024 * w), 16, 0, 0);
+    constexpr int FULL = MAIN / 4096 * 4096;
+    if (MAIN % 4096 != 0 && w < (MAIN % 4096) / 1024)
+        __builtin_amdgcn_global_load_lds(src + FULL + 16 * tid, (lds_ptr)(dst + FULL + 1024 * w), 16, 0, 0);
+    if (TAIL && w == 0)
+        __builtin_amdgcn_global_load_lds(src + MAIN + 16 * (lane & 15), (lds_ptr)(dst + MAIN), 16, 0, 0);
+}
+
+template <int E, int M, bool KEYMAJOR>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void sblocal_bwd_x3_kernel(BwdX3Args a) {
+    using TL = BwdTile<E, M>;
+    constexpr int NT = 256, TQ = 64, TK = 32, KB = 2;
+    constexpr int D = E, KS1 = E / 32, KS2 = M / 32, EC = E / 16, FC = M / 16, DB = D / 16, MH = M / 2;
+    constexpr int STAGE = TL::MAIN + 1024;                 // the image and a full wave load for its 256-byte tail
+    constexpr int LDK = E + 4, LDV = D + 4;                // epilogue operands, floats per row
+    constexpr float LOG2E = 1.4426950408889634f;
+    static_assert((M * LDV + M + MH * LDK) * 4 <= 2 * STAGE, "epilogue operands must fit the tile stages");
+    extern __shared__ __attribute__((aligned(256))) char smem[];
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
+    const int Lo = KEYMAJOR ? a.S : a.T, Li = KEYMAJOR ? a.T : a.S;
+    const int n_ot = (Lo + TQ - 1) / TQ;
+    const int n_items = a.BH * n_ot;
+    const int per_xcd = (n_items + a.n_xcd - 1) / a.n_xcd;
+    const int item = (blockIdx.x % a.n_xcd) * per_xcd + blockIdx.x / a.n_xcd;   // neighbouring tiles share a die's L2
+    if (item >= n_items) return;                           // workgroup-uniform
+    const int ot = item % n_ot, bh = item / n_ot, b = bh / a.H;
+    const int o0 = ot * TQ, ow0 = o0 + 16 * w, o = ow0 + r16;
+    const int len = a.lens ? min((int)a.lens[b], a.S) : a.S;
+    const int lc_lo = a.lc / 2, lc_hi = (a.lc + 1) / 2;    // band: -lc_lo <= s - i < lc_hi
+    const int lo = KEYMAJOR ? -(lc_hi - 1) : -lc_lo, hi = KEYMAJOR ? lc_lo + 1 : lc_hi;     // seen from the outer row
+    const int o_limit = KEYMAJOR ? len : a.T, n_limit = KEYMAJOR ? a.T : len;
+    const bool ovalid = o < o_limit;
+    const int n_oimg = 2 * ((Lo + 63) / 64), n_iimg = 2 * ((Li + 63) / 64);
+    const char* itiles = a.iimg + (long)bh * n_iimg * TL::BYTES;
+
+    const int o_last = min(o0 + TQ - 1, o_limit - 1);
+    const int n_lo = max(0, o0 + lo), n_hi = min(n_limit, o_last + hi);
+    const int kt_lo = n_lo / TK;
+    const int kt_hi = (o_last >= o0 && n_hi > n_lo) ? (n_hi + TK - 1) / TK : kt_lo;
+
+    if (kt_lo < kt_hi) bwd_tile_to_lds<TL::MAIN, KEYMAJOR>(itiles + (long)kt_lo * TL::BYTES, smem, tid);
+
+    // outer operands (B side: column = outer row, k-slots 8g .. 8g + 7 of every 32-wide step) from the row's image
+    const int orow = min(o, Lo - 1), trow = orow & 31;
+    const char* otile = a.oimg + ((long)bh * n_oimg + (orow >> 5)) * TL::BYTES;
+    uintx4 x1h[KS1], x1l[KS1], x3h[KS1], x3m[KS1], x3l[KS1], x2h[KEYMAJOR ? KS2 : 1], x2l[KEYMAJOR ? KS2 : 1];
+#pragma unroll
+    for (int ks = 0; ks < KS1; ++ks) {
+        const int off = trow * TL::X_ROW + x3_swz(trow, 4 * ks + g, TL::X_ROW) * 16;
+        x1h[ks] = *reinterpret_cast<const uintx4*>(otile + TL::X_OFF + off);
+        x1l[ks] = *reinterpret_cast<const uintx4*>(otile + TL::X_OFF + TL::X_PIECE + off);
+        x3h[ks] = *reinterpret_cast<const uintx4*>(otile + TL::Y_OFF + off);
+        x3m[ks] = *reinterpret_cast<const uintx4*>(otile + TL::Y_OFF + TL::X_PIECE + off);
+        x3l[ks] = *reinterpret_cast<const uintx4*>(otile + TL::Y_OFF + 2 * TL::X_PIECE + off);
+    }
+    if (KEYMAJOR) {
+#pragma unroll
+        for (int ks = 0; ks < KS2; ++ks) {
+            const int off = trow * TL::F_ROW + x3_swz(trow, 4 * ks + g, TL::F_ROW) * 16;
+            x2h[ks] = *reinterpret_cast<const uintx4*>(otile + TL::F_OFF + off);
+            x2l[ks] = *reinterpret_cast<const uintx4*>(otile + TL::F_OFF + TL::F_PIECE + off);
+        }
+    }
+    const float ln_o = KEYMAJOR ? 0.f : a.ln[(long)bh * a.T + orow] * LOG2E, c_o = KEYMAJOR ? 0.f : a.c[(long)bh * a.T + orow];
+    const float sc = a.temp * LOG2E;                       // scores leave the MFMA unscaled; exponents are base 2
+    // inner rows this lane's outer row may meet: nmin <= n < nmin + span
+    const int nmin = max(o + lo, 0);
+    const unsigned span = ovalid ? (unsigned)max(min(o + hi, n_limit) - nmin, 0) : 0u;
+
+    floatx4 acc1[EC], acc2[FC], acc3[KEYMAJOR ? DB : 1];
+#pragma unroll
+    for (int c = 0; c < EC; ++c) acc1[c] = Frag<float>::zero();
+#pragma unroll
+    for (int c = 0; c < FC; ++c) acc2[c] = Frag<float>::zero();
+#pragma unroll
+    for (int c = 0; c < (KEYMAJOR ? DB : 1); ++c) acc3[c] = Frag<float>::zero();
+
+    // transposed reads: this lane passes the address of row 4g + r16/4 (and 16 rows further), columns 4 (r16 % 4) .. + 3
+    // of the 16-column block (half (r16 % 4) % 2 of chunk 2c + (r16 % 4) / 2); it receives column r16 of rows
+    // 4g .. 4g + 3 (16 + 4g ..): the k-slots of its weights
+    const int tr_row = 4 * g + (r16 >> 2), tr_cb = r16 & 3;
+
+    drain_loads();
+    __syncthreads();
+
+    for (int kt = kt_lo; kt < kt_hi; ++kt) {
+        const int n_base = kt * TK;
+        const int cur = (kt - kt_lo) & 1;
+        const char* st = smem + cur * STAGE;
+        if (kt + 1 < kt_hi)                                // every wave is past the barrier that ended that stage's last use
+            bwd_tile_to_lds<TL::MAIN, KEYMAJOR>(itiles + (long)(kt + 1) * TL::BYTES, smem + (cur ^ 1) * STAGE, tid);
+
+        // wave-uniform: does this tile meet the band of any of the wave's 16 outer rows?
+        const bool any = !(n_base + TK - 1 - ow0 < lo || n_base - (ow0 + 15) >= hi || n_base >= n_limit || ow0 >= o_limit);
+        if (any) {
+            floatx4 s1[KB], s2[KB], s3[KB];
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) { s1[kb] = Frag<float>::zero(); s2[kb] = Frag<float>::zero(); s3[kb] = Frag<float>::zero(); }
+#pragma unroll
+            for (int ks = 0; ks < KS1; ++ks)
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb) {
+                    const int row = 16 * kb + r16;
+                    const char* p = st + row * TL::X_ROW + x3_swz(row, 4 * ks + g, TL::X_ROW) * 16;
+                    const uintx4 yh = *reinterpret_cast<const uintx4*>(p + TL::X_OFF), yl = *reinterpret_cast<const uintx4*>(p + TL::X_OFF + TL::X_PIECE);
+                    const uintx4 vh = *reinterpret_cast<const uintx4*>(p + TL::Y_OFF), vm = *reinterpret_cast<const uintx4*>(p + TL::Y_OFF + TL::X_PIECE);
+                    const uintx4 vl = *reinterpret_cast<const uintx4*>(p + TL::Y_OFF + 2 * TL::X_PIECE);
+                    s1[kb] = mma_bf16(yl, x1h[ks], s1[kb]);
+                    s3[kb] = mma_bf16(vl, x3h[ks], s3[kb]);
+                    s1[kb] = mma_bf16(yh, x1l[ks], s1[kb]);
+                    s3[kb] = mma_bf16(vh, x3l[ks], s3[kb]);
+                    s1[kb] = mma_bf16(yh, x1h[ks], s1[kb]);
+                    s3[kb] = mma_bf16(vm, x3m[ks], s3[kb]);
+                    s3[kb] = mma_bf16(vm, x3h[ks], s3[kb]);
+                    s3[kb] = mma_bf16(vh, x3m[ks], s3[kb]);
+                    s3[kb] = mma_bf16(vh, x3h[ks], s3[kb]);
+                }
+            if (KEYMAJOR) {
+#pragma unroll
+                for (int ks = 0; ks < KS2; ++ks)
+#pragma unroll
+                    for (int kb = 0; kb < KB; ++kb) {
+                        const int row = 16 * kb + r16;
+                        const char* p = st + TL::F_OFF + row * TL::F_ROW + x3_swz(row, 4 * ks + g, TL::F_ROW) * 16;
+                        const uintx4 fh = *reinterpret_cast<const uintx4*>(p), fl = *reinterpret_cast<const uintx4*>(p + TL::F_PIECE);
+                        s2[kb] = mma_bf16(fl, x2l[ks], s2[kb]);
+                        s2[kb] = mma_bf16(fl, x2h[ks], s2[kb]);
+                        s2[kb] = mma_bf16(fh, x2l[ks], s2[kb]);
+                        s2[kb] = mma_bf16(fh, x2h[ks], s2[kb]);
+                    }
+            }
+            // lane holds the pair (outer row o, inner row n_base + 16kb + 4g + i)
+            floatx4 wdm[KB], wdf[KB], wak[KB];
+            const float* Ss = reinterpret_cast<const float*>(st + TL::S_OFF);
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) {
+                floatx4 lnq, cq;
+                if (KEYMAJOR) {
+                    lnq = *reinterpret_cast<const floatx4*>(Ss + 16 * kb + 4 * g);
+                    cq = *reinterpret_cast<const floatx4*>(Ss + TK + 16 * kb + 4 * g);
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int n = n_base + 16 * kb + 4 * g + i;
+                    const bool ok = (unsigned)(n - nmin) < span;
+                    const float av = ok ? __builtin_amdgcn_exp2f(s1[kb][i] * sc - (KEYMAJOR ? lnq[i] : ln_o)) : 0.f;
+                    const float df = ok ? s3[kb][i] - (KEYMAJOR ? cq[i] : c_o) : 0.f;
+                    wdm[kb][i] = av * df;
+                    wdf[kb][i] = df;
+                    wak[kb][i] = av - (ok ? s2[kb][i] : 0.f);
+                }
+            }
+            uintx4 dmh, dml, dfh, dfm, dfl, akh, akl;
+            split2(wdm[0], wdm[1], dmh, dml);
+            split3(wdf[0], wdf[1], dfh, dfm, dfl);
+            if (KEYMAJOR) split2(wak[0], wak[1], akh, akl);
+            // out^T[col][outer] += sum_inner Y[inner][col] w[inner][outer]
+#pragma unroll
+            for (int c = 0; c < EC; ++c) {
+                const char* p = st + tr_row * TL::X_ROW + x3_swz(tr_row, 2 * c + (tr_cb >> 1), TL::X_ROW) * 16 + 8 * (tr_cb & 1);
+                const uintx4 yh = lds_read_tr8(p + TL::X_OFF, p + TL::X_OFF + 16 * TL::X_ROW);
+                const uintx4 yl = lds_read_tr8(p + TL::X_OFF + TL::X_PIECE, p + TL::X_OFF + TL::X_PIECE + 16 * TL::X_ROW);
+                acc1[c] = mma_bf16(yl, dmh, acc1[c]);
+                acc1[c] = mma_bf16(yh, dml, acc1[c]);
+                acc1[c] = mma_bf16(yh, dmh, acc1[c]);
+                if (KEYMAJOR) {
+                    const uintx4 vh = lds_read_tr8(p + TL::Y_OFF, p + TL::Y_OFF + 16 * TL::X_ROW);
+                    const uintx4 vl = lds_read_tr8(p + TL::Y_OFF + TL::X_PIECE, p + TL::Y_OFF + TL::X_PIECE + 16 * TL::X_ROW);       // (the middle piece)
+                    acc3[c] = mma_bf16(vl, akh, acc3[c]);
+                    acc3[c] = mma_bf16(vh, akl, acc3[c]);
+                    acc3[c] = mma_bf16(vh, akh, acc3[c]);
+                }
+            }
+#pragma unroll
+            for (int c = 0; c < FC; ++c) {
+                const char* p = st + TL::F_OFF + tr_row * TL::F_ROW + x3_swz(tr_row, 2 * c + (tr_cb >> 1), TL::F_ROW) * 16 + 8 * (tr_cb & 1);
+                const uintx4 fh = lds_read_tr8(p, p + 16 * TL::F_ROW);
+                const uintx4 fl = lds_read_tr8(p + TL::F_PIECE, p + TL::F_PIECE + 16 * TL::F_ROW);
+                acc2[c] = mma_bf16(fl, dfm, acc2[c]);
+                acc2[c] = mma_bf16(fh, dfl, acc2[c]);
+                acc2[c] = mma_bf16(fl, dfh, acc2[c]);
+                acc2[c] = mma_bf16(fh, dfm, acc2[c]);
+                acc2[c] = mma_bf16(fh, dfh, acc2[c]);
+            }
+        }
+        drain_loads();                                     // this wave's share of the next tile is in LDS
+        __syncthreads();
+    }
+
+    // ---- epilogue: per-head matrices into the tile stages (dead now; the loop ended on a barrier) ----
+    float* GMs = reinterpret_cast<float*>(smem);           // gmat (M, D), rows of LDV
+    float* GVs = GMs + M * LDV;                            // gvec (M)
+    float* Ps = GVs + M;                                   // projection (M/2, E), rows of LDK
+    for (int idx = tid; idx < M * (D / 4); idx += NT) {
+        const int r = idx / (D / 4), c4 = idx % (D / 4);
+        *reinterpret_cast<floatx4*>(GMs + r * LDV + 4 * c4) = *reinterpret_cast<const floatx4*>(a.gmat + ((long)bh * M + r) * D + 4 * c4);
+    }
+    for (int idx = tid; idx < MH * (E / 4); idx += NT) {
+        const int r = idx / (E / 4), c4 = idx % (E / 4);
+        *reinterpret_cast<floatx4*>(Ps + r * LDK + 4 * c4) = *reinterpret_cast<const floatx4*>(a.proj + (long)r * E + 4 * c4);
+    }
+    if (tid < M) GVs[tid] = a.gvec[(long)bh * M + tid];
+    // the outer row itself in fp32 (x1, x3) and its features from their two pieces (exact)
+    floatx4 x1[EC], x3[DB], x2[FC];
+#pragma unroll
+    for (int c = 0; c < EC; ++c) x1[c] = load4_f32(a.x1 + ((long)bh * Lo + orow) * E + 16 * c + 4 * g);
+#pragma unroll
+    for (int c = 0; c < DB; ++c) x3[c] = load4_f32(a.x3 + ((long)bh * Lo + orow) * D + 16 * c + 4 * g);
+#pragma unroll
+    for (int c = 0; c < FC; ++c) {
+        const char* p = otile + TL::F_OFF + trow * TL::F_ROW + x3_swz(trow, 2 * c + (g >> 1), TL::F_ROW) * 16 + 8 * (g & 1);
+        const uint2 fh = *reinterpret_cast<const uint2*>(p), fl = *reinterpret_cast<const uint2*>(p + TL::F_PIECE);
+        x2[c][0] = __uint_as_float(fh.x << 16) + __uint_as_float(fl.x << 16);
+        x2[c][1] = __uint_as_float(fh.x & 0xffff0000u) + __uint_as_float(fl.x & 0xffff0000u);
+        x2[c][2] = __uint_as_float(fh.y << 16) + __uint_as_float(fl.y << 16);
+        x2[c][3] = __uint_as_float(fh.y & 0xffff0000u) + __uint_as_float(fl.y & 0xffff0000u);
+    }
+    __syncthreads();
+    // u^T[f][outer] = sum_d gmat[f][d] x3[d][outer]
+    floatx4 u[FC];
+#pragma unroll
+    for (int c = 0; c < FC; ++c) u[c] = Frag<float>::zero();
+#pragma unroll
+    for (int cd = 0; cd < DB; ++cd) {
+        floatx4 ga[FC];
+#pragma unroll
+        for (int c = 0; c < FC; ++c) ga[c] = *reinterpret_cast<const floatx4*>(GMs + (16 * c + r16) * LDV + 16 * cd + 4 * g);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int c = 0; c < FC; ++c) u[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(ga[c][j], x3[cd][j], u[c], 0, 0, 0);
+    }
+    const float cmul = KEYMAJOR ? 1.0f : c_o;
+    float usum = 0.f;
+#pragma unroll
+    for (int c = 0; c < FC; ++c) {
+        const floatx4 gv = *reinterpret_cast<const floatx4*>(GVs + 16 * c + 4 * g);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            u[c][i] = x2[c][i] * (u[c][i] - cmul * gv[i] - acc2[c][i]);
+            usum += u[c][i];
+        }
+    }
+    usum = group_sum(usum);
+    // chain rule through the projection: dp^T[e][outer] = sum_r P[r][e] (u_r - u_{r + M/2})
+    floatx4 dp[EC];
+#pragma unroll
+    for (int c = 0; c < EC; ++c) dp[c] = Frag<float>::zero();
+#pragma unroll
+    for (int c = 0; c < FC / 2; ++c) {
+        const floatx4 du = u[c] - u[c + FC / 2];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int eb = 0; eb < EC; ++eb)
+                dp[eb] = __builtin_amdgcn_mfma_f32_16x16x4f32(Ps[(16 * c + 4 * g + j) * LDK + 16 * eb + r16], du[j], dp[eb], 0, 0, 0);
+    }
+    if (KEYMAJOR) {
+        // d v^T[d][key] += sum_f gmat[f][d] phik[f][key]
+#pragma unroll
+        for (int c = 0; c < FC; ++c)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+                    acc3[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(GMs[(16 * c + 4 * g + j) * LDV + 16 * db + r16], x2[c][j], acc3[db], 0, 0, 0);
+    }
+    if (o < Lo) {
+        const float st_ = sqrtf(a.temp);
+        float* p1 = a.o1 + ((long)bh * Lo + o) * E;
+#pragma unroll
+        for (int c = 0; c < EC; ++c) store4_f32(p1 + 16 * c + 4 * g, acc1[c] * a.temp + dp[c] * st_ - x1[c] * (a.temp * usum));
+        if (KEYMAJOR) {
+            float* p3 = a.o3 + ((long)bh * Lo + o) * D;
+#pragma unroll
+            for (int c = 0; c < DB; ++c) store4_f32(p3 + 16 * c + 4 * g, acc3[c]);
+        }
+    }
+}
+
+// (explicit instantiations: the host stubs of this template are not emitted otherwise)
+#define FLY_BWD_X3_INST(EE, MM) \
+    template __global__ void sblocal_bwd_x3_kernel<EE, MM, false>(BwdX3Args); \
+    template __global__ void sblocal_bwd_x3_kernel<EE, MM, true>(BwdX3Args);
+FLY_BWD_X3_INST(32, 32) FLY_BWD_X3_INST(32, 64) FLY_BWD_X3_INST(64, 32) FLY_BWD_X3_INST(64, 64) FLY_BWD_X3_INST(64, 128)
+#undef FLY_BWD_X3_INST
+
+template <int E, int M, bool KEYMAJOR>
+static int launch_bwd_x3(const BwdX3Args& a, hipStream_t st) {
+    auto kern = sblocal_bwd_x3_kernel<E, M, KEYMAJOR>;
+    constexpr size_t smem = 2 * (BwdTile<E, M>::MAIN + 1024);
+    static std::atomic<unsigned long long> lds_set{0};     // (devices on which this kernel has its LDS limit)
+    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_set, "sblocal_bwd_x3")) return rc;
+    const Machine& mach = machine();
+    const long items = (long)a.BH * (((KEYMAJOR ? a.S : a.T) + 63) / 64);
+    const long grid = (items + mach.xcds - 1) / mach.xcds * mach.xcds;
+    if (grid > 2147483647L) return fail(ERR_ARG, "sblocal_bwd_x3: too many workgroups");
+    BwdX3Args args = a;
+    args.n_xcd = mach.xcds;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), smem, st, args);
+    return check_launch("sblocal_bwd_x3_kernel");
+}
+template <int E, int M>
+static int launch_bwd_x3_both(const BwdX3Args& a, bool key_major, hipStream_t st) {
+    return key_major ? launch_bwd_x3<E, M, true>(a, st) : launch_bwd_x3<E, M, false>(a, st);
+}
+
 static void prep_splits(int BH, int T, int S, int& n_kblk, int& n_split_k, int& n_split_q) {
     const int kc = (S + PREP_ROWS - 1) / PREP_ROWS, qc = (T + PREP_ROWS - 1) / PREP_ROWS;
     const int want = std::max(1, (machine().slots + 2 * BH - 1) / (2 * BH));       // workgroups per role and (batch, head)
@@ -332,23 +765,34 @@ extern "C" int64_t flyhip_sblocal_bwd_prep_scratch(int BH, int T, int S, int E, 
     return (long)BH * n_kblk + (long)BH * (nk + nq) * M * (E + 1);
 }
 
+extern "C" int64_t flyhip_sblocal_bwd_image_bytes(int BH, int rows, int E, int M) {
+    if (BH <= 0 || rows <= 0 || E <= 0 || M <= 0) return -1;
+    const int64_t tile = 32 * (10 * (int64_t)E + 4 * (int64_t)M) + 256;       // BwdTile<E, M>::BYTES
+    return (int64_t)BH * 2 * ((rows + PREP_ROWS - 1) / PREP_ROWS) * tile;
+}
+
 extern "C" int flyhip_sblocal_bwd_prep(const float* q, const float* k, const float* v, const float* grad_out,
                                        const float* out, const float* log_norm, const float* proj,
                                        const int64_t* key_lengths,
                                        float* psi, float* phik, float* c,
                                        float* kv, float* ksum, float* qg, float* qc,
+                                       void* q_images, void* k_images,
                                        float* scratch, int64_t scratch_floats,
                                        int BH, int H, int T, int S, int E, int M, int mh_valid,
                                        float softmax_temp, void* stream) {
-    FLY_REQUIRE(q && k && v && grad_out && out && log_norm && proj && psi && phik && c && kv && ksum && qg && qc && scratch,
+    FLY_REQUIRE(q && k && v && grad_out && out && log_norm && proj && c && kv && ksum && qg && qc && scratch,
                 "sblocal_bwd_prep: null pointer");
+    FLY_REQUIRE((psi && phik) || (q_images && k_images), "sblocal_bwd_prep: neither feature arrays nor images asked for");
+    FLY_REQUIRE(!psi == !phik && !q_images == !k_images, "sblocal_bwd_prep: psi / phik and the two image buffers come in pairs");
     FLY_REQUIRE(BH > 0 && H > 0 && BH % H == 0 && T > 0 && S > 0, "sblocal_bwd_prep: empty or inconsistent problem");
     FLY_REQUIRE(softmax_temp > 0.f, "sblocal_bwd_prep: softmax_temp must be positive");
     FLY_REQUIRE(mh_valid >= 1 && 2 * mh_valid <= M, "sblocal_bwd_prep: %d projection rows do not fit %d features", mh_valid, M);
     const int64_t need = flyhip_sblocal_bwd_prep_scratch(BH, T, S, E, M);
     FLY_REQUIRE(scratch_floats >= need, "sblocal_bwd_prep: scratch of %lld floats, %lld needed", (long long)scratch_floats, (long long)need);
     PrepArgs a{q, k, v, grad_out, out, log_norm, proj, key_lengths, psi, phik, c, kv, ksum, qg, qc,
-               scratch, scratch + (long)BH * ((S + PREP_ROWS - 1) / PREP_ROWS), BH, H, T, S, mh_valid, 0, 0, 0, softmax_temp};
+               scratch, scratch + (long)BH * ((S + PREP_ROWS - 1) / PREP_ROWS),
+               reinterpret_cast<char*>(q_images), reinterpret_cast<char*>(k_images),
+               BH, H, T, S, mh_valid, 0, 0, 0, softmax_temp};
     prep_splits(BH, T, S, a.n_kblk, a.n_split_k, a.n_split_q);
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     if (E == 32 && M == 32) return launch_prep<32, 32>(a, st);
@@ -357,5 +801,30 @@ extern "C" int flyhip_sblocal_bwd_prep(const float* q, const float* k, const flo
     if (E == 64 && M == 64) return launch_prep<64, 64>(a, st);
     if (E == 64 && M == 128) return launch_prep<64, 128>(a, st);
     return fail(ERR_UNSUPPORTED, "sblocal_bwd_prep: (head dim, features) = (%d, %d) not in "
+                                 "{(32,32), (32,64), (64,32), (64,64), (64,128)}", E, M);
+}
+
+extern "C" int flyhip_sblocal_bwd_pieces(const void* outer_images, const void* inner_images,
+                                         const float* x1, const float* x3,
+                                         const float* log_norm, const float* c, const int64_t* key_lengths,
+                                         const float* gmat, const float* gvec, const float* proj,
+                                         float* d1, float* d3,
+                                         int BH, int H, int T, int S, int E, int M, int local_context,
+                                         float softmax_temp, int key_major, void* stream) {
+    FLY_REQUIRE(outer_images && inner_images && x1 && x3 && log_norm && c && gmat && gvec && proj && d1,
+                "sblocal_bwd_pieces: null pointer");
+    FLY_REQUIRE(!key_major || d3, "sblocal_bwd_pieces: the key-major pass needs d3");
+    FLY_REQUIRE(BH > 0 && H > 0 && BH % H == 0 && T > 0 && S > 0, "sblocal_bwd_pieces: empty or inconsistent problem");
+    FLY_REQUIRE(local_context >= 1, "sblocal_bwd_pieces: local_context must be >= 1");
+    FLY_REQUIRE(softmax_temp > 0.f, "sblocal_bwd_pieces: softmax_temp must be positive");
+    BwdX3Args a{reinterpret_cast<const char*>(outer_images), reinterpret_cast<const char*>(inner_images), x1, x3,
+                log_norm, c, key_lengths, d1, d3, BH, H, T, S, local_context, softmax_temp, gmat, gvec, proj, 0};
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (E == 32 && M == 32) return launch_bwd_x3_both<32, 32>(a, key_major != 0, st);
+    if (E == 32 && M == 64) return launch_bwd_x3_both<32, 64>(a, key_major != 0, st);
+    if (E == 64 && M == 32) return launch_bwd_x3_both<64, 32>(a, key_major != 0, st);
+    if (E == 64 && M == 64) return launch_bwd_x3_both<64, 64>(a, key_major != 0, st);
+    if (E == 64 && M == 128) return launch_bwd_x3_both<64, 128>(a, key_major != 0, st);
+    return fail(ERR_UNSUPPORTED, "sblocal_bwd_pieces: (head dim, features) = (%d, %d) not in "
                                  "{(32,32), (32,64), (64,32), (64,64), (64,128)}", E, M);
 }

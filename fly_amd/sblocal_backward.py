@@ -125,11 +125,13 @@ def _fit_features(x, mk):
     return torch.cat([torch.nn.functional.pad(x[..., :mh], pad), torch.nn.functional.pad(x[..., mh:], pad)], dim=-1)
 
 
-def _backward_hip(Q, K, V, G, O, LN, P, lens_b, H, local_context, t, dims):
+def _backward_hip(Q, K, V, G, O, LN, P, lens_b, H, local_context, t, dims, pieces=True):
     """d query, d key, d value (BH, rows, width) in five launches: flyhip_sblocal_bwd_prep (scaled features of
-    queries and keys, c = g . out, and the per-head sums over all keys / all queries) and the two passes of
-    flyhip_sblocal_bwd (everything per (query, key) pair, the low-rank epilogue, the chain rule through the
-    feature map)."""
+    queries and keys, c = g . out, and the per-head sums over all keys / all queries) and the two passes of the
+    band kernel (everything per (query, key) pair, the low-rank epilogue, the chain rule through the feature map).
+    pieces: the band kernel on the bf16 matrix pipe from operands in two bf16 pieces (flyhip_sblocal_bwd_pieces;
+    the preparation pass leaves every 32 rows of either side as one image of such operands), else on the fp32
+    matrix pipe from the float arrays (flyhip_sblocal_bwd)."""
     from . import _lib
     BH, T, E = Q.shape
     S, D = K.shape[1], V.shape[2]
@@ -139,22 +141,37 @@ def _backward_hip(Q, K, V, G, O, LN, P, lens_b, H, local_context, t, dims):
     proj = _fit(torch.nn.functional.pad(P, (0, 0, 0, mk // 2 - mh)), dim)
     ln_ = LN.reshape(BH, T).contiguous()
     new = Q.new_empty
-    psi_, phik_, c_ = new(BH, T, mk), new(BH, S, mk), new(BH, T)
+    lib = _lib.load()
+    psi_ = phik_ = qimg = kimg = None
+    if pieces:
+        qimg = torch.empty(lib.flyhip_sblocal_bwd_image_bytes(BH, T, dim, mk), dtype=torch.uint8, device=Q.device)
+        kimg = torch.empty(lib.flyhip_sblocal_bwd_image_bytes(BH, S, dim, mk), dtype=torch.uint8, device=Q.device)
+    else:
+        psi_, phik_ = new(BH, T, mk), new(BH, S, mk)
+    c_ = new(BH, T)
     kv, ksum, qg, qc = new(BH, mk, dim), new(BH, mk), new(BH, mk, dim), new(BH, mk)
-    scratch = new(_lib.load().flyhip_sblocal_bwd_prep_scratch(BH, T, S, dim, mk))
+    scratch = new(lib.flyhip_sblocal_bwd_prep_scratch(BH, T, S, dim, mk))
     dq, dk, dv = new(BH, T, dim), new(BH, S, dim), new(BH, S, dim)
     with torch.cuda.device(Q.device):
         st = _lib.stream_ptr(Q.device)
         _lib.call('flyhip_sblocal_bwd_prep', q_.data_ptr(), k_.data_ptr(), v_.data_ptr(), g_.data_ptr(), o_.data_ptr(),
-                  ln_.data_ptr(), proj.data_ptr(), _lib.ptr(lens_b), psi_.data_ptr(), phik_.data_ptr(), c_.data_ptr(),
-                  kv.data_ptr(), ksum.data_ptr(), qg.data_ptr(), qc.data_ptr(), scratch.data_ptr(), scratch.numel(),
-                  BH, H, T, S, dim, mk, mh, float(t), st)
-        _lib.call('flyhip_sblocal_bwd', q_.data_ptr(), psi_.data_ptr(), g_.data_ptr(), k_.data_ptr(), phik_.data_ptr(),
-                  v_.data_ptr(), ln_.data_ptr(), c_.data_ptr(), _lib.ptr(lens_b), kv.data_ptr(), ksum.data_ptr(),
-                  proj.data_ptr(), dq.data_ptr(), None, BH, H, T, S, dim, mk, local_context, float(t), 0, st)
-        _lib.call('flyhip_sblocal_bwd', k_.data_ptr(), phik_.data_ptr(), v_.data_ptr(), q_.data_ptr(), psi_.data_ptr(),
-                  g_.data_ptr(), ln_.data_ptr(), c_.data_ptr(), _lib.ptr(lens_b), qg.data_ptr(), qc.data_ptr(),
-                  proj.data_ptr(), dk.data_ptr(), dv.data_ptr(), BH, H, T, S, dim, mk, local_context, float(t), 1, st)
+                  ln_.data_ptr(), proj.data_ptr(), _lib.ptr(lens_b), _lib.ptr(psi_), _lib.ptr(phik_), c_.data_ptr(),
+                  kv.data_ptr(), ksum.data_ptr(), qg.data_ptr(), qc.data_ptr(), _lib.ptr(qimg), _lib.ptr(kimg),
+                  scratch.data_ptr(), scratch.numel(), BH, H, T, S, dim, mk, mh, float(t), st)
+        if pieces:
+            _lib.call('flyhip_sblocal_bwd_pieces', qimg.data_ptr(), kimg.data_ptr(), q_.data_ptr(), g_.data_ptr(),
+                      ln_.data_ptr(), c_.data_ptr(), _lib.ptr(lens_b), kv.data_ptr(), ksum.data_ptr(), proj.data_ptr(),
+                      dq.data_ptr(), None, BH, H, T, S, dim, mk, local_context, float(t), 0, st)
+            _lib.call('flyhip_sblocal_bwd_pieces', kimg.data_ptr(), qimg.data_ptr(), k_.data_ptr(), v_.data_ptr(),
+                      ln_.data_ptr(), c_.data_ptr(), _lib.ptr(lens_b), qg.data_ptr(), qc.data_ptr(), proj.data_ptr(),
+                      dk.data_ptr(), dv.data_ptr(), BH, H, T, S, dim, mk, local_context, float(t), 1, st)
+        else:
+            _lib.call('flyhip_sblocal_bwd', q_.data_ptr(), psi_.data_ptr(), g_.data_ptr(), k_.data_ptr(), phik_.data_ptr(),
+                      v_.data_ptr(), ln_.data_ptr(), c_.data_ptr(), _lib.ptr(lens_b), kv.data_ptr(), ksum.data_ptr(),
+                      proj.data_ptr(), dq.data_ptr(), None, BH, H, T, S, dim, mk, local_context, float(t), 0, st)
+            _lib.call('flyhip_sblocal_bwd', k_.data_ptr(), phik_.data_ptr(), v_.data_ptr(), q_.data_ptr(), psi_.data_ptr(),
+                      g_.data_ptr(), ln_.data_ptr(), c_.data_ptr(), _lib.ptr(lens_b), qg.data_ptr(), qc.data_ptr(),
+                      proj.data_ptr(), dk.data_ptr(), dv.data_ptr(), BH, H, T, S, dim, mk, local_context, float(t), 1, st)
     return dq[..., :E], dk[..., :E], dv[..., :D]
 
 
@@ -247,7 +264,9 @@ def sblocal_backward(query, key, value, projection_matrix, local_context, softma
     size of the (batch, chunks, chunk, window) intermediates: chunks are taken in groups that stay below it.
     band_kernel: None = the fused kernels where they apply (GPU, head dims <= 64, <= 128 features): the
     feature maps and per-head sums in three launches, then band sums, global low-rank terms and the feature-map
-    chain rule in two; 'sums' = only the band sums on the kernels, the rest as tensor algebra; False = batched library products; True = the kernels or NotImplementedError.
+    chain rule in two, on the bf16 matrix pipe from operands in two bf16 pieces; 'fp32' = the same five launches
+    with the band kernel on the fp32 matrix pipe; 'sums' = only the band sums on the kernels, the rest as tensor
+    algebra; False = batched library products; True = the kernels or NotImplementedError.
     Returns (d query, d key, d value) in the dtypes of the inputs."""
     B, T, H, E = query.shape
     S, D = key.shape[1], value.shape[3]
@@ -272,7 +291,8 @@ def sblocal_backward(query, key, value, projection_matrix, local_context, softma
     lens_b = None if key_lengths is None else key_lengths.to(device=Q.device, dtype=torch.int64).contiguous()
     if on_kernels and band_kernel != 'sums':
         # features, per-head sums and the two passes of the fused kernel
-        dQ, dK, dV = _backward_hip(Q, K, V, G, O, LN, P, lens_b, H, local_context, t, dims)
+        dQ, dK, dV = _backward_hip(Q, K, V, G, O, LN, P, lens_b, H, local_context, t, dims,
+                                   pieces=band_kernel != 'fp32')
     else:
         psi, phik = _scaled_features(Q, K, P, t, LN, lens)
         c = (G * O).sum(-1, keepdim=True)

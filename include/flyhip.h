@@ -181,24 +181,43 @@ int flyhip_sblocal_bwd(const float* x1, const float* x2, const float* x3,
                        int BH, int H, int T, int S, int E, int M, int local_context,
                        float softmax_temp, int key_major, void* stream);
 
-/* Everything the two flyhip_sblocal_bwd calls need besides q, k, v and d out, in three launches (the reference
+/* Everything the two band passes of the backward need besides q, k, v and d out, in three launches (the reference
  * gets it from autograd through softmax_kernel, src/models/attention/feature_maps_sb.py:51-82, and the sums of
  * src/models/attention/sblocal_attention.py:76-80).  Inputs packed float32: q, grad_out, out (BH,T,E), k, v
  * (BH,S,E), log_norm (BH,T), proj (M/2,E) with rows >= mh_valid zero, key_lengths (BH / H) int64 or NULL.
  * Outputs: psi (BH,T,M) = Phi(q) exp(kappa - log_norm), phik (BH,S,M) = Phi(k) exp(-kappa), zero at and past the
  * key length, each row [exp(+.) | exp(-.)] in halves of M/2 with features >= mh_valid zero; kappa = the largest
  * log-feature of a valid key of the (batch, head); c (BH,T) = grad_out . out; kv (BH,M,E) = phik^T v,
- * ksum (BH,M) = sum phik, qg (BH,M,E) = psi^T grad_out, qc (BH,M) = psi^T c.  scratch: at least
- * flyhip_sblocal_bwd_prep_scratch(BH,T,S,E,M) floats.  (E, M) as for flyhip_sblocal_bwd. */
+ * ksum (BH,M) = sum phik, qg (BH,M,E) = psi^T grad_out, qc (BH,M) = psi^T c.
+ * q_images, k_images (both or neither; flyhip_sblocal_bwd_image_bytes(BH, rows, E, M) bytes each): per 32 rows of
+ * the side one image of (q, grad_out, psi) resp. (k, v, phik) in two bf16 pieces each, the operands of
+ * flyhip_sblocal_bwd_pieces; with them the features are rounded to 17 significant bits everywhere (their two
+ * pieces are exact), and psi / phik may be NULL.  scratch: flyhip_sblocal_bwd_prep_scratch(BH,T,S,E,M) floats.
+ * (E, M) as for flyhip_sblocal_bwd. */
 int64_t flyhip_sblocal_bwd_prep_scratch(int BH, int T, int S, int E, int M);
+int64_t flyhip_sblocal_bwd_image_bytes(int BH, int rows, int E, int M);
 int flyhip_sblocal_bwd_prep(const float* q, const float* k, const float* v, const float* grad_out,
                             const float* out, const float* log_norm, const float* proj,
                             const int64_t* key_lengths,
                             float* psi, float* phik, float* c,
                             float* kv, float* ksum, float* qg, float* qc,
+                            void* q_images, void* k_images,
                             float* scratch, int64_t scratch_floats,
                             int BH, int H, int T, int S, int E, int M, int mh_valid,
                             float softmax_temp, void* stream);
+
+/* flyhip_sblocal_bwd on the bf16 matrix pipe: the same sums and epilogue (same gmat | gvec, proj, d1, d3 and
+ * key_major), every product from operands in two bf16 pieces with float32 accumulation.  outer_images /
+ * inner_images: the images of flyhip_sblocal_bwd_prep of the outer and of the inner side (queries then keys for
+ * key_major = 0, keys then queries for key_major = 1); x1, x3 (BH, outer rows, E) float32: the outer rows
+ * themselves (q, grad_out resp. k, v), c from the same preparation call. */
+int flyhip_sblocal_bwd_pieces(const void* outer_images, const void* inner_images,
+                              const float* x1, const float* x3,
+                              const float* log_norm, const float* c, const int64_t* key_lengths,
+                              const float* gmat, const float* gvec, const float* proj,
+                              float* d1, float* d3,
+                              int BH, int H, int T, int S, int E, int M, int local_context,
+                              float softmax_temp, int key_major, void* stream);
 
 /* Scatterbrain attention on a block-sparse support (ref: src/models/attention/sbblocksparse_attention.py:109-213
  * for need_weights = False, no dropout, no masks): as flyhip_sblocal_fwd with one part per query tile, but the

@@ -396,7 +396,8 @@ def test_backward_band_kernels_match_library_products(B, T, S, H, E, D, mh, lc, 
     kl = None if lens is None else torch.tensor(lens, device=dev)
     out, ln = sblocal_forward(q, k, v, P, lc, key_lengths=kl)
     ref = sblocal_backward(q, k, v, P, lc, None, kl, out, ln, go, band_kernel=False)
-    for mode in ('sums', True):          # band sums only / everything after the features on the kernels
+    # band sums only / everything on the kernels, band terms on the fp32 matrix pipe / on the bf16 matrix pipe
+    for mode in ('sums', 'fp32', True):
         got = sblocal_backward(q, k, v, P, lc, None, kl, out, ln, go, band_kernel=mode)
         for a, b in zip(got, ref):
             assert rel_err(a, b) <= 1e-4, (mode, rel_err(a, b))
@@ -438,7 +439,7 @@ def test_backward_preparation_kernels_match_tensor_algebra(BH, H, T, S, dim, mk,
     scratch = new(_lib.load().flyhip_sblocal_bwd_prep_scratch(BH, T, S, dim, mk))
     _lib.call('flyhip_sblocal_bwd_prep', Q.data_ptr(), K.data_ptr(), V.data_ptr(), G.data_ptr(), O.data_ptr(),
               LN.data_ptr(), proj.data_ptr(), _lib.ptr(kl), *(got[n].data_ptr() for n in ('psi', 'phik', 'c', 'kv', 'ksum', 'qg', 'qc')),
-              scratch.data_ptr(), scratch.numel(), BH, H, T, S, dim, mk, mh, t, _lib.stream_ptr(dev))
+              None, None, scratch.data_ptr(), scratch.numel(), BH, H, T, S, dim, mk, mh, t, _lib.stream_ptr(dev))
     torch.cuda.synchronize()
 
     def unpad(x, axis):                            # (.., mk, ..) -> (.., 2 mh, ..)
