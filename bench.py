@@ -389,6 +389,9 @@ def main():
     ap.add_argument('--copy-calibration', action='store_true',
                     help='also run a plain 256 MiB device copy: its FETCH_SIZE / WRITE_SIZE readings '
                          'give the scale of the traffic counters')
+    ap.add_argument('--train-step', choices=['config1', 'config3'], default=None,
+                    help='profiling runs: only time --steps forward + backward steps of Scatterbrain-local attention at '
+                         'that configuration (fp32; config3 = first T2T layer, B=64 L=3136 window 256) and print their time')
     args = ap.parse_args()
     if args.gpus != 1:
         print('bench.py: this build measures one GPU; --gpus must be 1 (nothing here shards over devices)',
@@ -397,6 +400,25 @@ def main():
     if not torch.cuda.is_available():
         print('bench.py: no GPU visible', file=sys.stderr)
         sys.exit(1)
+    if args.train_step:
+        import fly_amd
+        dev = torch.device('cuda:0')
+        g = torch.Generator().manual_seed(0)
+        torch.manual_seed(0)
+        B, L, lc, temp, scale = (2, 3136, 512, None, 64 ** -0.25) if args.train_step == 'config1' else (64, 3136, 256, 147 ** -0.5, 1.0)
+        q, k, v = (torch.randn(B, L, 1, 64, generator=g).to(dev) * scale for _ in range(3))
+        P = fly_amd.gaussian_orthogonal_random_matrix(64, 64).to(dev)
+        step = sblocal_train_step(q, k, v, P, lc, temp)
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        print(json.dumps({'train_step': args.train_step, 'steps': args.steps,
+                          'fwd_bwd_ms': (time.perf_counter() - t0) / args.steps * 1e3}))
+        return
     if args.copy_calibration:
         src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device='cuda:0').normal_()
         dst = torch.empty_like(src)
