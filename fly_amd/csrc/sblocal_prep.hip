@@ -410,6 +410,9 @@ struct BwdX3Args {
     float temp;
     const float* gmat; const float* gvec; const float* proj;
     int n_xcd;
+    // small problems: every outer tile's inner range walked in n_parts parts by as many workgroups, whose sums go to
+    // part_ws ((tile, part): registers x 256 lanes x 4 floats) and are finished by sblocal_bwd_x3_finish_kernel
+    float* part_ws; int n_parts;
 };
 
 typedef short shortx4 __attribute__((ext_vector_type(4)));
@@ -438,7 +441,108 @@ __device__ __forceinline__ void bwd_tile_to_lds(const char* src, char* dst, int 
         __builtin_amdgcn_global_load_lds(src + MAIN + 16 * (lane & 15), (lds_ptr)(dst + MAIN), 16, 0, 0);
 }
 
+// The finishing step of an outer tile: the sums over all keys / queries through the per-head matrices, the chain rule
+// through the feature map, and the stores.  smem: (M (D + 4) + M + M/2 (E + 4)) floats, not in use by anyone (the
+// caller's last access to it lies behind a barrier).
 template <int E, int M, bool KEYMAJOR>
+__device__ __forceinline__ void bwd_x3_epilogue(const BwdX3Args& a, char* smem, int bh, int o, int orow, int Lo,
+                                                const char* otile, int trow, float c_o,
+                                                floatx4 (&acc1)[E / 16], floatx4 (&acc2)[M / 16], floatx4 (&acc3)[KEYMAJOR ? E / 16 : 1]) {
+    using TL = BwdTile<E, M>;
+    constexpr int NT = 256, D = E, EC = E / 16, FC = M / 16, DB = D / 16, MH = M / 2, LDK = E + 4, LDV = D + 4;
+    const int tid = threadIdx.x, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
+    // ---- epilogue: per-head matrices into the tile stages (dead now; the loop ended on a barrier) ----
+    float* GMs = reinterpret_cast<float*>(smem);           // gmat (M, D), rows of LDV
+    float* GVs = GMs + M * LDV;                            // gvec (M)
+    float* Ps = GVs + M;                                   // projection (M/2, E), rows of LDK
+    for (int idx = tid; idx < M * (D / 4); idx += NT) {
+        const int r = idx / (D / 4), c4 = idx % (D / 4);
+        *reinterpret_cast<floatx4*>(GMs + r * LDV + 4 * c4) = *reinterpret_cast<const floatx4*>(a.gmat + ((long)bh * M + r) * D + 4 * c4);
+    }
+    for (int idx = tid; idx < MH * (E / 4); idx += NT) {
+        const int r = idx / (E / 4), c4 = idx % (E / 4);
+        *reinterpret_cast<floatx4*>(Ps + r * LDK + 4 * c4) = *reinterpret_cast<const floatx4*>(a.proj + (long)r * E + 4 * c4);
+    }
+    if (tid < M) GVs[tid] = a.gvec[(long)bh * M + tid];
+    // the outer row itself in fp32 (x1, x3) and its features from their two pieces (exact)
+    floatx4 x1[EC], x3[DB], x2[FC];
+#pragma unroll
+    for (int c = 0; c < EC; ++c) x1[c] = load4_f32(a.x1 + ((long)bh * Lo + orow) * E + 16 * c + 4 * g);
+#pragma unroll
+    for (int c = 0; c < DB; ++c) x3[c] = load4_f32(a.x3 + ((long)bh * Lo + orow) * D + 16 * c + 4 * g);
+#pragma unroll
+    for (int c = 0; c < FC; ++c) {
+        const char* p = otile + TL::F_OFF + trow * TL::F_ROW + x3_swz(trow, 2 * c + (g >> 1), TL::F_ROW) * 16 + 8 * (g & 1);
+        const uint2 fh = *reinterpret_cast<const uint2*>(p), fl = *reinterpret_cast<const uint2*>(p + TL::F_PIECE);
+        x2[c][0] = __uint_as_float(fh.x << 16) + __uint_as_float(fl.x << 16);
+        x2[c][1] = __uint_as_float(fh.x & 0xffff0000u) + __uint_as_float(fl.x & 0xffff0000u);
+        x2[c][2] = __uint_as_float(fh.y << 16) + __uint_as_float(fl.y << 16);
+        x2[c][3] = __uint_as_float(fh.y & 0xffff0000u) + __uint_as_float(fl.y & 0xffff0000u);
+    }
+    __syncthreads();
+    // u^T[f][outer] = sum_d gmat[f][d] x3[d][outer]
+    floatx4 u[FC];
+#pragma unroll
+    for (int c = 0; c < FC; ++c) u[c] = Frag<float>::zero();
+#pragma unroll
+    for (int cd = 0; cd < DB; ++cd) {
+        floatx4 ga[FC];
+#pragma unroll
+        for (int c = 0; c < FC; ++c) ga[c] = *reinterpret_cast<const floatx4*>(GMs + (16 * c + r16) * LDV + 16 * cd + 4 * g);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int c = 0; c < FC; ++c) u[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(ga[c][j], x3[cd][j], u[c], 0, 0, 0);
+    }
+    const float cmul = KEYMAJOR ? 1.0f : c_o;
+    float usum = 0.f;
+#pragma unroll
+    for (int c = 0; c < FC; ++c) {
+        const floatx4 gv = *reinterpret_cast<const floatx4*>(GVs + 16 * c + 4 * g);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            u[c][i] = x2[c][i] * (u[c][i] - cmul * gv[i] - acc2[c][i]);
+            usum += u[c][i];
+        }
+    }
+    usum = group_sum(usum);
+    // chain rule through the projection: dp^T[e][outer] = sum_r P[r][e] (u_r - u_{r + M/2})
+    floatx4 dp[EC];
+#pragma unroll
+    for (int c = 0; c < EC; ++c) dp[c] = Frag<float>::zero();
+#pragma unroll
+    for (int c = 0; c < FC / 2; ++c) {
+        const floatx4 du = u[c] - u[c + FC / 2];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int eb = 0; eb < EC; ++eb)
+                dp[eb] = __builtin_amdgcn_mfma_f32_16x16x4f32(Ps[(16 * c + 4 * g + j) * LDK + 16 * eb + r16], du[j], dp[eb], 0, 0, 0);
+    }
+    if (KEYMAJOR) {
+        // d v^T[d][key] += sum_f gmat[f][d] phik[f][key]
+#pragma unroll
+        for (int c = 0; c < FC; ++c)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+                    acc3[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(GMs[(16 * c + 4 * g + j) * LDV + 16 * db + r16], x2[c][j], acc3[db], 0, 0, 0);
+    }
+    if (o < Lo) {
+        const float st_ = sqrtf(a.temp);
+        float* p1 = a.o1 + ((long)bh * Lo + o) * E;
+#pragma unroll
+        for (int c = 0; c < EC; ++c) store4_f32(p1 + 16 * c + 4 * g, acc1[c] * a.temp + dp[c] * st_ - x1[c] * (a.temp * usum));
+        if (KEYMAJOR) {
+            float* p3 = a.o3 + ((long)bh * Lo + o) * D;
+#pragma unroll
+            for (int c = 0; c < DB; ++c) store4_f32(p3 + 16 * c + 4 * g, acc3[c]);
+        }
+    }
+}
+
+template <int E, int M, bool KEYMAJOR, bool PARTS>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void sblocal_bwd_x3_kernel(BwdX3Args a) {
     using TL = BwdTile<E, M>;
     constexpr int NT = 256, TQ = 64, TK = 32, KB = 2;
@@ -451,11 +555,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
     const int Lo = KEYMAJOR ? a.S : a.T, Li = KEYMAJOR ? a.T : a.S;
     const int n_ot = (Lo + TQ - 1) / TQ;
-    const int n_items = a.BH * n_ot;
+    const int n_parts = PARTS ? a.n_parts : 1;
+    const int n_items = a.BH * n_ot * n_parts;
     const int per_xcd = (n_items + a.n_xcd - 1) / a.n_xcd;
     const int item = (blockIdx.x % a.n_xcd) * per_xcd + blockIdx.x / a.n_xcd;   // neighbouring tiles share a die's L2
     if (item >= n_items) return;                           // workgroup-uniform
-    const int ot = item % n_ot, bh = item / n_ot, b = bh / a.H;
+    const int part = item % n_parts, tile_id = item / n_parts;
+    const int ot = tile_id % n_ot, bh = tile_id / n_ot, b = bh / a.H;
     const int o0 = ot * TQ, ow0 = o0 + 16 * w, o = ow0 + r16;
     const int len = a.lens ? min((int)a.lens[b], a.S) : a.S;
     const int lc_lo = a.lc / 2, lc_hi = (a.lc + 1) / 2;    // band: -lc_lo <= s - i < lc_hi
@@ -467,8 +573,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
     const int o_last = min(o0 + TQ - 1, o_limit - 1);
     const int n_lo = max(0, o0 + lo), n_hi = min(n_limit, o_last + hi);
-    const int kt_lo = n_lo / TK;
-    const int kt_hi = (o_last >= o0 && n_hi > n_lo) ? (n_hi + TK - 1) / TK : kt_lo;
+    int kt_lo = n_lo / TK;
+    int kt_hi = (o_last >= o0 && n_hi > n_lo) ? (n_hi + TK - 1) / TK : kt_lo;
+    if (PARTS) {                                           // this part's share of the tiles
+        const int per = (kt_hi - kt_lo + n_parts - 1) / n_parts;
+        kt_lo = min(kt_hi, kt_lo + part * per);
+        kt_hi = min(kt_hi, kt_lo + per);
+    }
 
     if (kt_lo < kt_hi) bwd_tile_to_lds<TL::MAIN, KEYMAJOR>(itiles + (long)kt_lo * TL::BYTES, smem, tid);
 
@@ -619,122 +730,110 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         __syncthreads();
     }
 
-    // ---- epilogue: per-head matrices into the tile stages (dead now; the loop ended on a barrier) ----
-    float* GMs = reinterpret_cast<float*>(smem);           // gmat (M, D), rows of LDV
-    float* GVs = GMs + M * LDV;                            // gvec (M)
-    float* Ps = GVs + M;                                   // projection (M/2, E), rows of LDK
-    for (int idx = tid; idx < M * (D / 4); idx += NT) {
-        const int r = idx / (D / 4), c4 = idx % (D / 4);
-        *reinterpret_cast<floatx4*>(GMs + r * LDV + 4 * c4) = *reinterpret_cast<const floatx4*>(a.gmat + ((long)bh * M + r) * D + 4 * c4);
-    }
-    for (int idx = tid; idx < MH * (E / 4); idx += NT) {
-        const int r = idx / (E / 4), c4 = idx % (E / 4);
-        *reinterpret_cast<floatx4*>(Ps + r * LDK + 4 * c4) = *reinterpret_cast<const floatx4*>(a.proj + (long)r * E + 4 * c4);
-    }
-    if (tid < M) GVs[tid] = a.gvec[(long)bh * M + tid];
-    // the outer row itself in fp32 (x1, x3) and its features from their two pieces (exact)
-    floatx4 x1[EC], x3[DB], x2[FC];
+    if (PARTS) {
+        // this part's sums, register by register, 16 bytes per lane
+        float* ws = a.part_ws + (long)item * ((EC + FC + (KEYMAJOR ? DB : 0)) * NT * 4) + 4 * tid;
 #pragma unroll
-    for (int c = 0; c < EC; ++c) x1[c] = load4_f32(a.x1 + ((long)bh * Lo + orow) * E + 16 * c + 4 * g);
+        for (int c = 0; c < EC; ++c) *reinterpret_cast<floatx4*>(ws + c * NT * 4) = acc1[c];
 #pragma unroll
-    for (int c = 0; c < DB; ++c) x3[c] = load4_f32(a.x3 + ((long)bh * Lo + orow) * D + 16 * c + 4 * g);
-#pragma unroll
-    for (int c = 0; c < FC; ++c) {
-        const char* p = otile + TL::F_OFF + trow * TL::F_ROW + x3_swz(trow, 2 * c + (g >> 1), TL::F_ROW) * 16 + 8 * (g & 1);
-        const uint2 fh = *reinterpret_cast<const uint2*>(p), fl = *reinterpret_cast<const uint2*>(p + TL::F_PIECE);
-        x2[c][0] = __uint_as_float(fh.x << 16) + __uint_as_float(fl.x << 16);
-        x2[c][1] = __uint_as_float(fh.x & 0xffff0000u) + __uint_as_float(fl.x & 0xffff0000u);
-        x2[c][2] = __uint_as_float(fh.y << 16) + __uint_as_float(fl.y << 16);
-        x2[c][3] = __uint_as_float(fh.y & 0xffff0000u) + __uint_as_float(fl.y & 0xffff0000u);
-    }
-    __syncthreads();
-    // u^T[f][outer] = sum_d gmat[f][d] x3[d][outer]
-    floatx4 u[FC];
-#pragma unroll
-    for (int c = 0; c < FC; ++c) u[c] = Frag<float>::zero();
-#pragma unroll
-    for (int cd = 0; cd < DB; ++cd) {
-        floatx4 ga[FC];
-#pragma unroll
-        for (int c = 0; c < FC; ++c) ga[c] = *reinterpret_cast<const floatx4*>(GMs + (16 * c + r16) * LDV + 16 * cd + 4 * g);
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int c = 0; c < FC; ++c) u[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(ga[c][j], x3[cd][j], u[c], 0, 0, 0);
-    }
-    const float cmul = KEYMAJOR ? 1.0f : c_o;
-    float usum = 0.f;
-#pragma unroll
-    for (int c = 0; c < FC; ++c) {
-        const floatx4 gv = *reinterpret_cast<const floatx4*>(GVs + 16 * c + 4 * g);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            u[c][i] = x2[c][i] * (u[c][i] - cmul * gv[i] - acc2[c][i]);
-            usum += u[c][i];
-        }
-    }
-    usum = group_sum(usum);
-    // chain rule through the projection: dp^T[e][outer] = sum_r P[r][e] (u_r - u_{r + M/2})
-    floatx4 dp[EC];
-#pragma unroll
-    for (int c = 0; c < EC; ++c) dp[c] = Frag<float>::zero();
-#pragma unroll
-    for (int c = 0; c < FC / 2; ++c) {
-        const floatx4 du = u[c] - u[c + FC / 2];
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int eb = 0; eb < EC; ++eb)
-                dp[eb] = __builtin_amdgcn_mfma_f32_16x16x4f32(Ps[(16 * c + 4 * g + j) * LDK + 16 * eb + r16], du[j], dp[eb], 0, 0, 0);
-    }
-    if (KEYMAJOR) {
-        // d v^T[d][key] += sum_f gmat[f][d] phik[f][key]
-#pragma unroll
-        for (int c = 0; c < FC; ++c)
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-#pragma unroll
-                for (int db = 0; db < DB; ++db)
-                    acc3[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(GMs[(16 * c + 4 * g + j) * LDV + 16 * db + r16], x2[c][j], acc3[db], 0, 0, 0);
-    }
-    if (o < Lo) {
-        const float st_ = sqrtf(a.temp);
-        float* p1 = a.o1 + ((long)bh * Lo + o) * E;
-#pragma unroll
-        for (int c = 0; c < EC; ++c) store4_f32(p1 + 16 * c + 4 * g, acc1[c] * a.temp + dp[c] * st_ - x1[c] * (a.temp * usum));
+        for (int c = 0; c < FC; ++c) *reinterpret_cast<floatx4*>(ws + (EC + c) * NT * 4) = acc2[c];
         if (KEYMAJOR) {
-            float* p3 = a.o3 + ((long)bh * Lo + o) * D;
 #pragma unroll
-            for (int c = 0; c < DB; ++c) store4_f32(p3 + 16 * c + 4 * g, acc3[c]);
+            for (int c = 0; c < DB; ++c) *reinterpret_cast<floatx4*>(ws + (EC + FC + c) * NT * 4) = acc3[c];
+        }
+        return;
+    }
+    bwd_x3_epilogue<E, M, KEYMAJOR>(a, smem, bh, o, orow, Lo, otile, trow, c_o, acc1, acc2, acc3);
+}
+
+// the parts of an outer tile summed in order, then its epilogue
+template <int E, int M, bool KEYMAJOR>
+__global__ __launch_bounds__(256) void sblocal_bwd_x3_finish_kernel(BwdX3Args a) {
+    using TL = BwdTile<E, M>;
+    constexpr int NT = 256, TQ = 64, D = E, EC = E / 16, FC = M / 16, DB = D / 16, NREG = EC + FC + (KEYMAJOR ? DB : 0);
+    extern __shared__ __attribute__((aligned(256))) char smem[];
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15;
+    const int Lo = KEYMAJOR ? a.S : a.T;
+    const int n_ot = (Lo + TQ - 1) / TQ;
+    const int tile = blockIdx.x, ot = tile % n_ot, bh = tile / n_ot;
+    const int o = ot * TQ + 16 * w + r16, orow = min(o, Lo - 1), trow = orow & 31;
+    const int n_oimg = 2 * ((Lo + 63) / 64);
+    const char* otile = a.oimg + ((long)bh * n_oimg + (orow >> 5)) * TL::BYTES;
+    const float c_o = KEYMAJOR ? 0.f : a.c[(long)bh * a.T + orow];
+    floatx4 acc1[EC], acc2[FC], acc3[KEYMAJOR ? DB : 1];
+#pragma unroll
+    for (int c = 0; c < EC; ++c) acc1[c] = Frag<float>::zero();
+#pragma unroll
+    for (int c = 0; c < FC; ++c) acc2[c] = Frag<float>::zero();
+#pragma unroll
+    for (int c = 0; c < (KEYMAJOR ? DB : 1); ++c) acc3[c] = Frag<float>::zero();
+    for (int p = 0; p < a.n_parts; ++p) {
+        const float* ws = a.part_ws + ((long)tile * a.n_parts + p) * (NREG * NT * 4) + 4 * tid;
+#pragma unroll
+        for (int c = 0; c < EC; ++c) acc1[c] += *reinterpret_cast<const floatx4*>(ws + c * NT * 4);
+#pragma unroll
+        for (int c = 0; c < FC; ++c) acc2[c] += *reinterpret_cast<const floatx4*>(ws + (EC + c) * NT * 4);
+        if (KEYMAJOR) {
+#pragma unroll
+            for (int c = 0; c < DB; ++c) acc3[c] += *reinterpret_cast<const floatx4*>(ws + (EC + FC + c) * NT * 4);
         }
     }
+    bwd_x3_epilogue<E, M, KEYMAJOR>(a, smem, bh, o, orow, Lo, otile, trow, c_o, acc1, acc2, acc3);
 }
 
 // (explicit instantiations: the host stubs of this template are not emitted otherwise)
 #define FLY_BWD_X3_INST(EE, MM) \
-    template __global__ void sblocal_bwd_x3_kernel<EE, MM, false>(BwdX3Args); \
-    template __global__ void sblocal_bwd_x3_kernel<EE, MM, true>(BwdX3Args);
+    template __global__ void sblocal_bwd_x3_kernel<EE, MM, false, false>(BwdX3Args); \
+    template __global__ void sblocal_bwd_x3_kernel<EE, MM, true, false>(BwdX3Args); \
+    template __global__ void sblocal_bwd_x3_kernel<EE, MM, false, true>(BwdX3Args); \
+    template __global__ void sblocal_bwd_x3_kernel<EE, MM, true, true>(BwdX3Args); \
+    template __global__ void sblocal_bwd_x3_finish_kernel<EE, MM, false>(BwdX3Args); \
+    template __global__ void sblocal_bwd_x3_finish_kernel<EE, MM, true>(BwdX3Args);
 FLY_BWD_X3_INST(32, 32) FLY_BWD_X3_INST(32, 64) FLY_BWD_X3_INST(64, 32) FLY_BWD_X3_INST(64, 64) FLY_BWD_X3_INST(64, 128)
 #undef FLY_BWD_X3_INST
 
+// parts per outer tile: as many as fill the machine once, at least two inner tiles each, at most 8
+static int bwd_x3_parts(long items, int lc) {
+    const int tiles = (64 + lc + 31) / 32 + 1;
+    const long fit = machine().slots / std::max(1L, items);
+    return (int)std::max(1L, std::min({fit, (long)tiles / 2, 8L}));
+}
+
 template <int E, int M, bool KEYMAJOR>
-static int launch_bwd_x3(const BwdX3Args& a, hipStream_t st) {
-    auto kern = sblocal_bwd_x3_kernel<E, M, KEYMAJOR>;
+static int launch_bwd_x3(const BwdX3Args& a, long part_ws_floats, hipStream_t st) {
     constexpr size_t smem = 2 * (BwdTile<E, M>::MAIN + 1024);
-    static std::atomic<unsigned long long> lds_set{0};     // (devices on which this kernel has its LDS limit)
-    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_set, "sblocal_bwd_x3")) return rc;
+    constexpr size_t smem_fin = sizeof(float) * (M * (E + 4) + M + (M / 2) * (E + 4));
+    constexpr long per_part = (E / 16 + M / 16 + (KEYMAJOR ? E / 16 : 0)) * 256 * 4;      // floats of one part's sums
     const Machine& mach = machine();
-    const long items = (long)a.BH * (((KEYMAJOR ? a.S : a.T) + 63) / 64);
+    const long tiles = (long)a.BH * (((KEYMAJOR ? a.S : a.T) + 63) / 64);
+    int parts = bwd_x3_parts(tiles, a.lc);
+    if (!a.part_ws || part_ws_floats < tiles * parts * per_part) parts = 1;
+    const long items = tiles * parts;
     const long grid = (items + mach.xcds - 1) / mach.xcds * mach.xcds;
     if (grid > 2147483647L) return fail(ERR_ARG, "sblocal_bwd_x3: too many workgroups");
     BwdX3Args args = a;
     args.n_xcd = mach.xcds;
+    args.n_parts = parts;
+    if (parts == 1) {
+        auto kern = sblocal_bwd_x3_kernel<E, M, KEYMAJOR, false>;
+        static std::atomic<unsigned long long> lds_set{0};     // (devices on which this kernel has its LDS limit)
+        if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_set, "sblocal_bwd_x3")) return rc;
+        hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), smem, st, args);
+        return check_launch("sblocal_bwd_x3_kernel");
+    }
+    auto kern = sblocal_bwd_x3_kernel<E, M, KEYMAJOR, true>;
+    auto fin = sblocal_bwd_x3_finish_kernel<E, M, KEYMAJOR>;
+    static std::atomic<unsigned long long> lds_set_p{0}, lds_set_f{0};
+    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_set_p, "sblocal_bwd_x3 (parts)")) return rc;
+    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(fin), smem_fin, lds_set_f, "sblocal_bwd_x3_finish")) return rc;
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), smem, st, args);
-    return check_launch("sblocal_bwd_x3_kernel");
+    if (int rc = check_launch("sblocal_bwd_x3_kernel (parts)")) return rc;
+    hipLaunchKernelGGL(fin, dim3((unsigned)tiles), dim3(256), smem_fin, st, args);
+    return check_launch("sblocal_bwd_x3_finish_kernel");
 }
 template <int E, int M>
-static int launch_bwd_x3_both(const BwdX3Args& a, bool key_major, hipStream_t st) {
-    return key_major ? launch_bwd_x3<E, M, true>(a, st) : launch_bwd_x3<E, M, false>(a, st);
+static int launch_bwd_x3_both(const BwdX3Args& a, long part_ws_floats, bool key_major, hipStream_t st) {
+    return key_major ? launch_bwd_x3<E, M, true>(a, part_ws_floats, st) : launch_bwd_x3<E, M, false>(a, part_ws_floats, st);
 }
 
 static void prep_splits(int BH, int T, int S, int& n_kblk, int& n_split_k, int& n_split_q) {
@@ -804,11 +903,22 @@ extern "C" int flyhip_sblocal_bwd_prep(const float* q, const float* k, const flo
                                  "{(32,32), (32,64), (64,32), (64,64), (64,128)}", E, M);
 }
 
+extern "C" int64_t flyhip_sblocal_bwd_parts_floats(int BH, int T, int S, int E, int M, int local_context) {
+    if (BH <= 0 || T <= 0 || S <= 0 || E <= 0 || M <= 0 || local_context < 1) return -1;
+    int64_t need = 0;
+    for (int km = 0; km < 2; ++km) {
+        const long tiles = (long)BH * (((km ? S : T) + 63) / 64);
+        const int parts = bwd_x3_parts(tiles, local_context);
+        if (parts > 1) need = std::max<int64_t>(need, tiles * parts * (int64_t)((E / 16 + M / 16 + (km ? E / 16 : 0)) * 256 * 4));
+    }
+    return need;
+}
+
 extern "C" int flyhip_sblocal_bwd_pieces(const void* outer_images, const void* inner_images,
                                          const float* x1, const float* x3,
                                          const float* log_norm, const float* c, const int64_t* key_lengths,
                                          const float* gmat, const float* gvec, const float* proj,
-                                         float* d1, float* d3,
+                                         float* d1, float* d3, float* part_ws, int64_t part_ws_floats,
                                          int BH, int H, int T, int S, int E, int M, int local_context,
                                          float softmax_temp, int key_major, void* stream) {
     FLY_REQUIRE(outer_images && inner_images && x1 && x3 && log_norm && c && gmat && gvec && proj && d1,
@@ -818,13 +928,14 @@ extern "C" int flyhip_sblocal_bwd_pieces(const void* outer_images, const void* i
     FLY_REQUIRE(local_context >= 1, "sblocal_bwd_pieces: local_context must be >= 1");
     FLY_REQUIRE(softmax_temp > 0.f, "sblocal_bwd_pieces: softmax_temp must be positive");
     BwdX3Args a{reinterpret_cast<const char*>(outer_images), reinterpret_cast<const char*>(inner_images), x1, x3,
-                log_norm, c, key_lengths, d1, d3, BH, H, T, S, local_context, softmax_temp, gmat, gvec, proj, 0};
+                log_norm, c, key_lengths, d1, d3, BH, H, T, S, local_context, softmax_temp, gmat, gvec, proj, 0, part_ws, 1};
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    if (E == 32 && M == 32) return launch_bwd_x3_both<32, 32>(a, key_major != 0, st);
-    if (E == 32 && M == 64) return launch_bwd_x3_both<32, 64>(a, key_major != 0, st);
-    if (E == 64 && M == 32) return launch_bwd_x3_both<64, 32>(a, key_major != 0, st);
-    if (E == 64 && M == 64) return launch_bwd_x3_both<64, 64>(a, key_major != 0, st);
-    if (E == 64 && M == 128) return launch_bwd_x3_both<64, 128>(a, key_major != 0, st);
+    const long wsf = part_ws ? (long)part_ws_floats : 0;
+    if (E == 32 && M == 32) return launch_bwd_x3_both<32, 32>(a, wsf, key_major != 0, st);
+    if (E == 32 && M == 64) return launch_bwd_x3_both<32, 64>(a, wsf, key_major != 0, st);
+    if (E == 64 && M == 32) return launch_bwd_x3_both<64, 32>(a, wsf, key_major != 0, st);
+    if (E == 64 && M == 64) return launch_bwd_x3_both<64, 64>(a, wsf, key_major != 0, st);
+    if (E == 64 && M == 128) return launch_bwd_x3_both<64, 128>(a, wsf, key_major != 0, st);
     return fail(ERR_UNSUPPORTED, "sblocal_bwd_pieces: (head dim, features) = (%d, %d) not in "
                                  "{(32,32), (32,64), (64,32), (64,64), (64,128)}", E, M);
 }

@@ -138,7 +138,7 @@ def _backward_hip(Q, K, V, G, O, LN, P, lens_b, H, local_context, t, dims, piece
     dim, mk = dims
     q_, k_, v_, g_, o_ = _fit(Q, dim), _fit(K, dim), _fit(V, dim), _fit(G, dim), _fit(O, dim)
     mh = P.shape[0]
-    proj = _fit(torch.nn.functional.pad(P, (0, 0, 0, mk // 2 - mh)), dim)
+    proj = P.contiguous() if P.shape == (mk // 2, dim) else _fit(torch.nn.functional.pad(P, (0, 0, 0, mk // 2 - mh)), dim)
     ln_ = LN.reshape(BH, T).contiguous()
     new = Q.new_empty
     lib = _lib.load()
@@ -146,6 +146,8 @@ def _backward_hip(Q, K, V, G, O, LN, P, lens_b, H, local_context, t, dims, piece
     if pieces:
         qimg = torch.empty(lib.flyhip_sblocal_bwd_image_bytes(BH, T, dim, mk), dtype=torch.uint8, device=Q.device)
         kimg = torch.empty(lib.flyhip_sblocal_bwd_image_bytes(BH, S, dim, mk), dtype=torch.uint8, device=Q.device)
+        n_ws = lib.flyhip_sblocal_bwd_parts_floats(BH, T, S, dim, mk, local_context)     # small problems: sums of parts
+        part_ws = new(n_ws) if n_ws > 0 else None
     else:
         psi_, phik_ = new(BH, T, mk), new(BH, S, mk)
     c_ = new(BH, T)
@@ -161,10 +163,10 @@ def _backward_hip(Q, K, V, G, O, LN, P, lens_b, H, local_context, t, dims, piece
         if pieces:
             _lib.call('flyhip_sblocal_bwd_pieces', qimg.data_ptr(), kimg.data_ptr(), q_.data_ptr(), g_.data_ptr(),
                       ln_.data_ptr(), c_.data_ptr(), _lib.ptr(lens_b), kv.data_ptr(), ksum.data_ptr(), proj.data_ptr(),
-                      dq.data_ptr(), None, BH, H, T, S, dim, mk, local_context, float(t), 0, st)
+                      dq.data_ptr(), None, _lib.ptr(part_ws), n_ws, BH, H, T, S, dim, mk, local_context, float(t), 0, st)
             _lib.call('flyhip_sblocal_bwd_pieces', kimg.data_ptr(), qimg.data_ptr(), k_.data_ptr(), v_.data_ptr(),
                       ln_.data_ptr(), c_.data_ptr(), _lib.ptr(lens_b), qg.data_ptr(), qc.data_ptr(), proj.data_ptr(),
-                      dk.data_ptr(), dv.data_ptr(), BH, H, T, S, dim, mk, local_context, float(t), 1, st)
+                      dk.data_ptr(), dv.data_ptr(), _lib.ptr(part_ws), n_ws, BH, H, T, S, dim, mk, local_context, float(t), 1, st)
         else:
             _lib.call('flyhip_sblocal_bwd', q_.data_ptr(), psi_.data_ptr(), g_.data_ptr(), k_.data_ptr(), phik_.data_ptr(),
                       v_.data_ptr(), ln_.data_ptr(), c_.data_ptr(), _lib.ptr(lens_b), kv.data_ptr(), ksum.data_ptr(),
