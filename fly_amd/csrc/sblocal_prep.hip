@@ -402,7 +402,7 @@ __global__ __launch_bounds__(PREP_NT) void sb_prep_reduce_kernel(PrepArgs a) {
 // no transposed copy exists anywhere.
 struct BwdX3Args {
     const char* oimg; const char* iimg;        // images of the outer and of the inner side
-    const float* x1; const float* x3;          // the outer rows themselves (BH, Lo, E), for the epilogue
+    const float* x1;                           // the outer rows themselves (BH, Lo, E), for the epilogue
     const float* ln; const float* c;           // (BH, T)
     const int64_t* lens;
     float* o1; float* o3;                      // d x1 (BH, Lo, E); d v (BH, S, E), key-major only
@@ -441,35 +441,64 @@ __device__ __forceinline__ void bwd_tile_to_lds(const char* src, char* dst, int 
         __builtin_amdgcn_global_load_lds(src + MAIN + 16 * (lane & 15), (lds_ptr)(dst + MAIN), 16, 0, 0);
 }
 
+// LDS bytes of the finishing step: gmat (M, D) and the projection (at least 32 rows, E) in three bf16 pieces, gvec
+template <int E, int M>
+constexpr int bwd_x3_epilogue_bytes() { return 3 * M * 2 * E + 3 * (M / 2 < 32 ? 32 : M / 2) * 2 * E + M * 4; }
+
+// rows x W floats in global memory (row stride W) -> three bf16 pieces in LDS ([h | m | l], `piece` bytes apart, rows
+// of 2 W bytes in natural element order, 16-byte chunks swizzled); rows >= rows_valid are written as zeros
+template <int W>
+__device__ __forceinline__ void bwd_x3_stage3(const float* src, char* dst, int rows, int rows_valid, int piece, int tid) {
+    for (int idx = tid; idx < rows * (W / 8); idx += 256) {
+        const int r = idx / (W / 8), ch = idx % (W / 8);
+        floatx4 x0 = Frag<float>::zero(), x1 = x0;
+        if (r < rows_valid) {
+            x0 = *reinterpret_cast<const floatx4*>(src + (long)r * W + 8 * ch);
+            x1 = *reinterpret_cast<const floatx4*>(src + (long)r * W + 8 * ch + 4);
+        }
+        uintx4 h, m, l;
+        split3(x0, x1, h, m, l);
+        char* d = dst + r * (2 * W) + x3_swz(r, ch, 2 * W) * 16;
+        *reinterpret_cast<uintx4*>(d) = h;
+        *reinterpret_cast<uintx4*>(d + piece) = m;
+        *reinterpret_cast<uintx4*>(d + 2 * piece) = l;
+    }
+}
+
 // The finishing step of an outer tile: the sums over all keys / queries through the per-head matrices, the chain rule
-// through the feature map, and the stores.  smem: (M (D + 4) + M + M/2 (E + 4)) floats, not in use by anyone (the
-// caller's last access to it lies behind a barrier).
+// through the feature map, and the stores; with u_f = x2_f (gmat_f . x3 - c gvec_f - acc2_f),
+//   d x1 = t acc1 + sqrt(t) P^T (u+ - u-) - t x1 sum_f u_f,     d v = acc3 + gmat^T x2   (key-major).
+// The three products run on the bf16 matrix pipe like the band sums: gmat and P in three pieces (exact), x3 from the
+// three pieces of its image, u+ - u- in three pieces, x2 in its two; six, six and five piece products, everything
+// above 2^-24 relative, because gmat . x3 is the "all keys" term the band's sum acc2 is subtracted from.  Transposed
+// operands (P^T, gmat^T) by ds_read_b64_tr_b16 as in the band loop.  smem: bwd_x3_epilogue_bytes<E, M>() bytes, not in
+// use by anyone (the caller's last access to it lies behind a barrier).
 template <int E, int M, bool KEYMAJOR>
 __device__ __forceinline__ void bwd_x3_epilogue(const BwdX3Args& a, char* smem, int bh, int o, int orow, int Lo,
                                                 const char* otile, int trow, float c_o,
                                                 floatx4 (&acc1)[E / 16], floatx4 (&acc2)[M / 16], floatx4 (&acc3)[KEYMAJOR ? E / 16 : 1]) {
     using TL = BwdTile<E, M>;
-    constexpr int NT = 256, D = E, EC = E / 16, FC = M / 16, DB = D / 16, MH = M / 2, LDK = E + 4, LDV = D + 4;
+    constexpr int D = E, KS1 = E / 32, EC = E / 16, FC = M / 16, DB = D / 16, MH = M / 2, PR = MH < 32 ? 32 : MH;
+    constexpr int G_ROW = 2 * D, G_PIECE = M * G_ROW, P_ROW = 2 * E, P_PIECE = PR * P_ROW;
     const int tid = threadIdx.x, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
-    // ---- epilogue: per-head matrices into the tile stages (dead now; the loop ended on a barrier) ----
-    float* GMs = reinterpret_cast<float*>(smem);           // gmat (M, D), rows of LDV
-    float* GVs = GMs + M * LDV;                            // gvec (M)
-    float* Ps = GVs + M;                                   // projection (M/2, E), rows of LDK
-    for (int idx = tid; idx < M * (D / 4); idx += NT) {
-        const int r = idx / (D / 4), c4 = idx % (D / 4);
-        *reinterpret_cast<floatx4*>(GMs + r * LDV + 4 * c4) = *reinterpret_cast<const floatx4*>(a.gmat + ((long)bh * M + r) * D + 4 * c4);
-    }
-    for (int idx = tid; idx < MH * (E / 4); idx += NT) {
-        const int r = idx / (E / 4), c4 = idx % (E / 4);
-        *reinterpret_cast<floatx4*>(Ps + r * LDK + 4 * c4) = *reinterpret_cast<const floatx4*>(a.proj + (long)r * E + 4 * c4);
-    }
+    char* GMs = smem;                                      // gmat pieces
+    char* Ps = GMs + 3 * G_PIECE;                          // projection pieces
+    float* GVs = reinterpret_cast<float*>(Ps + 3 * P_PIECE);
+    bwd_x3_stage3<D>(a.gmat + (long)bh * M * D, GMs, M, M, G_PIECE, tid);
+    bwd_x3_stage3<E>(a.proj, Ps, PR, MH, P_PIECE, tid);
     if (tid < M) GVs[tid] = a.gvec[(long)bh * M + tid];
-    // the outer row itself in fp32 (x1, x3) and its features from their two pieces (exact)
-    floatx4 x1[EC], x3[DB], x2[FC];
+    // the outer row: x1 in fp32, x3 as the three pieces of its image, its features from their two pieces (exact)
+    floatx4 x1[EC], x2[FC];
+    uintx4 x3h[KS1], x3m[KS1], x3l[KS1];
 #pragma unroll
     for (int c = 0; c < EC; ++c) x1[c] = load4_f32(a.x1 + ((long)bh * Lo + orow) * E + 16 * c + 4 * g);
 #pragma unroll
-    for (int c = 0; c < DB; ++c) x3[c] = load4_f32(a.x3 + ((long)bh * Lo + orow) * D + 16 * c + 4 * g);
+    for (int ks = 0; ks < KS1; ++ks) {
+        const char* p = otile + TL::Y_OFF + trow * TL::X_ROW + x3_swz(trow, 4 * ks + g, TL::X_ROW) * 16;
+        x3h[ks] = *reinterpret_cast<const uintx4*>(p);
+        x3m[ks] = *reinterpret_cast<const uintx4*>(p + TL::X_PIECE);
+        x3l[ks] = *reinterpret_cast<const uintx4*>(p + 2 * TL::X_PIECE);
+    }
 #pragma unroll
     for (int c = 0; c < FC; ++c) {
         const char* p = otile + TL::F_OFF + trow * TL::F_ROW + x3_swz(trow, 2 * c + (g >> 1), TL::F_ROW) * 16 + 8 * (g & 1);
@@ -483,16 +512,21 @@ __device__ __forceinline__ void bwd_x3_epilogue(const BwdX3Args& a, char* smem, 
     // u^T[f][outer] = sum_d gmat[f][d] x3[d][outer]
     floatx4 u[FC];
 #pragma unroll
-    for (int c = 0; c < FC; ++c) u[c] = Frag<float>::zero();
+    for (int c = 0; c < FC; ++c) {
+        u[c] = Frag<float>::zero();
 #pragma unroll
-    for (int cd = 0; cd < DB; ++cd) {
-        floatx4 ga[FC];
-#pragma unroll
-        for (int c = 0; c < FC; ++c) ga[c] = *reinterpret_cast<const floatx4*>(GMs + (16 * c + r16) * LDV + 16 * cd + 4 * g);
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int c = 0; c < FC; ++c) u[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(ga[c][j], x3[cd][j], u[c], 0, 0, 0);
+        for (int ks = 0; ks < KS1; ++ks) {
+            const int row = 16 * c + r16;
+            const char* p = GMs + row * G_ROW + x3_swz(row, 4 * ks + g, G_ROW) * 16;
+            const uintx4 gh = *reinterpret_cast<const uintx4*>(p), gm = *reinterpret_cast<const uintx4*>(p + G_PIECE);
+            const uintx4 gl = *reinterpret_cast<const uintx4*>(p + 2 * G_PIECE);
+            u[c] = mma_bf16(gl, x3h[ks], u[c]);
+            u[c] = mma_bf16(gh, x3l[ks], u[c]);
+            u[c] = mma_bf16(gm, x3m[ks], u[c]);
+            u[c] = mma_bf16(gm, x3h[ks], u[c]);
+            u[c] = mma_bf16(gh, x3m[ks], u[c]);
+            u[c] = mma_bf16(gh, x3h[ks], u[c]);
+        }
     }
     const float cmul = KEYMAJOR ? 1.0f : c_o;
     float usum = 0.f;
@@ -506,28 +540,52 @@ __device__ __forceinline__ void bwd_x3_epilogue(const BwdX3Args& a, char* smem, 
         }
     }
     usum = group_sum(usum);
-    // chain rule through the projection: dp^T[e][outer] = sum_r P[r][e] (u_r - u_{r + M/2})
+    // transposed reads as in the band loop: rows 4g + r16/4 (+ 16) of a 32-row step, columns 4 (r16 % 4) .. + 3 of a block
+    const int tr_row = 4 * g + (r16 >> 2), tr_cb = r16 & 3;
+    // chain rule through the projection: dp^T[e][outer] = sum_r P[r][e] (u_r - u_{r + M/2}), 32 rows r per step
     floatx4 dp[EC];
 #pragma unroll
     for (int c = 0; c < EC; ++c) dp[c] = Frag<float>::zero();
 #pragma unroll
-    for (int c = 0; c < FC / 2; ++c) {
-        const floatx4 du = u[c] - u[c + FC / 2];
+    for (int ks = 0; ks < PR / 32; ++ks) {
+        const floatx4 du0 = u[2 * ks] - u[2 * ks + FC / 2];
+        floatx4 du1 = Frag<float>::zero();
+        if (2 * ks + 1 < FC / 2) du1 = u[(2 * ks + 1 < FC / 2) ? 2 * ks + 1 : 0] - u[(2 * ks + 1 < FC / 2) ? 2 * ks + 1 + FC / 2 : 0];
+        uintx4 dh, dm, dl;
+        split3(du0, du1, dh, dm, dl);
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int eb = 0; eb < EC; ++eb)
-                dp[eb] = __builtin_amdgcn_mfma_f32_16x16x4f32(Ps[(16 * c + 4 * g + j) * LDK + 16 * eb + r16], du[j], dp[eb], 0, 0, 0);
+        for (int eb = 0; eb < EC; ++eb) {
+            const int row = 32 * ks + tr_row;
+            const char* p = Ps + row * P_ROW + x3_swz(row, 2 * eb + (tr_cb >> 1), P_ROW) * 16 + 8 * (tr_cb & 1);
+            const uintx4 ph = lds_read_tr8(p, p + 16 * P_ROW), pm = lds_read_tr8(p + P_PIECE, p + P_PIECE + 16 * P_ROW);
+            const uintx4 pl = lds_read_tr8(p + 2 * P_PIECE, p + 2 * P_PIECE + 16 * P_ROW);
+            dp[eb] = mma_bf16(pl, dh, dp[eb]);
+            dp[eb] = mma_bf16(ph, dl, dp[eb]);
+            dp[eb] = mma_bf16(pm, dm, dp[eb]);
+            dp[eb] = mma_bf16(pm, dh, dp[eb]);
+            dp[eb] = mma_bf16(ph, dm, dp[eb]);
+            dp[eb] = mma_bf16(ph, dh, dp[eb]);
+        }
     }
     if (KEYMAJOR) {
-        // d v^T[d][key] += sum_f gmat[f][d] phik[f][key]
+        // d v^T[d][key] += sum_f gmat[f][d] phik[f][key], 32 features per step
 #pragma unroll
-        for (int c = 0; c < FC; ++c)
+        for (int ks = 0; ks < M / 32; ++ks) {
+            uintx4 xh, xl;
+            split2(x2[2 * ks], x2[2 * ks + 1], xh, xl);
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-#pragma unroll
-                for (int db = 0; db < DB; ++db)
-                    acc3[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(GMs[(16 * c + 4 * g + j) * LDV + 16 * db + r16], x2[c][j], acc3[db], 0, 0, 0);
+            for (int db = 0; db < DB; ++db) {
+                const int row = 32 * ks + tr_row;
+                const char* p = GMs + row * G_ROW + x3_swz(row, 2 * db + (tr_cb >> 1), G_ROW) * 16 + 8 * (tr_cb & 1);
+                const uintx4 gh = lds_read_tr8(p, p + 16 * G_ROW), gm = lds_read_tr8(p + G_PIECE, p + G_PIECE + 16 * G_ROW);
+                const uintx4 gl = lds_read_tr8(p + 2 * G_PIECE, p + 2 * G_PIECE + 16 * G_ROW);
+                acc3[db] = mma_bf16(gl, xh, acc3[db]);
+                acc3[db] = mma_bf16(gm, xl, acc3[db]);
+                acc3[db] = mma_bf16(gm, xh, acc3[db]);
+                acc3[db] = mma_bf16(gh, xl, acc3[db]);
+                acc3[db] = mma_bf16(gh, xh, acc3[db]);
+            }
+        }
     }
     if (o < Lo) {
         const float st_ = sqrtf(a.temp);
@@ -548,9 +606,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     constexpr int NT = 256, TQ = 64, TK = 32, KB = 2;
     constexpr int D = E, KS1 = E / 32, KS2 = M / 32, EC = E / 16, FC = M / 16, DB = D / 16, MH = M / 2;
     constexpr int STAGE = TL::MAIN + 1024;                 // the image and a full wave load for its 256-byte tail
-    constexpr int LDK = E + 4, LDV = D + 4;                // epilogue operands, floats per row
     constexpr float LOG2E = 1.4426950408889634f;
-    static_assert((M * LDV + M + MH * LDK) * 4 <= 2 * STAGE, "epilogue operands must fit the tile stages");
+    static_assert(bwd_x3_epilogue_bytes<E, M>() <= 2 * STAGE, "epilogue operands must fit the tile stages");
     extern __shared__ __attribute__((aligned(256))) char smem[];
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
     const int Lo = KEYMAJOR ? a.S : a.T, Li = KEYMAJOR ? a.T : a.S;
@@ -802,7 +859,7 @@ static int bwd_x3_parts(long items, int lc) {
 template <int E, int M, bool KEYMAJOR>
 static int launch_bwd_x3(const BwdX3Args& a, long part_ws_floats, hipStream_t st) {
     constexpr size_t smem = 2 * (BwdTile<E, M>::MAIN + 1024);
-    constexpr size_t smem_fin = sizeof(float) * (M * (E + 4) + M + (M / 2) * (E + 4));
+    constexpr size_t smem_fin = bwd_x3_epilogue_bytes<E, M>();
     constexpr long per_part = (E / 16 + M / 16 + (KEYMAJOR ? E / 16 : 0)) * 256 * 4;      // floats of one part's sums
     const Machine& mach = machine();
     const long tiles = (long)a.BH * (((KEYMAJOR ? a.S : a.T) + 63) / 64);
@@ -915,19 +972,19 @@ extern "C" int64_t flyhip_sblocal_bwd_parts_floats(int BH, int T, int S, int E, 
 }
 
 extern "C" int flyhip_sblocal_bwd_pieces(const void* outer_images, const void* inner_images,
-                                         const float* x1, const float* x3,
+                                         const float* x1,
                                          const float* log_norm, const float* c, const int64_t* key_lengths,
                                          const float* gmat, const float* gvec, const float* proj,
                                          float* d1, float* d3, float* part_ws, int64_t part_ws_floats,
                                          int BH, int H, int T, int S, int E, int M, int local_context,
                                          float softmax_temp, int key_major, void* stream) {
-    FLY_REQUIRE(outer_images && inner_images && x1 && x3 && log_norm && c && gmat && gvec && proj && d1,
+    FLY_REQUIRE(outer_images && inner_images && x1 && log_norm && c && gmat && gvec && proj && d1,
                 "sblocal_bwd_pieces: null pointer");
     FLY_REQUIRE(!key_major || d3, "sblocal_bwd_pieces: the key-major pass needs d3");
     FLY_REQUIRE(BH > 0 && H > 0 && BH % H == 0 && T > 0 && S > 0, "sblocal_bwd_pieces: empty or inconsistent problem");
     FLY_REQUIRE(local_context >= 1, "sblocal_bwd_pieces: local_context must be >= 1");
     FLY_REQUIRE(softmax_temp > 0.f, "sblocal_bwd_pieces: softmax_temp must be positive");
-    BwdX3Args a{reinterpret_cast<const char*>(outer_images), reinterpret_cast<const char*>(inner_images), x1, x3,
+    BwdX3Args a{reinterpret_cast<const char*>(outer_images), reinterpret_cast<const char*>(inner_images), x1,
                 log_norm, c, key_lengths, d1, d3, BH, H, T, S, local_context, softmax_temp, gmat, gvec, proj, 0, part_ws, 1};
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     const long wsf = part_ws ? (long)part_ws_floats : 0;

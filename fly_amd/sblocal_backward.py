@@ -161,10 +161,10 @@ def _backward_hip(Q, K, V, G, O, LN, P, lens_b, H, local_context, t, dims, piece
                   kv.data_ptr(), ksum.data_ptr(), qg.data_ptr(), qc.data_ptr(), _lib.ptr(qimg), _lib.ptr(kimg),
                   scratch.data_ptr(), scratch.numel(), BH, H, T, S, dim, mk, mh, float(t), st)
         if pieces:
-            _lib.call('flyhip_sblocal_bwd_pieces', qimg.data_ptr(), kimg.data_ptr(), q_.data_ptr(), g_.data_ptr(),
+            _lib.call('flyhip_sblocal_bwd_pieces', qimg.data_ptr(), kimg.data_ptr(), q_.data_ptr(),
                       ln_.data_ptr(), c_.data_ptr(), _lib.ptr(lens_b), kv.data_ptr(), ksum.data_ptr(), proj.data_ptr(),
                       dq.data_ptr(), None, _lib.ptr(part_ws), n_ws, BH, H, T, S, dim, mk, local_context, float(t), 0, st)
-            _lib.call('flyhip_sblocal_bwd_pieces', kimg.data_ptr(), qimg.data_ptr(), k_.data_ptr(), v_.data_ptr(),
+            _lib.call('flyhip_sblocal_bwd_pieces', kimg.data_ptr(), qimg.data_ptr(), k_.data_ptr(),
                       ln_.data_ptr(), c_.data_ptr(), _lib.ptr(lens_b), qg.data_ptr(), qc.data_ptr(), proj.data_ptr(),
                       dk.data_ptr(), dv.data_ptr(), _lib.ptr(part_ws), n_ws, BH, H, T, S, dim, mk, local_context, float(t), 1, st)
         else:

@@ -209,14 +209,15 @@ int flyhip_sblocal_bwd_prep(const float* q, const float* k, const float* v, cons
 /* flyhip_sblocal_bwd on the bf16 matrix pipe: the same sums and epilogue (same gmat | gvec, proj, d1, d3 and
  * key_major), every product from operands in two bf16 pieces with float32 accumulation.  outer_images /
  * inner_images: the images of flyhip_sblocal_bwd_prep of the outer and of the inner side (queries then keys for
- * key_major = 0, keys then queries for key_major = 1); x1, x3 (BH, outer rows, E) float32: the outer rows
- * themselves (q, grad_out resp. k, v), c from the same preparation call.
+ * key_major = 0, keys then queries for key_major = 1); x1 (BH, outer rows, E) float32: the outer rows themselves
+ * (q resp. k), c from the same preparation call.  The epilogue's products run on the bf16 matrix pipe as well
+ * (gmat, proj and the image's values in three pieces each).
  * part_ws (may be NULL) of part_ws_floats >= flyhip_sblocal_bwd_parts_floats(BH,T,S,E,M,local_context) floats: with
  * it, problems of fewer 64-row tiles than the GPU holds workgroups walk each tile's band in several parts by as many
  * workgroups and finish in a second launch; without it (or when that function returns 0) every tile is one workgroup. */
 int64_t flyhip_sblocal_bwd_parts_floats(int BH, int T, int S, int E, int M, int local_context);
 int flyhip_sblocal_bwd_pieces(const void* outer_images, const void* inner_images,
-                              const float* x1, const float* x3,
+                              const float* x1,
                               const float* log_norm, const float* c, const int64_t* key_lengths,
                               const float* gmat, const float* gvec, const float* proj,
                               float* d1, float* d3, float* part_ws, int64_t part_ws_floats,
