@@ -125,6 +125,29 @@ def _fit_features(x, mk):
     return torch.cat([torch.nn.functional.pad(x[..., :mh], pad), torch.nn.functional.pad(x[..., mh:], pad)], dim=-1)
 
 
+_SCRATCH_SIZES = {}
+
+
+def _scratch_sizes(BH, T, S, dim, mk, local_context):
+    """Bytes of the two operand-image buffers and floats of the two scratch buffers of the kernel path, as the
+    library states them; kept per problem shape."""
+    key = (BH, T, S, dim, mk, local_context)
+    got = _SCRATCH_SIZES.get(key)
+    if got is None:
+        from . import _lib
+        lib = _lib.load()
+        got = {'qimg': lib.flyhip_sblocal_bwd_image_bytes(BH, T, dim, mk),
+               'kimg': lib.flyhip_sblocal_bwd_image_bytes(BH, S, dim, mk),
+               'scratch': lib.flyhip_sblocal_bwd_prep_scratch(BH, T, S, dim, mk),
+               'parts': lib.flyhip_sblocal_bwd_parts_floats(BH, T, S, dim, mk, local_context)}
+        if min(got.values()) < 0:
+            raise ValueError(f'the backward kernels reject the problem shape {key}')
+        if len(_SCRATCH_SIZES) > 256:
+            _SCRATCH_SIZES.clear()
+        _SCRATCH_SIZES[key] = got
+    return got
+
+
 def _backward_hip(Q, K, V, G, O, LN, P, lens_b, H, local_context, t, dims, pieces=True):
     """d query, d key, d value (BH, rows, width) in five launches: flyhip_sblocal_bwd_prep (scaled features of
     queries and keys, c = g . out, and the per-head sums over all keys / all queries) and the two passes of the
@@ -141,18 +164,24 @@ def _backward_hip(Q, K, V, G, O, LN, P, lens_b, H, local_context, t, dims, piece
     proj = P.contiguous() if P.shape == (mk // 2, dim) else _fit(torch.nn.functional.pad(P, (0, 0, 0, mk // 2 - mh)), dim)
     ln_ = LN.reshape(BH, T).contiguous()
     new = Q.new_empty
-    lib = _lib.load()
-    psi_ = phik_ = qimg = kimg = None
+    sizes = _scratch_sizes(BH, T, S, dim, mk, local_context)
+    n_ws = sizes['parts']
+    psi_ = phik_ = qimg = kimg = part_ws = None
     if pieces:
-        qimg = torch.empty(lib.flyhip_sblocal_bwd_image_bytes(BH, T, dim, mk), dtype=torch.uint8, device=Q.device)
-        kimg = torch.empty(lib.flyhip_sblocal_bwd_image_bytes(BH, S, dim, mk), dtype=torch.uint8, device=Q.device)
-        n_ws = lib.flyhip_sblocal_bwd_parts_floats(BH, T, S, dim, mk, local_context)     # small problems: sums of parts
-        part_ws = new(n_ws) if n_ws > 0 else None
+        images = torch.empty(sizes['qimg'] + sizes['kimg'], dtype=torch.uint8, device=Q.device)
+        qimg, kimg = images[:sizes['qimg']], images[sizes['qimg']:]
     else:
         psi_, phik_ = new(BH, T, mk), new(BH, S, mk)
-    c_ = new(BH, T)
-    kv, ksum, qg, qc = new(BH, mk, dim), new(BH, mk), new(BH, mk, dim), new(BH, mk)
-    scratch = new(lib.flyhip_sblocal_bwd_prep_scratch(BH, T, S, dim, mk))
+    # the small operands and the scratch as pieces of one allocation (each a multiple of 64 floats long)
+    want = [BH * T, BH * mk * dim, BH * mk, BH * mk * dim, BH * mk, sizes['scratch'], n_ws if pieces else 0]
+    offs = [0]
+    for n in want:
+        offs.append(offs[-1] + (n + 63) // 64 * 64)
+    pool = new(offs[-1])
+    c_, kv, ksum, qg, qc, scratch, ws = (pool[a:a + n] for a, n in zip(offs, want))
+    kv, qg = kv.view(BH, mk, dim), qg.view(BH, mk, dim)
+    if pieces and n_ws > 0:
+        part_ws = ws
     dq, dk, dv = new(BH, T, dim), new(BH, S, dim), new(BH, S, dim)
     with torch.cuda.device(Q.device):
         st = _lib.stream_ptr(Q.device)
