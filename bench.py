@@ -325,7 +325,18 @@ def bench_other_configs():
     q, k, v = (torch.randn(B, L, 1, E, generator=g).to(dev) * E ** -0.25 for _ in range(3))
     with torch.no_grad():
         out['sbblocksparse_fp32_B64_L3136_block32_m32'] = {'ms': timeit(lambda: sbbs(q, k, v), n=5)}
-    del q, k, v, sbbs
+    # its training step: fused forward, backward kernels walking the layout's blocks; beside it the op-by-op path
+    qg, kg, vg = (x.clone().requires_grad_() for x in (q, k, v))
+    go = torch.randn_like(v)
+
+    def sbbs_step():
+        o, _ = sbbs(qg, kg, vg)
+        o.backward(go)
+        qg.grad = kg.grad = vg.grad = None
+    out['sbblocksparse_fp32_B64_L3136_block32_m32']['fwd_bwd_ms'] = timeit(sbbs_step, n=5)
+    sbbs.fuse = False
+    out['sbblocksparse_fp32_B64_L3136_block32_m32']['fwd_bwd_op_by_op_ms'] = timeit(sbbs_step, n=3)
+    del q, k, v, sbbs, qg, kg, vg, go
 
     cfg = fly_amd.FlatBlockButterflySparsityConfig(8, 2, block=32)
     torch.manual_seed(0)

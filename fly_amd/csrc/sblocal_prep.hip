@@ -413,6 +413,9 @@ struct BwdX3Args {
     // small problems: every outer tile's inner range walked in n_parts parts by as many workgroups, whose sums go to
     // part_ws ((tile, part): registers x 256 lanes x 4 floats) and are finished by sblocal_bwd_x3_finish_kernel
     float* part_ws; int n_parts;
+    // a block-sparse support instead of a band (LIST kernels; 32 x 32 blocks, no key lengths): per (head, 64-row outer
+    // tile) the union of the inner 32-row blocks its two block-rows meet, and per entry whether each of the two does
+    const int32_t* tl_ptr; const int32_t* tl_inner; const int32_t* tl_blk;
 };
 
 typedef short shortx4 __attribute__((ext_vector_type(4)));
@@ -600,8 +603,9 @@ __device__ __forceinline__ void bwd_x3_epilogue(const BwdX3Args& a, char* smem, 
     }
 }
 
-template <int E, int M, bool KEYMAJOR, bool PARTS>
+template <int E, int M, bool KEYMAJOR, bool PARTS, bool LIST = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void sblocal_bwd_x3_kernel(BwdX3Args a) {
+    static_assert(!(PARTS && LIST), "lists are walked whole");
     using TL = BwdTile<E, M>;
     constexpr int NT = 256, TQ = 64, TK = 32, KB = 2;
     constexpr int D = E, KS1 = E / 32, KS2 = M / 32, EC = E / 16, FC = M / 16, DB = D / 16, MH = M / 2;
@@ -630,15 +634,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
     const int o_last = min(o0 + TQ - 1, o_limit - 1);
     const int n_lo = max(0, o0 + lo), n_hi = min(n_limit, o_last + hi);
-    int kt_lo = n_lo / TK;
-    int kt_hi = (o_last >= o0 && n_hi > n_lo) ? (n_hi + TK - 1) / TK : kt_lo;
-    if (PARTS) {                                           // this part's share of the tiles
-        const int per = (kt_hi - kt_lo + n_parts - 1) / n_parts;
-        kt_lo = min(kt_hi, kt_lo + part * per);
-        kt_hi = min(kt_hi, kt_lo + per);
+    const int kt_lo = n_lo / TK;
+    const int kt_hi = (o_last >= o0 && n_hi > n_lo) ? (n_hi + TK - 1) / TK : kt_lo;
+    // the inner tiles this workgroup meets: tile_at(i_lo) .. tile_at(i_hi - 1) -- the band's, this part's share of
+    // them, or the entries of the outer tile's list
+    int e_lo = 0, i_lo = 0, i_hi = kt_hi - kt_lo;
+    if (LIST) {
+        const int grp = (bh % a.H) * n_ot + ot;
+        e_lo = a.tl_ptr[grp];
+        i_hi = a.tl_ptr[grp + 1] - e_lo;
     }
+    if (PARTS) {
+        const int per = (i_hi + n_parts - 1) / n_parts;
+        i_lo = min(i_hi, part * per);
+        i_hi = min(i_hi, i_lo + per);
+    }
+    auto tile_at = [&](int i) __attribute__((always_inline)) { return LIST ? a.tl_inner[e_lo + i] : kt_lo + i; };
 
-    if (kt_lo < kt_hi) bwd_tile_to_lds<TL::MAIN, KEYMAJOR>(itiles + (long)kt_lo * TL::BYTES, smem, tid);
+    if (i_lo < i_hi) bwd_tile_to_lds<TL::MAIN, KEYMAJOR>(itiles + (long)tile_at(i_lo) * TL::BYTES, smem, tid);
 
     // outer operands (B side: column = outer row, k-slots 8g .. 8g + 7 of every 32-wide step) from the row's image
     const int orow = min(o, Lo - 1), trow = orow & 31;
@@ -683,15 +696,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     drain_loads();
     __syncthreads();
 
-    for (int kt = kt_lo; kt < kt_hi; ++kt) {
-        const int n_base = kt * TK;
-        const int cur = (kt - kt_lo) & 1;
+    for (int it = i_lo; it < i_hi; ++it) {
+        const int n_base = tile_at(it) * TK;
+        const int cur = (it - i_lo) & 1;
         const char* st = smem + cur * STAGE;
-        if (kt + 1 < kt_hi)                                // every wave is past the barrier that ended that stage's last use
-            bwd_tile_to_lds<TL::MAIN, KEYMAJOR>(itiles + (long)(kt + 1) * TL::BYTES, smem + (cur ^ 1) * STAGE, tid);
+        if (it + 1 < i_hi)                                 // every wave is past the barrier that ended that stage's last use
+            bwd_tile_to_lds<TL::MAIN, KEYMAJOR>(itiles + (long)tile_at(it + 1) * TL::BYTES, smem + (cur ^ 1) * STAGE, tid);
 
-        // wave-uniform: does this tile meet the band of any of the wave's 16 outer rows?
-        const bool any = !(n_base + TK - 1 - ow0 < lo || n_base - (ow0 + 15) >= hi || n_base >= n_limit || ow0 >= o_limit);
+        // wave-uniform: does this tile meet the band of any of the wave's 16 outer rows (is the block of the wave's
+        // block-row and this block-column part of the support)?
+        const bool any = LIST ? a.tl_blk[2 * (e_lo + it) + (w >> 1)] >= 0
+                              : !(n_base + TK - 1 - ow0 < lo || n_base - (ow0 + 15) >= hi || n_base >= n_limit || ow0 >= o_limit);
         if (any) {
             floatx4 s1[KB], s2[KB], s3[KB];
 #pragma unroll
@@ -742,7 +757,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const int n = n_base + 16 * kb + 4 * g + i;
-                    const bool ok = (unsigned)(n - nmin) < span;
+                    const bool ok = LIST ? ovalid : (unsigned)(n - nmin) < span;      // (a block of the support is whole)
                     const float av = ok ? __builtin_amdgcn_exp2f(s1[kb][i] * sc - (KEYMAJOR ? lnq[i] : ln_o)) : 0.f;
                     const float df = ok ? s3[kb][i] - (KEYMAJOR ? cq[i] : c_o) : 0.f;
                     wdm[kb][i] = av * df;
@@ -844,6 +859,8 @@ __global__ __launch_bounds__(256) void sblocal_bwd_x3_finish_kernel(BwdX3Args a)
     template __global__ void sblocal_bwd_x3_kernel<EE, MM, true, false>(BwdX3Args); \
     template __global__ void sblocal_bwd_x3_kernel<EE, MM, false, true>(BwdX3Args); \
     template __global__ void sblocal_bwd_x3_kernel<EE, MM, true, true>(BwdX3Args); \
+    template __global__ void sblocal_bwd_x3_kernel<EE, MM, false, false, true>(BwdX3Args); \
+    template __global__ void sblocal_bwd_x3_kernel<EE, MM, true, false, true>(BwdX3Args); \
     template __global__ void sblocal_bwd_x3_finish_kernel<EE, MM, false>(BwdX3Args); \
     template __global__ void sblocal_bwd_x3_finish_kernel<EE, MM, true>(BwdX3Args);
 FLY_BWD_X3_INST(32, 32) FLY_BWD_X3_INST(32, 64) FLY_BWD_X3_INST(64, 32) FLY_BWD_X3_INST(64, 64) FLY_BWD_X3_INST(64, 128)
@@ -871,6 +888,15 @@ static int launch_bwd_x3(const BwdX3Args& a, long part_ws_floats, hipStream_t st
     BwdX3Args args = a;
     args.n_xcd = mach.xcds;
     args.n_parts = parts;
+    if (a.tl_ptr) {
+        auto kern = sblocal_bwd_x3_kernel<E, M, KEYMAJOR, false, true>;
+        static std::atomic<unsigned long long> lds_set_l{0};
+        if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_set_l, "sblocal_bwd_x3 (lists)")) return rc;
+        const long lgrid = (tiles + mach.xcds - 1) / mach.xcds * mach.xcds;
+        args.n_parts = 1;
+        hipLaunchKernelGGL(kern, dim3((unsigned)lgrid), dim3(256), smem, st, args);
+        return check_launch("sblocal_bwd_x3_kernel (lists)");
+    }
     if (parts == 1) {
         auto kern = sblocal_bwd_x3_kernel<E, M, KEYMAJOR, false>;
         static std::atomic<unsigned long long> lds_set{0};     // (devices on which this kernel has its LDS limit)
@@ -985,7 +1011,8 @@ extern "C" int flyhip_sblocal_bwd_pieces(const void* outer_images, const void* i
     FLY_REQUIRE(local_context >= 1, "sblocal_bwd_pieces: local_context must be >= 1");
     FLY_REQUIRE(softmax_temp > 0.f, "sblocal_bwd_pieces: softmax_temp must be positive");
     BwdX3Args a{reinterpret_cast<const char*>(outer_images), reinterpret_cast<const char*>(inner_images), x1,
-                log_norm, c, key_lengths, d1, d3, BH, H, T, S, local_context, softmax_temp, gmat, gvec, proj, 0, part_ws, 1};
+                log_norm, c, key_lengths, d1, d3, BH, H, T, S, local_context, softmax_temp, gmat, gvec, proj, 0, part_ws, 1,
+                nullptr, nullptr, nullptr};
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     const long wsf = part_ws ? (long)part_ws_floats : 0;
     if (E == 32 && M == 32) return launch_bwd_x3_both<32, 32>(a, wsf, key_major != 0, st);
@@ -994,5 +1021,31 @@ extern "C" int flyhip_sblocal_bwd_pieces(const void* outer_images, const void* i
     if (E == 64 && M == 64) return launch_bwd_x3_both<64, 64>(a, wsf, key_major != 0, st);
     if (E == 64 && M == 128) return launch_bwd_x3_both<64, 128>(a, wsf, key_major != 0, st);
     return fail(ERR_UNSUPPORTED, "sblocal_bwd_pieces: (head dim, features) = (%d, %d) not in "
+                                 "{(32,32), (32,64), (64,32), (64,64), (64,128)}", E, M);
+}
+
+extern "C" int flyhip_sbblocksparse_bwd_pieces(const void* outer_images, const void* inner_images,
+                                               const float* x1, const float* log_norm, const float* c,
+                                               const float* gmat, const float* gvec, const float* proj,
+                                               float* d1, float* d3,
+                                               const int32_t* tl_ptr, const int32_t* tl_inner, const int32_t* tl_blk,
+                                               int BH, int H, int T, int S, int E, int M,
+                                               float softmax_temp, int key_major, void* stream) {
+    FLY_REQUIRE(outer_images && inner_images && x1 && log_norm && c && gmat && gvec && proj && d1 && tl_ptr && tl_inner && tl_blk,
+                "sbblocksparse_bwd_pieces: null pointer");
+    FLY_REQUIRE(!key_major || d3, "sbblocksparse_bwd_pieces: the key-major pass needs d3");
+    FLY_REQUIRE(BH > 0 && H > 0 && BH % H == 0 && T > 0 && S > 0, "sbblocksparse_bwd_pieces: empty or inconsistent problem");
+    FLY_REQUIRE(T % 32 == 0 && S % 32 == 0, "sbblocksparse_bwd_pieces: sequence lengths %d, %d must be multiples of 32", T, S);
+    FLY_REQUIRE(softmax_temp > 0.f, "sbblocksparse_bwd_pieces: softmax_temp must be positive");
+    BwdX3Args a{reinterpret_cast<const char*>(outer_images), reinterpret_cast<const char*>(inner_images), x1,
+                log_norm, c, nullptr, d1, d3, BH, H, T, S, 1, softmax_temp, gmat, gvec, proj, 0, nullptr, 1,
+                tl_ptr, tl_inner, tl_blk};
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (E == 32 && M == 32) return launch_bwd_x3_both<32, 32>(a, 0, key_major != 0, st);
+    if (E == 32 && M == 64) return launch_bwd_x3_both<32, 64>(a, 0, key_major != 0, st);
+    if (E == 64 && M == 32) return launch_bwd_x3_both<64, 32>(a, 0, key_major != 0, st);
+    if (E == 64 && M == 64) return launch_bwd_x3_both<64, 64>(a, 0, key_major != 0, st);
+    if (E == 64 && M == 128) return launch_bwd_x3_both<64, 128>(a, 0, key_major != 0, st);
+    return fail(ERR_UNSUPPORTED, "sbblocksparse_bwd_pieces: (head dim, features) = (%d, %d) not in "
                                  "{(32,32), (32,64), (64,32), (64,64), (64,128)}", E, M);
 }

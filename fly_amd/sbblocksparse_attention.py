@@ -41,6 +41,27 @@ def fused_tables(layout, device):
     return tuple(x.to(device) for x in (ptr, inner, blk, order, heavy)) + (parts,)
 
 
+class _SBBlockSparseFn(torch.autograd.Function):
+    """The fused forward with gradients for query, key and value: the backward of Scatterbrain-local attention with
+    the band replaced by the layout's blocks (sblocal_backward.sblocal_backward, support=...)."""
+
+    @staticmethod
+    def forward(ctx, query, key, value, projection_matrix, tables, support, softmax_temp):
+        out, log_norm = sbblocksparse_forward(query, key, value, projection_matrix, tables, softmax_temp)
+        ctx.save_for_backward(query, key, value, projection_matrix, out, log_norm)
+        ctx.support, ctx.softmax_temp = support, softmax_temp
+        ctx.mark_non_differentiable(log_norm)
+        return out, log_norm
+
+    @staticmethod
+    def backward(ctx, grad_out, _grad_log_norm):
+        from .sblocal_backward import sblocal_backward
+        query, key, value, projection_matrix, out, log_norm = ctx.saved_tensors
+        dq, dk, dv = sblocal_backward(query, key, value, projection_matrix, 1, ctx.softmax_temp, None, out, log_norm,
+                                      grad_out, support=ctx.support)
+        return dq, dk, dv, None, None, None, None
+
+
 class SBBlockSparseAttention(nn.Module):
     """sparsity_config: an object with ``.block`` and ``.make_layout(seq_len) -> (H, nb, nb)`` or a
     mapping with ``_target_``.  forward(query (B,T,H,E), key (B,S,H,E), value (B,S,H,D)) returns
@@ -67,6 +88,7 @@ class SBBlockSparseAttention(nn.Module):
         self.ops_cache = dict()
         self._layout_cache = dict()
         self.fused_tables = dict()
+        self.backward_tables = dict()
         # eligible forward passes run on the fused kernels; set to False to force the op-by-op path
         self.fuse = True
 
@@ -126,17 +148,27 @@ class SBBlockSparseAttention(nn.Module):
         self.feature_map.new_feature_map(query.device)
         layout = self.get_layout(T, S)
         needs_grad = torch.is_grad_enabled() and any(x.requires_grad for x in (query, key, value))
-        if (self.fuse and not need_weights and not needs_grad and not (self.training and self.dropout.p > 0)
+        from .sblocal_backward import _band_kernel_dims
+        n_rows = self.feature_map.projection_matrix.shape[0]
+        if (self.fuse and not need_weights and not (self.training and self.dropout.p > 0)
                 and self.softmax_eps == 0
                 and query.dtype in (torch.float32, torch.bfloat16, torch.float16)
-                and sbblocksparse_forward_supported(block, torch.float32, E, value.shape[3],
-                                                    self.feature_map.projection_matrix.shape[0], layout.shape[0], H)):
+                and sbblocksparse_forward_supported(block, torch.float32, E, value.shape[3], n_rows, layout.shape[0], H)
+                # with gradients: the backward kernels' head dims and feature counts
+                and (not needs_grad or _band_kernel_dims(E, value.shape[3], 2 * n_rows) is not None)):
             key_ = (T, S, query.device)
             if key_ not in self.fused_tables:
                 self.fused_tables[key_] = fused_tables(layout, query.device)
             # (2-byte inputs are widened, as on the op-by-op path below)
-            out, _ = sbblocksparse_forward(query.float(), key.float(), value.float(),
-                                           self.feature_map.projection_matrix, self.fused_tables[key_], softmax_temp)
+            if not needs_grad:
+                out, _ = sbblocksparse_forward(query.float(), key.float(), value.float(),
+                                               self.feature_map.projection_matrix, self.fused_tables[key_], softmax_temp)
+                return out.to(query.dtype), None
+            if key_ not in self.backward_tables:     # the support seen from the keys: unions of block-rows per two block-columns
+                self.backward_tables[key_] = tuple(x.to(query.device) for x in union_table(layout, 2, transposed=True))
+            support = (self.fused_tables[key_][:3], self.backward_tables[key_])
+            out, _ = _SBBlockSparseFn.apply(query.float(), key.float(), value.float(), self.feature_map.projection_matrix,
+                                            self.fused_tables[key_], support, softmax_temp)
             return out.to(query.dtype), None
 
         # 2-byte inputs are widened: the scores pass through HBM between the stages, and a score kept

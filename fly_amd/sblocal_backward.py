@@ -148,13 +148,16 @@ def _scratch_sizes(BH, T, S, dim, mk, local_context):
     return got
 
 
-def _backward_hip(Q, K, V, G, O, LN, P, lens_b, H, local_context, t, dims, pieces=True):
+def _backward_hip(Q, K, V, G, O, LN, P, lens_b, H, local_context, t, dims, pieces=True, support=None):
     """d query, d key, d value (BH, rows, width) in five launches: flyhip_sblocal_bwd_prep (scaled features of
     queries and keys, c = g . out, and the per-head sums over all keys / all queries) and the two passes of the
     band kernel (everything per (query, key) pair, the low-rank epilogue, the chain rule through the feature map).
     pieces: the band kernel on the bf16 matrix pipe from operands in two bf16 pieces (flyhip_sblocal_bwd_pieces;
     the preparation pass leaves every 32 rows of either side as one image of such operands), else on the fp32
-    matrix pipe from the float arrays (flyhip_sblocal_bwd)."""
+    matrix pipe from the float arrays (flyhip_sblocal_bwd).  support: instead of a band, a block-sparse support of
+    32 x 32 blocks -- (tables of the query tiles, tables of the key tiles), each (ptr, inner, blk) of
+    blocksparse_utils.union_table(layout, 2) resp. union_table(layout, 2, transposed=True) as int32 tensors on the
+    device (flyhip_sbblocksparse_bwd_pieces; no key lengths)."""
     from . import _lib
     BH, T, E = Q.shape
     S, D = K.shape[1], V.shape[2]
@@ -189,7 +192,15 @@ def _backward_hip(Q, K, V, G, O, LN, P, lens_b, H, local_context, t, dims, piece
                   ln_.data_ptr(), proj.data_ptr(), _lib.ptr(lens_b), _lib.ptr(psi_), _lib.ptr(phik_), c_.data_ptr(),
                   kv.data_ptr(), ksum.data_ptr(), qg.data_ptr(), qc.data_ptr(), _lib.ptr(qimg), _lib.ptr(kimg),
                   scratch.data_ptr(), scratch.numel(), BH, H, T, S, dim, mk, mh, float(t), st)
-        if pieces:
+        if support is not None:
+            (qp, qi, qb), (kp, ki, kb) = support
+            _lib.call('flyhip_sbblocksparse_bwd_pieces', qimg.data_ptr(), kimg.data_ptr(), q_.data_ptr(), ln_.data_ptr(),
+                      c_.data_ptr(), kv.data_ptr(), ksum.data_ptr(), proj.data_ptr(), dq.data_ptr(), None,
+                      qp.data_ptr(), qi.data_ptr(), qb.data_ptr(), BH, H, T, S, dim, mk, float(t), 0, st)
+            _lib.call('flyhip_sbblocksparse_bwd_pieces', kimg.data_ptr(), qimg.data_ptr(), k_.data_ptr(), ln_.data_ptr(),
+                      c_.data_ptr(), qg.data_ptr(), qc.data_ptr(), proj.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+                      kp.data_ptr(), ki.data_ptr(), kb.data_ptr(), BH, H, T, S, dim, mk, float(t), 1, st)
+        elif pieces:
             _lib.call('flyhip_sblocal_bwd_pieces', qimg.data_ptr(), kimg.data_ptr(), q_.data_ptr(),
                       ln_.data_ptr(), c_.data_ptr(), _lib.ptr(lens_b), kv.data_ptr(), ksum.data_ptr(), proj.data_ptr(),
                       dq.data_ptr(), None, _lib.ptr(part_ws), n_ws, BH, H, T, S, dim, mk, local_context, float(t), 0, st)
@@ -288,7 +299,7 @@ def _scaled_features(Q, K, P, t, LN, lens):
 
 
 def sblocal_backward(query, key, value, projection_matrix, local_context, softmax_temp, key_lengths,
-                     out, log_normalization, grad_out, chunk=256, max_elements=1 << 27, band_kernel=None):
+                     out, log_normalization, grad_out, chunk=256, max_elements=1 << 27, band_kernel=None, support=None):
     """query (B,T,H,E), key (B,S,H,E), value (B,S,H,D), out / grad_out (B,T,H,D),
     log_normalization (B,H,T,1) as returned by the forward; key_lengths (B,) or None.
     max_elements bounds the
@@ -298,6 +309,9 @@ def sblocal_backward(query, key, value, projection_matrix, local_context, softma
     chain rule in two, on the bf16 matrix pipe from operands in two bf16 pieces; 'fp32' = the same five launches
     with the band kernel on the fp32 matrix pipe; 'sums' = only the band sums on the kernels, the rest as tensor
     algebra; False = batched library products; True = the kernels or NotImplementedError.
+    support: the exact part lives on a block-sparse support of 32 x 32 blocks instead of a band (Scatterbrain
+    attention on a block-sparse support, sbblocksparse_attention.py:161-212): see _backward_hip; kernels only, no key
+    lengths, local_context is ignored.
     Returns (d query, d key, d value) in the dtypes of the inputs."""
     B, T, H, E = query.shape
     S, D = key.shape[1], value.shape[3]
@@ -320,7 +334,13 @@ def sblocal_backward(query, key, value, projection_matrix, local_context, softma
         raise NotImplementedError(f'no band kernel for head dims ({E}, {D}) with {2 * mh} features')
     on_kernels = dims is not None and Q.is_cuda and wdt == torch.float32
     lens_b = None if key_lengths is None else key_lengths.to(device=Q.device, dtype=torch.int64).contiguous()
-    if on_kernels and band_kernel != 'sums':
+    if support is not None:
+        if not on_kernels or key_lengths is not None or T % 32 or S % 32:
+            raise NotImplementedError('the backward on a block-sparse support needs the GPU kernels (float32 or bfloat16 '
+                                      f'inputs, head dims <= 64, <= 128 features; got ({E}, {D}), {2 * mh}), sequence '
+                                      'lengths that are multiples of 32 and no key lengths')
+        dQ, dK, dV = _backward_hip(Q, K, V, G, O, LN, P, None, H, 1, t, dims, support=support)
+    elif on_kernels and band_kernel != 'sums':
         # features, per-head sums and the two passes of the fused kernel
         dQ, dK, dV = _backward_hip(Q, K, V, G, O, LN, P, lens_b, H, local_context, t, dims,
                                    pieces=band_kernel != 'fp32')

@@ -224,6 +224,21 @@ int flyhip_sblocal_bwd_pieces(const void* outer_images, const void* inner_images
                               int BH, int H, int T, int S, int E, int M, int local_context,
                               float softmax_temp, int key_major, void* stream);
 
+/* flyhip_sblocal_bwd_pieces for Scatterbrain attention on a block-sparse support (the reference takes these
+ * gradients from autograd through src/models/attention/sbblocksparse_attention.py:161-212): the exact weights live on
+ * the nonzero 32 x 32 blocks of a layout instead of a band.  tl_ptr (H * ceil(outer rows / 64) + 1), tl_inner, tl_blk
+ * (2 per entry): per (head, 64-row outer tile) the union of the inner 32-row blocks its two block-rows meet, and per
+ * entry the block id of each of the two or -1 -- union_table(layout, 2) for key_major = 0 (outer = queries),
+ * union_table(layout, 2, transposed) for key_major = 1 (outer = keys).  T, S multiples of 32, no key lengths; images,
+ * gmat | gvec, c as for flyhip_sblocal_bwd_pieces. */
+int flyhip_sbblocksparse_bwd_pieces(const void* outer_images, const void* inner_images,
+                                    const float* x1, const float* log_norm, const float* c,
+                                    const float* gmat, const float* gvec, const float* proj,
+                                    float* d1, float* d3,
+                                    const int32_t* tl_ptr, const int32_t* tl_inner, const int32_t* tl_blk,
+                                    int BH, int H, int T, int S, int E, int M,
+                                    float softmax_temp, int key_major, void* stream);
+
 /* Scatterbrain attention on a block-sparse support (ref: src/models/attention/sbblocksparse_attention.py:109-213
  * for need_weights = False, no dropout, no masks): as flyhip_sblocal_fwd with one part per query tile, but the
  * exact part covers the nonzero 32 x 32 blocks of a layout instead of a band.  Key-side inputs (kfeat,

@@ -711,6 +711,72 @@ def test_sbblocksparse_fused_forward(B, H, T, S, E, D, m, seed):
     assert torch.equal(out2, out) and torch.equal(ln2, ln)
 
 
+@pytest.mark.parametrize('B,H,T,S,E,D,m,seed', [(2, 2, 256, 256, 64, 64, 64, 1), (1, 3, 224, 352, 32, 32, 32, 2),
+                                                (1, 2, 416, 160, 40, 24, 26, 4), (3, 1, 160, 192, 64, 64, 128, 5)])
+def test_sbblocksparse_gradients_on_the_kernels(B, H, T, S, E, D, m, seed):
+    """Gradients of Scatterbrain attention on a block-sparse support from the backward kernels walking the layout's
+    blocks (flyhip_sblocal_bwd_prep, flyhip_sbblocksparse_bwd_pieces) against autograd through the oracle in float64
+    (sbblocksparse_attention.py:161-212): random layouts per head with an empty block-row, an odd number of
+    block-rows and block-columns, T != S, head dims and feature counts that need padding."""
+    from fly_amd import sblocal_backward
+    from fly_amd.blocksparse_utils import union_table
+    from fly_amd.sblocal_attention import sbblocksparse_forward
+    from oracle import sbblocksparse as osbb
+    from oracle import sblocal as osb
+    print('case', B, H, T, S, E, D, m, flush=True)
+    g = torch.Generator().manual_seed(seed)
+    layout = (torch.rand(H, T // 32, S // 32, generator=g) < 0.4).long()
+    layout[:, :, 0] = 1
+    layout[0, 1, :] = 0
+    q = torch.randn(B, T, H, E, generator=g) * E ** -0.25
+    k = torch.randn(B, S, H, E, generator=g) * E ** -0.25
+    v = torch.randn(B, S, H, D, generator=g)
+    w = torch.randn(B, T, H, D, generator=g)
+    P = osb.gaussian_orthogonal_random_matrix(m // 2, E, generator=g)
+    qd, kd, vd = (x.double().requires_grad_() for x in (q, k, v))
+    ref_out, _ = osbb.sbblocksparse_attention(qd, kd, vd, P.double(), layout, 32)
+    (ref_out * w.double()).sum().backward()
+    fwd = tuple(x.to(DEV) for x in union_table(layout, rows_per_group=2))
+    bwd = tuple(x.to(DEV) for x in union_table(layout, rows_per_group=2, transposed=True))
+    qg, kg, vg = q.to(DEV), k.to(DEV), v.to(DEV)
+    out, ln = sbblocksparse_forward(qg, kg, vg, P.to(DEV), fwd)
+    dq, dk, dv = sblocal_backward(qg, kg, vg, P.to(DEV), 1, None, None, out, ln, w.to(DEV), support=(fwd, bwd))
+    for got, ref in ((dq, qd.grad), (dk, kd.grad), (dv, vd.grad)):
+        assert got.shape == ref.shape and rel_err(got, ref) <= 2e-4, rel_err(got, ref)
+
+
+def test_sbblocksparse_module_trains_on_the_fused_kernels():
+    """SBBlockSparseAttention with gradients: the forward stays on the fused kernels and the backward walks the
+    layout's blocks; gradients of query, key and value against autograd through the oracle, and against the op-by-op
+    path of the same module."""
+    from fly_amd import SBBlockSparseAttention, FlatBlockButterflySparsityConfig
+    from oracle import sbblocksparse as osbb
+    B, T, H, E, block = 2, 256, 1, 64, 32
+    torch.manual_seed(0)
+    layer = SBBlockSparseAttention(FlatBlockButterflySparsityConfig(4, 2, block=block), dim_heads=E,
+                                   nb_features=64, max_seq_length=T).to(DEV)
+    g = torch.Generator().manual_seed(4)
+    q, k, v, w = (torch.randn(B, T, H, E, generator=g) for _ in range(4))
+    q, k = q * E ** -0.25 * 2, k * E ** -0.25 * 2
+    qg, kg, vg = (x.to(DEV).requires_grad_() for x in (q, k, v))
+    out, _ = layer(qg, kg, vg)
+    assert len(layer.backward_tables) == 1                  # the kernel path
+    (out * w.to(DEV)).sum().backward()
+    P = layer.feature_map.projection_matrix.cpu().double()
+    qd, kd, vd = (x.double().requires_grad_() for x in (q, k, v))
+    ref_out, _ = osbb.sbblocksparse_attention(qd, kd, vd, P, layer.get_layout(T), block)
+    (ref_out * w.double()).sum().backward()
+    assert rel_err(out, ref_out) <= 1e-4
+    for got, ref in ((qg.grad, qd.grad), (kg.grad, kd.grad), (vg.grad, vd.grad)):
+        assert rel_err(got, ref) <= 2e-4, rel_err(got, ref)
+    layer.fuse = False
+    q2, k2, v2 = (x.to(DEV).requires_grad_() for x in (q, k, v))
+    out2, _ = layer(q2, k2, v2)
+    (out2 * w.to(DEV)).sum().backward()
+    for got, ref in ((qg.grad, q2.grad), (kg.grad, k2.grad), (vg.grad, v2.grad)):
+        assert rel_err(got, ref) <= 2e-4, rel_err(got, ref)
+
+
 def test_sbblocksparse_long_lists_in_parts():
     """Block-rows of global tokens: their query tiles' lists are walked in parts by a second launch and merged
     (fused_tables marks them); output and log-normaliser against the oracle and against the one-part path."""
