@@ -416,6 +416,9 @@ struct BwdX3Args {
     // a block-sparse support instead of a band (LIST kernels; 32 x 32 blocks, no key lengths): per (head, 64-row outer
     // tile) the union of the inner 32-row blocks its two block-rows meet, and per entry whether each of the two does
     const int32_t* tl_ptr; const int32_t* tl_inner; const int32_t* tl_blk;
+    // long lists: tl_skip (one flag per (head, outer tile)) marks the tiles the main launch leaves out; the launch
+    // in parts takes (batch, tl_heavy[j], part) for the n_heavy listed (head, outer tile) indices, then the finish
+    const int32_t* tl_skip; const int32_t* tl_heavy; int n_heavy;
 };
 
 typedef short shortx4 __attribute__((ext_vector_type(4)));
@@ -605,7 +608,6 @@ __device__ __forceinline__ void bwd_x3_epilogue(const BwdX3Args& a, char* smem, 
 
 template <int E, int M, bool KEYMAJOR, bool PARTS, bool LIST = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void sblocal_bwd_x3_kernel(BwdX3Args a) {
-    static_assert(!(PARTS && LIST), "lists are walked whole");
     using TL = BwdTile<E, M>;
     constexpr int NT = 256, TQ = 64, TK = 32, KB = 2;
     constexpr int D = E, KS1 = E / 32, KS2 = M / 32, EC = E / 16, FC = M / 16, DB = D / 16, MH = M / 2;
@@ -617,12 +619,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int Lo = KEYMAJOR ? a.S : a.T, Li = KEYMAJOR ? a.T : a.S;
     const int n_ot = (Lo + TQ - 1) / TQ;
     const int n_parts = PARTS ? a.n_parts : 1;
-    const int n_items = a.BH * n_ot * n_parts;
+    const int n_items = (LIST && PARTS ? (a.BH / a.H) * a.n_heavy : a.BH * n_ot) * n_parts;
     const int per_xcd = (n_items + a.n_xcd - 1) / a.n_xcd;
     const int item = (blockIdx.x % a.n_xcd) * per_xcd + blockIdx.x / a.n_xcd;   // neighbouring tiles share a die's L2
     if (item >= n_items) return;                           // workgroup-uniform
     const int part = item % n_parts, tile_id = item / n_parts;
-    const int ot = tile_id % n_ot, bh = tile_id / n_ot, b = bh / a.H;
+    int ot = tile_id % n_ot, bh = tile_id / n_ot;
+    if (LIST && PARTS) {                                   // tile_id = batch entry * n_heavy + index into the long lists
+        const int hg = a.tl_heavy[tile_id % a.n_heavy];
+        ot = hg % n_ot;
+        bh = (tile_id / a.n_heavy) * a.H + hg / n_ot;
+    }
+    if (LIST && !PARTS && a.tl_skip && a.tl_skip[(bh % a.H) * n_ot + ot]) return;      // walked in parts by another launch
+    const int b = bh / a.H;
     const int o0 = ot * TQ, ow0 = o0 + 16 * w, o = ow0 + r16;
     const int len = a.lens ? min((int)a.lens[b], a.S) : a.S;
     const int lc_lo = a.lc / 2, lc_hi = (a.lc + 1) / 2;    // band: -lc_lo <= s - i < lc_hi
@@ -827,7 +836,13 @@ __global__ __launch_bounds__(256) void sblocal_bwd_x3_finish_kernel(BwdX3Args a)
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15;
     const int Lo = KEYMAJOR ? a.S : a.T;
     const int n_ot = (Lo + TQ - 1) / TQ;
-    const int tile = blockIdx.x, ot = tile % n_ot, bh = tile / n_ot;
+    const int tile = blockIdx.x;
+    int ot = tile % n_ot, bh = tile / n_ot;
+    if (a.tl_heavy) {                                      // tile = batch entry * n_heavy + index into the long lists
+        const int hg = a.tl_heavy[tile % a.n_heavy];
+        ot = hg % n_ot;
+        bh = (tile / a.n_heavy) * a.H + hg / n_ot;
+    }
     const int o = ot * TQ + 16 * w + r16, orow = min(o, Lo - 1), trow = orow & 31;
     const int n_oimg = 2 * ((Lo + 63) / 64);
     const char* otile = a.oimg + ((long)bh * n_oimg + (orow >> 5)) * TL::BYTES;
@@ -861,6 +876,8 @@ __global__ __launch_bounds__(256) void sblocal_bwd_x3_finish_kernel(BwdX3Args a)
     template __global__ void sblocal_bwd_x3_kernel<EE, MM, true, true>(BwdX3Args); \
     template __global__ void sblocal_bwd_x3_kernel<EE, MM, false, false, true>(BwdX3Args); \
     template __global__ void sblocal_bwd_x3_kernel<EE, MM, true, false, true>(BwdX3Args); \
+    template __global__ void sblocal_bwd_x3_kernel<EE, MM, false, true, true>(BwdX3Args); \
+    template __global__ void sblocal_bwd_x3_kernel<EE, MM, true, true, true>(BwdX3Args); \
     template __global__ void sblocal_bwd_x3_finish_kernel<EE, MM, false>(BwdX3Args); \
     template __global__ void sblocal_bwd_x3_finish_kernel<EE, MM, true>(BwdX3Args);
 FLY_BWD_X3_INST(32, 32) FLY_BWD_X3_INST(32, 64) FLY_BWD_X3_INST(64, 32) FLY_BWD_X3_INST(64, 64) FLY_BWD_X3_INST(64, 128)
@@ -890,10 +907,29 @@ static int launch_bwd_x3(const BwdX3Args& a, long part_ws_floats, hipStream_t st
     args.n_parts = parts;
     if (a.tl_ptr) {
         auto kern = sblocal_bwd_x3_kernel<E, M, KEYMAJOR, false, true>;
-        static std::atomic<unsigned long long> lds_set_l{0};
+        static std::atomic<unsigned long long> lds_set_l{0}, lds_set_lp{0}, lds_set_lf{0};
         if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_set_l, "sblocal_bwd_x3 (lists)")) return rc;
         const long lgrid = (tiles + mach.xcds - 1) / mach.xcds * mach.xcds;
         args.n_parts = 1;
+        if (a.n_heavy > 0) {
+            // long lists first (they are the longest pieces of work): (batch, long tile, part) workgroups, then their finish
+            auto kern_p = sblocal_bwd_x3_kernel<E, M, KEYMAJOR, true, true>;
+            auto fin = sblocal_bwd_x3_finish_kernel<E, M, KEYMAJOR>;
+            if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern_p), smem, lds_set_lp, "sblocal_bwd_x3 (long lists)")) return rc;
+            if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(fin), smem_fin, lds_set_lf, "sblocal_bwd_x3_finish")) return rc;
+            const long htiles = (long)(a.BH / a.H) * a.n_heavy;
+            if (part_ws_floats < htiles * a.n_parts * per_part)
+                return fail(ERR_ARG, "sbblocksparse_bwd_pieces: part_ws of %ld floats, %ld needed", part_ws_floats, htiles * a.n_parts * per_part);
+            BwdX3Args hargs = args;
+            hargs.n_parts = a.n_parts;
+            const long hgrid = (htiles * a.n_parts + mach.xcds - 1) / mach.xcds * mach.xcds;
+            hipLaunchKernelGGL(kern_p, dim3((unsigned)hgrid), dim3(256), smem, st, hargs);
+            if (int rc = check_launch("sblocal_bwd_x3_kernel (long lists)")) return rc;
+            hipLaunchKernelGGL(kern, dim3((unsigned)lgrid), dim3(256), smem, st, args);
+            if (int rc = check_launch("sblocal_bwd_x3_kernel (lists)")) return rc;
+            hipLaunchKernelGGL(fin, dim3((unsigned)htiles), dim3(256), smem_fin, st, hargs);
+            return check_launch("sblocal_bwd_x3_finish_kernel (long lists)");
+        }
         hipLaunchKernelGGL(kern, dim3((unsigned)lgrid), dim3(256), smem, st, args);
         return check_launch("sblocal_bwd_x3_kernel (lists)");
     }
@@ -1012,7 +1048,7 @@ extern "C" int flyhip_sblocal_bwd_pieces(const void* outer_images, const void* i
     FLY_REQUIRE(softmax_temp > 0.f, "sblocal_bwd_pieces: softmax_temp must be positive");
     BwdX3Args a{reinterpret_cast<const char*>(outer_images), reinterpret_cast<const char*>(inner_images), x1,
                 log_norm, c, key_lengths, d1, d3, BH, H, T, S, local_context, softmax_temp, gmat, gvec, proj, 0, part_ws, 1,
-                nullptr, nullptr, nullptr};
+                nullptr, nullptr, nullptr, nullptr, nullptr, 0};
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     const long wsf = part_ws ? (long)part_ws_floats : 0;
     if (E == 32 && M == 32) return launch_bwd_x3_both<32, 32>(a, wsf, key_major != 0, st);
@@ -1024,11 +1060,18 @@ extern "C" int flyhip_sblocal_bwd_pieces(const void* outer_images, const void* i
                                  "{(32,32), (32,64), (64,32), (64,64), (64,128)}", E, M);
 }
 
+extern "C" int64_t flyhip_sbblocksparse_bwd_parts_floats(int B, int n_heavy, int heavy_parts, int E, int M, int key_major) {
+    if (B <= 0 || n_heavy < 0 || heavy_parts < 1 || E <= 0 || M <= 0) return -1;
+    return (int64_t)B * n_heavy * heavy_parts * ((E / 16 + M / 16 + (key_major ? E / 16 : 0)) * 256 * 4);
+}
+
 extern "C" int flyhip_sbblocksparse_bwd_pieces(const void* outer_images, const void* inner_images,
                                                const float* x1, const float* log_norm, const float* c,
                                                const float* gmat, const float* gvec, const float* proj,
                                                float* d1, float* d3,
                                                const int32_t* tl_ptr, const int32_t* tl_inner, const int32_t* tl_blk,
+                                               const int32_t* tl_skip, const int32_t* tl_heavy, int n_heavy, int heavy_parts,
+                                               float* part_ws, int64_t part_ws_floats,
                                                int BH, int H, int T, int S, int E, int M,
                                                float softmax_temp, int key_major, void* stream) {
     FLY_REQUIRE(outer_images && inner_images && x1 && log_norm && c && gmat && gvec && proj && d1 && tl_ptr && tl_inner && tl_blk,
@@ -1037,15 +1080,18 @@ extern "C" int flyhip_sbblocksparse_bwd_pieces(const void* outer_images, const v
     FLY_REQUIRE(BH > 0 && H > 0 && BH % H == 0 && T > 0 && S > 0, "sbblocksparse_bwd_pieces: empty or inconsistent problem");
     FLY_REQUIRE(T % 32 == 0 && S % 32 == 0, "sbblocksparse_bwd_pieces: sequence lengths %d, %d must be multiples of 32", T, S);
     FLY_REQUIRE(softmax_temp > 0.f, "sbblocksparse_bwd_pieces: softmax_temp must be positive");
+    FLY_REQUIRE(n_heavy == 0 || (n_heavy > 0 && tl_skip && tl_heavy && part_ws && heavy_parts >= 2 && heavy_parts <= 64),
+                "sbblocksparse_bwd_pieces: long lists need tl_skip, tl_heavy, part_ws and 2..64 parts");
     BwdX3Args a{reinterpret_cast<const char*>(outer_images), reinterpret_cast<const char*>(inner_images), x1,
-                log_norm, c, nullptr, d1, d3, BH, H, T, S, 1, softmax_temp, gmat, gvec, proj, 0, nullptr, 1,
-                tl_ptr, tl_inner, tl_blk};
+                log_norm, c, nullptr, d1, d3, BH, H, T, S, 1, softmax_temp, gmat, gvec, proj, 0, part_ws, n_heavy ? heavy_parts : 1,
+                tl_ptr, tl_inner, tl_blk, n_heavy ? tl_skip : nullptr, n_heavy ? tl_heavy : nullptr, n_heavy};
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    if (E == 32 && M == 32) return launch_bwd_x3_both<32, 32>(a, 0, key_major != 0, st);
-    if (E == 32 && M == 64) return launch_bwd_x3_both<32, 64>(a, 0, key_major != 0, st);
-    if (E == 64 && M == 32) return launch_bwd_x3_both<64, 32>(a, 0, key_major != 0, st);
-    if (E == 64 && M == 64) return launch_bwd_x3_both<64, 64>(a, 0, key_major != 0, st);
-    if (E == 64 && M == 128) return launch_bwd_x3_both<64, 128>(a, 0, key_major != 0, st);
+    const long wsf = part_ws ? (long)part_ws_floats : 0;
+    if (E == 32 && M == 32) return launch_bwd_x3_both<32, 32>(a, wsf, key_major != 0, st);
+    if (E == 32 && M == 64) return launch_bwd_x3_both<32, 64>(a, wsf, key_major != 0, st);
+    if (E == 64 && M == 32) return launch_bwd_x3_both<64, 32>(a, wsf, key_major != 0, st);
+    if (E == 64 && M == 64) return launch_bwd_x3_both<64, 64>(a, wsf, key_major != 0, st);
+    if (E == 64 && M == 128) return launch_bwd_x3_both<64, 128>(a, wsf, key_major != 0, st);
     return fail(ERR_UNSUPPORTED, "sbblocksparse_bwd_pieces: (head dim, features) = (%d, %d) not in "
                                  "{(32,32), (32,64), (64,32), (64,64), (64,128)}", E, M);
 }

@@ -41,6 +41,18 @@ def fused_tables(layout, device):
     return tuple(x.to(device) for x in (ptr, inner, blk, order, heavy)) + (parts,)
 
 
+def backward_tables(layout, device, transposed=False, n_heavy_min=32, entries_per_part=12, max_parts=16):
+    """Index tables of one pass of the backward kernels for a (H, T/32, S/32) layout: the union lists of the 64-row
+    outer tiles (queries, or with transposed=True keys), a flag per tile for the lists long enough to be walked in
+    parts, those tiles, and the number of parts -- (ptr, inner, blk, skip, heavy, parts), tensors on `device`."""
+    ptr, inner, blk = union_table(layout, rows_per_group=2, transposed=transposed)
+    counts = (ptr[1:] - ptr[:-1]).long()
+    skip = (counts >= n_heavy_min).to(torch.int32)
+    heavy = skip.nonzero().flatten().to(torch.int32)
+    parts = max(2, min(max_parts, int(counts.max()) // entries_per_part)) if heavy.numel() else 1
+    return tuple(x.to(device) for x in (ptr, inner, blk, skip, heavy)) + (parts,)
+
+
 class _SBBlockSparseFn(torch.autograd.Function):
     """The fused forward with gradients for query, key and value: the backward of Scatterbrain-local attention with
     the band replaced by the layout's blocks (sblocal_backward.sblocal_backward, support=...)."""
@@ -164,9 +176,10 @@ class SBBlockSparseAttention(nn.Module):
                 out, _ = sbblocksparse_forward(query.float(), key.float(), value.float(),
                                                self.feature_map.projection_matrix, self.fused_tables[key_], softmax_temp)
                 return out.to(query.dtype), None
-            if key_ not in self.backward_tables:     # the support seen from the keys: unions of block-rows per two block-columns
-                self.backward_tables[key_] = tuple(x.to(query.device) for x in union_table(layout, 2, transposed=True))
-            support = (self.fused_tables[key_][:3], self.backward_tables[key_])
+            if key_ not in self.backward_tables:     # the support seen from the queries and from the keys
+                self.backward_tables[key_] = (backward_tables(layout, query.device),
+                                              backward_tables(layout, query.device, transposed=True))
+            support = self.backward_tables[key_]
             out, _ = _SBBlockSparseFn.apply(query.float(), key.float(), value.float(), self.feature_map.projection_matrix,
                                             self.fused_tables[key_], support, softmax_temp)
             return out.to(query.dtype), None

@@ -157,7 +157,8 @@ def _backward_hip(Q, K, V, G, O, LN, P, lens_b, H, local_context, t, dims, piece
     matrix pipe from the float arrays (flyhip_sblocal_bwd).  support: instead of a band, a block-sparse support of
     32 x 32 blocks -- (tables of the query tiles, tables of the key tiles), each (ptr, inner, blk) of
     blocksparse_utils.union_table(layout, 2) resp. union_table(layout, 2, transposed=True) as int32 tensors on the
-    device (flyhip_sbblocksparse_bwd_pieces; no key lengths)."""
+    device, optionally followed by (skip, heavy, parts) for long lists walked in parts
+    (sbblocksparse_attention.backward_tables; flyhip_sbblocksparse_bwd_pieces; no key lengths)."""
     from . import _lib
     BH, T, E = Q.shape
     S, D = K.shape[1], V.shape[2]
@@ -193,13 +194,20 @@ def _backward_hip(Q, K, V, G, O, LN, P, lens_b, H, local_context, t, dims, piece
                   kv.data_ptr(), ksum.data_ptr(), qg.data_ptr(), qc.data_ptr(), _lib.ptr(qimg), _lib.ptr(kimg),
                   scratch.data_ptr(), scratch.numel(), BH, H, T, S, dim, mk, mh, float(t), st)
         if support is not None:
-            (qp, qi, qb), (kp, ki, kb) = support
-            _lib.call('flyhip_sbblocksparse_bwd_pieces', qimg.data_ptr(), kimg.data_ptr(), q_.data_ptr(), ln_.data_ptr(),
-                      c_.data_ptr(), kv.data_ptr(), ksum.data_ptr(), proj.data_ptr(), dq.data_ptr(), None,
-                      qp.data_ptr(), qi.data_ptr(), qb.data_ptr(), BH, H, T, S, dim, mk, float(t), 0, st)
-            _lib.call('flyhip_sbblocksparse_bwd_pieces', kimg.data_ptr(), qimg.data_ptr(), k_.data_ptr(), ln_.data_ptr(),
-                      c_.data_ptr(), qg.data_ptr(), qc.data_ptr(), proj.data_ptr(), dk.data_ptr(), dv.data_ptr(),
-                      kp.data_ptr(), ki.data_ptr(), kb.data_ptr(), BH, H, T, S, dim, mk, float(t), 1, st)
+            passes = ((qimg, kimg, q_, kv, ksum, dq, None), (kimg, qimg, k_, qg, qc, dk, dv))
+            for key_major, (tabs, (oimg, iimg, x1, gmat, gvec, d1, d3)) in enumerate(zip(support, passes)):
+                tl_ptr, tl_inner, tl_blk = tabs[:3]
+                skip = heavy = hws = None
+                n_heavy, parts, n_hws = 0, 1, 0
+                if len(tabs) > 3 and tabs[4].numel() > 0:      # long lists: walked in parts, finished by a second launch
+                    skip, heavy, parts = tabs[3], tabs[4], int(tabs[5])
+                    n_heavy = heavy.numel()
+                    n_hws = _lib.load().flyhip_sbblocksparse_bwd_parts_floats(BH // H, n_heavy, parts, dim, mk, key_major)
+                    hws = new(n_hws)
+                _lib.call('flyhip_sbblocksparse_bwd_pieces', oimg.data_ptr(), iimg.data_ptr(), x1.data_ptr(), ln_.data_ptr(),
+                          c_.data_ptr(), gmat.data_ptr(), gvec.data_ptr(), proj.data_ptr(), d1.data_ptr(), _lib.ptr(d3),
+                          tl_ptr.data_ptr(), tl_inner.data_ptr(), tl_blk.data_ptr(), _lib.ptr(skip), _lib.ptr(heavy),
+                          n_heavy, parts, _lib.ptr(hws), n_hws, BH, H, T, S, dim, mk, float(t), key_major, st)
         elif pieces:
             _lib.call('flyhip_sblocal_bwd_pieces', qimg.data_ptr(), kimg.data_ptr(), q_.data_ptr(),
                       ln_.data_ptr(), c_.data_ptr(), _lib.ptr(lens_b), kv.data_ptr(), ksum.data_ptr(), proj.data_ptr(),

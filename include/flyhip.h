@@ -230,12 +230,19 @@ int flyhip_sblocal_bwd_pieces(const void* outer_images, const void* inner_images
  * (2 per entry): per (head, 64-row outer tile) the union of the inner 32-row blocks its two block-rows meet, and per
  * entry the block id of each of the two or -1 -- union_table(layout, 2) for key_major = 0 (outer = queries),
  * union_table(layout, 2, transposed) for key_major = 1 (outer = keys).  T, S multiples of 32, no key lengths; images,
- * gmat | gvec, c as for flyhip_sblocal_bwd_pieces. */
+ * gmat | gvec, c as for flyhip_sblocal_bwd_pieces.
+ * Long lists (n_heavy > 0): tl_skip (H * ceil(outer rows / 64) flags) marks the outer tiles the main launch leaves
+ * out, tl_heavy (n_heavy indices head * ceil(outer rows / 64) + tile) lists them; they are walked in heavy_parts
+ * parts (2..64) by (batch, tile, part) workgroups of a launch of their own and finished by a third; part_ws of at
+ * least flyhip_sbblocksparse_bwd_parts_floats(BH / H, n_heavy, heavy_parts, E, M, key_major) floats. */
+int64_t flyhip_sbblocksparse_bwd_parts_floats(int B, int n_heavy, int heavy_parts, int E, int M, int key_major);
 int flyhip_sbblocksparse_bwd_pieces(const void* outer_images, const void* inner_images,
                                     const float* x1, const float* log_norm, const float* c,
                                     const float* gmat, const float* gvec, const float* proj,
                                     float* d1, float* d3,
                                     const int32_t* tl_ptr, const int32_t* tl_inner, const int32_t* tl_blk,
+                                    const int32_t* tl_skip, const int32_t* tl_heavy, int n_heavy, int heavy_parts,
+                                    float* part_ws, int64_t part_ws_floats,
                                     int BH, int H, int T, int S, int E, int M,
                                     float softmax_temp, int key_major, void* stream);
 

@@ -777,6 +777,48 @@ def test_sbblocksparse_module_trains_on_the_fused_kernels():
         assert rel_err(got, ref) <= 2e-4, rel_err(got, ref)
 
 
+def test_sbblocksparse_gradients_with_long_lists_in_parts():
+    """Backward kernels on a support with block-rows and block-columns of global tokens: the outer tiles with long
+    lists (queries of the global rows, keys of the global columns) are walked in parts and finished by a second
+    launch (sbblocksparse_attention.backward_tables); gradients against autograd through the oracle and against the
+    walk of whole lists."""
+    from fly_amd import sblocal_backward
+    from fly_amd.blocksparse_utils import union_table
+    from fly_amd.sbblocksparse_attention import backward_tables
+    from fly_amd.sblocal_attention import sbblocksparse_forward
+    from oracle import sbblocksparse as osbb
+    from oracle import sblocal as osb
+    B, H, L, E, m = 2, 2, 1280, 64, 64
+    nb = L // 32
+    g = torch.Generator().manual_seed(12)
+    idx = torch.arange(nb)
+    window = ((idx[:, None] - idx[None, :]).abs() <= 1).long()
+    layout = torch.stack([window.clone(), window.clone()])
+    layout[0, 0, :] = 1                       # head 0: a global block-row and a global block-column
+    layout[0, :, 0] = 1
+    layout[1, 21, :] = 1                      # head 1: a global block-row in the second half of its tile,
+    layout[1, :, 38:40] = 1                   # and a key tile whose two block-columns are both global
+    q = torch.randn(B, L, H, E, generator=g) * E ** -0.25
+    k = torch.randn(B, L, H, E, generator=g) * E ** -0.25
+    v = torch.randn(B, L, H, E, generator=g)
+    w = torch.randn(B, L, H, E, generator=g)
+    P = osb.gaussian_orthogonal_random_matrix(m // 2, E, generator=g)
+    tq, tk = backward_tables(layout, DEV), backward_tables(layout, DEV, transposed=True)
+    assert sorted(tq[4].tolist()) == [0, 20 + 10] and sorted(tk[4].tolist()) == [0, 20 + 19]
+    assert tq[5] >= 2 and tk[5] >= 2
+    qd, kd, vd = (x.double().requires_grad_() for x in (q, k, v))
+    ref_out, _ = osbb.sbblocksparse_attention(qd, kd, vd, P.double(), layout, 32)
+    (ref_out * w.double()).sum().backward()
+    qg, kg, vg = q.to(DEV), k.to(DEV), v.to(DEV)
+    out, ln = sbblocksparse_forward(qg, kg, vg, P.to(DEV), tq[:3])
+    got = sblocal_backward(qg, kg, vg, P.to(DEV), 1, None, None, out, ln, w.to(DEV), support=(tq, tk))
+    for x, ref in zip(got, (qd.grad, kd.grad, vd.grad)):
+        assert rel_err(x, ref) <= 2e-4, rel_err(x, ref)
+    whole = sblocal_backward(qg, kg, vg, P.to(DEV), 1, None, None, out, ln, w.to(DEV), support=(tq[:3], tk[:3]))
+    for x, y in zip(got, whole):
+        assert rel_err(x, y) <= 1e-5, rel_err(x, y)
+
+
 def test_sbblocksparse_long_lists_in_parts():
     """Block-rows of global tokens: their query tiles' lists are walked in parts by a second launch and merged
     (fused_tables marks them); output and log-normaliser against the oracle and against the one-part path."""

@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
     lib = _lib.load()
     for name in declared:
         assert hasattr(lib, name), f'{name} declared in include/flyhip.h but not exported'
-    assert set(_lib.SIGNATURES) | {'flyhip_last_error', 'flyhip_sb_workspace_bytes', 'flyhip_sblocal_bwd_prep_scratch', 'flyhip_sblocal_bwd_image_bytes', 'flyhip_sblocal_bwd_parts_floats'} == declared
+    assert set(_lib.SIGNATURES) | {'flyhip_last_error', 'flyhip_sb_workspace_bytes', 'flyhip_sblocal_bwd_prep_scratch', 'flyhip_sblocal_bwd_image_bytes', 'flyhip_sblocal_bwd_parts_floats', 'flyhip_sbblocksparse_bwd_parts_floats'} == declared
     assert lib.flyhip_version() >= 100
     # pure host entry point: the launch plan
     nc, ns, npart = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
