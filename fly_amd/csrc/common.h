@@ -294,4 +294,33 @@ __device__ __forceinline__ void split3(floatx4 x0, floatx4 x1, uintx4& h, uintx4
     split2(r0, r1, m, l);
 }
 
+// four floats -> bf16 head and rest, four k-slots each
+__device__ __forceinline__ void split2_4(floatx4 x, uint2& hi, uint2& lo) {
+    hi = make_uint2(pack_bf16x2(x[0], x[1]), pack_bf16x2(x[2], x[3]));
+    const floatx4 r = {x[0] - __uint_as_float(hi.x << 16), x[1] - __uint_as_float(hi.x & 0xffff0000u),
+                       x[2] - __uint_as_float(hi.y << 16), x[3] - __uint_as_float(hi.y & 0xffff0000u)};
+    lo = make_uint2(pack_bf16x2(r[0], r[1]), pack_bf16x2(r[2], r[3]));
+}
+
+__device__ __forceinline__ void split3_4(floatx4 x, uint2& h, uint2& m, uint2& l) {
+    h = make_uint2(pack_bf16x2(x[0], x[1]), pack_bf16x2(x[2], x[3]));
+    const floatx4 r = {x[0] - __uint_as_float(h.x << 16), x[1] - __uint_as_float(h.x & 0xffff0000u),
+                       x[2] - __uint_as_float(h.y << 16), x[3] - __uint_as_float(h.y & 0xffff0000u)};
+    split2_4(r, m, l);
+}
+
+// Transposed operand reads (ds_read_b64_tr_b16): within each group of 16 lanes, lane s passes the address of four
+// consecutive 16-bit elements -- row s / 4, columns 4 (s % 4) .. + 3 of a 4 x 16 block -- and lane l receives column l of
+// the four rows.
+typedef short shortx4 __attribute__((ext_vector_type(4)));
+typedef short shortx8 __attribute__((ext_vector_type(8)));
+// eight k-slots (inner rows) of one column: two transposed reads of 4 rows each
+__device__ __forceinline__ uintx4 lds_read_tr8(const char* p0, const char* p1) {
+    typedef __attribute__((address_space(3))) shortx4* lds_ptr;
+    const shortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)p0);
+    const shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)p1);
+    return __builtin_bit_cast(uintx4, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+}
+
+
 }  // namespace flyhip

@@ -162,6 +162,49 @@ struct RowTile {
     }
 };
 
+// K'^T V for the global low-rank term on the bf16 matrix pipe.  stash_pieces3: the rows a RowTile holds -> three bf16
+// pieces in LDS ([h | m | l], M * 2 COLS bytes apart; rows of 2 COLS bytes in natural element order, 16-byte chunks
+// swizzled): exact to fp32.  lowrank_pieces: lacc^T[d][query] += sum_f KV[f][d] q'[query][f] from those pieces, read
+// transposed (k = feature), and the query features in two pieces (exact: they are rounded to 17 bits where they are
+// formed); lane's k-slots of step ks are features 32 ks + 4 g + j and 32 ks + 16 + 4 g + j, as the overlap product
+// holds them.  Five piece products, everything above 2^-24: the term cancels against the band's own low-rank part.
+template <int M, int COLS>
+__device__ __forceinline__ void stash_pieces3(const RowTile<M, COLS>& t, char* dst, int tid) {
+    constexpr int V4 = COLS / 4, ROWB = 2 * COLS, PIECE = M * ROWB;
+#pragma unroll
+    for (int j = 0; j < RowTile<M, COLS>::N; ++j) {
+        const int idx = tid + NT * j, row = idx / V4, c4 = idx % V4;
+        if (RowTile<M, COLS>::N * NT == M * V4 || idx < M * V4) {
+            uint2 h, m, l;
+            split3_4(t.r[j], h, m, l);
+            char* d = dst + row * ROWB + x3_swz(row, c4 >> 1, ROWB) * 16 + 8 * (c4 & 1);
+            *reinterpret_cast<uint2*>(d) = h;
+            *reinterpret_cast<uint2*>(d + PIECE) = m;
+            *reinterpret_cast<uint2*>(d + 2 * PIECE) = l;
+        }
+    }
+}
+template <int M, int COLS, int NDB>
+__device__ __forceinline__ void lowrank_pieces(const char* kvp, const uintx4 (&qh)[M / 32], const uintx4 (&ql)[M / 32],
+                                               floatx4 (&lacc)[NDB], int r16, int g) {
+    constexpr int ROWB = 2 * COLS, PIECE = M * ROWB;
+    const int tr_row = 4 * g + (r16 >> 2), cb = r16 & 3;
+#pragma unroll
+    for (int ks = 0; ks < M / 32; ++ks)
+#pragma unroll
+        for (int db = 0; db < NDB; ++db) {
+            const int row = 32 * ks + tr_row;
+            const char* p = kvp + row * ROWB + x3_swz(row, 2 * db + (cb >> 1), ROWB) * 16 + 8 * (cb & 1);
+            const uintx4 kh = lds_read_tr8(p, p + 16 * ROWB), km = lds_read_tr8(p + PIECE, p + PIECE + 16 * ROWB);
+            const uintx4 kl = lds_read_tr8(p + 2 * PIECE, p + 2 * PIECE + 16 * ROWB);
+            lacc[db] = mma_bf16(kl, qh[ks], lacc[db]);
+            lacc[db] = mma_bf16(km, ql[ks], lacc[db]);
+            lacc[db] = mma_bf16(km, qh[ks], lacc[db]);
+            lacc[db] = mma_bf16(kh, ql[ks], lacc[db]);
+            lacc[db] = mma_bf16(kh, qh[ks], lacc[db]);
+        }
+}
+
 // projection matrix (MH, E) -> LDS rows of E+4 floats, scaled by sqrt(t)
 template <int E, int MH>
 __device__ __forceinline__ void load_proj(float* Ps, const float* proj, float scale, int tid) {
@@ -3197,16 +3240,23 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
     for (int db = 0; db < DB; ++db) lacc[db] = Frag<float>::zero();
     float qk1 = 0.f;
     if (!SPLIT) {
-        // global low-rank term on the fp32 MFMA from the rounded query features (hi + lo is exact)
-        float* KVs = smem;
-        float* KSs = smem + M * LDV;
-        {
-            RowTile<M, D> kvt;
-            kvt.fetch(a.kv + (long)bh * M * D, D, 0, M - 1, tid);
-            if (tid < M) KSs[tid] = a.ksum[(long)bh * M + tid];
-            kvt.template stash<LDV>(KVs, tid);
+        // global low-rank term on the bf16 matrix pipe: K'^T V in three pieces, the rounded query features in their two;
+        // as many of the D columns at a time as the three pieces fit into the tile stages
+        constexpr int ROOM = 2 * X3Tile<E, D, M>::BYTES - (int)sizeof(float) * M;
+        constexpr int CW = 3 * M * 2 * D <= ROOM ? D : (3 * M * D <= ROOM ? D / 2 : D / 4);
+        static_assert(3 * M * 2 * CW <= ROOM && CW % 16 == 0, "K'^T V pieces must fit the tile stages");
+        char* KVp = reinterpret_cast<char*>(smem);
+        float* KSs = reinterpret_cast<float*>(KVp + 3 * M * 2 * CW);
+        if (tid < M) KSs[tid] = a.ksum[(long)bh * M + tid];
+#pragma unroll
+        for (int sl = 0; sl < D / CW; ++sl) {
+            RowTile<M, CW> kvt;
+            kvt.fetch(a.kv + (long)bh * M * D + sl * CW, D, 0, M - 1, tid);
+            if (sl) __syncthreads();                 // the last slice's pieces have been read
+            stash_pieces3<M, CW>(kvt, KVp, tid);
+            __syncthreads();
+            lowrank_pieces<M, CW, CW / 16>(KVp, qfh, qfl, *reinterpret_cast<floatx4(*)[CW / 16]>(&lacc[sl * (CW / 16)]), r16, g);
         }
-        __syncthreads();
 #pragma unroll
         for (int c = 0; c < 2 * FB; ++c) {
             const uintx4 hw = qfh[c >> 1], lw = qfl[c >> 1];
@@ -3219,12 +3269,6 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
             }
             const floatx4 ks = *reinterpret_cast<const floatx4*>(KSs + 16 * c + 4 * g);
             qk1 += qf[0] * ks[0] + qf[1] * ks[1] + qf[2] * ks[2] + qf[3] * ks[3];
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-#pragma unroll
-                for (int db = 0; db < DB; ++db)
-                    lacc[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(
-                        KVs[(16 * c + 4 * g + j) * LDV + 16 * db + r16], qf[j], lacc[db], 0, 0, 0);
         }
         qk1 = group_sum(qk1);
     }
@@ -3358,9 +3402,9 @@ __global__ __launch_bounds__(NT) void sb_merge_kernel(FwdArgs a) {
 // read once), and the one-dimensional grid is laid out so that a tile is finished on the XCD whose
 // workgroups wrote its parts (the dispatcher deals consecutive workgroup ids to the XCDs in turn): the
 // partials are then still in that XCD's L2.  xcd_items = band items (tile, part) per XCD of the band launch.
-// (the finish of tile tl, columns 16 NDB slice .. of it, by one workgroup; KVs: M rows of 16 NDB + 4 floats, KSs: M floats of LDS)
+// (the finish of tile tl, columns 16 NDB slice .. of it, by one workgroup; KVp: 3 M rows of 32 NDB bytes, KSs: M floats of LDS)
 template <int D, int M, int NDB>
-__device__ __forceinline__ void sb_merge_tile(const FwdArgs& a, int tl, int slice, float* KVs, float* KSs) {
+__device__ __forceinline__ void sb_merge_tile(const FwdArgs& a, int tl, int slice, char* KVp, float* KSs) {
     constexpr float LN2 = 0.6931471805599453f;
     constexpr int FC = M / 16, COLS = 16 * NDB, LDV = COLS + 4;
     constexpr int PB = NDB >= 4 ? 5 : 8;              // parts per batch (their loads are all in flight together)
@@ -3401,7 +3445,7 @@ __device__ __forceinline__ void sb_merge_tile(const FwdArgs& a, int tl, int slic
                 ov[jj][db] = *reinterpret_cast<const floatx4*>(ws + off + ql * D + col0 + 16 * db + 4 * g);
         }
         if (p0 == 0) {
-            kvt.template stash<LDV>(KVs, tid);
+            stash_pieces3<M, COLS>(kvt, KVp, tid);
             if (tid < M) KSs[tid] = ksv;
         }
         float m_new = m_star;
@@ -3428,16 +3472,14 @@ __device__ __forceinline__ void sb_merge_tile(const FwdArgs& a, int tl, int slic
 #pragma unroll
     for (int db = 0; db < NDB; ++db) lacc[db] = Frag<float>::zero();
     float qk1 = 0.f;
+    uintx4 qph[M / 32], qpl[M / 32];
 #pragma unroll
     for (int c = 0; c < FC; ++c) {
         const floatx4 ks = *reinterpret_cast<const floatx4*>(KSs + 16 * c + 4 * g);
         qk1 += qf[c][0] * ks[0] + qf[c][1] * ks[1] + qf[c][2] * ks[2] + qf[c][3] * ks[3];
-#pragma unroll
-        for (int jj = 0; jj < 4; ++jj)
-#pragma unroll
-            for (int db = 0; db < NDB; ++db)
-                lacc[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(KVs[(16 * c + 4 * g + jj) * LDV + 16 * db + r16], qf[c][jj], lacc[db], 0, 0, 0);
+        if (c & 1) split2(qf[c - 1], qf[c], qph[c >> 1], qpl[c >> 1]);      // (exact: the features carry 17 bits)
     }
+    lowrank_pieces<M, COLS, NDB>(KVp, qph, qpl, lacc, r16, g);
     qk1 = group_sum(qk1);
     if (iq >= a.T) return;
     const float gamma = __builtin_amdgcn_exp2f(c0 - m_star);
@@ -3451,8 +3493,8 @@ __device__ __forceinline__ void sb_merge_tile(const FwdArgs& a, int tl, int slic
 
 template <int D, int M, int NDB>
 __global__ __launch_bounds__(NT) void sb_merge_x_kernel(FwdArgs a, int xcd_items, int tiles_per_xcd) {
-    constexpr int COLS = 16 * NDB, LDV = COLS + 4, NSL = D / COLS;
-    __shared__ __attribute__((aligned(16))) float KVs[M * LDV];
+    constexpr int COLS = 16 * NDB, NSL = D / COLS;
+    __shared__ __attribute__((aligned(16))) char KVp[3 * M * 2 * COLS];
     __shared__ __attribute__((aligned(16))) float KSs[M];
     const int n_qt = (a.T + TQ - 1) / TQ, n_tiles = a.B * a.H * n_qt;
     const int x = blockIdx.x % a.n_xcd, i = blockIdx.x / a.n_xcd, slice = i % NSL, j = i / NSL;
@@ -3461,7 +3503,7 @@ __global__ __launch_bounds__(NT) void sb_merge_x_kernel(FwdArgs a, int xcd_items
     const int t_hi = min(((x + 1) * xcd_items + a.n_parts - 1) / a.n_parts, n_tiles);
     const int tl = t_lo + j;
     if (j >= tiles_per_xcd || tl >= t_hi) return;     // workgroup-uniform
-    sb_merge_tile<D, M, NDB>(a, tl, slice, KVs, KSs);
+    sb_merge_tile<D, M, NDB>(a, tl, slice, KVp, KSs);
 }
 
 // ---------------------------------------------------------------------------------------

@@ -35,14 +35,6 @@ struct PrepArgs {
 constexpr int PREP_ROWS = 64;        // rows per step of a workgroup: 16 per wave
 constexpr int PREP_NT = 256;
 
-// four floats -> bf16 head and rest, four k-slots each
-__device__ __forceinline__ void split2_4(floatx4 x, uint2& hi, uint2& lo) {
-    hi = make_uint2(pack_bf16x2(x[0], x[1]), pack_bf16x2(x[2], x[3]));
-    const floatx4 r = {x[0] - __uint_as_float(hi.x << 16), x[1] - __uint_as_float(hi.x & 0xffff0000u),
-                       x[2] - __uint_as_float(hi.y << 16), x[3] - __uint_as_float(hi.y & 0xffff0000u)};
-    lo = make_uint2(pack_bf16x2(r[0], r[1]), pack_bf16x2(r[2], r[3]));
-}
-
 // 64 rows x W floats in LDS (row stride LD floats) -> their NP-piece images in the two 32-row tiles at `tile0` and
 // `tile0 + tile_stride`: chunk c of a row = elements 8c .. 8c + 7, 16 bytes per piece
 template <int W, int LD, int NP>
@@ -420,16 +412,6 @@ struct BwdX3Args {
     // in parts takes (batch, tl_heavy[j], part) for the n_heavy listed (head, outer tile) indices, then the finish
     const int32_t* tl_skip; const int32_t* tl_heavy; int n_heavy;
 };
-
-typedef short shortx4 __attribute__((ext_vector_type(4)));
-typedef short shortx8 __attribute__((ext_vector_type(8)));
-// eight k-slots (inner rows) of one column: two transposed reads of 4 rows each
-__device__ __forceinline__ uintx4 lds_read_tr8(const char* p0, const char* p1) {
-    typedef __attribute__((address_space(3))) shortx4* lds_ptr;
-    const shortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)p0);
-    const shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)p1);
-    return __builtin_bit_cast(uintx4, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-}
 
 // one tile image, global memory -> LDS stage `dst` (linear; each wave load writes 1024 consecutive bytes); TAIL: also
 // the 256 bytes behind the MAIN ones (log Z and c of the tile's queries; a full wave load, lanes 16.. repeat them)
