@@ -171,6 +171,7 @@ struct RowTile {
 template <int M, int COLS>
 __device__ __forceinline__ void stash_pieces3(const RowTile<M, COLS>& t, char* dst, int tid) {
     constexpr int V4 = COLS / 4, ROWB = 2 * COLS, PIECE = M * ROWB;
+    static_assert(COLS >= 32, "the chunk swizzle needs rows of four chunks or more");
 #pragma unroll
     for (int j = 0; j < RowTile<M, COLS>::N; ++j) {
         const int idx = tid + NT * j, row = idx / V4, c4 = idx % V4;
