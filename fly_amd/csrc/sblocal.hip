@@ -214,6 +214,24 @@ __device__ __forceinline__ void load_proj(float* Ps, const float* proj, float sc
     t.template stash<E + 4>(Ps, tid, scale);
 }
 
+// projection matrix (MH, E) times `scale` -> three bf16 pieces in LDS ([h | m | l], MH * 2 E bytes apart; rows of 2 E
+// bytes with position 32 ks + 8 g + 4 h + i <- element 32 ks + 16 h + 4 g + i, the k-slot order of an operand that
+// is split from fragments of elements 16 c + 4 g + i; 16-byte chunks swizzled): exact to fp32
+template <int E, int MH>
+__device__ __forceinline__ void load_proj_pieces(char* Pp, const float* proj, float scale, int tid) {
+    constexpr int CH8 = E / 8, ROWB = 2 * E, PIECE = MH * ROWB;
+    for (int idx = tid; idx < MH * CH8; idx += NT) {
+        const int row = idx / CH8, cch = idx % CH8, ks = cch >> 2, gq = cch & 3;
+        const float* sp = proj + (long)row * E + 32 * ks + 4 * gq;
+        uintx4 h, m, l;
+        split3(*reinterpret_cast<const floatx4*>(sp) * scale, *reinterpret_cast<const floatx4*>(sp + 16) * scale, h, m, l);
+        char* d = Pp + row * ROWB + x3_swz(row, cch, ROWB) * 16;
+        *reinterpret_cast<uintx4*>(d) = h;
+        *reinterpret_cast<uintx4*>(d + PIECE) = m;
+        *reinterpret_cast<uintx4*>(d + 2 * PIECE) = l;
+    }
+}
+
 // KV = sum_s exp(part_max_s - kmax) KV_s, same for Ksum, of one (batch, head) by `wpb` workgroups
 // (this is number `ci` of them; the output elements are dealt to their threads round-robin), the
 // weights staged in LDS (`wgt`, n_split floats) so that the loads over s are independent and stay
@@ -2997,22 +3015,31 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
             for (int c = 0; c < 2 * FB; ++c) qf[c] = *reinterpret_cast<const floatx4*>(a.qfeat + qrow * M + 16 * c + 4 * g);
             lsq = a.q_lsq[qrow];
         } else {
-            load_proj<E, MH>(Ps, a.proj, sqrtf(a.temp), tid);
+            // sqrt(t) P q on the bf16 matrix pipe: P in three pieces (exact), q in two, five piece products
+            char* Pp = reinterpret_cast<char*>(smem);
+            constexpr int P_ROW = 2 * E, P_PIECE = MH * P_ROW;
+            static_assert(3 * P_PIECE <= 2 * TL::BYTES, "the projection pieces must fit the tile stages");
+            load_proj_pieces<E, MH>(Pp, a.proj, sqrtf(a.temp), tid);
             __syncthreads();
             float qmax = 0.f;
 #pragma unroll
             for (int fb = 0; fb < FB; ++fb) qf[fb] = Frag<float>::zero();
 #pragma unroll
-            for (int c = 0; c < EC; ++c) {
-                floatx4 pa[FB];
+            for (int ks = 0; ks < E / 32; ++ks) {
+                uintx4 uh, ul;
+                split2(qr[2 * ks], qr[2 * ks + 1], uh, ul);
 #pragma unroll
-                for (int fb = 0; fb < FB; ++fb)
-                    pa[fb] = *reinterpret_cast<const floatx4*>(Ps + (16 * fb + r16) * LDK + 16 * c + 4 * g);
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-#pragma unroll
-                    for (int fb = 0; fb < FB; ++fb)
-                        qf[fb] = __builtin_amdgcn_mfma_f32_16x16x4f32(pa[fb][j], qr[c][j], qf[fb], 0, 0, 0);
+                for (int fb = 0; fb < FB; ++fb) {
+                    const int row = 16 * fb + r16;
+                    const char* pp_ = Pp + row * P_ROW + x3_swz(row, 4 * ks + g, P_ROW) * 16;
+                    const uintx4 ph = *reinterpret_cast<const uintx4*>(pp_), pm = *reinterpret_cast<const uintx4*>(pp_ + P_PIECE);
+                    const uintx4 pl = *reinterpret_cast<const uintx4*>(pp_ + 2 * P_PIECE);
+                    qf[fb] = mma_bf16(pl, uh, qf[fb]);
+                    qf[fb] = mma_bf16(pm, ul, qf[fb]);
+                    qf[fb] = mma_bf16(ph, ul, qf[fb]);
+                    qf[fb] = mma_bf16(pm, uh, qf[fb]);
+                    qf[fb] = mma_bf16(ph, uh, qf[fb]);
+                }
             }
 #pragma unroll
             for (int fb = 0; fb < FB; ++fb)
