@@ -383,7 +383,7 @@ __global__ __launch_bounds__(PREP_NT) void sb_prep_reduce_kernel(PrepArgs a) {
 // The arithmetic of sblocal_bwd_band_kernel (pair weights a = exp(t q.k - log Z), kb = psi.phik, df = g.v - c,
 // dm = a df; five band-limited sums; the finishing epilogue with the per-head matrices and the chain rule through
 // the feature map), with every product on v_mfma_f32_16x16x32_bf16 from operands in two bf16 pieces and fp32
-// accumulation: three piece products for q.k and two of the output sums (the rest-times-rest product, 2^-16
+// accumulation: three piece products for q.k and the sum over dm; six for (a - kb) g (its low-rank part cancels against Q'^T g) (the rest-times-rest product, 2^-16
 // relative, is dropped); six for g.v from three pieces each (exact to fp32: df = g.v - c cancels where one key carries
 // a query's weight) and five for phik^T df with df in three pieces; all four for psi.phik, whose operands are exact in two pieces -- the band's low-rank
 // weight then cancels against the per-head sums, which the preparation pass forms from the same rounded features.
@@ -756,10 +756,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                     wak[kb][i] = av - (ok ? s2[kb][i] : 0.f);
                 }
             }
-            uintx4 dmh, dml, dfh, dfm, dfl, akh, akl;
+            uintx4 dmh, dml, dfh, dfm, dfl, akh, akm, akl;
             split2(wdm[0], wdm[1], dmh, dml);
             split3(wdf[0], wdf[1], dfh, dfm, dfl);
-            if (KEYMAJOR) split2(wak[0], wak[1], akh, akl);
+            if (KEYMAJOR) split3(wak[0], wak[1], akh, akm, akl);
             // out^T[col][outer] += sum_inner Y[inner][col] w[inner][outer]
 #pragma unroll
             for (int c = 0; c < EC; ++c) {
@@ -770,10 +770,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 acc1[c] = mma_bf16(yh, dml, acc1[c]);
                 acc1[c] = mma_bf16(yh, dmh, acc1[c]);
                 if (KEYMAJOR) {
+                    // (a - kb) g: the band's low-rank part cancels against the per-head sum Q'^T g, so all six products
                     const uintx4 vh = lds_read_tr8(p + TL::Y_OFF, p + TL::Y_OFF + 16 * TL::X_ROW);
-                    const uintx4 vl = lds_read_tr8(p + TL::Y_OFF + TL::X_PIECE, p + TL::Y_OFF + TL::X_PIECE + 16 * TL::X_ROW);       // (the middle piece)
+                    const uintx4 vm = lds_read_tr8(p + TL::Y_OFF + TL::X_PIECE, p + TL::Y_OFF + TL::X_PIECE + 16 * TL::X_ROW);
+                    const uintx4 vl = lds_read_tr8(p + TL::Y_OFF + 2 * TL::X_PIECE, p + TL::Y_OFF + 2 * TL::X_PIECE + 16 * TL::X_ROW);
                     acc3[c] = mma_bf16(vl, akh, acc3[c]);
                     acc3[c] = mma_bf16(vh, akl, acc3[c]);
+                    acc3[c] = mma_bf16(vm, akm, acc3[c]);
+                    acc3[c] = mma_bf16(vm, akh, acc3[c]);
+                    acc3[c] = mma_bf16(vh, akm, acc3[c]);
                     acc3[c] = mma_bf16(vh, akh, acc3[c]);
                 }
             }
