@@ -162,6 +162,20 @@ struct RowTile {
     }
 };
 
+// every value of the rows a RowTile holds -> the sum of its two bf16 pieces (head and rounded rest)
+template <int ROWS, int W>
+__device__ __forceinline__ void round_to_pieces2(RowTile<ROWS, W>& t) {
+#pragma unroll
+    for (int j = 0; j < RowTile<ROWS, W>::N; ++j) {
+        uint2 h, l;
+        split2_4(t.r[j], h, l);
+        t.r[j] = floatx4{__uint_as_float(h.x << 16) + __uint_as_float(l.x << 16),
+                         __uint_as_float(h.x & 0xffff0000u) + __uint_as_float(l.x & 0xffff0000u),
+                         __uint_as_float(h.y << 16) + __uint_as_float(l.y << 16),
+                         __uint_as_float(h.y & 0xffff0000u) + __uint_as_float(l.y & 0xffff0000u)};
+    }
+}
+
 // K'^T V for the global low-rank term on the bf16 matrix pipe.  stash_pieces3: the rows a RowTile holds -> three bf16
 // pieces in LDS ([h | m | l], M * 2 COLS bytes apart; rows of 2 COLS bytes in natural element order, 16-byte chunks
 // swizzled): exact to fp32.  lowrank_pieces: lacc^T[d][query] += sum_f KV[f][d] q'[query][f] from those pieces, read
@@ -537,6 +551,7 @@ void sb_kfeat_kernel(KvArgs a) {
     const float pscale = sqrtf(a.temp) * LOG2E;                      // projections come out in base-2 units
     if (c0 < c1) {
         kt.template stash<LDK>(Ks, tid);
+        if (X3 && X3_VP == 2) round_to_pieces2(vt);      // K'^T V multiplies the V the band kernel sees: its two pieces
         vt.template stash<LDV>(Vs, tid);
     }
     __syncthreads();
@@ -695,6 +710,7 @@ void sb_kfeat_kernel(KvArgs a) {
         __syncthreads();                          // everyone is done with this chunk's tiles
         if (c + 1 < c1) {
             kt.template stash<LDK>(Ks, tid);
+            if (X3 && X3_VP == 2) round_to_pieces2(vt);      // K'^T V multiplies the V the band kernel sees: its two pieces
             vt.template stash<LDV>(Vs, tid);
         }
         __syncthreads();                          // next tile visible; Fs and red free again
