@@ -162,6 +162,15 @@ struct RowTile {
     }
 };
 
+// a value as the bfloat16 kernels see it: rounded to bf16.  Every product of a feature -- the overlap inside the band,
+// K'^T V, sum K', q'.sum K', the global low-rank term -- must use the same rounded value, or the band's low-rank part and
+// the global term no longer cancel to more than three digits.
+__device__ __forceinline__ float bf16_round(float x) { return bf16_to_f32(f32_to_bf16(x)); }
+__device__ __forceinline__ floatx4 bf16_round(floatx4 x) {
+    floatx4 r = {bf16_round(x[0]), bf16_round(x[1]), bf16_round(x[2]), bf16_round(x[3])};
+    return r;
+}
+
 // every value of the rows a RowTile holds -> the sum of its two bf16 pieces (head and rounded rest)
 template <int ROWS, int W>
 __device__ __forceinline__ void round_to_pieces2(RowTile<ROWS, W>& t) {
@@ -298,7 +307,11 @@ __device__ __forceinline__ void sb_combine_body(float* wgt, const float* kv_part
                 kv[(long)bh * M * D + r * D + d] = acc[i];
                 if (kvt) {      // bf16 copy for the bf16 band kernel: [d][slot], feature r in the k-slot order of its MFMA
                     const int c = r >> 4, slot = 32 * (c >> 1) + 8 * ((r >> 2) & 3) + 4 * (c & 1) + (r & 3);
-                    kvt[(long)bh * M * D + d * M + slot] = f32_to_bf16(acc[i]);
+                    // two pieces, M D elements apart: the term cancels against the band's low-rank part, and one bf16
+                    // (three digits) of it would show in the result
+                    const uint16_t hi = f32_to_bf16(acc[i]);
+                    kvt[(long)bh * 2 * M * D + d * M + slot] = hi;
+                    kvt[(long)bh * 2 * M * D + (long)M * D + d * M + slot] = f32_to_bf16(acc[i] - bf16_to_f32(hi));
                 }
             }
         } else {
@@ -526,6 +539,7 @@ void sb_kfeat_kernel(KvArgs a) {
                     fn[i] = ok ? __expf(-qf[fb][i] - qmax) : 0.f;
                 }
                 if (X3) { fp = quant16(fp); fn = quant16(fn); }
+                if (sizeof(T) == 2) { fp = bf16_round(fp); fn = bf16_round(fn); }
                 *reinterpret_cast<floatx4*>(dst + 16 * fb + 4 * g) = fp;
                 *reinterpret_cast<floatx4*>(dst + MH + 16 * fb + 4 * g) = fn;
             }
@@ -668,6 +682,7 @@ void sb_kfeat_kernel(KvArgs a) {
                     fn[i] = ok ? __builtin_amdgcn_exp2f(-dd[fb][i] + off) : 0.f;
                 }
                 if (X3) { fp = quant16(fp); fn = quant16(fn); }     // every later use sees the rounded features
+                if (sizeof(T) == 2) { fp = bf16_round(fp); fn = bf16_round(fn); }
                 ksp[fb] = ksp[fb] * rescale + fp;
                 ksn[fb] = ksn[fb] * rescale + fn;
                 *reinterpret_cast<floatx4*>(frow_s + 16 * fb + 4 * g) = fp;
@@ -1374,14 +1389,14 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const float keep = (16 * fb + 4 * g + i < a.mh_valid) ? 1.f : 0.f;
-                qf[fb][i] = keep * __builtin_amdgcn_exp2f((dd[i] - qmax) * LOG2E);
-                qf[FB + fb][i] = keep * __builtin_amdgcn_exp2f((-dd[i] - qmax) * LOG2E);
+                qf[fb][i] = keep * bf16_round(__builtin_amdgcn_exp2f((dd[i] - qmax) * LOG2E));
+                qf[FB + fb][i] = keep * bf16_round(__builtin_amdgcn_exp2f((-dd[i] - qmax) * LOG2E));
             }
         }
         __syncthreads();                 // the projection rows are dead; the tile buffers may overwrite them
     }
     FLY_PROF(1);
-    // normaliser of the global low-rank term, from the fp32 features
+    // normaliser of the global low-rank term, from the features as the overlap product sees them (bf16 values)
     float qk1 = 0.f;
     if (lowrank_here) {
 #pragma unroll
@@ -1583,20 +1598,24 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
     if (lowrank_here) {
         uint16_t* KVt = lds;
         // written by the combine kernel as bf16 [d][slot]: a plain copy in 16-byte pieces
-        const uint16_t* kvg = reinterpret_cast<const uint16_t*>(a.kvt) + (long)bh * M * D;
         constexpr int KVC = D * M / 8;
 #pragma unroll
-        for (int j = 0; j < (KVC + NT - 1) / NT; ++j) {
-            const int idx = tid + NT * j, d = idx / (M / 8), c8 = idx % (M / 8);
-            if (KVC % NT == 0 || idx < KVC)
-                *reinterpret_cast<uint4*>(KVt + d * LDKV + 8 * c8) = *reinterpret_cast<const uint4*>(kvg + (long)d * M + 8 * c8);
+        for (int piece = 1; piece >= 0; --piece) {       // the rest first, then the head (two bf16 pieces of K'^T V)
+            const uint16_t* kvg = reinterpret_cast<const uint16_t*>(a.kvt) + ((long)bh * 2 + piece) * M * D;
+            if (piece == 0) __syncthreads();             // the first piece has been read
+#pragma unroll
+            for (int j = 0; j < (KVC + NT - 1) / NT; ++j) {
+                const int idx = tid + NT * j, d = idx / (M / 8), c8 = idx % (M / 8);
+                if (KVC % NT == 0 || idx < KVC)
+                    *reinterpret_cast<uint4*>(KVt + d * LDKV + 8 * c8) = *reinterpret_cast<const uint4*>(kvg + (long)d * M + 8 * c8);
+            }
+            __syncthreads();
+#pragma unroll
+            for (int ks = 0; ks < M / 32; ++ks)
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+                    lacc[db] = mma_bf16(*reinterpret_cast<const uint4*>(KVt + (16 * db + r16) * LDKV + 32 * ks + 8 * g), qfb[ks], lacc[db]);
         }
-        __syncthreads();
-#pragma unroll
-        for (int ks = 0; ks < M / 32; ++ks)
-#pragma unroll
-            for (int db = 0; db < DB; ++db)
-                lacc[db] = mma_bf16(*reinterpret_cast<const uint4*>(KVt + (16 * db + r16) * LDKV + 32 * ks + 8 * g), qfb[ks], lacc[db]);
     }
     FLY_PROF(4);
     ze = group_sum(ze);
@@ -1856,7 +1875,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
                     for (int i = 0; i < 4; ++i) {
                         const float x = sg ? -dd[pb][4 * bq + i] : dd[pb][4 * bq + i];
                         const bool ok = 32 * pb + 8 * bq + 4 * h + i < a.mh_valid;
-                        f[4 * bq + i] = ok ? __builtin_amdgcn_exp2f((x - qmax) * LOG2E) : 0.f;
+                        f[4 * bq + i] = ok ? bf16_round(__builtin_amdgcn_exp2f((x - qmax) * LOG2E)) : 0.f;     // (as the operand holds it)
                         qk1 += f[4 * bq + i] * ks4[i];
                     }
                 }
@@ -2033,20 +2052,24 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
         for (int e = 0; e < 16; ++e) lacc[db][e] = 0.f;
     if (!SPLIT) {
         uint16_t* KVt = lds;
-        const uint16_t* kvg = reinterpret_cast<const uint16_t*>(a.kvt) + (long)bh * M * D;
         constexpr int KVC = D * M / 8;
+#pragma nounroll                                 // (unrolled, the copies cost the key loop registers)
+        for (int piece = 1; piece >= 0; --piece) {       // the rest first, then the head (two bf16 pieces of K'^T V)
+            const uint16_t* kvg = reinterpret_cast<const uint16_t*>(a.kvt) + ((long)bh * 2 + piece) * M * D;
+            if (piece == 0) __syncthreads();             // the first piece has been read
 #pragma unroll
-        for (int j = 0; j < (KVC + NT - 1) / NT; ++j) {
-            const int idx = tid + NT * j, d = idx / (M / 8), c8 = idx % (M / 8);
-            if (KVC % NT == 0 || idx < KVC)
-                *reinterpret_cast<uint4*>(KVt + d * LDKV + 8 * c8) = *reinterpret_cast<const uint4*>(kvg + (long)d * M + 8 * c8);
+            for (int j = 0; j < (KVC + NT - 1) / NT; ++j) {
+                const int idx = tid + NT * j, d = idx / (M / 8), c8 = idx % (M / 8);
+                if (KVC % NT == 0 || idx < KVC)
+                    *reinterpret_cast<uint4*>(KVt + d * LDKV + 8 * c8) = *reinterpret_cast<const uint4*>(kvg + (long)d * M + 8 * c8);
+            }
+            __syncthreads();
+#pragma unroll
+            for (int s = 0; s < FS; ++s)
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+                    lacc[db] = mma32_bf16(*reinterpret_cast<const uint4*>(KVt + (32 * db + c) * LDKV + 16 * s + 8 * h), qfb[s], lacc[db]);
         }
-        __syncthreads();
-#pragma unroll
-        for (int s = 0; s < FS; ++s)
-#pragma unroll
-            for (int db = 0; db < DB; ++db)
-                lacc[db] = mma32_bf16(*reinterpret_cast<const uint4*>(KVt + (32 * db + c) * LDKV + 16 * s + 8 * h), qfb[s], lacc[db]);
     }
     ze = pair32_sum(ze);
     zp = pair32_sum(zp);
@@ -2278,17 +2301,25 @@ __global__ __launch_bounds__(NT) void sb_kfeat_bf16_kernel(KvArgs a) {
             for (int sg = 0; sg < 2; ++sg) {
 #pragma unroll
                 for (int db = 0; db < DB; ++db) kvacc[fi][sg][db] *= rescale;
-                floatx4 fv[KBN];
+                // the features as the bf16 pairs every later product reads; their sum is taken from
+                // the same rounded values, so that numerator and normaliser see one set of features
+                uint32_t fp[KBN][2];
                 float tot = 0.f;
 #pragma unroll
-                for (int kb = 0; kb < KBN; ++kb)
+                for (int kb = 0; kb < KBN; ++kb) {
+                    float f[4];
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         const bool ok = live && fvalid && (s_base + 16 * kb + 4 * g + i) < len;
                         const float x = sg ? -dd[fi][kb][i] : dd[fi][kb][i];
-                        fv[kb][i] = ok ? __builtin_amdgcn_exp2f(x - dg[kb][i] - lnm_half2 - new_max) : 0.f;
-                        tot += fv[kb][i];
+                        f[i] = ok ? __builtin_amdgcn_exp2f(x - dg[kb][i] - lnm_half2 - new_max) : 0.f;
                     }
+                    fp[kb][0] = pack_bf16x2(f[0], f[1]);
+                    fp[kb][1] = pack_bf16x2(f[2], f[3]);
+#pragma unroll
+                    for (int h = 0; h < 2; ++h)
+                        tot += __uint_as_float(fp[kb][h] << 16) + __uint_as_float(fp[kb][h] & 0xffff0000u);
+                }
                 if (sg) ksum_n[fi] += tot; else ksum_p[fi] += tot;
                 if ((w + 4 * fi) < FB) {
                     const int bm = sg * FB + w + 4 * fi;
@@ -2296,14 +2327,13 @@ __global__ __launch_bounds__(NT) void sb_kfeat_bf16_kernel(KvArgs a) {
 #pragma unroll
                     for (int kb = 0; kb < KBN; ++kb)
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) Fo[(16 * kb + 4 * g + i) * LDFO + pos] = f32_to_bf16(fv[kb][i]);
+                        for (int i = 0; i < 4; ++i)
+                            Fo[(16 * kb + 4 * g + i) * LDFO + pos] = (uint16_t)(fp[kb][i >> 1] >> (16 * (i & 1)));
                 }
                 // KV[feature][d] += sum_keys F[key][feature] V[key][d], 32 keys per MFMA step
 #pragma unroll
                 for (int t = 0; t < CH / 32; ++t) {
-                    const floatx4 f0 = fv[2 * t], f1 = fv[2 * t + 1];
-                    const uint4 fa = make_uint4(pack_bf16x2(f0[0], f0[1]), pack_bf16x2(f0[2], f0[3]),
-                                                pack_bf16x2(f1[0], f1[1]), pack_bf16x2(f1[2], f1[3]));
+                    const uint4 fa = make_uint4(fp[2 * t][0], fp[2 * t][1], fp[2 * t + 1][0], fp[2 * t + 1][1]);
 #pragma unroll
                     for (int db = 0; db < DB; ++db)
                         kvacc[fi][sg][db] = mma_bf16(fa, *reinterpret_cast<const uint4*>(Vt + (16 * db + r16) * LDVT + 32 * t + 8 * g),
@@ -4354,7 +4384,7 @@ SbWorkspace sb_workspace(int B, int H, int T, int S, int E, int mh, int local_co
     w.ksum = take(bh * m * 4);
     w.kmax = take(bh * 4);
     w.vt = take(dtype == F32 ? bh * nc * 2 * (128 * (size_t)E + 64 * (size_t)X3_VP * (size_t)E) : bh * nc * CH * E * 2);
-    w.kvt = take(dtype == F32 ? 0 : bh * E * m * 2);
+    w.kvt = take(dtype == F32 ? 0 : bh * E * m * 2 * 2);      // two bf16 pieces
     w.part_ws = take(w.n_parts > 1 ? bh * n_qt * w.n_parts * TQ * (E + NSTAT) * 4 : 0);
     w.qfeat = take(w.n_parts > 1 ? bh * T * m * 4 : 0);
     w.q_lsq = take(w.n_parts > 1 ? bh * T * 4 : 0);

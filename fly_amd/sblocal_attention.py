@@ -91,7 +91,7 @@ class SBLocalPlan:
         if dtype == torch.bfloat16:
             # bf16 inputs: V per 32-key tile and K'^T V in the operand order of the bf16 MFMA (opaque)
             self.vt = torch.empty(B, H, self.n_chunks * 64, dim, dtype=dtype, device=device)
-            self.kvt = torch.empty(B, H, dim, m, dtype=dtype, device=device)
+            self.kvt = torch.empty(B, H, 2, dim, m, dtype=dtype, device=device)     # (two bf16 pieces)
         # with several parts per query tile the key pass also computes the query features, once
         self.part_ws = self.qfeat = self.q_lsq = None
         if self.n_parts > 1:

@@ -57,7 +57,7 @@ int flyhip_sb_plan(int B, int H, int T, int S, int local_context,
  * -t|q|^2/2 + rowmax - log(m)/2.  With q given, kv / ksum / kmax are NOT written: the partial
  * reductions (kv_part, part_max) are combined inside flyhip_sblocal_fwd's launch instead, which
  * saves a launch on problems this small.
- * bfloat16 inputs: vt (B,H,n_chunks*64,D) bf16 and kvt (B,H,D,m) bf16, opaque scratch for
+ * bfloat16 inputs: vt (B,H,n_chunks*64,D) bf16 and kvt (B,H,2,D,m) bf16 (K'^T V in two bf16 pieces), opaque scratch for
  * flyhip_sblocal_fwd -- V per 32-key tile and K'^T V, transposed into the operand order of the bf16
  * MFMA.
  * float inputs: vt may be NULL (all products on the fp32 matrix pipe, kfeat holds fp32 features).
