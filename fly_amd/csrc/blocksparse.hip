@@ -1188,21 +1188,36 @@ __device__ __forceinline__ float group_max_finite(float v) {
     rows_pair32(v, a, b); return max2_finite(a, b);
 }
 
-constexpr int ATT_LDT = 40;     // LDS row stride of the transposed V tile in elements (32 slots + 8)
-
+#ifndef FLY_ATTN_EXP
+#define FLY_ATTN_EXP 0
+#endif
+// LDS image of a block-column's K and V tiles: rows of 2 D bytes without padding (a wave's direct-to-LDS load
+// fills 1024 consecutive bytes), 16-byte chunks permuted within a row so that the fragment reads spread over the
+// banks: the eight lanes of a 16-byte K read (eight consecutive keys, one chunk) and the sixteen lanes of a
+// transposing V read (four consecutive keys, 32 bytes each) then cover a 128-byte line exactly.  Both maps are
+// their own inverses.  CPR = chunks per row.
+template <int CPR> __device__ __forceinline__ int attn_kslot(int row, int c) {
+    constexpr int RPL = CPR >= 8 ? 1 : 8 / CPR;           // rows per 128-byte line
+    return c ^ ((row / RPL) & (CPR - 1));
+}
+template <int CPR> __device__ __forceinline__ int attn_vslot(int row, int c) {
+    constexpr int RPL = CPR >= 8 ? 1 : 8 / CPR;
+    return c ^ ((((row / RPL) & 3) & (CPR / 2 - 1)) << 1);
+}
 template <typename T, int KS, int NW, bool MASKED>     // head dim 32*KS, NW block-rows (waves) per workgroup
 __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
-    constexpr int D = 32 * KS, LDK = D + 8, LDT = ATT_LDT, DT = D / 16, NTH = 64 * NW;
+    constexpr int D = 32 * KS, DT = D / 16, RB = 2 * D;   // RB: bytes of a tile row
+    constexpr int CP = KS <= 2 ? 4 : 2;                   // block-columns per step (what 64 KB of LDS hold twice over)
     constexpr int CPR = D / 8;                            // 16-byte chunks per tile row
-    constexpr int NCH = (64 * CPR + NTH - 1) / NTH;       // chunks per thread (K and V tiles together)
+    constexpr int COLB = 64 * RB;                         // one column's image: rows 0..31 keys of K, 32..63 the same keys of V
+    constexpr int U = COLB / 1024, NCH = (U + NW - 1) / NW;      // wave loads per column, and per wave
     constexpr float LOG2E = 1.4426950408889634f;
     // The running reference exponent of a query is only raised (and its accumulators rescaled) when
     // a block's maximum exceeds it by more than LAZY binary orders of magnitude; until then the
     // probabilities may exceed 1 (by at most 2^LAZY), which fp32 sums and 2-byte operands hold
     // without loss, and the result is the same quotient.
     constexpr float LAZY = 8.f;
-    __shared__ __attribute__((aligned(16))) uint16_t ks_[2][32 * LDK];
-    __shared__ __attribute__((aligned(16))) uint16_t vs_[3][D * LDT];
+    __shared__ __attribute__((aligned(1024))) char tiles[2][CP][COLB];
     const int tid = threadIdx.x, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     int unit, grp;
@@ -1224,44 +1239,22 @@ __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) fq[qt][ks] = *reinterpret_cast<const uintx4*>(qp + 16 * qt * a.q_sm + 32 * ks);
 
-    // staging: chunk c = tid + NTH i (16 bytes).  The first 32 CPR chunks are the K tile, row-major
-    // (row c / CPR); the rest are the V tile with the key running fastest over the lanes (row c % 32),
-    // so that the 2-byte stores that transpose it spread over the LDS banks.
-    uintx4 reg[NCH];
-    const T* src[NCH];           // the chunk's address in block-column 0
+    // staging: wave load x = w + NW i of a column fills bytes 1024 x .. of its image; this lane's 16 of them are
+    // chunk slot `p` of image row `row`
+    const T* src[NCH];           // the lane's chunk in block-column 0
     long src_step[NCH];          // elements from one block-column to the next (wave-uniform)
-    int dst[NCH];                // the chunk's LDS position in buffer 0 (K: elements of ks_, V: of vs_)
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
-        const int c = tid + NTH * i;
-        const bool is_k = 64 * w + NTH * i < 32 * CPR;      // whole waves stage K or V
-        if (is_k) {
-            src[i] = kz + (long)(c / CPR) * a.k_sn + 8 * (c % CPR);
-            src_step[i] = 32 * a.k_sn;
-            dst[i] = (c / CPR) * LDK + 8 * (c % CPR);
-        } else {
-            const int row = c & 31, ch = (c - 32 * CPR) >> 5;
-            src[i] = vz + (long)row * a.v_sn + 8 * ch;
-            src_step[i] = 32 * a.v_sn;
-            dst[i] = 8 * ch * LDT + 8 * ((row >> 2) & 3) + 4 * (row >> 4) + (row & 3);
-        }
+        const int pos = 1024 * (w + NW * i) + 16 * lane, row = (pos / RB) & 63, p = (pos % RB) / 16;
+        const bool is_k = 1024 * (w + NW * i) < 32 * RB;    // whole wave loads are K or V
+        src[i] = is_k ? kz + (long)row * a.k_sn + 8 * attn_kslot<CPR>(row, p)
+                      : vz + (long)(row - 32) * a.v_sn + 8 * attn_vslot<CPR>(row - 32, p);
+        src_step[i] = is_k ? 32 * a.k_sn : 32 * a.v_sn;
     }
-    auto fetch = [&](int inner) __attribute__((always_inline)) {
+    auto fetch = [&](int j, int stage, int inner) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < NCH; ++i)
-            if (64 * w + NTH * i < 64 * CPR) reg[i] = *reinterpret_cast<const uintx4*>(src[i] + inner * src_step[i]);
-    };
-    auto stash = [&](int kbuf, int vbuf) __attribute__((always_inline)) {
-#pragma unroll
-        for (int i = 0; i < NCH; ++i) {
-            if (64 * w + NTH * i < 32 * CPR) {
-                *reinterpret_cast<uintx4*>(&ks_[kbuf][dst[i]]) = reg[i];
-            } else if (64 * w + NTH * i < 64 * CPR) {
-#pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    vs_[vbuf][dst[i] + e * LDT] = (uint16_t)(reg[i][e >> 1] >> (16 * (e & 1)));
-            }
-        }
+            if (U % NW == 0 || w + NW * i < U) dma_to_lds(src[i] + inner * src_step[i], tiles[stage][j] + 1024 * (w + NW * i));
     };
 
     floatx4 o[DT][2];                                     // O^T[d = 16dt + 4g + i][query 16qt + r16]
@@ -1273,11 +1266,11 @@ __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
     const uintx4 ones = {one2, one2, one2, one2};
     const float scale2 = a.scale * LOG2E;
 
-    // S^T[key 16kt + 4g + i][query 16qt + r16] of the tile in K buffer `buf`
+    // S^T[key 16kt + 4g + i][query 16qt + r16] of the K tile at `tile`
     floatx4 sc[2][2];
     floatx4 amk[2][2];                                    // the attention-mask entries of sc (asked for with the scores)
     const float* amrow = (MASKED && a.am) ? a.am + (long)(min(bi, a.brows_per_head - 1) * 32 + r16) * a.am_stride + 4 * g : nullptr;
-    auto score = [&](int buf, int inner) __attribute__((always_inline)) {
+    auto score = [&](const char* tile, int inner) __attribute__((always_inline)) {
         if (MASKED && amrow) {
 #pragma unroll
             for (int kt = 0; kt < 2; ++kt)
@@ -1285,13 +1278,12 @@ __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
                 for (int qt = 0; qt < 2; ++qt)
                     amk[kt][qt] = *reinterpret_cast<const floatx4*>(amrow + 16 * qt * a.am_stride + (long)inner * 32 + 16 * kt);
         }
-        const uint16_t* kp = ks_[buf];
         uintx4 fk[2][KS];
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks)
-                fk[kt][ks] = *reinterpret_cast<const uintx4*>(kp + (16 * kt + r16) * LDK + 32 * ks + 8 * g);
+                fk[kt][ks] = *reinterpret_cast<const uintx4*>(tile + (16 * kt + r16) * RB + 16 * attn_kslot<CPR>(16 * kt + r16, 4 * ks + g));
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
@@ -1301,12 +1293,17 @@ __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
                 for (int ks = 0; ks < KS; ++ks) sc[kt][qt] = mma32<T>(fk[kt][ks], fq[qt][ks], sc[kt][qt]);
             }
     };
-    // online softmax of sc and O^T += V^T P with the tile in V buffer `buf`; `inner` = its block-column
-    auto soft_pv = [&](int buf, int inner) __attribute__((always_inline)) {
-        const uint16_t* vp = vs_[buf];
+    // online softmax of sc and O^T += V^T P with the V tile that follows the K tile at `tile`; `inner` = its block-column
+    auto soft_pv = [&](const char* tile, int inner) __attribute__((always_inline)) {
+        // A operand: column d = 16dt + r16 of V, keys 4g .. 4g+3 and 16+4g .. 16+4g+3
+        const int vrow = 4 * g + (r16 >> 2);
+        const char* vp = tile + (32 + vrow) * RB + 8 * (r16 & 1);
         uintx4 fv[DT];
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) fv[dt] = *reinterpret_cast<const uintx4*>(vp + (16 * dt + r16) * LDT + 8 * g);
+        for (int dt = 0; dt < DT; ++dt) {
+            const char* p0 = vp + 16 * attn_vslot<CPR>(vrow, 2 * dt + ((r16 & 3) >> 1));
+            fv[dt] = lds_read_tr8(p0, p0 + 16 * RB);
+        }
         uintx4 pb[2];
         if (!MASKED) {
             // scale > 0 and no mask: the maximum is taken on the raw scores and the scale rides in
@@ -1375,40 +1372,54 @@ __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
     };
 
     // The index lists are read two steps (block-column) and one step (presence) ahead of their use,
-    // so that no step waits for a table load.
-    // The upper half of the waves runs half a step behind the lower half: in iteration s an early
-    // wave does scores(s), softmax(s), PV(s); a late wave does softmax(s-1), PV(s-1), scores(s).
-    // A SIMD holds one wave of each kind per workgroup, so one's matrix phase coincides with the
-    // other's vector phase instead of both queueing for the same pipe.  K tiles are double-buffered,
-    // V tiles (still read one iteration later by the late waves) triple-buffered.
-    const bool late = w >= NW / 2;
-    int inner_cur = n > 0 ? a.uni_inner[p0] : 0, inner_n1 = n > 1 ? a.uni_inner[p0 + 1] : 0, inner_prev = 0;
-    int blk_cur = n > 0 ? a.uni_blk[(long)p0 * NW + w] : -1;
-    bool had_prev = false;
+    // so that no step waits for a table load.  A step: ask for the next step's tiles (they go into the
+    // other stage, which every wave has finished reading before the last barrier), work through this
+    // step's columns, wait for the own loads, barrier.
+    const int n_steps = (n + CP - 1) / CP;
+    int inner_cur[CP], inner_n1[CP], blk_cur[CP];
+#pragma unroll
+    for (int j = 0; j < CP; ++j) {
+        inner_cur[j] = j < n ? a.uni_inner[p0 + j] : 0;
+        inner_n1[j] = CP + j < n ? a.uni_inner[p0 + CP + j] : 0;
+        blk_cur[j] = j < n ? a.uni_blk[(long)(p0 + j) * NW + w] : -1;
+    }
     if (n > 0) {
-        fetch(inner_cur);
-        stash(0, 0);
+#pragma unroll
+        for (int j = 0; j < CP; ++j)
+            if (j < n) fetch(j, 0, inner_cur[j]);
     }
     drain_loads();
     __syncthreads();
-    int vb = 0;                                           // V buffer of step s (s % 3)
-    for (int s = 0; s <= n; ++s) {
-        const int inner_n2 = s + 2 < n ? a.uni_inner[p0 + s + 2] : 0;
-        const int blk_n1 = s + 1 < n ? a.uni_blk[(long)(p0 + s + 1) * NW + w] : -1;
-        const bool present = s < n && have_row && blk_cur >= 0;
-        const int vb_next = vb == 2 ? 0 : vb + 1, vb_prev = vb == 0 ? 2 : vb - 1;
-        if (s + 1 < n) fetch(inner_n1);
-        if (late && had_prev) soft_pv(vb_prev, inner_prev);
-        if (present) score(s & 1, inner_cur);
-        if (!late && present) soft_pv(vb, inner_cur);
-        if (s + 1 < n) stash((s + 1) & 1, vb_next);
-        had_prev = present;
-        inner_prev = inner_cur;
-        inner_cur = inner_n1;
-        inner_n1 = inner_n2;
-        blk_cur = blk_n1;
-        vb = vb_next;
+    for (int st = 0; st < n_steps; ++st) {
+        const int s1 = CP * (st + 1), s2 = CP * (st + 2);
+        int inner_n2[CP], blk_n1[CP];
+#pragma unroll
+        for (int j = 0; j < CP; ++j) {
+            inner_n2[j] = s2 + j < n ? a.uni_inner[p0 + s2 + j] : 0;
+            blk_n1[j] = s1 + j < n ? a.uni_blk[(long)(p0 + s1 + j) * NW + w] : -1;
+        }
+#if !(FLY_ATTN_EXP & 1)
+#pragma unroll
+        for (int j = 0; j < CP; ++j)
+            if (s1 + j < n) fetch(j, (st + 1) & 1, inner_n1[j]);
+#endif
+#pragma unroll
+        for (int j = 0; j < CP; ++j) {
+            if (have_row && blk_cur[j] >= 0) {
+                score(tiles[st & 1][j], inner_cur[j]);
+                soft_pv(tiles[st & 1][j], inner_cur[j]);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < CP; ++j) {
+            inner_cur[j] = inner_n1[j];
+            inner_n1[j] = inner_n2[j];
+            blk_cur[j] = blk_n1[j];
+        }
+#if !(FLY_ATTN_EXP & 2)
+        drain_loads();                                    // this wave's part of the next step's tiles has landed
         __syncthreads();
+#endif
     }
     if (!have_row) return;
     T* op = reinterpret_cast<T*>(a.out) + z * a.o_sz + head * a.o_sh;

@@ -309,6 +309,17 @@ __device__ __forceinline__ void split3_4(floatx4 x, uint2& h, uint2& m, uint2& l
     split2_4(r, m, l);
 }
 
+// One wave's 1024 bytes straight from global memory into LDS (lane l's 16 bytes land at wave_base + 16 l), issued as
+// assembly: the compiler then does not know of a transfer in flight, and does not drain the load counter in front of
+// LDS reads of the other stage (it does so before every transposing read, whose address it cannot tell from the
+// transfer's destination, which would leave the prefetch a fraction of a tile to arrive in).  The caller waits for
+// its transfers (drain_loads) before the barrier that publishes them.
+__device__ __forceinline__ void dma_to_lds(const void* lane_src, const char* wave_base) {
+    typedef __attribute__((address_space(3))) const char* lds_ptr;
+    const uint32_t base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr)wave_base);
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(lane_src), "s"(base) : "m0", "memory");
+}
+
 // Transposed operand reads (ds_read_b64_tr_b16): within each group of 16 lanes, lane s passes the address of four
 // consecutive 16-bit elements -- row s / 4, columns 4 (s % 4) .. + 3 of a 4 x 16 block -- and lane l receives column l of
 // the four rows.

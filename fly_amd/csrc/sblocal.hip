@@ -1703,19 +1703,18 @@ struct B32Loads {
         }
     }
     __device__ __forceinline__ void issue(char* st, int w, bool last, const char* kg, const char* fg, const char* vg) const {
-        typedef __attribute__((address_space(3))) void* lds_ptr;
 #pragma unroll
         for (int x = 0; x < NKL; ++x)
             if (K_BYTES / 1024 % NW == 0 || NW * x + w < K_BYTES / 1024)
-                __builtin_amdgcn_global_load_lds(kg + (last ? kgo_last[x] : kgo[x]), (lds_ptr)(st + 1024 * (NW * x + w)), 16, 0, 0);
+                dma_to_lds(kg + (last ? kgo_last[x] : kgo[x]), st + 1024 * (NW * x + w));
 #pragma unroll
         for (int x = 0; x < NFL; ++x)
             if (F_BYTES / 1024 % NW == 0 || NW * x + w < F_BYTES / 1024)
-                __builtin_amdgcn_global_load_lds(fg + fgo[x], (lds_ptr)(st + K_BYTES + 1024 * (NW * x + w)), 16, 0, 0);
+                dma_to_lds(fg + fgo[x], st + K_BYTES + 1024 * (NW * x + w));
 #pragma unroll
         for (int x = 0; x < NVL; ++x)
             if (V_BYTES / 1024 % NW == 0 || NW * x + w < V_BYTES / 1024)
-                __builtin_amdgcn_global_load_lds(vg + vgo[x], (lds_ptr)(st + K_BYTES + F_BYTES + 1024 * (NW * x + w)), 16, 0, 0);
+                dma_to_lds(vg + vgo[x], st + K_BYTES + F_BYTES + 1024 * (NW * x + w));
     }
 };
 

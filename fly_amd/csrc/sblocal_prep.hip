@@ -417,16 +417,12 @@ struct BwdX3Args {
 // the 256 bytes behind the MAIN ones (log Z and c of the tile's queries; a full wave load, lanes 16.. repeat them)
 template <int MAIN, bool TAIL>
 __device__ __forceinline__ void bwd_tile_to_lds(const char* src, char* dst, int tid) {
-    typedef __attribute__((address_space(3))) void* lds_ptr;
-    const int w = tid >> 6, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
 #pragma unroll
-    for (int j = 0; j < MAIN / 4096; ++j)
-        __builtin_amdgcn_global_load_lds(src + 4096 * j + 16 * tid, (lds_ptr)(dst + 4096 * j + 1024 * w), 16, 0, 0);
+    for (int j = 0; j < MAIN / 4096; ++j) dma_to_lds(src + 4096 * j + 16 * tid, dst + 4096 * j + 1024 * w);
     constexpr int FULL = MAIN / 4096 * 4096;
-    if (MAIN % 4096 != 0 && w < (MAIN % 4096) / 1024)
-        __builtin_amdgcn_global_load_lds(src + FULL + 16 * tid, (lds_ptr)(dst + FULL + 1024 * w), 16, 0, 0);
-    if (TAIL && w == 0)
-        __builtin_amdgcn_global_load_lds(src + MAIN + 16 * (lane & 15), (lds_ptr)(dst + MAIN), 16, 0, 0);
+    if (MAIN % 4096 != 0 && w < (MAIN % 4096) / 1024) dma_to_lds(src + FULL + 16 * tid, dst + FULL + 1024 * w);
+    if (TAIL && w == 0) dma_to_lds(src + MAIN + 16 * (lane & 15), dst + MAIN);
 }
 
 // LDS bytes of the finishing step: gmat (M, D) and the projection (at least 32 rows, E) in three bf16 pieces, gvec
