@@ -1188,9 +1188,6 @@ __device__ __forceinline__ float group_max_finite(float v) {
     rows_pair32(v, a, b); return max2_finite(a, b);
 }
 
-#ifndef FLY_ATTN_EXP
-#define FLY_ATTN_EXP 0
-#endif
 // LDS image of a block-column's K and V tiles: rows of 2 D bytes without padding (a wave's direct-to-LDS load
 // fills 1024 consecutive bytes), 16-byte chunks permuted within a row so that the fragment reads spread over the
 // banks: the eight lanes of a 16-byte K read (eight consecutive keys, one chunk) and the sixteen lanes of a
@@ -1398,11 +1395,9 @@ __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
             inner_n2[j] = s2 + j < n ? a.uni_inner[p0 + s2 + j] : 0;
             blk_n1[j] = s1 + j < n ? a.uni_blk[(long)(p0 + s1 + j) * NW + w] : -1;
         }
-#if !(FLY_ATTN_EXP & 1)
 #pragma unroll
         for (int j = 0; j < CP; ++j)
             if (s1 + j < n) fetch(j, (st + 1) & 1, inner_n1[j]);
-#endif
 #pragma unroll
         for (int j = 0; j < CP; ++j) {
             if (have_row && blk_cur[j] >= 0) {
@@ -1416,10 +1411,8 @@ __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
             inner_n1[j] = inner_n2[j];
             blk_cur[j] = blk_n1[j];
         }
-#if !(FLY_ATTN_EXP & 2)
         drain_loads();                                    // this wave's part of the next step's tiles has landed
         __syncthreads();
-#endif
     }
     if (!have_row) return;
     T* op = reinterpret_cast<T*>(a.out) + z * a.o_sz + head * a.o_sh;

@@ -3032,6 +3032,21 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
         for (int j = 0; j < NF; ++j)
             if (F_EXACT || tid + NT * j < TL::F_BYTES / 16) df[tid + NT * j] = rf[j];
     };
+    // the tiles after the first go straight from global memory into the stage (the first is asked for here, through
+    // registers, because the stages hold the projection until the query features are done)
+    auto transfer = [&](int kt, int stage) __attribute__((always_inline)) {
+        const char* gk = kv_img + (long)kt * TL::KV_BYTES;
+        const char* gf = f_img + (long)kt * TL::F_BYTES;
+        const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+#pragma unroll
+        for (int j = 0; j < NKV; ++j)
+            if (KV_EXACT || tid + NT * j < TL::KV_BYTES / 16)
+                dma_to_lds(gk + 16 * (tid + NT * j), lds + stage * TL::BYTES + 16 * (NT * j + 64 * wv));
+#pragma unroll
+        for (int j = 0; j < NF; ++j)
+            if (F_EXACT || tid + NT * j < TL::F_BYTES / 16)
+                dma_to_lds(gf + 16 * (tid + NT * j), lds + stage * TL::BYTES + TL::KV_BYTES + 16 * (NT * j + 64 * wv));
+    };
     if (kt_lo < kt_hi) fetch(kt_lo);
     const float* csp = a.chunk_scale + (long)bh * a.n_chunks;
     float cscale = (kt_lo < kt_hi) ? csp[kt_lo * TK / CH] : 0.f;
@@ -3143,8 +3158,8 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
         const char* st = lds + cur * TL::BYTES;
         const bool more = kt + 1 < kt_hi;
         float cscale_next = cscale;
-        if (more) {                                      // next tile's loads fly during the MFMAs
-            fetch(kt + 1);
+        if (more) {                                      // next tile's transfer flies during the MFMAs (every wave is past
+            transfer(kt + 1, cur ^ 1);                   // the barrier that ended the last use of that stage)
             cscale_next = csp[(s_base + TK) / CH];
         }
         const float wc = __builtin_amdgcn_exp2f((cscale - kmax) * LOG2E);
@@ -3300,7 +3315,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
             for (int db = 0; db < DB; ++db) oacc[db] = mma_bf16(vf[db][0], ph, oacc[db]);
         }
         FLY_PROF2(stamp, 6);
-        if (more) stash(cur ^ 1);
+        drain_loads();                                   // this wave's share of the next tile is in LDS
         cscale = cscale_next;
         FLY_PROF2(stamp, 7);
         __syncthreads();
