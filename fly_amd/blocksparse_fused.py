@@ -61,6 +61,10 @@ class fused_attention:
             attn_mask = attn_mask.to(device=q.device, dtype=torch.float32).contiguous()
             am, am_stride = attn_mask.data_ptr(), attn_mask.stride(0)
         uni_ptr, uni_inner, uni_blk = self.make_lut(q.device)
+        if uni_inner.numel() == 0:                      # a layout without blocks: every row is empty
+            out = torch.zeros((Z, p * 32, H, D), dtype=q.dtype, device=q.device).permute(0, 2, 1, 3)
+            lse2 = torch.full((Z, H, p * 32), float('inf'), dtype=torch.float32, device=q.device)
+            return (out, lse2) if return_lse else out
         out = torch.empty((Z, p * 32, H, D), dtype=q.dtype, device=q.device).permute(0, 2, 1, 3)
         # base-2 log of every row's softmax denominator (+inf for a row without a finite score): what a
         # backward pass needs to form the probabilities again

@@ -2136,8 +2136,10 @@ FLY_B32_INST(64, 64) FLY_B32_INST(64, 128) FLY_B32_INST(64, 256)
 // Wave w owns the projection rows of blocks w, w+4, ... (both signs of each), for all 64 keys of
 // the chunk.  The feature scratch for the band kernel ([key][k-slot order]) is assembled in LDS
 // from 2-byte writes and leaves as 16-byte stores.
+// (two workgroups per compute unit: the pass streams, and one workgroup's loads in flight do not fill the memory pipe;
+//  the few registers this spills cost less than that)
 template <int E, int D, int M>
-__global__ __launch_bounds__(NT) void sb_kfeat_bf16_kernel(KvArgs a) {
+__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void sb_kfeat_bf16_kernel(KvArgs a) {
     constexpr int MH = M / 2, FB = MH / 16, DB = D / 16, KS = E / 32, KBN = CH / 16;
     constexpr int FPW = (FB + 3) / 4;                       // projection-row blocks per wave
     constexpr int LDK = E + 8, LDVT = CH + 8, LDFO = M + 8; // LDS row strides in 2-byte elements

@@ -337,6 +337,15 @@ def test_fused_attention_matches_oracle(p, r, D, rpg, dtype):
         assert rel_err(out, o3.float()) <= 2 * TOL[dtype]
 
 
+def test_fused_attention_with_an_empty_layout():
+    """No nonzero block at all: zeros (the value of a row without blocks), and +inf as the rows' log-denominator."""
+    from fly_amd.blocksparse_fused import fused_attention
+    q, k, v = (torch.randn(2, 1, 64, 32, device=DEV).bfloat16() for _ in range(3))
+    out, lse2 = fused_attention(torch.zeros(1, 2, 2, dtype=torch.long), 32)(q, k, v, 0.5, return_lse=True)
+    assert out.shape == (2, 1, 64, 32) and float(out.abs().max()) == 0.0
+    assert bool(torch.isinf(lse2).all())
+
+
 def test_blocksparse_attention_module_fused_path():
     """BlockSparseAttention.forward takes the one-kernel path for eligible calls (eval / no grad, no
     attention mask) and the three-op path otherwise; both agree with the oracle, including padded
