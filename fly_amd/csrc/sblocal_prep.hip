@@ -138,8 +138,10 @@ __global__ __launch_bounds__(PREP_NT) void sb_prep_kmax_kernel(PrepArgs a) {
     if (tid == 0) a.pmax[(long)bh * a.n_kblk + blockIdx.x] = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
 }
 
+// (at least two workgroups per compute unit: the kernel streams, and at 128 features the registers it would like to take
+//  leave room for one only; the few it spills instead cost less)
 template <int DIM, int MK>
-__global__ __launch_bounds__(PREP_NT) void sb_prep_kernel(PrepArgs a) {
+__global__ __launch_bounds__(PREP_NT) __attribute__((amdgpu_waves_per_eu(2, 8))) void sb_prep_kernel(PrepArgs a) {
     constexpr int MH = MK / 2, FB = MK / 32, RBN = MK / 16, RB = (RBN + 3) / 4, DB = DIM / 16;
     constexpr int LDF = MK + 4, LDY = DIM + 4;
     __shared__ float Fs[PREP_ROWS * LDF];         // features of the current rows
