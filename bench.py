@@ -272,11 +272,18 @@ def bench_other_configs():
     out = {}
 
     def timeit(fn, n=10, w=2):
-        for _ in range(w):
+        # warm-up by time as well as by count: the clocks take tens of milliseconds of load to settle on a workload
+        # (a 0.3 ms forward timed after two calls reads 15 - 20 % above its steady state)
+        t0 = time.perf_counter()
+        done = 0
+        while done < w or time.perf_counter() - t0 < 0.05:
             fn()
+            done += 1
+            if done % 8 == 0:
+                torch.cuda.synchronize()
         torch.cuda.synchronize()
         reps = []
-        for _ in range(3):                      # median of three timed runs of n calls (clocks settle between workloads)
+        for _ in range(3):                      # median of three timed runs of n calls
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
             for _ in range(n):

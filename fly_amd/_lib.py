@@ -17,6 +17,7 @@ c_int, c_i64, c_float, c_vp = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctyp
 SIGNATURES = {
     'flyhip_version': [],
     'flyhip_sb_plan': [c_int] * 5 + [ctypes.POINTER(c_int)] * 3,
+    'flyhip_sb_plan_for': [c_int] * 8 + [ctypes.POINTER(c_int)] * 3,
     'flyhip_sb_time_next_fwd': [c_vp, c_vp],
     'flyhip_sb_kv_reduce': [c_vp] * 14 + [c_int] + [c_i64] * 3 + [c_vp] * 2 + [c_int] * 8 + [c_i64] * 6 + [c_float, c_int, c_vp],
     'flyhip_sblocal_fwd': [c_vp] * 13 + [c_vp] * 2 + [c_int] + [c_vp] * 4 + [c_int] * 10 + [c_i64] * 12 + [c_float, c_int, c_vp],

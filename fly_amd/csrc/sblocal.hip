@@ -4198,7 +4198,11 @@ static int plan_parts(int B, int H, int T, int S, int lc) {
     return want < 1 ? 1 : (int)want;
 }
 
-static int plan(int B, int H, int S, int* n_chunks, int* n_split) {
+// workgroups of the key pass that a compute unit holds together: the fp32 pass that writes the bf16 operand images
+// (sb_kfeat_x3_kernel: more than 256 registers a lane and 108 KB of LDS) runs one, the others two
+static int key_pass_wgs_per_cu(int dtype, int E, int mh) { return (dtype == F32 && E <= 64 && 2 * mh <= 128) ? 1 : 2; }
+
+static int plan(int B, int H, int S, int wgs_per_cu, int* n_chunks, int* n_split) {
     const int nc = (S + CH - 1) / CH;
     // aim for about four workgroups per CU over the chip, at least one chunk each
     const long slots = machine().slots;
@@ -4206,14 +4210,15 @@ static int plan(int B, int H, int S, int* n_chunks, int* n_split) {
     if (want < 1) want = 1;
     if (want > nc) want = nc;
     int per = (nc + (int)want - 1) / (int)want;
-    if ((long)B * H * nc > slots) {
-        // more work than one residency round (two workgroups per CU): the pass takes about
-        // rounds x chunks per workgroup, and a round that is full costs no more than one that is not; among
-        // equals the larger share wins (fewer partial reductions to combine)
+    const long resident = (long)machine().cus * wgs_per_cu;
+    if ((long)B * H * nc > resident) {
+        // more work than one residency round: the pass takes about rounds x chunks per workgroup, and a round that
+        // is full costs no more than one that is not; among equals the larger share wins (fewer partial reductions
+        // to combine)
         long best = -1;
         for (int p = 1; p <= nc; ++p) {
             const long wgs = (long)B * H * ((nc + p - 1) / p);
-            const long cost = ((wgs + slots - 1) / slots) * p;
+            const long cost = ((wgs + resident - 1) / resident) * p;
             if (best < 0 || cost <= best) { best = cost; per = p; }
         }
     }
@@ -4264,7 +4269,15 @@ extern "C" int flyhip_sb_plan(int B, int H, int T, int S, int local_context,
     FLY_REQUIRE(B > 0 && H > 0 && T > 0 && S > 0 && local_context > 0 && n_chunks && n_split && n_parts,
                 "sb_plan: bad arguments");
     *n_parts = plan_parts(B, H, T, S, local_context);
-    return plan(B, H, S, n_chunks, n_split);
+    return plan(B, H, S, 2, n_chunks, n_split);
+}
+
+extern "C" int flyhip_sb_plan_for(int B, int H, int T, int S, int local_context, int E, int mh, int dtype,
+                                  int* n_chunks, int* n_split, int* n_parts) {
+    FLY_REQUIRE(B > 0 && H > 0 && T > 0 && S > 0 && local_context > 0 && E > 0 && mh > 0 && n_chunks && n_split && n_parts,
+                "sb_plan_for: bad arguments");
+    *n_parts = plan_parts(B, H, T, S, local_context);
+    return plan(B, H, S, key_pass_wgs_per_cu(dtype, E, mh), n_chunks, n_split);
 }
 
 static int check_sb_dims(const char* who, int E, int D, int mh, int mh_valid, int dtype,
@@ -4293,7 +4306,7 @@ extern "C" int flyhip_sb_kv_reduce(const void* k, const void* v, const float* pr
     int rc = check_sb_dims("sb_kv_reduce", E, D, mh, mh_valid, dtype, k_sb | k_sh, k_ss, v_sb | v_sh | v_ss);
     if (rc) return rc;
     int nc, ns;
-    plan(B, H, S, &nc, &ns);
+    plan(B, H, S, 2, &nc, &ns);
     FLY_REQUIRE(n_split >= 1 && n_split <= nc && n_split <= MAX_SPLIT,
                 "sb_kv_reduce: n_split=%d outside [1, min(%d, %d)]", n_split, nc, MAX_SPLIT);
     FLY_REQUIRE((long)B * H <= 65535, "sb_kv_reduce: B*H=%ld exceeds the grid limit 65535", (long)B * H);
@@ -4347,7 +4360,7 @@ static int sblocal_fwd_checked(const void* q, const void* k, const void* v, cons
                 "sblocal_fwd: n_parts > 1 needs the partial workspace, the query features and the partial "
                 "reductions (kv_part, part_max, n_split) of the key pass");
     int nc, ns;
-    plan(B, H, S, &nc, &ns);
+    plan(B, H, S, 2, &nc, &ns);
     FwdArgs a{q, k, v, proj, kfeat, chunk_scale, kv, ksum, kmax, qfeat, q_lsq, vt, kvt, kv_part, part_max, n_split, 0, 1, key_lengths, out, log_norm, part_ws,
               B, H, T, S, mh_valid, local_context, nc, n_parts,
               q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss, softmax_temp,
@@ -4386,7 +4399,7 @@ struct SbWorkspace {
 // Every piece starts at a multiple of 256 bytes.  E: padded head dim (= D), mh: padded projection rows.
 SbWorkspace sb_workspace(int B, int H, int T, int S, int E, int mh, int local_context, int dtype) {
     SbWorkspace w{};
-    plan(B, H, S, &w.n_chunks, &w.n_split);
+    plan(B, H, S, key_pass_wgs_per_cu(dtype, E, mh), &w.n_chunks, &w.n_split);
     w.n_parts = plan_parts(B, H, T, S, local_context);
     const size_t bh = (size_t)B * H, nc = w.n_chunks, ns = w.n_split, m = 2 * (size_t)mh, n_qt = (T + TQ - 1) / TQ;
     const size_t esize = dtype == F32 ? 4 : 2;
@@ -4539,7 +4552,7 @@ extern "C" int flyhip_sbblocksparse_fwd(const void* q, const void* k, const void
                            v_sb | v_sh | v_ss, o_sb | o_sh | o_ss);
     if (rc) return rc;
     int nc, ns;
-    plan(B, H, S, &nc, &ns);
+    plan(B, H, S, 2, &nc, &ns);
     FLY_REQUIRE(n_heavy >= 0 && (n_heavy == 0 || (tl_heavy && tl_order && part_ws && qfeat && heavy_parts >= 2 && heavy_parts <= 64)),
                 "sbblocksparse_fwd: long lists need tl_heavy, tl_order (with the long tiles marked), part_ws, qfeat and "
                 "2 <= heavy_parts <= 64");

@@ -44,8 +44,8 @@ class SBLocalPlan:
     def __init__(self, B, H, T, S, dim, mh, mh_valid, dtype, device, local_context, n_parts=None,
                  operand_images=True):
         n_chunks, n_split, parts = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
-        _lib.call('flyhip_sb_plan', B, H, T, S, local_context, ctypes.byref(n_chunks), ctypes.byref(n_split),
-                  ctypes.byref(parts))
+        _lib.call('flyhip_sb_plan_for', B, H, T, S, local_context, dim, mh, _lib.DTYPE_CODE[dtype],
+                  ctypes.byref(n_chunks), ctypes.byref(n_split), ctypes.byref(parts))
         self.n_chunks, self.n_split = n_chunks.value, n_split.value
         self.planned_parts = parts.value
         self.n_parts = parts.value if n_parts is None else n_parts

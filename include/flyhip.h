@@ -34,6 +34,12 @@ const char* flyhip_last_error(void);
  * every 64-query tile is split into by flyhip_sblocal_fwd (1 = no partial workspace needed). */
 int flyhip_sb_plan(int B, int H, int T, int S, int local_context,
                    int* n_chunks, int* n_split, int* n_parts);
+/* The same for a known kernel choice: E the padded head dim, mh the padded projection rows, dtype the code of the
+ * inputs.  n_split then accounts for how many workgroups of that key pass a compute unit holds (one for fp32 inputs on
+ * the bf16-piece kernels, two otherwise); n_chunks and n_parts as above.  (No counterpart in the reference: launch
+ * geometry.) */
+int flyhip_sb_plan_for(int B, int H, int T, int S, int local_context, int E, int mh, int dtype,
+                       int* n_chunks, int* n_split, int* n_parts);
 
 /* Key-side pass.  Replaces feature_map.forward_keys (ref: feature_maps_sb.py:51-82, key branch),
  * the masking of padded keys (sblocal_attention.py:83-85) and the global reductions

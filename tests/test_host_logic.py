@@ -38,6 +38,12 @@ def test_library_exports_every_declared_symbol():
     assert nc.value == 49 and 1 <= ns.value <= 49 and 1 <= npart.value <= 8
     with pytest.raises(RuntimeError, match='bad arguments'):
         _lib.call('flyhip_sb_plan', 0, 1, 10, 10, 4, ctypes.byref(nc), ctypes.byref(ns), ctypes.byref(npart))
+    # the first T2T layer (B=64, L=3136): 49 chunks a head; the fp32 key pass on bf16 pieces holds one workgroup per
+    # compute unit, so one full round of 256 workgroups (4 a head, 13 chunks each) beats two rounds of 7 chunks
+    _lib.call('flyhip_sb_plan_for', 64, 1, 3136, 3136, 256, 64, 64, 0, ctypes.byref(nc), ctypes.byref(ns), ctypes.byref(npart))
+    assert (nc.value, ns.value, npart.value) == (49, 4, 1)
+    _lib.call('flyhip_sb_plan_for', 64, 1, 3136, 3136, 256, 64, 64, 1, ctypes.byref(nc), ctypes.byref(ns), ctypes.byref(npart))
+    assert (nc.value, ns.value) == (49, 7)
 
 
 @pytest.mark.parametrize('args', [(3072, 768, 8, 2, 32), (768, 3072, 8, 2, 32), (4096, 4096, 8, 2, 32),
