@@ -171,8 +171,13 @@ def bench_blocksparse(steps, warmup):
     out = {}
 
     def timeit(fn):
-        for _ in range(warmup):
+        t0 = time.perf_counter()                 # warm-up by time as well as by count (settled clocks)
+        done = 0
+        while done < warmup or time.perf_counter() - t0 < 0.05:
             fn()
+            done += 1
+            if done % 8 == 0:
+                torch.cuda.synchronize()
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
