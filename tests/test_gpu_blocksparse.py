@@ -337,6 +337,43 @@ def test_fused_attention_matches_oracle(p, r, D, rpg, dtype):
         assert rel_err(out, o3.float()) <= 2 * TOL[dtype]
 
 
+def test_fused_attention_random_shapes():
+    """Seeded random layouts, sizes, head dims, group sizes, dtypes, scales, key and attention masks against the
+    oracle's SDD -> softmax -> nan_to_num -> DSD in float64: union lists of any length modulo the four block-columns a
+    step takes, rows without blocks, heads without blocks, fully masked rows."""
+    import random
+    from fly_amd.blocksparse_fused import fused_attention
+    rng = random.Random(20)
+    for case in range(40):
+        Z, H = rng.randint(1, 3), rng.randint(1, 3)
+        p, r = rng.randint(1, 20), rng.randint(1, 20)
+        D, rpg = rng.choice([32, 64, 128]), rng.choice([4, 8])
+        dtype = rng.choice([torch.bfloat16, torch.float16])
+        dens = rng.choice([0.1, 0.4, 0.8, 1.0])
+        g = torch.Generator().manual_seed(case)
+        layout = (torch.rand(H, p, r, generator=g) < dens).long()
+        layout[0, 0, 0] = 1
+        q = torch.randn(Z, p * 32, H, D, generator=g).to(dtype)
+        k = torch.randn(Z, r * 32, H, D, generator=g).to(dtype)
+        v = torch.randn(Z, r * 32, H, D, generator=g).to(dtype)
+        kpm = am = None
+        if rng.random() < 0.5:
+            lens = torch.tensor([rng.randint(1, r * 32) for _ in range(Z)])
+            kpm = torch.log((torch.arange(r * 32).view(1, -1) < lens.view(Z, 1)).float())
+        if rng.random() < 0.3:
+            am = torch.log((torch.rand(p * 32, r * 32, generator=g) < 0.7).float())
+        scale = rng.choice([0.125, 0.31, 1.0])
+        print('case', case, Z, H, p, r, D, rpg, dtype, dens, kpm is not None, am is not None, scale, flush=True)
+        qh, kh, vh = (x.permute(0, 2, 1, 3) for x in (q, k, v))
+        qk = ob.sdd(qh.double(), kh.double(), layout, 32, trans_b=True)
+        pr = ob.block_softmax(qk, layout, 32, scale=scale, key_padding_mask=kpm, attn_mask=am).nan_to_num()
+        ref = ob.dsd(pr, vh.double(), layout, 32)
+        out = fused_attention(layout, 32, rows_per_group=rpg)(
+            qh.to(DEV), kh.to(DEV), vh.to(DEV), scale, None if kpm is None else kpm.to(DEV),
+            attn_mask=None if am is None else am.to(DEV))
+        assert rel_err(out, ref) <= TOL[dtype], (case, rel_err(out, ref))
+
+
 def test_fused_attention_with_an_empty_layout():
     """No nonzero block at all: zeros (the value of a row without blocks), and +inf as the rows' log-denominator."""
     from fly_amd.blocksparse_fused import fused_attention
