@@ -91,6 +91,19 @@ def call(name, *args):
 DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
 
 
+def table_ptr(t):
+    """Address of an index table that the kernels only read through the ranges of another one: an empty table (a
+    layout without blocks) has no storage, so a one-element stand-in is passed; no range points into it."""
+    if t.numel() == 0:
+        t = torch.zeros(1, dtype=t.dtype, device=t.device)
+        _KEEP_ALIVE.append(t)
+        del _KEEP_ALIVE[:-8]
+    return t.data_ptr()
+
+
+_KEEP_ALIVE = []
+
+
 def dtype_code(t):
     try:
         return DTYPE_CODE[t.dtype]

@@ -170,8 +170,8 @@ class SBLocalPlan:
             self.run_keys(q, k, v, proj, None, t, stream)
             _lib.call('flyhip_sbblocksparse_fwd', q.data_ptr(), k.data_ptr(), v.data_ptr(), proj.data_ptr(),
                       self.kfeat.data_ptr(), self.chunk_scale.data_ptr(), self.kv.data_ptr(),
-                      self.ksum.data_ptr(), self.kmax.data_ptr(), tl_ptr.data_ptr(), tl_inner.data_ptr(),
-                      tl_blk.data_ptr(), _lib.ptr(tl_order), _lib.ptr(tl_heavy), n_heavy, parts,
+                      self.ksum.data_ptr(), self.kmax.data_ptr(), tl_ptr.data_ptr(), _lib.table_ptr(tl_inner),
+                      _lib.table_ptr(tl_blk), _lib.ptr(tl_order), _lib.ptr(tl_heavy), n_heavy, parts,
                       _lib.ptr(self.part_ws) if n_heavy else None, _lib.ptr(self.qfeat) if n_heavy else None,
                       out.data_ptr(), log_norm.data_ptr(),
                       B, H, T, S, dim, dim, mh, mh_valid,

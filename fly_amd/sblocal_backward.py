@@ -206,7 +206,7 @@ def _backward_hip(Q, K, V, G, O, LN, P, lens_b, H, local_context, t, dims, piece
                     hws = new(n_hws)
                 _lib.call('flyhip_sbblocksparse_bwd_pieces', oimg.data_ptr(), iimg.data_ptr(), x1.data_ptr(), ln_.data_ptr(),
                           c_.data_ptr(), gmat.data_ptr(), gvec.data_ptr(), proj.data_ptr(), d1.data_ptr(), _lib.ptr(d3),
-                          tl_ptr.data_ptr(), tl_inner.data_ptr(), tl_blk.data_ptr(), _lib.ptr(skip), _lib.ptr(heavy),
+                          tl_ptr.data_ptr(), _lib.table_ptr(tl_inner), _lib.table_ptr(tl_blk), _lib.ptr(skip), _lib.ptr(heavy),
                           n_heavy, parts, _lib.ptr(hws), n_hws, BH, H, T, S, dim, mk, float(t), key_major, st)
         elif pieces:
             _lib.call('flyhip_sblocal_bwd_pieces', qimg.data_ptr(), kimg.data_ptr(), q_.data_ptr(),

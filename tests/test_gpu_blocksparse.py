@@ -757,6 +757,26 @@ def test_sbblocksparse_fused_forward(B, H, T, S, E, D, m, seed):
     assert torch.equal(out2, out) and torch.equal(ln2, ln)
 
 
+def test_sbblocksparse_fused_forward_with_an_empty_layout():
+    """A support without any block: what remains is the low-rank estimate alone (linear attention on the features)."""
+    from fly_amd.blocksparse_utils import union_table
+    from fly_amd.sblocal_attention import sbblocksparse_forward
+    from oracle import sbblocksparse as osbb
+    from oracle import sblocal as osb
+    g = torch.Generator().manual_seed(7)
+    B, H, T, S, E, D, m = 2, 1, 32, 96, 64, 64, 64
+    layout = torch.zeros(H, T // 32, S // 32, dtype=torch.long)
+    q = torch.randn(B, T, H, E, generator=g) * E ** -0.25
+    k = torch.randn(B, S, H, E, generator=g) * E ** -0.25
+    v = torch.randn(B, S, H, D, generator=g)
+    P = osb.gaussian_orthogonal_random_matrix(m // 2, E, generator=g)
+    tables = tuple(x.to(DEV) for x in union_table(layout, rows_per_group=2))
+    out, ln = sbblocksparse_forward(q.to(DEV), k.to(DEV), v.to(DEV), P.to(DEV), tables)
+    ref_out, ref_ln = osbb.sbblocksparse_attention(q.double(), k.double(), v.double(), P.double(), layout, 32)
+    assert rel_err(out, ref_out) <= 1e-4, rel_err(out, ref_out)
+    assert rel_err(ln.reshape(ref_ln.shape), ref_ln) <= 1e-4
+
+
 @pytest.mark.parametrize('B,H,T,S,E,D,m,seed', [(2, 2, 256, 256, 64, 64, 64, 1), (1, 3, 224, 352, 32, 32, 32, 2),
                                                 (1, 2, 416, 160, 40, 24, 26, 4), (3, 1, 160, 192, 64, 64, 128, 5)])
 def test_sbblocksparse_gradients_on_the_kernels(B, H, T, S, E, D, m, seed):
