@@ -1204,7 +1204,9 @@ template <int CPR> __device__ __forceinline__ int attn_vslot(int row, int c) {
 template <typename T, int KS, int NW, bool MASKED>     // head dim 32*KS, NW block-rows (waves) per workgroup
 __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
     constexpr int D = 32 * KS, DT = D / 16, RB = 2 * D;   // RB: bytes of a tile row
-    constexpr int CP = KS <= 2 ? 4 : 2;                   // block-columns per step (what 64 KB of LDS hold twice over)
+    // block-columns per step: what 64 KB of LDS hold twice over -- half of that for workgroups of four waves at 64 dims,
+    // of which a compute unit then holds four (the registers allow it) instead of two
+    constexpr int CP = KS == 1 ? 4 : (KS == 2 && NW >= 8 ? 4 : 2);
     constexpr int CPR = D / 8;                            // 16-byte chunks per tile row
     constexpr int COLB = 64 * RB;                         // one column's image: rows 0..31 keys of K, 32..63 the same keys of V
     constexpr int U = COLB / 1024, NCH = (U + NW - 1) / NW;      // wave loads per column, and per wave
