@@ -341,6 +341,9 @@ def sblocal_backward(query, key, value, projection_matrix, local_context, softma
     if band_kernel and dims is None:
         raise NotImplementedError(f'no band kernel for head dims ({E}, {D}) with {2 * mh} features')
     on_kernels = dims is not None and Q.is_cuda and wdt == torch.float32
+    if not Q.is_cuda and wdt != torch.float64:
+        # host tensors are accepted for one purpose: checking the written-out gradient formulas in float64 against autograd
+        raise NotImplementedError('sblocal_backward runs on the GPU; host tensors only in float64 (the check of the formulas)')
     lens_b = None if key_lengths is None else key_lengths.to(device=Q.device, dtype=torch.int64).contiguous()
     if support is not None:
         if not on_kernels or key_lengths is not None or T % 32 or S % 32:
