@@ -63,8 +63,8 @@ def local_backward(query, key, value, local_context, softmax_temp, key_lengths, 
     key get zero gradients.  Given the forward's out and lse (local_forward(..., return_lse=True)), float32
     or bfloat16 GPU tensors and head dims <= 64, the sums run on the backward band kernel of
     Scatterbrain-local attention with its feature operands zero (flyhip_sblocal_bwd_band: P_is =
-    exp(t q_i.k_s - lse_i), delta_i = g_i.out_i); otherwise as ordinary tensor algebra on whatever device
-    the tensors live on."""
+    exp(t q_i.k_s - lse_i), delta_i = g_i.out_i); otherwise as batched library products on the GPU (host tensors are
+    accepted in float64 only: the check of these formulas against autograd)."""
     B, T, H, E = query.shape
     S, D = key.shape[1], value.shape[3]
     t = softmax_temp or 1 / math.sqrt(E)
@@ -76,6 +76,9 @@ def local_backward(query, key, value, local_context, softmax_temp, key_lengths, 
 
     def back(x, like):                           # (B*H, L, C) -> (B,L,H,C)
         return x.reshape(B, H, x.shape[1], x.shape[2]).permute(0, 2, 1, 3).to(like.dtype)
+    if not Q.is_cuda and wdt != torch.float64:
+        # host tensors are accepted for one purpose: checking the written-out gradient formulas in float64 against autograd
+        raise NotImplementedError('local_backward runs on the GPU; host tensors only in float64 (the check of the formulas)')
     dims = _band_kernel_dims(E, D, 0)
     if out is not None and lse is not None and Q.is_cuda and wdt == torch.float32 and dims is not None:
         zq, zk = Q.new_zeros(B * H, T, dims[1]), Q.new_zeros(B * H, S, dims[1])
