@@ -74,9 +74,10 @@ def bench_sblocal(steps, warmup, cpu_baseline=True):
     for _ in range(warmup):
         plan.run(qd, kd, vd, Pd, None, lc, t, out, ln)
     torch.cuda.synchronize()
-    # The dominant kernel is timed inside the timed region: on sampled steps the library records two events
-    # right around the band kernel, on its stream.  At least 16 samples whatever the step count (an event pair
-    # costs a few microseconds of a 35 microsecond step, so it is not put around every launch of a long run).
+    # The dominant kernel is timed inside the timed region: on sampled steps the library launches the band kernel
+    # with two events that take the launch's own begin and end time stamps, on its stream.  At least 16 samples
+    # whatever the step count (timed launches cost a few microseconds of a 31 microsecond step, so not every launch of
+    # a long run is one).
     every = max(1, steps // 16)
     sampled = [i for i in range(steps) if i % every == 0]
     ev = {i: (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for i in sampled}

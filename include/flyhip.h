@@ -305,9 +305,10 @@ int flyhip_local_fwd_lse(const void* q, const void* k, const void* v, const int6
                          int64_t o_sb, int64_t o_sh, int64_t o_ss,
                          float softmax_temp, int dtype, void* stream);
 
-/* Measurement hook (no counterpart in the reference): the two caller-owned hipEvent_t are recorded
- * on the launch stream immediately before and after the fused band kernel of the NEXT
- * flyhip_sblocal_fwd call of the calling thread, then forgotten.  Pass NULLs to clear. */
+/* Measurement hook (no counterpart in the reference): the two caller-owned hipEvent_t receive the begin
+ * and the end time stamp of the fused band kernel's launch (hipExtLaunchKernelGGL) in the NEXT
+ * flyhip_sblocal_fwd call of the calling thread, on its stream, and are then forgotten: their elapsed time
+ * is the kernel's duration.  Pass NULLs to clear. */
 int flyhip_sb_time_next_fwd(void* event_before, void* event_after);
 
 /* ------------------------------------------------------------------------------------------
