@@ -23,6 +23,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_BF16_MFMA_TFLOPS = 2500.0
 PEAK_HBM_GBS = 8000.0
 # HBM bytes one launch of the dominant kernel moves at the benchmarked workload: rocprofv3 FETCH_SIZE / WRITE_SIZE
 # readings scaled by a plain copy of known size, kept with the profile summaries they come from
@@ -37,6 +38,24 @@ def band_kernel_traffic():
         return float(t['band_kernel']['hbm_read_bytes']) + float(t['band_kernel']['hbm_write_bytes'])
     except (OSError, KeyError, ValueError):
         return None
+
+
+def band_kernel_pipe_view(kernel_ms):
+    """The band kernel against the pipe it issues on: executed bf16 MFMA FLOPs per launch (counter
+    SQ_INSTS_VALU_MFMA_MOPS_BF16 x 512, from the committed summary) over the live kernel time against the bf16 MFMA
+    peak, and the share of the launch's SIMD cycles the matrix pipe was busy (SQ_VALU_MFMA_BUSY_CYCLES over
+    1024 SIMDs x the kernel time the counters were taken at x the shader clock of that run)."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            m = json.load(f)['band_kernel']['mfma']
+        executed = float(m['mops_bf16']) * 512.0
+        view = {'mfma_pipe': 'bf16', 'executed_flops_per_launch': executed, 'pipe_peak': PEAK_BF16_MFMA_TFLOPS,
+                'pipe_frac': executed / (kernel_ms * 1e-3) / 1e12 / PEAK_BF16_MFMA_TFLOPS,
+                'mfma_busy_share': float(m['busy_cycles']) / (1024.0 * float(m['kernel_us']) * float(m['clock_mhz']))}
+        return view
+    except (OSError, KeyError, ValueError):
+        return {'mfma_pipe': 'bf16', 'executed_flops_per_launch': None, 'pipe_peak': PEAK_BF16_MFMA_TFLOPS,
+                'pipe_frac': None, 'mfma_busy_share': None}
 
 
 def sblocal_flops(B, H, T, S, E, D, m, lc):
@@ -71,27 +90,37 @@ def bench_sblocal(steps, warmup, cpu_baseline=True):
     out = torch.empty(B, L, H, D, device=dev)
     ln = torch.empty(B, H, L, device=dev)
 
-    for _ in range(warmup):
+    # Warm-up: the counted steps, then the same step until 50 ms have passed -- the clocks need tens of
+    # milliseconds of load to settle on a workload, and a count of a few 30 microsecond steps is over long before that.
+    w0 = time.perf_counter()
+    done = 0
+    while done < warmup or time.perf_counter() - w0 < 0.05:
         plan.run(qd, kd, vd, Pd, None, lc, t, out, ln)
+        done += 1
+        if done % 64 == 0:
+            torch.cuda.synchronize()
     torch.cuda.synchronize()
-    # The dominant kernel is timed inside the timed region: on sampled steps the library launches the band kernel
-    # with two events that take the launch's own begin and end time stamps, on its stream.  At least 16 samples
-    # whatever the step count (timed launches cost a few microseconds of a 31 microsecond step, so not every launch of
-    # a long run is one).
-    every = max(1, steps // 16)
-    sampled = [i for i in range(steps) if i % every == 0]
-    ev = {i: (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for i in sampled}
-    for a, b in ev.values():             # create the underlying hipEvent_t objects before timing
-        a.record(); b.record()
-    torch.cuda.synchronize()
+    warmup_ms = (time.perf_counter() - w0) * 1e3
     t0 = time.perf_counter()
-    for i in range(steps):
-        if i in ev:
-            _lib.call('flyhip_sb_time_next_fwd', ev[i][0].cuda_event, ev[i][1].cuda_event)
+    for _ in range(steps):
         plan.run(qd, kd, vd, Pd, None, lc, t, out, ln)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    fwd_ms = sum(a.elapsed_time(b) for a, b in ev.values()) / len(ev)
+    # The dominant kernel is timed live on steps of the same loop that follow the timed ones (so that `wall` carries
+    # no timing hook): the library launches the band kernel of a sampled step with two events that take the launch's
+    # own begin and end time stamps, on its stream.  16 samples at least, one step in four at most.
+    n_samples = max(16, min(64, steps // 4))
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_samples)]
+    for a, b in ev:                      # create the underlying hipEvent_t objects before use
+        a.record(); b.record()
+    torch.cuda.synchronize()
+    for a, b in ev:
+        for _ in range(3):
+            plan.run(qd, kd, vd, Pd, None, lc, t, out, ln)
+        _lib.call('flyhip_sb_time_next_fwd', a.cuda_event, b.cuda_event)
+        plan.run(qd, kd, vd, Pd, None, lc, t, out, ln)
+    torch.cuda.synchronize()
+    fwd_ms = sum(a.elapsed_time(b) for a, b in ev) / len(ev)
 
     # the same forward through the drop-in module (reference signature sblocal_attention.py:43-44): argument
     # checks, cached scratch, two result tensors per call
@@ -102,26 +131,32 @@ def bench_sblocal(steps, warmup, cpu_baseline=True):
         for _ in range(max(warmup, 3)):
             mod(qd, kd, vd)
         torch.cuda.synchronize()
+        n_mod = max(steps, 200)
         t1 = time.perf_counter()
-        for _ in range(steps):
+        for _ in range(n_mod):
             mod(qd, kd, vd)
         torch.cuda.synchronize()
-        module_ms = (time.perf_counter() - t1) / steps * 1e3
+        module_ms = (time.perf_counter() - t1) / n_mod * 1e3
 
     total_flops, fwd_flops = sblocal_flops(B, H, L, L, E, D, 2 * mh, lc)
     ms_per_step = wall / steps * 1e3
     achieved = fwd_flops / (fwd_ms * 1e-3) / 1e12
+    roofline = {'bound': 'mfma', 'kernel': 'sblocal_fwd_x3_kernel<64,64,128,split>',
+                'achieved': achieved, 'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s',
+                'frac': achieved / PEAK_FP32_MFMA_TFLOPS, 'traffic': band_kernel_traffic(),
+                'kernel_ms': fwd_ms, 'flops_per_launch': fwd_flops, 'launches_timed': len(ev),
+                'arithmetic': 'fp32 inputs, outputs and accumulation; products on v_mfma_f32_16x16x32_bf16 from '
+                              'operands split into bf16 pieces (scores 3 piece products, feature overlap 4 on '
+                              'features rounded to 17 bits, P V 5 with V rounded to 16 bits).  achieved / peak / frac '
+                              'price the ALGORITHMIC fp32 FLOPs against the fp32 MFMA peak; mfma_pipe .. pipe_frac '
+                              'price the piece products actually issued against the peak of the pipe they run on'}
+    roofline.update(band_kernel_pipe_view(fwd_ms))
     res = {
         'tokens_per_s': B * L / (wall / steps),
         'ms_per_step': ms_per_step,
+        'warmup_ms': warmup_ms,
         'module_forward_ms': module_ms,
-        'roofline': {'bound': 'mfma', 'kernel': 'sblocal_fwd_x3_kernel<64,64,128,split>',
-                     'achieved': achieved, 'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s',
-                     'frac': achieved / PEAK_FP32_MFMA_TFLOPS, 'traffic': band_kernel_traffic(),
-                     'kernel_ms': fwd_ms, 'flops_per_launch': fwd_flops, 'launches_timed': len(ev),
-                     'arithmetic': 'fp32 inputs, outputs and accumulation; products on v_mfma_f32_16x16x32_bf16 from '
-                                   'operands split into bf16 pieces (scores 3 piece products, feature overlap 4 on '
-                                   'features rounded to 17 bits, P V 5 with V rounded to 16 bits); priced against the fp32 MFMA peak'},
+        'roofline': roofline,
         'parity': None,
         'flops_per_step': total_flops,
     }
@@ -453,7 +488,7 @@ def main():
     line = {
         'metric': 'SBLocal attention forward tokens/s (fp32, L=3136, d=64)',
         'value': sb['tokens_per_s'], 'unit': 'tokens/s', 'n_gpus': 1, 'steps': args.steps,
-        'warmup': args.warmup, 'ms_per_step': sb['ms_per_step'], 'higher_is_better': True,
+        'warmup': args.warmup, 'warmup_ms': sb['warmup_ms'], 'ms_per_step': sb['ms_per_step'], 'higher_is_better': True,
         'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f32', 'data': 'synthetic',
         'config': {'workload': 'BASELINE config 1 (configs[0]): SBLocal fwd fp32 B=2 H=1 L=3136 d=64 '
                                'local_context=512 nb_features=128, seeded orthogonal-Gaussian projection'},

@@ -191,37 +191,30 @@ class SBBlockSparseAttention(nn.Module):
         key = key.permute(0, 2, 1, 3).float().contiguous()
         value = value.permute(0, 2, 1, 3).float().contiguous()
 
-        q_prime, q_prime_log_scale = self.feature_map.forward_queries(query)
-        k_prime, k_prime_log_scale = self.feature_map.forward_keys(key)
-        prime_log_scale = q_prime_log_scale + k_prime_log_scale     # (b h t 1)
-        q_prime_k_prime_1 = linear_attention_normalization(q_prime, k_prime)
-        q_prime_k_prime_v, attn_prime = linear_attention(q_prime, k_prime, value, need_weights=need_weights)
-
-        layout = self.get_layout(T, S)
+        # op by op (:170-213): feature maps and the sums over all keys as library products, everything on the
+        # support through the block-sparse operators.  Per query: Z = sum_support e^{t q.k} + max(phi(q).sum_all phi(k)
+        # - sum_support phi(q).phi(k), 1e-24) e^{ls}; the weights on the support are e^{t q.k} / Z minus the feature
+        # weight, which the all-keys term adds back; dropout touches the exact part only (:200).
+        feat_q, ls_q = self.feature_map.forward_queries(query)
+        feat_k, ls_k = self.feature_map.forward_keys(key)
+        ls = (ls_q + ls_k).squeeze(-1)                                               # (b h t)
+        mass_all = linear_attention_normalization(feat_q, feat_k)                    # phi(q) . sum_s phi(k_s)
+        out_all, attn_prime = linear_attention(feat_q, feat_k, value, need_weights=need_weights)
         sdd_nt, dsd_nn, sparse_logsumexp, sparse_sum = self.get_ops(T, S)
-        QK = sdd_nt(query, key)
-        QK.mul_(softmax_temp)
-        dots_prime = sdd_nt(q_prime, k_prime)
+        scores = sdd_nt(query, key).mul_(softmax_temp)
+        overlap = sdd_nt(feat_q, feat_k)
+        mass_off_support = (mass_all - sparse_sum(overlap)).clamp_min(1e-24)
+        log_z = torch.logaddexp(sparse_logsumexp(scores), mass_off_support.log() + ls)
+        feat_weight = (ls - log_z).exp()
 
-        # joint normalisation first (:185-190)
-        QK_lse = sparse_logsumexp(QK).unsqueeze(-1)
-        dots_prime_sum = sparse_sum(dots_prime).unsqueeze(-1)
-        lr_log_normalization = torch.log((q_prime_k_prime_1.unsqueeze(-1) - dots_prime_sum).clamp_min_(1e-24)) \
-            + prime_log_scale
-        log_normalization = torch.logaddexp(QK_lse, lr_log_normalization)
-        prime_scale = torch.exp(prime_log_scale - log_normalization)
-
-        # weights on the support: exp(QK - log Z) with the low-rank overlap taken out (:195-200);
-        # dropout acts on the exact part only
-        log_normalization_sparse = sparsify_broadcast_tensor(log_normalization.squeeze(-1), layout, block)
-        prime_scale_sparse = sparsify_broadcast_tensor(prime_scale.squeeze(-1), layout, block)
-        dots = self.dropout(torch.exp(QK - log_normalization_sparse)) - dots_prime * prime_scale_sparse
-
-        out = (dsd_nn(dots, value) + q_prime_k_prime_v * prime_scale).to(in_dtype)
+        def per_block(rows):                     # a (b h t) vector spread over the columns of the support's blocks
+            return sparsify_broadcast_tensor(rows, layout, block)
+        dots = self.dropout((scores - per_block(log_z)).exp()) - overlap * per_block(feat_weight)
+        out = (dsd_nn(dots, value) + out_all * feat_weight.unsqueeze(-1)).to(in_dtype)
 
         attn = None
         if need_weights:
-            attn = densify_tensor(dots, layout) + attn_prime * prime_scale
+            attn = densify_tensor(dots, layout) + attn_prime * feat_weight.unsqueeze(-1)
             if return_attn_unnormalized:
-                attn = (attn, attn * torch.exp(log_normalization), attn_prime * torch.exp(prime_log_scale))
+                attn = (attn, attn * log_z.exp().unsqueeze(-1), attn_prime * ls.exp().unsqueeze(-1))
         return out.permute(0, 2, 1, 3), attn
