@@ -21,7 +21,7 @@ SIGNATURES = {
     'flyhip_sb_time_next_fwd': [c_vp, c_vp],
     'flyhip_sb_kv_reduce': [c_vp] * 14 + [c_int] + [c_i64] * 3 + [c_vp] * 2 + [c_int] * 8 + [c_i64] * 6 + [c_float, c_int, c_vp],
     'flyhip_sblocal_fwd': [c_vp] * 13 + [c_vp] * 2 + [c_int] + [c_vp] * 4 + [c_int] * 10 + [c_i64] * 12 + [c_float, c_int, c_vp],
-    'flyhip_sblocal_forward': [c_vp] * 8 + [c_i64] + [c_int] * 9 + [c_i64] * 12 + [c_float, c_int, c_vp],
+    'flyhip_sblocal_forward': [c_vp] * 8 + [c_i64] + [c_int] * 9 + [c_i64] * 12 + [c_float, c_int, c_int, c_vp],
     'flyhip_sblocal_fwd_static': [c_vp] * 13 + [c_vp] * 2 + [c_int] + [c_vp] * 3 + [c_int] * 10 + [c_i64] * 12 + [c_float, c_int, c_vp],
     'flyhip_sblocal_bwd_band': [c_vp] * 12 + [c_int] * 7 + [c_float, c_int, c_vp],
     'flyhip_sblocal_bwd': [c_vp] * 14 + [c_int] * 7 + [c_float, c_int, c_vp],
@@ -63,7 +63,7 @@ def load():
         fn = getattr(lib, name)
         fn.argtypes = argtypes
         fn.restype = c_int
-    lib.flyhip_sb_workspace_bytes.argtypes = [c_int] * 8
+    lib.flyhip_sb_workspace_bytes.argtypes = [c_int] * 9
     lib.flyhip_sb_workspace_bytes.restype = c_i64
     lib.flyhip_sblocal_bwd_prep_scratch.argtypes = [c_int] * 5
     lib.flyhip_sblocal_bwd_prep_scratch.restype = c_i64
@@ -89,6 +89,7 @@ def call(name, *args):
 
 
 DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
+SB_EXACT_FP32 = 1          # flag of flyhip_sblocal_forward / flyhip_sb_workspace_bytes (FLYHIP_SB_EXACT_FP32)
 
 
 def table_ptr(t):

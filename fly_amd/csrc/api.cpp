@@ -40,6 +40,20 @@ int ensure_dynamic_lds(const void* kernel, size_t bytes, std::atomic<unsigned lo
     done.fetch_or(bit, std::memory_order_release);
     return OK;
 }
+
+int refuse_capture(hipStream_t st) {
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    const hipError_t e = hipStreamIsCapturing(st, &status);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(ERR_UNSUPPORTED, "the stream cannot be launched on (%s): another stream of this process is under graph "
+                                     "capture, and calls of this library are not capturable", hipGetErrorString(e));
+    }
+    if (status != hipStreamCaptureStatusNone)
+        return fail(ERR_UNSUPPORTED, "the stream is under graph capture: calls of this library are not capturable "
+                                     "(run them eagerly, outside the capture)");
+    return OK;
+}
 }  // namespace flyhip
 
 extern "C" int flyhip_version(void) { return 100; }

@@ -1792,6 +1792,7 @@ extern "C" int flyhip_bs_sdd(const void* a, const void* b, void* c, const int32_
     if (b_sk == 1) FLY_REQUIRE(((b_sz | b_sh | b_sn) % 4) == 0, "bs_sdd: B strides must be multiples of 4 elements");
     if (nnz == 0) return OK;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (int rc_capture = refuse_capture(st)) return rc_capture;
     if (row_ptr && row_blk && row_col && blk == 32 && (dtype == BF16 || dtype == F16) && a_sk == 1 && b_sk == 1 &&
         K % 32 == 0 && K <= 128 && ((a_sz | a_sh | a_sm | b_sz | b_sh | b_sn) % 8) == 0 && n_brow > 0 &&
         brows_per_head > 0) {
@@ -1856,6 +1857,7 @@ static int launch_sdd_epilogue(const char* what, const void* a_dn, const void* b
     FLY_REQUIRE(nnz > 0 && n_heads > 0 && brows_per_head > 0, "%s: bad sizes", what);
     FLY_REQUIRE(((a_sz | a_sh | a_sm | b_sz | b_sh | b_sn) % 8) == 0, "%s: strides must be multiples of 8 elements", what);
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (int rc_capture = refuse_capture(st)) return rc_capture;
     const int gph = (brows_per_head + 3) / 4;
     SddUniArgs ua{a_dn, b_dn, c, uni_ptr, uni_inner, uni_blk, nnz, brows_per_head, gph, n_heads, Z,
                   a_sz, a_sh, a_sm, b_sz, b_sh, b_sn, p, rowvec, scale};
@@ -1949,6 +1951,7 @@ extern "C" int flyhip_bs_sdd_kmajor(const void* a, const void* b, float* c32,
     const int chunks = (max_row_nnz + 3) / 4, slices = (K + k_slice - 1) / k_slice;
     FLY_REQUIRE((long)n_grp * chunks <= 2147483647L && slices <= 65535, "bs_sdd_kmajor: too many workgroups");
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (int rc_capture = refuse_capture(st)) return rc_capture;
     SddKArgs args{a, b, c32, row_ptr, row_blk, row_col, grp_row0, grp_n, brows_per_head, K, k_slice, chunks, nnz,
                   a_sz, a_sh, a_sk, b_sz, b_sh, b_sk};
     dim3 grid((unsigned)(n_grp * chunks), slices, Z);
@@ -1974,6 +1977,7 @@ extern "C" int flyhip_bs_dsd(const void* a_sp, const void* b, void* c,
     if (c_sn == 1) FLY_REQUIRE(((c_sz | c_sh | c_sm) % 4) == 0, "bs_dsd: C strides must be multiples of 4 elements");
     FLY_REQUIRE(a_sz % 4 == 0, "bs_dsd: sparse batch stride must be a multiple of 4 elements");
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (int rc_capture = refuse_capture(st)) return rc_capture;
     DxdArgs args{a_sp, b, c, seg_ptr, seg_blk, seg_inner, n_seg, rows_per_head, N, trans_a,
                  a_sz, b_sz, b_sh, b_sk, b_sn, c_sz, c_sh, c_sm, c_sn, Z};
     if (blk == 32 && (dtype == BF16 || dtype == F16) && (!trans_a || (uni_ptr && uni_inner && uni_blk)) && b_sn == 1 &&
@@ -2029,6 +2033,7 @@ extern "C" int flyhip_bs_dds(const void* a, const void* b_sp, void* c,
     if (c_sn == 1) FLY_REQUIRE(((c_sz | c_sh | c_sm) % 4) == 0, "bs_dds: C strides must be multiples of 4 elements");
     FLY_REQUIRE(b_sz % 4 == 0, "bs_dds: sparse batch stride must be a multiple of 4 elements");
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (int rc_capture = refuse_capture(st)) return rc_capture;
     if (grp_row0 && grp_n && n_grp > 0 && max_seg_len >= 0 && max_seg_len <= DDS_MAX_STEPS && blk == 32 &&
         (dtype == BF16 || dtype == F16) && a_sk == 1 && (long)M * a_sm * 2 < (1L << 32) &&
         c_sn == 1 && ((a_sz | a_sh | a_sm | b_sz | c_sz | c_sh | c_sm) % 8) == 0 && (M + 127) / 128 <= 65535) {
@@ -2104,6 +2109,7 @@ extern "C" int flyhip_bs_attn_masks(const void* q, const void* k, const void* v,
     FLY_REQUIRE(!key_mask || key_mask_stride % 4 == 0, "bs_attn: key mask stride must be a multiple of 4");
     FLY_REQUIRE(!attn_mask || attn_mask_stride % 4 == 0, "bs_attn: attention mask stride must be a multiple of 4");
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (int rc_capture = refuse_capture(st)) return rc_capture;
     const int gph = (brows_per_head + rows_per_group - 1) / rows_per_group;
     AttnArgs args{q, k, v, out, uni_ptr, uni_inner, uni_blk, key_mask, key_mask_stride, brows_per_head, gph, H, Z,
                   q_sz, q_sh, q_sm, k_sz, k_sh, k_sn, v_sz, v_sh, v_sn, o_sz, o_sh, o_sm, scale, lse2};
@@ -2165,6 +2171,7 @@ extern "C" int flyhip_bs_softmax(void* x, const int32_t* row_ptr, const int32_t*
     FLY_REQUIRE(n_brow > 0 && brows_per_head > 0 && n_brow % brows_per_head == 0, "bs_softmax: bad row counts");
     FLY_REQUIRE(max_row_nnz >= 0, "bs_softmax: negative max_row_nnz");
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (int rc_capture = refuse_capture(st)) return rc_capture;
     RowArgs args{x, nullptr, row_ptr, row_blk, row_col, n_brow, brows_per_head, blk_shift_of(blk), x_sz, scale,
                  kpm, kpm_stride, kpm_mul, am, am_stride, am_mul, 0};
     const long nblocks = waves_to_blocks((long)n_brow * blk);
@@ -2188,6 +2195,7 @@ extern "C" int flyhip_bs_softmax_bwd(const void* y, const void* dy, void* dx,
     FLY_REQUIRE(n_brow > 0 && max_row_nnz >= 0 && max_row_nnz <= 64, "bs_softmax_bwd: at most 64 blocks per block-row (got %d)", max_row_nnz);
     FLY_REQUIRE(y_sz % 8 == 0, "bs_softmax_bwd: batch stride must be a multiple of 8 elements");
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (int rc_capture = refuse_capture(st)) return rc_capture;
     RowBwdArgs args{y, dy, dx, row_ptr, row_blk, y_sz, scale};
     dim3 grid(2 * n_brow, Z);
     const int slots = (max_row_nnz + 3) / 4;
@@ -2208,6 +2216,7 @@ extern "C" int flyhip_bs_rowreduce(const void* x, void* out, const int32_t* row_
     FLY_REQUIRE(op == 0 || op == 1, "bs_rowreduce: op must be 0 (logsumexp) or 1 (sum)");
     FLY_REQUIRE(n_brow > 0, "bs_rowreduce: no rows");
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (int rc_capture = refuse_capture(st)) return rc_capture;
     RowArgs args{const_cast<void*>(x), out, row_ptr, row_blk, nullptr, n_brow, 1, blk_shift_of(blk), x_sz, 1.f,
                  nullptr, 0, 0, nullptr, 0, 0, op};
     dim3 grid((unsigned)waves_to_blocks((long)n_brow * blk), Z);

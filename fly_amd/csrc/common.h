@@ -41,6 +41,12 @@ const Machine& machine();      // (without a device: the MI355X's 256 compute un
 // per-kernel set of devices already served (one bit each)
 int ensure_dynamic_lds(const void* kernel, size_t bytes, std::atomic<unsigned long long>& done, const char* what);
 
+// Every entry point that launches calls this first: a stream under capture into a HIP graph is refused with an error
+// (ERR_UNSUPPORTED).  The launchers do things on first use that are not stream operations (the LDS limit of a kernel,
+// the address of the built-in scratch array), and a capture of calls of this library has ended in a crash of the host
+// process whose cause is not known; until it is, capture is an error here rather than a crash.
+int refuse_capture(hipStream_t st);
+
 enum DType { F32 = 0, BF16 = 1, F16 = 2 };
 
 // ---------------------------------------------------------------------------------------

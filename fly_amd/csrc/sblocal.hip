@@ -4326,6 +4326,7 @@ extern "C" int flyhip_sb_kv_reduce(const void* k, const void* v, const float* pr
              q, qfeat, q_lsq, q ? T : 0, q_sb, q_sh, q_ss,
              q ? (T + TQ - 1) / TQ : 0, vt};
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (int rc_capture = refuse_capture(st)) return rc_capture;
     const int m = 2 * mh;
     rc = dispatch_kfeat(dtype, E, m, a, st);
     if (rc || q) return rc;          // with query features asked for (several parts per query tile) the
@@ -4370,7 +4371,9 @@ static int sblocal_fwd_checked(const void* q, const void* k, const void* v, cons
               B, H, T, S, mh_valid, local_context, nc, n_parts,
               q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss, softmax_temp,
               nullptr, nullptr, nullptr};
-    return dispatch_fwd(dtype, E, 2 * mh, a, reinterpret_cast<hipStream_t>(stream));
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (int rc_capture = refuse_capture(st)) return rc_capture;
+    return dispatch_fwd(dtype, E, 2 * mh, a, st);
 }
 
 extern "C" int flyhip_sblocal_fwd(const void* q, const void* k, const void* v, const float* proj,
@@ -4402,9 +4405,10 @@ struct SbWorkspace {
     int n_chunks, n_split, n_parts;
 };
 // Every piece starts at a multiple of 256 bytes.  E: padded head dim (= D), mh: padded projection rows.
-SbWorkspace sb_workspace(int B, int H, int T, int S, int E, int mh, int local_context, int dtype) {
+SbWorkspace sb_workspace(int B, int H, int T, int S, int E, int mh, int local_context, int dtype, bool exact_fp32) {
     SbWorkspace w{};
-    plan(B, H, S, key_pass_wgs_per_cu(dtype, E, mh), &w.n_chunks, &w.n_split);
+    // (the fp32-pipe key pass, like the bf16 one, keeps two workgroups per compute unit resident)
+    plan(B, H, S, exact_fp32 ? 2 : key_pass_wgs_per_cu(dtype, E, mh), &w.n_chunks, &w.n_split);
     w.n_parts = plan_parts(B, H, T, S, local_context);
     const size_t bh = (size_t)B * H, nc = w.n_chunks, ns = w.n_split, m = 2 * (size_t)mh, n_qt = (T + TQ - 1) / TQ;
     const size_t esize = dtype == F32 ? 4 : 2;
@@ -4427,9 +4431,13 @@ SbWorkspace sb_workspace(int B, int H, int T, int S, int E, int mh, int local_co
 }
 }  // namespace
 
-extern "C" int64_t flyhip_sb_workspace_bytes(int B, int H, int T, int S, int E, int mh, int local_context, int dtype) {
+// flags of flyhip_sblocal_forward / flyhip_sb_workspace_bytes
+constexpr int SB_EXACT_FP32 = 1;
+
+extern "C" int64_t flyhip_sb_workspace_bytes(int B, int H, int T, int S, int E, int mh, int local_context, int dtype, int flags) {
     if (B <= 0 || H <= 0 || T <= 0 || S <= 0 || E <= 0 || mh <= 0 || local_context <= 0 || (dtype != F32 && dtype != BF16)) return -1;
-    return (int64_t)sb_workspace(B, H, T, S, E, mh, local_context, dtype).total;
+    if (flags & ~SB_EXACT_FP32) return -1;
+    return (int64_t)sb_workspace(B, H, T, S, E, mh, local_context, dtype, dtype == F32 && (flags & SB_EXACT_FP32)).total;
 }
 
 extern "C" int flyhip_sblocal_forward(const void* q, const void* k, const void* v, const float* proj,
@@ -4440,19 +4448,23 @@ extern "C" int flyhip_sblocal_forward(const void* q, const void* k, const void* 
                                       int64_t k_sb, int64_t k_sh, int64_t k_ss,
                                       int64_t v_sb, int64_t v_sh, int64_t v_ss,
                                       int64_t o_sb, int64_t o_sh, int64_t o_ss,
-                                      float softmax_temp, int dtype, void* stream) {
+                                      float softmax_temp, int dtype, int flags, void* stream) {
     FLY_REQUIRE(q && k && v && proj && out && log_norm && workspace, "sblocal_forward: null pointer");
+    FLY_REQUIRE((flags & ~SB_EXACT_FP32) == 0, "sblocal_forward: unknown flags 0x%x", flags);
     FLY_REQUIRE(B > 0 && H > 0 && T > 0 && S > 0 && local_context >= 1, "sblocal_forward: empty problem");
     FLY_REQUIRE(dtype == F32 || dtype == BF16, "sblocal_forward supports float32 and bfloat16, got dtype code %d", dtype);
     FLY_REQUIRE(E == D && E > 0 && mh > 0, "sblocal_forward: padded head dims must be equal (E=%d, D=%d)", E, D);
     FLY_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0, "sblocal_forward: the workspace must be aligned to 256 bytes");
-    const SbWorkspace w = sb_workspace(B, H, T, S, E, mh, local_context, dtype);
+    // float inputs: products on the bf16 matrix pipe from operands in bf16 pieces (the key pass leaves tile images in
+    // `vt`), unless the caller asks for the fp32 matrix pipe throughout (no images: vt stays unused)
+    const bool exact_fp32 = dtype == F32 && (flags & SB_EXACT_FP32);
+    const SbWorkspace w = sb_workspace(B, H, T, S, E, mh, local_context, dtype, exact_fp32);
     FLY_REQUIRE(workspace_bytes >= (int64_t)w.total, "sblocal_forward: the workspace holds %lld bytes, this problem needs %lld "
                 "(flyhip_sb_workspace_bytes)", (long long)workspace_bytes, (long long)w.total);
     char* ws = reinterpret_cast<char*>(workspace);
     auto f = [&](size_t at) { return reinterpret_cast<float*>(ws + at); };
     const bool split = w.n_parts > 1;
-    void* vt = ws + w.vt;
+    void* vt = exact_fp32 ? nullptr : ws + w.vt;
     void* kvt = dtype == BF16 ? ws + w.kvt : nullptr;
     int rc = flyhip_sb_kv_reduce(k, v, proj, key_lengths, ws + w.kfeat, f(w.chunk_scale), f(w.kv_part), f(w.part_max),
                                  f(w.kv), f(w.ksum), f(w.kmax),
@@ -4567,6 +4579,7 @@ extern "C" int flyhip_sbblocksparse_fwd(const void* q, const void* k, const void
               q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss, softmax_temp,
               tl_ptr, tl_inner, tl_blk, tl_order, tl_heavy, n_heavy};
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (int rc_capture = refuse_capture(st)) return rc_capture;
     const int m = 2 * mh;
     SB_DISPATCH_E(launch_fwd_list, float, a)
 }
@@ -4589,6 +4602,7 @@ extern "C" int flyhip_local_fwd_lse(const void* q, const void* k, const void* v,
     LocalArgs a{q, k, v, key_lengths, out, B, H, T, S, local_context,
                 q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss, softmax_temp, lse};
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (int rc_capture = refuse_capture(st)) return rc_capture;
 #define LOCAL_DISPATCH(TT)                                                                          \
     switch (E) {                                                                                    \
         case 32: return launch_local<TT, 32>(a, st);                                                \
@@ -4652,6 +4666,7 @@ extern "C" int flyhip_sblocal_bwd(const float* x1, const float* x2, const float*
 
 static int dispatch_bwd_band(const BwdArgs& a, int E, int M, int key_major, void* stream) {
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (int rc_capture = refuse_capture(st)) return rc_capture;
     if (E == 32 && M == 32) return launch_bwd_band_both<32, 32>(a, key_major != 0, st);
     if (E == 32 && M == 64) return launch_bwd_band_both<32, 64>(a, key_major != 0, st);
     if (E == 64 && M == 32) return launch_bwd_band_both<64, 32>(a, key_major != 0, st);

@@ -998,6 +998,7 @@ extern "C" int flyhip_sblocal_bwd_prep(const float* q, const float* k, const flo
                BH, H, T, S, mh_valid, 0, 0, 0, softmax_temp};
     prep_splits(BH, T, S, a.n_kblk, a.n_split_k, a.n_split_q);
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (int rc_capture = refuse_capture(st)) return rc_capture;
     if (E == 32 && M == 32) return launch_prep<32, 32>(a, st);
     if (E == 32 && M == 64) return launch_prep<32, 64>(a, st);
     if (E == 64 && M == 32) return launch_prep<64, 32>(a, st);
@@ -1035,6 +1036,7 @@ extern "C" int flyhip_sblocal_bwd_pieces(const void* outer_images, const void* i
                 log_norm, c, key_lengths, d1, d3, BH, H, T, S, local_context, softmax_temp, gmat, gvec, proj, 0, part_ws, 1,
                 nullptr, nullptr, nullptr, nullptr, nullptr, 0};
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (int rc_capture = refuse_capture(st)) return rc_capture;
     const long wsf = part_ws ? (long)part_ws_floats : 0;
     if (E == 32 && M == 32) return launch_bwd_x3_both<32, 32>(a, wsf, key_major != 0, st);
     if (E == 32 && M == 64) return launch_bwd_x3_both<32, 64>(a, wsf, key_major != 0, st);
@@ -1071,6 +1073,7 @@ extern "C" int flyhip_sbblocksparse_bwd_pieces(const void* outer_images, const v
                 log_norm, c, nullptr, d1, d3, BH, H, T, S, 1, softmax_temp, gmat, gvec, proj, 0, part_ws, n_heavy ? heavy_parts : 1,
                 tl_ptr, tl_inner, tl_blk, n_heavy ? tl_skip : nullptr, n_heavy ? tl_heavy : nullptr, n_heavy};
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (int rc_capture = refuse_capture(st)) return rc_capture;
     const long wsf = part_ws ? (long)part_ws_floats : 0;
     if (E == 32 && M == 32) return launch_bwd_x3_both<32, 32>(a, wsf, key_major != 0, st);
     if (E == 32 && M == 64) return launch_bwd_x3_both<32, 64>(a, wsf, key_major != 0, st);

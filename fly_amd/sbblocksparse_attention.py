@@ -16,7 +16,7 @@ from .blocksparse_attention import instantiate
 from .blocksparse_matmul import matmul
 from .blocksparse_softmax import blocksparse_sum, logsumexp
 from .blocksparse_utils import densify_tensor, sparsify_broadcast_tensor, union_heavy, union_order, union_table
-from .sblocal_attention import sbblocksparse_forward, sbblocksparse_forward_supported
+from .sblocal_attention import ScratchCache, sbblocksparse_forward, sbblocksparse_forward_supported
 from .feature_maps_sb import SBPerformerFeatures
 from .padding import pad_to_multiple
 from .scatterbrain_utils import linear_attention, linear_attention_normalization
@@ -58,8 +58,8 @@ class _SBBlockSparseFn(torch.autograd.Function):
     the band replaced by the layout's blocks (sblocal_backward.sblocal_backward, support=...)."""
 
     @staticmethod
-    def forward(ctx, query, key, value, projection_matrix, tables, support, softmax_temp):
-        out, log_norm = sbblocksparse_forward(query, key, value, projection_matrix, tables, softmax_temp)
+    def forward(ctx, query, key, value, projection_matrix, tables, support, softmax_temp, cache=None):
+        out, log_norm = sbblocksparse_forward(query, key, value, projection_matrix, tables, softmax_temp, cache=cache)
         ctx.save_for_backward(query, key, value, projection_matrix, out, log_norm)
         ctx.support, ctx.softmax_temp = support, softmax_temp
         ctx.mark_non_differentiable(log_norm)
@@ -71,7 +71,7 @@ class _SBBlockSparseFn(torch.autograd.Function):
         query, key, value, projection_matrix, out, log_norm = ctx.saved_tensors
         dq, dk, dv = sblocal_backward(query, key, value, projection_matrix, 1, ctx.softmax_temp, None, out, log_norm,
                                       grad_out, support=ctx.support)
-        return dq, dk, dv, None, None, None, None
+        return dq, dk, dv, None, None, None, None, None
 
 
 class SBBlockSparseAttention(nn.Module):
@@ -103,6 +103,8 @@ class SBBlockSparseAttention(nn.Module):
         self.backward_tables = dict()
         # eligible forward passes run on the fused kernels; set to False to force the op-by-op path
         self.fuse = True
+        # their device scratch (plan) and padded projection, kept between calls
+        self._scratch_cache = ScratchCache()
 
     def get_layout(self, T, S=None):
         if S is None:
@@ -174,14 +176,15 @@ class SBBlockSparseAttention(nn.Module):
             # (2-byte inputs are widened, as on the op-by-op path below)
             if not needs_grad:
                 out, _ = sbblocksparse_forward(query.float(), key.float(), value.float(),
-                                               self.feature_map.projection_matrix, self.fused_tables[key_], softmax_temp)
+                                               self.feature_map.projection_matrix, self.fused_tables[key_], softmax_temp,
+                                               cache=self._scratch_cache)
                 return out.to(query.dtype), None
             if key_ not in self.backward_tables:     # the support seen from the queries and from the keys
                 self.backward_tables[key_] = (backward_tables(layout, query.device),
                                               backward_tables(layout, query.device, transposed=True))
             support = self.backward_tables[key_]
             out, _ = _SBBlockSparseFn.apply(query.float(), key.float(), value.float(), self.feature_map.projection_matrix,
-                                            self.fused_tables[key_], support, softmax_temp)
+                                            self.fused_tables[key_], support, softmax_temp, self._scratch_cache)
             return out.to(query.dtype), None
 
         # 2-byte inputs are widened: the scores pass through HBM between the stages, and a score kept

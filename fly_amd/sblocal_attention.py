@@ -2,6 +2,7 @@
 src/models/attention/sblocal_attention.py (class SBLocalAttention, :15-137)."""
 import ctypes
 import math
+import weakref
 
 import torch
 import torch.nn as nn
@@ -42,7 +43,7 @@ class SBLocalPlan:
     flyhip_sblocal_fwd) on individually allocated buffers, which are created on first use."""
 
     def __init__(self, B, H, T, S, dim, mh, mh_valid, dtype, device, local_context, n_parts=None,
-                 operand_images=True):
+                 operand_images=True, exact_fp32=False):
         n_chunks, n_split, parts = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
         _lib.call('flyhip_sb_plan_for', B, H, T, S, local_context, dim, mh, _lib.DTYPE_CODE[dtype],
                   ctypes.byref(n_chunks), ctypes.byref(n_split), ctypes.byref(parts))
@@ -55,13 +56,16 @@ class SBLocalPlan:
         self.dtype = dtype
         self.code = _lib.DTYPE_CODE[dtype]
         self.operand_images = operand_images
+        # float inputs only: every product on the fp32 matrix pipe (flag FLYHIP_SB_EXACT_FP32 of the one-call entry
+        # point) instead of bf16 pieces on the bf16 pipe
+        self.flags = _lib.SB_EXACT_FP32 if (exact_fp32 and dtype == torch.float32) else 0
         self.workspace = None
         self._buffers = False
 
     def _workspace(self):
         if self.workspace is None:
             B, H, T, S, dim, mh, _ = self.shape
-            size = _lib.load().flyhip_sb_workspace_bytes(B, H, T, S, dim, mh, self.local_context, self.code)
+            size = _lib.load().flyhip_sb_workspace_bytes(B, H, T, S, dim, mh, self.local_context, self.code, self.flags)
             if size < 0:
                 raise ValueError('flyhip_sb_workspace_bytes rejected the problem shape')
             self.workspace = torch.empty(size, dtype=torch.uint8, device=self.device)
@@ -195,28 +199,80 @@ class SBLocalPlan:
                       B, H, T, S, dim, dim, mh, mh_valid, local_context,
                       q.stride(0), q.stride(2), q.stride(1), k.stride(0), k.stride(2), k.stride(1),
                       v.stride(0), v.stride(2), v.stride(1), out.stride(0), out.stride(2), out.stride(1),
-                      t, self.code, _lib.stream_ptr(self.device))
+                      t, self.code, self.flags, _lib.stream_ptr(self.device))
+
+
+class ScratchCache:
+    """What a caller keeps between forwards so that a repeated call allocates nothing but its results: the plans
+    (device scratch) of the most recently used problem shapes and the padded projection.
+
+    At most ``max_plans`` plans are kept, least recently used dropped first (a plan holds the scratch of its shape:
+    roughly 200 MB at batch 64, L = 3136); callers with ever-changing sequence lengths therefore do not grow device
+    memory without bound.  The cache is per process and per object: copies and pickles of its owner start empty."""
+
+    def __init__(self, max_plans=4):
+        self.max_plans = max_plans
+        self.plans = {}                  # insertion-ordered: oldest use first
+        self._proj_src = None            # weak reference to the caller's projection tensor the padded copy was made from
+        self._proj_stamp = None
+        self._proj = None
+
+    def plan(self, key, make):
+        got = self.plans.pop(key, None)
+        if got is None:
+            got = make()
+            while len(self.plans) >= self.max_plans:
+                self.plans.pop(next(iter(self.plans)))
+        self.plans[key] = got            # (re-)inserted as the most recent
+        return got
+
+    def padded_projection(self, projection_matrix, mh, dim):
+        """The padded float32 copy of `projection_matrix`, remade when the caller's tensor is another object than the
+        one the copy was made from (same address and version are not enough: a replaced buffer often gets both)
+        or has been written to since."""
+        src = None if self._proj_src is None else self._proj_src()
+        stamp = (projection_matrix._version, mh, dim, projection_matrix.device)
+        if src is projection_matrix and stamp == self._proj_stamp:
+            return self._proj
+        self._proj = _pad_projection(projection_matrix, mh, dim)
+        self._proj_src, self._proj_stamp = weakref.ref(projection_matrix), stamp
+        return self._proj
+
+    def clear(self):
+        self.plans.clear()
+        self._proj_src = self._proj_stamp = self._proj = None
+
+    def __len__(self):
+        return len(self.plans)
+
+    def __deepcopy__(self, memo):
+        return ScratchCache(self.max_plans)
+
+    def __reduce__(self):
+        return (ScratchCache, (self.max_plans,))
+
+
+def _pad_projection(projection_matrix, mh, dim):
+    mh_valid, E = projection_matrix.shape
+    proj = torch.zeros(mh, dim, dtype=torch.float32, device=projection_matrix.device)
+    proj[:mh_valid, :E] = projection_matrix.to(torch.float32)
+    return proj
 
 
 def _padded_projection(projection_matrix, mh, dim, cache):
     """The projection as the kernels want it: float32, (mh, dim), zero rows / columns as padding.  The caller's
-    tensor itself when it already has that form; otherwise a padded copy, kept in `cache` until the
+    tensor itself when it already has that form; otherwise a padded copy, kept in `cache` (a ScratchCache) until the
     caller's tensor is replaced or written to."""
-    mh_valid, E = projection_matrix.shape
-    if (mh_valid, E) == (mh, dim) and projection_matrix.dtype == torch.float32 and projection_matrix.is_contiguous():
+    if (tuple(projection_matrix.shape) == (mh, dim) and projection_matrix.dtype == torch.float32
+            and projection_matrix.is_contiguous()):
         return projection_matrix
-    stamp = (projection_matrix.data_ptr(), projection_matrix._version, mh, dim)
-    if cache is not None and cache.get('projection_stamp') == stamp:
-        return cache['projection']
-    proj = torch.zeros(mh, dim, dtype=torch.float32, device=projection_matrix.device)
-    proj[:mh_valid, :E] = projection_matrix.to(torch.float32)
-    if cache is not None:
-        cache['projection_stamp'], cache['projection'] = stamp, proj
-    return proj
+    if cache is None:
+        return _pad_projection(projection_matrix, mh, dim)
+    return cache.padded_projection(projection_matrix, mh, dim)
 
 
 def sblocal_forward(query, key, value, projection_matrix, local_context, softmax_temp=None,
-                    key_lengths=None, cache=None):
+                    key_lengths=None, cache=None, exact_fp32=False):
     """Scatterbrain-local attention forward on the GPU.
 
     query (B,T,H,E), key (B,S,H,E), value (B,S,H,D) float32 or bfloat16 CUDA tensors;
@@ -224,9 +280,13 @@ def sblocal_forward(query, key, value, projection_matrix, local_context, softmax
     sblocal_attention.py:73-122 computes for causal=False, attn_mask=None, eps=0, no dropout.
     Returns (out (B,T,H,D) in the input dtype, log_normalization (B,H,T,1) float32).
 
-    cache: an optional dict the caller keeps between calls (SBLocalAttention keeps one per module).  It holds
-    the plan -- the device scratch -- of every problem shape seen and the padded projection, so that a repeated
-    call allocates nothing but its two results.  Calls that share a cache share scratch: one at a time.
+    cache: an optional ScratchCache the caller keeps between calls (SBLocalAttention keeps one per module).  It
+    holds the plans -- the device scratch -- of the last few problem shapes and the padded projection, so that a
+    repeated call allocates nothing but its two results.  Calls that share a cache share scratch: one at a time.
+
+    exact_fp32: float32 inputs only.  False (default): products on the bf16 matrix pipe from operands split into bf16
+    pieces with fp32 accumulation (V rounded to 16, the features to 17 significant bits; about 5e-6 of the float64
+    result at the benchmark configuration).  True: every product on the fp32 matrix pipe (about 1e-6; 1.6 times the time).
     """
     _lib.require_gpu(query, key, value, projection_matrix, key_lengths)
     if query.dtype not in (torch.float32, torch.bfloat16):
@@ -261,12 +321,13 @@ def sblocal_forward(query, key, value, projection_matrix, local_context, softmax
         if lens.shape != (B,):
             raise ValueError(f'key_lengths must have shape ({B},)')
 
-    plan_key = (B, H, T, S, dim, mh, mh_valid, query.dtype, query.device, local_context)
-    plan = None if cache is None else cache.get(plan_key)
-    if plan is None:
-        plan = SBLocalPlan(B, H, T, S, dim, mh, mh_valid, query.dtype, query.device, local_context)
-        if cache is not None:
-            cache[plan_key] = plan
+    exact_fp32 = bool(exact_fp32) and query.dtype == torch.float32
+    plan_key = (B, H, T, S, dim, mh, mh_valid, query.dtype, query.device, local_context, exact_fp32)
+
+    def make_plan():
+        return SBLocalPlan(B, H, T, S, dim, mh, mh_valid, query.dtype, query.device, local_context,
+                           exact_fp32=exact_fp32)
+    plan = make_plan() if cache is None else cache.plan(plan_key, make_plan)
     out = torch.empty(B, T, H, dim, dtype=query.dtype, device=query.device)
     log_norm = torch.empty(B, H, T, dtype=torch.float32, device=query.device)
     plan.run(q, k, v, proj, lens, local_context, t, out, log_norm)
@@ -279,13 +340,15 @@ def sbblocksparse_forward_supported(block, dtype, E, D, n_projection_rows, layou
             and n_projection_rows <= _FEATURE_ROWS[-1] and layout_heads == H)
 
 
-def sbblocksparse_forward(query, key, value, projection_matrix, tables, softmax_temp=None):
+def sbblocksparse_forward(query, key, value, projection_matrix, tables, softmax_temp=None, cache=None):
     """Scatterbrain attention on a block-sparse support (sbblocksparse_attention.py:109-213 for
     need_weights=False, no dropout) on the fused kernels: exact softmax weights on the nonzero 32 x 32
     blocks, the Performer estimate everywhere else, one normaliser.  query (B,T,H,E), key (B,S,H,E), value
     (B,S,H,D) float32 GPU tensors, T and S multiples of 32; tables = union_table(layout, rows_per_group=2)
     as int32 tensors on the device, optionally followed by union_order(tables[0], H), or the six entries of
-    sbblocksparse_attention.fused_tables (start order with the long lists marked, those lists, their parts).  Returns (out (B,T,H,D), log_normalization (B,H,T,1))."""
+    sbblocksparse_attention.fused_tables (start order with the long lists marked, those lists, their parts).
+    cache: an optional ScratchCache kept by the caller (plan and padded projection, as for sblocal_forward).
+    Returns (out (B,T,H,D), log_normalization (B,H,T,1))."""
     _lib.require_gpu(query, key, value, projection_matrix)
     B, T, H, E = query.shape
     S, D = key.shape[1], value.shape[3]
@@ -301,10 +364,13 @@ def sbblocksparse_forward(query, key, value, projection_matrix, tables, softmax_
             x = F.pad(x, (0, dim - x.shape[-1]))
         return x if _vector_ready(x) else x.contiguous()
     q, k, v = prep(query), prep(key), prep(value)
-    proj = torch.zeros(mh, dim, dtype=torch.float32, device=query.device)
-    proj[:mh_valid, :E] = projection_matrix.to(torch.float32)
-    plan = SBLocalPlan(B, H, T, S, dim, mh, mh_valid, query.dtype, query.device, 64, n_parts=1,
-                       operand_images=False)
+    proj = _padded_projection(projection_matrix, mh, dim, cache)
+
+    def make_plan():
+        return SBLocalPlan(B, H, T, S, dim, mh, mh_valid, query.dtype, query.device, 64, n_parts=1,
+                           operand_images=False)
+    plan_key = ('block-sparse', B, H, T, S, dim, mh, mh_valid, query.dtype, query.device)
+    plan = make_plan() if cache is None else cache.plan(plan_key, make_plan)
     out = torch.empty(B, T, H, dim, dtype=query.dtype, device=query.device)
     log_norm = torch.empty(B, H, T, dtype=torch.float32, device=query.device)
     plan.run_block_sparse(q, k, v, proj, t, tables, out, log_norm)
@@ -316,9 +382,11 @@ class _SBLocalFn(torch.autograd.Function):
     forward is the fused kernel path; the backward is sblocal_backward.sblocal_backward."""
 
     @staticmethod
-    def forward(ctx, query, key, value, projection_matrix, local_context, softmax_temp, key_lengths, cache=None):
+    def forward(ctx, query, key, value, projection_matrix, local_context, softmax_temp, key_lengths, cache=None,
+                exact_fp32=False):
         out, log_norm = sblocal_forward(query, key, value, projection_matrix, local_context,
-                                        softmax_temp=softmax_temp, key_lengths=key_lengths, cache=cache)
+                                        softmax_temp=softmax_temp, key_lengths=key_lengths, cache=cache,
+                                        exact_fp32=exact_fp32)
         ctx.save_for_backward(query, key, value, projection_matrix, out, log_norm)
         ctx.args = (local_context, softmax_temp, key_lengths)
         ctx.mark_non_differentiable(log_norm)
@@ -331,16 +399,17 @@ class _SBLocalFn(torch.autograd.Function):
         local_context, softmax_temp, key_lengths = ctx.args
         dq, dk, dv = sblocal_backward(query, key, value, projection_matrix, local_context, softmax_temp,
                                       key_lengths, out, log_norm, grad_out)
-        return dq, dk, dv, None, None, None, None, None
+        return dq, dk, dv, None, None, None, None, None, None
 
 
 def sblocal_attention_fn(query, key, value, projection_matrix, local_context, softmax_temp=None,
-                         key_lengths=None, cache=None):
+                         key_lengths=None, cache=None, exact_fp32=False):
     """sblocal_forward, differentiable with respect to query, key and value."""
     if torch.is_grad_enabled() and any(x.requires_grad for x in (query, key, value)):
-        return _SBLocalFn.apply(query, key, value, projection_matrix, local_context, softmax_temp, key_lengths, cache)
+        return _SBLocalFn.apply(query, key, value, projection_matrix, local_context, softmax_temp, key_lengths, cache,
+                                exact_fp32)
     return sblocal_forward(query, key, value, projection_matrix, local_context, softmax_temp=softmax_temp,
-                           key_lengths=key_lengths, cache=cache)
+                           key_lengths=key_lengths, cache=cache, exact_fp32=exact_fp32)
 
 
 class SBLocalAttention(nn.Module):
@@ -368,8 +437,10 @@ class SBLocalAttention(nn.Module):
         self.softmax_temp = softmax_temp
         self.dropout = nn.Dropout(attention_dropout)
         self.softmax_eps = softmax_eps
-        # device scratch per problem shape and the padded projection, kept between calls (see sblocal_forward)
-        self._scratch_cache = {}
+        # device scratch of the last few problem shapes and the padded projection, kept between calls (see sblocal_forward)
+        self._scratch_cache = ScratchCache()
+        # float32 inputs: True selects the fp32 matrix pipe for every product instead of bf16 pieces (see sblocal_forward)
+        self.exact_fp32 = False
         # need_weights builds the dense (B,H,T,S) matrix with library products: an inspection aid, not a fast path
         self.max_weight_elements = 1 << 26
 
@@ -395,7 +466,8 @@ class SBLocalAttention(nn.Module):
         self.feature_map.new_feature_map(query.device)
         out, log_norm = sblocal_attention_fn(query, key, value, self.feature_map.projection_matrix,
                                              self.local_context, softmax_temp=self.softmax_temp,
-                                             key_lengths=lengths, cache=self._scratch_cache)
+                                             key_lengths=lengths, cache=self._scratch_cache,
+                                             exact_fp32=self.exact_fp32)
         self.last_log_normalization = log_norm.detach()
         attn = None
         if need_weights or return_attn_unnormalized:

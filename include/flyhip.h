@@ -8,7 +8,10 @@
  *   - entry points return 0 on success and a negative code otherwise; the message is
  *     available from flyhip_last_error() (thread-local);
  *   - dtype: 0 = float32, 1 = bfloat16, 2 = float16 (storage type; accumulation is fp32);
- *   - strides are in elements.
+ *   - strides are in elements;
+ *   - a stream that is under capture into a HIP graph is refused (negative return, message): the
+ *     launchers do work on first use that is not a stream operation, so calls of this library
+ *     are to be made eagerly.
  *
  * "ref:" comments name the interface in the reference checkout that each entry point replaces.
  */
@@ -118,8 +121,12 @@ int flyhip_sblocal_fwd(const void* q, const void* k, const void* v, const float*
  * kernel runs on the bf16 matrix pipe).  flyhip_sb_workspace_bytes gives its size for a problem (E = D: padded
  * head dim, mh: padded projection rows; -1 for bad arguments).  The workspace must be aligned to 256 bytes; its
  * contents need no initialisation and mean nothing between calls; one call at a time may use it.
- * Arguments as for flyhip_sb_kv_reduce / flyhip_sblocal_fwd. */
-int64_t flyhip_sb_workspace_bytes(int B, int H, int T, int S, int E, int mh, int local_context, int dtype);
+ * flags: 0, or FLYHIP_SB_EXACT_FP32 -- float inputs then take the fp32 matrix pipe for every product (no bf16
+ * pieces, V and the features not rounded: about 1e-6 of the float64 result instead of 5e-6, at 1.6 times the
+ * time); pass the same flags to both functions.  Arguments otherwise as for flyhip_sb_kv_reduce /
+ * flyhip_sblocal_fwd. */
+#define FLYHIP_SB_EXACT_FP32 1
+int64_t flyhip_sb_workspace_bytes(int B, int H, int T, int S, int E, int mh, int local_context, int dtype, int flags);
 int flyhip_sblocal_forward(const void* q, const void* k, const void* v, const float* proj,
                            const int64_t* key_lengths, void* out, float* log_norm,
                            void* workspace, int64_t workspace_bytes,
@@ -128,17 +135,18 @@ int flyhip_sblocal_forward(const void* q, const void* k, const void* v, const fl
                            int64_t k_sb, int64_t k_sh, int64_t k_ss,
                            int64_t v_sb, int64_t v_sh, int64_t v_ss,
                            int64_t o_sb, int64_t o_sh, int64_t o_ss,
-                           float softmax_temp, int dtype, void* stream);
+                           float softmax_temp, int dtype, int flags, void* stream);
 
-/* flyhip_sblocal_fwd for callers that cannot allocate device memory -- code under HIP graph capture,
- * tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.
+/* flyhip_sblocal_fwd for callers that cannot allocate device memory -- tight serving loops, harnesses
+ * that forbid hipMalloc.  It has no counterpart in the reference.
  * Same arguments and results as flyhip_sblocal_fwd except that there is no part_ws: the partial
  * outputs of the parts of a query tile go to a fixed 16 MiB array inside the library (one copy per
  * GPU, held until the process ends).  The call allocates and frees nothing.  It fails with a
  * message when B*H*ceil(T/64)*n_parts*64*(D+5) exceeds 4 Mi floats (n_parts > 1 only; with
  * n_parts == 1 no scratch is used).  All calls on one GPU share that array: calls that overlap in
  * time on one GPU (different streams or threads) race.  Its address is looked up on the first call
- * on each device, with that device current; make that first call outside a graph capture. */
+ * on each device, with that device current.  (Like every entry point of this library it refuses a stream
+ * that is under graph capture.) */
 int flyhip_sblocal_fwd_static(const void* q, const void* k, const void* v, const float* proj,
                               const void* kfeat, const float* chunk_scale,
                               float* kv, float* ksum, float* kmax,

@@ -61,16 +61,33 @@ def test_config3_t2t_vit_logits_parity():
         assert rel_err(full[:2].cpu(), want) <= 1e-4
 
 
+def atol_needed(got, ref, rtol=1e-4):
+    """The smallest atol with which torch.allclose(got, ref, rtol, atol) holds (negative: rtol alone suffices)."""
+    got, ref = got.detach().double().cpu(), ref.detach().double().cpu()
+    return float(((got - ref).abs() - rtol * ref.abs()).max())
+
+
 @pytest.mark.parametrize('L,dim', [(3136, 147), (784, 576)])
 def test_config3_attention_layers_parity(L, dim):
+    """Both Scatterbrain-local layers of T2T-ViT at their real size (batch 4): 1e-4 of the tensor's maximum, and
+    elementwise rtol 1e-4 with a stated atol.  The outputs are of order one here (unscaled N(0,1) values), so an atol
+    of 1e-6 is float32 resolution: the float32 oracle itself needs 5e-7.  The fp32-pipe kernels hold 1e-6; the default
+    kernels (bf16 pieces, V rounded to 16 bits) need 2e-6 .. 4.2e-6 and are held to 6e-6 -- the measured values are
+    printed."""
     from fly_amd import sblocal_forward
     g = torch.Generator().manual_seed(L)
     q, k, v = (torch.randn(4, L, 1, 64, generator=g) for _ in range(3))
     P = osb.gaussian_orthogonal_random_matrix(64, 64, generator=g)
     t = dim ** -0.5
-    out, ln = sblocal_forward(q.to(DEV), k.to(DEV), v.to(DEV), P.to(DEV), 256, softmax_temp=t)
     ref_out, ref_ln = osb.sblocal_attention(q.double(), k.double(), v.double(), P.double(), 256, softmax_temp=t)
-    assert rel_err(out, ref_out) <= 1e-4 and rel_err(ln, ref_ln) <= 1e-4
+    for exact, atol in ((False, 6e-6), (True, 1e-6)):
+        out, ln = sblocal_forward(q.to(DEV), k.to(DEV), v.to(DEV), P.to(DEV), 256, softmax_temp=t, exact_fp32=exact)
+        need = atol_needed(out, ref_out)
+        print('exact_fp32', exact, 'out', rel_err(out, ref_out), 'log-normaliser', rel_err(ln, ref_ln),
+              'atol needed at rtol 1e-4', need, flush=True)
+        assert rel_err(out, ref_out) <= 1e-4 and rel_err(ln, ref_ln) <= 1e-4
+        assert need <= atol, need
+        assert torch.allclose(ln.double().cpu(), ref_ln, rtol=1e-4, atol=1e-6)
 
 
 def test_config4_pixelfly_mlp_bf16():

@@ -32,12 +32,16 @@ def run_both(q, k, v, P, lc, t=None, lengths=None):
     return out.float().cpu(), ln.cpu(), ref_out, ref_ln
 
 
-# fp32: 1e-4 relative to the tensor's max, and elementwise rtol 1e-4 with atol 1e-6 * max
-def check_fp32(out, ln, ref_out, ref_ln, tol=1e-4):
+# fp32: 1e-4 relative to the tensor's max, elementwise rtol 1e-4 on the log-normaliser, and -- with `elementwise` --
+# elementwise rtol 1e-4 with atol 1e-6 on the output as well
+def check_fp32(out, ln, ref_out, ref_ln, tol=1e-4, elementwise=False):
     assert out.shape == ref_out.shape and ln.shape == ref_ln.shape
     assert rel_err(out, ref_out) <= tol, rel_err(out, ref_out)
     assert rel_err(ln, ref_ln) <= tol, rel_err(ln, ref_ln)
     assert torch.allclose(ln.double(), ref_ln, rtol=tol, atol=1e-5)
+    if elementwise:
+        need = float(((out.double() - ref_out).abs() - tol * ref_out.abs()).max())
+        assert need <= 1e-6, f'elementwise rtol {tol} needs atol {need:.2e} (bar 1e-6)'
 
 
 @pytest.mark.parametrize('case', [
@@ -102,7 +106,33 @@ def test_fp32_wide_heads_with_unscaled_inputs(B, H, T, S, E, D, mh, lc, lens):
 def test_config1_full_size():
     """BASELINE config 1: B=2, H=1, L=3136, d=64, window 512, 128 features, fp32; q, k, v ~ N(0,1) d^-1/4."""
     q, k, v, P = make_inputs(2, 3136, 3136, 1, 64, 64, 64, seed=0, scale_v=True)
-    check_fp32(*run_both(q, k, v, P, 512))
+    check_fp32(*run_both(q, k, v, P, 512), elementwise=True)
+
+
+def test_config1_both_arithmetics_pinned():
+    """Config 1 on the default kernels (products on the bf16 matrix pipe from bf16 pieces, V rounded to 16 and the
+    features to 17 significant bits) and with exact_fp32=True (the fp32 matrix pipe throughout, the flag
+    FLYHIP_SB_EXACT_FP32 of the one-call entry point): both within 1e-4 elementwise (atol 1e-6); the pieces within
+    1e-5 of the maximum, the fp32 pipe within 2e-6 (measured 4.0e-6 and 6.2e-7; the float32 oracle 1.1e-6)."""
+    from fly_amd import sblocal_forward, SBLocalAttention
+    dev = torch.device('cuda:0')
+    q, k, v, P = make_inputs(2, 3136, 3136, 1, 64, 64, 64, seed=0, scale_v=True)
+    ref_out, ref_ln = osb.sblocal_attention(q.double(), k.double(), v.double(), P.double(), 512)
+    outs = {}
+    for exact, bar in ((False, 1e-5), (True, 2e-6)):
+        out, ln = sblocal_forward(q.to(dev), k.to(dev), v.to(dev), P.to(dev), 512, exact_fp32=exact)
+        check_fp32(out.cpu(), ln.cpu(), ref_out, ref_ln, elementwise=True)
+        print('exact_fp32', exact, rel_err(out, ref_out), rel_err(ln, ref_ln), flush=True)
+        assert rel_err(out, ref_out) <= bar and rel_err(ln, ref_ln) <= 1e-6
+        outs[exact] = out
+    assert not torch.equal(outs[False], outs[True])                  # two different arithmetics did run
+    attn = SBLocalAttention(512, dim_heads=64, nb_features=128).to(dev).eval()
+    attn.feature_map.projection_matrix.copy_(P.to(dev))
+    attn.feature_map.freeze_projection()
+    attn.exact_fp32 = True
+    with torch.no_grad():
+        got, _ = attn(q.to(dev), k.to(dev), v.to(dev))
+    assert torch.equal(got, outs[True])                              # the module's switch reaches the same kernels
 
 
 @pytest.mark.parametrize('n_parts', [5, 3, 8, 12, 1])
@@ -541,3 +571,28 @@ def test_random_shapes_sweep():
             got = sblocal_backward(*args, band_kernel=True)
             for a, b in zip(got, ref):
                 assert rel_err(a, b) <= 2e-4, rel_err(a, b)
+
+
+def test_module_scratch_stays_bounded_over_many_shapes():
+    """More problem shapes than the module's cache keeps plans for: the cache stays at its bound and a second round
+    over the same shapes leaves the allocated device memory where the first round left it."""
+    from fly_amd import SBLocalAttention
+    dev = torch.device('cuda:0')
+    attn = SBLocalAttention(local_context=64, dim_heads=64, nb_features=64).to(dev).eval()
+    lengths = [128, 192, 256, 320, 384, 448, 512]
+    assert len(lengths) > attn._scratch_cache.max_plans
+
+    def one_round():
+        for L in lengths:
+            q, k, v, _ = make_inputs(1, L, L, 2, 64, 64, 32, seed=L)
+            with torch.no_grad():
+                out, _ = attn(q.to(dev), k.to(dev), v.to(dev))
+            assert out.shape == (1, L, 2, 64) and bool(torch.isfinite(out).all())
+            del out
+        torch.cuda.synchronize()
+    one_round()
+    assert len(attn._scratch_cache) == attn._scratch_cache.max_plans
+    held = torch.cuda.memory_allocated(dev)
+    one_round()
+    assert len(attn._scratch_cache) == attn._scratch_cache.max_plans
+    assert torch.cuda.memory_allocated(dev) == held

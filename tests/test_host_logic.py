@@ -289,3 +289,44 @@ def test_sbblocksparse_module_interface_and_refusals():
         layer(q, q, q, key_padding_mask=fly_amd.LengthMask(torch.tensor([64]), max_len=64))
     with pytest.raises(ValueError, match='head dim'):
         layer(torch.zeros(1, 64, 1, 16), q, q)
+
+
+def test_scratch_cache_is_bounded_and_tracks_the_projection_object():
+    """The per-module cache of Scatterbrain-local attention: at most max_plans plans, least recently used dropped
+    first; the padded projection is remade when the caller's tensor is REPLACED by another of the same shape (same
+    version counter, possibly the same address) or written to; copies and pickles of the cache start empty."""
+    import copy
+    import pickle
+    from fly_amd.sblocal_attention import ScratchCache, _padded_projection
+    cache = ScratchCache(max_plans=3)
+    made = []
+
+    def maker(tag):
+        def make():
+            made.append(tag)
+            return tag
+        return make
+    for tag in 'abc':
+        assert cache.plan(tag, maker(tag)) == tag
+    assert cache.plan('a', maker('a')) == 'a' and made == ['a', 'b', 'c']       # hit: nothing made, 'a' now most recent
+    cache.plan('d', maker('d'))                                                 # evicts 'b', the least recently used
+    assert len(cache) == 3 and set(cache.plans) == {'a', 'c', 'd'}
+    cache.plan('b', maker('b'))
+    assert made == ['a', 'b', 'c', 'd', 'b'] and set(cache.plans) == {'a', 'd', 'b'}
+
+    P1 = torch.randn(13, 21)
+    pad1 = _padded_projection(P1, 16, 32, cache)
+    assert pad1.shape == (16, 32) and torch.equal(pad1[:13, :21], P1) and float(pad1[13:].abs().sum()) == 0
+    assert _padded_projection(P1, 16, 32, cache) is pad1                        # unchanged tensor: the kept copy
+    P2 = torch.randn(13, 21)                                                    # a replacement: same shape, version 0
+    assert P2._version == P1._version
+    pad2 = _padded_projection(P2, 16, 32, cache)
+    assert torch.equal(pad2[:13, :21], P2)
+    P2.mul_(2.0)                                                                # written to in place
+    assert torch.equal(_padded_projection(P2, 16, 32, cache)[:13, :21], P2)
+    exact = torch.randn(16, 32)
+    assert _padded_projection(exact, 16, 32, cache) is exact                    # already in kernel form: used as is
+    assert len(copy.deepcopy(cache)) == 0 and len(pickle.loads(pickle.dumps(cache))) == 0
+    mod = fly_amd.SBLocalAttention(8, dim_heads=16, nb_features=8)
+    mod._scratch_cache.plan('x', maker('x'))
+    assert len(copy.deepcopy(mod)._scratch_cache) == 0
