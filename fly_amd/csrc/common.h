@@ -323,7 +323,13 @@ __device__ __forceinline__ void split3_4(floatx4 x, uint2& h, uint2& m, uint2& l
 __device__ __forceinline__ void dma_to_lds(const void* lane_src, const char* wave_base) {
     typedef __attribute__((address_space(3))) const char* lds_ptr;
     const uint32_t base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr)wave_base);
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(lane_src), "s"(base) : "m0", "memory");
+    // m0 carries the LDS destination of the transfer.  The compiler does not accept m0 in a clobber list (it is a
+    // reserved register), so the statement itself puts back what m0 held: whatever the compiler keeps in m0 across
+    // this point (LDS-direct reads, register-indexed moves, SGPR spills) survives.  The transfer reads m0 when it is
+    // issued, so the restore may follow it directly.
+    uint32_t saved_m0;
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b32 m0, %0"
+                 : "=&s"(saved_m0) : "v"(lane_src), "s"(base) : "memory");
 }
 
 // Transposed operand reads (ds_read_b64_tr_b16): within each group of 16 lanes, lane s passes the address of four
