@@ -1214,6 +1214,26 @@ struct TileKV16 {
 };
 
 
+#ifndef FLY_TWO_PIECE_MAX
+#define FLY_TWO_PIECE_MAX 128      // most features for which the bf16 band kernels carry the two-piece path (at 256 the
+                                   // 32-queries-per-wave kernel has no registers left for it: +13 % on every input)
+#endif
+// bf16 band kernels: the probabilities p = e - (q'.k') beta go to the P V product as bf16, 2^-9 of their size.  Where
+// the features approximate the exact weights that size is the size of the weights; where they do not (unscaled inputs,
+// few features) the band's low-rank part can be hundreds of times the exact mass for some queries, cancels against the
+// sums over all keys only in the result, and its rounding would show in the output at 2^-9 times that ratio.  Once the
+// low-rank mass a lane has gathered on its keys of the band exceeds three times their exact mass, the wave hands P over
+// in two pieces (head and rest, 2^-17) for that tile: one more pass of the tile's P V products, taken by no tile of
+// well-conditioned inputs (for them the two masses are about equal), and what passes in one piece is bounded by four
+// times the exact mass, i.e. by the normaliser.  Both masses in units of 2^m_run.
+__device__ __forceinline__ bool second_piece_wanted(float lowrank_mass_so_far, float exact_mass_so_far) {
+    return __builtin_amdgcn_ballot_w64(lowrank_mass_so_far > 3.f * exact_mass_so_far) != 0;
+}
+// what two floats lose when they are packed into the bf16 pair `head`, as a bf16 pair
+__device__ __forceinline__ uint32_t pack_rest(float a, float b, uint32_t head) {
+    return pack_bf16x2(a - __uint_as_float(head << 16), b - __uint_as_float(head & 0xffff0000u));
+}
+
 template <int E, int M> constexpr size_t fwd_bf16_smem() {
     constexpr size_t stage = (size_t)TK * (E + 8) + (size_t)TK * (M + 8) + (size_t)E * (TK + 8);   // 2-byte elements
     constexpr size_t tiles = 2 * stage * 2;
@@ -1233,6 +1253,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
     constexpr int NT = 64 * NW, TQ = 16 * NW;          // shadow the 4-wave constants of the fp32 kernels
     constexpr int TQ64 = 64;                           // queries per tile of the partial workspace / merge
     typedef bf16_t T;
+    constexpr bool TWO_PIECE = M <= FLY_TWO_PIECE_MAX;
     constexpr int MH = M / 2, FB = MH / 16, EC = E / 16, DB = D / 16, KB = TK / 16;
     constexpr int LDK = E + 8, LDF = M + 8, LDT = TK + 8, LDKV = M + 8;   // LDS row strides in elements
     constexpr int STAGE = TK * LDK + TK * LDF + D * LDT;                  // elements per stage
@@ -1535,12 +1556,21 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
                 }
         };
         if (inside) soft(std::false_type{}); else soft(std::true_type{});
+        // (see second_piece_wanted: where the band's low-rank part dwarfs the exact weights the probabilities go to
+        //  the matrix pipe in two bf16 pieces)
         zp += ovs * wc;
+        const bool two = TWO_PIECE && second_piece_wanted(zp * __builtin_amdgcn_exp2f(c0 - m_run), ze);
         // O^T[d][query] += sum_keys V[key][d] p[key][query]: one MFMA step per 16 value dims
         const uint4 pb = make_uint4(pack_bf16x2(p[0][0], p[0][1]), pack_bf16x2(p[0][2], p[0][3]),
                                     pack_bf16x2(p[1][0], p[1][1]), pack_bf16x2(p[1][2], p[1][3]));
 #pragma unroll
         for (int db = 0; db < DB; ++db) oacc[db] = mma_bf16(vf[db], pb, oacc[db]);
+        if (two) {                                               // wave-uniform
+            const uint4 pl = make_uint4(pack_rest(p[0][0], p[0][1], pb.x), pack_rest(p[0][2], p[0][3], pb.y),
+                                        pack_rest(p[1][0], p[1][1], pb.z), pack_rest(p[1][2], p[1][3], pb.w));
+#pragma unroll
+            for (int db = 0; db < DB; ++db) oacc[db] = mma_bf16(vf[db], pl, oacc[db]);
+        }
     };
     const bool late = w >= NW / 2;        // wave-uniform: this wave runs half a tile behind
     float cs_prev = 0.f;                  // chunk scale of the tile a late wave still owes its softmax
@@ -1732,6 +1762,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
     constexpr int NT = 64 * NW, TQ = 32 * NW;          // shadow the constants of the fp32 kernels
     constexpr int TQ64 = 64;                           // queries per tile of the partial workspace / merge
     typedef bf16_t T;
+    constexpr bool TWO_PIECE = M <= FLY_TWO_PIECE_MAX;
     constexpr int MH = M / 2, PB = MH / 32, KS = E / 16, FS = M / 16, DB = D / 32;
     static_assert(MH % 32 == 0 && D % 32 == 0, "whole 32-row blocks");
     constexpr int LDK = E + 8, LDKV = M + 8;           // LDS row strides in elements (projection rows, K'^T V)
@@ -2003,7 +2034,10 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
             }
         };
         if (inside) soft(std::false_type{}); else soft(std::true_type{});
+        // (see second_piece_wanted: where the band's low-rank part dwarfs the exact weights the probabilities go to
+        //  the matrix pipe in two bf16 pieces)
         zp += ovs * wc;
+        const bool two = TWO_PIECE && second_piece_wanted(zp * __builtin_amdgcn_exp2f(c0 - m_run), ze);
         // O^T[d][query] += sum_keys V[key][d] p[key][query]: step t takes the lane's elements 4t + i and 4(2 + t) + i
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
@@ -2011,6 +2045,13 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
                                          pack_bf16x2(p[4 * (2 + t)], p[4 * (2 + t) + 1]), pack_bf16x2(p[4 * (2 + t) + 2], p[4 * (2 + t) + 3]));
 #pragma unroll
             for (int db = 0; db < DB; ++db) oacc[db] = mma32_bf16(vf[db][t], pb_, oacc[db]);
+            if (two) {                                           // wave-uniform
+                const uint4 pl_ = make_uint4(pack_rest(p[4 * t], p[4 * t + 1], pb_.x), pack_rest(p[4 * t + 2], p[4 * t + 3], pb_.y),
+                                             pack_rest(p[4 * (2 + t)], p[4 * (2 + t) + 1], pb_.z),
+                                             pack_rest(p[4 * (2 + t) + 2], p[4 * (2 + t) + 3], pb_.w));
+#pragma unroll
+                for (int db = 0; db < DB; ++db) oacc[db] = mma32_bf16(vf[db][t], pl_, oacc[db]);
+            }
         }
     };
     const bool late = NW > 4 && w >= NW / 2;      // wave-uniform: this wave runs half a tile behind

@@ -146,11 +146,15 @@ def local_weighted_average(A, V, chunk=256):
 # SBLocalAttention.forward -- src/models/attention/sblocal_attention.py:43-137
 # --------------------------------------------------------------------------------------
 def sblocal_attention(query, key, value, projection_matrix, local_context, softmax_temp=None,
-                      key_lengths=None, chunk=256):
+                      key_lengths=None, chunk=256, return_band_lowrank_mass=False):
     """sblocal_attention.py:56-122 for causal=False, attn_mask=None, eps=0, dropout off.
     query (B,T,H,E), key (B,S,H,E), value (B,S,H,D); projection_matrix (m/2, E);
     key_lengths (B,) int64 or None.  The reference's ``softmax_temp or 1/sqrt(E)`` (:59)
-    treats 0/None as unset.  Returns (out (B,T,H,D), log_normalization (B,H,T,1))."""
+    treats 0/None as unset.  Returns (out (B,T,H,D), log_normalization (B,H,T,1)); with
+    return_band_lowrank_mass also (B,H,T,1): the normalised low-rank weight a query's band carries,
+    sum_band q'.k' * prime_scale -- the amount that is subtracted on the band and added back through the
+    sums over all keys (a condition number of the estimator: of order one or below when the features
+    approximate the exact weights, hundreds when they do not)."""
     B, T, H, E = query.shape
     _, S, _, D = value.shape
     t = softmax_temp or 1 / math.sqrt(E)
@@ -185,6 +189,8 @@ def sblocal_attention(query, key, value, projection_matrix, local_context, softm
     prime_scale = torch.exp(prime_log_scale - log_normalization)                  # :115
     dots = torch.exp(QK - log_normalization) - dots_prime * prime_scale           # :119
     out = local_weighted_average(dots, v, chunk) + qkv * prime_scale              # :121-122
+    if return_band_lowrank_mass:
+        return out.permute(0, 2, 1, 3), log_normalization, dots_prime_sum * prime_scale
     return out.permute(0, 2, 1, 3), log_normalization
 
 
