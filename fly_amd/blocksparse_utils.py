@@ -127,6 +127,32 @@ def union_table(layout, rows_per_group=4, transposed=False):
     return ptr.to(torch.int32), nz[:, 2].to(torch.int32).contiguous(), blk.to(torch.int32).contiguous()
 
 
+def tile_mask_table(layout, block):
+    """The support of a layout of 16 x 16 or 32 x 32 blocks as the fused Scatterbrain kernels walk it: per (head,
+    64-query tile) the 32-key tiles that hold a block of any of the tile's block-rows, and per entry four masks, one per
+    group of 16 queries (16 w .. 16 w + 15 of the tile): bit 0 / bit 1 = that group sees keys 0..15 / 16..31 of the
+    entry's key tile.  Returns (ptr int32 (H * ceil(rows / 64) + 1), inner int32 (n) key tiles in increasing order per
+    query tile, mask int32 (n, 4)); rows and columns past the layout's end count as absent."""
+    if block not in (16, 32):
+        raise ValueError(f'block size {block}: the fused kernels walk supports of 16 x 16 or 32 x 32 blocks')
+    fine = _as_layout3(layout).cpu() > 0
+    rep = block // 16
+    if rep > 1:
+        fine = fine.repeat_interleave(rep, dim=1).repeat_interleave(rep, dim=2)
+    H, p16, r16 = fine.shape
+    G, C = (p16 + 3) // 4, (r16 + 1) // 2
+    padded = torch.zeros(H, 4 * G, 2 * C, dtype=torch.bool)
+    padded[:, :p16, :r16] = fine
+    halves = padded.view(H, G, 4, C, 2).long()
+    mask = (halves[..., 0] + 2 * halves[..., 1]).permute(0, 1, 3, 2)           # (H, G, C, 4)
+    nz = (mask > 0).any(dim=3).nonzero(as_tuple=False)                        # (h, g, c), sorted
+    counts = torch.bincount(nz[:, 0] * G + nz[:, 1], minlength=H * G)
+    ptr = torch.zeros(H * G + 1, dtype=torch.int64)
+    ptr[1:] = torch.cumsum(counts, 0)
+    return (ptr.to(torch.int32), nz[:, 2].to(torch.int32).contiguous(),
+            mask[nz[:, 0], nz[:, 1], nz[:, 2]].to(torch.int32).contiguous())
+
+
 def union_order(uni_ptr, n_heads):
     """Per head, its groups of union_table sorted by the length of their lists, longest first (ties in
     index order): int32 (n_heads * groups_per_head), entries are group indices within the head."""

@@ -100,9 +100,10 @@ struct FwdArgs {
     int B, H, T, S, mh_valid, lc, n_chunks, n_parts;
     long q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss;
     float temp;
-    // block-sparse support instead of a band (32 x 32 blocks; the fp32 kernel's LIST variant): per (head,
-    // 64-query tile) the key blocks its two block-rows touch -- tl_ptr (H * tiles + 1), tl_inner (block
-    // column per entry), tl_blk (2 per entry: block id of block-row 2 tile, 2 tile + 1, or -1 if absent)
+    // block-sparse support instead of a band (blocks of 16 x 16 or 32 x 32; the fp32 kernel's LIST variant): per (head,
+    // 64-query tile) the 32-key tiles its block-rows touch -- tl_ptr (H * tiles + 1), tl_inner (tile per entry),
+    // tl_blk (4 per entry: for queries 16 w .. 16 w + 15 of the tile bit 0 / bit 1 = keys 0..15 / 16..31 of the entry's
+    // tile are on the support)
     const int32_t* tl_ptr; const int32_t* tl_inner; const int32_t* tl_blk;
     // optional: per head the query tiles in the order they should start (longest list first); an entry
     // -1 - tile marks a tile that is left to the workgroups walking long lists in parts
@@ -2658,13 +2659,15 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
         kt_lo = first;
         kt_hi = first + base + (part < extra ? 1 : 0);
     }
-    // LIST: the loop counter walks the tile's list of key blocks instead of a range of key tiles (a key
-    // block is a key tile: both are 32 keys); the block column and this wave's presence flag of an entry
+    // LIST: the loop counter walks the tile's list of 32-key tiles instead of a range of them; the tile index and
+    // this wave's presence mask of an entry (bit h: the wave's 16 queries see keys 16 h .. 16 h + 15 of the tile --
+    // a block-row of 16 x 16 blocks is one wave, two waves share a block-row of 32 x 32 blocks and see whole tiles)
     // are read one iteration ahead of their use
     const int32_t* tl_inner = nullptr;
     const int32_t* tl_blk = nullptr;
     int tile_cur = 0, tile_next = 0;
-    bool pres_cur = false, pres_next = false, seen_block = false;
+    int pres_cur = 0, pres_next = 0;
+    bool seen_block = false;
     if (LIST) {
         int lp0 = a.tl_ptr[h * n_qt + qt];
         kt_lo = 0;
@@ -2676,9 +2679,9 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
             kt_hi = base + (part < extra ? 1 : 0);
         }
         tl_inner = a.tl_inner + lp0;
-        tl_blk = a.tl_blk + 2 * (long)lp0 + (w >> 1);       // waves 0, 1: block-row 2 qt; waves 2, 3: 2 qt + 1
-        if (kt_hi > 0) { tile_cur = tl_inner[0]; pres_cur = tl_blk[0] >= 0; }
-        if (kt_hi > 1) { tile_next = tl_inner[1]; pres_next = tl_blk[2] >= 0; }
+        tl_blk = a.tl_blk + 4 * (long)lp0 + w;              // four masks per entry, one per wave
+        if (kt_hi > 0) { tile_cur = tl_inner[0]; pres_cur = tl_blk[0] & 3; }
+        if (kt_hi > 1) { tile_next = tl_inner[1]; pres_next = tl_blk[4] & 3; }
     }
     const int first_tile = LIST ? tile_cur : kt_lo;
 
@@ -2803,8 +2806,8 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
         float cscale_next = cscale;
         // LIST: the entry after the next one (block column, presence) is requested now
         int tile_n2 = 0;
-        bool pres_n2 = false;
-        if (LIST && kt + 2 < kt_hi) { tile_n2 = tl_inner[kt + 2]; pres_n2 = tl_blk[2 * (kt + 2)] >= 0; }
+        int pres_n2 = 0;
+        if (LIST && kt + 2 < kt_hi) { tile_n2 = tl_inner[kt + 2]; pres_n2 = tl_blk[4 * (kt + 2)] & 3; }
         if (more) {                                      // next tile's loads fly during the MFMAs
             if (s_next + TK <= a.S) {
                 rk.fetch_fast(kptr + (long)s_next * a.k_ss, offk, tid);
@@ -2823,7 +2826,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
 
         // wave-uniform: does this tile touch the band of any of the wave's 16 queries?  (Blocks of a
         // touched tile that lie outside the band are computed and masked: no branches among the MFMAs.)
-        const bool any = LIST ? pres_cur
+        const bool any = LIST ? pres_cur != 0
                               : !(s_base + TK - 1 - qw0 < -lc_lo || s_base - (qw0 + 15) >= lc_hi || s_base >= len);
         if (any) {
             // scores^T: s1 = (t log2e) K q, s2 = K' q'.  The accumulation chains of the two key
@@ -2853,9 +2856,10 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
             // lane holds the scores of query iq against keys s_base + 16kb + 4g + i.  A tile that lies
             // inside the band of all 16 queries of the wave and below the key length (wave-uniform) needs
             // no masks.
-            // (LIST: a present block is wholly visible; the caller guarantees whole blocks of keys and queries)
-            const bool interior = LIST || (s_base - (qw0 + 15) >= -lc_lo && s_base + TK - 1 - qw0 < lc_hi &&
-                                           s_base + TK <= len && qw0 + 15 < a.T);
+            // (LIST: a present half tile is wholly visible; the caller guarantees whole blocks of keys and queries)
+            const bool interior = LIST ? pres_cur == 3
+                                       : (s_base - (qw0 + 15) >= -lc_lo && s_base + TK - 1 - qw0 < lc_hi &&
+                                          s_base + TK <= len && qw0 + 15 < a.T);
             floatx4 p[KB];
             float ovs = 0.f;
             auto soft = [&](auto masked_tag) __attribute__((always_inline)) {
@@ -2867,7 +2871,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         const int s = s_base + 16 * kb + 4 * g + i;
-                        ok[kb][i] = !MASKED || (unsigned)(s - smin) < span;
+                        ok[kb][i] = !MASKED || (LIST ? ((pres_cur >> kb) & 1) != 0 : (unsigned)(s - smin) < span);
                         mx = fmaxf(mx, ok[kb][i] ? s1[kb][i] : -INFINITY);
                     }
                 mx = group_max(mx);
@@ -2913,7 +2917,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
             rf.template stash<LDF>(nxt + TK * (LDK + LDV), tid);
         }
         cscale = cscale_next;
-        if (LIST) { seen_block |= pres_cur; tile_cur = tile_next; tile_next = tile_n2; pres_cur = pres_next; pres_next = pres_n2; }
+        if (LIST) { seen_block |= pres_cur != 0; tile_cur = tile_next; tile_next = tile_n2; pres_cur = pres_next; pres_next = pres_n2; }
         __syncthreads();
     }
     if (LIST && !part_role && !seen_block) {
@@ -4603,7 +4607,7 @@ extern "C" int flyhip_sbblocksparse_fwd(const void* q, const void* k, const void
     FLY_REQUIRE(q && k && v && proj && kfeat && chunk_scale && kv && ksum && kmax && tl_ptr && tl_inner && tl_blk &&
                 out && log_norm, "sbblocksparse_fwd: null pointer");
     FLY_REQUIRE(B > 0 && H > 0 && T > 0 && S > 0, "sbblocksparse_fwd: empty problem");
-    FLY_REQUIRE(T % 32 == 0 && S % 32 == 0, "sbblocksparse_fwd: sequence lengths %d, %d must be multiples of the block size 32", T, S);
+    FLY_REQUIRE(T % 16 == 0 && S % 16 == 0, "sbblocksparse_fwd: sequence lengths %d, %d must be multiples of 16", T, S);
     FLY_REQUIRE(softmax_temp > 0.f, "sbblocksparse_fwd: softmax_temp must be positive");
     FLY_REQUIRE(dtype == F32, "sbblocksparse_fwd: float32 inputs only (got dtype code %d)", dtype);
     int rc = check_sb_dims("sbblocksparse_fwd", E, D, mh, mh_valid, dtype, q_sb | q_sh | q_ss | k_sb | k_sh | k_ss,

@@ -15,21 +15,23 @@ from torch import distributed as dist
 from .blocksparse_attention import instantiate
 from .blocksparse_matmul import matmul
 from .blocksparse_softmax import blocksparse_sum, logsumexp
-from .blocksparse_utils import densify_tensor, sparsify_broadcast_tensor, union_heavy, union_order, union_table
+from .blocksparse_utils import (densify_tensor, sparsify_broadcast_tensor, tile_mask_table, union_heavy, union_order,
+                                union_table)
 from .sblocal_attention import ScratchCache, sbblocksparse_forward, sbblocksparse_forward_supported
 from .feature_maps_sb import SBPerformerFeatures
 from .padding import pad_to_multiple
 from .scatterbrain_utils import linear_attention, linear_attention_normalization
 
 
-def fused_tables(layout, device):
-    """Index tables of the fused forward for a (H, T/32, S/32) layout: the union lists of the query tiles
-    (two block-rows each), their start order (longest first), and the tiles whose lists are long enough to
-    be walked in parts -- (ptr, inner, blk, order, heavy, parts), tensors on `device`."""
-    ptr, inner, blk = union_table(layout, rows_per_group=2)
+def fused_tables(layout, device, block=32):
+    """Index tables of the fused forward for a (H, T/block, S/block) layout of 16 x 16 or 32 x 32 blocks: per
+    64-query tile the 32-key tiles on its support with the masks of its four groups of 16 queries
+    (blocksparse_utils.tile_mask_table), the tiles' start order (longest list first), and the tiles whose lists are long
+    enough to be walked in parts -- (ptr, inner, mask, order, heavy, parts), tensors on `device`."""
+    ptr, inner, mask = tile_mask_table(layout, block)
     H = layout.shape[0]
     order = union_order(ptr, H)
-    heavy, parts = union_heavy(ptr, blk)
+    heavy, parts = union_heavy(ptr, mask - 1)        # (mask 0 = absent, as a block id of -1)
     if heavy.numel():
         groups = order.numel() // H
         marked = order.reshape(H, groups).clone()
@@ -38,7 +40,7 @@ def fused_tables(layout, device):
         flat = torch.arange(H).unsqueeze(1) * groups + marked.long()
         marked[is_heavy[flat]] = -1 - marked[is_heavy[flat]]
         order = marked.reshape(-1).contiguous()
-    return tuple(x.to(device) for x in (ptr, inner, blk, order, heavy)) + (parts,)
+    return tuple(x.to(device) for x in (ptr, inner, mask, order, heavy)) + (parts,)
 
 
 def backward_tables(layout, device, transposed=False, n_heavy_min=32, entries_per_part=12, max_parts=16):
@@ -157,8 +159,9 @@ class SBBlockSparseAttention(nn.Module):
         S = value.shape[1]
         softmax_temp = self.softmax_temp or 1 / math.sqrt(E)       # :131
 
-        # 32 x 32 blocks, float32, nothing but the output wanted: the whole forward on the fused kernels of
-        # Scatterbrain-local attention, walking the layout's blocks instead of a band
+        # blocks of 16 x 16 or 32 x 32, nothing but the output wanted: the whole forward on the fused kernels of
+        # Scatterbrain-local attention, walking the layout's blocks instead of a band (with gradients: 32 x 32 blocks,
+        # whose backward kernels exist)
         self.feature_map.new_feature_map(query.device)
         layout = self.get_layout(T, S)
         needs_grad = torch.is_grad_enabled() and any(x.requires_grad for x in (query, key, value))
@@ -169,10 +172,10 @@ class SBBlockSparseAttention(nn.Module):
                 and query.dtype in (torch.float32, torch.bfloat16, torch.float16)
                 and sbblocksparse_forward_supported(block, torch.float32, E, value.shape[3], n_rows, layout.shape[0], H)
                 # with gradients: the backward kernels' head dims and feature counts
-                and (not needs_grad or _band_kernel_dims(E, value.shape[3], 2 * n_rows) is not None)):
+                and (not needs_grad or (block == 32 and _band_kernel_dims(E, value.shape[3], 2 * n_rows) is not None))):
             key_ = (T, S, query.device)
             if key_ not in self.fused_tables:
-                self.fused_tables[key_] = fused_tables(layout, query.device)
+                self.fused_tables[key_] = fused_tables(layout, query.device, block)
             # (2-byte inputs are widened, as on the op-by-op path below)
             if not needs_grad:
                 out, _ = sbblocksparse_forward(query.float(), key.float(), value.float(),

@@ -154,8 +154,8 @@ class SBLocalPlan:
 
     def run_block_sparse(self, q, k, v, proj, t, tables, out, log_norm):
         """Scatterbrain attention whose exact part lives on a block-sparse support instead of a band: the
-        key pass as in ``run``, then the fp32 band kernel walking lists of 32-key blocks (``tables`` =
-        union_table(layout, rows_per_group=2) on the device).  One part per query tile, no key lengths."""
+        key pass as in ``run``, then the fp32 band kernel walking lists of 32-key tiles (``tables`` =
+        blocksparse_utils.tile_mask_table(layout, block) on the device).  One part per query tile, no key lengths."""
         B, H, T, S, dim, mh, mh_valid = self.shape
         self._make_buffers()
         tl_ptr, tl_inner, tl_blk = tables[:3]
@@ -335,25 +335,25 @@ def sblocal_forward(query, key, value, projection_matrix, local_context, softmax
 
 
 def sbblocksparse_forward_supported(block, dtype, E, D, n_projection_rows, layout_heads, H):
-    """Whether sbblocksparse_forward applies: 32 x 32 blocks, float32, one layout per attention head."""
-    return (block == 32 and dtype == torch.float32 and max(E, D) <= _HEAD_DIMS[-1]
+    """Whether sbblocksparse_forward applies: blocks of 16 x 16 or 32 x 32, float32, one layout per attention head."""
+    return (block in (16, 32) and dtype == torch.float32 and max(E, D) <= _HEAD_DIMS[-1]
             and n_projection_rows <= _FEATURE_ROWS[-1] and layout_heads == H)
 
 
 def sbblocksparse_forward(query, key, value, projection_matrix, tables, softmax_temp=None, cache=None):
     """Scatterbrain attention on a block-sparse support (sbblocksparse_attention.py:109-213 for
-    need_weights=False, no dropout) on the fused kernels: exact softmax weights on the nonzero 32 x 32
-    blocks, the Performer estimate everywhere else, one normaliser.  query (B,T,H,E), key (B,S,H,E), value
-    (B,S,H,D) float32 GPU tensors, T and S multiples of 32; tables = union_table(layout, rows_per_group=2)
-    as int32 tensors on the device, optionally followed by union_order(tables[0], H), or the six entries of
+    need_weights=False, no dropout) on the fused kernels: exact softmax weights on the nonzero blocks (16 x 16 or
+    32 x 32), the Performer estimate everywhere else, one normaliser.  query (B,T,H,E), key (B,S,H,E), value
+    (B,S,H,D) float32 GPU tensors, T and S multiples of the block size; tables = blocksparse_utils.tile_mask_table(layout,
+    block) as int32 tensors on the device, optionally followed by union_order(tables[0], H), or the six entries of
     sbblocksparse_attention.fused_tables (start order with the long lists marked, those lists, their parts).
     cache: an optional ScratchCache kept by the caller (plan and padded projection, as for sblocal_forward).
     Returns (out (B,T,H,D), log_normalization (B,H,T,1))."""
     _lib.require_gpu(query, key, value, projection_matrix)
     B, T, H, E = query.shape
     S, D = key.shape[1], value.shape[3]
-    if T % 32 or S % 32:
-        raise ValueError(f'sequence lengths {T}, {S} must be multiples of the block size 32')
+    if T % 16 or S % 16:
+        raise ValueError(f'sequence lengths {T}, {S} must be multiples of the block size (16 or 32)')
     t = softmax_temp or 1 / math.sqrt(E)
     dim = _round_up_choice(max(E, D), _HEAD_DIMS, 'head dimension')
     mh_valid = projection_matrix.shape[0]

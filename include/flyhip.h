@@ -262,21 +262,23 @@ int flyhip_sbblocksparse_bwd_pieces(const void* outer_images, const void* inner_
 
 /* Scatterbrain attention on a block-sparse support (ref: src/models/attention/sbblocksparse_attention.py:109-213
  * for need_weights = False, no dropout, no masks): as flyhip_sblocal_fwd with one part per query tile, but the
- * exact part covers the nonzero 32 x 32 blocks of a layout instead of a band.  Key-side inputs (kfeat,
- * chunk_scale, kv, ksum, kmax) from flyhip_sb_kv_reduce.  tl_ptr (H * ceil(T/64) + 1), tl_inner, tl_blk (2 per
- * entry): per (head, 64-query tile) the union of the block columns of its two block-rows, and per entry the block
- * id of each of the two rows or -1 where the row lacks that column.  tl_order (H * ceil(T/64), may be NULL): per
+ * exact part covers the nonzero blocks of a layout (16 x 16 or 32 x 32) instead of a band.  Key-side inputs (kfeat,
+ * chunk_scale, kv, ksum, kmax) from flyhip_sb_kv_reduce.  tl_ptr (H * ceil(T/64) + 1), tl_inner, tl_mask (4 per
+ * entry): per (head, 64-query tile) the 32-key tiles that any of its queries sees on the support, and per entry and
+ * group of 16 queries (16 w .. 16 w + 15 of the tile) a mask: bit 0 = keys 0..15, bit 1 = keys 16..31 of that tile
+ * are on the support for those queries (32 x 32 blocks: 0 or 3, the same for w = 0, 1 and for w = 2, 3).
+ * tl_order (H * ceil(T/64), may be NULL): per
  * head a permutation of its query tiles, the order in which they are started -- longest list first keeps a
  * block-row of global tokens from becoming the tail of the launch.
  * Long lists (n_heavy > 0): tl_heavy (n_heavy entries head * ceil(T/64) + tile) names query tiles whose lists are
  * walked in heavy_parts parts (2..64) by the first workgroups of the launch and finished by a merge launch; those
  * tiles carry the entry -1 - tile in tl_order so that no workgroup takes them whole, and every block-row of such
  * a tile must have at least one block.  Scratch for them: part_ws of B*n_heavy*heavy_parts*64*(D+5) floats and qfeat of
- * B*n_heavy*64*m floats (both NULL when n_heavy == 0).  float32 only; T, S multiples of 32. */
+ * B*n_heavy*64*m floats (both NULL when n_heavy == 0).  float32 only; T, S multiples of 16. */
 int flyhip_sbblocksparse_fwd(const void* q, const void* k, const void* v, const float* proj,
                              const void* kfeat, const float* chunk_scale,
                              const float* kv, const float* ksum, const float* kmax,
-                             const int32_t* tl_ptr, const int32_t* tl_inner, const int32_t* tl_blk,
+                             const int32_t* tl_ptr, const int32_t* tl_inner, const int32_t* tl_mask,
                              const int32_t* tl_order, const int32_t* tl_heavy, int n_heavy, int heavy_parts,
                              float* part_ws, float* qfeat,
                              void* out, float* log_norm,

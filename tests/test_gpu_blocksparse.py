@@ -287,10 +287,10 @@ def test_sbblocksparse_attention_module(dtype, block):
     assert float((rows.float().cpu() - 1).abs().max()) <= (1e-4 if dtype == torch.float32 else 3e-2)
     ref_from_attn = torch.einsum('bhts,bshd->bthd', attn.double().cpu(), v.double())
     assert rel_err(ref_from_attn, ref_out) <= tol
-    # without the weights: 32 x 32 blocks take the fused kernels (the band kernel of Scatterbrain-local attention
-    # walking the layout's blocks), other block sizes the same ops as above
+    # without the weights: the fused kernels (the band kernel of Scatterbrain-local attention walking the layout's
+    # blocks, 16 x 16 or 32 x 32)
     out2, none = layer(q.to(DEV), k.to(DEV), v.to(DEV))
-    assert none is None and (len(layer.fused_tables) == 1) == (block == 32)
+    assert none is None and len(layer.fused_tables) == 1
     assert rel_err(out2, ref_out) <= tol
     layer.fuse = False
     out3, _ = layer(q.to(DEV), k.to(DEV), v.to(DEV))
@@ -731,7 +731,7 @@ def test_sbblocksparse_fused_forward(B, H, T, S, E, D, m, seed):
     """Scatterbrain attention on a block-sparse support on the fused kernels (flyhip_sbblocksparse_fwd): random
     layouts per head with an empty block-row, an odd number of block-rows (a query tile with one block-row),
     T != S, head dims and feature counts that need padding; output and log-normaliser against the oracle."""
-    from fly_amd.blocksparse_utils import union_table
+    from fly_amd.blocksparse_utils import tile_mask_table, union_table
     from fly_amd.sblocal_attention import sbblocksparse_forward
     from oracle import sbblocksparse as osbb
     from oracle import sblocal as osb
@@ -744,7 +744,7 @@ def test_sbblocksparse_fused_forward(B, H, T, S, E, D, m, seed):
     k = torch.randn(B, S, H, E, generator=g) * E ** -0.25
     v = torch.randn(B, S, H, D, generator=g)
     P = osb.gaussian_orthogonal_random_matrix(m // 2, E, generator=g)
-    tables = tuple(x.to(DEV) for x in union_table(layout, rows_per_group=2))
+    tables = tuple(x.to(DEV) for x in tile_mask_table(layout, 32))
     out, ln = sbblocksparse_forward(q.to(DEV), k.to(DEV), v.to(DEV), P.to(DEV), tables)
     ref_out, ref_ln = osbb.sbblocksparse_attention(q.double(), k.double(), v.double(), P.double(), layout, 32)
     assert out.shape == (B, T, H, D) and ln.shape == (B, H, T, 1)
@@ -757,9 +757,39 @@ def test_sbblocksparse_fused_forward(B, H, T, S, E, D, m, seed):
     assert torch.equal(out2, out) and torch.equal(ln2, ln)
 
 
+@pytest.mark.parametrize('B,H,T,S,E,D,m,seed', [(2, 2, 208, 144, 64, 64, 64, 11), (1, 3, 784, 784, 64, 64, 16, 12),
+                                                (2, 1, 48, 400, 32, 48, 32, 13)])
+def test_sbblocksparse_fused_forward_on_16x16_blocks(B, H, T, S, E, D, m, seed):
+    """The fused forward on a support of 16 x 16 blocks (the block size of the reference's second T2T layer,
+    configs/model/t2tattn_cfg/sbbs-*.yaml): a wave of the band kernel is one block-row, a 32-key tile two
+    block-columns, each present or not.  Sequence lengths that are no multiples of 32 or 64, block-rows without
+    blocks, a column of global keys; output and log-normaliser against the oracle."""
+    from fly_amd.blocksparse_utils import tile_mask_table
+    from fly_amd.sblocal_attention import sbblocksparse_forward
+    from oracle import sbblocksparse as osbb
+    from oracle import sblocal as osb
+    print('case', B, H, T, S, E, D, m, seed, flush=True)
+    g = torch.Generator().manual_seed(seed)
+    layout = (torch.rand(H, T // 16, S // 16, generator=g) < 0.3).long()
+    layout[:, :, 0] = 1
+    layout[0, 1, :] = 0                                        # a block-row without blocks
+    if T // 16 > 5:
+        layout[-1, 5, :] = 0
+    q = torch.randn(B, T, H, E, generator=g) * E ** -0.25
+    k = torch.randn(B, S, H, E, generator=g) * E ** -0.25
+    v = torch.randn(B, S, H, D, generator=g)
+    P = osb.gaussian_orthogonal_random_matrix(m // 2, E, generator=g)
+    tables = tuple(x.to(DEV) for x in tile_mask_table(layout, 16))
+    out, ln = sbblocksparse_forward(q.to(DEV), k.to(DEV), v.to(DEV), P.to(DEV), tables)
+    ref_out, ref_ln = osbb.sbblocksparse_attention(q.double(), k.double(), v.double(), P.double(), layout, 16)
+    assert out.shape == (B, T, H, D) and ln.shape == (B, H, T, 1)
+    assert rel_err(out, ref_out) <= 1e-4, rel_err(out, ref_out)
+    assert rel_err(ln.reshape(ref_ln.shape), ref_ln) <= 1e-4, rel_err(ln.reshape(ref_ln.shape), ref_ln)
+
+
 def test_sbblocksparse_fused_forward_with_an_empty_layout():
     """A support without any block: what remains is the low-rank estimate alone (linear attention on the features)."""
-    from fly_amd.blocksparse_utils import union_table
+    from fly_amd.blocksparse_utils import tile_mask_table, union_table
     from fly_amd.sblocal_attention import sbblocksparse_forward
     from oracle import sbblocksparse as osbb
     from oracle import sblocal as osb
@@ -770,7 +800,7 @@ def test_sbblocksparse_fused_forward_with_an_empty_layout():
     k = torch.randn(B, S, H, E, generator=g) * E ** -0.25
     v = torch.randn(B, S, H, D, generator=g)
     P = osb.gaussian_orthogonal_random_matrix(m // 2, E, generator=g)
-    tables = tuple(x.to(DEV) for x in union_table(layout, rows_per_group=2))
+    tables = tuple(x.to(DEV) for x in tile_mask_table(layout, 32))
     out, ln = sbblocksparse_forward(q.to(DEV), k.to(DEV), v.to(DEV), P.to(DEV), tables)
     ref_out, ref_ln = osbb.sbblocksparse_attention(q.double(), k.double(), v.double(), P.double(), layout, 32)
     assert rel_err(out, ref_out) <= 1e-4, rel_err(out, ref_out)
@@ -785,7 +815,7 @@ def test_sbblocksparse_gradients_on_the_kernels(B, H, T, S, E, D, m, seed):
     (sbblocksparse_attention.py:161-212): random layouts per head with an empty block-row, an odd number of
     block-rows and block-columns, T != S, head dims and feature counts that need padding."""
     from fly_amd import sblocal_backward
-    from fly_amd.blocksparse_utils import union_table
+    from fly_amd.blocksparse_utils import tile_mask_table, union_table
     from fly_amd.sblocal_attention import sbblocksparse_forward
     from oracle import sbblocksparse as osbb
     from oracle import sblocal as osb
@@ -805,7 +835,7 @@ def test_sbblocksparse_gradients_on_the_kernels(B, H, T, S, E, D, m, seed):
     fwd = tuple(x.to(DEV) for x in union_table(layout, rows_per_group=2))
     bwd = tuple(x.to(DEV) for x in union_table(layout, rows_per_group=2, transposed=True))
     qg, kg, vg = q.to(DEV), k.to(DEV), v.to(DEV)
-    out, ln = sbblocksparse_forward(qg, kg, vg, P.to(DEV), fwd)
+    out, ln = sbblocksparse_forward(qg, kg, vg, P.to(DEV), tuple(x.to(DEV) for x in tile_mask_table(layout, 32)))
     dq, dk, dv = sblocal_backward(qg, kg, vg, P.to(DEV), 1, None, None, out, ln, w.to(DEV), support=(fwd, bwd))
     for got, ref in ((dq, qd.grad), (dk, kd.grad), (dv, vd.grad)):
         assert got.shape == ref.shape and rel_err(got, ref) <= 2e-4, rel_err(got, ref)
@@ -849,7 +879,7 @@ def test_sbblocksparse_gradients_with_long_lists_in_parts():
     launch (sbblocksparse_attention.backward_tables); gradients against autograd through the oracle and against the
     walk of whole lists."""
     from fly_amd import sblocal_backward
-    from fly_amd.blocksparse_utils import union_table
+    from fly_amd.blocksparse_utils import tile_mask_table, union_table
     from fly_amd.sbblocksparse_attention import backward_tables
     from fly_amd.sblocal_attention import sbblocksparse_forward
     from oracle import sbblocksparse as osbb
@@ -876,7 +906,7 @@ def test_sbblocksparse_gradients_with_long_lists_in_parts():
     ref_out, _ = osbb.sbblocksparse_attention(qd, kd, vd, P.double(), layout, 32)
     (ref_out * w.double()).sum().backward()
     qg, kg, vg = q.to(DEV), k.to(DEV), v.to(DEV)
-    out, ln = sbblocksparse_forward(qg, kg, vg, P.to(DEV), tq[:3])
+    out, ln = sbblocksparse_forward(qg, kg, vg, P.to(DEV), tuple(x.to(DEV) for x in tile_mask_table(layout, 32)))
     got = sblocal_backward(qg, kg, vg, P.to(DEV), 1, None, None, out, ln, w.to(DEV), support=(tq, tk))
     for x, ref in zip(got, (qd.grad, kd.grad, vd.grad)):
         assert rel_err(x, ref) <= 2e-4, rel_err(x, ref)
@@ -888,7 +918,7 @@ def test_sbblocksparse_gradients_with_long_lists_in_parts():
 def test_sbblocksparse_long_lists_in_parts():
     """Block-rows of global tokens: their query tiles' lists are walked in parts by a second launch and merged
     (fused_tables marks them); output and log-normaliser against the oracle and against the one-part path."""
-    from fly_amd.blocksparse_utils import union_table
+    from fly_amd.blocksparse_utils import tile_mask_table, union_table
     from fly_amd.sbblocksparse_attention import fused_tables
     from fly_amd.sblocal_attention import sbblocksparse_forward
     from oracle import sbblocksparse as osbb
@@ -915,6 +945,6 @@ def test_sbblocksparse_long_lists_in_parts():
     ref_out, ref_ln = osbb.sbblocksparse_attention(q.double(), k.double(), v.double(), P.double(), layout, 32)
     assert rel_err(out, ref_out) <= 1e-4, rel_err(out, ref_out)
     assert rel_err(ln.reshape(ref_ln.shape), ref_ln) <= 1e-4, rel_err(ln.reshape(ref_ln.shape), ref_ln)
-    plain = tuple(x.to(DEV) for x in union_table(layout, rows_per_group=2))
+    plain = tuple(x.to(DEV) for x in tile_mask_table(layout, 32))
     out1, ln1 = sbblocksparse_forward(q.to(DEV), k.to(DEV), v.to(DEV), P.to(DEV), plain)
     assert rel_err(out, out1) <= 1e-5 and rel_err(ln, ln1) <= 1e-5

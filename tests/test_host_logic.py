@@ -330,3 +330,42 @@ def test_scratch_cache_is_bounded_and_tracks_the_projection_object():
     mod = fly_amd.SBLocalAttention(8, dim_heads=16, nb_features=8)
     mod._scratch_cache.plan('x', maker('x'))
     assert len(copy.deepcopy(mod)._scratch_cache) == 0
+
+
+@pytest.mark.parametrize('block', [16, 32])
+def test_tile_mask_table_against_loops(block):
+    """The support table of the fused Scatterbrain kernels (per 64-query tile its 32-key tiles, per entry and group of
+    16 queries which halves of the tile are on the support) against explicit loops over the layout."""
+    from fly_amd.blocksparse_utils import tile_mask_table
+    g = torch.Generator().manual_seed(block)
+    H, p, r = 3, 11 if block == 16 else 5, 9 if block == 16 else 7
+    layout = (torch.rand(H, p, r, generator=g) < 0.35).long()
+    layout[1, 2, :] = 0
+    ptr, inner, mask = tile_mask_table(layout, block)
+    rows, cols = p * block, r * block
+    n_qt, n_kt = (rows + 63) // 64, (cols + 31) // 32
+    assert ptr.shape == (H * n_qt + 1,) and ptr.dtype == inner.dtype == mask.dtype == torch.int32
+    want = []
+    for h in range(H):
+        for qt in range(n_qt):
+            for kt in range(n_kt):
+                m4 = []
+                for w in range(4):
+                    bits = 0
+                    for half in range(2):
+                        i, j = 64 * qt + 16 * w, 32 * kt + 16 * half
+                        if i < rows and j < cols and layout[h, i // block, j // block]:
+                            bits |= 1 << half
+                    m4.append(bits)
+                if any(m4):
+                    want.append((h * n_qt + qt, kt, m4))
+    assert int(ptr[-1]) == len(want) == inner.numel() and mask.shape == (len(want), 4)
+    at = 0
+    for grp in range(H * n_qt):
+        mine = [e for e in want if e[0] == grp]
+        assert int(ptr[grp + 1]) - int(ptr[grp]) == len(mine)
+        for e in mine:
+            assert int(inner[at]) == e[1] and mask[at].tolist() == e[2]
+            at += 1
+    with pytest.raises(ValueError):
+        tile_mask_table(layout, 64)
