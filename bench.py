@@ -359,7 +359,8 @@ def bench_other_configs():
     # Scatterbrain on a block-sparse support at the first T2T layer's size (the sbbs-* attention configs:
     # block 32, three sliding-window blocks, 32 features; here with one global block row / column)
     class WindowPlusGlobal:
-        block = 32
+        def __init__(self, block):
+            self.block = block
 
         def make_layout(self, seqlen):
             nb = seqlen // self.block
@@ -369,7 +370,7 @@ def bench_other_configs():
             lay[0, :] = 1
             return lay.unsqueeze(0)
     B, L, E = 64, 3136, 64
-    sbbs = fly_amd.SBBlockSparseAttention(WindowPlusGlobal(), dim_heads=E, nb_features=32, max_seq_length=L).to(dev)
+    sbbs = fly_amd.SBBlockSparseAttention(WindowPlusGlobal(32), dim_heads=E, nb_features=32, max_seq_length=L).to(dev)
     q, k, v = (torch.randn(B, L, 1, E, generator=g).to(dev) * E ** -0.25 for _ in range(3))
     with torch.no_grad():
         out['sbblocksparse_fp32_B64_L3136_block32_m32'] = {'ms': timeit(lambda: sbbs(q, k, v), n=5)}
@@ -385,6 +386,17 @@ def bench_other_configs():
     sbbs.fuse = False
     out['sbblocksparse_fp32_B64_L3136_block32_m32']['fwd_bwd_op_by_op_ms'] = timeit(sbbs_step, n=3)
     del q, k, v, sbbs, qg, kg, vg, go
+    # the second T2T layer's size with the reference's settings for it (sbbs-*.yaml: block 16, 16 features): forward
+    # on the fused kernels (a wave per block-row, half-tile masks) and op by op
+    L = 784
+    sbbs = fly_amd.SBBlockSparseAttention(WindowPlusGlobal(16), dim_heads=E, nb_features=16, max_seq_length=L).to(dev)
+    q, k, v = (torch.randn(B, L, 1, E, generator=g).to(dev) * E ** -0.25 for _ in range(3))
+    with torch.no_grad():
+        ms_f = timeit(lambda: sbbs(q, k, v), n=5)
+        sbbs.fuse = False
+        ms_o = timeit(lambda: sbbs(q, k, v), n=3)
+    out['sbblocksparse_fp32_B64_L784_block16_m16'] = {'ms': ms_f, 'op_by_op_ms': ms_o}
+    del q, k, v, sbbs
 
     cfg = fly_amd.FlatBlockButterflySparsityConfig(8, 2, block=32)
     torch.manual_seed(0)
