@@ -963,10 +963,20 @@ struct DdsGroupArgs {
     int per_head, M;
     long sp_sz, dn_sz, dn_sh, dn_sm, c_sz, c_sh, c_sm;
     int n_xcd;          // dies the dispatcher deals workgroup ids to (set where the kernel is launched)
+    int n_grp;          // groups (the weight-stationary kernel deals (token stream, group) pairs itself)
 };
 constexpr int DDS_MAX_STEPS = 128;   // longest reduction list the tiled kernel accepts
+#ifndef FLY_DDS_STATIONARY
+#define FLY_DDS_STATIONARY 1         // weight-stationary kernel where the group's weights fit the LDS
+#endif
+#ifndef FLY_DDS_DEPTH
+#define FLY_DDS_DEPTH 2              // steps (of two input blocks) its activation loads run ahead
+#endif
+#ifndef FLY_DDS_DIST
+#define FLY_DDS_DIST 2               // steps the loads of the 128-token kernel run ahead of its MFMAs
+#endif
 
-template <typename T, bool WT>     // WT: blocks are [k][n] (y = x W) and are transposed on their way into LDS
+template <typename T, bool WT, int DIST = FLY_DDS_DIST>     // WT: blocks are [k][n] (y = x W) and are transposed on their way into LDS
 __global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
     constexpr int KB = 1;                                   // input blocks per pipeline step
     // LDS tiles are [row][32 k] with 64-byte rows and no padding; the four 16-byte chunks of a row are
@@ -1018,8 +1028,8 @@ __global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
     // Every fetch issues the same number of loads on every path (a step past the end re-reads the last
     // one, an absent weight block reads block 0 and is zeroed when it is parked): only then can the
     // compiler count how many newer loads may stay in flight when it waits for the older set.
-    uintx4 rxa[KB][2], rwa[KB][2], rxb[KB][2], rwb[KB][2];
-    bool wla[KB][2], wlb[KB][2];                            // weight block present?
+    uintx4 rx[DIST][KB][2], rw[DIST][KB][2];                // set j holds the steps congruent to j modulo DIST
+    bool wl[DIST][KB][2];                                   // weight block present?
     int f_tile = 0, f_t = 0;                                // fetch cursor: (token tile, step inside it)
     // A load is "wave-uniform base + per-thread byte offset": the input block and the weight block of a
     // step are the same for the whole wave (a wave stages rows of one output block: (tid / 4) / 32 = w / 2),
@@ -1127,24 +1137,170 @@ __global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
             for (int tile = 0; tile < my_tiles; ++tile) store_tile(tile);
         return;
     }
-    fetch(rxa, rwa, wla);
-    stash(0, rxa, rwa, wla);
-    fetch(rxb, rwb, wlb);                                   // set B holds odd steps, set A even steps
-    drain_loads_but<4 * KB>();                              // only set B (4 KB loads a thread) is in flight
+    // Loads run DIST steps ahead of the MFMAs in DIST register sets: a step's tiles are asked for, parked in LDS
+    // DIST - 1 iterations later (one iteration before they are used), and every global load has that long to arrive.
+    // The loop is unrolled over the least common multiple of the two LDS stages and the DIST sets, so that every
+    // register set and stage index is a constant.
+#pragma unroll
+    for (int j = 0; j < DIST; ++j) fetch(rx[j], rw[j], wl[j]);
+    drain_loads_but<4 * KB * (DIST - 1)>();                  // set 0 has arrived
+    stash(0, rx[0], rw[0], wl[0]);
     __syncthreads();
-    for (int step = 0; step < n_steps; step += 2) {
-        fetch(rxa, rwa, wla);
-        compute(0);
-        stash(1, rxb, rwb, wlb);
-        drain_loads_but<4 * KB>();                          // set B is parked: only set A is in flight
-        __syncthreads();
-        // (no early exit between the halves: the compiler would count a path that leaves here, with
-        // set A in flight, as a way back to the top of the loop, and drain before every refill)
-        fetch(rxb, rwb, wlb);
-        if (step + 1 < n_steps) compute(1);
-        stash(0, rxa, rwa, wla);
-        drain_loads_but<4 * KB>();
-        __syncthreads();
+    constexpr int U = (DIST % 2 == 0) ? DIST : 2 * DIST;
+    for (int step = 0; step < n_steps; step += U) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            // (no early exit inside: every path through the body issues the same loads, so the compiler can count how
+            //  many newer ones may stay in flight when it waits for a set)
+            fetch(rx[u % DIST], rw[u % DIST], wl[u % DIST]);                    // step + u + DIST; its set was parked an iteration ago
+            if (step + u < n_steps) compute(u & 1);
+            stash((u + 1) & 1, rx[(u + 1) % DIST], rw[(u + 1) % DIST], wl[(u + 1) % DIST]);
+            drain_loads_but<4 * KB * (DIST - 1)>();         // the set parked next iteration has arrived
+            __syncthreads();
+        }
+    }
+}
+
+// Weight-stationary DDS for groups whose weights fit the LDS (reduction lists of up to 9 input blocks: layers that
+// widen, such as the first linear of a channel MLP).  The group's weight tiles -- the same for every token tile -- are
+// brought into LDS once; after that a wave needs nothing from its neighbours: it owns 64 tokens against all outputs of
+// the group, takes its activation fragments STRAIGHT from global memory in MFMA operand order (lane (r, g): token r,
+// inputs 8 g .. 8 g + 7 of the step's block, 16 contiguous bytes), DEPTH steps ahead in DEPTH register sets, and reads
+// the step's weight fragments from LDS.  No barrier in the loop, no activation staging, no weight traffic per token
+// tile; every weight fragment read feeds four MFMAs.  Tokens are the rows of the products and the weight tiles are
+// dealt so that tile n holds outputs 8 r + n (r = 0..15): a lane then ends up with eight CONSECUTIVE outputs of four
+// tokens, and one store instruction writes four whole 256-byte rows of the result (with 64-byte pieces per row the
+// stores of the 308 MB result were 40 % of the kernel's time).  Two workgroups of four waves per compute unit; the
+// (token stream, group) pairs are dealt to the XCDs in contiguous runs, so that the groups reading one stream's
+// activations share an L2.
+constexpr int DDS_STAT_STEPS = 9;         // longest reduction list: 8 KB of weight tiles per step, 72 KB, two workgroups per CU
+
+template <typename T, bool WT, int DEPTH>
+__global__ __launch_bounds__(256) void bs_dds32s_kernel(DdsGroupArgs a, int n_streams) {
+    constexpr int STEP = 8 * 16 * 32;                       // elements of a step's eight weight tiles
+    extern __shared__ __attribute__((aligned(16))) uint16_t wres[];     // [step][tile n][row r][32 k]: output 8 r + n of the group
+    __shared__ int s_inner[DDS_STAT_STEPS];
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
+    const int z = blockIdx.y;
+    // pair index: the dispatcher deals workgroup ids to the XCDs in turn; XCD x takes the pairs x * per_xcd ...
+    const int per_xcd = (int)gridDim.x / a.n_xcd;
+    const int pair = ((int)blockIdx.x % a.n_xcd) * per_xcd + (int)blockIdx.x / a.n_xcd;
+    const int n_grp = a.n_grp;
+    if (pair >= n_streams * n_grp) return;                  // workgroup-uniform
+    const int ty = pair / n_grp, grp = pair % n_grp, gy = n_streams;
+    const int tiles_all = (a.M + 255) / 256;
+    if (ty >= tiles_all) return;
+    const int my_tiles = (tiles_all - ty + gy - 1) / gy;
+    const int row0 = a.grp_row0[grp], gn = a.grp_n[grp];
+    const int head = row0 / a.per_head, bcol0 = row0 % a.per_head;
+    const int p0 = a.seg_ptr[row0], nin = a.seg_ptr[row0 + 1] - p0;
+    const uint16_t* spz = reinterpret_cast<const uint16_t*>(a.sp) + z * a.sp_sz;
+    const uint16_t* xp = reinterpret_cast<const uint16_t*>(a.dn) + z * a.dn_sz + head * a.dn_sh;
+    T* cp = reinterpret_cast<T*>(a.c) + z * a.c_sz + head * a.c_sh;
+
+    for (int i = tid; i < nin; i += 256) s_inner[i] = a.seg_inner[p0 + i];
+    // the group's weights, once (output blocks the group lacks: zeros)
+    for (int idx = tid; idx < nin * 512; idx += 256) {
+        const int chunk = idx & 3, row = (idx >> 2) & 31, ob = (idx >> 7) & 3, t = idx >> 9;
+        const int blk_id = ob < gn ? a.seg_blk[a.seg_ptr[row0 + ob] + t] : -1;
+        uintx4 v = {0, 0, 0, 0};
+        if (blk_id >= 0) v = *reinterpret_cast<const uintx4*>(spz + (long)blk_id * 1024 + row * 32 + chunk * 8);
+        uint16_t* dst = wres + (size_t)t * STEP;
+        if (!WT) {
+            // block row `row` is output 32 ob + row: tile row % 8, row 4 ob + row / 8; the thread's 8 inputs stay together
+            *reinterpret_cast<uintx4*>(dst + (row & 7) * 512 + (4 * ob + (row >> 3)) * 32 + 8 * chunk) = v;
+        } else {
+            // the block is [input][output]: the thread holds input `row`, outputs 32 ob + 8 chunk + e -> tile e, row 4 ob + chunk
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                dst[e * 512 + (4 * ob + chunk) * 32 + row] = (uint16_t)(v[e >> 1] >> (16 * (e & 1)));
+        }
+    }
+    __syncthreads();
+
+    floatx4 acc[4][8];
+#pragma unroll
+    for (int tm = 0; tm < 4; ++tm)
+#pragma unroll
+        for (int n = 0; n < 8; ++n) acc[tm][n] = Frag<float>::zero();
+    const bool col_live = 8 * r16 < 32 * gn;                // this lane's eight outputs exist in the group
+    // lane holds y[m = 64 w + 16 tm + 4 g + i][n0 + 8 r16 .. + 7]: one 16-byte store per (tm, i), 256 bytes per row and
+    // instruction
+    auto store_tile = [&](int tile) __attribute__((always_inline)) {
+        const long m0 = ((long)ty + (long)tile * gy) * 256 + 64 * w + 4 * g;
+        T* base = cp + (long)bcol0 * 32 + 8 * r16;
+#pragma unroll
+        for (int tm = 0; tm < 4; ++tm) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const long m = m0 + 16 * tm + i;
+                if (m < a.M && col_live) {
+                    const floatx4 lo = {acc[tm][0][i], acc[tm][1][i], acc[tm][2][i], acc[tm][3][i]};
+                    const floatx4 hi = {acc[tm][4][i], acc[tm][5][i], acc[tm][6][i], acc[tm][7][i]};
+                    store8_f32(base + m * a.c_sm, lo, hi);
+                }
+            }
+#pragma unroll
+            for (int n = 0; n < 8; ++n) acc[tm][n] = Frag<float>::zero();
+        }
+    };
+    if (nin == 0) {                                         // no input block: zero rows
+        for (int tile = 0; tile < my_tiles; ++tile) store_tile(tile);
+        return;
+    }
+
+    // a step takes two entries of the reduction list: neighbouring input blocks share their 128-byte lines, and asked for
+    // together the second block's loads find them on their way (a step apart they had left the L1 again)
+    const int npair = (nin + 1) / 2;
+    const int n_steps = my_tiles * npair;
+    uintx4 fx[DEPTH][2][4];
+    int f_tile = 0, f_t = 0;                                // fetch cursor: (token tile, pair of entries inside it)
+    uint32_t xoff[4] = {0, 0, 0, 0};
+    auto fetch = [&](uintx4 (&rx)[2][4]) __attribute__((always_inline)) {
+        const int tp = f_tile < my_tiles ? f_t : npair - 1; // past the end: re-read the last step (never used)
+        if (f_t == 0) {
+            const long m0 = ((long)ty + (long)min(f_tile, my_tiles - 1) * gy) * 256 + 64 * w;
+#pragma unroll
+            for (int tm = 0; tm < 4; ++tm) {
+                const long m = min(m0 + 16 * tm + r16, (long)a.M - 1);           // clamped: masked at the store
+                xoff[tm] = (uint32_t)((m * a.dn_sm + 8 * g) * 2);
+            }
+        }
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {                    // (an odd list's last step reads its last entry twice and uses it once)
+            const int inner = __builtin_amdgcn_readfirstlane(s_inner[min(2 * tp + hf, nin - 1)]);
+            const char* xb = reinterpret_cast<const char*>(xp + (long)inner * 32);
+#pragma unroll
+            for (int tm = 0; tm < 4; ++tm) rx[hf][tm] = *reinterpret_cast<const uintx4*>(xb + xoff[tm]);
+        }
+        if (++f_t == npair) { f_t = 0; ++f_tile; }
+    };
+    int c_tile = 0, c_t = 0;                                // compute cursor
+    const int frag_off = r16 * 32 + 8 * g;                  // this lane's 16 bytes of a weight tile: a wave reads its 1 KB in lane order
+    auto compute = [&](const uintx4 (&rx)[2][4]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+            if (2 * c_t + hf < nin) {                       // workgroup-uniform
+                const uint16_t* wt = wres + (size_t)(2 * c_t + hf) * STEP + frag_off;
+#pragma unroll
+                for (int n = 0; n < 8; ++n) {
+                    const uint4 fw = *reinterpret_cast<const uint4*>(wt + n * 512);
+#pragma unroll
+                    for (int tm = 0; tm < 4; ++tm)
+                        acc[tm][n] = Frag32<T>::mma(__builtin_bit_cast(uint4, rx[hf][tm]), fw, acc[tm][n]);
+                }
+            }
+        }
+        if (++c_t == npair) { store_tile(c_tile); c_t = 0; ++c_tile; }   // the tile's last entries: results out
+    };
+#pragma unroll
+    for (int j = 0; j < DEPTH; ++j) fetch(fx[j]);
+    for (int step = 0; step < n_steps; step += DEPTH) {
+#pragma unroll
+        for (int u = 0; u < DEPTH; ++u) {
+            if (step + u < n_steps) compute(fx[u]);
+            fetch(fx[u]);                                   // step + u + DEPTH
+        }
     }
 }
 
@@ -2039,10 +2195,34 @@ extern "C" int flyhip_bs_dds(const void* a, const void* b_sp, void* c,
         c_sn == 1 && ((a_sz | a_sh | a_sm | b_sz | c_sz | c_sh | c_sm) % 8) == 0 && (M + 127) / 128 <= 65535) {
         DdsGroupArgs ga{b_sp, a, c, seg_ptr, seg_blk, seg_inner, grp_row0, grp_n, cols_per_head, M,
                         b_sz, a_sz, a_sh, a_sm, c_sz, c_sh, c_sm};
-        // as many workgroups as are resident together (three fit a CU); each walks its share of the token tiles
-        const long tiles = (M + 127) / 128;
         const Machine& mach = machine();
         ga.n_xcd = mach.xcds;
+        ga.n_grp = n_grp;
+        // groups whose weights fit the LDS (four output blocks times the longest reduction list) and enough tokens to
+        // amortise bringing them in: the weight-stationary kernel, two workgroups per compute unit
+        if (FLY_DDS_STATIONARY && max_seg_len > 0 && max_seg_len <= DDS_STAT_STEPS && (long)M >= 256L * 8) {
+            const long tiles = (M + 255) / 256;
+            long n_streams = 2L * mach.cus / ((long)n_grp * Z);
+            if (n_streams < 1) n_streams = 1;
+            if (n_streams > tiles) n_streams = tiles;
+            const long pairs = n_streams * n_grp;
+            const long gx = (pairs + mach.xcds - 1) / mach.xcds * mach.xcds;
+            const size_t smem = (size_t)max_seg_len * 8192;
+            dim3 grid((unsigned)gx, Z);
+#define DDS_STAT(TT, WTT)                                                                                          \
+    {                                                                                                              \
+        auto kern = bs_dds32s_kernel<TT, WTT, FLY_DDS_DEPTH>;                                                       \
+        static std::atomic<unsigned long long> lds_set{0};                                                         \
+        if (int rc2 = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_set, "bs_dds (stationary)")) return rc2; \
+        hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, ga, (int)n_streams);                                   \
+    }
+            if (dtype == BF16) { if (trans_b) DDS_STAT(bf16_t, false) else DDS_STAT(bf16_t, true) }
+            else { if (trans_b) DDS_STAT(f16_t, false) else DDS_STAT(f16_t, true) }
+#undef DDS_STAT
+            return check_launch("bs_dds32s_kernel");
+        }
+        // as many workgroups as are resident together (three fit a CU); each walks its share of the token tiles
+        const long tiles = (M + 127) / 128;
         long gy = (3L * mach.cus + (long)n_grp * Z - 1) / ((long)n_grp * Z);
         if (gy > tiles) gy = tiles;
         gy = (gy + mach.xcds - 1) / mach.xcds * mach.xcds;   // the kernel deals streams of token tiles to the XCDs

@@ -569,6 +569,33 @@ def test_fast_dds_many_token_tiles_per_workgroup(trans_b):
 
 
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('trans_b', [True, False])
+def test_dds_weight_stationary_kernel(trans_b, dtype):
+    """Reduction lists of at most nine blocks and a few thousand tokens: the dds kernel that keeps a group's weights in
+    LDS and reads its activations straight from memory.  Two batch entries, two heads, groups of one to four segments
+    (the last lanes of a short group store nothing), a segment without blocks, a token count that ends inside a
+    256-token tile, both block orientations."""
+    from fly_amd import matmul
+    print('case', trans_b, dtype, flush=True)
+    Z, H, block, M = 2, 2, 32, 2048 + 77
+    p, r = (11, 9) if trans_b else (9, 11)                # segments: the output blocks, 11 of them either way
+    g = torch.Generator().manual_seed(31)
+    seg = (torch.rand(H, 11, 9, generator=g) < 0.45).long()   # (head, output block, input block): lists of <= 9
+    seg[0, 1:4] = seg[0, 0]                                # a full group of four
+    seg[1, 5:7] = seg[1, 4]                                # a group of three
+    seg[1, 9] = 0                                          # an output block without inputs
+    layout = seg if trans_b else seg.transpose(1, 2).contiguous()
+    nnz = int(layout.sum())
+    w = torch.randn(Z, nnz, block, block, generator=g).to(dtype)
+    x = torch.randn(Z, H, M, 9 * block, generator=g).to(dtype)
+    out = matmul(layout, block, 'dds', trans_a=False, trans_b=trans_b)(x.to(DEV), w.to(DEV))
+    ref = ob.dds(x.double(), w.double(), layout, block, False, trans_b)
+    assert out.shape == ref.shape == (Z, H, M, 11 * block)
+    assert rel_err(out, ref) <= TOL[dtype]
+    assert float(out[1, 1, :, 9 * block:10 * block].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize('p,r,N', [(8, 8, 64), (11, 6, 72), (5, 13, 128)])
 def test_dsd_with_transposed_sparse_operand(p, r, N, dtype):
     """dense = sparse^T . dense (dV = P^T dO, and dK = dS^T Q which arrives as a transposed dds) on the
