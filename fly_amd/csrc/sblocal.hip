@@ -115,6 +115,10 @@ struct FwdArgs {
     // index partials / query features by batch * n_heavy + entry.
     const int32_t* tl_heavy; int n_heavy;
     int n_xcd;                      // dies the dispatcher deals workgroup ids to (set at launch)
+    // dropout of the exact weights (sblocal_attention.py:119: dropout(exp(QK - ln)); the normaliser sees no dropout):
+    // drop_thresh = 0 means none; pair (query i of (batch, head) bh, key s) is kept iff
+    // drop_keep(drop_row_hash(drop_seed, bh T + i), s, drop_thresh), kept weights times drop_scale (bf16-piece kernel)
+    uint32_t drop_seed, drop_thresh; float drop_scale;
 };
 
 // ROWS x W tile of a (seq, W) matrix, moved global -> registers -> LDS in two steps so that all of
@@ -3001,7 +3005,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
 // overlap (four), 5 D / 16 for P V (five; six with three V pieces) instead of (E + M + D) / 2 fp32 MFMAs of twice the duration.
 // A tile image is copied global -> registers -> LDS as it is (16-byte pieces in thread order), two LDS
 // stages.
-template <int E, int D, int M, bool SPLIT>
+template <int E, int D, int M, bool SPLIT, bool DROPOUT = false>
 __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
     typedef X3Tile<E, D, M> TL;
     constexpr int MH = M / 2, LDK = E + 4, LDV = D + 4;
@@ -3187,6 +3191,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
     const int qw0 = q0 + 16 * w;
     const int smin = max(iq - lc_lo, 0);
     const unsigned span = qvalid ? (unsigned)max(min(iq + lc_hi, len) - smin, 0) : 0u;
+    const uint32_t drop_row = DROPOUT ? drop_row_hash(a.drop_seed, (uint32_t)(bh * a.T + iq)) : 0u;
 
     // fragment addresses inside a stage (bytes): rows 16 kb + r16 share the swizzle of r16
     int koff[KS], foff[FS];
@@ -3302,8 +3307,8 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
                                   s_base + TK <= len && qw0 + 15 < a.T;
             floatx4 p[KB];
             float ovs = 0.f;
-            auto soft = [&](auto masked_tag) __attribute__((always_inline)) {
-                constexpr bool MASKED = decltype(masked_tag)::value;
+            auto soft = [&](auto masked_tag, auto drop_tag) __attribute__((always_inline)) {
+                constexpr bool MASKED = decltype(masked_tag)::value, DROP = decltype(drop_tag)::value;
                 bool ok[KB][4];
                 float mx = -INFINITY;
 #pragma unroll
@@ -3330,12 +3335,15 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
                     for (int i = 0; i < 4; ++i) {
                         const float e = ok[kb][i] ? __builtin_amdgcn_exp2f(s1[kb][i] - m_run) : 0.f;
                         const float ov = ok[kb][i] ? s2[kb][i] : 0.f;
-                        ze += e;
+                        ze += e;                                   // the normaliser sees no dropout
                         ovs += ov;
-                        p[kb][i] = e - ov * beta;
+                        float ek = e;
+                        if (DROP) ek = drop_keep(drop_row, (uint32_t)(s_base + 16 * kb + 4 * g + i), a.drop_thresh) ? e * a.drop_scale : 0.f;
+                        p[kb][i] = ek - ov * beta;
                     }
             };
-            if (interior) soft(std::false_type{}); else soft(std::true_type{});
+            if (interior) soft(std::false_type{}, std::integral_constant<bool, DROPOUT>{});
+            else soft(std::true_type{}, std::integral_constant<bool, DROPOUT>{});
             FLY_PROF2(stamp, 5);
             zp += ovs * wc;
             // O^T[d][query] += sum_keys V[key][d] p[key][query]: P exactly in three pieces, five or six products
@@ -3782,9 +3790,9 @@ template <int E, int M> constexpr size_t fwd_x3_smem() {
     constexpr size_t lowrank = sizeof(float) * ((size_t)M * (E + 4) + M);
     return tiles > proj ? (tiles > lowrank ? tiles : lowrank) : (proj > lowrank ? proj : lowrank);
 }
-template <int E, int M, bool SPLIT>
+template <int E, int M, bool SPLIT, bool DROPOUT = false>
 static int launch_fwd_x3(const FwdArgs& a, hipStream_t st) {
-    auto kern = sblocal_fwd_x3_kernel<E, E, M, SPLIT>;
+    auto kern = sblocal_fwd_x3_kernel<E, E, M, SPLIT, DROPOUT>;
 #ifdef FLY_X3_PAD
     constexpr size_t smem = fwd_x3_smem<E, M>() + FLY_X3_PAD;
 #else
@@ -3830,8 +3838,15 @@ static int launch_fwd_x3(const FwdArgs& a, hipStream_t st) {
 }
 template <typename T, int E, int M>
 static int launch_fwd(const FwdArgs& a, hipStream_t st) {
-    if (sizeof(T) == 4 && a.vt)
+    if (sizeof(T) == 4 && a.vt) {
+        // (dropout of the exact weights: a variant of its own, so that the kernel without it carries nothing of it)
+        if (a.drop_thresh) {
+            if constexpr (E <= 64 && M <= 128)
+                return a.n_parts > 1 ? launch_fwd_x3<E, M, true, true>(a, st) : launch_fwd_x3<E, M, false, true>(a, st);
+            return fail(ERR_UNSUPPORTED, "sblocal_fwd: no dropout variant for head dim %d with %d features", E, M);
+        }
         return a.n_parts > 1 ? launch_fwd_x3<E, M, true>(a, st) : launch_fwd_x3<E, M, false>(a, st);
+    }
     return a.n_parts > 1 ? launch_fwd_impl<T, E, M, true>(a, st) : launch_fwd_impl<T, E, M, false>(a, st);
 }
 
@@ -4395,9 +4410,13 @@ static int sblocal_fwd_checked(const void* q, const void* k, const void* v, cons
                                   int64_t k_sb, int64_t k_sh, int64_t k_ss,
                                   int64_t v_sb, int64_t v_sh, int64_t v_ss,
                                   int64_t o_sb, int64_t o_sh, int64_t o_ss,
-                                  float softmax_temp, int dtype, void* stream) {
+                                  float softmax_temp, int dtype, void* stream, DropArgs drop = DropArgs{0, 0, 1.f}) {
     FLY_REQUIRE(q && k && v && proj && kfeat && chunk_scale && kv && ksum && kmax && out && log_norm,
                 "sblocal_fwd: null pointer");
+    // dropout lives in the band kernel on bf16 pieces (float inputs with the key pass's tile images)
+    FLY_REQUIRE(drop.thresh == 0 || (dtype == F32 && vt && E <= 64 && 2 * mh <= 128),
+                "sblocal_fwd: dropout is implemented for float32 inputs with head dims up to 64 and up to 128 features "
+                "(the kernels on bf16 pieces)");
     FLY_REQUIRE(B > 0 && H > 0 && T > 0 && S > 0, "sblocal_fwd: empty problem");
     FLY_REQUIRE(local_context >= 1, "sblocal_fwd: local_context must be >= 1");
     FLY_REQUIRE(softmax_temp > 0.f, "sblocal_fwd: softmax_temp must be positive");
@@ -4416,6 +4435,7 @@ static int sblocal_fwd_checked(const void* q, const void* k, const void* v, cons
               B, H, T, S, mh_valid, local_context, nc, n_parts,
               q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss, softmax_temp,
               nullptr, nullptr, nullptr};
+    a.drop_seed = drop.seed; a.drop_thresh = drop.thresh; a.drop_scale = drop.scale;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     if (int rc_capture = refuse_capture(st)) return rc_capture;
     return dispatch_fwd(dtype, E, 2 * mh, a, st);
@@ -4493,8 +4513,11 @@ extern "C" int flyhip_sblocal_forward(const void* q, const void* k, const void* 
                                       int64_t k_sb, int64_t k_sh, int64_t k_ss,
                                       int64_t v_sb, int64_t v_sh, int64_t v_ss,
                                       int64_t o_sb, int64_t o_sh, int64_t o_ss,
-                                      float softmax_temp, int dtype, int flags, void* stream) {
+                                      float softmax_temp, int dtype, int flags,
+                                      float dropout_p, uint64_t dropout_seed, void* stream) {
     FLY_REQUIRE(q && k && v && proj && out && log_norm && workspace, "sblocal_forward: null pointer");
+    FLY_REQUIRE(dropout_p >= 0.f && dropout_p < 1.f, "sblocal_forward: dropout probability %g outside [0, 1)", (double)dropout_p);
+    FLY_REQUIRE(dropout_p == 0.f || !(flags & SB_EXACT_FP32), "sblocal_forward: dropout is not implemented on the fp32-pipe kernels");
     FLY_REQUIRE((flags & ~SB_EXACT_FP32) == 0, "sblocal_forward: unknown flags 0x%x", flags);
     FLY_REQUIRE(B > 0 && H > 0 && T > 0 && S > 0 && local_context >= 1, "sblocal_forward: empty problem");
     FLY_REQUIRE(dtype == F32 || dtype == BF16, "sblocal_forward supports float32 and bfloat16, got dtype code %d", dtype);
@@ -4522,7 +4545,7 @@ extern "C" int flyhip_sblocal_forward(const void* q, const void* k, const void* 
                                f(w.kv_part), f(w.part_max), w.n_split, key_lengths, out, log_norm,
                                split ? f(w.part_ws) : nullptr, w.n_parts, B, H, T, S, E, D, mh, mh_valid, local_context,
                                q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss,
-                               softmax_temp, dtype, stream);
+                               softmax_temp, dtype, stream, drop_args(dropout_p, dropout_seed));
 }
 
 // ---------------------------------------------------------------------------------------

@@ -413,6 +413,9 @@ struct BwdX3Args {
     // long lists: tl_skip (one flag per (head, outer tile)) marks the tiles the main launch leaves out; the launch
     // in parts takes (batch, tl_heavy[j], part) for the n_heavy listed (head, outer tile) indices, then the finish
     const int32_t* tl_skip; const int32_t* tl_heavy; int n_heavy;
+    // dropout of the exact weights in the forward (drop_thresh = 0: none): the same mask again from the seed --
+    // pair (query i of bh, key s) was kept iff drop_keep(drop_row_hash(drop_seed, bh T + i), s, drop_thresh)
+    uint32_t drop_seed, drop_thresh; float drop_scale;
 };
 
 // one tile image, global memory -> LDS stage `dst` (linear; each wave load writes 1024 consecutive bytes); TAIL: also
@@ -665,6 +668,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
     const float ln_o = KEYMAJOR ? 0.f : a.ln[(long)bh * a.T + orow] * LOG2E, c_o = KEYMAJOR ? 0.f : a.c[(long)bh * a.T + orow];
     const float sc = a.temp * LOG2E;                       // scores leave the MFMA unscaled; exponents are base 2
+    const bool drop_on = a.drop_thresh != 0;               // (kernel-uniform)
+    const uint32_t drop_row = drop_row_hash(a.drop_seed, (uint32_t)(bh * a.T + (KEYMAJOR ? 0 : orow)));   // query-major: the lane's query
     // inner rows this lane's outer row may meet: nmin <= n < nmin + span
     const int nmin = max(o + lo, 0);
     const unsigned span = ovalid ? (unsigned)max(min(o + hi, n_limit) - nmin, 0) : 0u;
@@ -748,10 +753,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                     const int n = n_base + 16 * kb + 4 * g + i;
                     const bool ok = LIST ? ovalid : (unsigned)(n - nmin) < span;      // (a block of the support is whole)
                     const float av = ok ? __builtin_amdgcn_exp2f(s1[kb][i] * sc - (KEYMAJOR ? lnq[i] : ln_o)) : 0.f;
-                    const float df = ok ? s3[kb][i] - (KEYMAJOR ? cq[i] : c_o) : 0.f;
-                    wdm[kb][i] = av * df;
+                    const float cc = KEYMAJOR ? cq[i] : c_o;
+                    const float df = ok ? s3[kb][i] - cc : 0.f;
+                    // with dropout D (0 or 1 / (1 - p)) on the exact weight: out = sum (D a - kb) v + ..., and the
+                    // normaliser sees no dropout: dm = a (D g.v - c), the weight of g in d v is D a - kb
+                    float dk = 1.f;
+                    if (drop_on) {
+                        const uint32_t rh = KEYMAJOR ? drop_row_hash(a.drop_seed, (uint32_t)(bh * a.T + n)) : drop_row;
+                        dk = drop_keep(rh, (uint32_t)(KEYMAJOR ? o : n), a.drop_thresh) ? a.drop_scale : 0.f;
+                    }
+                    wdm[kb][i] = drop_on ? av * (ok ? dk * s3[kb][i] - cc : 0.f) : av * df;
                     wdf[kb][i] = df;
-                    wak[kb][i] = av - (ok ? s2[kb][i] : 0.f);
+                    wak[kb][i] = av * dk - (ok ? s2[kb][i] : 0.f);
                 }
             }
             uintx4 dmh, dml, dfh, dfm, dfl, akh, akm, akl;
@@ -1025,9 +1038,11 @@ extern "C" int flyhip_sblocal_bwd_pieces(const void* outer_images, const void* i
                                          const float* gmat, const float* gvec, const float* proj,
                                          float* d1, float* d3, float* part_ws, int64_t part_ws_floats,
                                          int BH, int H, int T, int S, int E, int M, int local_context,
-                                         float softmax_temp, int key_major, void* stream) {
+                                         float softmax_temp, int key_major, float dropout_p, uint64_t dropout_seed,
+                                         void* stream) {
     FLY_REQUIRE(outer_images && inner_images && x1 && log_norm && c && gmat && gvec && proj && d1,
                 "sblocal_bwd_pieces: null pointer");
+    FLY_REQUIRE(dropout_p >= 0.f && dropout_p < 1.f, "sblocal_bwd_pieces: dropout probability %g outside [0, 1)", (double)dropout_p);
     FLY_REQUIRE(!key_major || d3, "sblocal_bwd_pieces: the key-major pass needs d3");
     FLY_REQUIRE(BH > 0 && H > 0 && BH % H == 0 && T > 0 && S > 0, "sblocal_bwd_pieces: empty or inconsistent problem");
     FLY_REQUIRE(local_context >= 1, "sblocal_bwd_pieces: local_context must be >= 1");
@@ -1035,6 +1050,8 @@ extern "C" int flyhip_sblocal_bwd_pieces(const void* outer_images, const void* i
     BwdX3Args a{reinterpret_cast<const char*>(outer_images), reinterpret_cast<const char*>(inner_images), x1,
                 log_norm, c, key_lengths, d1, d3, BH, H, T, S, local_context, softmax_temp, gmat, gvec, proj, 0, part_ws, 1,
                 nullptr, nullptr, nullptr, nullptr, nullptr, 0};
+    const DropArgs dr = drop_args(dropout_p, dropout_seed);
+    a.drop_seed = dr.seed; a.drop_thresh = dr.thresh; a.drop_scale = dr.scale;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     if (int rc_capture = refuse_capture(st)) return rc_capture;
     const long wsf = part_ws ? (long)part_ws_floats : 0;

@@ -183,8 +183,12 @@ class SBLocalPlan:
                       v.stride(0), v.stride(2), v.stride(1), out.stride(0), out.stride(2), out.stride(1),
                       t, self.code, stream)
 
-    def run(self, q, k, v, proj, lens, local_context, t, out, log_norm):
+    def run(self, q, k, v, proj, lens, local_context, t, out, log_norm, dropout=(0.0, 0)):
+        """dropout: (probability, seed) -- dropout of the exact weights inside the band kernel (float32 inputs on the
+        bf16-piece kernels; the library refuses it elsewhere); the one-call path only."""
         B, H, T, S, dim, mh, mh_valid = self.shape
+        if dropout[0] > 0 and (self.n_parts != self.planned_parts or not self.operand_images or local_context != self.local_context):
+            raise NotImplementedError('dropout needs the one-call path of the plan (its own part count and band)')
         if self.n_parts != self.planned_parts or not self.operand_images or local_context != self.local_context:
             # a part count or band the library would not choose itself: the two-call path takes them as arguments
             with torch.cuda.device(self.device):
@@ -199,7 +203,7 @@ class SBLocalPlan:
                       B, H, T, S, dim, dim, mh, mh_valid, local_context,
                       q.stride(0), q.stride(2), q.stride(1), k.stride(0), k.stride(2), k.stride(1),
                       v.stride(0), v.stride(2), v.stride(1), out.stride(0), out.stride(2), out.stride(1),
-                      t, self.code, self.flags, _lib.stream_ptr(self.device))
+                      t, self.code, self.flags, float(dropout[0]), int(dropout[1]), _lib.stream_ptr(self.device))
 
 
 class ScratchCache:
@@ -272,7 +276,7 @@ def _padded_projection(projection_matrix, mh, dim, cache):
 
 
 def sblocal_forward(query, key, value, projection_matrix, local_context, softmax_temp=None,
-                    key_lengths=None, cache=None, exact_fp32=False):
+                    key_lengths=None, cache=None, exact_fp32=False, dropout_p=0.0, dropout_seed=0):
     """Scatterbrain-local attention forward on the GPU.
 
     query (B,T,H,E), key (B,S,H,E), value (B,S,H,D) float32 or bfloat16 CUDA tensors;
@@ -287,6 +291,11 @@ def sblocal_forward(query, key, value, projection_matrix, local_context, softmax
     exact_fp32: float32 inputs only.  False (default): products on the bf16 matrix pipe from operands split into bf16
     pieces with fp32 accumulation (V rounded to 16, the features to 17 significant bits; about 5e-6 of the float64
     result at the benchmark configuration).  True: every product on the fp32 matrix pipe (about 1e-6; 1.6 times the time).
+
+    dropout_p, dropout_seed: dropout of the exact band weights exp(QK - log_normalization) (sblocal_attention.py:116-119:
+    the normaliser and the low-rank part see none) inside the band kernel.  No mask is stored: a weight is kept
+    according to a hash of (seed, batch, head, query, key), which the backward kernels evaluate again, and kept
+    weights are scaled by 1 / (1 - p).  float32 inputs with head dims <= 64 and <= 128 features.
     """
     _lib.require_gpu(query, key, value, projection_matrix, key_lengths)
     if query.dtype not in (torch.float32, torch.bfloat16):
@@ -330,7 +339,10 @@ def sblocal_forward(query, key, value, projection_matrix, local_context, softmax
     plan = make_plan() if cache is None else cache.plan(plan_key, make_plan)
     out = torch.empty(B, T, H, dim, dtype=query.dtype, device=query.device)
     log_norm = torch.empty(B, H, T, dtype=torch.float32, device=query.device)
-    plan.run(q, k, v, proj, lens, local_context, t, out, log_norm)
+    if dropout_p > 0 and (query.dtype != torch.float32 or exact_fp32 or dim > 64 or m > 128):
+        raise NotImplementedError('attention dropout is implemented in the band kernel on bf16 pieces: float32 inputs, '
+                                  f'head dims <= 64, <= 128 features (got {query.dtype}, {max(E, D)}, {2 * mh_valid})')
+    plan.run(q, k, v, proj, lens, local_context, t, out, log_norm, dropout=(float(dropout_p), int(dropout_seed)))
     return out[..., :D], log_norm.unsqueeze(-1)
 
 
@@ -383,12 +395,13 @@ class _SBLocalFn(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, query, key, value, projection_matrix, local_context, softmax_temp, key_lengths, cache=None,
-                exact_fp32=False):
+                exact_fp32=False, dropout_p=0.0, dropout_seed=0):
         out, log_norm = sblocal_forward(query, key, value, projection_matrix, local_context,
                                         softmax_temp=softmax_temp, key_lengths=key_lengths, cache=cache,
-                                        exact_fp32=exact_fp32)
+                                        exact_fp32=exact_fp32, dropout_p=dropout_p, dropout_seed=dropout_seed)
         ctx.save_for_backward(query, key, value, projection_matrix, out, log_norm)
         ctx.args = (local_context, softmax_temp, key_lengths)
+        ctx.dropout = (float(dropout_p), int(dropout_seed))
         ctx.mark_non_differentiable(log_norm)
         return out, log_norm
 
@@ -398,18 +411,19 @@ class _SBLocalFn(torch.autograd.Function):
         query, key, value, projection_matrix, out, log_norm = ctx.saved_tensors
         local_context, softmax_temp, key_lengths = ctx.args
         dq, dk, dv = sblocal_backward(query, key, value, projection_matrix, local_context, softmax_temp,
-                                      key_lengths, out, log_norm, grad_out)
-        return dq, dk, dv, None, None, None, None, None, None
+                                      key_lengths, out, log_norm, grad_out, dropout=ctx.dropout)
+        return dq, dk, dv, None, None, None, None, None, None, None, None
 
 
 def sblocal_attention_fn(query, key, value, projection_matrix, local_context, softmax_temp=None,
-                         key_lengths=None, cache=None, exact_fp32=False):
+                         key_lengths=None, cache=None, exact_fp32=False, dropout_p=0.0, dropout_seed=0):
     """sblocal_forward, differentiable with respect to query, key and value."""
     if torch.is_grad_enabled() and any(x.requires_grad for x in (query, key, value)):
         return _SBLocalFn.apply(query, key, value, projection_matrix, local_context, softmax_temp, key_lengths, cache,
-                                exact_fp32)
+                                exact_fp32, dropout_p, dropout_seed)
     return sblocal_forward(query, key, value, projection_matrix, local_context, softmax_temp=softmax_temp,
-                           key_lengths=key_lengths, cache=cache, exact_fp32=exact_fp32)
+                           key_lengths=key_lengths, cache=cache, exact_fp32=exact_fp32, dropout_p=dropout_p,
+                           dropout_seed=dropout_seed)
 
 
 class SBLocalAttention(nn.Module):
@@ -419,7 +433,8 @@ class SBLocalAttention(nn.Module):
 
     Same constructor and forward signature as the reference class (sblocal_attention.py:29-44).
     The GPU path covers what the reference itself exercises: non-causal, no attn_mask, optional
-    length-style key_padding_mask, softmax_eps = 0, dropout inactive.  ``need_weights`` /
+    length-style key_padding_mask, softmax_eps = 0; attention dropout in training mode for float32 inputs with head
+    dims <= 64 and <= 128 features (inside the band kernel, see sblocal_forward).  ``need_weights`` /
     ``return_attn_unnormalized`` (:124-136) give the dense matrix for small problems, formed with library products around
     the fused kernels' ``log_normalization``; ``out`` always comes from the kernels.  Any other request raises
     NotImplementedError -- there is no slower fallback inside this module.
@@ -458,8 +473,15 @@ class SBLocalAttention(nn.Module):
                                       f'of small problems only (at most {self.max_weight_elements} elements)')
         if self.softmax_eps != 0.0:
             raise NotImplementedError('softmax_eps != 0 is not supported by the fused kernel')
+        # attention dropout (:116-119) runs inside the band kernel: a fresh seed per call from the CPU generator
+        # (torch.manual_seed makes a run reproducible; no device synchronisation), the mask never exists in memory
+        dropout_p, dropout_seed = 0.0, 0
         if self.training and self.dropout.p > 0.0:
-            raise NotImplementedError('attention dropout is not implemented in the fused kernel')
+            if need_weights or return_attn_unnormalized:
+                raise NotImplementedError('need_weights with active attention dropout is not implemented')
+            dropout_p = float(self.dropout.p)
+            dropout_seed = int(torch.randint(0, 2 ** 62, (1,)).item())
+            self.last_dropout_seed = dropout_seed
         lengths = None
         if key_padding_mask is not None and not bool(key_padding_mask.all_ones):
             lengths = key_padding_mask.lengths          # raises ValueError unless a length mask
@@ -467,7 +489,7 @@ class SBLocalAttention(nn.Module):
         out, log_norm = sblocal_attention_fn(query, key, value, self.feature_map.projection_matrix,
                                              self.local_context, softmax_temp=self.softmax_temp,
                                              key_lengths=lengths, cache=self._scratch_cache,
-                                             exact_fp32=self.exact_fp32)
+                                             exact_fp32=self.exact_fp32, dropout_p=dropout_p, dropout_seed=dropout_seed)
         self.last_log_normalization = log_norm.detach()
         attn = None
         if need_weights or return_attn_unnormalized:

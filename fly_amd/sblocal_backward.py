@@ -148,7 +148,7 @@ def _scratch_sizes(BH, T, S, dim, mk, local_context):
     return got
 
 
-def _backward_hip(Q, K, V, G, O, LN, P, lens_b, H, local_context, t, dims, pieces=True, support=None):
+def _backward_hip(Q, K, V, G, O, LN, P, lens_b, H, local_context, t, dims, pieces=True, support=None, dropout=(0.0, 0)):
     """d query, d key, d value (BH, rows, width) in five launches: flyhip_sblocal_bwd_prep (scaled features of
     queries and keys, c = g . out, and the per-head sums over all keys / all queries) and the two passes of the
     band kernel (everything per (query, key) pair, the low-rank epilogue, the chain rule through the feature map).
@@ -211,10 +211,12 @@ def _backward_hip(Q, K, V, G, O, LN, P, lens_b, H, local_context, t, dims, piece
         elif pieces:
             _lib.call('flyhip_sblocal_bwd_pieces', qimg.data_ptr(), kimg.data_ptr(), q_.data_ptr(),
                       ln_.data_ptr(), c_.data_ptr(), _lib.ptr(lens_b), kv.data_ptr(), ksum.data_ptr(), proj.data_ptr(),
-                      dq.data_ptr(), None, _lib.ptr(part_ws), n_ws, BH, H, T, S, dim, mk, local_context, float(t), 0, st)
+                      dq.data_ptr(), None, _lib.ptr(part_ws), n_ws, BH, H, T, S, dim, mk, local_context, float(t), 0,
+                      float(dropout[0]), int(dropout[1]), st)
             _lib.call('flyhip_sblocal_bwd_pieces', kimg.data_ptr(), qimg.data_ptr(), k_.data_ptr(),
                       ln_.data_ptr(), c_.data_ptr(), _lib.ptr(lens_b), qg.data_ptr(), qc.data_ptr(), proj.data_ptr(),
-                      dk.data_ptr(), dv.data_ptr(), _lib.ptr(part_ws), n_ws, BH, H, T, S, dim, mk, local_context, float(t), 1, st)
+                      dk.data_ptr(), dv.data_ptr(), _lib.ptr(part_ws), n_ws, BH, H, T, S, dim, mk, local_context, float(t), 1,
+                      float(dropout[0]), int(dropout[1]), st)
         else:
             _lib.call('flyhip_sblocal_bwd', q_.data_ptr(), psi_.data_ptr(), g_.data_ptr(), k_.data_ptr(), phik_.data_ptr(),
                       v_.data_ptr(), ln_.data_ptr(), c_.data_ptr(), _lib.ptr(lens_b), kv.data_ptr(), ksum.data_ptr(),
@@ -307,7 +309,8 @@ def _scaled_features(Q, K, P, t, LN, lens):
 
 
 def sblocal_backward(query, key, value, projection_matrix, local_context, softmax_temp, key_lengths,
-                     out, log_normalization, grad_out, chunk=256, max_elements=1 << 27, band_kernel=None, support=None):
+                     out, log_normalization, grad_out, chunk=256, max_elements=1 << 27, band_kernel=None, support=None,
+                     dropout=(0.0, 0)):
     """query (B,T,H,E), key (B,S,H,E), value (B,S,H,D), out / grad_out (B,T,H,D),
     log_normalization (B,H,T,1) as returned by the forward; key_lengths (B,) or None.
     max_elements bounds the
@@ -320,6 +323,8 @@ def sblocal_backward(query, key, value, projection_matrix, local_context, softma
     support: the exact part lives on a block-sparse support of 32 x 32 blocks instead of a band (Scatterbrain
     attention on a block-sparse support, sbblocksparse_attention.py:161-212): see _backward_hip; kernels only, no key
     lengths, local_context is ignored.
+    dropout: (probability, seed) the forward was called with; the band kernels on bf16 pieces form the forward's mask
+    again from the seed (other paths: NotImplementedError when the probability is not zero).
     Returns (d query, d key, d value) in the dtypes of the inputs."""
     B, T, H, E = query.shape
     S, D = key.shape[1], value.shape[3]
@@ -345,6 +350,9 @@ def sblocal_backward(query, key, value, projection_matrix, local_context, softma
         # host tensors are accepted for one purpose: checking the written-out gradient formulas in float64 against autograd
         raise NotImplementedError('sblocal_backward runs on the GPU; host tensors only in float64 (the check of the formulas)')
     lens_b = None if key_lengths is None else key_lengths.to(device=Q.device, dtype=torch.int64).contiguous()
+    if dropout[0] > 0 and (support is not None or not on_kernels or band_kernel in ('sums', 'fp32')):
+        raise NotImplementedError('the backward under attention dropout runs on the band kernels on bf16 pieces only '
+                                  f'(GPU, head dims <= 64, <= 128 features; got ({E}, {D}), {2 * mh})')
     if support is not None:
         if not on_kernels or key_lengths is not None or T % 32 or S % 32:
             raise NotImplementedError('the backward on a block-sparse support needs the GPU kernels (float32 or bfloat16 '
@@ -354,7 +362,7 @@ def sblocal_backward(query, key, value, projection_matrix, local_context, softma
     elif on_kernels and band_kernel != 'sums':
         # features, per-head sums and the two passes of the fused kernel
         dQ, dK, dV = _backward_hip(Q, K, V, G, O, LN, P, lens_b, H, local_context, t, dims,
-                                   pieces=band_kernel != 'fp32')
+                                   pieces=band_kernel != 'fp32', dropout=dropout)
     else:
         psi, phik = _scaled_features(Q, K, P, t, LN, lens)
         c = (G * O).sum(-1, keepdim=True)

@@ -123,8 +123,13 @@ int flyhip_sblocal_fwd(const void* q, const void* k, const void* v, const float*
  * contents need no initialisation and mean nothing between calls; one call at a time may use it.
  * flags: 0, or FLYHIP_SB_EXACT_FP32 -- float inputs then take the fp32 matrix pipe for every product (no bf16
  * pieces, V and the features not rounded: about 1e-6 of the float64 result instead of 5e-6, at 1.6 times the
- * time); pass the same flags to both functions.  Arguments otherwise as for flyhip_sb_kv_reduce /
- * flyhip_sblocal_fwd. */
+ * time); pass the same flags to both functions.
+ * dropout_p in [0, 1), dropout_seed: dropout of the exact weights exp(QK - log_normalization) as in
+ * sblocal_attention.py:119 (the normaliser and the low-rank part see none).  No mask is stored: whether the weight of
+ * (query i, key s) of (batch b, head h) is kept is a hash of (seed, (b H + h) T + i, s), and kept weights are scaled by
+ * 1 / (1 - p); flyhip_sblocal_bwd_pieces forms the same mask from the same seed.  float32 inputs with head dims up to
+ * 64 and up to 128 features (the kernels on bf16 pieces), not with FLYHIP_SB_EXACT_FP32; 0 = no dropout.
+ * Arguments otherwise as for flyhip_sb_kv_reduce / flyhip_sblocal_fwd. */
 #define FLYHIP_SB_EXACT_FP32 1
 int64_t flyhip_sb_workspace_bytes(int B, int H, int T, int S, int E, int mh, int local_context, int dtype, int flags);
 int flyhip_sblocal_forward(const void* q, const void* k, const void* v, const float* proj,
@@ -135,7 +140,8 @@ int flyhip_sblocal_forward(const void* q, const void* k, const void* v, const fl
                            int64_t k_sb, int64_t k_sh, int64_t k_ss,
                            int64_t v_sb, int64_t v_sh, int64_t v_ss,
                            int64_t o_sb, int64_t o_sh, int64_t o_ss,
-                           float softmax_temp, int dtype, int flags, void* stream);
+                           float softmax_temp, int dtype, int flags,
+                           float dropout_p, uint64_t dropout_seed, void* stream);
 
 /* flyhip_sblocal_fwd for callers that cannot allocate device memory -- tight serving loops, harnesses
  * that forbid hipMalloc.  It has no counterpart in the reference.
@@ -228,7 +234,9 @@ int flyhip_sblocal_bwd_prep(const float* q, const float* k, const float* v, cons
  * (gmat, proj and the image's values in three pieces each).
  * part_ws (may be NULL) of part_ws_floats >= flyhip_sblocal_bwd_parts_floats(BH,T,S,E,M,local_context) floats: with
  * it, problems of fewer 64-row tiles than the GPU holds workgroups walk each tile's band in several parts by as many
- * workgroups and finish in a second launch; without it (or when that function returns 0) every tile is one workgroup. */
+ * workgroups and finish in a second launch; without it (or when that function returns 0) every tile is one workgroup.
+ * dropout_p, dropout_seed: what the forward was called with (0: none) -- the kernel forms the forward's mask again
+ * from the seed (ref: the nn.Dropout of src/models/attention/sblocal_attention.py:119 under autograd). */
 int64_t flyhip_sblocal_bwd_parts_floats(int BH, int T, int S, int E, int M, int local_context);
 int flyhip_sblocal_bwd_pieces(const void* outer_images, const void* inner_images,
                               const float* x1,
@@ -236,7 +244,8 @@ int flyhip_sblocal_bwd_pieces(const void* outer_images, const void* inner_images
                               const float* gmat, const float* gvec, const float* proj,
                               float* d1, float* d3, float* part_ws, int64_t part_ws_floats,
                               int BH, int H, int T, int S, int E, int M, int local_context,
-                              float softmax_temp, int key_major, void* stream);
+                              float softmax_temp, int key_major, float dropout_p, uint64_t dropout_seed,
+                              void* stream);
 
 /* flyhip_sblocal_bwd_pieces for Scatterbrain attention on a block-sparse support (the reference takes these
  * gradients from autograd through src/models/attention/sbblocksparse_attention.py:161-212): the exact weights live on

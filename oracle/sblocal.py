@@ -145,8 +145,36 @@ def local_weighted_average(A, V, chunk=256):
 # --------------------------------------------------------------------------------------
 # SBLocalAttention.forward -- src/models/attention/sblocal_attention.py:43-137
 # --------------------------------------------------------------------------------------
+def _mix32(h):
+    """The 32-bit finaliser of MurmurHash3 on int64 tensors holding values below 2^32 (products wrap modulo 2^64, which
+    leaves their low 32 bits intact)."""
+    m = 0xFFFFFFFF
+    h = h ^ (h >> 16)
+    h = (h * 0x85EBCA6B) & m
+    h = h ^ (h >> 13)
+    h = (h * 0xC2B2AE35) & m
+    return h ^ (h >> 16)
+
+
+def dropout_keep(seed, p, B, H, T, S):
+    """The dropout multiplier of the HIP band kernels, restated on the host so that tests can hand the kernels' own
+    mask to the reference algebra: (B,H,T,S) float64, 1 / (1 - p) where the weight of (query i, key s) of (batch b,
+    head h) is kept and 0 where it is dropped.  Kept iff mix(mix((b H + h) T + i) * 0x9E3779B1 + seed') + s * 0x632BE5AB)
+    >= floor(p 2^32), seed' the 64-bit seed folded to 32 bits (fly_amd/csrc/common.h: drop_args, drop_row_hash,
+    drop_keep).  This has no counterpart in the reference, whose mask comes from torch's generator
+    (sblocal_attention.py:119); the statistics -- independent keeps with probability 1 - p -- are what both share."""
+    m = 0xFFFFFFFF
+    seed32 = (seed & m) ^ (((seed >> 32) * 0x9E3779B1) & m)
+    thresh = min(max(int(p * 4294967296.0), 1), 0xFFFFFFFF) if p > 0 else 0
+    rows = torch.arange(B * H * T, dtype=torch.int64)
+    row_hash = _mix32((rows * 0x9E3779B1 + seed32) & m).view(B, H, T, 1)
+    cols = torch.arange(S, dtype=torch.int64).view(1, 1, 1, S)
+    h = _mix32((row_hash + cols * 0x632BE5AB) & m)
+    return (h >= thresh).to(torch.float64) / (1.0 - p)
+
+
 def sblocal_attention(query, key, value, projection_matrix, local_context, softmax_temp=None,
-                      key_lengths=None, chunk=256, return_band_lowrank_mass=False):
+                      key_lengths=None, chunk=256, return_band_lowrank_mass=False, dropout_multiplier=None):
     """sblocal_attention.py:56-122 for causal=False, attn_mask=None, eps=0, dropout off.
     query (B,T,H,E), key (B,S,H,E), value (B,S,H,D); projection_matrix (m/2, E);
     key_lengths (B,) int64 or None.  The reference's ``softmax_temp or 1/sqrt(E)`` (:59)
@@ -154,7 +182,9 @@ def sblocal_attention(query, key, value, projection_matrix, local_context, softm
     return_band_lowrank_mass also (B,H,T,1): the normalised low-rank weight a query's band carries,
     sum_band q'.k' * prime_scale -- the amount that is subtracted on the band and added back through the
     sums over all keys (a condition number of the estimator: of order one or below when the features
-    approximate the exact weights, hundreds when they do not)."""
+    approximate the exact weights, hundreds when they do not).
+    dropout_multiplier: None, or (B,H,T,S) -- the mask of nn.Dropout times 1 / (1 - p) as it falls on the pair (query,
+    key); it multiplies exp(QK - log_normalization) and nothing else (:116-119)."""
     B, T, H, E = query.shape
     _, S, _, D = value.shape
     t = softmax_temp or 1 / math.sqrt(E)
@@ -187,7 +217,10 @@ def sblocal_attention(query, key, value, projection_matrix, local_context, softm
     lr_ln = torch.log((qk1.unsqueeze(-1) - dots_prime_sum).clamp_min(1e-24)) + prime_log_scale
     log_normalization = torch.logaddexp(QK_lse, lr_ln)                            # :113
     prime_scale = torch.exp(prime_log_scale - log_normalization)                  # :115
-    dots = torch.exp(QK - log_normalization) - dots_prime * prime_scale           # :119
+    exact = torch.exp(QK - log_normalization)
+    if dropout_multiplier is not None:                                            # self.dropout(...), :119
+        exact = exact * torch.gather(dropout_multiplier.to(exact.dtype), 3, local_idx.clamp(0, S - 1).expand(B, H, T, lc))
+    dots = exact - dots_prime * prime_scale                                       # :119
     out = local_weighted_average(dots, v, chunk) + qkv * prime_scale              # :121-122
     if return_band_lowrank_mass:
         return out.permute(0, 2, 1, 3), log_normalization, dots_prime_sum * prime_scale

@@ -628,3 +628,85 @@ def test_module_scratch_stays_bounded_over_many_shapes():
     one_round()
     assert len(attn._scratch_cache) == attn._scratch_cache.max_plans
     assert torch.cuda.memory_allocated(dev) == held
+
+
+@pytest.mark.parametrize('case', [
+    # B, T, S, H, E, D, mh, lc, lens, p
+    (2, 3136, 3136, 1, 64, 64, 64, 512, None, 0.1),           # config 1: the band of a tile walked in parts
+    (6, 700, 700, 4, 64, 64, 64, 200, None, 0.25),            # one part per tile
+    (2, 300, 260, 3, 32, 32, 16, 33, [260, 111], 0.5),        # T != S, odd window, key lengths
+    (1, 130, 130, 2, 40, 24, 13, 64, None, 0.1),              # padded head dims and features
+])
+def test_attention_dropout_in_the_band_kernel(case):
+    """Dropout of the exact weights (sblocal_attention.py:116-119) inside the band kernel: the kernel's mask is a hash
+    of (seed, batch, head, query, key); restated on the host and handed to the oracle as nn.Dropout's multiplier, the
+    oracle gives the kernel's output (1e-4) and, through autograd, the backward kernels' gradients (2e-4).  The
+    log-normaliser is the one without dropout; p = 0 is bit-identical to the call without the arguments; another seed
+    gives another output."""
+    from fly_amd import sblocal_attention_fn, sblocal_forward
+    B, T, S, H, E, D, mh, lc, lens, p = case
+    print('case', case, flush=True)
+    dev = torch.device('cuda:0')
+    q, k, v, P = make_inputs(B, T, S, H, E, D, mh, seed=77)
+    kl = None if lens is None else torch.tensor(lens)
+    seed = 0x1234_5678_9ABC + T
+    keep = osb.dropout_keep(seed, p, B, H, T, S)
+    assert abs(float((keep > 0).double().mean()) - (1 - p)) < 0.02
+    qd, kd, vd = (x.double().requires_grad_() for x in (q, k, v))
+    ref_out, ref_ln = osb.sblocal_attention(qd, kd, vd, P.double(), lc, key_lengths=kl, dropout_multiplier=keep)
+    plain_out, plain_ln = osb.sblocal_attention(q.double(), k.double(), v.double(), P.double(), lc, key_lengths=kl)
+    assert torch.equal(ref_ln.detach(), plain_ln) and rel_err(ref_out, plain_out) > 1e-2     # the mask matters
+    w = torch.randn(B, T, H, D, generator=torch.Generator().manual_seed(5))
+    (ref_out * w.double()).sum().backward()
+
+    qg, kg, vg = (x.to(dev).requires_grad_() for x in (q, k, v))
+    kld = None if kl is None else kl.to(dev)
+    out, ln = sblocal_attention_fn(qg, kg, vg, P.to(dev), lc, key_lengths=kld, dropout_p=p, dropout_seed=seed)
+    assert rel_err(out, ref_out) <= 1e-4, rel_err(out, ref_out)
+    assert rel_err(ln, ref_ln) <= 1e-4
+    (out * w.to(dev)).sum().backward()
+    for name, got, ref in (('dq', qg.grad, qd.grad), ('dk', kg.grad, kd.grad), ('dv', vg.grad, vd.grad)):
+        assert rel_err(got, ref) <= 2e-4, (name, rel_err(got, ref))
+    with torch.no_grad():
+        base, _ = sblocal_forward(qg, kg, vg, P.to(dev), lc, key_lengths=kld)
+        zero, _ = sblocal_forward(qg, kg, vg, P.to(dev), lc, key_lengths=kld, dropout_p=0.0, dropout_seed=seed)
+        other, _ = sblocal_forward(qg, kg, vg, P.to(dev), lc, key_lengths=kld, dropout_p=p, dropout_seed=seed + 1)
+    assert torch.equal(base, zero) and not torch.equal(other, out.detach())
+
+
+def test_attention_dropout_module_and_refusals():
+    """SBLocalAttention with attention_dropout: eval mode ignores it, training mode drops (a fresh seed per call from
+    the CPU generator, reproducible under torch.manual_seed), the mean over many masks is the output without dropout,
+    and configurations off the bf16-piece kernels raise."""
+    from fly_amd import SBLocalAttention, sblocal_forward
+    dev = torch.device('cuda:0')
+    q, k, v, P = make_inputs(2, 256, 256, 2, 64, 64, 32, seed=8)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    attn = SBLocalAttention(local_context=64, dim_heads=64, nb_features=64, attention_dropout=0.2).to(dev)
+    attn.feature_map.projection_matrix.copy_(P.to(dev))
+    attn.feature_map.freeze_projection()
+    attn.eval()
+    with torch.no_grad():
+        plain, _ = attn(qd, kd, vd)
+        attn.train()
+        torch.manual_seed(3)
+        a1, _ = attn(qd, kd, vd)
+        a2, _ = attn(qd, kd, vd)
+        torch.manual_seed(3)
+        b1, _ = attn(qd, kd, vd)
+        assert torch.equal(a1, b1) and not torch.equal(a1, a2) and not torch.equal(a1, plain)
+        mean = torch.zeros_like(plain)
+        n = 400
+        for _ in range(n):
+            mean += attn(qd, kd, vd)[0]
+        mean /= n
+    # per output the mask's variance is at most p / (1 - p) sum a^2 v^2 <= 0.25 max|v|^2: 400 draws leave ~ 0.03 max|v|
+    assert float((mean - plain).abs().max()) <= 0.1 * float(plain.abs().max() + vd.abs().max() * 0.3)
+    assert rel_err(mean, plain) <= 0.15
+    with pytest.raises(NotImplementedError):
+        sblocal_forward(qd.bfloat16(), kd.bfloat16(), vd.bfloat16(), P.to(dev), 64, dropout_p=0.1, dropout_seed=1)
+    q2, k2, v2, P2 = make_inputs(1, 128, 128, 1, 128, 128, 32, seed=9)
+    with pytest.raises(NotImplementedError):
+        sblocal_forward(q2.to(dev), k2.to(dev), v2.to(dev), P2.to(dev), 64, dropout_p=0.1, dropout_seed=1)
+    with pytest.raises(NotImplementedError):
+        attn(qd, kd, vd, need_weights=True)

@@ -242,3 +242,46 @@ def test_local_backward_matches_autograd_through_the_oracle(B, T, S, H, E, D, lc
         assert float((got - ref).abs().max()) < 1e-12
     if lens is not None:
         assert float(dk[1, lens[1]:].abs().max()) == 0.0 and float(dv[1, lens[1]:].abs().max()) == 0.0
+
+
+def test_dropout_multiplier_of_the_oracle_and_the_restated_hash():
+    """dropout_multiplier multiplies exp(QK - log_normalization) and nothing else (sblocal_attention.py:116-119):
+    with an all-ones multiplier the oracle is unchanged, with zeros only the low-rank part remains, the normaliser never
+    moves; a multiplier that drops one pair removes exactly that pair's exact weight times its value.  The restated
+    hash of the kernels: keeps with probability 1 - p, independent of one another to what a chi-square on pairs of
+    neighbours can see, scaled by 1 / (1 - p), all kept at p = 0, different for different seeds."""
+    g = torch.Generator().manual_seed(0)
+    B, T, S, H, E, D, lc = 2, 20, 17, 2, 8, 5, 6
+    q, k, v = (torch.randn(B, n, H, c, generator=g, dtype=torch.float64) * 0.5 for n, c in ((T, E), (S, E), (S, D)))
+    P = osb.gaussian_orthogonal_random_matrix(6, E, generator=g, dtype=torch.float64)
+    out, ln = osb.sblocal_attention(q, k, v, P, lc)
+    ones = torch.ones(B, H, T, S, dtype=torch.float64)
+    out1, ln1 = osb.sblocal_attention(q, k, v, P, lc, dropout_multiplier=ones)
+    assert torch.equal(out1, out) and torch.equal(ln1, ln)
+    one_gone = ones.clone()
+    b, h, i, s = 1, 0, 9, 10                                   # inside the band of query 9: keys 6 .. 11
+    one_gone[b, h, i, s] = 0
+    out2, ln2 = osb.sblocal_attention(q, k, v, P, lc, dropout_multiplier=one_gone)
+    t = 1 / math.sqrt(E)
+    weight = torch.exp(t * (q[b, i, h] @ k[b, s, h]) - ln[b, h, i, 0])
+    diff = out - out2
+    assert torch.equal(ln2, ln)
+    assert torch.allclose(diff[b, i, h], weight * v[b, s, h], rtol=1e-12, atol=1e-15)
+    diff[b, i, h] = 0
+    assert float(diff.abs().max()) == 0.0
+    far = ones.clone()
+    far[b, h, i, 0] = 0                                        # outside the band: no exact weight there, nothing changes
+    assert torch.equal(osb.sblocal_attention(q, k, v, P, lc, dropout_multiplier=far)[0], out)
+
+    for p in (0.1, 0.5, 0.9):
+        keep = osb.dropout_keep(2024, p, 2, 3, 300, 257)
+        kept = keep > 0
+        assert abs(float(kept.double().mean()) - (1 - p)) < 4 * math.sqrt(p * (1 - p) / kept.numel()) + 1e-4
+        assert torch.equal(keep[kept].unique(), torch.tensor([1 / (1 - p)], dtype=torch.float64))
+        # neighbouring keys and neighbouring queries: joint keep frequency = (1 - p)^2 within sampling error
+        for a_, b_ in ((kept[..., :-1], kept[..., 1:]), (kept[..., :-1, :], kept[..., 1:, :])):
+            joint = float((a_ & b_).double().mean())
+            assert abs(joint - (1 - p) ** 2) < 5 * math.sqrt((1 - p) ** 2 / a_.numel()) + 2e-3, (p, joint)
+    assert bool((osb.dropout_keep(7, 0.0, 1, 1, 10, 10) == 1).all())
+    assert not torch.equal(osb.dropout_keep(7, 0.5, 1, 2, 64, 64), osb.dropout_keep(8, 0.5, 1, 2, 64, 64))
+    assert not torch.equal(osb.dropout_keep(7, 0.5, 1, 2, 64, 64), osb.dropout_keep(7 + (1 << 40), 0.5, 1, 2, 64, 64))
