@@ -275,7 +275,21 @@ def bench_blocksparse(steps, warmup):
         o.backward(gm)
         qm.grad = km.grad = vm.grad = None
     out['module_fwd_bwd_ms'] = timeit(module_step)
-    del qm, km, vm, gm, mod
+    # ... and with the constructor's default attention dropout of 0.1 (blocksparse_attention.py:31,160): the mask
+    # is a hash formed inside the same kernels; `fuse = False` is the op-by-op chain with nn.Dropout on the
+    # stored probabilities
+    mod_drop = BlockSparseAttention(Layout(), max_seq_length=L).to(dev).train()
+
+    def module_drop_step():
+        o, _ = mod_drop(qm, km, vm)
+        o.backward(gm)
+        qm.grad = km.grad = vm.grad = None
+    out['module_dropout_fwd_bwd_ms'] = timeit(module_drop_step)
+    with torch.no_grad():
+        out['module_dropout_fwd_ms'] = timeit(lambda: mod_drop(qm, km, vm))
+    mod_drop.fuse = False
+    out['module_dropout_op_by_op_fwd_bwd_ms'] = timeit(module_drop_step)
+    del qm, km, vm, gm, mod, mod_drop
     out['fused_attention'] = {'ms': ms, 'tflops': 2 * flops / ms / 1e9, 'mfma_bf16_frac': 2 * flops / ms / 1e9 / 2500.0,
                               'speedup_over_three_stages': ms3 / ms,
                               'max_diff_vs_three_stages': float((got - ref).abs().max() / ref.abs().max())}

@@ -40,6 +40,8 @@ SIGNATURES = {
     'flyhip_bs_attn_lse': [c_vp] * 8 + [c_int, c_vp, c_i64] + [c_int] * 5 + [c_i64] * 12 + [c_float, c_int, c_vp],
     'flyhip_bs_attn_masks': [c_vp] * 8 + [c_int, c_vp, c_i64, c_vp, c_i64] + [c_int] * 5 + [c_i64] * 12 + [c_float, c_int, c_vp],
     'flyhip_bs_sdd_prob_dsoftmax': [c_vp] * 13 + [c_int] * 6 + [c_i64] * 18 + [c_float, c_int, c_vp],
+    'flyhip_bs_sdd_prob_dsoftmax_dropout': [c_vp] * 13 + [c_int] * 6 + [c_i64] * 18 + [c_float, c_int, c_float, c_u64, c_vp],
+    'flyhip_bs_attn_dropout': [c_vp] * 8 + [c_int, c_vp, c_i64, c_vp, c_i64] + [c_int] * 5 + [c_i64] * 12 + [c_float, c_int, c_float, c_u64, c_vp],
     'flyhip_bs_sdd_prob': [c_vp] * 7 + [c_int] * 6 + [c_i64] * 6 + [c_float, c_int, c_vp],
     'flyhip_bs_attn': [c_vp] * 7 + [c_int, c_vp, c_i64] + [c_int] * 5 + [c_i64] * 12 + [c_float, c_int, c_vp],
     'flyhip_bs_softmax': [c_vp] * 4 + [c_int] * 5 + [c_i64, c_float, c_vp, c_i64, c_int, c_vp, c_i64,

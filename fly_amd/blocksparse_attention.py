@@ -23,15 +23,20 @@ class _AttentionCoreFn(torch.autograd.Function):
     and the backward forms the probabilities again.  The backward runs four kernels instead of the
     op-by-op chain's six plus elementwise passes:
     dV = P^T dO, dS = scale * P * (dO V^T - rowsum(dO * O)) in one kernel (the sdd fused with the softmax
-    gradient), dQ = dS K, dK = dS^T Q.  32x32 blocks of bf16 / fp16 with shared-tile tables only."""
+    gradient), dQ = dS K, dK = dS^T Q.  32x32 blocks of bf16 / fp16 with shared-tile tables only.
+    ``dropout=(p, seed)`` (one-kernel forward only): the dropout of blocksparse_attention.py:160 with the mask
+    a hash of (seed, batch, head, query, key) that the backward kernel forms again: it writes M * P for dV and
+    dS = scale * P * (M * dO V^T - rowsum(dO * O)), M = kept / (1 - p)."""
 
     @staticmethod
-    def forward(ctx, q, k, v, sdd, dsd, sm, scale, kpm, am, fused):
-        ctx.ops, ctx.scale = (sdd, dsd), scale
+    def forward(ctx, q, k, v, sdd, dsd, sm, scale, kpm, am, fused, dropout=(0.0, 0)):
+        ctx.ops, ctx.scale, ctx.dropout = (sdd, dsd), scale, dropout
+        if dropout[0] > 0 and not (fused is not None and kpm is None and am is None):
+            raise NotImplementedError('dropout inside the kernels needs the one-kernel forward without masks')
         if fused is not None and kpm is None and am is None:
             # no masks: the one-kernel forward; it keeps the rows' log-denominators instead of the
             # probabilities, which the backward forms again (one sdd with an exponential epilogue)
-            out, lse2 = fused(q, k, v, scale, None, return_lse=True)
+            out, lse2 = fused(q, k, v, scale, None, return_lse=True, dropout=dropout)
             ctx.save_for_backward(q, k, v, out, lse2)
             ctx.recompute = True
             return out
@@ -65,14 +70,15 @@ class _AttentionCoreFn(torch.autograd.Function):
             qq, kk, vv, oo = vec(q), vec(k), vec(v), vec(out)
             dq = torch.empty(q.shape, dtype=q.dtype, device=q.device)
             with torch.cuda.device(q.device):
-                _lib.call('flyhip_bs_sdd_prob_dsoftmax', dout.data_ptr(), vv.data_ptr(), qq.data_ptr(), kk.data_ptr(),
+                _lib.call('flyhip_bs_sdd_prob_dsoftmax_dropout', dout.data_ptr(), vv.data_ptr(), qq.data_ptr(), kk.data_ptr(),
                           None, oo.data_ptr(), lse2.data_ptr(), ds.data_ptr(), p.data_ptr(), dq.data_ptr(),
                           uni_ptr.data_ptr(), uni_inner.data_ptr(), uni_blk.data_ptr(),
                           nnz, H, rows, q.shape[0], q.shape[3], 32,
                           dout.stride(0), dout.stride(1), dout.stride(2), vv.stride(0), vv.stride(1), vv.stride(2),
                           qq.stride(0), qq.stride(1), qq.stride(2), kk.stride(0), kk.stride(1), kk.stride(2),
                           dq.stride(0), dq.stride(1), dq.stride(2), oo.stride(0), oo.stride(1), oo.stride(2),
-                          float(ctx.scale), _lib.dtype_code(q), _lib.stream_ptr(q.device))
+                          float(ctx.scale), _lib.dtype_code(q), float(ctx.dropout[0]), int(ctx.dropout[1]),
+                          _lib.stream_ptr(q.device))
             dv = dsd._run('dsd', p, dout, True, False, False)
         else:
             dq = None
@@ -90,7 +96,7 @@ class _AttentionCoreFn(torch.autograd.Function):
         if dq is None:
             dq = dsd._run('dsd', ds, k, False, False, False)
         dk = dsd._run('dsd', ds, q, True, False, False)
-        return dq, dk, dv, None, None, None, None, None, None, None
+        return dq, dk, dv, None, None, None, None, None, None, None, None
 
     @staticmethod
     def supports(sdd, block, dtype, head_dim, device):
@@ -140,8 +146,8 @@ class BlockSparseAttention(nn.Module):
         self.ops_cache = dict()
         self.fused_cache = dict()
         self._layout_cache = dict()
-        # forward passes that need neither gradients, attention weights, an attention mask nor
-        # dropout run as ONE kernel (no score tensor in memory); set to False to force the three ops
+        # forward passes that need neither gradients nor attention weights run as ONE kernel (no score
+        # tensor in memory), dropout included; set to False to force the three ops
         self.fuse = True
 
     def get_layout(self, T, S=None):
@@ -199,8 +205,14 @@ class BlockSparseAttention(nn.Module):
         q, k, v = (x.permute(0, 2, 1, 3) for x in (query, key, value))
         layout = self.get_layout(T, S)
         needs_grad = torch.is_grad_enabled() and any(x.requires_grad for x in (query, key, value))
-        if (self.fuse and not need_weights and not needs_grad
-                and not (self.training and self.dropout.p > 0)
+        # training-mode dropout (:160) runs inside the kernels: the mask is a hash of (seed, batch, head, query, key),
+        # the seed drawn per call from torch's CPU generator (torch.manual_seed makes it repeatable) and kept in
+        # last_dropout_seed
+        dropout = (0.0, 0)
+        if self.training and self.dropout.p > 0:
+            dropout = (float(self.dropout.p), int(torch.randint(0, 2 ** 62, (1,)).item()))
+        self.last_dropout_seed = None                       # set where a kernel uses the seed
+        if (self.fuse and not need_weights and not needs_grad and dropout[0] < 1.0
                 and fused_attention.supports(block, query.dtype, E, value.shape[3])):
             if (T, S) not in self.fused_cache:
                 self.fused_cache[T, S] = fused_attention(layout, block)
@@ -209,22 +221,27 @@ class BlockSparseAttention(nn.Module):
                 key_mask = key_padding_mask.additive_matrix
             if attn_mask is not None and not attn_mask.all_ones:
                 add_mask = attn_mask.additive_matrix        # (T, S), read per nonzero block inside the kernel
-            out = self.fused_cache[T, S](q, k, v, softmax_temp, key_mask, attn_mask=add_mask)
+            out = self.fused_cache[T, S](q, k, v, softmax_temp, key_mask, attn_mask=add_mask, dropout=dropout)
+            self.last_dropout_seed = dropout[1] if dropout[0] > 0 else None
             return out.permute(0, 2, 1, 3)[:, :q_seqlen_og, :, :v_dim_og], None
         sdd_nt, dsd_nn, sparse_softmax = self.get_ops(T, S)
-        if (needs_grad and not need_weights and not (self.training and self.dropout.p > 0)
+        unmasked = ((key_padding_mask is None or key_padding_mask.all_ones)
+                    and (attn_mask is None or attn_mask.all_ones))
+        one_kernel = self.fuse and unmasked and fused_attention.supports(block, query.dtype, E, value.shape[3])
+        # (with masks AND dropout a training step stays on the three ops below: the backward that forms the
+        # probabilities again does not read masks)
+        if (needs_grad and not need_weights and (dropout[0] == 0.0 or (one_kernel and dropout[0] < 1.0))
                 and E == value.shape[3] and _AttentionCoreFn.supports(sdd_nt, block, query.dtype, E, query.device)):
             fused = None
-            if (self.fuse and (key_padding_mask is None or key_padding_mask.all_ones)
-                    and (attn_mask is None or attn_mask.all_ones)
-                    and fused_attention.supports(block, query.dtype, E, value.shape[3])):
+            if one_kernel:
                 if (T, S) not in self.fused_cache:
                     self.fused_cache[T, S] = fused_attention(layout, block)
                 fused = self.fused_cache[T, S]
+            self.last_dropout_seed = dropout[1] if dropout[0] > 0 else None
             out = _AttentionCoreFn.apply(
                 q, k, v, sdd_nt, dsd_nn, sparse_softmax, softmax_temp,
                 None if fused is not None or key_padding_mask is None else key_padding_mask.additive_matrix,
-                None if fused is not None or attn_mask is None else attn_mask.additive_matrix, fused)
+                None if fused is not None or attn_mask is None else attn_mask.additive_matrix, fused, dropout)
             return out.permute(0, 2, 1, 3)[:, :q_seqlen_og, :, :v_dim_og], None
         qk = sdd_nt(q, k)
         attn = sparse_softmax(qk, scale=softmax_temp,

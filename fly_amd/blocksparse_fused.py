@@ -12,8 +12,11 @@ class fused_attention:
     k / v (Z,H,cols,D) (any batch / head / row strides, D contiguous) returns
     softmax(scale * q k^T + key_mask[z, col] + attn_mask[row, col]) v over the nonzero blocks of `layout`, shaped
     (Z,H,rows,D) over memory laid out (Z,rows,H,D).  key_mask: fp32 (Z, cols), attn_mask: fp32 (rows, cols), both
-    additive (0 / -inf from the mask classes, blocksparse_attention.py:146-152).  Forward only, 32x32 blocks of
-    bf16 / fp16, D in {32,64,128}: `supports()` says whether a call qualifies."""
+    additive (0 / -inf from the mask classes, blocksparse_attention.py:146-152).  ``dropout=(p, seed)`` with p > 0
+    drops probabilities the way ``self.dropout(attn)`` of blocksparse_attention.py:160 does -- after the softmax,
+    kept ones scaled by 1 / (1 - p) -- with the mask a hash of (seed, batch, head, query, key) formed inside the
+    kernel instead of a stored tensor.  Forward only, 32x32 blocks of bf16 / fp16, D in {32,64,128}: `supports()`
+    says whether a call qualifies."""
 
     def __init__(self, layout, block, rows_per_group=8):
         self.layout = _as_layout3(layout)
@@ -32,7 +35,7 @@ class fused_attention:
             self.lut_cache[device] = tuple(t.to(device) for t in union_table(self.layout, self.rows_per_group))
         return self.lut_cache[device]
 
-    def __call__(self, q, k, v, scale, key_mask=None, return_lse=False, attn_mask=None):
+    def __call__(self, q, k, v, scale, key_mask=None, return_lse=False, attn_mask=None, dropout=(0.0, 0)):
         _lib.require_gpu(q, k, v)
         H, p, r = self.spdims
         Z, D = q.shape[0], q.shape[3]
@@ -69,11 +72,18 @@ class fused_attention:
         # base-2 log of every row's softmax denominator (+inf for a row without a finite score): what a
         # backward pass needs to form the probabilities again
         lse2 = torch.empty((Z, H, p * 32), dtype=torch.float32, device=q.device) if return_lse else None
+        drop_p, drop_seed = float(dropout[0]), int(dropout[1])
+        if not 0.0 <= drop_p < 1.0:
+            raise ValueError(f'dropout probability {drop_p} not in [0, 1)')
         with torch.cuda.device(q.device):
-            _lib.call('flyhip_bs_attn_masks', q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), _lib.ptr(lse2),
+            common = (q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), _lib.ptr(lse2),
                       uni_ptr.data_ptr(), uni_inner.data_ptr(), uni_blk.data_ptr(), self.rows_per_group,
                       km, km_stride, am, am_stride, Z, H, p, D, 32,
                       q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
                       v.stride(0), v.stride(1), v.stride(2), out.stride(0), out.stride(1), out.stride(2),
-                      float(scale), _lib.dtype_code(q), _lib.stream_ptr(q.device))
+                      float(scale), _lib.dtype_code(q))
+            if drop_p > 0.0:
+                _lib.call('flyhip_bs_attn_dropout', *common, drop_p, drop_seed, _lib.stream_ptr(q.device))
+            else:
+                _lib.call('flyhip_bs_attn_masks', *common, _lib.stream_ptr(q.device))
         return (out, lse2) if return_lse else out

@@ -225,10 +225,15 @@ struct SddUniArgs {
     // ... with delta formed here when `out` is given (delta may then be null): rowsum(a * out), out laid out like a
     const void* out; long o_sz, o_sh, o_sm;
     int n_xcd;          // dies the dispatcher deals workgroup ids to (set where the kernel is launched)
+    // EPI 3 with DROP: the forward dropped probabilities by the hash of (seed, row = (z H + head) L + query, key)
+    // (drop_keep): p2 is then written with the dropped ones zeroed and the kept ones scaled by 1 / (1 - p) -- the
+    // operand of dV -- and c = scale * p * (m * (a b^T) - delta[row]) with m that 0 or 1 / (1 - p)
+    uint32_t drop_seed, drop_thresh; float drop_scale;
 };
 
-template <typename T, int KS, int EPI = 0>     // KS = K / 32; EPI: 0 product, 1 softmax gradient, 2 probabilities
+template <typename T, int KS, int EPI = 0, bool DROP = false>     // KS = K / 32; EPI: 0 product, 1 softmax gradient, 2 probabilities
 __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
+    static_assert(!DROP || EPI == 3, "dropout belongs to the epilogue that forms the probabilities again");
     constexpr bool DSOFT = EPI == 1, PROB = EPI == 2, BOTH = EPI == 3;
     constexpr int K = 32 * KS, LD = K + 8;              // LDS row stride: 16 rows of a tile hit all banks once
     constexpr int CPR = K / 8;                          // 16-byte chunks per tile row
@@ -301,6 +306,12 @@ __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
         }
         bz2 = reinterpret_cast<const T*>(a.b2) + z * a.b2_sz + head * a.b2_sh;
     }
+    uint32_t drop_row[2] = {0u, 0u};
+    if (DROP) {
+        const uint32_t row0 = (uint32_t)rowvec_off;     // (z H + head) L + 32 bi + r16
+        drop_row[0] = drop_row_hash(a.drop_seed, row0);
+        drop_row[1] = drop_row_hash(a.drop_seed, row0 + 16u);
+    }
 
     // staging: chunk c = tid + 256 i is 16 bytes of tile row c / CPR.  Block column n lands in LDS row
     // 16*((n>>2)&1) + 4*(n>>3) + (n&3), so that MFMA tile tn reads the 16 consecutive LDS rows
@@ -334,7 +345,8 @@ __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
     // the index lists are read two steps (block-column) and one step (block id) ahead of their use
     int inner_n1 = n > 1 ? a.uni_inner[p0 + 1] : 0;
     int blk = a.uni_blk[(long)p0 * 4 + w];
-    fetch(a.uni_inner[p0]);
+    int inner_cur = a.uni_inner[p0];
+    fetch(inner_cur);
     stash(0);
     drain_loads();
     __syncthreads();
@@ -411,8 +423,15 @@ __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
 #pragma unroll
                         for (int i = 0; i < 4; ++i) {
                             const float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(acc2[tm][tn][i], a.scale2, -lse_row[tm]));
-                            acc2[tm][tn][i] = pr;
-                            acc[tm][tn][i] = a.scale * pr * (acc[tm][tn][i] - dl_row[tm]);
+                            if (DROP) {
+                                const uint32_t col = (uint32_t)inner_cur * 32u + 8u * g + 4u * tn + i;
+                                const float m = drop_keep(drop_row[tm], col, a.drop_thresh) ? a.drop_scale : 0.f;
+                                acc2[tm][tn][i] = m * pr;
+                                acc[tm][tn][i] = a.scale * pr * (m * acc[tm][tn][i] - dl_row[tm]);
+                            } else {
+                                acc2[tm][tn][i] = pr;
+                                acc[tm][tn][i] = a.scale * pr * (acc[tm][tn][i] - dl_row[tm]);
+                            }
                         }
                     T* pp2 = reinterpret_cast<T*>(a.p2) + ((long)z * a.nnz + blk) * 1024;
                     store8_f32(pp2 + (16 * tm + r16) * 32 + 8 * g, acc2[tm][0], acc2[tm][1]);
@@ -442,6 +461,7 @@ __global__ __launch_bounds__(256) void bs_sdd32u_kernel(const SddUniArgs a) {
                 store8_f32(cp + (16 * tm + r16) * 32 + 8 * g, acc[tm][0], acc[tm][1]);
             }
         }
+        inner_cur = inner_n1;
         inner_n1 = inner_n2;
         blk = blk_n1;
         __syncthreads();
@@ -1327,6 +1347,9 @@ struct AttnArgs {
     float* lse2;        // optional (Z, H, 32 * brows_per_head): base-2 log of every row's softmax denominator
     int n_xcd;          // dies the dispatcher deals workgroup ids to (set where the kernel is launched)
     const float* am; long am_stride;     // optional (rows, cols) additive term per (query, key), shared by batch and heads
+    // dropout of the probabilities (DROP kernels): element (z, head, query, key) is kept when the hash of
+    // (seed, row = (z H + head) L + query, key) reaches the threshold; kept ones are scaled by 1 / (1 - p)
+    uint32_t drop_seed, drop_thresh; float drop_scale;
 };
 
 // Maxima of scores.  A two-operand fmaxf costs three instructions here (each operand is first quieted
@@ -1357,8 +1380,9 @@ template <int CPR> __device__ __forceinline__ int attn_vslot(int row, int c) {
     constexpr int RPL = CPR >= 8 ? 1 : 8 / CPR;
     return c ^ ((((row / RPL) & 3) & (CPR / 2 - 1)) << 1);
 }
-template <typename T, int KS, int NW, bool MASKED>     // head dim 32*KS, NW block-rows (waves) per workgroup
+template <typename T, int KS, int NW, bool MASKED, bool DROP = false>     // head dim 32*KS, NW block-rows (waves) per workgroup
 __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
+    static_assert(!DROP || MASKED, "the dropout variant is built on the general (masked) softmax");
     constexpr int D = 32 * KS, DT = D / 16, RB = 2 * D;   // RB: bytes of a tile row
     // block-columns per step: what 64 KB of LDS hold twice over -- half of that for workgroups of four waves at 64 dims,
     // of which a compute unit then holds four (the registers allow it) instead of two
@@ -1425,6 +1449,13 @@ __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
     floatx4 sc[2][2];
     floatx4 amk[2][2];                                    // the attention-mask entries of sc (asked for with the scores)
     const float* amrow = (MASKED && a.am) ? a.am + (long)(min(bi, a.brows_per_head - 1) * 32 + r16) * a.am_stride + 4 * g : nullptr;
+    uint32_t drop_row[2] = {0u, 0u};                      // DROP: hash of (seed, global row) of the lane's two queries
+    if (DROP) {
+        const uint32_t row0 = (uint32_t)(z * a.n_heads + head) * (uint32_t)(a.brows_per_head * 32) +
+                              (uint32_t)(min(bi, a.brows_per_head - 1) * 32 + r16);
+        drop_row[0] = drop_row_hash(a.drop_seed, row0);
+        drop_row[1] = drop_row_hash(a.drop_seed, row0 + 16u);
+    }
     auto score = [&](const char* tile, int inner) __attribute__((always_inline)) {
         if (MASKED && amrow) {
 #pragma unroll
@@ -1459,7 +1490,7 @@ __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
             const char* p0 = vp + 16 * attn_vslot<CPR>(vrow, 2 * dt + ((r16 & 3) >> 1));
             fv[dt] = lds_read_tr8(p0, p0 + 16 * RB);
         }
-        uintx4 pb[2];
+        uintx4 pb[2], pd[2];                              // probabilities, and (DROP) the kept ones
         if (!MASKED) {
             // scale > 0 and no mask: the maximum is taken on the raw scores and the scale rides in
             // the exponent's fma
@@ -1514,6 +1545,16 @@ __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
                     e1[i] = __builtin_amdgcn_exp2f(t1[i] - mref);
                 }
                 pb[qt] = uintx4{pack2<T>(e0[0], e0[1]), pack2<T>(e0[2], e0[3]), pack2<T>(e1[0], e1[1]), pack2<T>(e1[2], e1[3])};
+                if (DROP) {
+                    // the dropped probabilities go to the product with V only: the denominator below sums all of them
+                    const uint32_t col0 = (uint32_t)inner * 32u + 4u * g;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        if (!drop_keep(drop_row[qt], col0 + i, a.drop_thresh)) e0[i] = 0.f;
+                        if (!drop_keep(drop_row[qt], col0 + 16u + i, a.drop_thresh)) e1[i] = 0.f;
+                    }
+                    pd[qt] = uintx4{pack2<T>(e0[0], e0[1]), pack2<T>(e0[2], e0[3]), pack2<T>(e1[0], e1[1]), pack2<T>(e1[2], e1[3])};
+                }
             }
         }
         // the row sums come from the matrix pipe as well: a row of ones times the rounded probabilities
@@ -1521,8 +1562,8 @@ __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
         lsum[1] = mma32<T>(ones, pb[1], lsum[1]);
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
-            o[dt][0] = mma32<T>(fv[dt], pb[0], o[dt][0]);
-            o[dt][1] = mma32<T>(fv[dt], pb[1], o[dt][1]);
+            o[dt][0] = mma32<T>(fv[dt], DROP ? pd[0] : pb[0], o[dt][0]);
+            o[dt][1] = mma32<T>(fv[dt], DROP ? pd[1] : pb[1], o[dt][1]);
         }
     };
 
@@ -1577,7 +1618,8 @@ __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
 #pragma unroll
     for (int qt = 0; qt < 2; ++qt) {
         const float l = lsum[qt][0];
-        const float inv = l > 0.f ? 1.0f / l : 0.f;       // rows without a finite score come out as zeros
+        float inv = l > 0.f ? 1.0f / l : 0.f;             // rows without a finite score come out as zeros
+        if (DROP) inv *= a.drop_scale;
         T* row = op + ((long)bi * 32 + 16 * qt + r16) * a.o_sm + 4 * g;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) store4_f32(row + 16 * dt, o[dt][qt] * inv);
@@ -2042,6 +2084,22 @@ static int launch_sdd_epilogue(const char* what, const void* a_dn, const void* b
         case 3: hipLaunchKernelGGL((bs_sdd32u_kernel<T, 3, EPI>), grid, dim3(256), 0, st, ua); break;  \
         default: hipLaunchKernelGGL((bs_sdd32u_kernel<T, 4, EPI>), grid, dim3(256), 0, st, ua); break; \
     }
+    if constexpr (EPI == 3) {
+        if (second->drop_thresh != 0u) {
+            ua.drop_seed = second->drop_seed; ua.drop_thresh = second->drop_thresh; ua.drop_scale = second->drop_scale;
+            FLY_REQUIRE((long)Z * n_heads * brows_per_head * 32 <= 4294967295L, "%s: more than 2^32 rows", what);
+#define SDDS_DROP_LAUNCH(T)                                                                                   \
+    switch (K / 32) {                                                                                         \
+        case 1: hipLaunchKernelGGL((bs_sdd32u_kernel<T, 1, 3, true>), grid, dim3(256), 0, st, ua); break;    \
+        case 2: hipLaunchKernelGGL((bs_sdd32u_kernel<T, 2, 3, true>), grid, dim3(256), 0, st, ua); break;    \
+        case 3: hipLaunchKernelGGL((bs_sdd32u_kernel<T, 3, 3, true>), grid, dim3(256), 0, st, ua); break;    \
+        default: hipLaunchKernelGGL((bs_sdd32u_kernel<T, 4, 3, true>), grid, dim3(256), 0, st, ua); break;   \
+    }
+            if (dtype == BF16) { SDDS_DROP_LAUNCH(bf16_t) } else { SDDS_DROP_LAUNCH(f16_t) }
+#undef SDDS_DROP_LAUNCH
+            return check_launch(what);
+        }
+    }
     if (dtype == BF16) { SDDS_LAUNCH(bf16_t) } else { SDDS_LAUNCH(f16_t) }
 #undef SDDS_LAUNCH
     return check_launch(what);
@@ -2057,6 +2115,18 @@ extern "C" int flyhip_bs_sdd_dsoftmax(const void* dout, const void* v, const voi
                                   brows_per_head, Z, K, blk, a_sz, a_sh, a_sm, b_sz, b_sh, b_sn, scale, dtype, stream);
 }
 
+extern "C" int flyhip_bs_sdd_prob_dsoftmax_dropout(const void* dout, const void* v, const void* q, const void* k,
+                                           const float* delta, const void* out, const float* lse2, void* ds, void* p, void* dq,
+                                           const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
+                                           int nnz, int n_heads, int brows_per_head, int Z, int K, int blk,
+                                           int64_t do_sz, int64_t do_sh, int64_t do_sm,
+                                           int64_t v_sz, int64_t v_sh, int64_t v_sn,
+                                           int64_t q_sz, int64_t q_sh, int64_t q_sm,
+                                           int64_t k_sz, int64_t k_sh, int64_t k_sn,
+                                           int64_t dq_sz, int64_t dq_sh, int64_t dq_sm,
+                                           int64_t o_sz, int64_t o_sh, int64_t o_sm,
+                                           float scale, int dtype, float dropout_p, uint64_t dropout_seed, void* stream);
+
 extern "C" int flyhip_bs_sdd_prob_dsoftmax(const void* dout, const void* v, const void* q, const void* k,
                                            const float* delta, const void* out, const float* lse2, void* ds, void* p, void* dq,
                                            const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
@@ -2068,7 +2138,27 @@ extern "C" int flyhip_bs_sdd_prob_dsoftmax(const void* dout, const void* v, cons
                                            int64_t dq_sz, int64_t dq_sh, int64_t dq_sm,
                                            int64_t o_sz, int64_t o_sh, int64_t o_sm,
                                            float scale, int dtype, void* stream) {
+    return flyhip_bs_sdd_prob_dsoftmax_dropout(dout, v, q, k, delta, out, lse2, ds, p, dq, uni_ptr, uni_inner, uni_blk, nnz,
+                                               n_heads, brows_per_head, Z, K, blk, do_sz, do_sh, do_sm, v_sz, v_sh, v_sn,
+                                               q_sz, q_sh, q_sm, k_sz, k_sh, k_sn, dq_sz, dq_sh, dq_sm, o_sz, o_sh, o_sm,
+                                               scale, dtype, 0.f, 0, stream);
+}
+
+extern "C" int flyhip_bs_sdd_prob_dsoftmax_dropout(const void* dout, const void* v, const void* q, const void* k,
+                                           const float* delta, const void* out, const float* lse2, void* ds, void* p, void* dq,
+                                           const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
+                                           int nnz, int n_heads, int brows_per_head, int Z, int K, int blk,
+                                           int64_t do_sz, int64_t do_sh, int64_t do_sm,
+                                           int64_t v_sz, int64_t v_sh, int64_t v_sn,
+                                           int64_t q_sz, int64_t q_sh, int64_t q_sm,
+                                           int64_t k_sz, int64_t k_sh, int64_t k_sn,
+                                           int64_t dq_sz, int64_t dq_sh, int64_t dq_sm,
+                                           int64_t o_sz, int64_t o_sh, int64_t o_sm,
+                                           float scale, int dtype, float dropout_p, uint64_t dropout_seed, void* stream) {
+    FLY_REQUIRE(dropout_p >= 0.f && dropout_p < 1.f, "bs_sdd_prob_dsoftmax: dropout_p %g not in [0, 1)", (double)dropout_p);
     SddUniArgs second{};
+    const DropArgs drop = drop_args(dropout_p, dropout_seed);
+    second.drop_seed = drop.seed; second.drop_thresh = drop.thresh; second.drop_scale = drop.scale;
     second.out = out; second.o_sz = o_sz; second.o_sh = o_sh; second.o_sm = o_sm;
     second.dq = dq; second.dq_sz = dq_sz; second.dq_sh = dq_sh; second.dq_sm = dq_sm;
     second.a2 = q; second.b2 = k; second.lse2 = lse2; second.p2 = p; second.scale2 = scale * 1.4426950408889634f;
@@ -2266,7 +2356,7 @@ static int launch_softmax(const RowArgs& args, dim3 grid, int max_elems, hipStre
     return check_launch("bs_softmax_kernel");
 }
 
-extern "C" int flyhip_bs_attn_masks(const void* q, const void* k, const void* v, void* out, float* lse2,
+static int bs_attn_checked(const void* q, const void* k, const void* v, void* out, float* lse2,
                               const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
                               int rows_per_group, const float* key_mask, int64_t key_mask_stride,
                               const float* attn_mask, int64_t attn_mask_stride,
@@ -2275,7 +2365,7 @@ extern "C" int flyhip_bs_attn_masks(const void* q, const void* k, const void* v,
                               int64_t k_sz, int64_t k_sh, int64_t k_sn,
                               int64_t v_sz, int64_t v_sh, int64_t v_sn,
                               int64_t o_sz, int64_t o_sh, int64_t o_sm,
-                              float scale, int dtype, void* stream) {
+                              float scale, int dtype, void* stream, DropArgs drop) {
     int rc = check_common("bs_attn", blk, dtype, Z);
     if (rc) return rc;
     FLY_REQUIRE(q && k && v && out && uni_ptr && uni_inner && uni_blk, "bs_attn: null pointer");
@@ -2300,9 +2390,14 @@ extern "C" int flyhip_bs_attn_masks(const void* q, const void* k, const void* v,
     FLY_REQUIRE(nwg <= 2147483647L, "bs_attn: too many workgroups");
     dim3 grid((unsigned)nwg);
     const bool masked = key_mask != nullptr || attn_mask != nullptr || !(scale > 0.f);
+    const bool dropping = drop.thresh != 0u;
+    args.drop_seed = drop.seed;
+    args.drop_thresh = drop.thresh;
+    args.drop_scale = drop.scale;
 #define ATTN_LAUNCH(T, KS, NW)                                                                                  \
     do {                                                                                                        \
-        if (masked) hipLaunchKernelGGL((bs_attn32_kernel<T, KS, NW, true>), grid, dim3(64 * NW), 0, st, args);  \
+        if (dropping) hipLaunchKernelGGL((bs_attn32_kernel<T, KS, NW, true, true>), grid, dim3(64 * NW), 0, st, args); \
+        else if (masked) hipLaunchKernelGGL((bs_attn32_kernel<T, KS, NW, true>), grid, dim3(64 * NW), 0, st, args);  \
         else hipLaunchKernelGGL((bs_attn32_kernel<T, KS, NW, false>), grid, dim3(64 * NW), 0, st, args);        \
     } while (0)
 #define ATTN_KS(T, NW) do { if (D == 32) ATTN_LAUNCH(T, 1, NW); else if (D == 64) ATTN_LAUNCH(T, 2, NW); else ATTN_LAUNCH(T, 4, NW); } while (0)
@@ -2311,6 +2406,38 @@ extern "C" int flyhip_bs_attn_masks(const void* q, const void* k, const void* v,
 #undef ATTN_KS
 #undef ATTN_LAUNCH
     return check_launch("bs_attn32_kernel");
+}
+
+extern "C" int flyhip_bs_attn_masks(const void* q, const void* k, const void* v, void* out, float* lse2,
+                              const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
+                              int rows_per_group, const float* key_mask, int64_t key_mask_stride,
+                              const float* attn_mask, int64_t attn_mask_stride,
+                              int Z, int H, int brows_per_head, int D, int blk,
+                              int64_t q_sz, int64_t q_sh, int64_t q_sm,
+                              int64_t k_sz, int64_t k_sh, int64_t k_sn,
+                              int64_t v_sz, int64_t v_sh, int64_t v_sn,
+                              int64_t o_sz, int64_t o_sh, int64_t o_sm,
+                              float scale, int dtype, void* stream) {
+    return bs_attn_checked(q, k, v, out, lse2, uni_ptr, uni_inner, uni_blk, rows_per_group, key_mask, key_mask_stride,
+                           attn_mask, attn_mask_stride, Z, H, brows_per_head, D, blk, q_sz, q_sh, q_sm, k_sz, k_sh, k_sn,
+                           v_sz, v_sh, v_sn, o_sz, o_sh, o_sm, scale, dtype, stream, DropArgs{0u, 0u, 1.f});
+}
+
+extern "C" int flyhip_bs_attn_dropout(const void* q, const void* k, const void* v, void* out, float* lse2,
+                              const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
+                              int rows_per_group, const float* key_mask, int64_t key_mask_stride,
+                              const float* attn_mask, int64_t attn_mask_stride,
+                              int Z, int H, int brows_per_head, int D, int blk,
+                              int64_t q_sz, int64_t q_sh, int64_t q_sm,
+                              int64_t k_sz, int64_t k_sh, int64_t k_sn,
+                              int64_t v_sz, int64_t v_sh, int64_t v_sn,
+                              int64_t o_sz, int64_t o_sh, int64_t o_sm,
+                              float scale, int dtype, float dropout_p, uint64_t dropout_seed, void* stream) {
+    FLY_REQUIRE(dropout_p >= 0.f && dropout_p < 1.f, "bs_attn_dropout: dropout_p %g not in [0, 1)", (double)dropout_p);
+    FLY_REQUIRE((long)Z * H * brows_per_head * 32 <= 4294967295L, "bs_attn_dropout: more than 2^32 rows");
+    return bs_attn_checked(q, k, v, out, lse2, uni_ptr, uni_inner, uni_blk, rows_per_group, key_mask, key_mask_stride,
+                           attn_mask, attn_mask_stride, Z, H, brows_per_head, D, blk, q_sz, q_sh, q_sm, k_sz, k_sh, k_sn,
+                           v_sz, v_sh, v_sn, o_sz, o_sh, o_sm, scale, dtype, stream, drop_args(dropout_p, dropout_seed));
 }
 
 extern "C" int flyhip_bs_attn_lse(const void* q, const void* k, const void* v, void* out, float* lse2,

@@ -472,6 +472,25 @@ int flyhip_bs_attn_masks(const void* q, const void* k, const void* v, void* out,
                          int64_t o_sz, int64_t o_sh, int64_t o_sm,
                          float scale, int dtype, void* stream);
 
+/* flyhip_bs_attn_masks with the dropout of BlockSparseAttention.forward (ref:
+ * src/models/attention/blocksparse_attention.py:160, `dsd_nn(self.dropout(attn), v)`; the constructor's default
+ * attention_dropout is 0.1, :31): every probability is dropped with probability dropout_p in [0, 1) after the softmax
+ * (the denominator sums all of them) and the kept ones are scaled by 1 / (1 - dropout_p).  No mask tensor exists:
+ * (batch z, head h, query i, key j) is kept iff mix(mix(((z H + h) L + i) * 0x9E3779B1 + s) + j * 0x632BE5AB) >=
+ * floor(dropout_p 2^32), L = 32 * brows_per_head, mix = the 32-bit finaliser of MurmurHash3, s = the 64-bit seed
+ * folded to 32 bits (low ^ high * 0x9E3779B1); flyhip_bs_sdd_prob_dsoftmax_dropout forms the same mask again.
+ * lse2 is that of the undropped softmax.  dropout_p = 0 is flyhip_bs_attn_masks. */
+int flyhip_bs_attn_dropout(const void* q, const void* k, const void* v, void* out, float* lse2,
+                           const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
+                           int rows_per_group, const float* key_mask, int64_t key_mask_stride,
+                           const float* attn_mask, int64_t attn_mask_stride,
+                           int Z, int H, int brows_per_head, int D, int blk,
+                           int64_t q_sz, int64_t q_sh, int64_t q_sm,
+                           int64_t k_sz, int64_t k_sh, int64_t k_sn,
+                           int64_t v_sz, int64_t v_sh, int64_t v_sn,
+                           int64_t o_sz, int64_t o_sh, int64_t o_sm,
+                           float scale, int dtype, float dropout_p, uint64_t dropout_seed, void* stream);
+
 /* The probabilities of that attention again, in the block-sparse format: p = exp(scale * q k^T - lse) on
  * the nonzero blocks, as one sdd (blocksparse_matmul.py:279-346) with an exponential epilogue;
  * lse2 as written by flyhip_bs_attn_lse; tables as for flyhip_bs_sdd's shared-tile path (four
@@ -501,6 +520,23 @@ int flyhip_bs_sdd_prob_dsoftmax(const void* dout, const void* v, const void* q, 
                                 int64_t dq_sz, int64_t dq_sh, int64_t dq_sm,
                                 int64_t o_sz, int64_t o_sh, int64_t o_sm,
                                 float scale, int dtype, void* stream);
+
+/* flyhip_bs_sdd_prob_dsoftmax for a forward that dropped probabilities (flyhip_bs_attn_dropout with the same
+ * dropout_p, dropout_seed and shapes): with m = 0 on dropped pairs and 1 / (1 - dropout_p) on kept ones, p receives
+ * m * p -- the operand of dv = (m p)^T d out -- and ds = scale * p * (m * d out v^T - delta[row]); delta =
+ * rowsum(d out * out) as before (out being the dropped forward's result).  The chain is the one autograd builds
+ * through blocksparse_attention.py:146-160 with nn.Dropout's mask kept. */
+int flyhip_bs_sdd_prob_dsoftmax_dropout(const void* dout, const void* v, const void* q, const void* k,
+                                const float* delta, const void* out, const float* lse2, void* ds, void* p, void* dq,
+                                const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
+                                int nnz, int n_heads, int brows_per_head, int Z, int K, int blk,
+                                int64_t do_sz, int64_t do_sh, int64_t do_sm,
+                                int64_t v_sz, int64_t v_sh, int64_t v_sn,
+                                int64_t q_sz, int64_t q_sh, int64_t q_sm,
+                                int64_t k_sz, int64_t k_sh, int64_t k_sn,
+                                int64_t dq_sz, int64_t dq_sh, int64_t dq_sm,
+                                int64_t o_sz, int64_t o_sh, int64_t o_sm,
+                                float scale, int dtype, float dropout_p, uint64_t dropout_seed, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Block-sparse row operations.  row_ptr (n_brow+1) / row_blk / row_col int32: for every

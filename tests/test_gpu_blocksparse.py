@@ -722,6 +722,66 @@ def test_blocksparse_attention_gradients_with_fully_masked_rows(dtype, dropout):
             assert rel_err(got, want) <= 1e-4, rel_err(got, want)
 
 
+@pytest.mark.parametrize('E,dtype,p_drop', [(64, torch.bfloat16, 0.25), (32, torch.float16, 0.1), (128, torch.bfloat16, 0.5)])
+def test_blocksparse_attention_dropout_inside_the_kernels(E, dtype, p_drop):
+    """Training-mode dropout of BlockSparseAttention (blocksparse_attention.py:160, constructor default 0.1) on the
+    one-kernel forward and the recomputing backward: the mask is a hash of (seed, batch, head, query, key), restated
+    on the host (oracle.sblocal.dropout_keep), so output and gradients are compared with float64 autograd through
+    softmax -> mask / (1 - p) -> product on the kernels' own mask.  The reference draws its mask from torch's
+    generator; independent keeps with probability 1 - p are what both share."""
+    from fly_amd import BlockSparseAttention
+    from oracle.sblocal import dropout_keep
+
+    class Cfg:
+        block = 32
+
+        def make_layout(self, seqlen):
+            nb = seqlen // self.block
+            lay = ob.band_layout(nb, nb, 2)
+            lay[:, 0] = 1
+            lay[5, :] = 1
+            return lay.unsqueeze(0).repeat(2, 1, 1)
+
+    B, T, H = 2, 352, 2
+    print('case', E, dtype, p_drop, flush=True)
+    g = torch.Generator().manual_seed(21)
+    q, k, v = (torch.randn(B, T, H, E, generator=g).to(dtype) for _ in range(3))
+    w = torch.randn(B, T, H, E, generator=g)
+    mod = BlockSparseAttention(Cfg(), attention_dropout=p_drop, max_seq_length=T).to(DEV).train()
+    qg, kg, vg = (x.to(DEV).requires_grad_() for x in (q, k, v))
+    torch.manual_seed(5)
+    out, _ = mod(qg, kg, vg)
+    seed = mod.last_dropout_seed
+    assert seed is not None and len(mod.fused_cache) == 1 and len(mod.ops_cache) == 1
+    (out.float() * w.to(DEV)).sum().backward()
+
+    qd, kd, vd = (x.double().requires_grad_() for x in (q, k, v))
+    lay = ob.densify_tensor(torch.ones(1, int(mod.master_layout.sum()), 32, 32), mod.master_layout.cpu())[0].bool()
+    s = torch.einsum('bthe,bshe->bhts', qd, kd) / math.sqrt(E)
+    prob = torch.softmax(s.masked_fill(~lay.unsqueeze(0), float('-inf')), -1)
+    mult = dropout_keep(seed, p_drop, B, H, T, T)
+    kept = float((mult > 0)[:, lay].double().mean())
+    assert abs(kept - (1 - p_drop)) < 0.01, kept
+    ref = torch.einsum('bhts,bshd->bthd', prob * mult, vd)
+    (ref * w.double()).sum().backward()
+    tol = 2e-2 if dtype == torch.bfloat16 else 4e-3
+    assert rel_err(out, ref) <= tol, rel_err(out, ref)
+    for got, want, name in ((qg.grad, qd.grad, 'dq'), (kg.grad, kd.grad, 'dk'), (vg.grad, vd.grad, 'dv')):
+        assert rel_err(got.float(), want) <= 1.5 * tol, (name, rel_err(got.float(), want))
+    # without gradients the same module call is the same kernel with the same mask for the same seed
+    torch.manual_seed(5)
+    with torch.no_grad():
+        again, _ = mod(qg, kg, vg)
+    assert mod.last_dropout_seed == seed and torch.equal(again, out.detach())
+    # another seed, another mask; evaluation mode: none
+    with torch.no_grad():
+        other, _ = mod(qg, kg, vg)
+        plain, _ = mod.eval()(qg, kg, vg)
+    assert mod.last_dropout_seed is None
+    assert rel_err(other, ref) > 0.1
+    assert rel_err(plain, torch.einsum('bhts,bshd->bthd', prob, vd).detach()) <= tol
+
+
 def test_probabilities_from_log_denominators():
     """flyhip_bs_attn_lse + flyhip_bs_sdd_prob: the one-kernel attention's per-row log-denominators
     turn an sdd into the softmax probabilities (what the training path's backward starts from); against
