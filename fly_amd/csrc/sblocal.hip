@@ -2445,6 +2445,9 @@ struct LocalArgs {
     float temp;
     float* lse;                     // optional (B, H, T): log of the softmax denominator, for the backward pass
     int n_xcd;                      // dies the dispatcher deals workgroup ids to (set at launch)
+    // dropout of the probabilities (drop_thresh != 0): pair (query i, key s) of (b, h) is kept when the hash of
+    // (seed, row = (b H + h) T + i, s) reaches the threshold, and scaled by 1 / (1 - p); the denominator sums all
+    uint32_t drop_seed, drop_thresh; float drop_scale;
 };
 
 template <typename T, int E, int D>
@@ -2491,6 +2494,7 @@ __global__ __launch_bounds__(NT) void local_fwd_kernel(LocalArgs a) {
     const int qw0 = q0 + 16 * w;
     const int smin = max(iq - lc_lo, 0);
     const unsigned span = qvalid ? (unsigned)max(min(iq + lc_hi, len) - smin, 0) : 0u;
+    const uint32_t drop_row = a.drop_thresh != 0u ? drop_row_hash(a.drop_seed, (uint32_t)(bh * a.T + iq)) : 0u;
     if (kt_lo < kt_hi) {
         rk.template stash<LDK>(smem, tid);
         rv.template stash<LDV>(smem + TK * LDK, tid);
@@ -2549,6 +2553,13 @@ __global__ __launch_bounds__(NT) void local_fwd_kernel(LocalArgs a) {
                     p[kb][i] = ok[kb][i] ? __builtin_amdgcn_exp2f(s1[kb][i] - m_run) : 0.f;
                     ze += p[kb][i];
                 }
+            if (a.drop_thresh != 0u) {                   // (uniform) dropped weights leave the product, not the denominator
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        if (!drop_keep(drop_row, (uint32_t)(s_base + 16 * kb + 4 * g + i), a.drop_thresh)) p[kb][i] = 0.f;
+            }
 #pragma unroll
             for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
@@ -2567,7 +2578,7 @@ __global__ __launch_bounds__(NT) void local_fwd_kernel(LocalArgs a) {
     }
     ze = group_sum(ze);
     if (qvalid) {
-        const float inv = ze > 0.f ? 1.0f / ze : 0.f;
+        const float inv = (ze > 0.f ? 1.0f / ze : 0.f) * (a.drop_thresh != 0u ? a.drop_scale : 1.0f);
         T* optr = reinterpret_cast<T*>(a.out) + b * a.o_sb + h * a.o_sh + (long)iq * a.o_ss;
 #pragma unroll
         for (int db = 0; db < DB; ++db) store4_f32(optr + 16 * db + 4 * g, oacc[db] * inv);
@@ -3920,6 +3931,10 @@ struct BwdArgs {
     // finishing pass: global low-rank terms and the chain rule through the feature map in the epilogue
     const float* gmat; const float* gvec; const float* proj;
     int n_xcd;                      // dies the dispatcher deals workgroup ids to (set at launch)
+    // dropout of the exact weights in the forward (drop_thresh != 0): with m = 0 on dropped pairs (the hash of
+    // (seed, (b H + h) T + query, key), see drop_keep) and 1 / (1 - p) on kept ones, dm = a (m g.v - c) and the
+    // weight of g in d v is m a - kb
+    uint32_t drop_seed, drop_thresh; float drop_scale;
 };
 
 //
@@ -4005,6 +4020,7 @@ __global__ __launch_bounds__(NT) void sblocal_bwd_band_kernel(BwdArgs a) {
     // inner rows this lane's outer row may meet: nmin <= n < nmin + span
     const int nmin = max(o + lo, 0);
     const unsigned span = ovalid ? (unsigned)max(min(o + hi, n_limit) - nmin, 0) : 0u;
+    const uint32_t drop_row = (!KEYMAJOR && a.drop_thresh != 0u) ? drop_row_hash(a.drop_seed, (uint32_t)(bh * a.T + o)) : 0u;
 
     floatx4 acc1[EC], acc2[FC], acc3[KEYMAJOR ? DB : 1];
 #pragma unroll
@@ -4078,9 +4094,16 @@ __global__ __launch_bounds__(NT) void sblocal_bwd_band_kernel(BwdArgs a) {
                     const bool ok = (unsigned)(n - nmin) < span;
                     const float av = ok ? __builtin_amdgcn_exp2f(s1[kb][i] - (KEYMAJOR ? lnq[i] : ln_o)) : 0.f;
                     const float df = ok ? s3[kb][i] - (KEYMAJOR ? cq[i] : c_o) : 0.f;
-                    wdm[kb][i] = av * df;
                     wdf[kb][i] = df;
-                    wak[kb][i] = av - (ok ? s2[kb][i] : 0.f);
+                    if (a.drop_thresh != 0u) {               // (uniform)
+                        const uint32_t rh = KEYMAJOR ? drop_row_hash(a.drop_seed, (uint32_t)(bh * a.T + n)) : drop_row;
+                        const float m = drop_keep(rh, (uint32_t)(KEYMAJOR ? o : n), a.drop_thresh) ? a.drop_scale : 0.f;
+                        wdm[kb][i] = ok ? av * (m * s3[kb][i] - (KEYMAJOR ? cq[i] : c_o)) : 0.f;
+                        wak[kb][i] = av * m - (ok ? s2[kb][i] : 0.f);
+                    } else {
+                        wdm[kb][i] = av * df;
+                        wak[kb][i] = av - (ok ? s2[kb][i] : 0.f);
+                    }
                 }
             }
             // out^T[col][outer] += sum_inner Y[inner][col] w[inner][outer]
@@ -4652,6 +4675,22 @@ extern "C" int flyhip_sbblocksparse_fwd(const void* q, const void* k, const void
     SB_DISPATCH_E(launch_fwd_list, float, a)
 }
 
+extern "C" int flyhip_local_fwd_dropout(const void* q, const void* k, const void* v, const int64_t* key_lengths, void* out,
+                                    float* lse,
+                                int B, int H, int T, int S, int E, int D, int local_context,
+                                int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                                int64_t k_sb, int64_t k_sh, int64_t k_ss,
+                                int64_t v_sb, int64_t v_sh, int64_t v_ss,
+                                int64_t o_sb, int64_t o_sh, int64_t o_ss,
+                                float softmax_temp, int dtype, float dropout_p, uint64_t dropout_seed, void* stream);
+extern "C" int flyhip_sblocal_bwd_band_dropout(const float* x1, const float* x2, const float* x3,
+                                       const float* y1, const float* y2, const float* y3,
+                                       const float* log_norm, const float* c, const int64_t* key_lengths,
+                                       float* o1, float* o2, float* o3,
+                                       int BH, int H, int T, int S, int E, int M, int local_context,
+                                       float softmax_temp, int key_major, float dropout_p, uint64_t dropout_seed,
+                                       void* stream);
+
 extern "C" int flyhip_local_fwd_lse(const void* q, const void* k, const void* v, const int64_t* key_lengths, void* out,
                                     float* lse,
                                 int B, int H, int T, int S, int E, int D, int local_context,
@@ -4660,7 +4699,22 @@ extern "C" int flyhip_local_fwd_lse(const void* q, const void* k, const void* v,
                                 int64_t v_sb, int64_t v_sh, int64_t v_ss,
                                 int64_t o_sb, int64_t o_sh, int64_t o_ss,
                                 float softmax_temp, int dtype, void* stream) {
+    return flyhip_local_fwd_dropout(q, k, v, key_lengths, out, lse, B, H, T, S, E, D, local_context,
+                                    q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss,
+                                    softmax_temp, dtype, 0.f, 0, stream);
+}
+
+extern "C" int flyhip_local_fwd_dropout(const void* q, const void* k, const void* v, const int64_t* key_lengths, void* out,
+                                    float* lse,
+                                int B, int H, int T, int S, int E, int D, int local_context,
+                                int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                                int64_t k_sb, int64_t k_sh, int64_t k_ss,
+                                int64_t v_sb, int64_t v_sh, int64_t v_ss,
+                                int64_t o_sb, int64_t o_sh, int64_t o_ss,
+                                float softmax_temp, int dtype, float dropout_p, uint64_t dropout_seed, void* stream) {
     FLY_REQUIRE(q && k && v && out, "local_fwd: null pointer");
+    FLY_REQUIRE(dropout_p >= 0.f && dropout_p < 1.f, "local_fwd: dropout_p %g not in [0, 1)", (double)dropout_p);
+    FLY_REQUIRE((long)B * H * T <= 4294967295L, "local_fwd: more than 2^32 query rows");
     FLY_REQUIRE(B > 0 && H > 0 && T > 0 && S > 0, "local_fwd: empty problem");
     FLY_REQUIRE(local_context >= 1, "local_fwd: local_context must be >= 1");
     FLY_REQUIRE(softmax_temp > 0.f, "local_fwd: softmax_temp must be positive");
@@ -4669,6 +4723,8 @@ extern "C" int flyhip_local_fwd_lse(const void* q, const void* k, const void* v,
                 "local_fwd: strides must be multiples of 4 elements (16-byte vector access)");
     LocalArgs a{q, k, v, key_lengths, out, B, H, T, S, local_context,
                 q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss, softmax_temp, lse};
+    const DropArgs drop = drop_args(dropout_p, dropout_seed);
+    a.drop_seed = drop.seed; a.drop_thresh = drop.thresh; a.drop_scale = drop.scale;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     if (int rc_capture = refuse_capture(st)) return rc_capture;
 #define LOCAL_DISPATCH(TT)                                                                          \
@@ -4704,13 +4760,28 @@ extern "C" int flyhip_sblocal_bwd_band(const float* x1, const float* x2, const f
                                        float* o1, float* o2, float* o3,
                                        int BH, int H, int T, int S, int E, int M, int local_context,
                                        float softmax_temp, int key_major, void* stream) {
+    return flyhip_sblocal_bwd_band_dropout(x1, x2, x3, y1, y2, y3, log_norm, c, key_lengths, o1, o2, o3, BH, H, T, S, E, M,
+                                           local_context, softmax_temp, key_major, 0.f, 0, stream);
+}
+
+extern "C" int flyhip_sblocal_bwd_band_dropout(const float* x1, const float* x2, const float* x3,
+                                       const float* y1, const float* y2, const float* y3,
+                                       const float* log_norm, const float* c, const int64_t* key_lengths,
+                                       float* o1, float* o2, float* o3,
+                                       int BH, int H, int T, int S, int E, int M, int local_context,
+                                       float softmax_temp, int key_major, float dropout_p, uint64_t dropout_seed,
+                                       void* stream) {
     FLY_REQUIRE(x1 && x3 && y1 && y2 && y3 && log_norm && c && o1 && o2, "sblocal_bwd_band: null pointer");
+    FLY_REQUIRE(dropout_p >= 0.f && dropout_p < 1.f, "sblocal_bwd_band: dropout_p %g not in [0, 1)", (double)dropout_p);
+    FLY_REQUIRE((long)BH * T <= 4294967295L, "sblocal_bwd_band: more than 2^32 query rows");
     FLY_REQUIRE(!key_major || (x2 && o3), "sblocal_bwd_band: the key-major pass needs x2 and o3");
     FLY_REQUIRE(BH > 0 && H > 0 && BH % H == 0 && T > 0 && S > 0, "sblocal_bwd_band: empty or inconsistent problem");
     FLY_REQUIRE(local_context >= 1, "sblocal_bwd_band: local_context must be >= 1");
     FLY_REQUIRE(softmax_temp > 0.f, "sblocal_bwd_band: softmax_temp must be positive");
     BwdArgs a{x1, x2, x3, y1, y2, y3, log_norm, c, key_lengths, o1, o2, o3, BH, H, T, S, local_context, softmax_temp,
               nullptr, nullptr, nullptr};
+    const DropArgs drop = drop_args(dropout_p, dropout_seed);
+    a.drop_seed = drop.seed; a.drop_thresh = drop.thresh; a.drop_scale = drop.scale;
     return dispatch_bwd_band(a, E, M, key_major, stream);
 }
 

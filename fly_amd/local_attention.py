@@ -11,11 +11,15 @@ from .sblocal_attention import _HEAD_DIMS, _round_up_choice, _vector_ready
 from .sblocal_backward import BandWindows, _band_kernel_dims, _band_terms_hip
 
 
-def local_forward(query, key, value, local_context, softmax_temp=None, key_lengths=None, return_lse=False):
+def local_forward(query, key, value, local_context, softmax_temp=None, key_lengths=None, return_lse=False,
+                  dropout=(0.0, 0)):
     """query (B,T,H,E), key (B,S,H,E), value (B,S,H,D) float32 or bfloat16 GPU tensors ->
     out (B,T,H,D): query i attends to keys j with -(local_context // 2) <= j - i < (local_context + 1) // 2
-    and j < key_lengths[b] (local_attention.py:68-92 for attn_mask=None, no dropout).  With return_lse
-    also the log of every query's softmax denominator, (B,H,T) float32 (0 for a query without keys)."""
+    and j < key_lengths[b] (local_attention.py:68-92 for attn_mask=None).  With return_lse
+    also the log of every query's softmax denominator, (B,H,T) float32 (0 for a query without keys).
+    dropout = (p, seed) with p > 0: the weights are dropped after the softmax with probability p and the kept ones
+    scaled by 1 / (1 - p) (local_attention.py:91, `self.dropout(torch.softmax(...))`), by a hash of (seed, batch,
+    head, query, key) formed inside the kernel instead of a stored mask."""
     _lib.require_gpu(query, key, value, key_lengths)
     if query.dtype not in (torch.float32, torch.bfloat16):
         raise NotImplementedError(f'the local attention kernel supports float32 and bfloat16, got {query.dtype}')
@@ -44,16 +48,16 @@ def local_forward(query, key, value, local_context, softmax_temp=None, key_lengt
     out = torch.empty(B, T, H, dim, dtype=query.dtype, device=query.device)
     lse = torch.empty(B, H, T, dtype=torch.float32, device=query.device) if return_lse else None
     with torch.cuda.device(query.device):
-        _lib.call('flyhip_local_fwd_lse', q.data_ptr(), k.data_ptr(), v.data_ptr(), _lib.ptr(lens), out.data_ptr(),
+        _lib.call('flyhip_local_fwd_dropout', q.data_ptr(), k.data_ptr(), v.data_ptr(), _lib.ptr(lens), out.data_ptr(),
                   _lib.ptr(lse), B, H, T, S, dim, dim, local_context,
                   q.stride(0), q.stride(2), q.stride(1), k.stride(0), k.stride(2), k.stride(1),
                   v.stride(0), v.stride(2), v.stride(1), out.stride(0), out.stride(2), out.stride(1),
-                  t, _lib.dtype_code(q), _lib.stream_ptr(query.device))
+                  t, _lib.dtype_code(q), float(dropout[0]), int(dropout[1]), _lib.stream_ptr(query.device))
     return (out[..., :D], lse) if return_lse else out[..., :D]
 
 
 def local_backward(query, key, value, local_context, softmax_temp, key_lengths, grad_out, chunk=256,
-                   max_elements=1 << 27, out=None, lse=None):
+                   max_elements=1 << 27, out=None, lse=None, dropout=(0.0, 0)):
     """Gradients of local attention with respect to query, key and value (the reference takes them from
     autograd through fast_transformers.local_product, local_attention.py:68-92).  The band softmax is
     evaluated again for all chunks of queries at once against the windows of keys their bands touch
@@ -64,7 +68,9 @@ def local_backward(query, key, value, local_context, softmax_temp, key_lengths, 
     or bfloat16 GPU tensors and head dims <= 64, the sums run on the backward band kernel of
     Scatterbrain-local attention with its feature operands zero (flyhip_sblocal_bwd_band: P_is =
     exp(t q_i.k_s - lse_i), delta_i = g_i.out_i); otherwise as batched library products on the GPU (host tensors are
-    accepted in float64 only: the check of these formulas against autograd)."""
+    accepted in float64 only: the check of these formulas against autograd).  dropout = (p, seed) of the forward:
+    with M the kept / (1 - p) mask, d v_s = sum_i M_is P_is g_i and d(t q_i.k_s) = P_is (M_is g_i.v_s - delta_i),
+    delta_i = g_i.out_i as before; on the band kernel only."""
     B, T, H, E = query.shape
     S, D = key.shape[1], value.shape[3]
     t = softmax_temp or 1 / math.sqrt(E)
@@ -85,8 +91,11 @@ def local_backward(query, key, value, local_context, softmax_temp, key_lengths, 
         delta = (G * bh(out)).sum(-1, keepdim=True)
         lens_b = None if key_lengths is None else key_lengths.to(device=Q.device, dtype=torch.int64).contiguous()
         dQ, _, dK, _, dV = _band_terms_hip(Q, K, V, G, zq, zk, lse.reshape(B * H, T, 1), delta, lens_b, H,
-                                           local_context, t, dims)
+                                           local_context, t, dims, dropout)
         return back(dQ, query), back(dK, key), back(dV, value)
+    if dropout[0] > 0:
+        raise NotImplementedError('the gradients of dropped local attention run on the band kernel only: float32 or '
+                                  'bfloat16 GPU tensors, head dims <= 64, the forward\'s out and lse given')
     lens = None
     if key_lengths is not None:
         lens = key_lengths.to(Q.device).repeat_interleave(H).view(B * H, 1, 1)
@@ -113,31 +122,31 @@ class _LocalFn(torch.autograd.Function):
     """Forward on the fused kernel, gradients from local_backward."""
 
     @staticmethod
-    def forward(ctx, query, key, value, local_context, softmax_temp, key_lengths):
+    def forward(ctx, query, key, value, local_context, softmax_temp, key_lengths, dropout=(0.0, 0)):
         out, lse = local_forward(query, key, value, local_context, softmax_temp=softmax_temp, key_lengths=key_lengths,
-                                 return_lse=True)
+                                 return_lse=True, dropout=dropout)
         ctx.save_for_backward(query, key, value, key_lengths, out, lse)
-        ctx.local_context, ctx.softmax_temp = local_context, softmax_temp
+        ctx.local_context, ctx.softmax_temp, ctx.dropout = local_context, softmax_temp, dropout
         return out
 
     @staticmethod
     def backward(ctx, grad_out):
         query, key, value, key_lengths, out, lse = ctx.saved_tensors
         dq, dk, dv = local_backward(query, key, value, ctx.local_context, ctx.softmax_temp, key_lengths, grad_out,
-                                    out=out, lse=lse)
-        return dq, dk, dv, None, None, None
+                                    out=out, lse=lse, dropout=ctx.dropout)
+        return dq, dk, dv, None, None, None, None
 
 
-def local_attention_fn(query, key, value, local_context, softmax_temp=None, key_lengths=None):
+def local_attention_fn(query, key, value, local_context, softmax_temp=None, key_lengths=None, dropout=(0.0, 0)):
     """local_forward that autograd can differentiate."""
-    return _LocalFn.apply(query, key, value, local_context, softmax_temp, key_lengths)
+    return _LocalFn.apply(query, key, value, local_context, softmax_temp, key_lengths, dropout)
 
 
 class LocalAttention(nn.Module):
     """Softmax attention in which query i only sees keys j with
     -(local_context // 2) <= j - i < (local_context + 1) // 2.  Same constructor and forward signature
     as the reference class.  Covered on the GPU: no attn_mask, optional length-style key_padding_mask,
-    dropout inactive; anything else raises NotImplementedError.  need_weights=True also returns the dense
+    attention dropout in training mode (inside the kernels); anything else raises NotImplementedError.  need_weights=True also returns the dense
     (B,H,T,S) matrix (local_attention.py:94-106), exp(t q.k - lse) on the band with the kernel's own
     log-denominators, as ordinary tensor algebra: an inspection path for problems of up to
     max_weight_elements entries."""
@@ -152,14 +161,23 @@ class LocalAttention(nn.Module):
     def forward(self, query, key, value, attn_mask=None, key_padding_mask=None, need_weights=False):
         if attn_mask is not None and not bool(attn_mask.all_ones):
             raise NotImplementedError('attn_mask other than all-ones is not supported by the fused kernel')
+        # training-mode dropout (local_attention.py:91) runs inside the kernels: the mask is a hash of (seed, batch,
+        # head, query, key); the seed is drawn per call from torch's CPU generator and kept in last_dropout_seed
+        dropout = (0.0, 0)
+        self.last_dropout_seed = None
         if self.training and self.dropout.p > 0.0:
-            raise NotImplementedError('attention dropout is not implemented in the fused kernel')
+            if not self.dropout.p < 1.0:
+                raise NotImplementedError('attention dropout with p = 1 is not implemented in the fused kernel')
+            if need_weights:
+                raise NotImplementedError('need_weights with active attention dropout is not implemented')
+            dropout = (float(self.dropout.p), int(torch.randint(0, 2 ** 62, (1,)).item()))
+            self.last_dropout_seed = dropout[1]
         lengths = None
         if key_padding_mask is not None and not bool(key_padding_mask.all_ones):
             lengths = key_padding_mask.lengths
         if not need_weights:
             out = local_attention_fn(query, key, value, self.local_context, softmax_temp=self.softmax_temp,
-                                     key_lengths=lengths)
+                                     key_lengths=lengths, dropout=dropout)
             return out, None
         B, T, H, E = query.shape
         S = key.shape[1]

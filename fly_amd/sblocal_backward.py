@@ -227,10 +227,11 @@ def _backward_hip(Q, K, V, G, O, LN, P, lens_b, H, local_context, t, dims, piece
     return dq[..., :E], dk[..., :E], dv[..., :D]
 
 
-def _band_terms_hip(Q, K, V, G, psi, phik, LN, c, lens_b, H, local_context, t, dims):
+def _band_terms_hip(Q, K, V, G, psi, phik, LN, c, lens_b, H, local_context, t, dims, dropout=(0.0, 0)):
     """The five band-limited sums on flyhip_sblocal_bwd_band.  Q, G, psi, LN, c: (BH, T, .); K, V, phik:
     (BH, S, .); float32 on the GPU.  Returns (t sum_s dm k, sum_s df phik, t sum_i dm q, sum_i df psi,
-    sum_i (a - kb) g) cut back to the callers' widths."""
+    sum_i (a - kb) g) cut back to the callers' widths.  dropout = (p, seed) of a forward that dropped exact
+    weights: the kernels form the same mask again from the seed."""
     from . import _lib
     BH, T, E = Q.shape
     S, D, M = K.shape[1], V.shape[2], psi.shape[2]
@@ -242,12 +243,13 @@ def _band_terms_hip(Q, K, V, G, psi, phik, LN, c, lens_b, H, local_context, t, d
     dk, uk, dv = Q.new_empty(BH, S, dim), Q.new_empty(BH, S, mk), Q.new_empty(BH, S, dim)
     with torch.cuda.device(Q.device):
         st = _lib.stream_ptr(Q.device)
-        _lib.call('flyhip_sblocal_bwd_band', q_.data_ptr(), None, g_.data_ptr(), k_.data_ptr(), phik_.data_ptr(),
+        drop = (float(dropout[0]), int(dropout[1]))
+        _lib.call('flyhip_sblocal_bwd_band_dropout', q_.data_ptr(), None, g_.data_ptr(), k_.data_ptr(), phik_.data_ptr(),
                   v_.data_ptr(), ln_.data_ptr(), c_.data_ptr(), _lib.ptr(lens_b), dq.data_ptr(), uq.data_ptr(), None,
-                  BH, H, T, S, dim, mk, local_context, float(t), 0, st)
-        _lib.call('flyhip_sblocal_bwd_band', k_.data_ptr(), phik_.data_ptr(), v_.data_ptr(), q_.data_ptr(),
+                  BH, H, T, S, dim, mk, local_context, float(t), 0, *drop, st)
+        _lib.call('flyhip_sblocal_bwd_band_dropout', k_.data_ptr(), phik_.data_ptr(), v_.data_ptr(), q_.data_ptr(),
                   psi_.data_ptr(), g_.data_ptr(), ln_.data_ptr(), c_.data_ptr(), _lib.ptr(lens_b), dk.data_ptr(),
-                  uk.data_ptr(), dv.data_ptr(), BH, H, T, S, dim, mk, local_context, float(t), 1, st)
+                  uk.data_ptr(), dv.data_ptr(), BH, H, T, S, dim, mk, local_context, float(t), 1, *drop, st)
     return dq[..., :E], uq[..., :M], dk[..., :E], uk[..., :M], dv[..., :D]
 
 

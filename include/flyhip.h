@@ -185,6 +185,19 @@ int flyhip_sblocal_bwd_band(const float* x1, const float* x2, const float* x3,
                             int BH, int H, int T, int S, int E, int M, int local_context,
                             float softmax_temp, int key_major, void* stream);
 
+/* flyhip_sblocal_bwd_band for a forward that dropped exact weights with (dropout_p, dropout_seed) (the dropout of
+ * sblocal_attention.py:119 / local_attention.py:91, whose mask autograd keeps; here it is formed again from the seed,
+ * the hash of flyhip_sblocal_forward): with m = 0 on dropped pairs and 1 / (1 - dropout_p) on kept ones,
+ * dm = a (m g_i.v_s - c_i) and o3 = sum_i (m a - kb) g_i; df and o2 are unchanged (the low-rank part is not dropped).
+ * dropout_p = 0 is flyhip_sblocal_bwd_band. */
+int flyhip_sblocal_bwd_band_dropout(const float* x1, const float* x2, const float* x3,
+                                    const float* y1, const float* y2, const float* y3,
+                                    const float* log_norm, const float* c, const int64_t* key_lengths,
+                                    float* o1, float* o2, float* o3,
+                                    int BH, int H, int T, int S, int E, int M, int local_context,
+                                    float softmax_temp, int key_major, float dropout_p, uint64_t dropout_seed,
+                                    void* stream);
+
 /* The whole backward pass after the feature maps, one call per side (same operand roles as
  * flyhip_sblocal_bwd_band, x2 = the outer rows' own features in both passes: psi for key_major = 0,
  * phik for key_major = 1).  The epilogue adds the low-rank weight outside the band ("all keys minus the
@@ -323,6 +336,20 @@ int flyhip_local_fwd_lse(const void* q, const void* k, const void* v, const int6
                          int64_t v_sb, int64_t v_sh, int64_t v_ss,
                          int64_t o_sb, int64_t o_sh, int64_t o_ss,
                          float softmax_temp, int dtype, void* stream);
+
+/* flyhip_local_fwd_lse with the dropout of LocalAttention.forward (ref: src/models/attention/local_attention.py:91,
+ * `self.dropout(torch.softmax(...))`): every weight is dropped with probability dropout_p in [0, 1) after the softmax
+ * (lse is that of the undropped softmax) and the kept ones are scaled by 1 / (1 - dropout_p).  The mask is the hash
+ * of (seed, (b H + h) T + query, key) that flyhip_sblocal_forward documents; flyhip_sblocal_bwd_band_dropout forms
+ * it again.  dropout_p = 0 is flyhip_local_fwd_lse. */
+int flyhip_local_fwd_dropout(const void* q, const void* k, const void* v, const int64_t* key_lengths, void* out,
+                             float* lse,
+                             int B, int H, int T, int S, int E, int D, int local_context,
+                             int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                             int64_t k_sb, int64_t k_sh, int64_t k_ss,
+                             int64_t v_sb, int64_t v_sh, int64_t v_ss,
+                             int64_t o_sb, int64_t o_sh, int64_t o_ss,
+                             float softmax_temp, int dtype, float dropout_p, uint64_t dropout_seed, void* stream);
 
 /* Measurement hook (no counterpart in the reference): the two caller-owned hipEvent_t receive the begin
  * and the end time stamp of the fused band kernel's launch (hipExtLaunchKernelGGL) in the NEXT

@@ -477,6 +477,55 @@ def test_local_attention_module_gradients(dtype, tol):
     assert float(kg.grad[1, 200:].abs().max()) == 0.0
 
 
+@pytest.mark.parametrize('dtype,tol,E,p_drop', [(torch.float32, 1e-4, 64, 0.25), (torch.bfloat16, 3e-2, 64, 0.1),
+                                                 (torch.float32, 1e-4, 24, 0.5)])
+def test_local_attention_dropout_inside_the_kernels(dtype, tol, E, p_drop):
+    """Training-mode dropout of LocalAttention (local_attention.py:91) inside the forward kernel and both band kernels
+    of the backward: the mask is the hash of (seed, batch, head, query, key) restated in oracle.sblocal.dropout_keep, so
+    output and gradients are compared with float64 autograd through band softmax -> mask / (1 - p) -> product on the
+    kernels' own mask -- T != S, key lengths (queries without a visible key), a head dim that needs padding.  The
+    reference draws its mask from torch's generator; independent keeps with probability 1 - p are what both share."""
+    from fly_amd import LocalAttention, LengthMask
+    B, T, S, H, D, lc = 2, 300, 280, 2, E, 64
+    print('case', dtype, E, p_drop, flush=True)
+    g = torch.Generator().manual_seed(33)
+    q, k, v = (torch.randn(B, L, H, C, generator=g).to(dtype) for L, C in ((T, E), (S, E), (S, D)))
+    lengths = torch.tensor([S, 200])
+    w = torch.randn(B, T, H, D, generator=g)
+    dev = torch.device('cuda:0')
+    mod = LocalAttention(lc, attention_dropout=p_drop).to(dev).train()
+    qg, kg, vg = (x.to(dev).requires_grad_() for x in (q, k, v))
+    torch.manual_seed(11)
+    out, _ = mod(qg, kg, vg, key_padding_mask=LengthMask(lengths.to(dev), max_len=S))
+    seed = mod.last_dropout_seed
+    assert seed is not None
+    (out.float() * w.to(dev)).sum().backward()
+
+    qd, kd, vd = (x.double().requires_grad_() for x in (q, k, v))
+    i, j = torch.arange(T).view(T, 1), torch.arange(S).view(1, S)
+    vis = ((j - i >= -(lc // 2)) & (j - i < (lc + 1) // 2)).view(1, 1, T, S) & (j.view(1, 1, 1, S) < lengths.view(B, 1, 1, 1))
+    live = vis.any(-1, keepdim=True)
+    sc = torch.einsum('bthe,bshe->bhts', qd, kd) / math.sqrt(E)
+    prob = torch.softmax(torch.where(live, sc.masked_fill(~vis, float('-inf')), torch.zeros_like(sc)), -1) * live
+    mult = osb.dropout_keep(seed, p_drop, B, H, T, S)
+    ref = torch.einsum('bhts,bshd->bthd', prob * mult, vd)
+    (ref * w.double()).sum().backward()
+    assert rel_err(out.float(), ref) <= (1e-4 if dtype == torch.float32 else 2e-2), rel_err(out.float(), ref)
+    for got, want, name in ((qg.grad, qd.grad, 'dq'), (kg.grad, kd.grad, 'dk'), (vg.grad, vd.grad, 'dv')):
+        assert got.dtype == dtype and rel_err(got.float(), want) <= tol, (name, rel_err(got.float(), want))
+    assert float(kg.grad[1, 200:].abs().max()) == 0.0
+    # same seed, same mask; evaluation mode: no mask; need_weights with active dropout is refused
+    torch.manual_seed(11)
+    with torch.no_grad():
+        again, _ = mod(qg, kg, vg, key_padding_mask=LengthMask(lengths.to(dev), max_len=S))
+        assert torch.equal(again, out.detach())
+        with pytest.raises(NotImplementedError):
+            mod(qg, kg, vg, need_weights=True)
+        plain, _ = mod.eval()(qg, kg, vg, key_padding_mask=LengthMask(lengths.to(dev), max_len=S))
+    assert mod.last_dropout_seed is None
+    assert rel_err(plain.float(), torch.einsum('bhts,bshd->bthd', prob, vd).detach()) <= (1e-4 if dtype == torch.float32 else 2e-2)
+
+
 @pytest.mark.parametrize('B,T,S,H,E,D,mh,lc,lens', [(2, 300, 280, 2, 64, 64, 32, 64, [280, 200]),
                                                     (1, 257, 391, 3, 50, 40, 24, 77, None),
                                                     (2, 130, 130, 1, 32, 32, 16, 301, [130, 1]),
