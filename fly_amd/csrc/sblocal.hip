@@ -2801,6 +2801,8 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
     // keys this lane's query may see: smin <= s < smin + span
     const int smin = max(iq - lc_lo, 0);
     const unsigned span = qvalid ? (unsigned)max(min(iq + lc_hi, len) - smin, 0) : 0u;
+    const bool drop_on = a.drop_thresh != 0u;          // (kernel-uniform) dropout of the exact weights
+    const uint32_t drop_row = drop_on ? drop_row_hash(a.drop_seed, (uint32_t)(bh * a.T + iq)) : 0u;
 
     if (kt_lo < kt_hi) {
         rk.template stash<LDK>(smem, tid);
@@ -2907,9 +2909,11 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
                     for (int i = 0; i < 4; ++i) {
                         const float e = ok[kb][i] ? __builtin_amdgcn_exp2f(s1[kb][i] - m_run) : 0.f;
                         const float ov = ok[kb][i] ? s2[kb][i] : 0.f;
-                        ze += e;
+                        ze += e;                                   // the normaliser sees no dropout
                         ovs += ov;
-                        p[kb][i] = e - ov * beta;
+                        float ek = e;
+                        if (drop_on) ek = drop_keep(drop_row, (uint32_t)(s_base + 16 * kb + 4 * g + i), a.drop_thresh) ? e * a.drop_scale : 0.f;
+                        p[kb][i] = ek - ov * beta;
                     }
             };
             if (interior) soft(std::false_type{}); else soft(std::true_type{});
@@ -4649,9 +4653,11 @@ extern "C" int flyhip_sbblocksparse_fwd(const void* q, const void* k, const void
                                         int64_t k_sb, int64_t k_sh, int64_t k_ss,
                                         int64_t v_sb, int64_t v_sh, int64_t v_ss,
                                         int64_t o_sb, int64_t o_sh, int64_t o_ss,
-                                        float softmax_temp, int dtype, void* stream) {
+                                        float softmax_temp, int dtype, float dropout_p, uint64_t dropout_seed, void* stream) {
     FLY_REQUIRE(q && k && v && proj && kfeat && chunk_scale && kv && ksum && kmax && tl_ptr && tl_inner && tl_blk &&
                 out && log_norm, "sbblocksparse_fwd: null pointer");
+    FLY_REQUIRE(dropout_p >= 0.f && dropout_p < 1.f, "sbblocksparse_fwd: dropout_p %g not in [0, 1)", (double)dropout_p);
+    FLY_REQUIRE((long)B * H * T <= 4294967295L, "sbblocksparse_fwd: more than 2^32 query rows");
     FLY_REQUIRE(B > 0 && H > 0 && T > 0 && S > 0, "sbblocksparse_fwd: empty problem");
     FLY_REQUIRE(T % 16 == 0 && S % 16 == 0, "sbblocksparse_fwd: sequence lengths %d, %d must be multiples of 16", T, S);
     FLY_REQUIRE(softmax_temp > 0.f, "sbblocksparse_fwd: softmax_temp must be positive");
@@ -4669,6 +4675,8 @@ extern "C" int flyhip_sbblocksparse_fwd(const void* q, const void* k, const void
               B, H, T, S, mh_valid, 1, nc, n_heavy > 0 ? heavy_parts : 1,
               q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss, softmax_temp,
               tl_ptr, tl_inner, tl_blk, tl_order, tl_heavy, n_heavy};
+    const DropArgs drop = drop_args(dropout_p, dropout_seed);
+    a.drop_seed = drop.seed; a.drop_thresh = drop.thresh; a.drop_scale = drop.scale;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     if (int rc_capture = refuse_capture(st)) return rc_capture;
     const int m = 2 * mh;

@@ -1077,9 +1077,11 @@ extern "C" int flyhip_sbblocksparse_bwd_pieces(const void* outer_images, const v
                                                const int32_t* tl_skip, const int32_t* tl_heavy, int n_heavy, int heavy_parts,
                                                float* part_ws, int64_t part_ws_floats,
                                                int BH, int H, int T, int S, int E, int M,
-                                               float softmax_temp, int key_major, void* stream) {
+                                               float softmax_temp, int key_major, float dropout_p, uint64_t dropout_seed,
+                                               void* stream) {
     FLY_REQUIRE(outer_images && inner_images && x1 && log_norm && c && gmat && gvec && proj && d1 && tl_ptr && tl_inner && tl_blk,
                 "sbblocksparse_bwd_pieces: null pointer");
+    FLY_REQUIRE(dropout_p >= 0.f && dropout_p < 1.f, "sbblocksparse_bwd_pieces: dropout probability %g outside [0, 1)", (double)dropout_p);
     FLY_REQUIRE(!key_major || d3, "sbblocksparse_bwd_pieces: the key-major pass needs d3");
     FLY_REQUIRE(BH > 0 && H > 0 && BH % H == 0 && T > 0 && S > 0, "sbblocksparse_bwd_pieces: empty or inconsistent problem");
     FLY_REQUIRE(T % 32 == 0 && S % 32 == 0, "sbblocksparse_bwd_pieces: sequence lengths %d, %d must be multiples of 32", T, S);
@@ -1089,6 +1091,8 @@ extern "C" int flyhip_sbblocksparse_bwd_pieces(const void* outer_images, const v
     BwdX3Args a{reinterpret_cast<const char*>(outer_images), reinterpret_cast<const char*>(inner_images), x1,
                 log_norm, c, nullptr, d1, d3, BH, H, T, S, 1, softmax_temp, gmat, gvec, proj, 0, part_ws, n_heavy ? heavy_parts : 1,
                 tl_ptr, tl_inner, tl_blk, n_heavy ? tl_skip : nullptr, n_heavy ? tl_heavy : nullptr, n_heavy};
+    const DropArgs dr = drop_args(dropout_p, dropout_seed);
+    a.drop_seed = dr.seed; a.drop_thresh = dr.thresh; a.drop_scale = dr.scale;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     if (int rc_capture = refuse_capture(st)) return rc_capture;
     const long wsf = part_ws ? (long)part_ws_floats : 0;

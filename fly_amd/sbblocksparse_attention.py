@@ -60,10 +60,11 @@ class _SBBlockSparseFn(torch.autograd.Function):
     the band replaced by the layout's blocks (sblocal_backward.sblocal_backward, support=...)."""
 
     @staticmethod
-    def forward(ctx, query, key, value, projection_matrix, tables, support, softmax_temp, cache=None):
-        out, log_norm = sbblocksparse_forward(query, key, value, projection_matrix, tables, softmax_temp, cache=cache)
+    def forward(ctx, query, key, value, projection_matrix, tables, support, softmax_temp, cache=None, dropout=(0.0, 0)):
+        out, log_norm = sbblocksparse_forward(query, key, value, projection_matrix, tables, softmax_temp, cache=cache,
+                                              dropout_p=dropout[0], dropout_seed=dropout[1])
         ctx.save_for_backward(query, key, value, projection_matrix, out, log_norm)
-        ctx.support, ctx.softmax_temp = support, softmax_temp
+        ctx.support, ctx.softmax_temp, ctx.dropout = support, softmax_temp, dropout
         ctx.mark_non_differentiable(log_norm)
         return out, log_norm
 
@@ -72,8 +73,8 @@ class _SBBlockSparseFn(torch.autograd.Function):
         from .sblocal_backward import sblocal_backward
         query, key, value, projection_matrix, out, log_norm = ctx.saved_tensors
         dq, dk, dv = sblocal_backward(query, key, value, projection_matrix, 1, ctx.softmax_temp, None, out, log_norm,
-                                      grad_out, support=ctx.support)
-        return dq, dk, dv, None, None, None, None, None
+                                      grad_out, support=ctx.support, dropout=ctx.dropout)
+        return dq, dk, dv, None, None, None, None, None, None
 
 
 class SBBlockSparseAttention(nn.Module):
@@ -167,7 +168,13 @@ class SBBlockSparseAttention(nn.Module):
         needs_grad = torch.is_grad_enabled() and any(x.requires_grad for x in (query, key, value))
         from .sblocal_backward import _band_kernel_dims
         n_rows = self.feature_map.projection_matrix.shape[0]
-        if (self.fuse and not need_weights and not (self.training and self.dropout.p > 0)
+        # training-mode dropout (:200: of the exact weights only) runs inside the kernels: the mask is a hash of (seed,
+        # batch, head, query, key), the seed drawn per call from torch's CPU generator and kept in last_dropout_seed
+        dropout = (0.0, 0)
+        self.last_dropout_seed = None
+        if self.training and 0 < self.dropout.p < 1:
+            dropout = (float(self.dropout.p), int(torch.randint(0, 2 ** 62, (1,)).item()))
+        if (self.fuse and not need_weights and not (self.training and self.dropout.p >= 1)
                 and self.softmax_eps == 0
                 and query.dtype in (torch.float32, torch.bfloat16, torch.float16)
                 and sbblocksparse_forward_supported(block, torch.float32, E, value.shape[3], n_rows, layout.shape[0], H)
@@ -180,14 +187,16 @@ class SBBlockSparseAttention(nn.Module):
             if not needs_grad:
                 out, _ = sbblocksparse_forward(query.float(), key.float(), value.float(),
                                                self.feature_map.projection_matrix, self.fused_tables[key_], softmax_temp,
-                                               cache=self._scratch_cache)
+                                               cache=self._scratch_cache, dropout_p=dropout[0], dropout_seed=dropout[1])
+                self.last_dropout_seed = dropout[1] if dropout[0] > 0 else None
                 return out.to(query.dtype), None
             if key_ not in self.backward_tables:     # the support seen from the queries and from the keys
                 self.backward_tables[key_] = (backward_tables(layout, query.device),
                                               backward_tables(layout, query.device, transposed=True))
             support = self.backward_tables[key_]
             out, _ = _SBBlockSparseFn.apply(query.float(), key.float(), value.float(), self.feature_map.projection_matrix,
-                                            self.fused_tables[key_], support, softmax_temp, self._scratch_cache)
+                                            self.fused_tables[key_], support, softmax_temp, self._scratch_cache, dropout)
+            self.last_dropout_seed = dropout[1] if dropout[0] > 0 else None
             return out.to(query.dtype), None
 
         # 2-byte inputs are widened: the scores pass through HBM between the stages, and a score kept

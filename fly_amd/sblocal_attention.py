@@ -152,10 +152,11 @@ class SBLocalPlan:
                   v.stride(0), v.stride(2), v.stride(1), out.stride(0), out.stride(2), out.stride(1),
                   t, self.code, stream)
 
-    def run_block_sparse(self, q, k, v, proj, t, tables, out, log_norm):
+    def run_block_sparse(self, q, k, v, proj, t, tables, out, log_norm, dropout=(0.0, 0)):
         """Scatterbrain attention whose exact part lives on a block-sparse support instead of a band: the
         key pass as in ``run``, then the fp32 band kernel walking lists of 32-key tiles (``tables`` =
-        blocksparse_utils.tile_mask_table(layout, block) on the device).  One part per query tile, no key lengths."""
+        blocksparse_utils.tile_mask_table(layout, block) on the device).  One part per query tile, no key lengths.
+        dropout: (probability, seed) of the dropout of the exact weights inside that kernel."""
         B, H, T, S, dim, mh, mh_valid = self.shape
         self._make_buffers()
         tl_ptr, tl_inner, tl_blk = tables[:3]
@@ -181,7 +182,7 @@ class SBLocalPlan:
                       B, H, T, S, dim, dim, mh, mh_valid,
                       q.stride(0), q.stride(2), q.stride(1), k.stride(0), k.stride(2), k.stride(1),
                       v.stride(0), v.stride(2), v.stride(1), out.stride(0), out.stride(2), out.stride(1),
-                      t, self.code, stream)
+                      t, self.code, float(dropout[0]), int(dropout[1]), stream)
 
     def run(self, q, k, v, proj, lens, local_context, t, out, log_norm, dropout=(0.0, 0)):
         """dropout: (probability, seed) -- dropout of the exact weights inside the band kernel (float32 inputs on the
@@ -352,9 +353,11 @@ def sbblocksparse_forward_supported(block, dtype, E, D, n_projection_rows, layou
             and n_projection_rows <= _FEATURE_ROWS[-1] and layout_heads == H)
 
 
-def sbblocksparse_forward(query, key, value, projection_matrix, tables, softmax_temp=None, cache=None):
+def sbblocksparse_forward(query, key, value, projection_matrix, tables, softmax_temp=None, cache=None,
+                          dropout_p=0.0, dropout_seed=0):
     """Scatterbrain attention on a block-sparse support (sbblocksparse_attention.py:109-213 for
-    need_weights=False, no dropout) on the fused kernels: exact softmax weights on the nonzero blocks (16 x 16 or
+    need_weights=False; dropout_p, dropout_seed: the dropout of the exact weights of :200, by the hash mask of
+    sblocal_forward) on the fused kernels: exact softmax weights on the nonzero blocks (16 x 16 or
     32 x 32), the Performer estimate everywhere else, one normaliser.  query (B,T,H,E), key (B,S,H,E), value
     (B,S,H,D) float32 GPU tensors, T and S multiples of the block size; tables = blocksparse_utils.tile_mask_table(layout,
     block) as int32 tensors on the device, optionally followed by union_order(tables[0], H), or the six entries of
@@ -385,7 +388,9 @@ def sbblocksparse_forward(query, key, value, projection_matrix, tables, softmax_
     plan = make_plan() if cache is None else cache.plan(plan_key, make_plan)
     out = torch.empty(B, T, H, dim, dtype=query.dtype, device=query.device)
     log_norm = torch.empty(B, H, T, dtype=torch.float32, device=query.device)
-    plan.run_block_sparse(q, k, v, proj, t, tables, out, log_norm)
+    if not 0.0 <= dropout_p < 1.0:
+        raise ValueError(f'dropout probability {dropout_p} not in [0, 1)')
+    plan.run_block_sparse(q, k, v, proj, t, tables, out, log_norm, dropout=(float(dropout_p), int(dropout_seed)))
     return out[..., :D], log_norm.unsqueeze(-1)
 
 

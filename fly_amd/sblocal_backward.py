@@ -207,7 +207,8 @@ def _backward_hip(Q, K, V, G, O, LN, P, lens_b, H, local_context, t, dims, piece
                 _lib.call('flyhip_sbblocksparse_bwd_pieces', oimg.data_ptr(), iimg.data_ptr(), x1.data_ptr(), ln_.data_ptr(),
                           c_.data_ptr(), gmat.data_ptr(), gvec.data_ptr(), proj.data_ptr(), d1.data_ptr(), _lib.ptr(d3),
                           tl_ptr.data_ptr(), _lib.table_ptr(tl_inner), _lib.table_ptr(tl_blk), _lib.ptr(skip), _lib.ptr(heavy),
-                          n_heavy, parts, _lib.ptr(hws), n_hws, BH, H, T, S, dim, mk, float(t), key_major, st)
+                          n_heavy, parts, _lib.ptr(hws), n_hws, BH, H, T, S, dim, mk, float(t), key_major,
+                          float(dropout[0]), int(dropout[1]), st)
         elif pieces:
             _lib.call('flyhip_sblocal_bwd_pieces', qimg.data_ptr(), kimg.data_ptr(), q_.data_ptr(),
                       ln_.data_ptr(), c_.data_ptr(), _lib.ptr(lens_b), kv.data_ptr(), ksum.data_ptr(), proj.data_ptr(),
@@ -352,7 +353,7 @@ def sblocal_backward(query, key, value, projection_matrix, local_context, softma
         # host tensors are accepted for one purpose: checking the written-out gradient formulas in float64 against autograd
         raise NotImplementedError('sblocal_backward runs on the GPU; host tensors only in float64 (the check of the formulas)')
     lens_b = None if key_lengths is None else key_lengths.to(device=Q.device, dtype=torch.int64).contiguous()
-    if dropout[0] > 0 and (support is not None or not on_kernels or band_kernel in ('sums', 'fp32')):
+    if dropout[0] > 0 and (not on_kernels or band_kernel in ('sums', 'fp32')):
         raise NotImplementedError('the backward under attention dropout runs on the band kernels on bf16 pieces only '
                                   f'(GPU, head dims <= 64, <= 128 features; got ({E}, {D}), {2 * mh})')
     if support is not None:
@@ -360,7 +361,7 @@ def sblocal_backward(query, key, value, projection_matrix, local_context, softma
             raise NotImplementedError('the backward on a block-sparse support needs the GPU kernels (float32 or bfloat16 '
                                       f'inputs, head dims <= 64, <= 128 features; got ({E}, {D}), {2 * mh}), sequence '
                                       'lengths that are multiples of 32 and no key lengths')
-        dQ, dK, dV = _backward_hip(Q, K, V, G, O, LN, P, None, H, 1, t, dims, support=support)
+        dQ, dK, dV = _backward_hip(Q, K, V, G, O, LN, P, None, H, 1, t, dims, support=support, dropout=dropout)
     elif on_kernels and band_kernel != 'sums':
         # features, per-head sums and the two passes of the fused kernel
         dQ, dK, dV = _backward_hip(Q, K, V, G, O, LN, P, lens_b, H, local_context, t, dims,

@@ -270,7 +270,8 @@ int flyhip_sblocal_bwd_pieces(const void* outer_images, const void* inner_images
  * Long lists (n_heavy > 0): tl_skip (H * ceil(outer rows / 64) flags) marks the outer tiles the main launch leaves
  * out, tl_heavy (n_heavy indices head * ceil(outer rows / 64) + tile) lists them; they are walked in heavy_parts
  * parts (2..64) by (batch, tile, part) workgroups of a launch of their own and finished by a third; part_ws of at
- * least flyhip_sbblocksparse_bwd_parts_floats(BH / H, n_heavy, heavy_parts, E, M, key_major) floats. */
+ * least flyhip_sbblocksparse_bwd_parts_floats(BH / H, n_heavy, heavy_parts, E, M, key_major) floats.
+ * dropout_p, dropout_seed: those of the forward (flyhip_sbblocksparse_fwd), as for flyhip_sblocal_bwd_pieces. */
 int64_t flyhip_sbblocksparse_bwd_parts_floats(int B, int n_heavy, int heavy_parts, int E, int M, int key_major);
 int flyhip_sbblocksparse_bwd_pieces(const void* outer_images, const void* inner_images,
                                     const float* x1, const float* log_norm, const float* c,
@@ -280,10 +281,11 @@ int flyhip_sbblocksparse_bwd_pieces(const void* outer_images, const void* inner_
                                     const int32_t* tl_skip, const int32_t* tl_heavy, int n_heavy, int heavy_parts,
                                     float* part_ws, int64_t part_ws_floats,
                                     int BH, int H, int T, int S, int E, int M,
-                                    float softmax_temp, int key_major, void* stream);
+                                    float softmax_temp, int key_major, float dropout_p, uint64_t dropout_seed,
+                                    void* stream);
 
 /* Scatterbrain attention on a block-sparse support (ref: src/models/attention/sbblocksparse_attention.py:109-213
- * for need_weights = False, no dropout, no masks): as flyhip_sblocal_fwd with one part per query tile, but the
+ * for need_weights = False, no masks): as flyhip_sblocal_fwd with one part per query tile, but the
  * exact part covers the nonzero blocks of a layout (16 x 16 or 32 x 32) instead of a band.  Key-side inputs (kfeat,
  * chunk_scale, kv, ksum, kmax) from flyhip_sb_kv_reduce.  tl_ptr (H * ceil(T/64) + 1), tl_inner, tl_mask (4 per
  * entry): per (head, 64-query tile) the 32-key tiles that any of its queries sees on the support, and per entry and
@@ -296,7 +298,10 @@ int flyhip_sbblocksparse_bwd_pieces(const void* outer_images, const void* inner_
  * walked in heavy_parts parts (2..64) by the first workgroups of the launch and finished by a merge launch; those
  * tiles carry the entry -1 - tile in tl_order so that no workgroup takes them whole, and every block-row of such
  * a tile must have at least one block.  Scratch for them: part_ws of B*n_heavy*heavy_parts*64*(D+5) floats and qfeat of
- * B*n_heavy*64*m floats (both NULL when n_heavy == 0).  float32 only; T, S multiples of 16. */
+ * B*n_heavy*64*m floats (both NULL when n_heavy == 0).  float32 only; T, S multiples of 16.
+ * dropout_p in [0, 1), dropout_seed: the dropout of the exact weights of sbblocksparse_attention.py:200 (the low-rank
+ * part and the normaliser see none), by the hash mask that flyhip_sblocal_forward documents;
+ * flyhip_sbblocksparse_bwd_pieces takes the same two values and forms the mask again. */
 int flyhip_sbblocksparse_fwd(const void* q, const void* k, const void* v, const float* proj,
                              const void* kfeat, const float* chunk_scale,
                              const float* kv, const float* ksum, const float* kmax,
@@ -309,7 +314,7 @@ int flyhip_sbblocksparse_fwd(const void* q, const void* k, const void* v, const 
                              int64_t k_sb, int64_t k_sh, int64_t k_ss,
                              int64_t v_sb, int64_t v_sh, int64_t v_ss,
                              int64_t o_sb, int64_t o_sh, int64_t o_ss,
-                             float softmax_temp, int dtype, void* stream);
+                             float softmax_temp, int dtype, float dropout_p, uint64_t dropout_seed, void* stream);
 
 /* Plain local attention, no random features (ref: src/models/attention/local_attention.py:68-92;
  * fast_transformers.local_product): out[i] = softmax over the band -(lc/2) <= s - i < (lc+1)/2, s below

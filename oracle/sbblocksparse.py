@@ -25,9 +25,12 @@ def support_mask(layout, block):
     return layout.bool().repeat_interleave(block, dim=1).repeat_interleave(block, dim=2)
 
 
-def sbblocksparse_attention(query, key, value, projection_matrix, layout, block, softmax_temp=None):
+def sbblocksparse_attention(query, key, value, projection_matrix, layout, block, softmax_temp=None,
+                            dropout_multiplier=None):
     """query (B,T,H,E), key (B,S,H,E), value (B,S,H,D) -> out (B,T,H,D), log_normalization (B,H,T,1).
-    Same op sequence as the reference layer (sbblocksparse_attention.py:161-212), dense."""
+    Same op sequence as the reference layer (sbblocksparse_attention.py:161-212), dense.
+    dropout_multiplier: None, or (B,H,T,S) -- the mask of nn.Dropout times 1 / (1 - p); it multiplies
+    exp(QK - log_normalization) and nothing else (:196-200)."""
     B, T, H, E = query.shape
     t = softmax_temp or 1 / math.sqrt(E)
     q = query.permute(0, 2, 1, 3)
@@ -47,7 +50,10 @@ def sbblocksparse_attention(query, key, value, projection_matrix, layout, block,
     lr_log_norm = torch.log((qk1.unsqueeze(-1) - dots_prime_sum).clamp_min(1e-24)) + prime_log_scale   # :189-190
     log_norm = torch.logaddexp(QK_lse, lr_log_norm)                                   # :191
     prime_scale = torch.exp(prime_log_scale - log_norm)                               # :193
-    dots = (torch.exp(QK - log_norm) - dots_prime * prime_scale) * mask               # :200
+    exact = torch.exp(QK - log_norm)
+    if dropout_multiplier is not None:
+        exact = exact * dropout_multiplier
+    dots = (exact - dots_prime * prime_scale) * mask                                  # :200
     out = dots @ v + qkv * prime_scale                                                # :203-204
     return out.permute(0, 2, 1, 3), log_norm
 

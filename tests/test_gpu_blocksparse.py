@@ -928,6 +928,47 @@ def test_sbblocksparse_gradients_on_the_kernels(B, H, T, S, E, D, m, seed):
         assert got.shape == ref.shape and rel_err(got, ref) <= 2e-4, rel_err(got, ref)
 
 
+@pytest.mark.parametrize('block,p_drop', [(32, 0.25), (16, 0.1)])
+def test_sbblocksparse_dropout_inside_the_kernels(block, p_drop):
+    """Training-mode dropout of SBBlockSparseAttention (sbblocksparse_attention.py:196-200: of the exact weights only)
+    inside the fused forward and, for 32 x 32 blocks, the backward kernels: the mask is the hash of (seed, batch, head,
+    query, key) restated in oracle.sblocal.dropout_keep, handed to the oracle as nn.Dropout's multiplier.  16 x 16
+    blocks have no backward kernels: forward only (a training step there runs op by op with torch's dropout)."""
+    from fly_amd import SBBlockSparseAttention, FlatBlockButterflySparsityConfig
+    from oracle import sbblocksparse as osbb
+    from oracle.sblocal import dropout_keep
+    B, T, H, E = 2, 256, 1, 64
+    print('case', block, p_drop, flush=True)
+    torch.manual_seed(0)
+    layer = SBBlockSparseAttention(FlatBlockButterflySparsityConfig(4, 2, block=block), dim_heads=E, nb_features=64,
+                                   attention_dropout=p_drop, max_seq_length=T).to(DEV).train()
+    g = torch.Generator().manual_seed(6)
+    q, k, v, w = (torch.randn(B, T, H, E, generator=g) for _ in range(4))
+    q, k = q * E ** -0.25 * 2, k * E ** -0.25 * 2
+    train = block == 32
+    qg, kg, vg = (x.to(DEV).requires_grad_(train) for x in (q, k, v))
+    torch.manual_seed(9)
+    out, _ = layer(qg, kg, vg)
+    seed = layer.last_dropout_seed
+    assert seed is not None and len(layer.fused_tables) == 1 and len(layer.ops_cache) == 0
+    P = layer.feature_map.projection_matrix.cpu().double()
+    qd, kd, vd = (x.double().requires_grad_() for x in (q, k, v))
+    mult = dropout_keep(seed, p_drop, B, H, T, T)
+    ref_out, _ = osbb.sbblocksparse_attention(qd, kd, vd, P, layer.get_layout(T), block, dropout_multiplier=mult)
+    assert rel_err(out, ref_out) <= 1e-4, rel_err(out, ref_out)
+    plain_ref, _ = osbb.sbblocksparse_attention(qd, kd, vd, P, layer.get_layout(T), block)
+    assert rel_err(out, plain_ref) > 1e-2
+    if train:
+        assert len(layer.backward_tables) == 1
+        (out * w.to(DEV)).sum().backward()
+        (ref_out * w.double()).sum().backward()
+        for got, ref in ((qg.grad, qd.grad), (kg.grad, kd.grad), (vg.grad, vd.grad)):
+            assert rel_err(got, ref) <= 2e-4, rel_err(got, ref)
+    with torch.no_grad():
+        plain, _ = layer.eval()(qg, kg, vg)
+    assert layer.last_dropout_seed is None and rel_err(plain, plain_ref) <= 1e-4
+
+
 def test_sbblocksparse_module_trains_on_the_fused_kernels():
     """SBBlockSparseAttention with gradients: the forward stays on the fused kernels and the backward walks the
     layout's blocks; gradients of query, key and value against autograd through the oracle, and against the op-by-op
