@@ -176,9 +176,13 @@ class LocalAttention(nn.Module):
         if key_padding_mask is not None and not bool(key_padding_mask.all_ones):
             lengths = key_padding_mask.lengths
         if not need_weights:
+            # float16 inputs are widened to float32 for the kernels (exact) and the result goes back to float16
+            in_dtype = query.dtype
+            if in_dtype == torch.float16:
+                query, key, value = query.float(), key.float(), value.float()
             out = local_attention_fn(query, key, value, self.local_context, softmax_temp=self.softmax_temp,
                                      key_lengths=lengths, dropout=dropout)
-            return out, None
+            return (out.to(in_dtype) if in_dtype == torch.float16 else out), None
         B, T, H, E = query.shape
         S = key.shape[1]
         if B * H * T * S > self.max_weight_elements:

@@ -491,10 +491,18 @@ class SBLocalAttention(nn.Module):
         if key_padding_mask is not None and not bool(key_padding_mask.all_ones):
             lengths = key_padding_mask.lengths          # raises ValueError unless a length mask
         self.feature_map.new_feature_map(query.device)
+        # float16 inputs (the reference's modules take whatever dtype autocast hands them) are widened to float32
+        # for the kernels -- exact, and the feature exponentials do not fit float16's range -- and the result goes
+        # back to float16; the casts are ordinary autograd nodes
+        in_dtype = query.dtype
+        if in_dtype == torch.float16:
+            query, key, value = query.float(), key.float(), value.float()
         out, log_norm = sblocal_attention_fn(query, key, value, self.feature_map.projection_matrix,
                                              self.local_context, softmax_temp=self.softmax_temp,
                                              key_lengths=lengths, cache=self._scratch_cache,
                                              exact_fp32=self.exact_fp32, dropout_p=dropout_p, dropout_seed=dropout_seed)
+        if in_dtype == torch.float16:
+            out = out.to(in_dtype)
         self.last_log_normalization = log_norm.detach()
         attn = None
         if need_weights or return_attn_unnormalized:

@@ -452,6 +452,38 @@ def test_gradients_at_benchmark_sizes_match_autograd_through_the_oracle(case):
         assert rel_err(got, ref) <= 2e-4, (name, rel_err(got, ref))
 
 
+def test_float16_inputs_are_widened_for_the_kernels():
+    """SBLocalAttention and LocalAttention with float16 inputs (the dtype autocast hands the reference's modules):
+    widened to float32 for the kernels, results and gradients back in float16 -- against the oracle on the same
+    (float16-rounded) inputs, to float16's rounding of the result."""
+    from fly_amd import SBLocalAttention, LocalAttention, LengthMask
+    dev = torch.device('cuda:0')
+    B, T, S, H, E, lc = 2, 200, 232, 2, 64, 64
+    g = torch.Generator().manual_seed(41)
+    q, k, v = (torch.randn(B, L, H, E, generator=g).half() for L in (T, S, S))
+    q, k = q * 0.4, k * 0.4
+    w = torch.randn(B, T, H, E, generator=g)
+    lengths = torch.tensor([S, 150])
+    mask = LengthMask(lengths.to(dev), max_len=S)
+    sb = SBLocalAttention(lc, dim_heads=E, nb_features=64).to(dev).eval()
+    loc = LocalAttention(lc).to(dev).eval()
+    qg, kg, vg = (x.to(dev).requires_grad_() for x in (q, k, v))
+    out, _ = sb(qg, kg, vg, key_padding_mask=mask)
+    assert out.dtype == torch.float16
+    P = sb.feature_map.projection_matrix.cpu().double()
+    qd, kd, vd = (x.double().requires_grad_() for x in (q, k, v))
+    ref, _ = osb.sblocal_attention(qd, kd, vd, P, lc, key_lengths=lengths)
+    assert rel_err(out.float(), ref) <= 1e-3, rel_err(out.float(), ref)
+    (out.float() * w.to(dev)).sum().backward()
+    (ref * w.double()).sum().backward()
+    for got, want in ((qg.grad, qd.grad), (kg.grad, kd.grad), (vg.grad, vd.grad)):
+        assert got.dtype == torch.float16 and rel_err(got.float(), want) <= 2e-3, rel_err(got.float(), want)
+    with torch.no_grad():
+        out2, _ = loc(qg, kg, vg, key_padding_mask=mask)
+    assert out2.dtype == torch.float16
+    assert rel_err(out2.float(), osb.local_attention(q.double(), k.double(), v.double(), lc, key_lengths=lengths)) <= 1e-3
+
+
 @pytest.mark.parametrize('dtype,tol', [(torch.float32, 1e-4), (torch.bfloat16, 3e-2)])
 def test_local_attention_module_gradients(dtype, tol):
     """LocalAttention is trainable: forward on the fused kernel, gradients against autograd through the
