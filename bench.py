@@ -215,13 +215,18 @@ def bench_blocksparse(steps, warmup):
             if done % 8 == 0:
                 torch.cuda.synchronize()
         torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(steps):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / steps
+        # median of three batches: one stall of the issuing thread (tens of milliseconds now and then on a shared
+        # host) would otherwise land in a single stage's figure
+        reps = []
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(steps):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            reps.append(e0.elapsed_time(e1) / steps)
+        return sorted(reps)[1]
 
     qk = sdd(q, k)
     flops = 2 * B * nnz * block * block * d

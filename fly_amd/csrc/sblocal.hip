@@ -1760,6 +1760,9 @@ template <int E, int M> constexpr size_t fwd_b32_smem() { return fwd_bf16_smem<E
 #ifndef B32_WAVES
 #define B32_WAVES 4
 #endif
+#ifndef FLY_B32_FUSED_TILE
+#define FLY_B32_FUSED_TILE 1
+#endif
 
 template <int E, int D, int M, bool SPLIT, int NW>
 __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2))) void sblocal_fwd_b32_kernel(FwdArgs a) {
@@ -1779,7 +1782,9 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
     extern __shared__ __attribute__((aligned(128))) float smem[];
     uint16_t* lds = reinterpret_cast<uint16_t*>(smem);
 
-    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c = lane & 31, h = lane >> 5;
+    const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6), c = lane & 31, h = lane >> 5;
+    // (the wave index as a scalar: the tests on the wave's range of queries -- does a tile touch its band, does it lie inside
+    //  every query's band -- are then scalar branches, and the accumulators are not copied around exec-masked regions)
     if (SPLIT && (int)blockIdx.x >= a.band_wgs) {       // combine role, see sblocal_fwd_kernel
         const int ci = blockIdx.x - a.band_wgs;
         sb_combine_body(smem, a.kv_part, a.part_max, const_cast<float*>(a.kv), const_cast<float*>(a.ksum),
@@ -2019,9 +2024,13 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
                 mx = fmaxf(mx, ok[e] ? s1[e] : -INFINITY);
             }
             mx = pair32_max(mx) * sc;                               // sc > 0
-            // (the reference exponent is raised only when a tile exceeds it by more than 2^8)
-            if (__builtin_amdgcn_ballot_w64(mx > m_run + 8.f) != 0) {      // wave-uniform
-                const float m_new = fmaxf(m_run, mx);
+            // The reference exponent is raised only when a tile exceeds it by more than 2^8 (wave-uniform vote), but the
+            // rescale itself is unconditional (by 1 when nothing was raised): inside a branch the compiler gave the scaled
+            // accumulators new registers and copied all 32 of them on the usual path and back at the end of every tile
+            // (33 multiplies instead of 32 two-register moves and two waits for the matrix pipe).
+            {
+                const bool grow = __builtin_amdgcn_ballot_w64(mx > m_run + 8.f) != 0;
+                const float m_new = grow ? fmaxf(m_run, mx) : m_run;
                 const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
                 m_run = m_new;
                 ze *= alpha;
@@ -2059,6 +2068,125 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
             }
         }
     };
+    // Both phases of a tile in one piece, for waves that are not skewed.  The overlap products q'.k' of a tile are one chain of
+    // FS MFMAs on one accumulator: each waits for the one before it, and a wave that has nothing else to issue waits with
+    // it.  Everything of the softmax that needs only the scores -- maximum, reference exponent, rescale, the
+    // exponentials and their sum -- is therefore placed between the links of that chain (sched_group_barrier: one MFMA,
+    // then a share of the vector instructions), and only the subtraction of the overlap follows it.
+    auto tile_phase = [&](int kt, int stage, float cs) __attribute__((always_inline)) {
+        if (!touches(kt)) return;
+        const char* Ks = reinterpret_cast<const char*>(lds) + stage * STAGE_BYTES;
+        const char* Fs = Ks + K_BYTES;
+        const char* Vt = Fs + F_BYTES;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) { s1[e] = 0.f; s2[e] = 0.f; }
+        uint4 kf[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) kf[ks] = *reinterpret_cast<const uint4*>(Ks + koff4[ks & 3] + 128 * (ks >> 2));
+        constexpr int FBATCH = FS >= 16 ? 2 : (FS < 4 ? FS : 4), NBATCH = FS / FBATCH;
+        static_assert(FS % FBATCH == 0, "whole batches");
+        uint4 ff[2][FBATCH];
+#pragma unroll
+        for (int s = 0; s < FBATCH; ++s) ff[0][s] = *reinterpret_cast<const uint4*>(Fs + foff4[s & 3] + 128 * (s >> 2));
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) s1 = mma32_bf16(kf[ks], qb[ks], s1);
+        __builtin_amdgcn_sched_barrier(0);
+        const int s_base = kt * TK;
+        const float wc = __builtin_amdgcn_exp2f((cs - kmax) * LOG2E);
+        const bool inside = s_base >= max(qw0 + 31 - lc_lo, 0) && s_base + TK <= min(qw0 + lc_hi, len) && qw0 + 31 < a.T;
+        float p[16];
+        float ovs = 0.f;
+        auto soft = [&](auto masked_t) __attribute__((always_inline)) {
+            constexpr bool MASKED = decltype(masked_t)::value;
+            // the chain, its fragments a batch ahead (V^T fragments with the last batch)
+#pragma unroll
+            for (int bt = 0; bt < NBATCH; ++bt) {
+                if (bt + 1 < NBATCH) {
+#pragma unroll
+                    for (int s = 0; s < FBATCH; ++s) {
+                        const int sn = (bt + 1) * FBATCH + s;
+                        ff[(bt + 1) & 1][s] = *reinterpret_cast<const uint4*>(Fs + foff4[sn & 3] + 128 * (sn >> 2));
+                    }
+                } else {
+#pragma unroll
+                    for (int db = 0; db < DB; ++db)
+#pragma unroll
+                        for (int t = 0; t < 2; ++t)
+                            vf[db][t] = *reinterpret_cast<const uint4*>(Vt + (32 * db + c) * V_ROW + x3_swz(32 * db + c, 2 * t + h, V_ROW) * 16);
+                }
+#pragma unroll
+                for (int s = 0; s < FBATCH; ++s) s2 = mma32_bf16(ff[bt & 1][s], qfb[bt * FBATCH + s], s2);
+            }
+            // in its shadow: what the scores alone decide
+            bool ok[16];
+            float mx = -INFINITY;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int s = s_base + 8 * (e >> 2) + 4 * h + (e & 3);
+                ok[e] = !MASKED || (unsigned)(s - smin) < span;
+                mx = fmaxf(mx, ok[e] ? s1[e] : -INFINITY);
+            }
+            mx = pair32_max(mx) * sc;                               // sc > 0
+            {   // (see soft_phase: the vote is wave-uniform, the rescale unconditional)
+                const bool grow = __builtin_amdgcn_ballot_w64(mx > m_run + 8.f) != 0;
+                const float m_new = grow ? fmaxf(m_run, mx) : m_run;
+                const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+                m_run = m_new;
+                ze *= alpha;
+#pragma unroll
+                for (int db = 0; db < DB; ++db) oacc[db] *= alpha;
+            }
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                p[e] = ok[e] ? __builtin_amdgcn_exp2f(__builtin_fmaf(s1[e], sc, -m_run)) : 0.f;
+                ze += p[e];
+            }
+            // the order asked of the scheduler: per batch its LDS reads, then link by link one MFMA and a share of the
+            // vector work
+            constexpr int VSHARE = (MASKED ? 176 : 144) / FS;
+#pragma unroll
+            for (int bt = 0; bt + 1 < NBATCH; ++bt) {
+                __builtin_amdgcn_sched_group_barrier(0x100, FBATCH, 0);
+#pragma unroll
+                for (int s = 0; s < FBATCH; ++s) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, VSHARE, 0);
+                }
+            }
+            __builtin_amdgcn_sched_group_barrier(0x100, 2 * DB, 0);
+#pragma unroll
+            for (int s = 0; s < FBATCH; ++s) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, VSHARE, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            const float beta = wc * __builtin_amdgcn_exp2f(c0 - m_run);      // scale of the overlap term
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const float ov = ok[e] ? s2[e] : 0.f;
+                ovs += ov;
+                p[e] = __builtin_fmaf(-ov, beta, p[e]);
+            }
+        };
+        if (inside) soft(std::false_type{}); else soft(std::true_type{});
+        zp += ovs * wc;
+        const bool two = TWO_PIECE && second_piece_wanted(zp * __builtin_amdgcn_exp2f(c0 - m_run), ze);
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const uint4 pb_ = make_uint4(pack_bf16x2(p[4 * t], p[4 * t + 1]), pack_bf16x2(p[4 * t + 2], p[4 * t + 3]),
+                                         pack_bf16x2(p[4 * (2 + t)], p[4 * (2 + t) + 1]), pack_bf16x2(p[4 * (2 + t) + 2], p[4 * (2 + t) + 3]));
+#pragma unroll
+            for (int db = 0; db < DB; ++db) oacc[db] = mma32_bf16(vf[db][t], pb_, oacc[db]);
+            if (two) {                                           // wave-uniform
+                const uint4 pl_ = make_uint4(pack_rest(p[4 * t], p[4 * t + 1], pb_.x), pack_rest(p[4 * t + 2], p[4 * t + 3], pb_.y),
+                                             pack_rest(p[4 * (2 + t)], p[4 * (2 + t) + 1], pb_.z),
+                                             pack_rest(p[4 * (2 + t) + 2], p[4 * (2 + t) + 3], pb_.w));
+#pragma unroll
+                for (int db = 0; db < DB; ++db) oacc[db] = mma32_bf16(vf[db][t], pl_, oacc[db]);
+            }
+        }
+    };
     const bool late = NW > 4 && w >= NW / 2;      // wave-uniform: this wave runs half a tile behind
     float cs_prev = 0.f;                          // chunk scale of the tile a late wave still owes its softmax
     // (the first pass, kt = kt_lo - 1, only brings the first tile in)
@@ -2075,8 +2203,12 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
         }
         if (kt >= kt_lo) {
             if (!late) {
+#if FLY_B32_FUSED_TILE
+                tile_phase(kt, cur, cscale);
+#else
                 score_phase(kt, cur);
                 soft_phase(kt, cscale);
+#endif
             } else {
                 if (kt > kt_lo) soft_phase(kt - 1, cs_prev);
                 score_phase(kt, cur);
