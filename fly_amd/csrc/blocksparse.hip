@@ -1382,7 +1382,6 @@ template <int CPR> __device__ __forceinline__ int attn_vslot(int row, int c) {
 }
 template <typename T, int KS, int NW, bool MASKED, bool DROP = false>     // head dim 32*KS, NW block-rows (waves) per workgroup
 __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
-    static_assert(!DROP || MASKED, "the dropout variant is built on the general (masked) softmax");
     constexpr int D = 32 * KS, DT = D / 16, RB = 2 * D;   // RB: bytes of a tile row
     // block-columns per step: what 64 KB of LDS hold twice over -- half of that for workgroups of four waves at 64 dims,
     // of which a compute unit then holds four (the registers allow it) instead of two
@@ -1479,6 +1478,16 @@ __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
                 for (int ks = 0; ks < KS; ++ks) sc[kt][qt] = mma32<T>(fk[kt][ks], fq[qt][ks], sc[kt][qt]);
             }
     };
+    // DROP: the probabilities that go to the product with V, the dropped ones zeroed (the denominator sums all of them)
+    auto dropped = [&](float (&e0)[4], float (&e1)[4], uint32_t row_hash, int inner) __attribute__((always_inline)) {
+        const uint32_t col0 = (uint32_t)inner * 32u + 4u * g;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if (!drop_keep(row_hash, col0 + i, a.drop_thresh)) e0[i] = 0.f;
+            if (!drop_keep(row_hash, col0 + 16u + i, a.drop_thresh)) e1[i] = 0.f;
+        }
+        return uintx4{pack2<T>(e0[0], e0[1]), pack2<T>(e0[2], e0[3]), pack2<T>(e1[0], e1[1]), pack2<T>(e1[2], e1[3])};
+    };
     // online softmax of sc and O^T += V^T P with the V tile that follows the K tile at `tile`; `inner` = its block-column
     auto soft_pv = [&](const char* tile, int inner) __attribute__((always_inline)) {
         // A operand: column d = 16dt + r16 of V, keys 4g .. 4g+3 and 16+4g .. 16+4g+3
@@ -1514,6 +1523,7 @@ __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
                     e1[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s1[i], scale2, nm));
                 }
                 pb[qt] = uintx4{pack2<T>(e0[0], e0[1]), pack2<T>(e0[2], e0[3]), pack2<T>(e1[0], e1[1]), pack2<T>(e1[2], e1[3])};
+                if (DROP) pd[qt] = dropped(e0, e1, drop_row[qt], inner);
             }
         } else {
             floatx4 mk[2] = {Frag<float>::zero(), Frag<float>::zero()};
@@ -1545,16 +1555,7 @@ __global__ __launch_bounds__(64 * NW) void bs_attn32_kernel(const AttnArgs a) {
                     e1[i] = __builtin_amdgcn_exp2f(t1[i] - mref);
                 }
                 pb[qt] = uintx4{pack2<T>(e0[0], e0[1]), pack2<T>(e0[2], e0[3]), pack2<T>(e1[0], e1[1]), pack2<T>(e1[2], e1[3])};
-                if (DROP) {
-                    // the dropped probabilities go to the product with V only: the denominator below sums all of them
-                    const uint32_t col0 = (uint32_t)inner * 32u + 4u * g;
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        if (!drop_keep(drop_row[qt], col0 + i, a.drop_thresh)) e0[i] = 0.f;
-                        if (!drop_keep(drop_row[qt], col0 + 16u + i, a.drop_thresh)) e1[i] = 0.f;
-                    }
-                    pd[qt] = uintx4{pack2<T>(e0[0], e0[1]), pack2<T>(e0[2], e0[3]), pack2<T>(e1[0], e1[1]), pack2<T>(e1[2], e1[3])};
-                }
+                if (DROP) pd[qt] = dropped(e0, e1, drop_row[qt], inner);
             }
         }
         // the row sums come from the matrix pipe as well: a row of ones times the rounded probabilities
@@ -2396,7 +2397,8 @@ static int bs_attn_checked(const void* q, const void* k, const void* v, void* ou
     args.drop_scale = drop.scale;
 #define ATTN_LAUNCH(T, KS, NW)                                                                                  \
     do {                                                                                                        \
-        if (dropping) hipLaunchKernelGGL((bs_attn32_kernel<T, KS, NW, true, true>), grid, dim3(64 * NW), 0, st, args); \
+        if (dropping && masked) hipLaunchKernelGGL((bs_attn32_kernel<T, KS, NW, true, true>), grid, dim3(64 * NW), 0, st, args); \
+        else if (dropping) hipLaunchKernelGGL((bs_attn32_kernel<T, KS, NW, false, true>), grid, dim3(64 * NW), 0, st, args); \
         else if (masked) hipLaunchKernelGGL((bs_attn32_kernel<T, KS, NW, true>), grid, dim3(64 * NW), 0, st, args);  \
         else hipLaunchKernelGGL((bs_attn32_kernel<T, KS, NW, false>), grid, dim3(64 * NW), 0, st, args);        \
     } while (0)

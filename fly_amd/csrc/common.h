@@ -317,15 +317,18 @@ __device__ __forceinline__ void split3_4(floatx4 x, uint2& h, uint2& m, uint2& l
 
 // Dropout of attention weights without a stored mask: whether the pair (row, col) is kept is a hash of (seed, row, col),
 // so the backward forms the same mask again from the seed.  row_hash depends on the row alone (one query: once per
-// lane); the column enters through a multiply-add and the 32-bit finaliser of MurmurHash3 (full avalanche).  A pair is
-// kept when its hash is at least thresh = floor(p 2^32); kept weights are scaled by 1 / (1 - p).
+// lane).  A pair of neighbouring columns (2c, 2c + 1) shares one 32-bit hash -- the pair index enters through a
+// multiply-add and the 32-bit finaliser of MurmurHash3 (full avalanche) -- and each column takes one 16-bit half of it:
+// the hash's two multiplies are quarter-rate instructions, and a lane's columns come in consecutive runs.  A pair is
+// kept when its half is at least thresh = floor(p 2^16); kept weights are scaled by 1 / (1 - thresh 2^-16).
 __device__ __forceinline__ uint32_t drop_mix(uint32_t h) {
     h ^= h >> 16; h *= 0x85EBCA6Bu; h ^= h >> 13; h *= 0xC2B2AE35u; h ^= h >> 16;
     return h;
 }
 __device__ __forceinline__ uint32_t drop_row_hash(uint32_t seed, uint32_t row) { return drop_mix(row * 0x9E3779B1u + seed); }
 __device__ __forceinline__ bool drop_keep(uint32_t row_hash, uint32_t col, uint32_t thresh) {
-    return drop_mix(row_hash + col * 0x632BE5ABu) >= thresh;
+    const uint32_t h = drop_mix(row_hash + (col >> 1) * 0x632BE5ABu);
+    return ((col & 1u) ? (h >> 16) : (h & 0xffffu)) >= thresh;
 }
 // host side: the kernels' dropout arguments from a probability and a 64-bit seed (p = 0: thresh = 0 = off)
 struct DropArgs { uint32_t seed, thresh; float scale; };
@@ -333,10 +336,10 @@ inline DropArgs drop_args(float p, uint64_t seed) {
     DropArgs d{0, 0, 1.f};
     if (p > 0.f) {
         d.seed = (uint32_t)seed ^ ((uint32_t)(seed >> 32) * 0x9E3779B1u);
-        const double t = (double)p * 4294967296.0;
-        d.thresh = t >= 4294967295.0 ? 4294967295u : (uint32_t)t;
+        const double t = (double)p * 65536.0;
+        d.thresh = t >= 65535.0 ? 65535u : (uint32_t)t;
         if (d.thresh == 0) d.thresh = 1;
-        d.scale = 1.f / (1.f - p);
+        d.scale = (float)(1.0 / (1.0 - d.thresh / 65536.0));       // of the probability actually realised: the mean stays exact
     }
     return d;
 }

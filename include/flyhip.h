@@ -126,8 +126,9 @@ int flyhip_sblocal_fwd(const void* q, const void* k, const void* v, const float*
  * time); pass the same flags to both functions.
  * dropout_p in [0, 1), dropout_seed: dropout of the exact weights exp(QK - log_normalization) as in
  * sblocal_attention.py:119 (the normaliser and the low-rank part see none).  No mask is stored: whether the weight of
- * (query i, key s) of (batch b, head h) is kept is a hash of (seed, (b H + h) T + i, s), and kept weights are scaled by
- * 1 / (1 - p); flyhip_sblocal_bwd_pieces forms the same mask from the same seed.  float32 inputs with head dims up to
+ * (query i, key s) of (batch b, head h) is kept is a hash of (seed, (b H + h) T + i, s) -- written out at
+ * flyhip_bs_attn_dropout, with L = T -- and kept weights are scaled by 1 / (1 - p); flyhip_sblocal_bwd_pieces forms
+ * the same mask from the same seed.  float32 inputs with head dims up to
  * 64 and up to 128 features (the kernels on bf16 pieces), not with FLYHIP_SB_EXACT_FP32; 0 = no dropout.
  * Arguments otherwise as for flyhip_sb_kv_reduce / flyhip_sblocal_fwd. */
 #define FLYHIP_SB_EXACT_FP32 1
@@ -508,9 +509,10 @@ int flyhip_bs_attn_masks(const void* q, const void* k, const void* v, void* out,
  * src/models/attention/blocksparse_attention.py:160, `dsd_nn(self.dropout(attn), v)`; the constructor's default
  * attention_dropout is 0.1, :31): every probability is dropped with probability dropout_p in [0, 1) after the softmax
  * (the denominator sums all of them) and the kept ones are scaled by 1 / (1 - dropout_p).  No mask tensor exists:
- * (batch z, head h, query i, key j) is kept iff mix(mix(((z H + h) L + i) * 0x9E3779B1 + s) + j * 0x632BE5AB) >=
- * floor(dropout_p 2^32), L = 32 * brows_per_head, mix = the 32-bit finaliser of MurmurHash3, s = the 64-bit seed
- * folded to 32 bits (low ^ high * 0x9E3779B1); flyhip_bs_sdd_prob_dsoftmax_dropout forms the same mask again.
+ * keys 2c and 2c + 1 of (batch z, head h, query i) share the 32-bit hash mix(mix(((z H + h) L + i) * 0x9E3779B1 + s)
+ * + c * 0x632BE5AB) -- L = 32 * brows_per_head, mix = the 32-bit finaliser of MurmurHash3, s = the 64-bit seed folded
+ * to 32 bits (low ^ high * 0x9E3779B1) -- key 2c takes its low and key 2c + 1 its high 16 bits, and a probability is
+ * kept iff its half >= floor(dropout_p 2^16); flyhip_bs_sdd_prob_dsoftmax_dropout forms the same mask again.
  * lse2 is that of the undropped softmax.  dropout_p = 0 is flyhip_bs_attn_masks. */
 int flyhip_bs_attn_dropout(const void* q, const void* k, const void* v, void* out, float* lse2,
                            const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,

@@ -157,20 +157,23 @@ def _mix32(h):
 
 
 def dropout_keep(seed, p, B, H, T, S):
-    """The dropout multiplier of the HIP band kernels, restated on the host so that tests can hand the kernels' own
-    mask to the reference algebra: (B,H,T,S) float64, 1 / (1 - p) where the weight of (query i, key s) of (batch b,
-    head h) is kept and 0 where it is dropped.  Kept iff mix(mix((b H + h) T + i) * 0x9E3779B1 + seed') + s * 0x632BE5AB)
-    >= floor(p 2^32), seed' the 64-bit seed folded to 32 bits (fly_amd/csrc/common.h: drop_args, drop_row_hash,
-    drop_keep).  This has no counterpart in the reference, whose mask comes from torch's generator
-    (sblocal_attention.py:119); the statistics -- independent keeps with probability 1 - p -- are what both share."""
+    """The dropout multiplier of the HIP kernels, restated on the host so that tests can hand the kernels' own
+    mask to the reference algebra: (B,H,T,S) float64, 1 / (1 - p') where the weight of (query i, key s) of (batch b,
+    head h) is kept and 0 where it is dropped, p' = floor(p 2^16) 2^-16 the probability actually realised.  A pair of neighbouring keys (2c, 2c + 1) shares the 32-bit hash
+    mix(mix(((b H + h) T + i) * 0x9E3779B1 + seed') + c * 0x632BE5AB), key 2c takes its low and key 2c + 1 its high 16
+    bits, and a weight is kept iff its half >= floor(p 2^16); seed' is the 64-bit seed folded to 32 bits
+    (fly_amd/csrc/common.h: drop_args, drop_row_hash, drop_keep).  This has no counterpart in the reference, whose mask
+    comes from torch's generator (sblocal_attention.py:119); the statistics -- independent keeps with probability 1 - p
+    (p rounded down to a multiple of 2^-16) -- are what both share."""
     m = 0xFFFFFFFF
     seed32 = (seed & m) ^ (((seed >> 32) * 0x9E3779B1) & m)
-    thresh = min(max(int(p * 4294967296.0), 1), 0xFFFFFFFF) if p > 0 else 0
+    thresh = min(max(int(p * 65536.0), 1), 0xFFFF) if p > 0 else 0
     rows = torch.arange(B * H * T, dtype=torch.int64)
     row_hash = _mix32((rows * 0x9E3779B1 + seed32) & m).view(B, H, T, 1)
     cols = torch.arange(S, dtype=torch.int64).view(1, 1, 1, S)
-    h = _mix32((row_hash + cols * 0x632BE5AB) & m)
-    return (h >= thresh).to(torch.float64) / (1.0 - p)
+    h = _mix32((row_hash + (cols >> 1) * 0x632BE5AB) & m)
+    half = torch.where((cols & 1) == 1, h >> 16, h & 0xFFFF)
+    return (half >= thresh).to(torch.float64) / (1.0 - thresh / 65536.0)
 
 
 def sblocal_attention(query, key, value, projection_matrix, local_context, softmax_temp=None,
