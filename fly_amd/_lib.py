@@ -30,7 +30,7 @@ SIGNATURES = {
     'flyhip_sblocal_bwd_prep': [c_vp] * 18 + [c_i64] + [c_int] * 7 + [c_float, c_vp],
     'flyhip_sblocal_bwd_pieces': [c_vp] * 12 + [c_i64] + [c_int] * 7 + [c_float, c_int, c_float, c_u64, c_vp],
     'flyhip_sbblocksparse_bwd_pieces': [c_vp] * 15 + [c_int] * 2 + [c_vp, c_i64] + [c_int] * 6 + [c_float, c_int, c_float, c_u64, c_vp],
-    'flyhip_sbblocksparse_fwd': [c_vp] * 14 + [c_int] * 2 + [c_vp] * 4 + [c_int] * 8 + [c_i64] * 12 + [c_float, c_int, c_float, c_u64, c_vp],
+    'flyhip_sbblocksparse_fwd': [c_vp] * 15 + [c_int] * 2 + [c_vp] * 4 + [c_int] * 8 + [c_i64] * 12 + [c_float, c_int, c_float, c_u64, c_vp],
     'flyhip_local_fwd_lse': [c_vp] * 6 + [c_int] * 7 + [c_i64] * 12 + [c_float, c_int, c_vp],
     'flyhip_local_fwd_dropout': [c_vp] * 6 + [c_int] * 7 + [c_i64] * 12 + [c_float, c_int, c_float, c_u64, c_vp],
     'flyhip_local_fwd': [c_vp] * 5 + [c_int] * 7 + [c_i64] * 12 + [c_float, c_int, c_vp],

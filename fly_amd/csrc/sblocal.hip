@@ -3152,8 +3152,12 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
 // overlap (four), 5 D / 16 for P V (five; six with three V pieces) instead of (E + M + D) / 2 fp32 MFMAs of twice the duration.
 // A tile image is copied global -> registers -> LDS as it is (16-byte pieces in thread order), two LDS
 // stages.
-template <int E, int D, int M, bool SPLIT, bool DROPOUT = false>
+// LIST: the exact part lives on a block-sparse support instead of a band (see sblocal_fwd_kernel: the same lists of 32-key
+// tiles with a two-bit mask per wave and entry, the same start order, long lists walked in parts by the first workgroups
+// of the launch, which write un-normalised partials for sb_merge_kernel).  One part per ordinary tile: SPLIT is false.
+template <int E, int D, int M, bool SPLIT, bool DROPOUT = false, bool LIST = false>
 __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
+    static_assert(!(LIST && SPLIT), "a block-sparse support is walked with one part per tile (long lists: a runtime role)");
     typedef X3Tile<E, D, M> TL;
     constexpr int MH = M / 2, LDK = E + 4, LDV = D + 4;
     constexpr int FB = MH / 16, EC = E / 16, DB = D / 16, KB = TK / 16, KS = E / 32, FS = M / 32;
@@ -3164,11 +3168,12 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
     const int n_qt = (a.T + TQ - 1) / TQ;
-    const int n_items = a.B * a.H * n_qt * a.n_parts;
+    // (LIST: every workgroup has an item of the lists below; n_items = 0 keeps the band's mapping out of the way)
+    const int n_items = LIST ? 0 : a.B * a.H * n_qt * a.n_parts;
     const int per_xcd = (n_items + a.n_xcd - 1) / a.n_xcd;
     const bool tail = (int)blockIdx.x >= a.band_wgs;
     const int item = tail ? n_items : (blockIdx.x % a.n_xcd) * per_xcd + blockIdx.x / a.n_xcd;   // see sblocal_fwd_kernel
-    if (item >= n_items) {                             // workgroup-uniform
+    if (!LIST && item >= n_items) {                    // workgroup-uniform
         // Combine role, see sblocal_fwd_kernel: the workgroups behind the band workgroups, and the band range's own
         // padding (its size is a whole number of rounds over the XCDs), which would otherwise hold a slot for nothing
         if (!SPLIT) return;
@@ -3181,9 +3186,36 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
         FLY_PROF(7);
         return;
     }
-    const int part = item % a.n_parts;
-    const int qt = (item / a.n_parts) % n_qt;
-    const int bh = item / (a.n_parts * n_qt), b = bh / a.H, h = bh % a.H;
+    int part = LIST ? 0 : item % a.n_parts;
+    int qt = LIST ? 0 : (item / a.n_parts) % n_qt;
+    int bh = LIST ? 0 : item / (a.n_parts * n_qt);
+    // part_role: this workgroup writes an un-normalised partial instead of the result (always with SPLIT; with LIST the
+    // first workgroups of the launch, which walk the long lists in parts)
+    bool part_role = SPLIT;
+    long slot = 0;                  // long lists: index of the tile's partials and compact query features
+    if (LIST) {                     // (as in sblocal_fwd_kernel)
+        const int n_part_wgs = (a.B * a.n_heavy * a.n_parts + a.n_xcd - 1) / a.n_xcd * a.n_xcd;
+        if ((int)blockIdx.x < n_part_wgs) {
+            const int idx = blockIdx.x;
+            if (idx >= a.B * a.n_heavy * a.n_parts) return;            // workgroup-uniform
+            part_role = true;
+            part = idx % a.n_parts;
+            slot = idx / a.n_parts;
+            const int hq = a.tl_heavy[slot % a.n_heavy];
+            qt = hq % n_qt;
+            bh = (int)(slot / a.n_heavy) * a.H + hq / n_qt;
+        } else {
+            const int blk_id = blockIdx.x - n_part_wgs;
+            const int nbh = a.B * a.H, x = blk_id % a.n_xcd, i = blk_id / a.n_xcd;
+            const int mine = (nbh - x + a.n_xcd - 1) / a.n_xcd;            // (batch, head) pairs of this XCD
+            if (mine <= 0 || i >= mine * n_qt) return;                 // workgroup-uniform
+            const int rank = i / mine;
+            bh = x + a.n_xcd * (i % mine);
+            qt = a.tl_order ? a.tl_order[(bh % a.H) * n_qt + rank] : rank;
+            if (qt < 0) return;                                        // a long list: walked in parts by the first workgroups
+        }
+    }
+    const int b = bh / a.H, h = bh % a.H;
     const int q0 = qt * TQ;
     const int iq = q0 + 16 * w + r16;
     const bool qvalid = iq < a.T;
@@ -3206,6 +3238,28 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
         kt_lo = first;
         kt_hi = first + base + (part < extra ? 1 : 0);
     }
+    // LIST: the loop counter walks the tile's list; tile index and this wave's presence mask of an entry (bit h: the wave's
+    // 16 queries see keys 16 h .. 16 h + 15 of the tile) are read one iteration ahead of their use
+    const int32_t* tl_inner = nullptr;
+    const int32_t* tl_blk = nullptr;
+    int tile_cur = 0, tile_next = 0;
+    int pres_cur = 0, pres_next = 0;
+    bool seen_block = false;
+    if (LIST) {
+        int lp0 = a.tl_ptr[h * n_qt + qt];
+        kt_lo = 0;
+        kt_hi = a.tl_ptr[h * n_qt + qt + 1] - lp0;
+        if (part_role) {
+            const int base = kt_hi / a.n_parts, extra = kt_hi % a.n_parts;
+            lp0 += part * base + min(part, extra);
+            kt_hi = base + (part < extra ? 1 : 0);
+        }
+        tl_inner = a.tl_inner + lp0;
+        tl_blk = a.tl_blk + 4 * (long)lp0 + w;              // four masks per entry, one per wave
+        if (kt_hi > 0) { tile_cur = tl_inner[0]; pres_cur = tl_blk[0] & 3; }
+        if (kt_hi > 1) { tile_next = tl_inner[1]; pres_next = tl_blk[4] & 3; }
+    }
+    const int first_tile = LIST ? tile_cur : kt_lo;
 
     // tile images: flat copies, 16-byte pieces in thread order
     constexpr int NKV = (TL::KV_BYTES / 16 + NT - 1) / NT, NF = (TL::F_BYTES / 16 + NT - 1) / NT;
@@ -3246,9 +3300,9 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
             if (F_EXACT || tid + NT * j < TL::F_BYTES / 16)
                 dma_to_lds(gf + 16 * (tid + NT * j), lds + stage * TL::BYTES + TL::KV_BYTES + 16 * (NT * j + 64 * wv));
     };
-    if (kt_lo < kt_hi) fetch(kt_lo);
+    if (kt_lo < kt_hi) fetch(first_tile);
     const float* csp = a.chunk_scale + (long)bh * a.n_chunks;
-    float cscale = (kt_lo < kt_hi) ? csp[kt_lo * TK / CH] : 0.f;
+    float cscale = (kt_lo < kt_hi) ? csp[first_tile * TK / CH] : 0.f;
     const float kmax = SPLIT ? split_kmax(a.part_max, bh, a.n_split) : a.kmax[bh];
 
     // query operand: lane (r16, g) holds elements 16c + 4g + i of its query row
@@ -3319,6 +3373,12 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
             }
             __syncthreads();      // Ps is dead; the tile buffers may overwrite it
         }
+        if (LIST && part_role && part == 0) {
+            // the merge kernel's operand for the global low-rank term
+            float* dst = const_cast<float*>(a.qfeat) + (slot * TQ + 16 * w + r16) * M;
+#pragma unroll
+            for (int c = 0; c < 2 * FB; ++c) *reinterpret_cast<floatx4*>(dst + 16 * c + 4 * g) = qf[c];
+        }
 #pragma unroll
         for (int ks = 0; ks < FS; ++ks) split2(qf[2 * ks], qf[2 * ks + 1], qfh[ks], qfl[ks]);   // exact: 17-bit values
     }
@@ -3353,17 +3413,22 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
 
     FLY_PROF(2);
     for (int kt = kt_lo; kt < kt_hi; ++kt) {
-        const int s_base = kt * TK;
+        const int s_base = (LIST ? tile_cur : kt) * TK;
         const int cur = (kt - kt_lo) & 1;
         const char* st = lds + cur * TL::BYTES;
         const bool more = kt + 1 < kt_hi;
         float cscale_next = cscale;
+        // LIST: the entry after the next one (tile, presence) is requested now
+        int tile_n2 = 0, pres_n2 = 0;
+        if (LIST && kt + 2 < kt_hi) { tile_n2 = tl_inner[kt + 2]; pres_n2 = tl_blk[4 * (kt + 2)] & 3; }
         if (more) {                                      // next tile's transfer flies during the MFMAs (every wave is past
-            transfer(kt + 1, cur ^ 1);                   // the barrier that ended the last use of that stage)
-            cscale_next = csp[(s_base + TK) / CH];
+            const int nxt = LIST ? tile_next : kt + 1;   // the barrier that ended the last use of that stage)
+            transfer(nxt, cur ^ 1);
+            cscale_next = csp[nxt * TK / CH];
         }
         const float wc = __builtin_amdgcn_exp2f((cscale - kmax) * LOG2E);
-        const bool any = !(s_base + TK - 1 - qw0 < -lc_lo || s_base - (qw0 + 15) >= lc_hi || s_base >= len);
+        const bool any = LIST ? pres_cur != 0
+                              : !(s_base + TK - 1 - qw0 < -lc_lo || s_base - (qw0 + 15) >= lc_hi || s_base >= len);
         const bool stamp = kt == kt_lo + 1;
         FLY_PROF2(stamp, 0);
         if (any) {
@@ -3450,8 +3515,10 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
 #pragma unroll
                 for (int ks = 0; ks < FS; ++ks) { load_f(ks); overlap(ks); }
             }
-            const bool interior = s_base - (qw0 + 15) >= -lc_lo && s_base + TK - 1 - qw0 < lc_hi &&
-                                  s_base + TK <= len && qw0 + 15 < a.T;
+            // (LIST: a present half tile is wholly visible; the caller guarantees whole blocks of keys and queries)
+            const bool interior = LIST ? pres_cur == 3
+                                       : (s_base - (qw0 + 15) >= -lc_lo && s_base + TK - 1 - qw0 < lc_hi &&
+                                          s_base + TK <= len && qw0 + 15 < a.T);
             floatx4 p[KB];
             float ovs = 0.f;
             auto soft = [&](auto masked_tag, auto drop_tag) __attribute__((always_inline)) {
@@ -3463,7 +3530,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         const int s = s_base + 16 * kb + 4 * g + i;
-                        ok[kb][i] = !MASKED || (unsigned)(s - smin) < span;
+                        ok[kb][i] = !MASKED || (LIST ? ((pres_cur >> kb) & 1) != 0 : (unsigned)(s - smin) < span);
                         mx = fmaxf(mx, ok[kb][i] ? s1[kb][i] : -INFINITY);
                     }
                 mx = group_max(mx);
@@ -3520,9 +3587,16 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
         FLY_PROF2(stamp, 6);
         drain_loads();                                   // this wave's share of the next tile is in LDS
         cscale = cscale_next;
+        if (LIST) { seen_block |= pres_cur != 0; tile_cur = tile_next; tile_next = tile_n2; pres_cur = pres_next; pres_next = pres_n2; }
         FLY_PROF2(stamp, 7);
         __syncthreads();
         FLY_PROF2(stamp, 8);
+    }
+    if (LIST && !part_role && !seen_block) {
+        // A block-row without any block: the reference's row logsumexp returns 0 there, not -inf
+        // (blocksparse_logsumexp.py:132), so its normaliser carries an extra exp(0); reproduced.
+        m_run = fmaxf(m_run, 0.f);
+        ze = g == 0 ? __builtin_amdgcn_exp2f(-m_run) : 0.f;
     }
 
     FLY_PROF(3);
@@ -3530,7 +3604,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
 #pragma unroll
     for (int db = 0; db < DB; ++db) lacc[db] = Frag<float>::zero();
     float qk1 = 0.f;
-    if (!SPLIT) {
+    if (!part_role) {
         // global low-rank term on the bf16 matrix pipe: K'^T V in three pieces, the rounded query features in their two;
         // as many of the D columns at a time as the three pieces fit into the tile stages
         constexpr int ROOM = 2 * X3Tile<E, D, M>::BYTES - (int)sizeof(float) * M;
@@ -3567,8 +3641,8 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
     zp = group_sum(zp);
     FLY_PROF(4);
     const float gamma = __builtin_amdgcn_exp2f(c0 - m_run);               // <= 1
-    if (SPLIT) {
-        float* ws = a.part_ws + (((long)bh * n_qt + qt) * a.n_parts + part) * (TQ * (D + NSTAT));
+    if (part_role) {
+        float* ws = a.part_ws + ((LIST ? slot : (long)bh * n_qt + qt) * a.n_parts + part) * (TQ * (D + NSTAT));
         const int ql_ = 16 * w + r16;
         float* stp = ws + TQ * D;
 #pragma unroll
@@ -3997,13 +4071,26 @@ static int launch_fwd(const FwdArgs& a, hipStream_t st) {
     return a.n_parts > 1 ? launch_fwd_impl<T, E, M, true>(a, st) : launch_fwd_impl<T, E, M, false>(a, st);
 }
 
-// fp32 kernel on a block-sparse support (lists of key blocks per query tile), one part per tile
+// band kernel on a block-sparse support (lists of key tiles per query tile), one part per tile: on bf16 pieces when the
+// key pass has left tile images (a.vt; head dims up to 64, up to 128 features, no dropout), else the fp32 kernel
 template <typename T, int E, int M>
 static int launch_fwd_list(const FwdArgs& a, hipStream_t st) {
-    auto kern = sblocal_fwd_kernel<float, E, E, M, false, true>;
-    constexpr size_t smem = fwd_smem<E, M>();
-    static std::atomic<unsigned long long> lds_set{0};     // (devices on which this kernel has its LDS limit)
-    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_set, "sbblocksparse_fwd")) return rc;
+    constexpr bool X3 = E <= 64 && M <= 128;
+    const bool pieces = X3 && a.vt != nullptr;
+    if (a.vt && !(X3 && a.drop_thresh == 0))
+        return fail(ERR_UNSUPPORTED, "sbblocksparse_fwd: tile images are for head dims up to 64, up to 128 features and no "
+                                     "dropout (got %d, %d)", E, M);
+    const void* kern_fp32 = reinterpret_cast<const void*>(sblocal_fwd_kernel<float, E, E, M, false, true>);
+    const void* kern = kern_fp32;
+    size_t smem = fwd_smem<E, M>();
+    static std::atomic<unsigned long long> lds_set{0}, lds_set_x3{0};     // (devices on which the kernels have their LDS limit)
+    if constexpr (X3) {
+        if (pieces) {
+            kern = reinterpret_cast<const void*>(sblocal_fwd_x3_kernel<E, E, M, false, false, true>);
+            smem = fwd_x3_smem<E, M>();
+        }
+    }
+    if (int rc = ensure_dynamic_lds(kern, smem, pieces ? lds_set_x3 : lds_set, "sbblocksparse_fwd")) return rc;
     // every XCD gets room for ceil(B H / dies) (batch, head) pairs
     const Machine& mach = machine();
     const long grid = (((long)a.B * a.H + mach.xcds - 1) / mach.xcds) * ((a.T + TQ - 1) / TQ) * mach.xcds;
@@ -4015,7 +4102,12 @@ static int launch_fwd_list(const FwdArgs& a, hipStream_t st) {
     FwdArgs args = a;
     args.n_xcd = mach.xcds;
     args.band_wgs = (int)(grid + part_wgs);
-    hipLaunchKernelGGL(kern, dim3((unsigned)(grid + part_wgs)), dim3(NT), smem, st, args);
+    if constexpr (X3) {
+        if (pieces)
+            hipLaunchKernelGGL((sblocal_fwd_x3_kernel<E, E, M, false, false, true>), dim3((unsigned)(grid + part_wgs)), dim3(NT), smem, st, args);
+    }
+    if (!pieces)
+        hipLaunchKernelGGL((sblocal_fwd_kernel<float, E, E, M, false, true>), dim3((unsigned)(grid + part_wgs)), dim3(NT), smem, st, args);
     int rc = check_launch("sblocal_fwd_kernel (block-sparse support)");
     if (rc || a.n_heavy <= 0) return rc;
     hipLaunchKernelGGL((sb_merge_kernel<float, E, M>), dim3((unsigned)tiles, E / 16, 1), dim3(NT), 0, st, args);
@@ -4775,7 +4867,7 @@ extern "C" int flyhip_sblocal_fwd_static(const void* q, const void* k, const voi
 }
 
 extern "C" int flyhip_sbblocksparse_fwd(const void* q, const void* k, const void* v, const float* proj,
-                                        const void* kfeat, const float* chunk_scale,
+                                        const void* kfeat, const void* vt, const float* chunk_scale,
                                         const float* kv, const float* ksum, const float* kmax,
                                         const int32_t* tl_ptr, const int32_t* tl_inner, const int32_t* tl_blk,
                                         const int32_t* tl_order, const int32_t* tl_heavy, int n_heavy, int heavy_parts,
@@ -4802,7 +4894,7 @@ extern "C" int flyhip_sbblocksparse_fwd(const void* q, const void* k, const void
     FLY_REQUIRE(n_heavy >= 0 && (n_heavy == 0 || (tl_heavy && tl_order && part_ws && qfeat && heavy_parts >= 2 && heavy_parts <= 64)),
                 "sbblocksparse_fwd: long lists need tl_heavy, tl_order (with the long tiles marked), part_ws, qfeat and "
                 "2 <= heavy_parts <= 64");
-    FwdArgs a{q, k, v, proj, kfeat, chunk_scale, kv, ksum, kmax, qfeat, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 1,
+    FwdArgs a{q, k, v, proj, kfeat, chunk_scale, kv, ksum, kmax, qfeat, nullptr, vt, nullptr, nullptr, nullptr, 0, 0, 1,
               nullptr, out, log_norm, part_ws,
               B, H, T, S, mh_valid, 1, nc, n_heavy > 0 ? heavy_parts : 1,
               q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss, softmax_temp,

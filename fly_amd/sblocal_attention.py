@@ -154,9 +154,11 @@ class SBLocalPlan:
 
     def run_block_sparse(self, q, k, v, proj, t, tables, out, log_norm, dropout=(0.0, 0)):
         """Scatterbrain attention whose exact part lives on a block-sparse support instead of a band: the
-        key pass as in ``run``, then the fp32 band kernel walking lists of 32-key tiles (``tables`` =
-        blocksparse_utils.tile_mask_table(layout, block) on the device).  One part per query tile, no key lengths.
-        dropout: (probability, seed) of the dropout of the exact weights inside that kernel."""
+        key pass as in ``run``, then the band kernel walking lists of 32-key tiles (``tables`` =
+        blocksparse_utils.tile_mask_table(layout, block) on the device) -- on bf16 pieces from the key pass's tile images
+        when the plan has them (``operand_images``: float32, head dims up to 64, up to 128 features, no dropout), else on
+        the fp32 matrix pipe.  One part per query tile, no key lengths.
+        dropout: (probability, seed) of the dropout of the exact weights inside the fp32 kernel."""
         B, H, T, S, dim, mh, mh_valid = self.shape
         self._make_buffers()
         tl_ptr, tl_inner, tl_blk = tables[:3]
@@ -174,7 +176,7 @@ class SBLocalPlan:
             stream = _lib.stream_ptr(self.device)
             self.run_keys(q, k, v, proj, None, t, stream)
             _lib.call('flyhip_sbblocksparse_fwd', q.data_ptr(), k.data_ptr(), v.data_ptr(), proj.data_ptr(),
-                      self.kfeat.data_ptr(), self.chunk_scale.data_ptr(), self.kv.data_ptr(),
+                      self.kfeat.data_ptr(), _lib.ptr(self.vt), self.chunk_scale.data_ptr(), self.kv.data_ptr(),
                       self.ksum.data_ptr(), self.kmax.data_ptr(), tl_ptr.data_ptr(), _lib.table_ptr(tl_inner),
                       _lib.table_ptr(tl_blk), _lib.ptr(tl_order), _lib.ptr(tl_heavy), n_heavy, parts,
                       _lib.ptr(self.part_ws) if n_heavy else None, _lib.ptr(self.qfeat) if n_heavy else None,
@@ -381,10 +383,13 @@ def sbblocksparse_forward(query, key, value, projection_matrix, tables, softmax_
     q, k, v = prep(query), prep(key), prep(value)
     proj = _padded_projection(projection_matrix, mh, dim, cache)
 
+    # tile images of the key pass (the band kernel on bf16 pieces) where that kernel exists; dropout lives in the fp32 kernel
+    images = dropout_p == 0 and dim <= 64 and mh <= 64
+
     def make_plan():
         return SBLocalPlan(B, H, T, S, dim, mh, mh_valid, query.dtype, query.device, 64, n_parts=1,
-                           operand_images=False)
-    plan_key = ('block-sparse', B, H, T, S, dim, mh, mh_valid, query.dtype, query.device)
+                           operand_images=images)
+    plan_key = ('block-sparse', B, H, T, S, dim, mh, mh_valid, query.dtype, query.device, images)
     plan = make_plan() if cache is None else cache.plan(plan_key, make_plan)
     out = torch.empty(B, T, H, dim, dtype=query.dtype, device=query.device)
     log_norm = torch.empty(B, H, T, dtype=torch.float32, device=query.device)

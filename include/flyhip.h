@@ -288,7 +288,9 @@ int flyhip_sbblocksparse_bwd_pieces(const void* outer_images, const void* inner_
 /* Scatterbrain attention on a block-sparse support (ref: src/models/attention/sbblocksparse_attention.py:109-213
  * for need_weights = False, no masks): as flyhip_sblocal_fwd with one part per query tile, but the
  * exact part covers the nonzero blocks of a layout (16 x 16 or 32 x 32) instead of a band.  Key-side inputs (kfeat,
- * chunk_scale, kv, ksum, kmax) from flyhip_sb_kv_reduce.  tl_ptr (H * ceil(T/64) + 1), tl_inner, tl_mask (4 per
+ * chunk_scale, kv, ksum, kmax) from flyhip_sb_kv_reduce; vt = the tile images that pass leaves when asked for them
+ * (then kfeat holds feature images and the band kernel runs on bf16 pieces: head dims up to 64, up to 128 features,
+ * dropout_p = 0), or NULL (fp32 features in kfeat, the kernel on the fp32 matrix pipe).  tl_ptr (H * ceil(T/64) + 1), tl_inner, tl_mask (4 per
  * entry): per (head, 64-query tile) the 32-key tiles that any of its queries sees on the support, and per entry and
  * group of 16 queries (16 w .. 16 w + 15 of the tile) a mask: bit 0 = keys 0..15, bit 1 = keys 16..31 of that tile
  * are on the support for those queries (32 x 32 blocks: 0 or 3, the same for w = 0, 1 and for w = 2, 3).
@@ -304,7 +306,7 @@ int flyhip_sbblocksparse_bwd_pieces(const void* outer_images, const void* inner_
  * part and the normaliser see none), by the hash mask that flyhip_sblocal_forward documents;
  * flyhip_sbblocksparse_bwd_pieces takes the same two values and forms the mask again. */
 int flyhip_sbblocksparse_fwd(const void* q, const void* k, const void* v, const float* proj,
-                             const void* kfeat, const float* chunk_scale,
+                             const void* kfeat, const void* vt, const float* chunk_scale,
                              const float* kv, const float* ksum, const float* kmax,
                              const int32_t* tl_ptr, const int32_t* tl_inner, const int32_t* tl_mask,
                              const int32_t* tl_order, const int32_t* tl_heavy, int n_heavy, int heavy_parts,
