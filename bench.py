@@ -415,6 +415,18 @@ def bench_other_configs():
         sbbs.fuse = False
         ms_o = timeit(lambda: sbbs(q, k, v), n=3)
     out['sbblocksparse_fp32_B64_L784_block16_m16'] = {'ms': ms_f, 'op_by_op_ms': ms_o}
+    qg, kg, vg = (x.clone().requires_grad_() for x in (q, k, v))
+    go = torch.randn_like(v)
+
+    def sbbs16_step():
+        o, _ = sbbs(qg, kg, vg)
+        o.backward(go)
+        qg.grad = kg.grad = vg.grad = None
+    sbbs.fuse = True
+    out['sbblocksparse_fp32_B64_L784_block16_m16']['fwd_bwd_ms'] = timeit(sbbs16_step, n=5)
+    sbbs.fuse = False
+    out['sbblocksparse_fp32_B64_L784_block16_m16']['fwd_bwd_op_by_op_ms'] = timeit(sbbs16_step, n=3)
+    del qg, kg, vg, go
     del q, k, v, sbbs
 
     cfg = fly_amd.FlatBlockButterflySparsityConfig(8, 2, block=32)

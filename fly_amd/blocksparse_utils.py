@@ -127,15 +127,18 @@ def union_table(layout, rows_per_group=4, transposed=False):
     return ptr.to(torch.int32), nz[:, 2].to(torch.int32).contiguous(), blk.to(torch.int32).contiguous()
 
 
-def tile_mask_table(layout, block):
+def tile_mask_table(layout, block, transposed=False):
     """The support of a layout of 16 x 16 or 32 x 32 blocks as the fused Scatterbrain kernels walk it: per (head,
     64-query tile) the 32-key tiles that hold a block of any of the tile's block-rows, and per entry four masks, one per
     group of 16 queries (16 w .. 16 w + 15 of the tile): bit 0 / bit 1 = that group sees keys 0..15 / 16..31 of the
     entry's key tile.  Returns (ptr int32 (H * ceil(rows / 64) + 1), inner int32 (n) key tiles in increasing order per
-    query tile, mask int32 (n, 4)); rows and columns past the layout's end count as absent."""
+    query tile, mask int32 (n, 4)); rows and columns past the layout's end count as absent.  transposed: the same with
+    the roles of queries and keys exchanged (64-key tiles against 32-query tiles: the key-major pass of the backward)."""
     if block not in (16, 32):
         raise ValueError(f'block size {block}: the fused kernels walk supports of 16 x 16 or 32 x 32 blocks')
     fine = _as_layout3(layout).cpu() > 0
+    if transposed:
+        fine = fine.transpose(1, 2)
     rep = block // 16
     if rep > 1:
         fine = fine.repeat_interleave(rep, dim=1).repeat_interleave(rep, dim=2)

@@ -407,8 +407,9 @@ struct BwdX3Args {
     // small problems: every outer tile's inner range walked in n_parts parts by as many workgroups, whose sums go to
     // part_ws ((tile, part): registers x 256 lanes x 4 floats) and are finished by sblocal_bwd_x3_finish_kernel
     float* part_ws; int n_parts;
-    // a block-sparse support instead of a band (LIST kernels; 32 x 32 blocks, no key lengths): per (head, 64-row outer
-    // tile) the union of the inner 32-row blocks its two block-rows meet, and per entry whether each of the two does
+    // a block-sparse support instead of a band (LIST kernels; 16 x 16 or 32 x 32 blocks, no key lengths): per (head,
+    // 64-row outer tile) the inner 32-row tiles that any of its rows meets on the support, and per entry four masks, one
+    // per group of 16 outer rows (a wave): bit 0 / bit 1 = that group meets inner rows 0..15 / 16..31 of the entry's tile
     const int32_t* tl_ptr; const int32_t* tl_inner; const int32_t* tl_blk;
     // long lists: tl_skip (one flag per (head, outer tile)) marks the tiles the main launch leaves out; the launch
     // in parts takes (batch, tl_heavy[j], part) for the n_heavy listed (head, outer tile) indices, then the finish
@@ -699,7 +700,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
         // wave-uniform: does this tile meet the band of any of the wave's 16 outer rows (is the block of the wave's
         // block-row and this block-column part of the support)?
-        const bool any = LIST ? a.tl_blk[2 * (e_lo + it) + (w >> 1)] >= 0
+        const int pres = LIST ? a.tl_blk[4 * (e_lo + it) + w] & 3 : 3;      // (LIST: the wave's mask of this entry)
+        const bool any = LIST ? pres != 0
                               : !(n_base + TK - 1 - ow0 < lo || n_base - (ow0 + 15) >= hi || n_base >= n_limit || ow0 >= o_limit);
         if (any) {
             floatx4 s1[KB], s2[KB], s3[KB];
@@ -751,7 +753,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const int n = n_base + 16 * kb + 4 * g + i;
-                    const bool ok = LIST ? ovalid : (unsigned)(n - nmin) < span;      // (a block of the support is whole)
+                    const bool ok = LIST ? (ovalid && ((pres >> kb) & 1) != 0) : (unsigned)(n - nmin) < span;      // (a present half tile is whole)
                     const float av = ok ? __builtin_amdgcn_exp2f(s1[kb][i] * sc - (KEYMAJOR ? lnq[i] : ln_o)) : 0.f;
                     const float cc = KEYMAJOR ? cq[i] : c_o;
                     const float df = ok ? s3[kb][i] - cc : 0.f;
@@ -1084,7 +1086,7 @@ extern "C" int flyhip_sbblocksparse_bwd_pieces(const void* outer_images, const v
     FLY_REQUIRE(dropout_p >= 0.f && dropout_p < 1.f, "sbblocksparse_bwd_pieces: dropout probability %g outside [0, 1)", (double)dropout_p);
     FLY_REQUIRE(!key_major || d3, "sbblocksparse_bwd_pieces: the key-major pass needs d3");
     FLY_REQUIRE(BH > 0 && H > 0 && BH % H == 0 && T > 0 && S > 0, "sbblocksparse_bwd_pieces: empty or inconsistent problem");
-    FLY_REQUIRE(T % 32 == 0 && S % 32 == 0, "sbblocksparse_bwd_pieces: sequence lengths %d, %d must be multiples of 32", T, S);
+    FLY_REQUIRE(T % 16 == 0 && S % 16 == 0, "sbblocksparse_bwd_pieces: sequence lengths %d, %d must be multiples of 16", T, S);
     FLY_REQUIRE(softmax_temp > 0.f, "sbblocksparse_bwd_pieces: softmax_temp must be positive");
     FLY_REQUIRE(n_heavy == 0 || (n_heavy > 0 && tl_skip && tl_heavy && part_ws && heavy_parts >= 2 && heavy_parts <= 64),
                 "sbblocksparse_bwd_pieces: long lists need tl_skip, tl_heavy, part_ws and 2..64 parts");

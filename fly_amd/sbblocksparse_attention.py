@@ -43,11 +43,12 @@ def fused_tables(layout, device, block=32):
     return tuple(x.to(device) for x in (ptr, inner, mask, order, heavy)) + (parts,)
 
 
-def backward_tables(layout, device, transposed=False, n_heavy_min=32, entries_per_part=12, max_parts=16):
-    """Index tables of one pass of the backward kernels for a (H, T/32, S/32) layout: the union lists of the 64-row
-    outer tiles (queries, or with transposed=True keys), a flag per tile for the lists long enough to be walked in
-    parts, those tiles, and the number of parts -- (ptr, inner, blk, skip, heavy, parts), tensors on `device`."""
-    ptr, inner, blk = union_table(layout, rows_per_group=2, transposed=transposed)
+def backward_tables(layout, device, transposed=False, n_heavy_min=32, entries_per_part=12, max_parts=16, block=32):
+    """Index tables of one pass of the backward kernels for a (H, T/block, S/block) layout of 16 x 16 or 32 x 32 blocks:
+    the lists of the 64-row outer tiles (queries, or with transposed=True keys) with the masks of their four groups of 16
+    rows (blocksparse_utils.tile_mask_table), a flag per tile for the lists long enough to be walked in parts, those
+    tiles, and the number of parts -- (ptr, inner, mask, skip, heavy, parts), tensors on `device`."""
+    ptr, inner, blk = tile_mask_table(layout, block, transposed=transposed)
     counts = (ptr[1:] - ptr[:-1]).long()
     skip = (counts >= n_heavy_min).to(torch.int32)
     heavy = skip.nonzero().flatten().to(torch.int32)
@@ -161,8 +162,8 @@ class SBBlockSparseAttention(nn.Module):
         softmax_temp = self.softmax_temp or 1 / math.sqrt(E)       # :131
 
         # blocks of 16 x 16 or 32 x 32, nothing but the output wanted: the whole forward on the fused kernels of
-        # Scatterbrain-local attention, walking the layout's blocks instead of a band (with gradients: 32 x 32 blocks,
-        # whose backward kernels exist)
+        # Scatterbrain-local attention, walking the layout's blocks instead of a band (with gradients: head dims and
+        # feature counts of the backward kernels)
         self.feature_map.new_feature_map(query.device)
         layout = self.get_layout(T, S)
         needs_grad = torch.is_grad_enabled() and any(x.requires_grad for x in (query, key, value))
@@ -179,7 +180,7 @@ class SBBlockSparseAttention(nn.Module):
                 and query.dtype in (torch.float32, torch.bfloat16, torch.float16)
                 and sbblocksparse_forward_supported(block, torch.float32, E, value.shape[3], n_rows, layout.shape[0], H)
                 # with gradients: the backward kernels' head dims and feature counts
-                and (not needs_grad or (block == 32 and _band_kernel_dims(E, value.shape[3], 2 * n_rows) is not None))):
+                and (not needs_grad or _band_kernel_dims(E, value.shape[3], 2 * n_rows) is not None)):
             key_ = (T, S, query.device)
             if key_ not in self.fused_tables:
                 self.fused_tables[key_] = fused_tables(layout, query.device, block)
@@ -191,8 +192,8 @@ class SBBlockSparseAttention(nn.Module):
                 self.last_dropout_seed = dropout[1] if dropout[0] > 0 else None
                 return out.to(query.dtype), None
             if key_ not in self.backward_tables:     # the support seen from the queries and from the keys
-                self.backward_tables[key_] = (backward_tables(layout, query.device),
-                                              backward_tables(layout, query.device, transposed=True))
+                self.backward_tables[key_] = (backward_tables(layout, query.device, block=block),
+                                              backward_tables(layout, query.device, transposed=True, block=block))
             support = self.backward_tables[key_]
             out, _ = _SBBlockSparseFn.apply(query.float(), key.float(), value.float(), self.feature_map.projection_matrix,
                                             self.fused_tables[key_], support, softmax_temp, self._scratch_cache, dropout)

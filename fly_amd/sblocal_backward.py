@@ -155,9 +155,9 @@ def _backward_hip(Q, K, V, G, O, LN, P, lens_b, H, local_context, t, dims, piece
     pieces: the band kernel on the bf16 matrix pipe from operands in two bf16 pieces (flyhip_sblocal_bwd_pieces;
     the preparation pass leaves every 32 rows of either side as one image of such operands), else on the fp32
     matrix pipe from the float arrays (flyhip_sblocal_bwd).  support: instead of a band, a block-sparse support of
-    32 x 32 blocks -- (tables of the query tiles, tables of the key tiles), each (ptr, inner, blk) of
-    blocksparse_utils.union_table(layout, 2) resp. union_table(layout, 2, transposed=True) as int32 tensors on the
-    device, optionally followed by (skip, heavy, parts) for long lists walked in parts
+    16 x 16 or 32 x 32 blocks -- (tables of the query tiles, tables of the key tiles), each (ptr, inner, mask) of
+    blocksparse_utils.tile_mask_table(layout, block) resp. tile_mask_table(layout, block, transposed=True) as int32
+    tensors on the device, optionally followed by (skip, heavy, parts) for long lists walked in parts
     (sbblocksparse_attention.backward_tables; flyhip_sbblocksparse_bwd_pieces; no key lengths)."""
     from . import _lib
     BH, T, E = Q.shape
@@ -323,7 +323,7 @@ def sblocal_backward(query, key, value, projection_matrix, local_context, softma
     chain rule in two, on the bf16 matrix pipe from operands in two bf16 pieces; 'fp32' = the same five launches
     with the band kernel on the fp32 matrix pipe; 'sums' = only the band sums on the kernels, the rest as tensor
     algebra; False = batched library products; True = the kernels or NotImplementedError.
-    support: the exact part lives on a block-sparse support of 32 x 32 blocks instead of a band (Scatterbrain
+    support: the exact part lives on a block-sparse support of 16 x 16 or 32 x 32 blocks instead of a band (Scatterbrain
     attention on a block-sparse support, sbblocksparse_attention.py:161-212): see _backward_hip; kernels only, no key
     lengths, local_context is ignored.
     dropout: (probability, seed) the forward was called with; the band kernels on bf16 pieces form the forward's mask
@@ -357,10 +357,10 @@ def sblocal_backward(query, key, value, projection_matrix, local_context, softma
         raise NotImplementedError('the backward under attention dropout runs on the band kernels on bf16 pieces only '
                                   f'(GPU, head dims <= 64, <= 128 features; got ({E}, {D}), {2 * mh})')
     if support is not None:
-        if not on_kernels or key_lengths is not None or T % 32 or S % 32:
+        if not on_kernels or key_lengths is not None or T % 16 or S % 16:
             raise NotImplementedError('the backward on a block-sparse support needs the GPU kernels (float32 or bfloat16 '
                                       f'inputs, head dims <= 64, <= 128 features; got ({E}, {D}), {2 * mh}), sequence '
-                                      'lengths that are multiples of 32 and no key lengths')
+                                      'lengths that are multiples of 16 and no key lengths')
         dQ, dK, dV = _backward_hip(Q, K, V, G, O, LN, P, None, H, 1, t, dims, support=support, dropout=dropout)
     elif on_kernels and band_kernel != 'sums':
         # features, per-head sums and the two passes of the fused kernel

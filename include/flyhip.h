@@ -263,11 +263,13 @@ int flyhip_sblocal_bwd_pieces(const void* outer_images, const void* inner_images
 
 /* flyhip_sblocal_bwd_pieces for Scatterbrain attention on a block-sparse support (the reference takes these
  * gradients from autograd through src/models/attention/sbblocksparse_attention.py:161-212): the exact weights live on
- * the nonzero 32 x 32 blocks of a layout instead of a band.  tl_ptr (H * ceil(outer rows / 64) + 1), tl_inner, tl_blk
- * (2 per entry): per (head, 64-row outer tile) the union of the inner 32-row blocks its two block-rows meet, and per
- * entry the block id of each of the two or -1 -- union_table(layout, 2) for key_major = 0 (outer = queries),
- * union_table(layout, 2, transposed) for key_major = 1 (outer = keys).  T, S multiples of 32, no key lengths; images,
- * gmat | gvec, c as for flyhip_sblocal_bwd_pieces.
+ * the nonzero blocks (16 x 16 or 32 x 32) of a layout instead of a band.  tl_ptr (H * ceil(outer rows / 64) + 1),
+ * tl_inner, tl_blk (4 per entry): per (head, 64-row outer tile) the 32-row inner tiles that any of its rows meets on
+ * the support, and per entry and group of 16 outer rows (16 w .. 16 w + 15 of the tile) a mask: bit 0 = inner rows
+ * 0..15, bit 1 = inner rows 16..31 of that tile are on the support for those rows -- the tables of
+ * flyhip_sbblocksparse_fwd for key_major = 0 (outer = queries), the same built from the transposed layout for
+ * key_major = 1 (outer = keys).  T, S multiples of 16, no key lengths; images, gmat | gvec, c as for
+ * flyhip_sblocal_bwd_pieces.
  * Long lists (n_heavy > 0): tl_skip (H * ceil(outer rows / 64) flags) marks the outer tiles the main launch leaves
  * out, tl_heavy (n_heavy indices head * ceil(outer rows / 64) + tile) lists them; they are walked in heavy_parts
  * parts (2..64) by (batch, tile, part) workgroups of a launch of their own and finished by a third; part_ws of at

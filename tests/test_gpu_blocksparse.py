@@ -894,21 +894,24 @@ def test_sbblocksparse_fused_forward_with_an_empty_layout():
     assert rel_err(ln.reshape(ref_ln.shape), ref_ln) <= 1e-4
 
 
-@pytest.mark.parametrize('B,H,T,S,E,D,m,seed', [(2, 2, 256, 256, 64, 64, 64, 1), (1, 3, 224, 352, 32, 32, 32, 2),
-                                                (1, 2, 416, 160, 40, 24, 26, 4), (3, 1, 160, 192, 64, 64, 128, 5)])
-def test_sbblocksparse_gradients_on_the_kernels(B, H, T, S, E, D, m, seed):
+@pytest.mark.parametrize('B,H,T,S,E,D,m,seed,block', [(2, 2, 256, 256, 64, 64, 64, 1, 32), (1, 3, 224, 352, 32, 32, 32, 2, 32),
+                                                      (1, 2, 416, 160, 40, 24, 26, 4, 32), (3, 1, 160, 192, 64, 64, 128, 5, 32),
+                                                      (2, 2, 208, 144, 64, 64, 64, 6, 16), (1, 3, 784, 784, 64, 64, 16, 7, 16),
+                                                      (2, 1, 48, 400, 32, 48, 32, 8, 16)])
+def test_sbblocksparse_gradients_on_the_kernels(B, H, T, S, E, D, m, seed, block):
     """Gradients of Scatterbrain attention on a block-sparse support from the backward kernels walking the layout's
     blocks (flyhip_sblocal_bwd_prep, flyhip_sbblocksparse_bwd_pieces) against autograd through the oracle in float64
     (sbblocksparse_attention.py:161-212): random layouts per head with an empty block-row, an odd number of
-    block-rows and block-columns, T != S, head dims and feature counts that need padding."""
+    block-rows and block-columns, T != S, head dims and feature counts that need padding; 32 x 32 and 16 x 16 blocks (the
+    latter with lengths that are not multiples of 32: half tiles past the end)."""
     from fly_amd import sblocal_backward
     from fly_amd.blocksparse_utils import tile_mask_table, union_table
     from fly_amd.sblocal_attention import sbblocksparse_forward
     from oracle import sbblocksparse as osbb
     from oracle import sblocal as osb
-    print('case', B, H, T, S, E, D, m, flush=True)
+    print('case', B, H, T, S, E, D, m, block, flush=True)
     g = torch.Generator().manual_seed(seed)
-    layout = (torch.rand(H, T // 32, S // 32, generator=g) < 0.4).long()
+    layout = (torch.rand(H, T // block, S // block, generator=g) < (0.4 if block == 32 else 0.2)).long()
     layout[:, :, 0] = 1
     layout[0, 1, :] = 0
     q = torch.randn(B, T, H, E, generator=g) * E ** -0.25
@@ -917,12 +920,12 @@ def test_sbblocksparse_gradients_on_the_kernels(B, H, T, S, E, D, m, seed):
     w = torch.randn(B, T, H, D, generator=g)
     P = osb.gaussian_orthogonal_random_matrix(m // 2, E, generator=g)
     qd, kd, vd = (x.double().requires_grad_() for x in (q, k, v))
-    ref_out, _ = osbb.sbblocksparse_attention(qd, kd, vd, P.double(), layout, 32)
+    ref_out, _ = osbb.sbblocksparse_attention(qd, kd, vd, P.double(), layout, block)
     (ref_out * w.double()).sum().backward()
-    fwd = tuple(x.to(DEV) for x in union_table(layout, rows_per_group=2))
-    bwd = tuple(x.to(DEV) for x in union_table(layout, rows_per_group=2, transposed=True))
+    fwd = tuple(x.to(DEV) for x in tile_mask_table(layout, block))
+    bwd = tuple(x.to(DEV) for x in tile_mask_table(layout, block, transposed=True))
     qg, kg, vg = q.to(DEV), k.to(DEV), v.to(DEV)
-    out, ln = sbblocksparse_forward(qg, kg, vg, P.to(DEV), tuple(x.to(DEV) for x in tile_mask_table(layout, 32)))
+    out, ln = sbblocksparse_forward(qg, kg, vg, P.to(DEV), fwd)
     dq, dk, dv = sblocal_backward(qg, kg, vg, P.to(DEV), 1, None, None, out, ln, w.to(DEV), support=(fwd, bwd))
     for got, ref in ((dq, qd.grad), (dk, kd.grad), (dv, vd.grad)):
         assert got.shape == ref.shape and rel_err(got, ref) <= 2e-4, rel_err(got, ref)
@@ -931,9 +934,8 @@ def test_sbblocksparse_gradients_on_the_kernels(B, H, T, S, E, D, m, seed):
 @pytest.mark.parametrize('block,p_drop', [(32, 0.25), (16, 0.1)])
 def test_sbblocksparse_dropout_inside_the_kernels(block, p_drop):
     """Training-mode dropout of SBBlockSparseAttention (sbblocksparse_attention.py:196-200: of the exact weights only)
-    inside the fused forward and, for 32 x 32 blocks, the backward kernels: the mask is the hash of (seed, batch, head,
-    query, key) restated in oracle.sblocal.dropout_keep, handed to the oracle as nn.Dropout's multiplier.  16 x 16
-    blocks have no backward kernels: forward only (a training step there runs op by op with torch's dropout)."""
+    inside the fused forward and the backward kernels (32 x 32 and 16 x 16 blocks): the mask is the hash of (seed, batch,
+    head, query, key) restated in oracle.sblocal.dropout_keep, handed to the oracle as nn.Dropout's multiplier."""
     from fly_amd import SBBlockSparseAttention, FlatBlockButterflySparsityConfig
     from oracle import sbblocksparse as osbb
     from oracle.sblocal import dropout_keep
@@ -945,7 +947,7 @@ def test_sbblocksparse_dropout_inside_the_kernels(block, p_drop):
     g = torch.Generator().manual_seed(6)
     q, k, v, w = (torch.randn(B, T, H, E, generator=g) for _ in range(4))
     q, k = q * E ** -0.25 * 2, k * E ** -0.25 * 2
-    train = block == 32
+    train = True
     qg, kg, vg = (x.to(DEV).requires_grad_(train) for x in (q, k, v))
     torch.manual_seed(9)
     out, _ = layer(qg, kg, vg)

@@ -367,5 +367,8 @@ def test_tile_mask_table_against_loops(block):
         for e in mine:
             assert int(inner[at]) == e[1] and mask[at].tolist() == e[2]
             at += 1
+    # transposed: the table of the transposed layout (64-key tiles against 32-query tiles, the backward's key-major pass)
+    for a_, b_ in zip(tile_mask_table(layout, block, transposed=True), tile_mask_table(layout.transpose(1, 2).contiguous(), block)):
+        assert torch.equal(a_, b_)
     with pytest.raises(ValueError):
         tile_mask_table(layout, 64)
