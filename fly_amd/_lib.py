@@ -26,6 +26,7 @@ SIGNATURES = {
     'flyhip_sblocal_fwd_static': [c_vp] * 13 + [c_vp] * 2 + [c_int] + [c_vp] * 3 + [c_int] * 10 + [c_i64] * 12 + [c_float, c_int, c_vp],
     'flyhip_sblocal_bwd_band': [c_vp] * 12 + [c_int] * 7 + [c_float, c_int, c_vp],
     'flyhip_sblocal_bwd_band_dropout': [c_vp] * 12 + [c_int] * 7 + [c_float, c_int, c_float, c_u64, c_vp],
+    'flyhip_sblocal_bwd_band_masked': [c_vp] * 13 + [c_int] * 7 + [c_float, c_int, c_float, c_u64, c_vp],
     'flyhip_sblocal_bwd': [c_vp] * 14 + [c_int] * 7 + [c_float, c_int, c_vp],
     'flyhip_sblocal_bwd_prep': [c_vp] * 18 + [c_i64] + [c_int] * 7 + [c_float, c_vp],
     'flyhip_sblocal_bwd_pieces': [c_vp] * 12 + [c_i64] + [c_int] * 7 + [c_float, c_int, c_float, c_u64, c_vp],
@@ -33,6 +34,7 @@ SIGNATURES = {
     'flyhip_sbblocksparse_fwd': [c_vp] * 15 + [c_int] * 2 + [c_vp] * 4 + [c_int] * 8 + [c_i64] * 12 + [c_float, c_int, c_float, c_u64, c_vp],
     'flyhip_local_fwd_lse': [c_vp] * 6 + [c_int] * 7 + [c_i64] * 12 + [c_float, c_int, c_vp],
     'flyhip_local_fwd_dropout': [c_vp] * 6 + [c_int] * 7 + [c_i64] * 12 + [c_float, c_int, c_float, c_u64, c_vp],
+    'flyhip_local_fwd_masked': [c_vp] * 7 + [c_int] * 7 + [c_i64] * 12 + [c_float, c_int, c_float, c_u64, c_vp],
     'flyhip_local_fwd': [c_vp] * 5 + [c_int] * 7 + [c_i64] * 12 + [c_float, c_int, c_vp],
     'flyhip_bs_sdd': [c_vp] * 4 + [c_int] + [c_vp] * 3 + [c_int] * 2 + [c_vp] * 3 + [c_int] * 3 + [c_i64] * 8 + [c_int, c_vp],
     'flyhip_bs_sdd_dsoftmax': [c_vp] * 8 + [c_int] * 6 + [c_i64] * 6 + [c_float, c_int, c_vp],

@@ -2580,6 +2580,11 @@ struct LocalArgs {
     // dropout of the probabilities (drop_thresh != 0): pair (query i, key s) of (b, h) is kept when the hash of
     // (seed, row = (b H + h) T + i, s) reaches the threshold, and scaled by 1 / (1 - p); the denominator sums all
     uint32_t drop_seed, drop_thresh; float drop_scale;
+    // optional additive mask (T, S), float32, rows contiguous: added to q.k before the temperature.  Entries of -1e24
+    // absorb the product (every masked score is the same float), so a query whose visible keys are all masked gets
+    // equal weights 1 / local_context -- over the positions of its band that fall outside the keys as well, which
+    // count in the denominator only; its lse entry is -inf, the marker the backward kernel reads.
+    const float* add_mask;
 };
 
 template <typename T, int E, int D>
@@ -2666,8 +2671,20 @@ __global__ __launch_bounds__(NT) void local_fwd_kernel(LocalArgs a) {
                 for (int i = 0; i < 4; ++i) {
                     const int s = s_base + 16 * kb + 4 * g + i;
                     ok[kb][i] = (unsigned)(s - smin) < span;
-                    mx = fmaxf(mx, ok[kb][i] ? s1[kb][i] : -INFINITY);
                 }
+            if (a.add_mask) {                                // (uniform)
+                const float* am = a.add_mask + (long)min(iq, a.T - 1) * a.S;
+                const float cs = a.temp * LOG2E;
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        if (ok[kb][i]) s1[kb][i] += am[s_base + 16 * kb + 4 * g + i] * cs;
+            }
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) mx = fmaxf(mx, ok[kb][i] ? s1[kb][i] : -INFINITY);
             mx = group_max(mx);
             if (__builtin_amdgcn_ballot_w64(mx > m_run + 8.f) != 0) {
                 const float m_new = fmaxf(m_run, mx);
@@ -2709,13 +2726,18 @@ __global__ __launch_bounds__(NT) void local_fwd_kernel(LocalArgs a) {
         __syncthreads();
     }
     ze = group_sum(ze);
+    // every visible key masked: the positions of the band outside the keys carry the same score in the reference's
+    // softmax over the packed band (local_attention.py:68-81), so they count in the denominator
+    const bool all_masked = a.add_mask != nullptr && span > 0u && m_run < -1e20f;
+    if (all_masked) ze += (float)(a.lc - (int)span);
     if (qvalid) {
         const float inv = (ze > 0.f ? 1.0f / ze : 0.f) * (a.drop_thresh != 0u ? a.drop_scale : 1.0f);
         T* optr = reinterpret_cast<T*>(a.out) + b * a.o_sb + h * a.o_sh + (long)iq * a.o_ss;
 #pragma unroll
         for (int db = 0; db < DB; ++db) store4_f32(optr + 16 * db + 4 * g, oacc[db] * inv);
         if (a.lse && g == 0)        // a query without visible keys has no pair that would read its entry
-            a.lse[((long)b * a.H + h) * a.T + iq] = ze > 0.f ? m_run * 0.6931471805599453f + __logf(ze) : 0.f;
+            a.lse[((long)b * a.H + h) * a.T + iq] = all_masked ? -INFINITY
+                                                    : ze > 0.f ? m_run * 0.6931471805599453f + __logf(ze) : 0.f;
     }
 }
 
@@ -4163,6 +4185,9 @@ struct BwdArgs {
     // (seed, (b H + h) T + query, key), see drop_keep) and 1 / (1 - p) on kept ones, dm = a (m g.v - c) and the
     // weight of g in d v is m a - kb
     uint32_t drop_seed, drop_thresh; float drop_scale;
+    // optional additive mask (T, S) of plain local attention, added to q.k before the temperature (see LocalArgs); a
+    // query whose log Z entry is -inf had all its visible keys masked and weighs each of them 1 / local_context
+    const float* add_mask;
 };
 
 //
@@ -4320,7 +4345,13 @@ __global__ __launch_bounds__(NT) void sblocal_bwd_band_kernel(BwdArgs a) {
                 for (int i = 0; i < 4; ++i) {
                     const int n = n_base + 16 * kb + 4 * g + i;
                     const bool ok = (unsigned)(n - nmin) < span;
-                    const float av = ok ? __builtin_amdgcn_exp2f(s1[kb][i] - (KEYMAJOR ? lnq[i] : ln_o)) : 0.f;
+                    float av = ok ? __builtin_amdgcn_exp2f(s1[kb][i] - (KEYMAJOR ? lnq[i] : ln_o)) : 0.f;
+                    if (a.add_mask) {                        // (uniform)
+                        const float lq = KEYMAJOR ? lnq[i] : ln_o;
+                        const long at = KEYMAJOR ? (long)n * a.S + o : (long)o * a.S + n;
+                        const float sm = ok ? s1[kb][i] + a.add_mask[at] * (a.temp * LOG2E) : 0.f;
+                        av = !ok ? 0.f : lq == -INFINITY ? 1.0f / (float)a.lc : __builtin_amdgcn_exp2f(sm - lq);
+                    }
                     const float df = ok ? s3[kb][i] - (KEYMAJOR ? cq[i] : c_o) : 0.f;
                     wdf[kb][i] = df;
                     if (a.drop_thresh != 0u) {               // (uniform)
@@ -4936,6 +4967,16 @@ extern "C" int flyhip_local_fwd_lse(const void* q, const void* k, const void* v,
                                     softmax_temp, dtype, 0.f, 0, stream);
 }
 
+extern "C" int flyhip_local_fwd_masked(const void* q, const void* k, const void* v, const int64_t* key_lengths,
+                                       const float* attn_mask, void* out, float* lse,
+                                       int B, int H, int T, int S, int E, int D, int local_context,
+                                       int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                                       int64_t k_sb, int64_t k_sh, int64_t k_ss,
+                                       int64_t v_sb, int64_t v_sh, int64_t v_ss,
+                                       int64_t o_sb, int64_t o_sh, int64_t o_ss,
+                                       float softmax_temp, int dtype, float dropout_p, uint64_t dropout_seed,
+                                       void* stream);
+
 extern "C" int flyhip_local_fwd_dropout(const void* q, const void* k, const void* v, const int64_t* key_lengths, void* out,
                                     float* lse,
                                 int B, int H, int T, int S, int E, int D, int local_context,
@@ -4944,6 +4985,20 @@ extern "C" int flyhip_local_fwd_dropout(const void* q, const void* k, const void
                                 int64_t v_sb, int64_t v_sh, int64_t v_ss,
                                 int64_t o_sb, int64_t o_sh, int64_t o_ss,
                                 float softmax_temp, int dtype, float dropout_p, uint64_t dropout_seed, void* stream) {
+    return flyhip_local_fwd_masked(q, k, v, key_lengths, nullptr, out, lse, B, H, T, S, E, D, local_context,
+                                   q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss,
+                                   softmax_temp, dtype, dropout_p, dropout_seed, stream);
+}
+
+extern "C" int flyhip_local_fwd_masked(const void* q, const void* k, const void* v, const int64_t* key_lengths,
+                                       const float* attn_mask, void* out, float* lse,
+                                       int B, int H, int T, int S, int E, int D, int local_context,
+                                       int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                                       int64_t k_sb, int64_t k_sh, int64_t k_ss,
+                                       int64_t v_sb, int64_t v_sh, int64_t v_ss,
+                                       int64_t o_sb, int64_t o_sh, int64_t o_ss,
+                                       float softmax_temp, int dtype, float dropout_p, uint64_t dropout_seed,
+                                       void* stream) {
     FLY_REQUIRE(q && k && v && out, "local_fwd: null pointer");
     FLY_REQUIRE(dropout_p >= 0.f && dropout_p < 1.f, "local_fwd: dropout_p %g not in [0, 1)", (double)dropout_p);
     FLY_REQUIRE((long)B * H * T <= 4294967295L, "local_fwd: more than 2^32 query rows");
@@ -4957,6 +5012,7 @@ extern "C" int flyhip_local_fwd_dropout(const void* q, const void* k, const void
                 q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss, softmax_temp, lse};
     const DropArgs drop = drop_args(dropout_p, dropout_seed);
     a.drop_seed = drop.seed; a.drop_thresh = drop.thresh; a.drop_scale = drop.scale;
+    a.add_mask = attn_mask;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     if (int rc_capture = refuse_capture(st)) return rc_capture;
 #define LOCAL_DISPATCH(TT)                                                                          \
@@ -4996,9 +5052,31 @@ extern "C" int flyhip_sblocal_bwd_band(const float* x1, const float* x2, const f
                                            local_context, softmax_temp, key_major, 0.f, 0, stream);
 }
 
+extern "C" int flyhip_sblocal_bwd_band_masked(const float* x1, const float* x2, const float* x3,
+                                       const float* y1, const float* y2, const float* y3,
+                                       const float* log_norm, const float* c, const int64_t* key_lengths,
+                                       const float* attn_mask,
+                                       float* o1, float* o2, float* o3,
+                                       int BH, int H, int T, int S, int E, int M, int local_context,
+                                       float softmax_temp, int key_major, float dropout_p, uint64_t dropout_seed,
+                                       void* stream);
+
 extern "C" int flyhip_sblocal_bwd_band_dropout(const float* x1, const float* x2, const float* x3,
                                        const float* y1, const float* y2, const float* y3,
                                        const float* log_norm, const float* c, const int64_t* key_lengths,
+                                       float* o1, float* o2, float* o3,
+                                       int BH, int H, int T, int S, int E, int M, int local_context,
+                                       float softmax_temp, int key_major, float dropout_p, uint64_t dropout_seed,
+                                       void* stream) {
+    return flyhip_sblocal_bwd_band_masked(x1, x2, x3, y1, y2, y3, log_norm, c, key_lengths, nullptr, o1, o2, o3,
+                                          BH, H, T, S, E, M, local_context, softmax_temp, key_major, dropout_p,
+                                          dropout_seed, stream);
+}
+
+extern "C" int flyhip_sblocal_bwd_band_masked(const float* x1, const float* x2, const float* x3,
+                                       const float* y1, const float* y2, const float* y3,
+                                       const float* log_norm, const float* c, const int64_t* key_lengths,
+                                       const float* attn_mask,
                                        float* o1, float* o2, float* o3,
                                        int BH, int H, int T, int S, int E, int M, int local_context,
                                        float softmax_temp, int key_major, float dropout_p, uint64_t dropout_seed,
@@ -5014,6 +5092,7 @@ extern "C" int flyhip_sblocal_bwd_band_dropout(const float* x1, const float* x2,
               nullptr, nullptr, nullptr};
     const DropArgs drop = drop_args(dropout_p, dropout_seed);
     a.drop_seed = drop.seed; a.drop_thresh = drop.thresh; a.drop_scale = drop.scale;
+    a.add_mask = attn_mask;
     return dispatch_bwd_band(a, E, M, key_major, stream);
 }
 

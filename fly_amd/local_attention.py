@@ -11,16 +11,30 @@ from .sblocal_attention import _HEAD_DIMS, _round_up_choice, _vector_ready
 from .sblocal_backward import BandWindows, _band_kernel_dims, _band_terms_hip
 
 
+def _additive_mask(attn_mask, T, S, device):
+    """The (T, S) additive matrix as the kernels read it: float32, contiguous, on the device; finite entries only
+    (the reference hands over additive_matrix_finite, 0 / -1e24, local_attention.py:53-56)."""
+    if attn_mask is None:
+        return None
+    if tuple(attn_mask.shape) != (T, S):
+        raise ValueError(f'attn_mask must have shape ({T}, {S}), got {tuple(attn_mask.shape)}')
+    return attn_mask.to(device=device, dtype=torch.float32).contiguous()
+
+
 def local_forward(query, key, value, local_context, softmax_temp=None, key_lengths=None, return_lse=False,
-                  dropout=(0.0, 0)):
+                  dropout=(0.0, 0), attn_mask=None):
     """query (B,T,H,E), key (B,S,H,E), value (B,S,H,D) float32 or bfloat16 GPU tensors ->
     out (B,T,H,D): query i attends to keys j with -(local_context // 2) <= j - i < (local_context + 1) // 2
     and j < key_lengths[b] (local_attention.py:68-92 for attn_mask=None).  With return_lse
     also the log of every query's softmax denominator, (B,H,T) float32 (0 for a query without keys).
     dropout = (p, seed) with p > 0: the weights are dropped after the softmax with probability p and the kept ones
     scaled by 1 / (1 - p) (local_attention.py:91, `self.dropout(torch.softmax(...))`), by a hash of (seed, batch,
-    head, query, key) formed inside the kernel instead of a stored mask."""
-    _lib.require_gpu(query, key, value, key_lengths)
+    head, query, key) formed inside the kernel instead of a stored mask.
+    attn_mask: None or a (T, S) float tensor added to q.k before the temperature (local_attention.py:53-56, 68-75:
+    additive_matrix_finite, 0 / -1e24).  -1e24 absorbs the product in float32, so a query whose visible keys are all
+    masked weighs each position of its band 1 / local_context, the positions outside the keys included (they add
+    nothing to the output; :76-81 leaves such rows as they are); its lse entry is -inf."""
+    _lib.require_gpu(query, key, value, key_lengths, attn_mask)
     if query.dtype not in (torch.float32, torch.bfloat16):
         raise NotImplementedError(f'the local attention kernel supports float32 and bfloat16, got {query.dtype}')
     if key.dtype != query.dtype or value.dtype != query.dtype:
@@ -47,9 +61,10 @@ def local_forward(query, key, value, local_context, softmax_temp=None, key_lengt
             raise ValueError(f'key_lengths must have shape ({B},)')
     out = torch.empty(B, T, H, dim, dtype=query.dtype, device=query.device)
     lse = torch.empty(B, H, T, dtype=torch.float32, device=query.device) if return_lse else None
+    add = _additive_mask(attn_mask, T, S, query.device)
     with torch.cuda.device(query.device):
-        _lib.call('flyhip_local_fwd_dropout', q.data_ptr(), k.data_ptr(), v.data_ptr(), _lib.ptr(lens), out.data_ptr(),
-                  _lib.ptr(lse), B, H, T, S, dim, dim, local_context,
+        _lib.call('flyhip_local_fwd_masked', q.data_ptr(), k.data_ptr(), v.data_ptr(), _lib.ptr(lens), _lib.ptr(add),
+                  out.data_ptr(), _lib.ptr(lse), B, H, T, S, dim, dim, local_context,
                   q.stride(0), q.stride(2), q.stride(1), k.stride(0), k.stride(2), k.stride(1),
                   v.stride(0), v.stride(2), v.stride(1), out.stride(0), out.stride(2), out.stride(1),
                   t, _lib.dtype_code(q), float(dropout[0]), int(dropout[1]), _lib.stream_ptr(query.device))
@@ -57,7 +72,7 @@ def local_forward(query, key, value, local_context, softmax_temp=None, key_lengt
 
 
 def local_backward(query, key, value, local_context, softmax_temp, key_lengths, grad_out, chunk=256,
-                   max_elements=1 << 27, out=None, lse=None, dropout=(0.0, 0)):
+                   max_elements=1 << 27, out=None, lse=None, dropout=(0.0, 0), attn_mask=None):
     """Gradients of local attention with respect to query, key and value (the reference takes them from
     autograd through fast_transformers.local_product, local_attention.py:68-92).  The band softmax is
     evaluated again for all chunks of queries at once against the windows of keys their bands touch
@@ -70,7 +85,8 @@ def local_backward(query, key, value, local_context, softmax_temp, key_lengths, 
     exp(t q_i.k_s - lse_i), delta_i = g_i.out_i); otherwise as batched library products on the GPU (host tensors are
     accepted in float64 only: the check of these formulas against autograd).  dropout = (p, seed) of the forward:
     with M the kept / (1 - p) mask, d v_s = sum_i M_is P_is g_i and d(t q_i.k_s) = P_is (M_is g_i.v_s - delta_i),
-    delta_i = g_i.out_i as before; on the band kernel only."""
+    delta_i = g_i.out_i as before; on the band kernel only.  attn_mask: the forward's additive matrix (the scores are
+    t (q.k + mask); a query with lse = -inf weighs its visible keys 1 / local_context each); on the band kernel only."""
     B, T, H, E = query.shape
     S, D = key.shape[1], value.shape[3]
     t = softmax_temp or 1 / math.sqrt(E)
@@ -91,8 +107,11 @@ def local_backward(query, key, value, local_context, softmax_temp, key_lengths, 
         delta = (G * bh(out)).sum(-1, keepdim=True)
         lens_b = None if key_lengths is None else key_lengths.to(device=Q.device, dtype=torch.int64).contiguous()
         dQ, _, dK, _, dV = _band_terms_hip(Q, K, V, G, zq, zk, lse.reshape(B * H, T, 1), delta, lens_b, H,
-                                           local_context, t, dims, dropout)
+                                           local_context, t, dims, dropout, _additive_mask(attn_mask, T, S, Q.device))
         return back(dQ, query), back(dK, key), back(dV, value)
+    if attn_mask is not None:
+        raise NotImplementedError('the gradients of local attention with an attn_mask run on the band kernel only: '
+                                  'float32 or bfloat16 GPU tensors, head dims <= 64, the forward\'s out and lse given')
     if dropout[0] > 0:
         raise NotImplementedError('the gradients of dropped local attention run on the band kernel only: float32 or '
                                   'bfloat16 GPU tensors, head dims <= 64, the forward\'s out and lse given')
@@ -122,31 +141,33 @@ class _LocalFn(torch.autograd.Function):
     """Forward on the fused kernel, gradients from local_backward."""
 
     @staticmethod
-    def forward(ctx, query, key, value, local_context, softmax_temp, key_lengths, dropout=(0.0, 0)):
+    def forward(ctx, query, key, value, local_context, softmax_temp, key_lengths, dropout=(0.0, 0), attn_mask=None):
         out, lse = local_forward(query, key, value, local_context, softmax_temp=softmax_temp, key_lengths=key_lengths,
-                                 return_lse=True, dropout=dropout)
-        ctx.save_for_backward(query, key, value, key_lengths, out, lse)
+                                 return_lse=True, dropout=dropout, attn_mask=attn_mask)
+        ctx.save_for_backward(query, key, value, key_lengths, out, lse, attn_mask)
         ctx.local_context, ctx.softmax_temp, ctx.dropout = local_context, softmax_temp, dropout
         return out
 
     @staticmethod
     def backward(ctx, grad_out):
-        query, key, value, key_lengths, out, lse = ctx.saved_tensors
+        query, key, value, key_lengths, out, lse, attn_mask = ctx.saved_tensors
         dq, dk, dv = local_backward(query, key, value, ctx.local_context, ctx.softmax_temp, key_lengths, grad_out,
-                                    out=out, lse=lse, dropout=ctx.dropout)
-        return dq, dk, dv, None, None, None, None
+                                    out=out, lse=lse, dropout=ctx.dropout, attn_mask=attn_mask)
+        return dq, dk, dv, None, None, None, None, None
 
 
-def local_attention_fn(query, key, value, local_context, softmax_temp=None, key_lengths=None, dropout=(0.0, 0)):
-    """local_forward that autograd can differentiate."""
-    return _LocalFn.apply(query, key, value, local_context, softmax_temp, key_lengths, dropout)
+def local_attention_fn(query, key, value, local_context, softmax_temp=None, key_lengths=None, dropout=(0.0, 0),
+                       attn_mask=None):
+    """local_forward that autograd can differentiate (no gradient reaches attn_mask)."""
+    return _LocalFn.apply(query, key, value, local_context, softmax_temp, key_lengths, dropout, attn_mask)
 
 
 class LocalAttention(nn.Module):
     """Softmax attention in which query i only sees keys j with
     -(local_context // 2) <= j - i < (local_context + 1) // 2.  Same constructor and forward signature
-    as the reference class.  Covered on the GPU: no attn_mask, optional length-style key_padding_mask,
-    attention dropout in training mode (inside the kernels); anything else raises NotImplementedError.  need_weights=True also returns the dense
+    as the reference class.  Covered on the GPU: optional attn_mask (its additive_matrix_finite is added inside the
+    kernels), optional length-style key_padding_mask, attention dropout in training mode (inside the kernels);
+    anything else raises NotImplementedError.  need_weights=True also returns the dense
     (B,H,T,S) matrix (local_attention.py:94-106), exp(t q.k - lse) on the band with the kernel's own
     log-denominators, as ordinary tensor algebra: an inspection path for problems of up to
     max_weight_elements entries."""
@@ -159,8 +180,9 @@ class LocalAttention(nn.Module):
         self.max_weight_elements = 1 << 26
 
     def forward(self, query, key, value, attn_mask=None, key_padding_mask=None, need_weights=False):
+        additive = None
         if attn_mask is not None and not bool(attn_mask.all_ones):
-            raise NotImplementedError('attn_mask other than all-ones is not supported by the fused kernel')
+            additive = attn_mask.additive_matrix_finite.to(query.device)    # local_attention.py:53-56
         # training-mode dropout (local_attention.py:91) runs inside the kernels: the mask is a hash of (seed, batch,
         # head, query, key); the seed is drawn per call from torch's CPU generator and kept in last_dropout_seed
         dropout = (0.0, 0)
@@ -181,7 +203,7 @@ class LocalAttention(nn.Module):
             if in_dtype == torch.float16:
                 query, key, value = query.float(), key.float(), value.float()
             out = local_attention_fn(query, key, value, self.local_context, softmax_temp=self.softmax_temp,
-                                     key_lengths=lengths, dropout=dropout)
+                                     key_lengths=lengths, dropout=dropout, attn_mask=additive)
             return (out.to(in_dtype) if in_dtype == torch.float16 else out), None
         B, T, H, E = query.shape
         S = key.shape[1]
@@ -189,12 +211,17 @@ class LocalAttention(nn.Module):
             raise NotImplementedError(f'need_weights=True materialises the (B,H,T,S) matrix: {B * H * T * S} entries '
                                       f'exceed max_weight_elements = {self.max_weight_elements}')
         out, lse = local_forward(query, key, value, self.local_context, softmax_temp=self.softmax_temp,
-                                 key_lengths=lengths, return_lse=True)
+                                 key_lengths=lengths, return_lse=True, attn_mask=additive)
         t = self.softmax_temp or 1 / math.sqrt(E)
-        scores = t * torch.einsum('bthe,bshe->bhts', query.float(), key.float())
+        scores = torch.einsum('bthe,bshe->bhts', query.float(), key.float())
+        if additive is not None:
+            scores = scores + additive.to(scores)
+        scores = t * scores
         idx = torch.arange(S, device=query.device).view(1, S) - torch.arange(T, device=query.device).view(T, 1)
         band = ((idx >= -(self.local_context // 2)) & (idx < (self.local_context + 1) // 2)).view(1, 1, T, S)
         if lengths is not None:
             band = band & (torch.arange(S, device=query.device).view(1, 1, 1, S) < lengths.view(B, 1, 1, 1))
         attn = torch.where(band, torch.exp(scores - lse.unsqueeze(-1)), scores.new_zeros(()))
+        if additive is not None:         # every visible key masked (lse = -inf): equal weights over the packed band
+            attn = torch.where(torch.isinf(lse).unsqueeze(-1), band.to(attn.dtype) / self.local_context, attn)
         return out, attn

@@ -442,7 +442,8 @@ class SBLocalAttention(nn.Module):
     -(local_context // 2) <= j - i < (local_context + 1) // 2 and through random features to the rest.
 
     Same constructor and forward signature as the reference class (sblocal_attention.py:29-44).
-    The GPU path covers what the reference itself exercises: non-causal, no attn_mask, optional
+    The GPU path covers what the reference itself exercises: non-causal, an attn_mask that hides no pair inside the
+    band (one that does fails the reference's own assertion, and so it does here), optional
     length-style key_padding_mask, softmax_eps = 0; attention dropout in training mode for float32 inputs with head
     dims <= 64 and <= 128 features (inside the band kernel, see sblocal_forward).  ``need_weights`` /
     ``return_attn_unnormalized`` (:124-136) give the dense matrix for small problems, formed with library products around
@@ -476,7 +477,18 @@ class SBLocalAttention(nn.Module):
             raise NotImplementedError('causal SBLocalAttention is not implemented (the reference '
                                       'marks it unverified, sblocal_attention.py:61)')
         if attn_mask is not None and not bool(attn_mask.all_ones):
-            raise NotImplementedError('attn_mask other than all-ones is not supported by the fused kernel')
+            # The reference adds the mask's -1e24 to the band entries of Q K^T and of Q' K'^T alike (:90-97) and then
+            # asserts that the latter are >= 0 (:105): a mask that hides any pair inside the band fails that assertion,
+            # and a mask that only hides pairs outside the band changes nothing (the low-rank part never sees it).
+            T, S = query.shape[1], key.shape[1]
+            hidden = ~attn_mask.bool_matrix
+            idx = torch.arange(S, device=hidden.device).view(1, S) - torch.arange(T, device=hidden.device).view(T, 1)
+            band = (idx >= -(self.local_context // 2)) & (idx < (self.local_context + 1) // 2)
+            if key_padding_mask is not None:
+                band = band & (torch.arange(S, device=hidden.device).view(1, S) < int(key_padding_mask.lengths.max()))
+            if bool((hidden & band).any()):
+                raise AssertionError('attn_mask hides a pair inside the band: the reference adds -1e24 to its feature '
+                                     'product and fails its own assertion (sblocal_attention.py:105)')
         if (need_weights or return_attn_unnormalized) and (
                 query.shape[0] * query.shape[2] * query.shape[1] * key.shape[1] > self.max_weight_elements):
             raise NotImplementedError('need_weights=True materialises the (B,H,T,S) matrix; supported for inspection '

@@ -228,11 +228,12 @@ def _backward_hip(Q, K, V, G, O, LN, P, lens_b, H, local_context, t, dims, piece
     return dq[..., :E], dk[..., :E], dv[..., :D]
 
 
-def _band_terms_hip(Q, K, V, G, psi, phik, LN, c, lens_b, H, local_context, t, dims, dropout=(0.0, 0)):
+def _band_terms_hip(Q, K, V, G, psi, phik, LN, c, lens_b, H, local_context, t, dims, dropout=(0.0, 0), attn_mask=None):
     """The five band-limited sums on flyhip_sblocal_bwd_band.  Q, G, psi, LN, c: (BH, T, .); K, V, phik:
     (BH, S, .); float32 on the GPU.  Returns (t sum_s dm k, sum_s df phik, t sum_i dm q, sum_i df psi,
     sum_i (a - kb) g) cut back to the callers' widths.  dropout = (p, seed) of a forward that dropped exact
-    weights: the kernels form the same mask again from the seed."""
+    weights: the kernels form the same mask again from the seed.  attn_mask: the (T, S) float32 additive matrix of
+    plain local attention (local_forward), or None."""
     from . import _lib
     BH, T, E = Q.shape
     S, D, M = K.shape[1], V.shape[2], psi.shape[2]
@@ -245,12 +246,12 @@ def _band_terms_hip(Q, K, V, G, psi, phik, LN, c, lens_b, H, local_context, t, d
     with torch.cuda.device(Q.device):
         st = _lib.stream_ptr(Q.device)
         drop = (float(dropout[0]), int(dropout[1]))
-        _lib.call('flyhip_sblocal_bwd_band_dropout', q_.data_ptr(), None, g_.data_ptr(), k_.data_ptr(), phik_.data_ptr(),
-                  v_.data_ptr(), ln_.data_ptr(), c_.data_ptr(), _lib.ptr(lens_b), dq.data_ptr(), uq.data_ptr(), None,
-                  BH, H, T, S, dim, mk, local_context, float(t), 0, *drop, st)
-        _lib.call('flyhip_sblocal_bwd_band_dropout', k_.data_ptr(), phik_.data_ptr(), v_.data_ptr(), q_.data_ptr(),
-                  psi_.data_ptr(), g_.data_ptr(), ln_.data_ptr(), c_.data_ptr(), _lib.ptr(lens_b), dk.data_ptr(),
-                  uk.data_ptr(), dv.data_ptr(), BH, H, T, S, dim, mk, local_context, float(t), 1, *drop, st)
+        _lib.call('flyhip_sblocal_bwd_band_masked', q_.data_ptr(), None, g_.data_ptr(), k_.data_ptr(), phik_.data_ptr(),
+                  v_.data_ptr(), ln_.data_ptr(), c_.data_ptr(), _lib.ptr(lens_b), _lib.ptr(attn_mask), dq.data_ptr(),
+                  uq.data_ptr(), None, BH, H, T, S, dim, mk, local_context, float(t), 0, *drop, st)
+        _lib.call('flyhip_sblocal_bwd_band_masked', k_.data_ptr(), phik_.data_ptr(), v_.data_ptr(), q_.data_ptr(),
+                  psi_.data_ptr(), g_.data_ptr(), ln_.data_ptr(), c_.data_ptr(), _lib.ptr(lens_b), _lib.ptr(attn_mask),
+                  dk.data_ptr(), uk.data_ptr(), dv.data_ptr(), BH, H, T, S, dim, mk, local_context, float(t), 1, *drop, st)
     return dq[..., :E], uq[..., :M], dk[..., :E], uk[..., :M], dv[..., :D]
 
 

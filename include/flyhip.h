@@ -199,6 +199,19 @@ int flyhip_sblocal_bwd_band_dropout(const float* x1, const float* x2, const floa
                                     float softmax_temp, int key_major, float dropout_p, uint64_t dropout_seed,
                                     void* stream);
 
+/* flyhip_sblocal_bwd_band_dropout for a forward with an additive attn_mask (flyhip_local_fwd_masked; the reference
+ * takes these gradients from autograd through src/models/attention/local_attention.py:68-92): the pair weight is
+ * exp(t (q.k + attn_mask[query][key]) - log_norm[query]), and 1 / local_context where log_norm[query] is -inf.
+ * attn_mask NULL is flyhip_sblocal_bwd_band_dropout. */
+int flyhip_sblocal_bwd_band_masked(const float* x1, const float* x2, const float* x3,
+                                   const float* y1, const float* y2, const float* y3,
+                                   const float* log_norm, const float* c, const int64_t* key_lengths,
+                                   const float* attn_mask,
+                                   float* o1, float* o2, float* o3,
+                                   int BH, int H, int T, int S, int E, int M, int local_context,
+                                   float softmax_temp, int key_major, float dropout_p, uint64_t dropout_seed,
+                                   void* stream);
+
 /* The whole backward pass after the feature maps, one call per side (same operand roles as
  * flyhip_sblocal_bwd_band, x2 = the outer rows' own features in both passes: psi for key_major = 0,
  * phik for key_major = 1).  The epilogue adds the low-rank weight outside the band ("all keys minus the
@@ -360,6 +373,21 @@ int flyhip_local_fwd_dropout(const void* q, const void* k, const void* v, const 
                              int64_t v_sb, int64_t v_sh, int64_t v_ss,
                              int64_t o_sb, int64_t o_sh, int64_t o_ss,
                              float softmax_temp, int dtype, float dropout_p, uint64_t dropout_seed, void* stream);
+
+/* flyhip_local_fwd_dropout with the attn_mask of LocalAttention.forward (ref: src/models/attention/local_attention.py:
+ * 53-56, 68-81): attn_mask (T, S) float32, rows contiguous, or NULL -- the mask's additive_matrix_finite (0 / -1e24; any
+ * finite bias is allowed), added to q.k before the temperature.  -1e24 absorbs the product in float32, so a query
+ * whose visible keys are all masked weighs every position of its band 1 / local_context, those outside the keys
+ * included (they add nothing to the output), as the reference's softmax over the packed band does; its lse entry is
+ * -inf, which flyhip_sblocal_bwd_band_masked reads as that case. */
+int flyhip_local_fwd_masked(const void* q, const void* k, const void* v, const int64_t* key_lengths,
+                            const float* attn_mask, void* out, float* lse,
+                            int B, int H, int T, int S, int E, int D, int local_context,
+                            int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                            int64_t k_sb, int64_t k_sh, int64_t k_ss,
+                            int64_t v_sb, int64_t v_sh, int64_t v_ss,
+                            int64_t o_sb, int64_t o_sh, int64_t o_ss,
+                            float softmax_temp, int dtype, float dropout_p, uint64_t dropout_seed, void* stream);
 
 /* Measurement hook (no counterpart in the reference): the two caller-owned hipEvent_t receive the begin
  * and the end time stamp of the fused band kernel's launch (hipExtLaunchKernelGGL) in the NEXT

@@ -274,8 +274,9 @@ def dense_closed_form(query, key, value, projection_matrix, local_context, softm
     return out.permute(0, 2, 1, 3), torch.log(Z), A
 
 
-def local_attention(query, key, value, local_context, softmax_temp=None, key_lengths=None):
-    """LocalAttention.forward for attn_mask=None, no dropout (local_attention.py:50-92): band-packed
+def local_attention(query, key, value, local_context, softmax_temp=None, key_lengths=None, attn_mask_additive=None):
+    """LocalAttention.forward without dropout (local_attention.py:50-92; attn_mask_additive = the (T,S)
+    additive_matrix_finite of :53-56, default zeros): band-packed
     scores from local_dot_product, softmax over the packed axis, rows without a valid key zeroed when
     a key padding mask is given, local_weighted_average.  query (B,T,H,E) -> out (B,T,H,D)."""
     B, T, H, E = query.shape
@@ -285,7 +286,8 @@ def local_attention(query, key, value, local_context, softmax_temp=None, key_len
     k = key.permute(0, 2, 1, 3)
     v = value.permute(0, 2, 1, 3)
     lengths = torch.full((B,), S, dtype=torch.long) if key_lengths is None else key_lengths
-    QK = local_dot_product(q, k, torch.zeros(T, S, dtype=q.dtype), lengths, local_context)     # :68-74
+    add = torch.zeros(T, S, dtype=q.dtype) if attn_mask_additive is None else attn_mask_additive.to(q.dtype)
+    QK = local_dot_product(q, k, add, lengths, local_context)                                  # :68-74
     attn = torch.softmax(t * QK, dim=-1)                                                       # :75
     if key_lengths is not None:                                                                # :82-88
         i = torch.arange(T).view(1, 1, T, 1)

@@ -558,6 +558,81 @@ def test_local_attention_dropout_inside_the_kernels(dtype, tol, E, p_drop):
     assert rel_err(plain.float(), torch.einsum('bhts,bshd->bthd', prob, vd).detach()) <= (1e-4 if dtype == torch.float32 else 2e-2)
 
 
+@pytest.mark.parametrize('dtype,tol,E,p_keep', [(torch.float32, 2e-4, 64, 0.6), (torch.float32, 2e-4, 40, 0.9),
+                                                (torch.bfloat16, 3e-2, 64, 0.6)])
+def test_local_attention_with_attn_mask(dtype, tol, E, p_keep):
+    """LocalAttention with an attn_mask (local_attention.py:53-56, 68-81): its additive matrix (0 / -1e24) is added
+    inside the forward kernel and both band kernels of the backward.  Output, gradients and need_weights against the
+    oracle in float64 (autograd through it for the gradients): a random FullMask with queries whose visible keys are
+    all hidden (equal weights 1 / local_context there, as the reference's packed softmax gives), T != S, key lengths,
+    a head dim that needs padding; then a mask that hides nothing (bit-identical to no mask)."""
+    from fly_amd import LocalAttention, LengthMask, FullMask
+    B, T, S, H, D, lc = 2, 300, 280, 2, E, 64
+    print('case', dtype, E, p_keep, flush=True)
+    g = torch.Generator().manual_seed(35)
+    q, k, v = (torch.randn(B, L, H, C, generator=g).to(dtype) for L, C in ((T, E), (S, E), (S, D)))
+    keep = torch.rand(T, S, generator=g) < p_keep
+    keep[5] = False
+    keep[130:133] = False
+    keep[250, :230] = False                   # its visible keys lie beyond the second batch entry's length
+    lengths = torch.tensor([S, 200])
+    w = torch.randn(B, T, H, D, generator=g)
+    dev = torch.device('cuda:0')
+    mod = LocalAttention(lc).to(dev)
+    qg, kg, vg = (x.to(dev).requires_grad_() for x in (q, k, v))
+    amask, kmask = FullMask(keep.to(dev)), LengthMask(lengths.to(dev), max_len=S)
+    out, none = mod(qg, kg, vg, attn_mask=amask, key_padding_mask=kmask)
+    assert none is None and out.dtype == dtype
+    (out.float() * w.to(dev)).sum().backward()
+
+    qd, kd, vd = (x.double().requires_grad_() for x in (q, k, v))
+    add = (~keep).double() * -1e24
+    ref = osb.local_attention(qd, kd, vd, lc, key_lengths=lengths, attn_mask_additive=add)
+    (ref * w.double()).sum().backward()
+    assert rel_err(out.float(), ref.detach()) <= (1e-4 if dtype == torch.float32 else 2e-2), rel_err(out.float(), ref.detach())
+    for got, want, name in ((qg.grad, qd.grad, 'dq'), (kg.grad, kd.grad, 'dk'), (vg.grad, vd.grad, 'dv')):
+        assert got.dtype == dtype and rel_err(got.float(), want) <= tol, (name, rel_err(got.float(), want))
+    assert float(kg.grad[1, 200:].abs().max()) == 0.0
+    # the hidden rows: the mean of their visible values times (visible count / local_context)
+    vis5 = v[:, max(0, 5 - lc // 2):5 + (lc + 1) // 2].double().sum(1) / lc
+    assert rel_err(out[:, 5].float(), vis5) <= (1e-5 if dtype == torch.float32 else 2e-2)
+    # dense weights (local_attention.py:94-106) from the kernel's own log-denominators
+    with torch.no_grad():
+        out_w, attn = mod(qg, kg, vg, attn_mask=amask, key_padding_mask=kmask, need_weights=True)
+    assert torch.equal(out_w, out.detach())
+    again = torch.einsum('bhts,bshd->bthd', attn.double().cpu(), v.double())
+    assert rel_err(again, ref.detach()) <= (1e-4 if dtype == torch.float32 else 2e-2)
+    assert abs(float(attn[0, 0, 5].sum()) - min(5 + (lc + 1) // 2, S) / lc) < 1e-5
+    # a mask that hides nothing is the unmasked kernel
+    with torch.no_grad():
+        a, _ = mod(qg, kg, vg, attn_mask=FullMask(torch.ones(T, S, dtype=torch.bool, device=dev)), key_padding_mask=kmask)
+        b, _ = mod(qg, kg, vg, key_padding_mask=kmask)
+    assert torch.equal(a, b)
+
+
+def test_sblocal_attn_mask_follows_the_references_assertion():
+    """SBLocalAttention with an attn_mask (sblocal_attention.py:62-65, 90-105): a mask that hides a pair inside the
+    band fails the reference's own assertion on the feature products, one that only hides pairs outside the band
+    changes nothing."""
+    from fly_amd import SBLocalAttention, FullMask
+    dev = torch.device('cuda:0')
+    B, L, H, E, lc = 1, 192, 2, 64, 32
+    g = torch.Generator().manual_seed(36)
+    q, k, v = (torch.randn(B, L, H, E, generator=g).to(dev) * 0.5 for _ in range(3))
+    mod = SBLocalAttention(lc, dim_heads=E, nb_features=64).to(dev).eval()
+    i, j = torch.arange(L).view(L, 1), torch.arange(L).view(1, L)
+    band = (j - i >= -(lc // 2)) & (j - i < (lc + 1) // 2)
+    outside = band | (torch.rand(L, L, generator=g) < 0.5)
+    with torch.no_grad():
+        plain, _ = mod(q, k, v)
+        same, _ = mod(q, k, v, attn_mask=FullMask(outside.to(dev)))
+        assert torch.equal(plain, same)
+        inside = outside.clone()
+        inside[100, 101] = False
+        with pytest.raises(AssertionError):
+            mod(q, k, v, attn_mask=FullMask(inside.to(dev)))
+
+
 @pytest.mark.parametrize('B,T,S,H,E,D,mh,lc,lens', [(2, 300, 280, 2, 64, 64, 32, 64, [280, 200]),
                                                     (1, 257, 391, 3, 50, 40, 24, 77, None),
                                                     (2, 130, 130, 1, 32, 32, 16, 301, [130, 1]),

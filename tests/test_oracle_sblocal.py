@@ -189,6 +189,42 @@ def test_local_attention_equals_dense_masked_softmax():
         assert (out - ref).abs().max() < 1e-12
 
 
+def test_local_attention_with_an_additive_mask():
+    """LocalAttention with attn_mask (local_attention.py:53-56, 68-81: additive_matrix_finite added to Q K^T inside
+    the band-packed product).  Rows that keep a visible key equal a dense softmax with -inf on band, lengths and mask;
+    a row whose visible keys are all masked has equal scores everywhere in its packed band, i.e. weights
+    1 / local_context, and its output is the sum of its visible values over local_context (the reference leaves such
+    rows as they are, :76-81); a general finite bias equals the dense softmax of t (q.k + bias)."""
+    g = torch.Generator().manual_seed(18)
+    for (B, T, S, H, E, D, lc, lens) in [(2, 40, 40, 2, 8, 5, 7, None), (2, 33, 50, 1, 4, 6, 12, [50, 21])]:
+        q = torch.randn(B, T, H, E, generator=g, dtype=torch.float64)
+        k = torch.randn(B, S, H, E, generator=g, dtype=torch.float64)
+        v = torch.randn(B, S, H, D, generator=g, dtype=torch.float64)
+        kl = None if lens is None else torch.tensor(lens)
+        keep = torch.rand(T, S, generator=g) < 0.6
+        keep[3] = False                                     # a query with every key hidden
+        keep[T - 2] = False
+        add = (~keep).double() * -1e24
+        out = osb.local_attention(q, k, v, lc, softmax_temp=0.4, key_lengths=kl, attn_mask_additive=add)
+        i = torch.arange(T).view(T, 1)
+        j = torch.arange(S).view(1, S)
+        band = ((j - i) >= -(lc // 2)) & ((j - i) < (lc + 1) // 2)
+        limit = torch.full((B,), S) if kl is None else kl
+        vis = band.view(1, 1, T, S) & (j.view(1, 1, 1, S) < limit.view(B, 1, 1, 1))
+        ok = vis & keep.view(1, 1, T, S)
+        s = 0.4 * torch.einsum('bthe,bshe->bhts', q, k)
+        w = torch.softmax(s.masked_fill(~ok, float('-inf')), dim=-1).nan_to_num(0.0)
+        hidden_row = vis.any(-1, keepdim=True) & ~ok.any(-1, keepdim=True)
+        w = torch.where(hidden_row, vis.double() / lc, w)
+        ref = torch.einsum('bhts,bshd->bthd', w, v)
+        assert bool(hidden_row.any()) and (out - ref).abs().max() < 1e-12
+        bias = torch.randn(T, S, generator=g, dtype=torch.float64)
+        out = osb.local_attention(q, k, v, lc, softmax_temp=0.4, key_lengths=kl, attn_mask_additive=bias)
+        w = torch.softmax((0.4 * (torch.einsum('bthe,bshe->bhts', q, k) + bias)).masked_fill(~vis, float('-inf')), -1)
+        ref = torch.einsum('bhts,bshd->bthd', w.nan_to_num(0.0), v)
+        assert (out - ref).abs().max() < 1e-12
+
+
 @pytest.mark.parametrize('B,T,S,H,E,D,mh,lc,lens', [(1, 40, 40, 2, 16, 16, 8, 12, None),
                                                     (2, 70, 55, 2, 16, 24, 8, 13, [55, 31]),
                                                     (1, 300, 300, 1, 8, 8, 4, 64, None)])
