@@ -393,6 +393,11 @@ def bench_other_configs():
     q, k, v = (torch.randn(B, L, 1, E, generator=g).to(dev) * E ** -0.25 for _ in range(3))
     with torch.no_grad():
         out['sbblocksparse_fp32_B64_L3136_block32_m32'] = {'ms': timeit(lambda: sbbs(q, k, v), n=5)}
+        # training-mode dropout of the exact weights inside the same kernels (a fresh seed per call)
+        sbbs_drop = fly_amd.SBBlockSparseAttention(WindowPlusGlobal(32), dim_heads=E, nb_features=32, max_seq_length=L,
+                                                   attention_dropout=0.1).to(dev).train()
+        out['sbblocksparse_fp32_B64_L3136_block32_m32']['dropout_fwd_ms'] = timeit(lambda: sbbs_drop(q, k, v), n=5)
+        del sbbs_drop
     # its training step: fused forward, backward kernels walking the layout's blocks; beside it the op-by-op path
     qg, kg, vg = (x.clone().requires_grad_() for x in (q, k, v))
     go = torch.randn_like(v)

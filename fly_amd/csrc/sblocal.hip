@@ -4099,20 +4099,23 @@ template <typename T, int E, int M>
 static int launch_fwd_list(const FwdArgs& a, hipStream_t st) {
     constexpr bool X3 = E <= 64 && M <= 128;
     const bool pieces = X3 && a.vt != nullptr;
-    if (a.vt && !(X3 && a.drop_thresh == 0))
-        return fail(ERR_UNSUPPORTED, "sbblocksparse_fwd: tile images are for head dims up to 64, up to 128 features and no "
-                                     "dropout (got %d, %d)", E, M);
+    if (a.vt && !X3)
+        return fail(ERR_UNSUPPORTED, "sbblocksparse_fwd: tile images are for head dims up to 64 and up to 128 features "
+                                     "(got %d, %d)", E, M);
+    const bool dropping = a.drop_thresh != 0u;
     const void* kern_fp32 = reinterpret_cast<const void*>(sblocal_fwd_kernel<float, E, E, M, false, true>);
     const void* kern = kern_fp32;
     size_t smem = fwd_smem<E, M>();
     static std::atomic<unsigned long long> lds_set{0}, lds_set_x3{0};     // (devices on which the kernels have their LDS limit)
     if constexpr (X3) {
         if (pieces) {
-            kern = reinterpret_cast<const void*>(sblocal_fwd_x3_kernel<E, E, M, false, false, true>);
+            kern = dropping ? reinterpret_cast<const void*>(sblocal_fwd_x3_kernel<E, E, M, false, true, true>)
+                            : reinterpret_cast<const void*>(sblocal_fwd_x3_kernel<E, E, M, false, false, true>);
             smem = fwd_x3_smem<E, M>();
         }
     }
-    if (int rc = ensure_dynamic_lds(kern, smem, pieces ? lds_set_x3 : lds_set, "sbblocksparse_fwd")) return rc;
+    static std::atomic<unsigned long long> lds_set_x3d{0};
+    if (int rc = ensure_dynamic_lds(kern, smem, pieces ? (dropping ? lds_set_x3d : lds_set_x3) : lds_set, "sbblocksparse_fwd")) return rc;
     // every XCD gets room for ceil(B H / dies) (batch, head) pairs
     const Machine& mach = machine();
     const long grid = (((long)a.B * a.H + mach.xcds - 1) / mach.xcds) * ((a.T + TQ - 1) / TQ) * mach.xcds;
@@ -4125,7 +4128,9 @@ static int launch_fwd_list(const FwdArgs& a, hipStream_t st) {
     args.n_xcd = mach.xcds;
     args.band_wgs = (int)(grid + part_wgs);
     if constexpr (X3) {
-        if (pieces)
+        if (pieces && dropping)
+            hipLaunchKernelGGL((sblocal_fwd_x3_kernel<E, E, M, false, true, true>), dim3((unsigned)(grid + part_wgs)), dim3(NT), smem, st, args);
+        else if (pieces)
             hipLaunchKernelGGL((sblocal_fwd_x3_kernel<E, E, M, false, false, true>), dim3((unsigned)(grid + part_wgs)), dim3(NT), smem, st, args);
     }
     if (!pieces)

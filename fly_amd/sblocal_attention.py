@@ -383,8 +383,8 @@ def sbblocksparse_forward(query, key, value, projection_matrix, tables, softmax_
     q, k, v = prep(query), prep(key), prep(value)
     proj = _padded_projection(projection_matrix, mh, dim, cache)
 
-    # tile images of the key pass (the band kernel on bf16 pieces) where that kernel exists; dropout lives in the fp32 kernel
-    images = dropout_p == 0 and dim <= 64 and mh <= 64
+    # tile images of the key pass (the band kernel on bf16 pieces) where that kernel exists
+    images = dim <= 64 and mh <= 64
 
     def make_plan():
         return SBLocalPlan(B, H, T, S, dim, mh, mh_valid, query.dtype, query.device, 64, n_parts=1,

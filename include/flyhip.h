@@ -304,8 +304,8 @@ int flyhip_sbblocksparse_bwd_pieces(const void* outer_images, const void* inner_
  * for need_weights = False, no masks): as flyhip_sblocal_fwd with one part per query tile, but the
  * exact part covers the nonzero blocks of a layout (16 x 16 or 32 x 32) instead of a band.  Key-side inputs (kfeat,
  * chunk_scale, kv, ksum, kmax) from flyhip_sb_kv_reduce; vt = the tile images that pass leaves when asked for them
- * (then kfeat holds feature images and the band kernel runs on bf16 pieces: head dims up to 64, up to 128 features,
- * dropout_p = 0), or NULL (fp32 features in kfeat, the kernel on the fp32 matrix pipe).  tl_ptr (H * ceil(T/64) + 1), tl_inner, tl_mask (4 per
+ * (then kfeat holds feature images and the band kernel runs on bf16 pieces: head dims up to 64, up to 128
+ * features), or NULL (fp32 features in kfeat, the kernel on the fp32 matrix pipe).  tl_ptr (H * ceil(T/64) + 1), tl_inner, tl_mask (4 per
  * entry): per (head, 64-query tile) the 32-key tiles that any of its queries sees on the support, and per entry and
  * group of 16 queries (16 w .. 16 w + 15 of the tile) a mask: bit 0 = keys 0..15, bit 1 = keys 16..31 of that tile
  * are on the support for those queries (32 x 32 blocks: 0 or 3, the same for w = 0, 1 and for w = 2, 3).
