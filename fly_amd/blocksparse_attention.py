@@ -16,6 +16,16 @@ from .masking import FullMask, LengthMask, pad_mask
 from .padding import pad_to_multiple
 
 
+def _cut(out, seqlen, dim):
+    """out[:, :seqlen, :, :dim] -- sliced only where something is cut off: under autograd every slice, also one that
+    keeps everything, costs a zero-fill and a copy of the whole tensor in the backward pass."""
+    if out.shape[1] != seqlen:
+        out = out[:, :seqlen]
+    if out.shape[3] != dim:
+        out = out[..., :dim]
+    return out
+
+
 class _AttentionCoreFn(torch.autograd.Function):
     """softmax(scale * q k^T + masks) v on the nonzero blocks, for calls that need gradients.  With masks
     the forward is the reference's three ops (blocksparse_attention.py:134-160; the probabilities are
@@ -223,7 +233,7 @@ class BlockSparseAttention(nn.Module):
                 add_mask = attn_mask.additive_matrix        # (T, S), read per nonzero block inside the kernel
             out = self.fused_cache[T, S](q, k, v, softmax_temp, key_mask, attn_mask=add_mask, dropout=dropout)
             self.last_dropout_seed = dropout[1] if dropout[0] > 0 else None
-            return out.permute(0, 2, 1, 3)[:, :q_seqlen_og, :, :v_dim_og], None
+            return _cut(out.permute(0, 2, 1, 3), q_seqlen_og, v_dim_og), None
         sdd_nt, dsd_nn, sparse_softmax = self.get_ops(T, S)
         unmasked = ((key_padding_mask is None or key_padding_mask.all_ones)
                     and (attn_mask is None or attn_mask.all_ones))
@@ -242,7 +252,7 @@ class BlockSparseAttention(nn.Module):
                 q, k, v, sdd_nt, dsd_nn, sparse_softmax, softmax_temp,
                 None if fused is not None or key_padding_mask is None else key_padding_mask.additive_matrix,
                 None if fused is not None or attn_mask is None else attn_mask.additive_matrix, fused, dropout)
-            return out.permute(0, 2, 1, 3)[:, :q_seqlen_og, :, :v_dim_og], None
+            return _cut(out.permute(0, 2, 1, 3), q_seqlen_og, v_dim_og), None
         qk = sdd_nt(q, k)
         attn = sparse_softmax(qk, scale=softmax_temp,
                               key_padding_mask=None if key_padding_mask is None else key_padding_mask.additive_matrix,
@@ -257,4 +267,4 @@ class BlockSparseAttention(nn.Module):
         weights = None
         if need_weights:
             weights = densify_tensor(attn, layout)[:, :, :q_seqlen_og, :k_seqlen_og]
-        return out.permute(0, 2, 1, 3)[:, :q_seqlen_og, :, :v_dim_og], weights
+        return _cut(out.permute(0, 2, 1, 3), q_seqlen_og, v_dim_og), weights

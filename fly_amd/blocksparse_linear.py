@@ -153,8 +153,14 @@ class BlockSparseLinear(nn.Module):
             pad_tok = -n_tok % self.block_size
             if pad_in or pad_tok:
                 tokens = F.pad(tokens, (0, pad_in, 0, pad_tok))
-            y = self.get_ops()(tokens[None, None], self.weight)[0, 0]
-            y = y[:n_tok].reshape(*lead, y.shape[-1])
-        y = y[..., :self.out_features]
+            # (views only, and slices only where something is cut off: under autograd a select or a slice of the
+            #  result, also one that keeps everything, costs a zero-fill and a copy of the whole tensor on the way back)
+            y = self.get_ops()(tokens.view(1, 1, *tokens.shape), self.weight)
+            y = y.view(y.shape[2], y.shape[3])
+            if pad_tok:
+                y = y[:n_tok]
+            y = y.reshape(*lead, y.shape[-1])
+        if y.shape[-1] != self.out_features:
+            y = y[..., :self.out_features]
         # the bias joins in the dtype of the product (under autocast the product is half precision)
         return y if self.bias is None else y + self.bias.to(y.dtype)

@@ -998,15 +998,16 @@ constexpr int DDS_MAX_STEPS = 128;   // longest reduction list the tiled kernel 
 
 template <typename T, bool WT, int DIST = FLY_DDS_DIST>     // WT: blocks are [k][n] (y = x W) and are transposed on their way into LDS
 __global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
-    constexpr int KB = 1;                                   // input blocks per pipeline step
-    // LDS tiles are [row][32 k] with 64-byte rows and no padding; the four 16-byte chunks of a row are
-    // stored at chunk ^ swz(row), swz(r) = ((r >> 1) & 3) ^ ((r >> 3) & 1).  Then both the 16-byte
-    // fragment reads (16 consecutive rows, one chunk) and the staging writes (4 rows x 4 chunks per 16
-    // lanes) spread evenly over the banks, whether 8 or 16 lanes are served per clock.
-    constexpr int LD = 32;
-    __shared__ __attribute__((aligned(16))) uint16_t xs[2][128 * LD];
-    __shared__ __attribute__((aligned(16))) uint16_t ws[2][128 * LD];
-    auto swz = [](int r) { return ((r >> 1) & 3) ^ ((r >> 3) & 1); };
+    // A pipeline step takes TWO entries of the reduction list.  The LDS tiles are [row][64 k] with 128-byte rows, the
+    // first entry's 32 inputs in front; the eight 16-byte chunks of a row are stored at chunk ^ ((row >> 1) & 7).  Then
+    // both the 16-byte fragment reads (16 consecutive rows, one chunk) and the staging writes (2 rows x 8 chunks per 16
+    // lanes) cover all 64 banks.  Neighbouring entries of a list are mostly neighbouring input blocks: a staging wave
+    // then reads whole 128-byte lines of eight token rows (a compute unit's vector memory path takes one line about
+    // every four cycles whether half of it is used or all of it).
+    constexpr int LD = 64;
+    extern __shared__ __attribute__((aligned(16))) uint16_t dds_smem[];
+    uint16_t (*xs)[128 * LD] = reinterpret_cast<uint16_t (*)[128 * LD]>(dds_smem);
+    uint16_t (*ws)[128 * LD] = reinterpret_cast<uint16_t (*)[128 * LD]>(dds_smem + 2 * 128 * LD);
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r16 = lane & 15, g = lane >> 4;
     const int wm = w >> 1, wn = w & 1;                      // this wave: tokens 64wm.., outputs 64wn..
     const int z = blockIdx.z;
@@ -1026,7 +1027,7 @@ __global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
     const uint16_t* spz = reinterpret_cast<const uint16_t*>(a.sp) + z * a.sp_sz;
     const uint16_t* xp = reinterpret_cast<const uint16_t*>(a.dn) + z * a.dn_sz + head * a.dn_sh;
 
-    // the group's reduction list (inner block per step, block id per step and output block-row) is
+    // the group's reduction list (inner block per entry, block id per entry and output block-row) is
     // read once into LDS: the per-step loads then depend on no other global load
     __shared__ int s_inner[DDS_MAX_STEPS];
     __shared__ int s_blk[4][DDS_MAX_STEPS];
@@ -1037,71 +1038,71 @@ __global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
     }
     __syncthreads();
 
-    // staging roles: thread -> (row = tid/4 [+64], 16-byte chunk = tid%4) of the x and W tiles of one
-    // input block; a step moves KB input blocks
-    const int srow = tid >> 2, schunk = (tid & 3) * 8;
-    static_assert(KB == 1, "the tile cursors below advance one input block per step");
-    const int n_steps = my_tiles * nin;
-    // two register sets: the loads of step s+2 are issued while step s computes and are parked in LDS
-    // one iteration later, so every global load has two steps to arrive
+    // staging roles: thread -> (row = tid/8 + 32 hh, 16-byte chunk = tid%8) of the x and W tiles; chunks 0..3 belong
+    // to the step's first entry, 4..7 to its second
+    const int srow = tid >> 3, sc = tid & 7, sel = sc >> 2, schunk = (sc & 3) * 8;
+    const int npair = (nin + 1) / 2;
+    const int n_steps = my_tiles * npair;
+    // DIST register sets: the loads of step s+DIST are issued while step s computes and are parked in LDS
+    // one iteration before they are used
     // (native vectors: arrays of the uint4 struct passed by reference do not stay in registers)
     // Every fetch issues the same number of loads on every path (a step past the end re-reads the last
     // one, an absent weight block reads block 0 and is zeroed when it is parked): only then can the
     // compiler count how many newer loads may stay in flight when it waits for the older set.
-    uintx4 rx[DIST][KB][2], rw[DIST][KB][2];                // set j holds the steps congruent to j modulo DIST
-    bool wl[DIST][KB][2];                                   // weight block present?
+    uintx4 rx[DIST][4], rw[DIST][4];                        // set j holds the steps congruent to j modulo DIST
+    bool wl[DIST][4];                                       // weight block present?
     int f_tile = 0, f_t = 0;                                // fetch cursor: (token tile, step inside it)
-    // A load is "wave-uniform base + per-thread byte offset": the input block and the weight block of a
-    // step are the same for the whole wave (a wave stages rows of one output block: (tid / 4) / 32 = w / 2),
-    // so they come out of LDS once through the first lane and the bases are formed on the scalar unit;
-    // the per-thread offsets change only with the token tile.
-    const int obw = w >> 1;                                 // output block (of the group's four) of this wave's rows, +2 for the upper half
-    const uint32_t woff = (uint32_t)(((srow & 31) * 32 + schunk) * 2);
-    uint32_t xoff[2] = {0, 0};
-    auto fetch = [&](uintx4 (&rx)[KB][2], uintx4 (&rw)[KB][2], bool (&wl)[KB][2]) __attribute__((always_inline)) {
+    // A load is "base + per-thread byte offset": the two input blocks of a step and the weight blocks of its eight
+    // (output block, entry) pairs come out of LDS once through the first lane; a thread picks the entry its chunk
+    // belongs to; the per-thread offsets change only with the token tile.
+    const uint32_t woff = (uint32_t)((srow * 32 + schunk) * 2);
+    uint32_t xoff[4] = {0, 0, 0, 0};
+    auto fetch = [&](uintx4 (&rx)[4], uintx4 (&rw)[4], bool (&wl)[4]) __attribute__((always_inline)) {
         const bool live = f_tile < my_tiles;                 // past the end: re-read the last step, zero weights
-        const int tc = live ? f_t : nin - 1;
+        const int tc = live ? f_t : npair - 1;
         if (f_t == 0) {
             const long m0 = ((long)ty + (long)min(f_tile, my_tiles - 1) * gy) * 128;
 #pragma unroll
-            for (int hh = 0; hh < 2; ++hh) {
-                const long m = min(m0 + srow + 64 * hh, (long)a.M - 1);          // clamped: masked at the store
+            for (int hh = 0; hh < 4; ++hh) {
+                const long m = min(m0 + srow + 32 * hh, (long)a.M - 1);          // clamped: masked at the store
                 xoff[hh] = (uint32_t)((m * a.dn_sm + schunk) * 2);
             }
         }
-        const int inner = __builtin_amdgcn_readfirstlane(s_inner[tc]);
-        const char* xb = reinterpret_cast<const char*>(xp + (long)inner * 32);
+        const int t0 = 2 * tc, t1 = min(2 * tc + 1, nin - 1);
+        const bool second = 2 * tc + 1 < nin;                // an odd list's last step: its second entry is absent
+        const int in0 = __builtin_amdgcn_readfirstlane(s_inner[t0]), in1 = __builtin_amdgcn_readfirstlane(s_inner[t1]);
+        const char* xb = reinterpret_cast<const char*>(xp + (long)(sel ? in1 : in0) * 32);
 #pragma unroll
-        for (int hh = 0; hh < 2; ++hh) {
-            rx[0][hh] = *reinterpret_cast<const uintx4*>(xb + xoff[hh]);
-            const int blk_id = __builtin_amdgcn_readfirstlane(s_blk[obw + 2 * hh][tc]);
-            wl[0][hh] = live && blk_id >= 0;                 // a missing block contributes zero weights
-            rw[0][hh] = *reinterpret_cast<const uintx4*>(reinterpret_cast<const char*>(spz + (long)max(blk_id, 0) * 1024) + woff);
+        for (int hh = 0; hh < 4; ++hh) {
+            rx[hh] = *reinterpret_cast<const uintx4*>(xb + xoff[hh]);
+            const int b0 = __builtin_amdgcn_readfirstlane(s_blk[hh][t0]), b1 = __builtin_amdgcn_readfirstlane(s_blk[hh][t1]);
+            const int blk_id = sel ? (second ? b1 : -1) : b0;
+            wl[hh] = live && blk_id >= 0;                    // a missing block contributes zero weights
+            rw[hh] = *reinterpret_cast<const uintx4*>(reinterpret_cast<const char*>(spz + (long)max(blk_id, 0) * 1024) + woff);
         }
-        if (++f_t == nin) { f_t = 0; ++f_tile; }
+        if (++f_t == npair) { f_t = 0; ++f_tile; }
     };
     // The weight tile sits in LDS in the order the MFMAs read it: row 64*(n/64) + 16*i + r holds output
     // n = 64*(n/64) + 32*(i/2) + 8*(r/4) + 4*(i%2) + r%4, so that a wave's fragment read walks 16
-    // consecutive LDS rows (rows 16 apart share their banks at this row stride).
+    // consecutive LDS rows.
     auto wrow = [](int n) { const int b = n & 31; return (n & 64) + 16 * (2 * ((n >> 5) & 1) + ((b >> 2) & 1)) + 4 * (b >> 3) + (b & 3); };
-    const int wrow0 = wrow(srow);
-    const int xs_off = srow * LD + 8 * ((tid & 3) ^ swz(srow));        // + 64 rows for the upper half (same swizzle)
-    const int ws_off = wrow0 * LD + 8 * ((tid & 3) ^ swz(wrow0));
-    auto stash = [&](int buf, const uintx4 (&rx)[KB][2], const uintx4 (&rw)[KB][2], const bool (&wl)[KB][2]) __attribute__((always_inline)) {
+    auto slot_of = [](int row, int chunk) { return row * LD + 8 * (chunk ^ ((row >> 1) & 7)); };
+    auto stash = [&](int buf, const uintx4 (&rx)[4], const uintx4 (&rw)[4], const bool (&wl)[4]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int hh = 0; hh < 2; ++hh) {
-            *reinterpret_cast<uintx4*>(&xs[buf][xs_off + 64 * hh * LD]) = rx[0][hh];
-            const uintx4 wv = wl[0][hh] ? rw[0][hh] : uintx4{0, 0, 0, 0};
+        for (int hh = 0; hh < 4; ++hh) {
+            *reinterpret_cast<uintx4*>(&xs[buf][slot_of(srow + 32 * hh, sc)]) = rx[hh];
+            const uintx4 wv = wl[hh] ? rw[hh] : uintx4{0, 0, 0, 0};
             if (!WT) {
-                *reinterpret_cast<uintx4*>(&ws[buf][ws_off + 64 * hh * LD]) = wv;
+                // block row srow of output block hh, inputs schunk .. of entry `sel`
+                *reinterpret_cast<uintx4*>(&ws[buf][slot_of(wrow(32 * hh + srow), sc)]) = wv;
             } else {
-                // the thread holds row k = orow % 32 of the block, columns n = schunk .. schunk + 7: the
+                // the thread holds row k = srow of the block [k][n], columns n = schunk .. schunk + 7: the
                 // LDS tile is [n][k] either way, so these eight go out one by one
-                const int orow = srow + 64 * hh, k = orow & 31;
+                const int kk = 32 * sel + srow;
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
-                    const int n = wrow(32 * (orow >> 5) + schunk + e);
-                    ws[buf][n * LD + 8 * ((k >> 3) ^ swz(n)) + (k & 7)] = (uint16_t)(wv[e >> 1] >> (16 * (e & 1)));
+                    const int n = wrow(32 * hh + schunk + e);
+                    ws[buf][slot_of(n, kk >> 3) + (kk & 7)] = (uint16_t)(wv[e >> 1] >> (16 * (e & 1)));
                 }
             }
         }
@@ -1132,24 +1133,25 @@ __global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
         }
     };
     int c_tile = 0, c_t = 0;                                // compute cursor
-    const int frag_off = r16 * LD + 8 * (g ^ swz(r16));     // this lane's 16 bytes inside a 16-row fragment
+    // this lane's 16 bytes inside a 16-row fragment, per entry of the step (fragments start at multiples of 16 rows)
+    const int frag_off[2] = {r16 * LD + 8 * (g ^ (r16 >> 1)), r16 * LD + 8 * ((4 + g) ^ (r16 >> 1))};
     auto compute = [&](int cur) __attribute__((always_inline)) {
         if (wave_active) {
 #pragma unroll
-            for (int kb = 0; kb < KB; ++kb) {
+            for (int kb = 0; kb < 2; ++kb) {
                 uint4 fx[4], fw[4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    fx[i] = *reinterpret_cast<const uint4*>(&xs[cur][(64 * wm + 16 * i) * LD + frag_off]);
+                    fx[i] = *reinterpret_cast<const uint4*>(&xs[cur][(64 * wm + 16 * i) * LD + frag_off[kb]]);
                     // W-tile i covers output block i/2; its MFMA row r is block row 8*(r/4) + 4*(i%2) + r%4
-                    fw[i] = *reinterpret_cast<const uint4*>(&ws[cur][(64 * wn + 16 * i) * LD + frag_off]);
+                    fw[i] = *reinterpret_cast<const uint4*>(&ws[cur][(64 * wn + 16 * i) * LD + frag_off[kb]]);
                 }
 #pragma unroll
                 for (int tm = 0; tm < 4; ++tm)
 #pragma unroll
                     for (int tn = 0; tn < 4; ++tn) acc[tm][tn] = Frag32<T>::mma(fw[tn], fx[tm], acc[tm][tn]);
             }
-            if (++c_t == nin) { store_tile(c_tile); c_t = 0; ++c_tile; }     // the tile's last input block
+            if (++c_t == npair) { store_tile(c_tile); c_t = 0; ++c_tile; }   // the tile's last entries
         }
     };
     if (nin == 0) {                                         // no input block: zero rows
@@ -1163,7 +1165,7 @@ __global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
     // register set and stage index is a constant.
 #pragma unroll
     for (int j = 0; j < DIST; ++j) fetch(rx[j], rw[j], wl[j]);
-    drain_loads_but<4 * KB * (DIST - 1)>();                  // set 0 has arrived
+    drain_loads_but<8 * (DIST - 1)>();                       // set 0 has arrived
     stash(0, rx[0], rw[0], wl[0]);
     __syncthreads();
     constexpr int U = (DIST % 2 == 0) ? DIST : 2 * DIST;
@@ -1175,7 +1177,7 @@ __global__ __launch_bounds__(256) void bs_dds32_kernel(DdsGroupArgs a) {
             fetch(rx[u % DIST], rw[u % DIST], wl[u % DIST]);                    // step + u + DIST; its set was parked an iteration ago
             if (step + u < n_steps) compute(u & 1);
             stash((u + 1) & 1, rx[(u + 1) % DIST], rw[(u + 1) % DIST], wl[(u + 1) % DIST]);
-            drain_loads_but<4 * KB * (DIST - 1)>();         // the set parked next iteration has arrived
+            drain_loads_but<8 * (DIST - 1)>();              // the set parked next iteration has arrived
             __syncthreads();
         }
     }
@@ -2312,19 +2314,24 @@ extern "C" int flyhip_bs_dds(const void* a, const void* b_sp, void* c,
 #undef DDS_STAT
             return check_launch("bs_dds32s_kernel");
         }
-        // as many workgroups as are resident together (three fit a CU); each walks its share of the token tiles
+        // as many workgroups as are resident together (two fit a CU: 64 KB of tiles each); each walks its share of the
+        // token tiles
         const long tiles = (M + 127) / 128;
-        long gy = (3L * mach.cus + (long)n_grp * Z - 1) / ((long)n_grp * Z);
+        long gy = (2L * mach.cus + (long)n_grp * Z - 1) / ((long)n_grp * Z);
         if (gy > tiles) gy = tiles;
         gy = (gy + mach.xcds - 1) / mach.xcds * mach.xcds;   // the kernel deals streams of token tiles to the XCDs
         dim3 grid(n_grp, (unsigned)gy, Z);
-        if (dtype == BF16) {
-            if (trans_b) hipLaunchKernelGGL((bs_dds32_kernel<bf16_t, false>), grid, dim3(256), 0, st, ga);
-            else hipLaunchKernelGGL((bs_dds32_kernel<bf16_t, true>), grid, dim3(256), 0, st, ga);
-        } else {
-            if (trans_b) hipLaunchKernelGGL((bs_dds32_kernel<f16_t, false>), grid, dim3(256), 0, st, ga);
-            else hipLaunchKernelGGL((bs_dds32_kernel<f16_t, true>), grid, dim3(256), 0, st, ga);
-        }
+        constexpr size_t smem_t = 4 * 128 * 64 * 2;          // two stages of the activation and the weight tile
+#define DDS_TILED(TT, WTT)                                                                                         \
+    {                                                                                                              \
+        auto kern = bs_dds32_kernel<TT, WTT>;                                                                      \
+        static std::atomic<unsigned long long> lds_set{0};                                                         \
+        if (int rc2 = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem_t, lds_set, "bs_dds (tiled)")) return rc2; \
+        hipLaunchKernelGGL(kern, grid, dim3(256), smem_t, st, ga);                                                 \
+    }
+        if (dtype == BF16) { if (trans_b) DDS_TILED(bf16_t, false) else DDS_TILED(bf16_t, true) }
+        else { if (trans_b) DDS_TILED(f16_t, false) else DDS_TILED(f16_t, true) }
+#undef DDS_TILED
         return check_launch("bs_dds32_kernel");
     }
     DxdArgs args{b_sp, a, c, seg_ptr, seg_blk, seg_inner, n_seg, cols_per_head, M, trans_b,
