@@ -307,13 +307,16 @@ def bench_blocksparse(steps, warmup):
 
 
 def sblocal_train_step(q, k, v, P, lc, temp):
-    """A closure running one forward + backward of Scatterbrain-local attention with respect to q, k, v."""
+    """A closure running one forward + backward of Scatterbrain-local attention with respect to q, k, v (with the
+    per-shape scratch cache that the module SBLocalAttention keeps between its calls)."""
     import fly_amd
+    from fly_amd.sblocal_attention import ScratchCache
     qg, kg, vg = (x.clone().requires_grad_() for x in (q, k, v))
     go = torch.randn_like(v)
+    cache = ScratchCache()
 
     def run():
-        o = fly_amd.sblocal_attention_fn(qg, kg, vg, P, lc, temp, None)
+        o = fly_amd.sblocal_attention_fn(qg, kg, vg, P, lc, temp, None, cache=cache)
         o = o[0] if isinstance(o, tuple) else o
         o.backward(go)
         qg.grad = kg.grad = vg.grad = None
