@@ -140,7 +140,7 @@ __global__ __launch_bounds__(PREP_NT) void sb_prep_kmax_kernel(PrepArgs a) {
 
 // (at least two workgroups per compute unit: the kernel streams, and at 128 features the registers it would like to take
 //  leave room for one only; the few it spills instead cost less)
-template <int DIM, int MK>
+template <int DIM, int MK, bool WRITE_F>     // WRITE_F: the float32 feature arrays are wanted (not only the images)
 __global__ __launch_bounds__(PREP_NT) __attribute__((amdgpu_waves_per_eu(2, 8))) void sb_prep_kernel(PrepArgs a) {
     constexpr int MH = MK / 2, FB = MK / 32, RBN = MK / 16, RB = (RBN + 3) / 4, DB = DIM / 16;
     constexpr int LDF = MK + 4, LDY = DIM + 4;
@@ -156,7 +156,7 @@ __global__ __launch_bounds__(PREP_NT) __attribute__((amdgpu_waves_per_eu(2, 8)))
     const int rows = key_role ? a.S : a.T;
     const int len = key_role ? (a.lens ? min((int)a.lens[b], a.S) : a.S) : a.T;
     const float* X = (key_role ? a.k : a.q) + (long)bh * rows * DIM;
-    float* F = key_role ? a.phik : a.psi;        // may be null: only the images are wanted
+    float* F = WRITE_F ? (key_role ? a.phik : a.psi) : nullptr;
     if (F) F += (long)bh * rows * MK;
 
     // kappa: the maximum over the key blocks of pass 1 (0 when no key is valid)
@@ -271,7 +271,7 @@ __global__ __launch_bounds__(PREP_NT) __attribute__((amdgpu_waves_per_eu(2, 8)))
         else bias = kappa - ln_row - 0.5f * a.temp * sq - off;
         __syncthreads();                          // every c of this chunk has been read
         float* frow_s = Fs + (16 * w + r16) * LDF;
-        floatx4 fblk[2 * FB];                     // the row's features: blocks of 16, [exp(+.) | exp(-.)]
+        floatx4 fblk[WRITE_F ? 2 * FB : 1];       // the row's features: blocks of 16, [exp(+.) | exp(-.)]
 #pragma unroll
         for (int fb = 0; fb < FB; ++fb) {
             floatx4 fp, fn;
@@ -286,10 +286,9 @@ __global__ __launch_bounds__(PREP_NT) __attribute__((amdgpu_waves_per_eu(2, 8)))
             sn_[fb] += fn * wrow;
             *reinterpret_cast<floatx4*>(frow_s + 16 * fb + 4 * g) = fp;
             *reinterpret_cast<floatx4*>(frow_s + MH + 16 * fb + 4 * g) = fn;
-            fblk[fb] = fp;
-            fblk[FB + fb] = fn;
+            if (WRITE_F) { fblk[fb] = fp; fblk[FB + fb] = fn; }
         }
-        if (F && row < rows) {
+        if (WRITE_F && F && row < rows) {
             float* frow_g = F + (long)row * MK;
 #pragma unroll
             for (int fb = 0; fb < 2 * FB; ++fb) *reinterpret_cast<floatx4*>(frow_g + 16 * fb + 4 * g) = fblk[fb];
@@ -966,7 +965,10 @@ static void prep_splits(int BH, int T, int S, int& n_kblk, int& n_split_k, int& 
 template <int DIM, int MK>
 static int launch_prep(PrepArgs a, hipStream_t st) {
     hipLaunchKernelGGL((sb_prep_kmax_kernel<DIM, MK>), dim3(a.n_kblk, a.BH), dim3(PREP_NT), 0, st, a);
-    hipLaunchKernelGGL((sb_prep_kernel<DIM, MK>), dim3(a.n_split_k + a.n_split_q, a.BH), dim3(PREP_NT), 0, st, a);
+    if (a.psi || a.phik)
+        hipLaunchKernelGGL((sb_prep_kernel<DIM, MK, true>), dim3(a.n_split_k + a.n_split_q, a.BH), dim3(PREP_NT), 0, st, a);
+    else
+        hipLaunchKernelGGL((sb_prep_kernel<DIM, MK, false>), dim3(a.n_split_k + a.n_split_q, a.BH), dim3(PREP_NT), 0, st, a);
     hipLaunchKernelGGL((sb_prep_reduce_kernel<DIM, MK>), dim3((MK * (DIM + 1) + PREP_NT - 1) / PREP_NT, 2, a.BH),
                        dim3(PREP_NT), 0, st, a);
     return check_launch("sblocal_bwd_prep");
