@@ -568,6 +568,31 @@ def test_fast_dds_many_token_tiles_per_workgroup(trans_b):
     assert rel_err(out, ref) <= TOL[torch.bfloat16]
 
 
+@pytest.mark.parametrize('trans_b', [True, False])
+def test_tiled_dds_with_long_odd_reduction_lists(trans_b):
+    """The tiled dds kernel takes two entries of a reduction list per step: lists of 10 to 12 input blocks (too long for
+    the weight-stationary kernel; odd lengths end on a step with one entry), neighbouring and scattered input blocks,
+    groups of one to four output blocks, a few thousand tokens (several tiles per workgroup) ending inside a tile."""
+    from fly_amd import matmul
+    print('case', trans_b, flush=True)
+    Z, H, block, n_out, n_in, M = 2, 2, 32, 7, 13, 128 * 21 + 5
+    g = torch.Generator().manual_seed(41)
+    seg = (torch.rand(H, n_out, n_in, generator=g) < 0.85).long()   # (head, output block, input block)
+    seg[0, 0] = 1
+    seg[0, 0, 4] = 0                                       # 12 entries
+    seg[0, 1:3] = seg[0, 0]                                # a group of three
+    seg[1, 3, ::2] = 1
+    seg[1, 3, 1::2] = (torch.arange(6) < 4).long()         # 11 entries, half of them without a neighbour
+    assert int(seg.sum(-1).max()) > 9 and int(seg.sum(-1).min()) > 9 and bool((seg.sum(-1) % 2 == 1).any())
+    layout = seg if trans_b else seg.transpose(1, 2).contiguous()
+    w = torch.randn(Z, int(layout.sum()), block, block, generator=g).bfloat16()
+    x = torch.randn(Z, H, M, n_in * block, generator=g).bfloat16()
+    out = matmul(layout, block, 'dds', trans_a=False, trans_b=trans_b)(x.to(DEV), w.to(DEV))
+    ref = ob.dds(x.float(), w.float(), layout, block, False, trans_b)
+    assert out.shape == ref.shape == (Z, H, M, n_out * block)
+    assert rel_err(out, ref) <= TOL[torch.bfloat16]
+
+
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize('trans_b', [True, False])
 def test_dds_weight_stationary_kernel(trans_b, dtype):
