@@ -608,6 +608,31 @@ def test_local_attention_with_attn_mask(dtype, tol, E, p_keep):
         a, _ = mod(qg, kg, vg, attn_mask=FullMask(torch.ones(T, S, dtype=torch.bool, device=dev)), key_padding_mask=kmask)
         b, _ = mod(qg, kg, vg, key_padding_mask=kmask)
     assert torch.equal(a, b)
+    # mask and training-mode dropout together: the dense form of the same weights (equal weights on the hidden rows)
+    # times the kernels' own keep / (1 - p) multipliers, output and gradients
+    drop = LocalAttention(lc, attention_dropout=0.2).to(dev).train()
+    for x in (qg, kg, vg):
+        x.grad = None
+    torch.manual_seed(3)
+    out_d, _ = drop(qg, kg, vg, attn_mask=amask, key_padding_mask=kmask)
+    (out_d.float() * w.to(dev)).sum().backward()
+    qd, kd, vd = (x.double().requires_grad_() for x in (q, k, v))
+    i, j = torch.arange(T).view(T, 1), torch.arange(S).view(1, S)
+    vis = ((j - i >= -(lc // 2)) & (j - i < (lc + 1) // 2)).view(1, 1, T, S) & (j.view(1, 1, 1, S) < lengths.view(B, 1, 1, 1))
+    ok = vis & keep.view(1, 1, T, S)
+    sc = torch.einsum('bthe,bshe->bhts', qd, kd) / math.sqrt(E)
+    live = ok.any(-1, keepdim=True)
+    prob = torch.softmax(torch.where(live, sc.masked_fill(~ok, float('-inf')), torch.zeros_like(sc)), -1) * live
+    # hidden rows: equal scores in all local_context slots of the packed band; the scores of the visible slots still
+    # depend on q and k (their value is absorbed by the -1e24, their derivative is not), the other slots are constants
+    hidden_row = vis.any(-1, keepdim=True) & ~live
+    z = torch.exp(sc - sc.detach()) * vis
+    prob = torch.where(hidden_row, z / (z.sum(-1, keepdim=True) + (lc - vis.sum(-1, keepdim=True))), prob)
+    ref_d = torch.einsum('bhts,bshd->bthd', prob * osb.dropout_keep(drop.last_dropout_seed, 0.2, B, H, T, S), vd)
+    (ref_d * w.double()).sum().backward()
+    assert rel_err(out_d.float(), ref_d.detach()) <= (1e-4 if dtype == torch.float32 else 2e-2)
+    for got, want, name in ((qg.grad, qd.grad, 'dq'), (kg.grad, kd.grad, 'dk'), (vg.grad, vd.grad, 'dv')):
+        assert rel_err(got.float(), want) <= tol, (name, rel_err(got.float(), want))
 
 
 def test_sblocal_attn_mask_follows_the_references_assertion():
