@@ -278,8 +278,9 @@ __global__ __launch_bounds__(PREP_NT) __attribute__((amdgpu_waves_per_eu(2, 8)))
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const bool ok = valid && (16 * fb + 4 * g + i < a.mh_valid);
-                fp[i] = ok ? expf(dd[fb][i] + bias) : 0.f;
-                fn[i] = ok ? expf(bias - dd[fb][i]) : 0.f;
+                // (the hardware exponential: its last-bit differences vanish in the rounding to 17 bits below)
+                fp[i] = ok ? __expf(dd[fb][i] + bias) : 0.f;
+                fn[i] = ok ? __expf(bias - dd[fb][i]) : 0.f;
             }
             if (img) { fp = quant16(fp); fn = quant16(fn); }     // every use sees the features rounded to 17 bits
             sp_[fb] += fp * wrow;
