@@ -319,7 +319,7 @@ __device__ __forceinline__ void split3_4(floatx4 x, uint2& h, uint2& m, uint2& l
 // so the backward forms the same mask again from the seed.  row_hash depends on the row alone (one query: once per
 // lane).  A pair of neighbouring columns (2c, 2c + 1) shares one 32-bit hash -- the pair index enters through a
 // multiply-add and the 32-bit finaliser of MurmurHash3 (full avalanche) -- and each column takes one 16-bit half of it:
-// the hash's two multiplies are quarter-rate instructions, and a lane's columns come in consecutive runs.  A pair is
+// the hash is ten vector instructions, and a lane's columns come in consecutive runs.  A pair is
 // kept when its half is at least thresh = floor(p 2^16); kept weights are scaled by 1 / (1 - thresh 2^-16).
 __device__ __forceinline__ uint32_t drop_mix(uint32_t h) {
     h ^= h >> 16; h *= 0x85EBCA6Bu; h ^= h >> 13; h *= 0xC2B2AE35u; h ^= h >> 16;
