@@ -987,8 +987,8 @@ struct DdsGroupArgs {
 };
 constexpr int DDS_MAX_STEPS = 128;   // longest reduction list the tiled kernel accepts
 #ifndef FLY_DDS_STATIONARY
-#define FLY_DDS_STATIONARY 1         // weight-stationary kernel where the group's weights fit the LDS
-#endif
+#define FLY_DDS_STATIONARY 2         // weight-stationary kernels where the group's weights fit the LDS: 1 = activation
+#endif                               // fragments straight from memory, 2 = staged through LDS when there are enough tokens
 #ifndef FLY_DDS_DEPTH
 #define FLY_DDS_DEPTH 2              // steps (of two input blocks) its activation loads run ahead
 #endif
@@ -1323,6 +1323,155 @@ __global__ __launch_bounds__(256) void bs_dds32s_kernel(DdsGroupArgs a, int n_st
             if (step + u < n_steps) compute(fx[u]);
             fetch(fx[u]);                                   // step + u + DEPTH
         }
+    }
+}
+
+// The weight-stationary DDS with the activations staged through LDS by direct-to-LDS transfers.  A compute unit's
+// vector memory path takes about one 128-byte line every four cycles whether half of the line is asked for or all of
+// it, and bs_dds32s_kernel's fragment loads (64-byte pieces of 16 token rows per instruction) are what bounds it.  Here
+// a wave fetches a step's two input blocks of its 64 tokens as whole 128-byte pieces of token rows (eight rows per
+// instruction, the two blocks side by side when they are neighbours) into a stage of its own, 8 KB, and reads the MFMA
+// fragments from there.  One workgroup of eight waves per compute unit shares the group's weights (72 KB) and leaves
+// room for the eight stages; a wave touches no other wave's stage, so the loop has no barrier: it waits for its
+// transfer, reads the step's fragments into registers, starts the next step's transfer into the same stage and then
+// multiplies.  16-byte chunk c of token t sits at chunk c ^ ((t >> 1) & 7) of the token's 128 bytes: the transfer
+// writes lane by lane, so the lane asks for the chunk that belongs in its slot, and the 16 lanes of a fragment read
+// cover all 64 banks.
+template <typename T, bool WT>
+__global__ __launch_bounds__(512) void bs_dds32d_kernel(DdsGroupArgs a, int n_streams) {
+    constexpr int STEP = 8 * 16 * 32;                       // elements of a step's eight weight tiles
+    constexpr int WBYTES = DDS_STAT_STEPS * 8192;           // the weights' share of the LDS
+    extern __shared__ __attribute__((aligned(1024))) uint16_t wres[];   // [step][tile n][row r][32 k], then 8 stages of 8 KB
+    __shared__ int s_inner[DDS_STAT_STEPS];
+    const int tid = threadIdx.x, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int z = blockIdx.y;
+    const int per_xcd = (int)gridDim.x / a.n_xcd;
+    const int pair = ((int)blockIdx.x % a.n_xcd) * per_xcd + (int)blockIdx.x / a.n_xcd;
+    const int n_grp = a.n_grp;
+    if (pair >= n_streams * n_grp) return;                  // workgroup-uniform
+    const int ty = pair / n_grp, grp = pair % n_grp, gy = n_streams;
+    const int tiles_all = (a.M + 511) / 512;
+    if (ty >= tiles_all) return;
+    const int my_tiles = (tiles_all - ty + gy - 1) / gy;
+    const int row0 = a.grp_row0[grp], gn = a.grp_n[grp];
+    const int head = row0 / a.per_head, bcol0 = row0 % a.per_head;
+    const int p0 = a.seg_ptr[row0], nin = a.seg_ptr[row0 + 1] - p0;
+    const uint16_t* spz = reinterpret_cast<const uint16_t*>(a.sp) + z * a.sp_sz;
+    const uint16_t* xp = reinterpret_cast<const uint16_t*>(a.dn) + z * a.dn_sz + head * a.dn_sh;
+    T* cp = reinterpret_cast<T*>(a.c) + z * a.c_sz + head * a.c_sh;
+
+    for (int i = tid; i < nin; i += 512) s_inner[i] = a.seg_inner[p0 + i];
+    for (int idx = tid; idx < nin * 512; idx += 512) {      // the group's weights, once (see bs_dds32s_kernel)
+        const int chunk = idx & 3, row = (idx >> 2) & 31, ob = (idx >> 7) & 3, t = idx >> 9;
+        const int blk_id = ob < gn ? a.seg_blk[a.seg_ptr[row0 + ob] + t] : -1;
+        uintx4 v = {0, 0, 0, 0};
+        if (blk_id >= 0) v = *reinterpret_cast<const uintx4*>(spz + (long)blk_id * 1024 + row * 32 + chunk * 8);
+        uint16_t* dst = wres + (size_t)t * STEP;
+        if (!WT) {
+            *reinterpret_cast<uintx4*>(dst + (row & 7) * 512 + (4 * ob + (row >> 3)) * 32 + 8 * chunk) = v;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                dst[e * 512 + (4 * ob + chunk) * 32 + row] = (uint16_t)(v[e >> 1] >> (16 * (e & 1)));
+        }
+    }
+    __syncthreads();
+
+    floatx4 acc[4][8];
+#pragma unroll
+    for (int tm = 0; tm < 4; ++tm)
+#pragma unroll
+        for (int n = 0; n < 8; ++n) acc[tm][n] = Frag<float>::zero();
+    const bool col_live = 8 * r16 < 32 * gn;
+    auto store_tile = [&](int tile) __attribute__((always_inline)) {
+        const long m0 = ((long)ty + (long)tile * gy) * 512 + 64 * w + 4 * g;
+        T* base = cp + (long)bcol0 * 32 + 8 * r16;
+#pragma unroll
+        for (int tm = 0; tm < 4; ++tm) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const long m = m0 + 16 * tm + i;
+                if (m < a.M && col_live) {
+                    const floatx4 lo = {acc[tm][0][i], acc[tm][1][i], acc[tm][2][i], acc[tm][3][i]};
+                    const floatx4 hi = {acc[tm][4][i], acc[tm][5][i], acc[tm][6][i], acc[tm][7][i]};
+                    store8_f32(base + m * a.c_sm, lo, hi);
+                }
+            }
+#pragma unroll
+            for (int n = 0; n < 8; ++n) acc[tm][n] = Frag<float>::zero();
+        }
+    };
+    if (nin == 0) {                                         // no input block: zero rows
+        for (int tile = 0; tile < my_tiles; ++tile) store_tile(tile);
+        return;
+    }
+
+    const int npair = (nin + 1) / 2;
+    const int n_steps = my_tiles * npair;
+    char* stage = reinterpret_cast<char*>(wres) + WBYTES + 8192 * w;
+    // transfer j of a step brings tokens 8 j .. 8 j + 7 of the wave: this lane's slot is chunk slot lane % 8 of token
+    // 8 j + lane / 8, i.e. chunk (lane % 8) ^ ((token >> 1) & 7) of that token's two blocks
+    const int tl = lane >> 3;
+    uint32_t xoff[8];
+    int sel[8];                                             // which of the step's two blocks the lane's chunk belongs to
+#pragma unroll
+    for (int j = 0; j < 8; ++j) { xoff[j] = 0; sel[j] = 0; }
+    int f_tile = 0, f_t = 0;                                // transfer cursor: (token tile, pair of entries inside it)
+    auto transfer = [&]() __attribute__((always_inline)) {
+        if (f_t == 0) {
+            const long m0 = ((long)ty + (long)f_tile * gy) * 512 + 64 * w;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int t = 8 * j + tl, c = (lane & 7) ^ ((t >> 1) & 7);
+                const long m = min(m0 + t, (long)a.M - 1);                       // clamped: masked at the store
+                xoff[j] = (uint32_t)((m * a.dn_sm + 8 * (c & 3)) * 2);
+                sel[j] = c >> 2;
+            }
+        }
+        const int in0 = __builtin_amdgcn_readfirstlane(s_inner[2 * f_t]);
+        const int in1 = __builtin_amdgcn_readfirstlane(s_inner[min(2 * f_t + 1, nin - 1)]);   // (an odd list's last step: twice the same)
+        const char* xb = reinterpret_cast<const char*>(xp);
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            dma_to_lds(xb + xoff[j] + (uint32_t)((sel[j] ? in1 : in0) * 64), stage + 1024 * j);
+        if (++f_t == npair) { f_t = 0; ++f_tile; }
+    };
+    int c_tile = 0, c_t = 0;                                // compute cursor
+    const int wfrag = r16 * 32 + 8 * g;                     // this lane's 16 bytes of a weight tile
+    // fragment of (token 16 tm + r16, block hf): chunk 4 hf + g, stored at chunk ^ ((token >> 1) & 7)
+    int xfrag[2][4];
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+        for (int tm = 0; tm < 4; ++tm) {
+            const int t = 16 * tm + r16;
+            xfrag[hf][tm] = t * 128 + 16 * ((4 * hf + g) ^ ((t >> 1) & 7));
+        }
+    transfer();
+    for (int step = 0; step < n_steps; ++step) {
+        drain_loads();                                      // this step's activations are in the stage
+        uintx4 fx[2][4];
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+            for (int tm = 0; tm < 4; ++tm) fx[hf][tm] = *reinterpret_cast<const uintx4*>(stage + xfrag[hf][tm]);
+        __builtin_amdgcn_s_waitcnt(0xC07F);                 // lgkmcnt(0): the fragments are in registers, the stage is free
+        if (step + 1 < n_steps) transfer();                 // (workgroup-uniform) flies under the products below
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+            if (2 * c_t + hf < nin) {                       // workgroup-uniform
+                const uint16_t* wt = wres + (size_t)(2 * c_t + hf) * STEP + wfrag;
+#pragma unroll
+                for (int n = 0; n < 8; ++n) {
+                    const uint4 fw = *reinterpret_cast<const uint4*>(wt + n * 512);
+#pragma unroll
+                    for (int tm = 0; tm < 4; ++tm)
+                        acc[tm][n] = Frag32<T>::mma(__builtin_bit_cast(uint4, fx[hf][tm]), fw, acc[tm][n]);
+                }
+            }
+        }
+        if (++c_t == npair) { store_tile(c_tile); c_t = 0; ++c_tile; }
     }
 }
 
@@ -2293,6 +2442,31 @@ extern "C" int flyhip_bs_dds(const void* a, const void* b_sp, void* c,
         ga.n_grp = n_grp;
         // groups whose weights fit the LDS (four output blocks times the longest reduction list) and enough tokens to
         // amortise bringing them in: the weight-stationary kernel, two workgroups per compute unit
+        if (FLY_DDS_STATIONARY == 2 && max_seg_len > 0 && max_seg_len <= DDS_STAT_STEPS && (long)M >= 512L * 8) {
+            // one workgroup of eight waves per compute unit: the group's weights and a stage of activations per wave
+            // streams of token tiles per group: the count that minimises (rounds of workgroups) x (tiles per workgroup)
+            const long tiles = (M + 511) / 512;
+            long n_streams = 1, best = -1;
+            for (long n = 1; n <= tiles && n * n_grp * Z <= 4L * mach.cus + (long)n_grp * Z; ++n) {
+                const long cost = ((n * n_grp * Z + mach.cus - 1) / mach.cus) * ((tiles + n - 1) / n);
+                if (best < 0 || cost < best) { best = cost; n_streams = n; }
+            }
+            const long pairs = n_streams * n_grp;
+            const long gx = (pairs + mach.xcds - 1) / mach.xcds * mach.xcds;
+            const size_t smem = (size_t)DDS_STAT_STEPS * 8192 + 8 * 8192;
+            dim3 grid((unsigned)gx, Z);
+#define DDS_DMA(TT, WTT)                                                                                           \
+    {                                                                                                              \
+        auto kern = bs_dds32d_kernel<TT, WTT>;                                                                     \
+        static std::atomic<unsigned long long> lds_set{0};                                                         \
+        if (int rc2 = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_set, "bs_dds (staged)")) return rc2; \
+        hipLaunchKernelGGL(kern, grid, dim3(512), smem, st, ga, (int)n_streams);                                   \
+    }
+            if (dtype == BF16) { if (trans_b) DDS_DMA(bf16_t, false) else DDS_DMA(bf16_t, true) }
+            else { if (trans_b) DDS_DMA(f16_t, false) else DDS_DMA(f16_t, true) }
+#undef DDS_DMA
+            return check_launch("bs_dds32d_kernel");
+        }
         if (FLY_DDS_STATIONARY && max_seg_len > 0 && max_seg_len <= DDS_STAT_STEPS && (long)M >= 256L * 8) {
             const long tiles = (M + 255) / 256;
             long n_streams = 2L * mach.cus / ((long)n_grp * Z);

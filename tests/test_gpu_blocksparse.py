@@ -595,14 +595,17 @@ def test_tiled_dds_with_long_odd_reduction_lists(trans_b):
 
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize('trans_b', [True, False])
-def test_dds_weight_stationary_kernel(trans_b, dtype):
-    """Reduction lists of at most nine blocks and a few thousand tokens: the dds kernel that keeps a group's weights in
-    LDS and reads its activations straight from memory.  Two batch entries, two heads, groups of one to four segments
-    (the last lanes of a short group store nothing), a segment without blocks, a token count that ends inside a
-    256-token tile, both block orientations."""
+@pytest.mark.parametrize('M', [2048 + 77, 4096 + 1024 + 77])
+def test_dds_weight_stationary_kernel(M, trans_b, dtype):
+    """Reduction lists of at most nine blocks and a few thousand tokens: the dds kernels that keep a group's weights in
+    LDS -- with activation fragments straight from memory (from 2048 tokens) and with the activations staged through
+    LDS by direct-to-LDS transfers of whole 128-byte pieces of token rows (from 4096 tokens).  Two batch entries, two
+    heads, groups of one to four segments (the last lanes of a short group store nothing), lists of odd and even
+    length with neighbouring and scattered input blocks, a segment without blocks, a token count that ends inside a
+    tile, both block orientations."""
     from fly_amd import matmul
-    print('case', trans_b, dtype, flush=True)
-    Z, H, block, M = 2, 2, 32, 2048 + 77
+    print('case', M, trans_b, dtype, flush=True)
+    Z, H, block = 2, 2, 32
     p, r = (11, 9) if trans_b else (9, 11)                # segments: the output blocks, 11 of them either way
     g = torch.Generator().manual_seed(31)
     seg = (torch.rand(H, 11, 9, generator=g) < 0.45).long()   # (head, output block, input block): lists of <= 9
