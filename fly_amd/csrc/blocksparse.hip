@@ -1475,6 +1475,207 @@ __global__ __launch_bounds__(512) void bs_dds32d_kernel(DdsGroupArgs a, int n_st
     }
 }
 
+// The same per-wave scheme for reduction lists that do not fit the LDS (layers that narrow: 36 input blocks per output
+// block in the second linear of a channel MLP).  The group's weights pass through LDS in chunks of DDS_CK list entries
+// (32 KB), double-buffered and shared by the eight waves: a thread asks for its 64 bytes of the next chunk at the head
+// of a chunk, parks them in the other buffer at its end, and one barrier per chunk (two steps of 64 MFMAs per wave)
+// publishes them -- the tiled kernel pays a barrier, eight LDS writes and the wait for its loads per 32 MFMAs.  The
+// activations go through a stage per wave exactly as in bs_dds32d_kernel.  The weights are fetched again for every tile
+// of 512 tokens (from L2: a quarter of what the tiled kernel's 128-token tiles fetch).
+constexpr int DDS_CK = 4;
+typedef unsigned int uintx2 __attribute__((ext_vector_type(2)));
+
+template <typename T, bool WT>
+__global__ __launch_bounds__(512) void bs_dds32c_kernel(DdsGroupArgs a, int n_streams) {
+    constexpr int STEP = 8 * 16 * 32;                       // elements of an entry's eight weight tiles
+    constexpr int CHUNK = DDS_CK * STEP;                    // elements of a chunk buffer
+    extern __shared__ __attribute__((aligned(1024))) uint16_t wres[];   // 2 x [entry][tile n][row r][32 k], then 8 stages of 8 KB
+    __shared__ int s_inner[DDS_MAX_STEPS];
+    __shared__ int s_blk[4][DDS_MAX_STEPS];
+    const int tid = threadIdx.x, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int z = blockIdx.y;
+    const int per_xcd = (int)gridDim.x / a.n_xcd;
+    const int pair = ((int)blockIdx.x % a.n_xcd) * per_xcd + (int)blockIdx.x / a.n_xcd;
+    const int n_grp = a.n_grp;
+    if (pair >= n_streams * n_grp) return;                  // workgroup-uniform
+    const int ty = pair / n_grp, grp = pair % n_grp, gy = n_streams;
+    const int tiles_all = (a.M + 511) / 512;
+    if (ty >= tiles_all) return;
+    const int my_tiles = (tiles_all - ty + gy - 1) / gy;
+    const int row0 = a.grp_row0[grp], gn = a.grp_n[grp];
+    const int head = row0 / a.per_head, bcol0 = row0 % a.per_head;
+    const int p0 = a.seg_ptr[row0], nin = a.seg_ptr[row0 + 1] - p0;
+    const uint16_t* spz = reinterpret_cast<const uint16_t*>(a.sp) + z * a.sp_sz;
+    const uint16_t* xp = reinterpret_cast<const uint16_t*>(a.dn) + z * a.dn_sz + head * a.dn_sh;
+    T* cp = reinterpret_cast<T*>(a.c) + z * a.c_sz + head * a.c_sh;
+
+    for (int i = tid; i < nin; i += 512) s_inner[i] = a.seg_inner[p0 + i];
+    for (int i = tid; i < 4 * nin; i += 512) {
+        const int ob = i / nin, t = i % nin;
+        s_blk[ob][t] = ob < gn ? a.seg_blk[a.seg_ptr[row0 + ob] + t] : -1;
+    }
+    __syncthreads();
+
+    floatx4 acc[4][8];
+#pragma unroll
+    for (int tm = 0; tm < 4; ++tm)
+#pragma unroll
+        for (int n = 0; n < 8; ++n) acc[tm][n] = Frag<float>::zero();
+    // The group's 32 gn outputs are dealt to NT = 2 gn tiles of 16: tile n holds outputs NT r + n (r = 0..15), so no MFMA
+    // column is padding whatever the group's size, and a lane ends up with NT consecutive outputs of four tokens.
+    const int NT = 2 * gn;
+    auto store_tile = [&](int tile) __attribute__((always_inline)) {
+        const long m0 = ((long)ty + (long)tile * gy) * 512 + 64 * w + 4 * g;
+        T* base = cp + (long)bcol0 * 32 + NT * r16;
+#pragma unroll
+        for (int tm = 0; tm < 4; ++tm) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const long m = m0 + 16 * tm + i;
+                if (m < a.M) {
+                    uint32_t* dst = reinterpret_cast<uint32_t*>(base + m * a.c_sm);
+                    const uint32_t p0_ = pack2<T>(acc[tm][0][i], acc[tm][1][i]), p1_ = pack2<T>(acc[tm][2][i], acc[tm][3][i]);
+                    const uint32_t p2_ = pack2<T>(acc[tm][4][i], acc[tm][5][i]), p3_ = pack2<T>(acc[tm][6][i], acc[tm][7][i]);
+                    if (NT == 8) __builtin_nontemporal_store(uintx4{p0_, p1_, p2_, p3_}, reinterpret_cast<uintx4*>(dst));
+                    else if (NT == 6) { __builtin_nontemporal_store(uintx2{p0_, p1_}, reinterpret_cast<uintx2*>(dst)); __builtin_nontemporal_store(p2_, dst + 2); }
+                    else if (NT == 4) __builtin_nontemporal_store(uintx2{p0_, p1_}, reinterpret_cast<uintx2*>(dst));
+                    else __builtin_nontemporal_store(p0_, dst);
+                }
+            }
+#pragma unroll
+            for (int n = 0; n < 8; ++n) acc[tm][n] = Frag<float>::zero();
+        }
+    };
+    if (nin == 0) {                                         // no input block: zero rows
+        for (int tile = 0; tile < my_tiles; ++tile) store_tile(tile);
+        return;
+    }
+
+    const int npair = (nin + 1) / 2, nchunk = (npair + DDS_CK / 2 - 1) / (DDS_CK / 2);      // steps and chunks per tile
+    const int n_steps = my_tiles * npair, n_chunks = my_tiles * nchunk;
+    // the weights of a chunk: this thread's 16 bytes of each of its DDS_CK entries -- row `wrow` (its 8 inputs `wch`..) of
+    // output block `wob`, parked at the place the MFMAs read (see bs_dds32s_kernel)
+    const int wch = tid & 3, wrow = (tid >> 2) & 31, wob = (tid >> 7) & 3;
+    const uint32_t wsrc = (uint32_t)((wrow * 32 + wch * 8) * 2);
+    // where they go: output o of the group sits in tile o % NT, row o / NT
+    int wdst[WT ? 8 : 1];
+    if (!WT) {
+        const int o = 32 * wob + wrow;
+        wdst[0] = (o % NT) * 512 + (o / NT) * 32 + 8 * wch;
+    } else {
+#pragma unroll
+        for (int e = 0; e < (WT ? 8 : 1); ++e) {
+            const int o = 32 * wob + 8 * wch + e;
+            wdst[e] = (o % NT) * 512 + (o / NT) * 32 + wrow;
+        }
+    }
+    uintx4 rwq[DDS_CK];
+    bool wlive[DDS_CK];
+    auto fetch_w = [&](int q) __attribute__((always_inline)) {
+        const int e0 = DDS_CK * (q % nchunk);
+#pragma unroll
+        for (int j = 0; j < DDS_CK; ++j) {
+            const int blk_id = e0 + j < nin ? s_blk[wob][e0 + j] : -1;
+            wlive[j] = blk_id >= 0;
+            rwq[j] = *reinterpret_cast<const uintx4*>(reinterpret_cast<const char*>(spz + (long)max(blk_id, 0) * 1024) + wsrc);
+        }
+    };
+    auto stash_w = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < DDS_CK; ++j) {
+            const uintx4 v = wlive[j] ? rwq[j] : uintx4{0, 0, 0, 0};
+            uint16_t* dst = wres + (size_t)buf * CHUNK + (size_t)j * STEP;
+            if (wob < gn) {                                 // (an output block the group lacks has no place in the tiles)
+                if (!WT) {
+                    *reinterpret_cast<uintx4*>(dst + wdst[0]) = v;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < (WT ? 8 : 1); ++e) dst[wdst[e]] = (uint16_t)(v[e >> 1] >> (16 * (e & 1)));
+                }
+            }
+        }
+    };
+
+    char* stage = reinterpret_cast<char*>(wres) + 2 * CHUNK * 2 + 8192 * w;
+    const int tl = lane >> 3;
+    uint32_t xoff[8];
+    int sel[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) { xoff[j] = 0; sel[j] = 0; }
+    int f_tile = 0, f_t = 0;                                // transfer cursor: (token tile, pair of entries inside it)
+    auto transfer = [&]() __attribute__((always_inline)) {  // (see bs_dds32d_kernel)
+        if (f_t == 0) {
+            const long m0 = ((long)ty + (long)f_tile * gy) * 512 + 64 * w;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int t = 8 * j + tl, c = (lane & 7) ^ ((t >> 1) & 7);
+                const long m = min(m0 + t, (long)a.M - 1);
+                xoff[j] = (uint32_t)((m * a.dn_sm + 8 * (c & 3)) * 2);
+                sel[j] = c >> 2;
+            }
+        }
+        const int in0 = __builtin_amdgcn_readfirstlane(s_inner[2 * f_t]);
+        const int in1 = __builtin_amdgcn_readfirstlane(s_inner[min(2 * f_t + 1, nin - 1)]);
+        const char* xb = reinterpret_cast<const char*>(xp);
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            dma_to_lds(xb + xoff[j] + (uint32_t)((sel[j] ? in1 : in0) * 64), stage + 1024 * j);
+        if (++f_t == npair) { f_t = 0; ++f_tile; }
+    };
+    const int wfrag = r16 * 32 + 8 * g;
+    int xfrag[2][4];
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+        for (int tm = 0; tm < 4; ++tm) {
+            const int t = 16 * tm + r16;
+            xfrag[hf][tm] = t * 128 + 16 * ((4 * hf + g) ^ ((t >> 1) & 7));
+        }
+
+    fetch_w(0);
+    stash_w(0);
+    __syncthreads();
+    transfer();
+    int c_tile = 0, c_t = 0, q = 0;                         // compute cursor: tile, step inside it; chunks done so far
+    for (int step = 0; step < n_steps; ++step) {
+        drain_loads();                                      // this step's activations are in the stage
+        const bool chunk_head = (c_t & (DDS_CK / 2 - 1)) == 0;
+        if (chunk_head && q + 1 < n_chunks) fetch_w(q + 1); // (workgroup-uniform) parked at the chunk's end
+        uintx4 fx[2][4];
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+            for (int tm = 0; tm < 4; ++tm) fx[hf][tm] = *reinterpret_cast<const uintx4*>(stage + xfrag[hf][tm]);
+        __builtin_amdgcn_s_waitcnt(0xC07F);                 // lgkmcnt(0): the fragments are in registers, the stage is free
+        if (step + 1 < n_steps) transfer();
+        const uint16_t* wbuf = wres + (size_t)(q & 1) * CHUNK + (size_t)(2 * (c_t & (DDS_CK / 2 - 1))) * STEP + wfrag;
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+            if (2 * c_t + hf < nin) {                       // workgroup-uniform
+                const uint16_t* wt = wbuf + (size_t)hf * STEP;
+#pragma unroll
+                for (int n = 0; n < 8; ++n) {
+                    if (n < NT) {                           // workgroup-uniform
+                        const uint4 fw = *reinterpret_cast<const uint4*>(wt + n * 512);
+#pragma unroll
+                        for (int tm = 0; tm < 4; ++tm)
+                            acc[tm][n] = Frag32<T>::mma(__builtin_bit_cast(uint4, fx[hf][tm]), fw, acc[tm][n]);
+                    }
+                }
+            }
+        }
+        bool chunk_end = false;
+        if (++c_t == npair) { store_tile(c_tile); c_t = 0; ++c_tile; chunk_end = true; }
+        else chunk_end = (c_t & (DDS_CK / 2 - 1)) == 0;
+        if (chunk_end) {                                    // (workgroup-uniform)
+            if (q + 1 < n_chunks) stash_w((q + 1) & 1);
+            __syncthreads();
+            ++q;
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------------------
 // fused block-sparse attention: out = softmax(scale * Q K^T + key mask) V over the nonzero blocks
 // ---------------------------------------------------------------------------------------
@@ -2466,6 +2667,30 @@ extern "C" int flyhip_bs_dds(const void* a, const void* b_sp, void* c,
             else { if (trans_b) DDS_DMA(f16_t, false) else DDS_DMA(f16_t, true) }
 #undef DDS_DMA
             return check_launch("bs_dds32d_kernel");
+        }
+        if (FLY_DDS_STATIONARY == 2 && max_seg_len > DDS_STAT_STEPS && max_seg_len <= DDS_MAX_STEPS && (long)M >= 512L * 8) {
+            // longer lists: the same workgroup shape with the weights passing through LDS in chunks
+            const long tiles = (M + 511) / 512;
+            long n_streams = 1, best = -1;
+            for (long n = 1; n <= tiles && n * n_grp * Z <= 4L * mach.cus + (long)n_grp * Z; ++n) {
+                const long cost = ((n * n_grp * Z + mach.cus - 1) / mach.cus) * ((tiles + n - 1) / n);
+                if (best < 0 || cost < best) { best = cost; n_streams = n; }
+            }
+            const long pairs = n_streams * n_grp;
+            const long gx = (pairs + mach.xcds - 1) / mach.xcds * mach.xcds;
+            const size_t smem = (size_t)2 * DDS_CK * 8192 + 8 * 8192;
+            dim3 grid((unsigned)gx, Z);
+#define DDS_CHUNKED(TT, WTT)                                                                                       \
+    {                                                                                                              \
+        auto kern = bs_dds32c_kernel<TT, WTT>;                                                                     \
+        static std::atomic<unsigned long long> lds_set{0};                                                         \
+        if (int rc2 = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_set, "bs_dds (chunked)")) return rc2; \
+        hipLaunchKernelGGL(kern, grid, dim3(512), smem, st, ga, (int)n_streams);                                   \
+    }
+            if (dtype == BF16) { if (trans_b) DDS_CHUNKED(bf16_t, false) else DDS_CHUNKED(bf16_t, true) }
+            else { if (trans_b) DDS_CHUNKED(f16_t, false) else DDS_CHUNKED(f16_t, true) }
+#undef DDS_CHUNKED
+            return check_launch("bs_dds32c_kernel");
         }
         if (FLY_DDS_STATIONARY && max_seg_len > 0 && max_seg_len <= DDS_STAT_STEPS && (long)M >= 256L * 8) {
             const long tiles = (M + 255) / 256;

@@ -624,6 +624,37 @@ def test_dds_weight_stationary_kernel(M, trans_b, dtype):
 
 
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('trans_b', [True, False])
+def test_dds_staged_kernel_with_weights_in_chunks(trans_b, dtype):
+    """Reduction lists longer than nine blocks and more than 4096 tokens: the staged dds kernel whose group weights
+    pass through LDS in double-buffered chunks of four list entries.  Lists of 10 to 21 entries (the last chunk of a
+    list holds one to four entries, odd lengths end on a step with one entry), groups of one to four output blocks
+    (the lanes of a short group store fewer outputs), two batch entries, two heads, a token count that ends inside a
+    tile, both block orientations."""
+    from fly_amd import matmul
+    print('case', trans_b, dtype, flush=True)
+    Z, H, block, n_out, n_in, M = 2, 2, 32, 10, 21, 4096 + 1024 + 77
+    g = torch.Generator().manual_seed(43)
+    seg = (torch.rand(H, n_out, n_in, generator=g) < 0.7).long()    # (head, output block, input block)
+    seg[0, 0] = 1                                          # 21 entries: five chunks and one entry more
+    seg[0, 1:4] = seg[0, 0]                                # a full group of four
+    seg[0, 4] = (torch.arange(n_in) % 2 == 0).long()       # 11 entries, none with a neighbour
+    seg[1, 0, :] = 0
+    seg[1, 0, :10] = 1                                     # 10 entries: two chunks and half a chunk
+    seg[1, 1:3] = seg[1, 0]                                # a group of three
+    seg[1, 3] = (torch.arange(n_in) < 17).long()           # 17 entries: the last chunk holds one
+    lens = seg.sum(-1)
+    assert int(lens.max()) == 21 and all(bool((lens % 4 == k).any()) for k in range(4))
+    layout = seg if trans_b else seg.transpose(1, 2).contiguous()
+    w = torch.randn(Z, int(layout.sum()), block, block, generator=g).to(dtype)
+    x = torch.randn(Z, H, M, n_in * block, generator=g).to(dtype)
+    out = matmul(layout, block, 'dds', trans_a=False, trans_b=trans_b)(x.to(DEV), w.to(DEV))
+    ref = ob.dds(x.double(), w.double(), layout, block, False, trans_b)
+    assert out.shape == ref.shape == (Z, H, M, n_out * block)
+    assert rel_err(out, ref) <= TOL[dtype]
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize('p,r,N', [(8, 8, 64), (11, 6, 72), (5, 13, 128)])
 def test_dsd_with_transposed_sparse_operand(p, r, N, dtype):
     """dense = sparse^T . dense (dV = P^T dO, and dK = dS^T Q which arrives as a transposed dds) on the
