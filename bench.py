@@ -482,9 +482,14 @@ def bench_other_configs():
     ln = torch.empty(B, H, L, device=dev)
     ms = timeit(lambda: plan.run(q, k, v, P, None, lc, 0.125, o, ln))
     msk = timeit(lambda: plan.run_keys(q, k, v, P, None, 0.125))
-    fl, _ = sblocal_flops(B, H, L, L, E, E, 2 * mh, lc)
+    fl, band_fl = sblocal_flops(B, H, L, L, E, E, 2 * mh, lc)
     out['config5_sblocal_bf16_L16384'] = {'ms': ms, 'key_pass_ms': msk, 'tflops': fl / ms / 1e9,
                                           'tokens_per_s': B * L / ms * 1e3, 'mfma_bf16_frac': fl / ms / 1e9 / 2500.0}
+    # plain local attention (LocalAttention, local_attention.py:50-92) on the same inputs: the band softmax alone
+    from fly_amd.local_attention import local_forward
+    pairs = band_fl / (2 * (E + 2 * mh + E))                 # band pairs, from the count above
+    ms = timeit(lambda: local_forward(q, k, v, lc, softmax_temp=0.125))
+    out['local_attention_bf16_L16384'] = {'ms': ms, 'tflops': pairs * 2 * (E + E) / ms / 1e9}
     return out
 
 

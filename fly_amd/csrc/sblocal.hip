@@ -2742,6 +2742,228 @@ __global__ __launch_bounds__(NT) void local_fwd_kernel(LocalArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------
+// plain local attention for 2-byte inputs: both products on the 16x16x32 MFMA of the input type
+// ---------------------------------------------------------------------------------------
+// The same work decomposition, masks, online softmax and outputs as local_fwd_kernel; key tiles of 64 keys, K and V
+// row-major in LDS as they are in memory (rows padded by 16 bytes).
+//   scores^T block (hf, b) = K rows {32 hf + 8 (r / 4) + 4 b + r % 4 : r = 0 .. 15} . q : lane (query r16, group g)
+//       receives keys 32 hf + 8 g + 4 b + i, i = 0 .. 3 -- over b = 0, 1 the eight consecutive keys 32 hf + 8 g .. + 7,
+//       which is the contraction slot order of the second product, so the weights go from registers into it;
+//   out^T[d][query] += V^T[d][key] P[key][query], 32 keys per step: V^T fragments by transposing LDS reads
+//       (ds_read_b64_tr_b16: column d of four consecutive key rows per read).
+template <typename T> __device__ __forceinline__ uint32_t pack_pair(float lo, float hi);
+template <> __device__ __forceinline__ uint32_t pack_pair<bf16_t>(float lo, float hi) { return pack_bf16x2(lo, hi); }
+template <> __device__ __forceinline__ uint32_t pack_pair<f16_t>(float lo, float hi) {
+    const _Float16 l = (_Float16)lo, h = (_Float16)hi;
+    return (uint32_t)__builtin_bit_cast(uint16_t, l) | ((uint32_t)__builtin_bit_cast(uint16_t, h) << 16);
+}
+constexpr int TKL = 64;                                // keys per tile of local_fwd_b16_kernel
+template <int E> constexpr size_t local_b16_smem() { return (size_t)2 * TKL * 2 * (E + 8) * 2; }
+
+// QB: 16-query blocks per wave.  With two, every K and V^T fragment read from LDS feeds two products (the LDS fragment
+// traffic is what bounds the one-block form on long problems); a workgroup then covers 128 queries.
+template <typename T, int E, int D, int QB>
+__global__ __launch_bounds__(NT) void local_fwd_b16_kernel(LocalArgs a) {
+    static_assert(sizeof(T) == 2 && E % 32 == 0 && D % 16 == 0, "2-byte inputs, whole MFMA steps");
+    constexpr int LDK = E + 8, LDV = D + 8, KS = E / 32, DB = D / 16;
+    constexpr int STAGE = TKL * (LDK + LDV);           // 2-byte elements of a stage
+    constexpr int QW = 16 * QB, TQB = 4 * QW;          // queries per wave, per workgroup
+    constexpr float LOG2E = 1.4426950408889634f;
+    extern __shared__ __attribute__((aligned(128))) float smem[];
+    uint16_t* lds = reinterpret_cast<uint16_t*>(smem);
+    const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6), r16 = lane & 15, g = lane >> 4;
+    const int n_qt = (a.T + TQB - 1) / TQB;
+    const int n_items = a.B * a.H * n_qt;
+    const int per_xcd = (n_items + a.n_xcd - 1) / a.n_xcd;
+    const int item = (blockIdx.x % a.n_xcd) * per_xcd + blockIdx.x / a.n_xcd;   // see sblocal_fwd_kernel
+    if (item >= n_items) return;                       // workgroup-uniform
+    const int qt = item % n_qt, bh = item / n_qt, b = bh / a.H, h = bh % a.H;
+    const int q0 = qt * TQB, qw0 = q0 + QW * w;
+    const uint16_t* qptr = reinterpret_cast<const uint16_t*>(a.q) + b * a.q_sb + h * a.q_sh;
+    const uint16_t* kptr = reinterpret_cast<const uint16_t*>(a.k) + b * a.k_sb + h * a.k_sh;
+    const uint16_t* vptr = reinterpret_cast<const uint16_t*>(a.v) + b * a.v_sb + h * a.v_sh;
+    const int len = a.lens ? min((int)a.lens[b], a.S) : a.S;
+    const int lc_lo = a.lc / 2, lc_hi = (a.lc + 1) / 2;    // band: -lc_lo <= s - i < lc_hi
+
+    const int q_last = min(q0 + TQB - 1, a.T - 1);
+    const int lo = max(0, q0 - lc_lo), hi = min(len, q_last + lc_hi);
+    const int kt_lo = lo / TKL, kt_hi = (hi > lo) ? (hi + TKL - 1) / TKL : kt_lo;
+    Tile16<TKL, E, NT> rk;
+    Tile16<TKL, D, NT> rv;
+    if (kt_lo < kt_hi) {
+        rk.fetch(kptr, a.k_ss, kt_lo * TKL, a.S - 1, tid);
+        rv.fetch(vptr, a.v_ss, kt_lo * TKL, a.S - 1, tid);
+    }
+    // score operands: the query rows as they are in memory, dims 32 c + 8 g .. + 7 (the scale goes into the exponent)
+    int iq[QB], smin[QB];
+    unsigned span[QB];
+    uint32_t drop_row[QB];
+    uint4 qb[QB][KS];
+    float m_run[QB], ze[QB];
+    floatx4 oacc[QB][DB];
+#pragma unroll
+    for (int qq = 0; qq < QB; ++qq) {
+        iq[qq] = qw0 + 16 * qq + r16;
+        const uint16_t* qrow = qptr + (long)min(iq[qq], a.T - 1) * a.q_ss;
+#pragma unroll
+        for (int c = 0; c < KS; ++c) qb[qq][c] = *reinterpret_cast<const uint4*>(qrow + 32 * c + 8 * g);
+        m_run[qq] = -1e30f;         // finite, so that the first rescale is exp2(-huge) = 0 and not inf - inf
+        ze[qq] = 0.f;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) oacc[qq][db] = Frag<float>::zero();
+        smin[qq] = max(iq[qq] - lc_lo, 0);
+        span[qq] = iq[qq] < a.T ? (unsigned)max(min(iq[qq] + lc_hi, len) - smin[qq], 0) : 0u;
+        drop_row[qq] = a.drop_thresh != 0u ? drop_row_hash(a.drop_seed, (uint32_t)(bh * a.T + iq[qq])) : 0u;
+    }
+    const float sc = a.temp * LOG2E;
+    // fragment addresses inside a stage: the K row of this lane in block (hf, b), the two V rows of its transposing reads
+    const int koff = (8 * (r16 >> 2) + (r16 & 3)) * LDK + 8 * g;        // + (32 hf + 4 b) LDK + 32 c
+    const int voff = (8 * g + (r16 >> 2)) * LDV + 4 * (r16 & 3);        // + 32 hf LDV (+ 4 LDV) + 16 db
+    if (kt_lo < kt_hi) {
+        rk.template stash<LDK>(lds, tid);
+        rv.template stash<LDV>(lds + TKL * LDK, tid);
+    }
+    __syncthreads();
+    for (int kt = kt_lo; kt < kt_hi; ++kt) {
+        const int s_base = kt * TKL, cur = (kt - kt_lo) & 1;
+        const uint16_t* Ks = lds + cur * STAGE;
+        const uint16_t* Vs = Ks + TKL * LDK;
+        const bool more = kt + 1 < kt_hi;
+        if (more) {
+            rk.fetch(kptr, a.k_ss, s_base + TKL, a.S - 1, tid);
+            rv.fetch(vptr, a.v_ss, s_base + TKL, a.S - 1, tid);
+        }
+        // (wave-uniform, scalar: w is) does the tile touch the band of one of the wave's queries; does it lie inside all
+        const bool any = !(s_base + TKL - 1 - qw0 < -lc_lo || s_base - (qw0 + QW - 1) >= lc_hi || s_base >= len);
+        const bool inside = s_base - (qw0 + QW - 1) >= -lc_lo && s_base + TKL - 1 - qw0 < lc_hi && s_base + TKL <= len &&
+                            qw0 + QW - 1 < a.T;
+        if (any) {
+            floatx4 s1[QB][4];                           // block 2 hf + b, unscaled
+#pragma unroll
+            for (int qq = 0; qq < QB; ++qq)
+#pragma unroll
+                for (int hb = 0; hb < 4; ++hb) s1[qq][hb] = Frag<float>::zero();
+#pragma unroll
+            for (int hb = 0; hb < 4; ++hb)
+#pragma unroll
+                for (int c = 0; c < KS; ++c) {
+                    const uint4 kf = *reinterpret_cast<const uint4*>(Ks + koff + (32 * (hb >> 1) + 4 * (hb & 1)) * LDK + 32 * c);
+#pragma unroll
+                    for (int qq = 0; qq < QB; ++qq) s1[qq][hb] = Frag32<T>::mma(kf, qb[qq][c], s1[qq][hb]);
+                }
+            if (a.add_mask) {                                // (uniform)
+#pragma unroll
+                for (int qq = 0; qq < QB; ++qq) {
+                    const float* am = a.add_mask + (long)min(iq[qq], a.T - 1) * a.S;
+#pragma unroll
+                    for (int hb = 0; hb < 4; ++hb)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const int s = s_base + 32 * (hb >> 1) + 8 * g + 4 * (hb & 1) + i;
+                            // (an absorbing entry becomes -2^80: its product with the scale is exact, so the multiply-add
+                            //  of the exponent below gives exactly 0 for a row whose keys are all hidden)
+                            if ((unsigned)(s - smin[qq]) < span[qq])
+                                s1[qq][hb][i] = am[s] < -1e20f ? -0x1p80f : s1[qq][hb][i] + am[s];
+                        }
+                }
+            }
+            if (!inside) {
+#pragma unroll
+                for (int qq = 0; qq < QB; ++qq)
+#pragma unroll
+                    for (int hb = 0; hb < 4; ++hb)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const int s = s_base + 32 * (hb >> 1) + 8 * g + 4 * (hb & 1) + i;
+                            if (!((unsigned)(s - smin[qq]) < span[qq])) s1[qq][hb][i] = -INFINITY;
+                        }
+            }
+            float mx[QB];
+            bool moved = false;
+#pragma unroll
+            for (int qq = 0; qq < QB; ++qq) {
+                mx[qq] = -INFINITY;
+#pragma unroll
+                for (int hb = 0; hb < 4; ++hb)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) mx[qq] = fmaxf(mx[qq], s1[qq][hb][i]);
+                mx[qq] = group_max(mx[qq]) * sc;
+                moved = moved || mx[qq] > m_run[qq] + 8.f;
+            }
+            if (__builtin_amdgcn_ballot_w64(moved) != 0) {
+#pragma unroll
+                for (int qq = 0; qq < QB; ++qq) {
+                    const float m_new = fmaxf(m_run[qq], mx[qq]);
+                    const float alpha = __builtin_amdgcn_exp2f(m_run[qq] - m_new);
+                    m_run[qq] = m_new;
+                    ze[qq] *= alpha;
+#pragma unroll
+                    for (int db = 0; db < DB; ++db) oacc[qq][db] *= alpha;
+                }
+            }
+#pragma unroll
+            for (int qq = 0; qq < QB; ++qq)
+#pragma unroll
+                for (int hb = 0; hb < 4; ++hb)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        s1[qq][hb][i] = __builtin_amdgcn_exp2f(fmaf(s1[qq][hb][i], sc, -m_run[qq]));   // (masked: -inf, weight 0)
+                        ze[qq] += s1[qq][hb][i];
+                    }
+            if (a.drop_thresh != 0u) {                   // (uniform) dropped weights leave the product, not the denominator
+#pragma unroll
+                for (int qq = 0; qq < QB; ++qq)
+#pragma unroll
+                    for (int hb = 0; hb < 4; ++hb)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                            if (!drop_keep(drop_row[qq], (uint32_t)(s_base + 32 * (hb >> 1) + 8 * g + 4 * (hb & 1) + i), a.drop_thresh))
+                                s1[qq][hb][i] = 0.f;
+            }
+#pragma unroll
+            for (int hf = 0; hf < 2; ++hf) {
+                uint4 pb[QB];
+#pragma unroll
+                for (int qq = 0; qq < QB; ++qq)
+                    pb[qq] = make_uint4(pack_pair<T>(s1[qq][2 * hf][0], s1[qq][2 * hf][1]), pack_pair<T>(s1[qq][2 * hf][2], s1[qq][2 * hf][3]),
+                                        pack_pair<T>(s1[qq][2 * hf + 1][0], s1[qq][2 * hf + 1][1]),
+                                        pack_pair<T>(s1[qq][2 * hf + 1][2], s1[qq][2 * hf + 1][3]));
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+                    const uint16_t* vp = Vs + voff + 32 * hf * LDV + 16 * db;
+                    const uint4 va = __builtin_bit_cast(uint4, lds_read_tr8(reinterpret_cast<const char*>(vp),
+                                                                             reinterpret_cast<const char*>(vp + 4 * LDV)));
+#pragma unroll
+                    for (int qq = 0; qq < QB; ++qq) oacc[qq][db] = Frag32<T>::mma(va, pb[qq], oacc[qq][db]);
+                }
+            }
+        }
+        if (more) {
+            uint16_t* nxt = lds + (cur ^ 1) * STAGE;
+            rk.template stash<LDK>(nxt, tid);
+            rv.template stash<LDV>(nxt + TKL * LDK, tid);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int qq = 0; qq < QB; ++qq) {
+        float z = group_sum(ze[qq]);
+        // (every visible key masked: see local_fwd_kernel)
+        const bool all_masked = a.add_mask != nullptr && span[qq] > 0u && m_run[qq] < -1e20f;
+        if (all_masked) z += (float)(a.lc - (int)span[qq]);
+        if (iq[qq] < a.T) {
+            const float inv = (z > 0.f ? 1.0f / z : 0.f) * (a.drop_thresh != 0u ? a.drop_scale : 1.0f);
+            T* optr = reinterpret_cast<T*>(a.out) + b * a.o_sb + h * a.o_sh + (long)iq[qq] * a.o_ss;
+#pragma unroll
+            for (int db = 0; db < DB; ++db) store4_f32(optr + 16 * db + 4 * g, oacc[qq][db] * inv);
+            if (a.lse && g == 0)
+                a.lse[((long)b * a.H + h) * a.T + iq[qq]] = all_masked ? -INFINITY
+                                                            : z > 0.f ? m_run[qq] * 0.6931471805599453f + __logf(z) : 0.f;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
 // fused band kernel
 // ---------------------------------------------------------------------------------------
 template <typename T, int E, int D, int M, bool SPLIT, bool LIST = false>
@@ -4141,6 +4363,48 @@ static int launch_fwd_list(const FwdArgs& a, hipStream_t st) {
     return check_launch("sb_merge_kernel (long lists)");
 }
 
+#ifndef FLY_LOCAL_B16
+#define FLY_LOCAL_B16 1
+#endif
+// 2-byte inputs whose rows allow 16-byte loads: the kernel on the 16x16x32 MFMA of the input type
+template <typename T, int E, int QB>
+static int launch_local_b16_as(const LocalArgs& a, hipStream_t st) {
+    auto kern = local_fwd_b16_kernel<T, E, E, QB>;
+    constexpr size_t smem = local_b16_smem<E>();
+    static std::atomic<unsigned long long> lds_set{0};     // (devices on which this kernel has its LDS limit)
+    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_set, "local_fwd_b16")) return rc;
+    const Machine& mach = machine();
+    const long items = (long)a.B * a.H * ((a.T + 64 * QB - 1) / (64 * QB));
+    const long grid = (items + mach.xcds - 1) / mach.xcds * mach.xcds;
+    if (grid > 2147483647L) return fail(ERR_ARG, "local_fwd: too many workgroups");
+    LocalArgs args = a;
+    args.n_xcd = mach.xcds;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NT), smem, st, args);
+    return check_launch("local_fwd_b16_kernel");
+}
+#ifndef FLY_LOCAL_B16_WIDE
+#define FLY_LOCAL_B16_WIDE 1
+#endif
+#ifndef FLY_LOCAL_B16_WIDE_ROUNDS
+#define FLY_LOCAL_B16_WIDE_ROUNDS 2
+#endif
+// 32 queries per wave once workgroups of 128 queries still fill the device twice over (three of them share a compute
+// unit; measured at 2.7 rounds: 0.152 -> 0.129 ms at 16 heads of 16384 tokens; head dims up to 64: the wide form's
+// accumulators and score sets need the registers)
+template <typename T, int E>
+static int launch_local_b16(const LocalArgs& a, hipStream_t st) {
+    if constexpr (E <= 64) {
+        const long wide_items = (long)a.B * a.H * ((a.T + 127) / 128);
+        if (FLY_LOCAL_B16_WIDE && wide_items >= (long)FLY_LOCAL_B16_WIDE_ROUNDS * 3 * machine().cus) return launch_local_b16_as<T, E, 2>(a, st);
+    }
+    return launch_local_b16_as<T, E, 1>(a, st);
+}
+static bool local_b16_ready(const LocalArgs& a) {
+    const long strides = a.q_sb | a.q_sh | a.q_ss | a.k_sb | a.k_sh | a.k_ss | a.v_sb | a.v_sh | a.v_ss;
+    const uintptr_t ptrs = reinterpret_cast<uintptr_t>(a.q) | reinterpret_cast<uintptr_t>(a.k) | reinterpret_cast<uintptr_t>(a.v);
+    return FLY_LOCAL_B16 && strides % 8 == 0 && ptrs % 16 == 0;
+}
+
 template <typename T, int E>
 static int launch_local(const LocalArgs& a, hipStream_t st) {
     auto kern = local_fwd_kernel<T, E, E>;
@@ -5028,9 +5292,22 @@ extern "C" int flyhip_local_fwd_masked(const void* q, const void* k, const void*
         default: return fail(ERR_UNSUPPORTED, "local_fwd: head dim E=%d not in {32,64,128}", E);     \
     }
     if (dtype == F32) { LOCAL_DISPATCH(float) }
+#define LOCAL_DISPATCH_B16(TT)                                                                      \
+    switch (E) {                                                                                    \
+        case 32: return launch_local_b16<TT, 32>(a, st);                                            \
+        case 64: return launch_local_b16<TT, 64>(a, st);                                            \
+        case 128: return launch_local_b16<TT, 128>(a, st);                                          \
+        default: return fail(ERR_UNSUPPORTED, "local_fwd: head dim E=%d not in {32,64,128}", E);     \
+    }
+    if (dtype == BF16 && local_b16_ready(a)) { LOCAL_DISPATCH_B16(bf16_t) }
     if (dtype == BF16) { LOCAL_DISPATCH(bf16_t) }
+    if (dtype == F16) {
+        FLY_REQUIRE(local_b16_ready(a), "local_fwd: float16 rows must allow 16-byte loads (strides in multiples of 8 elements, aligned pointers)");
+        LOCAL_DISPATCH_B16(f16_t)
+    }
 #undef LOCAL_DISPATCH
-    return fail(ERR_UNSUPPORTED, "local_fwd supports float32 and bfloat16, got dtype code %d", dtype);
+#undef LOCAL_DISPATCH_B16
+    return fail(ERR_UNSUPPORTED, "local_fwd supports float32, bfloat16 and float16, got dtype code %d", dtype);
 }
 
 extern "C" int flyhip_local_fwd(const void* q, const void* k, const void* v, const int64_t* key_lengths, void* out,

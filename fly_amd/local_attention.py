@@ -23,7 +23,7 @@ def _additive_mask(attn_mask, T, S, device):
 
 def local_forward(query, key, value, local_context, softmax_temp=None, key_lengths=None, return_lse=False,
                   dropout=(0.0, 0), attn_mask=None):
-    """query (B,T,H,E), key (B,S,H,E), value (B,S,H,D) float32 or bfloat16 GPU tensors ->
+    """query (B,T,H,E), key (B,S,H,E), value (B,S,H,D) float32, bfloat16 or float16 GPU tensors ->
     out (B,T,H,D): query i attends to keys j with -(local_context // 2) <= j - i < (local_context + 1) // 2
     and j < key_lengths[b] (local_attention.py:68-92 for attn_mask=None).  With return_lse
     also the log of every query's softmax denominator, (B,H,T) float32 (0 for a query without keys).
@@ -35,8 +35,8 @@ def local_forward(query, key, value, local_context, softmax_temp=None, key_lengt
     masked weighs each position of its band 1 / local_context, the positions outside the keys included (they add
     nothing to the output; :76-81 leaves such rows as they are); its lse entry is -inf."""
     _lib.require_gpu(query, key, value, key_lengths, attn_mask)
-    if query.dtype not in (torch.float32, torch.bfloat16):
-        raise NotImplementedError(f'the local attention kernel supports float32 and bfloat16, got {query.dtype}')
+    if query.dtype not in (torch.float32, torch.bfloat16, torch.float16):
+        raise NotImplementedError(f'the local attention kernel supports float32, bfloat16 and float16, got {query.dtype}')
     if key.dtype != query.dtype or value.dtype != query.dtype:
         raise ValueError('query, key and value must share a dtype')
     B, T, H, E = query.shape
@@ -52,7 +52,9 @@ def local_forward(query, key, value, local_context, softmax_temp=None, key_lengt
     def prep(x):
         if x.shape[-1] != dim:
             x = F.pad(x, (0, dim - x.shape[-1]))      # zero columns change no dot product
-        return x if _vector_ready(x) else x.contiguous()
+        # (2-byte rows are loaded 8 elements at a time: strides in multiples of 8)
+        ready = _vector_ready(x) and (x.element_size() == 4 or all(st % 8 == 0 for st in x.stride()[:-1]))
+        return x if ready else x.contiguous()
     q, k, v = prep(query), prep(key), prep(value)
     lens = None
     if key_lengths is not None:
@@ -198,13 +200,9 @@ class LocalAttention(nn.Module):
         if key_padding_mask is not None and not bool(key_padding_mask.all_ones):
             lengths = key_padding_mask.lengths
         if not need_weights:
-            # float16 inputs are widened to float32 for the kernels (exact) and the result goes back to float16
-            in_dtype = query.dtype
-            if in_dtype == torch.float16:
-                query, key, value = query.float(), key.float(), value.float()
             out = local_attention_fn(query, key, value, self.local_context, softmax_temp=self.softmax_temp,
                                      key_lengths=lengths, dropout=dropout, attn_mask=additive)
-            return (out.to(in_dtype) if in_dtype == torch.float16 else out), None
+            return out, None
         B, T, H, E = query.shape
         S = key.shape[1]
         if B * H * T * S > self.max_weight_elements:

@@ -338,7 +338,10 @@ int flyhip_sbblocksparse_fwd(const void* q, const void* k, const void* v, const 
  * fast_transformers.local_product): out[i] = softmax over the band -(lc/2) <= s - i < (lc+1)/2, s below
  * the key length, of t q_i.k_s, times v.  q (B,T,H,E), k (B,S,H,E), v (B,S,H,D), out (B,T,H,D) via
  * (batch, head, seq) strides, innermost contiguous; E = D in {32,64,128}; key_lengths (B) int64 or
- * NULL.  A query with no valid key gets a zero row (local_attention.py:74-84). */
+ * NULL.  A query with no valid key gets a zero row (local_attention.py:74-84).
+ * dtype: float32 (both products on the fp32 matrix pipe), bfloat16 or float16 (both on the 16x16x32 MFMA of the
+ * type, the weights rounded to it for the second product; float16 needs strides in multiples of 8 elements and
+ * 16-byte aligned pointers, bfloat16 with other strides runs on the fp32 pipe). */
 int flyhip_local_fwd(const void* q, const void* k, const void* v, const int64_t* key_lengths, void* out,
                      int B, int H, int T, int S, int E, int D, int local_context,
                      int64_t q_sb, int64_t q_sh, int64_t q_ss,
