@@ -490,6 +490,14 @@ def bench_other_configs():
     pairs = band_fl / (2 * (E + 2 * mh + E))                 # band pairs, from the count above
     ms = timeit(lambda: local_forward(q, k, v, lc, softmax_temp=0.125))
     out['local_attention_bf16_L16384'] = {'ms': ms, 'tflops': pairs * 2 * (E + E) / ms / 1e9}
+    from fly_amd.local_attention import local_attention_fn
+    qg, kg, vg = (x.clone().requires_grad_() for x in (q, k, v))
+    go = torch.randn(B, L, H, E, generator=g).bfloat16().to(dev)
+
+    def local_step():
+        local_attention_fn(qg, kg, vg, lc, softmax_temp=0.125).backward(go)
+        qg.grad = kg.grad = vg.grad = None
+    out['local_attention_bf16_L16384']['fwd_bwd_ms'] = timeit(local_step, n=5)
     return out
 
 

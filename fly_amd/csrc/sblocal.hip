@@ -2964,6 +2964,245 @@ __global__ __launch_bounds__(NT) void local_fwd_b16_kernel(LocalArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------
+// gradients of plain local attention for 2-byte inputs
+// ---------------------------------------------------------------------------------------
+// With P_is = exp(t q_i.k_s - lse_i) on the band, g = d out and delta_i = g_i.out_i (local_attention.py:68-92 leaves
+// these to autograd):  d v_s = sum_i P_is g_i,  dS_is = P_is (g_i.v_s - delta_i),  d q_i = t sum_s dS_is k_s,
+// d k_s = t sum_i dS_is q_i.  One kernel in two orientations, built like local_fwd_b16_kernel: a wave owns QB blocks
+// of 16 "outer" rows (queries, or keys when KEYMAJOR) whose two operands stay in registers, and walks 64-row tiles of
+// the "inner" side (keys with values, or queries with their output gradients) through LDS.
+//   S^T  = Y1 . x1  and  G^T = Y2 . x2   (inner rows of a 16-row block picked so that a lane's results over two
+//                                         blocks are eight consecutive inner rows, the contraction slots below)
+//   P = exp2(sc S - lse log2e) where the pair is in the band, dS = P (G - delta)   (lse, delta: of the query)
+//   d x^T[e][outer] += Y^T[e][inner] . {P, dS}[inner][outer]   (Y^T fragments by transposing LDS reads)
+// Query-major: d q from (K, dS).  Key-major: d v from (d out, P) and d k from (Q, dS).
+struct LocalBwdArgs {
+    const void* q; const void* k; const void* v; const void* go; const void* out;
+    const float* lse; float* delta;                 // (B, H, T); delta is written by the query-major launch
+    const int64_t* lens;
+    void* dq; void* dk; void* dv;
+    int B, H, T, S, lc;
+    long q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, g_sb, g_sh, g_ss, o_sb, o_sh, o_ss;
+    long dq_sb, dq_sh, dq_ss, dk_sb, dk_sh, dk_ss, dv_sb, dv_sh, dv_ss;
+    float temp;
+    int n_xcd;
+};
+template <typename T> __device__ __forceinline__ float unpack_lo(uint32_t w);
+template <typename T> __device__ __forceinline__ float unpack_hi(uint32_t w);
+template <> __device__ __forceinline__ float unpack_lo<bf16_t>(uint32_t w) { return __uint_as_float(w << 16); }
+template <> __device__ __forceinline__ float unpack_hi<bf16_t>(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+template <> __device__ __forceinline__ float unpack_lo<f16_t>(uint32_t w) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xffffu)); }
+template <> __device__ __forceinline__ float unpack_hi<f16_t>(uint32_t w) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16)); }
+template <int E> constexpr size_t local_bwd_smem() { return (size_t)2 * (TKL * 2 * (E + 8) * 2 + 2 * TKL * sizeof(float)); }
+
+template <typename T, int E, bool KEYMAJOR, int QB>
+__global__ __launch_bounds__(NT) void local_bwd_b16_kernel(LocalBwdArgs a) {
+    static_assert(sizeof(T) == 2 && E % 32 == 0, "2-byte inputs, whole MFMA steps");
+    constexpr int LD = E + 8, KS = E / 32, EB = E / 16;
+    constexpr int STAGE_BYTES = TKL * 2 * LD * 2 + 2 * TKL * (int)sizeof(float);
+    constexpr int QW = 16 * QB, TQB = 4 * QW;          // outer rows per wave, per workgroup
+    constexpr float LOG2E = 1.4426950408889634f;
+    extern __shared__ __attribute__((aligned(128))) float smem[];
+    char* lds = reinterpret_cast<char*>(smem);
+    const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6), r16 = lane & 15, g = lane >> 4;
+    const int R_out = KEYMAJOR ? a.S : a.T, R_in = KEYMAJOR ? a.T : a.S;
+    const int n_ot = (R_out + TQB - 1) / TQB;
+    const int n_items = a.B * a.H * n_ot;
+    const int per_xcd = (n_items + a.n_xcd - 1) / a.n_xcd;
+    const int item = (blockIdx.x % a.n_xcd) * per_xcd + blockIdx.x / a.n_xcd;   // see sblocal_fwd_kernel
+    if (item >= n_items) return;                       // workgroup-uniform
+    const int ot = item % n_ot, bh = item / n_ot, b = bh / a.H, h = bh % a.H;
+    const int o0 = ot * TQB, ow0 = o0 + QW * w;
+    const uint16_t* qptr = reinterpret_cast<const uint16_t*>(a.q) + b * a.q_sb + h * a.q_sh;
+    const uint16_t* kptr = reinterpret_cast<const uint16_t*>(a.k) + b * a.k_sb + h * a.k_sh;
+    const uint16_t* vptr = reinterpret_cast<const uint16_t*>(a.v) + b * a.v_sb + h * a.v_sh;
+    const uint16_t* gptr = reinterpret_cast<const uint16_t*>(a.go) + b * a.g_sb + h * a.g_sh;
+    const uint16_t* x1p = KEYMAJOR ? kptr : qptr;  const long x1s = KEYMAJOR ? a.k_ss : a.q_ss;     // outer operands
+    const uint16_t* x2p = KEYMAJOR ? vptr : gptr;  const long x2s = KEYMAJOR ? a.v_ss : a.g_ss;
+    const uint16_t* y1p = KEYMAJOR ? qptr : kptr;  const long y1s = KEYMAJOR ? a.q_ss : a.k_ss;     // inner tiles
+    const uint16_t* y2p = KEYMAJOR ? gptr : vptr;  const long y2s = KEYMAJOR ? a.g_ss : a.v_ss;
+    const float* lsep = a.lse + (long)bh * a.T;
+    const float* delp = a.delta + (long)bh * a.T;
+    const int len = a.lens ? min((int)a.lens[b], a.S) : a.S;
+    // the pair (outer o, inner n) is in the band when n - o lies in [-A, Bq), o < Lo and n < Ln
+    const int lc_lo = a.lc / 2, lc_hi = (a.lc + 1) / 2;
+    const int A = KEYMAJOR ? lc_hi - 1 : lc_lo, Bq = KEYMAJOR ? lc_lo + 1 : lc_hi;
+    const int Lo = KEYMAJOR ? len : a.T, Ln = KEYMAJOR ? a.T : len;
+
+    const int o_last = min(min(o0 + TQB - 1, R_out - 1), Lo - 1);
+    const int lo = max(0, o0 - A), hi = o_last >= o0 ? min(Ln, o_last + Bq) : 0;
+    const int it_lo = lo / TKL, it_hi = (hi > lo) ? (hi + TKL - 1) / TKL : it_lo;
+    Tile16<TKL, E, NT> r1, r2;
+    float rl = 0.f, rd = 0.f;                          // key-major: lse log2e and delta of inner row tid (threads 0 .. 63)
+    auto fetch = [&](int it) __attribute__((always_inline)) {
+        r1.fetch(y1p, y1s, it * TKL, R_in - 1, tid);
+        r2.fetch(y2p, y2s, it * TKL, R_in - 1, tid);
+        if (KEYMAJOR && tid < TKL) {
+            const int i = min(it * TKL + tid, a.T - 1);
+            rl = lsep[i] * LOG2E;
+            rd = delp[i];
+        }
+    };
+    auto stash = [&](int stage) __attribute__((always_inline)) {
+        uint16_t* t1 = reinterpret_cast<uint16_t*>(lds + stage * STAGE_BYTES);
+        r1.template stash<LD>(t1, tid);
+        r2.template stash<LD>(t1 + TKL * LD, tid);
+        if (KEYMAJOR && tid < TKL) {
+            float* sc_ = reinterpret_cast<float*>(lds + stage * STAGE_BYTES + TKL * 2 * LD * 2);
+            sc_[tid] = rl;
+            sc_[TKL + tid] = rd;
+        }
+    };
+    if (it_lo < it_hi) fetch(it_lo);
+
+    int io[QB], vmin[QB];
+    unsigned vspan[QB];
+    uint4 x1[QB][KS], x2[QB][KS];
+    float l_own[QB], d_own[QB];
+    floatx4 acc1[QB][EB], acc2[KEYMAJOR ? QB : 1][KEYMAJOR ? EB : 1];     // d q | d k, and d v
+#pragma unroll
+    for (int qq = 0; qq < QB; ++qq) {
+        io[qq] = ow0 + 16 * qq + r16;
+        const long row = min(io[qq], R_out - 1);
+#pragma unroll
+        for (int c = 0; c < KS; ++c) {
+            x1[qq][c] = *reinterpret_cast<const uint4*>(x1p + row * x1s + 32 * c + 8 * g);
+            x2[qq][c] = *reinterpret_cast<const uint4*>(x2p + row * x2s + 32 * c + 8 * g);
+        }
+        vmin[qq] = max(io[qq] - A, 0);
+        vspan[qq] = io[qq] < Lo ? (unsigned)max(min(io[qq] + Bq, Ln) - vmin[qq], 0) : 0u;
+        l_own[qq] = d_own[qq] = 0.f;
+        if (!KEYMAJOR) {
+            l_own[qq] = lsep[min(io[qq], a.T - 1)] * LOG2E;
+            // delta of the query, g . out, from the output row in the layout of the gradient row; kept for the key-major launch
+            const uint16_t* orow = reinterpret_cast<const uint16_t*>(a.out) + b * a.o_sb + h * a.o_sh + row * a.o_ss;
+            float dsum = 0.f;
+#pragma unroll
+            for (int c = 0; c < KS; ++c) {
+                const uint4 ov = *reinterpret_cast<const uint4*>(orow + 32 * c + 8 * g);
+                const uint32_t ow[4] = {ov.x, ov.y, ov.z, ov.w}, gw[4] = {x2[qq][c].x, x2[qq][c].y, x2[qq][c].z, x2[qq][c].w};
+#pragma unroll
+                for (int x = 0; x < 4; ++x)
+                    dsum += unpack_lo<T>(ow[x]) * unpack_lo<T>(gw[x]) + unpack_hi<T>(ow[x]) * unpack_hi<T>(gw[x]);
+            }
+            d_own[qq] = group_sum(dsum);
+            if (g == 0 && io[qq] < a.T) a.delta[(long)bh * a.T + io[qq]] = d_own[qq];
+        }
+#pragma unroll
+        for (int eb = 0; eb < EB; ++eb) acc1[qq][eb] = Frag<float>::zero();
+    }
+    if (KEYMAJOR) {
+#pragma unroll
+        for (int qq = 0; qq < QB; ++qq)
+#pragma unroll
+            for (int eb = 0; eb < EB; ++eb) acc2[qq][eb] = Frag<float>::zero();
+    }
+    const float sc = a.temp * LOG2E;
+    const int foff = (8 * (r16 >> 2) + (r16 & 3)) * LD + 8 * g;         // + (32 hf + 4 b) LD + 32 c   (elements)
+    const int toff = (8 * g + (r16 >> 2)) * LD + 4 * (r16 & 3);         // + 32 hf LD (+ 4 LD) + 16 eb
+    if (it_lo < it_hi) stash(0);
+    __syncthreads();
+    for (int it = it_lo; it < it_hi; ++it) {
+        const int i_base = it * TKL, cur = (it - it_lo) & 1;
+        const uint16_t* Y1 = reinterpret_cast<const uint16_t*>(lds + cur * STAGE_BYTES);
+        const uint16_t* Y2 = Y1 + TKL * LD;
+        const float* Ls = reinterpret_cast<const float*>(lds + cur * STAGE_BYTES + TKL * 2 * LD * 2);
+        const bool more = it + 1 < it_hi;
+        if (more) fetch(it + 1);
+        // (wave-uniform, scalar) does the tile touch the band of one of the wave's outer rows; does it lie inside all
+        const bool any = !(i_base + TKL - 1 - ow0 < -A || i_base - (ow0 + QW - 1) >= Bq || i_base >= Ln || ow0 >= Lo);
+        const bool inside = i_base - (ow0 + QW - 1) >= -A && i_base + TKL - 1 - ow0 < Bq && i_base + TKL <= Ln && ow0 + QW - 1 < Lo;
+        if (any) {
+            floatx4 s1[QB][4], gp[QB][4];                // block 2 hf + b: scores (unscaled) and g.v
+#pragma unroll
+            for (int qq = 0; qq < QB; ++qq)
+#pragma unroll
+                for (int hb = 0; hb < 4; ++hb) { s1[qq][hb] = Frag<float>::zero(); gp[qq][hb] = Frag<float>::zero(); }
+#pragma unroll
+            for (int hb = 0; hb < 4; ++hb)
+#pragma unroll
+                for (int c = 0; c < KS; ++c) {
+                    const int off = foff + (32 * (hb >> 1) + 4 * (hb & 1)) * LD + 32 * c;
+                    const uint4 f1 = *reinterpret_cast<const uint4*>(Y1 + off);
+                    const uint4 f2 = *reinterpret_cast<const uint4*>(Y2 + off);
+#pragma unroll
+                    for (int qq = 0; qq < QB; ++qq) {
+                        s1[qq][hb] = Frag32<T>::mma(f1, x1[qq][c], s1[qq][hb]);
+                        gp[qq][hb] = Frag32<T>::mma(f2, x2[qq][c], gp[qq][hb]);
+                    }
+                }
+            floatx4 ln4[4], dl4[4];                      // key-major: the queries' lse log2e and delta, by block
+            if (KEYMAJOR) {
+#pragma unroll
+                for (int hb = 0; hb < 4; ++hb) {
+                    ln4[hb] = *reinterpret_cast<const floatx4*>(Ls + 32 * (hb >> 1) + 8 * g + 4 * (hb & 1));
+                    dl4[hb] = *reinterpret_cast<const floatx4*>(Ls + TKL + 32 * (hb >> 1) + 8 * g + 4 * (hb & 1));
+                }
+            }
+            // weights P into s1, dS into gp
+#pragma unroll
+            for (int qq = 0; qq < QB; ++qq)
+#pragma unroll
+                for (int hb = 0; hb < 4; ++hb)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int n = i_base + 32 * (hb >> 1) + 8 * g + 4 * (hb & 1) + i;
+                        const float lrow = KEYMAJOR ? ln4[hb][i] : l_own[qq], drow = KEYMAJOR ? dl4[hb][i] : d_own[qq];
+                        float pr = __builtin_amdgcn_exp2f(fmaf(s1[qq][hb][i], sc, -lrow));
+                        if (!inside && !((unsigned)(n - vmin[qq]) < vspan[qq])) pr = 0.f;
+                        s1[qq][hb][i] = pr;
+                        gp[qq][hb][i] = pr * (gp[qq][hb][i] - drow);
+                    }
+#pragma unroll
+            for (int hf = 0; hf < 2; ++hf) {
+                uint4 pb[KEYMAJOR ? QB : 1], sb[QB];
+#pragma unroll
+                for (int qq = 0; qq < QB; ++qq) {
+                    sb[qq] = make_uint4(pack_pair<T>(gp[qq][2 * hf][0], gp[qq][2 * hf][1]), pack_pair<T>(gp[qq][2 * hf][2], gp[qq][2 * hf][3]),
+                                        pack_pair<T>(gp[qq][2 * hf + 1][0], gp[qq][2 * hf + 1][1]),
+                                        pack_pair<T>(gp[qq][2 * hf + 1][2], gp[qq][2 * hf + 1][3]));
+                    if (KEYMAJOR)
+                        pb[qq] = make_uint4(pack_pair<T>(s1[qq][2 * hf][0], s1[qq][2 * hf][1]), pack_pair<T>(s1[qq][2 * hf][2], s1[qq][2 * hf][3]),
+                                            pack_pair<T>(s1[qq][2 * hf + 1][0], s1[qq][2 * hf + 1][1]),
+                                            pack_pair<T>(s1[qq][2 * hf + 1][2], s1[qq][2 * hf + 1][3]));
+                }
+#pragma unroll
+                for (int eb = 0; eb < EB; ++eb) {
+                    const uint16_t* p1 = Y1 + toff + 32 * hf * LD + 16 * eb;
+                    const uint4 t1 = __builtin_bit_cast(uint4, lds_read_tr8(reinterpret_cast<const char*>(p1),
+                                                                             reinterpret_cast<const char*>(p1 + 4 * LD)));
+#pragma unroll
+                    for (int qq = 0; qq < QB; ++qq) acc1[qq][eb] = Frag32<T>::mma(t1, sb[qq], acc1[qq][eb]);
+                    if (KEYMAJOR) {
+                        const uint16_t* p2 = Y2 + toff + 32 * hf * LD + 16 * eb;
+                        const uint4 t2 = __builtin_bit_cast(uint4, lds_read_tr8(reinterpret_cast<const char*>(p2),
+                                                                                 reinterpret_cast<const char*>(p2 + 4 * LD)));
+#pragma unroll
+                        for (int qq = 0; qq < QB; ++qq) acc2[qq][eb] = Frag32<T>::mma(t2, pb[qq], acc2[qq][eb]);
+                    }
+                }
+            }
+        }
+        if (more) stash(cur ^ 1);
+        __syncthreads();
+    }
+#pragma unroll
+    for (int qq = 0; qq < QB; ++qq) {
+        if (io[qq] < R_out) {
+            T* d1 = KEYMAJOR ? reinterpret_cast<T*>(a.dk) + b * a.dk_sb + h * a.dk_sh + (long)io[qq] * a.dk_ss
+                             : reinterpret_cast<T*>(a.dq) + b * a.dq_sb + h * a.dq_sh + (long)io[qq] * a.dq_ss;
+#pragma unroll
+            for (int eb = 0; eb < EB; ++eb) store4_f32(d1 + 16 * eb + 4 * g, acc1[qq][eb] * a.temp);
+            if (KEYMAJOR) {
+                T* d2 = reinterpret_cast<T*>(a.dv) + b * a.dv_sb + h * a.dv_sh + (long)io[qq] * a.dv_ss;
+#pragma unroll
+                for (int eb = 0; eb < EB; ++eb) store4_f32(d2 + 16 * eb + 4 * g, acc2[qq][eb]);
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
 // fused band kernel
 // ---------------------------------------------------------------------------------------
 template <typename T, int E, int D, int M, bool SPLIT, bool LIST = false>
@@ -4405,6 +4644,32 @@ static bool local_b16_ready(const LocalArgs& a) {
     return FLY_LOCAL_B16 && strides % 8 == 0 && ptrs % 16 == 0;
 }
 
+#ifndef FLY_LOCAL_BWD_QB
+#define FLY_LOCAL_BWD_QB 1
+#endif
+template <typename T, int E, bool KEYMAJOR, int QB>
+static int launch_local_bwd_as(const LocalBwdArgs& a, hipStream_t st) {
+    auto kern = local_bwd_b16_kernel<T, E, KEYMAJOR, QB>;
+    constexpr size_t smem = local_bwd_smem<E>();
+    static std::atomic<unsigned long long> lds_set{0};     // (devices on which this kernel has its LDS limit)
+    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_set, "local_bwd_b16")) return rc;
+    const Machine& mach = machine();
+    const int rows = KEYMAJOR ? a.S : a.T;
+    const long items = (long)a.B * a.H * ((rows + 64 * QB - 1) / (64 * QB));
+    const long grid = (items + mach.xcds - 1) / mach.xcds * mach.xcds;
+    if (grid > 2147483647L) return fail(ERR_ARG, "local_bwd: too many workgroups");
+    LocalBwdArgs args = a;
+    args.n_xcd = mach.xcds;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NT), smem, st, args);
+    return check_launch("local_bwd_b16_kernel");
+}
+template <typename T, int E>
+static int launch_local_bwd(const LocalBwdArgs& a, hipStream_t st) {
+    // (query-major first: it leaves delta for the key-major launch)
+    if (int rc = launch_local_bwd_as<T, E, false, FLY_LOCAL_BWD_QB>(a, st)) return rc;
+    return launch_local_bwd_as<T, E, true, FLY_LOCAL_BWD_QB>(a, st);
+}
+
 template <typename T, int E>
 static int launch_local(const LocalArgs& a, hipStream_t st) {
     auto kern = local_fwd_kernel<T, E, E>;
@@ -5308,6 +5573,49 @@ extern "C" int flyhip_local_fwd_masked(const void* q, const void* k, const void*
 #undef LOCAL_DISPATCH
 #undef LOCAL_DISPATCH_B16
     return fail(ERR_UNSUPPORTED, "local_fwd supports float32, bfloat16 and float16, got dtype code %d", dtype);
+}
+
+extern "C" int flyhip_local_bwd(const void* q, const void* k, const void* v, const void* out, const void* grad_out,
+                               const float* lse, const int64_t* key_lengths, float* delta,
+                               void* dq, void* dk, void* dv,
+                               int B, int H, int T, int S, int E, int local_context,
+                               int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                               int64_t k_sb, int64_t k_sh, int64_t k_ss,
+                               int64_t v_sb, int64_t v_sh, int64_t v_ss,
+                               int64_t o_sb, int64_t o_sh, int64_t o_ss,
+                               int64_t g_sb, int64_t g_sh, int64_t g_ss,
+                               int64_t dq_sb, int64_t dq_sh, int64_t dq_ss,
+                               int64_t dk_sb, int64_t dk_sh, int64_t dk_ss,
+                               int64_t dv_sb, int64_t dv_sh, int64_t dv_ss,
+                               float softmax_temp, int dtype, void* stream) {
+    FLY_REQUIRE(q && k && v && out && grad_out && lse && delta && dq && dk && dv, "local_bwd: null pointer");
+    FLY_REQUIRE(B > 0 && H > 0 && T > 0 && S > 0, "local_bwd: empty problem");
+    FLY_REQUIRE(local_context >= 1, "local_bwd: local_context must be >= 1");
+    FLY_REQUIRE(softmax_temp > 0.f, "local_bwd: softmax_temp must be positive");
+    FLY_REQUIRE(((q_sb | q_sh | q_ss | k_sb | k_sh | k_ss | v_sb | v_sh | v_ss | g_sb | g_sh | g_ss | o_sb | o_sh | o_ss) % 8) == 0,
+                "local_bwd: input strides must be multiples of 8 elements (16-byte loads)");
+    FLY_REQUIRE(((dq_sb | dq_sh | dq_ss | dk_sb | dk_sh | dk_ss | dv_sb | dv_sh | dv_ss) % 4) == 0,
+                "local_bwd: output strides must be multiples of 4 elements (8-byte stores)");
+    FLY_REQUIRE(((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
+                  reinterpret_cast<uintptr_t>(grad_out) | reinterpret_cast<uintptr_t>(out)) % 16) == 0 &&
+                ((reinterpret_cast<uintptr_t>(dq) | reinterpret_cast<uintptr_t>(dk) | reinterpret_cast<uintptr_t>(dv)) % 8) == 0,
+                "local_bwd: pointers must be 16-byte (inputs) and 8-byte (outputs) aligned");
+    LocalBwdArgs a{q, k, v, grad_out, out, lse, delta, key_lengths, dq, dk, dv, B, H, T, S, local_context,
+                   q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, g_sb, g_sh, g_ss, o_sb, o_sh, o_ss,
+                   dq_sb, dq_sh, dq_ss, dk_sb, dk_sh, dk_ss, dv_sb, dv_sh, dv_ss, softmax_temp, 0};
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (int rc_capture = refuse_capture(st)) return rc_capture;
+#define LOCAL_BWD_DISPATCH(TT)                                                                      \
+    switch (E) {                                                                                    \
+        case 32: return launch_local_bwd<TT, 32>(a, st);                                            \
+        case 64: return launch_local_bwd<TT, 64>(a, st);                                            \
+        case 128: return launch_local_bwd<TT, 128>(a, st);                                          \
+        default: return fail(ERR_UNSUPPORTED, "local_bwd: head dim E=%d not in {32,64,128}", E);     \
+    }
+    if (dtype == BF16) { LOCAL_BWD_DISPATCH(bf16_t) }
+    if (dtype == F16) { LOCAL_BWD_DISPATCH(f16_t) }
+#undef LOCAL_BWD_DISPATCH
+    return fail(ERR_UNSUPPORTED, "local_bwd supports bfloat16 and float16, got dtype code %d", dtype);
 }
 
 extern "C" int flyhip_local_fwd(const void* q, const void* k, const void* v, const int64_t* key_lengths, void* out,

@@ -81,8 +81,10 @@ def local_backward(query, key, value, local_context, softmax_temp, key_lengths, 
     (sblocal_backward.BandWindows); with
     P = softmax over the band, g = d out and delta_i = sum_s P_is g_i.v_s:
     d v_s = sum_i P_is g_i,  d(t q_i.k_s) = P_is (g_i.v_s - delta_i).  Queries without any visible
-    key get zero gradients.  Given the forward's out and lse (local_forward(..., return_lse=True)), float32
-    or bfloat16 GPU tensors and head dims <= 64, the sums run on the backward band kernel of
+    key get zero gradients.  bfloat16 and float16 GPU tensors with the forward's out and lse, no attn_mask and no
+    dropout: flyhip_local_bwd, on the matrix pipe of the input type (_local_backward_2byte).  Otherwise, given the
+    forward's out and lse (local_forward(..., return_lse=True)), GPU tensors
+    and head dims <= 64, the sums run in float32 on the backward band kernel of
     Scatterbrain-local attention with its feature operands zero (flyhip_sblocal_bwd_band: P_is =
     exp(t q_i.k_s - lse_i), delta_i = g_i.out_i); otherwise as batched library products on the GPU (host tensors are
     accepted in float64 only: the check of these formulas against autograd).  dropout = (p, seed) of the forward:
@@ -92,6 +94,9 @@ def local_backward(query, key, value, local_context, softmax_temp, key_lengths, 
     B, T, H, E = query.shape
     S, D = key.shape[1], value.shape[3]
     t = softmax_temp or 1 / math.sqrt(E)
+    if (query.dtype in (torch.bfloat16, torch.float16) and query.is_cuda and out is not None and lse is not None
+            and attn_mask is None and dropout[0] == 0 and max(E, D) <= _HEAD_DIMS[-1]):
+        return _local_backward_2byte(query, key, value, local_context, t, key_lengths, grad_out, out, lse)
     wdt = torch.float64 if query.dtype == torch.float64 else torch.float32
 
     def bh(x):                                   # (B,L,H,C) -> (B*H, L, C)
@@ -137,6 +142,36 @@ def local_backward(query, key, value, local_context, softmax_temp, key_lengths, 
         band.add_windows(acc_v, j0, p.transpose(2, 3) @ Gc[:, sl])
     dQ, dK, dV = band.unchunk(dQc), band.fold(acc_k), band.fold(acc_v)
     return back(dQ, query), back(dK, key), back(dV, value)
+
+
+def _local_backward_2byte(query, key, value, local_context, t, key_lengths, grad_out, out, lse):
+    """local_backward for bfloat16 / float16 GPU tensors on flyhip_local_bwd: the band softmax is formed again from the
+    forward's lse on the matrix pipe of the input type; delta_i = g_i . out_i is formed by the first launch."""
+    B, T, H, E = query.shape
+    S, D = key.shape[1], value.shape[3]
+    dim = _round_up_choice(max(E, D), _HEAD_DIMS, 'head dimension')
+
+    def prep(x):
+        if x.shape[-1] != dim:
+            x = F.pad(x, (0, dim - x.shape[-1]))      # zero columns change no dot product
+        ready = _vector_ready(x) and all(st % 8 == 0 for st in x.stride()[:-1])
+        return x if ready else x.contiguous()
+    q, k, v, g, o = prep(query), prep(key), prep(value), prep(grad_out.to(query.dtype)), prep(out.to(query.dtype))
+    delta = torch.empty(B, H, T, dtype=torch.float32, device=query.device)     # g . out per query, filled by the kernels
+    lse_ = lse.reshape(B, H, T).float().contiguous()
+    lens = None if key_lengths is None else key_lengths.to(device=query.device, dtype=torch.int64).contiguous()
+    dq = torch.empty(B, T, H, dim, dtype=query.dtype, device=query.device)
+    dk = torch.empty(B, S, H, dim, dtype=query.dtype, device=query.device)
+    dv = torch.empty(B, S, H, dim, dtype=query.dtype, device=query.device)
+
+    def strides(x):
+        return x.stride(0), x.stride(2), x.stride(1)
+    with torch.cuda.device(query.device):
+        _lib.call('flyhip_local_bwd', q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), g.data_ptr(),
+                  lse_.data_ptr(), _lib.ptr(lens), delta.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+                  B, H, T, S, dim, local_context, *strides(q), *strides(k), *strides(v), *strides(o), *strides(g),
+                  *strides(dq), *strides(dk), *strides(dv), t, _lib.dtype_code(q), _lib.stream_ptr(query.device))
+    return dq[..., :E], dk[..., :E], dv[..., :D]
 
 
 class _LocalFn(torch.autograd.Function):

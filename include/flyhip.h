@@ -392,6 +392,30 @@ int flyhip_local_fwd_masked(const void* q, const void* k, const void* v, const i
                             int64_t o_sb, int64_t o_sh, int64_t o_ss,
                             float softmax_temp, int dtype, float dropout_p, uint64_t dropout_seed, void* stream);
 
+/* Gradients of flyhip_local_fwd for bfloat16 or float16 tensors (the reference takes them from autograd through
+ * fast_transformers.local_product, src/models/attention/local_attention.py:68-92): with P = the band softmax formed again
+ * as exp(t q.k - lse), g = grad_out and delta[b][h][i] = g_i . out_i (float32 (B,H,T) like lse: caller-owned scratch
+ * that the first launch fills from out, the forward's output, and the second reads):
+ * dv_s = sum_i P_is g_i, dS_is = P_is (g_i.v_s - delta_i), dq_i = t sum_s dS_is k_s, dk_s = t sum_i dS_is q_i.  Two
+ * launches (query-major for dq, key-major for dk and dv) on the 16x16x32 MFMA of the input type, P and dS rounded to it.
+ * q, out, grad_out, dq (B,T,H,E) and k, v, dk, dv (B,S,H,E) via (batch, head, seq) strides in elements, innermost
+ * contiguous, E in {32,64,128}; input strides in multiples of 8 elements and 16-byte aligned pointers, output strides in
+ * multiples of 4.  Every row of dq, dk, dv is written (zeros where a row has no pair in the band).  No attn_mask, no
+ * dropout: those gradients run on flyhip_sblocal_bwd_band_masked. */
+int flyhip_local_bwd(const void* q, const void* k, const void* v, const void* out, const void* grad_out,
+                     const float* lse, const int64_t* key_lengths, float* delta,
+                     void* dq, void* dk, void* dv,
+                     int B, int H, int T, int S, int E, int local_context,
+                     int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                     int64_t k_sb, int64_t k_sh, int64_t k_ss,
+                     int64_t v_sb, int64_t v_sh, int64_t v_ss,
+                     int64_t o_sb, int64_t o_sh, int64_t o_ss,
+                     int64_t g_sb, int64_t g_sh, int64_t g_ss,
+                     int64_t dq_sb, int64_t dq_sh, int64_t dq_ss,
+                     int64_t dk_sb, int64_t dk_sh, int64_t dk_ss,
+                     int64_t dv_sb, int64_t dv_sh, int64_t dv_ss,
+                     float softmax_temp, int dtype, void* stream);
+
 /* Measurement hook (no counterpart in the reference): the two caller-owned hipEvent_t receive the begin
  * and the end time stamp of the fused band kernel's launch (hipExtLaunchKernelGGL) in the NEXT
  * flyhip_sblocal_fwd call of the calling thread, on its stream, and are then forgotten: their elapsed time

@@ -550,6 +550,46 @@ def test_local_attention_module_gradients(dtype, tol):
     assert float(kg.grad[1, 200:].abs().max()) == 0.0
 
 
+@pytest.mark.parametrize('case', [
+    dict(B=2, T=300, S=280, H=2, E=64, D=64, lc=64, lens=[280, 200], dtype=torch.float16),
+    dict(B=2, T=130, S=257, H=1, E=21, D=17, lc=33, lens=[257, 100], dtype=torch.bfloat16),
+    dict(B=1, T=200, S=70, H=2, E=128, D=128, lc=40, lens=[50], dtype=torch.bfloat16),
+    dict(B=1, T=700, S=900, H=2, E=32, D=32, lc=301, lens=None, dtype=torch.float16),
+    dict(B=1, T=1100, S=900, H=2, E=64, D=64, lc=512, lens=[801], dtype=torch.bfloat16),
+    dict(B=2, T=96, S=96, H=3, E=64, D=32, lc=1, lens=None, dtype=torch.bfloat16),
+], ids=['fp16-lengths', 'odd-sizes-lengths', 'rows-without-keys-128', 'fp16-long-band', 'long-band-lengths', 'window-of-one'])
+def test_local_attention_gradients_on_the_2byte_kernels(case):
+    """Gradients of LocalAttention for bfloat16 / float16 inputs (flyhip_local_bwd: query-major launch for d query,
+    key-major launch for d key and d value, both on the matrix pipe of the input type) against autograd through the
+    oracle in float64 on the same rounded inputs: padded head dims, more keys than queries and the reverse, key
+    lengths, queries and keys without a partner (zero gradients), bands long enough for tiles that skip the masks."""
+    from fly_amd import LocalAttention, LengthMask
+    c = dict(case)
+    dtype, lens = c.pop('dtype'), c.pop('lens')
+    print('case', c, dtype, flush=True)
+    B, T, S, H, E, D, lc = (c[x] for x in 'B T S H E D lc'.split())
+    g = torch.Generator().manual_seed(61)
+    q, k, v = (torch.randn(B, L, H, C, generator=g).to(dtype) for L, C in ((T, E), (S, E), (S, D)))
+    w = torch.randn(B, T, H, D, generator=g).to(dtype)
+    lengths = None if lens is None else torch.tensor(lens)
+    qd, kd, vd = (x.double().requires_grad_() for x in (q, k, v))
+    ref_out = osb.local_attention(qd, kd, vd, lc, key_lengths=lengths)
+    (ref_out * w.double()).sum().backward()
+    dev = torch.device('cuda:0')
+    mod = LocalAttention(lc).to(dev)
+    qg, kg, vg = (x.to(dev).requires_grad_() for x in (q, k, v))
+    mask = None if lengths is None else LengthMask(lengths.to(dev), max_len=S)
+    out, _ = mod(qg, kg, vg, key_padding_mask=mask)
+    out.backward(w.to(dev))
+    tol = 3e-2 if dtype == torch.bfloat16 else 4e-3
+    for name, got, ref in (('dq', qg.grad, qd.grad), ('dk', kg.grad, kd.grad), ('dv', vg.grad, vd.grad)):
+        assert got.dtype == dtype and got.shape == ref.shape
+        diff = float((got.double().cpu() - ref).abs().max()) / max(float(ref.abs().max()), 1e-2)
+        assert diff <= tol, (name, diff)       # (d query is all zeros where a query sees one key: window-of-one)
+        zero = ref.abs().amax(-1) == 0         # rows without a partner in the band, or with a single one (d query)
+        assert float(got.float().cpu()[zero].abs().max() if bool(zero.any()) else 0.0) <= 1e-5, name
+
+
 @pytest.mark.parametrize('dtype,tol,E,p_drop', [(torch.float32, 1e-4, 64, 0.25), (torch.bfloat16, 3e-2, 64, 0.1),
                                                  (torch.float32, 1e-4, 24, 0.5)])
 def test_local_attention_dropout_inside_the_kernels(dtype, tol, E, p_drop):
