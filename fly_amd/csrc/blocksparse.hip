@@ -2522,6 +2522,285 @@ extern "C" int flyhip_bs_sdd_prob_dsoftmax_dropout(const void* dout, const void*
                                   stream, &second);
 }
 
+// ---------------------------------------------------------------------------------------
+// gradients of the one-kernel block-sparse attention without the probabilities in memory
+// ---------------------------------------------------------------------------------------
+// With P = 2^(scale log2e q.k - lse2[query]) on the nonzero 32 x 32 blocks, g = d out and delta = rowsum(g * out):
+// d v = P^T g, dS = P (g v^T - delta), d q = scale dS k, d k = scale dS^T q.  One kernel in two orientations, neither
+// of which writes P or dS: a workgroup owns four block-rows (query-major: d q, and delta on the way) or four
+// block-columns (key-major: d k and d v), a wave one of them with its two operands in registers (q and g rows; k and v
+// rows), and walks the union of their lists (union_table, transposed for key-major), every 32-row tile of the other
+// side (K with V; Q with g, lse2 and delta) staged once in LDS for the four waves.  Per block S^T = Y1 . x1 and
+// G^T = Y2 . x2 (the tile's rows picked so that a lane's results over the two 16-row blocks are eight consecutive
+// inner rows, the contraction slots of what follows), then d x^T[e][outer] += Y^T[e][inner] . {dS, P}[inner][outer]
+// with Y^T fragments by transposing LDS reads of the same tiles.
+struct AttnBwdArgs {
+    const void* q; const void* k; const void* v; const void* go; const void* out;
+    const float* lse2; float* delta;                 // (Z, H, 32 * query blocks); delta is written by the query-major launch
+    void* dq; void* dk; void* dv;
+    const int32_t* uni_ptr; const int32_t* uni_inner; const int32_t* uni_blk;      // of the launch's orientation
+    int outer_blocks, inner_blocks, q_blocks, grps_per_head, n_heads, Z;
+    long q_sz, q_sh, q_sm, k_sz, k_sh, k_sm, v_sz, v_sh, v_sm, g_sz, g_sh, g_sm, o_sz, o_sh, o_sm;
+    long dq_sz, dq_sh, dq_sm, dk_sz, dk_sh, dk_sm, dv_sz, dv_sh, dv_sm;
+    float scale;
+    int n_xcd;
+};
+
+// (registers for three waves per SIMD: the key-major form at 64 dims takes 176 without the bound, two waves per SIMD,
+//  and runs 7 % slower; a two-step register prefetch of the tiles costs more registers than it hides latency)
+template <typename T, int E, bool KEYMAJOR>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 8))) void bs_attn32_bwd_kernel(const AttnBwdArgs a) {
+    static_assert(sizeof(T) == 2 && E % 32 == 0, "2-byte inputs, whole MFMA steps");
+    constexpr int LD = E + 8, KS = E / 32, EB = E / 16;
+    constexpr int CPR = E / 8, NCH = (32 * CPR + 255) / 256;        // 16-byte chunks per tile row, per thread
+    constexpr float LOG2E = 1.4426950408889634f;
+    __shared__ __attribute__((aligned(16))) uint16_t tiles[2][2][32 * LD];      // [stage][Y1 | Y2]
+    __shared__ __attribute__((aligned(16))) float rowv[2][2][32];              // key-major: [stage][lse2 | delta] of the tile's queries
+    const int tid = threadIdx.x, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    int unit, grp;
+    if (!unit_of(blockIdx.x, a.n_xcd, a.grps_per_head, a.n_heads * a.Z, unit, grp)) return;
+    const int z = unit / a.n_heads, head = unit % a.n_heads;
+    const int ug = head * a.grps_per_head + grp;
+    const int p0 = a.uni_ptr[ug], n = a.uni_ptr[ug + 1] - p0;
+    const int bo = grp * 4 + w;
+    const bool have = bo < a.outer_blocks;
+    const int bo_c = min(bo, a.outer_blocks - 1);
+    const uint16_t* qz = reinterpret_cast<const uint16_t*>(a.q) + z * a.q_sz + head * a.q_sh;
+    const uint16_t* kz = reinterpret_cast<const uint16_t*>(a.k) + z * a.k_sz + head * a.k_sh;
+    const uint16_t* vz = reinterpret_cast<const uint16_t*>(a.v) + z * a.v_sz + head * a.v_sh;
+    const uint16_t* gz = reinterpret_cast<const uint16_t*>(a.go) + z * a.g_sz + head * a.g_sh;
+    const uint16_t* x1p = KEYMAJOR ? kz : qz;  const long x1s = KEYMAJOR ? a.k_sm : a.q_sm;     // outer operands
+    const uint16_t* x2p = KEYMAJOR ? vz : gz;  const long x2s = KEYMAJOR ? a.v_sm : a.g_sm;
+    const uint16_t* y1p = KEYMAJOR ? qz : kz;  const long y1s = KEYMAJOR ? a.q_sm : a.k_sm;     // inner tiles
+    const uint16_t* y2p = KEYMAJOR ? gz : vz;  const long y2s = KEYMAJOR ? a.g_sm : a.v_sm;
+    const long qvec = ((long)z * a.n_heads + head) * a.q_blocks * 32;                          // row vectors of this (z, head)
+    T* d1 = KEYMAJOR ? reinterpret_cast<T*>(a.dk) + z * a.dk_sz + head * a.dk_sh : reinterpret_cast<T*>(a.dq) + z * a.dq_sz + head * a.dq_sh;
+    const long d1s = KEYMAJOR ? a.dk_sm : a.dq_sm;
+    T* d2 = reinterpret_cast<T*>(a.dv) + z * a.dv_sz + head * a.dv_sh;
+
+    uintx4 x1[2][KS], x2[2][KS];
+    float l_own[2] = {0.f, 0.f}, d_own[2] = {0.f, 0.f};
+    floatx4 acc1[2][EB], acc2[KEYMAJOR ? 2 : 1][KEYMAJOR ? EB : 1];     // d q | d k, and d v
+#pragma unroll
+    for (int qq = 0; qq < 2; ++qq) {
+        const long row = (long)bo_c * 32 + 16 * qq + r16;
+#pragma unroll
+        for (int c = 0; c < KS; ++c) {
+            x1[qq][c] = *reinterpret_cast<const uintx4*>(x1p + row * x1s + 32 * c + 8 * g);
+            x2[qq][c] = *reinterpret_cast<const uintx4*>(x2p + row * x2s + 32 * c + 8 * g);
+        }
+        if (!KEYMAJOR) {
+            l_own[qq] = a.lse2[qvec + row];
+            // delta of the query, g . out, from the output row in the layout of the gradient row; kept for the key-major launch
+            const uint16_t* orow = reinterpret_cast<const uint16_t*>(a.out) + z * a.o_sz + head * a.o_sh + row * a.o_sm;
+            float part = 0.f;
+#pragma unroll
+            for (int c = 0; c < KS; ++c) {
+                const uintx4 ov = *reinterpret_cast<const uintx4*>(orow + 32 * c + 8 * g);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    T x, y;
+                    *reinterpret_cast<uint16_t*>(&x) = (uint16_t)(x2[qq][c][e >> 1] >> (16 * (e & 1)));
+                    *reinterpret_cast<uint16_t*>(&y) = (uint16_t)(ov[e >> 1] >> (16 * (e & 1)));
+                    part += Elem<T>::to_f32(x) * Elem<T>::to_f32(y);
+                }
+            }
+            d_own[qq] = group_sum(part);
+            if (have && g == 0) a.delta[qvec + row] = d_own[qq];
+        }
+#pragma unroll
+        for (int eb = 0; eb < EB; ++eb) acc1[qq][eb] = Frag<float>::zero();
+    }
+    if (KEYMAJOR) {
+#pragma unroll
+        for (int qq = 0; qq < 2; ++qq)
+#pragma unroll
+            for (int eb = 0; eb < EB; ++eb) acc2[qq][eb] = Frag<float>::zero();
+    }
+
+    uintx4 r1[NCH], r2[NCH];
+    float rl = 0.f, rd = 0.f;
+    auto fetch = [&](int inner) __attribute__((always_inline)) {
+        const long row0 = (long)inner * 32;
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int c = tid + 256 * i;
+            if (c < 32 * CPR) {
+                r1[i] = *reinterpret_cast<const uintx4*>(y1p + (row0 + c / CPR) * y1s + 8 * (c % CPR));
+                r2[i] = *reinterpret_cast<const uintx4*>(y2p + (row0 + c / CPR) * y2s + 8 * (c % CPR));
+            }
+        }
+        if (KEYMAJOR && tid < 32) {
+            rl = a.lse2[qvec + row0 + tid];
+            rd = a.delta[qvec + row0 + tid];
+        }
+    };
+    auto stash = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int c = tid + 256 * i;
+            if (c < 32 * CPR) {
+                *reinterpret_cast<uintx4*>(&tiles[buf][0][(c / CPR) * LD + 8 * (c % CPR)]) = r1[i];
+                *reinterpret_cast<uintx4*>(&tiles[buf][1][(c / CPR) * LD + 8 * (c % CPR)]) = r2[i];
+            }
+        }
+        if (KEYMAJOR && tid < 32) {
+            rowv[buf][0][tid] = rl;
+            rowv[buf][1][tid] = rd;
+        }
+    };
+    const float sc = a.scale * LOG2E;
+    const int foff = (8 * (r16 >> 2) + (r16 & 3)) * LD + 8 * g;         // + 4 b LD + 32 c   (elements)
+    const int toff = (8 * g + (r16 >> 2)) * LD + 4 * (r16 & 3);         // (+ 4 LD) + 16 eb
+    if (n > 0) {
+        fetch(a.uni_inner[p0]);
+        stash(0);
+    }
+    __syncthreads();
+    for (int s = 0; s < n; ++s) {
+        const int cur = s & 1;
+        const bool more = s + 1 < n;
+        if (more) fetch(a.uni_inner[p0 + s + 1]);
+        const bool present = have && a.uni_blk[(long)(p0 + s) * 4 + w] >= 0;      // wave-uniform
+        if (present) {
+            const uint16_t* Y1 = tiles[cur][0];
+            const uint16_t* Y2 = tiles[cur][1];
+            floatx4 s1[2][2], gp[2][2];                  // [outer block][inner block b]: scores (unscaled) and g.v
+#pragma unroll
+            for (int qq = 0; qq < 2; ++qq)
+#pragma unroll
+                for (int hb = 0; hb < 2; ++hb) { s1[qq][hb] = Frag<float>::zero(); gp[qq][hb] = Frag<float>::zero(); }
+#pragma unroll
+            for (int hb = 0; hb < 2; ++hb)
+#pragma unroll
+                for (int c = 0; c < KS; ++c) {
+                    const int off = foff + 4 * hb * LD + 32 * c;
+                    const uintx4 f1 = *reinterpret_cast<const uintx4*>(Y1 + off);
+                    const uintx4 f2 = *reinterpret_cast<const uintx4*>(Y2 + off);
+#pragma unroll
+                    for (int qq = 0; qq < 2; ++qq) {
+                        s1[qq][hb] = mma32<T>(f1, x1[qq][c], s1[qq][hb]);
+                        gp[qq][hb] = mma32<T>(f2, x2[qq][c], gp[qq][hb]);
+                    }
+                }
+            floatx4 ln4[2], dl4[2];                      // key-major: the tile's queries' lse2 and delta, by block
+            if (KEYMAJOR) {
+#pragma unroll
+                for (int hb = 0; hb < 2; ++hb) {
+                    ln4[hb] = *reinterpret_cast<const floatx4*>(&rowv[cur][0][8 * g + 4 * hb]);
+                    dl4[hb] = *reinterpret_cast<const floatx4*>(&rowv[cur][1][8 * g + 4 * hb]);
+                }
+            }
+#pragma unroll
+            for (int qq = 0; qq < 2; ++qq)
+#pragma unroll
+                for (int hb = 0; hb < 2; ++hb)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float lrow = KEYMAJOR ? ln4[hb][i] : l_own[qq], drow = KEYMAJOR ? dl4[hb][i] : d_own[qq];
+                        const float pr = __builtin_amdgcn_exp2f(fmaf(s1[qq][hb][i], sc, -lrow));   // (a row without scores: lse2 = +inf)
+                        s1[qq][hb][i] = pr;
+                        gp[qq][hb][i] = pr * (gp[qq][hb][i] - drow);
+                    }
+            uintx4 pb[KEYMAJOR ? 2 : 1], sb[2];
+#pragma unroll
+            for (int qq = 0; qq < 2; ++qq) {
+                sb[qq] = uintx4{pack2<T>(gp[qq][0][0], gp[qq][0][1]), pack2<T>(gp[qq][0][2], gp[qq][0][3]),
+                                pack2<T>(gp[qq][1][0], gp[qq][1][1]), pack2<T>(gp[qq][1][2], gp[qq][1][3])};
+                if (KEYMAJOR)
+                    pb[qq] = uintx4{pack2<T>(s1[qq][0][0], s1[qq][0][1]), pack2<T>(s1[qq][0][2], s1[qq][0][3]),
+                                    pack2<T>(s1[qq][1][0], s1[qq][1][1]), pack2<T>(s1[qq][1][2], s1[qq][1][3])};
+            }
+#pragma unroll
+            for (int eb = 0; eb < EB; ++eb) {
+                const uint16_t* p1 = Y1 + toff + 16 * eb;
+                const uintx4 t1 = lds_read_tr8(reinterpret_cast<const char*>(p1), reinterpret_cast<const char*>(p1 + 4 * LD));
+#pragma unroll
+                for (int qq = 0; qq < 2; ++qq) acc1[qq][eb] = mma32<T>(t1, sb[qq], acc1[qq][eb]);
+                if (KEYMAJOR) {
+                    const uint16_t* p2 = Y2 + toff + 16 * eb;
+                    const uintx4 t2 = lds_read_tr8(reinterpret_cast<const char*>(p2), reinterpret_cast<const char*>(p2 + 4 * LD));
+#pragma unroll
+                    for (int qq = 0; qq < 2; ++qq) acc2[qq][eb] = mma32<T>(t2, pb[qq], acc2[qq][eb]);
+                }
+            }
+        }
+        if (more) stash(cur ^ 1);
+        __syncthreads();
+    }
+    if (have) {
+#pragma unroll
+        for (int qq = 0; qq < 2; ++qq) {
+            const long row = (long)bo * 32 + 16 * qq + r16;
+#pragma unroll
+            for (int eb = 0; eb < EB; ++eb) store4_f32(d1 + row * d1s + 16 * eb + 4 * g, acc1[qq][eb] * a.scale);
+            if (KEYMAJOR) {
+#pragma unroll
+                for (int eb = 0; eb < EB; ++eb) store4_f32(d2 + row * a.dv_sm + 16 * eb + 4 * g, acc2[qq][eb]);
+            }
+        }
+    }
+}
+
+template <typename T, int E, bool KEYMAJOR>
+static int launch_attn_bwd(const AttnBwdArgs& a, hipStream_t st) {
+    AttnBwdArgs args = a;
+    args.n_xcd = machine().xcds;
+    const long grid = unit_grid((long)a.n_heads * a.Z, a.grps_per_head);
+    if (grid > 2147483647L) return fail(ERR_ARG, "bs_attn_bwd: too many workgroups");
+    hipLaunchKernelGGL((bs_attn32_bwd_kernel<T, E, KEYMAJOR>), dim3((unsigned)grid), dim3(256), 0, st, args);
+    return check_launch("bs_attn32_bwd_kernel");
+}
+
+extern "C" int flyhip_bs_attn_bwd(const void* q, const void* k, const void* v, const void* out, const void* grad_out,
+                                  const float* lse2, float* delta, void* dq, void* dk, void* dv,
+                                  const int32_t* row_ptr, const int32_t* row_inner, const int32_t* row_blk,
+                                  const int32_t* col_ptr, const int32_t* col_inner, const int32_t* col_blk,
+                                  int n_heads, int brows_per_head, int bcols_per_head, int Z, int E,
+                                  int64_t q_sz, int64_t q_sh, int64_t q_sm, int64_t k_sz, int64_t k_sh, int64_t k_sm,
+                                  int64_t v_sz, int64_t v_sh, int64_t v_sm, int64_t o_sz, int64_t o_sh, int64_t o_sm,
+                                  int64_t g_sz, int64_t g_sh, int64_t g_sm,
+                                  int64_t dq_sz, int64_t dq_sh, int64_t dq_sm, int64_t dk_sz, int64_t dk_sh, int64_t dk_sm,
+                                  int64_t dv_sz, int64_t dv_sh, int64_t dv_sm,
+                                  float scale, int dtype, void* stream) {
+    FLY_REQUIRE(q && k && v && out && grad_out && lse2 && delta && dq && dk && dv, "bs_attn_bwd: null pointer");
+    FLY_REQUIRE(row_ptr && row_inner && row_blk && col_ptr && col_inner && col_blk, "bs_attn_bwd: null table");
+    FLY_REQUIRE(n_heads > 0 && brows_per_head > 0 && bcols_per_head > 0 && Z > 0, "bs_attn_bwd: empty problem");
+    FLY_REQUIRE(E == 32 || E == 64, "bs_attn_bwd: head dim %d not in {32, 64}", E);
+    FLY_REQUIRE(dtype == BF16 || dtype == F16, "bs_attn_bwd supports bfloat16 and float16, got dtype code %d", dtype);
+    FLY_REQUIRE(((q_sz | q_sh | q_sm | k_sz | k_sh | k_sm | v_sz | v_sh | v_sm | o_sz | o_sh | o_sm | g_sz | g_sh | g_sm) % 8) == 0,
+                "bs_attn_bwd: input strides must be multiples of 8 elements (16-byte loads)");
+    FLY_REQUIRE(((dq_sz | dq_sh | dq_sm | dk_sz | dk_sh | dk_sm | dv_sz | dv_sh | dv_sm) % 4) == 0,
+                "bs_attn_bwd: output strides must be multiples of 4 elements (8-byte stores)");
+    FLY_REQUIRE(((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
+                  reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(grad_out)) % 16) == 0 &&
+                ((reinterpret_cast<uintptr_t>(dq) | reinterpret_cast<uintptr_t>(dk) | reinterpret_cast<uintptr_t>(dv)) % 8) == 0,
+                "bs_attn_bwd: pointers must be 16-byte (inputs) and 8-byte (outputs) aligned");
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (int rc_capture = refuse_capture(st)) return rc_capture;
+    AttnBwdArgs a{};
+    a.q = q; a.k = k; a.v = v; a.go = grad_out; a.out = out; a.lse2 = lse2; a.delta = delta; a.dq = dq; a.dk = dk; a.dv = dv;
+    a.q_blocks = brows_per_head; a.n_heads = n_heads; a.Z = Z; a.scale = scale;
+    a.q_sz = q_sz; a.q_sh = q_sh; a.q_sm = q_sm; a.k_sz = k_sz; a.k_sh = k_sh; a.k_sm = k_sm; a.v_sz = v_sz; a.v_sh = v_sh; a.v_sm = v_sm;
+    a.g_sz = g_sz; a.g_sh = g_sh; a.g_sm = g_sm; a.o_sz = o_sz; a.o_sh = o_sh; a.o_sm = o_sm;
+    a.dq_sz = dq_sz; a.dq_sh = dq_sh; a.dq_sm = dq_sm; a.dk_sz = dk_sz; a.dk_sh = dk_sh; a.dk_sm = dk_sm;
+    a.dv_sz = dv_sz; a.dv_sh = dv_sh; a.dv_sm = dv_sm;
+    for (int km = 0; km < 2; ++km) {                 // query-major first: it leaves delta for the key-major launch
+        a.uni_ptr = km ? col_ptr : row_ptr; a.uni_inner = km ? col_inner : row_inner; a.uni_blk = km ? col_blk : row_blk;
+        a.outer_blocks = km ? bcols_per_head : brows_per_head;
+        a.inner_blocks = km ? brows_per_head : bcols_per_head;
+        a.grps_per_head = (a.outer_blocks + 3) / 4;
+        int rc;
+#define ATTN_BWD_LAUNCH(TT, EE) rc = km ? launch_attn_bwd<TT, EE, true>(a, st) : launch_attn_bwd<TT, EE, false>(a, st)
+        if (dtype == BF16) { if (E == 32) ATTN_BWD_LAUNCH(bf16_t, 32); else ATTN_BWD_LAUNCH(bf16_t, 64); }
+        else { if (E == 32) ATTN_BWD_LAUNCH(f16_t, 32); else ATTN_BWD_LAUNCH(f16_t, 64); }
+#undef ATTN_BWD_LAUNCH
+        if (rc) return rc;
+    }
+    return 0;
+}
+
 extern "C" int flyhip_bs_sdd_prob(const void* q, const void* k, const float* lse2, void* p,
                                   const int32_t* uni_ptr, const int32_t* uni_inner, const int32_t* uni_blk,
                                   int nnz, int n_heads, int brows_per_head, int Z, int K, int blk,

@@ -564,6 +564,27 @@ int flyhip_bs_attn_masks(const void* q, const void* k, const void* v, void* out,
                          int64_t o_sz, int64_t o_sh, int64_t o_sm,
                          float scale, int dtype, void* stream);
 
+/* Gradients of flyhip_bs_attn_lse (the one-kernel block-sparse attention without masks; the reference takes them from
+ * autograd through sdd, softmax and dsd, src/models/attention/blocksparse_attention.py:134-160) without the
+ * probabilities in memory: with P = 2^(scale log2e q.k - lse2[query]) on the nonzero 32 x 32 blocks, g = grad_out and
+ * delta = rowsum(g * out): dv = P^T g, dS = P (g v^T - delta), dq = scale dS k, dk = scale dS^T q.  Two launches on
+ * the 16x16x32 MFMA of the input type: query-major over groups of four block-rows (dq; fills delta, caller-owned
+ * float32 scratch shaped like lse2) and key-major over groups of four block-columns (dk, dv).  row_* = union_table of
+ * the layout, col_* = the same of the transposed layout (block ids are only tested for >= 0).  q, out, grad_out, dq
+ * (Z, H, 32 brows, E) and k, v, dk, dv (Z, H, 32 bcols, E) via (batch, head, row) strides in elements, E in {32, 64},
+ * bfloat16 or float16; input strides in multiples of 8 and 16-byte aligned pointers, output strides in multiples of 4. */
+int flyhip_bs_attn_bwd(const void* q, const void* k, const void* v, const void* out, const void* grad_out,
+                       const float* lse2, float* delta, void* dq, void* dk, void* dv,
+                       const int32_t* row_ptr, const int32_t* row_inner, const int32_t* row_blk,
+                       const int32_t* col_ptr, const int32_t* col_inner, const int32_t* col_blk,
+                       int n_heads, int brows_per_head, int bcols_per_head, int Z, int E,
+                       int64_t q_sz, int64_t q_sh, int64_t q_sm, int64_t k_sz, int64_t k_sh, int64_t k_sm,
+                       int64_t v_sz, int64_t v_sh, int64_t v_sm, int64_t o_sz, int64_t o_sh, int64_t o_sm,
+                       int64_t g_sz, int64_t g_sh, int64_t g_sm,
+                       int64_t dq_sz, int64_t dq_sh, int64_t dq_sm, int64_t dk_sz, int64_t dk_sh, int64_t dk_sm,
+                       int64_t dv_sz, int64_t dv_sh, int64_t dv_sm,
+                       float scale, int dtype, void* stream);
+
 /* flyhip_bs_attn_masks with the dropout of BlockSparseAttention.forward (ref:
  * src/models/attention/blocksparse_attention.py:160, `dsd_nn(self.dropout(attn), v)`; the constructor's default
  * attention_dropout is 0.1, :31): every probability is dropped with probability dropout_p in [0, 1) after the softmax

@@ -732,6 +732,50 @@ def test_blocksparse_attention_module_gradients(masked, E, dtype):
         assert float(kg.grad[1, 200:].abs().max()) == 0.0
 
 
+@pytest.mark.parametrize('E,dtype,nb', [(64, torch.bfloat16, 13), (32, torch.float16, 13), (64, torch.float16, 6),
+                                          (32, torch.bfloat16, 22)])
+def test_blocksparse_attention_gradients_without_stored_probabilities(E, dtype, nb, monkeypatch):
+    """The backward after the one-kernel forward (flyhip_bs_attn_bwd: query-major launch for d query, key-major launch
+    for d key and d value, probabilities and score gradients formed per block and never written): ragged layouts that
+    differ by head -- a band on one, a band plus scattered blocks on the other -- with a block-row without blocks (zero
+    output, zero d query), a block-column without blocks (zero d key and d value), a number of block-rows that is no
+    multiple of four; against autograd through the oracle in float64 on the same rounded inputs."""
+    from fly_amd import BlockSparseAttention, _lib
+    print('case', E, dtype, nb, flush=True)
+    called, call = [], _lib.call
+    monkeypatch.setattr(_lib, 'call', lambda name, *args: (called.append(name), call(name, *args))[1])
+    g = torch.Generator().manual_seed(100 + nb)
+    lay = torch.stack([ob.band_layout(nb, nb, 1), ((torch.rand(nb, nb, generator=g) < 0.3) | (ob.band_layout(nb, nb, 2) > 0)).long()])
+    lay[0, 2, :] = 0                                      # a block-row without blocks
+    lay[1, :, 3] = 0                                      # a block-column without blocks
+    lay[:, nb - 1, nb - 1] = 1
+
+    class Cfg:
+        block = 32
+
+        def make_layout(self, seqlen):
+            return lay.clone()
+
+    B, T, H = 2, 32 * nb, 2
+    q, k, v = (torch.randn(B, T, H, E, generator=g).to(dtype) for _ in range(3))
+    w = torch.randn(B, T, H, E, generator=g).to(dtype)
+    mod = BlockSparseAttention(Cfg(), attention_dropout=0.0, max_seq_length=T).to(DEV)
+    qd, kd, vd = (x.double().requires_grad_() for x in (q, k, v))
+    ref = ob.blocksparse_attention(qd, kd, vd, lay, 32)
+    (ref * w.double()).sum().backward()
+    qg, kg, vg = (x.to(DEV).requires_grad_() for x in (q, k, v))
+    out, _ = mod(qg, kg, vg)
+    assert len(mod.fused_cache) == 1
+    tol = 3e-2 if dtype == torch.bfloat16 else 4e-3
+    assert rel_err(out, ref) <= tol
+    out.backward(w.to(DEV))
+    assert 'flyhip_bs_attn_bwd' in called and not any('dsoftmax' in name for name in called), called
+    for got, want, name in ((qg.grad, qd.grad, 'dq'), (kg.grad, kd.grad, 'dk'), (vg.grad, vd.grad, 'dv')):
+        assert got.dtype == dtype and rel_err(got.float(), want) <= tol, (name, rel_err(got.float(), want))
+    assert float(out.detach()[:, 64:96, 0].abs().max()) == 0.0 and float(qg.grad[:, 64:96, 0].abs().max()) == 0.0
+    assert float(kg.grad[:, 96:128, 1].abs().max()) == 0.0 and float(vg.grad[:, 96:128, 1].abs().max()) == 0.0
+
+
 @pytest.mark.parametrize('dtype,dropout', [(torch.float32, 0.0), (torch.bfloat16, 0.3)])
 def test_blocksparse_attention_gradients_with_fully_masked_rows(dtype, dropout):
     """Band-only layout plus a length mask: the query rows past the band of the last valid key see no key
