@@ -34,7 +34,7 @@ class _AttentionCoreFn(torch.autograd.Function):
     op-by-op chain's six plus elementwise passes:
     dV = P^T dO, dS = scale * P * (dO V^T - rowsum(dO * O)) in one kernel (the sdd fused with the softmax
     gradient), dQ = dS K, dK = dS^T Q.  32x32 blocks of bf16 / fp16 with shared-tile tables only.
-    After the one-kernel forward without dropout and with head dims up to 64 the backward is flyhip_bs_attn_bwd: two
+    After the one-kernel forward with head dims up to 64 the backward is flyhip_bs_attn_bwd: two
     launches (query-major for dQ, key-major for dK and dV) that form P and dS per block and never write them.
     ``dropout=(p, seed)`` (one-kernel forward only): the dropout of blocksparse_attention.py:160 with the mask
     a hash of (seed, batch, head, query, key) that the backward kernel forms again: it writes M * P for dV and
@@ -72,8 +72,8 @@ class _AttentionCoreFn(torch.autograd.Function):
             ok = x.stride(3) == 1 and all(s_ % 8 == 0 for s_ in x.stride()[:3]) and x.data_ptr() % 16 == 0
             return x if ok else x.contiguous()
         dout = vec(dout)
-        if ctx.recompute and ctx.dropout[0] == 0 and ctx.saved_tensors[0].shape[3] in (32, 64):
-            # no dropout, head dims up to 64: both orientations on one kernel that keeps neither P nor dS
+        if ctx.recompute and ctx.saved_tensors[0].shape[3] in (32, 64):
+            # head dims up to 64: both orientations on one kernel that keeps neither P nor dS (a dropout mask is formed again)
             q, k, v, out, lse2 = ctx.saved_tensors
             col_tabs = sdd._table('union_t', dout.device)
             if len(col_tabs) == 3:
@@ -90,7 +90,7 @@ class _AttentionCoreFn(torch.autograd.Function):
                               col_tabs[0].data_ptr(), col_tabs[1].data_ptr(), col_tabs[2].data_ptr(),
                               H, rows, cols, q.shape[0], q.shape[3], *st3(qq), *st3(kk), *st3(vv), *st3(oo), *st3(dout),
                               *st3(dq), *st3(dk), *st3(dv), float(ctx.scale), _lib.dtype_code(q),
-                              _lib.stream_ptr(q.device))
+                              float(ctx.dropout[0]), int(ctx.dropout[1]), _lib.stream_ptr(q.device))
                 return dq, dk, dv, None, None, None, None, None, None, None, None
         if ctx.recompute:
             # probabilities, score gradient, dq and the rows' delta = rowsum(d out * out) from one kernel: both

@@ -2544,18 +2544,21 @@ struct AttnBwdArgs {
     long dq_sz, dq_sh, dq_sm, dk_sz, dk_sh, dk_sm, dv_sz, dv_sh, dv_sm;
     float scale;
     int n_xcd;
+    // DROP: the forward dropped probabilities by the hash of (seed, row = (z H + head) L + query, key) (drop_keep): d v takes
+    // m P and dS = P (m g.v - delta), m = 0 or 1 / (1 - p)
+    uint32_t drop_seed, drop_thresh; float drop_scale;
 };
 
 // (registers for three waves per SIMD: the key-major form at 64 dims takes 176 without the bound, two waves per SIMD,
 //  and runs 7 % slower; a two-step register prefetch of the tiles costs more registers than it hides latency)
-template <typename T, int E, bool KEYMAJOR>
+template <typename T, int E, bool KEYMAJOR, bool DROP = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 8))) void bs_attn32_bwd_kernel(const AttnBwdArgs a) {
     static_assert(sizeof(T) == 2 && E % 32 == 0, "2-byte inputs, whole MFMA steps");
     constexpr int LD = E + 8, KS = E / 32, EB = E / 16;
     constexpr int CPR = E / 8, NCH = (32 * CPR + 255) / 256;        // 16-byte chunks per tile row, per thread
     constexpr float LOG2E = 1.4426950408889634f;
     __shared__ __attribute__((aligned(16))) uint16_t tiles[2][2][32 * LD];      // [stage][Y1 | Y2]
-    __shared__ __attribute__((aligned(16))) float rowv[2][2][32];              // key-major: [stage][lse2 | delta] of the tile's queries
+    __shared__ __attribute__((aligned(16))) float rowv[2][3][32];              // key-major: [stage][lse2 | delta | row hash] of the tile's queries
     const int tid = threadIdx.x, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     int unit, grp;
@@ -2581,6 +2584,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 8))) voi
 
     uintx4 x1[2][KS], x2[2][KS];
     float l_own[2] = {0.f, 0.f}, d_own[2] = {0.f, 0.f};
+    uint32_t h_own[2] = {0u, 0u};                     // DROP, query-major: hash of (seed, global row) of the lane's queries
     floatx4 acc1[2][EB], acc2[KEYMAJOR ? 2 : 1][KEYMAJOR ? EB : 1];     // d q | d k, and d v
 #pragma unroll
     for (int qq = 0; qq < 2; ++qq) {
@@ -2592,6 +2596,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 8))) voi
         }
         if (!KEYMAJOR) {
             l_own[qq] = a.lse2[qvec + row];
+            if (DROP) h_own[qq] = drop_row_hash(a.drop_seed, (uint32_t)(qvec + row));
             // delta of the query, g . out, from the output row in the layout of the gradient row; kept for the key-major launch
             const uint16_t* orow = reinterpret_cast<const uint16_t*>(a.out) + z * a.o_sz + head * a.o_sh + row * a.o_sm;
             float part = 0.f;
@@ -2621,6 +2626,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 8))) voi
 
     uintx4 r1[NCH], r2[NCH];
     float rl = 0.f, rd = 0.f;
+    uint32_t rh = 0u;
     auto fetch = [&](int inner) __attribute__((always_inline)) {
         const long row0 = (long)inner * 32;
 #pragma unroll
@@ -2634,6 +2640,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 8))) voi
         if (KEYMAJOR && tid < 32) {
             rl = a.lse2[qvec + row0 + tid];
             rd = a.delta[qvec + row0 + tid];
+            if (DROP) rh = drop_row_hash(a.drop_seed, (uint32_t)(qvec + row0 + tid));
         }
     };
     auto stash = [&](int buf) __attribute__((always_inline)) {
@@ -2648,6 +2655,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 8))) voi
         if (KEYMAJOR && tid < 32) {
             rowv[buf][0][tid] = rl;
             rowv[buf][1][tid] = rd;
+            if (DROP) rowv[buf][2][tid] = __uint_as_float(rh);
         }
     };
     const float sc = a.scale * LOG2E;
@@ -2684,14 +2692,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 8))) voi
                         gp[qq][hb] = mma32<T>(f2, x2[qq][c], gp[qq][hb]);
                     }
                 }
-            floatx4 ln4[2], dl4[2];                      // key-major: the tile's queries' lse2 and delta, by block
+            floatx4 ln4[2], dl4[2], hh4[2];              // key-major: the tile's queries' lse2, delta and row hashes, by block
             if (KEYMAJOR) {
 #pragma unroll
                 for (int hb = 0; hb < 2; ++hb) {
                     ln4[hb] = *reinterpret_cast<const floatx4*>(&rowv[cur][0][8 * g + 4 * hb]);
                     dl4[hb] = *reinterpret_cast<const floatx4*>(&rowv[cur][1][8 * g + 4 * hb]);
+                    if (DROP) hh4[hb] = *reinterpret_cast<const floatx4*>(&rowv[cur][2][8 * g + 4 * hb]);
                 }
             }
+            const int inner_cur = a.uni_inner[p0 + s];
 #pragma unroll
             for (int qq = 0; qq < 2; ++qq)
 #pragma unroll
@@ -2700,8 +2710,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 8))) voi
                     for (int i = 0; i < 4; ++i) {
                         const float lrow = KEYMAJOR ? ln4[hb][i] : l_own[qq], drow = KEYMAJOR ? dl4[hb][i] : d_own[qq];
                         const float pr = __builtin_amdgcn_exp2f(fmaf(s1[qq][hb][i], sc, -lrow));   // (a row without scores: lse2 = +inf)
-                        s1[qq][hb][i] = pr;
-                        gp[qq][hb][i] = pr * (gp[qq][hb][i] - drow);
+                        if (DROP) {
+                            // (query, key) of the element: the inner row 8 g + 4 hb + i of the tile, the outer row 16 qq + r16
+                            const uint32_t inner_row = (uint32_t)inner_cur * 32u + 8u * g + 4u * hb + i;
+                            const uint32_t outer_row = (uint32_t)bo_c * 32u + 16u * qq + r16;
+                            const uint32_t rhash = KEYMAJOR ? __float_as_uint(hh4[hb][i]) : h_own[qq];
+                            const float m = drop_keep(rhash, KEYMAJOR ? outer_row : inner_row, a.drop_thresh) ? a.drop_scale : 0.f;
+                            s1[qq][hb][i] = m * pr;
+                            gp[qq][hb][i] = pr * (m * gp[qq][hb][i] - drow);
+                        } else {
+                            s1[qq][hb][i] = pr;
+                            gp[qq][hb][i] = pr * (gp[qq][hb][i] - drow);
+                        }
                     }
             uintx4 pb[KEYMAJOR ? 2 : 1], sb[2];
 #pragma unroll
@@ -2743,14 +2763,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 8))) voi
     }
 }
 
-template <typename T, int E, bool KEYMAJOR>
-static int launch_attn_bwd(const AttnBwdArgs& a, hipStream_t st) {
+template <typename T, int E, bool KEYMAJOR, bool DROP>
+static int launch_attn_bwd_as(const AttnBwdArgs& a, hipStream_t st) {
     AttnBwdArgs args = a;
     args.n_xcd = machine().xcds;
     const long grid = unit_grid((long)a.n_heads * a.Z, a.grps_per_head);
     if (grid > 2147483647L) return fail(ERR_ARG, "bs_attn_bwd: too many workgroups");
-    hipLaunchKernelGGL((bs_attn32_bwd_kernel<T, E, KEYMAJOR>), dim3((unsigned)grid), dim3(256), 0, st, args);
+    hipLaunchKernelGGL((bs_attn32_bwd_kernel<T, E, KEYMAJOR, DROP>), dim3((unsigned)grid), dim3(256), 0, st, args);
     return check_launch("bs_attn32_bwd_kernel");
+}
+template <typename T, int E, bool KEYMAJOR>
+static int launch_attn_bwd(const AttnBwdArgs& a, hipStream_t st) {
+    return a.drop_thresh != 0u ? launch_attn_bwd_as<T, E, KEYMAJOR, true>(a, st) : launch_attn_bwd_as<T, E, KEYMAJOR, false>(a, st);
 }
 
 extern "C" int flyhip_bs_attn_bwd(const void* q, const void* k, const void* v, const void* out, const void* grad_out,
@@ -2763,8 +2787,10 @@ extern "C" int flyhip_bs_attn_bwd(const void* q, const void* k, const void* v, c
                                   int64_t g_sz, int64_t g_sh, int64_t g_sm,
                                   int64_t dq_sz, int64_t dq_sh, int64_t dq_sm, int64_t dk_sz, int64_t dk_sh, int64_t dk_sm,
                                   int64_t dv_sz, int64_t dv_sh, int64_t dv_sm,
-                                  float scale, int dtype, void* stream) {
+                                  float scale, int dtype, float dropout_p, uint64_t dropout_seed, void* stream) {
     FLY_REQUIRE(q && k && v && out && grad_out && lse2 && delta && dq && dk && dv, "bs_attn_bwd: null pointer");
+    FLY_REQUIRE(dropout_p >= 0.f && dropout_p < 1.f, "bs_attn_bwd: dropout_p %g not in [0, 1)", (double)dropout_p);
+    FLY_REQUIRE((long)Z * n_heads * brows_per_head * 32 <= 4294967295L, "bs_attn_bwd: more than 2^32 query rows");
     FLY_REQUIRE(row_ptr && row_inner && row_blk && col_ptr && col_inner && col_blk, "bs_attn_bwd: null table");
     FLY_REQUIRE(n_heads > 0 && brows_per_head > 0 && bcols_per_head > 0 && Z > 0, "bs_attn_bwd: empty problem");
     FLY_REQUIRE(E == 32 || E == 64, "bs_attn_bwd: head dim %d not in {32, 64}", E);
@@ -2782,6 +2808,8 @@ extern "C" int flyhip_bs_attn_bwd(const void* q, const void* k, const void* v, c
     AttnBwdArgs a{};
     a.q = q; a.k = k; a.v = v; a.go = grad_out; a.out = out; a.lse2 = lse2; a.delta = delta; a.dq = dq; a.dk = dk; a.dv = dv;
     a.q_blocks = brows_per_head; a.n_heads = n_heads; a.Z = Z; a.scale = scale;
+    const DropArgs drop = drop_args(dropout_p, dropout_seed);
+    a.drop_seed = drop.seed; a.drop_thresh = drop.thresh; a.drop_scale = drop.scale;
     a.q_sz = q_sz; a.q_sh = q_sh; a.q_sm = q_sm; a.k_sz = k_sz; a.k_sh = k_sh; a.k_sm = k_sm; a.v_sz = v_sz; a.v_sh = v_sh; a.v_sm = v_sm;
     a.g_sz = g_sz; a.g_sh = g_sh; a.g_sm = g_sm; a.o_sz = o_sz; a.o_sh = o_sh; a.o_sm = o_sm;
     a.dq_sz = dq_sz; a.dq_sh = dq_sh; a.dq_sm = dq_sm; a.dk_sz = dk_sz; a.dk_sh = dk_sh; a.dk_sm = dk_sm;

@@ -572,7 +572,9 @@ int flyhip_bs_attn_masks(const void* q, const void* k, const void* v, void* out,
  * float32 scratch shaped like lse2) and key-major over groups of four block-columns (dk, dv).  row_* = union_table of
  * the layout, col_* = the same of the transposed layout (block ids are only tested for >= 0).  q, out, grad_out, dq
  * (Z, H, 32 brows, E) and k, v, dk, dv (Z, H, 32 bcols, E) via (batch, head, row) strides in elements, E in {32, 64},
- * bfloat16 or float16; input strides in multiples of 8 and 16-byte aligned pointers, output strides in multiples of 4. */
+ * bfloat16 or float16; input strides in multiples of 8 and 16-byte aligned pointers, output strides in multiples of 4.
+ * dropout_p, dropout_seed: those of a flyhip_bs_attn_dropout forward (0 for none): the mask is formed again from the
+ * hash of (seed, (z H + head) L + query, key); dv takes m P and dS = P (m g.v - delta), m = 0 or 1 / (1 - p). */
 int flyhip_bs_attn_bwd(const void* q, const void* k, const void* v, const void* out, const void* grad_out,
                        const float* lse2, float* delta, void* dq, void* dk, void* dv,
                        const int32_t* row_ptr, const int32_t* row_inner, const int32_t* row_blk,
@@ -583,7 +585,7 @@ int flyhip_bs_attn_bwd(const void* q, const void* k, const void* v, const void* 
                        int64_t g_sz, int64_t g_sh, int64_t g_sm,
                        int64_t dq_sz, int64_t dq_sh, int64_t dq_sm, int64_t dk_sz, int64_t dk_sh, int64_t dk_sm,
                        int64_t dv_sz, int64_t dv_sh, int64_t dv_sm,
-                       float scale, int dtype, void* stream);
+                       float scale, int dtype, float dropout_p, uint64_t dropout_seed, void* stream);
 
 /* flyhip_bs_attn_masks with the dropout of BlockSparseAttention.forward (ref:
  * src/models/attention/blocksparse_attention.py:160, `dsd_nn(self.dropout(attn), v)`; the constructor's default
