@@ -78,7 +78,8 @@ class _AttentionCoreFn(torch.autograd.Function):
             col_tabs = sdd._table('union_t', dout.device)
             if len(col_tabs) == 3:
                 qq, kk, vv, oo = vec(q), vec(k), vec(v), vec(out)
-                dq, dk, dv = (torch.empty(x.shape, dtype=x.dtype, device=x.device) for x in (q, k, v))
+                # (in the layout of the inputs -- (B, T, H, E) seen as (B, H, T, E) -- so that autograd hands them on as they are)
+                dq, dk, dv = (torch.empty_like(x) for x in (qq, kk, vv))
                 delta = torch.empty_like(lse2)
 
                 def st3(x):
