@@ -2550,9 +2550,11 @@ struct AttnBwdArgs {
 };
 
 // (registers for three waves per SIMD: the key-major form at 64 dims takes 176 without the bound, two waves per SIMD,
-//  and runs 7 % slower; a two-step register prefetch of the tiles costs more registers than it hides latency)
+//  and runs 7 % slower; with the dropout hashes it would spill 24 registers inside the loop at that bound -- 703 us
+//  against 365 without dropout -- and keeps two waves; a two-step register prefetch of the tiles costs more registers
+//  than it hides latency)
 template <typename T, int E, bool KEYMAJOR, bool DROP = false>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 8))) void bs_attn32_bwd_kernel(const AttnBwdArgs a) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(KEYMAJOR && DROP ? 2 : 3, 8))) void bs_attn32_bwd_kernel(const AttnBwdArgs a) {
     static_assert(sizeof(T) == 2 && E % 32 == 0, "2-byte inputs, whole MFMA steps");
     constexpr int LD = E + 8, KS = E / 32, EB = E / 16;
     constexpr int CPR = E / 8, NCH = (32 * CPR + 255) / 256;        // 16-byte chunks per tile row, per thread
