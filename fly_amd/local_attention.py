@@ -104,7 +104,8 @@ def local_backward(query, key, value, local_context, softmax_temp, key_lengths, 
     Q, K, V, G = bh(query), bh(key), bh(value), bh(grad_out)
 
     def back(x, like):                           # (B*H, L, C) -> (B,L,H,C)
-        return x.reshape(B, H, x.shape[1], x.shape[2]).permute(0, 2, 1, 3).to(like.dtype)
+        # (in the inputs' own memory order: autograd then accumulates the gradient without another copy)
+        return x.reshape(B, H, x.shape[1], x.shape[2]).permute(0, 2, 1, 3).to(like.dtype, memory_format=torch.contiguous_format)
     if not Q.is_cuda and wdt != torch.float64:
         # host tensors are accepted for one purpose: checking the written-out gradient formulas in float64 against autograd
         raise NotImplementedError('local_backward runs on the GPU; host tensors only in float64 (the check of the formulas)')

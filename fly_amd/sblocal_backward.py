@@ -395,5 +395,6 @@ def sblocal_backward(query, key, value, projection_matrix, local_context, softma
         dK += st * ((uk[..., :mh] - uk[..., mh:]) @ P) - t * K * uk.sum(-1, keepdim=True)
 
     def back(x, like):                           # (B*H, L, C) -> (B,L,H,C)
-        return x.reshape(B, H, x.shape[1], x.shape[2]).permute(0, 2, 1, 3).to(like.dtype)
+        # (in the inputs' own memory order: autograd then accumulates the gradient without another copy)
+        return x.reshape(B, H, x.shape[1], x.shape[2]).permute(0, 2, 1, 3).to(like.dtype, memory_format=torch.contiguous_format)
     return back(dQ, query), back(dK, key), back(dV, value)
