@@ -87,6 +87,8 @@ struct KvArgs {
     long q_sb, q_sh, q_ss;
     int q_tiles;                    // query-role workgroups per (batch, head), after the n_split key-role ones
     void* vt;                       // bf16 inputs: V per 32-key tile, transposed ([d][k-slot]) for the band kernel's P V
+    // float path with operand images only: the element type of q, k, v in memory (0 float, 1 bfloat16, 2 float16)
+    int in_code = 0;
 };
 
 struct FwdArgs {
@@ -119,6 +121,8 @@ struct FwdArgs {
     // drop_thresh = 0 means none; pair (query i of (batch, head) bh, key s) is kept iff
     // drop_keep(drop_row_hash(drop_seed, bh T + i), s, drop_thresh), kept weights times drop_scale (bf16-piece kernel)
     uint32_t drop_seed, drop_thresh; float drop_scale;
+    // block-sparse support on operand images only: the element type of q and out in memory (0 float, 1 bfloat16, 2 float16)
+    int io_code = 0;
 };
 
 // ROWS x W tile of a (seq, W) matrix, moved global -> registers -> LDS in two steps so that all of
@@ -782,7 +786,9 @@ void sb_kfeat_kernel(KvArgs a) {
 //                the partial leaves in the natural feature order the combine step expects
 // One chunk of 64 keys = two tile images = 2 * X3Tile::BYTES of LDS, copied to global memory in 16-byte
 // pieces.  Instantiated where that fits next to the fp32 V chunk and the projection image (E <= 64, m <= 128).
-template <int E, int D, int M>
+// TIN: the element type of q, k and v in memory (float, or a 2-byte type widened as it is loaded: its values are exact
+// in two bf16 pieces at most).
+template <int E, int D, int M, typename TIN = float>
 __global__ __launch_bounds__(NT) void sb_kfeat_x3_kernel(KvArgs a) {
     typedef X3Tile<E, D, M> TL;
     constexpr int MH = M / 2, FB = MH / 16, EC = E / 16, DB = D / 16, KS = E / 32, FS = M / 32;
@@ -803,7 +809,7 @@ __global__ __launch_bounds__(NT) void sb_kfeat_x3_kernel(KvArgs a) {
         // Query role: the features of 64 queries, rounded to 17 bits, and their log-scales (see sb_kfeat_kernel)
         const float* pp = a.proj + r16 * E + 4 * g;
         const int iq = (sp - a.n_split) * TQ + 16 * w + r16;
-        const float* qrow = reinterpret_cast<const float*>(a.q) + b * a.q_sb + h * a.q_sh + (long)min(iq, a.T - 1) * a.q_ss;
+        const TIN* qrow = reinterpret_cast<const TIN*>(a.q) + b * a.q_sb + h * a.q_sh + (long)min(iq, a.T - 1) * a.q_ss;
         floatx4 qr[EC];
         float sq = 0.f;
 #pragma unroll
@@ -855,8 +861,8 @@ __global__ __launch_bounds__(NT) void sb_kfeat_x3_kernel(KvArgs a) {
         return;
     }
 
-    const float* kptr = reinterpret_cast<const float*>(a.k) + b * a.k_sb + h * a.k_sh;
-    const float* vptr = reinterpret_cast<const float*>(a.v) + b * a.v_sb + h * a.v_sh;
+    const TIN* kptr = reinterpret_cast<const TIN*>(a.k) + b * a.k_sb + h * a.k_sh;
+    const TIN* vptr = reinterpret_cast<const TIN*>(a.v) + b * a.v_sb + h * a.v_sh;
     const int len = a.lens ? min((int)a.lens[b], a.S) : a.S;
     const float lnm_half2 = 0.5f * __log2f(2.0f * a.mh_valid);
     const int per = (a.n_chunks + a.n_split - 1) / a.n_split;
@@ -870,7 +876,7 @@ __global__ __launch_bounds__(NT) void sb_kfeat_x3_kernel(KvArgs a) {
 #pragma unroll
         for (int j = 0; j < KNJ; ++j) {
             const int idx = tid + NT * j, row64 = idx / KCH8, cch = idx % KCH8;
-            const float* sp_ = kptr + (long)min(s_base + row64, a.S - 1) * a.k_ss + 32 * (cch >> 2) + 4 * (cch & 3);
+            const TIN* sp_ = kptr + (long)min(s_base + row64, a.S - 1) * a.k_ss + 32 * (cch >> 2) + 4 * (cch & 3);
             kq0[j] = load4_f32(sp_);
             kq1[j] = load4_f32(sp_ + 16);
         }
@@ -3638,7 +3644,8 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_kernel(FwdArgs a) {
 // LIST: the exact part lives on a block-sparse support instead of a band (see sblocal_fwd_kernel: the same lists of 32-key
 // tiles with a two-bit mask per wave and entry, the same start order, long lists walked in parts by the first workgroups
 // of the launch, which write un-normalised partials for sb_merge_kernel).  One part per ordinary tile: SPLIT is false.
-template <int E, int D, int M, bool SPLIT, bool DROPOUT = false, bool LIST = false>
+// TIO: the element type of q and out in memory (float, or a 2-byte type widened as it is loaded / rounded as it is stored).
+template <int E, int D, int M, bool SPLIT, bool DROPOUT = false, bool LIST = false, typename TIO = float>
 __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
     static_assert(!(LIST && SPLIT), "a block-sparse support is walked with one part per tile (long lists: a runtime role)");
     typedef X3Tile<E, D, M> TL;
@@ -3702,7 +3709,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
     const int q0 = qt * TQ;
     const int iq = q0 + 16 * w + r16;
     const bool qvalid = iq < a.T;
-    const float* qptr = reinterpret_cast<const float*>(a.q) + b * a.q_sb + h * a.q_sh;
+    const TIO* qptr = reinterpret_cast<const TIO*>(a.q) + b * a.q_sb + h * a.q_sh;
     const char* kv_img = reinterpret_cast<const char*>(a.vt) + (long)bh * a.n_chunks * (2 * (long)TL::KV_BYTES);
     const char* f_img = reinterpret_cast<const char*>(a.kfeat) + (long)bh * a.n_chunks * (2 * (long)TL::F_BYTES);
     const int len = a.lens ? min((int)a.lens[b], a.S) : a.S;
@@ -4141,7 +4148,7 @@ __global__ __launch_bounds__(NT) void sblocal_fwd_x3_kernel(FwdArgs a) {
         const float Z = ze + gamma * fmaxf(qk1 - zp, 1e-24f);
         const float inv = 1.0f / Z;
         if (qvalid) {
-            float* optr = reinterpret_cast<float*>(a.out) + b * a.o_sb + h * a.o_sh + (long)iq * a.o_ss;
+            TIO* optr = reinterpret_cast<TIO*>(a.out) + b * a.o_sb + h * a.o_sh + (long)iq * a.o_ss;
 #pragma unroll
             for (int db = 0; db < DB; ++db) store4_f32(optr + 16 * db + 4 * g, (oacc[db] + gamma * lacc[db]) * inv);
             if (g == 0) a.log_norm[(long)bh * a.T + iq] = m_run * LN2 + __logf(Z);
@@ -4381,14 +4388,20 @@ template <int E, int M>
 static int launch_kfeat_x3(const KvArgs& a, hipStream_t st) {
     if constexpr (E <= 64 && M <= 128) {
         // both products on the bf16 matrix pipe, images assembled in LDS
-        auto kern = sb_kfeat_x3_kernel<E, E, M>;
         constexpr size_t smem = kfeat_x3_smem<E, M>();
         static_assert(smem <= 160 * 1024, "two tile images, the V chunk and the projection image must fit the LDS");
-        static std::atomic<unsigned long long> lds_set{0};     // (devices on which this kernel has its LDS limit)
-        if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_set, "sb_kfeat_x3")) return rc;
-        hipLaunchKernelGGL(kern, dim3(a.n_split + a.q_tiles, a.B * a.H), dim3(NT), smem, st, a);
+        static std::atomic<unsigned long long> lds_set[3] = {{0}, {0}, {0}};     // (devices on which a kernel has its LDS limit)
+        const void* kern = a.in_code == 1   ? reinterpret_cast<const void*>(sb_kfeat_x3_kernel<E, E, M, bf16_t>)
+                           : a.in_code == 2 ? reinterpret_cast<const void*>(sb_kfeat_x3_kernel<E, E, M, f16_t>)
+                                            : reinterpret_cast<const void*>(sb_kfeat_x3_kernel<E, E, M, float>);
+        if (int rc = ensure_dynamic_lds(kern, smem, lds_set[a.in_code], "sb_kfeat_x3")) return rc;
+        const dim3 grid(a.n_split + a.q_tiles, a.B * a.H);
+        if (a.in_code == 1) hipLaunchKernelGGL((sb_kfeat_x3_kernel<E, E, M, bf16_t>), grid, dim3(NT), smem, st, a);
+        else if (a.in_code == 2) hipLaunchKernelGGL((sb_kfeat_x3_kernel<E, E, M, f16_t>), grid, dim3(NT), smem, st, a);
+        else hipLaunchKernelGGL((sb_kfeat_x3_kernel<E, E, M, float>), grid, dim3(NT), smem, st, a);
         return check_launch("sb_kfeat_x3_kernel");
     }
+    if (a.in_code != 0) return fail(ERR_UNSUPPORTED, "sb_kv_reduce: 2-byte inputs on the image path need head dims up to 64 and up to 128 features");
     auto kern = sb_kfeat_kernel<float, E, E, M, true>;
     constexpr size_t smem = kfeat_smem<E, M>();
     static std::atomic<unsigned long long> lds_set{0};     // (devices on which this kernel has its LDS limit)
@@ -4567,16 +4580,21 @@ static int launch_fwd_list(const FwdArgs& a, hipStream_t st) {
     const void* kern_fp32 = reinterpret_cast<const void*>(sblocal_fwd_kernel<float, E, E, M, false, true>);
     const void* kern = kern_fp32;
     size_t smem = fwd_smem<E, M>();
-    static std::atomic<unsigned long long> lds_set{0}, lds_set_x3{0};     // (devices on which the kernels have their LDS limit)
+    static std::atomic<unsigned long long> lds_set{0};     // (devices on which the kernels have their LDS limit)
+    if (a.io_code != 0 && !pieces)
+        return fail(ERR_UNSUPPORTED, "sbblocksparse_fwd: 2-byte q and out are read and written by the kernel on operand images only");
+    static std::atomic<unsigned long long> lds_set_x3v[6] = {{0}, {0}, {0}, {0}, {0}, {0}};
     if constexpr (X3) {
         if (pieces) {
-            kern = dropping ? reinterpret_cast<const void*>(sblocal_fwd_x3_kernel<E, E, M, false, true, true>)
-                            : reinterpret_cast<const void*>(sblocal_fwd_x3_kernel<E, E, M, false, false, true>);
+#define FLY_X3_LIST(DROP_, TIO_) reinterpret_cast<const void*>(sblocal_fwd_x3_kernel<E, E, M, false, DROP_, true, TIO_>)
+            kern = a.io_code == 1   ? (dropping ? FLY_X3_LIST(true, bf16_t) : FLY_X3_LIST(false, bf16_t))
+                   : a.io_code == 2 ? (dropping ? FLY_X3_LIST(true, f16_t) : FLY_X3_LIST(false, f16_t))
+                                    : (dropping ? FLY_X3_LIST(true, float) : FLY_X3_LIST(false, float));
+#undef FLY_X3_LIST
             smem = fwd_x3_smem<E, M>();
         }
     }
-    static std::atomic<unsigned long long> lds_set_x3d{0};
-    if (int rc = ensure_dynamic_lds(kern, smem, pieces ? (dropping ? lds_set_x3d : lds_set_x3) : lds_set, "sbblocksparse_fwd")) return rc;
+    if (int rc = ensure_dynamic_lds(kern, smem, pieces ? lds_set_x3v[2 * a.io_code + (dropping ? 1 : 0)] : lds_set, "sbblocksparse_fwd")) return rc;
     // every XCD gets room for ceil(B H / dies) (batch, head) pairs
     const Machine& mach = machine();
     const long grid = (((long)a.B * a.H + mach.xcds - 1) / mach.xcds) * ((a.T + TQ - 1) / TQ) * mach.xcds;
@@ -4589,16 +4607,23 @@ static int launch_fwd_list(const FwdArgs& a, hipStream_t st) {
     args.n_xcd = mach.xcds;
     args.band_wgs = (int)(grid + part_wgs);
     if constexpr (X3) {
-        if (pieces && dropping)
-            hipLaunchKernelGGL((sblocal_fwd_x3_kernel<E, E, M, false, true, true>), dim3((unsigned)(grid + part_wgs)), dim3(NT), smem, st, args);
-        else if (pieces)
-            hipLaunchKernelGGL((sblocal_fwd_x3_kernel<E, E, M, false, false, true>), dim3((unsigned)(grid + part_wgs)), dim3(NT), smem, st, args);
+        if (pieces) {
+            const dim3 grd((unsigned)(grid + part_wgs));
+#define FLY_X3_LIST_GO(DROP_, TIO_) hipLaunchKernelGGL((sblocal_fwd_x3_kernel<E, E, M, false, DROP_, true, TIO_>), grd, dim3(NT), smem, st, args)
+            if (a.io_code == 1) { if (dropping) FLY_X3_LIST_GO(true, bf16_t); else FLY_X3_LIST_GO(false, bf16_t); }
+            else if (a.io_code == 2) { if (dropping) FLY_X3_LIST_GO(true, f16_t); else FLY_X3_LIST_GO(false, f16_t); }
+            else { if (dropping) FLY_X3_LIST_GO(true, float); else FLY_X3_LIST_GO(false, float); }
+#undef FLY_X3_LIST_GO
+        }
     }
     if (!pieces)
         hipLaunchKernelGGL((sblocal_fwd_kernel<float, E, E, M, false, true>), dim3((unsigned)(grid + part_wgs)), dim3(NT), smem, st, args);
     int rc = check_launch("sblocal_fwd_kernel (block-sparse support)");
     if (rc || a.n_heavy <= 0) return rc;
-    hipLaunchKernelGGL((sb_merge_kernel<float, E, M>), dim3((unsigned)tiles, E / 16, 1), dim3(NT), 0, st, args);
+    const dim3 mgrid((unsigned)tiles, E / 16, 1);
+    if (a.io_code == 1) hipLaunchKernelGGL((sb_merge_kernel<bf16_t, E, M>), mgrid, dim3(NT), 0, st, args);
+    else if (a.io_code == 2) hipLaunchKernelGGL((sb_merge_kernel<f16_t, E, M>), mgrid, dim3(NT), 0, st, args);
+    else hipLaunchKernelGGL((sb_merge_kernel<float, E, M>), mgrid, dim3(NT), 0, st, args);
     return check_launch("sb_merge_kernel (long lists)");
 }
 
@@ -5184,6 +5209,10 @@ extern "C" int flyhip_sb_kv_reduce(const void* k, const void* v, const float* pr
                 "sb_kv_reduce: null pointer");
     FLY_REQUIRE(B > 0 && H > 0 && S > 0, "sb_kv_reduce: empty problem B=%d H=%d S=%d", B, H, S);
     FLY_REQUIRE(softmax_temp > 0.f, "sb_kv_reduce: softmax_temp must be positive");
+    // (float32 with operand images: bits 8..15 of dtype name the element type of q, k, v in memory, see flyhip_sbblocksparse_fwd)
+    const int in_code = (dtype >> 8) & 0xff;
+    dtype &= 0xff;
+    FLY_REQUIRE(in_code >= 0 && in_code <= 2 && (in_code == 0 || (dtype == F32 && vt)), "sb_kv_reduce: 2-byte tensors (code %d) go with float32 arithmetic on operand images", in_code);
     int rc = check_sb_dims("sb_kv_reduce", E, D, mh, mh_valid, dtype, k_sb | k_sh, k_ss, v_sb | v_sh | v_ss);
     if (rc) return rc;
     int nc, ns;
@@ -5201,6 +5230,7 @@ extern "C" int flyhip_sb_kv_reduce(const void* k, const void* v, const float* pr
              B, H, S, mh_valid, nc, n_split, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, softmax_temp,
              q, qfeat, q_lsq, q ? T : 0, q_sb, q_sh, q_ss,
              q ? (T + TQ - 1) / TQ : 0, vt};
+    a.in_code = in_code;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     if (int rc_capture = refuse_capture(st)) return rc_capture;
     const int m = 2 * mh;
@@ -5450,7 +5480,12 @@ extern "C" int flyhip_sbblocksparse_fwd(const void* q, const void* k, const void
     FLY_REQUIRE(B > 0 && H > 0 && T > 0 && S > 0, "sbblocksparse_fwd: empty problem");
     FLY_REQUIRE(T % 16 == 0 && S % 16 == 0, "sbblocksparse_fwd: sequence lengths %d, %d must be multiples of 16", T, S);
     FLY_REQUIRE(softmax_temp > 0.f, "sbblocksparse_fwd: softmax_temp must be positive");
-    FLY_REQUIRE(dtype == F32, "sbblocksparse_fwd: float32 inputs only (got dtype code %d)", dtype);
+    // dtype: float32, optionally with the element type of q, k, v and out in memory in bits 8..15 (FLYHIP_IO_BF16 /
+    // FLYHIP_IO_F16: the kernels on operand images widen what they load and round what they store)
+    const int io_code = (dtype >> 8) & 0xff;
+    dtype &= 0xff;
+    FLY_REQUIRE(dtype == F32, "sbblocksparse_fwd: float32 arithmetic only (got dtype code %d)", dtype);
+    FLY_REQUIRE(io_code >= 0 && io_code <= 2 && (io_code == 0 || vt), "sbblocksparse_fwd: 2-byte tensors (code %d) need the operand images", io_code);
     int rc = check_sb_dims("sbblocksparse_fwd", E, D, mh, mh_valid, dtype, q_sb | q_sh | q_ss | k_sb | k_sh | k_ss,
                            v_sb | v_sh | v_ss, o_sb | o_sh | o_ss);
     if (rc) return rc;
@@ -5466,6 +5501,7 @@ extern "C" int flyhip_sbblocksparse_fwd(const void* q, const void* k, const void
               tl_ptr, tl_inner, tl_blk, tl_order, tl_heavy, n_heavy};
     const DropArgs drop = drop_args(dropout_p, dropout_seed);
     a.drop_seed = drop.seed; a.drop_thresh = drop.thresh; a.drop_scale = drop.scale;
+    a.io_code = io_code;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     if (int rc_capture = refuse_capture(st)) return rc_capture;
     const int m = 2 * mh;

@@ -184,10 +184,12 @@ class SBBlockSparseAttention(nn.Module):
             key_ = (T, S, query.device)
             if key_ not in self.fused_tables:
                 self.fused_tables[key_] = fused_tables(layout, query.device, block)
-            # (2-byte inputs are widened, as on the op-by-op path below)
             if not needs_grad:
-                out, _ = sbblocksparse_forward(query.float(), key.float(), value.float(),
-                                               self.feature_map.projection_matrix, self.fused_tables[key_], softmax_temp,
+                # 2-byte inputs go to the kernels as they are where the kernels on operand images run (they widen what
+                # they load); otherwise they are widened here, as on the op-by-op path below
+                native = sbblocksparse_forward_supported(block, query.dtype, E, value.shape[3], n_rows, layout.shape[0], H)
+                qkv = (query, key, value) if native else (query.float(), key.float(), value.float())
+                out, _ = sbblocksparse_forward(*qkv, self.feature_map.projection_matrix, self.fused_tables[key_], softmax_temp,
                                                cache=self._scratch_cache, dropout_p=dropout[0], dropout_seed=dropout[1])
                 self.last_dropout_seed = dropout[1] if dropout[0] > 0 else None
                 return out.to(query.dtype), None
@@ -195,6 +197,7 @@ class SBBlockSparseAttention(nn.Module):
                 self.backward_tables[key_] = (backward_tables(layout, query.device, block=block),
                                               backward_tables(layout, query.device, transposed=True, block=block))
             support = self.backward_tables[key_]
+            # (with gradients 2-byte inputs are widened: the backward kernels take float32)
             out, _ = _SBBlockSparseFn.apply(query.float(), key.float(), value.float(), self.feature_map.projection_matrix,
                                             self.fused_tables[key_], support, softmax_temp, self._scratch_cache, dropout)
             self.last_dropout_seed = dropout[1] if dropout[0] > 0 else None

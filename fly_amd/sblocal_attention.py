@@ -105,7 +105,7 @@ class SBLocalPlan:
             self.q_lsq = torch.empty(B, H, T, dtype=f32, device=device)
         self._buffers = True
 
-    def run_keys(self, q, k, v, proj, lens, t, stream=None):
+    def run_keys(self, q, k, v, proj, lens, t, stream=None, io_code=0):
         """The key-side pass (features of the keys, K'^T V, sum K'); with several parts per query
         tile also the features of the queries `q`."""
         B, H, T, S, dim, mh, mh_valid = self.shape
@@ -120,7 +120,7 @@ class SBLocalPlan:
                   self.part_max.data_ptr(), self.kv.data_ptr(), self.ksum.data_ptr(), self.kmax.data_ptr(),
                   *q_args, _lib.ptr(self.vt), _lib.ptr(self.kvt), B, H, S, dim, dim, mh, mh_valid, self.n_split,
                   k.stride(0), k.stride(2), k.stride(1), v.stride(0), v.stride(2), v.stride(1),
-                  t, self.code, stream)
+                  t, self.code | (io_code << 8), stream)
 
     def run_queries(self, q, k, v, proj, lens, local_context, t, out, log_norm, stream=None):
         B, H, T, S, dim, mh, mh_valid = self.shape
@@ -152,13 +152,15 @@ class SBLocalPlan:
                   v.stride(0), v.stride(2), v.stride(1), out.stride(0), out.stride(2), out.stride(1),
                   t, self.code, stream)
 
-    def run_block_sparse(self, q, k, v, proj, t, tables, out, log_norm, dropout=(0.0, 0)):
+    def run_block_sparse(self, q, k, v, proj, t, tables, out, log_norm, dropout=(0.0, 0), io_code=0):
         """Scatterbrain attention whose exact part lives on a block-sparse support instead of a band: the
         key pass as in ``run``, then the band kernel walking lists of 32-key tiles (``tables`` =
         blocksparse_utils.tile_mask_table(layout, block) on the device) -- on bf16 pieces from the key pass's tile images
         when the plan has them (``operand_images``: float32, head dims up to 64, up to 128 features, no dropout), else on
         the fp32 matrix pipe.  One part per query tile, no key lengths.
-        dropout: (probability, seed) of the dropout of the exact weights inside the fp32 kernel."""
+        dropout: (probability, seed) of the dropout of the exact weights inside the fp32 kernel.
+        io_code: with operand images, q, k, v and out are tensors of that 2-byte element type (_lib.DTYPE_CODE of bfloat16 or
+        float16), widened as the kernels load them and rounded as they store: no float32 copies of them."""
         B, H, T, S, dim, mh, mh_valid = self.shape
         self._make_buffers()
         tl_ptr, tl_inner, tl_blk = tables[:3]
@@ -174,7 +176,7 @@ class SBLocalPlan:
                 self._heavy_sizes = need
         with torch.cuda.device(self.device):
             stream = _lib.stream_ptr(self.device)
-            self.run_keys(q, k, v, proj, None, t, stream)
+            self.run_keys(q, k, v, proj, None, t, stream, io_code=io_code)
             _lib.call('flyhip_sbblocksparse_fwd', q.data_ptr(), k.data_ptr(), v.data_ptr(), proj.data_ptr(),
                       self.kfeat.data_ptr(), _lib.ptr(self.vt), self.chunk_scale.data_ptr(), self.kv.data_ptr(),
                       self.ksum.data_ptr(), self.kmax.data_ptr(), tl_ptr.data_ptr(), _lib.table_ptr(tl_inner),
@@ -184,7 +186,7 @@ class SBLocalPlan:
                       B, H, T, S, dim, dim, mh, mh_valid,
                       q.stride(0), q.stride(2), q.stride(1), k.stride(0), k.stride(2), k.stride(1),
                       v.stride(0), v.stride(2), v.stride(1), out.stride(0), out.stride(2), out.stride(1),
-                      t, self.code, float(dropout[0]), int(dropout[1]), stream)
+                      t, self.code | (io_code << 8), float(dropout[0]), int(dropout[1]), stream)
 
     def run(self, q, k, v, proj, lens, local_context, t, out, log_norm, dropout=(0.0, 0)):
         """dropout: (probability, seed) -- dropout of the exact weights inside the band kernel (float32 inputs on the
@@ -350,9 +352,12 @@ def sblocal_forward(query, key, value, projection_matrix, local_context, softmax
 
 
 def sbblocksparse_forward_supported(block, dtype, E, D, n_projection_rows, layout_heads, H):
-    """Whether sbblocksparse_forward applies: blocks of 16 x 16 or 32 x 32, float32, one layout per attention head."""
-    return (block in (16, 32) and dtype == torch.float32 and max(E, D) <= _HEAD_DIMS[-1]
-            and n_projection_rows <= _FEATURE_ROWS[-1] and layout_heads == H)
+    """Whether sbblocksparse_forward applies: blocks of 16 x 16 or 32 x 32, one layout per attention head, float32 --
+    or bfloat16 / float16 where the kernels on operand images run (head dims up to 64, up to 64 projection rows)."""
+    fits = block in (16, 32) and max(E, D) <= _HEAD_DIMS[-1] and n_projection_rows <= _FEATURE_ROWS[-1] and layout_heads == H
+    if dtype in (torch.bfloat16, torch.float16):
+        return fits and max(E, D) <= 64 and n_projection_rows <= 64
+    return fits and dtype == torch.float32
 
 
 def sbblocksparse_forward(query, key, value, projection_matrix, tables, softmax_temp=None, cache=None,
@@ -361,7 +366,8 @@ def sbblocksparse_forward(query, key, value, projection_matrix, tables, softmax_
     need_weights=False; dropout_p, dropout_seed: the dropout of the exact weights of :200, by the hash mask of
     sblocal_forward) on the fused kernels: exact softmax weights on the nonzero blocks (16 x 16 or
     32 x 32), the Performer estimate everywhere else, one normaliser.  query (B,T,H,E), key (B,S,H,E), value
-    (B,S,H,D) float32 GPU tensors, T and S multiples of the block size; tables = blocksparse_utils.tile_mask_table(layout,
+    (B,S,H,D) float32 GPU tensors (bfloat16 / float16 with head dims up to 64 and up to 64 projection rows: read and
+    written as they are by the kernels on operand images, the arithmetic is the float32 path's), T and S multiples of the block size; tables = blocksparse_utils.tile_mask_table(layout,
     block) as int32 tensors on the device, optionally followed by union_order(tables[0], H), or the six entries of
     sbblocksparse_attention.fused_tables (start order with the long lists marked, those lists, their parts).
     cache: an optional ScratchCache kept by the caller (plan and padded projection, as for sblocal_forward).
@@ -386,16 +392,25 @@ def sbblocksparse_forward(query, key, value, projection_matrix, tables, softmax_
     # tile images of the key pass (the band kernel on bf16 pieces) where that kernel exists
     images = dim <= 64 and mh <= 64
 
+    io_code = 0
+    if query.dtype != torch.float32:
+        if not (images and query.dtype in (torch.bfloat16, torch.float16)
+                and key.dtype == query.dtype and value.dtype == query.dtype):
+            raise NotImplementedError('sbblocksparse_forward takes float32 tensors, or bfloat16 / float16 ones with head '
+                                      f'dims up to 64 and up to 64 projection rows (got {query.dtype}, {dim}, {mh})')
+        io_code = _lib.DTYPE_CODE[query.dtype]
+
     def make_plan():
-        return SBLocalPlan(B, H, T, S, dim, mh, mh_valid, query.dtype, query.device, 64, n_parts=1,
+        return SBLocalPlan(B, H, T, S, dim, mh, mh_valid, torch.float32, query.device, 64, n_parts=1,
                            operand_images=images)
-    plan_key = ('block-sparse', B, H, T, S, dim, mh, mh_valid, query.dtype, query.device, images)
+    plan_key = ('block-sparse', B, H, T, S, dim, mh, mh_valid, torch.float32, query.device, images)
     plan = make_plan() if cache is None else cache.plan(plan_key, make_plan)
     out = torch.empty(B, T, H, dim, dtype=query.dtype, device=query.device)
     log_norm = torch.empty(B, H, T, dtype=torch.float32, device=query.device)
     if not 0.0 <= dropout_p < 1.0:
         raise ValueError(f'dropout probability {dropout_p} not in [0, 1)')
-    plan.run_block_sparse(q, k, v, proj, t, tables, out, log_norm, dropout=(float(dropout_p), int(dropout_seed)))
+    plan.run_block_sparse(q, k, v, proj, t, tables, out, log_norm, dropout=(float(dropout_p), int(dropout_seed)),
+                          io_code=io_code)
     return out[..., :D], log_norm.unsqueeze(-1)
 
 

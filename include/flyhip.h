@@ -316,7 +316,9 @@ int flyhip_sbblocksparse_bwd_pieces(const void* outer_images, const void* inner_
  * walked in heavy_parts parts (2..64) by the first workgroups of the launch and finished by a merge launch; those
  * tiles carry the entry -1 - tile in tl_order so that no workgroup takes them whole, and every block-row of such
  * a tile must have at least one block.  Scratch for them: part_ws of B*n_heavy*heavy_parts*64*(D+5) floats and qfeat of
- * B*n_heavy*64*m floats (both NULL when n_heavy == 0).  float32 only; T, S multiples of 16.
+ * B*n_heavy*64*m floats (both NULL when n_heavy == 0).  float32 arithmetic only; T, S multiples of 16.  With the tile
+ * images (vt) q, k, v and out may be bfloat16 or float16 tensors: dtype = 0 | (1 << 8) resp. 0 | (2 << 8), here and in the
+ * flyhip_sb_kv_reduce call that precedes it -- the kernels widen what they load and round what they store.
  * dropout_p in [0, 1), dropout_seed: the dropout of the exact weights of sbblocksparse_attention.py:200 (the low-rank
  * part and the normaliser see none), by the hash mask that flyhip_sblocal_forward documents;
  * flyhip_sbblocksparse_bwd_pieces takes the same two values and forms the mask again. */

@@ -1148,6 +1148,56 @@ def test_sbblocksparse_gradients_with_long_lists_in_parts():
         assert rel_err(x, y) <= 1e-5, rel_err(x, y)
 
 
+@pytest.mark.parametrize('dtype,block', [(torch.bfloat16, 32), (torch.float16, 32), (torch.bfloat16, 16), (torch.float16, 16)])
+def test_sbblocksparse_forward_reads_2byte_tensors_as_they_are(dtype, block):
+    """bfloat16 / float16 q, k, v go to the kernels on operand images without float32 copies (the key pass and the band
+    kernel widen what they load, the band kernel and the merge of long lists round what they store): the arithmetic is the
+    float32 path's on the same values, so the output equals the float32 path's output rounded, bit for bit, and the
+    log-normaliser is the same.  Supports with a block-row of global tokens (a long list walked in parts and merged) and
+    windows, two heads that differ; against the oracle on the rounded inputs as well; through the module too."""
+    from fly_amd import SBBlockSparseAttention
+    from fly_amd.sbblocksparse_attention import fused_tables
+    from fly_amd.sblocal_attention import sbblocksparse_forward
+    from oracle import sbblocksparse as osbb
+    from oracle import sblocal as osb
+    print('case', dtype, block, flush=True)
+    B, H, L, E, m = 2, 2, 40 * block, 64, 64
+    nb = L // block
+    g = torch.Generator().manual_seed(13)
+    idx = torch.arange(nb)
+    window = ((idx[:, None] - idx[None, :]).abs() <= 1).long()
+    layout = torch.stack([window.clone(), window.clone()])
+    layout[0, 0, :] = 1
+    layout[0, :, 0] = 1
+    layout[1, 21, :] = 1
+    q, k, v = (torch.randn(B, L, H, E, generator=g) for _ in range(3))
+    q, k = (q * E ** -0.25).to(dtype), (k * E ** -0.25).to(dtype)
+    v = v.to(dtype)
+    P = osb.gaussian_orthogonal_random_matrix(m // 2, E, generator=g)
+    tables = fused_tables(layout, DEV, block)
+    out, ln = sbblocksparse_forward(q.to(DEV), k.to(DEV), v.to(DEV), P.to(DEV), tables)
+    assert out.dtype == dtype and ln.dtype == torch.float32
+    wide, ln_w = sbblocksparse_forward(q.float().to(DEV), k.float().to(DEV), v.float().to(DEV), P.to(DEV), tables)
+    assert torch.equal(out, wide.to(dtype)) and torch.equal(ln, ln_w)
+    ref_out, ref_ln = osbb.sbblocksparse_attention(q.double(), k.double(), v.double(), P.double(), layout, block)
+    assert rel_err(out, ref_out) <= (1e-2 if dtype == torch.bfloat16 else 2e-3)
+    assert rel_err(ln.reshape(ref_ln.shape), ref_ln) <= 1e-4
+
+    class Cfg:
+        def __init__(self):
+            self.block = block
+
+        def make_layout(self, seqlen):
+            return layout.clone()
+
+    layer = SBBlockSparseAttention(Cfg(), dim_heads=E, nb_features=m, max_seq_length=L).to(DEV).eval()
+    with torch.no_grad():
+        layer(q.to(DEV), k.to(DEV), v.to(DEV))                     # (the first call draws the projection)
+        layer.feature_map.projection_matrix.copy_(P)
+        got, _ = layer(q.to(DEV), k.to(DEV), v.to(DEV))
+    assert got.dtype == dtype and torch.equal(got, out)
+
+
 def test_sbblocksparse_long_lists_in_parts():
     """Block-rows of global tokens: their query tiles' lists are walked in parts by a second launch and merged
     (fused_tables marks them); output and log-normaliser against the oracle and against the one-part path."""
