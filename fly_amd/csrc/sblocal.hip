@@ -4258,7 +4258,7 @@ __global__ __launch_bounds__(NT) void sb_merge_kernel(FwdArgs a) {
 // workgroups wrote its parts (the dispatcher deals consecutive workgroup ids to the XCDs in turn): the
 // partials are then still in that XCD's L2.  xcd_items = band items (tile, part) per XCD of the band launch.
 // (the finish of tile tl, columns 16 NDB slice .. of it, by one workgroup; KVp: 3 M rows of 32 NDB bytes, KSs: M floats of LDS)
-template <int D, int M, int NDB>
+template <int D, int M, int NDB, typename TOUT = float>
 __device__ __forceinline__ void sb_merge_tile(const FwdArgs& a, int tl, int slice, char* KVp, float* KSs) {
     constexpr float LN2 = 0.6931471805599453f;
     constexpr int FC = M / 16, COLS = 16 * NDB, LDV = COLS + 4;
@@ -4340,13 +4340,13 @@ __device__ __forceinline__ void sb_merge_tile(const FwdArgs& a, int tl, int slic
     const float gamma = __builtin_amdgcn_exp2f(c0 - m_star);
     const float Z = ze + gamma * fmaxf(qk1 - zp, 1e-24f);
     const float inv = 1.0f / Z;
-    float* optr = reinterpret_cast<float*>(a.out) + b * a.o_sb + h * a.o_sh + (long)iq * a.o_ss + col0;
+    TOUT* optr = reinterpret_cast<TOUT*>(a.out) + b * a.o_sb + h * a.o_sh + (long)iq * a.o_ss + col0;
 #pragma unroll
     for (int db = 0; db < NDB; ++db) store4_f32(optr + 16 * db + 4 * g, (acc[db] + gamma * lacc[db]) * inv);
     if (g == 0 && slice == 0) a.log_norm[(long)bh * a.T + iq] = m_star * LN2 + __logf(Z);
 }
 
-template <int D, int M, int NDB>
+template <int D, int M, int NDB, typename TOUT = float>
 __global__ __launch_bounds__(NT) void sb_merge_x_kernel(FwdArgs a, int xcd_items, int tiles_per_xcd) {
     constexpr int COLS = 16 * NDB, NSL = D / COLS;
     __shared__ __attribute__((aligned(16))) char KVp[3 * M * 2 * COLS];
@@ -4358,7 +4358,7 @@ __global__ __launch_bounds__(NT) void sb_merge_x_kernel(FwdArgs a, int xcd_items
     const int t_hi = min(((x + 1) * xcd_items + a.n_parts - 1) / a.n_parts, n_tiles);
     const int tl = t_lo + j;
     if (j >= tiles_per_xcd || tl >= t_hi) return;     // workgroup-uniform
-    sb_merge_tile<D, M, NDB>(a, tl, slice, KVp, KSs);
+    sb_merge_tile<D, M, NDB, TOUT>(a, tl, slice, KVp, KSs);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -4507,9 +4507,9 @@ template <int E, int M> constexpr size_t fwd_x3_smem() {
     constexpr size_t lowrank = sizeof(float) * ((size_t)M * (E + 4) + M);
     return tiles > proj ? (tiles > lowrank ? tiles : lowrank) : (proj > lowrank ? proj : lowrank);
 }
-template <int E, int M, bool SPLIT, bool DROPOUT = false>
+template <int E, int M, bool SPLIT, bool DROPOUT = false, typename TIO = float>
 static int launch_fwd_x3(const FwdArgs& a, hipStream_t st) {
-    auto kern = sblocal_fwd_x3_kernel<E, E, M, SPLIT, DROPOUT>;
+    auto kern = sblocal_fwd_x3_kernel<E, E, M, SPLIT, DROPOUT, false, TIO>;
 #ifdef FLY_X3_PAD
     constexpr size_t smem = fwd_x3_smem<E, M>() + FLY_X3_PAD;
 #else
@@ -4549,12 +4549,24 @@ static int launch_fwd_x3(const FwdArgs& a, hipStream_t st) {
     constexpr int NDB = MERGE_NDB < E / 16 ? MERGE_NDB : E / 16;
     const int xcd_items = (int)((items + mach.xcds - 1) / mach.xcds);
     const int tiles_per_xcd = (xcd_items + a.n_parts - 1) / a.n_parts + 1;
-    hipLaunchKernelGGL((sb_merge_x_kernel<E, M, NDB>), dim3((unsigned)(mach.xcds * tiles_per_xcd * (E / 16 / NDB))), dim3(NT), 0, st,
+    hipLaunchKernelGGL((sb_merge_x_kernel<E, M, NDB, TIO>), dim3((unsigned)(mach.xcds * tiles_per_xcd * (E / 16 / NDB))), dim3(NT), 0, st,
                        args, xcd_items, tiles_per_xcd);
     return check_launch("sb_merge_x_kernel");
 }
 template <typename T, int E, int M>
 static int launch_fwd(const FwdArgs& a, hipStream_t st) {
+    if (a.io_code != 0) {
+        // float16 q and out on the kernels on operand images (bfloat16 tensors have kernels of their own)
+        if constexpr (sizeof(T) == 4 && E <= 64 && M <= 128) {
+            if (a.vt && a.io_code == 2) {
+                if (a.drop_thresh)
+                    return a.n_parts > 1 ? launch_fwd_x3<E, M, true, true, f16_t>(a, st) : launch_fwd_x3<E, M, false, true, f16_t>(a, st);
+                return a.n_parts > 1 ? launch_fwd_x3<E, M, true, false, f16_t>(a, st) : launch_fwd_x3<E, M, false, false, f16_t>(a, st);
+            }
+        }
+        return fail(ERR_UNSUPPORTED, "sblocal_fwd: 2-byte q and out (code %d) are read and written by the kernels on operand images "
+                                     "only: float16, head dims up to 64, up to 128 features", a.io_code);
+    }
     if (sizeof(T) == 4 && a.vt) {
         // (dropout of the exact weights: a variant of its own, so that the kernel without it carries nothing of it)
         if (a.drop_thresh) {
@@ -5259,6 +5271,10 @@ static int sblocal_fwd_checked(const void* q, const void* k, const void* v, cons
                                   float softmax_temp, int dtype, void* stream, DropArgs drop = DropArgs{0, 0, 1.f}) {
     FLY_REQUIRE(q && k && v && proj && kfeat && chunk_scale && kv && ksum && kmax && out && log_norm,
                 "sblocal_fwd: null pointer");
+    // (float32 with operand images: bits 8..15 of dtype name the element type of q and out in memory, see flyhip_sbblocksparse_fwd)
+    const int io_code = (dtype >> 8) & 0xff;
+    dtype &= 0xff;
+    FLY_REQUIRE(io_code == 0 || (io_code == 2 && dtype == F32 && vt), "sblocal_fwd: 2-byte tensors (code %d) are float16 with float32 arithmetic on operand images", io_code);
     // dropout lives in the band kernel on bf16 pieces (float inputs with the key pass's tile images)
     FLY_REQUIRE(drop.thresh == 0 || (dtype == F32 && vt && E <= 64 && 2 * mh <= 128),
                 "sblocal_fwd: dropout is implemented for float32 inputs with head dims up to 64 and up to 128 features "
@@ -5282,6 +5298,7 @@ static int sblocal_fwd_checked(const void* q, const void* k, const void* v, cons
               q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss, softmax_temp,
               nullptr, nullptr, nullptr};
     a.drop_seed = drop.seed; a.drop_thresh = drop.thresh; a.drop_scale = drop.scale;
+    a.io_code = io_code;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     if (int rc_capture = refuse_capture(st)) return rc_capture;
     return dispatch_fwd(dtype, E, 2 * mh, a, st);
@@ -5366,6 +5383,11 @@ extern "C" int flyhip_sblocal_forward(const void* q, const void* k, const void* 
     FLY_REQUIRE(dropout_p == 0.f || !(flags & SB_EXACT_FP32), "sblocal_forward: dropout is not implemented on the fp32-pipe kernels");
     FLY_REQUIRE((flags & ~SB_EXACT_FP32) == 0, "sblocal_forward: unknown flags 0x%x", flags);
     FLY_REQUIRE(B > 0 && H > 0 && T > 0 && S > 0 && local_context >= 1, "sblocal_forward: empty problem");
+    // (float32 on operand images: bits 8..15 of dtype = 2 for float16 q, k, v and out, widened as they are loaded, rounded as stored)
+    const int io_bits = dtype & 0xff00;
+    dtype &= 0xff;
+    FLY_REQUIRE(io_bits == 0 || (io_bits == (2 << 8) && dtype == F32 && !(flags & SB_EXACT_FP32)),
+                "sblocal_forward: 2-byte tensors are float16 with float32 arithmetic on operand images (dtype 0x%x)", dtype | io_bits);
     FLY_REQUIRE(dtype == F32 || dtype == BF16, "sblocal_forward supports float32 and bfloat16, got dtype code %d", dtype);
     FLY_REQUIRE(E == D && E > 0 && mh > 0, "sblocal_forward: padded head dims must be equal (E=%d, D=%d)", E, D);
     FLY_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0, "sblocal_forward: the workspace must be aligned to 256 bytes");
@@ -5384,14 +5406,14 @@ extern "C" int flyhip_sblocal_forward(const void* q, const void* k, const void* 
                                  f(w.kv), f(w.ksum), f(w.kmax),
                                  split ? q : nullptr, split ? f(w.qfeat) : nullptr, split ? f(w.q_lsq) : nullptr, T,
                                  q_sb, q_sh, q_ss, vt, kvt, B, H, S, E, D, mh, mh_valid, w.n_split,
-                                 k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, softmax_temp, dtype, stream);
+                                 k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, softmax_temp, dtype | io_bits, stream);
     if (rc) return rc;
     return sblocal_fwd_checked(q, k, v, proj, ws + w.kfeat, f(w.chunk_scale), f(w.kv), f(w.ksum), f(w.kmax),
                                split ? f(w.qfeat) : nullptr, split ? f(w.q_lsq) : nullptr, vt, kvt,
                                f(w.kv_part), f(w.part_max), w.n_split, key_lengths, out, log_norm,
                                split ? f(w.part_ws) : nullptr, w.n_parts, B, H, T, S, E, D, mh, mh_valid, local_context,
                                q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss,
-                               softmax_temp, dtype, stream, drop_args(dropout_p, dropout_seed));
+                               softmax_temp, dtype | io_bits, stream, drop_args(dropout_p, dropout_seed));
 }
 
 // ---------------------------------------------------------------------------------------

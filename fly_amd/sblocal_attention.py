@@ -188,12 +188,17 @@ class SBLocalPlan:
                       v.stride(0), v.stride(2), v.stride(1), out.stride(0), out.stride(2), out.stride(1),
                       t, self.code | (io_code << 8), float(dropout[0]), int(dropout[1]), stream)
 
-    def run(self, q, k, v, proj, lens, local_context, t, out, log_norm, dropout=(0.0, 0)):
+    def run(self, q, k, v, proj, lens, local_context, t, out, log_norm, dropout=(0.0, 0), io_code=0):
         """dropout: (probability, seed) -- dropout of the exact weights inside the band kernel (float32 inputs on the
-        bf16-piece kernels; the library refuses it elsewhere); the one-call path only."""
+        bf16-piece kernels; the library refuses it elsewhere); the one-call path only.
+        io_code: a float32 plan on operand images takes float16 q, k, v and out as they are (_lib.DTYPE_CODE[torch.float16]);
+        the one-call path only."""
         B, H, T, S, dim, mh, mh_valid = self.shape
         if dropout[0] > 0 and (self.n_parts != self.planned_parts or not self.operand_images or local_context != self.local_context):
             raise NotImplementedError('dropout needs the one-call path of the plan (its own part count and band)')
+        if io_code and (self.n_parts != self.planned_parts or not self.operand_images or local_context != self.local_context
+                        or self.flags):
+            raise NotImplementedError('float16 tensors are read as they are on the one-call path of a plan with operand images')
         if self.n_parts != self.planned_parts or not self.operand_images or local_context != self.local_context:
             # a part count or band the library would not choose itself: the two-call path takes them as arguments
             with torch.cuda.device(self.device):
@@ -208,7 +213,8 @@ class SBLocalPlan:
                       B, H, T, S, dim, dim, mh, mh_valid, local_context,
                       q.stride(0), q.stride(2), q.stride(1), k.stride(0), k.stride(2), k.stride(1),
                       v.stride(0), v.stride(2), v.stride(1), out.stride(0), out.stride(2), out.stride(1),
-                      t, self.code, self.flags, float(dropout[0]), int(dropout[1]), _lib.stream_ptr(self.device))
+                      t, self.code | (io_code << 8), self.flags, float(dropout[0]), int(dropout[1]),
+                      _lib.stream_ptr(self.device))
 
 
 class ScratchCache:
@@ -284,7 +290,8 @@ def sblocal_forward(query, key, value, projection_matrix, local_context, softmax
                     key_lengths=None, cache=None, exact_fp32=False, dropout_p=0.0, dropout_seed=0):
     """Scatterbrain-local attention forward on the GPU.
 
-    query (B,T,H,E), key (B,S,H,E), value (B,S,H,D) float32 or bfloat16 CUDA tensors;
+    query (B,T,H,E), key (B,S,H,E), value (B,S,H,D) float32 or bfloat16 CUDA tensors (float16 with head dims up to 64 and up
+    to 128 features: float32 arithmetic on the values as they are, no widened copies);
     projection_matrix (m/2, E); key_lengths (B,) int64 or None.  Computes what
     sblocal_attention.py:73-122 computes for causal=False, attn_mask=None, eps=0, no dropout.
     Returns (out (B,T,H,D) in the input dtype, log_normalization (B,H,T,1) float32).
@@ -303,8 +310,8 @@ def sblocal_forward(query, key, value, projection_matrix, local_context, softmax
     weights are scaled by 1 / (1 - p).  float32 inputs with head dims <= 64 and <= 128 features.
     """
     _lib.require_gpu(query, key, value, projection_matrix, key_lengths)
-    if query.dtype not in (torch.float32, torch.bfloat16):
-        raise NotImplementedError(f'SBLocal kernels support float32 and bfloat16, got {query.dtype}')
+    if query.dtype not in (torch.float32, torch.bfloat16, torch.float16):
+        raise NotImplementedError(f'SBLocal kernels support float32, bfloat16 and float16, got {query.dtype}')
     if key.dtype != query.dtype or value.dtype != query.dtype:
         raise ValueError('query, key and value must share a dtype')
     B, T, H, E = query.shape
@@ -336,18 +343,26 @@ def sblocal_forward(query, key, value, projection_matrix, local_context, softmax
             raise ValueError(f'key_lengths must have shape ({B},)')
 
     exact_fp32 = bool(exact_fp32) and query.dtype == torch.float32
-    plan_key = (B, H, T, S, dim, mh, mh_valid, query.dtype, query.device, local_context, exact_fp32)
+    # float16 tensors: the float32 plan on operand images, whose kernels widen what they load and round what they store
+    io_code, plan_dtype = 0, query.dtype
+    if query.dtype == torch.float16:
+        if dim > 64 or m > 128:
+            raise NotImplementedError('float16 tensors are read by the kernels on operand images: head dims up to 64, up '
+                                      f'to 128 features (got {max(E, D)}, {2 * mh_valid}); widen them to float32')
+        io_code, plan_dtype = _lib.DTYPE_CODE[torch.float16], torch.float32
+    plan_key = (B, H, T, S, dim, mh, mh_valid, plan_dtype, query.device, local_context, exact_fp32)
 
     def make_plan():
-        return SBLocalPlan(B, H, T, S, dim, mh, mh_valid, query.dtype, query.device, local_context,
+        return SBLocalPlan(B, H, T, S, dim, mh, mh_valid, plan_dtype, query.device, local_context,
                            exact_fp32=exact_fp32)
     plan = make_plan() if cache is None else cache.plan(plan_key, make_plan)
     out = torch.empty(B, T, H, dim, dtype=query.dtype, device=query.device)
     log_norm = torch.empty(B, H, T, dtype=torch.float32, device=query.device)
-    if dropout_p > 0 and (query.dtype != torch.float32 or exact_fp32 or dim > 64 or m > 128):
+    if dropout_p > 0 and (plan_dtype != torch.float32 or exact_fp32 or dim > 64 or m > 128):
         raise NotImplementedError('attention dropout is implemented in the band kernel on bf16 pieces: float32 inputs, '
                                   f'head dims <= 64, <= 128 features (got {query.dtype}, {max(E, D)}, {2 * mh_valid})')
-    plan.run(q, k, v, proj, lens, local_context, t, out, log_norm, dropout=(float(dropout_p), int(dropout_seed)))
+    plan.run(q, k, v, proj, lens, local_context, t, out, log_norm, dropout=(float(dropout_p), int(dropout_seed)),
+             io_code=io_code)
     return out[..., :D], log_norm.unsqueeze(-1)
 
 
@@ -523,17 +538,22 @@ class SBLocalAttention(nn.Module):
         if key_padding_mask is not None and not bool(key_padding_mask.all_ones):
             lengths = key_padding_mask.lengths          # raises ValueError unless a length mask
         self.feature_map.new_feature_map(query.device)
-        # float16 inputs (the reference's modules take whatever dtype autocast hands them) are widened to float32
-        # for the kernels -- exact, and the feature exponentials do not fit float16's range -- and the result goes
-        # back to float16; the casts are ordinary autograd nodes
+        # float16 inputs (the reference's modules take whatever dtype autocast hands them): the arithmetic is float32
+        # either way (exact widening; the feature exponentials do not fit float16's range).  Without gradients the
+        # kernels on operand images read them as they are and store the float16 result (head dims up to 64, up to 128
+        # features); otherwise they are widened here and the result goes back to float16, the casts being ordinary
+        # autograd nodes
         in_dtype = query.dtype
-        if in_dtype == torch.float16:
+        needs_grad = torch.is_grad_enabled() and any(x.requires_grad for x in (query, key, value))
+        as_it_is = (in_dtype == torch.float16 and not needs_grad and not self.exact_fp32
+                    and max(query.shape[3], value.shape[3]) <= 64 and self.feature_map.projection_matrix.shape[0] <= 64)
+        if in_dtype == torch.float16 and not as_it_is:
             query, key, value = query.float(), key.float(), value.float()
         out, log_norm = sblocal_attention_fn(query, key, value, self.feature_map.projection_matrix,
                                              self.local_context, softmax_temp=self.softmax_temp,
                                              key_lengths=lengths, cache=self._scratch_cache,
                                              exact_fp32=self.exact_fp32, dropout_p=dropout_p, dropout_seed=dropout_seed)
-        if in_dtype == torch.float16:
+        if in_dtype == torch.float16 and not as_it_is:
             out = out.to(in_dtype)
         self.last_log_normalization = log_norm.detach()
         attn = None

@@ -492,6 +492,32 @@ def test_gradients_at_benchmark_sizes_match_autograd_through_the_oracle(case):
         assert rel_err(got, ref) <= 2e-4, (name, rel_err(got, ref))
 
 
+@pytest.mark.parametrize('B,T,S,H,E,mh,lc,lens', [(2, 700, 700, 1, 64, 64, 256, None), (40, 512, 576, 2, 64, 32, 128, True),
+                                                 (3, 300, 300, 2, 48, 20, 64, True)])
+def test_sblocal_forward_reads_float16_as_it_is(B, T, S, H, E, mh, lc, lens):
+    """float16 q, k, v go to the kernels on operand images without float32 copies (key pass, band kernel, merge: they
+    widen what they load and round what they store): the float32 path's arithmetic on the same values, so the output is
+    that path's output rounded to float16, bit for bit, and the log-normaliser the same -- with the band split over
+    several workgroups and merged (small problems) and with one part per tile, key lengths, padded head dims."""
+    from fly_amd.sblocal_attention import sblocal_forward, SBLocalPlan
+    print('case', B, T, S, H, E, mh, lc, flush=True)
+    dev = torch.device('cuda:0')
+    g = torch.Generator().manual_seed(71)
+    q, k, v = (torch.randn(B, L, H, E, generator=g) for L in (T, S, S))
+    q, k, v = (q * E ** -0.25).half(), (k * E ** -0.25).half(), v.half()
+    P = osb.gaussian_orthogonal_random_matrix(mh, E, generator=g)
+    kl = None if lens is None else torch.randint(S // 2, S + 1, (B,), generator=g)
+    args = dict(key_lengths=None if kl is None else kl.to(dev))
+    out, ln = sblocal_forward(q.to(dev), k.to(dev), v.to(dev), P.to(dev), lc, **args)
+    wide, ln_w = sblocal_forward(q.float().to(dev), k.float().to(dev), v.float().to(dev), P.to(dev), lc, **args)
+    assert out.dtype == torch.float16 and ln.dtype == torch.float32
+    assert torch.equal(out, wide.half()) and torch.equal(ln, ln_w)
+    ref_out, ref_ln = osb.sblocal_attention(q.double(), k.double(), v.double(), P.double(), lc, key_lengths=kl)
+    assert rel_err(out, ref_out) <= 1e-3 and rel_err(ln.reshape(ref_ln.shape), ref_ln) <= 1e-4
+    parts = SBLocalPlan(B, H, T, S, 64, 64 if mh > 32 else 32, mh, torch.float32, dev, lc).n_parts
+    assert (parts > 1) == (B <= 3), parts
+
+
 def test_float16_inputs_are_widened_for_the_kernels():
     """SBLocalAttention and LocalAttention with float16 inputs (the dtype autocast hands the reference's modules):
     SBLocalAttention widens them to float32 for the kernels, LocalAttention runs its forward on the float16 matrix
