@@ -130,8 +130,9 @@ int flyhip_sblocal_fwd(const void* q, const void* k, const void* v, const float*
  * flyhip_bs_attn_dropout, with L = T -- and kept weights are scaled by 1 / (1 - p); flyhip_sblocal_bwd_pieces forms
  * the same mask from the same seed.  float32 inputs with head dims up to
  * 64 and up to 128 features (the kernels on bf16 pieces), not with FLYHIP_SB_EXACT_FP32; 0 = no dropout.
- * Arguments otherwise as for flyhip_sb_kv_reduce / flyhip_sblocal_fwd. * float16 tensors: dtype = 0 | (2 << 8) -- float32 arithmetic on operand images (not with FLYHIP_SB_EXACT_FP32; head dims up to
- * 64, up to 128 features) with q, k, v read and out written as float16: the kernels widen what they load and round
+ * Arguments otherwise as for flyhip_sb_kv_reduce / flyhip_sblocal_fwd.
+ * float16 tensors: dtype = 0 | (2 << 8) -- float32 arithmetic on operand images (not with FLYHIP_SB_EXACT_FP32; head dims
+ * up to 64, up to 128 features) with q, k, v read and out written as float16: the kernels widen what they load and round
  * what they store. */
 #define FLYHIP_SB_EXACT_FP32 1
 int64_t flyhip_sb_workspace_bytes(int B, int H, int T, int S, int E, int mh, int local_context, int dtype, int flags);
