@@ -38,7 +38,7 @@ SIGNATURES = {
     'flyhip_local_fwd': [c_vp] * 5 + [c_int] * 7 + [c_i64] * 12 + [c_float, c_int, c_vp],
     'flyhip_local_bwd': [c_vp] * 11 + [c_int] * 6 + [c_i64] * 24 + [c_float, c_int, c_vp],
     'flyhip_bs_sdd': [c_vp] * 4 + [c_int] + [c_vp] * 3 + [c_int] * 2 + [c_vp] * 3 + [c_int] * 3 + [c_i64] * 8 + [c_int, c_vp],
-    'flyhip_bs_attn_bwd': [c_vp] * 16 + [c_int] * 5 + [c_i64] * 24 + [c_float, c_int, c_float, c_u64, c_vp],
+    'flyhip_bs_attn_bwd': [c_vp] * 16 + [c_int] * 5 + [c_i64] * 24 + [c_float, c_int, c_float, c_u64, c_vp, c_i64, c_vp, c_i64, c_vp],
     'flyhip_bs_sdd_dsoftmax': [c_vp] * 8 + [c_int] * 6 + [c_i64] * 6 + [c_float, c_int, c_vp],
     'flyhip_bs_sdd_kmajor': [c_vp] * 8 + [c_int] * 8 + [c_i64] * 6 + [c_int, c_vp],
     'flyhip_bs_dsd': [c_vp] * 9 + [c_int] * 6 + [c_i64] * 9 + [c_int, c_vp],

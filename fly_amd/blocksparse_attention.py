@@ -43,13 +43,16 @@ class _AttentionCoreFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, sdd, dsd, sm, scale, kpm, am, fused, dropout=(0.0, 0)):
         ctx.ops, ctx.scale, ctx.dropout = (sdd, dsd), scale, dropout
-        if dropout[0] > 0 and not (fused is not None and kpm is None and am is None):
+        masked = kpm is not None or am is not None
+        if dropout[0] > 0 and not (fused is not None and not masked):
             raise NotImplementedError('dropout inside the kernels needs the one-kernel forward without masks')
-        if fused is not None and kpm is None and am is None:
-            # no masks: the one-kernel forward; it keeps the rows' log-denominators instead of the
-            # probabilities, which the backward forms again (one sdd with an exponential epilogue)
-            out, lse2 = fused(q, k, v, scale, None, return_lse=True, dropout=dropout)
+        ctx.masks = (None, None)
+        if fused is not None and (not masked or (dropout[0] == 0 and q.shape[3] in (32, 64))):
+            # the one-kernel forward; it keeps the rows' log-denominators instead of the probabilities, which the
+            # backward forms again.  With masks (head dims up to 64, no dropout) the backward kernels read them too.
+            out, lse2 = fused(q, k, v, scale, kpm, return_lse=True, attn_mask=am, dropout=dropout)
             ctx.save_for_backward(q, k, v, out, lse2)
+            ctx.masks = (kpm, am)
             ctx.recompute = True
             return out
         p = sm(sdd._run('sdd', q, k, False, True, False), scale=scale, key_padding_mask=kpm, attn_mask=am,
@@ -81,6 +84,9 @@ class _AttentionCoreFn(torch.autograd.Function):
                 # (in the layout of the inputs -- (B, T, H, E) seen as (B, H, T, E) -- so that autograd hands them on as they are)
                 dq, dk, dv = (torch.empty_like(x) for x in (qq, kk, vv))
                 delta = torch.empty_like(lse2)
+                kpm, am = ctx.masks
+                kpm = None if kpm is None else kpm.to(device=q.device, dtype=torch.float32).contiguous()
+                am = None if am is None else am.to(device=q.device, dtype=torch.float32).contiguous()
 
                 def st3(x):
                     return x.stride(0), x.stride(1), x.stride(2)
@@ -91,8 +97,11 @@ class _AttentionCoreFn(torch.autograd.Function):
                               col_tabs[0].data_ptr(), col_tabs[1].data_ptr(), col_tabs[2].data_ptr(),
                               H, rows, cols, q.shape[0], q.shape[3], *st3(qq), *st3(kk), *st3(vv), *st3(oo), *st3(dout),
                               *st3(dq), *st3(dk), *st3(dv), float(ctx.scale), _lib.dtype_code(q),
-                              float(ctx.dropout[0]), int(ctx.dropout[1]), _lib.stream_ptr(q.device))
+                              float(ctx.dropout[0]), int(ctx.dropout[1]), _lib.ptr(kpm), 0 if kpm is None else kpm.stride(0),
+                              _lib.ptr(am), 0 if am is None else am.stride(0), _lib.stream_ptr(q.device))
                 return dq, dk, dv, None, None, None, None, None, None, None, None
+            if ctx.masks != (None, None):
+                raise NotImplementedError('the backward with masks needs the shared-tile tables of the transposed layout')
         if ctx.recompute:
             # probabilities, score gradient, dq and the rows' delta = rowsum(d out * out) from one kernel: both
             # products (q k^T, d out v^T) per block
@@ -260,9 +269,12 @@ class BlockSparseAttention(nn.Module):
         sdd_nt, dsd_nn, sparse_softmax = self.get_ops(T, S)
         unmasked = ((key_padding_mask is None or key_padding_mask.all_ones)
                     and (attn_mask is None or attn_mask.all_ones))
-        one_kernel = self.fuse and unmasked and fused_attention.supports(block, query.dtype, E, value.shape[3])
-        # (with masks AND dropout a training step stays on the three ops below: the backward that forms the
-        # probabilities again does not read masks)
+        one_kernel = self.fuse and fused_attention.supports(block, query.dtype, E, value.shape[3])
+        if one_kernel and not unmasked:
+            # with masks: the backward kernels that read them take head dims up to 64 and no dropout (with masks AND
+            # dropout a training step stays on the three ops below)
+            one_kernel = (needs_grad and dropout[0] == 0.0 and E in (32, 64)
+                          and len(sdd_nt._table('union_t', query.device)) == 3)
         if (needs_grad and not need_weights and (dropout[0] == 0.0 or (one_kernel and dropout[0] < 1.0))
                 and E == value.shape[3] and _AttentionCoreFn.supports(sdd_nt, block, query.dtype, E, query.device)):
             fused = None
@@ -273,8 +285,8 @@ class BlockSparseAttention(nn.Module):
             self.last_dropout_seed = dropout[1] if dropout[0] > 0 else None
             out = _AttentionCoreFn.apply(
                 q, k, v, sdd_nt, dsd_nn, sparse_softmax, softmax_temp,
-                None if fused is not None or key_padding_mask is None else key_padding_mask.additive_matrix,
-                None if fused is not None or attn_mask is None else attn_mask.additive_matrix, fused, dropout)
+                None if unmasked or key_padding_mask is None else key_padding_mask.additive_matrix,
+                None if unmasked or attn_mask is None else attn_mask.additive_matrix, fused, dropout)
             return _cut(out.permute(0, 2, 1, 3), q_seqlen_og, v_dim_og), None
         qk = sdd_nt(q, k)
         attn = sparse_softmax(qk, scale=softmax_temp,

@@ -2547,14 +2547,20 @@ struct AttnBwdArgs {
     // DROP: the forward dropped probabilities by the hash of (seed, row = (z H + head) L + query, key) (drop_keep): d v takes
     // m P and dS = P (m g.v - delta), m = 0 or 1 / (1 - p)
     uint32_t drop_seed, drop_thresh; float drop_scale;
+    // the forward's additive masks (flyhip_bs_attn_masks), optional: key_mask (Z, keys) and attn_mask (queries, keys),
+    // float32, added to scale * q.k (0 / -inf, or any finite bias)
+    const float* key_mask; long km_stride; const float* attn_mask; long am_stride;
 };
 
 // (registers for three waves per SIMD: the key-major form at 64 dims takes 176 without the bound, two waves per SIMD,
 //  and runs 7 % slower; with the dropout hashes it would spill 24 registers inside the loop at that bound -- 703 us
 //  against 365 without dropout -- and keeps two waves; a two-step register prefetch of the tiles costs more registers
 //  than it hides latency)
-template <typename T, int E, bool KEYMAJOR, bool DROP = false>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(KEYMAJOR && DROP ? 2 : 3, 8))) void bs_attn32_bwd_kernel(const AttnBwdArgs a) {
+// MASKED: a variant of its own, so that the kernels without masks carry nothing of them (as a kernel-uniform branch the
+// mask code cost the key-major form 35 more spilled registers and the query-major form a wave per SIMD)
+template <typename T, int E, bool KEYMAJOR, bool DROP = false, bool MASKED = false>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(KEYMAJOR && (DROP || MASKED) ? 2 : 3, 8))) void bs_attn32_bwd_kernel(const AttnBwdArgs a) {
+    static_assert(!(DROP && MASKED), "the forward with masks has no dropout");
     static_assert(sizeof(T) == 2 && E % 32 == 0, "2-byte inputs, whole MFMA steps");
     constexpr int LD = E + 8, KS = E / 32, EB = E / 16;
     constexpr int CPR = E / 8, NCH = (32 * CPR + 255) / 256;        // 16-byte chunks per tile row, per thread
@@ -2586,6 +2592,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(KEYMAJOR &&
 
     uintx4 x1[2][KS], x2[2][KS];
     float l_own[2] = {0.f, 0.f}, d_own[2] = {0.f, 0.f};
+    float km_own[2] = {0.f, 0.f};                     // key-major: the key mask entries of the lane's keys
     uint32_t h_own[2] = {0u, 0u};                     // DROP, query-major: hash of (seed, global row) of the lane's queries
     floatx4 acc1[2][EB], acc2[KEYMAJOR ? 2 : 1][KEYMAJOR ? EB : 1];     // d q | d k, and d v
 #pragma unroll
@@ -2596,6 +2603,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(KEYMAJOR &&
             x1[qq][c] = *reinterpret_cast<const uintx4*>(x1p + row * x1s + 32 * c + 8 * g);
             x2[qq][c] = *reinterpret_cast<const uintx4*>(x2p + row * x2s + 32 * c + 8 * g);
         }
+        if (MASKED && KEYMAJOR && a.key_mask) km_own[qq] = a.key_mask[z * a.km_stride + row];
         if (!KEYMAJOR) {
             l_own[qq] = a.lse2[qvec + row];
             if (DROP) h_own[qq] = drop_row_hash(a.drop_seed, (uint32_t)(qvec + row));
@@ -2704,6 +2712,28 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(KEYMAJOR &&
                 }
             }
             const int inner_cur = a.uni_inner[p0 + s];
+            if constexpr (MASKED) {                                     // the masks, in units of the unscaled scores
+                const float inv_scale = 1.0f / a.scale;
+#pragma unroll
+                for (int qq = 0; qq < 2; ++qq)
+#pragma unroll
+                    for (int hb = 0; hb < 2; ++hb) {
+                        const long in0 = (long)inner_cur * 32 + 8 * g + 4 * hb;        // the element's four inner rows
+                        const long orow = (long)bo_c * 32 + 16 * qq + r16;             // its outer row
+                        floatx4 add = Frag<float>::zero();
+                        if (!KEYMAJOR) {
+                            if (a.key_mask) add += *reinterpret_cast<const floatx4*>(a.key_mask + z * a.km_stride + in0);
+                            if (a.attn_mask) add += *reinterpret_cast<const floatx4*>(a.attn_mask + orow * a.am_stride + in0);
+                        } else {
+                            if (a.key_mask) add += km_own[qq];
+                            if (a.attn_mask) {
+#pragma unroll
+                                for (int i = 0; i < 4; ++i) add[i] += a.attn_mask[(in0 + i) * a.am_stride + orow];
+                            }
+                        }
+                        s1[qq][hb] += add * inv_scale;
+                    }
+            }
 #pragma unroll
             for (int qq = 0; qq < 2; ++qq)
 #pragma unroll
@@ -2765,17 +2795,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(KEYMAJOR &&
     }
 }
 
-template <typename T, int E, bool KEYMAJOR, bool DROP>
+template <typename T, int E, bool KEYMAJOR, bool DROP, bool MASKED = false>
 static int launch_attn_bwd_as(const AttnBwdArgs& a, hipStream_t st) {
     AttnBwdArgs args = a;
     args.n_xcd = machine().xcds;
     const long grid = unit_grid((long)a.n_heads * a.Z, a.grps_per_head);
     if (grid > 2147483647L) return fail(ERR_ARG, "bs_attn_bwd: too many workgroups");
-    hipLaunchKernelGGL((bs_attn32_bwd_kernel<T, E, KEYMAJOR, DROP>), dim3((unsigned)grid), dim3(256), 0, st, args);
+    hipLaunchKernelGGL((bs_attn32_bwd_kernel<T, E, KEYMAJOR, DROP, MASKED>), dim3((unsigned)grid), dim3(256), 0, st, args);
     return check_launch("bs_attn32_bwd_kernel");
 }
 template <typename T, int E, bool KEYMAJOR>
 static int launch_attn_bwd(const AttnBwdArgs& a, hipStream_t st) {
+    if (a.key_mask != nullptr || a.attn_mask != nullptr) return launch_attn_bwd_as<T, E, KEYMAJOR, false, true>(a, st);
     return a.drop_thresh != 0u ? launch_attn_bwd_as<T, E, KEYMAJOR, true>(a, st) : launch_attn_bwd_as<T, E, KEYMAJOR, false>(a, st);
 }
 
@@ -2789,8 +2820,15 @@ extern "C" int flyhip_bs_attn_bwd(const void* q, const void* k, const void* v, c
                                   int64_t g_sz, int64_t g_sh, int64_t g_sm,
                                   int64_t dq_sz, int64_t dq_sh, int64_t dq_sm, int64_t dk_sz, int64_t dk_sh, int64_t dk_sm,
                                   int64_t dv_sz, int64_t dv_sh, int64_t dv_sm,
-                                  float scale, int dtype, float dropout_p, uint64_t dropout_seed, void* stream) {
+                                  float scale, int dtype, float dropout_p, uint64_t dropout_seed,
+                                  const float* key_mask, int64_t key_mask_stride, const float* attn_mask, int64_t attn_mask_stride,
+                                  void* stream) {
     FLY_REQUIRE(q && k && v && out && grad_out && lse2 && delta && dq && dk && dv, "bs_attn_bwd: null pointer");
+    FLY_REQUIRE(scale > 0.f, "bs_attn_bwd: scale must be positive");
+    FLY_REQUIRE((!key_mask || key_mask_stride % 4 == 0) && (!attn_mask || attn_mask_stride % 4 == 0) &&
+                ((reinterpret_cast<uintptr_t>(key_mask) | reinterpret_cast<uintptr_t>(attn_mask)) % 16) == 0,
+                "bs_attn_bwd: mask rows must be 16-byte aligned (strides in multiples of 4 floats)");
+    FLY_REQUIRE(dropout_p == 0.f || (!key_mask && !attn_mask), "bs_attn_bwd: no dropout together with masks (the forward has none)");
     FLY_REQUIRE(dropout_p >= 0.f && dropout_p < 1.f, "bs_attn_bwd: dropout_p %g not in [0, 1)", (double)dropout_p);
     FLY_REQUIRE((long)Z * n_heads * brows_per_head * 32 <= 4294967295L, "bs_attn_bwd: more than 2^32 query rows");
     FLY_REQUIRE(row_ptr && row_inner && row_blk && col_ptr && col_inner && col_blk, "bs_attn_bwd: null table");
@@ -2812,6 +2850,7 @@ extern "C" int flyhip_bs_attn_bwd(const void* q, const void* k, const void* v, c
     a.q_blocks = brows_per_head; a.n_heads = n_heads; a.Z = Z; a.scale = scale;
     const DropArgs drop = drop_args(dropout_p, dropout_seed);
     a.drop_seed = drop.seed; a.drop_thresh = drop.thresh; a.drop_scale = drop.scale;
+    a.key_mask = key_mask; a.km_stride = key_mask_stride; a.attn_mask = attn_mask; a.am_stride = attn_mask_stride;
     a.q_sz = q_sz; a.q_sh = q_sh; a.q_sm = q_sm; a.k_sz = k_sz; a.k_sh = k_sh; a.k_sm = k_sm; a.v_sz = v_sz; a.v_sh = v_sh; a.v_sm = v_sm;
     a.g_sz = g_sz; a.g_sh = g_sh; a.g_sm = g_sm; a.o_sz = o_sz; a.o_sh = o_sh; a.o_sm = o_sm;
     a.dq_sz = dq_sz; a.dq_sh = dq_sh; a.dq_sm = dq_sm; a.dk_sz = dk_sz; a.dk_sh = dk_sh; a.dk_sm = dk_sm;

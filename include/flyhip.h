@@ -579,7 +579,9 @@ int flyhip_bs_attn_masks(const void* q, const void* k, const void* v, void* out,
  * (Z, H, 32 brows, E) and k, v, dk, dv (Z, H, 32 bcols, E) via (batch, head, row) strides in elements, E in {32, 64},
  * bfloat16 or float16; input strides in multiples of 8 and 16-byte aligned pointers, output strides in multiples of 4.
  * dropout_p, dropout_seed: those of a flyhip_bs_attn_dropout forward (0 for none): the mask is formed again from the
- * hash of (seed, (z H + head) L + query, key); dv takes m P and dS = P (m g.v - delta), m = 0 or 1 / (1 - p). */
+ * hash of (seed, (z H + head) L + query, key); dv takes m P and dS = P (m g.v - delta), m = 0 or 1 / (1 - p).
+ * key_mask (Z, keys) and attn_mask (queries, keys), both optional: the additive masks of a flyhip_bs_attn_masks forward
+ * (float32, row strides in multiples of 4), added to scale q.k before the exponential; not together with dropout. */
 int flyhip_bs_attn_bwd(const void* q, const void* k, const void* v, const void* out, const void* grad_out,
                        const float* lse2, float* delta, void* dq, void* dk, void* dv,
                        const int32_t* row_ptr, const int32_t* row_inner, const int32_t* row_blk,
@@ -590,7 +592,9 @@ int flyhip_bs_attn_bwd(const void* q, const void* k, const void* v, const void* 
                        int64_t g_sz, int64_t g_sh, int64_t g_sm,
                        int64_t dq_sz, int64_t dq_sh, int64_t dq_sm, int64_t dk_sz, int64_t dk_sh, int64_t dk_sm,
                        int64_t dv_sz, int64_t dv_sh, int64_t dv_sm,
-                       float scale, int dtype, float dropout_p, uint64_t dropout_seed, void* stream);
+                       float scale, int dtype, float dropout_p, uint64_t dropout_seed,
+                       const float* key_mask, int64_t key_mask_stride, const float* attn_mask, int64_t attn_mask_stride,
+                       void* stream);
 
 /* flyhip_bs_attn_masks with the dropout of BlockSparseAttention.forward (ref:
  * src/models/attention/blocksparse_attention.py:160, `dsd_nn(self.dropout(attn), v)`; the constructor's default

@@ -685,13 +685,14 @@ def test_dsd_with_transposed_sparse_operand(p, r, N, dtype):
 
 
 @pytest.mark.parametrize('masked,E,dtype', [(True, 64, torch.bfloat16), (False, 64, torch.bfloat16), (False, 32, torch.bfloat16),
-                                            (False, 128, torch.bfloat16), (False, 64, torch.float16)])
+                                            (False, 128, torch.bfloat16), (False, 64, torch.float16), (True, 32, torch.float16),
+                                            (True, 128, torch.bfloat16)])
 def test_blocksparse_attention_module_gradients(masked, E, dtype):
-    """Training path of BlockSparseAttention for 2-byte inputs: one autograd node whose backward runs
-    dV, the fused score gradient, dQ and dK on the tiled kernels; gradients against autograd through
-    the oracle in float64 on the same rounded inputs.  With padded keys the forward is the three ops and
-    keeps the probabilities; without masks it is the one-kernel attention and the backward forms the
-    probabilities again from the rows' log-denominators."""
+    """Training path of BlockSparseAttention for 2-byte inputs: one autograd node; gradients against autograd through
+    the oracle in float64 on the same rounded inputs.  The forward is the one-kernel attention and the backward forms
+    the probabilities again from the rows' log-denominators -- per block, without writing them, for head dims up to 64
+    (with padded keys the backward kernels read the key mask too); at 128 dims dV, the fused score gradient, dQ and dK on
+    the tiled kernels."""
     from fly_amd import BlockSparseAttention, LengthMask
 
     class Cfg:
@@ -715,7 +716,7 @@ def test_blocksparse_attention_module_gradients(masked, E, dtype):
     (ref * w.double()).sum().backward()
     qg, kg, vg = (x.to(DEV).requires_grad_() for x in (q, k, v))
     out, _ = mod(qg, kg, vg, key_padding_mask=LengthMask(lengths.to(DEV), max_len=T) if masked else None)
-    assert (len(mod.fused_cache) == 1) == (not masked)
+    assert (len(mod.fused_cache) == 1) == (not masked or E <= 64)      # (with masks: the backward kernels that read them)
     seen, todo = set(), [out.grad_fn]
     while todo:                                           # the node sits behind the views that un-pad the output
         fn = todo.pop()
@@ -823,6 +824,58 @@ def test_blocksparse_attention_gradients_with_fully_masked_rows(dtype, dropout):
                                                      key_lengths=lengths)) <= 1e-4
         for got, want in ((qg.grad, qd.grad), (kg.grad, kd.grad), (vg.grad, vd.grad)):
             assert rel_err(got, want) <= 1e-4, rel_err(got, want)
+
+
+@pytest.mark.parametrize('dtype,E,with_attn_mask', [(torch.bfloat16, 64, False), (torch.float16, 32, True), (torch.bfloat16, 64, True)])
+def test_blocksparse_attention_masked_gradients_without_stored_probabilities(dtype, E, with_attn_mask, monkeypatch):
+    """Training with masks on the one-kernel forward and the backward that forms the probabilities again per block
+    (flyhip_bs_attn_masks, flyhip_bs_attn_bwd with key_mask / attn_mask): a band-only layout plus a length mask, so that
+    the query rows past the band of the last valid key see no key at all (zero output, zero gradients, nothing
+    non-finite), optionally a FullMask attention mask that hides scattered pairs; output and gradients against a dense
+    masked softmax in float64 whose rows without a visible key are zero rows."""
+    from fly_amd import BlockSparseAttention, LengthMask, FullMask, _lib
+    print('case', dtype, E, with_attn_mask, flush=True)
+    called, call = [], _lib.call
+    monkeypatch.setattr(_lib, 'call', lambda name, *args: (called.append(name), call(name, *args))[1])
+
+    class Cfg:
+        block = 32
+
+        def make_layout(self, seqlen):
+            nb = seqlen // self.block
+            return ob.band_layout(nb, nb, 1).unsqueeze(0).repeat(2, 1, 1)
+
+    B, T, H = 2, 256, 2
+    g = torch.Generator().manual_seed(19)
+    q, k, v = (torch.randn(B, T, H, E, generator=g).to(dtype) for _ in range(3))
+    w = torch.randn(B, T, H, E, generator=g).to(dtype)
+    lengths = torch.tensor([T, 70])              # batch 1: block-rows 4.. see only masked keys
+    keep = torch.rand(T, T, generator=g) < 0.8 if with_attn_mask else torch.ones(T, T, dtype=torch.bool)
+    keep[torch.arange(T), torch.arange(T)] = True
+    mod = BlockSparseAttention(Cfg(), attention_dropout=0.0, max_seq_length=T).to(DEV).train()
+    qg, kg, vg = (x.to(DEV).requires_grad_() for x in (q, k, v))
+    out, _ = mod(qg, kg, vg, key_padding_mask=LengthMask(lengths.to(DEV), max_len=T),
+                 attn_mask=FullMask(keep.to(DEV)) if with_attn_mask else None)
+    assert len(mod.fused_cache) == 1
+    assert float(out[1, 128:].detach().abs().max()) == 0.0
+    out.backward(w.to(DEV))
+    assert 'flyhip_bs_attn_bwd' in called and 'flyhip_bs_attn_masks' in called, called
+    for grad in (qg.grad, kg.grad, vg.grad):
+        assert bool(torch.isfinite(grad).all())
+    assert float(kg.grad[1, 70:].abs().max()) == 0.0 and float(vg.grad[1, 70:].abs().max()) == 0.0
+    assert float(qg.grad[1, 128:].abs().max()) == 0.0
+    qd, kd, vd = (x.double().requires_grad_() for x in (q, k, v))
+    lay = ob.densify_tensor(torch.ones(1, int(mod.master_layout.sum()), 32, 32), mod.master_layout.cpu())[0].bool()
+    vis = lay.unsqueeze(0) & keep.view(1, 1, T, T) & (torch.arange(T).view(1, 1, 1, T) < lengths.view(B, 1, 1, 1))
+    sc = torch.einsum('bthe,bshe->bhts', qd, kd) / math.sqrt(E)
+    live = vis.any(-1, keepdim=True)
+    p = torch.softmax(torch.where(live, sc.masked_fill(~vis, float('-inf')), torch.zeros_like(sc)), -1) * live
+    ref = torch.einsum('bhts,bshd->bthd', p, vd)
+    (ref * w.double()).sum().backward()
+    tol = 3e-2 if dtype == torch.bfloat16 else 4e-3
+    assert rel_err(out, ref) <= tol
+    for got, want, name in ((qg.grad, qd.grad, 'dq'), (kg.grad, kd.grad, 'dk'), (vg.grad, vd.grad, 'dv')):
+        assert rel_err(got.float(), want) <= tol, (name, rel_err(got.float(), want))
 
 
 @pytest.mark.parametrize('E,dtype,p_drop', [(64, torch.bfloat16, 0.25), (32, torch.float16, 0.1), (128, torch.bfloat16, 0.5)])
