@@ -280,6 +280,18 @@ def bench_blocksparse(steps, warmup):
         o.backward(gm)
         qm.grad = km.grad = vm.grad = None
     out['module_fwd_bwd_ms'] = timeit(module_step)
+    # ... with a key-padding mask (every second batch entry 500 keys short): the one-kernel forward reads it, and so do
+    # the two launches of the backward (blocksparse_attention.py:117-127,146-152)
+    from fly_amd import LengthMask
+    lens = torch.full((B,), L, dtype=torch.long)
+    lens[1::2] = L - 500
+    pad_mask = LengthMask(lens.to(dev), max_len=L)
+
+    def module_masked_step():
+        o, _ = mod(qm, km, vm, key_padding_mask=pad_mask)
+        o.backward(gm)
+        qm.grad = km.grad = vm.grad = None
+    out['module_key_padding_fwd_bwd_ms'] = timeit(module_masked_step)
     # ... and with the constructor's default attention dropout of 0.1 (blocksparse_attention.py:31,160): the mask
     # is a hash formed inside the same kernels; `fuse = False` is the op-by-op chain with nn.Dropout on the
     # stored probabilities
